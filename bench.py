@@ -1,0 +1,145 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: DCGAN-64 generator forward, fp32, batch 256.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step is one forward pass of the generator over one batch of synthetic latents that are already resident in HBM
+(the fused C-ABI path: Linear, 4 x (BatchNorm + ReLU, transposed conv 4x4 s2 p1), tanh).  Prints ONE JSON line:
+value = images/s of the whole step; conv_gflops / conv_frac_of_fp32_mfma_peak = algorithmic FLOPs (2*MAC, non-zero
+taps only) of the four transposed convolutions over the time of their kernels; roofline = the dominant kernel
+(the matrix-core implicit GEMM of the three large transposed convolutions) measured with HIP events on the
+library's stream inside the timed region; cpu_baseline = the reference's CPU path (oracle/_ref when built, else
+the C restatement) timed on this host on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "cuda-cnn-gan-vae_amd"))
+
+FP32_MFMA_PEAK_TFLOPS = 157.3
+BATCH = 256
+
+
+def hip_events():
+    """hipEvent helpers on the library's stream (torch.cuda.Event would watch torch's own stream)."""
+    hip = ctypes.CDLL("libamdhip64.so")
+    def create():
+        e = ctypes.c_void_p()
+        assert hip.hipEventCreate(ctypes.byref(e)) == 0
+        return e
+    def record(e, stream):
+        assert hip.hipEventRecord(e, ctypes.c_void_p(stream)) == 0
+    def elapsed_ms(a, b):
+        assert hip.hipEventSynchronize(b) == 0
+        ms = ctypes.c_float()
+        assert hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+        return ms.value
+    return create, record, elapsed_ms
+
+
+def cpu_baseline(sample_batch):
+    """The CPU path on this host, single thread (the reference has no active OpenMP), on `sample_batch` images."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle_api                       # the checker's library, timed here as the reported baseline only
+    import layer_sequences as seq
+    import generator as G
+    kind = "reference" if oracle_api.available("ref") else "port"
+    cpu = oracle_api.Oracle("ref" if kind == "reference" else "oracle")
+    params, z = G.make_parameters(), G.make_latent(sample_batch)
+    t0 = time.perf_counter()
+    seq.dcgan_generator_forward(cpu, params, z)
+    dt = time.perf_counter() - t0
+    return {"value": sample_batch / dt, "unit": "images/s", "cores": 1, "kind": kind,
+            "sample": "one generator forward at batch %d (%.1f s), scaled linearly; host has %d cores" % (sample_batch, dt, os.cpu_count() or 0)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--cpu-sample-batch", type=int, default=4)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the path shards along the batch axis, see DESIGN.md")
+
+    import mi355tensor as mt
+    import generator as G
+
+    net = G.DcganGenerator(BATCH)
+    net.set_latent(G.make_latent(BATCH))
+    stream = mt.get_stream()
+    create, record, elapsed_ms = hip_events()
+
+    for _ in range(args.warmup):
+        net.forward_fused()
+    mt.synchronize()
+
+    # timed region: K steps between two events on the work stream, host wall clock beside it
+    e0, e1 = create(), create()
+    mt.profile_enable(True)          # per-kernel events inside the same region
+    mt.synchronize()
+    t0 = time.perf_counter()
+    record(e0, stream)
+    for _ in range(args.steps):
+        net.forward_fused()
+    record(e1, stream)
+    mt.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = elapsed_ms(e0, e1)
+    prof = mt.profile_report()
+    mt.profile_enable(False)
+
+    ms_per_step = max(gpu_ms, wall_ms) / args.steps
+    flops = G.conv_flops(BATCH)
+    conv_kernels = {k: v for k, v in prof.items() if k.startswith("mt_backward_convolution")}
+    conv_ms = sum(v[1] for v in conv_kernels.values()) / args.steps
+    conv_tflops = sum(flops) / (conv_ms * 1e-3) / 1e12
+
+    # dominant kernel: the implicit GEMM of the three large layers (12 launches per step, 2*256*512*16*256*4/4 FLOP each)
+    big = [(k, v) for k, v in conv_kernels.items() if "32x128" not in k and "direct" not in k]
+    dom_label = max(big, key=lambda kv: kv[1][1])[0] if big else None
+    dom_launches = sum(v[0] for _, v in big)
+    dom_ms = sum(v[1] for _, v in big)
+    flop_per_launch = sum(flops[:3]) / 12.0
+    achieved = flop_per_launch / (dom_ms / dom_launches * 1e-3) / 1e12 if dom_launches else 0.0
+
+    result = {
+        "metric": "images/sec, DCGAN-64 generator fwd fp32 b=256 (conv GFLOP/s and % fp32 MFMA peak beside it)",
+        "value": BATCH / (ms_per_step * 1e-3),
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: DCGAN-64 generator forward, batch 256, latent 100 -> 512x4x4 -> 256 -> 128 -> 64 -> 3x64x64, BN(batch stats)+ReLU, tanh",
+                   "global_batch": BATCH, "path": "fused C-ABI entry points"},
+        "conv_gflops": conv_tflops * 1e3,
+        "conv_ms_per_step": conv_ms,
+        "conv_frac_of_fp32_mfma_peak": conv_tflops / FP32_MFMA_PEAK_TFLOPS,
+        "gpu_ms_per_step_events": gpu_ms / args.steps,
+        "host_ms_per_step_wall": wall_ms / args.steps,
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None, "kernel": dom_label,
+                     "launches_per_step": dom_launches / args.steps, "avg_launch_ms": dom_ms / dom_launches if dom_launches else None,
+                     "flop_per_launch": flop_per_launch},
+        "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,118 @@
+// Shared host/device helpers of libmi355tensor (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "mi355_tensor.h"
+
+namespace mt {
+
+// ---- host side: stream, error latch -------------------------------------------------------
+hipStream_t stream();
+int fail(int code, const char *fmt, ...);  // records the message, returns `code`
+int hip_fail(hipError_t e, const char *what);
+int set_conv_path(int v);  // 0 auto, 1 direct kernels, 2 matrix cores wherever they apply
+
+// Brackets the launches made inside its lifetime with two events on the work stream when profiling is enabled
+// (mt_profile_enable); `label` must be a string literal.
+struct ProfileScope {
+  explicit ProfileScope(const char *label);
+  ~ProfileScope();
+  int slot;
+};
+bool profiling();
+const char *intern_label(const char *name, const char *suffix);  // "name[suffix]" with process lifetime
+
+#define MT_HIP(call)                                         \
+  do {                                                       \
+    hipError_t e_ = (call);                                  \
+    if (e_ != hipSuccess) return mt::hip_fail(e_, #call);    \
+  } while (0)
+
+// after a kernel launch
+#define MT_LAUNCH_CHECK(name)                                \
+  do {                                                       \
+    hipError_t e_ = hipGetLastError();                       \
+    if (e_ != hipSuccess) return mt::hip_fail(e_, name);     \
+  } while (0)
+
+inline bool same_zyx(const mt_tensor *a, const mt_tensor *b) { return a->x == b->x && a->y == b->y && a->z == b->z; }
+inline size_t count(const mt_tensor *t) { return (size_t)t->w * t->z * t->y * t->x; }
+inline bool bad(const mt_tensor *t) { return t == nullptr || (t->p == nullptr && count(t) != 0); }
+inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+// ---- device side ---------------------------------------------------------------------------
+// The reference's scalar functions (cpu/ctensorapplyfunc.h:111-255) with the same float/double
+// promotions, so that results differ from the CPU path only by the libm implementation.
+__device__ __forceinline__ float f_sigmoid(float v) {
+  if (v > 30.f) v = 29.99999f;
+  if (v < -30.f) v = -29.99999f;
+  return (float)(1.0 / (1.0 + (double)expf(-v)));
+}
+__device__ __forceinline__ float f_tangence(float v) {
+  if (v > 30.f) v = 29.99999f;
+  if (v < -30.f) v = -29.99999f;
+  return tanhf(v);
+}
+__device__ __forceinline__ float f_gelu_inner(float v) {
+  const float pi = 3.141592654f;
+  double dv = v;
+  return (float)((double)sqrtf(2.f / pi) * (dv + 0.044715 * dv * dv * dv));
+}
+__device__ __forceinline__ float f_gelu(float v) {
+  float ft = tanhf(f_gelu_inner(v));
+  return (float)(0.5 * (double)v * (double)(1.f + ft));
+}
+__device__ __forceinline__ float f_dgelu(float v) {
+  const float pi = 3.141592654f;
+  double dv = v;
+  float ft = f_gelu_inner(v);
+  float fa = (float)((double)sqrtf(2.f / pi) * (1.0 + 3 * 0.044715 * dv * dv));
+  float sech = 1.f / coshf(ft);
+  return (float)(0.5 * ((double)(1.f + tanhf(ft)) + 0.5 * dv * (double)sech * (double)sech) * (double)fa);
+}
+
+__device__ __forceinline__ float apply_func(int func, float v) {
+  switch (func) {
+    case MT_F_SIGMOID: return f_sigmoid(v);
+    case MT_F_RELU: return v > 0.f ? v : 0.f;
+    case MT_F_GELU: return f_gelu(v);
+    case MT_F_LEAKY_RELU: return v > 0.f ? v : (float)(0.1 * (double)v);
+    case MT_F_LINEAR: return v;
+    case MT_F_TANGENCE: return f_tangence(v);
+    case MT_F_DIFFERENTIAL + MT_F_SIGMOID: { float s = f_sigmoid(v); return (float)((1.0 - (double)s) * (double)s); }
+    case MT_F_DIFFERENTIAL + MT_F_RELU: return v >= 0.f ? 1.f : 0.f;
+    case MT_F_DIFFERENTIAL + MT_F_GELU: return f_dgelu(v);
+    case MT_F_DIFFERENTIAL + MT_F_LEAKY_RELU: return v >= 0.f ? 1.f : 0.1f;
+    case MT_F_DIFFERENTIAL + MT_F_LINEAR: return 1.f;
+    case MT_F_DIFFERENTIAL + MT_F_TANGENCE: { float t = f_tangence(v); return 1.f - t * t; }
+    default: return v;  // MT_F_NONE
+  }
+}
+
+// For matrix-core epilogues, where the store loop is unrolled 64 times: the cheap functions stay inline, the
+// transcendental ones are one shared out-of-line body (func is uniform, so the branch costs nothing).
+__device__ __attribute__((noinline)) inline float apply_func_outlined(int func, float v) { return apply_func(func, v); }
+__device__ __forceinline__ float apply_func_epilogue(int func, float v) {
+  if (func == MT_F_NONE || func == MT_F_LINEAR) return v;
+  if (func == MT_F_RELU) return v > 0.f ? v : 0.f;
+  if (func == MT_F_LEAKY_RELU) return v > 0.f ? v : (float)(0.1 * (double)v);
+  return apply_func_outlined(func, v);
+}
+
+inline bool valid_func(int func, bool allow_none) {
+  if (func == MT_F_NONE) return allow_none;
+  int base = func & ~MT_F_DIFFERENTIAL;
+  return func >= 0 && func < 16 && base >= MT_F_SIGMOID && base <= MT_F_TANGENCE;
+}
+
+// 64-lane wavefront sum
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+}  // namespace mt

@@ -1,0 +1,396 @@
+// CTensorConv on gfx950: forward convolution, transposed convolution (also the input delta of a convolution)
+// and the per-sample weight / bias gradient.
+//
+// Fast path: implicit GEMM on the fp32 matrix cores (mt_igemm.h).
+//   forward      C[k][(b,oy,ox)]   = sum_{c,ky,kx} kernel[k][(c,ky,kx)] * image[b][c][oy*s-p+ky][ox*s-p+kx]
+//   transposed   the output is split into its sy*sx stride phases.  All pixels of one phase use the same subset of
+//                kernel taps, so each phase is a dense stride-1 convolution of the (un-dilated) delta with a packed
+//                sub-kernel: only non-zero taps are multiplied, 1/(sy*sx) of the dense-over-zeros product.
+//   gradient     per sample, dK[f][(c,i,j)] += sum_{oy,ox} delta[f][(oy,ox)] * image[c][oy*s-p+i][ox*s-p+j]
+// Slow path ("direct"): one thread per output element, same loop and summation order as the CPU path, used
+// for shapes the fast path does not cover (kernels that differ per sample, strides above 4) and as a
+// bit-for-bit cross-check of the fast path in the tests.
+#include "mt_igemm.h"
+
+namespace {
+
+using namespace mt::igemm;
+using mt::cdiv;
+
+int g_conv_path = 0;  // 0 auto, 1 direct, 2 implicit GEMM wherever it applies
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+// ---- library-owned workspace: packed phase kernels and bias sums of the transposed convolution ----------------
+float *g_ws = nullptr;
+size_t g_ws_floats = 0;
+int workspace(size_t floats, float **p) {
+  if (floats > g_ws_floats) {
+    if (g_ws) { MT_HIP(hipStreamSynchronize(mt::stream())); MT_HIP(hipFree(g_ws)); g_ws = nullptr; g_ws_floats = 0; }
+    size_t want = floats + floats / 4 + 1024;
+    MT_HIP(hipMalloc((void **)&g_ws, want * sizeof(float)));
+    g_ws_floats = want;
+  }
+  *p = g_ws;
+  return MT_OK;
+}
+
+struct ConvGeo {
+  uint32_t out_w, in_w, ker_w, bias_w;
+  int32_t C, H, W;      // input depth and size (image of a forward conv, delta of a transposed one)
+  int32_t KA;           // kernel_amount
+  int32_t KY, KX, SY, SX, PY, PX;
+  int32_t OH, OW, OZ;   // output size and depth
+  uint32_t ker_ld, ker_rows;
+};
+
+// ---- direct kernels: CPU loop order, no contraction, so results equal the CPU path bit for bit ------------------
+__global__ __launch_bounds__(256) void fwd_direct_kernel(float *out, const float *image, const float *kernel, const float *bias, ConvGeo g, size_t total) {
+  size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  int32_t x = idx % g.OW, y = (idx / g.OW) % g.OH, k = (idx / ((size_t)g.OW * g.OH)) % g.OZ;
+  uint32_t w = idx / ((size_t)g.OW * g.OH * g.OZ);
+  const float *img = image + (size_t)(w % g.in_w) * g.C * g.H * g.W;
+  const float *ker = kernel + ((size_t)(w % g.ker_w) * g.ker_rows + k) * g.ker_ld;
+  float acc = bias[(size_t)(w % g.bias_w) * g.KA + k];
+  int32_t taps = g.KX * g.KY;
+  for (int32_t ky = 0; ky < g.KY; ky++) {
+    int32_t iy = g.SY * y + ky - g.PY;
+    if (iy < 0 || iy >= g.H) continue;
+    for (int32_t kx = 0; kx < g.KX; kx++) {
+      int32_t ix = g.SX * x + kx - g.PX;
+      if (ix < 0 || ix >= g.W) continue;
+      for (int32_t c = 0; c < g.C; c++) acc += ker[c * taps + ky * g.KX + kx] * img[((size_t)c * g.H + iy) * g.W + ix];
+    }
+  }
+  out[idx] = acc;
+}
+
+__global__ __launch_bounds__(256) void tconv_direct_kernel(float *out, const float *delta, const float *kernel, const float *bias, ConvGeo g, size_t total, int func) {
+  size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  int32_t x = idx % g.OW, y = (idx / g.OW) % g.OH, z = (idx / ((size_t)g.OW * g.OH)) % g.OZ;
+  uint32_t w = idx / ((size_t)g.OW * g.OH * g.OZ);
+  const float *dl = delta + (size_t)(w % g.in_w) * g.C * g.H * g.W;
+  const float *ker = kernel + (size_t)(w % g.ker_w) * g.ker_rows * g.ker_ld;
+  const float *bs = bias + (size_t)(w % g.bias_w) * g.KA;
+  int32_t pad_y = g.KY - 1 - g.PY, pad_x = g.KX - 1 - g.PX, taps = g.KX * g.KY;
+  float acc = 0.f;
+  for (int32_t ky = 0; ky < g.KY; ky++) {
+    int32_t py = y + ky - pad_y;
+    if (py % g.SY != 0) continue;
+    int32_t dy = py / g.SY;
+    if (dy < 0 || dy >= g.H) continue;
+    for (int32_t kx = 0; kx < g.KX; kx++) {
+      int32_t px = x + kx - pad_x;
+      if (px % g.SX != 0) continue;
+      int32_t dx = px / g.SX;
+      if (dx < 0 || dx >= g.W) continue;
+      int32_t col = z * taps + (g.KY - 1 - ky) * g.KX + (g.KX - 1 - kx);
+      for (int32_t f = 0; f < g.KA; f++) {
+        acc += bs[f];
+        acc += ker[(size_t)f * g.ker_ld + col] * dl[((size_t)f * g.H + dy) * g.W + dx];
+      }
+    }
+  }
+  out[idx] = mt::apply_func(func, acc);
+}
+
+// one thread per gradient coefficient (w, f, c, i, j); pixels are visited in the CPU order
+__global__ __launch_bounds__(256) void wgrad_direct_kernel(float *dk, const float *image, const float *delta, ConvGeo g, uint32_t delta_w, int32_t DH, int32_t DW, size_t total) {
+  size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  int32_t taps = g.KX * g.KY, ncol = g.C * taps;
+  int32_t col = idx % ncol, f = (idx / ncol) % g.KA;
+  uint32_t w = idx / ((size_t)ncol * g.KA);
+  int32_t c = col / taps, i = (col % taps) / g.KX, j = col % g.KX;
+  const float *img = image + ((size_t)(w % g.in_w) * g.C + c) * g.H * g.W;
+  const float *dl = delta + ((size_t)(w % delta_w) * g.KA + f) * DH * DW;
+  float *dst = dk + ((size_t)w * g.ker_rows + f) * g.ker_ld + col;
+  float acc = *dst;
+  for (int32_t oy = 0; oy < DH; oy++) {
+    int32_t iy = i + oy * g.SY - g.PY;
+    if (iy < 0 || iy >= g.H) continue;
+    for (int32_t ox = 0; ox < DW; ox++) {
+      int32_t ix = j + ox * g.SX - g.PX;
+      if (ix < 0 || ix >= g.W) continue;
+      acc += dl[oy * DW + ox] * img[(size_t)iy * g.W + ix];
+    }
+  }
+  *dst = acc;
+}
+
+// bias gradient, CPU order: for each stored row (wb, f), samples w = wb, wb + Wb, ... then pixels in order
+__global__ __launch_bounds__(256) void dbias_serial_kernel(float *dbias, uint32_t dbias_w, const float *delta, uint32_t delta_w, uint32_t KA, uint32_t DHW, uint32_t W) {
+  uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= dbias_w * KA) return;
+  uint32_t wb = idx / KA, f = idx % KA;
+  float b = dbias[idx];
+  for (uint32_t w = wb; w < W; w += dbias_w) {
+    const float *dl = delta + ((size_t)(w % delta_w) * KA + f) * DHW;
+    for (uint32_t i = 0; i < DHW; i++) b += dl[i];
+  }
+  dbias[idx] = b;
+}
+
+// bias gradient when every sample owns its row of dbias: one wavefront per (w, f)
+__global__ __launch_bounds__(256) void dbias_wave_kernel(float *dbias, const float *delta, uint32_t delta_w, uint32_t KA, uint32_t DHW, uint32_t rows) {
+  uint32_t row = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x % 64;
+  if (row >= rows) return;
+  uint32_t w = row / KA, f = row % KA;
+  const float *dl = delta + ((size_t)(w % delta_w) * KA + f) * DHW;
+  float s = 0.f;
+  for (uint32_t i = lane; i < DHW; i += 64) s += dl[i];
+  s = mt::wave_sum(s);
+  if (lane == 0) dbias[row] += s;
+}
+
+// ---- transposed convolution: phase geometry, kernel packing, bias sums ----------------------------------------
+struct Phase1D {
+  int32_t k0, taps, off, q;  // first tap, tap count, input offset, number of output rows/columns in the phase
+};
+// outputs y = q*s + ph (q = 0..); taps ky = k0 + t*s; the input row of (q, t) is q + t + off
+Phase1D phase_1d(int32_t ph, int32_t K, int32_t s, int32_t p, int32_t O) {
+  int32_t pad = K - 1 - p;
+  Phase1D r;
+  r.k0 = ((pad - ph) % s + s) % s;
+  r.taps = r.k0 < K ? (K - r.k0 + s - 1) / s : 0;
+  r.off = (ph + r.k0 - pad) / s;  // exact: ph + k0 - pad is a multiple of s
+  r.q = O > ph ? (O - ph + s - 1) / s : 0;
+  return r;
+}
+
+// packed[co][(ci, ty, tx)] = kernel[ci][co*KY*KX + (KY-1-(ky0+ty*sy))*KX + (KX-1-(kx0+tx*sx))]
+__global__ __launch_bounds__(256) void pack_phase_kernel(float *packed, const float *kernel, uint32_t ker_ld, int32_t CO, int32_t CI, int32_t KY, int32_t KX,
+                                                         int32_t SY, int32_t SX, int32_t ky0, int32_t kx0, int32_t TY, int32_t TX) {
+  uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+  uint32_t kp = CI * TY * TX;
+  if (idx >= (uint32_t)CO * kp) return;
+  uint32_t co = idx / kp, k = idx % kp, ci = k / (TY * TX), t = k % (TY * TX), ty = t / TX, tx = t % TX;
+  int32_t ky = ky0 + ty * SY, kx = kx0 + tx * SX;
+  packed[idx] = kernel[(size_t)ci * ker_ld + co * KY * KX + (KY - 1 - ky) * KX + (KX - 1 - kx)];
+}
+
+__global__ __launch_bounds__(64) void bias_sum_kernel(float *sums, const float *bias, uint32_t KA) {
+  const float *b = bias + (size_t)blockIdx.x * KA;
+  float s = 0.f;
+  for (uint32_t i = threadIdx.x; i < KA; i += 64) s += b[i];
+  s = mt::wave_sum(s);
+  if (threadIdx.x == 0) sums[blockIdx.x] = s;
+}
+
+// ---- argument checks shared by the plain and the fused entry points ---------------------------------------------
+int check_forward(const char *name, const mt_tensor *out, const mt_tensor *image, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz,
+                  uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py) {
+  if (mt::bad(out) || mt::bad(image) || mt::bad(kernel) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel is required", name);
+  if (ka != bias->z) return mt::fail(MT_E_BIAS_COUNT, "%s: kernel_amount %u but %u biases", name, ka, bias->z);
+  if (kx <= 0 || ky <= 0 || sx <= 0 || sy <= 0 || px < 0 || py < 0) return mt::fail(MT_E_ARGUMENT, "%s: kernel and stride must be positive, padding non-negative", name);
+  int32_t ox = ((int32_t)image->x - kx + 2 * px) / sx + 1, oy = ((int32_t)image->y - ky + 2 * py) / sy + 1;
+  if ((int32_t)out->x != ox || (int32_t)out->y != oy || out->z != ka) return mt::fail(MT_E_OUTPUT_SHAPE, "%s: output must be [W,%u,%d,%d]", name, ka, oy, ox);
+  if ((int32_t)image->z != kz) return mt::fail(MT_E_DEPTH, "%s: image depth %u but kernel depth %d", name, image->z, kz);
+  return MT_OK;
+}
+
+int check_kernel_tensor(const char *name, const mt_tensor *kernel, uint32_t rows, uint32_t cols) {
+  if (kernel->w == 0 || kernel->z == 0 || kernel->y < rows || kernel->x < cols)
+    return mt::fail(MT_E_ARGUMENT, "%s: kernel tensor [%u,%u,%u,%u] is smaller than [1,1,%u,%u]", name, kernel->w, kernel->z, kernel->y, kernel->x, rows, cols);
+  return MT_OK;
+}
+
+int forward(const char *name, const mt_tensor *out, const mt_tensor *image, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
+            const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
+  int rc = check_forward(name, out, image, kernel, kx, ky, kz, ka, bias, sx, sy, px, py);
+  if (rc) return rc;
+  if (mt::count(out) == 0) return MT_OK;
+  if (image->w == 0 || bias->w == 0) return mt::fail(MT_E_ARGUMENT, "%s: empty operand", name);
+  uint32_t K = (uint32_t)kz * kx * ky;
+  if ((rc = check_kernel_tensor(name, kernel, ka, K))) return rc;
+  ConvGeo g{out->w, image->w, kernel->w, bias->w, kz, (int32_t)image->y, (int32_t)image->x, (int32_t)ka, ky, kx, sy, sx, py, px,
+            (int32_t)out->y, (int32_t)out->x, (int32_t)ka, kernel->x, kernel->z * kernel->y};
+  bool direct = g_conv_path == 1;
+  if (direct) {
+    size_t total = mt::count(out);
+    mt::ProfileScope prof("fwd_direct");
+    fwd_direct_kernel<<<cdiv(total, 256), 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, total);
+    MT_LAUNCH_CHECK(name);
+    if (func != MT_F_NONE) return mt_apply_func(out, out, func);
+    return MT_OK;
+  }
+  uint32_t OHW = out->y * out->x;
+  SrcRowK a{};
+  a.p = kernel->p; a.ld = kernel->x; a.R = ka; a.K = K; a.vec = (kernel->x % 4 == 0) && aligned16(kernel->p);
+  SrcIm2col b{};
+  b.p = image->p; b.in_w = image->w; b.C = kz; b.H = image->y; b.W = image->x; b.KY = ky; b.KX = kx; b.OHW = OHW; b.OW = out->x; b.K = K;
+  b.sy = sy; b.sx = sx; b.py = py; b.px = px;
+  Epilogue ep{};
+  ep.C = out->p; ep.row_stride = OHW; ep.inner = OHW; ep.g_stride = (size_t)ka * OHW;
+  ep.bias = bias->p; ep.bias_mode = 1; ep.bias_w = bias->w; ep.bias_stride = ka; ep.func = func;
+  if (kernel->w == 1) {  // one kernel set for the whole batch: fold the batch into the columns
+    b.R = out->w * OHW;
+    return launch(name, a, b, ep, ka, out->w * OHW, K, 1);
+  }
+  // kernels differ per sample: one product per output image
+  a.bt.wmod = kernel->w; a.bt.stride = (size_t)kernel->z * kernel->y * kernel->x;
+  b.bt.wmod = image->w; b.bt.stride = (size_t)kz * image->y * image->x; b.in_w = 1; b.R = OHW;
+  ep.bt.wmod = out->w; ep.bt.stride = (size_t)ka * OHW;
+  return launch(name, a, b, ep, ka, OHW, K, out->w);
+}
+
+int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
+             const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
+  if (mt::bad(out) || mt::bad(delta) || mt::bad(kernel) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel is required", name);
+  if (ka != bias->z) return mt::fail(MT_E_BIAS_COUNT, "%s: kernel_amount %u but %u biases", name, ka, bias->z);
+  if (kx <= 0 || ky <= 0 || kz <= 0 || sx <= 0 || sy <= 0) return mt::fail(MT_E_ARGUMENT, "%s: kernel and stride must be positive", name);
+  if (out->z != (uint32_t)kz) return mt::fail(MT_E_OUTPUT_SHAPE, "%s: output depth %u but kernel depth %d", name, out->z, kz);
+  if (delta->z != ka) return mt::fail(MT_E_DEPTH, "%s: delta depth %u but kernel_amount %u", name, delta->z, ka);
+  if (mt::count(out) == 0) return MT_OK;
+  if (delta->w == 0 || bias->w == 0) return mt::fail(MT_E_ARGUMENT, "%s: empty operand", name);
+  int rc = check_kernel_tensor(name, kernel, ka, (uint32_t)kz * kx * ky);
+  if (rc) return rc;
+  ConvGeo g{out->w, delta->w, kernel->w, bias->w, (int32_t)ka, (int32_t)delta->y, (int32_t)delta->x, (int32_t)ka, ky, kx, sy, sx, py, px,
+            (int32_t)out->y, (int32_t)out->x, kz, kernel->x, kernel->z * kernel->y};
+  bool direct = g_conv_path == 1 || kernel->w != 1 || sx > 4 || sy > 4 || delta->y == 0 || delta->x == 0;
+  if (direct) {
+    size_t total = mt::count(out);
+    mt::ProfileScope prof("tconv_direct");
+    tconv_direct_kernel<<<cdiv(total, 256), 256, 0, mt::stream()>>>(out->p, delta->p, kernel->p, bias->p, g, total, func);
+    MT_LAUNCH_CHECK(name);
+    return MT_OK;
+  }
+
+  // workspace: [bias sums (bias_w, padded to 64)] [packed kernels of all phases: kz*ka*ky*kx floats]
+  size_t sums = (bias->w + 63u) & ~(size_t)63u;
+  float *ws = nullptr;
+  if ((rc = workspace(sums + (size_t)kz * ka * ky * kx + 64, &ws))) return rc;
+  {
+    mt::ProfileScope prof("tconv_bias_sum");
+    bias_sum_kernel<<<bias->w, 64, 0, mt::stream()>>>(ws, bias->p, ka);
+  }
+  MT_LAUNCH_CHECK("bias_sum");
+  float *packed = ws + sums;
+  const uint32_t OHW = out->y * out->x;
+  for (int32_t phy = 0; phy < sy; phy++) {
+    Phase1D Y = phase_1d(phy, ky, sy, py, out->y);
+    if (Y.q == 0) continue;
+    for (int32_t phx = 0; phx < sx; phx++) {
+      Phase1D X = phase_1d(phx, kx, sx, px, out->x);
+      if (X.q == 0) continue;
+      uint32_t kp = ka * Y.taps * X.taps;
+      if (kp) {
+        mt::ProfileScope prof("tconv_pack_phase");
+        pack_phase_kernel<<<cdiv((size_t)kz * kp, 256), 256, 0, mt::stream()>>>(packed, kernel->p, kernel->x, kz, ka, ky, kx, sy, sx, Y.k0, X.k0, Y.taps, X.taps);
+        MT_LAUNCH_CHECK("pack_phase");
+      }
+      SrcRowK a{};
+      a.p = packed; a.ld = kp; a.R = kz; a.K = kp; a.vec = (kp % 4 == 0) && aligned16(packed);
+      SrcIm2col b{};
+      uint32_t QHW = (uint32_t)Y.q * X.q;
+      b.p = delta->p; b.in_w = delta->w; b.C = ka; b.H = delta->y; b.W = delta->x; b.KY = Y.taps ? Y.taps : 1; b.KX = X.taps ? X.taps : 1;
+      b.OHW = QHW; b.OW = X.q; b.R = out->w * QHW; b.K = kp; b.sy = 1; b.sx = 1; b.py = -Y.off; b.px = -X.off;
+      Epilogue ep{};
+      ep.C = out->p; ep.row_stride = OHW; ep.inner = QHW; ep.g_stride = (size_t)kz * OHW;
+      ep.qw = X.q; ep.sy = sy; ep.sx = sx; ep.py = phy; ep.px = phx; ep.OW = out->x;
+      ep.tap_bias = ws; ep.bias_w = bias->w; ep.ty_cnt = Y.taps; ep.tx_cnt = X.taps; ep.offy = Y.off; ep.offx = X.off; ep.IH = delta->y; ep.IW = delta->x;
+      ep.func = func;
+      if ((rc = launch(name, a, b, ep, kz, out->w * QHW, kp, 1))) return rc;
+      packed += ((size_t)kz * kp + 3) & ~(size_t)3;  // keep every phase 16-byte aligned
+    }
+  }
+  return MT_OK;
+}
+
+int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
+          const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py, bool bias_too) {
+  if (mt::bad(dk) || mt::bad(db) || mt::bad(image) || mt::bad(delta)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel gradient is required", name);
+  if (db->z != ka) return mt::fail(MT_E_BIAS_COUNT, "%s: kernel_amount %u but %u bias gradients", name, ka, db->z);
+  if (kx <= 0 || ky <= 0 || kz <= 0 || sx <= 0 || sy <= 0) return mt::fail(MT_E_ARGUMENT, "%s: kernel and stride must be positive", name);
+  if ((uint32_t)kz != image->z) return mt::fail(MT_E_SHAPE, "%s: kernel depth %d but image depth %u", name, kz, image->z);
+  if (delta->z != ka) return mt::fail(MT_E_DEPTH, "%s: delta depth %u but kernel_amount %u", name, delta->z, ka);
+  if (dk->w == 0) return MT_OK;
+  if (image->w == 0 || delta->w == 0 || db->w == 0) return mt::fail(MT_E_ARGUMENT, "%s: empty operand", name);
+  uint32_t ncol = (uint32_t)kz * kx * ky, DHW = delta->y * delta->x;
+  int rc = check_kernel_tensor(name, dk, ka, ncol);
+  if (rc) return rc;
+  if (DHW == 0) return MT_OK;
+  ConvGeo g{dk->w, image->w, dk->w, db->w, kz, (int32_t)image->y, (int32_t)image->x, (int32_t)ka, ky, kx, sy, sx, py, px, 0, 0, 0, dk->x, dk->z * dk->y};
+  bool direct = g_conv_path == 1 || dk->w > 65535u;
+  if (direct) {
+    size_t total = (size_t)dk->w * ka * ncol;
+    wgrad_direct_kernel<<<cdiv(total, 256), 256, 0, mt::stream()>>>(dk->p, image->p, delta->p, g, delta->w, delta->y, delta->x, total);
+    MT_LAUNCH_CHECK(name);
+  } else {
+    SrcRowK a{};
+    a.p = delta->p; a.ld = DHW; a.R = ka; a.K = DHW; a.vec = (DHW % 4 == 0) && aligned16(delta->p);
+    a.bt.wmod = delta->w; a.bt.stride = (size_t)ka * DHW;
+    SrcWgradImage b{};
+    b.p = image->p; b.H = image->y; b.W = image->x; b.KY = ky; b.KX = kx; b.OW = delta->x; b.R = ncol; b.K = DHW; b.sy = sy; b.sx = sx; b.py = py; b.px = px;
+    b.bt.wmod = image->w; b.bt.stride = (size_t)kz * image->y * image->x;
+    Epilogue ep{};
+    ep.C = dk->p; ep.row_stride = dk->x; ep.inner = ncol; ep.g_stride = 0; ep.accumulate = true;
+    ep.bt.wmod = dk->w; ep.bt.stride = (size_t)dk->z * dk->y * dk->x;
+    if ((rc = launch(name, a, b, ep, ka, ncol, DHW, dk->w))) return rc;
+  }
+  if (!bias_too) return MT_OK;
+  if (db->y != 1 || db->x != 1) return mt::fail(MT_E_ARGUMENT, "%s: bias gradient must be [W,Z,1,1]", name);
+  if (db->w >= dk->w && g_conv_path != 1) {
+    uint32_t rows = dk->w * ka;
+    dbias_wave_kernel<<<cdiv(rows, 4), 256, 0, mt::stream()>>>(db->p, delta->p, delta->w, ka, DHW, rows);
+  } else {
+    uint32_t wb = db->w < dk->w ? db->w : dk->w;
+    dbias_serial_kernel<<<cdiv((size_t)wb * ka, 256), 256, 0, mt::stream()>>>(db->p, wb, delta->p, delta->w, ka, DHW, dk->w);
+  }
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
+}  // namespace
+
+namespace mt {
+int set_conv_path(int v) {
+  if (v < 0 || v > 2) return fail(MT_E_ARGUMENT, "conv_path must be 0 (auto), 1 (direct) or 2 (matrix cores)");
+  g_conv_path = v;
+  return MT_OK;
+}
+}  // namespace mt
+
+extern "C" {
+
+int mt_forward_convolution(const mt_tensor *out, const mt_tensor *image, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
+                           const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py) {
+  return forward("mt_forward_convolution", out, image, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, MT_F_NONE);
+}
+
+int mt_forward_convolution_func(const mt_tensor *out, const mt_tensor *image, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
+                                const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
+  if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_forward_convolution_func: unknown function id %d", func);
+  return forward("mt_forward_convolution_func", out, image, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);
+}
+
+int mt_backward_convolution(const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
+                            const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py) {
+  return backward("mt_backward_convolution", out, delta, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, MT_F_NONE);
+}
+
+int mt_backward_convolution_func(const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
+                                 const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
+  if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_backward_convolution_func: unknown function id %d", func);
+  return backward("mt_backward_convolution_func", out, delta, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);
+}
+
+int mt_create_delta_weight_and_bias(const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
+                                    const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py) {
+  return wgrad("mt_create_delta_weight_and_bias", dk, kx, ky, kz, ka, db, image, delta, sx, sy, px, py, true);
+}
+
+// the transposed layer: image and delta trade places, and the bias gradient is cleared (cpu/ctensorconv.h:393-397)
+int mt_create_back_delta_weight_and_bias(const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
+                                         const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py) {
+  int rc = wgrad("mt_create_back_delta_weight_and_bias", dk, kx, ky, kz, ka, db, delta, image, sx, sy, px, py, false);
+  if (rc) return rc;
+  return mt_fill(db, 0.f);
+}
+
+}  // extern "C"

@@ -1,0 +1,580 @@
+// HBM-bound part of the tensor-op path for gfx950: elementwise ops, reductions over the batch axis
+// and over Y*X, resampling, pooling, Adam and the activation functions.
+//
+// Layout rule shared by every kernel here: the output is walked as [W][S] with S = Z*Y*X;
+// blockIdx.y is the output layer w, so a broadcast operand (w % W_operand) costs no per-element
+// division, and threads along blockIdx.x/threadIdx.x touch consecutive addresses (coalesced,
+// 16-byte vectors when S and the pointers allow it).
+#include "mt_common.h"
+
+namespace {
+
+using mt::cdiv;
+
+constexpr int EW_THREADS = 256;
+
+struct Operand {
+  const float *p;
+  uint32_t w;  // layers; layer used for output layer w is w % this
+};
+
+__device__ __forceinline__ const float *layer(const Operand &o, uint32_t w, size_t S) {
+  return o.p + (size_t)(o.w == 1 ? 0u : w % o.w) * S;
+}
+
+// out[w][i] = f(a[w%Wa][i])
+template <class F>
+__global__ __launch_bounds__(EW_THREADS) void ew1_kernel(float *out, Operand a, uint32_t S, uint32_t W, bool vec, F f) {
+  for (uint32_t w = blockIdx.y; w < W; w += gridDim.y) {
+    const float *pa = layer(a, w, S);
+    float *po = out + (size_t)w * S;
+    uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+    if (vec) {
+      if (i * 4 < S) {
+        float4 v = reinterpret_cast<const float4 *>(pa)[i];
+        v.x = f(v.x); v.y = f(v.y); v.z = f(v.z); v.w = f(v.w);
+        reinterpret_cast<float4 *>(po)[i] = v;
+      }
+    } else if (i < S) {
+      po[i] = f(pa[i]);
+    }
+  }
+}
+
+// out[w][i] = f(a[w%Wa][i], b[w%Wb][i])
+template <class F>
+__global__ __launch_bounds__(EW_THREADS) void ew2_kernel(float *out, Operand a, Operand b, uint32_t S, uint32_t W, bool vec, F f) {
+  for (uint32_t w = blockIdx.y; w < W; w += gridDim.y) {
+    const float *pa = layer(a, w, S), *pb = layer(b, w, S);
+    float *po = out + (size_t)w * S;
+    uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+    if (vec) {
+      if (i * 4 < S) {
+        float4 x = reinterpret_cast<const float4 *>(pa)[i], y = reinterpret_cast<const float4 *>(pb)[i], o;
+        o.x = f(x.x, y.x); o.y = f(x.y, y.y); o.z = f(x.z, y.z); o.w = f(x.w, y.w);
+        reinterpret_cast<float4 *>(po)[i] = o;
+      }
+    } else if (i < S) {
+      po[i] = f(pa[i], pb[i]);
+    }
+  }
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <class F>
+int launch1(const char *name, const mt_tensor *out, const mt_tensor *in, F f) {
+  if (mt::bad(out) || mt::bad(in)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (!mt::same_zyx(in, out)) return mt::fail(MT_E_SHAPE, "%s: Z/Y/X of input and output differ", name);
+  size_t S = (size_t)out->z * out->y * out->x;
+  if (S == 0 || out->w == 0) return MT_OK;
+  if (in->w == 0) return mt::fail(MT_E_ARGUMENT, "%s: empty input", name);
+  bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p);
+  dim3 grid(cdiv(vec ? S / 4 : S, EW_THREADS), out->w < 65535u ? out->w : 65535u);
+  mt::ProfileScope prof(name);
+  ew1_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, Operand{in->p, in->w}, (uint32_t)S, out->w, vec, f);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
+template <class F>
+int launch2(const char *name, const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, F f) {
+  if (mt::bad(out) || mt::bad(l) || mt::bad(r)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (!mt::same_zyx(l, r) || !mt::same_zyx(out, r)) return mt::fail(MT_E_SHAPE, "%s: Z/Y/X of the operands differ", name);
+  size_t S = (size_t)out->z * out->y * out->x;
+  if (S == 0 || out->w == 0) return MT_OK;
+  if (l->w == 0 || r->w == 0) return mt::fail(MT_E_ARGUMENT, "%s: empty operand", name);
+  bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(l->p) && aligned16(r->p);
+  dim3 grid(cdiv(vec ? S / 4 : S, EW_THREADS), out->w < 65535u ? out->w : 65535u);
+  mt::ProfileScope prof(name);
+  ew2_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, Operand{l->p, l->w}, Operand{r->p, r->w}, (uint32_t)S, out->w, vec, f);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
+// ---- functors: arithmetic exactly as the CPU path writes it (no fused multiply-add: see the build flags) ----
+struct FInv { __device__ float operator()(float i) const { return (float)(1.0 / (double)i); } };
+struct FPow2 { float s; __device__ float operator()(float i) const { return i * i * s; } };
+struct FSqrt { float s, add; __device__ float operator()(float i) const { return sqrtf(i + add) * s; } };
+struct FScale { float v; __device__ float operator()(float i) const { return i * v; } };
+struct FAffine { float s, add; __device__ float operator()(float i) const { return i * s + add; } };
+struct FClip { float lo, hi; __device__ float operator()(float v) const { if (v < lo) v = lo; if (v > hi) v = hi; return v; } };
+struct FSign { __device__ float operator()(float v) const { if (v < 0.f) v = -1.f; if (v > 0.f) v = 1.f; return v; } };
+struct FFunc { int func; __device__ float operator()(float v) const { return mt::apply_func(func, v); } };
+struct FAdd { float ls, rs; __device__ float operator()(float l, float r) const { return (ls * l) + (rs * r); } };
+struct FSub { float ls, rs; __device__ float operator()(float l, float r) const { return (ls * l) - (rs * r); } };
+struct FDiv { float ls, rs; __device__ float operator()(float l, float r) const { return (ls * l) / (rs * r); } };
+struct FMul { __device__ float operator()(float l, float r) const { return l * r; } };
+
+__global__ __launch_bounds__(EW_THREADS) void fill_kernel(float *out, size_t n, float v) {
+  size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * EW_THREADS;
+  for (; i < n; i += stride) out[i] = v;
+}
+
+// ---- AddSumW: out[0][r] = ls*sum_w L[w][r] + rs*sum_w R[w][r], out[w>0][r] = 0 --------------------------------
+// A block owns RB consecutive r and splits the batch axis over WS = 256/RB slices that are combined in LDS,
+// so short tensors (S of a few thousand) still fill the chip and every load is coalesced along r.
+template <int RB>
+__global__ __launch_bounds__(EW_THREADS) void add_sum_w_kernel(float *out, uint32_t Wout, const float *L, uint32_t Wl, const float *R,
+                                                               uint32_t Wr, uint32_t S, float ls, float rs) {
+  constexpr int WS = EW_THREADS / RB;
+  __shared__ float part[2][WS][RB];
+  int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
+  uint32_t r = blockIdx.x * RB + rl;
+  float sl = 0.f, sr = 0.f;
+  if (r < S) {
+    for (uint32_t w = ws; w < Wl; w += WS) sl += L[(size_t)w * S + r];
+    for (uint32_t w = ws; w < Wr; w += WS) sr += R[(size_t)w * S + r];
+  }
+  part[0][ws][rl] = sl;
+  part[1][ws][rl] = sr;
+  __syncthreads();
+  if (ws == 0 && r < S) {
+    sl = 0.f; sr = 0.f;
+#pragma unroll
+    for (int i = 0; i < WS; i++) { sl += part[0][i][rl]; sr += part[1][i][rl]; }
+    sl *= ls;
+    sr *= rs;
+    out[r] = sl + sr;
+  }
+  if (r < S)
+    for (uint32_t w = 1 + ws; w < Wout; w += WS) out[(size_t)w * S + r] = 0.f;
+}
+
+// ---- SummXY: one wavefront per (w,z) row of Y*X elements ---------------------------------------------------------
+__global__ __launch_bounds__(EW_THREADS) void summ_xy_kernel(float *out, const float *in, uint32_t Win, uint32_t Z, uint32_t YX, uint32_t rows) {
+  uint32_t row = blockIdx.x * (EW_THREADS / 64) + threadIdx.x / 64;
+  if (row >= rows) return;
+  uint32_t w = row / Z, z = row % Z, lane = threadIdx.x % 64;
+  const float *p = in + ((size_t)(w % Win) * Z + z) * YX;
+  float s = 0.f;
+  for (uint32_t i = lane; i < YX; i += 64) s += p[i];
+  s = mt::wave_sum(s);
+  if (lane == 0) out[row] = s;
+}
+
+// ---- AddBias: working[w][z][.] += bias[w%Wb][z] ------------------------------------------------------------------
+__global__ __launch_bounds__(EW_THREADS) void add_bias_kernel(float *t, const float *bias, uint32_t Wb, uint32_t Z, uint32_t YX, uint32_t rows) {
+  for (uint32_t row = blockIdx.y; row < rows; row += gridDim.y) {
+    uint32_t w = row / Z, z = row % Z;
+    float b = bias[(size_t)(w % Wb) * Z + z];
+    uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+    if (i < YX) t[(size_t)row * YX + i] += b;
+  }
+}
+
+// ---- Transponse ---------------------------------------------------------------------------------------------------
+__global__ void transponse_kernel(float *out, const float *in, uint32_t Y, uint32_t X) {
+  __shared__ float tile[32][33];
+  const float *pi = in + (size_t)blockIdx.z * Y * X;
+  float *po = out + (size_t)blockIdx.z * Y * X;
+  uint32_t x = blockIdx.x * 32 + threadIdx.x;
+  for (int j = threadIdx.y; j < 32; j += 8) {
+    uint32_t y = blockIdx.y * 32 + j;
+    if (x < X && y < Y) tile[j][threadIdx.x] = pi[(size_t)y * X + x];
+  }
+  __syncthreads();
+  uint32_t oy = blockIdx.y * 32 + threadIdx.x;  // becomes the fast index of the output
+  for (int j = threadIdx.y; j < 32; j += 8) {
+    uint32_t ox = blockIdx.x * 32 + j;
+    if (ox < X && oy < Y) po[(size_t)ox * Y + oy] = tile[threadIdx.x][j];
+  }
+}
+
+// ---- resampling and pooling: one thread per output element, x fastest ---------------------------------------------
+struct Geo {
+  uint32_t Win, Z, iy, ix, oy, ox;  // input layers, depth, input / output rows and columns
+};
+
+__global__ __launch_bounds__(EW_THREADS) void upsampling_kernel(float *out, const float *in, Geo g, uint32_t ux, uint32_t uy, uint32_t planes) {
+  uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, n = g.oy * g.ox;
+  if (i >= n) return;
+  uint32_t y = i / g.ox, x = i % g.ox, sy = y / uy, sx = x / ux;
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    uint32_t w = pl / g.Z, z = pl % g.Z;
+    float v = 0.f;
+    if (sx < g.ix && sy < g.iy) v = in[(((size_t)(w % g.Win) * g.Z + z) * g.iy + sy) * g.ix + sx];
+    out[(size_t)pl * n + i] = v;
+  }
+}
+
+__global__ __launch_bounds__(EW_THREADS) void downsampling_kernel(float *out, const float *in, Geo g, uint32_t dsx, uint32_t dsy, uint32_t planes) {
+  uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, n = g.oy * g.ox;
+  if (i >= n) return;
+  uint32_t y = i / g.ox, x = i % g.ox;
+  float div = (float)(dsx * dsy);
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const float *p = in + (size_t)pl * g.iy * g.ix;
+    float s = 0.f;
+    for (uint32_t dx = 0; dx < dsx; dx++) {  // dx outer, dy inner: the CPU path's summation order
+      uint32_t xp = x * dsx + dx;
+      if (xp >= g.ix) continue;
+      for (uint32_t dy = 0; dy < dsy; dy++) {
+        uint32_t yp = y * dsy + dy;
+        if (yp >= g.iy) continue;
+        s += p[(size_t)yp * g.ix + xp];
+      }
+    }
+    out[(size_t)pl * n + i] = s / div;
+  }
+}
+
+__global__ __launch_bounds__(EW_THREADS) void max_pooling_kernel(float *out, mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t px_, uint32_t py_, uint32_t planes) {
+  uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, n = g.oy * g.ox;
+  if (i >= n) return;
+  uint32_t y = i / g.ox, x = i % g.ox, ix = x * px_, iy = y * py_;
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    uint32_t w = pl / g.Z, z = pl % g.Z;
+    const float *p = in + (size_t)pl * g.iy * g.ix;
+    float best = p[(size_t)iy * g.ix + ix];
+    uint32_t bx = ix, by = iy;
+    for (uint32_t py = 0; py < py_; py++)
+      for (uint32_t px = 0; px < px_; px++) {
+        float e = p[(size_t)(iy + py) * g.ix + ix + px];
+        if (e > best) { best = e; bx = ix + px; by = iy + py; }  // first strict maximum, rows then columns
+      }
+    out[(size_t)pl * n + i] = best;
+    mt_spos s; s.X = bx; s.Y = by;
+    pos[((size_t)(w % Wpos) * g.Z + z) * n + i] = s;
+  }
+}
+
+// Gather form of the CPU path's scatter: output (y,x) takes the delta of its window when that window's stored
+// maximum is (x,y), else 0.  Equal to the scatter for positions that lie inside their own window, which is what
+// max_pooling writes.
+__global__ __launch_bounds__(EW_THREADS) void max_pooling_backward_kernel(float *out, const mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t px_, uint32_t py_, uint32_t planes) {
+  uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, n = g.oy * g.ox;
+  if (i >= n) return;
+  uint32_t y = i / g.ox, x = i % g.ox, sy = y / py_, sx = x / px_;
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    uint32_t w = pl / g.Z, z = pl % g.Z;
+    float v = 0.f;
+    if (sy < g.iy && sx < g.ix) {
+      size_t k = (size_t)sy * g.ix + sx;
+      mt_spos s = pos[((size_t)(w % Wpos) * g.Z + z) * g.iy * g.ix + k];
+      if (s.X == x && s.Y == y) v = in[(size_t)pl * g.iy * g.ix + k];
+    }
+    out[(size_t)pl * n + i] = v;
+  }
+}
+
+// ---- Adam: fp32 state, update arithmetic in double as on the CPU path ------------------------------------------------
+__global__ __launch_bounds__(EW_THREADS) void adam_kernel(float *weight, const float *dweight, float *m, float *v, size_t n, float batch,
+                                                          double speed, double beta1, double beta2, double epsilon, double c1, double c2) {
+  size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
+  if (i >= n) return;
+  float dw = dweight[i] / batch, mi = m[i], vi = v[i];
+  mi = (float)(beta1 * (double)mi + (1.0 - beta1) * (double)dw);
+  vi = (float)(beta2 * (double)vi + (1.0 - beta2) * (double)dw * (double)dw);
+  float mc = (float)((double)mi / c1);  // c1 = 1 - beta1^iteration
+  float vc = (float)((double)vi / c2);
+  dw = (float)(speed * (double)mc / ((double)sqrtf(vc) + epsilon));
+  m[i] = mi;
+  v[i] = vi;
+  weight[i] = weight[i] - dw;
+}
+
+// ---- batch normalisation over the batch axis, statistics per element (z,y,x) --------------------------------------
+// Pass 1: per column r, sums of d = x - x[0][r] and d*d over w (the shift keeps the one-pass variance stable),
+// the batch split over WS slices like add_sum_w.  Produces mean, biased variance and 1/sqrt(var+eps).
+template <int RB>
+__global__ __launch_bounds__(EW_THREADS) void bn_stats_kernel(const float *x, uint32_t W, uint32_t S, float inv_n, float eps, float *mean,
+                                                              float *var, float *ivar, float *new_mean, float *new_var, float mom_old, float mom_new) {
+  constexpr int WS = EW_THREADS / RB;
+  __shared__ float part[2][WS][RB];
+  int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
+  uint32_t r = blockIdx.x * RB + rl;
+  float s1 = 0.f, s2 = 0.f, shift = 0.f;
+  if (r < S) {
+    shift = x[r];
+    for (uint32_t w = ws; w < W; w += WS) {
+      float d = x[(size_t)w * S + r] - shift;
+      s1 += d;
+      s2 += d * d;
+    }
+  }
+  part[0][ws][rl] = s1;
+  part[1][ws][rl] = s2;
+  __syncthreads();
+  if (ws != 0 || r >= S) return;
+  s1 = 0.f; s2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < WS; i++) { s1 += part[0][i][rl]; s2 += part[1][i][rl]; }
+  float md = s1 * inv_n;                  // mean of the shifted data
+  float mu = shift + md;
+  float vr = (s2 - s1 * md) * inv_n;      // sum((d-md)^2)/N
+  if (vr < 0.f) vr = 0.f;
+  float iv = (float)(1.0 / (double)(sqrtf(vr + eps) * 1.f));
+  mean[r] = mu;
+  var[r] = vr;
+  ivar[r] = iv;
+  if (new_mean) new_mean[r] = (mom_old * new_mean[r]) + (mom_new * mu);
+  if (new_var) new_var[r] = (mom_old * new_var[r]) + (mom_new * vr);
+}
+
+// Pass 2: out = func(gamma * ((x - mean) * ivar) + beta), optionally storing xhat.
+__global__ __launch_bounds__(EW_THREADS) void bn_apply_kernel(float *out, float *xhat, const float *x, const float *mean, const float *ivar,
+                                                              const float *gamma, const float *beta, uint32_t S, uint32_t W, bool vec, int func) {
+  uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (vec) {
+    if (i * 4 >= S) return;
+    float4 mu = reinterpret_cast<const float4 *>(mean)[i], iv = reinterpret_cast<const float4 *>(ivar)[i];
+    float4 g = reinterpret_cast<const float4 *>(gamma)[i], b = reinterpret_cast<const float4 *>(beta)[i];
+    for (uint32_t w = blockIdx.y; w < W; w += gridDim.y) {
+      float4 v = reinterpret_cast<const float4 *>(x + (size_t)w * S)[i], h, o;
+      h.x = (v.x - mu.x) * iv.x; h.y = (v.y - mu.y) * iv.y; h.z = (v.z - mu.z) * iv.z; h.w = (v.w - mu.w) * iv.w;
+      o.x = mt::apply_func(func, (g.x * h.x) + b.x); o.y = mt::apply_func(func, (g.y * h.y) + b.y);
+      o.z = mt::apply_func(func, (g.z * h.z) + b.z); o.w = mt::apply_func(func, (g.w * h.w) + b.w);
+      if (xhat) reinterpret_cast<float4 *>(xhat + (size_t)w * S)[i] = h;
+      reinterpret_cast<float4 *>(out + (size_t)w * S)[i] = o;
+    }
+  } else {
+    if (i >= S) return;
+    float mu = mean[i], iv = ivar[i], g = gamma[i], b = beta[i];
+    for (uint32_t w = blockIdx.y; w < W; w += gridDim.y) {
+      float h = (x[(size_t)w * S + i] - mu) * iv;
+      if (xhat) xhat[(size_t)w * S + i] = h;
+      out[(size_t)w * S + i] = mt::apply_func(func, (g * h) + b);
+    }
+  }
+}
+
+__global__ __launch_bounds__(EW_THREADS) void bn_ivar_kernel(float *ivar, const float *var, uint32_t S, float eps) {
+  uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (i < S) ivar[i] = (float)(1.0 / (double)sqrtf(var[i] + eps));
+}
+
+}  // namespace
+
+// a small pool of scratch statistics for the fused batch-norm entry points when the caller passes NULL
+namespace {
+float *g_bn_scratch = nullptr;
+size_t g_bn_scratch_floats = 0;
+int bn_scratch(size_t floats, float **p) {
+  if (floats > g_bn_scratch_floats) {
+    if (g_bn_scratch) { MT_HIP(hipStreamSynchronize(mt::stream())); MT_HIP(hipFree(g_bn_scratch)); g_bn_scratch = nullptr; g_bn_scratch_floats = 0; }
+    MT_HIP(hipMalloc((void **)&g_bn_scratch, floats * sizeof(float)));
+    g_bn_scratch_floats = floats;
+  }
+  *p = g_bn_scratch;
+  return MT_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int mt_fill(const mt_tensor *out, float value) {
+  if (mt::bad(out)) return mt::fail(MT_E_ARGUMENT, "mt_fill: null tensor");
+  size_t n = mt::count(out);
+  if (n == 0) return MT_OK;
+  unsigned blocks = cdiv(n, EW_THREADS);
+  if (blocks > 65536u * 4) blocks = 65536u * 4;
+  fill_kernel<<<blocks, EW_THREADS, 0, mt::stream()>>>(out->p, n, value);
+  MT_LAUNCH_CHECK("mt_fill");
+  return MT_OK;
+}
+
+int mt_inv(const mt_tensor *out, const mt_tensor *in) { return launch1("mt_inv", out, in, FInv{}); }
+int mt_pow2(const mt_tensor *out, const mt_tensor *in, float scale) { return launch1("mt_pow2", out, in, FPow2{scale}); }
+int mt_sqrt(const mt_tensor *out, const mt_tensor *in, float scale, float add) { return launch1("mt_sqrt", out, in, FSqrt{scale, add}); }
+int mt_mul_value(const mt_tensor *out, const mt_tensor *in, float v) { return launch1("mt_mul_value", out, in, FScale{v}); }
+int mt_add_value(const mt_tensor *out, const mt_tensor *in, float s, float v) { return launch1("mt_add_value", out, in, FAffine{s, v}); }
+int mt_sub_value(const mt_tensor *out, const mt_tensor *in, float s, float v) { return launch1("mt_sub_value", out, in, FAffine{s, -v}); }
+int mt_set(const mt_tensor *out, const mt_tensor *in, float s, float add) { return launch1("mt_set", out, in, FAffine{s, add}); }
+int mt_clip(const mt_tensor *t, float lo, float hi) { return launch1("mt_clip", t, t, FClip{lo, hi}); }
+int mt_signum(const mt_tensor *t) { return launch1("mt_signum", t, t, FSign{}); }
+
+int mt_add(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, float ls, float rs) { return launch2("mt_add", out, l, r, FAdd{ls, rs}); }
+int mt_sub(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, float ls, float rs) { return launch2("mt_sub", out, l, r, FSub{ls, rs}); }
+int mt_div(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, float ls, float rs) { return launch2("mt_div", out, l, r, FDiv{ls, rs}); }
+int mt_tensor_item_production(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r) { return launch2("mt_tensor_item_production", out, l, r, FMul{}); }
+
+int mt_apply_func(const mt_tensor *out, const mt_tensor *in, int func) {
+  if (!mt::valid_func(func, false)) return mt::fail(MT_E_ARGUMENT, "mt_apply_func: unknown function id %d", func);
+  if (mt::bad(out) || mt::bad(in)) return mt::fail(MT_E_ARGUMENT, "mt_apply_func: null tensor");
+  if (!mt::same_zyx(in, out) || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_apply_func: sizes of input and output differ");
+  return launch1("mt_apply_func", out, in, FFunc{func});
+}
+
+int mt_add_sum_w(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, float ls, float rs) {
+  if (mt::bad(out) || mt::bad(l) || mt::bad(r)) return mt::fail(MT_E_ARGUMENT, "mt_add_sum_w: null tensor");
+  if (!mt::same_zyx(l, r) || !mt::same_zyx(out, r)) return mt::fail(MT_E_SHAPE, "mt_add_sum_w: Z/Y/X of the operands differ");
+  size_t S = (size_t)out->z * out->y * out->x;
+  if (S == 0 || out->w == 0) return MT_OK;
+  mt::ProfileScope prof("mt_add_sum_w");
+  // the output may alias an operand (dW = dW + sum_w TmpdW): every column is read completely before it is written
+  if (S >= 65536)
+    add_sum_w_kernel<256><<<cdiv(S, 256), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
+  else
+    add_sum_w_kernel<32><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
+  MT_LAUNCH_CHECK("mt_add_sum_w");
+  return MT_OK;
+}
+
+int mt_summ_xy(const mt_tensor *out, const mt_tensor *in) {
+  if (mt::bad(out) || mt::bad(in)) return mt::fail(MT_E_ARGUMENT, "mt_summ_xy: null tensor");
+  if (in->z != out->z) return mt::fail(MT_E_SHAPE, "mt_summ_xy: depth of input and output differ");
+  uint32_t rows = out->w * out->z;
+  if (rows == 0) return MT_OK;
+  if (out->y != 1 || out->x != 1) {  // the reference writes element (w,z,0,0) of a larger output; keep that addressing
+    return mt::fail(MT_E_ARGUMENT, "mt_summ_xy: output must be [W,Z,1,1]");
+  }
+  summ_xy_kernel<<<cdiv(rows, EW_THREADS / 64), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, in->w, in->z, in->y * in->x, rows);
+  MT_LAUNCH_CHECK("mt_summ_xy");
+  return MT_OK;
+}
+
+int mt_add_bias(const mt_tensor *t, const mt_tensor *bias) {
+  if (mt::bad(t) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "mt_add_bias: null tensor");
+  if (t->z != bias->z) return mt::fail(MT_E_SHAPE, "mt_add_bias: depth of tensor and bias differ");
+  uint32_t rows = t->w * t->z, YX = t->y * t->x;
+  if (rows == 0 || YX == 0) return MT_OK;
+  if (bias->y != 1 || bias->x != 1) return mt::fail(MT_E_ARGUMENT, "mt_add_bias: bias must be [W,Z,1,1]");
+  dim3 grid(cdiv(YX, EW_THREADS), rows < 65535u ? rows : 65535u);
+  add_bias_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(t->p, bias->p, bias->w, t->z, YX, rows);
+  MT_LAUNCH_CHECK("mt_add_bias");
+  return MT_OK;
+}
+
+int mt_transponse(const mt_tensor *out, const mt_tensor *in) {
+  if (mt::bad(out) || mt::bad(in)) return mt::fail(MT_E_ARGUMENT, "mt_transponse: null tensor");
+  if (out->y != in->x || out->x != in->y || out->z != in->z || out->w != in->w) return mt::fail(MT_E_SHAPE, "mt_transponse: sizes do not match");
+  if (mt::count(in) == 0) return MT_OK;
+  uint32_t planes = in->w * in->z;
+  if (planes > 65535u) return mt::fail(MT_E_ARGUMENT, "mt_transponse: more than 65535 matrices");
+  dim3 grid(cdiv(in->x, 32), cdiv(in->y, 32), planes);
+  transponse_kernel<<<grid, dim3(32, 8), 0, mt::stream()>>>(out->p, in->p, in->y, in->x);
+  MT_LAUNCH_CHECK("mt_transponse");
+  return MT_OK;
+}
+
+int mt_upsampling(const mt_tensor *out, const mt_tensor *in, uint32_t ux, uint32_t uy) {
+  if (mt::bad(out) || mt::bad(in) || ux == 0 || uy == 0) return mt::fail(MT_E_ARGUMENT, "mt_upsampling: bad argument");
+  if (in->x != out->x / ux || in->y != out->y / uy || in->z != out->z) return mt::fail(MT_E_SHAPE, "mt_upsampling: sizes do not match");
+  uint32_t planes = out->w * out->z, n = out->y * out->x;
+  if (planes == 0 || n == 0) return MT_OK;
+  Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
+  upsampling_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, ux, uy, planes);
+  MT_LAUNCH_CHECK("mt_upsampling");
+  return MT_OK;
+}
+
+int mt_downsampling(const mt_tensor *out, const mt_tensor *in, uint32_t dx, uint32_t dy) {
+  if (mt::bad(out) || mt::bad(in) || dx == 0 || dy == 0) return mt::fail(MT_E_ARGUMENT, "mt_downsampling: bad argument");
+  if (in->x / dx != out->x || in->y / dy != out->y || in->z != out->z || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_downsampling: sizes do not match");
+  uint32_t planes = out->w * out->z, n = out->y * out->x;
+  if (planes == 0 || n == 0) return MT_OK;
+  Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
+  downsampling_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, dx, dy, planes);
+  MT_LAUNCH_CHECK("mt_downsampling");
+  return MT_OK;
+}
+
+int mt_max_pooling(const mt_tensor *out, const mt_pos_tensor *pos, const mt_tensor *in, uint32_t px, uint32_t py) {
+  if (mt::bad(out) || mt::bad(in) || pos == nullptr || px == 0 || py == 0) return mt::fail(MT_E_ARGUMENT, "mt_max_pooling: bad argument");
+  if (in->x / px != out->x || in->y / py != out->y || in->z != out->z || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_max_pooling: sizes do not match");
+  uint32_t planes = out->w * out->z, n = out->y * out->x;
+  if (planes == 0 || n == 0) return MT_OK;
+  if (pos->p == nullptr || pos->w == 0 || pos->z != out->z || pos->y != out->y || pos->x != out->x)
+    return mt::fail(MT_E_ARGUMENT, "mt_max_pooling: position tensor must be [W',Z,Y,X] of the output");
+  Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
+  max_pooling_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, px, py, planes);
+  MT_LAUNCH_CHECK("mt_max_pooling");
+  return MT_OK;
+}
+
+int mt_max_pooling_backward(const mt_tensor *out, const mt_pos_tensor *pos, const mt_tensor *in, uint32_t px, uint32_t py) {
+  if (mt::bad(out) || mt::bad(in) || pos == nullptr || px == 0 || py == 0) return mt::fail(MT_E_ARGUMENT, "mt_max_pooling_backward: bad argument");
+  if (in->x != out->x / px || in->y != out->y / py || in->z != out->z || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_max_pooling_backward: sizes do not match");
+  uint32_t planes = out->w * out->z, n = out->y * out->x;
+  if (planes == 0 || n == 0) return MT_OK;
+  if (pos->p == nullptr || pos->w == 0 || pos->z != in->z || pos->y != in->y || pos->x != in->x)
+    return mt::fail(MT_E_ARGUMENT, "mt_max_pooling_backward: position tensor must be [W',Z,Y,X] of the input");
+  Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
+  max_pooling_backward_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, px, py, planes);
+  MT_LAUNCH_CHECK("mt_max_pooling_backward");
+  return MT_OK;
+}
+
+int mt_adam(const mt_tensor *weight, const mt_tensor *dweight, const mt_tensor *m, const mt_tensor *v, uint32_t batch_size, double speed,
+            double beta1, double beta2, double epsilon, double iteration) {
+  if (mt::bad(weight) || mt::bad(dweight) || mt::bad(m) || mt::bad(v)) return mt::fail(MT_E_ARGUMENT, "mt_adam: null tensor");
+  const mt_tensor *o[3] = {dweight, m, v};
+  for (auto t : o)
+    if (!mt::same_zyx(weight, t) || weight->w != t->w) return mt::fail(MT_E_SHAPE, "mt_adam: sizes do not match");
+  size_t n = mt::count(weight);
+  if (n == 0) return MT_OK;
+  double c1 = 1.0 - pow(beta1, iteration), c2 = 1.0 - pow(beta2, iteration);
+  adam_kernel<<<cdiv(n, EW_THREADS), EW_THREADS, 0, mt::stream()>>>(weight->p, dweight->p, m->p, v->p, n, (float)batch_size, speed, beta1, beta2, epsilon, c1, c2);
+  MT_LAUNCH_CHECK("mt_adam");
+  return MT_OK;
+}
+
+int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
+                                    const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
+                                    const mt_tensor *new_variable, float momentum, float epsilon, int func) {
+  if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: unknown function id %d", func);
+  if (mt::bad(out) || mt::bad(in) || mt::bad(gamma) || mt::bad(beta)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: null tensor");
+  if (!mt::same_zyx(in, out) || in->w != out->w || !mt::same_zyx(gamma, in) || !mt::same_zyx(beta, in))
+    return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_func: sizes do not match");
+  const mt_tensor *stats[5] = {ivar, batch_mean, batch_var, new_mean, new_variable};
+  for (auto t : stats)
+    if (t && (mt::bad(t) || !mt::same_zyx(t, in))) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_func: statistics must be [1,Z,Y,X]");
+  if (xhat && (mt::bad(xhat) || !mt::same_zyx(xhat, in) || xhat->w != in->w)) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_func: xhat must match the input");
+  size_t S = (size_t)in->z * in->y * in->x;
+  uint32_t W = in->w;
+  if (S == 0 || W == 0) return MT_OK;
+  float *scratch = nullptr;
+  int rc = bn_scratch(3 * S, &scratch);
+  if (rc) return rc;
+  float *pm = batch_mean ? batch_mean->p : scratch, *pv = batch_var ? batch_var->p : scratch + S, *pi = ivar ? ivar->p : scratch + 2 * S;
+  float inv_n = (float)(1.0 / (double)(float)W);  // the layer passes 1.0/N with N a float
+  float mom_new = (float)(1.0 - (double)momentum);  // and 1.0-Momentum, rounded once
+  {
+  mt::ProfileScope prof("bn_stats");
+  if (S >= 65536)
+    bn_stats_kernel<256><<<cdiv(S, 256), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, new_mean ? new_mean->p : nullptr, new_variable ? new_variable->p : nullptr, momentum, mom_new);
+  else
+    bn_stats_kernel<32><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, new_mean ? new_mean->p : nullptr, new_variable ? new_variable->p : nullptr, momentum, mom_new);
+  }
+  MT_LAUNCH_CHECK("bn_stats");
+  bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(pm) && aligned16(pi) && (!xhat || aligned16(xhat->p));
+  unsigned gx = cdiv(vec ? S / 4 : S, EW_THREADS);
+  unsigned gy = W < 16 ? W : 16;  // a few batch slices per column block keeps the per-column loads in registers
+  mt::ProfileScope prof("bn_apply");
+  bn_apply_kernel<<<dim3(gx, gy), EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, pm, pi, gamma->p, beta->p, (uint32_t)S, W, vec, func);
+  MT_LAUNCH_CHECK("bn_apply");
+  return MT_OK;
+}
+
+int mt_batchnorm_forward_infer_func(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *mean,
+                                    const mt_tensor *variable, float epsilon, int func) {
+  if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_infer_func: unknown function id %d", func);
+  const mt_tensor *all[6] = {out, in, gamma, beta, mean, variable};
+  for (auto t : all)
+    if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_infer_func: null tensor");
+  if (!mt::same_zyx(in, out) || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_infer_func: sizes do not match");
+  for (int i = 2; i < 6; i++)
+    if (!mt::same_zyx(all[i], in)) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_infer_func: parameters must be [1,Z,Y,X]");
+  size_t S = (size_t)in->z * in->y * in->x;
+  uint32_t W = in->w;
+  if (S == 0 || W == 0) return MT_OK;
+  float *scratch = nullptr;
+  int rc = bn_scratch(3 * S, &scratch);
+  if (rc) return rc;
+  bn_ivar_kernel<<<cdiv(S, EW_THREADS), EW_THREADS, 0, mt::stream()>>>(scratch, variable->p, (uint32_t)S, epsilon);
+  MT_LAUNCH_CHECK("bn_ivar");
+  bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(mean->p);
+  unsigned gx = cdiv(vec ? S / 4 : S, EW_THREADS);
+  unsigned gy = W < 16 ? W : 16;
+  bn_apply_kernel<<<dim3(gx, gy), EW_THREADS, 0, mt::stream()>>>(out->p, nullptr, in->p, mean->p, scratch, gamma->p, beta->p, (uint32_t)S, W, vec, func);
+  MT_LAUNCH_CHECK("bn_apply");
+  return MT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,107 @@
+// CTensorMath::Mul / TransponseMul and the Linear layer's forward pass on the fp32 matrix cores.
+//
+// The reference runs one small product per batch entry (grid.z = W, N = 1 for a Linear layer).  Here a batch
+// that shares one operand is folded into a single wide product before it reaches the matrix cores:
+//   left  has W == 1:  C[w] = A * B[w]   ->  one product with N' = W*N columns
+//   right has W == 1:  C[w] = A[w] * B   ->  one product with M' = W*M rows
+// With N == 1 (matrix times a batch of vectors) the folded product is computed transposed, C'[w][m], so that
+// the 64 lanes of a wavefront write consecutive addresses.
+#include "mt_igemm.h"
+
+namespace {
+
+using namespace mt::igemm;
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+SrcRowK row_k(const float *p, uint32_t ld, uint32_t R, uint32_t K) {
+  SrcRowK s{};
+  s.p = p; s.ld = ld; s.R = R; s.K = K;
+  s.vec = (ld % 4 == 0) && aligned16(p);
+  return s;
+}
+SrcColK col_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, uint32_t inner, size_t gstride) {
+  SrcColK s{};
+  s.p = p; s.ld = ld; s.R = R; s.K = K; s.inner = inner; s.gstride = gstride;
+  return s;
+}
+
+// C[w,z] = op(A[w%Wa,z]) * B[w%Wb,z];  op = transpose when `ta` (A stored [K][M]).
+// bias (optional) holds one value per output row m; func is applied last.
+int product(const char *name, const mt_tensor *out, const mt_tensor *left, const mt_tensor *right, bool ta, const float *bias, int func) {
+  if (mt::bad(out) || mt::bad(left) || mt::bad(right)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  const uint32_t M = ta ? left->x : left->y, K = ta ? left->y : left->x, N = right->x, Z = left->z;
+  if (K != right->y || left->z != right->z || out->y != M || out->x != N || out->z != right->z)
+    return mt::fail(MT_E_SHAPE, "%s: sizes do not match", name);
+  const uint32_t W = out->w;
+  if (W == 0 || Z == 0 || M == 0 || N == 0) return MT_OK;
+  if (left->w == 0 || right->w == 0) return mt::fail(MT_E_ARGUMENT, "%s: empty operand", name);
+  if (K == 0) return mt_fill(out, 0.f);
+
+  Epilogue ep{};
+  ep.C = out->p;
+  ep.func = func;
+  const bool fold_ok = Z == 1 && W > 1;
+
+  if (fold_ok && left->w == 1 && right->w >= W) {
+    if (N == 1) {
+      // C'[w][m] = sum_k B[w][k] * op(A)[m][k]: rows are batch entries, columns are the output rows m
+      ep.row_stride = M; ep.inner = M; ep.g_stride = 0;
+      if (bias) { ep.bias = bias; ep.bias_mode = 2; }
+      SrcRowK a = row_k(right->p, K, W, K);
+      if (ta) return launch(name, a, col_k(left->p, M, M, K, M, 0), ep, W, M, K, 1);
+      return launch(name, a, row_k(left->p, K, M, K), ep, W, M, K, 1);
+    }
+    // one product with N' = W*N columns; column n' = (w, n)
+    ep.row_stride = N; ep.inner = N; ep.g_stride = (size_t)M * N;
+    if (bias) { ep.bias = bias; ep.bias_mode = 1; }
+    SrcColK b = col_k(right->p, N, W * N, K, N, (size_t)K * N);
+    if (ta) return launch(name, col_k(left->p, M, M, K, M, 0), b, ep, M, W * N, K, 1);
+    return launch(name, row_k(left->p, K, M, K), b, ep, M, W * N, K, 1);
+  }
+  if (fold_ok && right->w == 1 && left->w >= W && !ta && !bias) {
+    // rows (w, m) of A and of C are contiguous: one product with M' = W*M rows
+    ep.row_stride = N; ep.inner = N; ep.g_stride = 0;
+    return launch(name, row_k(left->p, K, W * M, K), col_k(right->p, N, N, K, N, 0), ep, W * M, N, K, 1);
+  }
+
+  // general case: one product per (w, z)
+  ep.row_stride = N; ep.inner = N; ep.g_stride = 0;
+  ep.bt.wmod = W; ep.bt.zcount = Z; ep.bt.stride = (size_t)M * N;
+  if (bias) { ep.bias = bias; ep.bias_mode = 1; }
+  SrcColK b = col_k(right->p, N, N, K, N, 0);
+  b.bt.wmod = right->w; b.bt.zcount = Z; b.bt.stride = (size_t)K * N;
+  if (ta) {
+    SrcColK a = col_k(left->p, M, M, K, M, 0);
+    a.bt.wmod = left->w; a.bt.zcount = Z; a.bt.stride = (size_t)K * M;
+    return launch(name, a, b, ep, M, N, K, W * Z);
+  }
+  SrcRowK a = row_k(left->p, K, M, K);
+  a.bt.wmod = left->w; a.bt.zcount = Z; a.bt.stride = (size_t)M * K;
+  return launch(name, a, b, ep, M, N, K, W * Z);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mt_mul(const mt_tensor *out, const mt_tensor *left, const mt_tensor *right) { return product("mt_mul", out, left, right, false, nullptr, MT_F_NONE); }
+
+int mt_transponse_mul(const mt_tensor *out, const mt_tensor *left, const mt_tensor *right) {
+  return product("mt_transponse_mul", out, left, right, true, nullptr, MT_F_NONE);
+}
+
+int mt_linear_forward_func(const mt_tensor *out, const mt_tensor *weight, const mt_tensor *input, const mt_tensor *bias, int func) {
+  if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_linear_forward_func: unknown function id %d", func);
+  if (mt::bad(out) || mt::bad(weight) || mt::bad(input) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "mt_linear_forward_func: null tensor");
+  // the layer views its input as [B,1,In,1] (ReinterpretSize, netlayer/cnetlayerlinear.cu.h:271)
+  mt_tensor in = *input;
+  in.y = input->z * input->y * input->x;
+  in.z = 1;
+  in.x = 1;
+  if (weight->w != 1 || weight->z != 1 || bias->w != 1 || bias->z != 1 || bias->x != 1 || bias->y != weight->y || out->w != input->w)
+    return mt::fail(MT_E_SHAPE, "mt_linear_forward_func: weight must be [1,1,Out,In], bias [1,1,Out,1], output [B,1,Out,1]");
+  return product("mt_linear_forward_func", out, weight, &in, false, bias->p, func);
+}
+
+}  // extern "C"

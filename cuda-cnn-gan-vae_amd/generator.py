@@ -1,0 +1,120 @@
+"""DCGAN-64 generator forward pass as the reference's layers would run it, on device-resident tensors.
+
+Layer stack (the reference's layer classes in brackets):
+    latent [B,1,100,1]
+    -> Linear 100 -> 512*4*4              [CNetLayerLinear, netlayer/cnetlayerlinear.cu.h:262-282]
+    -> BatchNorm (batch statistics) + ReLU [CNetLayerBatchNormalization :268-380, CNetLayerFunction :203-213]
+    -> transposed conv 4x4 s2 p1, 512 -> 256 -> 128 -> 64, each followed by BatchNorm + ReLU
+                                           [CNetLayerBackConvolution, netlayer/cnetlayerbackconvolution.cu.h:303-315]
+    -> transposed conv 4x4 s2 p1, 64 -> 3, tanh -> images [B,3,64,64]
+
+Batch-norm statistics are per element (z,y,x) over the batch axis, as in the reference.
+`forward_fused` uses the fused C-ABI entry points (one or two launches per layer); `forward_literal`
+issues the reference layers' exact op sequences, one C-ABI call per tensor op.
+"""
+import numpy as np
+
+import mi355tensor as mt
+from mi355tensor import CTensor, CTensorApplyFunc, CTensorConv, CTensorMath, Fused
+
+LATENT = 100
+CHANNELS = (512, 256, 128, 64, 3)
+BN_EPSILON = 1e-6
+MOMENTUM = 0.9
+
+
+def make_parameters(seed=3, std=0.02):
+    """Random-init parameters (N(0, std)), biases 0, gamma 1, beta 0, as numpy arrays in the reference's layouts."""
+    rng = np.random.default_rng(seed)
+    p = {"lin_w": (rng.standard_normal((1, 1, CHANNELS[0] * 16, LATENT)) * std).astype(np.float32),
+         "lin_b": np.zeros((1, 1, CHANNELS[0] * 16, 1), np.float32)}
+    size = 4
+    for i in range(4):
+        cin, cout = CHANNELS[i], CHANNELS[i + 1]
+        p["gamma%d" % i] = np.ones((1, cin, size, size), np.float32)
+        p["beta%d" % i] = np.zeros((1, cin, size, size), np.float32)
+        # kernel of BackwardConvolution: row f = input channel, column z*16 + i*4 + j (cpu/ctensorconv.h:256)
+        p["kernel%d" % i] = (rng.standard_normal((1, 1, cin, cout * 16)) * std).astype(np.float32)
+        p["bias%d" % i] = np.zeros((1, cin, 1, 1), np.float32)
+        size *= 2
+    return p
+
+
+def make_latent(batch, seed=3):
+    return np.random.default_rng(seed + 1000).standard_normal((batch, 1, LATENT, 1)).astype(np.float32)
+
+
+def conv_flops(batch):
+    """Algorithmic FLOPs (2*MAC, non-zero taps only) of the four transposed convolutions, per layer."""
+    out, size = [], 4
+    for i in range(4):
+        out.append(2.0 * batch * CHANNELS[i] * size * size * CHANNELS[i + 1] * 16)
+        size *= 2
+    return out
+
+
+class DcganGenerator:
+    def __init__(self, batch, params=None):
+        mt.init(0)
+        self.batch = batch
+        host = params or make_parameters()
+        self.p = {k: CTensor.from_numpy(v) for k, v in host.items()}
+        b = batch
+        self.latent = CTensor(b, 1, LATENT, 1)
+        self.h = [CTensor(b, CHANNELS[0], 4, 4)]            # pre-normalisation activations
+        self.a = []                                          # post BN+ReLU activations
+        size = 4
+        for i in range(4):
+            self.a.append(CTensor(b, CHANNELS[i], size, size))
+            size *= 2
+            self.h.append(CTensor(b, CHANNELS[i + 1], size, size))
+        self.lin_out = self.h[0].reinterpret(b, 1, CHANNELS[0] * 16, 1)
+        self.literal_tmp = None
+
+    def set_latent(self, z):
+        self.latent.upload(z)
+
+    @property
+    def output(self):
+        return self.h[4]
+
+    def forward_fused(self):
+        p = self.p
+        Fused.LinearForward(self.lin_out, p["lin_w"], self.latent, p["lin_b"], None)
+        for i in range(4):
+            Fused.BatchNormForwardTrain(self.a[i], self.h[i], p["gamma%d" % i], p["beta%d" % i], momentum=MOMENTUM, epsilon=BN_EPSILON, func="relu")
+            CTensorConv.BackwardConvolution(self.h[i + 1], self.a[i], p["kernel%d" % i], 4, 4, CHANNELS[i + 1], CHANNELS[i], p["bias%d" % i], 2, 2, 1, 1,
+                                            func="tangence" if i == 3 else None)
+        return self.h[4]
+
+    def forward_literal(self):
+        """Every layer as the reference issues it: Mul + Add; the 11 tensor ops of a training-mode batch norm;
+        ApplyReLU; BackwardConvolution; ApplyTangence."""
+        p = self.p
+        if self.literal_tmp is None:
+            self.literal_tmp = []
+            for i in range(4):
+                s = self.h[i].shape
+                one = (1,) + s[1:]
+                self.literal_tmp.append(dict(mean=CTensor(*one), var=CTensor(*one), sqrtvar=CTensor(*one), ivar=CTensor(*one),
+                                             xhat=CTensor(*s), tmp=CTensor(*s), bn=CTensor(*s)))
+        CTensorMath.Mul(self.lin_out, p["lin_w"], self.latent)
+        CTensorMath.Add(self.lin_out, self.lin_out, p["lin_b"])
+        inv_n = float(np.float32(1.0 / np.float64(np.float32(self.batch))))
+        for i in range(4):
+            t, x = self.literal_tmp[i], self.h[i]
+            CTensorMath.Fill(t["mean"], 0)
+            CTensorMath.AddSumW(t["mean"], t["mean"], x, 1, inv_n)
+            CTensorMath.Sub(t["xhat"], x, t["mean"], 1.0, 1.0)
+            CTensorMath.Fill(t["var"], 0)
+            CTensorMath.Pow2(t["tmp"], t["xhat"], 1)
+            CTensorMath.AddSumW(t["var"], t["var"], t["tmp"], 1, inv_n)
+            CTensorMath.SQRT(t["sqrtvar"], t["var"], 1, BN_EPSILON)
+            CTensorMath.Inv(t["ivar"], t["sqrtvar"])
+            CTensorMath.TensorItemProduction(t["xhat"], t["xhat"], t["ivar"])
+            CTensorMath.TensorItemProduction(t["tmp"], p["gamma%d" % i], t["xhat"])
+            CTensorMath.Add(t["bn"], t["tmp"], p["beta%d" % i])
+            CTensorApplyFunc.ApplyReLU(self.a[i], t["bn"])
+            CTensorConv.BackwardConvolution(self.h[i + 1], self.a[i], p["kernel%d" % i], 4, 4, CHANNELS[i + 1], CHANNELS[i], p["bias%d" % i], 2, 2, 1, 1)
+        CTensorApplyFunc.ApplyTangence(self.h[4], self.h[4])
+        return self.h[4]

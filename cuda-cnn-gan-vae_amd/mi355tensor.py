@@ -1,0 +1,347 @@
+"""ctypes binding of libmi355tensor.so for tests and benchmarks.
+
+The names mirror the reference's C++ classes (`CTensor`, `CTensorMath`, `CTensorConv`,
+`CTensorApplyFunc`; cuda/ctensor.cu.h:69-168, cuda/ctensormath.cu.h:52-138,
+cuda/ctensorconv.cu.h:48-69, cuda/ctensorapplyfunc.cu.h) with the same argument order, so a test
+written against the reference reads the same here.  Every call goes through the C ABI declared in
+include/mi355_tensor.h; there is no CPU fallback: without the built library and a gfx950 device
+this module raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmi355tensor.so")
+
+FUNC = {"sigmoid": 0, "relu": 1, "gelu": 2, "leaky_relu": 3, "linear": 4, "tangence": 5, None: -1, "none": -1}
+DIFFERENTIAL = 8
+
+
+class MtTensor(C.Structure):
+    _fields_ = [("p", C.c_void_p), ("w", C.c_uint32), ("z", C.c_uint32), ("y", C.c_uint32), ("x", C.c_uint32)]
+
+
+class TensorError(RuntimeError):
+    """A non-zero status of the C ABI (the C++ classes `throw` a message in the same place)."""
+
+    def __init__(self, name, code, message):
+        super().__init__("%s failed with code %d: %s" % (name, code, message))
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libmi355tensor.so is not built: run `make -C cuda-cnn-gan-vae_amd` (or __graft_entry__.build())")
+        _lib = C.CDLL(LIB_PATH)
+        _lib.mt_last_error.restype = C.c_char_p
+        _lib.mt_get_stream.restype = C.c_void_p
+        _lib.mt_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+        _lib.mt_free.argtypes = [C.c_void_p]
+        for f in ("mt_copy_h2d", "mt_copy_d2h", "mt_copy_d2d"):
+            getattr(_lib, f).argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        _lib.mt_set_stream.argtypes = [C.c_void_p]
+        _lib.mt_set_option.argtypes = [C.c_char_p, C.c_int]
+    return _lib
+
+
+def call(name, *args):
+    fn = getattr(lib(), name)
+    fn.restype = C.c_int
+    rc = fn(*args)
+    if rc != 0:
+        raise TensorError(name, rc, lib().mt_last_error().decode(errors="replace"))
+
+
+def init(device=0):
+    call("mt_init", C.c_int(device))
+
+
+def synchronize():
+    call("mt_synchronize")
+
+
+def set_option(name, value):
+    call("mt_set_option", name.encode(), C.c_int(value))
+
+
+def profile_enable(on=True):
+    call("mt_profile_enable", C.c_int(1 if on else 0))
+
+
+def profile_report():
+    """{label: (launches, total_ms)} of the kernels launched since profile_enable(True); waits for the stream."""
+    n = lib().mt_profile_entries()
+    if n < 0:
+        raise TensorError("mt_profile_entries", n, lib().mt_last_error().decode(errors="replace"))
+    out = {}
+    for i in range(n):
+        label, launches, ms = C.c_char_p(), C.c_uint64(), C.c_double()
+        call("mt_profile_entry", C.c_int(i), C.byref(label), C.byref(launches), C.byref(ms))
+        out[label.value.decode()] = (launches.value, ms.value)
+    return out
+
+
+def get_stream():
+    return lib().mt_get_stream()
+
+
+def set_stream(handle):
+    call("mt_set_stream", C.c_void_p(handle))
+
+
+class CTensor:
+    """Device-resident [W,Z,Y,X] fp32 tensor (uint32 pairs for pooling positions when `pos` is set)."""
+
+    def __init__(self, size_w=1, size_z=1, size_y=1, size_x=1, pos=False):
+        self.shape = (int(size_w), int(size_z), int(size_y), int(size_x))
+        self.pos = pos
+        self.item = 8 if pos else 4
+        self.ptr = C.c_void_p()
+        self.owned = True
+        call("mt_malloc", C.byref(self.ptr), C.c_size_t(self.count * self.item))
+
+    @property
+    def count(self):
+        w, z, y, x = self.shape
+        return w * z * y * x
+
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        assert a.ndim == 4, "tensors are [W,Z,Y,X]"
+        t = cls(*a.shape)
+        t.upload(a)
+        return t
+
+    @classmethod
+    def wrap(cls, ptr, shape):
+        """Borrow device memory owned by someone else (e.g. a torch tensor's data_ptr())."""
+        t = cls.__new__(cls)
+        t.shape, t.pos, t.item, t.ptr, t.owned = tuple(int(s) for s in shape), False, 4, C.c_void_p(ptr), False
+        return t
+
+    def upload(self, a):
+        a = np.ascontiguousarray(a, dtype=np.uint32 if self.pos else np.float32)
+        assert a.size == self.count * (2 if self.pos else 1)
+        if a.size:
+            call("mt_copy_h2d", self.ptr, C.c_void_p(a.ctypes.data), C.c_size_t(a.nbytes))
+
+    def numpy(self):
+        out = np.empty(self.shape + ((2,) if self.pos else ()), np.uint32 if self.pos else np.float32)
+        if out.size:
+            call("mt_copy_d2h", C.c_void_p(out.ctypes.data), self.ptr, C.c_size_t(out.nbytes))
+        else:
+            synchronize()
+        return out
+
+    def reinterpret(self, w, z, y, x):
+        """ReinterpretSize: the same memory under other sizes (cuda/ctensor.cu.h:587-601)."""
+        assert w * z * y * x == self.count, "the element count must not change"
+        return CTensor.wrap(self.ptr.value, (w, z, y, x))
+
+    def desc(self):
+        return MtTensor(self.ptr.value, *self.shape)
+
+    def free(self):
+        if self.owned and self.ptr:
+            call("mt_free", self.ptr)
+            self.ptr = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _d(t):
+    return C.byref(t.desc())
+
+
+def _i(v):
+    return C.c_int32(int(v))
+
+
+def _u(v):
+    return C.c_uint32(int(v))
+
+
+def _f(v):
+    return C.c_float(float(v))
+
+
+class CTensorConv:
+    @staticmethod
+    def ForwardConvolution(out, image, kernel, kernel_x, kernel_y, kernel_z, kernel_amount, bias, stride_x, stride_y, padding_x, padding_y, func=None):
+        args = (_d(out), _d(image), _d(kernel), _i(kernel_x), _i(kernel_y), _i(kernel_z), _u(kernel_amount), _d(bias), _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y))
+        if func is None:
+            call("mt_forward_convolution", *args)
+        else:
+            call("mt_forward_convolution_func", *args, C.c_int(FUNC[func]))
+
+    @staticmethod
+    def BackwardConvolution(out, delta, kernel, kernel_x, kernel_y, kernel_z, kernel_amount, bias, stride_x, stride_y, padding_x, padding_y, func=None):
+        args = (_d(out), _d(delta), _d(kernel), _i(kernel_x), _i(kernel_y), _i(kernel_z), _u(kernel_amount), _d(bias), _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y))
+        if func is None:
+            call("mt_backward_convolution", *args)
+        else:
+            call("mt_backward_convolution_func", *args, C.c_int(FUNC[func]))
+
+    @staticmethod
+    def CreateDeltaWeightAndBias(dkernel, dkernel_x, dkernel_y, dkernel_z, dkernel_amount, dbias, image, delta, stride_x, stride_y, padding_x, padding_y):
+        call("mt_create_delta_weight_and_bias", _d(dkernel), _i(dkernel_x), _i(dkernel_y), _i(dkernel_z), _u(dkernel_amount), _d(dbias), _d(image), _d(delta),
+             _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y))
+
+    @staticmethod
+    def CreateBackDeltaWeightAndBias(dkernel, dkernel_x, dkernel_y, dkernel_z, dkernel_amount, dbias, image, delta, stride_x, stride_y, padding_x, padding_y):
+        call("mt_create_back_delta_weight_and_bias", _d(dkernel), _i(dkernel_x), _i(dkernel_y), _i(dkernel_z), _u(dkernel_amount), _d(dbias), _d(image), _d(delta),
+             _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y))
+
+
+class CTensorMath:
+    @staticmethod
+    def Fill(out, value=0.0):
+        call("mt_fill", _d(out), _f(value))
+
+    @staticmethod
+    def Inv(out, inp):
+        call("mt_inv", _d(out), _d(inp))
+
+    @staticmethod
+    def Div(out, left, right, left_scale=1.0, right_scale=1.0):
+        call("mt_div", _d(out), _d(left), _d(right), _f(left_scale), _f(right_scale))
+
+    @staticmethod
+    def Add(out, left, right, left_scale=1.0, right_scale=1.0):
+        call("mt_add", _d(out), _d(left), _d(right), _f(left_scale), _f(right_scale))
+
+    @staticmethod
+    def Sub(out, left, right, left_scale=1.0, right_scale=1.0):
+        call("mt_sub", _d(out), _d(left), _d(right), _f(left_scale), _f(right_scale))
+
+    @staticmethod
+    def AddSumW(out, left, right, left_scale=1.0, right_scale=1.0):
+        call("mt_add_sum_w", _d(out), _d(left), _d(right), _f(left_scale), _f(right_scale))
+
+    @staticmethod
+    def AddValue(out, inp, tensor_scale, value):
+        call("mt_add_value", _d(out), _d(inp), _f(tensor_scale), _f(value))
+
+    @staticmethod
+    def SubValue(out, inp, tensor_scale, value):
+        call("mt_sub_value", _d(out), _d(inp), _f(tensor_scale), _f(value))
+
+    @staticmethod
+    def Set(out, inp, scale=1.0, add_value=0.0):
+        call("mt_set", _d(out), _d(inp), _f(scale), _f(add_value))
+
+    @staticmethod
+    def Pow2(out, inp, scale=1.0):
+        call("mt_pow2", _d(out), _d(inp), _f(scale))
+
+    @staticmethod
+    def SQRT(out, inp, scale, add_sqrt_value):
+        call("mt_sqrt", _d(out), _d(inp), _f(scale), _f(add_sqrt_value))
+
+    @staticmethod
+    def AddBias(working, bias):
+        call("mt_add_bias", _d(working), _d(bias))
+
+    @staticmethod
+    def SummXY(out, inp):
+        call("mt_summ_xy", _d(out), _d(inp))
+
+    @staticmethod
+    def Mul(out, left, right):
+        """Tensor * tensor, or tensor * scalar / scalar * tensor (the reference overloads Mul the same way)."""
+        if isinstance(right, (int, float)):
+            call("mt_mul_value", _d(out), _d(left), _f(right))
+        elif isinstance(left, (int, float)):
+            call("mt_mul_value", _d(out), _d(right), _f(left))
+        else:
+            call("mt_mul", _d(out), _d(left), _d(right))
+
+    @staticmethod
+    def TransponseMul(out, left, right):
+        call("mt_transponse_mul", _d(out), _d(left), _d(right))
+
+    @staticmethod
+    def Transponse(out, inp):
+        call("mt_transponse", _d(out), _d(inp))
+
+    @staticmethod
+    def TensorItemProduction(out, left, right):
+        call("mt_tensor_item_production", _d(out), _d(left), _d(right))
+
+    @staticmethod
+    def UpSampling(out, inp, upsampling_x, upsampling_y):
+        call("mt_upsampling", _d(out), _d(inp), _u(upsampling_x), _u(upsampling_y))
+
+    @staticmethod
+    def DownSampling(out, inp, downsampling_x, downsampling_y):
+        call("mt_downsampling", _d(out), _d(inp), _u(downsampling_x), _u(downsampling_y))
+
+    @staticmethod
+    def MaxPooling(out, position, inp, pooling_x, pooling_y):
+        call("mt_max_pooling", _d(out), _d(position), _d(inp), _u(pooling_x), _u(pooling_y))
+
+    @staticmethod
+    def MaxPoolingBackward(out, position, inp, pooling_x, pooling_y):
+        call("mt_max_pooling_backward", _d(out), _d(position), _d(inp), _u(pooling_x), _u(pooling_y))
+
+    @staticmethod
+    def Clip(tensor, min_value, max_value):
+        call("mt_clip", _d(tensor), _f(min_value), _f(max_value))
+
+    @staticmethod
+    def Signum(tensor):
+        call("mt_signum", _d(tensor))
+
+    @staticmethod
+    def Adam(weight, dweight, m, v, batch_size, speed, beta1, beta2, epsilon, iteration):
+        call("mt_adam", _d(weight), _d(dweight), _d(m), _d(v), _u(batch_size), C.c_double(speed), C.c_double(beta1), C.c_double(beta2),
+             C.c_double(epsilon), C.c_double(iteration))
+
+
+class CTensorApplyFunc:
+    @staticmethod
+    def Apply(out, inp, func, differential=False):
+        call("mt_apply_func", _d(out), _d(inp), C.c_int(FUNC[func] + (DIFFERENTIAL if differential else 0)))
+
+
+for _name, _key in (("Sigmoid", "sigmoid"), ("ReLU", "relu"), ("GeLU", "gelu"), ("LeakyReLU", "leaky_relu"), ("Linear", "linear"), ("Tangence", "tangence")):
+    setattr(CTensorApplyFunc, "Apply" + _name, staticmethod(lambda out, inp, k=_key: CTensorApplyFunc.Apply(out, inp, k)))
+    setattr(CTensorApplyFunc, "ApplyDifferential" + _name, staticmethod(lambda out, inp, k=_key: CTensorApplyFunc.Apply(out, inp, k, True)))
+
+
+class Fused:
+    """The fused layer entry points of the C ABI (one reference layer Forward() each)."""
+
+    @staticmethod
+    def LinearForward(out, weight, inp, bias, func=None):
+        call("mt_linear_forward_func", _d(out), _d(weight), _d(inp), _d(bias), C.c_int(FUNC[func]))
+
+    @staticmethod
+    def BatchNormForwardTrain(out, inp, gamma, beta, xhat=None, ivar=None, batch_mean=None, batch_var=None, new_mean=None, new_variable=None,
+                              momentum=0.9, epsilon=1e-6, func=None):
+        opt = lambda t: _d(t) if t is not None else None
+        call("mt_batchnorm_forward_train_func", _d(out), _d(inp), _d(gamma), _d(beta), opt(xhat), opt(ivar), opt(batch_mean), opt(batch_var),
+             opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
+
+    @staticmethod
+    def BatchNormForwardInfer(out, inp, gamma, beta, mean, variable, epsilon=1e-6, func=None):
+        call("mt_batchnorm_forward_infer_func", _d(out), _d(inp), _d(gamma), _d(beta), _d(mean), _d(variable), _f(epsilon), C.c_int(FUNC[func]))
+
+
+def exported_symbols():
+    """Names declared in include/mi355_tensor.h (used by the CPU-side ABI test)."""
+    import re
+    header = open(os.path.join(HERE, "..", "include", "mi355_tensor.h")).read()
+    return sorted(set(re.findall(r"\b(mt_[a-z0-9_]+)\s*\(", header)))

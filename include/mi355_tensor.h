@@ -1,0 +1,175 @@
+/*
+ * mi355_tensor.h -- C ABI of libmi355tensor.so, the MI355X (gfx950) tensor-op library
+ * that backs the reference's CTensor / CTensorMath / CTensorConv / CTensorApplyFunc
+ * classes.  Each entry point below replaces one static member function of the
+ * reference's GPU classes (file:line given per function, relative to the reference
+ * tree) and keeps its argument order, argument meaning and precondition checks.
+ *
+ * Conventions
+ *  - Tensors are dense fp32 [W,Z,Y,X] arrays in DEVICE memory, X contiguous; element
+ *    (w,z,y,x) is at x + X*(y + Y*(z + Z*w))  (cuda/ctensor.cu.h:293).  The library
+ *    borrows the pointers for the duration of the call and never owns them.
+ *  - An operand whose W is smaller than the output's broadcasts by w % W
+ *    (cuda/ctensormath.cu.h:141-145).
+ *  - Every function returns 0 on success.  MT_E_* (1..5) are the reference's
+ *    precondition failures (where the C++ classes `throw` a message); values >= 1000
+ *    are 1000 + hipError_t.  mt_last_error() returns a readable message.
+ *  - Work is enqueued on one HIP stream (mt_get_stream) and is asynchronous with
+ *    respect to the host; mt_copy_d2h and mt_synchronize wait for it.  The reference
+ *    blocks after every launch (cudaDeviceSynchronize); callers see the same results
+ *    because every host read goes through mt_copy_d2h.
+ *  - Not thread safe: one host thread per process, as in the reference.
+ */
+#ifndef MI355_TENSOR_H
+#define MI355_TENSOR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct {
+  float *p;            /* device pointer */
+  uint32_t w, z, y, x; /* sizes, [W,Z,Y,X] */
+} mt_tensor;
+
+/* CTensorMath<T>::SPos (cuda/ctensormath.cu.h:63-67): absolute input coordinates of a pooling maximum */
+typedef struct {
+  uint32_t X, Y;
+} mt_spos;
+
+typedef struct {
+  mt_spos *p; /* device pointer */
+  uint32_t w, z, y, x;
+} mt_pos_tensor;
+
+enum {
+  MT_OK = 0,
+  MT_E_NO_KERNELS = 1,   /* kernel_amount == 0                                  (cpu/ctensorconv.h:88,199,321)  */
+  MT_E_BIAS_COUNT = 2,   /* bias Z != kernel_amount                             (cpu/ctensorconv.h:89,200,322)  */
+  MT_E_OUTPUT_SHAPE = 3, /* output tensor has the wrong Z/Y/X                   (cpu/ctensorconv.h:103,220)     */
+  MT_E_DEPTH = 4,        /* image/delta depth does not match the kernels        (cpu/ctensorconv.h:105,221,335) */
+  MT_E_SHAPE = 5,        /* "sizes do not match" of the tensor-math functions   (cpu/ctensormath.h, every head) */
+  MT_E_ARGUMENT = 6,     /* null pointer, zero stride, unknown function id ...  (no counterpart: the C++ API cannot express these) */
+  MT_E_UNAVAILABLE = 7,  /* no usable gfx950 device                             */
+  MT_E_HIP = 1000        /* + hipError_t                                         (cuda/handle_error.cu.h:7-19)  */
+};
+
+/* activation ids (cuda/ctensorapplyfunc.cu.h:60-...): add MT_F_DIFFERENTIAL for the derivative */
+enum {
+  MT_F_SIGMOID = 0, MT_F_RELU = 1, MT_F_GELU = 2, MT_F_LEAKY_RELU = 3, MT_F_LINEAR = 4, MT_F_TANGENCE = 5,
+  MT_F_DIFFERENTIAL = 8,
+  MT_F_NONE = -1 /* fused entry points only: no activation */
+};
+
+/* ---- runtime: replaces CCUDADeviceVector (cuda/ccudadevicevector.cu.h:41-72) and HANDLE_ERROR ---- */
+int mt_init(int device);                 /* cuda/cuda.cu:81 (cudaSetDevice); checks the device is gfx950 */
+const char *mt_last_error(void);
+int mt_malloc(void **ptr, size_t bytes); /* ccudadevicevector.cu.h resize   */
+int mt_free(void *ptr);                  /* ccudadevicevector.cu.h clear    */
+int mt_copy_h2d(void *dst, const void *src, size_t bytes); /* copy_host_to_device */
+int mt_copy_d2h(void *dst, const void *src, size_t bytes); /* copy_device_to_host; waits for queued work */
+int mt_copy_d2d(void *dst, const void *src, size_t bytes); /* operator= (device copy, :159-170) */
+int mt_synchronize(void);
+void *mt_get_stream(void);               /* the hipStream_t all work is queued on */
+int mt_set_stream(void *hip_stream);     /* queue on a caller-owned stream (NULL: back to the library's own) */
+/* "conv_path": 0 choose per shape (default), 1 one-thread-per-output kernels in the CPU path's summation order,
+ * 2 matrix-core kernels wherever they apply.  For tests and measurements; results agree within fp32 rounding. */
+int mt_set_option(const char *name, int value);
+
+/* ---- convolutions: CTensorConv<T> (cuda/ctensorconv.cu.h:63-66) ---- */
+/* ForwardConvolution, cuda/ctensorconv.cu.h:276-315 (+ the AddBias launch it ends with); CPU: cpu/ctensorconv.h:84-148 */
+int mt_forward_convolution(const mt_tensor *output, const mt_tensor *image, const mt_tensor *kernel,
+                           int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
+                           const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y);
+/* BackwardConvolution, cuda/ctensorconv.cu.h:683-725; CPU: cpu/ctensorconv.h:196-266 (the per-tap bias of the CPU path is kept) */
+int mt_backward_convolution(const mt_tensor *output_delta, const mt_tensor *delta, const mt_tensor *kernel,
+                            int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
+                            const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y);
+/* CreateDeltaWeightAndBias, cuda/ctensorconv.cu.h:1168-1211; CPU: cpu/ctensorconv.h:319-386. Accumulates into dkernel and dbias. */
+int mt_create_delta_weight_and_bias(const mt_tensor *dkernel, int32_t dkernel_x, int32_t dkernel_y, int32_t dkernel_z,
+                                    uint32_t dkernel_amount, const mt_tensor *dbias, const mt_tensor *image,
+                                    const mt_tensor *delta, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y);
+/* CreateBackDeltaWeightAndBias, cuda/ctensorconv.cu.h:1218-1222; CPU: cpu/ctensorconv.h:393-397 */
+int mt_create_back_delta_weight_and_bias(const mt_tensor *dkernel, int32_t dkernel_x, int32_t dkernel_y, int32_t dkernel_z,
+                                         uint32_t dkernel_amount, const mt_tensor *dbias, const mt_tensor *image,
+                                         const mt_tensor *delta, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y);
+
+/* ---- matrix products: CTensorMath<T> ---- */
+int mt_mul(const mt_tensor *output, const mt_tensor *left, const mt_tensor *right);            /* Mul, cuda/ctensormath.cu.h:2237-2243 (MulAbstract :1949-2067); CPU :531-595 */
+int mt_transponse_mul(const mt_tensor *output, const mt_tensor *left, const mt_tensor *right); /* TransponseMul, cuda :2249-2255; CPU :643-712 */
+int mt_transponse(const mt_tensor *output, const mt_tensor *input);                            /* Transponse, cuda :2362 (a host loop there); CPU :787-816 */
+
+/* ---- elementwise and reductions: CTensorMath<T> (line numbers: cuda/ctensormath.cu.h host entry; CPU twin in cpu/ctensormath.h) ---- */
+int mt_fill(const mt_tensor *output, float value);                                                                               /* Fill :637; CPU :154-157 */
+int mt_inv(const mt_tensor *output, const mt_tensor *input);                                                                     /* Inv :702; CPU :163-190 */
+int mt_div(const mt_tensor *output, const mt_tensor *left, const mt_tensor *right, float left_scale, float right_scale);         /* Div :768; CPU :197-229 */
+int mt_add(const mt_tensor *output, const mt_tensor *left, const mt_tensor *right, float left_scale, float right_scale);         /* Add :837; CPU :235-266 */
+int mt_sub(const mt_tensor *output, const mt_tensor *left, const mt_tensor *right, float left_scale, float right_scale);         /* Sub :1021; CPU :314-346 */
+int mt_add_sum_w(const mt_tensor *output, const mt_tensor *left, const mt_tensor *right, float left_scale, float right_scale);   /* AddSumW :914; CPU :273-307 */
+int mt_add_bias(const mt_tensor *working, const mt_tensor *bias);                                                                /* AddBias :1328; CPU :352-381 */
+int mt_pow2(const mt_tensor *output, const mt_tensor *input, float scale);                                                       /* Pow2 :1196; CPU :387-415 */
+int mt_sqrt(const mt_tensor *output, const mt_tensor *input, float scale, float add_sqrt_value);                                 /* SQRT :1262; CPU :421-449 */
+int mt_summ_xy(const mt_tensor *output, const mt_tensor *input);                                                                 /* SummXY :1396; CPU :455-483 */
+int mt_mul_value(const mt_tensor *output, const mt_tensor *input, float value);                                                  /* Mul(T,scalar) x2 :2291,:2326; CPU :721-782 */
+int mt_tensor_item_production(const mt_tensor *output, const mt_tensor *left, const mt_tensor *right);                           /* TensorItemProduction :2425; CPU :822-851 */
+int mt_clip(const mt_tensor *tensor, float min_value, float max_value);                                                          /* Clip :2834; CPU :1061-1084 */
+int mt_signum(const mt_tensor *tensor);                                                                                          /* Signum :2892; CPU :1090-1113 */
+int mt_add_value(const mt_tensor *output, const mt_tensor *input, float tensor_scale, float value);                              /* AddValue :985 (GPU class only) */
+int mt_sub_value(const mt_tensor *output, const mt_tensor *input, float tensor_scale, float value);                              /* SubValue :1061 (GPU class only) */
+int mt_set(const mt_tensor *output, const mt_tensor *input, float scale, float add_value);                                       /* Set :1128 (GPU class only) */
+
+/* ---- resampling and pooling: CTensorMath<T> ---- */
+int mt_upsampling(const mt_tensor *output, const mt_tensor *input, uint32_t upsampling_x, uint32_t upsampling_y);       /* UpSampling :2518; CPU :868-902 */
+int mt_downsampling(const mt_tensor *output, const mt_tensor *input, uint32_t downsampling_x, uint32_t downsampling_y); /* DownSampling :2600; CPU :908-949 (CPU edge rule kept) */
+int mt_max_pooling(const mt_tensor *output, const mt_pos_tensor *position, const mt_tensor *input, uint32_t pooling_x, uint32_t pooling_y);          /* MaxPooling :2693; CPU :955-1013 */
+int mt_max_pooling_backward(const mt_tensor *output, const mt_pos_tensor *position, const mt_tensor *input, uint32_t pooling_x, uint32_t pooling_y); /* MaxPoolingBackward :2767; CPU :1019-1055 */
+
+/* ---- optimiser: Adam, cuda/ctensormath.cu.h:2978-3022; CPU :1119-1165 (`iteration` used as passed, as on the CPU path) ---- */
+int mt_adam(const mt_tensor *weight, const mt_tensor *dweight, const mt_tensor *m, const mt_tensor *v, uint32_t batch_size,
+            double speed, double beta1, double beta2, double epsilon, double iteration);
+
+/* ---- activations: CTensorApplyFunc<T>::Apply* / ApplyDifferential* (cuda/ctensorapplyfunc.cu.h:297-866; CPU :261-629) ---- */
+int mt_apply_func(const mt_tensor *output, const mt_tensor *input, int func);
+
+/* ---- fused entry points -----------------------------------------------------------------------
+ * Each one is the exact op sequence of one reference layer's Forward(), lowered to fewer launches.
+ * They have no single counterpart function in the reference; the sequence each replaces is cited. */
+
+/* CNetLayerConvolution::Forward + CNetLayerFunction::Forward (netlayer/cnetlayerconvolution.cu.h:310-322,
+ * netlayer/cnetlayerfunction.cu.h:203-213): convolution, bias and activation `func` in one kernel. */
+int mt_forward_convolution_func(const mt_tensor *output, const mt_tensor *image, const mt_tensor *kernel,
+                                int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
+                                const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y, int func);
+/* CNetLayerBackConvolution::Forward + CNetLayerFunction::Forward (netlayer/cnetlayerbackconvolution.cu.h:303-315) */
+int mt_backward_convolution_func(const mt_tensor *output, const mt_tensor *delta, const mt_tensor *kernel,
+                                 int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
+                                 const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y, int func);
+/* CNetLayerLinear::Forward + CNetLayerFunction::Forward (netlayer/cnetlayerlinear.cu.h:262-282): output[B,1,Out,1] =
+ * func(weight[1,1,Out,In] * input[B,1,In,1] + bias[1,1,Out,1]); `input` may have any [B,Z,Y,X] with Z*Y*X == In. */
+int mt_linear_forward_func(const mt_tensor *output, const mt_tensor *weight, const mt_tensor *input, const mt_tensor *bias, int func);
+/* CNetLayerBatchNormalization::Forward in training mode followed by CNetLayerFunction::Forward
+ * (netlayer/cnetlayerbatchnormalization.cu.h:301-371): statistics per element (z,y,x) over the batch axis W.
+ * Writes output = func(gamma*xhat+beta); optionally xhat [B,Z,Y,X], ivar / batch mean / batch variance [1,Z,Y,X]
+ * (NULL to skip), and blends new_mean / new_variable with `momentum` as lines 311 and 324 do (NULL to skip). */
+int mt_batchnorm_forward_train_func(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
+                                    const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var,
+                                    const mt_tensor *new_mean, const mt_tensor *new_variable, float momentum, float epsilon, int func);
+/* The same layer in inference mode (lines 326-371): stored mean / variable instead of batch statistics. */
+int mt_batchnorm_forward_infer_func(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
+                                    const mt_tensor *mean, const mt_tensor *variable, float epsilon, int func);
+
+/* ---- timing: replaces CCUDATimeSpent / CTimeStamp (cuda/ccudatimespent.cu:38-52, cuda/ctimestamp.cu:17-32) ----
+ * While enabled, every kernel launch of the hot path is bracketed by two events on the work stream and its
+ * duration is accumulated under the kernel's label.  mt_profile_entries() waits for the stream and returns the
+ * number of labels seen since profiling was enabled; mt_profile_entry() reads one of them. */
+int mt_profile_enable(int on);
+int mt_profile_entries(void);
+int mt_profile_entry(int index, const char **label, uint64_t *launches, double *total_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,132 @@
+"""TEST INFRASTRUCTURE ONLY (checker side).
+
+The reference layers' Forward()/TrainingBackward() as literal sequences of tensor ops, written
+against the shared numpy API of oracle_api.Oracle and gpu_api.Gpu.  Running one sequence on both
+back ends is the "same op sequence on oracle vs GPU" parity check; the fused C-ABI entry points
+are compared with the oracle's literal sequence."""
+import numpy as np
+
+BN_EPSILON = 1e-6  # netlayer/cnetlayerbatchnormalization.cu.h:26
+
+
+def flat(x):
+    """ReinterpretSize(B,1,Z*Y*X,1) (netlayer/cnetlayerlinear.cu.h:268-271)."""
+    return np.ascontiguousarray(x).reshape(x.shape[0], 1, -1, 1)
+
+
+def linear_forward(lib, weight, x, bias):
+    """CNetLayerLinear::Forward, netlayer/cnetlayerlinear.cu.h:262-280: Mul then Add of the bias."""
+    h = lib.mul(weight, flat(x))
+    return lib.add(h, bias)
+
+
+def linear_backward(lib, weight, delta, h_prev):
+    """CNetLayerLinear::TrainingBackward, netlayer/cnetlayerlinear.cu.h:415-447.
+    Returns (previous layer error, dW, dB) starting from zero gradients."""
+    prev_err = lib.transponse_mul(weight, delta)
+    b = delta.shape[0]
+    tmp = lib.mul(delta, np.ascontiguousarray(h_prev).reshape(b, 1, 1, -1))          # per-sample outer products
+    zero_w = np.zeros((1, 1) + weight.shape[2:], np.float32)
+    dw = lib.add_sum_w(zero_w, tmp, out_init=zero_w)
+    zero_b = np.zeros((1, 1, weight.shape[2], 1), np.float32)
+    db = lib.add_sum_w(zero_b, delta, out_init=zero_b)
+    return prev_err, dw, db
+
+
+def function_forward(lib, x, func):
+    """CNetLayerFunction::Forward, netlayer/cnetlayerfunction.cu.h:203-213."""
+    return lib.apply_func(x, func)
+
+
+def batchnorm_forward_train(lib, x, gamma, beta, new_mean=None, new_var=None, momentum=0.9):
+    """CNetLayerBatchNormalization::Forward in training mode, netlayer/cnetlayerbatchnormalization.cu.h:301-371.
+    Statistics are per element (z,y,x) over the batch axis.  Returns a dict of every tensor the layer keeps."""
+    n = np.float32(x.shape[0])
+    inv_n = float(np.float32(1.0 / np.float64(n)))
+    zero = np.zeros((1,) + x.shape[1:], np.float32)
+    mean = lib.add_sum_w(zero, x, 1.0, inv_n, out_init=zero)                        # :308-309
+    res = {}
+    if new_mean is not None:
+        res["new_mean"] = lib.add(new_mean, mean, momentum, float(np.float32(1.0 - np.float64(np.float32(momentum)))))  # :311
+    xmu = lib.sub(x, mean, 1.0, 1.0)                                               # :315
+    sq = lib.pow2(xmu, 1.0)                                                        # :321
+    var = lib.add_sum_w(zero, sq, 1.0, inv_n, out_init=zero)                       # :322
+    if new_var is not None:
+        res["new_var"] = lib.add(new_var, var, momentum, float(np.float32(1.0 - np.float64(np.float32(momentum)))))     # :324
+    sqrtvar = lib.sqrt(var, 1.0, BN_EPSILON)                                       # :356
+    ivar = lib.inv(sqrtvar)                                                        # :359
+    xhat = lib.tensor_item_production(xmu, ivar)                                   # :363
+    gx = lib.tensor_item_production(gamma, xhat)                                   # :369
+    out = lib.add(gx, beta)                                                        # :371
+    res.update(out=out, xhat=xhat, ivar=ivar, mean=mean, var=var)
+    return res
+
+
+def batchnorm_forward_infer(lib, x, gamma, beta, mean, var):
+    """The same layer in inference mode, lines 326-371."""
+    xmu = lib.sub(x, mean, 1.0, 1.0)
+    ivar = lib.inv(lib.sqrt(var, 1.0, BN_EPSILON))
+    xhat = lib.tensor_item_production(xmu, ivar)
+    return lib.add(lib.tensor_item_production(gamma, xhat), beta)
+
+
+def batchnorm_backward(lib, delta, gamma, xhat, ivar):
+    """CNetLayerBatchNormalization::TrainingBackward, lines 578-604 (with create_delta_weight).
+    Returns (previous layer error, dGamma, dBeta) starting from zero gradients."""
+    n = np.float32(delta.shape[0])
+    zero = np.zeros((1,) + delta.shape[1:], np.float32)
+    dxhat = lib.tensor_item_production(delta, gamma)
+    s1 = lib.add_sum_w(zero, dxhat, out_init=zero)
+    s2 = lib.add_sum_w(zero, lib.tensor_item_production(dxhat, xhat), out_init=zero)
+    dgamma = lib.add_sum_w(zero, lib.tensor_item_production(delta, xhat), out_init=zero)
+    dbeta = lib.add_sum_w(zero, delta, out_init=zero)
+    err = lib.mul_value(dxhat, float(n))
+    err = lib.sub(err, lib.tensor_item_production(xhat, s2))
+    err = lib.sub(err, s1)
+    err = lib.tensor_item_production(err, ivar)
+    err = lib.mul_value(err, float(np.float32(1.0 / np.float64(n))))
+    return err, dgamma, dbeta
+
+
+def conv_forward(lib, x, kernel, bias, k, s, p):
+    """CNetLayerConvolution::Forward, netlayer/cnetlayerconvolution.cu.h:310-322."""
+    ka, c = kernel.shape[2], x.shape[1]
+    return lib.forward_convolution(x, kernel, bias, k, k, c, ka, s, s, p, p)
+
+
+def conv_backward(lib, x, kernel, delta, k, s, p):
+    """CNetLayerConvolution::TrainingBackward, netlayer/cnetlayerconvolution.cu.h:484-516: input delta with a zero
+    bias, per-sample gradients, then their sum over the batch.  Returns (previous layer error, dK, dB)."""
+    b, c, ka = x.shape[0], x.shape[1], kernel.shape[2]
+    zero_bias = np.zeros((1, ka, 1, 1), np.float32)
+    prev_err = lib.backward_convolution(delta, kernel, zero_bias, k, k, c, ka, s, s, p, p, x.shape)
+    dk_batch, db_batch = lib.create_delta_weight_and_bias(np.zeros((b, 1, ka, c * k * k), np.float32), np.zeros((b, ka, 1, 1), np.float32),
+                                                          x, delta, k, k, c, ka, s, s, p, p)
+    zk, zb = np.zeros((1, 1, ka, c * k * k), np.float32), np.zeros((1, ka, 1, 1), np.float32)
+    dk = lib.add_sum_w(zk, dk_batch, out_init=zk)
+    db = lib.add_sum_w(zb, db_batch, out_init=zb)
+    return prev_err, dk, db
+
+
+def backconv_forward(lib, x, kernel, bias, k, s, p, out_depth):
+    """CNetLayerBackConvolution::Forward, netlayer/cnetlayerbackconvolution.cu.h:303-315; output size
+    s*(in-1)+k-2p (lines 198-232).  kernel is [1,1,Cin,Cout*k*k]."""
+    b, cin, h, w = x.shape
+    oh, ow = s * (h - 1) + k - 2 * p, s * (w - 1) + k - 2 * p
+    return lib.backward_convolution(x, kernel, bias, k, k, out_depth, cin, s, s, p, p, (b, out_depth, oh, ow))
+
+
+def dcgan_generator_forward(lib, params, latent, channels=(512, 256, 128, 64, 3)):
+    """DCGAN-64 generator forward as a stack of the reference's layers: Linear, then four times
+    (BatchNorm in training mode, ReLU, transposed conv 4x4 stride 2 padding 1), tanh on the last output.
+    `params` uses the names of generator.make_parameters().  Returns every layer output."""
+    b = latent.shape[0]
+    h = linear_forward(lib, params["lin_w"], latent, params["lin_b"]).reshape(b, channels[0], 4, 4)
+    outs = {"h0": h}
+    for i in range(4):
+        bn = batchnorm_forward_train(lib, h, params["gamma%d" % i], params["beta%d" % i])["out"]
+        a = function_forward(lib, bn, "relu")
+        h = backconv_forward(lib, a, params["kernel%d" % i], params["bias%d" % i], 4, 2, 1, channels[i + 1])
+        outs["a%d" % i], outs["h%d" % (i + 1)] = a, h
+    outs["image"] = function_forward(lib, h, "tangence")
+    return outs

@@ -384,13 +384,13 @@ int oracle_signum(ot_tensor *t) {
   return ORACLE_OK;
 }
 
-/* cuda/ctensormath.cu.h:957-979 (kernel), 985-1015 (host) */
+/* cuda/ctensormath.cu.h:957-979 (kernel), :985 (host) */
 int oracle_add_value(ot_tensor *out, const ot_tensor *in, float tensor_scale, float value) {
   if (!same_zyx(in, out)) return ORACLE_E_SHAPE;
   UNARY_LOOP(i * tensor_scale + value)
   return ORACLE_OK;
 }
-/* cuda/ctensormath.cu.h:1060-1090 -- AddValue with the value negated */
+/* cuda/ctensormath.cu.h:1061 -- AddValue with the value negated */
 int oracle_sub_value(ot_tensor *out, const ot_tensor *in, float tensor_scale, float value) {
   return oracle_add_value(out, in, tensor_scale, -value);
 }

@@ -1,0 +1,90 @@
+"""The benchmark configurations through the C ABI: the DCGAN-64 generator (the measured workload) against
+the CPU oracle at a batch the oracle finishes in seconds, and at the full batch of 256 through
+size-independent properties; the Linear stack and the single-conv configuration at full size."""
+import numpy as np
+import pytest
+
+import layer_sequences as seq
+from cases import rng_normal as Nrm, rng_uniform as U
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-4  # max|gpu-cpu| / max|cpu| per tensor, fp32
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    from gpu_api import Gpu
+    return Gpu()
+
+
+def test_config1_single_conv_layer(gpu, oracle):
+    """16x3x64x64 uniform[-1,1], 32 filters 5x5x3 He-normal seed 1, bias 0, stride 1, padding 2, leaky ReLU."""
+    image = U(1, 16, 3, 64, 64)
+    kernel = Nrm(1, 1, 1, 32, 75, std=float(np.sqrt(2.0 / 75)))
+    bias = np.zeros((1, 32, 1, 1), np.float32)
+    want = oracle.apply_func(oracle.forward_convolution(image, kernel, bias, 5, 5, 3, 32, 1, 1, 2, 2), "leaky_relu")  # slope 0.1, the reference's
+    got = gpu.forward_convolution(image, kernel, bias, 5, 5, 3, 32, 1, 1, 2, 2, func="leaky_relu")
+    assert got.shape == (16, 32, 64, 64) and rel_err(got, want) <= REL
+    lit = gpu.apply_func(gpu.forward_convolution(image, kernel, bias, 5, 5, 3, 32, 1, 1, 2, 2), "leaky_relu")
+    assert rel_err(lit, want) <= REL
+
+
+def test_config2_linear_stack(gpu, oracle):
+    """Batch 256, 4096 -> 3072 -> ReLU -> 768, Xavier-uniform seed 2."""
+    x = Nrm(2, 256, 1, 4096, 1)
+    w1 = U(3, 1, 1, 3072, 4096, lo=-np.sqrt(6 / 7168), hi=np.sqrt(6 / 7168))
+    w2 = U(4, 1, 1, 768, 3072, lo=-np.sqrt(6 / 3840), hi=np.sqrt(6 / 3840))
+    b1, b2 = np.full((1, 1, 3072, 1), 0.1, np.float32), np.full((1, 1, 768, 1), 0.1, np.float32)
+    h = oracle.apply_func(seq.linear_forward(oracle, w1, x, b1), "relu")
+    want = seq.linear_forward(oracle, w2, h, b2)
+    got = gpu.linear_forward(w2, gpu.linear_forward(w1, x, b1, func="relu"), b2)
+    assert got.shape == (256, 1, 768, 1) and rel_err(got, want) <= REL
+    lit = seq.linear_forward(gpu, w2, gpu.apply_func(seq.linear_forward(gpu, w1, x, b1), "relu"), b2)
+    assert rel_err(lit, want) <= REL
+
+
+def test_config3_generator_against_oracle(gpu, oracle):
+    """DCGAN-64 generator forward, every layer output, batch 8 (the oracle needs ~0.2 GFLOP per image)."""
+    import generator as G
+    params, z = G.make_parameters(), G.make_latent(8)
+    want = seq.dcgan_generator_forward(oracle, params, z)
+    net = G.DcganGenerator(8, params)
+    net.set_latent(z)
+    for forward in (net.forward_fused, net.forward_literal):
+        forward()
+        assert rel_err(net.h[0].numpy(), want["h0"]) <= REL
+        for i in range(4):
+            assert rel_err(net.a[i].numpy(), want["a%d" % i]) <= REL, "a%d" % i
+            if i < 3:
+                assert rel_err(net.h[i + 1].numpy(), want["h%d" % (i + 1)]) <= REL, "h%d" % (i + 1)
+        image = net.output.numpy()
+        assert image.shape == (8, 3, 64, 64) and rel_err(image, want["image"]) <= REL
+
+
+def test_config3_full_batch_properties(gpu, oracle):
+    """Batch 256: (1) the fused and the literal op sequences agree; (2) the transposed convolutions are linear and
+    per-sample independent, so any sample of the big batch equals the same sample run alone through the oracle."""
+    import generator as G
+    params, z = G.make_parameters(), G.make_latent(256)
+    net = G.DcganGenerator(256, params)
+    net.set_latent(z)
+    fused = net.forward_fused().numpy()
+    a = [t.numpy() for t in net.a]
+    h = [t.numpy() for t in net.h[:4]]
+    literal = net.forward_literal().numpy()
+    assert fused.shape == (256, 3, 64, 64) and np.all(np.isfinite(fused)) and np.all(np.abs(fused) <= 1)
+    assert rel_err(fused, literal) <= REL
+    for i in range(4):
+        # batch-norm output before ReLU has zero mean and unit variance over the batch, per element
+        x = h[i].astype(np.float64)
+        xhat = (x - x.mean(0)) / np.sqrt(x.var(0) + G.BN_EPSILON)
+        assert rel_err(a[i], np.maximum(xhat, 0)) <= REL
+    for i, sample in ((0, 255), (1, 17), (2, 100), (3, 3)):
+        cin, cout = G.CHANNELS[i], G.CHANNELS[i + 1]
+        want = seq.backconv_forward(oracle, a[i][sample:sample + 1], params["kernel%d" % i], params["bias%d" % i], 4, 2, 1, cout)
+        got = h[i + 1][sample:sample + 1] if i < 3 else None
+        if i == 3:
+            want, got = oracle.apply_func(want, "tangence"), fused[sample:sample + 1]
+        assert rel_err(got, want) <= REL, "layer %d" % i
