@@ -102,12 +102,20 @@ def main():
     conv_ms = sum(v[1] for v in conv_kernels.values()) / args.steps
     conv_tflops = sum(flops) / (conv_ms * 1e-3) / 1e12
 
-    # dominant kernel: the implicit GEMM of the three large layers (12 launches per step, 2*256*512*16*256*4/4 FLOP each)
-    big = [(k, v) for k, v in conv_kernels.items() if "32x128" not in k and "direct" not in k]
-    dom_label = max(big, key=lambda kv: kv[1][1])[0] if big else None
-    dom_launches = sum(v[0] for _, v in big)
-    dom_ms = sum(v[1] for _, v in big)
-    flop_per_launch = sum(flops[:3]) / 12.0
+    # dominant kernel: the matrix-core implicit GEMM of the three large layers.  Its label carries the GEMM shape
+    # "M<Cout> N<batch*pixels per phase> K<Cin*taps> x<phases>", i.e. 2*M*N*K*phases algorithmic FLOP per launch
+    # (= 2*B*Cin*Hin*Win*Cout*16 of the layer: every phase multiplies only its own non-zero taps).
+    import re
+    big = []
+    for k, v in conv_kernels.items():
+        m = re.search(r"M(\d+) N(\d+) K(\d+) x(\d+)", k)
+        if m:
+            M_, N_, K_, X_ = (int(g) for g in m.groups())
+            big.append((k, v[0], v[1], 2.0 * M_ * N_ * K_ * X_))
+    dom_label = big[0][0].split(" M")[0] if big else None
+    dom_launches = sum(b[1] for b in big)
+    dom_ms = sum(b[2] for b in big)
+    flop_per_launch = sum(b[1] * b[3] for b in big) / dom_launches if dom_launches else 0.0
     achieved = flop_per_launch / (dom_ms / dom_launches * 1e-3) / 1e12 if dom_launches else 0.0
 
     result = {
@@ -133,7 +141,8 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None, "kernel": dom_label,
                      "launches_per_step": dom_launches / args.steps, "avg_launch_ms": dom_ms / dom_launches if dom_launches else None,
-                     "flop_per_launch": flop_per_launch},
+                     "flop_per_launch": flop_per_launch,
+                     "per_layer": {b[0]: {"avg_launch_ms": b[2] / b[1], "tflops": b[3] / (b[2] / b[1] * 1e-3) / 1e12} for b in big}},
         "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])},
     }
     if not args.no_cpu_baseline:

@@ -21,6 +21,19 @@ int g_conv_path = 0;  // 0 auto, 1 direct, 2 implicit GEMM wherever it applies
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
+// Calls f with a row-major, k-contiguous source; 128-bit loads when the layout allows them.
+template <class F>
+int with_row_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, Batch bt, F &&f) {
+  if (ld % 4 == 0 && K % 4 == 0 && aligned16(p) && bt.stride % 4 == 0) {
+    SrcRowK<true> s{};
+    s.p = p; s.ld = ld; s.R = R; s.K = K; s.bt = bt;
+    return f(s);
+  }
+  SrcRowK<false> s{};
+  s.p = p; s.ld = ld; s.R = R; s.K = K; s.bt = bt;
+  return f(s);
+}
+
 // ---- library-owned workspace: packed phase kernels and bias sums of the transposed convolution ----------------
 float *g_ws = nullptr;
 size_t g_ws_floats = 0;
@@ -160,23 +173,110 @@ Phase1D phase_1d(int32_t ph, int32_t K, int32_t s, int32_t p, int32_t O) {
   return r;
 }
 
-// packed[co][(ci, ty, tx)] = kernel[ci][co*KY*KX + (KY-1-(ky0+ty*sy))*KX + (KX-1-(kx0+tx*sx))]
-__global__ __launch_bounds__(256) void pack_phase_kernel(float *packed, const float *kernel, uint32_t ker_ld, int32_t CO, int32_t CI, int32_t KY, int32_t KX,
-                                                         int32_t SY, int32_t SX, int32_t ky0, int32_t kx0, int32_t TY, int32_t TX) {
-  uint32_t idx = blockIdx.x * 256 + threadIdx.x;
-  uint32_t kp = CI * TY * TX;
-  if (idx >= (uint32_t)CO * kp) return;
-  uint32_t co = idx / kp, k = idx % kp, ci = k / (TY * TX), t = k % (TY * TX), ty = t / TX, tx = t % TX;
-  int32_t ky = ky0 + ty * SY, kx = kx0 + tx * SX;
-  packed[idx] = kernel[(size_t)ci * ker_ld + co * KY * KX + (KY - 1 - ky) * KX + (KX - 1 - kx)];
+// One launch prepares a transposed convolution: blockIdx.y < nphase packs that phase's sub-kernel,
+//   packed_f[co][(ci, ty, tx)] = kernel[ci][co*KY*KX + (KY-1-(ky0+ty*sy))*KX + (KX-1-(kx0+tx*sx))],
+// and blockIdx.y == nphase sums the biases of every bias layer (the CPU path adds all of them per tap).
+struct PackPhase {
+  uint32_t begin, kp, ld;  // offset of the phase in the packed buffer (floats), coefficients per row, padded row length
+  int32_t ky0, kx0, ty, tx;
+};
+struct PackArgs {
+  PackPhase ph[MAX_PHASES];
+  uint32_t nphase, ker_ld, bias_w;
+  int32_t CO, CI, KY, KX, SY, SX;
+};
+__global__ __launch_bounds__(256) void tconv_prepare_kernel(float *packed, float *sums, const float *kernel, const float *bias, PackArgs pa) {
+  if (blockIdx.y == pa.nphase) {
+    uint32_t wave = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x % 64, waves = gridDim.x * 4;
+    for (uint32_t w = wave; w < pa.bias_w; w += waves) {
+      float acc = 0.f;
+      for (uint32_t i = lane; i < (uint32_t)pa.CI; i += 64) acc += bias[(size_t)w * pa.CI + i];
+      acc = mt::wave_sum(acc);
+      if (lane == 0) sums[w] = acc;
+    }
+    return;
+  }
+  const PackPhase ph = pa.ph[blockIdx.y];
+  const uint32_t taps = ph.ty * ph.tx, total = (uint32_t)pa.CO * ph.ld;
+  for (uint32_t idx = blockIdx.x * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
+    uint32_t co = idx / ph.ld, k = idx % ph.ld;
+    float v = 0.f;  // rows are zero-padded to a multiple of four coefficients
+    if (k < ph.kp) {
+      uint32_t ci = k / taps, t = k % taps, ty = t / ph.tx, tx = t % ph.tx;
+      int32_t ky = ph.ky0 + ty * pa.SY, kx = ph.kx0 + tx * pa.SX;
+      v = kernel[(size_t)ci * pa.ker_ld + co * pa.KY * pa.KX + (pa.KY - 1 - ky) * pa.KX + (pa.KX - 1 - kx)];
+    }
+    packed[ph.begin + idx] = v;
+  }
 }
 
-__global__ __launch_bounds__(64) void bias_sum_kernel(float *sums, const float *bias, uint32_t KA) {
-  const float *b = bias + (size_t)blockIdx.x * KA;
-  float s = 0.f;
-  for (uint32_t i = threadIdx.x; i < KA; i += 64) s += b[i];
-  s = mt::wave_sum(s);
-  if (threadIdx.x == 0) sums[blockIdx.x] = s;
+// ---- transposed convolution with very few output channels (the image-producing last layer) --------------------
+// A 32-row matrix-core tile would be 90% padding for 3 output channels, so this case runs on the vector ALUs:
+// one thread per output pixel of one stride phase (blockIdx.y), CO accumulators, the packed sub-kernel read
+// through the scalar cache (its address is uniform), the delta read with lanes along x (coalesced, neighbours
+// share cache lines).  TY/TX = 0 means "tap counts known only at run time".
+template <int CO, int TY, int TX>
+__global__ __launch_bounds__(256) void tconv_small_kernel(TconvArgs args) {
+  const TconvPhase ph = args.ph[blockIdx.y];
+  const uint32_t qhw = ph.qh * ph.qw, N = args.out_w * qhw;
+  const uint32_t n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  const int ty_cnt = TY ? TY : ph.taps_y, tx_cnt = TX ? TX : ph.taps_x;
+  const uint32_t g = n / qhw, r = n % qhw, qy = r / ph.qw, qx = r % ph.qw;
+  const uint32_t H = args.H, W = args.W, C = args.C;
+  const float *in = args.delta + (size_t)(g % args.in_w) * C * H * W;
+  const int32_t y0 = (int32_t)qy + ph.offy, x0 = (int32_t)qx + ph.offx;
+  float acc[CO];
+#pragma unroll
+  for (int co = 0; co < CO; co++) acc[co] = 0.f;
+  const uint32_t taps = ty_cnt * tx_cnt;
+  for (uint32_t ci = 0; ci < C; ci++) {
+    const float *plane = in + (size_t)ci * H * W;
+    const float *wrow = ph.packed + ci * taps;
+#pragma unroll
+    for (int ty = 0; ty < (TY ? TY : 4); ty++) {
+      if (!TY && ty >= ty_cnt) break;
+      const int32_t iy = y0 + ty;
+      const bool yok = (uint32_t)iy < H;
+#pragma unroll
+      for (int tx = 0; tx < (TX ? TX : 4); tx++) {
+        if (!TX && tx >= tx_cnt) break;
+        const int32_t ix = x0 + tx;
+        const bool ok = yok && (uint32_t)ix < W;
+        const float v = ok ? plane[(size_t)(ok ? iy : 0) * W + (ok ? ix : 0)] : 0.f;
+#pragma unroll
+        for (int co = 0; co < CO; co++)
+          if (co < (int)args.M) acc[co] = __builtin_fmaf(wrow[(size_t)co * ph.ld + ty * tx_cnt + tx], v, acc[co]);
+      }
+    }
+  }
+  Epilogue ep = args.ep;
+  ep.inner = qhw; ep.qw = ph.qw; ep.py = ph.py; ep.px = ph.px;
+  ep.ty_cnt = ph.taps_y; ep.tx_cnt = ph.taps_x; ep.offy = ph.offy; ep.offx = ph.offx;
+  Epilogue::Col col = ep.column(n);
+#pragma unroll
+  for (int co = 0; co < CO; co++)
+    if (co < (int)args.M) ep.store(col, co, acc[co]);
+}
+
+int launch_tconv_small(const char *name, TconvArgs &args, uint32_t max_n) {
+  mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "vector ALU, few output channels") : name);
+  dim3 grid(cdiv(max_n, 256), args.nphase);
+  bool t22 = true, small = true;
+  for (uint32_t f = 0; f < args.nphase; f++) {
+    t22 = t22 && args.ph[f].taps_y == 2 && args.ph[f].taps_x == 2;
+    small = small && args.ph[f].taps_y <= 4 && args.ph[f].taps_x <= 4;
+  }
+  if (!small) return -1;  // caller falls back to the matrix-core path
+  if (t22) {
+    if (args.M <= 2) tconv_small_kernel<2, 2, 2><<<grid, 256, 0, mt::stream()>>>(args);
+    else tconv_small_kernel<4, 2, 2><<<grid, 256, 0, mt::stream()>>>(args);
+  } else {
+    if (args.M <= 2) tconv_small_kernel<2, 0, 0><<<grid, 256, 0, mt::stream()>>>(args);
+    else tconv_small_kernel<4, 0, 0><<<grid, 256, 0, mt::stream()>>>(args);
+  }
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
 }
 
 // ---- argument checks shared by the plain and the fused entry points ---------------------------------------------
@@ -218,8 +318,6 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
     return MT_OK;
   }
   uint32_t OHW = out->y * out->x;
-  SrcRowK a{};
-  a.p = kernel->p; a.ld = kernel->x; a.R = ka; a.K = K; a.vec = (kernel->x % 4 == 0) && aligned16(kernel->p);
   SrcIm2col b{};
   b.p = image->p; b.in_w = image->w; b.C = kz; b.H = image->y; b.W = image->x; b.KY = ky; b.KX = kx; b.OHW = OHW; b.OW = out->x; b.K = K;
   b.sy = sy; b.sx = sx; b.py = py; b.px = px;
@@ -228,13 +326,21 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
   ep.bias = bias->p; ep.bias_mode = 1; ep.bias_w = bias->w; ep.bias_stride = ka; ep.func = func;
   if (kernel->w == 1) {  // one kernel set for the whole batch: fold the batch into the columns
     b.R = out->w * OHW;
-    return launch(name, a, b, ep, ka, out->w * OHW, K, 1);
+    const uint32_t taps = (uint32_t)ky * kx;
+    if (BK % taps == 0 && (uint32_t)kz % (BK / taps) == 0) {  // taps tile the k step: offsets precomputed per thread
+      SrcIm2colFixed bf{};
+      bf.p = b.p; bf.in_w = b.in_w; bf.C = b.C; bf.H = b.H; bf.W = b.W; bf.KY = b.KY; bf.KX = b.KX; bf.OHW = b.OHW; bf.OW = b.OW; bf.R = b.R; bf.K = b.K;
+      bf.sy = sy; bf.sx = sx; bf.py = py; bf.px = px;
+      return with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return launch(name, a, bf, ep, ka, out->w * OHW, K, 1); });
+    }
+    return with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return launch(name, a, b, ep, ka, out->w * OHW, K, 1); });
   }
   // kernels differ per sample: one product per output image
-  a.bt.wmod = kernel->w; a.bt.stride = (size_t)kernel->z * kernel->y * kernel->x;
+  Batch abt;
+  abt.wmod = kernel->w; abt.stride = (size_t)kernel->z * kernel->y * kernel->x;
   b.bt.wmod = image->w; b.bt.stride = (size_t)kz * image->y * image->x; b.in_w = 1; b.R = OHW;
   ep.bt.wmod = out->w; ep.bt.stride = (size_t)ka * OHW;
-  return launch(name, a, b, ep, ka, OHW, K, out->w);
+  return with_row_k(kernel->p, kernel->x, ka, K, abt, [&](auto a) { return launch(name, a, b, ep, ka, OHW, K, out->w); });
 }
 
 int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
@@ -260,16 +366,16 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     return MT_OK;
   }
 
-  // workspace: [bias sums (bias_w, padded to 64)] [packed kernels of all phases: kz*ka*ky*kx floats]
+  // workspace: [bias sums (bias_w, padded to 64)] [packed sub-kernels of all phases: kz*ka*ky*kx floats + alignment]
   size_t sums = (bias->w + 63u) & ~(size_t)63u;
   float *ws = nullptr;
-  if ((rc = workspace(sums + (size_t)kz * ka * ky * kx + 64, &ws))) return rc;
-  {
-    mt::ProfileScope prof("tconv_bias_sum");
-    bias_sum_kernel<<<bias->w, 64, 0, mt::stream()>>>(ws, bias->p, ka);
-  }
-  MT_LAUNCH_CHECK("bias_sum");
+  if ((rc = workspace(sums + (size_t)kz * ka * ky * kx + (size_t)4 * kz * sy * sx + 64, &ws))) return rc;
   float *packed = ws + sums;
+
+  TconvArgs args{};
+  PackArgs pa{};
+  pa.ker_ld = kernel->x; pa.bias_w = bias->w; pa.CO = kz; pa.CI = ka; pa.KY = ky; pa.KX = kx; pa.SY = sy; pa.SX = sx;
+  uint32_t max_n = 0, max_pack = 0, begin = 0;
   const uint32_t OHW = out->y * out->x;
   for (int32_t phy = 0; phy < sy; phy++) {
     Phase1D Y = phase_1d(phy, ky, sy, py, out->y);
@@ -277,28 +383,34 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     for (int32_t phx = 0; phx < sx; phx++) {
       Phase1D X = phase_1d(phx, kx, sx, px, out->x);
       if (X.q == 0) continue;
-      uint32_t kp = ka * Y.taps * X.taps;
-      if (kp) {
-        mt::ProfileScope prof("tconv_pack_phase");
-        pack_phase_kernel<<<cdiv((size_t)kz * kp, 256), 256, 0, mt::stream()>>>(packed, kernel->p, kernel->x, kz, ka, ky, kx, sy, sx, Y.k0, X.k0, Y.taps, X.taps);
-        MT_LAUNCH_CHECK("pack_phase");
-      }
-      SrcRowK a{};
-      a.p = packed; a.ld = kp; a.R = kz; a.K = kp; a.vec = (kp % 4 == 0) && aligned16(packed);
-      SrcIm2col b{};
-      uint32_t QHW = (uint32_t)Y.q * X.q;
-      b.p = delta->p; b.in_w = delta->w; b.C = ka; b.H = delta->y; b.W = delta->x; b.KY = Y.taps ? Y.taps : 1; b.KX = X.taps ? X.taps : 1;
-      b.OHW = QHW; b.OW = X.q; b.R = out->w * QHW; b.K = kp; b.sy = 1; b.sx = 1; b.py = -Y.off; b.px = -X.off;
-      Epilogue ep{};
-      ep.C = out->p; ep.row_stride = OHW; ep.inner = QHW; ep.g_stride = (size_t)kz * OHW;
-      ep.qw = X.q; ep.sy = sy; ep.sx = sx; ep.py = phy; ep.px = phx; ep.OW = out->x;
-      ep.tap_bias = ws; ep.bias_w = bias->w; ep.ty_cnt = Y.taps; ep.tx_cnt = X.taps; ep.offy = Y.off; ep.offx = X.off; ep.IH = delta->y; ep.IW = delta->x;
-      ep.func = func;
-      if ((rc = launch(name, a, b, ep, kz, out->w * QHW, kp, 1))) return rc;
-      packed += ((size_t)kz * kp + 3) & ~(size_t)3;  // keep every phase 16-byte aligned
+      uint32_t kp = ka * Y.taps * X.taps, ld = (kp + 3u) & ~3u, f = args.nphase++;
+      pa.ph[f] = PackPhase{begin, kp, ld, Y.k0, X.k0, Y.taps, X.taps};
+      args.ph[f] = TconvPhase{packed + begin, kp, ld, (uint32_t)Y.q, (uint32_t)X.q, Y.taps, X.taps, Y.off, X.off, (uint32_t)phy, (uint32_t)phx};
+      begin += (uint32_t)kz * ld;  // a multiple of four floats: every phase starts 16-byte aligned
+      uint32_t n = out->w * Y.q * X.q;
+      if (n > max_n) max_n = n;
+      if ((uint32_t)kz * ld > max_pack) max_pack = (uint32_t)kz * ld;
     }
   }
-  return MT_OK;
+  pa.nphase = args.nphase;
+  {
+    mt::ProfileScope prof("tconv_prepare");
+    unsigned gx = cdiv(max_pack ? max_pack : 1, 256 * 4);
+    if (gx > 1024) gx = 1024;
+    tconv_prepare_kernel<<<dim3(gx ? gx : 1, args.nphase + 1), 256, 0, mt::stream()>>>(packed, ws, kernel->p, bias->p, pa);
+    MT_LAUNCH_CHECK("tconv_prepare");
+  }
+  args.M = kz; args.out_w = out->w;
+  args.delta = delta->p; args.in_w = delta->w; args.C = ka; args.H = delta->y; args.W = delta->x;
+  args.ep.C = out->p; args.ep.row_stride = OHW; args.ep.g_stride = (size_t)kz * OHW;
+  args.ep.sy = sy; args.ep.sx = sx; args.ep.OW = out->x;
+  args.ep.tap_bias = ws; args.ep.bias_w = bias->w; args.ep.IH = delta->y; args.ep.IW = delta->x;
+  args.ep.func = func;
+  if (kz <= 4 && mt::igemm::tile_override() < 0) {
+    rc = launch_tconv_small(name, args, max_n);
+    if (rc >= 0) return rc;
+  }
+  return launch_tconv(name, args, max_n);
 }
 
 int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
@@ -322,16 +434,15 @@ int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t
     wgrad_direct_kernel<<<cdiv(total, 256), 256, 0, mt::stream()>>>(dk->p, image->p, delta->p, g, delta->w, delta->y, delta->x, total);
     MT_LAUNCH_CHECK(name);
   } else {
-    SrcRowK a{};
-    a.p = delta->p; a.ld = DHW; a.R = ka; a.K = DHW; a.vec = (DHW % 4 == 0) && aligned16(delta->p);
-    a.bt.wmod = delta->w; a.bt.stride = (size_t)ka * DHW;
+    Batch abt;
+    abt.wmod = delta->w; abt.stride = (size_t)ka * DHW;
     SrcWgradImage b{};
-    b.p = image->p; b.H = image->y; b.W = image->x; b.KY = ky; b.KX = kx; b.OW = delta->x; b.R = ncol; b.K = DHW; b.sy = sy; b.sx = sx; b.py = py; b.px = px;
+    b.p = image->p; b.C = kz; b.H = image->y; b.W = image->x; b.KY = ky; b.KX = kx; b.OW = delta->x; b.R = ncol; b.K = DHW; b.sy = sy; b.sx = sx; b.py = py; b.px = px;
     b.bt.wmod = image->w; b.bt.stride = (size_t)kz * image->y * image->x;
     Epilogue ep{};
     ep.C = dk->p; ep.row_stride = dk->x; ep.inner = ncol; ep.g_stride = 0; ep.accumulate = true;
     ep.bt.wmod = dk->w; ep.bt.stride = (size_t)dk->z * dk->y * dk->x;
-    if ((rc = launch(name, a, b, ep, ka, ncol, DHW, dk->w))) return rc;
+    if ((rc = with_row_k(delta->p, DHW, ka, DHW, abt, [&](auto a) { return launch(name, a, b, ep, ka, ncol, DHW, dk->w); }))) return rc;
   }
   if (!bias_too) return MT_OK;
   if (db->y != 1 || db->x != 1) return mt::fail(MT_E_ARGUMENT, "%s: bias gradient must be [W,Z,1,1]", name);
@@ -349,6 +460,17 @@ int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t
 }  // namespace
 
 namespace mt {
+namespace igemm {
+int &tile_override() {
+  static int v = -1;
+  return v;
+}
+}  // namespace igemm
+int set_igemm_tile(int v) {
+  if (v < -1 || v > 3) return fail(MT_E_ARGUMENT, "igemm_tile must be -1 (auto) or 0..3");
+  igemm::tile_override() = v;
+  return MT_OK;
+}
 int set_conv_path(int v) {
   if (v < 0 || v > 2) return fail(MT_E_ARGUMENT, "conv_path must be 0 (auto), 1 (direct) or 2 (matrix cores)");
   g_conv_path = v;

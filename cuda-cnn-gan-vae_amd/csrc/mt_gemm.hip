@@ -14,15 +14,22 @@ using namespace mt::igemm;
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
-SrcRowK row_k(const float *p, uint32_t ld, uint32_t R, uint32_t K) {
-  SrcRowK s{};
-  s.p = p; s.ld = ld; s.R = R; s.K = K;
-  s.vec = (ld % 4 == 0) && aligned16(p);
-  return s;
+// Calls f with a row-major, k-contiguous source; 128-bit loads when the layout allows them.
+template <class F>
+int with_row_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, Batch bt, F &&f) {
+  if (ld % 4 == 0 && K % 4 == 0 && aligned16(p) && bt.stride % 4 == 0) {
+    SrcRowK<true> s{};
+    s.p = p; s.ld = ld; s.R = R; s.K = K; s.bt = bt;
+    return f(s);
+  }
+  SrcRowK<false> s{};
+  s.p = p; s.ld = ld; s.R = R; s.K = K; s.bt = bt;
+  return f(s);
 }
 SrcColK col_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, uint32_t inner, size_t gstride) {
   SrcColK s{};
   s.p = p; s.ld = ld; s.R = R; s.K = K; s.inner = inner; s.gstride = gstride;
+  s.groups = inner ? (R + inner - 1) / inner : 1;
   return s;
 }
 
@@ -42,27 +49,30 @@ int product(const char *name, const mt_tensor *out, const mt_tensor *left, const
   ep.C = out->p;
   ep.func = func;
   const bool fold_ok = Z == 1 && W > 1;
+  const Batch none{};
 
   if (fold_ok && left->w == 1 && right->w >= W) {
     if (N == 1) {
       // C'[w][m] = sum_k B[w][k] * op(A)[m][k]: rows are batch entries, columns are the output rows m
       ep.row_stride = M; ep.inner = M; ep.g_stride = 0;
       if (bias) { ep.bias = bias; ep.bias_mode = 2; }
-      SrcRowK a = row_k(right->p, K, W, K);
-      if (ta) return launch(name, a, col_k(left->p, M, M, K, M, 0), ep, W, M, K, 1);
-      return launch(name, a, row_k(left->p, K, M, K), ep, W, M, K, 1);
+      return with_row_k(right->p, K, W, K, none, [&](auto a) {
+        if (ta) return launch(name, a, col_k(left->p, M, M, K, M, 0), ep, W, M, K, 1);
+        return with_row_k(left->p, K, M, K, none, [&](auto b) { return launch(name, a, b, ep, W, M, K, 1); });
+      });
     }
     // one product with N' = W*N columns; column n' = (w, n)
     ep.row_stride = N; ep.inner = N; ep.g_stride = (size_t)M * N;
     if (bias) { ep.bias = bias; ep.bias_mode = 1; }
     SrcColK b = col_k(right->p, N, W * N, K, N, (size_t)K * N);
     if (ta) return launch(name, col_k(left->p, M, M, K, M, 0), b, ep, M, W * N, K, 1);
-    return launch(name, row_k(left->p, K, M, K), b, ep, M, W * N, K, 1);
+    return with_row_k(left->p, K, M, K, none, [&](auto a) { return launch(name, a, b, ep, M, W * N, K, 1); });
   }
   if (fold_ok && right->w == 1 && left->w >= W && !ta && !bias) {
     // rows (w, m) of A and of C are contiguous: one product with M' = W*M rows
     ep.row_stride = N; ep.inner = N; ep.g_stride = 0;
-    return launch(name, row_k(left->p, K, W * M, K), col_k(right->p, N, N, K, N, 0), ep, W * M, N, K, 1);
+    SrcColK b = col_k(right->p, N, N, K, N, 0);
+    return with_row_k(left->p, K, W * M, K, none, [&](auto a) { return launch(name, a, b, ep, W * M, N, K, 1); });
   }
 
   // general case: one product per (w, z)
@@ -76,9 +86,9 @@ int product(const char *name, const mt_tensor *out, const mt_tensor *left, const
     a.bt.wmod = left->w; a.bt.zcount = Z; a.bt.stride = (size_t)K * M;
     return launch(name, a, b, ep, M, N, K, W * Z);
   }
-  SrcRowK a = row_k(left->p, K, M, K);
-  a.bt.wmod = left->w; a.bt.zcount = Z; a.bt.stride = (size_t)M * K;
-  return launch(name, a, b, ep, M, N, K, W * Z);
+  Batch abt;
+  abt.wmod = left->w; abt.zcount = Z; abt.stride = (size_t)M * K;
+  return with_row_k(left->p, K, M, K, abt, [&](auto a) { return launch(name, a, b, ep, M, N, K, W * Z); });
 }
 
 }  // namespace

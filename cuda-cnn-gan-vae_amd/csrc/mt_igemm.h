@@ -13,6 +13,8 @@
 //    rows of one k (coalesced NCHW rows); for k-contiguous sources each thread reads a 16/32-byte vector.
 #pragma once
 
+#include <type_traits>
+
 #include "mt_common.h"
 
 namespace mt {
@@ -33,39 +35,73 @@ struct Batch {
   }
 };
 
-// element(row, k) = p[row*ld + k]: k contiguous (weights [M][K], Linear activations [B][In])
+// ---- operand sources ----------------------------------------------------------------------------------------
+// Every source reads through a raw buffer descriptor (buffer_load_dword / _dwordx4).  The hardware range check
+// returns 0 for a lane whose byte offset is >= the buffer size, so "outside the operand" is encoded as the offset
+// OOB and costs no compare-and-select after the load and no branch around it: the loop body is straight-line
+// code and the loads of the next tile stay in flight behind the matrix instructions of the current one.
+// The scalar offset operand (uniform over the wavefront) carries what advances from tile to tile.
+// Operands must be smaller than 2 GiB (checked on the host); OOB plus any in-range offset stays out of range.
+//
+// Protocol:  bind(row) once per thread;  seek<E>(k) position at the thread's first k;  fetch<E>(v) load E
+// consecutive k;  next() advance by BK.
+constexpr uint32_t OOB = 0x80000000u;
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float *p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0));
+}
+__device__ __forceinline__ floatx2 buf_load2(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(floatx2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0));
+}
+__device__ __forceinline__ floatx4 buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
+}
+
+// element(row, k) = p[row*ld + k]: k contiguous (weights [M][K], Linear activations [B][In]).
+// VEC: ld % 4 == 0, K % 4 == 0 and p 16-byte aligned, so every aligned group of 4 (or 2) k is all real or all padding.
+template <bool VEC>
 struct SrcRowK {
   static constexpr bool K_CONTIG = true;
   const float *p;
   uint32_t ld, R, K;
-  bool vec;  // ld % 4 == 0 and p 16-byte aligned: vector loads allowed
   Batch bt;
-  const float *rowp;
-  bool rowok;
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff, kthread, ktile;
   __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
   __device__ void bind(uint32_t row) {
-    rowok = row < R;
-    rowp = p + (size_t)(rowok ? row : 0) * ld;
+    rsrc = make_rsrc(p, R * ld * 4u);
+    voff = row < R ? row * ld * 4u : OOB;
   }
   template <int E>
-  __device__ void fetch(uint32_t k0, float (&v)[E]) const {
-    if (rowok && vec && k0 + E <= K) {
-      if constexpr (E % 4 == 0) {
+  __device__ void seek(uint32_t k0) {
+    kthread = k0;
+    ktile = 0;
+    if (voff != OOB) voff += k0 * 4u;
+  }
+  __device__ void next() { ktile += BK; }
+  template <int E>
+  __device__ void fetch(float (&v)[E]) const {
+    const uint32_t soff = ktile * 4u, k = kthread + ktile;
+    if constexpr (VEC && E % 4 == 0) {
 #pragma unroll
-        for (int i = 0; i < E; i += 4) {
-          float4 t = *reinterpret_cast<const float4 *>(rowp + k0 + i);
-          v[i] = t.x; v[i + 1] = t.y; v[i + 2] = t.z; v[i + 3] = t.w;
-        }
-      } else {
+      for (int i = 0; i < E; i += 4) {
+        floatx4 t = buf_load4(rsrc, k + i + 4 <= K ? voff + i * 4u : OOB, soff);
+        v[i] = t.x; v[i + 1] = t.y; v[i + 2] = t.z; v[i + 3] = t.w;
+      }
+    } else if constexpr (VEC) {
 #pragma unroll
-        for (int i = 0; i < E; i += 2) {
-          float2 t = *reinterpret_cast<const float2 *>(rowp + k0 + i);
-          v[i] = t.x; v[i + 1] = t.y;
-        }
+      for (int i = 0; i < E; i += 2) {
+        floatx2 t = buf_load2(rsrc, k + i + 2 <= K ? voff + i * 4u : OOB, soff);
+        v[i] = t.x; v[i + 1] = t.y;
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < E; i++) v[i] = (rowok && k0 + i < K) ? rowp[k0 + i] : 0.f;
+      for (int i = 0; i < E; i++) v[i] = buf_load(rsrc, k + i < K ? voff + i * 4u : OOB, soff);
     }
   }
 };
@@ -75,56 +111,124 @@ struct SrcRowK {
 struct SrcColK {
   static constexpr bool K_CONTIG = false;
   const float *p;
-  uint32_t ld, R, K, inner;
+  uint32_t ld, R, K, inner, groups;  // groups = number of folded matrices (1 when not folded)
   size_t gstride;
   Batch bt;
-  const float *rowp;
-  bool rowok;
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff, k;
   __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
   __device__ void bind(uint32_t row) {
-    rowok = row < R;
-    uint32_t r = rowok ? row : 0;
-    rowp = p + (size_t)(r / inner) * gstride + r % inner;
+    rsrc = make_rsrc(p, (uint32_t)(((size_t)(groups - 1) * gstride + (size_t)K * ld) * 4u));
+    voff = row < R ? (uint32_t)((row / inner) * gstride + row % inner) * 4u : OOB;
   }
   template <int E>
-  __device__ void fetch(uint32_t k0, float (&v)[E]) const {
+  __device__ void seek(uint32_t k0) { k = k0; }
+  __device__ void next() { k += BK; }
+  template <int E>
+  __device__ void fetch(float (&v)[E]) const {
 #pragma unroll
-    for (int i = 0; i < E; i++) v[i] = (rowok && k0 + i < K) ? rowp[(size_t)(k0 + i) * ld] : 0.f;
+    for (int i = 0; i < E; i++) v[i] = buf_load(rsrc, k + i < K ? voff + (k + i) * ld * 4u : OOB, 0);
   }
 };
 
 // im2col view of NCHW images: row = (b, oy, ox), k = (c, ky, kx) with kx fastest;
 // element = image[b % in_w][c][oy*sy - py + ky][ox*sx - px + kx], 0 outside the image.
 // One stride phase of a transposed convolution is the same view with stride 1 and a (possibly negative) padding.
+// The k position is kept as (c, ky, kx); it is uniform over a wavefront (scalar registers) for tiles of >= 64 rows.
 struct SrcIm2col {
   static constexpr bool K_CONTIG = false;
   const float *p;
   uint32_t in_w, C, H, W, KY, KX, OHW, OW, R, K;
   int32_t sy, sx, py, px;
   Batch bt;  // per-image batching (kernels that differ per sample): stride = C*H*W, wmod = in_w
-  const float *base;
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t imgoff;  // byte offset of the row's image, OOB for rows outside the operand
   int32_t iy0, ix0;
-  bool rowok;
+  uint32_t k, c, ky, kx;
+  uint32_t step_c, step_ky, step_kx;  // BK = step_c*KY*KX + step_ky*KX + step_kx
   __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
   __device__ void bind(uint32_t row) {
-    rowok = row < R;
-    uint32_t r = rowok ? row : 0;
+    rsrc = make_rsrc(p, in_w * C * H * W * 4u);
+    uint32_t r = row < R ? row : 0;
     uint32_t b = r / OHW, q = r % OHW, oy = q / OW, ox = q % OW;
-    base = p + (size_t)(b % in_w) * C * H * W;
+    imgoff = row < R ? (b % in_w) * C * H * W * 4u : OOB;
     iy0 = (int32_t)oy * sy - py;
     ix0 = (int32_t)ox * sx - px;
   }
   template <int E>
-  __device__ void fetch(uint32_t k0, float (&v)[E]) const {
+  __device__ void seek(uint32_t k0) {
     uint32_t taps = KY * KX;
-    uint32_t c = k0 / taps, rem = k0 % taps, ky = rem / KX, kx = rem % KX;
+    k = k0; c = k0 / taps;
+    uint32_t rem = k0 % taps;
+    ky = rem / KX; kx = rem % KX;
+    step_c = BK / taps;
+    rem = BK % taps;
+    step_ky = rem / KX; step_kx = rem % KX;
+  }
+  __device__ void next() {
+    k += BK;
+    kx += step_kx;
+    if (kx >= KX) { kx -= KX; ky++; }
+    ky += step_ky;
+    if (ky >= KY) { ky -= KY; c++; }
+    c += step_c;
+  }
+  template <int E>
+  __device__ void fetch(float (&v)[E]) const {
+    uint32_t cc = c, yy = ky, xx = kx;
 #pragma unroll
     for (int i = 0; i < E; i++) {
-      int32_t iy = iy0 + (int32_t)ky, ix = ix0 + (int32_t)kx;
-      bool ok = rowok && (k0 + i < K) && (uint32_t)iy < H && (uint32_t)ix < W;
-      v[i] = ok ? base[((size_t)c * H + (uint32_t)iy) * W + (uint32_t)ix] : 0.f;
-      if (++kx == KX) { kx = 0; if (++ky == KY) { ky = 0; ++c; } }
+      int32_t iy = iy0 + (int32_t)yy, ix = ix0 + (int32_t)xx;
+      bool ok = (k + i < K) && (uint32_t)iy < H && (uint32_t)ix < W;
+      uint32_t off = imgoff + ((cc * H + (uint32_t)iy) * W + (uint32_t)ix) * 4u;
+      v[i] = buf_load(rsrc, ok ? off : OOB, 0);  // imgoff == OOB keeps a row outside the operand out of range
+      if (++xx == KX) { xx = 0; if (++yy == KY) { yy = 0; ++cc; } }
     }
+  }
+};
+
+// The same view when the taps tile the k step: KY*KX divides BK and C is a multiple of BK/(KY*KX) (so K is a
+// multiple of BK).  Then a thread's E elements always hit the same taps; their byte offsets (or OOB) are computed
+// once, and from tile to tile only the channel moves -- by the scalar offset.  Per tile: E loads, no vector ALU work.
+struct SrcIm2colFixed {
+  static constexpr bool K_CONTIG = false;
+  const float *p;
+  uint32_t in_w, C, H, W, KY, KX, OHW, OW, R, K;
+  int32_t sy, sx, py, px;
+  Batch bt;
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t imgoff;
+  int32_t iy0, ix0;
+  uint32_t voff[8];
+  uint32_t soff, sstep;
+  __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
+  __device__ void bind(uint32_t row) {
+    rsrc = make_rsrc(p, in_w * C * H * W * 4u);
+    uint32_t r = row < R ? row : 0;
+    uint32_t b = r / OHW, q = r % OHW, oy = q / OW, ox = q % OW;
+    imgoff = row < R ? (b % in_w) * C * H * W * 4u : OOB;
+    iy0 = (int32_t)oy * sy - py;
+    ix0 = (int32_t)ox * sx - px;
+  }
+  template <int E>
+  __device__ void seek(uint32_t k0) {  // k0 < BK
+    static_assert(E <= 8, "at most eight elements per thread");
+    const uint32_t taps = KY * KX;
+#pragma unroll
+    for (int i = 0; i < E; i++) {
+      uint32_t kk = k0 + i, cc = kk / taps, t = kk % taps, ty = t / KX, tx = t % KX;
+      int32_t iy = iy0 + (int32_t)ty, ix = ix0 + (int32_t)tx;
+      bool ok = imgoff != OOB && (uint32_t)iy < H && (uint32_t)ix < W;
+      voff[i] = ok ? imgoff + ((cc * H + (uint32_t)iy) * W + (uint32_t)ix) * 4u : OOB;
+    }
+    soff = 0;
+    sstep = (BK / taps) * H * W * 4u;
+  }
+  __device__ void next() { soff += sstep; }
+  template <int E>
+  __device__ void fetch(float (&v)[E]) const {
+#pragma unroll
+    for (int i = 0; i < E; i++) v[i] = buf_load(rsrc, voff[i], soff);
   }
 };
 
@@ -133,30 +237,43 @@ struct SrcIm2col {
 struct SrcWgradImage {
   static constexpr bool K_CONTIG = false;
   const float *p;
-  uint32_t H, W, KY, KX, OW, R, K;
+  uint32_t C, H, W, KY, KX, OW, R, K;
   int32_t sy, sx, py, px;
   Batch bt;
-  const float *base;
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t chanoff;
   int32_t iy0, ix0;
-  bool rowok;
+  uint32_t k, oy, ox, step_y, step_x;  // BK = step_y*OW + step_x
   __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
   __device__ void bind(uint32_t row) {
-    rowok = row < R;
-    uint32_t r = rowok ? row : 0;
+    rsrc = make_rsrc(p, C * H * W * 4u);
+    uint32_t r = row < R ? row : 0;
     uint32_t taps = KY * KX, c = r / taps, q = r % taps, i = q / KX, j = q % KX;
-    base = p + (size_t)c * H * W;
+    chanoff = row < R ? c * H * W * 4u : OOB;
     iy0 = (int32_t)i - py;
     ix0 = (int32_t)j - px;
   }
   template <int E>
-  __device__ void fetch(uint32_t k0, float (&v)[E]) const {
-    uint32_t oy = k0 / OW, ox = k0 % OW;
+  __device__ void seek(uint32_t k0) {
+    k = k0; oy = k0 / OW; ox = k0 % OW;
+    step_y = BK / OW; step_x = BK % OW;
+  }
+  __device__ void next() {
+    k += BK;
+    ox += step_x;
+    if (ox >= OW) { ox -= OW; oy++; }
+    oy += step_y;
+  }
+  template <int E>
+  __device__ void fetch(float (&v)[E]) const {
+    uint32_t yy = oy, xx = ox;
 #pragma unroll
     for (int i = 0; i < E; i++) {
-      int32_t iy = iy0 + (int32_t)oy * sy, ix = ix0 + (int32_t)ox * sx;
-      bool ok = rowok && (k0 + i < K) && (uint32_t)iy < H && (uint32_t)ix < W;
-      v[i] = ok ? base[(size_t)(uint32_t)iy * W + (uint32_t)ix] : 0.f;
-      if (++ox == OW) { ox = 0; ++oy; }
+      int32_t iy = iy0 + (int32_t)yy * sy, ix = ix0 + (int32_t)xx * sx;
+      bool ok = (k + i < K) && (uint32_t)iy < H && (uint32_t)ix < W;
+      uint32_t off = chanoff + ((uint32_t)iy * W + (uint32_t)ix) * 4u;
+      v[i] = buf_load(rsrc, ok ? off : OOB, 0);
+      if (++xx == OW) { xx = 0; ++yy; }
     }
   }
 };
@@ -214,21 +331,45 @@ struct Epilogue {
   }
 };
 
+// LDS tiles are [rows][LDK] with the 16 k of a tile contiguous per row and 4 floats of padding: a row is 80 bytes,
+// so eight consecutive rows start in eight different 16-byte bank groups and 128-bit LDS reads and writes of
+// consecutive rows are conflict free.
+constexpr int LDK = BK + 4;
+
+template <int TM, int TN, int WGM, int WGN>
+struct TileShape {
+  static constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+  static constexpr int LDS_FLOATS = 2 * (BM + BN) * LDK;
+};
+
+template <int E>
+__device__ __forceinline__ void lds_put(float *dst, const float (&v)[E]) {
+  if constexpr (E % 4 == 0) {
+#pragma unroll
+    for (int i = 0; i < E; i += 4) *reinterpret_cast<float4 *>(dst + i) = make_float4(v[i], v[i + 1], v[i + 2], v[i + 3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < E; i += 2) *reinterpret_cast<float2 *>(dst + i) = make_float2(v[i], v[i + 1]);
+  }
+}
+
+// One (BM x BN) block of C at (m0, n0).  `smem` holds LDS_FLOATS floats, 16-byte aligned.
+//
+// Feeding v_mfma_f32_32x32x2_f32: lanes 0-31 supply k = 2s and lanes 32-63 supply k = 2s+1 of step s, for the row
+// (lane % 32) of A and the column (lane % 32) of B.  Which k of the tile a step multiplies is free as long as A and
+// B agree, so lanes 0-31 take k = 0..3 and lanes 32-63 k = 4..7 from ONE 128-bit LDS read (steps 0-3), then
+// k = 8..11 / 12..15 from a second one (steps 4-7): two LDS reads per 32 rows and tile instead of eight.
 template <int TM, int TN, int WGM, int WGN, class SrcA, class SrcB>
-__global__ __launch_bounds__(THREADS) void igemm_kernel(SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K) {
+__device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep, uint32_t M, uint32_t N, uint32_t K, uint32_t m0, uint32_t n0, float *smem) {
   static_assert(WGM * WGN == 4, "four wavefronts per block");
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
   constexpr int EA = BM * BK / THREADS, EB = BN * BK / THREADS;
   static_assert(EA >= 2 && EB >= 2, "tile too small for the loader");
-  __shared__ float As[2][BK][BM];
-  __shared__ float Bs[2][BK][BN];
+  float *As = smem;                      // [2][BM][LDK]
+  float *Bs = smem + 2 * BM * LDK;       // [2][BN][LDK]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
-  const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  a.batch(blockIdx.z);
-  b.batch(blockIdx.z);
-  ep.batch(blockIdx.z);
 
   int a_row, a_k, b_row, b_k;
   if (SrcA::K_CONTIG) { constexpr int TPR = BK / EA; a_row = tid / TPR; a_k = (tid % TPR) * EA; }
@@ -251,39 +392,50 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(SrcA a, SrcB b, Epilogue
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
   const uint32_t nk = (K + BK - 1) / BK;
-  a.template fetch<EA>(a_k, ra);
-  b.template fetch<EB>(b_k, rb);
-#pragma unroll
-  for (int i = 0; i < EA; i++) As[0][a_k + i][a_row] = ra[i];
-#pragma unroll
-  for (int i = 0; i < EB; i++) Bs[0][b_k + i][b_row] = rb[i];
+  a.template seek<EA>(a_k);
+  b.template seek<EB>(b_k);
+  a.template fetch<EA>(ra);
+  b.template fetch<EB>(rb);
+  float *a_put = As + a_row * LDK + a_k, *b_put = Bs + b_row * LDK + b_k;
+  lds_put<EA>(a_put, ra);
+  lds_put<EB>(b_put, rb);
   __syncthreads();
 
   const int lrow = lane & 31, lk = lane >> 5;
+  const float *a_get = As + (wm * TM * 32 + lrow) * LDK + lk * 4;
+  const float *b_get = Bs + (wn * TN * 32 + lrow) * LDK + lk * 4;
   for (uint32_t kt = 0; kt < nk; kt++) {
     const int cur = kt & 1;
     const bool more = kt + 1 < nk;
-    if (more) {
-      a.template fetch<EA>((kt + 1) * BK + a_k, ra);
-      b.template fetch<EB>((kt + 1) * BK + b_k, rb);
+    // loads of the next tile: issued now, consumed after this tile's matrix instructions (the extra fetch of the
+    // last iteration lies beyond K, is answered with zeros by the range check and is never stored)
+    a.next();
+    b.next();
+    a.template fetch<EA>(ra);
+    b.template fetch<EB>(rb);
+    __builtin_amdgcn_sched_barrier(0);  // keep the loads above the matrix instructions: their latency hides behind them
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+      float4 av[TM], bv[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) av[i] = *reinterpret_cast<const float4 *>(a_get + cur * BM * LDK + i * 32 * LDK + half * 8);
+#pragma unroll
+      for (int j = 0; j < TN; j++) bv[j] = *reinterpret_cast<const float4 *>(b_get + cur * BN * LDK + j * 32 * LDK + half * 8);
+#pragma unroll
+      for (int c = 0; c < 4; c++)  // consecutive matrix instructions go to different accumulators
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++) {
+            float x = c == 0 ? av[i].x : c == 1 ? av[i].y : c == 2 ? av[i].z : av[i].w;
+            float y = c == 0 ? bv[j].x : c == 1 ? bv[j].y : c == 2 ? bv[j].z : bv[j].w;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[i][j], 0, 0, 0);
+          }
     }
-#pragma unroll
-    for (int ks = 0; ks < BK; ks += 2) {
-      float av[TM], bv[TN];
-#pragma unroll
-      for (int i = 0; i < TM; i++) av[i] = As[cur][ks + lk][(wm * TM + i) * 32 + lrow];
-#pragma unroll
-      for (int j = 0; j < TN; j++) bv[j] = Bs[cur][ks + lk][(wn * TN + j) * 32 + lrow];
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
-    }
+    __builtin_amdgcn_sched_barrier(0);
     if (more) {
-#pragma unroll
-      for (int i = 0; i < EA; i++) As[cur ^ 1][a_k + i][a_row] = ra[i];
-#pragma unroll
-      for (int i = 0; i < EB; i++) Bs[cur ^ 1][b_k + i][b_row] = rb[i];
+      lds_put<EA>(a_put + (cur ^ 1) * BM * LDK, ra);
+      lds_put<EB>(b_put + (cur ^ 1) * BN * LDK, rb);
     }
     __syncthreads();
   }
@@ -305,37 +457,140 @@ __global__ __launch_bounds__(THREADS) void igemm_kernel(SrcA a, SrcB b, Epilogue
   }
 }
 
-enum Tile { T128x128, T64x128, T32x128, T64x64 };
+// The hardware hands workgroup L of a 1-D grid to XCD (L % 8), each XCD with its own L2.  Renumbering gives
+// XCD x the contiguous logical range [x*total/8, (x+1)*total/8), so blocks that share operand tiles (neighbouring
+// logical indices) meet in one L2 instead of eight.
+__device__ __forceinline__ uint32_t xcd_swizzle(uint32_t L, uint32_t total) {
+  uint32_t per = total / 8;
+  if (L >= per * 8) return L;
+  return (L % 8) * per + L / 8;
+}
 
-inline Tile pick_tile(uint32_t M, uint32_t N) {
+// Generic launch: logical block index = (n tile, batch entry, m tile), n slowest, so concurrently running blocks
+// of one XCD share their B tile (the activations) and cycle through the A tiles (the weights).
+template <int TM, int TN, int WGM, int WGN, class SrcA, class SrcB>
+__global__ __launch_bounds__(THREADS) void igemm_kernel(SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, uint32_t tiles_m, uint32_t batches) {
+  using TS = TileShape<TM, TN, WGM, WGN>;
+  __shared__ float4 smem[TS::LDS_FLOATS / 4];
+  uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
+  uint32_t group = tiles_m * batches;
+  uint32_t nt = j / group, rem = j % group, bz = rem / tiles_m, mt = rem % tiles_m;
+  a.batch(bz);
+  b.batch(bz);
+  ep.batch(bz);
+  igemm_body<TM, TN, WGM, WGN>(a, b, ep, M, N, K, mt * TS::BM, nt * TS::BN, reinterpret_cast<float *>(smem));
+}
+
+enum Tile { T128x128, T64x128, T32x128, T64x64 };
+static const char *const tile_names[] = {"128x128", "64x128", "32x128", "64x64"};
+
+int &tile_override();  // -1: choose per shape; 0..3: force a Tile (measurements only)
+
+inline const char *shape_label(const char *name, Tile tile, uint32_t M, uint32_t N, uint32_t K, uint32_t batches) {
+  char buf[96];
+  snprintf(buf, sizeof buf, "%s M%u N%u K%u x%u", tile_names[tile], M, N, K, batches);
+  return intern_label(name, buf);
+}
+
+inline Tile pick_tile(uint32_t M, uint32_t N, uint32_t batches) {
+  if (tile_override() >= 0) return (Tile)tile_override();
   if (M <= 32) return T32x128;
-  if (M <= 64) return N >= 8192 ? T64x128 : T64x64;
-  size_t big = (size_t)cdiv(M, 128) * cdiv(N, 128);
-  if (big >= 512) return T128x128;  // at least two 128x128 blocks per compute unit
+  if (M <= 64) return (size_t)N * batches >= 8192 ? T64x128 : T64x64;
+  size_t big = (size_t)cdiv(M, 128) * cdiv(N, 128) * batches;
+  if (big >= 1024) return T128x128;  // at least four 128x128 blocks per compute unit
   return T64x128;
 }
 
 template <class SrcA, class SrcB>
 int launch(const char *name, SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, uint32_t batches) {
   if (M == 0 || N == 0 || batches == 0) return MT_OK;
-  if (batches > 65535u) return fail(MT_E_ARGUMENT, "%s: more than 65535 batched products", name);
   hipStream_t s = stream();
-  const Tile tile = pick_tile(M, N);
-  static const char *const tile_names[] = {"128x128", "64x128", "32x128", "64x64"};
-  ProfileScope prof(profiling() ? intern_label(name, tile_names[tile]) : name);
+  const Tile tile = pick_tile(M, N, batches);
+  ProfileScope prof(profiling() ? shape_label(name, tile, M, N, K, batches) : name);
+  const uint32_t bm = tile == T128x128 ? 128 : tile == T32x128 ? 32 : 64, bn = tile == T64x64 ? 64 : 128;
+  const uint32_t tm = cdiv(M, bm), tn = cdiv(N, bn);
+  const size_t total = (size_t)tm * tn * batches;
+  if (total > 0x7fffffffu) return fail(MT_E_ARGUMENT, "%s: problem too large for one launch", name);
   switch (tile) {
-    case T128x128:
-      igemm_kernel<2, 2, 2, 2><<<dim3(cdiv(N, 128), cdiv(M, 128), batches), THREADS, 0, s>>>(a, b, ep, M, N, K);
-      break;
-    case T64x128:
-      igemm_kernel<2, 1, 1, 4><<<dim3(cdiv(N, 128), cdiv(M, 64), batches), THREADS, 0, s>>>(a, b, ep, M, N, K);
-      break;
-    case T32x128:
-      igemm_kernel<1, 1, 1, 4><<<dim3(cdiv(N, 128), cdiv(M, 32), batches), THREADS, 0, s>>>(a, b, ep, M, N, K);
-      break;
-    case T64x64:
-      igemm_kernel<1, 1, 2, 2><<<dim3(cdiv(N, 64), cdiv(M, 64), batches), THREADS, 0, s>>>(a, b, ep, M, N, K);
-      break;
+    case T128x128: igemm_kernel<2, 2, 2, 2><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+    case T64x128: igemm_kernel<2, 1, 1, 4><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+    case T32x128: igemm_kernel<1, 1, 1, 4><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+    case T64x64: igemm_kernel<1, 1, 2, 2><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+  }
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
+// ---- all stride phases of a transposed convolution in one launch -------------------------------------------------
+// Phase f multiplies its packed sub-kernel [M][kp] with the stride-1 im2col view of the delta that has
+// taps_y x taps_x taps and offsets (offy, offx), and scatters to output pixels (qy*sy + py, qx*sx + px).
+struct TconvPhase {
+  const float *packed;
+  uint32_t kp, ld, qh, qw;  // packed rows hold kp coefficients, zero-padded to ld (a multiple of 4)
+  int32_t taps_y, taps_x, offy, offx;
+  uint32_t py, px;
+};
+constexpr int MAX_PHASES = 16;
+struct TconvArgs {
+  TconvPhase ph[MAX_PHASES];
+  uint32_t nphase, tiles_m, M, out_w;
+  const float *delta;          // [in_w][C][H][W]
+  uint32_t in_w, C, H, W;
+  Epilogue ep;   // C, row_stride, g_stride, sy, sx, OW, tap_bias, bias_w, IH, IW, func filled in
+};
+
+// FIXED: every phase has taps that tile the k step (see SrcIm2colFixed)
+template <int TM, int TN, int WGM, int WGN, bool FIXED>
+__global__ __launch_bounds__(THREADS) void tconv_kernel(TconvArgs args) {
+  using TS = TileShape<TM, TN, WGM, WGN>;
+  __shared__ float4 smem[TS::LDS_FLOATS / 4];
+  uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
+  uint32_t group = args.tiles_m * args.nphase;
+  uint32_t nt = j / group, rem = j % group, f = rem / args.tiles_m, mt = rem % args.tiles_m;
+  const TconvPhase &ph = args.ph[f];
+  const uint32_t qhw = ph.qh * ph.qw, N = args.out_w * qhw;
+  if (nt * TS::BN >= N) return;  // phases of an odd-sized output differ in size
+  SrcRowK<true> a{};
+  a.p = ph.packed; a.ld = ph.ld; a.R = args.M; a.K = ph.ld;  // rows are zero-padded to ld (a multiple of 4)
+  typename std::conditional<FIXED, SrcIm2colFixed, SrcIm2col>::type b{};
+  b.p = args.delta; b.in_w = args.in_w; b.C = args.C; b.H = args.H; b.W = args.W;
+  b.KY = ph.taps_y ? ph.taps_y : 1; b.KX = ph.taps_x ? ph.taps_x : 1; b.OHW = qhw; b.OW = ph.qw; b.R = N; b.K = ph.kp;
+  b.sy = 1; b.sx = 1; b.py = -ph.offy; b.px = -ph.offx;
+  Epilogue ep = args.ep;
+  ep.inner = qhw; ep.qw = ph.qw; ep.py = ph.py; ep.px = ph.px;
+  ep.ty_cnt = ph.taps_y; ep.tx_cnt = ph.taps_x; ep.offy = ph.offy; ep.offx = ph.offx;
+  igemm_body<TM, TN, WGM, WGN>(a, b, ep, args.M, N, ph.kp, mt * TS::BM, nt * TS::BN, reinterpret_cast<float *>(smem));
+}
+
+inline int launch_tconv(const char *name, TconvArgs &args, uint32_t max_n) {
+  if (args.M == 0 || max_n == 0 || args.nphase == 0) return MT_OK;
+  hipStream_t s = stream();
+  const Tile tile = pick_tile(args.M, max_n, args.nphase);
+  ProfileScope prof(profiling() ? shape_label(name, tile, args.M, max_n, args.ph[0].kp, args.nphase) : name);
+  const uint32_t bm = tile == T128x128 ? 128 : tile == T32x128 ? 32 : 64, bn = tile == T64x64 ? 64 : 128;
+  args.tiles_m = cdiv(args.M, bm);
+  const size_t total = (size_t)args.tiles_m * cdiv(max_n, bn) * args.nphase;
+  if (total > 0x7fffffffu) return fail(MT_E_ARGUMENT, "%s: problem too large for one launch", name);
+  bool fixed = true;
+  for (uint32_t f = 0; f < args.nphase; f++) {
+    uint32_t taps = args.ph[f].taps_y * args.ph[f].taps_x;
+    fixed = fixed && taps != 0 && BK % taps == 0 && args.C % (BK / taps) == 0;
+  }
+  const uint32_t grid = (uint32_t)total;
+  if (fixed) {
+    switch (tile) {
+      case T128x128: tconv_kernel<2, 2, 2, 2, true><<<grid, THREADS, 0, s>>>(args); break;
+      case T64x128: tconv_kernel<2, 1, 1, 4, true><<<grid, THREADS, 0, s>>>(args); break;
+      case T32x128: tconv_kernel<1, 1, 1, 4, true><<<grid, THREADS, 0, s>>>(args); break;
+      case T64x64: tconv_kernel<1, 1, 2, 2, true><<<grid, THREADS, 0, s>>>(args); break;
+    }
+  } else {
+    switch (tile) {
+      case T128x128: tconv_kernel<2, 2, 2, 2, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T64x128: tconv_kernel<2, 1, 1, 4, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T32x128: tconv_kernel<1, 1, 1, 4, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T64x64: tconv_kernel<1, 1, 2, 2, false><<<grid, THREADS, 0, s>>>(args); break;
+    }
   }
   MT_LAUNCH_CHECK(name);
   return MT_OK;

@@ -23,12 +23,17 @@ def gpu():
     return Gpu()
 
 
-@pytest.fixture(params=[2, 1], ids=["matrix-cores", "direct"])
+@pytest.fixture(params=[(2, -1), (2, 0), (2, 1), (2, 3), (1, -1)], ids=["auto", "mfma-128x128", "mfma-64x128", "mfma-64x64", "direct"])
 def path(request, gpu):
+    """Kernel family under test: per-shape choice (vector-ALU kernel for very few output channels, matrix cores
+    otherwise), the matrix-core kernels with one forced block tile, or the one-thread-per-output kernels."""
     import mi355tensor as mt
-    mt.set_option("conv_path", request.param)
-    yield request.param
+    conv_path, tile = request.param
+    mt.set_option("conv_path", conv_path)
+    mt.set_option("igemm_tile", tile)
+    yield conv_path
     mt.set_option("conv_path", 0)
+    mt.set_option("igemm_tile", -1)
 
 
 def close(got, want, tol=REL):
