@@ -259,6 +259,79 @@ __global__ __launch_bounds__(256) void tconv_small_kernel(TconvArgs args) {
     if (co < (int)args.M) ep.store(col, co, acc[co]);
 }
 
+// The same case for the common geometry kernel 4x4, stride 2, padding 1 (output exactly twice the input):
+// one thread per INPUT pixel computes the 2x2 output pixels it maps to, i.e. all four stride phases, for CO output
+// channels.  The four phases together read the 3x3 neighbourhood of the input pixel, so per input channel a
+// thread issues 9 loads for 16*CO multiply-adds.  The loads are buffer loads whose 9 byte offsets (or the
+// out-of-range marker for neighbours outside the image) are computed once; the channel advances through the
+// scalar offset.  The 16*CO coefficients of a channel are uniform and come through the scalar cache.
+template <int CO>
+__global__ __launch_bounds__(256) void tconv_k4s2_small_kernel(TconvArgs args) {
+  const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W;
+  const uint32_t n = blockIdx.x * 256 + threadIdx.x;
+  const bool live = n < args.out_w * HW;
+  const uint32_t g = (live ? n : 0) / HW, r = (live ? n : 0) % HW, qy = r / W, qx = r % W;
+  __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta, args.in_w * C * HW * 4u);
+  const uint32_t imgoff = (g % args.in_w) * C * HW * 4u;
+  uint32_t voff[3][3];
+#pragma unroll
+  for (int dy = 0; dy < 3; dy++)
+#pragma unroll
+    for (int dx = 0; dx < 3; dx++) {
+      int32_t iy = (int32_t)qy + dy - 1, ix = (int32_t)qx + dx - 1;
+      bool ok = live && (uint32_t)iy < H && (uint32_t)ix < W;
+      voff[dy][dx] = ok ? imgoff + ((uint32_t)iy * W + (uint32_t)ix) * 4u : OOB;
+    }
+  float acc[2][2][CO];
+#pragma unroll
+  for (int i = 0; i < 4 * CO; i++) (&acc[0][0][0])[i] = 0.f;
+  const uint32_t M = args.M;
+#pragma unroll 2
+  for (uint32_t ci = 0; ci < C; ci++) {
+    const uint32_t soff = ci * HW * 4u;
+    float v[3][3];
+#pragma unroll
+    for (int dy = 0; dy < 3; dy++)
+#pragma unroll
+      for (int dx = 0; dx < 3; dx++) v[dy][dx] = buf_load(rsrc, voff[dy][dx], soff);
+#pragma unroll
+    for (int py = 0; py < 2; py++)
+#pragma unroll
+      for (int px = 0; px < 2; px++) {
+        const TconvPhase &ph = args.ph[py * 2 + px];
+#pragma unroll
+        for (int co = 0; co < CO; co++) {
+          if (co >= (int)M) continue;
+          const float4 w = *reinterpret_cast<const float4 *>(ph.packed + (size_t)co * ph.ld + ci * 4u);  // taps (ty,tx) = 00 01 10 11
+          float a = acc[py][px][co];
+          a = __builtin_fmaf(w.x, v[py][px], a);
+          a = __builtin_fmaf(w.y, v[py][px + 1], a);
+          a = __builtin_fmaf(w.z, v[py + 1][px], a);
+          a = __builtin_fmaf(w.w, v[py + 1][px + 1], a);
+          acc[py][px][co] = a;
+        }
+      }
+  }
+  if (!live) return;
+  const uint32_t OW = 2 * W, OHW = 4 * HW;
+  const float bsum = args.ep.tap_bias ? args.ep.tap_bias[g % args.ep.bias_w] : 0.f;
+#pragma unroll
+  for (int py = 0; py < 2; py++) {
+    // contributing taps of output row 2*qy+py are input rows qy+py-1 and qy+py
+    const int ny = ((uint32_t)((int32_t)qy + py - 1) < H) + ((uint32_t)((int32_t)qy + py) < H);
+    const int nx0 = ((uint32_t)((int32_t)qx - 1) < W) + 1, nx1 = 1 + ((uint32_t)((int32_t)qx + 1) < W);
+#pragma unroll
+    for (int co = 0; co < CO; co++) {
+      if (co >= (int)M) continue;
+      float2 o;
+      o.x = mt::apply_func_epilogue(args.ep.func, acc[py][0][co] + bsum * (float)(ny * nx0));
+      o.y = mt::apply_func_epilogue(args.ep.func, acc[py][1][co] + bsum * (float)(ny * nx1));
+      float *dst = args.ep.C + ((size_t)g * M + co) * OHW + (size_t)(2 * qy + py) * OW + 2 * qx;
+      *reinterpret_cast<float2 *>(dst) = o;
+    }
+  }
+}
+
 int launch_tconv_small(const char *name, TconvArgs &args, uint32_t max_n) {
   mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "vector ALU, few output channels") : name);
   dim3 grid(cdiv(max_n, 256), args.nphase);
@@ -268,6 +341,21 @@ int launch_tconv_small(const char *name, TconvArgs &args, uint32_t max_n) {
     small = small && args.ph[f].taps_y <= 4 && args.ph[f].taps_x <= 4;
   }
   if (!small) return -1;  // caller falls back to the matrix-core path
+  // kernel 4x4, stride 2, padding 1 with the natural output size: four 2x2-tap phases with offsets -1 / 0
+  bool k4s2 = t22 && args.nphase == 4 && args.ep.sy == 2 && args.ep.sx == 2 && args.ep.OW == 2 * args.W && args.ep.row_stride == 4 * args.H * args.W &&
+              ((uintptr_t)args.ep.C & 7u) == 0;
+  for (uint32_t f = 0; k4s2 && f < 4; f++)
+    k4s2 = args.ph[f].py == f / 2 && args.ph[f].px == f % 2 && args.ph[f].offy == (int32_t)(f / 2) - 1 && args.ph[f].offx == (int32_t)(f % 2) - 1 &&
+           args.ph[f].qh == args.H && args.ph[f].qw == args.W;
+  if (k4s2) {
+    dim3 g4(cdiv((size_t)args.out_w * args.H * args.W, 256));
+    if (args.M <= 1) tconv_k4s2_small_kernel<1><<<g4, 256, 0, mt::stream()>>>(args);
+    else if (args.M <= 2) tconv_k4s2_small_kernel<2><<<g4, 256, 0, mt::stream()>>>(args);
+    else if (args.M == 3) tconv_k4s2_small_kernel<3><<<g4, 256, 0, mt::stream()>>>(args);
+    else tconv_k4s2_small_kernel<4><<<g4, 256, 0, mt::stream()>>>(args);
+    MT_LAUNCH_CHECK(name);
+    return MT_OK;
+  }
   if (t22) {
     if (args.M <= 2) tconv_small_kernel<2, 2, 2><<<grid, 256, 0, mt::stream()>>>(args);
     else tconv_small_kernel<4, 2, 2><<<grid, 256, 0, mt::stream()>>>(args);

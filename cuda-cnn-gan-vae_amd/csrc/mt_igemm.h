@@ -495,10 +495,12 @@ inline const char *shape_label(const char *name, Tile tile, uint32_t M, uint32_t
 inline Tile pick_tile(uint32_t M, uint32_t N, uint32_t batches) {
   if (tile_override() >= 0) return (Tile)tile_override();
   if (M <= 32) return T32x128;
-  if (M <= 64) return (size_t)N * batches >= 8192 ? T64x128 : T64x64;
+  if (M <= 64) return T64x64;
+  // 64x64 blocks need only 20 KB of LDS and 60 registers, so eight of them share a compute unit and hide each
+  // other's barriers and load latency; larger blocks only pay off when the grid is huge anyway
   size_t big = (size_t)cdiv(M, 128) * cdiv(N, 128) * batches;
-  if (big >= 1024) return T128x128;  // at least four 128x128 blocks per compute unit
-  return T64x128;
+  if (big >= 8192) return T128x128;
+  return T64x64;
 }
 
 template <class SrcA, class SrcB>
