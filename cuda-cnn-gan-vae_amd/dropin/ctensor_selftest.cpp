@@ -1,0 +1,221 @@
+// Self-test of the drop-in C++ classes: the checks of the reference's CTensorTest::Test()
+// (cuda/ctensortest.cu.h:725-928 and the five convolution tests at :77-652) written against the same public API,
+// plus the lazy host/device coherence and the error convention.  Every tensor op below runs on the GPU through
+// libmi355tensor.so.  Prints one line per check; exit code 0 when all pass.
+#include <stdio.h>
+#include <string.h>
+#include <string>
+
+#include "cuda/tensor.cu.h"
+
+namespace SYSTEM
+{
+ void PutMessage(const std::string &message) {printf("%s\n",message.c_str());}
+ void PutMessageToConsole(const std::string &message) {printf("%s\n",message.c_str());}
+}
+
+typedef float type_t;
+static const uint32_t BATCH=10;
+static int failures=0;
+
+static void Report(const char *name,bool ok)
+{
+ printf("%-64s %s\n",name,ok?"PASS":"FAIL");
+ if (!ok) failures++;
+}
+
+static bool AllEqual(const CTensor<type_t> &t,const type_t *expected)
+{
+ for(uint32_t w=0;w<t.GetSizeW();w++)
+ {
+  uint32_t n=0;
+  for(uint32_t z=0;z<t.GetSizeZ();z++)
+   for(uint32_t y=0;y<t.GetSizeY();y++)
+    for(uint32_t x=0;x<t.GetSizeX();x++,n++)
+     if (t.GetElement(w,z,y,x)!=expected[n]) return(false);
+ }
+ return(true);
+}
+
+// fills every batch layer with the same [Z,Y,X] data
+static void FillLayers(CTensor<type_t> &t,const type_t *data)
+{
+ for(uint32_t w=0;w<t.GetSizeW();w++)
+ {
+  uint32_t n=0;
+  for(uint32_t z=0;z<t.GetSizeZ();z++)
+   for(uint32_t y=0;y<t.GetSizeY();y++)
+    for(uint32_t x=0;x<t.GetSizeX();x++,n++) t.SetElement(w,z,y,x,data[n]);
+ }
+}
+
+static void MatrixChecks(void)
+{
+ const type_t m[4]={1,2,3,4};
+ CTensor<type_t> a(BATCH,1,2,2),b(BATCH,1,2,2),c(BATCH,1,2,2),a_one(1,1,2,2),b_one(1,1,2,2);
+ FillLayers(a,m);FillLayers(b,m);FillLayers(a_one,m);FillLayers(b_one,m);
+ Report("element set/get",AllEqual(a,m));
+ const type_t twice[4]={2,4,6,8};
+ c=a*static_cast<type_t>(2.0);
+ Report("tensor * scalar",AllEqual(c,twice));
+ c=static_cast<type_t>(2.0)*a;
+ Report("scalar * tensor",AllEqual(c,twice));
+ const type_t prod[4]={7,10,15,22};
+ c=a*b;
+ Report("Mul, equal batch",AllEqual(c,prod) && c.GetSizeW()==BATCH);
+ c=a_one*b;
+ Report("Mul, left operand broadcast over W",AllEqual(c,prod) && c.GetSizeW()==BATCH);
+ CTensorMath<type_t>::Mul(c,a,b_one);
+ Report("Mul, right operand broadcast over W",AllEqual(c,prod));
+ const type_t zero[4]={0,0,0,0};
+ c=a-b;
+ Report("Sub",AllEqual(c,zero));
+ c=a+b;
+ Report("Add",AllEqual(c,twice));
+ const type_t tr[4]={1,3,2,4};
+ c=CTensorMath<type_t>::Transpose(a);
+ Report("Transpose",AllEqual(c,tr));
+ const type_t sq[4]={1,4,9,16};
+ CTensor<type_t> e(BATCH,1,2,2);
+ CTensorMath<type_t>::TensorItemProduction(e,a,b);
+ Report("TensorItemProduction",AllEqual(e,sq));
+}
+
+static void ForwardConvolutionCheck(void)
+{
+ type_t kernel_a[12],kernel_b[12],image[27];
+ for(int n=0;n<12;n++) {kernel_a[n]=n+1;kernel_b[n]=12-n;}
+ for(int n=0;n<27;n++) image[n]=n+1;
+ CTensor<type_t> kernel(1,1,2,12),bias(1,2,1,1),img(BATCH,3,3,3),out(BATCH,2,2,2);
+ for(uint32_t n=0;n<12;n++) {kernel.SetElement(0,0,0,n,kernel_a[n]);kernel.SetElement(0,0,1,n,kernel_b[n]);}
+ CTensorMath<type_t>::Fill(bias,0);
+ FillLayers(img,image);
+ CTensorConv<type_t>::ForwardConvolution(out,img,kernel,2,2,3,2,bias,1,1,0,0);
+ const type_t expected[8]={1245,1323,1479,1557,627,705,861,939};
+ Report("ForwardConvolution 2x2x3, stride 1",AllEqual(out,expected));
+}
+
+static void DeltaWeightChecks(void)
+{
+ type_t image[49],delta[16];
+ for(int n=0;n<49;n++) image[n]=n+1;
+ for(int n=0;n<16;n++) delta[n]=n+1;
+ CTensor<type_t> img(BATCH,1,7,7),dl(BATCH,1,4,4),dk(BATCH,1,1,25),db(BATCH,1,1,1);
+ FillLayers(img,image);FillLayers(dl,delta);
+ CTensorMath<type_t>::Fill(db,0);
+ CTensorMath<type_t>::Fill(dk,0);
+ CTensorConv<type_t>::CreateDeltaWeightAndBias(dk,5,5,1,1,db,img,dl,2,2,2,2);
+ const type_t expected[25]={2031,2130,2746,1968,2058, 2724,2823,3628,2598,2688, 3448,3556,4560,3256,3352, 1860,1923,2428,1698,1752, 2301,2364,2974,2076,2130};
+ bool ok=true;
+ for(uint32_t w=0;w<BATCH;w++)
+ {
+  for(uint32_t n=0;n<25;n++) ok=ok && dk.GetElement(w,0,0,n)==expected[n];
+  ok=ok && db.GetElement(w,0,0,0)==136;
+ }
+ Report("CreateDeltaWeightAndBias 5x5, stride 2, padding 2",ok);
+
+ const type_t image2[16]={4,5,8,7, 1,8,8,8, 3,6,6,4, 6,5,7,8};
+ const type_t dout[4]={2,1,4,4};
+ CTensor<type_t> img2(BATCH,1,4,4),d2(BATCH,1,2,2),dk2(BATCH,1,1,9),db2(BATCH,1,1,1);
+ FillLayers(img2,image2);FillLayers(d2,dout);
+ CTensorMath<type_t>::Fill(dk2,0);
+ CTensorMath<type_t>::Fill(db2,0);
+ CTensorConv<type_t>::CreateDeltaWeightAndBias(dk2,3,3,1,1,db2,img2,d2,1,1,0,0);
+ const type_t expected2[9]={49,82,87,46,72,64,56,66,76};
+ ok=true;
+ for(uint32_t w=0;w<BATCH;w++)
+  for(uint32_t n=0;n<9;n++) ok=ok && dk2.GetElement(w,0,0,n)==expected2[n];
+ Report("CreateDeltaWeightAndBias 3x3, stride 1",ok);
+}
+
+static void BackwardConvolutionCheck(void)
+{
+ type_t delta[16];
+ for(int n=0;n<16;n++) delta[n]=n+1;
+ CTensor<type_t> kernel(1,1,1,25),bias(1,1,1,1),dl(BATCH,1,4,4),out(BATCH,1,7,7);
+ for(uint32_t n=0;n<25;n++) kernel.SetElement(0,0,0,n,n+1);
+ bias.Zero();
+ FillLayers(dl,delta);
+ CTensorConv<type_t>::BackwardConvolution(out,dl,kernel,5,5,1,1,bias,2,2,2,2);
+ const type_t expected[49]={56,70,124,102,172,134,156, 126,140,244,192,322,244,266, 233,266,450,344,567,422,467, 318,348,556,400,634,452,490,
+                            521,578,918,656,1035,734,803, 510,556,868,608,946,660,714, 740,786,1228,858,1336,930,984};
+ CTensor<type_t> control(BATCH,1,7,7);
+ FillLayers(control,expected);
+ Report("BackwardConvolution 5x5, stride 2, padding 2",out.Compare(control,"",false));
+}
+
+static void SummXYCheck(void)
+{
+ bool ok=true;
+ for(uint32_t size=1;size<512;size+=32)
+ {
+  CTensor<type_t> in(8,16,size,size),out(8,16,1,1);
+  in.Fill(1);
+  CTensorMath<type_t>::SummXY(out,in);
+  for(uint32_t w=0;w<8;w++)
+   for(uint32_t z=0;z<16;z++) ok=ok && static_cast<uint32_t>(out.GetElement(w,z,0,0))==size*size;
+ }
+ Report("SummXY of all-ones, sizes 1..481",ok);
+}
+
+static void CoherenceAndErrors(void)
+{
+ CTensor<type_t> a(2,1,2,3),b(2,1,2,3),c(2,1,2,3);
+ a.Fill(3);b.Fill(4);
+ CTensorMath<type_t>::Add(c,a,b);             // device result
+ bool ok=c.GetElement(1,0,1,2)==7;               // lazy download
+ c.SetElement(1,0,1,2,100);                      // host change
+ CTensorMath<type_t>::Mul(c,c,static_cast<type_t>(2));  // must upload before computing in place
+ ok=ok && c.GetElement(1,0,1,2)==200 && c.GetElement(0,0,0,0)==14;
+ CTensor<type_t> d=c;                            // deep copy, device data included
+ CTensorMath<type_t>::Fill(c,0);
+ ok=ok && d.GetElement(1,0,1,2)==200 && c.GetElement(1,0,1,2)==0;
+ c.ReinterpretSize(1,1,4,3);
+ ok=ok && c.GetSizeY()==4;
+ c.RestoreSize();
+ ok=ok && c.GetSizeW()==2 && c.GetSizeY()==2;
+ Report("host/device coherence, copies, reinterpretation",ok);
+
+ bool thrown=false;
+ try
+ {
+  CTensor<type_t> wrong(2,1,3,3);
+  CTensorMath<type_t>::Add(wrong,a,b);
+ }
+ catch(const char *message) {thrown=(message!=NULL && strlen(message)>0);}
+ Report("shape mismatch throws const char*",thrown);
+ thrown=false;
+ try {a.GetElement(0,0,5,0);} catch(const char*) {thrown=true;}
+ Report("out-of-range element access throws",thrown);
+
+ CTensor<CTensorMath<type_t>::SPos> pos(1,1,2,2);
+ CTensor<type_t> in(1,1,4,4),pooled(1,1,2,2),back(1,1,4,4);
+ for(uint32_t y=0;y<4;y++) for(uint32_t x=0;x<4;x++) in.SetElement(0,0,y,x,static_cast<type_t>((x*7+y*3)%5));
+ CTensorMath<type_t>::MaxPooling(pooled,pos,in,2,2);
+ CTensorMath<type_t>::SPos p=pos.GetElement(0,0,1,1);
+ ok=pooled.GetElement(0,0,1,1)==in.GetElement(0,0,p.Y,p.X) && p.X>=2 && p.Y>=2;
+ CTensorMath<type_t>::MaxPoolingBackward(back,pos,pooled,2,2);
+ ok=ok && back.GetElement(0,0,p.Y,p.X)==pooled.GetElement(0,0,1,1);
+ Report("MaxPooling positions and backward",ok);
+}
+
+int main(void)
+{
+ try
+ {
+  mi355::Check(mt_init(0));
+  MatrixChecks();
+  ForwardConvolutionCheck();
+  DeltaWeightChecks();
+  BackwardConvolutionCheck();
+  SummXYCheck();
+  CoherenceAndErrors();
+ }
+ catch(const char *message)
+ {
+  printf("exception: %s\n",message);
+  return(2);
+ }
+ printf("%s\n",failures==0?"ALL PASS":"SOME FAILED");
+ return(failures==0?0:1);
+}

@@ -1,0 +1,395 @@
+// Drop-in for the reference's cuda/ctensor.cu.h (class at :69-168): a dense [W,Z,Y,X] tensor with a host copy and a
+// device copy kept coherent lazily (HostOnChange / DeviceOnChange, :664-704).  Device memory goes through the C ABI of
+// libmi355tensor.so (mt_malloc / mt_copy_*), which replaces CCUDADeviceVector (cuda/ccudadevicevector.cu.h).
+// Failures are thrown as `const char *`, as the reference does.
+#ifndef C_TENSOR_CU_H
+#define C_TENSOR_CU_H
+
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../common/idatastream.h"
+#include "../system/system.h"
+#include "mi355_tensor.h"
+
+namespace mi355
+{
+ inline void Check(int rc)
+ {
+  if (rc!=MT_OK) throw static_cast<const char*>(mt_last_error());
+ }
+
+ // owning device buffer with value semantics (copying copies the device data, :159-170 of the reference vector)
+ class CDeviceBuffer
+ {
+   void *Ptr;
+   size_t Bytes;
+  public:
+   CDeviceBuffer(void):Ptr(NULL),Bytes(0) {}
+   CDeviceBuffer(const CDeviceBuffer &other):Ptr(NULL),Bytes(0) {*this=other;}
+   ~CDeviceBuffer() {clear();}
+   CDeviceBuffer& operator=(const CDeviceBuffer &other)
+   {
+    if (this==&other) return(*this);
+    resize(other.Bytes);
+    if (Bytes!=0) Check(mt_copy_d2d(Ptr,other.Ptr,Bytes));
+    return(*this);
+   }
+   void clear(void)
+   {
+    if (Ptr!=NULL) mt_free(Ptr);
+    Ptr=NULL;
+    Bytes=0;
+   }
+   void resize(size_t bytes)
+   {
+    if (bytes==Bytes) return;
+    clear();
+    if (bytes!=0) Check(mt_malloc(&Ptr,bytes));
+    Bytes=bytes;
+   }
+   void swap(CDeviceBuffer &other) {std::swap(Ptr,other.Ptr);std::swap(Bytes,other.Bytes);}
+   void* get(void) const {return(Ptr);}
+   size_t size(void) const {return(Bytes);}
+ };
+}
+
+template<class type_t> class CTensorMath;
+template<class type_t> class CTensorConv;
+template<class type_t> class CTensorApplyFunc;
+template<class type_t> class CTensor;
+
+template<class type_t> CTensor<type_t> operator+(const CTensor<type_t>& cTensor_Left,const CTensor<type_t>& cTensor_Right);
+template<class type_t> CTensor<type_t> operator-(const CTensor<type_t>& cTensor_Left,const CTensor<type_t>& cTensor_Right);
+template<class type_t> CTensor<type_t> operator*(const CTensor<type_t>& cTensor_Left,const CTensor<type_t>& cTensor_Right);
+template<class type_t> CTensor<type_t> operator*(const CTensor<type_t>& cTensor_Left,const type_t& value_right);
+template<class type_t> CTensor<type_t> operator*(const type_t& value_left,const CTensor<type_t>& cTensor_Right);
+
+template<class type_t>
+class CTensor
+{
+ template<class new_type_t> friend class CTensorMath;
+ template<class new_type_t> friend class CTensorConv;
+ template<class new_type_t> friend class CTensorApplyFunc;
+ template<class new_type_t> friend class CTensorTest;
+ private:
+  mutable uint32_t Size_X;
+  mutable uint32_t Size_Y;
+  mutable uint32_t Size_Z;
+  mutable uint32_t Size_W;
+  mutable uint32_t BasedSize_X;
+  mutable uint32_t BasedSize_Y;
+  mutable uint32_t BasedSize_Z;
+  mutable uint32_t BasedSize_W;
+  mutable std::vector<type_t> Item;
+  mutable mi355::CDeviceBuffer DeviceItem;
+  mutable bool HostOnChange;
+  mutable bool DeviceOnChange;
+ public:
+  CTensor(uint32_t size_w=1,uint32_t size_z=1,uint32_t size_y=1,uint32_t size_x=1)
+  {
+   Size_X=size_x;Size_Y=size_y;Size_Z=size_z;Size_W=size_w;
+   BasedSize_X=Size_X;BasedSize_Y=Size_Y;BasedSize_Z=Size_Z;BasedSize_W=Size_W;
+   Item.resize(Count());
+   DeviceItem.resize(Count()*sizeof(type_t));
+   HostOnChange=false;
+   DeviceOnChange=false;
+  }
+  CTensor(const CTensor<type_t> &cTensor)
+  {
+   Item=cTensor.Item;
+   DeviceItem=cTensor.DeviceItem;
+   Size_X=cTensor.Size_X;Size_Y=cTensor.Size_Y;Size_Z=cTensor.Size_Z;Size_W=cTensor.Size_W;
+   BasedSize_X=Size_X;BasedSize_Y=Size_Y;BasedSize_Z=Size_Z;BasedSize_W=Size_W;
+   HostOnChange=cTensor.HostOnChange;
+   DeviceOnChange=cTensor.DeviceOnChange;
+  }
+  ~CTensor() {}
+ public:
+  uint32_t GetSizeX(void) const {return(Size_X);}
+  uint32_t GetSizeY(void) const {return(Size_Y);}
+  uint32_t GetSizeZ(void) const {return(Size_Z);}
+  uint32_t GetSizeW(void) const {return(Size_W);}
+  type_t GetElement(uint32_t w,uint32_t z,uint32_t y,uint32_t x) const
+  {
+   if (x>=Size_X || y>=Size_Y || z>=Size_Z || w>=Size_W) throw("CTensor::GetElement: index outside the tensor");
+   CopyFromDevice();
+   return(Item[Index(w,z,y,x)]);
+  }
+  void SetElement(uint32_t w,uint32_t z,uint32_t y,uint32_t x,type_t value)
+  {
+   if (x>=Size_X || y>=Size_Y || z>=Size_Z || w>=Size_W) throw("CTensor::SetElement: index outside the tensor");
+   CopyFromDevice();
+   Item[Index(w,z,y,x)]=value;
+   SetHostOnChange();
+  }
+  type_t* GetColumnPtr(uint32_t w,uint32_t z,uint32_t y)
+  {
+   if (y>=Size_Y || z>=Size_Z || w>=Size_W) throw("CTensor::GetColumnPtr: row outside the tensor");
+   CopyFromDevice();
+   SetHostOnChange();
+   return(&Item[Index(w,z,y,0)]);
+  }
+  const type_t* GetColumnPtr(uint32_t w,uint32_t z,uint32_t y) const
+  {
+   if (y>=Size_Y || z>=Size_Z || w>=Size_W) throw("CTensor::GetColumnPtr: row outside the tensor");
+   CopyFromDevice();
+   SetHostOnChange();
+   return(&Item[Index(w,z,y,0)]);
+  }
+  void Unitary(void)
+  {
+   size_t n=0;
+   for(uint32_t w=0;w<Size_W;w++)
+    for(uint32_t z=0;z<Size_Z;z++)
+     for(uint32_t y=0;y<Size_Y;y++)
+      for(uint32_t x=0;x<Size_X;x++,n++) Item[n]=(x==y)?1:0;
+   SetHostOnChange();
+  }
+  void Zero(void) {Fill(0);}
+  void Fill(type_t value)
+  {
+   for(size_t n=0;n<Item.size();n++) Item[n]=value;
+   SetHostOnChange();
+  }
+  void Move(CTensor<type_t> &cTensor)
+  {
+   if (this==&cTensor) return;
+   Item=std::move(cTensor.Item);
+   DeviceItem.swap(cTensor.DeviceItem);
+   Size_X=cTensor.Size_X;Size_Y=cTensor.Size_Y;Size_Z=cTensor.Size_Z;Size_W=cTensor.Size_W;
+   BasedSize_X=cTensor.BasedSize_X;BasedSize_Y=cTensor.BasedSize_Y;BasedSize_Z=cTensor.BasedSize_Z;BasedSize_W=cTensor.BasedSize_W;
+   HostOnChange=cTensor.HostOnChange;
+   DeviceOnChange=cTensor.DeviceOnChange;
+   cTensor.Size_X=0;cTensor.Size_Y=0;cTensor.Size_Z=0;cTensor.Size_W=0;
+   cTensor.BasedSize_X=0;cTensor.BasedSize_Y=0;cTensor.BasedSize_Z=0;cTensor.BasedSize_W=0;
+   cTensor.Item.clear();
+   cTensor.HostOnChange=false;
+   cTensor.DeviceOnChange=false;
+  }
+  void CopyItem(CTensor<type_t> &cTensor)
+  {
+   if (Count()!=cTensor.Count()) throw("CTensor::CopyItem: element counts differ");
+   cTensor.CopyFromDevice();
+   Item=cTensor.Item;
+   SetHostOnChange();
+  }
+  void CopyItemToHost(type_t *item_array,uint32_t size)
+  {
+   if (Item.size()<size) throw("CTensor::CopyItemToHost: array larger than the tensor");
+   CopyFromDevice();
+   memcpy(&Item[0],item_array,size*sizeof(type_t));
+   SetHostOnChange();
+  }
+  void CopyItemToDevice(type_t *item_array,uint32_t size)
+  {
+   if (Item.size()<size) throw("CTensor::CopyItemToDevice: array larger than the tensor");
+   CopyToDevice();
+   mi355::Check(mt_copy_h2d(DeviceItem.get(),item_array,size*sizeof(type_t)));
+   SetDeviceOnChange();
+  }
+  void CopyItemLayerWToHost(uint32_t w,type_t *item_array,uint32_t size)
+  {
+   size_t offset=static_cast<size_t>(w)*Size_X*Size_Y*Size_Z;
+   if (Item.size()<size+offset) throw("CTensor::CopyItemLayerWToHost: array larger than the tensor");
+   CopyFromDevice();
+   memcpy(&Item[offset],item_array,size*sizeof(type_t));
+   SetHostOnChange();
+  }
+  void CopyItemLayerWToDevice(uint32_t w,type_t *item_array,uint32_t size)
+  {
+   size_t offset=static_cast<size_t>(w)*Size_X*Size_Y*Size_Z;
+   if (Item.size()<size+offset) throw("CTensor::CopyItemLayerWToDevice: array larger than the tensor");
+   CopyToDevice();
+   mi355::Check(mt_copy_h2d(static_cast<type_t*>(DeviceItem.get())+offset,item_array,size*sizeof(type_t)));
+   SetDeviceOnChange();
+  }
+  CTensor<type_t>& operator=(const CTensor<type_t> &cTensor)
+  {
+   if (this!=&cTensor)
+   {
+    Item=cTensor.Item;
+    DeviceItem=cTensor.DeviceItem;
+    Size_X=cTensor.Size_X;Size_Y=cTensor.Size_Y;Size_Z=cTensor.Size_Z;Size_W=cTensor.Size_W;
+    BasedSize_X=cTensor.BasedSize_X;BasedSize_Y=cTensor.BasedSize_Y;BasedSize_Z=cTensor.BasedSize_Z;BasedSize_W=cTensor.BasedSize_W;
+    HostOnChange=cTensor.HostOnChange;
+    DeviceOnChange=cTensor.DeviceOnChange;
+   }
+   return(*this);
+  }
+
+  friend CTensor<type_t> operator+<type_t>(const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right);
+  friend CTensor<type_t> operator-<type_t>(const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right);
+  friend CTensor<type_t> operator*<type_t>(const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right);
+  friend CTensor<type_t> operator*<type_t>(const CTensor<type_t> &cTensor_Left,const type_t &value_right);
+  friend CTensor<type_t> operator*<type_t>(const type_t &value_left,const CTensor<type_t> &cTensor_Right);
+
+  // on-disk form: W,Z,Y,X as uint32 then every element as a double (reference :525-571)
+  bool Save(IDataStream *iDataStream_Ptr)
+  {
+   CopyFromDevice();
+   iDataStream_Ptr->SaveUInt32(Size_W);
+   iDataStream_Ptr->SaveUInt32(Size_Z);
+   iDataStream_Ptr->SaveUInt32(Size_Y);
+   iDataStream_Ptr->SaveUInt32(Size_X);
+   for(size_t n=0;n<Count();n++) iDataStream_Ptr->SaveDouble(static_cast<double>(Item[n]));
+   return(true);
+  }
+  bool Load(IDataStream *iDataStream_Ptr,bool check_size=false)
+  {
+   if (check_size==true)
+   {
+    if (Size_W!=iDataStream_Ptr->LoadUInt32()) throw("CTensor::Load: stored W differs");
+    if (Size_Z!=iDataStream_Ptr->LoadUInt32()) throw("CTensor::Load: stored Z differs");
+    if (Size_Y!=iDataStream_Ptr->LoadUInt32()) throw("CTensor::Load: stored Y differs");
+    if (Size_X!=iDataStream_Ptr->LoadUInt32()) throw("CTensor::Load: stored X differs");
+   }
+   else
+   {
+    Size_W=iDataStream_Ptr->LoadUInt32();
+    Size_Z=iDataStream_Ptr->LoadUInt32();
+    Size_Y=iDataStream_Ptr->LoadUInt32();
+    Size_X=iDataStream_Ptr->LoadUInt32();
+   }
+   Item.assign(Count(),type_t());
+   DeviceItem.resize(Item.size()*sizeof(type_t));
+   for(size_t n=0;n<Count();n++) Item[n]=static_cast<type_t>(iDataStream_Ptr->LoadDouble());
+   SetHostOnChange();
+   return(true);
+  }
+
+  void ExchangeSizeXY(void) const {uint32_t tmp=Size_X;Size_X=Size_Y;Size_Y=tmp;}
+  void ReinterpretSize(uint32_t size_w,uint32_t size_z,uint32_t size_y,uint32_t size_x) const
+  {
+   if (Count()!=static_cast<size_t>(size_x)*size_y*size_z*size_w)
+   {
+    char str[256];
+    snprintf(str,sizeof(str),"%ux%ux%ux%u->%ux%ux%ux%u",Size_W,Size_Z,Size_Y,Size_X,size_w,size_z,size_y,size_x);
+    SYSTEM::PutMessageToConsole(str);
+    throw("CTensor::ReinterpretSize: the element count must not change");
+   }
+   Size_X=size_x;Size_Y=size_y;Size_Z=size_z;Size_W=size_w;
+  }
+  void RestoreSize(void) const {Size_X=BasedSize_X;Size_Y=BasedSize_Y;Size_Z=BasedSize_Z;Size_W=BasedSize_W;}
+
+  void Normalize(void)
+  {
+   CopyFromDevice();
+   for(uint32_t w=0;w<Size_W;w++)
+    for(uint32_t z=0;z<Size_Z;z++)
+    {
+     type_t norma=GetNorma(w,z);
+     if (norma<0.0000000001) continue;
+     for(uint32_t y=0;y<Size_Y;y++)
+      for(uint32_t x=0;x<Size_X;x++) Item[Index(w,z,y,x)]/=norma;
+    }
+   SetHostOnChange();
+  }
+  type_t GetNorma(uint32_t w,uint32_t z) const
+  {
+   CopyFromDevice();
+   type_t norma=0;
+   for(uint32_t y=0;y<Size_Y;y++)
+    for(uint32_t x=0;x<Size_X;x++)
+    {
+     type_t v=Item[Index(w,z,y,x)];
+     norma+=v*v;
+    }
+   return(sqrt(norma));
+  }
+
+  void CopyToDevice(bool force=false) const
+  {
+   if (HostOnChange==false && force==false) return;
+   if (!Item.empty()) mi355::Check(mt_copy_h2d(DeviceItem.get(),&Item[0],Item.size()*sizeof(type_t)));
+   HostOnChange=false;
+   DeviceOnChange=false;
+  }
+  void CopyFromDevice(bool force=false) const
+  {
+   if (DeviceOnChange==false && force==false) return;
+   if (!Item.empty()) mi355::Check(mt_copy_d2h(&Item[0],DeviceItem.get(),Item.size()*sizeof(type_t)));
+   HostOnChange=false;
+   DeviceOnChange=false;
+  }
+  void SetDeviceOnChange(void) const {DeviceOnChange=true;HostOnChange=false;}
+  void SetHostOnChange(void) const {DeviceOnChange=false;HostOnChange=true;}
+
+  void Print(const std::string &name,bool print_value=true) const
+  {
+   char str[255];
+   CopyFromDevice();
+   snprintf(str,sizeof(str),"***** %s *****",name.c_str());
+   SYSTEM::PutMessageToConsole(str);
+   snprintf(str,sizeof(str),"W:%u Z:%u Y:%u X:%u",Size_W,Size_Z,Size_Y,Size_X);
+   SYSTEM::PutMessageToConsole(str);
+   if (print_value==false) return;
+   for(uint32_t w=0;w<Size_W;w++)
+    for(uint32_t z=0;z<Size_Z;z++)
+     for(uint32_t y=0;y<Size_Y;y++)
+     {
+      std::string line;
+      for(uint32_t x=0;x<Size_X;x++)
+      {
+       snprintf(str,sizeof(str),"%f ",static_cast<double>(Item[Index(w,z,y,x)]));
+       line+=str;
+      }
+      SYSTEM::PutMessageToConsole(line);
+     }
+  }
+  void PrintToFile(const std::string &file_name,const std::string &name,bool print_value=true) const
+  {
+   CopyFromDevice();
+   FILE *file=fopen(file_name.c_str(),"wb");
+   if (file==NULL) return;
+   fprintf(file,"***** %s *****\r\nW:%u Z:%u Y:%u X:%u\r\n",name.c_str(),Size_W,Size_Z,Size_Y,Size_X);
+   if (print_value==true)
+   {
+    for(uint32_t w=0;w<Size_W;w++)
+     for(uint32_t z=0;z<Size_Z;z++)
+      for(uint32_t y=0;y<Size_Y;y++)
+      {
+       for(uint32_t x=0;x<Size_X;x++) fprintf(file,"%f ",static_cast<double>(Item[Index(w,z,y,x)]));
+       fprintf(file,"\r\n");
+      }
+   }
+   fclose(file);
+  }
+  // absolute tolerance 1e-5, as the reference (:787)
+  bool Compare(const CTensor<type_t> &cTensor_Control,const std::string &name="",bool print_value=true) const
+  {
+   CopyFromDevice();
+   cTensor_Control.CopyFromDevice();
+   if (print_value==true && !name.empty()) SYSTEM::PutMessageToConsole(name);
+   bool ret=true;
+   for(uint32_t w=0;w<Size_W;w++)
+    for(uint32_t z=0;z<Size_Z;z++)
+     for(uint32_t y=0;y<Size_Y;y++)
+      for(uint32_t x=0;x<Size_X;x++)
+      {
+       double e1=static_cast<double>(GetElement(w,z,y,x));
+       double e2=static_cast<double>(cTensor_Control.GetElement(w,z,y,x));
+       if (fabs(e1-e2)>0.00001) ret=false;
+      }
+   return(ret);
+  }
+ private:
+  size_t Count(void) const {return(static_cast<size_t>(Size_X)*Size_Y*Size_Z*Size_W);}
+  size_t Index(uint32_t w,uint32_t z,uint32_t y,uint32_t x) const {return(x+static_cast<size_t>(Size_X)*(y+static_cast<size_t>(Size_Y)*(z+static_cast<size_t>(Size_Z)*w)));}
+  // descriptor of the device copy for the C ABI; `upload` first brings the device copy up to date
+  mt_tensor Device(bool upload) const
+  {
+   if (upload==true) CopyToDevice();
+   mt_tensor t;
+   t.p=static_cast<float*>(DeviceItem.get());
+   t.w=Size_W;t.z=Size_Z;t.y=Size_Y;t.x=Size_X;
+   return(t);
+  }
+};
+
+#endif

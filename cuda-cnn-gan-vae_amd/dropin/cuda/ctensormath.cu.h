@@ -1,0 +1,267 @@
+// Drop-in for the reference's cuda/ctensormath.cu.h (class at :52-138): every static function keeps the reference's
+// name, argument order and defaults and forwards to one C-ABI call.  Inputs are brought up to date on the device
+// first and the output is marked device-side, as the reference does (:845-870).
+#ifndef C_TENSOR_MATH_CU_H
+#define C_TENSOR_MATH_CU_H
+
+#include <type_traits>
+
+#include "ctensor.cu.h"
+
+template<class type_t>
+class CTensorMath
+{
+ public:
+  struct SPos
+  {
+   uint32_t X;
+   uint32_t Y;
+  };
+ private:
+  static void OnlyFloat(void) {static_assert(std::is_same<type_t,float>::value,"the MI355X tensor path computes in fp32 only");}
+  static mt_pos_tensor Position(const CTensor<SPos> &cTensor,bool upload)
+  {
+   mt_tensor t=cTensor.Device(upload);
+   mt_pos_tensor p;
+   p.p=reinterpret_cast<mt_spos*>(t.p);
+   p.w=t.w;p.z=t.z;p.y=t.y;p.x=t.x;
+   return(p);
+  }
+ public:
+  static void Fill(CTensor<type_t> &cTensor_Output,type_t value=0)
+  {
+   OnlyFloat();
+   mt_tensor o=cTensor_Output.Device(false);
+   mi355::Check(mt_fill(&o,value));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Inv(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_inv(&o,&i));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Div(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
+  {
+   OnlyFloat();
+   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_div(&o,&l,&r,left_scale,right_scale));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Add(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
+  {
+   OnlyFloat();
+   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_add(&o,&l,&r,left_scale,right_scale));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  // The batch-norm layer of the reference calls Add(out,left,right,EMA_K,1,0-EMA_K) (netlayer/cnetlayerbatchnormalization.cu.h:655-658,
+  // a typo for 1.0-EMA_K that matches no overload of the reference): this overload gives it the intended right scale 1-EMA_K.
+  static void Add(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale,int right_scale_a,type_t right_scale_b)
+  {
+   Add(cTensor_Output,cTensor_Left,cTensor_Right,left_scale,static_cast<type_t>(right_scale_a+right_scale_b));
+  }
+  static void AddSumW(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
+  {
+   OnlyFloat();
+   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_add_sum_w(&o,&l,&r,left_scale,right_scale));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void AddValue(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t tensor_scale,type_t value)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_add_value(&o,&i,tensor_scale,value));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Sub(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
+  {
+   OnlyFloat();
+   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_sub(&o,&l,&r,left_scale,right_scale));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void SubValue(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t tensor_scale,type_t value)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_sub_value(&o,&i,tensor_scale,value));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Set(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t scale=1,type_t add_value=0)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_set(&o,&i,scale,add_value));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Pow2(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t scale=1)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_pow2(&o,&i,scale));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void SQRT(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t scale,type_t add_sqrt_value)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_sqrt(&o,&i,scale,add_sqrt_value));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void AddBias(CTensor<type_t> &cTensor_Working,const CTensor<type_t> &cTensor_Bias)
+  {
+   OnlyFloat();
+   mt_tensor b=cTensor_Bias.Device(true),o=cTensor_Working.Device(true);
+   mi355::Check(mt_add_bias(&o,&b));
+   cTensor_Working.SetDeviceOnChange();
+  }
+  static void SummXY(CTensor<type_t> &cTensor_Output,CTensor<type_t> &cTensor_Input)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(true);
+   mi355::Check(mt_summ_xy(&o,&i));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Mul(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,bool tensor_core=false)
+  {
+   OnlyFloat();
+   (void)tensor_core;  // the reference's fp16 tensor-core switch; this path is always fp32 on the matrix cores
+   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_mul(&o,&l,&r));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void TransponseMul(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,bool tensor_core=false)
+  {
+   OnlyFloat();
+   (void)tensor_core;
+   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_transponse_mul(&o,&l,&r));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Mul(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const type_t &value_right)
+  {
+   OnlyFloat();
+   mt_tensor l=cTensor_Left.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_mul_value(&o,&l,value_right));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Mul(CTensor<type_t> &cTensor_Output,const type_t &value_left,const CTensor<type_t> &cTensor_Right)
+  {
+   Mul(cTensor_Output,cTensor_Right,value_left);
+  }
+  static void Transponse(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_transponse(&o,&i));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void TensorItemProduction(CTensor<type_t> &cTensor_Output,CTensor<type_t> &cTensor_Left,CTensor<type_t> &cTensor_Right)
+  {
+   OnlyFloat();
+   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_tensor_item_production(&o,&l,&r));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static CTensor<type_t> Transpose(const CTensor<type_t> &cTensor_Input)
+  {
+   CTensor<type_t> cTensor(cTensor_Input.Size_W,cTensor_Input.Size_Z,cTensor_Input.Size_X,cTensor_Input.Size_Y);
+   Transponse(cTensor,cTensor_Input);
+   return(cTensor);
+  }
+  static void UpSampling(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,uint32_t upsampling_x,uint32_t upsampling_y)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_upsampling(&o,&i,upsampling_x,upsampling_y));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void DownSampling(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,uint32_t downsampling_x,uint32_t downsampling_y)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_downsampling(&o,&i,downsampling_x,downsampling_y));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void MaxPooling(CTensor<type_t> &cTensor_Output,const CTensor<SPos> &cTensor_Position,const CTensor<type_t> &cTensor_Input,uint32_t pooling_x,uint32_t pooling_y)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_pos_tensor p=Position(cTensor_Position,false);
+   mi355::Check(mt_max_pooling(&o,&p,&i,pooling_x,pooling_y));
+   cTensor_Output.SetDeviceOnChange();
+   cTensor_Position.SetDeviceOnChange();
+  }
+  static void MaxPoolingBackward(CTensor<type_t> &cTensor_Output,const CTensor<SPos> &cTensor_Position,const CTensor<type_t> &cTensor_Input,uint32_t pooling_x,uint32_t pooling_y)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_pos_tensor p=Position(cTensor_Position,true);
+   mi355::Check(mt_max_pooling_backward(&o,&p,&i,pooling_x,pooling_y));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void Clip(CTensor<type_t> &cTensor,type_t min_value,type_t max_value)
+  {
+   OnlyFloat();
+   mt_tensor o=cTensor.Device(true);
+   mi355::Check(mt_clip(&o,min_value,max_value));
+   cTensor.SetDeviceOnChange();
+  }
+  static void Signum(CTensor<type_t> &cTensor)
+  {
+   OnlyFloat();
+   mt_tensor o=cTensor.Device(true);
+   mi355::Check(mt_signum(&o));
+   cTensor.SetDeviceOnChange();
+  }
+  static void Adam(CTensor<type_t> &cTensor_Weight,CTensor<type_t> &cTensor_dWeight,CTensor<type_t> &cTensor_M,CTensor<type_t> &cTensor_V,uint32_t batch_size,double speed,double beta1,double beta2,double epsilon,double iteration)
+  {
+   OnlyFloat();
+   mt_tensor w=cTensor_Weight.Device(true),dw=cTensor_dWeight.Device(true),m=cTensor_M.Device(true),v=cTensor_V.Device(true);
+   mi355::Check(mt_adam(&w,&dw,&m,&v,batch_size,speed,beta1,beta2,epsilon,iteration));
+   cTensor_Weight.SetDeviceOnChange();
+   cTensor_M.SetDeviceOnChange();
+   cTensor_V.SetDeviceOnChange();
+  }
+};
+
+template<class type_t>
+CTensor<type_t> operator+(const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right)
+{
+ CTensor<type_t> cTensor(cTensor_Right.Size_W,cTensor_Left.Size_Z,cTensor_Left.Size_Y,cTensor_Left.Size_X);
+ CTensorMath<type_t>::Add(cTensor,cTensor_Left,cTensor_Right);
+ return(cTensor);
+}
+template<class type_t>
+CTensor<type_t> operator-(const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right)
+{
+ CTensor<type_t> cTensor(cTensor_Right.Size_W,cTensor_Left.Size_Z,cTensor_Left.Size_Y,cTensor_Left.Size_X);
+ CTensorMath<type_t>::Sub(cTensor,cTensor_Left,cTensor_Right);
+ return(cTensor);
+}
+template<class type_t>
+CTensor<type_t> operator*(const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right)
+{
+ CTensor<type_t> cTensor(cTensor_Right.Size_W,cTensor_Left.Size_Z,cTensor_Left.Size_Y,cTensor_Right.Size_X);
+ CTensorMath<type_t>::Mul(cTensor,cTensor_Left,cTensor_Right);
+ return(cTensor);
+}
+template<class type_t>
+CTensor<type_t> operator*(const CTensor<type_t> &cTensor_Left,const type_t &value_right)
+{
+ CTensor<type_t> cTensor(cTensor_Left.Size_W,cTensor_Left.Size_Z,cTensor_Left.Size_Y,cTensor_Left.Size_X);
+ CTensorMath<type_t>::Mul(cTensor,cTensor_Left,value_right);
+ return(cTensor);
+}
+template<class type_t>
+CTensor<type_t> operator*(const type_t &value_left,const CTensor<type_t> &cTensor_Right)
+{
+ CTensor<type_t> cTensor(cTensor_Right.Size_W,cTensor_Right.Size_Z,cTensor_Right.Size_Y,cTensor_Right.Size_X);
+ CTensorMath<type_t>::Mul(cTensor,value_left,cTensor_Right);
+ return(cTensor);
+}
+
+#endif

@@ -76,7 +76,9 @@ int mt_synchronize(void);
 void *mt_get_stream(void);               /* the hipStream_t all work is queued on */
 int mt_set_stream(void *hip_stream);     /* queue on a caller-owned stream (NULL: back to the library's own) */
 /* "conv_path": 0 choose per shape (default), 1 one-thread-per-output kernels in the CPU path's summation order,
- * 2 matrix-core kernels wherever they apply.  For tests and measurements; results agree within fp32 rounding. */
+ * 2 matrix-core kernels wherever they apply.  "igemm_tile": -1 choose per shape (default), 0..3 force the block
+ * tile 128x128 / 64x128 / 32x128 / 64x64 of the matrix-core kernels.  For tests and measurements; results agree
+ * within fp32 rounding. */
 int mt_set_option(const char *name, int value);
 
 /* ---- convolutions: CTensorConv<T> (cuda/ctensorconv.cu.h:63-66) ---- */

@@ -1,0 +1,279 @@
+// TEST INFRASTRUCTURE ONLY.
+//
+// Runs the reference's OWN layer classes (netlayer/cnetlayer*.cu.h, compiled from /root/reference where they lie)
+// on seeded inputs and writes every layer output, back-propagated error and updated weight to a file.
+// The same source is built twice by oracle/Makefile, only where /root/reference exists, into oracle/_ref/:
+//   layers_cpu    -DUSE_CPU: the layers on the reference's CPU tensor classes (cpu/tensor.h)
+//   layers_mi355  the layers on the drop-in tensor classes (cuda-cnn-gan-vae_amd/dropin) -> libmi355tensor.so
+// A GPU test runs both and compares the files: the unchanged layers produce the same numbers on the HIP path.
+// Weights enter through Load() from an in-memory stream (Reset() uses an unseeded RNG, and Load() is the only way
+// to give the transposed-convolution layer a correctly shaped kernel).
+//
+// Chain A: input [B,3,16,16] -> Convolution 8 x 4x4 s2 p1 -> LeakyReLU -> Linear 24 -> Sigmoid
+// Chain B: input [B,8,4,4]   -> BackConvolution 4x4 s2 p1 to 3 channels -> Tangence
+// Chain C: input [B,4,5,5]   -> BatchNormalization (training) -> ReLU            (layers_mi355 only: the reference's
+//          batch-norm layer does not compile on its own CPU classes, netlayer/cnetlayerbatchnormalization.cu.h:655)
+// Each chain: TrainingStart, Forward, SetOutputError, TrainingBackward, TrainingUpdateWeight (gradient descent), Save.
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+#include <algorithm>
+#include <memory>
+#include <string>
+#include <vector>
+
+#ifdef USE_CPU
+#include "common/idatastream.h"
+#include "system/system.h"
+#include "cuda/tensor.cu.h"   // with USE_CPU this is the reference's cpu/tensor.h
+#else
+#include "cuda/tensor.cu.h"   // the drop-in, found first on the include path
+#endif
+
+#include "netlayer/cnetlayerconvolutioninput.cu.h"
+#include "netlayer/cnetlayerconvolution.cu.h"
+#include "netlayer/cnetlayerbackconvolution.cu.h"
+#include "netlayer/cnetlayerlinear.cu.h"
+#include "netlayer/cnetlayerfunction.cu.h"
+#ifndef USE_CPU
+#include "netlayer/cnetlayerbatchnormalization.cu.h"
+#endif
+
+namespace SYSTEM
+{
+ void PutMessage(const std::string &) {}
+ void PutMessageToConsole(const std::string &) {}
+}
+// the reference's IDataStream declares a file factory that nothing here calls
+#ifdef USE_CPU
+IDataStream* IDataStream::CreateNewDataStreamFile(std::string,bool) {return(NULL);}
+#endif
+
+typedef float type_t;
+
+// bytes in memory, typed access in host byte order like the reference's file stream
+class CMemoryStream:public IDataStream
+{
+  std::vector<uint8_t> Data;
+  size_t Pos;
+  template<class T> T Get(void) {T v;memcpy(&v,&Data[Pos],sizeof(T));Pos+=sizeof(T);return(v);}
+  template<class T> void Put(T v) {const uint8_t *p=reinterpret_cast<const uint8_t*>(&v);Data.insert(Data.end(),p,p+sizeof(T));}
+ public:
+  CMemoryStream(void):Pos(0) {}
+  void Rewind(void) {Pos=0;}
+  int8_t LoadInt8(void) {return(Get<int8_t>());}
+  int16_t LoadInt16(void) {return(Get<int16_t>());}
+  int32_t LoadInt32(void) {return(Get<int32_t>());}
+  uint8_t LoadUInt8(void) {return(Get<uint8_t>());}
+  uint16_t LoadUInt16(void) {return(Get<uint16_t>());}
+  uint32_t LoadUInt32(void) {return(Get<uint32_t>());}
+  float LoadFloat(void) {return(Get<float>());}
+  double LoadDouble(void) {return(Get<double>());}
+  void SaveFloat(float value) {Put(value);}
+  void SaveDouble(double value) {Put(value);}
+  void SaveInt8(int8_t value) {Put(value);}
+  void SaveInt16(int16_t value) {Put(value);}
+  void SaveInt32(int32_t value) {Put(value);}
+  void SaveUInt8(int8_t value) {Put(value);}
+  void SaveUInt16(int16_t value) {Put(value);}
+  void SaveUInt32(int32_t value) {Put(value);}
+  bool IsFail(void) const {return(false);}
+  // a tensor as CTensor::Save writes it: four sizes, then doubles
+  void PutTensor(uint32_t w,uint32_t z,uint32_t y,uint32_t x,const std::vector<double> &v)
+  {
+   Put<uint32_t>(w);Put<uint32_t>(z);Put<uint32_t>(y);Put<uint32_t>(x);
+   for(size_t n=0;n<v.size();n++) Put<double>(v[n]);
+  }
+};
+
+// small deterministic generator (the same stream of numbers in both builds)
+static uint64_t rng_state=0x9E3779B97F4A7C15ull;
+static double Uniform(void)
+{
+ rng_state=rng_state*6364136223846793005ull+1442695040888963407ull;
+ return(static_cast<double>((rng_state>>11)&0xFFFFFFFFFFFFFull)/4503599627370496.0*2.0-1.0);
+}
+static std::vector<double> Values(size_t n,double scale)
+{
+ std::vector<double> v(n);
+ for(size_t i=0;i<n;i++) v[i]=static_cast<double>(static_cast<float>(Uniform()*scale));  // exactly representable in fp32
+ return(v);
+}
+static void FillTensor(CTensor<type_t> &t,double scale)
+{
+ for(uint32_t w=0;w<t.GetSizeW();w++)
+  for(uint32_t z=0;z<t.GetSizeZ();z++)
+   for(uint32_t y=0;y<t.GetSizeY();y++)
+    for(uint32_t x=0;x<t.GetSizeX();x++) t.SetElement(w,z,y,x,static_cast<type_t>(Uniform()*scale));
+}
+
+static FILE *out_file=NULL;
+static void Dump(const char *name,const CTensor<type_t> &t)
+{
+ char label[32];
+ memset(label,0,sizeof(label));
+ strncpy(label,name,sizeof(label)-1);
+ uint32_t dims[4]={t.GetSizeW(),t.GetSizeZ(),t.GetSizeY(),t.GetSizeX()};
+ fwrite(label,1,sizeof(label),out_file);
+ fwrite(dims,sizeof(uint32_t),4,out_file);
+ for(uint32_t w=0;w<dims[0];w++)
+  for(uint32_t z=0;z<dims[1];z++)
+   for(uint32_t y=0;y<dims[2];y++)
+    for(uint32_t x=0;x<dims[3];x++)
+    {
+     float v=t.GetElement(w,z,y,x);
+     fwrite(&v,sizeof(float),1,out_file);
+    }
+}
+// the saved form of a layer (what Save() wrote), as one row of doubles converted to float
+static void DumpStream(const char *name,CMemoryStream &stream,size_t skip_bytes,uint32_t tensors)
+{
+ stream.Rewind();
+ for(size_t n=0;n<skip_bytes;n++) stream.LoadUInt8();
+ for(uint32_t i=0;i<tensors;i++)
+ {
+  uint32_t w=stream.LoadUInt32(),z=stream.LoadUInt32(),y=stream.LoadUInt32(),x=stream.LoadUInt32();
+  CTensor<type_t> t(w,z,y,x);
+  for(uint32_t a=0;a<w;a++) for(uint32_t b=0;b<z;b++) for(uint32_t c=0;c<y;c++) for(uint32_t d=0;d<x;d++) t.SetElement(a,b,c,d,static_cast<type_t>(stream.LoadDouble()));
+  char label[32];
+  snprintf(label,sizeof(label),"%s.%u",name,i);
+  Dump(label,t);
+ }
+}
+
+static const uint32_t BATCH=6;
+
+static void ChainA(void)
+{
+ CNetLayerConvolutionInput<type_t> input(3,16,16,BATCH);
+ CNetLayerConvolution<type_t> conv(8,4,2,2,1,1,&input,BATCH);
+ CNetLayerFunction<type_t> f1(NNeuron::NEURON_FUNCTION_LEAKY_RELU,&conv,BATCH);
+ CNetLayerLinear<type_t> lin(24,&f1,BATCH);
+ CNetLayerFunction<type_t> f2(NNeuron::NEURON_FUNCTION_SIGMOID,&lin,BATCH);
+
+ CMemoryStream conv_w;
+ conv_w.SaveUInt32(8);conv_w.SaveInt32(4);conv_w.SaveInt32(4);conv_w.SaveInt32(3);conv_w.SaveInt32(2);conv_w.SaveInt32(2);conv_w.SaveInt32(1);conv_w.SaveInt32(1);
+ conv_w.PutTensor(1,1,8,3*16,Values(8*48,0.2));
+ conv_w.PutTensor(1,8,1,1,Values(8,0.1));
+ conv.Load(&conv_w);
+ CMemoryStream lin_w;
+ lin_w.PutTensor(1,1,24,8*8*8,Values(24*512,0.08));
+ lin_w.PutTensor(1,1,24,1,Values(24,0.1));
+ lin.Load(&lin_w);
+
+ CTensor<type_t> image(BATCH,3,16,16);
+ FillTensor(image,1.0);
+ input.SetOutput(image);
+ INetLayer<type_t> *layers[5]={&input,&conv,&f1,&lin,&f2};
+ for(int n=0;n<5;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+ for(int n=0;n<5;n++) layers[n]->Forward();
+ Dump("A.conv",conv.GetOutputTensor());
+ Dump("A.leaky",f1.GetOutputTensor());
+ Dump("A.linear",lin.GetOutputTensor());
+ Dump("A.sigmoid",f2.GetOutputTensor());
+
+ CTensor<type_t> error(BATCH,1,24,1);
+ FillTensor(error,0.5);
+ f2.SetOutputError(error);
+ for(int n=4;n>=1;n--) layers[n]->TrainingBackward(true);
+ Dump("A.delta_linear",lin.GetDeltaTensor());
+ Dump("A.delta_leaky",f1.GetDeltaTensor());
+ Dump("A.delta_conv",conv.GetDeltaTensor());
+ for(int n=1;n<5;n++) layers[n]->TrainingUpdateWeight(0.05,1);
+ CMemoryStream conv_saved,lin_saved;
+ conv.Save(&conv_saved);
+ lin.Save(&lin_saved);
+ DumpStream("A.conv_updated",conv_saved,8*sizeof(int32_t),2);
+ DumpStream("A.linear_updated",lin_saved,0,2);
+}
+
+static void ChainB(void)
+{
+ CNetLayerConvolutionInput<type_t> input(8,4,4,BATCH);
+ CNetLayerBackConvolution<type_t> tconv(4,3,2,2,1,1,&input,BATCH);
+ CNetLayerFunction<type_t> f(NNeuron::NEURON_FUNCTION_TANGENCE,&tconv,BATCH);
+
+ CMemoryStream w;
+ w.SaveUInt32(8);w.SaveInt32(4);w.SaveInt32(4);w.SaveInt32(3);w.SaveInt32(2);w.SaveInt32(2);w.SaveInt32(1);w.SaveInt32(1);
+ w.PutTensor(1,1,8,3*16,Values(8*48,0.3));   // row = input channel, column = output channel * 16 + tap
+ w.PutTensor(1,8,1,1,std::vector<double>(8,0.0));
+ tconv.Load(&w);
+
+ CTensor<type_t> x(BATCH,8,4,4);
+ FillTensor(x,1.0);
+ input.SetOutput(x);
+ INetLayer<type_t> *layers[3]={&input,&tconv,&f};
+ for(int n=0;n<3;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+ for(int n=0;n<3;n++) layers[n]->Forward();
+ Dump("B.tconv",tconv.GetOutputTensor());
+ Dump("B.tanh",f.GetOutputTensor());
+ CTensor<type_t> error(BATCH,3,8,8);
+ FillTensor(error,0.5);
+ f.SetOutputError(error);
+ for(int n=2;n>=1;n--) layers[n]->TrainingBackward(true);
+ Dump("B.delta_tconv",tconv.GetDeltaTensor());
+ for(int n=1;n<3;n++) layers[n]->TrainingUpdateWeight(0.05,1);
+ CMemoryStream saved;
+ tconv.Save(&saved);
+ DumpStream("B.tconv_updated",saved,8*sizeof(int32_t),2);
+}
+
+#ifndef USE_CPU
+static void ChainC(void)
+{
+ CNetLayerConvolutionInput<type_t> input(4,5,5,BATCH);
+ CNetLayerBatchNormalization<type_t> bn(0.9f,&input,BATCH);
+ CNetLayerFunction<type_t> f(NNeuron::NEURON_FUNCTION_RELU,&bn,BATCH);
+ CMemoryStream w;
+ std::vector<double> beta=Values(100,0.5),gamma=Values(100,1.0);
+ w.PutTensor(1,4,5,5,beta);
+ w.PutTensor(1,4,5,5,gamma);
+ w.PutTensor(1,4,5,5,std::vector<double>(100,0.0));
+ w.PutTensor(1,4,5,5,std::vector<double>(100,1.0));
+ w.SaveDouble(0.9);
+ bn.Load(&w);
+ CTensor<type_t> x(BATCH,4,5,5);
+ FillTensor(x,2.0);
+ input.SetOutput(x);
+ INetLayer<type_t> *layers[3]={&input,&bn,&f};
+ for(int n=0;n<3;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+ for(int n=0;n<3;n++) layers[n]->Forward();
+ Dump("C.input",x);
+ CTensor<type_t> tb(1,4,5,5),tg(1,4,5,5);
+ for(uint32_t n=0;n<100;n++) {tb.SetElement(0,n/25,(n%25)/5,n%5,static_cast<type_t>(beta[n]));tg.SetElement(0,n/25,(n%25)/5,n%5,static_cast<type_t>(gamma[n]));}
+ Dump("C.beta",tb);
+ Dump("C.gamma",tg);
+ Dump("C.bn",bn.GetOutputTensor());
+ Dump("C.relu",f.GetOutputTensor());
+ CTensor<type_t> error(BATCH,4,5,5);
+ FillTensor(error,0.5);
+ Dump("C.error",error);
+ f.SetOutputError(error);
+ for(int n=2;n>=1;n--) layers[n]->TrainingBackward(true);
+ Dump("C.delta_bn",bn.GetDeltaTensor());
+ Dump("C.prev_error",input.GetDeltaTensor());   // the input layer hands back its own tensor: unchanged input
+}
+#endif
+
+int main(int argc,char **argv)
+{
+ if (argc<2) {fprintf(stderr,"usage: %s <output file>\n",argv[0]);return(2);}
+ out_file=fopen(argv[1],"wb");
+ if (out_file==NULL) return(2);
+ try
+ {
+  ChainA();
+  ChainB();
+#ifndef USE_CPU
+  ChainC();
+#endif
+ }
+ catch(const char *message)
+ {
+  fprintf(stderr,"exception: %s\n",message);
+  return(1);
+ }
+ fclose(out_file);
+ return(0);
+}

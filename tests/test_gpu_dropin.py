@@ -1,0 +1,79 @@
+"""The drop-in boundary on the GPU, from C++:
+
+* `ctensor_selftest` -- the checks of the reference's CTensorTest::Test() written against the drop-in
+  CTensor / CTensorMath / CTensorConv classes (every op runs through libmi355tensor.so);
+* `layers_mi355` vs `layers_cpu` -- the reference's OWN layer classes (convolution, transposed convolution, linear,
+  function, batch normalisation), compiled in the authoring container from /root/reference, once on the drop-in
+  classes and once on the reference's CPU classes: forward outputs, back-propagated deltas and the weights after
+  one gradient step must agree within 1e-4 (max|a-b| / max|b| per tensor).  Skipped where those binaries are absent.
+"""
+import os
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+
+import layer_sequences as seq
+from conftest import ROOT, rel_err
+
+pytestmark = pytest.mark.gpu
+
+SELFTEST = os.path.join(ROOT, "cuda-cnn-gan-vae_amd", "dropin", "ctensor_selftest")
+LAYERS_GPU = os.path.join(ROOT, "oracle", "_ref", "layers_mi355")
+LAYERS_CPU = os.path.join(ROOT, "oracle", "_ref", "layers_cpu")
+
+
+def read_dump(path):
+    out, data, pos = {}, open(path, "rb").read(), 0
+    while pos < len(data):
+        name = data[pos:pos + 32].split(b"\0")[0].decode()
+        dims = struct.unpack_from("<4I", data, pos + 32)
+        n = int(np.prod(dims))
+        out[name] = np.frombuffer(data, np.float32, n, pos + 48).reshape(dims)
+        pos += 48 + 4 * n
+    return out
+
+
+def test_cpp_selftest_on_the_dropin_classes():
+    assert os.path.exists(SELFTEST), "build it with `make -C cuda-cnn-gan-vae_amd`"
+    run = subprocess.run([SELFTEST], capture_output=True, text=True, timeout=120)
+    print(run.stdout[-3000:], run.stderr[-2000:])
+    assert run.returncode == 0 and "ALL PASS" in run.stdout and "FAIL" not in run.stdout
+    assert run.stdout.count("PASS") >= 18
+
+
+@pytest.fixture(scope="module")
+def dumps(tmp_path_factory):
+    if not (os.path.exists(LAYERS_GPU) and os.path.exists(LAYERS_CPU)):
+        pytest.skip("oracle/_ref/layers_* not built (they need /root/reference)")
+    d = tmp_path_factory.mktemp("layers")
+    files = {}
+    for tag, exe in (("gpu", LAYERS_GPU), ("cpu", LAYERS_CPU)):
+        files[tag] = str(d / (tag + ".bin"))
+        run = subprocess.run([exe, files[tag]], capture_output=True, text=True, timeout=180)
+        assert run.returncode == 0, run.stderr
+    return read_dump(files["gpu"]), read_dump(files["cpu"])
+
+
+def test_reference_layers_agree_on_both_tensor_paths(dumps):
+    gpu, cpu = dumps
+    shared = [k for k in cpu if k in gpu]
+    assert len(shared) >= 16 and any(k.startswith("B.") for k in shared)
+    for key in shared:
+        assert gpu[key].shape == cpu[key].shape, key
+        assert rel_err(gpu[key], cpu[key]) <= 1e-4, key
+    # the update step really moved the weights (the comparison above is not between two untouched copies)
+    assert not np.array_equal(cpu["A.conv_updated.0"], cpu["A.conv_updated.0"] * 0)
+
+
+def test_reference_batchnorm_layer_matches_the_oracle_sequence(dumps, oracle):
+    """The reference's batch-norm layer does not build on its own CPU classes, so its run on the drop-in classes is
+    checked against the oracle's restatement of the layer's op sequence."""
+    gpu, _ = dumps
+    x, gamma, beta, err = gpu["C.input"], gpu["C.gamma"], gpu["C.beta"], gpu["C.error"]
+    want = seq.batchnorm_forward_train(oracle, x, gamma, beta)
+    assert rel_err(gpu["C.bn"], want["out"]) <= 1e-4
+    assert rel_err(gpu["C.relu"], oracle.apply_func(want["out"], "relu")) <= 1e-4
+    delta = oracle.tensor_item_production(err, oracle.apply_func(want["out"], "relu", differential=True))
+    assert rel_err(gpu["C.delta_bn"], delta) <= 1e-4
