@@ -265,10 +265,15 @@ __global__ __launch_bounds__(256) void tconv_small_kernel(TconvArgs args) {
 // thread issues 9 loads for 16*CO multiply-adds.  The loads are buffer loads whose 9 byte offsets (or the
 // out-of-range marker for neighbours outside the image) are computed once; the channel advances through the
 // scalar offset.  The 16*CO coefficients of a channel are uniform and come through the scalar cache.
+// The input channels are split over the 4 wavefronts of a block (64 input pixels per block): four times as many
+// loads in flight, partial sums combined through LDS.
 template <int CO>
 __global__ __launch_bounds__(256) void tconv_k4s2_small_kernel(TconvArgs args) {
+  constexpr int SLICES = 4, PIX = 64;
+  __shared__ float part[SLICES - 1][4 * CO][PIX];
   const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W;
-  const uint32_t n = blockIdx.x * 256 + threadIdx.x;
+  const uint32_t pix = threadIdx.x % PIX, slice = threadIdx.x / PIX;   // the slice is uniform over a wavefront
+  const uint32_t n = blockIdx.x * PIX + pix;
   const bool live = n < args.out_w * HW;
   const uint32_t g = (live ? n : 0) / HW, r = (live ? n : 0) % HW, qy = r / W, qx = r % W;
   __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta, args.in_w * C * HW * 4u);
@@ -286,8 +291,11 @@ __global__ __launch_bounds__(256) void tconv_k4s2_small_kernel(TconvArgs args) {
 #pragma unroll
   for (int i = 0; i < 4 * CO; i++) (&acc[0][0][0])[i] = 0.f;
   const uint32_t M = args.M;
-#pragma unroll 2
-  for (uint32_t ci = 0; ci < C; ci++) {
+  const uint32_t per = (C + SLICES - 1) / SLICES;
+  const uint32_t c_begin = __builtin_amdgcn_readfirstlane(slice * per);
+  const uint32_t c_end = c_begin + per < C ? c_begin + per : C;
+#pragma unroll 4
+  for (uint32_t ci = c_begin; ci < c_end; ci++) {
     const uint32_t soff = ci * HW * 4u;
     float v[3][3];
 #pragma unroll
@@ -312,7 +320,16 @@ __global__ __launch_bounds__(256) void tconv_k4s2_small_kernel(TconvArgs args) {
         }
       }
   }
-  if (!live) return;
+  if (slice > 0) {
+#pragma unroll
+    for (int i = 0; i < 4 * CO; i++) part[slice - 1][i][pix] = (&acc[0][0][0])[i];
+  }
+  __syncthreads();
+  if (slice > 0 || !live) return;
+#pragma unroll
+  for (int i = 0; i < 4 * CO; i++)
+#pragma unroll
+    for (int sl = 0; sl < SLICES - 1; sl++) (&acc[0][0][0])[i] += part[sl][i][pix];
   const uint32_t OW = 2 * W, OHW = 4 * HW;
   const float bsum = args.ep.tap_bias ? args.ep.tap_bias[g % args.ep.bias_w] : 0.f;
 #pragma unroll
@@ -348,7 +365,7 @@ int launch_tconv_small(const char *name, TconvArgs &args, uint32_t max_n) {
     k4s2 = args.ph[f].py == f / 2 && args.ph[f].px == f % 2 && args.ph[f].offy == (int32_t)(f / 2) - 1 && args.ph[f].offx == (int32_t)(f % 2) - 1 &&
            args.ph[f].qh == args.H && args.ph[f].qw == args.W;
   if (k4s2) {
-    dim3 g4(cdiv((size_t)args.out_w * args.H * args.W, 256));
+    dim3 g4(cdiv((size_t)args.out_w * args.H * args.W, 64));
     if (args.M <= 1) tconv_k4s2_small_kernel<1><<<g4, 256, 0, mt::stream()>>>(args);
     else if (args.M <= 2) tconv_k4s2_small_kernel<2><<<g4, 256, 0, mt::stream()>>>(args);
     else if (args.M == 3) tconv_k4s2_small_kernel<3><<<g4, 256, 0, mt::stream()>>>(args);

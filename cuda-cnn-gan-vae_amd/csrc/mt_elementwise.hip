@@ -276,41 +276,63 @@ __global__ __launch_bounds__(EW_THREADS) void adam_kernel(float *weight, const f
 }
 
 // ---- batch normalisation over the batch axis, statistics per element (z,y,x) --------------------------------------
-// Pass 1: per column r, sums of d = x - x[0][r] and d*d over w (the shift keeps the one-pass variance stable),
-// the batch split over WS slices like add_sum_w.  Produces mean, biased variance and 1/sqrt(var+eps).
-template <int RB>
+// Pass 1: per column r, sums of d = x - x[0][r] and d*d over w (the shift keeps the one-pass variance stable).
+// A block owns 32 column groups of V columns (V = 4: 128-bit loads) and splits the batch over 8 slices that are
+// combined in LDS; the slice loop is unrolled so that several loads per thread are in flight.
+// Produces mean, biased variance and 1/sqrt(var+eps), and blends the running statistics.
+template <int V>
 __global__ __launch_bounds__(EW_THREADS) void bn_stats_kernel(const float *x, uint32_t W, uint32_t S, float inv_n, float eps, float *mean,
                                                               float *var, float *ivar, float *new_mean, float *new_var, float mom_old, float mom_new) {
-  constexpr int WS = EW_THREADS / RB;
-  __shared__ float part[2][WS][RB];
-  int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
-  uint32_t r = blockIdx.x * RB + rl;
-  float s1 = 0.f, s2 = 0.f, shift = 0.f;
+  constexpr int RB = 32, WS = EW_THREADS / RB;
+  __shared__ float part[2][WS][RB * V];
+  const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
+  const uint32_t r = (blockIdx.x * RB + rl) * V;
+  float s1[V], s2[V], shift[V];
+#pragma unroll
+  for (int v = 0; v < V; v++) { s1[v] = 0.f; s2[v] = 0.f; shift[v] = 0.f; }
   if (r < S) {
-    shift = x[r];
-    for (uint32_t w = ws; w < W; w += WS) {
-      float d = x[(size_t)w * S + r] - shift;
-      s1 += d;
-      s2 += d * d;
+    if constexpr (V == 4) {
+      float4 t = *reinterpret_cast<const float4 *>(x + r);
+      shift[0] = t.x; shift[1] = t.y; shift[2] = t.z; shift[3] = t.w;
+#pragma unroll 4
+      for (uint32_t w = ws; w < W; w += WS) {
+        float4 q = *reinterpret_cast<const float4 *>(x + (size_t)w * S + r);
+        float d0 = q.x - shift[0], d1 = q.y - shift[1], d2 = q.z - shift[2], d3 = q.w - shift[3];
+        s1[0] += d0; s1[1] += d1; s1[2] += d2; s1[3] += d3;
+        s2[0] += d0 * d0; s2[1] += d1 * d1; s2[2] += d2 * d2; s2[3] += d3 * d3;
+      }
+    } else {
+      shift[0] = x[r];
+#pragma unroll 4
+      for (uint32_t w = ws; w < W; w += WS) {
+        float d = x[(size_t)w * S + r] - shift[0];
+        s1[0] += d;
+        s2[0] += d * d;
+      }
     }
   }
-  part[0][ws][rl] = s1;
-  part[1][ws][rl] = s2;
-  __syncthreads();
-  if (ws != 0 || r >= S) return;
-  s1 = 0.f; s2 = 0.f;
 #pragma unroll
-  for (int i = 0; i < WS; i++) { s1 += part[0][i][rl]; s2 += part[1][i][rl]; }
-  float md = s1 * inv_n;                  // mean of the shifted data
-  float mu = shift + md;
-  float vr = (s2 - s1 * md) * inv_n;      // sum((d-md)^2)/N
+  for (int v = 0; v < V; v++) { part[0][ws][rl * V + v] = s1[v]; part[1][ws][rl * V + v] = s2[v]; }
+  __syncthreads();
+  // the first RB*V threads finish one column each
+  const int c = threadIdx.x;
+  if (c >= RB * V) return;
+  const uint32_t rc = blockIdx.x * RB * V + c;
+  if (rc >= S) return;
+  float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < WS; i++) { a1 += part[0][i][c]; a2 += part[1][i][c]; }
+  const float sh = x[rc];
+  float md = a1 * inv_n;                  // mean of the shifted data
+  float mu = sh + md;
+  float vr = (a2 - a1 * md) * inv_n;      // sum((d-md)^2)/N
   if (vr < 0.f) vr = 0.f;
   float iv = (float)(1.0 / (double)(sqrtf(vr + eps) * 1.f));
-  mean[r] = mu;
-  var[r] = vr;
-  ivar[r] = iv;
-  if (new_mean) new_mean[r] = (mom_old * new_mean[r]) + (mom_new * mu);
-  if (new_var) new_var[r] = (mom_old * new_var[r]) + (mom_new * vr);
+  mean[rc] = mu;
+  var[rc] = vr;
+  ivar[rc] = iv;
+  if (new_mean) new_mean[rc] = (mom_old * new_mean[rc]) + (mom_new * mu);
+  if (new_var) new_var[rc] = (mom_old * new_var[rc]) + (mom_new * vr);
 }
 
 // Pass 2: out = func(gamma * ((x - mean) * ivar) + beta), optionally storing xhat.
@@ -537,10 +559,10 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
   float mom_new = (float)(1.0 - (double)momentum);  // and 1.0-Momentum, rounded once
   {
   mt::ProfileScope prof("bn_stats");
-  if (S >= 65536)
-    bn_stats_kernel<256><<<cdiv(S, 256), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, new_mean ? new_mean->p : nullptr, new_variable ? new_variable->p : nullptr, momentum, mom_new);
+  if (S % 4 == 0 && aligned16(in->p))
+    bn_stats_kernel<4><<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, new_mean ? new_mean->p : nullptr, new_variable ? new_variable->p : nullptr, momentum, mom_new);
   else
-    bn_stats_kernel<32><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, new_mean ? new_mean->p : nullptr, new_variable ? new_variable->p : nullptr, momentum, mom_new);
+    bn_stats_kernel<1><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, new_mean ? new_mean->p : nullptr, new_variable ? new_variable->p : nullptr, momentum, mom_new);
   }
   MT_LAUNCH_CHECK("bn_stats");
   bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(pm) && aligned16(pi) && (!xhat || aligned16(xhat->p));
