@@ -353,6 +353,14 @@ __device__ __forceinline__ void lds_put(float *dst, const float (&v)[E]) {
   }
 }
 
+// Workgroup barrier that orders LDS traffic only: global loads issued before it stay in flight across it
+// (__syncthreads() would also wait for them).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // One (BM x BN) block of C at (m0, n0).  `smem` holds LDS_FLOATS floats, 16-byte aligned.
 //
 // Feeding v_mfma_f32_32x32x2_f32: lanes 0-31 supply k = 2s and lanes 32-63 supply k = 2s+1 of step s, for the row
@@ -399,46 +407,74 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
   float *a_put = As + a_row * LDK + a_k, *b_put = Bs + b_row * LDK + b_k;
   lds_put<EA>(a_put, ra);
   lds_put<EB>(b_put, rb);
-  __syncthreads();
-
-  const int lrow = lane & 31, lk = lane >> 5;
-  const float *a_get = As + (wm * TM * 32 + lrow) * LDK + lk * 4;
-  const float *b_get = Bs + (wn * TN * 32 + lrow) * LDK + lk * 4;
-  for (uint32_t kt = 0; kt < nk; kt++) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < nk;
-    // loads of the next tile: issued now, consumed after this tile's matrix instructions (the extra fetch of the
-    // last iteration lies beyond K, is answered with zeros by the range check and is never stored)
+  if (nk > 1) {
     a.next();
     b.next();
     a.template fetch<EA>(ra);
     b.template fetch<EB>(rb);
-    __builtin_amdgcn_sched_barrier(0);  // keep the loads above the matrix instructions: their latency hides behind them
+  }
+  lds_barrier();
+
+  const int lrow = lane & 31, lk = lane >> 5;
+  const float *a_get = As + (wm * TM * 32 + lrow) * LDK + lk * 4;
+  const float *b_get = Bs + (wn * TN * 32 + lrow) * LDK + lk * 4;
+  // fragments of one half tile (8 k): one 128-bit LDS read per 32 rows
+  float4 fa[2][TM], fb[2][TN];
+  auto read_half = [&](float4 (&av)[TM], float4 (&bv)[TN], int buf, int half) {
 #pragma unroll
-    for (int half = 0; half < 2; half++) {
-      float4 av[TM], bv[TN];
+    for (int i = 0; i < TM; i++) av[i] = *reinterpret_cast<const float4 *>(a_get + buf * BM * LDK + i * 32 * LDK + half * 8);
 #pragma unroll
-      for (int i = 0; i < TM; i++) av[i] = *reinterpret_cast<const float4 *>(a_get + cur * BM * LDK + i * 32 * LDK + half * 8);
+    for (int j = 0; j < TN; j++) bv[j] = *reinterpret_cast<const float4 *>(b_get + buf * BN * LDK + j * 32 * LDK + half * 8);
+  };
+  auto multiply = [&](const float4 (&av)[TM], const float4 (&bv)[TN]) {
 #pragma unroll
-      for (int j = 0; j < TN; j++) bv[j] = *reinterpret_cast<const float4 *>(b_get + cur * BN * LDK + j * 32 * LDK + half * 8);
+    for (int c = 0; c < 4; c++)  // consecutive matrix instructions go to different accumulators
 #pragma unroll
-      for (int c = 0; c < 4; c++)  // consecutive matrix instructions go to different accumulators
+      for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-          for (int j = 0; j < TN; j++) {
-            float x = c == 0 ? av[i].x : c == 1 ? av[i].y : c == 2 ? av[i].z : av[i].w;
-            float y = c == 0 ? bv[j].x : c == 1 ? bv[j].y : c == 2 ? bv[j].z : bv[j].w;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[i][j], 0, 0, 0);
-          }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (more) {
+        for (int j = 0; j < TN; j++) {
+          float x = c == 0 ? av[i].x : c == 1 ? av[i].y : c == 2 ? av[i].z : av[i].w;
+          float y = c == 0 ? bv[j].x : c == 1 ? bv[j].y : c == 2 ? bv[j].z : bv[j].w;
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[i][j], 0, 0, 0);
+        }
+  };
+
+  // Software pipeline, two half tiles per step.  While the matrix instructions of one half run, the wavefront
+  // already holds the fragments of the next half in registers, tile t+1 is being written to the other LDS buffer
+  // and the global loads of tile t+2 are in flight, so a wavefront keeps its matrix pipe busy on its own:
+  //
+  //   first half   read fragments (t, half 1) | write tile t+1 to LDS | issue loads of tile t+2 | multiply (t, half 0)
+  //   barrier      tile t+1 is complete in LDS and nobody reads the buffer of tile t any more
+  //   second half  read fragments (t+1, half 0) | multiply (t, half 1)
+  // The last two steps have nothing left to write or load; peeling them keeps every step free of branches, so
+  // the compiler counts outstanding LDS operations exactly and waits for no more than it must.
+  auto step = [&](uint32_t kt, auto write_next, auto load_after_next) {
+    const int cur = kt & 1;
+    read_half(fa[1], fb[1], cur, 1);
+    if constexpr (decltype(write_next)::value) {
       lds_put<EA>(a_put + (cur ^ 1) * BM * LDK, ra);
       lds_put<EB>(b_put + (cur ^ 1) * BN * LDK, rb);
     }
-    __syncthreads();
-  }
+    if constexpr (decltype(load_after_next)::value) {  // never past K: the scalar part of a buffer address is not range checked
+      a.next();
+      b.next();
+      a.template fetch<EA>(ra);
+      b.template fetch<EB>(rb);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // memory instructions first, their latency hides behind the multiplies
+    multiply(fa[0], fb[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    lds_barrier();
+    if constexpr (decltype(write_next)::value) read_half(fa[0], fb[0], cur ^ 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(fa[1], fb[1]);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  read_half(fa[0], fb[0], 0, 0);
+  uint32_t kt = 0;
+  for (; kt + 2 < nk; kt++) step(kt, std::true_type{}, std::true_type{});
+  if (kt + 1 < nk) step(kt++, std::true_type{}, std::false_type{});
+  step(kt, std::false_type{}, std::false_type{});
 
   // accumulator layout of v_mfma_f32_32x32x2_f32: register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32]
 #pragma unroll
