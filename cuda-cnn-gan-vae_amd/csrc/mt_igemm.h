@@ -390,7 +390,7 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
   a.bind(m0 + a_row);
   b.bind(n0 + b_row);
 
-  float ra[EA], rb[EB];
+  float ra[2][EA], rb[2][EB];  // two register sets: the global loads run two tiles ahead of the LDS writes
   floatx16 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; i++)
@@ -402,18 +402,27 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
   const uint32_t nk = (K + BK - 1) / BK;
   a.template seek<EA>(a_k);
   b.template seek<EB>(b_k);
-  a.template fetch<EA>(ra);
-  b.template fetch<EB>(rb);
   float *a_put = As + a_row * LDK + a_k, *b_put = Bs + b_row * LDK + b_k;
-  lds_put<EA>(a_put, ra);
-  lds_put<EB>(b_put, rb);
-  if (nk > 1) {
-    a.next();
-    b.next();
-    a.template fetch<EA>(ra);
-    b.template fetch<EB>(rb);
-  }
-  lds_barrier();
+  // tile 0 goes to LDS, tiles 1 and 2 (where they exist) are requested; the two cases are separate straight-line
+  // paths so that the count of loads in flight is known at compile time on each of them
+  auto load_tile = [&](int set, bool advance) {
+    // the same issue order everywhere (A, then B), so that the wait before an LDS write names exactly the loads
+    // it needs and leaves the younger ones in flight
+    if (advance) { a.next(); b.next(); }
+    __builtin_amdgcn_sched_barrier(0);
+    a.template fetch<EA>(ra[set]);
+    __builtin_amdgcn_sched_barrier(0);
+    b.template fetch<EB>(rb[set]);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto prologue = [&](auto tiles) {
+    load_tile(0, false);
+    lds_put<EA>(a_put, ra[0]);
+    lds_put<EB>(b_put, rb[0]);
+    if constexpr (decltype(tiles)::value > 1) load_tile(1, true);
+    if constexpr (decltype(tiles)::value > 2) load_tile(0, true);
+    lds_barrier();
+  };
 
   const int lrow = lane & 31, lk = lane >> 5;
   const float *a_get = As + (wm * TM * 32 + lrow) * LDK + lk * 4;
@@ -441,40 +450,65 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
 
   // Software pipeline, two half tiles per step.  While the matrix instructions of one half run, the wavefront
   // already holds the fragments of the next half in registers, tile t+1 is being written to the other LDS buffer
-  // and the global loads of tile t+2 are in flight, so a wavefront keeps its matrix pipe busy on its own:
+  // and the global loads of tiles t+2 and t+3 are in flight, so a wavefront keeps its matrix pipe busy on its own:
   //
-  //   first half   read fragments (t, half 1) | write tile t+1 to LDS | issue loads of tile t+2 | multiply (t, half 0)
+  //   first half   read fragments (t, half 1) | write tile t+1 to LDS | issue loads of tile t+3 | multiply (t, half 0)
   //   barrier      tile t+1 is complete in LDS and nobody reads the buffer of tile t any more
   //   second half  read fragments (t+1, half 0) | multiply (t, half 1)
-  // The last two steps have nothing left to write or load; peeling them keeps every step free of branches, so
-  // the compiler counts outstanding LDS operations exactly and waits for no more than it must.
-  auto step = [&](uint32_t kt, auto write_next, auto load_after_next) {
-    const int cur = kt & 1;
+  //
+  // Steps come in pairs so that the LDS buffer and the register set of a step are compile-time constants, and the
+  // last (up to four) steps, which have less left to write or load, are peeled: every step is free of branches, the
+  // compiler counts outstanding memory operations exactly and waits for no more than it must.  Nothing is loaded
+  // past K: the scalar part of a buffer address is not range checked.
+  auto step = [&](auto parity, auto write_next, auto load_ahead) {
+    constexpr int cur = decltype(parity)::value, nxt = cur ^ 1;  // tile t lives in LDS buffer cur, tile t+1 in register set nxt
     read_half(fa[1], fb[1], cur, 1);
     if constexpr (decltype(write_next)::value) {
-      lds_put<EA>(a_put + (cur ^ 1) * BM * LDK, ra);
-      lds_put<EB>(b_put + (cur ^ 1) * BN * LDK, rb);
+      lds_put<EA>(a_put + nxt * BM * LDK, ra[nxt]);
+      lds_put<EB>(b_put + nxt * BN * LDK, rb[nxt]);
     }
-    if constexpr (decltype(load_after_next)::value) {  // never past K: the scalar part of a buffer address is not range checked
-      a.next();
-      b.next();
-      a.template fetch<EA>(ra);
-      b.template fetch<EB>(rb);
-    }
+    if constexpr (decltype(load_ahead)::value) load_tile(nxt, true);
     __builtin_amdgcn_sched_barrier(0);  // memory instructions first, their latency hides behind the multiplies
     multiply(fa[0], fb[0]);
     __builtin_amdgcn_sched_barrier(0);
     lds_barrier();
-    if constexpr (decltype(write_next)::value) read_half(fa[0], fb[0], cur ^ 1, 0);
+    if constexpr (decltype(write_next)::value) read_half(fa[0], fb[0], nxt, 0);
     __builtin_amdgcn_sched_barrier(0);
     multiply(fa[1], fb[1]);
     __builtin_amdgcn_sched_barrier(0);
   };
-  read_half(fa[0], fb[0], 0, 0);
-  uint32_t kt = 0;
-  for (; kt + 2 < nk; kt++) step(kt, std::true_type{}, std::true_type{});
-  if (kt + 1 < nk) step(kt++, std::true_type{}, std::false_type{});
-  step(kt, std::false_type{}, std::false_type{});
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
+  using Yes = std::true_type;
+  using No = std::false_type;
+  if (nk >= 3) {
+    prologue(std::integral_constant<int, 3>{});
+    read_half(fa[0], fb[0], 0, 0);
+    uint32_t left = nk;
+    for (; left > 4; left -= 2) {
+      step(Even{}, Yes{}, Yes{});
+      step(Odd{}, Yes{}, Yes{});
+    }
+    if (left == 4) {
+      step(Even{}, Yes{}, Yes{});
+      step(Odd{}, Yes{}, No{});
+      step(Even{}, Yes{}, No{});
+      step(Odd{}, No{}, No{});
+    } else {
+      step(Even{}, Yes{}, No{});
+      step(Odd{}, Yes{}, No{});
+      step(Even{}, No{}, No{});
+    }
+  } else if (nk == 2) {
+    prologue(std::integral_constant<int, 2>{});
+    read_half(fa[0], fb[0], 0, 0);
+    step(Even{}, Yes{}, No{});
+    step(Odd{}, No{}, No{});
+  } else {
+    prologue(std::integral_constant<int, 1>{});
+    read_half(fa[0], fb[0], 0, 0);
+    step(Even{}, No{}, No{});
+  }
 
   // accumulator layout of v_mfma_f32_32x32x2_f32: register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32]
 #pragma unroll
