@@ -93,8 +93,12 @@ __device__ __forceinline__ float apply_func(int func, float v) {
   }
 }
 
-// For matrix-core epilogues, where the store loop is unrolled 64 times: the cheap functions stay inline, the
-// transcendental ones are one shared out-of-line body (func is uniform, so the branch costs nothing).
+// Functions cheap enough to live in the epilogue of a matrix-core kernel; after the others the host runs the
+// elementwise kernel over the output (same arithmetic, one more pass).
+inline bool epilogue_func(int func) { return func == MT_F_NONE || func == MT_F_LINEAR || func == MT_F_RELU || func == MT_F_LEAKY_RELU; }
+
+// For kernels that hold few values per thread: the cheap functions stay inline, the transcendental ones are one
+// shared out-of-line body (func is uniform, so the branch costs nothing).
 __device__ __attribute__((noinline)) inline float apply_func_outlined(int func, float v) { return apply_func(func, v); }
 __device__ __forceinline__ float apply_func_epilogue(int func, float v) {
   if (func == MT_F_NONE || func == MT_F_LINEAR) return v;

@@ -428,7 +428,9 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
   b.sy = sy; b.sx = sx; b.py = py; b.px = px;
   Epilogue ep{};
   ep.C = out->p; ep.row_stride = OHW; ep.inner = OHW; ep.g_stride = (size_t)ka * OHW;
-  ep.bias = bias->p; ep.bias_mode = 1; ep.bias_w = bias->w; ep.bias_stride = ka; ep.func = func;
+  ep.bias = bias->p; ep.bias_mode = 1; ep.bias_w = bias->w; ep.bias_stride = ka;
+  const bool func_later = !mt::epilogue_func(func);
+  ep.func = func_later ? MT_F_NONE : func;
   if (kernel->w == 1) {  // one kernel set for the whole batch: fold the batch into the columns
     b.R = out->w * OHW;
     const uint32_t taps = (uint32_t)ky * kx;
@@ -436,16 +438,19 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
       SrcIm2colFixed bf{};
       bf.p = b.p; bf.in_w = b.in_w; bf.C = b.C; bf.H = b.H; bf.W = b.W; bf.KY = b.KY; bf.KX = b.KX; bf.OHW = b.OHW; bf.OW = b.OW; bf.R = b.R; bf.K = b.K;
       bf.sy = sy; bf.sx = sx; bf.py = py; bf.px = px;
-      return with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return launch(name, a, bf, ep, ka, out->w * OHW, K, 1); });
+      rc = with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return launch(name, a, bf, ep, ka, out->w * OHW, K, 1); });
+    } else {
+      rc = with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return launch(name, a, b, ep, ka, out->w * OHW, K, 1); });
     }
-    return with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return launch(name, a, b, ep, ka, out->w * OHW, K, 1); });
+  } else {
+    // kernels differ per sample: one product per output image
+    Batch abt;
+    abt.wmod = kernel->w; abt.stride = (size_t)kernel->z * kernel->y * kernel->x;
+    b.bt.wmod = image->w; b.bt.stride = (size_t)kz * image->y * image->x; b.in_w = 1; b.R = OHW;
+    ep.bt.wmod = out->w; ep.bt.stride = (size_t)ka * OHW;
+    rc = with_row_k(kernel->p, kernel->x, ka, K, abt, [&](auto a) { return launch(name, a, b, ep, ka, OHW, K, out->w); });
   }
-  // kernels differ per sample: one product per output image
-  Batch abt;
-  abt.wmod = kernel->w; abt.stride = (size_t)kernel->z * kernel->y * kernel->x;
-  b.bt.wmod = image->w; b.bt.stride = (size_t)kz * image->y * image->x; b.in_w = 1; b.R = OHW;
-  ep.bt.wmod = out->w; ep.bt.stride = (size_t)ka * OHW;
-  return with_row_k(kernel->p, kernel->x, ka, K, abt, [&](auto a) { return launch(name, a, b, ep, ka, OHW, K, out->w); });
+  return rc == MT_OK && func_later ? mt_apply_func(out, out, func) : rc;
 }
 
 int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
@@ -515,7 +520,10 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     rc = launch_tconv_small(name, args, max_n);
     if (rc >= 0) return rc;
   }
-  return launch_tconv(name, args, max_n);
+  if (mt::epilogue_func(func)) return launch_tconv(name, args, max_n);
+  args.ep.func = MT_F_NONE;
+  rc = launch_tconv(name, args, max_n);
+  return rc == MT_OK ? mt_apply_func(out, out, func) : rc;
 }
 
 int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,

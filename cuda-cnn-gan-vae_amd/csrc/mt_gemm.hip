@@ -111,7 +111,9 @@ int mt_linear_forward_func(const mt_tensor *out, const mt_tensor *weight, const 
   in.x = 1;
   if (weight->w != 1 || weight->z != 1 || bias->w != 1 || bias->z != 1 || bias->x != 1 || bias->y != weight->y || out->w != input->w)
     return mt::fail(MT_E_SHAPE, "mt_linear_forward_func: weight must be [1,1,Out,In], bias [1,1,Out,1], output [B,1,Out,1]");
-  return product("mt_linear_forward_func", out, weight, &in, false, bias->p, func);
+  if (mt::epilogue_func(func)) return product("mt_linear_forward_func", out, weight, &in, false, bias->p, func);
+  int rc = product("mt_linear_forward_func", out, weight, &in, false, bias->p, MT_F_NONE);
+  return rc == MT_OK ? mt_apply_func(out, out, func) : rc;
 }
 
 }  // extern "C"

@@ -213,10 +213,11 @@ struct SrcIm2colFixed {
   template <int E>
   __device__ void seek(uint32_t k0) {  // k0 < BK
     static_assert(E <= 8, "at most eight elements per thread");
-    const uint32_t taps = KY * KX;
+    const uint32_t taps = KY * KX;  // taps divides BK = 16, so taps and KX are powers of two
+    const int lt = __builtin_ctz(taps), lx = __builtin_ctz(KX);
 #pragma unroll
     for (int i = 0; i < E; i++) {
-      uint32_t kk = k0 + i, cc = kk / taps, t = kk % taps, ty = t / KX, tx = t % KX;
+      uint32_t kk = k0 + i, cc = kk >> lt, t = kk & (taps - 1), ty = t >> lx, tx = t & (KX - 1);
       int32_t iy = iy0 + (int32_t)ty, ix = ix0 + (int32_t)tx;
       bool ok = imgoff != OOB && (uint32_t)iy < H && (uint32_t)ix < W;
       voff[i] = ok ? imgoff + ((cc * H + (uint32_t)iy) * W + (uint32_t)ix) * 4u : OOB;
@@ -300,7 +301,7 @@ struct Epilogue {
 
   struct Col {
     size_t off;
-    uint32_t g;
+    uint32_t g, bias_row;
     float extra;
   };
   __device__ void batch(uint32_t bz) { C += bt.offset(bz); g0 = bz / bt.zcount; }
@@ -308,6 +309,7 @@ struct Epilogue {
     Col c;
     c.g = g0 + n / inner;
     uint32_t r = n % inner;
+    c.bias_row = (c.g % bias_w) * bias_stride;
     c.extra = (bias && bias_mode == 2) ? bias[r] : 0.f;
     if (qw) {
       uint32_t qy = r / qw, qx = r % qw;
@@ -322,12 +324,46 @@ struct Epilogue {
     c.off = (size_t)(c.g - g0) * g_stride + r;
     return c;
   }
+  // one value (kernels that hold few values per thread)
   __device__ void store(const Col &c, uint32_t m, float v) const {
     float *dst = C + c.off + (size_t)m * row_stride;
     if (accumulate) v += *dst;
-    if (bias && bias_mode == 1) v += bias[(size_t)(c.g % bias_w) * bias_stride + m];
+    if (bias && bias_mode == 1) v += bias[c.bias_row + m];
     v += c.extra;
     *dst = apply_func_epilogue(func, v);
+  }
+  // One accumulator of v_mfma_f32_32x32x2_f32 for column c: register r holds row m_base + 8*(r/4) + r%4.
+  // Every option is tested once for the sixteen values, not once per value: old C, then the bias of the row, then
+  // the column's extra term, then the function (none, linear, ReLU or leaky ReLU), in this order.
+  template <bool FULL>
+  __device__ __forceinline__ void store_rows(const Col &c, uint32_t m_base, uint32_t M, floatx16 &v) const {
+    float *dst = C + c.off + (size_t)m_base * row_stride;
+#define MT_EACH_ROW(body)                                    \
+  _Pragma("unroll") for (int r = 0; r < 16; r++) {           \
+    const uint32_t dm = 8 * (r / 4) + (r & 3);               \
+    if (FULL || m_base + dm < M) { body; }                   \
+  }
+    if (accumulate) MT_EACH_ROW(v[r] += dst[(size_t)dm * row_stride]);
+    if (bias && bias_mode == 1) {
+      const float *bp = bias + c.bias_row + m_base;
+      MT_EACH_ROW(v[r] += bp[dm]);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) v[r] += c.extra;
+    if (func == MT_F_RELU) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) v[r] = v[r] > 0.f ? v[r] : 0.f;
+    } else if (func == MT_F_LEAKY_RELU) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) v[r] = v[r] > 0.f ? v[r] : (float)(0.1 * (double)v[r]);
+    }  // any other function is applied by the host in a pass of its own (see epilogue_func)
+    MT_EACH_ROW(dst[(size_t)dm * row_stride] = v[r]);
+#undef MT_EACH_ROW
+  }
+  __device__ __forceinline__ void store_block(const Col &c, uint32_t m_base, uint32_t M, floatx16 &v) const {
+    if (m_base >= M) return;
+    if (m_base + 28 <= M) store_rows<true>(c, m_base, M, v);
+    else store_rows<false>(c, m_base, M, v);
   }
 };
 
@@ -517,13 +553,7 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
     if (n >= N) continue;
     Epilogue::Col col = ep.column(n);
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        uint32_t m = m0 + (wm * TM + i) * 32 + 8 * (r / 4) + 4 * lk + (r & 3);
-        if (m < M) ep.store(col, m, acc[i][j][r]);
-      }
-    }
+    for (int i = 0; i < TM; i++) ep.store_block(col, m0 + (wm * TM + i) * 32 + 4 * lk, M, acc[i][j]);
   }
 }
 
@@ -539,7 +569,7 @@ __device__ __forceinline__ uint32_t xcd_swizzle(uint32_t L, uint32_t total) {
 // Generic launch: logical block index = (n tile, batch entry, m tile), n slowest, so concurrently running blocks
 // of one XCD share their B tile (the activations) and cycle through the A tiles (the weights).
 template <int TM, int TN, int WGM, int WGN, class SrcA, class SrcB>
-__global__ __launch_bounds__(THREADS) void igemm_kernel(SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, uint32_t tiles_m, uint32_t batches) {
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN == 1 ? 5 : TM * TN == 2 ? 3 : 2))) void igemm_kernel(SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, uint32_t tiles_m, uint32_t batches) {
   using TS = TileShape<TM, TN, WGM, WGN>;
   __shared__ float4 smem[TS::LDS_FLOATS / 4];
   uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
@@ -613,7 +643,7 @@ struct TconvArgs {
 
 // FIXED: every phase has taps that tile the k step (see SrcIm2colFixed)
 template <int TM, int TN, int WGM, int WGN, bool FIXED>
-__global__ __launch_bounds__(THREADS) void tconv_kernel(TconvArgs args) {
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN == 1 ? 5 : TM * TN == 2 ? 3 : 2))) void tconv_kernel(TconvArgs args) {
   using TS = TileShape<TM, TN, WGM, WGN>;
   __shared__ float4 smem[TS::LDS_FLOATS / 4];
   uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
