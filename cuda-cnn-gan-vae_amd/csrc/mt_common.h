@@ -97,6 +97,12 @@ __device__ __forceinline__ float apply_func(int func, float v) {
 // elementwise kernel over the output (same arithmetic, one more pass).
 inline bool epilogue_func(int func) { return func == MT_F_NONE || func == MT_F_LINEAR || func == MT_F_RELU || func == MT_F_LEAKY_RELU; }
 
+__device__ __forceinline__ float apply_func_cheap(int func, float v) {  // func satisfies epilogue_func()
+  if (func == MT_F_RELU) return v > 0.f ? v : 0.f;
+  if (func == MT_F_LEAKY_RELU) return v > 0.f ? v : (float)(0.1 * (double)v);
+  return v;
+}
+
 // For kernels that hold few values per thread: the cheap functions stay inline, the transcendental ones are one
 // shared out-of-line body (func is uniform, so the branch costs nothing).
 __device__ __attribute__((noinline)) inline float apply_func_outlined(int func, float v) { return apply_func(func, v); }

@@ -175,10 +175,12 @@ Phase1D phase_1d(int32_t ph, int32_t K, int32_t s, int32_t p, int32_t O) {
 
 // One launch prepares a transposed convolution: blockIdx.y < nphase packs that phase's sub-kernel,
 //   packed_f[co][(ci, ty, tx)] = kernel[ci][co*KY*KX + (KY-1-(ky0+ty*sy))*KX + (KX-1-(kx0+tx*sx))],
+// (or, with other strides, [ci][phase][co][taps] for the kernel that reads all coefficients of a channel at once)
 // and blockIdx.y == nphase sums the biases of every bias layer (the CPU path adds all of them per tap).
 struct PackPhase {
   uint32_t begin, kp, ld;  // offset of the phase in the packed buffer (floats), coefficients per row, padded row length
   int32_t ky0, kx0, ty, tx;
+  uint32_t co_stride, ci_stride;  // coefficient (co, ci, t) goes to begin + co*co_stride + ci*ci_stride + t
 };
 struct PackArgs {
   PackPhase ph[MAX_PHASES];
@@ -200,13 +202,14 @@ __global__ __launch_bounds__(256) void tconv_prepare_kernel(float *packed, float
   const uint32_t taps = ph.ty * ph.tx, total = (uint32_t)pa.CO * ph.ld;
   for (uint32_t idx = blockIdx.x * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
     uint32_t co = idx / ph.ld, k = idx % ph.ld;
-    float v = 0.f;  // rows are zero-padded to a multiple of four coefficients
     if (k < ph.kp) {
       uint32_t ci = k / taps, t = k % taps, ty = t / ph.tx, tx = t % ph.tx;
       int32_t ky = ph.ky0 + ty * pa.SY, kx = ph.kx0 + tx * pa.SX;
-      v = kernel[(size_t)ci * pa.ker_ld + co * pa.KY * pa.KX + (pa.KY - 1 - ky) * pa.KX + (pa.KX - 1 - kx)];
+      packed[ph.begin + co * ph.co_stride + ci * ph.ci_stride + t] =
+          kernel[(size_t)ci * pa.ker_ld + co * pa.KY * pa.KX + (pa.KY - 1 - ky) * pa.KX + (pa.KX - 1 - kx)];
+    } else {
+      packed[ph.begin + idx] = 0.f;  // rows [co][k] are zero-padded to a multiple of four coefficients
     }
-    packed[ph.begin + idx] = v;
   }
 }
 
@@ -349,6 +352,153 @@ __global__ __launch_bounds__(256) void tconv_k4s2_small_kernel(TconvArgs args) {
   }
 }
 
+// The same geometry with the input staged through LDS: a block owns a tile of 32 x 16 input pixels of one image
+// (64 x 32 output pixels) and walks the input channels in chunks of CC.  A chunk's (16+2) x (32+2) halo tile per
+// channel is fetched with 128-bit buffer loads (zero outside the image through the range check), kept in registers
+// while the previous chunk is multiplied, then written to the other LDS buffer: one barrier per chunk.  A thread
+// computes two neighbouring input pixels, i.e. 2 x 4 output pixels: per channel 6 LDS reads for 32*CO multiply-adds
+// instead of 9 global loads for 16*CO, which moves the kernel from the texture-address path to the vector ALUs.
+// Needs W % 4 == 0, C % CC == 0, 16-byte aligned rows, exactly CO output channels and the coefficients packed
+// as [ci][phase][co][taps].
+template <int CO>
+__global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
+  constexpr int TW = 32, TH = 16, CC = 8, PITCH = 36, ROWS = TH + 2;
+  constexpr int VEC = CC * ROWS * (TW / 4), NVEC = (VEC + 255) / 256;  // 128-bit pieces of a chunk, per thread
+  constexpr int EDGE = CC * ROWS * 2, NEDGE = (EDGE + 255) / 256;      // halo columns left and right
+  __shared__ __attribute__((aligned(16))) float tile[2][CC][ROWS][PITCH];  // column 0 = x0-1, 1..32 = the tile, 33 = x0+32
+  const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W, M = args.M;
+  const uint32_t tiles_x = (W + TW - 1) / TW;
+  const uint32_t x0 = (blockIdx.x % tiles_x) * TW, y0 = (blockIdx.x / tiles_x) * TH, g = blockIdx.y;
+  const uint32_t tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta, args.in_w * C * HW * 4u);
+  const uint32_t imgoff = (g % args.in_w) * C * HW * 4u;
+
+  // byte offsets of this thread's pieces within a chunk (channel advance goes through the scalar offset)
+  uint32_t voff[NVEC], eoff[NEDGE], vdst[NVEC], edst[NEDGE];
+#pragma unroll
+  for (int i = 0; i < NVEC; i++) {
+    const uint32_t idx = tid + i * 256, row = idx / (TW / 4), seg = idx % (TW / 4), c = row / ROWS, yy = row % ROWS;
+    const int32_t iy = (int32_t)(y0 + yy) - 1;
+    const uint32_t ix = x0 + seg * 4;
+    const bool ok = idx < VEC && (uint32_t)iy < H && ix < W;
+    voff[i] = ok ? imgoff + ((c * H + (uint32_t)iy) * W + ix) * 4u : OOB;
+    vdst[i] = idx < VEC ? (c * ROWS + yy) * PITCH + 1 + seg * 4 : 0xffffffffu;
+  }
+#pragma unroll
+  for (int i = 0; i < NEDGE; i++) {
+    const uint32_t idx = tid + i * 256, row = idx / 2, side = idx % 2, c = row / ROWS, yy = row % ROWS;
+    const int32_t iy = (int32_t)(y0 + yy) - 1, ix = side ? (int32_t)(x0 + TW) : (int32_t)x0 - 1;
+    const bool ok = idx < EDGE && (uint32_t)iy < H && (uint32_t)ix < W;
+    eoff[i] = ok ? imgoff + ((c * H + (uint32_t)iy) * W + (uint32_t)ix) * 4u : OOB;
+    edst[i] = idx < EDGE ? (c * ROWS + yy) * PITCH + (side ? TW + 1 : 0) : 0xffffffffu;
+  }
+  floatx4 rv[NVEC];
+  float re[NEDGE];
+  auto fetch = [&](uint32_t chunk) {
+    const uint32_t soff = chunk * CC * HW * 4u;
+#pragma unroll
+    for (int i = 0; i < NVEC; i++) rv[i] = buf_load4(rsrc, voff[i], soff);
+#pragma unroll
+    for (int i = 0; i < NEDGE; i++) re[i] = buf_load(rsrc, eoff[i], soff);
+  };
+  auto put = [&](int buf) {
+    float *t = &tile[buf][0][0][0];
+#pragma unroll
+    for (int i = 0; i < NVEC; i++)
+      if (vdst[i] != 0xffffffffu) {  // the tile starts at an odd column: 4 + 8 + 4 bytes
+        t[vdst[i]] = rv[i].x;
+        *reinterpret_cast<float2 *>(t + vdst[i] + 1) = make_float2(rv[i].y, rv[i].z);
+        t[vdst[i] + 3] = rv[i].w;
+      }
+#pragma unroll
+    for (int i = 0; i < NEDGE; i++)
+      if (edst[i] != 0xffffffffu) t[edst[i]] = re[i];
+  };
+
+  float acc[2][2][2][CO];  // [pixel][py][px][co]
+#pragma unroll
+  for (int i = 0; i < 8 * CO; i++) (&acc[0][0][0][0])[i] = 0.f;
+  const uint32_t chunks = C / CC;
+  const float *coeff = args.ph[0].packed;
+  fetch(0);
+  put(0);
+  __syncthreads();
+  for (uint32_t ch = 0; ch < chunks; ch++) {
+    const int cur = ch & 1;
+    if (ch + 1 < chunks) fetch(ch + 1);
+#pragma unroll 2
+    for (int c = 0; c < CC; c++) {
+      const uint32_t ci = ch * CC + c;
+      float v[3][4];  // rows y-1..y+1, columns x-1..x+2 of the pixel pair (x, x+1)
+#pragma unroll
+      for (int dy = 0; dy < 3; dy++) {
+        const float *rowp = &tile[cur][c][ty + dy][2 * tx];
+        const float2 lo = *reinterpret_cast<const float2 *>(rowp), hi = *reinterpret_cast<const float2 *>(rowp + 2);
+        v[dy][0] = lo.x; v[dy][1] = lo.y; v[dy][2] = hi.x; v[dy][3] = hi.y;
+      }
+#pragma unroll
+      for (int py = 0; py < 2; py++)
+#pragma unroll
+        for (int px = 0; px < 2; px++) {
+#pragma unroll
+          for (int co = 0; co < CO; co++) {
+            // all 16*CO coefficients of a channel are contiguous: [ci][phase][co][taps (ty,tx) = 00 01 10 11]
+            const float4 w = *reinterpret_cast<const float4 *>(coeff + (size_t)ci * (16 * CO) + ((py * 2 + px) * CO + co) * 4);
+#pragma unroll
+            for (int p = 0; p < 2; p++) {
+              float a = acc[p][py][px][co];
+              a = __builtin_fmaf(w.x, v[py][p + px], a);
+              a = __builtin_fmaf(w.y, v[py][p + px + 1], a);
+              a = __builtin_fmaf(w.z, v[py + 1][p + px], a);
+              a = __builtin_fmaf(w.w, v[py + 1][p + px + 1], a);
+              acc[p][py][px][co] = a;
+            }
+          }
+        }
+    }
+    if (ch + 1 < chunks) put(cur ^ 1);
+    __syncthreads();
+  }
+
+  const uint32_t qy = y0 + ty, qx = x0 + 2 * tx;
+  if (qy >= H || qx >= W) return;  // W is even: a pair is inside or outside as a whole
+  const uint32_t OW = 2 * W, OHW = 4 * HW;
+  const float bsum = args.ep.tap_bias ? args.ep.tap_bias[g % args.ep.bias_w] : 0.f;
+#pragma unroll
+  for (int py = 0; py < 2; py++) {
+    // contributing taps of output row 2*qy+py are input rows qy+py-1 and qy+py; likewise along x
+    const int ny = ((uint32_t)((int32_t)qy + py - 1) < H) + ((uint32_t)((int32_t)qy + py) < H);
+    const int nx[4] = {((uint32_t)((int32_t)qx - 1) < W) + 1, 2, 2, 1 + ((uint32_t)((int32_t)qx + 2) < W)};
+#pragma unroll
+    for (int co = 0; co < CO; co++) {
+      float4 o;
+      o.x = mt::apply_func_epilogue(args.ep.func, acc[0][py][0][co] + bsum * (float)(ny * nx[0]));
+      o.y = mt::apply_func_epilogue(args.ep.func, acc[0][py][1][co] + bsum * (float)(ny * nx[1]));
+      o.z = mt::apply_func_epilogue(args.ep.func, acc[1][py][0][co] + bsum * (float)(ny * nx[2]));
+      o.w = mt::apply_func_epilogue(args.ep.func, acc[1][py][1][co] + bsum * (float)(ny * nx[3]));
+      float *dst = args.ep.C + ((size_t)g * M + co) * OHW + (size_t)(2 * qy + py) * OW + 2 * qx;
+      *reinterpret_cast<float4 *>(dst) = o;
+    }
+  }
+}
+
+// kernel 4x4, stride 2, padding 1, at most 4 output channels, and the shape the tile kernel is written for
+bool tile_kernel_fits(const mt_tensor *out, const mt_tensor *delta, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, int32_t sx, int32_t sy, int32_t px,
+                      int32_t py) {
+  return kz <= 4 && kx == 4 && ky == 4 && sx == 2 && sy == 2 && px == 1 && py == 1 && out->y == 2 * delta->y && out->x == 2 * delta->x &&
+         delta->x % 4 == 0 && ka % 8 == 0 && ka >= 16 && ((uintptr_t)out->p & 15u) == 0 && ((uintptr_t)delta->p & 15u) == 0 && out->w <= 65535u;
+}
+int launch_tconv_tile(const char *name, TconvArgs &args) {
+  mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "vector ALU, few output channels") : name);
+  dim3 gt(cdiv(args.W, 32) * cdiv(args.H, 16), args.out_w);
+  if (args.M == 1) tconv_k4s2_tile_kernel<1><<<gt, 256, 0, mt::stream()>>>(args);
+  else if (args.M == 2) tconv_k4s2_tile_kernel<2><<<gt, 256, 0, mt::stream()>>>(args);
+  else if (args.M == 3) tconv_k4s2_tile_kernel<3><<<gt, 256, 0, mt::stream()>>>(args);
+  else tconv_k4s2_tile_kernel<4><<<gt, 256, 0, mt::stream()>>>(args);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
 int launch_tconv_small(const char *name, TconvArgs &args, uint32_t max_n) {
   mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "vector ALU, few output channels") : name);
   dim3 grid(cdiv(max_n, 256), args.nphase);
@@ -487,6 +637,7 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   pa.ker_ld = kernel->x; pa.bias_w = bias->w; pa.CO = kz; pa.CI = ka; pa.KY = ky; pa.KX = kx; pa.SY = sy; pa.SX = sx;
   uint32_t max_n = 0, max_pack = 0, begin = 0;
   const uint32_t OHW = out->y * out->x;
+  const bool tile = mt::igemm::tile_override() < 0 && tile_kernel_fits(out, delta, kx, ky, kz, ka, sx, sy, px, py);
   for (int32_t phy = 0; phy < sy; phy++) {
     Phase1D Y = phase_1d(phy, ky, sy, py, out->y);
     if (Y.q == 0) continue;
@@ -494,8 +645,11 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
       Phase1D X = phase_1d(phx, kx, sx, px, out->x);
       if (X.q == 0) continue;
       uint32_t kp = ka * Y.taps * X.taps, ld = (kp + 3u) & ~3u, f = args.nphase++;
-      pa.ph[f] = PackPhase{begin, kp, ld, Y.k0, X.k0, Y.taps, X.taps};
-      args.ph[f] = TconvPhase{packed + begin, kp, ld, (uint32_t)Y.q, (uint32_t)X.q, Y.taps, X.taps, Y.off, X.off, (uint32_t)phy, (uint32_t)phx};
+      pa.ph[f] = PackPhase{begin, kp, ld, Y.k0, X.k0, Y.taps, X.taps, ld, (uint32_t)(Y.taps * X.taps)};
+      if (tile) {  // [ci][phase][co][2x2 taps]
+        pa.ph[f].begin = f * 4u * (uint32_t)kz; pa.ph[f].co_stride = 4; pa.ph[f].ci_stride = 16u * (uint32_t)kz;
+      }
+      args.ph[f] = TconvPhase{packed + pa.ph[f].begin, kp, ld, (uint32_t)Y.q, (uint32_t)X.q, Y.taps, X.taps, Y.off, X.off, (uint32_t)phy, (uint32_t)phx};
       begin += (uint32_t)kz * ld;  // a multiple of four floats: every phase starts 16-byte aligned
       uint32_t n = out->w * Y.q * X.q;
       if (n > max_n) max_n = n;
@@ -516,6 +670,7 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   args.ep.sy = sy; args.ep.sx = sx; args.ep.OW = out->x;
   args.ep.tap_bias = ws; args.ep.bias_w = bias->w; args.ep.IH = delta->y; args.ep.IW = delta->x;
   args.ep.func = func;
+  if (tile) return launch_tconv_tile(name, args);
   if (kz <= 4 && mt::igemm::tile_override() < 0) {
     rc = launch_tconv_small(name, args, max_n);
     if (rc >= 0) return rc;

@@ -362,6 +362,77 @@ __global__ __launch_bounds__(EW_THREADS) void bn_apply_kernel(float *out, float 
   }
 }
 
+// Both passes in one kernel when a thread's share of the batch fits in registers: a block owns RB groups of four
+// columns and splits the batch over 256/RB slices; a thread keeps its NW rows (128-bit each) in registers between
+// the statistics and the normalisation, so the input is read once.  Same sums, in the same order per thread, as
+// bn_stats_kernel<4>; only the cheap functions are applied here (see mt::epilogue_func).
+template <int RB, int NW>
+__global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float *xhat, const float *x, uint32_t W, uint32_t S, float inv_n, float eps,
+                                                              float *mean, float *var, float *ivar, float *new_mean, float *new_var, float mom_old,
+                                                              float mom_new, const float *gamma, const float *beta, int func) {
+  constexpr int WS = EW_THREADS / RB;
+  __shared__ float part[2][WS][RB * 4];
+  __shared__ float col_mean[RB * 4], col_ivar[RB * 4];
+  const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
+  const uint32_t r = (blockIdx.x * RB + rl) * 4;
+  float4 q[NW];
+  float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f};
+  if (r < S) {
+    const float4 sh = *reinterpret_cast<const float4 *>(x + r);
+#pragma unroll
+    for (int i = 0; i < NW; i++) {
+      const uint32_t w = ws + i * WS;
+      q[i] = w < W ? *reinterpret_cast<const float4 *>(x + (size_t)w * S + r) : sh;
+    }
+#pragma unroll
+    for (int i = 0; i < NW; i++) {
+      if (ws + i * WS < W) {
+        float d0 = q[i].x - sh.x, d1 = q[i].y - sh.y, d2 = q[i].z - sh.z, d3 = q[i].w - sh.w;
+        s1[0] += d0; s1[1] += d1; s1[2] += d2; s1[3] += d3;
+        s2[0] += d0 * d0; s2[1] += d1 * d1; s2[2] += d2 * d2; s2[3] += d3 * d3;
+      }
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 4; v++) { part[0][ws][rl * 4 + v] = s1[v]; part[1][ws][rl * 4 + v] = s2[v]; }
+  __syncthreads();
+  const int c = threadIdx.x;
+  const uint32_t rc = blockIdx.x * RB * 4 + c;
+  if (c < RB * 4 && rc < S) {  // the first RB*4 threads finish one column each
+    float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < WS; i++) { a1 += part[0][i][c]; a2 += part[1][i][c]; }
+    const float sh = x[rc];
+    float md = a1 * inv_n;
+    float mu = sh + md;
+    float vr = (a2 - a1 * md) * inv_n;
+    if (vr < 0.f) vr = 0.f;
+    float iv = (float)(1.0 / (double)(sqrtf(vr + eps) * 1.f));
+    mean[rc] = mu;
+    var[rc] = vr;
+    ivar[rc] = iv;
+    if (new_mean) new_mean[rc] = (mom_old * new_mean[rc]) + (mom_new * mu);
+    if (new_var) new_var[rc] = (mom_old * new_var[rc]) + (mom_new * vr);
+    col_mean[c] = mu;
+    col_ivar[c] = iv;
+  }
+  __syncthreads();
+  if (r >= S) return;
+  const float4 mu = *reinterpret_cast<const float4 *>(col_mean + rl * 4), iv = *reinterpret_cast<const float4 *>(col_ivar + rl * 4);
+  const float4 g = *reinterpret_cast<const float4 *>(gamma + r), b = *reinterpret_cast<const float4 *>(beta + r);
+#pragma unroll
+  for (int i = 0; i < NW; i++) {
+    const uint32_t w = ws + i * WS;
+    if (w >= W) break;
+    float4 h, o;
+    h.x = (q[i].x - mu.x) * iv.x; h.y = (q[i].y - mu.y) * iv.y; h.z = (q[i].z - mu.z) * iv.z; h.w = (q[i].w - mu.w) * iv.w;
+    o.x = mt::apply_func_cheap(func, (g.x * h.x) + b.x); o.y = mt::apply_func_cheap(func, (g.y * h.y) + b.y);
+    o.z = mt::apply_func_cheap(func, (g.z * h.z) + b.z); o.w = mt::apply_func_cheap(func, (g.w * h.w) + b.w);
+    if (xhat) *reinterpret_cast<float4 *>(xhat + (size_t)w * S + r) = h;
+    *reinterpret_cast<float4 *>(out + (size_t)w * S + r) = o;
+  }
+}
+
 __global__ __launch_bounds__(EW_THREADS) void bn_ivar_kernel(float *ivar, const float *var, uint32_t S, float eps) {
   uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
   if (i < S) ivar[i] = (float)(1.0 / (double)sqrtf(var[i] + eps));
@@ -557,15 +628,34 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
   float *pm = batch_mean ? batch_mean->p : scratch, *pv = batch_var ? batch_var->p : scratch + S, *pi = ivar ? ivar->p : scratch + 2 * S;
   float inv_n = (float)(1.0 / (double)(float)W);  // the layer passes 1.0/N with N a float
   float mom_new = (float)(1.0 - (double)momentum);  // and 1.0-Momentum, rounded once
+  float *nm = new_mean ? new_mean->p : nullptr, *nv = new_variable ? new_variable->p : nullptr;
+  bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(pm) && aligned16(pi) && (!xhat || aligned16(xhat->p));
+  if (vec && mt::epilogue_func(func)) {
+    // one pass: the widest column block that still gives every compute unit a few blocks, if the batch share fits
+    const int rb = S / 128 >= 512 ? 32 : S / 64 >= 512 ? 16 : 8;
+    const uint32_t nw = cdiv(W, EW_THREADS / rb);
+    if (nw <= 32) {
+      mt::ProfileScope prof("bn_fused");
+      const unsigned grid = cdiv(S, (size_t)rb * 4);
+#define MT_BN_FUSED(RB, NW) \
+  bn_fused_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func)
+#define MT_BN_FUSED_NW(RB) \
+  do { if (nw <= 8) MT_BN_FUSED(RB, 8); else if (nw <= 16) MT_BN_FUSED(RB, 16); else MT_BN_FUSED(RB, 32); } while (0)
+      if (rb == 32) MT_BN_FUSED_NW(32); else if (rb == 16) MT_BN_FUSED_NW(16); else MT_BN_FUSED_NW(8);
+#undef MT_BN_FUSED_NW
+#undef MT_BN_FUSED
+      MT_LAUNCH_CHECK("bn_fused");
+      return MT_OK;
+    }
+  }
   {
   mt::ProfileScope prof("bn_stats");
   if (S % 4 == 0 && aligned16(in->p))
-    bn_stats_kernel<4><<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, new_mean ? new_mean->p : nullptr, new_variable ? new_variable->p : nullptr, momentum, mom_new);
+    bn_stats_kernel<4><<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new);
   else
-    bn_stats_kernel<1><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, new_mean ? new_mean->p : nullptr, new_variable ? new_variable->p : nullptr, momentum, mom_new);
+    bn_stats_kernel<1><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new);
   }
   MT_LAUNCH_CHECK("bn_stats");
-  bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(pm) && aligned16(pi) && (!xhat || aligned16(xhat->p));
   unsigned gx = cdiv(vec ? S / 4 : S, EW_THREADS);
   unsigned gy = W < 16 ? W : 16;  // a few batch slices per column block keeps the per-column loads in registers
   mt::ProfileScope prof("bn_apply");
