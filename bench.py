@@ -42,6 +42,20 @@ def hip_events():
     return create, record, elapsed_ms
 
 
+def measured_traffic():
+    """HBM-side bytes per launch of the dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each
+    scaled by what the same counter reads for a plain copy of known size); the summary of those runs is kept under
+    profiles/ and carries the figure on a line of its own.  None when the summary is missing."""
+    path = os.path.join(ROOT, "profiles", "dcgan64_b256_forward_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def cpu_baseline(sample_batch):
     """The CPU path on this host, single thread (the reference has no active OpenMP), on `sample_batch` images."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
@@ -159,7 +173,8 @@ def main():
         "host_ms_per_step_wall": wall_ms / args.steps,
         "ms_per_step_with_per_kernel_events": profiled_wall_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None, "kernel": dom_label,
+                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": measured_traffic(), "traffic_unit": "bytes per launch",
+                     "kernel": dom_label,
                      "launches_per_step": dom_launches / args.steps, "avg_launch_ms": dom_ms / dom_launches if dom_launches else None,
                      "flop_per_launch": flop_per_launch,
                      "per_layer": {b[0]: {"avg_launch_ms": b[2] / b[1], "tflops": b[3] / (b[2] / b[1] * 1e-3) / 1e12} for b in big}},
