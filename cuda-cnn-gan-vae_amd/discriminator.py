@@ -1,0 +1,201 @@
+"""DCGAN-64 discriminator training step as the reference's layers would run it, on device-resident tensors.
+
+Layer stack (the reference's layer classes in brackets):
+    images [B,3,64,64]
+    -> conv 4x4 s2 p1, 3 -> 64 -> 128 -> 256 -> 512   [CNetLayerConvolution, netlayer/cnetlayerconvolution.cu.h:310-322]
+       each followed by BatchNorm (batch statistics)   [CNetLayerBatchNormalization :268-380]
+       and leaky ReLU                                  [CNetLayerFunction :203-213]
+    -> Linear 8192 -> 1, sigmoid                       [CNetLayerLinear :262-282]
+
+`forward` / `backward` issue the layers' op sequences one C-ABI call per tensor op (TrainingBackward of
+cnetlayerfunction.cu.h:347-358, cnetlayerbatchnormalization.cu.h:578-604, cnetlayerconvolution.cu.h:484-516,
+cnetlayerlinear.cu.h:415-447); `update` is the layers' TrainingUpdateWeight (Adam).  The error fed to the last
+function layer is p - label.
+"""
+import numpy as np
+
+import mi355tensor as mt
+from mi355tensor import CTensor, CTensorApplyFunc, CTensorConv, CTensorMath, Fused
+
+CHANNELS = (3, 64, 128, 256, 512)
+IMAGE = 64
+BN_EPSILON = 1e-6
+MOMENTUM = 0.9
+
+
+def make_parameters(seed=5, std=0.02):
+    """Random-init parameters as numpy arrays in the reference's layouts (kernel [1,1,Cout,Cin*16], bias [1,Cout,1,1])."""
+    rng = np.random.default_rng(seed)
+    p, size = {}, IMAGE
+    for i in range(4):
+        cin, cout = CHANNELS[i], CHANNELS[i + 1]
+        size //= 2
+        p["kernel%d" % i] = (rng.standard_normal((1, 1, cout, cin * 16)) * std).astype(np.float32)
+        p["bias%d" % i] = np.zeros((1, cout, 1, 1), np.float32)
+        p["gamma%d" % i] = np.ones((1, cout, size, size), np.float32)
+        p["beta%d" % i] = np.zeros((1, cout, size, size), np.float32)
+    p["lin_w"] = (rng.standard_normal((1, 1, 1, CHANNELS[4] * 16)) * std).astype(np.float32)
+    p["lin_b"] = np.full((1, 1, 1, 1), 0.1, np.float32)
+    return p
+
+
+def make_batch(batch, seed=5):
+    rng = np.random.default_rng(seed + 1000)
+    x = rng.uniform(-1, 1, size=(batch, 3, IMAGE, IMAGE)).astype(np.float32)
+    labels = (rng.uniform(size=(batch, 1, 1, 1)) < 0.5).astype(np.float32)
+    return x, labels
+
+
+def conv_flops(batch):
+    """Algorithmic FLOPs (2*MAC) of one pass over the four convolutions; forward, input gradient and weight
+    gradient each cost this much."""
+    out, size = [], IMAGE
+    for i in range(4):
+        size //= 2
+        out.append(2.0 * batch * CHANNELS[i + 1] * size * size * CHANNELS[i] * 16)
+    return out
+
+
+class Discriminator:
+    def __init__(self, batch, params=None):
+        mt.init(0)
+        self.batch = b = batch
+        host = params or make_parameters()
+        self.p = {k: CTensor.from_numpy(v) for k, v in host.items()}
+        self.x, self.labels = CTensor(b, 3, IMAGE, IMAGE), CTensor(b, 1, 1, 1)
+        self.c, self.bn, self.a, self.xhat, self.ivar = [], [], [], [], []
+        self.d_a, self.d_bn, self.d_c = [], [], []
+        self.dk_batch, self.db_batch, self.g = [], [], {}
+        self.stat = []
+        size = IMAGE
+        for i in range(4):
+            cin, cout = CHANNELS[i], CHANNELS[i + 1]
+            size //= 2
+            shape, s1 = (b, cout, size, size), (1, cout, size, size)
+            for lst in (self.c, self.bn, self.a, self.xhat, self.d_a, self.d_bn, self.d_c):
+                lst.append(CTensor(*shape))
+            self.ivar.append(CTensor(*s1))
+            self.stat.append([CTensor(*s1) for _ in range(4)])      # scratch of the batch-norm backward pass
+            self.dk_batch.append(CTensor(b, 1, cout, cin * 16))
+            self.db_batch.append(CTensor(b, cout, 1, 1))
+            for name in ("kernel", "bias", "gamma", "beta"):
+                self.g["%s%d" % (name, i)] = CTensor(*host["%s%d" % (name, i)].shape)
+        self.d_x = CTensor(b, 3, IMAGE, IMAGE)
+        self.logit, self.prob, self.err, self.d_logit = (CTensor(b, 1, 1, 1) for _ in range(4))
+        self.tmp = [CTensor(*t.shape) for t in self.c]               # elementwise scratch, one per layer size
+        self.tmp_dw = CTensor(b, 1, 1, CHANNELS[4] * 16)
+        self.g["lin_w"], self.g["lin_b"] = CTensor(1, 1, 1, CHANNELS[4] * 16), CTensor(1, 1, 1, 1)
+        self.zero_bias = [CTensor.from_numpy(np.zeros((1, CHANNELS[i + 1], 1, 1), np.float32)) for i in range(4)]
+        self.m = {k: CTensor.from_numpy(np.zeros(v.shape, np.float32)) for k, v in host.items()}
+        self.v = {k: CTensor.from_numpy(np.zeros(v.shape, np.float32)) for k, v in host.items()}
+        self.iteration = 0
+
+    def set_batch(self, x, labels):
+        self.x.upload(x)
+        self.labels.upload(labels)
+
+    # ---- forward -------------------------------------------------------------------------------------------
+    def forward(self, fused=False):
+        h, p = self.x, self.p
+        for i in range(4):
+            cin, cout = CHANNELS[i], CHANNELS[i + 1]
+            CTensorConv.ForwardConvolution(self.c[i], h, p["kernel%d" % i], 4, 4, cin, cout, p["bias%d" % i], 2, 2, 1, 1)
+            if fused:
+                Fused.BatchNormForwardTrain(self.bn[i], self.c[i], p["gamma%d" % i], p["beta%d" % i], self.xhat[i], self.ivar[i],
+                                            momentum=MOMENTUM, epsilon=BN_EPSILON)
+            else:
+                self._batchnorm_literal(i)
+            CTensorApplyFunc.ApplyLeakyReLU(self.a[i], self.bn[i])
+            h = self.a[i]
+        flat = h.reinterpret(self.batch, 1, CHANNELS[4] * 16, 1)
+        if fused:
+            Fused.LinearForward(self.logit, p["lin_w"], flat, p["lin_b"])
+        else:
+            CTensorMath.Mul(self.logit, p["lin_w"], flat)
+            CTensorMath.Add(self.logit, self.logit, p["lin_b"])
+        CTensorApplyFunc.ApplySigmoid(self.prob, self.logit)
+        return self.prob
+
+    def _batchnorm_literal(self, i):
+        """Training-mode forward of cnetlayerbatchnormalization.cu.h:301-371, op by op."""
+        x, p = self.c[i], self.p
+        mean, var, sq = self.stat[i][0], self.stat[i][1], self.stat[i][2]
+        inv_n = float(np.float32(1.0 / np.float64(np.float32(self.batch))))
+        CTensorMath.Fill(mean, 0.0)
+        CTensorMath.AddSumW(mean, mean, x, 1.0, inv_n)
+        xmu = self.tmp[i]
+        CTensorMath.Sub(xmu, x, mean, 1.0, 1.0)
+        CTensorMath.Pow2(self.xhat[i], xmu, 1.0)
+        CTensorMath.Fill(var, 0.0)
+        CTensorMath.AddSumW(var, var, self.xhat[i], 1.0, inv_n)
+        CTensorMath.SQRT(sq, var, 1.0, BN_EPSILON)
+        CTensorMath.Inv(self.ivar[i], sq)
+        CTensorMath.TensorItemProduction(self.xhat[i], xmu, self.ivar[i])
+        CTensorMath.TensorItemProduction(self.bn[i], p["gamma%d" % i], self.xhat[i])
+        CTensorMath.Add(self.bn[i], self.bn[i], p["beta%d" % i])
+
+    # ---- backward ------------------------------------------------------------------------------------------
+    def backward(self):
+        b, p, g = self.batch, self.p, self.g
+        CTensorMath.Sub(self.err, self.prob, self.labels)
+        CTensorApplyFunc.ApplyDifferentialSigmoid(self.d_logit, self.logit)
+        CTensorMath.TensorItemProduction(self.d_logit, self.err, self.d_logit)
+        # Linear: previous error, per-sample outer products, their sum over the batch
+        flat_err = self.d_a[3].reinterpret(b, 1, CHANNELS[4] * 16, 1)
+        CTensorMath.TransponseMul(flat_err, p["lin_w"], self.d_logit)
+        CTensorMath.Mul(self.tmp_dw, self.d_logit, self.a[3].reinterpret(b, 1, 1, CHANNELS[4] * 16))
+        CTensorMath.Fill(g["lin_w"], 0.0)
+        CTensorMath.AddSumW(g["lin_w"], g["lin_w"], self.tmp_dw)
+        CTensorMath.Fill(g["lin_b"], 0.0)
+        CTensorMath.AddSumW(g["lin_b"], g["lin_b"], self.d_logit)
+        for i in (3, 2, 1, 0):
+            cin, cout = CHANNELS[i], CHANNELS[i + 1]
+            # function layer
+            CTensorApplyFunc.ApplyDifferentialLeakyReLU(self.d_bn[i], self.bn[i])
+            CTensorMath.TensorItemProduction(self.d_bn[i], self.d_a[i], self.d_bn[i])
+            self._batchnorm_backward(i)
+            # convolution layer
+            inp, prev = (self.a[i - 1], self.d_a[i - 1]) if i else (self.x, self.d_x)
+            CTensorConv.BackwardConvolution(prev, self.d_c[i], p["kernel%d" % i], 4, 4, cin, cout, self.zero_bias[i], 2, 2, 1, 1)
+            CTensorMath.Fill(self.dk_batch[i], 0.0)
+            CTensorMath.Fill(self.db_batch[i], 0.0)
+            CTensorConv.CreateDeltaWeightAndBias(self.dk_batch[i], 4, 4, cin, cout, self.db_batch[i], inp, self.d_c[i], 2, 2, 1, 1)
+            CTensorMath.Fill(g["kernel%d" % i], 0.0)
+            CTensorMath.AddSumW(g["kernel%d" % i], g["kernel%d" % i], self.dk_batch[i])
+            CTensorMath.Fill(g["bias%d" % i], 0.0)
+            CTensorMath.AddSumW(g["bias%d" % i], g["bias%d" % i], self.db_batch[i])
+
+    def _batchnorm_backward(self, i):
+        """cnetlayerbatchnormalization.cu.h:578-604."""
+        n = np.float32(self.batch)
+        delta, gamma, xhat, ivar, g = self.d_bn[i], self.p["gamma%d" % i], self.xhat[i], self.ivar[i], self.g
+        s1, s2 = self.stat[i][0], self.stat[i][1]
+        dxhat, t, out = self.tmp[i], self.c[i], self.d_c[i]          # the conv output is no longer needed: reuse it as scratch
+        CTensorMath.TensorItemProduction(dxhat, delta, gamma)
+        CTensorMath.Fill(s1, 0.0)
+        CTensorMath.AddSumW(s1, s1, dxhat)
+        CTensorMath.TensorItemProduction(t, dxhat, xhat)
+        CTensorMath.Fill(s2, 0.0)
+        CTensorMath.AddSumW(s2, s2, t)
+        CTensorMath.TensorItemProduction(t, delta, xhat)
+        CTensorMath.Fill(g["gamma%d" % i], 0.0)
+        CTensorMath.AddSumW(g["gamma%d" % i], g["gamma%d" % i], t)
+        CTensorMath.Fill(g["beta%d" % i], 0.0)
+        CTensorMath.AddSumW(g["beta%d" % i], g["beta%d" % i], delta)
+        CTensorMath.Mul(out, dxhat, float(n))
+        CTensorMath.TensorItemProduction(t, xhat, s2)
+        CTensorMath.Sub(out, out, t)
+        CTensorMath.Sub(out, out, s1)
+        CTensorMath.TensorItemProduction(out, out, ivar)
+        CTensorMath.Mul(out, out, float(np.float32(1.0 / np.float64(n))))
+
+    # ---- optimiser ------------------------------------------------------------------------------------------
+    def update(self, speed=2e-4, beta1=0.5, beta2=0.999, epsilon=1e-8):
+        self.iteration += 1
+        for k in self.p:
+            CTensorMath.Adam(self.p[k], self.g[k], self.m[k], self.v[k], self.batch, speed, beta1, beta2, epsilon, float(self.iteration))
+
+    def step(self, fused=False):
+        self.forward(fused)
+        self.backward()
+        self.update()

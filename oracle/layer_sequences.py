@@ -130,3 +130,42 @@ def dcgan_generator_forward(lib, params, latent, channels=(512, 256, 128, 64, 3)
         outs["a%d" % i], outs["h%d" % (i + 1)] = a, h
     outs["image"] = function_forward(lib, h, "tangence")
     return outs
+
+
+def function_backward(lib, error, layer_input, func):
+    """CNetLayerFunction::SetOutputError, netlayer/cnetlayerfunction.cu.h:347-358: delta = error * f'(input)."""
+    return lib.tensor_item_production(error, lib.apply_func(layer_input, func, differential=True))
+
+
+def discriminator_forward(lib, params, x, channels=(3, 64, 128, 256, 512)):
+    """DCGAN-64 discriminator forward as a stack of the reference's layers: four times (conv 4x4 stride 2 padding 1,
+    BatchNorm in training mode, leaky ReLU), Linear to one logit, sigmoid.  `params` uses the names of
+    discriminator.make_parameters().  Returns every tensor the layers keep."""
+    acts, h = {"x": x}, x
+    for i in range(4):
+        c = conv_forward(lib, h, params["kernel%d" % i], params["bias%d" % i], 4, 2, 1)
+        bn = batchnorm_forward_train(lib, c, params["gamma%d" % i], params["beta%d" % i])
+        h = function_forward(lib, bn["out"], "leaky_relu")
+        acts["c%d" % i], acts["bn%d" % i], acts["a%d" % i] = c, bn, h
+    acts["logit"] = linear_forward(lib, params["lin_w"], h, params["lin_b"])
+    acts["prob"] = function_forward(lib, acts["logit"], "sigmoid")
+    return acts
+
+
+def discriminator_backward(lib, params, acts, labels):
+    """TrainingBackward of the same stack with the error p - label fed to the last function layer.
+    Returns the gradient of every parameter (same names) and "d_x", the error that reaches the images."""
+    grads = {}
+    err = lib.sub(acts["prob"], labels)
+    delta = function_backward(lib, err, acts["logit"], "sigmoid")
+    prev, grads["lin_w"], grads["lin_b"] = linear_backward(lib, params["lin_w"], delta, acts["a3"])
+    err = prev.reshape(acts["a3"].shape)
+    for i in (3, 2, 1, 0):
+        bn = acts["bn%d" % i]
+        d_bn = function_backward(lib, err, bn["out"], "leaky_relu")
+        d_c, grads["gamma%d" % i], grads["beta%d" % i] = batchnorm_backward(lib, d_bn, params["gamma%d" % i], bn["xhat"], bn["ivar"])
+        inp = acts["a%d" % (i - 1)] if i else acts["x"]
+        err, grads["kernel%d" % i], grads["bias%d" % i] = conv_backward(lib, inp, params["kernel%d" % i], d_c, 4, 2, 1)
+        grads["d_c%d" % i] = d_c
+    grads["d_x"] = err
+    return grads

@@ -88,3 +88,76 @@ def test_config3_full_batch_properties(gpu, oracle):
         if i == 3:
             want, got = oracle.apply_func(want, "tangence"), fused[sample:sample + 1]
         assert rel_err(got, want) <= REL, "layer %d" % i
+
+
+def test_config5_training_step_against_oracle(gpu, oracle):
+    """DCGAN-64 discriminator: forward, backward (input, weight and bias gradients, batch-norm gradients) and one Adam
+    step at batch 4, every tensor against the CPU oracle running the same layer sequences."""
+    import discriminator as D
+    params = D.make_parameters()
+    x, labels = D.make_batch(4)
+    acts = seq.discriminator_forward(oracle, params, x)
+    want = seq.discriminator_backward(oracle, params, acts, labels)
+    net = D.Discriminator(4, params)
+    net.set_batch(x, labels)
+    for fused in (False, True):
+        net.forward(fused)
+        for i in range(4):
+            assert rel_err(net.c[i].numpy(), acts["c%d" % i]) <= REL, "conv %d" % i
+            assert rel_err(net.xhat[i].numpy(), acts["bn%d" % i]["xhat"]) <= REL, "xhat %d" % i
+            assert rel_err(net.ivar[i].numpy(), acts["bn%d" % i]["ivar"]) <= REL, "ivar %d" % i
+            assert rel_err(net.a[i].numpy(), acts["a%d" % i]) <= REL, "activation %d" % i
+        assert rel_err(net.prob.numpy(), acts["prob"]) <= REL
+    net.backward()
+    for name in sorted(params):
+        if name.startswith("bias"):
+            # a bias in front of a batch norm has zero gradient: what is left is the rounding of a sum of cancelling
+            # terms, so the error is measured against the size of the summands
+            scale = np.abs(want["d_c" + name[4:]]).sum(axis=(0, 2, 3)).max()
+            assert np.max(np.abs(net.g[name].numpy() - want[name])) <= REL * scale, name
+        else:
+            assert rel_err(net.g[name].numpy(), want[name]) <= REL, name
+    for i in range(4):
+        assert rel_err(net.d_c[i].numpy(), want["d_c%d" % i]) <= REL, "delta %d" % i
+    assert rel_err(net.d_x.numpy(), want["d_x"]) <= REL
+    # Adam normalises every step to about +-speed, so it is checked on identical inputs: the device's own gradients
+    grads = {name: net.g[name].numpy() for name in ("kernel3", "gamma1", "lin_w")}
+    net.update()
+    for name, grad in grads.items():
+        zero = np.zeros_like(params[name])
+        w, m, v = oracle.adam(params[name], grad, zero, zero, 4, 2e-4, 0.5, 0.999, 1e-8, 1.0)
+        assert np.max(np.abs(net.p[name].numpy() - w)) <= 1e-7, name
+        assert rel_err(net.m[name].numpy(), m) <= 1e-6 and rel_err(net.v[name].numpy(), v) <= 1e-6, name
+
+
+def test_config5_full_batch_properties(gpu, oracle):
+    """Batch 128: (1) the fused and the literal forward agree; (2) convolution, its input gradient and its per-sample
+    weight gradient are independent per sample, so one sample of the big batch equals that sample alone through the
+    oracle; (3) the batch sum of the per-sample gradients equals their float64 sum."""
+    import discriminator as D
+    params = D.make_parameters()
+    x, labels = D.make_batch(128)
+    net = D.Discriminator(128, params)
+    net.set_batch(x, labels)
+    lit = net.forward(False).numpy()
+    a_lit = [t.numpy() for t in net.a]
+    fus = net.forward(True).numpy()
+    assert np.all(np.isfinite(fus)) and np.all((fus > 0) & (fus < 1)) and rel_err(fus, lit) <= REL
+    for i in range(4):
+        assert rel_err(net.a[i].numpy(), a_lit[i]) <= REL
+    net.backward()
+    for i, sample in ((0, 127), (1, 5), (2, 64), (3, 0)):
+        cin, cout = D.CHANNELS[i], D.CHANNELS[i + 1]
+        inp = (net.a[i - 1] if i else net.x).numpy()[sample:sample + 1]
+        delta = net.d_c[i].numpy()[sample:sample + 1]
+        zero_bias = np.zeros((1, cout, 1, 1), np.float32)
+        want_prev = oracle.backward_convolution(delta, params["kernel%d" % i], zero_bias, 4, 4, cin, cout, 2, 2, 1, 1, inp.shape)
+        got_prev = (net.d_a[i - 1] if i else net.d_x).numpy()[sample:sample + 1]
+        assert rel_err(got_prev, want_prev) <= REL, "input gradient %d" % i
+        dk, db = oracle.create_delta_weight_and_bias(np.zeros((1, 1, cout, cin * 16), np.float32), np.zeros((1, cout, 1, 1), np.float32),
+                                                     inp, delta, 4, 4, cin, cout, 2, 2, 1, 1)
+        dk_batch, db_batch = net.dk_batch[i].numpy(), net.db_batch[i].numpy()
+        assert rel_err(dk_batch[sample:sample + 1], dk) <= REL, "weight gradient %d" % i
+        assert rel_err(db_batch[sample:sample + 1], db) <= REL, "bias gradient %d" % i
+        assert rel_err(net.g["kernel%d" % i].numpy(), dk_batch.astype(np.float64).sum(0, keepdims=True)) <= REL
+        assert np.max(np.abs(net.g["bias%d" % i].numpy() - db_batch.astype(np.float64).sum(0, keepdims=True))) <= REL * np.abs(db_batch).sum(0).max()
