@@ -15,6 +15,7 @@ int fail(int code, const char *fmt, ...);  // records the message, returns `code
 int hip_fail(hipError_t e, const char *what);
 int set_conv_path(int v);  // 0 auto, 1 direct kernels, 2 matrix cores wherever they apply
 int set_igemm_tile(int v); // -1 auto, 0..3 force one block tile of the matrix-core kernels
+int set_wgrad_groups(int v);  // 0 auto, else batch groups of the batch-summed weight gradient
 
 // Brackets the launches made inside its lifetime with two events on the work stream when profiling is enabled
 // (mt_profile_enable); `label` must be a string literal.

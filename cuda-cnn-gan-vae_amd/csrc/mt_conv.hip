@@ -18,6 +18,7 @@ using namespace mt::igemm;
 using mt::cdiv;
 
 int g_conv_path = 0;  // 0 auto, 1 direct, 2 implicit GEMM wherever it applies
+int g_wgrad_groups = 0;  // 0 auto, else the number of batch groups of the batch-summed weight gradient (if it divides the batch)
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
@@ -156,6 +157,19 @@ __global__ __launch_bounds__(256) void dbias_wave_kernel(float *dbias, const flo
   for (uint32_t i = lane; i < DHW; i += 64) s += dl[i];
   s = mt::wave_sum(s);
   if (lane == 0) dbias[row] += s;
+}
+
+// dbias[f] += sum over the whole batch and all pixels of delta[w][f]: one wavefront per filter
+__global__ __launch_bounds__(256) void dbias_batch_sum_kernel(float *dbias, const float *delta, uint32_t B, uint32_t KA, uint32_t DHW) {
+  uint32_t f = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x % 64;
+  if (f >= KA) return;
+  float s = 0.f;
+  for (uint32_t w = 0; w < B; w++) {
+    const float *dl = delta + ((size_t)w * KA + f) * DHW;
+    for (uint32_t i = lane; i < DHW; i += 64) s += dl[i];
+  }
+  s = mt::wave_sum(s);
+  if (lane == 0) dbias[f] += s;
 }
 
 // ---- transposed convolution: phase geometry, kernel packing, bias sums ----------------------------------------
@@ -725,6 +739,84 @@ int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t
   return MT_OK;
 }
 
+// Weight and bias gradient of a convolution layer summed over the batch in one product: K runs over (sample, output
+// pixel), so dK[f][(c,i,j)] += sum_w sum_(oy,ox) delta[w][f][oy][ox] * image[w][c][oy*s-p+i][ox*s-p+j] without the
+// per-sample gradients ever being written.  When the product has few output tiles the batch is split into groups
+// whose partial sums go to the workspace and are added afterwards (fixed order: the result does not depend on timing).
+int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
+                    const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py) {
+  if (mt::bad(dk) || mt::bad(db) || mt::bad(image) || mt::bad(delta)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel gradient is required", name);
+  if (db->z != ka) return mt::fail(MT_E_BIAS_COUNT, "%s: kernel_amount %u but %u bias gradients", name, ka, db->z);
+  if (kx <= 0 || ky <= 0 || kz <= 0 || sx <= 0 || sy <= 0) return mt::fail(MT_E_ARGUMENT, "%s: kernel and stride must be positive", name);
+  if ((uint32_t)kz != image->z) return mt::fail(MT_E_SHAPE, "%s: kernel depth %d but image depth %u", name, kz, image->z);
+  if (delta->z != ka) return mt::fail(MT_E_DEPTH, "%s: delta depth %u but kernel_amount %u", name, delta->z, ka);
+  if (dk->w != 1 || db->w != 1 || db->y != 1 || db->x != 1) return mt::fail(MT_E_ARGUMENT, "%s: the summed gradients are [1,1,Kamt,C*Ky*Kx] and [1,Kamt,1,1]", name);
+  if (image->w != delta->w) return mt::fail(MT_E_SHAPE, "%s: image and delta batch sizes differ", name);
+  const uint32_t B = delta->w, ncol = (uint32_t)kz * kx * ky, DHW = delta->y * delta->x;
+  int rc = check_kernel_tensor(name, dk, ka, ncol);
+  if (rc) return rc;
+  if (B == 0 || DHW == 0) return MT_OK;
+  const size_t sample_image = (size_t)kz * image->y * image->x, sample_delta = (size_t)ka * DHW;
+  if (g_conv_path == 1 || DHW % BK != 0 || sample_image * 4 >= 0x80000000ull || sample_delta * 4 >= 0x80000000ull) {
+    // per-sample gradients into the workspace, then their sum: the op sequence of the layer itself
+    float *ws = nullptr;
+    if ((rc = workspace((size_t)B * ka * ncol + (size_t)B * ka, &ws))) return rc;
+    mt_tensor dkb{ws, B, 1, ka, ncol}, dbb{ws + (size_t)B * ka * ncol, B, ka, 1, 1};
+    if ((rc = mt_fill(&dkb, 0.f)) || (rc = mt_fill(&dbb, 0.f))) return rc;
+    if ((rc = wgrad(name, &dkb, kx, ky, kz, ka, &dbb, image, delta, sx, sy, px, py, true))) return rc;
+    mt_tensor flat{dk->p, 1, 1, ka, ncol};
+    const mt_tensor *dst = (dk->x == ncol && dk->z * dk->y == ka) ? &flat : nullptr;
+    if (!dst) return mt::fail(MT_E_ARGUMENT, "%s: the summed kernel gradient must be exactly [1,1,%u,%u]", name, ka, ncol);
+    if ((rc = mt_add_sum_w(dst, dst, &dkb, 1.f, 1.f))) return rc;
+    return mt_add_sum_w(db, db, &dbb, 1.f, 1.f);
+  }
+  // groups: enough blocks for every compute unit, and a divisor of the batch so that all groups have the same K
+  const uint32_t tiles = cdiv(ka, 64) * cdiv(ncol, 64);
+  uint32_t groups = 1;
+  while (groups < B && tiles * groups < 1024) {
+    uint32_t g = groups + 1;
+    while (g < B && B % g) g++;
+    groups = g;
+  }
+  if (g_wgrad_groups > 0 && B % (uint32_t)g_wgrad_groups == 0) groups = (uint32_t)g_wgrad_groups;
+  const uint32_t per = B / groups;
+  float *partial = nullptr;
+  if (groups > 1) {
+    if (dk->x != ncol || dk->z * dk->y != ka) return mt::fail(MT_E_ARGUMENT, "%s: the summed kernel gradient must be exactly [1,1,%u,%u]", name, ka, ncol);
+    if ((rc = workspace((size_t)groups * ka * ncol, &partial))) return rc;
+  }
+  SrcRowK<true> a{};
+  a.p = delta->p; a.ld = DHW; a.R = ka; a.K = per * DHW; a.seg = DHW; a.seg_stride = (uint32_t)sample_delta;
+  a.bt.wmod = groups; a.bt.stride = (size_t)per * sample_delta;
+  SrcWgradImage b{};
+  b.p = image->p; b.C = kz; b.H = image->y; b.W = image->x; b.KY = ky; b.KX = kx; b.OW = delta->x; b.OH = delta->y; b.R = ncol; b.K = per * DHW;
+  b.sy = sy; b.sx = sx; b.py = py; b.px = px;
+  b.bt.wmod = groups; b.bt.stride = (size_t)per * sample_image;
+  Epilogue ep{};
+  ep.inner = ncol; ep.g_stride = 0;
+  if (groups > 1) {
+    ep.C = partial; ep.row_stride = ncol; ep.bt.wmod = groups; ep.bt.stride = (size_t)ka * ncol;
+  } else {
+    ep.C = dk->p; ep.row_stride = dk->x; ep.accumulate = true;
+  }
+  if (DHW % 4 == 0 && ((uintptr_t)delta->p & 15u) == 0) {
+    rc = launch(name, a, b, ep, ka, ncol, per * DHW, groups);
+  } else {
+    SrcRowK<false> as{};
+    as.p = a.p; as.ld = a.ld; as.R = a.R; as.K = a.K; as.seg = a.seg; as.seg_stride = a.seg_stride; as.bt = a.bt;
+    rc = launch(name, as, b, ep, ka, ncol, per * DHW, groups);
+  }
+  if (rc) return rc;
+  if (groups > 1) {
+    mt_tensor pt{partial, groups, 1, ka, ncol}, flat{dk->p, 1, 1, ka, ncol};
+    if ((rc = mt_add_sum_w(&flat, &flat, &pt, 1.f, 1.f))) return rc;
+  }
+  dbias_batch_sum_kernel<<<cdiv(ka, 4), 256, 0, mt::stream()>>>(db->p, delta->p, B, ka, DHW);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
 }  // namespace
 
 namespace mt {
@@ -737,6 +829,11 @@ int &tile_override() {
 int set_igemm_tile(int v) {
   if (v < -1 || v > 3) return fail(MT_E_ARGUMENT, "igemm_tile must be -1 (auto) or 0..3");
   igemm::tile_override() = v;
+  return MT_OK;
+}
+int set_wgrad_groups(int v) {
+  if (v < 0) return fail(MT_E_ARGUMENT, "wgrad_groups must be 0 (auto) or a positive divisor of the batch");
+  g_wgrad_groups = v;
   return MT_OK;
 }
 int set_conv_path(int v) {
@@ -773,6 +870,11 @@ int mt_backward_convolution_func(const mt_tensor *out, const mt_tensor *delta, c
 int mt_create_delta_weight_and_bias(const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
                                     const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py) {
   return wgrad("mt_create_delta_weight_and_bias", dk, kx, ky, kz, ka, db, image, delta, sx, sy, px, py, true);
+}
+
+int mt_convolution_backward_weights_sum(const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
+                                        const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py) {
+  return wgrad_batch_sum("mt_convolution_backward_weights_sum", dk, kx, ky, kz, ka, db, image, delta, sx, sy, px, py);
 }
 
 // the transposed layer: image and delta trade places, and the bias gradient is cleared (cpu/ctensorconv.h:393-397)

@@ -64,29 +64,48 @@ __device__ __forceinline__ floatx4 buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t 
 
 // element(row, k) = p[row*ld + k]: k contiguous (weights [M][K], Linear activations [B][In]).
 // VEC: ld % 4 == 0, K % 4 == 0 and p 16-byte aligned, so every aligned group of 4 (or 2) k is all real or all padding.
+// seg > 0: k runs over several matrices of seg columns each (seg a multiple of BK), seg_stride floats apart -- the
+// deltas of a whole batch, [w][row][seg], as one long k axis.
 template <bool VEC>
 struct SrcRowK {
   static constexpr bool K_CONTIG = true;
   const float *p;
   uint32_t ld, R, K;
   Batch bt;
+  uint32_t seg = 0, seg_stride = 0;
+  uint32_t ksplit = 0;  // > 0: batch entry bz covers k in [bz*ksplit, (bz+1)*ksplit) of one matrix (split-K)
   __amdgpu_buffer_rsrc_t rsrc;
-  uint32_t voff, kthread, ktile;
-  __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
+  uint32_t voff, kthread, ktile, kseg, segjump;
+  __device__ void batch(uint32_t bz) {
+    if (ksplit) {
+      const uint32_t k0 = bz * ksplit;
+      p += k0;
+      K = K > k0 ? (K - k0 < ksplit ? K - k0 : ksplit) : 0;
+    } else {
+      p += bt.offset(bz);
+    }
+  }
   __device__ void bind(uint32_t row) {
-    rsrc = make_rsrc(p, R * ld * 4u);
+    // the range check applies to vector + scalar offset, so the descriptor spans every matrix of the k axis
+    rsrc = make_rsrc(p, seg ? ((K / seg - 1) * seg_stride + R * ld) * 4u : R * ld * 4u);
     voff = row < R ? row * ld * 4u : OOB;
   }
   template <int E>
   __device__ void seek(uint32_t k0) {
     kthread = k0;
-    ktile = 0;
+    ktile = 0; kseg = 0; segjump = 0;
     if (voff != OOB) voff += k0 * 4u;
   }
-  __device__ void next() { ktile += BK; }
+  __device__ void next() {
+    ktile += BK;
+    if (seg) {
+      kseg += BK;
+      if (kseg >= seg) { kseg = 0; segjump += (seg_stride - seg) * 4u; }
+    }
+  }
   template <int E>
   __device__ void fetch(float (&v)[E]) const {
-    const uint32_t soff = ktile * 4u, k = kthread + ktile;
+    const uint32_t soff = ktile * 4u + segjump, k = kthread + ktile;
     if constexpr (VEC && E % 4 == 0) {
 #pragma unroll
       for (int i = 0; i < E; i += 4) {
@@ -114,9 +133,18 @@ struct SrcColK {
   uint32_t ld, R, K, inner, groups;  // groups = number of folded matrices (1 when not folded)
   size_t gstride;
   Batch bt;
+  uint32_t ksplit = 0;  // > 0: batch entry bz covers k in [bz*ksplit, (bz+1)*ksplit) (split-K)
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t voff, k;
-  __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
+  __device__ void batch(uint32_t bz) {
+    if (ksplit) {
+      const uint32_t k0 = bz * ksplit;
+      p += (size_t)k0 * ld;
+      K = K > k0 ? (K - k0 < ksplit ? K - k0 : ksplit) : 0;
+    } else {
+      p += bt.offset(bz);
+    }
+  }
   __device__ void bind(uint32_t row) {
     rsrc = make_rsrc(p, (uint32_t)(((size_t)(groups - 1) * gstride + (size_t)K * ld) * 4u));
     voff = row < R ? (uint32_t)((row / inner) * gstride + row % inner) * 4u : OOB;
@@ -235,19 +263,21 @@ struct SrcIm2colFixed {
 
 // image view of a weight gradient: row = (c, i, j) (a kernel coefficient), k = (oy, ox) (an output pixel);
 // element = image[c][oy*sy - py + i][ox*sx - px + j], 0 outside.
+// OH > 0: k runs over the output pixels of several images in turn, (w, oy, ox), OH*OW a multiple of BK.
 struct SrcWgradImage {
   static constexpr bool K_CONTIG = false;
   const float *p;
   uint32_t C, H, W, KY, KX, OW, R, K;
   int32_t sy, sx, py, px;
   Batch bt;
+  uint32_t OH = 0;
   __amdgpu_buffer_rsrc_t rsrc;
-  uint32_t chanoff;
+  uint32_t chanoff, woff;
   int32_t iy0, ix0;
   uint32_t k, oy, ox, step_y, step_x;  // BK = step_y*OW + step_x
   __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
   __device__ void bind(uint32_t row) {
-    rsrc = make_rsrc(p, C * H * W * 4u);
+    rsrc = make_rsrc(p, (OH ? K / (OH * OW) : 1u) * C * H * W * 4u);  // all images of the k axis: the range check sees vector + scalar offset
     uint32_t r = row < R ? row : 0;
     uint32_t taps = KY * KX, c = r / taps, q = r % taps, i = q / KX, j = q % KX;
     chanoff = row < R ? c * H * W * 4u : OOB;
@@ -256,14 +286,19 @@ struct SrcWgradImage {
   }
   template <int E>
   __device__ void seek(uint32_t k0) {
-    k = k0; oy = k0 / OW; ox = k0 % OW;
+    k = k0; oy = k0 / OW; ox = k0 % OW; woff = 0;
     step_y = BK / OW; step_x = BK % OW;
+    if (OH) { step_y %= OH; }  // a tile may be longer than a whole image of very few pixels
   }
   __device__ void next() {
     k += BK;
     ox += step_x;
     if (ox >= OW) { ox -= OW; oy++; }
     oy += step_y;
+    if (OH) {
+      woff += (BK / (OH * OW)) * C * H * W * 4u;
+      if (oy >= OH) { oy -= OH; woff += C * H * W * 4u; }
+    }
   }
   template <int E>
   __device__ void fetch(float (&v)[E]) const {
@@ -273,7 +308,7 @@ struct SrcWgradImage {
       int32_t iy = iy0 + (int32_t)yy * sy, ix = ix0 + (int32_t)xx * sx;
       bool ok = (k + i < K) && (uint32_t)iy < H && (uint32_t)ix < W;
       uint32_t off = chanoff + ((uint32_t)iy * W + (uint32_t)ix) * 4u;
-      v[i] = buf_load(rsrc, ok ? off : OOB, 0);
+      v[i] = buf_load(rsrc, ok ? off : OOB, woff);
       if (++xx == OW) { xx = 0; ++yy; }
     }
   }
@@ -495,7 +530,7 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
   // Steps come in pairs so that the LDS buffer and the register set of a step are compile-time constants, and the
   // last (up to four) steps, which have less left to write or load, are peeled: every step is free of branches, the
   // compiler counts outstanding memory operations exactly and waits for no more than it must.  Nothing is loaded
-  // past K: the scalar part of a buffer address is not range checked.
+  // past K.
   auto step = [&](auto parity, auto write_next, auto load_ahead) {
     constexpr int cur = decltype(parity)::value, nxt = cur ^ 1;  // tile t lives in LDS buffer cur, tile t+1 in register set nxt
     read_half(fa[1], fb[1], cur, 1);

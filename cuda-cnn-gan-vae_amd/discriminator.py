@@ -135,7 +135,8 @@ class Discriminator:
         CTensorMath.Add(self.bn[i], self.bn[i], p["beta%d" % i])
 
     # ---- backward ------------------------------------------------------------------------------------------
-    def backward(self):
+    def backward(self, fused=False):
+        """fused: the batch-summed weight gradient in one product instead of per-sample gradients and their sum."""
         b, p, g = self.batch, self.p, self.g
         CTensorMath.Sub(self.err, self.prob, self.labels)
         CTensorApplyFunc.ApplyDifferentialSigmoid(self.d_logit, self.logit)
@@ -157,12 +158,15 @@ class Discriminator:
             # convolution layer
             inp, prev = (self.a[i - 1], self.d_a[i - 1]) if i else (self.x, self.d_x)
             CTensorConv.BackwardConvolution(prev, self.d_c[i], p["kernel%d" % i], 4, 4, cin, cout, self.zero_bias[i], 2, 2, 1, 1)
+            CTensorMath.Fill(g["kernel%d" % i], 0.0)
+            CTensorMath.Fill(g["bias%d" % i], 0.0)
+            if fused:
+                Fused.ConvolutionBackwardWeightsSum(g["kernel%d" % i], 4, 4, cin, cout, g["bias%d" % i], inp, self.d_c[i], 2, 2, 1, 1)
+                continue
             CTensorMath.Fill(self.dk_batch[i], 0.0)
             CTensorMath.Fill(self.db_batch[i], 0.0)
             CTensorConv.CreateDeltaWeightAndBias(self.dk_batch[i], 4, 4, cin, cout, self.db_batch[i], inp, self.d_c[i], 2, 2, 1, 1)
-            CTensorMath.Fill(g["kernel%d" % i], 0.0)
             CTensorMath.AddSumW(g["kernel%d" % i], g["kernel%d" % i], self.dk_batch[i])
-            CTensorMath.Fill(g["bias%d" % i], 0.0)
             CTensorMath.AddSumW(g["bias%d" % i], g["bias%d" % i], self.db_batch[i])
 
     def _batchnorm_backward(self, i):
@@ -197,5 +201,5 @@ class Discriminator:
 
     def step(self, fused=False):
         self.forward(fused)
-        self.backward()
+        self.backward(fused)
         self.update()

@@ -336,6 +336,11 @@ class Fused:
              opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
 
     @staticmethod
+    def ConvolutionBackwardWeightsSum(dkernel, dkernel_x, dkernel_y, dkernel_z, dkernel_amount, dbias, image, delta, stride_x, stride_y, padding_x, padding_y):
+        call("mt_convolution_backward_weights_sum", _d(dkernel), _i(dkernel_x), _i(dkernel_y), _i(dkernel_z), _u(dkernel_amount), _d(dbias), _d(image),
+             _d(delta), _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y))
+
+    @staticmethod
     def BatchNormForwardInfer(out, inp, gamma, beta, mean, variable, epsilon=1e-6, func=None):
         call("mt_batchnorm_forward_infer_func", _d(out), _d(inp), _d(gamma), _d(beta), _d(mean), _d(variable), _f(epsilon), C.c_int(FUNC[func]))
 

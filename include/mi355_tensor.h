@@ -77,8 +77,9 @@ void *mt_get_stream(void);               /* the hipStream_t all work is queued o
 int mt_set_stream(void *hip_stream);     /* queue on a caller-owned stream (NULL: back to the library's own) */
 /* "conv_path": 0 choose per shape (default), 1 one-thread-per-output kernels in the CPU path's summation order,
  * 2 matrix-core kernels wherever they apply.  "igemm_tile": -1 choose per shape (default), 0..3 force the block
- * tile 128x128 / 64x128 / 32x128 / 64x64 of the matrix-core kernels.  For tests and measurements; results agree
- * within fp32 rounding. */
+ * tile 128x128 / 64x128 / 32x128 / 64x64 of the matrix-core kernels.  "wgrad_groups": 0 choose per shape (default),
+ * n split the batch of mt_convolution_backward_weights_sum into n groups (when n divides the batch).  For tests and
+ * measurements; results agree within fp32 rounding. */
 int mt_set_option(const char *name, int value);
 
 /* ---- convolutions: CTensorConv<T> (cuda/ctensorconv.cu.h:63-66) ---- */
@@ -162,6 +163,14 @@ int mt_batchnorm_forward_train_func(const mt_tensor *output, const mt_tensor *in
 /* The same layer in inference mode (lines 326-371): stored mean / variable instead of batch statistics. */
 int mt_batchnorm_forward_infer_func(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
                                     const mt_tensor *mean, const mt_tensor *variable, float epsilon, int func);
+
+/* ---- fused backward sequences ---- */
+/* CNetLayerConvolution::TrainingBackward, netlayer/cnetlayerconvolution.cu.h:501-508, without the per-sample round trip:
+ * dkernel [1,1,Kamt,C*Ky*Kx] += sum over the batch of the per-sample weight gradients (CreateDeltaWeightAndBias into a
+ * zeroed batch tensor, then AddSumW), dbias [1,Kamt,1,1] += sum over the batch and the pixels of delta. */
+int mt_convolution_backward_weights_sum(const mt_tensor *dkernel, int32_t dkernel_x, int32_t dkernel_y, int32_t dkernel_z,
+                                        uint32_t dkernel_amount, const mt_tensor *dbias, const mt_tensor *image,
+                                        const mt_tensor *delta, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y);
 
 /* ---- timing: replaces CCUDATimeSpent / CTimeStamp (cuda/ccudatimespent.cu:38-52, cuda/ctimestamp.cu:17-32) ----
  * While enabled, every kernel launch of the hot path is bracketed by two events on the work stream and its

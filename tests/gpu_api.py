@@ -35,6 +35,11 @@ class Gpu:
         fn(dk, kx, ky, kz, ka, db, up(image), up(delta), sx, sy, px, py)
         return dk.numpy(), db.numpy()
 
+    def convolution_backward_weights_sum(self, dkernel, dbias, image, delta, kx, ky, kz, ka, sx, sy, px, py):
+        dk, db = up(dkernel), up(dbias)
+        Fused.ConvolutionBackwardWeightsSum(dk, kx, ky, kz, ka, db, up(image), up(delta), sx, sy, px, py)
+        return dk.numpy(), db.numpy()
+
     # ---- products -------------------------------------------------------
     def mul(self, left, right, out_w=None):
         left, right = np.asarray(left, np.float32), np.asarray(right, np.float32)

@@ -161,3 +161,12 @@ def test_config5_full_batch_properties(gpu, oracle):
         assert rel_err(db_batch[sample:sample + 1], db) <= REL, "bias gradient %d" % i
         assert rel_err(net.g["kernel%d" % i].numpy(), dk_batch.astype(np.float64).sum(0, keepdims=True)) <= REL
         assert np.max(np.abs(net.g["bias%d" % i].numpy() - db_batch.astype(np.float64).sum(0, keepdims=True))) <= REL * np.abs(db_batch).sum(0).max()
+    # (4) the batch-summed weight gradient in one product gives the same gradients
+    literal = {name: t.numpy() for name, t in net.g.items()}
+    net.backward(fused=True)
+    for name, want in literal.items():
+        if name.startswith("bias"):
+            i = int(name[4:])
+            assert np.max(np.abs(net.g[name].numpy() - want)) <= REL * np.abs(net.db_batch[i].numpy()).sum(0).max(), name
+        else:
+            assert rel_err(net.g[name].numpy(), want) <= REL, name

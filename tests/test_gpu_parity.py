@@ -221,6 +221,38 @@ def test_wgrad_w_broadcast(gpu, oracle, path):
     close(got[1], want[1])
 
 
+@pytest.mark.parametrize("case", [
+    # B, C, H, W, KA, k, s, p
+    (6, 3, 16, 16, 8, 4, 2, 1),      # 64 output pixels per sample: the batch is split into groups
+    (4, 5, 8, 8, 70, 3, 1, 1),       # sizes that are no multiple of a tile
+    (3, 2, 9, 7, 5, 3, 1, 1),        # 63 output pixels: not a multiple of the k step, per-sample path
+    (5, 16, 8, 8, 130, 4, 2, 1),     # 16 output pixels: one k step per sample
+    (2, 40, 32, 32, 64, 4, 2, 1),    # 256 output pixels, 640 columns
+    (7, 1, 4, 4, 1, 1, 1, 0),        # 1x1 kernel, one channel, odd batch
+])
+def test_convolution_backward_weights_sum(gpu, oracle, path, case):
+    """The batch-summed weight gradient against the layer's own sequence: per-sample gradients into zeroed batch
+    tensors, then AddSumW into gradients that already hold something (cnetlayerconvolution.cu.h:501-508)."""
+    B, C, H, Wd, KA, k, s, p = case
+    oy, ox = (H - k + 2 * p) // s + 1, (Wd - k + 2 * p) // s + 1
+    image, delta = U(11, B, C, H, Wd), U(12, B, KA, oy, ox)
+    dk0, db0 = U(13, 1, 1, KA, C * k * k), U(14, 1, KA, 1, 1)
+    dkb, dbb = oracle.create_delta_weight_and_bias(np.zeros((B, 1, KA, C * k * k), np.float32), np.zeros((B, KA, 1, 1), np.float32),
+                                                   image, delta, k, k, C, KA, s, s, p, p)
+    want_k, want_b = oracle.add_sum_w(dk0, dkb, out_init=dk0), oracle.add_sum_w(db0, dbb, out_init=db0)
+    import mi355tensor as mt
+    for groups in (0, 1, 2, B):   # chosen per shape; the whole batch in one product; several samples per group; one each
+        if groups and B % groups:
+            continue
+        mt.set_option("wgrad_groups", groups)
+        try:
+            got_k, got_b = gpu.convolution_backward_weights_sum(dk0, db0, image, delta, k, k, C, KA, s, s, p, p)
+        finally:
+            mt.set_option("wgrad_groups", 0)
+        close(got_k, want_k)
+        close(got_b, want_b)
+
+
 def test_fused_conv_activation(gpu, oracle, path):
     image, kernel, bias = U(1, 3, 4, 10, 10), U(2, 1, 1, 6, 4 * 9), U(3, 1, 6, 1, 1)
     for func in ("leaky_relu", "relu", "tangence", "sigmoid"):
@@ -234,7 +266,9 @@ def test_fused_conv_activation(gpu, oracle, path):
 
 
 @pytest.mark.parametrize("m,k,n,wl,wr,z", [(1, 1, 1, 1, 1, 1), (33, 65, 31, 1, 3, 2), (64, 100, 1, 1, 5, 1), (70, 32, 96, 2, 2, 1), (5, 300, 7, 3, 1, 1),
-                                           (200, 77, 150, 1, 4, 1), (130, 260, 1, 1, 70, 1), (96, 40, 1, 1, 1, 1), (17, 9, 40, 4, 4, 3)])
+                                           (200, 77, 150, 1, 4, 1), (130, 260, 1, 1, 70, 1), (96, 40, 1, 1, 1, 1), (17, 9, 40, 4, 4, 3),
+                                           # few output tiles and a long k axis: the product is split over k
+                                           (1, 8192, 1, 1, 128, 1), (70, 1000, 3, 1, 4, 1), (33, 650, 20, 5, 1, 1), (128, 2052, 1, 1, 64, 1)])
 def test_products(gpu, oracle, m, k, n, wl, wr, z):
     a, b, at = U(1, wl, z, m, k), U(2, wr, z, k, n), U(3, wl, z, k, m)
     close(gpu.mul(a, b), oracle.mul(a, b), 1e-5)
@@ -351,6 +385,15 @@ def test_empty_tensors(gpu):
 
 
 # ---- layers: literal op sequences on both back ends, and the fused entry points ----------------
+
+def test_linear_layer_split_over_k(gpu, oracle):
+    """Few outputs, many inputs (the last layer of a discriminator): bias and activation after the k ranges are added."""
+    w, x, b = U(1, 1, 1, 3, 2048) * 0.05, Nrm(2, 10, 8, 16, 16), U(3, 1, 1, 3, 1)
+    want = seq.linear_forward(oracle, w, x, b)
+    close(gpu.linear_forward(w, x, b), want, 1e-5)
+    close(gpu.linear_forward(w, x, b, func="sigmoid"), oracle.apply_func(want, "sigmoid"), 1e-5)
+    close(gpu.linear_forward(w, x, b, func="leaky_relu"), oracle.apply_func(want, "leaky_relu"), 1e-5)
+
 
 def test_linear_layer(gpu, oracle):
     w, x, b = U(1, 1, 1, 96, 8 * 4 * 4), Nrm(2, 12, 8, 4, 4), U(3, 1, 1, 96, 1)
