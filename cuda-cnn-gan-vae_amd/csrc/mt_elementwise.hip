@@ -433,6 +433,97 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
   }
 }
 
+// Backward pass of the same layer in one kernel (netlayer/cnetlayerbatchnormalization.cu.h:578-604):
+//   dxhat = delta*gamma;  s1 = sum_w dxhat;  s2 = sum_w dxhat*xhat;  dgamma += sum_w delta*xhat;  dbeta += sum_w delta;
+//   error = ((N*dxhat - xhat*s2) - s1) * ivar * (1/N)            (each step rounded to fp32, in this order)
+// Block layout as bn_fused_kernel.  NW > 0: a thread keeps its NW rows of delta and xhat in registers between the
+// sums and the error; NW == 0: any batch size, the rows are read a second time.
+template <int RB, int NW>
+__global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, float *dgamma, float *dbeta, const float *delta, const float *gamma,
+                                                                 const float *xhat, const float *ivar, uint32_t W, uint32_t S, float n, float inv_n) {
+  constexpr int WS = EW_THREADS / RB, HOLD = NW > 0 ? NW : 1;
+  __shared__ float part[4][WS][RB * 4];
+  __shared__ float col_s1[RB * 4], col_s2[RB * 4];
+  const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
+  const uint32_t r = (blockIdx.x * RB + rl) * 4;
+  float4 qd[HOLD], qx[HOLD];
+  float acc[4][4] = {};
+  float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
+  auto add = [&](const float4 &d, const float4 &x) {
+    const float dv[4] = {d.x, d.y, d.z, d.w}, xv[4] = {x.x, x.y, x.z, x.w}, gv[4] = {g.x, g.y, g.z, g.w};
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const float dx = dv[v] * gv[v];
+      acc[0][v] += dx;
+      acc[1][v] += dx * xv[v];
+      acc[2][v] += dv[v] * xv[v];
+      acc[3][v] += dv[v];
+    }
+  };
+  if (r < S) {
+    g = *reinterpret_cast<const float4 *>(gamma + r);
+    if constexpr (NW > 0) {
+#pragma unroll
+      for (int i = 0; i < NW; i++) {
+        const uint32_t w = ws + i * WS;
+        if (w < W) {
+          qd[i] = *reinterpret_cast<const float4 *>(delta + (size_t)w * S + r);
+          qx[i] = *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NW; i++)
+        if (ws + i * WS < W) add(qd[i], qx[i]);
+    } else {
+#pragma unroll 4
+      for (uint32_t w = ws; w < W; w += WS)
+        add(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r));
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 4; q++)
+#pragma unroll
+    for (int v = 0; v < 4; v++) part[q][ws][rl * 4 + v] = acc[q][v];
+  __syncthreads();
+  const int c = threadIdx.x;
+  const uint32_t rc = blockIdx.x * RB * 4 + c;
+  if (c < RB * 4 && rc < S) {  // the first RB*4 threads finish one column each
+    float t[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < WS; i++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) t[q] += part[q][i][c];
+    col_s1[c] = t[0];
+    col_s2[c] = t[1];
+    if (dgamma) dgamma[rc] = dgamma[rc] + t[2];
+    if (dbeta) dbeta[rc] = dbeta[rc] + t[3];
+  }
+  __syncthreads();
+  if (r >= S) return;
+  const float4 s1 = *reinterpret_cast<const float4 *>(col_s1 + rl * 4), s2 = *reinterpret_cast<const float4 *>(col_s2 + rl * 4);
+  const float4 iv = *reinterpret_cast<const float4 *>(ivar + r);
+  auto error = [&](const float4 &d, const float4 &x) {
+    float4 e;
+    e.x = (((n * (d.x * g.x)) - (x.x * s2.x)) - s1.x) * iv.x * inv_n;
+    e.y = (((n * (d.y * g.y)) - (x.y * s2.y)) - s1.y) * iv.y * inv_n;
+    e.z = (((n * (d.z * g.z)) - (x.z * s2.z)) - s1.z) * iv.z * inv_n;
+    e.w = (((n * (d.w * g.w)) - (x.w * s2.w)) - s1.w) * iv.w * inv_n;
+    return e;
+  };
+  if constexpr (NW > 0) {
+#pragma unroll
+    for (int i = 0; i < NW; i++) {
+      const uint32_t w = ws + i * WS;
+      if (w >= W) break;
+      *reinterpret_cast<float4 *>(err + (size_t)w * S + r) = error(qd[i], qx[i]);
+    }
+  } else {
+    for (uint32_t w = ws; w < W; w += WS)
+      *reinterpret_cast<float4 *>(err + (size_t)w * S + r) =
+          error(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r));
+  }
+}
+
 __global__ __launch_bounds__(EW_THREADS) void bn_ivar_kernel(float *ivar, const float *var, uint32_t S, float eps) {
   uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
   if (i < S) ivar[i] = (float)(1.0 / (double)sqrtf(var[i] + eps));
@@ -686,6 +777,55 @@ int mt_batchnorm_forward_infer_func(const mt_tensor *out, const mt_tensor *in, c
   unsigned gy = W < 16 ? W : 16;
   bn_apply_kernel<<<dim3(gx, gy), EW_THREADS, 0, mt::stream()>>>(out->p, nullptr, in->p, mean->p, scratch, gamma->p, beta->p, (uint32_t)S, W, vec, func);
   MT_LAUNCH_CHECK("bn_apply");
+  return MT_OK;
+}
+
+int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
+                          const mt_tensor *xhat, const mt_tensor *ivar) {
+  const mt_tensor *need[5] = {error, delta, gamma, xhat, ivar};
+  for (auto t : need)
+    if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: null tensor");
+  if (!mt::same_zyx(error, delta) || error->w != delta->w || !mt::same_zyx(xhat, delta) || xhat->w != delta->w || !mt::same_zyx(gamma, delta) ||
+      !mt::same_zyx(ivar, delta))
+    return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: sizes do not match");
+  for (auto t : {dgamma, dbeta})
+    if (t && (mt::bad(t) || !mt::same_zyx(t, delta))) return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: gradients must be [1,Z,Y,X]");
+  const size_t S = (size_t)delta->z * delta->y * delta->x;
+  const uint32_t W = delta->w;
+  if (S == 0 || W == 0) return MT_OK;
+  const float n = (float)W, inv_n = (float)(1.0 / (double)n);
+  float *pg = dgamma ? dgamma->p : nullptr, *pb = dbeta ? dbeta->p : nullptr;
+  const bool vec = S % 4 == 0 && aligned16(error->p) && aligned16(delta->p) && aligned16(gamma->p) && aligned16(xhat->p) && aligned16(ivar->p);
+  if (!vec) {
+    // any layout: the layer's own sequence of tensor operations, on workspace tensors
+    float *ws = nullptr;
+    int rc = bn_scratch(2 * S + 2 * (size_t)W * S, &ws);
+    if (rc) return rc;
+    mt_tensor s1{ws, 1, delta->z, delta->y, delta->x}, s2{ws + S, 1, delta->z, delta->y, delta->x};
+    mt_tensor dx{ws + 2 * S, W, delta->z, delta->y, delta->x}, t{ws + 2 * S + (size_t)W * S, W, delta->z, delta->y, delta->x};
+    if ((rc = mt_fill(&s1, 0.f)) || (rc = mt_fill(&s2, 0.f))) return rc;
+    if ((rc = mt_tensor_item_production(&dx, delta, gamma)) || (rc = mt_add_sum_w(&s1, &s1, &dx, 1.f, 1.f))) return rc;
+    if ((rc = mt_tensor_item_production(&t, &dx, xhat)) || (rc = mt_add_sum_w(&s2, &s2, &t, 1.f, 1.f))) return rc;
+    if (dgamma && ((rc = mt_tensor_item_production(&t, delta, xhat)) || (rc = mt_add_sum_w(dgamma, dgamma, &t, 1.f, 1.f)))) return rc;
+    if (dbeta && (rc = mt_add_sum_w(dbeta, dbeta, delta, 1.f, 1.f))) return rc;
+    if ((rc = mt_mul_value(error, &dx, n)) || (rc = mt_tensor_item_production(&t, xhat, &s2))) return rc;
+    if ((rc = mt_sub(error, error, &t, 1.f, 1.f)) || (rc = mt_sub(error, error, &s1, 1.f, 1.f))) return rc;
+    if ((rc = mt_tensor_item_production(error, error, ivar))) return rc;
+    return mt_mul_value(error, error, inv_n);
+  }
+  mt::ProfileScope prof("bn_backward");
+  int rb = S / 128 >= 512 ? 32 : S / 64 >= 512 ? 16 : 8;
+  while (rb > 8 && cdiv(W, EW_THREADS / rb) > 16) rb /= 2;
+  const uint32_t nw = cdiv(W, EW_THREADS / rb);
+  const unsigned grid = cdiv(S, (size_t)rb * 4);
+#define MT_BN_BWD(RB, NW) \
+  bn_backward_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(error->p, pg, pb, delta->p, gamma->p, xhat->p, ivar->p, W, (uint32_t)S, n, inv_n)
+#define MT_BN_BWD_NW(RB) \
+  do { if (nw <= 4) MT_BN_BWD(RB, 4); else if (nw <= 8) MT_BN_BWD(RB, 8); else if (nw <= 16) MT_BN_BWD(RB, 16); else MT_BN_BWD(RB, 0); } while (0)
+  if (rb == 32) MT_BN_BWD_NW(32); else if (rb == 16) MT_BN_BWD_NW(16); else MT_BN_BWD_NW(8);
+#undef MT_BN_BWD_NW
+#undef MT_BN_BWD
+  MT_LAUNCH_CHECK("mt_batchnorm_backward");
   return MT_OK;
 }
 

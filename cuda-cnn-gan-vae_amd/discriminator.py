@@ -136,7 +136,8 @@ class Discriminator:
 
     # ---- backward ------------------------------------------------------------------------------------------
     def backward(self, fused=False):
-        """fused: the batch-summed weight gradient in one product instead of per-sample gradients and their sum."""
+        """fused: the batch-norm backward pass as one kernel and the batch-summed weight gradient as one product,
+        instead of the layers' sequences of tensor operations."""
         b, p, g = self.batch, self.p, self.g
         CTensorMath.Sub(self.err, self.prob, self.labels)
         CTensorApplyFunc.ApplyDifferentialSigmoid(self.d_logit, self.logit)
@@ -154,7 +155,12 @@ class Discriminator:
             # function layer
             CTensorApplyFunc.ApplyDifferentialLeakyReLU(self.d_bn[i], self.bn[i])
             CTensorMath.TensorItemProduction(self.d_bn[i], self.d_a[i], self.d_bn[i])
-            self._batchnorm_backward(i)
+            if fused:
+                CTensorMath.Fill(g["gamma%d" % i], 0.0)
+                CTensorMath.Fill(g["beta%d" % i], 0.0)
+                Fused.BatchNormBackward(self.d_c[i], g["gamma%d" % i], g["beta%d" % i], self.d_bn[i], p["gamma%d" % i], self.xhat[i], self.ivar[i])
+            else:
+                self._batchnorm_backward(i)
             # convolution layer
             inp, prev = (self.a[i - 1], self.d_a[i - 1]) if i else (self.x, self.d_x)
             CTensorConv.BackwardConvolution(prev, self.d_c[i], p["kernel%d" % i], 4, 4, cin, cout, self.zero_bias[i], 2, 2, 1, 1)

@@ -336,6 +336,11 @@ class Fused:
              opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
 
     @staticmethod
+    def BatchNormBackward(error, dgamma, dbeta, delta, gamma, xhat, ivar):
+        opt = lambda t: _d(t) if t is not None else None
+        call("mt_batchnorm_backward", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), _d(xhat), _d(ivar))
+
+    @staticmethod
     def ConvolutionBackwardWeightsSum(dkernel, dkernel_x, dkernel_y, dkernel_z, dkernel_amount, dbias, image, delta, stride_x, stride_y, padding_x, padding_y):
         call("mt_convolution_backward_weights_sum", _d(dkernel), _i(dkernel_x), _i(dkernel_y), _i(dkernel_z), _u(dkernel_amount), _d(dbias), _d(image),
              _d(delta), _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y))

@@ -165,6 +165,12 @@ int mt_batchnorm_forward_infer_func(const mt_tensor *output, const mt_tensor *in
                                     const mt_tensor *mean, const mt_tensor *variable, float epsilon, int func);
 
 /* ---- fused backward sequences ---- */
+/* CNetLayerBatchNormalization::TrainingBackward, netlayer/cnetlayerbatchnormalization.cu.h:578-604, as one kernel:
+ * error [B,Z,Y,X] = ((N*dxhat - xhat*sum_w(dxhat*xhat)) - sum_w(dxhat)) * ivar * (1/N) with dxhat = delta*gamma;
+ * dgamma [1,Z,Y,X] += sum_w(delta*xhat), dbeta += sum_w(delta) (NULL to skip, as create_delta_weight == false does).
+ * `error` may be the same tensor as `delta`. */
+int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta,
+                          const mt_tensor *gamma, const mt_tensor *xhat, const mt_tensor *ivar);
 /* CNetLayerConvolution::TrainingBackward, netlayer/cnetlayerconvolution.cu.h:501-508, without the per-sample round trip:
  * dkernel [1,1,Kamt,C*Ky*Kx] += sum over the batch of the per-sample weight gradients (CreateDeltaWeightAndBias into a
  * zeroed batch tensor, then AddSumW), dbias [1,Kamt,1,1] += sum over the batch and the pixels of delta. */

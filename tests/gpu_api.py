@@ -198,6 +198,12 @@ class Gpu:
             res["new_mean"], res["new_var"] = nm.numpy(), nv.numpy()
         return res
 
+    def batchnorm_backward(self, delta, gamma, xhat, ivar, dgamma0, dbeta0):
+        delta = np.asarray(delta, np.float32)
+        err, dg, db = CTensor(*delta.shape), up(dgamma0), up(dbeta0)
+        Fused.BatchNormBackward(err, dg, db, up(delta), up(gamma), up(xhat), up(ivar))
+        return err.numpy(), dg.numpy(), db.numpy()
+
     def batchnorm_infer(self, x, gamma, beta, mean, var, eps=1e-6, func=None):
         x = np.asarray(x, np.float32)
         out = CTensor(*x.shape)

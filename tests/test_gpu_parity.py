@@ -433,6 +433,23 @@ def test_batchnorm_layer(gpu, oracle):
         close(got, exp, 1e-5)
 
 
+@pytest.mark.parametrize("shape", [(16, 3, 6, 6), (5, 2, 3, 3), (40, 8, 16, 16), (130, 4, 8, 8), (300, 1, 4, 8), (7, 64, 32, 32)])
+def test_batchnorm_backward_fused(gpu, oracle, shape):
+    """The one-kernel backward pass against the layer's sequence of tensor operations, gradients accumulating into
+    non-zero tensors; shapes cover register-resident and re-read batches, vector and scalar layouts."""
+    x, gamma, beta = Nrm(1, *shape) * 1.5 + 0.3, U(2, 1, *shape[1:]) + 1.5, U(3, 1, *shape[1:])
+    fwd = seq.batchnorm_forward_train(oracle, x, gamma, beta)
+    delta = U(4, *shape)
+    want_err, want_dg, want_db = seq.batchnorm_backward(oracle, delta, gamma, fwd["xhat"], fwd["ivar"])
+    dg0, db0 = U(5, 1, *shape[1:]), U(6, 1, *shape[1:])
+    err, dg, db = gpu.batchnorm_backward(delta, gamma, fwd["xhat"], fwd["ivar"], dg0, db0)
+    # the error is a difference of nearly equal terms: it is measured against the size of those terms
+    scale = float(shape[0]) * np.abs(delta * gamma).max() * np.abs(fwd["ivar"]).max() / shape[0]
+    assert np.max(np.abs(err - want_err)) <= 1e-5 * max(scale, np.abs(want_err).max())
+    close(dg - dg0, want_dg, 1e-5)
+    close(db - db0, want_db, 1e-5)
+
+
 def test_conv_layer_forward_backward(gpu, oracle, path):
     x, kernel, bias = U(1, 6, 3, 16, 16), Nrm(2, 1, 1, 8, 3 * 16, std=0.1), U(3, 1, 8, 1, 1) * 0.1
     want = seq.conv_forward(oracle, x, kernel, bias, 4, 2, 1)
