@@ -72,6 +72,51 @@ def cpu_baseline(sample_batch):
             "sample": "one generator forward at batch %d (%.1f s), scaled linearly; host has %d cores" % (sample_batch, dt, os.cpu_count() or 0)}
 
 
+def discriminator_step(args):
+    """Secondary workload (configs[4]): forward, backward and Adam update of the DCGAN-64 discriminator at batch 128
+    through the fused entry points.  Same two timed regions as the main workload; one JSON line."""
+    import mi355tensor as mt
+    import discriminator as D
+    batch = 128
+    net = D.Discriminator(batch)
+    net.set_batch(*D.make_batch(batch))
+    stream = mt.get_stream()
+    create, record, elapsed_ms = hip_events()
+    for _ in range(args.warmup):
+        net.step(fused=True)
+    mt.synchronize()
+    e0, e1 = create(), create()
+    t0 = time.perf_counter()
+    record(e0, stream)
+    for _ in range(args.steps):
+        net.step(fused=True)
+    record(e1, stream)
+    mt.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = elapsed_ms(e0, e1)
+    mt.profile_enable(True)
+    for _ in range(args.steps):
+        net.step(fused=True)
+    prof = mt.profile_report()
+    mt.profile_enable(False)
+    ms_per_step = max(gpu_ms, wall_ms) / args.steps
+    conv = {k: v for k, v in prof.items() if k.startswith(("mt_forward_convolution", "mt_backward_convolution", "mt_convolution_backward_weights_sum"))}
+    conv_ms = sum(v[1] for v in conv.values()) / args.steps
+    flop = 3.0 * sum(D.conv_flops(batch))   # forward, input gradient, weight gradient
+    print(json.dumps({
+        "metric": "images/sec, DCGAN-64 discriminator training step fp32 b=128 (secondary workload)",
+        "value": batch / (ms_per_step * 1e-3), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[4]: DCGAN-64 discriminator, batch 128: conv 4x4 s2 p1 3->64->128->256->512 with BN + leaky ReLU, "
+                               "Linear 8192->1, sigmoid; forward, backward (input, weight, bias, BN gradients), Adam", "global_batch": batch,
+                   "path": "fused C-ABI entry points"},
+        "gpu_ms_per_step_events": gpu_ms / args.steps, "host_ms_per_step_wall": wall_ms / args.steps,
+        "kernel_ms_per_step_sum": sum(v[1] for v in prof.values()) / args.steps,
+        "conv_gflops": flop / (conv_ms * 1e-3) / 1e9, "conv_ms_per_step": conv_ms,
+        "conv_frac_of_fp32_mfma_peak": flop / (conv_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+        "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -82,9 +127,14 @@ def main():
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also launch one plain copy (mt_set) of this many MiB before the timed region: the known-size kernel "
                          "that calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--workload", choices=["c3", "c5"], default="c3",
+                    help="c3 (default, the measured configuration): DCGAN-64 generator forward, batch 256; "
+                         "c5 (secondary): DCGAN-64 discriminator training step, batch 128")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the path shards along the batch axis, see DESIGN.md")
+    if args.workload == "c5":
+        return discriminator_step(args)
 
     import mi355tensor as mt
     import generator as G

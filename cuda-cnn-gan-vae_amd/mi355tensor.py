@@ -52,9 +52,7 @@ def lib():
 
 
 def call(name, *args):
-    fn = getattr(lib(), name)
-    fn.restype = C.c_int
-    rc = fn(*args)
+    rc = getattr(_lib or lib(), name)(*args)   # ctypes' default result type is int
     if rc != 0:
         raise TensorError(name, rc, lib().mt_last_error().decode(errors="replace"))
 
@@ -149,6 +147,14 @@ class CTensor:
     def desc(self):
         return MtTensor(self.ptr.value, *self.shape)
 
+    def ref(self):
+        """Pointer to this tensor's descriptor for a C-ABI call (built once: pointer and sizes never change)."""
+        r = self.__dict__.get("_ref")
+        if r is None:
+            self._desc = self.desc()
+            r = self._ref = C.byref(self._desc)
+        return r
+
     def free(self):
         if self.owned and self.ptr:
             call("mt_free", self.ptr)
@@ -162,7 +168,7 @@ class CTensor:
 
 
 def _d(t):
-    return C.byref(t.desc())
+    return t.ref()
 
 
 def _i(v):
