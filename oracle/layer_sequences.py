@@ -169,3 +169,26 @@ def discriminator_backward(lib, params, acts, labels):
         grads["d_c%d" % i] = d_c
     grads["d_x"] = err
     return grads
+
+
+def upsampling_forward(lib, x, u):
+    """CNetLayerUpSampling::Forward, netlayer/cnetlayerupsampling.cu.h:233-252."""
+    return lib.upsampling(x, u, u)
+
+
+def gan_generator_forward(lib, params, noise, channels=(512, 512, 256, 128, 64, 32, 16), image_depth=3):
+    """The generator the reference ships (cuda/netmodel/cmodel_gan.cu.h:131-230): Linear to 3*4*C0, leaky ReLU, viewed as
+    [B,C0,3,4]; six times (up-sampling x2, conv 3x3 stride 1 padding 1, BatchNorm in training mode, leaky ReLU); conv 3x3
+    to the image depth, tanh: [B,depth,192,256].  `channels[0]` is C0, `channels[1:]` the six convolution widths;
+    parameter names: lin_w, lin_b, kernel0..6, bias0..6, gamma0..5, beta0..5."""
+    b = noise.shape[0]
+    h = function_forward(lib, linear_forward(lib, params["lin_w"], noise, params["lin_b"]), "leaky_relu")
+    h = np.ascontiguousarray(h).reshape(b, channels[0], 3, 4)
+    outs = {"h0": h}
+    for i in range(6):
+        c = conv_forward(lib, upsampling_forward(lib, h, 2), params["kernel%d" % i], params["bias%d" % i], 3, 1, 1)
+        bn = batchnorm_forward_train(lib, c, params["gamma%d" % i], params["beta%d" % i])["out"]
+        h = function_forward(lib, bn, "leaky_relu")
+        outs["c%d" % i], outs["h%d" % (i + 1)] = c, h
+    outs["image"] = function_forward(lib, conv_forward(lib, h, params["kernel6"], params["bias6"], 3, 1, 1), "tangence")
+    return outs

@@ -170,3 +170,41 @@ def test_config5_full_batch_properties(gpu, oracle):
             assert np.max(np.abs(net.g[name].numpy() - want)) <= REL * np.abs(net.db_batch[i].numpy()).sum(0).max(), name
         else:
             assert rel_err(net.g[name].numpy(), want) <= REL, name
+
+
+def test_shipped_gan_generator_topology(gpu, oracle):
+    """The generator of the reference's own GAN model (Linear, then up-sampling + conv 3x3 + BatchNorm + leaky ReLU six
+    times, conv 3x3 + tanh; 3x4 -> 192x256), every layer output against the oracle, at a quarter of the shipped widths
+    and batch 4 so that the CPU side finishes in seconds."""
+    channels, noise_size, b = (128, 128, 64, 32, 16, 8, 4), 64, 4
+    rng = np.random.default_rng(6)
+    params = {"lin_w": (rng.standard_normal((1, 1, 12 * channels[0], noise_size)) * 0.1).astype(np.float32),
+              "lin_b": np.full((1, 1, 12 * channels[0], 1), 0.1, np.float32)}
+    size, widths = (3, 4), channels[1:] + (3,)
+    for i in range(7):
+        cin, cout = (channels[0] if i == 0 else widths[i - 1]), widths[i]
+        params["kernel%d" % i] = (rng.standard_normal((1, 1, cout, cin * 9)) * np.sqrt(2.0 / (cin * 9))).astype(np.float32)
+        params["bias%d" % i] = (rng.standard_normal((1, cout, 1, 1)) * 0.05).astype(np.float32)
+        if i < 6:
+            size = (size[0] * 2, size[1] * 2)
+            params["gamma%d" % i] = rng.uniform(0.5, 1.5, (1, cout) + size).astype(np.float32)
+            params["beta%d" % i] = rng.uniform(-0.2, 0.2, (1, cout) + size).astype(np.float32)
+    noise = rng.standard_normal((b, 1, noise_size, 1)).astype(np.float32)
+    want = seq.gan_generator_forward(oracle, params, noise, channels)
+    # layer by layer on the oracle's own inputs: a batch norm over four samples divides by spreads that can be tiny, so
+    # rounding differences of one layer would otherwise be amplified by the next ones
+    h0 = seq.function_forward(gpu, seq.linear_forward(gpu, params["lin_w"], noise, params["lin_b"]), "leaky_relu")
+    assert rel_err(h0.reshape(want["h0"].shape), want["h0"]) <= REL
+    for i in range(6):
+        up = seq.upsampling_forward(oracle, want["h%d" % i], 2)
+        assert np.array_equal(seq.upsampling_forward(gpu, want["h%d" % i], 2), up), "up-sampling %d is an index map: bit-exact" % i
+        assert rel_err(seq.conv_forward(gpu, up, params["kernel%d" % i], params["bias%d" % i], 3, 1, 1), want["c%d" % i]) <= REL, "conv %d" % i
+        bn = seq.batchnorm_forward_train(gpu, want["c%d" % i], params["gamma%d" % i], params["beta%d" % i])["out"]
+        assert rel_err(seq.function_forward(gpu, bn, "leaky_relu"), want["h%d" % (i + 1)]) <= REL, "batch norm %d" % i
+        fused = gpu.batchnorm_train(want["c%d" % i], params["gamma%d" % i], params["beta%d" % i], func="leaky_relu")["out"]
+        assert rel_err(fused, want["h%d" % (i + 1)]) <= REL, "fused batch norm %d" % i
+    image = gpu.forward_convolution(want["h6"], params["kernel6"], params["bias6"], 3, 3, widths[5], 3, 1, 1, 1, 1, func="tangence")
+    assert rel_err(image, want["image"]) <= REL
+    # end to end: the whole stack on the device, seven layers of accumulated rounding
+    got = seq.gan_generator_forward(gpu, params, noise, channels)
+    assert got["image"].shape == (b, 3, 192, 256) and rel_err(got["image"], want["image"]) <= 2e-3
