@@ -13,6 +13,9 @@ namespace mt {
 hipStream_t stream();
 int fail(int code, const char *fmt, ...);  // records the message, returns `code`
 int hip_fail(hipError_t e, const char *what);
+// split-K: workspace for S partial results, and out[i] = func(sum_s partial[s][i] + bias[(i / bias_div) % bias_mod])
+int split_workspace(size_t floats, float **p);
+int split_reduce(const char *name, float *out, const float *partial, uint32_t S, size_t n, const float *bias, uint32_t bias_div, uint32_t bias_mod, int func);
 int set_conv_path(int v);  // 0 auto, 1 direct kernels, 2 matrix cores wherever they apply
 int set_igemm_tile(int v); // -1 auto, 0..3 force one block tile of the matrix-core kernels
 int set_wgrad_groups(int v);  // 0 auto, else batch groups of the batch-summed weight gradient

@@ -548,6 +548,16 @@ int launch_tconv_small(const char *name, TconvArgs &args, uint32_t max_n) {
   return MT_OK;
 }
 
+// Weights of a forward convolution re-ordered tap-major for SrcIm2colTap: packed[m][t*C + c] = kernel[m][c*taps + t]
+__global__ __launch_bounds__(256) void conv_pack_tap_major_kernel(float *packed, const float *kernel, uint32_t ker_ld, uint32_t KA, uint32_t C, uint32_t taps) {
+  const uint32_t K = C * taps;
+  const size_t total = (size_t)KA * K;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
+    const uint32_t m = (uint32_t)(idx / K), k = (uint32_t)(idx % K), t = k / C, c = k % C;
+    packed[idx] = kernel[(size_t)m * ker_ld + c * taps + t];
+  }
+}
+
 // ---- argument checks shared by the plain and the fused entry points ---------------------------------------------
 int check_forward(const char *name, const mt_tensor *out, const mt_tensor *image, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz,
                   uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py) {
@@ -597,14 +607,34 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
   ep.func = func_later ? MT_F_NONE : func;
   if (kernel->w == 1) {  // one kernel set for the whole batch: fold the batch into the columns
     b.R = out->w * OHW;
-    const uint32_t taps = (uint32_t)ky * kx;
+    const uint32_t taps = (uint32_t)ky * kx, N = out->w * OHW;
+    const size_t out_floats = mt::count(out);
+    // one product, split over k when it has few output tiles (needs one bias set: the partial sums are added flat)
+    auto run = [&](auto a, auto src) {
+      if (bias->w == 1) return launch_split(name, a, src, ep, ka, N, K, out_floats, OHW, ka);
+      return launch(name, a, src, ep, ka, N, K, 1);
+    };
     if (BK % taps == 0 && (uint32_t)kz % (BK / taps) == 0) {  // taps tile the k step: offsets precomputed per thread
       SrcIm2colFixed bf{};
       bf.p = b.p; bf.in_w = b.in_w; bf.C = b.C; bf.H = b.H; bf.W = b.W; bf.KY = b.KY; bf.KX = b.KX; bf.OHW = b.OHW; bf.OW = b.OW; bf.R = b.R; bf.K = b.K;
       bf.sy = sy; bf.sx = sx; bf.py = py; bf.px = px;
-      rc = with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return launch(name, a, bf, ep, ka, out->w * OHW, K, 1); });
+      rc = with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return run(a, bf); });
+    } else if ((uint32_t)kz % BK == 0 && ka >= 16) {
+      // k ordered tap-major, 16 channels of one tap per k step; the weights are re-ordered to match (one small launch)
+      float *packed = nullptr;
+      if ((rc = workspace((size_t)ka * K, &packed))) return rc;
+      {
+        mt::ProfileScope prof("conv_pack_tap_major");
+        unsigned gx = cdiv((size_t)ka * K, 256 * 4);
+        conv_pack_tap_major_kernel<<<gx > 2048 ? 2048 : gx, 256, 0, mt::stream()>>>(packed, kernel->p, kernel->x, ka, (uint32_t)kz, taps);
+        MT_LAUNCH_CHECK("conv_pack_tap_major");
+      }
+      SrcIm2colTap bt{};
+      bt.p = b.p; bt.in_w = b.in_w; bt.C = b.C; bt.H = b.H; bt.W = b.W; bt.KY = b.KY; bt.KX = b.KX; bt.OHW = b.OHW; bt.OW = b.OW; bt.R = b.R; bt.K = b.K;
+      bt.sy = sy; bt.sx = sx; bt.py = py; bt.px = px;
+      rc = with_row_k(packed, K, ka, K, Batch{}, [&](auto a) { return run(a, bt); });
     } else {
-      rc = with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return launch(name, a, b, ep, ka, out->w * OHW, K, 1); });
+      rc = with_row_k(kernel->p, kernel->x, ka, K, Batch{}, [&](auto a) { return run(a, b); });
     }
   } else {
     // kernels differ per sample: one product per output image

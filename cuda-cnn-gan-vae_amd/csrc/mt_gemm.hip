@@ -34,22 +34,9 @@ SrcColK col_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, uint32_t inne
   return s;
 }
 
-// ---- split-K: products with few output tiles and a long k axis -----------------------------------------------------
-// A product of M x N < 128 tiles would leave most compute units idle while a few blocks walk the whole k axis
-// (a Linear layer with few outputs: 8192 -> 1 for a batch of 128 is two blocks of 512 steps).  The k axis is cut into
-// S ranges, each range is an ordinary product into its own partial result in the library's workspace, and one
-// elementwise kernel adds the S partials in a fixed order, then bias and activation.
+// ---- split-K support (see launch_split in mt_igemm.h): workspace for the partial results and the kernel that adds them
 float *g_split_ws = nullptr;
 size_t g_split_floats = 0;
-int split_workspace(size_t floats, float **p) {
-  if (floats > g_split_floats) {
-    if (g_split_ws) { MT_HIP(hipStreamSynchronize(mt::stream())); MT_HIP(hipFree(g_split_ws)); g_split_ws = nullptr; g_split_floats = 0; }
-    MT_HIP(hipMalloc((void **)&g_split_ws, (floats + floats / 4 + 1024) * sizeof(float)));
-    g_split_floats = floats + floats / 4 + 1024;
-  }
-  *p = g_split_ws;
-  return MT_OK;
-}
 
 // out[i] = func(sum_s partial[s][i] + bias[(i / bias_div) % bias_mod])
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *out, const float *partial, uint32_t S, size_t n, const float *bias, uint32_t bias_div,
@@ -60,32 +47,6 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *out, const fl
   for (uint32_t s = 0; s < S; s++) acc += partial[(size_t)s * n + i];
   if (bias) acc += bias[(i / bias_div) % bias_mod];
   out[i] = mt::apply_func(func, acc);
-}
-
-// One product, split over k when that fills the machine better.  `out` / `out_floats`: the contiguous output the
-// epilogue addresses from ep.C; bias is given as (pointer, divisor, modulus) over the flat output index.
-template <class SrcA, class SrcB>
-int launch_one(const char *name, SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, size_t out_floats, uint32_t bias_div, uint32_t bias_mod) {
-  const size_t tiles = (size_t)cdiv(M, 64) * cdiv(N, 64);
-  if (tiles >= 128 || K < 512 || out_floats > (1u << 22)) return launch(name, a, b, ep, M, N, K, 1);
-  uint32_t want = (uint32_t)(512 / tiles);                       // ranges wanted
-  uint32_t kc = (cdiv(K, want) + BK - 1) / BK * BK;              // range length, a multiple of the k step
-  if (kc < 2 * BK) kc = 2 * BK;
-  const uint32_t S = cdiv(K, kc);
-  if (S < 2) return launch(name, a, b, ep, M, N, K, 1);
-  float *partial = nullptr;
-  int rc = split_workspace((size_t)S * out_floats, &partial);
-  if (rc) return rc;
-  float *out = ep.C;
-  const float *bias = ep.bias;
-  const int func = ep.func;
-  a.ksplit = kc; b.ksplit = kc;
-  ep.C = partial; ep.bias = nullptr; ep.func = MT_F_NONE;
-  ep.bt.wmod = S; ep.bt.zcount = 1; ep.bt.stride = out_floats;
-  if ((rc = launch(name, a, b, ep, M, N, kc, S))) return rc;
-  splitk_reduce_kernel<<<cdiv(out_floats, 256), 256, 0, mt::stream()>>>(out, partial, S, out_floats, bias, bias_div, bias_mod, func);
-  MT_LAUNCH_CHECK(name);
-  return MT_OK;
 }
 
 // C[w,z] = op(A[w%Wa,z]) * B[w%Wb,z];  op = transpose when `ta` (A stored [K][M]).
@@ -113,8 +74,8 @@ int product(const char *name, const mt_tensor *out, const mt_tensor *left, const
       if (bias) { ep.bias = bias; ep.bias_mode = 2; }
       // bias per output row m = flat index % M
       return with_row_k(right->p, K, W, K, none, [&](auto a) {
-        if (ta) return launch_one(name, a, col_k(left->p, M, M, K, M, 0), ep, W, M, K, (size_t)W * M, 1, M);
-        return with_row_k(left->p, K, M, K, none, [&](auto b) { return launch_one(name, a, b, ep, W, M, K, (size_t)W * M, 1, M); });
+        if (ta) return launch_split(name, a, col_k(left->p, M, M, K, M, 0), ep, W, M, K, (size_t)W * M, 1, M);
+        return with_row_k(left->p, K, M, K, none, [&](auto b) { return launch_split(name, a, b, ep, W, M, K, (size_t)W * M, 1, M); });
       });
     }
     // one product with N' = W*N columns; column n' = (w, n)
@@ -122,14 +83,14 @@ int product(const char *name, const mt_tensor *out, const mt_tensor *left, const
     if (bias) { ep.bias = bias; ep.bias_mode = 1; }
     // output [w][m][n]: bias per row m = (flat index / N) % M
     SrcColK b = col_k(right->p, N, W * N, K, N, (size_t)K * N);
-    if (ta) return launch_one(name, col_k(left->p, M, M, K, M, 0), b, ep, M, W * N, K, (size_t)W * M * N, N, M);
-    return with_row_k(left->p, K, M, K, none, [&](auto a) { return launch_one(name, a, b, ep, M, W * N, K, (size_t)W * M * N, N, M); });
+    if (ta) return launch_split(name, col_k(left->p, M, M, K, M, 0), b, ep, M, W * N, K, (size_t)W * M * N, N, M);
+    return with_row_k(left->p, K, M, K, none, [&](auto a) { return launch_split(name, a, b, ep, M, W * N, K, (size_t)W * M * N, N, M); });
   }
   if (fold_ok && right->w == 1 && left->w >= W && !ta && !bias) {
     // rows (w, m) of A and of C are contiguous: one product with M' = W*M rows
     ep.row_stride = N; ep.inner = N; ep.g_stride = 0;
     SrcColK b = col_k(right->p, N, N, K, N, 0);
-    return with_row_k(left->p, K, W * M, K, none, [&](auto a) { return launch_one(name, a, b, ep, W * M, N, K, (size_t)W * M * N, 1, 1); });
+    return with_row_k(left->p, K, W * M, K, none, [&](auto a) { return launch_split(name, a, b, ep, W * M, N, K, (size_t)W * M * N, 1, 1); });
   }
 
   // general case: one product per (w, z)
@@ -149,6 +110,23 @@ int product(const char *name, const mt_tensor *out, const mt_tensor *left, const
 }
 
 }  // namespace
+
+namespace mt {
+int split_workspace(size_t floats, float **p) {
+  if (floats > g_split_floats) {
+    if (g_split_ws) { MT_HIP(hipStreamSynchronize(stream())); MT_HIP(hipFree(g_split_ws)); g_split_ws = nullptr; g_split_floats = 0; }
+    MT_HIP(hipMalloc((void **)&g_split_ws, (floats + floats / 4 + 1024) * sizeof(float)));
+    g_split_floats = floats + floats / 4 + 1024;
+  }
+  *p = g_split_ws;
+  return MT_OK;
+}
+int split_reduce(const char *name, float *out, const float *partial, uint32_t S, size_t n, const float *bias, uint32_t bias_div, uint32_t bias_mod, int func) {
+  splitk_reduce_kernel<<<cdiv(n, 256), 256, 0, stream()>>>(out, partial, S, n, bias, bias_div, bias_mod, func);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+}  // namespace mt
 
 extern "C" {
 

@@ -44,7 +44,7 @@ struct Batch {
 // Operands must be smaller than 2 GiB (checked on the host); OOB plus any in-range offset stays out of range.
 //
 // Protocol:  bind(row) once per thread;  seek<E>(k) position at the thread's first k;  fetch<E>(v) load E
-// consecutive k;  next() advance by BK.
+// consecutive k;  next<E>() advance by BK.
 constexpr uint32_t OOB = 0x80000000u;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
@@ -96,6 +96,7 @@ struct SrcRowK {
     ktile = 0; kseg = 0; segjump = 0;
     if (voff != OOB) voff += k0 * 4u;
   }
+  template <int E>
   __device__ void next() {
     ktile += BK;
     if (seg) {
@@ -151,6 +152,7 @@ struct SrcColK {
   }
   template <int E>
   __device__ void seek(uint32_t k0) { k = k0; }
+  template <int E>
   __device__ void next() { k += BK; }
   template <int E>
   __device__ void fetch(float (&v)[E]) const {
@@ -169,12 +171,20 @@ struct SrcIm2col {
   uint32_t in_w, C, H, W, KY, KX, OHW, OW, R, K;
   int32_t sy, sx, py, px;
   Batch bt;  // per-image batching (kernels that differ per sample): stride = C*H*W, wmod = in_w
+  uint32_t ksplit = 0, kbase = 0;  // ksplit > 0: batch entry bz covers k in [bz*ksplit, (bz+1)*ksplit) (split-K)
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t imgoff;  // byte offset of the row's image, OOB for rows outside the operand
   int32_t iy0, ix0;
   uint32_t k, c, ky, kx;
   uint32_t step_c, step_ky, step_kx;  // BK = step_c*KY*KX + step_ky*KX + step_kx
-  __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
+  __device__ void batch(uint32_t bz) {
+    if (ksplit) {
+      kbase = bz * ksplit;
+      if (K > kbase + ksplit) K = kbase + ksplit;
+    } else {
+      p += bt.offset(bz);
+    }
+  }
   __device__ void bind(uint32_t row) {
     rsrc = make_rsrc(p, in_w * C * H * W * 4u);
     uint32_t r = row < R ? row : 0;
@@ -186,6 +196,7 @@ struct SrcIm2col {
   template <int E>
   __device__ void seek(uint32_t k0) {
     uint32_t taps = KY * KX;
+    k0 += kbase;
     k = k0; c = k0 / taps;
     uint32_t rem = k0 % taps;
     ky = rem / KX; kx = rem % KX;
@@ -193,6 +204,7 @@ struct SrcIm2col {
     rem = BK % taps;
     step_ky = rem / KX; step_kx = rem % KX;
   }
+  template <int E>
   __device__ void next() {
     k += BK;
     kx += step_kx;
@@ -227,9 +239,17 @@ struct SrcIm2colFixed {
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t imgoff;
   int32_t iy0, ix0;
+  uint32_t ksplit = 0;  // > 0: batch entry bz covers k in [bz*ksplit, (bz+1)*ksplit), ksplit a multiple of BK (split-K)
   uint32_t voff[8];
-  uint32_t soff, sstep;
-  __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
+  uint32_t soff, sstep, kpos, kend, kbase = 0;
+  __device__ void batch(uint32_t bz) {
+    if (ksplit) kbase = bz * ksplit;
+    else p += bt.offset(bz);
+  }
+  __device__ void range() {  // [kpos, kend): this batch entry's part of the k axis
+    kpos = kbase;
+    kend = ksplit && K > kbase + ksplit ? kbase + ksplit : K;
+  }
   __device__ void bind(uint32_t row) {
     rsrc = make_rsrc(p, in_w * C * H * W * 4u);
     uint32_t r = row < R ? row : 0;
@@ -250,14 +270,85 @@ struct SrcIm2colFixed {
       bool ok = imgoff != OOB && (uint32_t)iy < H && (uint32_t)ix < W;
       voff[i] = ok ? imgoff + ((cc * H + (uint32_t)iy) * W + (uint32_t)ix) * 4u : OOB;
     }
-    soff = 0;
+    range();
     sstep = (BK / taps) * H * W * 4u;
+    soff = (kpos / BK) * sstep;
   }
-  __device__ void next() { soff += sstep; }
+  template <int E>
+  __device__ void next() { soff += sstep; kpos += BK; }
   template <int E>
   __device__ void fetch(float (&v)[E]) const {
+    const uint32_t so = kpos < kend ? soff : OOB;  // beyond this range of k: out of range for every lane (uniform select)
 #pragma unroll
-    for (int i = 0; i < E; i++) v[i] = buf_load(rsrc, voff[i], soff);
+    for (int i = 0; i < E; i++) v[i] = buf_load(rsrc, voff[i], so);
+  }
+};
+
+// The same view with k ordered tap-major, k = (ky*KX + kx)*C + c, for kernels whose taps do not tile the k step (3x3,
+// 5x5): C is a multiple of BK, so a tile holds 16 consecutive channels of ONE tap.  A thread's E elements are E
+// channels of the same input pixel: their byte offsets (or OOB) are recomputed only when the tap changes, every C/BK
+// tiles; in between only the scalar channel offset moves.  The weight matrix must be packed in the same k order.
+struct SrcIm2colTap {
+  static constexpr bool K_CONTIG = false;
+  const float *p;
+  uint32_t in_w, C, H, W, KY, KX, OHW, OW, R, K;
+  int32_t sy, sx, py, px;
+  Batch bt;
+  uint32_t ksplit = 0;  // > 0: batch entry bz covers k in [bz*ksplit, (bz+1)*ksplit), ksplit a multiple of BK (split-K)
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t imgoff, kthread;
+  int32_t iy0, ix0;
+  uint32_t voff[8];
+  uint32_t ky, kx, ctile, tiles_per_tap, kpos, kend, kbase = 0;
+  __device__ void batch(uint32_t bz) {
+    if (ksplit) kbase = bz * ksplit;
+    else p += bt.offset(bz);
+  }
+  __device__ void range() {  // [kpos, kend): this batch entry's part of the k axis
+    kpos = kbase;
+    kend = ksplit && K > kbase + ksplit ? kbase + ksplit : K;
+  }
+  __device__ void bind(uint32_t row) {
+    rsrc = make_rsrc(p, in_w * C * H * W * 4u);
+    uint32_t r = row < R ? row : 0;
+    uint32_t b = r / OHW, q = r % OHW, oy = q / OW, ox = q % OW;
+    imgoff = row < R ? (b % in_w) * C * H * W * 4u : OOB;
+    iy0 = (int32_t)oy * sy - py;
+    ix0 = (int32_t)ox * sx - px;
+  }
+  template <int E>
+  __device__ void retap() {
+    const int32_t iy = iy0 + (int32_t)ky, ix = ix0 + (int32_t)kx;
+    const bool ok = imgoff != OOB && ky < KY && (uint32_t)iy < H && (uint32_t)ix < W;
+    const uint32_t base = imgoff + ((kthread * H + (uint32_t)iy) * W + (uint32_t)ix) * 4u;
+#pragma unroll
+    for (int i = 0; i < E; i++) voff[i] = ok ? base + (uint32_t)i * H * W * 4u : OOB;
+  }
+  template <int E>
+  __device__ void seek(uint32_t k0) {  // k0 < BK: the thread's first channel within a tile
+    static_assert(E <= 8, "at most eight elements per thread");
+    kthread = k0;
+    range();
+    tiles_per_tap = C / BK;
+    const uint32_t tile = kpos / BK, t = tile / tiles_per_tap;
+    ctile = tile % tiles_per_tap;
+    ky = t / KX; kx = t % KX;
+    retap<E>();
+  }
+  template <int E>
+  __device__ void next() {
+    kpos += BK;
+    if (++ctile == tiles_per_tap) {  // uniform: next tap
+      ctile = 0;
+      if (++kx == KX) { kx = 0; ++ky; }
+      retap<E>();
+    }
+  }
+  template <int E>
+  __device__ void fetch(float (&v)[E]) const {
+    const uint32_t so = kpos < kend ? ctile * BK * H * W * 4u : OOB;
+#pragma unroll
+    for (int i = 0; i < E; i++) v[i] = buf_load(rsrc, voff[i], so);
   }
 };
 
@@ -290,6 +381,7 @@ struct SrcWgradImage {
     step_y = BK / OW; step_x = BK % OW;
     if (OH) { step_y %= OH; }  // a tile may be longer than a whole image of very few pixels
   }
+  template <int E>
   __device__ void next() {
     k += BK;
     ox += step_x;
@@ -479,7 +571,7 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
   auto load_tile = [&](int set, bool advance) {
     // the same issue order everywhere (A, then B), so that the wait before an LDS write names exactly the loads
     // it needs and leaves the younger ones in flight
-    if (advance) { a.next(); b.next(); }
+    if (advance) { a.template next<EA>(); b.template next<EB>(); }
     __builtin_amdgcn_sched_barrier(0);
     a.template fetch<EA>(ra[set]);
     __builtin_amdgcn_sched_barrier(0);
@@ -656,6 +748,35 @@ int launch(const char *name, SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N
   }
   MT_LAUNCH_CHECK(name);
   return MT_OK;
+}
+
+// ---- split-K: one product with few output tiles and a long k axis ------------------------------------------------
+// A product of fewer than 128 output tiles would leave most compute units idle while a few blocks walk the whole k
+// axis (a Linear layer 8192 -> 1 for a batch of 128 is two blocks of 512 steps; a 3x3 convolution of 512 channels on
+// 6x8 pixels is 96 blocks of 288 steps).  The k axis is cut into S ranges, each range is an ordinary product into its
+// own partial result in the library's workspace, and one elementwise kernel adds the S partials in a fixed order,
+// then bias and activation.  `out_floats`: the contiguous output the epilogue addresses from ep.C; the bias is given
+// as (divisor, modulus) over the flat output index.  Sources must understand `ksplit`.
+template <class SrcA, class SrcB>
+int launch_split(const char *name, SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, size_t out_floats, uint32_t bias_div, uint32_t bias_mod) {
+  const size_t tiles = (size_t)cdiv(M, 64) * cdiv(N, 64);
+  if (tiles >= 128 || K < 512 || out_floats > (1u << 22) || ep.accumulate) return launch(name, a, b, ep, M, N, K, 1);
+  uint32_t want = (uint32_t)(512 / tiles);                       // ranges wanted
+  uint32_t kc = (cdiv(K, want) + BK - 1) / BK * BK;              // range length, a multiple of the k step
+  if (kc < 2 * BK) kc = 2 * BK;
+  const uint32_t S = cdiv(K, kc);
+  if (S < 2) return launch(name, a, b, ep, M, N, K, 1);
+  float *partial = nullptr;
+  int rc = split_workspace((size_t)S * out_floats, &partial);
+  if (rc) return rc;
+  float *out = ep.C;
+  const float *bias = ep.bias;
+  const int func = ep.func;
+  a.ksplit = kc; b.ksplit = kc;
+  ep.C = partial; ep.bias = nullptr; ep.func = MT_F_NONE;
+  ep.bt.wmod = S; ep.bt.zcount = 1; ep.bt.stride = out_floats;
+  if ((rc = launch(name, a, b, ep, M, N, kc, S))) return rc;
+  return split_reduce(name, out, partial, S, out_floats, bias, bias_div, bias_mod, func);
 }
 
 // ---- all stride phases of a transposed convolution in one launch -------------------------------------------------

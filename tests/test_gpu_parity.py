@@ -168,6 +168,12 @@ CONV_CASES = [
     (3, 40, 12, 12, 130, 4, 4, 2, 2, 1, 1, 1, 1),   # more than one 128-row tile
     (2, 8, 20, 20, 16, 5, 5, 5, 5, 0, 0, 1, 1),     # stride above 4: transposed conv takes the direct kernel
     (2, 3, 6, 6, 2, 1, 1, 2, 2, 0, 0, 1, 1),        # 1x1 kernel, stride 2: stride phases without taps
+    (3, 16, 9, 10, 20, 3, 3, 1, 1, 1, 1, 1, 1),     # 3x3 with a multiple of 16 channels: tap-major k order
+    (2, 32, 11, 9, 70, 5, 5, 2, 2, 2, 2, 1, 1),     # 5x5 stride 2, tap-major
+    (2, 64, 6, 8, 40, 3, 3, 1, 1, 1, 1, 1, 1),      # few output tiles, k = 576: tap-major, split over k
+    (2, 64, 8, 8, 24, 4, 4, 2, 2, 1, 1, 1, 1),      # taps tile the k step, k = 1024, 32 columns: split over k
+    (2, 60, 6, 6, 8, 3, 3, 1, 1, 1, 1, 1, 1),       # k = 540 in channel-major order, split over k
+    (2, 48, 6, 6, 8, 3, 3, 1, 1, 1, 1, 1, 2),       # one bias set per sample: not split
 ]
 
 
