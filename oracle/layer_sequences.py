@@ -192,3 +192,44 @@ def gan_generator_forward(lib, params, noise, channels=(512, 512, 256, 128, 64, 
         outs["c%d" % i], outs["h%d" % (i + 1)] = c, h
     outs["image"] = function_forward(lib, conv_forward(lib, h, params["kernel6"], params["bias6"], 3, 1, 1), "tangence")
     return outs
+
+
+VAE_ENCODER = (3, 32, 64, 128, 256)
+VAE_DECODER = (256, 128, 64, 32, 3)
+
+
+def vae_encoder_forward(lib, params, x):
+    """VAE encoder of configuration 4: conv 3x3 stride 2 padding 1, 3 -> 32 -> 64 -> 128 -> 256, each followed by
+    BatchNorm (training mode) and leaky ReLU; two Linear heads to the mean and the log-variance of the latent
+    (netlayer/cnetlayervaecoderoutput.cu.h consumes them).  Parameter names: ekernel0..3, ebias0..3, egamma0..3,
+    ebeta0..3, mu_w, mu_b, lv_w, lv_b."""
+    outs, h = {}, x
+    for i in range(4):
+        c = conv_forward(lib, h, params["ekernel%d" % i], params["ebias%d" % i], 3, 2, 1)
+        bn = batchnorm_forward_train(lib, c, params["egamma%d" % i], params["ebeta%d" % i])["out"]
+        h = function_forward(lib, bn, "leaky_relu")
+        outs["ec%d" % i], outs["eh%d" % i] = c, h
+    outs["mu"] = linear_forward(lib, params["mu_w"], h, params["mu_b"])
+    outs["logvar"] = linear_forward(lib, params["lv_w"], h, params["lv_b"])
+    return outs
+
+
+def vae_reparameterize(mu, logvar, eps):
+    """z = mu + exp(clamp(logvar, -10, 10) / 2) * eps (netlayer/cnetlayervaecoderoutput.cu.h:266-274), on the host:
+    the same numbers feed both back ends."""
+    return (mu + np.exp(np.clip(logvar, -10.0, 10.0) * 0.5) * eps).astype(np.float32)
+
+
+def vae_decoder_forward(lib, params, z, size=8):
+    """VAE decoder: Linear latent -> 256*size*size, leaky ReLU, viewed [B,256,size,size]; transposed conv 4x4 stride 2
+    padding 1, 256 -> 128 -> 64 -> 32 -> 3 with leaky ReLU between, sigmoid at the end.  Parameter names: dec_w, dec_b,
+    dkernel0..3, dbias0..3."""
+    b = z.shape[0]
+    h = function_forward(lib, linear_forward(lib, params["dec_w"], z, params["dec_b"]), "leaky_relu")
+    h = np.ascontiguousarray(h).reshape(b, VAE_DECODER[0], size, size)
+    outs = {"dh0": h}
+    for i in range(4):
+        h = backconv_forward(lib, h, params["dkernel%d" % i], params["dbias%d" % i], 4, 2, 1, VAE_DECODER[i + 1])
+        h = function_forward(lib, h, "leaky_relu" if i < 3 else "sigmoid")
+        outs["dh%d" % (i + 1)] = h
+    return outs

@@ -208,3 +208,74 @@ def test_shipped_gan_generator_topology(gpu, oracle):
     # end to end: the whole stack on the device, seven layers of accumulated rounding
     got = seq.gan_generator_forward(gpu, params, noise, channels)
     assert got["image"].shape == (b, 3, 192, 256) and rel_err(got["image"], want["image"]) <= 2e-3
+
+
+def vae_parameters(latent=128, seed=4):
+    rng = np.random.default_rng(seed)
+    p, size = {}, 128
+    for i in range(4):
+        cin, cout = seq.VAE_ENCODER[i], seq.VAE_ENCODER[i + 1]
+        size //= 2
+        p["ekernel%d" % i] = (rng.standard_normal((1, 1, cout, cin * 9)) * np.sqrt(2.0 / (cin * 9))).astype(np.float32)
+        p["ebias%d" % i] = (rng.standard_normal((1, cout, 1, 1)) * 0.05).astype(np.float32)
+        p["egamma%d" % i] = rng.uniform(0.5, 1.5, (1, cout, size, size)).astype(np.float32)
+        p["ebeta%d" % i] = rng.uniform(-0.2, 0.2, (1, cout, size, size)).astype(np.float32)
+    flat = 256 * 8 * 8
+    for head in ("mu", "lv"):
+        p[head + "_w"] = (rng.standard_normal((1, 1, latent, flat)) / np.sqrt(flat)).astype(np.float32)
+        p[head + "_b"] = np.full((1, 1, latent, 1), 0.1, np.float32)
+    p["dec_w"] = (rng.standard_normal((1, 1, flat, latent)) / np.sqrt(latent)).astype(np.float32)
+    p["dec_b"] = np.full((1, 1, flat, 1), 0.1, np.float32)
+    for i in range(4):
+        cin, cout = seq.VAE_DECODER[i], seq.VAE_DECODER[i + 1]
+        p["dkernel%d" % i] = (rng.standard_normal((1, 1, cin, cout * 16)) * np.sqrt(1.0 / (cin * 4))).astype(np.float32)
+        p["dbias%d" % i] = np.zeros((1, cin, 1, 1), np.float32)
+    return p
+
+
+def test_config4_vae_against_oracle(gpu, oracle):
+    """VAE of configuration 4 at batch 4: encoder (conv 3x3 s2 p1 + BatchNorm + leaky ReLU x4, two Linear heads 16384 ->
+    128), reparameterisation on the host, decoder (Linear 128 -> 16384, transposed conv 4x4 s2 p1 x4, sigmoid)."""
+    params = vae_parameters()
+    x = U(40, 4, 3, 128, 128, lo=0.0, hi=1.0)
+    want = seq.vae_encoder_forward(oracle, params, x)
+    # layer by layer on the oracle's inputs (batch norms over four samples amplify rounding between layers)
+    h = x
+    for i in range(4):
+        c = seq.conv_forward(gpu, h, params["ekernel%d" % i], params["ebias%d" % i], 3, 2, 1)
+        assert rel_err(c, want["ec%d" % i]) <= REL, "encoder conv %d" % i
+        a = gpu.batchnorm_train(want["ec%d" % i], params["egamma%d" % i], params["ebeta%d" % i], func="leaky_relu")["out"]
+        assert rel_err(a, want["eh%d" % i]) <= REL, "encoder batch norm %d" % i
+        h = want["eh%d" % i]
+    for head, key in (("mu", "mu"), ("lv", "logvar")):   # 16384 -> 128 at batch 4: split over k
+        assert rel_err(gpu.linear_forward(params[head + "_w"], h, params[head + "_b"]), want[key]) <= REL, key
+    z = seq.vae_reparameterize(want["mu"], want["logvar"], Nrm(41, *want["mu"].shape))
+    dwant = seq.vae_decoder_forward(oracle, params, z)
+    dgot = seq.vae_decoder_forward(gpu, params, z)
+    for name in dwant:
+        assert rel_err(dgot[name], dwant[name]) <= REL, name
+    assert dgot["dh4"].shape == (4, 3, 128, 128) and np.all((dgot["dh4"] > 0) & (dgot["dh4"] < 1))
+    # the encoder end to end on the device
+    got = seq.vae_encoder_forward(gpu, params, x)
+    assert rel_err(got["mu"], want["mu"]) <= 2e-3 and rel_err(got["logvar"], want["logvar"]) <= 2e-3
+
+
+def test_config4_full_batch_properties(gpu, oracle):
+    """Batch 64: convolutions and transposed convolutions are independent per sample, so one sample of the full batch
+    equals that sample alone through the oracle; the Linear heads likewise."""
+    params = vae_parameters()
+    x = U(42, 64, 3, 128, 128, lo=0.0, hi=1.0)
+    h = x
+    for i, sample in ((0, 63), (1, 7)):
+        c = seq.conv_forward(gpu, h, params["ekernel%d" % i], params["ebias%d" % i], 3, 2, 1)
+        one = seq.conv_forward(oracle, h[sample:sample + 1], params["ekernel%d" % i], params["ebias%d" % i], 3, 2, 1)
+        assert rel_err(c[sample:sample + 1], one) <= REL, "encoder conv %d" % i
+        h = gpu.batchnorm_train(c, params["egamma%d" % i], params["ebeta%d" % i], func="leaky_relu")["out"]
+        x64 = c.astype(np.float64)
+        exact = params["egamma%d" % i] * (x64 - x64.mean(0)) / np.sqrt(x64.var(0) + seq.BN_EPSILON) + params["ebeta%d" % i]
+        assert rel_err(h, np.where(exact > 0, exact, 0.1 * exact)) <= REL, "batch norm %d" % i
+    z = Nrm(43, 64, 1, 128, 1)
+    d = seq.vae_decoder_forward(gpu, params, z)
+    one = seq.vae_decoder_forward(oracle, params, z[20:21])
+    for name in one:
+        assert rel_err(d[name][20:21], one[name]) <= REL, name
