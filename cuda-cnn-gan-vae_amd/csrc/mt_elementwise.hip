@@ -524,6 +524,35 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
   }
 }
 
+// VAE coder output (netlayer/cnetlayervaecoderoutput.cu.h:252-286, a host loop there): out = mu + exp(clamp(lv)/2)*eps
+// and per block the partial sum of 1 + lv - mu^2 - exp(lv); vae_kl_kernel adds the partials in block order.
+__global__ __launch_bounds__(EW_THREADS) void vae_coder_kernel(float *out, float *partial, const float *mu, const float *logvar, const float *eps, size_t n) {
+  __shared__ float red[EW_THREADS / 64];
+  float s = 0.f;
+  for (size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += (size_t)gridDim.x * EW_THREADS) {
+    float m = mu[i], lv = logvar[i];
+    if (lv > 10.f) lv = 10.f;
+    if (lv < -10.f) lv = -10.f;
+    const float e = (float)exp((double)lv / 2.0);
+    out[i] = m + e * eps[i];
+    s += 1.f + lv - m * m - expf(lv);
+  }
+  s = mt::wave_sum(s);
+  if (threadIdx.x % 64 == 0) red[threadIdx.x / 64] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.f;
+    for (int i = 0; i < EW_THREADS / 64; i++) t += red[i];
+    partial[blockIdx.x] = t;
+  }
+}
+__global__ void vae_kl_kernel(float *kl, const float *partial, uint32_t blocks, float batch) {
+  float t = 0.f;
+  for (uint32_t i = 0; i < blocks; i++) t += partial[i];
+  t = (float)((double)t * -0.5);
+  kl[0] = t / batch;
+}
+
 __global__ __launch_bounds__(EW_THREADS) void bn_ivar_kernel(float *ivar, const float *var, uint32_t S, float eps) {
   uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
   if (i < S) ivar[i] = (float)(1.0 / (double)sqrtf(var[i] + eps));
@@ -826,6 +855,29 @@ int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const
 #undef MT_BN_BWD_NW
 #undef MT_BN_BWD
   MT_LAUNCH_CHECK("mt_batchnorm_backward");
+  return MT_OK;
+}
+
+int mt_vae_coder_output(const mt_tensor *out, const mt_tensor *kl_loss, const mt_tensor *mu, const mt_tensor *logvar, const mt_tensor *epsilon) {
+  const mt_tensor *need[4] = {out, mu, logvar, epsilon};
+  for (auto t : need)
+    if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_vae_coder_output: null tensor");
+  for (auto t : {mu, logvar, epsilon})
+    if (!mt::same_zyx(t, out) || t->w != out->w) return mt::fail(MT_E_SHAPE, "mt_vae_coder_output: sizes do not match");
+  if (kl_loss && (mt::bad(kl_loss) || mt::count(kl_loss) < 1)) return mt::fail(MT_E_ARGUMENT, "mt_vae_coder_output: kl_loss must hold one value");
+  const size_t n = mt::count(out);
+  if (n == 0) return MT_OK;
+  unsigned blocks = cdiv(n, (size_t)EW_THREADS * 4);
+  if (blocks > 1024) blocks = 1024;
+  float *partial = nullptr;
+  int rc = bn_scratch(blocks, &partial);
+  if (rc) return rc;
+  vae_coder_kernel<<<blocks, EW_THREADS, 0, mt::stream()>>>(out->p, partial, mu->p, logvar->p, epsilon->p, n);
+  MT_LAUNCH_CHECK("mt_vae_coder_output");
+  if (kl_loss) {
+    vae_kl_kernel<<<1, 1, 0, mt::stream()>>>(kl_loss->p, partial, blocks, (float)out->w);
+    MT_LAUNCH_CHECK("mt_vae_coder_output");
+  }
   return MT_OK;
 }
 

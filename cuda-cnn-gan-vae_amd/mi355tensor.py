@@ -342,6 +342,10 @@ class Fused:
              opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
 
     @staticmethod
+    def VaeCoderOutput(out, kl_loss, mu, logvar, epsilon):
+        call("mt_vae_coder_output", _d(out), _d(kl_loss) if kl_loss is not None else None, _d(mu), _d(logvar), _d(epsilon))
+
+    @staticmethod
     def BatchNormBackward(error, dgamma, dbeta, delta, gamma, xhat, ivar):
         opt = lambda t: _d(t) if t is not None else None
         call("mt_batchnorm_backward", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), _d(xhat), _d(ivar))

@@ -164,6 +164,12 @@ int mt_batchnorm_forward_train_func(const mt_tensor *output, const mt_tensor *in
 int mt_batchnorm_forward_infer_func(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
                                     const mt_tensor *mean, const mt_tensor *variable, float epsilon, int func);
 
+/* CNetLayerVAECoderOutput::Forward, netlayer/cnetlayervaecoderoutput.cu.h:244-287 (a host loop over GetElement there),
+ * with the noise supplied by the caller instead of drawn from an unseedable generator:
+ * output = mu + exp(clamp(logvar, -10, 10) / 2) * epsilon;  kl_loss[0] = -0.5 * sum(1 + logvar - mu^2 - exp(logvar)) / W
+ * (kl_loss: device tensor of at least one value, NULL to skip). */
+int mt_vae_coder_output(const mt_tensor *output, const mt_tensor *kl_loss, const mt_tensor *mu, const mt_tensor *logvar, const mt_tensor *epsilon);
+
 /* ---- fused backward sequences ---- */
 /* CNetLayerBatchNormalization::TrainingBackward, netlayer/cnetlayerbatchnormalization.cu.h:578-604, as one kernel:
  * error [B,Z,Y,X] = ((N*dxhat - xhat*sum_w(dxhat*xhat)) - sum_w(dxhat)) * ivar * (1/N) with dxhat = delta*gamma;

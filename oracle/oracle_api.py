@@ -242,6 +242,13 @@ class Oracle:
                    C.c_double(speed), C.c_double(beta1), C.c_double(beta2), C.c_double(epsilon), C.c_double(iteration))
         return weight, m, v
 
+    # ---- VAE coder output ----------------------------------------------
+    def vae_coder_output(self, mu, logvar, epsilon):
+        mu, logvar, epsilon = _f32(mu), _f32(logvar), _f32(epsilon)
+        out, kl = np.zeros(mu.shape, np.float32), C.c_float()
+        self._call("vae_coder_output", self._p(out), C.byref(kl), self._p(mu), self._p(logvar), self._p(epsilon))
+        return out, kl.value
+
     # ---- activations --------------------------------------------------
     def apply_func(self, a, func, differential=False):
         a = _f32(a)

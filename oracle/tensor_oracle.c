@@ -505,6 +505,29 @@ int oracle_adam(ot_tensor *weight, const ot_tensor *dweight, ot_tensor *m, ot_te
   return ORACLE_OK;
 }
 
+/* netlayer/cnetlayervaecoderoutput.cu.h:252-286 with type_t = float: log_var/2.0 is a double division, exp of it a
+ * double exp rounded to float; exp(log_var) in the KL term is the float overload; the sum runs in float in
+ * w, z, y, x order; "*=-0.5" multiplies in double, "/=BatchSize" divides by the batch size converted to float. */
+int oracle_vae_coder_output(ot_tensor *out, float *kl, const ot_tensor *mu, const ot_tensor *logvar, const ot_tensor *epsilon) {
+  if (!same_zyx(out, mu) || out->w != mu->w || !same_zyx(out, logvar) || out->w != logvar->w || !same_zyx(out, epsilon) ||
+      out->w != epsilon->w)
+    return ORACLE_E_SHAPE;
+  size_t n = count(out);
+  float kl_loss = 0;
+  for (size_t i = 0; i < n; i++) {
+    float m = mu->p[i], log_var = logvar->p[i];
+    if (log_var > 10) log_var = 10;
+    if (log_var < -10) log_var = -10;
+    float e = (float)exp(log_var / 2.0);
+    out->p[i] = m + e * epsilon->p[i];
+    kl_loss += 1 + log_var - m * m - expf(log_var);
+  }
+  kl_loss = (float)(kl_loss * -0.5);
+  kl_loss /= (float)out->w;
+  if (kl) *kl = kl_loss;
+  return ORACLE_OK;
+}
+
 /* ------------------------------------------------------------------------ */
 /* cpu/ctensorapplyfunc.h:111-255.  The float/double mix follows the C++
  * overload resolution of the reference with type_t=float: math calls on a

@@ -105,6 +105,12 @@ int oracle_max_pooling_backward(ot_tensor *out, const ot_pos_tensor *pos, const 
 int oracle_adam(ot_tensor *weight, const ot_tensor *dweight, ot_tensor *m, ot_tensor *v, uint32_t batch_size,
                 double speed, double beta1, double beta2, double epsilon, double iteration);
 
+/* ---- VAE coder output (netlayer/cnetlayervaecoderoutput.cu.h:244-287) ----
+ * The layer's host loop with the noise given instead of drawn: out = mu + exp(clamp(logvar,-10,10)/2) * epsilon and
+ * *kl = -0.5 * sum(1 + logvar - mu^2 - exp(logvar)) / W (clamped logvar).  Pinned by its float64 closed form and by
+ * special cases (tests/test_oracle_math.py); the layer itself draws from an unseedable generator. */
+int oracle_vae_coder_output(ot_tensor *out, float *kl, const ot_tensor *mu, const ot_tensor *logvar, const ot_tensor *epsilon);
+
 /* ---- activations (cpu/ctensorapplyfunc.h) -------------------------------
  * func ids: 0 sigmoid, 1 ReLU, 2 GeLU, 3 LeakyReLU(0.1), 4 linear, 5 tanh;
  * add 8 for the derivative of the same function. */

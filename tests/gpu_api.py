@@ -204,6 +204,12 @@ class Gpu:
         Fused.BatchNormBackward(err, dg, db, up(delta), up(gamma), up(xhat), up(ivar))
         return err.numpy(), dg.numpy(), db.numpy()
 
+    def vae_coder_output(self, mu, logvar, epsilon):
+        mu = np.asarray(mu, np.float32)
+        out, kl = CTensor(*mu.shape), CTensor(1, 1, 1, 1)
+        Fused.VaeCoderOutput(out, kl, up(mu), up(logvar), up(epsilon))
+        return out.numpy(), float(kl.numpy().ravel()[0])
+
     def batchnorm_infer(self, x, gamma, beta, mean, var, eps=1e-6, func=None):
         x = np.asarray(x, np.float32)
         out = CTensor(*x.shape)

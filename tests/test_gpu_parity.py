@@ -456,6 +456,20 @@ def test_batchnorm_backward_fused(gpu, oracle, shape):
     close(db - db0, want_db, 1e-5)
 
 
+def test_vae_coder_output(gpu, oracle):
+    mu, logvar, eps = Nrm(1, 6, 1, 128, 1), Nrm(2, 6, 1, 128, 1) * 6, Nrm(3, 6, 1, 128, 1)   # log-variances beyond the +-10 clamp
+    want, want_kl = oracle.vae_coder_output(mu, logvar, eps)
+    got, got_kl = gpu.vae_coder_output(mu, logvar, eps)
+    close(got, want, 1e-6)
+    assert abs(got_kl - want_kl) <= 1e-5 * abs(want_kl)
+    big = (300, 2, 16, 16)
+    mu, logvar, eps = Nrm(4, *big), Nrm(5, *big), Nrm(6, *big)
+    want, want_kl = oracle.vae_coder_output(mu, logvar, eps)
+    got, got_kl = gpu.vae_coder_output(mu, logvar, eps)
+    close(got, want, 1e-6)
+    assert abs(got_kl - want_kl) <= 1e-4 * abs(want_kl)      # a float sum of 150 000 terms in another order
+
+
 def test_conv_layer_forward_backward(gpu, oracle, path):
     x, kernel, bias = U(1, 6, 3, 16, 16), Nrm(2, 1, 1, 8, 3 * 16, std=0.1), U(3, 1, 8, 1, 1) * 0.1
     want = seq.conv_forward(oracle, x, kernel, bias, 4, 2, 1)

@@ -207,3 +207,25 @@ def test_adam_closed_form(oracle):
     v64 = b2 * v + (1 - b2) * g * g
     step = lr * (m64 / (1 - b1 ** it)) / (np.sqrt(v64 / (1 - b2 ** it)) + eps)
     assert rel_err(m1, m64) < 1e-6 and rel_err(v1, v64) < 1e-6 and rel_err(w1, w - step) < 1e-6
+
+
+def test_vae_coder_output_closed_form(oracle):
+    """out = mu + exp(clamp(logvar)/2)*eps and the KL term against float64; special cases that a dropped term, a wrong
+    sign or a missing clamp would break."""
+    rng = np.random.default_rng(7)
+    mu, lv, eps = (rng.standard_normal((5, 1, 64, 1)).astype(np.float32) for _ in range(3))
+    lv *= 7                                                     # some beyond +-10
+    out, kl = oracle.vae_coder_output(mu, lv, eps)
+    c = np.clip(lv.astype(np.float64), -10, 10)
+    assert np.max(np.abs(out - (mu + np.exp(c / 2) * eps))) <= 1e-5 * np.abs(out).max()
+    exact = -0.5 * np.sum(1 + c - mu.astype(np.float64) ** 2 - np.exp(c)) / 5
+    assert abs(kl - exact) <= 1e-5 * abs(exact)
+    zero = np.zeros((3, 1, 8, 1), np.float32)
+    out, kl = oracle.vae_coder_output(zero + 0.5, zero, zero)   # no noise: the mean comes through; KL = 0.5*mu^2 per element
+    assert np.array_equal(out, zero + 0.5) and abs(kl - 0.5 * 0.25 * 8) <= 1e-6
+    out, kl = oracle.vae_coder_output(zero, zero, zero + 2)     # unit variance: the noise comes through, KL = 0
+    assert np.array_equal(out, zero + 2) and kl == 0
+    out, _ = oracle.vae_coder_output(zero, zero + 50, zero + 1)  # clamp at 10: exp(5)
+    assert np.allclose(out, np.exp(5.0), rtol=1e-6)
+    out, _ = oracle.vae_coder_output(zero, zero - 50, zero + 1)
+    assert np.allclose(out, np.exp(-5.0), rtol=1e-6)
