@@ -47,6 +47,9 @@ inline bool same_zyx(const mt_tensor *a, const mt_tensor *b) { return a->x == b-
 inline size_t count(const mt_tensor *t) { return (size_t)t->w * t->z * t->y * t->x; }
 inline bool bad(const mt_tensor *t) { return t == nullptr || (t->p == nullptr && count(t) != 0); }
 inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+// The matrix-core kernels address an operand through a 32-bit buffer descriptor, with 0x80000000 as "outside".
+inline bool fits_buffer(size_t floats) { return floats * 4 < 0x80000000ull; }
+inline bool fits_buffer(const mt_tensor *t) { return fits_buffer(count(t)); }
 
 // ---- device side ---------------------------------------------------------------------------
 // The reference's scalar functions (cpu/ctensorapplyfunc.h:111-255) with the same float/double

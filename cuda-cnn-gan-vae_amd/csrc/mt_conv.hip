@@ -588,6 +588,22 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
   ConvGeo g{out->w, image->w, kernel->w, bias->w, kz, (int32_t)image->y, (int32_t)image->x, (int32_t)ka, ky, kx, sy, sx, py, px,
             (int32_t)out->y, (int32_t)out->x, (int32_t)ka, kernel->x, kernel->z * kernel->y};
   bool direct = g_conv_path == 1;
+  const size_t image_sample = (size_t)kz * image->y * image->x;
+  if (!direct && kernel->w == 1 && !mt::fits_buffer(image)) {
+    // the folded batch is addressed through one 32-bit descriptor: run it in parts of less than 2 GiB of input
+    if (image->w == out->w && bias->w == 1 && mt::fits_buffer(image_sample)) {
+      const uint32_t part = (uint32_t)((0x80000000ull / 4 - 1) / image_sample);
+      const size_t out_sample = (size_t)ka * out->y * out->x;
+      for (uint32_t w0 = 0; w0 < out->w; w0 += part) {
+        const uint32_t n = out->w - w0 < part ? out->w - w0 : part;
+        mt_tensor o{out->p + w0 * out_sample, n, out->z, out->y, out->x}, im{image->p + w0 * image_sample, n, image->z, image->y, image->x};
+        if ((rc = forward(name, &o, &im, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func))) return rc;
+      }
+      return MT_OK;
+    }
+    direct = true;
+  }
+  if (!direct && kernel->w != 1 && !mt::fits_buffer(image_sample)) direct = true;
   if (direct) {
     size_t total = mt::count(out);
     mt::ProfileScope prof("fwd_direct");
@@ -662,6 +678,20 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   ConvGeo g{out->w, delta->w, kernel->w, bias->w, (int32_t)ka, (int32_t)delta->y, (int32_t)delta->x, (int32_t)ka, ky, kx, sy, sx, py, px,
             (int32_t)out->y, (int32_t)out->x, kz, kernel->x, kernel->z * kernel->y};
   bool direct = g_conv_path == 1 || kernel->w != 1 || sx > 4 || sy > 4 || delta->y == 0 || delta->x == 0;
+  if (!direct && !mt::fits_buffer(delta)) {
+    // the batch is addressed through one 32-bit descriptor: run it in parts of less than 2 GiB of input
+    const size_t delta_sample = (size_t)ka * delta->y * delta->x, out_sample = (size_t)kz * out->y * out->x;
+    if (delta->w == out->w && bias->w == 1 && mt::fits_buffer(delta_sample)) {
+      const uint32_t part = (uint32_t)((0x80000000ull / 4 - 1) / delta_sample);
+      for (uint32_t w0 = 0; w0 < out->w; w0 += part) {
+        const uint32_t n = out->w - w0 < part ? out->w - w0 : part;
+        mt_tensor o{out->p + w0 * out_sample, n, out->z, out->y, out->x}, d{delta->p + w0 * delta_sample, n, delta->z, delta->y, delta->x};
+        if ((rc = backward(name, &o, &d, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func))) return rc;
+      }
+      return MT_OK;
+    }
+    direct = true;
+  }
   if (direct) {
     size_t total = mt::count(out);
     mt::ProfileScope prof("tconv_direct");
@@ -740,7 +770,7 @@ int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t
   if (rc) return rc;
   if (DHW == 0) return MT_OK;
   ConvGeo g{dk->w, image->w, dk->w, db->w, kz, (int32_t)image->y, (int32_t)image->x, (int32_t)ka, ky, kx, sy, sx, py, px, 0, 0, 0, dk->x, dk->z * dk->y};
-  bool direct = g_conv_path == 1 || dk->w > 65535u;
+  bool direct = g_conv_path == 1 || dk->w > 65535u || !mt::fits_buffer((size_t)kz * image->y * image->x) || !mt::fits_buffer((size_t)ka * DHW);
   if (direct) {
     size_t total = (size_t)dk->w * ka * ncol;
     wgrad_direct_kernel<<<cdiv(total, 256), 256, 0, mt::stream()>>>(dk->p, image->p, delta->p, g, delta->w, delta->y, delta->x, total);
@@ -810,6 +840,11 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     groups = g;
   }
   if (g_wgrad_groups > 0 && B % (uint32_t)g_wgrad_groups == 0) groups = (uint32_t)g_wgrad_groups;
+  while (groups < B && (!mt::fits_buffer((size_t)(B / groups) * sample_image) || !mt::fits_buffer((size_t)(B / groups) * sample_delta))) {
+    uint32_t g = groups + 1;   // a group's samples are addressed through one descriptor: keep its span below 2 GiB
+    while (g < B && B % g) g++;
+    groups = g;
+  }
   const uint32_t per = B / groups;
   float *partial = nullptr;
   if (groups > 1) {

@@ -64,7 +64,10 @@ int product(const char *name, const mt_tensor *out, const mt_tensor *left, const
   Epilogue ep{};
   ep.C = out->p;
   ep.func = func;
-  const bool fold_ok = Z == 1 && W > 1;
+  // a folded batch is addressed through one 32-bit descriptor; otherwise every matrix has its own
+  const bool fold_ok = Z == 1 && W > 1 && mt::fits_buffer(left) && mt::fits_buffer(right);
+  if (!mt::fits_buffer((size_t)M * K) || !mt::fits_buffer((size_t)K * N))
+    return mt::fail(MT_E_UNAVAILABLE, "%s: a single matrix of 2 GiB or more is not supported", name);
   const Batch none{};
 
   if (fold_ok && left->w == 1 && right->w >= W) {

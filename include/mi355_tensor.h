@@ -53,7 +53,7 @@ enum {
   MT_E_DEPTH = 4,        /* image/delta depth does not match the kernels        (cpu/ctensorconv.h:105,221,335) */
   MT_E_SHAPE = 5,        /* "sizes do not match" of the tensor-math functions   (cpu/ctensormath.h, every head) */
   MT_E_ARGUMENT = 6,     /* null pointer, zero stride, unknown function id ...  (no counterpart: the C++ API cannot express these) */
-  MT_E_UNAVAILABLE = 7,  /* no usable gfx950 device                             */
+  MT_E_UNAVAILABLE = 7,  /* no usable gfx950 device; a single matrix of 2 GiB+   */
   MT_E_HIP = 1000        /* + hipError_t                                         (cuda/handle_error.cu.h:7-19)  */
 };
 

@@ -479,3 +479,29 @@ def test_conv_layer_forward_backward(gpu, oracle, path):
         close(got, exp)
     tk = Nrm(5, 1, 1, 8, 3 * 16, std=0.1)
     close(seq.backconv_forward(gpu, want, tk, np.zeros((1, 8, 1, 1)), 4, 2, 1, 3), seq.backconv_forward(oracle, want, tk, np.zeros((1, 8, 1, 1)), 4, 2, 1, 3))
+
+
+def test_operands_beyond_two_gib(gpu, oracle):
+    """An input tensor of 2.4 GB: the matrix-core kernels address operands through 32-bit descriptors, so the library
+    runs the batch in parts.  Samples from the first part, the seam and the last part against the oracle."""
+    from mi355tensor import CTensor, CTensorConv
+    rng = np.random.default_rng(50)
+    W, C, H = 36, 16, 1024
+    base = rng.standard_normal((1, C, H, H)).astype(np.float32)
+    scale = (1.0 + np.arange(W, dtype=np.float32) / W).reshape(W, 1, 1, 1)
+    host = base * scale                                                   # 2.4 GB, every sample different
+    assert host.nbytes > 2**31
+    x = CTensor.from_numpy(host)
+    kernel, bias = U(51, 1, 1, 2, C * 9) * 0.1, U(52, 1, 2, 1, 1)
+    out = CTensor(W, 2, H // 2, H // 2)
+    CTensorConv.ForwardConvolution(out, x, CTensor.from_numpy(kernel), 3, 3, C, 2, CTensor.from_numpy(bias), 2, 2, 1, 1)
+    got = out.numpy()
+    for w in (0, 30, 31, 32, 35):   # 32 samples of 64 MiB make 2 GiB: the seam lies at sample 31/32
+        close(got[w:w + 1], oracle.forward_convolution(host[w:w + 1], kernel, bias, 3, 3, C, 2, 2, 2, 1, 1))
+    tk = U(53, 1, 1, C, 1 * 9) * 0.1                                       # transposed conv 3x3 stride 1 to one channel
+    zero = np.zeros((1, C, 1, 1), np.float32)
+    back = CTensor(W, 1, H, H)
+    CTensorConv.BackwardConvolution(back, x, CTensor.from_numpy(tk), 3, 3, 1, C, CTensor.from_numpy(zero), 1, 1, 1, 1)
+    got = back.numpy()
+    for w in (0, 31, 32, 35):
+        close(got[w:w + 1], oracle.backward_convolution(host[w:w + 1], tk, zero, 3, 3, 1, C, 1, 1, 1, 1, (1, 1, H, H)))
