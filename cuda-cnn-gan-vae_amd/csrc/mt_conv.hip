@@ -366,57 +366,49 @@ __global__ __launch_bounds__(256) void tconv_k4s2_small_kernel(TconvArgs args) {
   }
 }
 
-// The same geometry with the input staged through LDS: a block owns a tile of 32 x 16 input pixels of one image
-// (64 x 32 output pixels) and walks the input channels in chunks of CC.  A chunk's (16+2) x (32+2) halo tile per
-// channel is fetched with 128-bit buffer loads (zero outside the image through the range check), kept in registers
-// while the previous chunk is multiplied, then written to the other LDS buffer: one barrier per chunk.  A thread
-// computes two neighbouring input pixels, i.e. 2 x 4 output pixels: per channel 6 LDS reads for 32*CO multiply-adds
-// instead of 9 global loads for 16*CO, which moves the kernel from the texture-address path to the vector ALUs.
-// Needs W % 4 == 0, C % CC == 0, 16-byte aligned rows, exactly CO output channels and the coefficients packed
-// as [ci][phase][co][taps].
-template <int CO>
-__global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
-  constexpr int TW = 32, TH = 16, CC = 8, PITCH = 36, ROWS = TH + 2;
-  constexpr int VEC = CC * ROWS * (TW / 4), NVEC = (VEC + 255) / 256;  // 128-bit pieces of a chunk, per thread
-  constexpr int EDGE = CC * ROWS * 2, NEDGE = (EDGE + 255) / 256;      // halo columns left and right
-  __shared__ __attribute__((aligned(16))) float tile[2][CC][ROWS][PITCH];  // column 0 = x0-1, 1..32 = the tile, 33 = x0+32
-  const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W, M = args.M;
-  const uint32_t tiles_x = (W + TW - 1) / TW;
-  const uint32_t x0 = (blockIdx.x % tiles_x) * TW, y0 = (blockIdx.x / tiles_x) * TH, g = blockIdx.y;
-  const uint32_t tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
-  __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta, args.in_w * C * HW * 4u);
-  const uint32_t imgoff = (g % args.in_w) * C * HW * 4u;
-
-  // byte offsets of this thread's pieces within a chunk (channel advance goes through the scalar offset)
-  uint32_t voff[NVEC], eoff[NEDGE], vdst[NVEC], edst[NEDGE];
-#pragma unroll
-  for (int i = 0; i < NVEC; i++) {
-    const uint32_t idx = tid + i * 256, row = idx / (TW / 4), seg = idx % (TW / 4), c = row / ROWS, yy = row % ROWS;
-    const int32_t iy = (int32_t)(y0 + yy) - 1;
-    const uint32_t ix = x0 + seg * 4;
-    const bool ok = idx < VEC && (uint32_t)iy < H && ix < W;
-    voff[i] = ok ? imgoff + ((c * H + (uint32_t)iy) * W + ix) * 4u : OOB;
-    vdst[i] = idx < VEC ? (c * ROWS + yy) * PITCH + 1 + seg * 4 : 0xffffffffu;
-  }
-#pragma unroll
-  for (int i = 0; i < NEDGE; i++) {
-    const uint32_t idx = tid + i * 256, row = idx / 2, side = idx % 2, c = row / ROWS, yy = row % ROWS;
-    const int32_t iy = (int32_t)(y0 + yy) - 1, ix = side ? (int32_t)(x0 + TW) : (int32_t)x0 - 1;
-    const bool ok = idx < EDGE && (uint32_t)iy < H && (uint32_t)ix < W;
-    eoff[i] = ok ? imgoff + ((c * H + (uint32_t)iy) * W + (uint32_t)ix) * 4u : OOB;
-    edst[i] = idx < EDGE ? (c * ROWS + yy) * PITCH + (side ? TW + 1 : 0) : 0xffffffffu;
-  }
+// Staging of an input tile with a one-pixel halo through registers into LDS, shared by the vector-ALU kernels below:
+// per channel (TH+2) rows of [x0-1 | x0 .. x0+TW-1 | x0+TW] (PITCH floats, the tile itself starts at column 1), CC
+// channels per chunk.  The tile columns are fetched with 128-bit buffer loads, the two halo columns with 32-bit ones;
+// everything outside the image comes back as zero through the range check.  The byte offsets of a thread's pieces are
+// computed once; the chunk advances through the scalar offset.  Needs W % 4 == 0 and 16-byte aligned rows.
+template <int TW, int TH, int CC>
+struct HaloTile {
+  static constexpr int PITCH = TW + 4, ROWS = TH + 2, FLOATS = CC * ROWS * PITCH;
+  static constexpr int VEC = CC * ROWS * (TW / 4), NVEC = (VEC + 255) / 256;
+  static constexpr int EDGE = CC * ROWS * 2, NEDGE = (EDGE + 255) / 256;
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff[NVEC], eoff[NEDGE], vdst[NVEC], edst[NEDGE], chunk_bytes;
   floatx4 rv[NVEC];
   float re[NEDGE];
-  auto fetch = [&](uint32_t chunk) {
-    const uint32_t soff = chunk * CC * HW * 4u;
+  __device__ void setup(const float *p, uint32_t bytes, uint32_t imgoff, uint32_t H, uint32_t W, uint32_t x0, uint32_t y0, uint32_t tid) {
+    rsrc = make_rsrc(p, bytes);
+    chunk_bytes = CC * H * W * 4u;
+#pragma unroll
+    for (int i = 0; i < NVEC; i++) {
+      const uint32_t idx = tid + i * 256, row = idx / (TW / 4), seg = idx % (TW / 4), c = row / ROWS, yy = row % ROWS;
+      const int32_t iy = (int32_t)(y0 + yy) - 1;
+      const uint32_t ix = x0 + seg * 4;
+      const bool ok = idx < VEC && (uint32_t)iy < H && ix < W;
+      voff[i] = ok ? imgoff + ((c * H + (uint32_t)iy) * W + ix) * 4u : OOB;
+      vdst[i] = idx < VEC ? (c * ROWS + yy) * PITCH + 1 + seg * 4 : 0xffffffffu;
+    }
+#pragma unroll
+    for (int i = 0; i < NEDGE; i++) {
+      const uint32_t idx = tid + i * 256, row = idx / 2, side = idx % 2, c = row / ROWS, yy = row % ROWS;
+      const int32_t iy = (int32_t)(y0 + yy) - 1, ix = side ? (int32_t)(x0 + TW) : (int32_t)x0 - 1;
+      const bool ok = idx < EDGE && (uint32_t)iy < H && (uint32_t)ix < W;
+      eoff[i] = ok ? imgoff + ((c * H + (uint32_t)iy) * W + (uint32_t)ix) * 4u : OOB;
+      edst[i] = idx < EDGE ? (c * ROWS + yy) * PITCH + (side ? TW + 1 : 0) : 0xffffffffu;
+    }
+  }
+  __device__ void fetch(uint32_t chunk) {
+    const uint32_t soff = chunk * chunk_bytes;
 #pragma unroll
     for (int i = 0; i < NVEC; i++) rv[i] = buf_load4(rsrc, voff[i], soff);
 #pragma unroll
     for (int i = 0; i < NEDGE; i++) re[i] = buf_load(rsrc, eoff[i], soff);
-  };
-  auto put = [&](int buf) {
-    float *t = &tile[buf][0][0][0];
+  }
+  __device__ void put(float *t) const {
 #pragma unroll
     for (int i = 0; i < NVEC; i++)
       if (vdst[i] != 0xffffffffu) {  // the tile starts at an odd column: 4 + 8 + 4 bytes
@@ -427,7 +419,30 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
 #pragma unroll
     for (int i = 0; i < NEDGE; i++)
       if (edst[i] != 0xffffffffu) t[edst[i]] = re[i];
-  };
+  }
+};
+
+// The same geometry with the input staged through LDS: a block owns a tile of 32 x 16 input pixels of one image
+// (64 x 32 output pixels) and walks the input channels in chunks of CC.  A chunk's (16+2) x (32+2) halo tile per
+// channel is fetched with 128-bit buffer loads (zero outside the image through the range check), kept in registers
+// while the previous chunk is multiplied, then written to the other LDS buffer: one barrier per chunk.  A thread
+// computes two neighbouring input pixels, i.e. 2 x 4 output pixels: per channel 6 LDS reads for 32*CO multiply-adds
+// instead of 9 global loads for 16*CO, which moves the kernel from the texture-address path to the vector ALUs.
+// Needs W % 4 == 0, C % CC == 0, 16-byte aligned rows, exactly CO output channels and the coefficients packed
+// as [ci][phase][co][taps].
+template <int CO>
+__global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
+  using Tile = HaloTile<32, 16, 8>;
+  constexpr int TW = 32, TH = 16, CC = 8, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
+  __shared__ __attribute__((aligned(16))) float tile[2][CC][ROWS][PITCH];
+  const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W, M = args.M;
+  const uint32_t tiles_x = (W + TW - 1) / TW;
+  const uint32_t x0 = (blockIdx.x % tiles_x) * TW, y0 = (blockIdx.x / tiles_x) * TH, g = blockIdx.y;
+  const uint32_t tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  Tile stage;
+  stage.setup(args.delta, args.in_w * C * HW * 4u, (g % args.in_w) * C * HW * 4u, H, W, x0, y0, tid);
+  auto fetch = [&](uint32_t chunk) { stage.fetch(chunk); };
+  auto put = [&](int buf) { stage.put(&tile[buf][0][0][0]); };
 
   float acc[2][2][2][CO];  // [pixel][py][px][co]
 #pragma unroll
@@ -493,6 +508,68 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
       float *dst = args.ep.C + ((size_t)g * M + co) * OHW + (size_t)(2 * qy + py) * OW + 2 * qx;
       *reinterpret_cast<float4 *>(dst) = o;
     }
+  }
+}
+
+// Forward convolution 3x3, stride 1, padding 1 with at most 4 output channels (an image-producing last layer) on the
+// vector ALUs, same staging: a thread computes two neighbouring output pixels for all KA channels, per input channel
+// 6 LDS reads and 18*KA multiply-adds; the 9 coefficients of (k, c) are contiguous in the kernel tensor and come
+// through the scalar cache.  Needs W % 4 == 0, C % 8 == 0, 16-byte aligned rows.
+template <int KA>
+__global__ __launch_bounds__(256) void conv3x3_tile_kernel(float *out, const float *image, const float *kernel, const float *bias, ConvGeo g, int func) {
+  using Tile = HaloTile<32, 16, 8>;
+  constexpr int TW = 32, TH = 16, CC = 8, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
+  __shared__ __attribute__((aligned(16))) float tile[2][CC][ROWS][PITCH];
+  const uint32_t H = g.H, W = g.W, C = g.C, HW = H * W;
+  const uint32_t tiles_x = (W + TW - 1) / TW;
+  const uint32_t x0 = (blockIdx.x % tiles_x) * TW, y0 = (blockIdx.x / tiles_x) * TH, w = blockIdx.y;
+  const uint32_t tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  Tile stage;
+  stage.setup(image, g.in_w * C * HW * 4u, (w % g.in_w) * C * HW * 4u, H, W, x0, y0, tid);
+  float acc[2][KA];
+#pragma unroll
+  for (int k = 0; k < KA; k++) acc[0][k] = acc[1][k] = bias[(size_t)(w % g.bias_w) * KA + k];
+  const uint32_t chunks = C / CC;
+  stage.fetch(0);
+  stage.put(&tile[0][0][0][0]);
+  __syncthreads();
+  for (uint32_t ch = 0; ch < chunks; ch++) {
+    const int cur = ch & 1;
+    if (ch + 1 < chunks) stage.fetch(ch + 1);
+#pragma unroll 2
+    for (int c = 0; c < CC; c++) {
+      const uint32_t ci = ch * CC + c;
+      float v[3][4];  // rows y-1..y+1, columns x-1..x+2 of the pixel pair (x, x+1)
+#pragma unroll
+      for (int dy = 0; dy < 3; dy++) {
+        const float *rowp = &tile[cur][c][ty + dy][2 * tx];
+        const float2 lo = *reinterpret_cast<const float2 *>(rowp), hi = *reinterpret_cast<const float2 *>(rowp + 2);
+        v[dy][0] = lo.x; v[dy][1] = lo.y; v[dy][2] = hi.x; v[dy][3] = hi.y;
+      }
+#pragma unroll
+      for (int k = 0; k < KA; k++) {
+        const float *wk = kernel + (size_t)k * g.ker_ld + ci * 9u;
+#pragma unroll
+        for (int dy = 0; dy < 3; dy++)
+#pragma unroll
+          for (int dx = 0; dx < 3; dx++) {
+            const float wv = wk[dy * 3 + dx];
+            acc[0][k] = __builtin_fmaf(wv, v[dy][dx], acc[0][k]);
+            acc[1][k] = __builtin_fmaf(wv, v[dy][dx + 1], acc[1][k]);
+          }
+      }
+    }
+    if (ch + 1 < chunks) stage.put(&tile[cur ^ 1][0][0][0]);
+    __syncthreads();
+  }
+  const uint32_t y = y0 + ty, x = x0 + 2 * tx;
+  if (y >= H || x >= W) return;  // W is even: a pair is inside or outside as a whole
+#pragma unroll
+  for (int k = 0; k < KA; k++) {
+    float2 o;
+    o.x = mt::apply_func_epilogue(func, acc[0][k]);
+    o.y = mt::apply_func_epilogue(func, acc[1][k]);
+    *reinterpret_cast<float2 *>(out + ((size_t)w * KA + k) * HW + (size_t)y * W + x) = o;
   }
 }
 
@@ -610,6 +687,17 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
     fwd_direct_kernel<<<cdiv(total, 256), 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, total);
     MT_LAUNCH_CHECK(name);
     if (func != MT_F_NONE) return mt_apply_func(out, out, func);
+    return MT_OK;
+  }
+  if (ka <= 4 && kernel->w == 1 && mt::igemm::tile_override() < 0 && kx == 3 && ky == 3 && sx == 1 && sy == 1 && px == 1 && py == 1 &&
+      image->x % 4 == 0 && kz % 8 == 0 && ((uintptr_t)image->p & 15u) == 0 && ((uintptr_t)out->p & 7u) == 0 && out->w <= 65535u) {
+    mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "vector ALU, few output channels") : name);
+    dim3 grid(cdiv(image->x, 32) * cdiv(image->y, 16), out->w);
+    if (ka == 1) conv3x3_tile_kernel<1><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);
+    else if (ka == 2) conv3x3_tile_kernel<2><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);
+    else if (ka == 3) conv3x3_tile_kernel<3><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);
+    else conv3x3_tile_kernel<4><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);
+    MT_LAUNCH_CHECK(name);
     return MT_OK;
   }
   uint32_t OHW = out->y * out->x;

@@ -174,6 +174,8 @@ CONV_CASES = [
     (2, 64, 8, 8, 24, 4, 4, 2, 2, 1, 1, 1, 1),      # taps tile the k step, k = 1024, 32 columns: split over k
     (2, 60, 6, 6, 8, 3, 3, 1, 1, 1, 1, 1, 1),       # k = 540 in channel-major order, split over k
     (2, 48, 6, 6, 8, 3, 3, 1, 1, 1, 1, 1, 2),       # one bias set per sample: not split
+    (3, 16, 20, 24, 3, 3, 3, 1, 1, 1, 1, 1, 1),     # 3x3 to three channels: LDS-tiled vector-ALU kernel
+    (2, 8, 18, 36, 4, 3, 3, 1, 1, 1, 1, 1, 2),      # the same with partial tiles and one bias set per sample
 ]
 
 
