@@ -465,14 +465,19 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
         const float2 lo = *reinterpret_cast<const float2 *>(rowp), hi = *reinterpret_cast<const float2 *>(rowp + 2);
         v[dy][0] = lo.x; v[dy][1] = lo.y; v[dy][2] = hi.x; v[dy][3] = hi.y;
       }
+      // all 16*CO coefficients of a channel are contiguous, [ci][phase][co][taps (ty,tx) = 00 01 10 11]: CO uniform
+      // 64-byte loads through the scalar cache
+      floatx16 wv[CO];
+#pragma unroll
+      for (int j = 0; j < CO; j++) wv[j] = reinterpret_cast<const floatx16 *>(coeff + (size_t)ci * (16 * CO))[j];
 #pragma unroll
       for (int py = 0; py < 2; py++)
 #pragma unroll
         for (int px = 0; px < 2; px++) {
 #pragma unroll
           for (int co = 0; co < CO; co++) {
-            // all 16*CO coefficients of a channel are contiguous: [ci][phase][co][taps (ty,tx) = 00 01 10 11]
-            const float4 w = *reinterpret_cast<const float4 *>(coeff + (size_t)ci * (16 * CO) + ((py * 2 + px) * CO + co) * 4);
+            const int f = ((py * 2 + px) * CO + co) * 4;
+            const float4 w = make_float4(wv[f / 16][f % 16], wv[f / 16][f % 16 + 1], wv[f / 16][f % 16 + 2], wv[f / 16][f % 16 + 3]);
 #pragma unroll
             for (int p = 0; p < 2; p++) {
               float a = acc[p][py][px][co];
@@ -493,6 +498,7 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
   if (qy >= H || qx >= W) return;  // W is even: a pair is inside or outside as a whole
   const uint32_t OW = 2 * W, OHW = 4 * HW;
   const float bsum = args.ep.tap_bias ? args.ep.tap_bias[g % args.ep.bias_w] : 0.f;
+  const int func = args.ep.func;
 #pragma unroll
   for (int py = 0; py < 2; py++) {
     // contributing taps of output row 2*qy+py are input rows qy+py-1 and qy+py; likewise along x
@@ -500,13 +506,18 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
     const int nx[4] = {((uint32_t)((int32_t)qx - 1) < W) + 1, 2, 2, 1 + ((uint32_t)((int32_t)qx + 2) < W)};
 #pragma unroll
     for (int co = 0; co < CO; co++) {
-      float4 o;
-      o.x = mt::apply_func_epilogue(args.ep.func, acc[0][py][0][co] + bsum * (float)(ny * nx[0]));
-      o.y = mt::apply_func_epilogue(args.ep.func, acc[0][py][1][co] + bsum * (float)(ny * nx[1]));
-      o.z = mt::apply_func_epilogue(args.ep.func, acc[1][py][0][co] + bsum * (float)(ny * nx[2]));
-      o.w = mt::apply_func_epilogue(args.ep.func, acc[1][py][1][co] + bsum * (float)(ny * nx[3]));
+      float o[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) o[i] = acc[i / 2][py][i % 2][co] + bsum * (float)(ny * nx[i]);
+      if (func == MT_F_TANGENCE) {  // the usual end of an image generator: inline, the other functions share one body
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = mt::f_tangence(o[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = mt::apply_func_epilogue(func, o[i]);
+      }
       float *dst = args.ep.C + ((size_t)g * M + co) * OHW + (size_t)(2 * qy + py) * OW + 2 * qx;
-      *reinterpret_cast<float4 *>(dst) = o;
+      *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
     }
   }
 }
