@@ -227,6 +227,50 @@ __global__ __launch_bounds__(256) void tconv_prepare_kernel(float *packed, float
   }
 }
 
+// The same preparation for the common geometry kernel 4x4, stride 2 (four phases of 2x2 taps): one thread per
+// (input channel, output channel) reads the 16 contiguous coefficients of that pair once (four 128-bit loads) and
+// writes each phase its four; consecutive threads take consecutive input channels, so the writes of a wavefront are
+// contiguous.  blockIdx.y == CO sums the biases.
+__global__ __launch_bounds__(256) void tconv_prepare_k4s2_kernel(float *packed, float *sums, const float *kernel, const float *bias, PackArgs pa) {
+  if (blockIdx.y == (uint32_t)pa.CO) {
+    uint32_t wave = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x % 64, waves = gridDim.x * 4;
+    for (uint32_t w = wave; w < pa.bias_w; w += waves) {
+      float acc = 0.f;
+      for (uint32_t i = lane; i < (uint32_t)pa.CI; i += 64) acc += bias[(size_t)w * pa.CI + i];
+      acc = mt::wave_sum(acc);
+      if (lane == 0) sums[w] = acc;
+    }
+    return;
+  }
+  const uint32_t ci = blockIdx.x * 256 + threadIdx.x, co = blockIdx.y;
+  if (ci >= (uint32_t)pa.CI) return;
+  float k[16];
+  const float4 *src = reinterpret_cast<const float4 *>(kernel + (size_t)ci * pa.ker_ld + co * 16);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const float4 t = src[i];
+    k[4 * i] = t.x; k[4 * i + 1] = t.y; k[4 * i + 2] = t.z; k[4 * i + 3] = t.w;
+  }
+#pragma unroll
+  for (int f = 0; f < 4; f++) {
+    const PackPhase &ph = pa.ph[f];
+    float4 o;
+    // tap (ty, tx) of the phase is coefficient (3 - (ky0 + 2*ty), 3 - (kx0 + 2*tx)) of the kernel
+    float v[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const int ky = ph.ky0 + 2 * (t / 2), kx = ph.kx0 + 2 * (t % 2);
+      const int idx = (3 - ky) * 4 + (3 - kx);
+      float r = k[0];
+#pragma unroll
+      for (int q = 1; q < 16; q++) r = idx == q ? k[q] : r;   // ky0, kx0 are uniform: selects, no indexed registers
+      v[t] = r;
+    }
+    o = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4 *>(packed + ph.begin + (size_t)co * ph.co_stride + (size_t)ci * ph.ci_stride) = o;
+  }
+}
+
 // ---- transposed convolution with very few output channels (the image-producing last layer) --------------------
 // A 32-row matrix-core tile would be 90% padding for 3 output channels, so this case runs on the vector ALUs:
 // one thread per output pixel of one stride phase (blockIdx.y), CO accumulators, the packed sub-kernel read
@@ -832,9 +876,15 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   pa.nphase = args.nphase;
   {
     mt::ProfileScope prof("tconv_prepare");
-    unsigned gx = cdiv(max_pack ? max_pack : 1, 256 * 4);
-    if (gx > 1024) gx = 1024;
-    tconv_prepare_kernel<<<dim3(gx ? gx : 1, args.nphase + 1), 256, 0, mt::stream()>>>(packed, ws, kernel->p, bias->p, pa);
+    bool k4s2 = kx == 4 && ky == 4 && sx == 2 && sy == 2 && args.nphase == 4 && kernel->x % 4 == 0 && ((uintptr_t)kernel->p & 15u) == 0 && kz <= 65534;
+    for (uint32_t f = 0; k4s2 && f < 4; f++) k4s2 = pa.ph[f].ty == 2 && pa.ph[f].tx == 2 && pa.ph[f].ci_stride % 4 == 0 && pa.ph[f].co_stride % 4 == 0;
+    if (k4s2) {
+      tconv_prepare_k4s2_kernel<<<dim3(cdiv(ka, 256), kz + 1), 256, 0, mt::stream()>>>(packed, ws, kernel->p, bias->p, pa);
+    } else {
+      unsigned gx = cdiv(max_pack ? max_pack : 1, 256 * 4);
+      if (gx > 1024) gx = 1024;
+      tconv_prepare_kernel<<<dim3(gx ? gx : 1, args.nphase + 1), 256, 0, mt::stream()>>>(packed, ws, kernel->p, bias->p, pa);
+    }
     MT_LAUNCH_CHECK("tconv_prepare");
   }
   args.M = kz; args.out_w = out->w;
