@@ -85,15 +85,26 @@ def discriminator_step(args):
     for _ in range(args.warmup):
         net.step(fused=True)
     mt.synchronize()
+    # the step is recorded once as a HIP graph and replayed; Adam's iteration count is an argument of the recorded
+    # kernels, so the replays repeat iteration `warmup + 1` (same work, same arithmetic)
+    graph = mt.Graph(lambda: net.step(fused=True))
+    for _ in range(3):
+        graph.launch()
+    mt.synchronize()
     e0, e1 = create(), create()
     t0 = time.perf_counter()
     record(e0, stream)
     for _ in range(args.steps):
-        net.step(fused=True)
+        graph.launch()
     record(e1, stream)
     mt.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     gpu_ms = elapsed_ms(e0, e1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        net.step(fused=True)
+    mt.synchronize()
+    eager_ms = (time.perf_counter() - t0) * 1e3
     mt.profile_enable(True)
     for _ in range(args.steps):
         net.step(fused=True)
@@ -109,8 +120,9 @@ def discriminator_step(args):
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[4]: DCGAN-64 discriminator, batch 128: conv 4x4 s2 p1 3->64->128->256->512 with BN + leaky ReLU, "
                                "Linear 8192->1, sigmoid; forward, backward (input, weight, bias, BN gradients), Adam", "global_batch": batch,
-                   "path": "fused C-ABI entry points"},
+                   "path": "fused C-ABI entry points, step replayed as a HIP graph"},
         "gpu_ms_per_step_events": gpu_ms / args.steps, "host_ms_per_step_wall": wall_ms / args.steps,
+        "ms_per_step_eager_from_python": eager_ms / args.steps,
         "kernel_ms_per_step_sum": sum(v[1] for v in prof.values()) / args.steps,
         "conv_gflops": flop / (conv_ms * 1e-3) / 1e9, "conv_ms_per_step": conv_ms,
         "conv_frac_of_fp32_mfma_peak": flop / (conv_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
@@ -127,6 +139,9 @@ def main():
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also launch one plain copy (mt_set) of this many MiB before the timed region: the known-size kernel "
                          "that calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--graph", action="store_true",
+                    help="time region 1 as replays of the step recorded once as a HIP graph (c5 does so by default: its step "
+                         "is about a hundred short kernels and the Python host would be the bottleneck)")
     ap.add_argument("--workload", choices=["c3", "c5"], default="c3",
                     help="c3 (default, the measured configuration): DCGAN-64 generator forward, batch 256; "
                          "c5 (secondary): DCGAN-64 discriminator training step, batch 128")
@@ -155,12 +170,18 @@ def main():
         mt.synchronize()
 
     # Timed region 1 (-> value): K steps between two events on the work stream, host wall clock beside it.
+    step = net.forward_fused
+    if args.graph:
+        graph = mt.Graph(net.forward_fused)
+        step = graph.launch
+        for _ in range(3):
+            step()
     e0, e1 = create(), create()
     mt.synchronize()
     t0 = time.perf_counter()
     record(e0, stream)
     for _ in range(args.steps):
-        net.forward_fused()
+        step()
     record(e1, stream)
     mt.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3

@@ -145,9 +145,14 @@ class Discriminator:
         # Linear: previous error, per-sample outer products, their sum over the batch
         flat_err = self.d_a[3].reinterpret(b, 1, CHANNELS[4] * 16, 1)
         CTensorMath.TransponseMul(flat_err, p["lin_w"], self.d_logit)
-        CTensorMath.Mul(self.tmp_dw, self.d_logit, self.a[3].reinterpret(b, 1, 1, CHANNELS[4] * 16))
-        CTensorMath.Fill(g["lin_w"], 0.0)
-        CTensorMath.AddSumW(g["lin_w"], g["lin_w"], self.tmp_dw)
+        if fused:
+            # dW = sum_b delta_b (x) h_b is one product delta^T * H over the batch axis: the same tensors viewed as
+            # [1,1,B,Out] and [1,1,B,In] (ReinterpretSize), no per-sample outer products
+            CTensorMath.TransponseMul(g["lin_w"], self.d_logit.reinterpret(1, 1, b, 1), self.a[3].reinterpret(1, 1, b, CHANNELS[4] * 16))
+        else:
+            CTensorMath.Mul(self.tmp_dw, self.d_logit, self.a[3].reinterpret(b, 1, 1, CHANNELS[4] * 16))
+            CTensorMath.Fill(g["lin_w"], 0.0)
+            CTensorMath.AddSumW(g["lin_w"], g["lin_w"], self.tmp_dw)
         CTensorMath.Fill(g["lin_b"], 0.0)
         CTensorMath.AddSumW(g["lin_b"], g["lin_b"], self.d_logit)
         for i in (3, 2, 1, 0):

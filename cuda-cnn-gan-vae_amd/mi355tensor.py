@@ -94,6 +94,41 @@ def set_stream(handle):
     call("mt_set_stream", C.c_void_p(handle))
 
 
+class Graph:
+    """A sequence of library calls recorded once as a HIP graph and replayed with one launch: for steps made of many
+    short kernels, where the host would otherwise be the bottleneck.  Everything the calls allocate (workspaces) must
+    exist before the recording, so run the sequence once eagerly first.  The recorded kernels keep the pointers and
+    sizes of the recording."""
+
+    def __init__(self, record):
+        hip = C.CDLL("libamdhip64.so")
+        self._hip, self._stream = hip, C.c_void_p(get_stream())
+        graph, self._exec = C.c_void_p(), C.c_void_p()
+        self._check(hip.hipStreamBeginCapture(self._stream, C.c_int(2)), "hipStreamBeginCapture")   # relaxed mode
+        try:
+            record()
+        finally:
+            rc = hip.hipStreamEndCapture(self._stream, C.byref(graph))
+        self._check(rc, "hipStreamEndCapture")
+        self._check(hip.hipGraphInstantiate(C.byref(self._exec), graph, None, None, C.c_size_t(0)), "hipGraphInstantiate")
+        hip.hipGraphDestroy(graph)
+
+    @staticmethod
+    def _check(rc, what):
+        if rc != 0:
+            raise RuntimeError("%s failed with hipError %d" % (what, rc))
+
+    def launch(self):
+        self._check(self._hip.hipGraphLaunch(self._exec, self._stream), "hipGraphLaunch")
+
+    def __del__(self):
+        try:
+            if self._exec:
+                self._hip.hipGraphExecDestroy(self._exec)
+        except Exception:
+            pass
+
+
 class CTensor:
     """Device-resident [W,Z,Y,X] fp32 tensor (uint32 pairs for pooling positions when `pos` is set)."""
 

@@ -279,3 +279,27 @@ def test_config4_full_batch_properties(gpu, oracle):
     one = seq.vae_decoder_forward(oracle, params, z[20:21])
     for name in one:
         assert rel_err(d[name][20:21], one[name]) <= REL, name
+
+
+def test_recorded_graph_replays(gpu, oracle):
+    """A discriminator forward pass recorded as a HIP graph: every replay, with eager work and synchronisations of the
+    program between the replays, gives the eager result for the input that is in the tensors at that moment."""
+    import discriminator as D
+    import mi355tensor as mt
+    net = D.Discriminator(8)
+    batches = [D.make_batch(8, seed=s) for s in (60, 61, 62, 63)]
+    net.set_batch(*batches[0])
+    net.forward(True)                                   # allocates the workspaces
+    mt.synchronize()
+    graph = mt.Graph(lambda: net.forward(True))
+    for x, labels in batches:
+        net.set_batch(x, labels)
+        eager = net.forward(True).numpy()
+        acts = [t.numpy() for t in net.a]
+        for t in net.a + [net.prob]:
+            mt.CTensorMath.Fill(t, 7.0)                 # eager work in between; the replay must overwrite it
+        mt.synchronize()
+        graph.launch()
+        assert np.array_equal(net.prob.numpy(), eager)
+        for t, want in zip(net.a, acts):
+            assert np.array_equal(t.numpy(), want)
