@@ -72,6 +72,70 @@ def cpu_baseline(sample_batch):
             "sample": "one generator forward at batch %d (%.1f s), scaled linearly; host has %d cores" % (sample_batch, dt, os.cpu_count() or 0)}
 
 
+def memory_bound_ops(args):
+    """Secondary workload: the HBM-bound tensor operations on the largest activation of the measured configuration,
+    [256,64,32,32] fp32 (67 MB), each timed on its own with HIP events; achieved = algorithmic bytes / time against the
+    8 TB/s HBM peak.  One JSON line."""
+    import numpy as np
+    import mi355tensor as mt
+    from mi355tensor import CTensor, CTensorApplyFunc as F, CTensorMath as M, Fused
+    mt.init(0)
+    shape, s1 = (256, 64, 32, 32), (1, 64, 32, 32)
+    n = 256 * 64 * 32 * 32
+    rng = np.random.default_rng(0)
+    a, b, out = (CTensor.from_numpy(rng.standard_normal(shape).astype(np.float32)) for _ in range(3))
+    g, be, m1, v1 = (CTensor.from_numpy(np.abs(rng.standard_normal(s1)).astype(np.float32) + 0.5) for _ in range(4))
+    xhat, sums, bias = CTensor(*shape), CTensor(256, 64, 1, 1), CTensor.from_numpy(np.ones((1, 64, 1, 1), np.float32))
+    half, pos, up = CTensor(256, 64, 16, 16), CTensor(256, 64, 16, 16, pos=True), CTensor(256, 64, 64, 64)
+    big = CTensor(256, 64, 64, 64)
+    mom, vel = CTensor.from_numpy(np.zeros(shape, np.float32)), CTensor.from_numpy(np.zeros(shape, np.float32))
+    B = 4.0 * n
+    ops = [  # name, callable, algorithmic bytes
+        ("Fill", lambda: M.Fill(out, 1.0), B),
+        ("Set (copy)", lambda: M.Set(out, a, 1.0, 0.0), 2 * B),
+        ("Add", lambda: M.Add(out, a, b, 1.0, 1.0), 3 * B),
+        ("Add, broadcast right operand [1,Z,Y,X]", lambda: M.Add(out, a, g, 1.0, 1.0), 2 * B),
+        ("TensorItemProduction", lambda: M.TensorItemProduction(out, a, b), 3 * B),
+        ("Pow2", lambda: M.Pow2(out, a, 1.0), 2 * B),
+        ("ApplyReLU", lambda: F.ApplyReLU(out, a), 2 * B),
+        ("ApplyTangence", lambda: F.ApplyTangence(out, a), 2 * B),
+        ("ApplyDifferentialLeakyReLU", lambda: F.ApplyDifferentialLeakyReLU(out, a), 2 * B),
+        ("AddBias", lambda: M.AddBias(out, bias), 2 * B),
+        ("AddSumW (sum over the batch)", lambda: M.AddSumW(m1, m1, a, 1.0, 1.0 / 256), B),
+        ("SummXY", lambda: M.SummXY(sums, a), B),
+        ("batch norm forward, training mode, fused + ReLU", lambda: Fused.BatchNormForwardTrain(out, a, g, be, func="relu"), 2 * B),
+        ("batch norm forward, training mode, keeping xhat", lambda: Fused.BatchNormForwardTrain(out, a, g, be, xhat, v1), 3 * B),
+        ("batch norm forward, inference mode, fused + ReLU", lambda: Fused.BatchNormForwardInfer(out, a, g, be, m1, v1, func="relu"), 2 * B),
+        ("batch norm backward, fused", lambda: Fused.BatchNormBackward(out, m1, v1, a, g, b, be), 3 * B),
+        ("MaxPooling 2x2 (+ positions)", lambda: M.MaxPooling(half, pos, a, 2, 2), B + 3 * B / 4),
+        ("MaxPoolingBackward 2x2", lambda: M.MaxPoolingBackward(out, pos, half, 2, 2), B + 3 * B / 4),
+        ("UpSampling x2", lambda: M.UpSampling(up, a, 2, 2), B + 4 * B),
+        ("DownSampling x2", lambda: M.DownSampling(a, big, 2, 2), 4 * B + B),
+        ("Adam", lambda: M.Adam(out, a, mom, vel, 256, 2e-4, 0.5, 0.999, 1e-8, 1.0), 7 * B),
+    ]
+    stream = mt.get_stream()
+    create, record, elapsed_ms = hip_events()
+    results = {}
+    for name, fn, nbytes in ops:
+        for _ in range(args.warmup):
+            fn()
+        e0, e1 = create(), create()
+        record(e0, stream)
+        for _ in range(args.steps):
+            fn()
+        record(e1, stream)
+        us = elapsed_ms(e0, e1) / args.steps * 1e3
+        results[name] = {"us": us, "GB/s": nbytes / us / 1e3, "frac_of_hbm_peak": nbytes / us / 1e3 / 8000.0, "algorithmic_MB": nbytes / 1e6}
+    rates = [r["GB/s"] for r in results.values()]
+    print(json.dumps({
+        "metric": "GB/s of the HBM-bound tensor operations on a [256,64,32,32] fp32 activation (secondary workload)",
+        "value": float(np.median(rates)), "unit": "GB/s (median over the operations)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sum(r["us"] for r in results.values()) / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic", "config": {"workload": "every HBM-bound operation of the tensor-op layer, one launch each per step"},
+        "roofline": {"bound": "hbm", "peak": 8000.0, "unit": "GB/s", "achieved": float(np.median(rates)), "frac": float(np.median(rates)) / 8000.0},
+        "operations": results}))
+
+
 def discriminator_step(args):
     """Secondary workload (configs[4]): forward, backward and Adam update of the DCGAN-64 discriminator at batch 128
     through the fused entry points.  Same two timed regions as the main workload; one JSON line."""
@@ -142,14 +206,17 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="time region 1 as replays of the step recorded once as a HIP graph (c5 does so by default: its step "
                          "is about a hundred short kernels and the Python host would be the bottleneck)")
-    ap.add_argument("--workload", choices=["c3", "c5"], default="c3",
+    ap.add_argument("--workload", choices=["c3", "c5", "ops"], default="c3",
                     help="c3 (default, the measured configuration): DCGAN-64 generator forward, batch 256; "
-                         "c5 (secondary): DCGAN-64 discriminator training step, batch 128")
+                         "c5 (secondary): DCGAN-64 discriminator training step, batch 128; "
+                         "ops (secondary): every HBM-bound tensor operation on a [256,64,32,32] activation, GB/s each")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the path shards along the batch axis, see DESIGN.md")
     if args.workload == "c5":
         return discriminator_step(args)
+    if args.workload == "ops":
+        return memory_bound_ops(args)
 
     import mi355tensor as mt
     import generator as G

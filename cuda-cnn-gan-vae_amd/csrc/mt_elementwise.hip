@@ -61,6 +61,12 @@ __global__ __launch_bounds__(EW_THREADS) void ew2_kernel(float *out, Operand a, 
 }
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+// grid.y of the kernels that loop over planes: enough blocks to fill the machine, few enough that a thread's index
+// arithmetic is spread over several planes
+inline unsigned plane_blocks(unsigned blocks_x, uint32_t planes) {
+  unsigned want = blocks_x >= 8192u ? 1u : 8192u / blocks_x;
+  return planes < want ? planes : want;
+}
 
 template <class F>
 int launch1(const char *name, const mt_tensor *out, const mt_tensor *in, F f) {
@@ -106,6 +112,12 @@ struct FSub { float ls, rs; __device__ float operator()(float l, float r) const 
 struct FDiv { float ls, rs; __device__ float operator()(float l, float r) const { return (ls * l) / (rs * r); } };
 struct FMul { __device__ float operator()(float l, float r) const { return l * r; } };
 
+__global__ __launch_bounds__(EW_THREADS) void fill4_kernel(float4 *out, size_t n4, float v) {
+  size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * EW_THREADS;
+  const float4 q = make_float4(v, v, v, v);
+  for (; i < n4; i += stride) out[i] = q;
+}
 __global__ __launch_bounds__(EW_THREADS) void fill_kernel(float *out, size_t n, float v) {
   size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
   size_t stride = (size_t)gridDim.x * EW_THREADS;
@@ -155,6 +167,58 @@ __global__ __launch_bounds__(EW_THREADS) void summ_xy_kernel(float *out, const f
 }
 
 // ---- AddBias: working[w][z][.] += bias[w%Wb][z] ------------------------------------------------------------------
+// The same with 128-bit accesses: a block owns 32 groups of four columns and splits the batch over 8 slices that are
+// combined in LDS; the slice loop is unrolled so that several loads per thread are in flight.
+__global__ __launch_bounds__(EW_THREADS) void add_sum_w_vec_kernel(float *out, uint32_t Wout, const float *L, uint32_t Wl, const float *R, uint32_t Wr,
+                                                                   uint32_t S, float ls, float rs) {
+  constexpr int RB = 32, WS = EW_THREADS / RB;
+  __shared__ float4 part[2][WS][RB];
+  const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
+  const uint32_t r = (blockIdx.x * RB + rl) * 4;
+  float4 sl = make_float4(0.f, 0.f, 0.f, 0.f), sr = sl;
+  if (r < S) {
+#pragma unroll 4
+    for (uint32_t w = ws; w < Wl; w += WS) {
+      const float4 q = *reinterpret_cast<const float4 *>(L + (size_t)w * S + r);
+      sl.x += q.x; sl.y += q.y; sl.z += q.z; sl.w += q.w;
+    }
+#pragma unroll 4
+    for (uint32_t w = ws; w < Wr; w += WS) {
+      const float4 q = *reinterpret_cast<const float4 *>(R + (size_t)w * S + r);
+      sr.x += q.x; sr.y += q.y; sr.z += q.z; sr.w += q.w;
+    }
+  }
+  part[0][ws][rl] = sl;
+  part[1][ws][rl] = sr;
+  __syncthreads();
+  if (r >= S) return;
+  if (ws == 0) {
+    sl = make_float4(0.f, 0.f, 0.f, 0.f); sr = sl;
+#pragma unroll
+    for (int i = 0; i < WS; i++) {
+      const float4 a = part[0][i][rl], b = part[1][i][rl];
+      sl.x += a.x; sl.y += a.y; sl.z += a.z; sl.w += a.w;
+      sr.x += b.x; sr.y += b.y; sr.z += b.z; sr.w += b.w;
+    }
+    float4 o;
+    o.x = sl.x * ls + sr.x * rs; o.y = sl.y * ls + sr.y * rs; o.z = sl.z * ls + sr.z * rs; o.w = sl.w * ls + sr.w * rs;
+    *reinterpret_cast<float4 *>(out + r) = o;
+  }
+  for (uint32_t w = 1 + ws; w < Wout; w += WS) *reinterpret_cast<float4 *>(out + (size_t)w * S + r) = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+__global__ __launch_bounds__(EW_THREADS) void add_bias4_kernel(float *t, const float *bias, uint32_t Wb, uint32_t Z, uint32_t YX4, uint32_t rows) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (i >= YX4) return;
+  for (uint32_t row = blockIdx.y; row < rows; row += gridDim.y) {
+    const uint32_t w = row / Z, z = row % Z;
+    const float b = bias[(size_t)(w % Wb) * Z + z];
+    float4 *p = reinterpret_cast<float4 *>(t + (size_t)row * YX4 * 4) + i;
+    float4 q = *p;
+    q.x += b; q.y += b; q.z += b; q.w += b;
+    *p = q;
+  }
+}
 __global__ __launch_bounds__(EW_THREADS) void add_bias_kernel(float *t, const float *bias, uint32_t Wb, uint32_t Z, uint32_t YX, uint32_t rows) {
   for (uint32_t row = blockIdx.y; row < rows; row += gridDim.y) {
     uint32_t w = row / Z, z = row % Z;
@@ -199,6 +263,46 @@ __global__ __launch_bounds__(EW_THREADS) void upsampling_kernel(float *out, cons
   }
 }
 
+// Four consecutive output columns per thread (one 128-bit store); ox is a multiple of 4.
+__global__ __launch_bounds__(EW_THREADS) void upsampling4_kernel(float *out, const float *in, Geo g, uint32_t ux, uint32_t uy, uint32_t planes) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ox4 = g.ox / 4, n4 = g.oy * ox4;
+  if (i >= n4) return;
+  const uint32_t y = i / ox4, x = (i % ox4) * 4, sy = y / uy;
+  uint32_t sx[4];
+#pragma unroll
+  for (int k = 0; k < 4; k++) sx[k] = (x + k) / ux;
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const uint32_t w = pl / g.Z, z = pl % g.Z;
+    const float *src = in + (((size_t)(w % g.Win) * g.Z + z) * g.iy + sy) * g.ix;
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = (sy < g.iy && sx[k] < g.ix) ? src[sx[k]] : 0.f;
+    reinterpret_cast<float4 *>(out + (size_t)pl * g.oy * g.ox)[i] = make_float4(v[0], v[1], v[2], v[3]);
+  }
+}
+__global__ __launch_bounds__(EW_THREADS) void max_pooling_backward4_kernel(float *out, const mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t px_, uint32_t py_, uint32_t planes) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ox4 = g.ox / 4, n4 = g.oy * ox4;
+  if (i >= n4) return;
+  const uint32_t y = i / ox4, x = (i % ox4) * 4, sy = y / py_;
+  uint32_t sx[4];
+#pragma unroll
+  for (int k = 0; k < 4; k++) sx[k] = (x + k) / px_;
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const uint32_t w = pl / g.Z, z = pl % g.Z;
+    const mt_spos *prow = pos + (((size_t)(w % Wpos) * g.Z + z) * g.iy + sy) * g.ix;
+    const float *irow = in + ((size_t)pl * g.iy + sy) * g.ix;
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      v[k] = 0.f;
+      if (sy < g.iy && sx[k] < g.ix) {
+        const mt_spos s = prow[sx[k]];
+        if (s.X == x + k && s.Y == y) v[k] = irow[sx[k]];
+      }
+    }
+    reinterpret_cast<float4 *>(out + (size_t)pl * g.oy * g.ox)[i] = make_float4(v[0], v[1], v[2], v[3]);
+  }
+}
 __global__ __launch_bounds__(EW_THREADS) void downsampling_kernel(float *out, const float *in, Geo g, uint32_t dsx, uint32_t dsy, uint32_t planes) {
   uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, n = g.oy * g.ox;
   if (i >= n) return;
@@ -581,6 +685,13 @@ int mt_fill(const mt_tensor *out, float value) {
   if (mt::bad(out)) return mt::fail(MT_E_ARGUMENT, "mt_fill: null tensor");
   size_t n = mt::count(out);
   if (n == 0) return MT_OK;
+  if (n % 4 == 0 && aligned16(out->p)) {
+    unsigned blocks = cdiv(n / 4, EW_THREADS);
+    if (blocks > 8192u) blocks = 8192u;
+    fill4_kernel<<<blocks, EW_THREADS, 0, mt::stream()>>>(reinterpret_cast<float4 *>(out->p), n / 4, value);
+    MT_LAUNCH_CHECK("mt_fill");
+    return MT_OK;
+  }
   unsigned blocks = cdiv(n, EW_THREADS);
   if (blocks > 65536u * 4) blocks = 65536u * 4;
   fill_kernel<<<blocks, EW_THREADS, 0, mt::stream()>>>(out->p, n, value);
@@ -617,7 +728,9 @@ int mt_add_sum_w(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, f
   if (S == 0 || out->w == 0) return MT_OK;
   mt::ProfileScope prof("mt_add_sum_w");
   // the output may alias an operand (dW = dW + sum_w TmpdW): every column is read completely before it is written
-  if (S >= 65536)
+  if (S % 4 == 0 && S >= 4096 && aligned16(out->p) && aligned16(l->p) && aligned16(r->p))
+    add_sum_w_vec_kernel<<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
+  else if (S >= 65536)
     add_sum_w_kernel<256><<<cdiv(S, 256), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
   else
     add_sum_w_kernel<32><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
@@ -644,6 +757,12 @@ int mt_add_bias(const mt_tensor *t, const mt_tensor *bias) {
   uint32_t rows = t->w * t->z, YX = t->y * t->x;
   if (rows == 0 || YX == 0) return MT_OK;
   if (bias->y != 1 || bias->x != 1) return mt::fail(MT_E_ARGUMENT, "mt_add_bias: bias must be [W,Z,1,1]");
+  if (YX % 4 == 0 && aligned16(t->p)) {
+    dim3 grid4(cdiv(YX / 4, EW_THREADS), plane_blocks(cdiv(YX / 4, EW_THREADS), rows));
+    add_bias4_kernel<<<grid4, EW_THREADS, 0, mt::stream()>>>(t->p, bias->p, bias->w, t->z, YX / 4, rows);
+    MT_LAUNCH_CHECK("mt_add_bias");
+    return MT_OK;
+  }
   dim3 grid(cdiv(YX, EW_THREADS), rows < 65535u ? rows : 65535u);
   add_bias_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(t->p, bias->p, bias->w, t->z, YX, rows);
   MT_LAUNCH_CHECK("mt_add_bias");
@@ -668,6 +787,12 @@ int mt_upsampling(const mt_tensor *out, const mt_tensor *in, uint32_t ux, uint32
   uint32_t planes = out->w * out->z, n = out->y * out->x;
   if (planes == 0 || n == 0) return MT_OK;
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  if (out->x % 4 == 0 && aligned16(out->p)) {
+    dim3 grid4(cdiv(n / 4, EW_THREADS), plane_blocks(cdiv(n / 4, EW_THREADS), planes));
+    upsampling4_kernel<<<grid4, EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, ux, uy, planes);
+    MT_LAUNCH_CHECK("mt_upsampling");
+    return MT_OK;
+  }
   dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
   upsampling_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, ux, uy, planes);
   MT_LAUNCH_CHECK("mt_upsampling");
@@ -708,6 +833,12 @@ int mt_max_pooling_backward(const mt_tensor *out, const mt_pos_tensor *pos, cons
   if (pos->p == nullptr || pos->w == 0 || pos->z != in->z || pos->y != in->y || pos->x != in->x)
     return mt::fail(MT_E_ARGUMENT, "mt_max_pooling_backward: position tensor must be [W',Z,Y,X] of the input");
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  if (out->x % 4 == 0 && aligned16(out->p)) {
+    dim3 grid4(cdiv(n / 4, EW_THREADS), plane_blocks(cdiv(n / 4, EW_THREADS), planes));
+    max_pooling_backward4_kernel<<<grid4, EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, px, py, planes);
+    MT_LAUNCH_CHECK("mt_max_pooling_backward");
+    return MT_OK;
+  }
   dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
   max_pooling_backward_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, px, py, planes);
   MT_LAUNCH_CHECK("mt_max_pooling_backward");
