@@ -159,17 +159,61 @@ __global__ __launch_bounds__(256) void dbias_wave_kernel(float *dbias, const flo
   if (lane == 0) dbias[row] += s;
 }
 
-// dbias[f] += sum over the whole batch and all pixels of delta[w][f]: one wavefront per filter
-__global__ __launch_bounds__(256) void dbias_batch_sum_kernel(float *dbias, const float *delta, uint32_t B, uint32_t KA, uint32_t DHW) {
-  uint32_t f = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x % 64;
+// Sum over the whole batch and all pixels of delta[w][f], one value per filter.  Block (f, c) adds the samples
+// c*per .. (c+1)*per-1 of filter f (V = float4 when the rows allow it, else float) and writes partial[f*chunks + c],
+// or adds to dbias[f] itself when chunks == 1.  The partials are added in a fixed order by dbias_finish_kernel.
+template <class V>
+__global__ __launch_bounds__(256) void dbias_batch_sum_kernel(float *dbias, float *partial, const V *delta, uint32_t per, uint32_t KA, uint32_t DV, uint32_t chunks) {
+  const uint32_t f = blockIdx.x, c = blockIdx.y, t = threadIdx.x;
+  const uint32_t count = per * DV;  // vectors of this block
+  const V *base = delta + ((size_t)c * per * KA + f) * DV;
+  const size_t sample = (size_t)KA * DV;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  auto at = [&](uint32_t i) -> float {
+    if (i >= count) return 0.f;
+    const uint32_t w = i / DV, x = i - w * DV;
+    const V v = base[(size_t)w * sample + x];
+    if constexpr (sizeof(V) == 16) return (v.x + v.y) + (v.z + v.w);
+    else return v;
+  };
+  for (uint32_t i = t; i < count; i += 1024) {
+    s0 += at(i); s1 += at(i + 256); s2 += at(i + 512); s3 += at(i + 768);
+  }
+  __shared__ float part[4];
+  const float s = mt::wave_sum((s0 + s1) + (s2 + s3));
+  if (t % 64 == 0) part[t / 64] = s;
+  __syncthreads();
+  if (t == 0) {
+    const float sum = (part[0] + part[1]) + (part[2] + part[3]);
+    if (chunks == 1) dbias[f] += sum;
+    else partial[f * chunks + c] = sum;
+  }
+}
+__global__ __launch_bounds__(256) void dbias_finish_kernel(float *dbias, const float *partial, uint32_t KA, uint32_t chunks) {
+  const uint32_t f = blockIdx.x * 256 + threadIdx.x;
   if (f >= KA) return;
   float s = 0.f;
-  for (uint32_t w = 0; w < B; w++) {
-    const float *dl = delta + ((size_t)w * KA + f) * DHW;
-    for (uint32_t i = lane; i < DHW; i += 64) s += dl[i];
+  for (uint32_t c = 0; c < chunks; c++) s += partial[f * chunks + c];
+  dbias[f] += s;
+}
+// chunks of the batch per filter: enough blocks to fill the device, each with at least a few thousand values
+uint32_t dbias_chunks(uint32_t B, uint32_t KA, uint32_t DHW) {
+  uint32_t chunks = 1;
+  while (chunks * 2 <= B && B % (chunks * 2) == 0 && KA * chunks < 1024 && (size_t)(B / (chunks * 2)) * DHW >= 4096) chunks *= 2;
+  return chunks;
+}
+int dbias_batch_sum(const char *name, float *dbias, float *partial, const float *delta, uint32_t B, uint32_t KA, uint32_t DHW, uint32_t chunks) {
+  const dim3 grid(KA, chunks);
+  if (DHW % 4 == 0 && ((uintptr_t)delta & 15u) == 0)
+    dbias_batch_sum_kernel<float4><<<grid, 256, 0, mt::stream()>>>(dbias, partial, (const float4 *)delta, B / chunks, KA, DHW / 4, chunks);
+  else
+    dbias_batch_sum_kernel<float><<<grid, 256, 0, mt::stream()>>>(dbias, partial, delta, B / chunks, KA, DHW, chunks);
+  MT_LAUNCH_CHECK(name);
+  if (chunks > 1) {
+    dbias_finish_kernel<<<cdiv(KA, 256), 256, 0, mt::stream()>>>(dbias, partial, KA, chunks);
+    MT_LAUNCH_CHECK(name);
   }
-  s = mt::wave_sum(s);
-  if (lane == 0) dbias[f] += s;
+  return MT_OK;
 }
 
 // ---- transposed convolution: phase geometry, kernel packing, bias sums ----------------------------------------
@@ -995,10 +1039,14 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     groups = g;
   }
   const uint32_t per = B / groups;
-  float *partial = nullptr;
-  if (groups > 1) {
-    if (dk->x != ncol || dk->z * dk->y != ka) return mt::fail(MT_E_ARGUMENT, "%s: the summed kernel gradient must be exactly [1,1,%u,%u]", name, ka, ncol);
-    if ((rc = workspace((size_t)groups * ka * ncol, &partial))) return rc;
+  float *partial = nullptr, *dbias_partial = nullptr;
+  const uint32_t chunks = dbias_chunks(B, ka, DHW);
+  const size_t wgrad_floats = groups > 1 ? (size_t)groups * ka * ncol : 0;
+  if (groups > 1 && (dk->x != ncol || dk->z * dk->y != ka))
+    return mt::fail(MT_E_ARGUMENT, "%s: the summed kernel gradient must be exactly [1,1,%u,%u]", name, ka, ncol);
+  if (wgrad_floats + (chunks > 1 ? (size_t)ka * chunks : 0) > 0) {
+    if ((rc = workspace(wgrad_floats + (size_t)ka * chunks, &partial))) return rc;
+    dbias_partial = partial + wgrad_floats;
   }
   SrcRowK<true> a{};
   a.p = delta->p; a.ld = DHW; a.R = ka; a.K = per * DHW; a.seg = DHW; a.seg_stride = (uint32_t)sample_delta;
@@ -1026,9 +1074,7 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     mt_tensor pt{partial, groups, 1, ka, ncol}, flat{dk->p, 1, 1, ka, ncol};
     if ((rc = mt_add_sum_w(&flat, &flat, &pt, 1.f, 1.f))) return rc;
   }
-  dbias_batch_sum_kernel<<<cdiv(ka, 4), 256, 0, mt::stream()>>>(db->p, delta->p, B, ka, DHW);
-  MT_LAUNCH_CHECK(name);
-  return MT_OK;
+  return dbias_batch_sum(name, db->p, dbias_partial, delta->p, B, ka, DHW, chunks);
 }
 
 }  // namespace

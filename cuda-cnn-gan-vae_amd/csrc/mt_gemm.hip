@@ -44,9 +44,34 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *out, const fl
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float acc = 0.f;
-  for (uint32_t s = 0; s < S; s++) acc += partial[(size_t)s * n + i];
+  const float *p = partial + i;
+  uint32_t s = 0;
+  for (; s + 4 <= S; s += 4, p += 4 * n) {  // four loads in flight
+    const float v0 = p[0], v1 = p[n], v2 = p[2 * n], v3 = p[3 * n];
+    acc += v0; acc += v1; acc += v2; acc += v3;
+  }
+  for (; s < S; s++, p += n) acc += p[0];
   if (bias) acc += bias[(i / bias_div) % bias_mod];
   out[i] = mt::apply_func(func, acc);
+}
+// The same for a small output: 16 outputs per block, 16 threads per output each adding every 16th partial, then the
+// 16 sums in a fixed order (one thread per output over all S partials would be a long chain of dependent loads).
+__global__ __launch_bounds__(256) void splitk_reduce_small_kernel(float *out, const float *partial, uint32_t S, uint32_t n, const float *bias, uint32_t bias_div,
+                                                                  uint32_t bias_mod, int func) {
+  const uint32_t t = threadIdx.x, il = t % 16, g = t / 16, i = blockIdx.x * 16 + il;
+  __shared__ float part[16][17];
+  float acc = 0.f;
+  if (i < n)
+    for (uint32_t s = g; s < S; s += 16) acc += partial[(size_t)s * n + i];
+  part[g][il] = acc;
+  __syncthreads();
+  if (g == 0 && i < n) {
+    float sum = 0.f;
+#pragma unroll
+    for (uint32_t k = 0; k < 16; k++) sum += part[k][il];
+    if (bias) sum += bias[(i / bias_div) % bias_mod];
+    out[i] = mt::apply_func(func, sum);
+  }
 }
 
 // C[w,z] = op(A[w%Wa,z]) * B[w%Wb,z];  op = transpose when `ta` (A stored [K][M]).
@@ -125,7 +150,10 @@ int split_workspace(size_t floats, float **p) {
   return MT_OK;
 }
 int split_reduce(const char *name, float *out, const float *partial, uint32_t S, size_t n, const float *bias, uint32_t bias_div, uint32_t bias_mod, int func) {
-  splitk_reduce_kernel<<<cdiv(n, 256), 256, 0, stream()>>>(out, partial, S, n, bias, bias_div, bias_mod, func);
+  if (n <= 16384 && S >= 32)
+    splitk_reduce_small_kernel<<<cdiv(n, 16), 256, 0, stream()>>>(out, partial, S, (uint32_t)n, bias, bias_div, bias_mod, func);
+  else
+    splitk_reduce_kernel<<<cdiv(n, 256), 256, 0, stream()>>>(out, partial, S, n, bias, bias_div, bias_mod, func);
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }

@@ -237,6 +237,8 @@ def test_wgrad_w_broadcast(gpu, oracle, path):
     (5, 16, 8, 8, 130, 4, 2, 1),     # 16 output pixels: one k step per sample
     (2, 40, 32, 32, 64, 4, 2, 1),    # 256 output pixels, 640 columns
     (7, 1, 4, 4, 1, 1, 1, 0),        # 1x1 kernel, one channel, odd batch
+    (16, 2, 64, 64, 3, 4, 2, 1),     # 1024 output pixels, 16 samples: the bias sum runs over the batch in four chunks
+    (8, 1, 35, 35, 2, 3, 1, 0),      # 33x33 output pixels: rows that are no multiple of four floats, two chunks
 ])
 def test_convolution_backward_weights_sum(gpu, oracle, path, case):
     """The batch-summed weight gradient against the layer's own sequence: per-sample gradients into zeroed batch
