@@ -743,6 +743,7 @@ int mt_summ_xy(const mt_tensor *out, const mt_tensor *in) {
   if (in->z != out->z) return mt::fail(MT_E_SHAPE, "mt_summ_xy: depth of input and output differ");
   uint32_t rows = out->w * out->z;
   if (rows == 0) return MT_OK;
+  if (in->w == 0) return mt::fail(MT_E_ARGUMENT, "mt_summ_xy: empty input");
   if (out->y != 1 || out->x != 1) {  // the reference writes element (w,z,0,0) of a larger output; keep that addressing
     return mt::fail(MT_E_ARGUMENT, "mt_summ_xy: output must be [W,Z,1,1]");
   }
@@ -756,7 +757,7 @@ int mt_add_bias(const mt_tensor *t, const mt_tensor *bias) {
   if (t->z != bias->z) return mt::fail(MT_E_SHAPE, "mt_add_bias: depth of tensor and bias differ");
   uint32_t rows = t->w * t->z, YX = t->y * t->x;
   if (rows == 0 || YX == 0) return MT_OK;
-  if (bias->y != 1 || bias->x != 1) return mt::fail(MT_E_ARGUMENT, "mt_add_bias: bias must be [W,Z,1,1]");
+  if (bias->w == 0 || bias->y != 1 || bias->x != 1) return mt::fail(MT_E_ARGUMENT, "mt_add_bias: bias must be [W,Z,1,1], W >= 1");
   if (YX % 4 == 0 && aligned16(t->p)) {
     dim3 grid4(cdiv(YX / 4, EW_THREADS), plane_blocks(cdiv(YX / 4, EW_THREADS), rows));
     add_bias4_kernel<<<grid4, EW_THREADS, 0, mt::stream()>>>(t->p, bias->p, bias->w, t->z, YX / 4, rows);
@@ -786,6 +787,7 @@ int mt_upsampling(const mt_tensor *out, const mt_tensor *in, uint32_t ux, uint32
   if (in->x != out->x / ux || in->y != out->y / uy || in->z != out->z) return mt::fail(MT_E_SHAPE, "mt_upsampling: sizes do not match");
   uint32_t planes = out->w * out->z, n = out->y * out->x;
   if (planes == 0 || n == 0) return MT_OK;
+  if (in->w == 0) return mt::fail(MT_E_ARGUMENT, "mt_upsampling: empty input");
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
   if (out->x % 4 == 0 && aligned16(out->p)) {
     dim3 grid4(cdiv(n / 4, EW_THREADS), plane_blocks(cdiv(n / 4, EW_THREADS), planes));
@@ -864,11 +866,11 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
                                     const mt_tensor *new_variable, float momentum, float epsilon, int func) {
   if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: unknown function id %d", func);
   if (mt::bad(out) || mt::bad(in) || mt::bad(gamma) || mt::bad(beta)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: null tensor");
-  if (!mt::same_zyx(in, out) || in->w != out->w || !mt::same_zyx(gamma, in) || !mt::same_zyx(beta, in))
+  if (!mt::same_zyx(in, out) || in->w != out->w || !mt::same_zyx(gamma, in) || !mt::same_zyx(beta, in) || gamma->w == 0 || beta->w == 0)
     return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_func: sizes do not match");
   const mt_tensor *stats[5] = {ivar, batch_mean, batch_var, new_mean, new_variable};
   for (auto t : stats)
-    if (t && (mt::bad(t) || !mt::same_zyx(t, in))) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_func: statistics must be [1,Z,Y,X]");
+    if (t && (mt::bad(t) || !mt::same_zyx(t, in) || t->w == 0)) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_func: statistics must be [1,Z,Y,X]");
   if (xhat && (mt::bad(xhat) || !mt::same_zyx(xhat, in) || xhat->w != in->w)) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_func: xhat must match the input");
   size_t S = (size_t)in->z * in->y * in->x;
   uint32_t W = in->w;
@@ -923,7 +925,7 @@ int mt_batchnorm_forward_infer_func(const mt_tensor *out, const mt_tensor *in, c
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_infer_func: null tensor");
   if (!mt::same_zyx(in, out) || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_infer_func: sizes do not match");
   for (int i = 2; i < 6; i++)
-    if (!mt::same_zyx(all[i], in)) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_infer_func: parameters must be [1,Z,Y,X]");
+    if (!mt::same_zyx(all[i], in) || all[i]->w == 0) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_infer_func: parameters must be [1,Z,Y,X]");
   size_t S = (size_t)in->z * in->y * in->x;
   uint32_t W = in->w;
   if (S == 0 || W == 0) return MT_OK;
@@ -946,10 +948,10 @@ int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const
   for (auto t : need)
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: null tensor");
   if (!mt::same_zyx(error, delta) || error->w != delta->w || !mt::same_zyx(xhat, delta) || xhat->w != delta->w || !mt::same_zyx(gamma, delta) ||
-      !mt::same_zyx(ivar, delta))
+      !mt::same_zyx(ivar, delta) || gamma->w == 0 || ivar->w == 0)
     return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: sizes do not match");
   for (auto t : {dgamma, dbeta})
-    if (t && (mt::bad(t) || !mt::same_zyx(t, delta))) return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: gradients must be [1,Z,Y,X]");
+    if (t && (mt::bad(t) || !mt::same_zyx(t, delta) || t->w == 0)) return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: gradients must be [1,Z,Y,X]");
   const size_t S = (size_t)delta->z * delta->y * delta->x;
   const uint32_t W = delta->w;
   if (S == 0 || W == 0) return MT_OK;

@@ -392,6 +392,30 @@ def test_empty_tensors(gpu):
     assert gpu.add(np.zeros((0, 2, 3, 4), np.float32), np.zeros((0, 2, 3, 4), np.float32)).shape == (0, 2, 3, 4)
     assert gpu.fill((2, 0, 3, 4), 1.0).size == 0
     assert gpu.forward_convolution(np.zeros((0, 2, 5, 5), np.float32), U(1, 1, 1, 3, 18), U(2, 1, 3, 1, 1), 3, 3, 2, 3, 1, 1, 1, 1).shape == (0, 3, 5, 5)
+    # no input channels: every output pixel is its bias (a product with an empty k axis)
+    bias = U(2, 1, 3, 1, 1)
+    got = gpu.forward_convolution(np.zeros((2, 0, 5, 5), np.float32), np.zeros((1, 1, 3, 0), np.float32), bias, 3, 3, 0, 3, 1, 1, 1, 1)
+    assert np.array_equal(got, np.broadcast_to(bias, (2, 3, 5, 5)))
+    assert np.array_equal(gpu.mul(np.zeros((1, 1, 4, 0), np.float32), np.zeros((1, 1, 0, 5), np.float32)), np.zeros((1, 1, 4, 5), np.float32))
+
+
+def test_empty_broadcast_operand_is_an_error(gpu):
+    """An operand that broadcasts by w % W needs W >= 1 when the output is not empty: refused on the host, before
+    any kernel would index with it."""
+    import mi355tensor as mt
+    z = np.zeros
+    probes = [
+        lambda: gpu.add_bias(U(1, 2, 3, 4, 4), z((0, 3, 1, 1), np.float32)),
+        lambda: gpu.summ_xy(z((0, 3, 4, 4), np.float32), out_w=2),
+        lambda: gpu.upsampling(z((0, 3, 4, 4), np.float32), 2, 2, out_shape=(2, 3, 8, 8)),
+        lambda: gpu.add(U(1, 2, 3, 4, 4), z((0, 3, 4, 4), np.float32)),
+        lambda: gpu.mul(U(1, 2, 1, 4, 4), z((0, 1, 4, 4), np.float32)),
+        lambda: gpu.forward_convolution(U(1, 1, 2, 5, 5), U(2, 1, 1, 3, 18), z((0, 3, 1, 1), np.float32), 3, 3, 2, 3, 1, 1, 1, 1),
+    ]
+    for i, probe in enumerate(probes):
+        with pytest.raises(mt.TensorError) as e:
+            probe()
+        assert e.value.code == 6, "probe %d" % i
 
 
 # ---- layers: literal op sequences on both back ends, and the fused entry points ----------------
