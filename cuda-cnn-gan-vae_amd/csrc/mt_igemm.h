@@ -394,6 +394,19 @@ struct SrcWgradImage {
   }
   template <int E>
   __device__ void fetch(float (&v)[E]) const {
+    if (OW % E == 0) {  // the E elements are consecutive pixels of one output row (k and ox are multiples of E)
+      const int32_t iy = iy0 + (int32_t)oy * sy;
+      int32_t ix = ix0 + (int32_t)ox * sx;
+      const bool row_ok = k < K && (uint32_t)iy < H;
+      uint32_t off = chanoff + ((uint32_t)iy * W + (uint32_t)ix) * 4u;
+#pragma unroll
+      for (int i = 0; i < E; i++) {
+        v[i] = buf_load(rsrc, row_ok && (uint32_t)ix < W ? off : OOB, woff);
+        ix += sx;
+        off += (uint32_t)sx * 4u;
+      }
+      return;
+    }
     uint32_t yy = oy, xx = ox;
 #pragma unroll
     for (int i = 0; i < E; i++) {
@@ -760,10 +773,13 @@ int launch(const char *name, SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N
 template <class SrcA, class SrcB>
 int launch_split(const char *name, SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, size_t out_floats, uint32_t bias_div, uint32_t bias_mod) {
   const size_t tiles = (size_t)cdiv(M, 64) * cdiv(N, 64);
-  if (tiles >= 128 || K < 512 || out_floats > (1u << 22) || ep.accumulate) return launch(name, a, b, ep, M, N, K, 1);
-  uint32_t want = (uint32_t)(512 / tiles);                       // ranges wanted
+  // up to two blocks per compute unit (one wave per SIMD each) and a long k axis: split down to ranges of 64 steps
+  const bool few = tiles < 128 && K >= 512, thin = tiles >= 128 && tiles <= 512 && K >= 2048;
+  if (!(few || thin) || out_floats > (1u << 22) || ep.accumulate) return launch(name, a, b, ep, M, N, K, 1);
+  uint32_t want = (uint32_t)((few ? 512 : 1024) / tiles);        // ranges wanted
   uint32_t kc = (cdiv(K, want) + BK - 1) / BK * BK;              // range length, a multiple of the k step
   if (kc < 2 * BK) kc = 2 * BK;
+  if (thin && kc < 64 * BK) kc = 64 * BK;
   const uint32_t S = cdiv(K, kc);
   if (S < 2) return launch(name, a, b, ep, M, N, K, 1);
   float *partial = nullptr;
