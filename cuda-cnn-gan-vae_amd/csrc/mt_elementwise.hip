@@ -364,10 +364,13 @@ __global__ __launch_bounds__(EW_THREADS) void max_pooling_backward_kernel(float 
 }
 
 // ---- Adam: fp32 state, update arithmetic in double as on the CPU path ------------------------------------------------
-__global__ __launch_bounds__(EW_THREADS) void adam_kernel(float *weight, const float *dweight, float *m, float *v, size_t n, float batch,
-                                                          double speed, double beta1, double beta2, double epsilon, double c1, double c2) {
-  size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
-  if (i >= n) return;
+struct AdamStep {
+  float batch;
+  double speed, beta1, beta2, epsilon, c1, c2;
+};
+__device__ __forceinline__ void adam_update(float *weight, const float *dweight, float *m, float *v, size_t i, const AdamStep &a) {
+  const float batch = a.batch;
+  const double speed = a.speed, beta1 = a.beta1, beta2 = a.beta2, epsilon = a.epsilon, c1 = a.c1, c2 = a.c2;
   float dw = dweight[i] / batch, mi = m[i], vi = v[i];
   mi = (float)(beta1 * (double)mi + (1.0 - beta1) * (double)dw);
   vi = (float)(beta2 * (double)vi + (1.0 - beta2) * (double)dw * (double)dw);
@@ -377,6 +380,44 @@ __global__ __launch_bounds__(EW_THREADS) void adam_kernel(float *weight, const f
   m[i] = mi;
   v[i] = vi;
   weight[i] = weight[i] - dw;
+}
+__global__ __launch_bounds__(EW_THREADS) void adam_kernel(float *weight, const float *dweight, float *m, float *v, size_t n, AdamStep a) {
+  size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
+  if (i < n) adam_update(weight, dweight, m, v, i, a);
+}
+
+// ---- one launch over several tensors (all gradients of a network, all its parameters) ------------------------------
+// Tensor t owns the blocks first_block[t] .. first_block[t+1]-1, which walk it with a grid stride.
+constexpr int MANY = 32;
+struct ManyFill {
+  float *p[MANY];
+  size_t n[MANY];
+  uint32_t first_block[MANY + 1];
+};
+struct ManyAdam {
+  float *weight[MANY];
+  const float *dweight[MANY];
+  float *m[MANY], *v[MANY];
+  size_t n[MANY];
+  uint32_t first_block[MANY + 1];
+};
+template <class T>
+__device__ __forceinline__ uint32_t many_owner(const T &a, uint32_t count) {
+  uint32_t t = 0;
+  while (t + 1 < count && blockIdx.x >= a.first_block[t + 1]) t++;
+  return t;
+}
+__global__ __launch_bounds__(EW_THREADS) void fill_many_kernel(ManyFill a, uint32_t count, float value) {
+  const uint32_t t = many_owner(a, count);
+  const size_t stride = (size_t)(a.first_block[t + 1] - a.first_block[t]) * EW_THREADS;
+  float *p = a.p[t];
+  for (size_t i = (size_t)(blockIdx.x - a.first_block[t]) * EW_THREADS + threadIdx.x; i < a.n[t]; i += stride) p[i] = value;
+}
+__global__ __launch_bounds__(EW_THREADS) void adam_many_kernel(ManyAdam a, uint32_t count, AdamStep step) {
+  const uint32_t t = many_owner(a, count);
+  const size_t stride = (size_t)(a.first_block[t + 1] - a.first_block[t]) * EW_THREADS;
+  for (size_t i = (size_t)(blockIdx.x - a.first_block[t]) * EW_THREADS + threadIdx.x; i < a.n[t]; i += stride)
+    adam_update(a.weight[t], a.dweight[t], a.m[t], a.v[t], i, step);
 }
 
 // ---- batch normalisation over the batch axis, statistics per element (z,y,x) --------------------------------------
@@ -542,9 +583,12 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
 //   error = ((N*dxhat - xhat*s2) - s1) * ivar * (1/N)            (each step rounded to fp32, in this order)
 // Block layout as bn_fused_kernel.  NW > 0: a thread keeps its NW rows of delta and xhat in registers between the
 // sums and the error; NW == 0: any batch size, the rows are read a second time.
+// func (ReLU or leaky ReLU, else MT_F_NONE): the layer's output went through that function and `delta` is the
+// gradient behind it; the function layer's step delta * f'(gamma*xhat + beta) happens as delta is loaded.
 template <int RB, int NW>
 __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, float *dgamma, float *dbeta, const float *delta, const float *gamma,
-                                                                 const float *xhat, const float *ivar, uint32_t W, uint32_t S, float n, float inv_n) {
+                                                                 const float *beta, const float *xhat, const float *ivar, uint32_t W, uint32_t S, float n,
+                                                                 float inv_n, int func) {
   constexpr int WS = EW_THREADS / RB, HOLD = NW > 0 ? NW : 1;
   __shared__ float part[4][WS][RB * 4];
   __shared__ float col_s1[RB * 4], col_s2[RB * 4];
@@ -552,7 +596,17 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
   const uint32_t r = (blockIdx.x * RB + rl) * 4;
   float4 qd[HOLD], qx[HOLD];
   float acc[4][4] = {};
-  float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 g = make_float4(0.f, 0.f, 0.f, 0.f), bt = g;
+  const float below = func == MT_F_RELU ? 0.f : 0.1f;  // f'(z) for z < 0
+  auto behind = [&](float4 d, const float4 &x) {  // the gradient in front of the function
+    if (func != MT_F_NONE) {
+      d.x = d.x * (((g.x * x.x) + bt.x) >= 0.f ? 1.f : below);
+      d.y = d.y * (((g.y * x.y) + bt.y) >= 0.f ? 1.f : below);
+      d.z = d.z * (((g.z * x.z) + bt.z) >= 0.f ? 1.f : below);
+      d.w = d.w * (((g.w * x.w) + bt.w) >= 0.f ? 1.f : below);
+    }
+    return d;
+  };
   auto add = [&](const float4 &d, const float4 &x) {
     const float dv[4] = {d.x, d.y, d.z, d.w}, xv[4] = {x.x, x.y, x.z, x.w}, gv[4] = {g.x, g.y, g.z, g.w};
 #pragma unroll
@@ -566,6 +620,7 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
   };
   if (r < S) {
     g = *reinterpret_cast<const float4 *>(gamma + r);
+    if (func != MT_F_NONE) bt = *reinterpret_cast<const float4 *>(beta + r);
     if constexpr (NW > 0) {
 #pragma unroll
       for (int i = 0; i < NW; i++) {
@@ -577,11 +632,16 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
       }
 #pragma unroll
       for (int i = 0; i < NW; i++)
-        if (ws + i * WS < W) add(qd[i], qx[i]);
+        if (ws + i * WS < W) {
+          qd[i] = behind(qd[i], qx[i]);
+          add(qd[i], qx[i]);
+        }
     } else {
 #pragma unroll 4
-      for (uint32_t w = ws; w < W; w += WS)
-        add(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r));
+      for (uint32_t w = ws; w < W; w += WS) {
+        const float4 x = *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r);
+        add(behind(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), x), x);
+      }
     }
   }
 #pragma unroll
@@ -622,9 +682,10 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
       *reinterpret_cast<float4 *>(err + (size_t)w * S + r) = error(qd[i], qx[i]);
     }
   } else {
-    for (uint32_t w = ws; w < W; w += WS)
-      *reinterpret_cast<float4 *>(err + (size_t)w * S + r) =
-          error(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r));
+    for (uint32_t w = ws; w < W; w += WS) {
+      const float4 x = *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r);
+      *reinterpret_cast<float4 *>(err + (size_t)w * S + r) = error(behind(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), x), x);
+    }
   }
 }
 
@@ -855,9 +916,62 @@ int mt_adam(const mt_tensor *weight, const mt_tensor *dweight, const mt_tensor *
     if (!mt::same_zyx(weight, t) || weight->w != t->w) return mt::fail(MT_E_SHAPE, "mt_adam: sizes do not match");
   size_t n = mt::count(weight);
   if (n == 0) return MT_OK;
-  double c1 = 1.0 - pow(beta1, iteration), c2 = 1.0 - pow(beta2, iteration);
-  adam_kernel<<<cdiv(n, EW_THREADS), EW_THREADS, 0, mt::stream()>>>(weight->p, dweight->p, m->p, v->p, n, (float)batch_size, speed, beta1, beta2, epsilon, c1, c2);
+  const AdamStep step{(float)batch_size, speed, beta1, beta2, epsilon, 1.0 - pow(beta1, iteration), 1.0 - pow(beta2, iteration)};
+  adam_kernel<<<cdiv(n, EW_THREADS), EW_THREADS, 0, mt::stream()>>>(weight->p, dweight->p, m->p, v->p, n, step);
   MT_LAUNCH_CHECK("mt_adam");
+  return MT_OK;
+}
+
+int mt_fill_many(uint32_t count, const mt_tensor *const *tensors, float value) {
+  if (count && tensors == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_fill_many: null list");
+  for (uint32_t i = 0; i < count; i++)
+    if (mt::bad(tensors[i])) return mt::fail(MT_E_ARGUMENT, "mt_fill_many: null tensor (entry %u)", i);
+  for (uint32_t first = 0; first < count;) {
+    ManyFill a{};
+    uint32_t used = 0;
+    for (; first < count && used < (uint32_t)MANY; first++) {
+      const size_t n = mt::count(tensors[first]);
+      if (n == 0) continue;
+      unsigned blocks = cdiv(n, (size_t)EW_THREADS * 4);  // a few stores per thread
+      if (blocks > 2048u) blocks = 2048u;
+      a.p[used] = tensors[first]->p; a.n[used] = n; a.first_block[used + 1] = a.first_block[used] + blocks;
+      used++;
+    }
+    if (used == 0) continue;
+    mt::ProfileScope prof("mt_fill_many");
+    fill_many_kernel<<<a.first_block[used], EW_THREADS, 0, mt::stream()>>>(a, used, value);
+    MT_LAUNCH_CHECK("mt_fill_many");
+  }
+  return MT_OK;
+}
+
+int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor *const *dweight, const mt_tensor *const *m, const mt_tensor *const *v,
+                 uint32_t batch_size, double speed, double beta1, double beta2, double epsilon, double iteration) {
+  if (count && (weight == nullptr || dweight == nullptr || m == nullptr || v == nullptr)) return mt::fail(MT_E_ARGUMENT, "mt_adam_many: null list");
+  for (uint32_t i = 0; i < count; i++) {
+    if (mt::bad(weight[i]) || mt::bad(dweight[i]) || mt::bad(m[i]) || mt::bad(v[i])) return mt::fail(MT_E_ARGUMENT, "mt_adam_many: null tensor (entry %u)", i);
+    const mt_tensor *o[3] = {dweight[i], m[i], v[i]};
+    for (auto t : o)
+      if (!mt::same_zyx(weight[i], t) || weight[i]->w != t->w) return mt::fail(MT_E_SHAPE, "mt_adam_many: sizes do not match (entry %u)", i);
+  }
+  const AdamStep step{(float)batch_size, speed, beta1, beta2, epsilon, 1.0 - pow(beta1, iteration), 1.0 - pow(beta2, iteration)};
+  for (uint32_t first = 0; first < count;) {
+    ManyAdam a{};
+    uint32_t used = 0;
+    for (; first < count && used < (uint32_t)MANY; first++) {
+      const size_t n = mt::count(weight[first]);
+      if (n == 0) continue;
+      unsigned blocks = cdiv(n, EW_THREADS);
+      if (blocks > 4096u) blocks = 4096u;
+      a.weight[used] = weight[first]->p; a.dweight[used] = dweight[first]->p; a.m[used] = m[first]->p; a.v[used] = v[first]->p;
+      a.n[used] = n; a.first_block[used + 1] = a.first_block[used] + blocks;
+      used++;
+    }
+    if (used == 0) continue;
+    mt::ProfileScope prof("mt_adam_many");
+    adam_many_kernel<<<a.first_block[used], EW_THREADS, 0, mt::stream()>>>(a, used, step);
+    MT_LAUNCH_CHECK("mt_adam_many");
+  }
   return MT_OK;
 }
 
@@ -944,9 +1058,18 @@ int mt_batchnorm_forward_infer_func(const mt_tensor *out, const mt_tensor *in, c
 
 int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
                           const mt_tensor *xhat, const mt_tensor *ivar) {
+  return mt_batchnorm_backward_func(error, dgamma, dbeta, delta, gamma, nullptr, xhat, ivar, MT_F_NONE);
+}
+
+int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
+                               const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func) {
+  if (!mt::valid_func(func, true) || (func != MT_F_NONE && (func & MT_F_DIFFERENTIAL))) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: unknown function id %d", func);
+  if (func == MT_F_LINEAR) func = MT_F_NONE;  // derivative 1
   const mt_tensor *need[5] = {error, delta, gamma, xhat, ivar};
   for (auto t : need)
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: null tensor");
+  if (func != MT_F_NONE && (mt::bad(beta) || !mt::same_zyx(beta, delta) || beta->w == 0))
+    return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: beta must be [1,Z,Y,X] when a function is given");
   if (!mt::same_zyx(error, delta) || error->w != delta->w || !mt::same_zyx(xhat, delta) || xhat->w != delta->w || !mt::same_zyx(gamma, delta) ||
       !mt::same_zyx(ivar, delta) || gamma->w == 0 || ivar->w == 0)
     return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: sizes do not match");
@@ -957,14 +1080,22 @@ int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const
   if (S == 0 || W == 0) return MT_OK;
   const float n = (float)W, inv_n = (float)(1.0 / (double)n);
   float *pg = dgamma ? dgamma->p : nullptr, *pb = dbeta ? dbeta->p : nullptr;
-  const bool vec = S % 4 == 0 && aligned16(error->p) && aligned16(delta->p) && aligned16(gamma->p) && aligned16(xhat->p) && aligned16(ivar->p);
+  const bool cheap = func == MT_F_NONE || func == MT_F_RELU || func == MT_F_LEAKY_RELU;
+  const bool vec = cheap && S % 4 == 0 && aligned16(error->p) && aligned16(delta->p) && aligned16(gamma->p) && aligned16(xhat->p) && aligned16(ivar->p) &&
+                   (func == MT_F_NONE || aligned16(beta->p));
   if (!vec) {
-    // any layout: the layer's own sequence of tensor operations, on workspace tensors
+    // any layout, any function: the layers' own sequences of tensor operations, on workspace tensors
     float *ws = nullptr;
-    int rc = bn_scratch(2 * S + 2 * (size_t)W * S, &ws);
+    int rc = bn_scratch(2 * S + 3 * (size_t)W * S, &ws);
     if (rc) return rc;
     mt_tensor s1{ws, 1, delta->z, delta->y, delta->x}, s2{ws + S, 1, delta->z, delta->y, delta->x};
     mt_tensor dx{ws + 2 * S, W, delta->z, delta->y, delta->x}, t{ws + 2 * S + (size_t)W * S, W, delta->z, delta->y, delta->x};
+    mt_tensor front{ws + 2 * S + 2 * (size_t)W * S, W, delta->z, delta->y, delta->x};
+    if (func != MT_F_NONE) {  // the function layer: delta * f'(gamma*xhat + beta)
+      if ((rc = mt_tensor_item_production(&t, gamma, xhat)) || (rc = mt_add(&t, &t, beta, 1.f, 1.f))) return rc;
+      if ((rc = mt_apply_func(&t, &t, MT_F_DIFFERENTIAL + func)) || (rc = mt_tensor_item_production(&front, delta, &t))) return rc;
+      delta = &front;
+    }
     if ((rc = mt_fill(&s1, 0.f)) || (rc = mt_fill(&s2, 0.f))) return rc;
     if ((rc = mt_tensor_item_production(&dx, delta, gamma)) || (rc = mt_add_sum_w(&s1, &s1, &dx, 1.f, 1.f))) return rc;
     if ((rc = mt_tensor_item_production(&t, &dx, xhat)) || (rc = mt_add_sum_w(&s2, &s2, &t, 1.f, 1.f))) return rc;
@@ -981,7 +1112,8 @@ int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const
   const uint32_t nw = cdiv(W, EW_THREADS / rb);
   const unsigned grid = cdiv(S, (size_t)rb * 4);
 #define MT_BN_BWD(RB, NW) \
-  bn_backward_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(error->p, pg, pb, delta->p, gamma->p, xhat->p, ivar->p, W, (uint32_t)S, n, inv_n)
+  bn_backward_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(error->p, pg, pb, delta->p, gamma->p, beta ? beta->p : nullptr, xhat->p, ivar->p, W, \
+                                                                    (uint32_t)S, n, inv_n, func)
 #define MT_BN_BWD_NW(RB) \
   do { if (nw <= 4) MT_BN_BWD(RB, 4); else if (nw <= 8) MT_BN_BWD(RB, 8); else if (nw <= 16) MT_BN_BWD(RB, 16); else MT_BN_BWD(RB, 0); } while (0)
   if (rb == 32) MT_BN_BWD_NW(32); else if (rb == 16) MT_BN_BWD_NW(16); else MT_BN_BWD_NW(8);

@@ -100,12 +100,12 @@ class Discriminator:
         for i in range(4):
             cin, cout = CHANNELS[i], CHANNELS[i + 1]
             CTensorConv.ForwardConvolution(self.c[i], h, p["kernel%d" % i], 4, 4, cin, cout, p["bias%d" % i], 2, 2, 1, 1)
-            if fused:
-                Fused.BatchNormForwardTrain(self.bn[i], self.c[i], p["gamma%d" % i], p["beta%d" % i], self.xhat[i], self.ivar[i],
-                                            momentum=MOMENTUM, epsilon=BN_EPSILON)
+            if fused:  # batch norm and the function layer behind it in one pass
+                Fused.BatchNormForwardTrain(self.a[i], self.c[i], p["gamma%d" % i], p["beta%d" % i], self.xhat[i], self.ivar[i],
+                                            momentum=MOMENTUM, epsilon=BN_EPSILON, func="leaky_relu")
             else:
                 self._batchnorm_literal(i)
-            CTensorApplyFunc.ApplyLeakyReLU(self.a[i], self.bn[i])
+                CTensorApplyFunc.ApplyLeakyReLU(self.a[i], self.bn[i])
             h = self.a[i]
         flat = h.reinterpret(self.batch, 1, CHANNELS[4] * 16, 1)
         if fused:
@@ -136,9 +136,11 @@ class Discriminator:
 
     # ---- backward ------------------------------------------------------------------------------------------
     def backward(self, fused=False):
-        """fused: the batch-norm backward pass as one kernel and the batch-summed weight gradient as one product,
-        instead of the layers' sequences of tensor operations."""
+        """fused: function and batch-norm backward as one kernel, the batch-summed weight gradient as one product and
+        one launch that zeroes every gradient, instead of the layers' sequences of tensor operations."""
         b, p, g = self.batch, self.p, self.g
+        if fused:
+            Fused.FillMany([g[k] for k in g if k != "lin_w"], 0.0)      # lin_w is written, not accumulated
         CTensorMath.Sub(self.err, self.prob, self.labels)
         CTensorApplyFunc.ApplyDifferentialSigmoid(self.d_logit, self.logit)
         CTensorMath.TensorItemProduction(self.d_logit, self.err, self.d_logit)
@@ -153,24 +155,24 @@ class Discriminator:
             CTensorMath.Mul(self.tmp_dw, self.d_logit, self.a[3].reinterpret(b, 1, 1, CHANNELS[4] * 16))
             CTensorMath.Fill(g["lin_w"], 0.0)
             CTensorMath.AddSumW(g["lin_w"], g["lin_w"], self.tmp_dw)
-        CTensorMath.Fill(g["lin_b"], 0.0)
+        if not fused:
+            CTensorMath.Fill(g["lin_b"], 0.0)
         CTensorMath.AddSumW(g["lin_b"], g["lin_b"], self.d_logit)
         for i in (3, 2, 1, 0):
             cin, cout = CHANNELS[i], CHANNELS[i + 1]
-            # function layer
-            CTensorApplyFunc.ApplyDifferentialLeakyReLU(self.d_bn[i], self.bn[i])
-            CTensorMath.TensorItemProduction(self.d_bn[i], self.d_a[i], self.d_bn[i])
-            if fused:
-                CTensorMath.Fill(g["gamma%d" % i], 0.0)
-                CTensorMath.Fill(g["beta%d" % i], 0.0)
-                Fused.BatchNormBackward(self.d_c[i], g["gamma%d" % i], g["beta%d" % i], self.d_bn[i], p["gamma%d" % i], self.xhat[i], self.ivar[i])
+            if fused:  # function layer and batch norm
+                Fused.BatchNormBackward(self.d_c[i], g["gamma%d" % i], g["beta%d" % i], self.d_a[i], p["gamma%d" % i], self.xhat[i], self.ivar[i],
+                                        beta=p["beta%d" % i], func="leaky_relu")
             else:
+                CTensorApplyFunc.ApplyDifferentialLeakyReLU(self.d_bn[i], self.bn[i])
+                CTensorMath.TensorItemProduction(self.d_bn[i], self.d_a[i], self.d_bn[i])
                 self._batchnorm_backward(i)
             # convolution layer
             inp, prev = (self.a[i - 1], self.d_a[i - 1]) if i else (self.x, self.d_x)
             CTensorConv.BackwardConvolution(prev, self.d_c[i], p["kernel%d" % i], 4, 4, cin, cout, self.zero_bias[i], 2, 2, 1, 1)
-            CTensorMath.Fill(g["kernel%d" % i], 0.0)
-            CTensorMath.Fill(g["bias%d" % i], 0.0)
+            if not fused:
+                CTensorMath.Fill(g["kernel%d" % i], 0.0)
+                CTensorMath.Fill(g["bias%d" % i], 0.0)
             if fused:
                 Fused.ConvolutionBackwardWeightsSum(g["kernel%d" % i], 4, 4, cin, cout, g["bias%d" % i], inp, self.d_c[i], 2, 2, 1, 1)
                 continue
@@ -205,12 +207,17 @@ class Discriminator:
         CTensorMath.Mul(out, out, float(np.float32(1.0 / np.float64(n))))
 
     # ---- optimiser ------------------------------------------------------------------------------------------
-    def update(self, speed=2e-4, beta1=0.5, beta2=0.999, epsilon=1e-8):
+    def update(self, speed=2e-4, beta1=0.5, beta2=0.999, epsilon=1e-8, fused=False):
         self.iteration += 1
+        if fused:
+            keys = list(self.p)
+            Fused.AdamMany([self.p[k] for k in keys], [self.g[k] for k in keys], [self.m[k] for k in keys], [self.v[k] for k in keys],
+                           self.batch, speed, beta1, beta2, epsilon, float(self.iteration))
+            return
         for k in self.p:
             CTensorMath.Adam(self.p[k], self.g[k], self.m[k], self.v[k], self.batch, speed, beta1, beta2, epsilon, float(self.iteration))
 
     def step(self, fused=False):
         self.forward(fused)
         self.backward(fused)
-        self.update()
+        self.update(fused=fused)

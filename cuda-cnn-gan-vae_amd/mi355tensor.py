@@ -206,6 +206,12 @@ def _d(t):
     return t.ref()
 
 
+def _list(tensors):
+    """Array of descriptor pointers for the entry points that take several tensors."""
+    descs = [t.ref() and t._desc for t in tensors]
+    return (C.POINTER(MtTensor) * len(descs))(*[C.pointer(d) for d in descs])
+
+
 def _i(v):
     return C.c_int32(int(v))
 
@@ -381,9 +387,22 @@ class Fused:
         call("mt_vae_coder_output", _d(out), _d(kl_loss) if kl_loss is not None else None, _d(mu), _d(logvar), _d(epsilon))
 
     @staticmethod
-    def BatchNormBackward(error, dgamma, dbeta, delta, gamma, xhat, ivar):
+    def BatchNormBackward(error, dgamma, dbeta, delta, gamma, xhat, ivar, beta=None, func=None):
+        """func: the function the forward pass applied to gamma*xhat+beta (`delta` is the gradient behind it)."""
         opt = lambda t: _d(t) if t is not None else None
-        call("mt_batchnorm_backward", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), _d(xhat), _d(ivar))
+        if func is None:
+            call("mt_batchnorm_backward", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), _d(xhat), _d(ivar))
+        else:
+            call("mt_batchnorm_backward_func", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), opt(beta), _d(xhat), _d(ivar), C.c_int(FUNC[func]))
+
+    @staticmethod
+    def FillMany(tensors, value):
+        call("mt_fill_many", _u(len(tensors)), _list(tensors), _f(value))
+
+    @staticmethod
+    def AdamMany(weights, dweights, ms, vs, batch_size, speed, beta1, beta2, epsilon, iteration):
+        call("mt_adam_many", _u(len(weights)), _list(weights), _list(dweights), _list(ms), _list(vs), _u(batch_size), C.c_double(speed),
+             C.c_double(beta1), C.c_double(beta2), C.c_double(epsilon), C.c_double(iteration))
 
     @staticmethod
     def ConvolutionBackwardWeightsSum(dkernel, dkernel_x, dkernel_y, dkernel_z, dkernel_amount, dbias, image, delta, stride_x, stride_y, padding_x, padding_y):

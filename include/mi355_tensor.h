@@ -177,12 +177,25 @@ int mt_vae_coder_output(const mt_tensor *output, const mt_tensor *kl_loss, const
  * `error` may be the same tensor as `delta`. */
 int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta,
                           const mt_tensor *gamma, const mt_tensor *xhat, const mt_tensor *ivar);
+/* The same behind a function layer (CNetLayerFunction::SetOutputError, netlayer/cnetlayerfunction.cu.h:347-358, then the
+ * sequence above): `delta` is the gradient of func(gamma*xhat+beta) as the forward pass wrote it with that `func`; it is
+ * multiplied by f'(gamma*xhat+beta) on the way in.  `beta` [1,Z,Y,X] is needed unless func is MT_F_NONE / MT_F_LINEAR. */
+int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta,
+                               const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func);
 /* CNetLayerConvolution::TrainingBackward, netlayer/cnetlayerconvolution.cu.h:501-508, without the per-sample round trip:
  * dkernel [1,1,Kamt,C*Ky*Kx] += sum over the batch of the per-sample weight gradients (CreateDeltaWeightAndBias into a
  * zeroed batch tensor, then AddSumW), dbias [1,Kamt,1,1] += sum over the batch and the pixels of delta. */
 int mt_convolution_backward_weights_sum(const mt_tensor *dkernel, int32_t dkernel_x, int32_t dkernel_y, int32_t dkernel_z,
                                         uint32_t dkernel_amount, const mt_tensor *dbias, const mt_tensor *image,
                                         const mt_tensor *delta, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y);
+
+/* TrainingResetDeltaWeight of every layer of a network (netlayer/cnetlayerconvolution.cu.h:522-526 and the same
+ * function of the other layers) as one launch: Fill(tensors[i], value) for i < count. */
+int mt_fill_many(uint32_t count, const mt_tensor *const *tensors, float value);
+/* TrainingUpdateWeight of every layer in Adam mode (netlayer/cnetlayerconvolution.cu.h:533-539 and the same function of
+ * the other layers) as one launch: mt_adam on (weight[i], dweight[i], m[i], v[i]) for i < count, same arithmetic. */
+int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor *const *dweight, const mt_tensor *const *m,
+                 const mt_tensor *const *v, uint32_t batch_size, double speed, double beta1, double beta2, double epsilon, double iteration);
 
 /* ---- timing: replaces CCUDATimeSpent / CTimeStamp (cuda/ccudatimespent.cu:38-52, cuda/ctimestamp.cu:17-32) ----
  * While enabled, every kernel launch of the hot path is bracketed by two events on the work stream and its

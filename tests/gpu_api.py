@@ -198,11 +198,21 @@ class Gpu:
             res["new_mean"], res["new_var"] = nm.numpy(), nv.numpy()
         return res
 
-    def batchnorm_backward(self, delta, gamma, xhat, ivar, dgamma0, dbeta0):
+    def batchnorm_backward(self, delta, gamma, xhat, ivar, dgamma0, dbeta0, beta=None, func=None):
         delta = np.asarray(delta, np.float32)
         err, dg, db = CTensor(*delta.shape), up(dgamma0), up(dbeta0)
-        Fused.BatchNormBackward(err, dg, db, up(delta), up(gamma), up(xhat), up(ivar))
+        Fused.BatchNormBackward(err, dg, db, up(delta), up(gamma), up(xhat), up(ivar), beta=up(beta) if beta is not None else None, func=func)
         return err.numpy(), dg.numpy(), db.numpy()
+
+    def fill_many(self, arrays, value):
+        ts = [up(a) for a in arrays]
+        Fused.FillMany(ts, value)
+        return [t.numpy() for t in ts]
+
+    def adam_many(self, weights, dweights, ms, vs, batch_size, speed, beta1, beta2, epsilon, iteration):
+        w, dw, m, v = ([up(a) for a in group] for group in (weights, dweights, ms, vs))
+        Fused.AdamMany(w, dw, m, v, batch_size, speed, beta1, beta2, epsilon, iteration)
+        return [t.numpy() for t in w], [t.numpy() for t in m], [t.numpy() for t in v]
 
     def vae_coder_output(self, mu, logvar, epsilon):
         mu = np.asarray(mu, np.float32)

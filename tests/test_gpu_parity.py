@@ -278,7 +278,9 @@ def test_fused_conv_activation(gpu, oracle, path):
 @pytest.mark.parametrize("m,k,n,wl,wr,z", [(1, 1, 1, 1, 1, 1), (33, 65, 31, 1, 3, 2), (64, 100, 1, 1, 5, 1), (70, 32, 96, 2, 2, 1), (5, 300, 7, 3, 1, 1),
                                            (200, 77, 150, 1, 4, 1), (130, 260, 1, 1, 70, 1), (96, 40, 1, 1, 1, 1), (17, 9, 40, 4, 4, 3),
                                            # few output tiles and a long k axis: the product is split over k
-                                           (1, 8192, 1, 1, 128, 1), (70, 1000, 3, 1, 4, 1), (33, 650, 20, 5, 1, 1), (128, 2052, 1, 1, 64, 1)])
+                                           (1, 8192, 1, 1, 128, 1), (70, 1000, 3, 1, 4, 1), (33, 650, 20, 5, 1, 1), (128, 2052, 1, 1, 64, 1),
+                                           # one block per compute unit and a long k axis: split as well
+                                           (512, 2048, 1024, 1, 1, 1)])
 def test_products(gpu, oracle, m, k, n, wl, wr, z):
     a, b, at = U(1, wl, z, m, k), U(2, wr, z, k, n), U(3, wl, z, k, m)
     close(gpu.mul(a, b), oracle.mul(a, b), 1e-5)
@@ -482,6 +484,46 @@ def test_batchnorm_backward_fused(gpu, oracle, shape):
     assert np.max(np.abs(err - want_err)) <= 1e-5 * max(scale, np.abs(want_err).max())
     close(dg - dg0, want_dg, 1e-5)
     close(db - db0, want_db, 1e-5)
+
+
+@pytest.mark.parametrize("shape", [(16, 3, 6, 6), (5, 2, 3, 3), (130, 4, 8, 8), (300, 1, 4, 8)])
+@pytest.mark.parametrize("func", ["leaky_relu", "relu", "linear", "tangence"])
+def test_batchnorm_backward_behind_a_function(gpu, oracle, shape, func):
+    """Function layer and batch-norm layer backward in one call: delta * f'(gamma*xhat + beta) first
+    (cnetlayerfunction.cu.h:347-358), then the batch-norm sequence; ReLU-like functions inside the kernel, the others
+    (and layouts the kernel does not take) through the library's own op-by-op path."""
+    x, gamma, beta = Nrm(1, *shape) * 1.5 + 0.3, U(2, 1, *shape[1:]) + 1.5, U(3, 1, *shape[1:])
+    fwd = seq.batchnorm_forward_train(oracle, x, gamma, beta)
+    error = U(4, *shape)
+    delta = seq.function_backward(oracle, error, fwd["out"], func)
+    want_err, want_dg, want_db = seq.batchnorm_backward(oracle, delta, gamma, fwd["xhat"], fwd["ivar"])
+    zero = np.zeros((1,) + shape[1:], np.float32)
+    err, dg, db = gpu.batchnorm_backward(error, gamma, fwd["xhat"], fwd["ivar"], zero, zero, beta=beta, func=func)
+    scale = np.abs(delta * gamma).max() * np.abs(fwd["ivar"]).max()
+    assert np.max(np.abs(err - want_err)) <= 1e-5 * max(scale, np.abs(want_err).max())
+    close(dg, want_dg, 1e-5)
+    close(db, want_db, 1e-5)
+
+
+def test_fill_and_adam_over_many_tensors(gpu, oracle):
+    """One launch over a list of tensors against the single-tensor operations: bit-identical (same arithmetic per
+    element); 40 tensors need two launches, sizes from one element to beyond one block's stride."""
+    shapes = [(1, 1, 1, 1), (1, 1, 64, 48), (1, 64, 1, 1), (2, 3, 5, 7), (1, 1, 128, 1024), (1, 1, 3, 700001)] + [(1, 1, i + 1, 3) for i in range(34)]
+    arrays = [U(10 + i, *sh) for i, sh in enumerate(shapes)]
+    for got, a in zip(gpu.fill_many(arrays, 0.25), arrays):
+        assert got.shape == a.shape and np.all(got == np.float32(0.25))
+    w, dw = arrays, [U(100 + i, *sh) * 30 for i, sh in enumerate(shapes)]
+    m, v = [U(200 + i, *sh) * 0.2 for i, sh in enumerate(shapes)], [np.abs(U(300 + i, *sh)) * 0.05 for i, sh in enumerate(shapes)]
+    got_w, got_m, got_v = gpu.adam_many(w, dw, m, v, 32, 1e-3, 0.9, 0.999, 1e-8, 3.0)
+    for i in range(len(shapes)):
+        one = gpu.adam(w[i], dw[i], m[i], v[i], 32, 1e-3, 0.9, 0.999, 1e-8, 3.0)
+        assert np.array_equal(got_w[i], one[0]) and np.array_equal(got_m[i], one[1]) and np.array_equal(got_v[i], one[2]), i
+    small = slice(0, 4)
+    want = [oracle.adam(w[i], dw[i], m[i], v[i], 32, 1e-3, 0.9, 0.999, 1e-8, 3.0) for i in range(4)]
+    for i in range(4):
+        assert np.array_equal(got_m[i], want[i][1]) and np.array_equal(got_v[i], want[i][2])
+        close(got_w[i], want[i][0], 1e-6)
+    assert gpu.fill_many([], 1.0) == []
 
 
 def test_vae_coder_output(gpu, oracle):
