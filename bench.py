@@ -193,6 +193,79 @@ def discriminator_step(args):
         "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}}))
 
 
+def secondary_forward(args):
+    """Secondary workloads configs[0], configs[1], configs[3]: one forward pass per step, recorded once as a HIP graph
+    and replayed (the steps are a few short kernels); the same two timed regions as the main workload."""
+    import numpy as np
+    import mi355tensor as mt
+    from mi355tensor import CTensor, CTensorConv, Fused
+    mt.init(0)
+    rng = np.random.default_rng({"c1": 1, "c2": 2, "c4": 4}[args.workload])
+    if args.workload == "c1":
+        batch, name = 16, "configs[0]: one convolution layer, batch 16: 3x64x64 -> 32 filters 5x5 stride 1 padding 2, leaky ReLU"
+        image = CTensor.from_numpy(rng.uniform(-1, 1, (16, 3, 64, 64)).astype(np.float32))
+        kernel = CTensor.from_numpy((rng.standard_normal((1, 1, 32, 75)) * np.sqrt(2.0 / 75)).astype(np.float32))
+        bias, out = CTensor.from_numpy(np.zeros((1, 32, 1, 1), np.float32)), CTensor(16, 32, 64, 64)
+        flop = {"conv": 2.0 * 16 * 32 * 64 * 64 * 75}
+        step = lambda: CTensorConv.ForwardConvolution(out, image, kernel, 5, 5, 3, 32, bias, 1, 1, 2, 2, func="leaky_relu")
+    elif args.workload == "c2":
+        batch, name = 256, "configs[1]: Linear 4096 -> 3072, ReLU, Linear 3072 -> 768, batch 256"
+        x = CTensor.from_numpy(rng.standard_normal((256, 1, 4096, 1)).astype(np.float32))
+        w1 = CTensor.from_numpy(rng.uniform(-1, 1, (1, 1, 3072, 4096)).astype(np.float32) * np.float32(np.sqrt(6 / 7168)))
+        w2 = CTensor.from_numpy(rng.uniform(-1, 1, (1, 1, 768, 3072)).astype(np.float32) * np.float32(np.sqrt(6 / 3840)))
+        b1, b2 = CTensor.from_numpy(np.full((1, 1, 3072, 1), 0.1, np.float32)), CTensor.from_numpy(np.full((1, 1, 768, 1), 0.1, np.float32))
+        h, out = CTensor(256, 1, 3072, 1), CTensor(256, 1, 768, 1)
+        flop = {"linear": 2.0 * 256 * (4096 * 3072 + 3072 * 768)}
+
+        def step():
+            Fused.LinearForward(h, w1, x, b1, "relu")
+            Fused.LinearForward(out, w2, h, b2)
+    else:
+        import vae
+        batch, name = 64, ("configs[3]: VAE forward, batch 64: conv 3x3 s2 p1 3->32->64->128->256 with BN + leaky ReLU, Linear 16384->128 x2, "
+                           "reparameterisation + KL, Linear 128->16384, transposed conv 4x4 s2 p1 256->128->64->32->3, sigmoid")
+        net = vae.Vae(batch)
+        net.set_batch(*vae.make_batch(batch))
+        flop = vae.flops(batch)
+        step = net.forward
+    stream = mt.get_stream()
+    create, record, elapsed_ms = hip_events()
+    for _ in range(max(args.warmup, 1)):
+        step()
+    mt.synchronize()
+    graph = mt.Graph(step)
+    for _ in range(3):
+        graph.launch()
+    mt.synchronize()
+    e0, e1 = create(), create()
+    t0 = time.perf_counter()
+    record(e0, stream)
+    for _ in range(args.steps):
+        graph.launch()
+    record(e1, stream)
+    mt.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = elapsed_ms(e0, e1)
+    mt.profile_enable(True)
+    for _ in range(args.steps):
+        step()
+    prof = mt.profile_report()
+    mt.profile_enable(False)
+    ms_per_step = max(gpu_ms, wall_ms) / args.steps
+    kernel_ms = sum(v[1] for v in prof.values()) / args.steps
+    total = sum(flop.values())
+    print(json.dumps({
+        "metric": "images/sec, forward fp32 (secondary workload)" if args.workload != "c2" else "samples/sec, forward fp32 (secondary workload)",
+        "value": batch / (ms_per_step * 1e-3), "unit": "images/s" if args.workload != "c2" else "samples/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic", "config": {"workload": name, "global_batch": batch, "path": "fused C-ABI entry points, step replayed as a HIP graph"},
+        "gpu_ms_per_step_events": gpu_ms / args.steps, "host_ms_per_step_wall": wall_ms / args.steps, "kernel_ms_per_step_sum": kernel_ms,
+        "gflop_per_step": {k: v / 1e9 for k, v in flop.items()},
+        "tflops_over_the_step": total / (ms_per_step * 1e-3) / 1e12,
+        "frac_of_fp32_mfma_peak_over_the_step": total / (ms_per_step * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+        "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -206,9 +279,10 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="time region 1 as replays of the step recorded once as a HIP graph (c5 does so by default: its step "
                          "is about a hundred short kernels and the Python host would be the bottleneck)")
-    ap.add_argument("--workload", choices=["c3", "c5", "ops"], default="c3",
+    ap.add_argument("--workload", choices=["c3", "c5", "ops", "c1", "c2", "c4"], default="c3",
                     help="c3 (default, the measured configuration): DCGAN-64 generator forward, batch 256; "
                          "c5 (secondary): DCGAN-64 discriminator training step, batch 128; "
+                         "c1, c2, c4 (secondary): one convolution layer at batch 16, a two-layer MLP at batch 256, the VAE forward at batch 64; "
                          "ops (secondary): every HBM-bound tensor operation on a [256,64,32,32] activation, GB/s each")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -217,6 +291,8 @@ def main():
         return discriminator_step(args)
     if args.workload == "ops":
         return memory_bound_ops(args)
+    if args.workload in ("c1", "c2", "c4"):
+        return secondary_forward(args)
 
     import mi355tensor as mt
     import generator as G

@@ -212,27 +212,9 @@ def test_shipped_gan_generator_topology(gpu, oracle):
     assert got["image"].shape == (b, 3, 192, 256) and rel_err(got["image"], want["image"]) <= 2e-3
 
 
-def vae_parameters(latent=128, seed=4):
-    rng = np.random.default_rng(seed)
-    p, size = {}, 128
-    for i in range(4):
-        cin, cout = seq.VAE_ENCODER[i], seq.VAE_ENCODER[i + 1]
-        size //= 2
-        p["ekernel%d" % i] = (rng.standard_normal((1, 1, cout, cin * 9)) * np.sqrt(2.0 / (cin * 9))).astype(np.float32)
-        p["ebias%d" % i] = (rng.standard_normal((1, cout, 1, 1)) * 0.05).astype(np.float32)
-        p["egamma%d" % i] = rng.uniform(0.5, 1.5, (1, cout, size, size)).astype(np.float32)
-        p["ebeta%d" % i] = rng.uniform(-0.2, 0.2, (1, cout, size, size)).astype(np.float32)
-    flat = 256 * 8 * 8
-    for head in ("mu", "lv"):
-        p[head + "_w"] = (rng.standard_normal((1, 1, latent, flat)) / np.sqrt(flat)).astype(np.float32)
-        p[head + "_b"] = np.full((1, 1, latent, 1), 0.1, np.float32)
-    p["dec_w"] = (rng.standard_normal((1, 1, flat, latent)) / np.sqrt(latent)).astype(np.float32)
-    p["dec_b"] = np.full((1, 1, flat, 1), 0.1, np.float32)
-    for i in range(4):
-        cin, cout = seq.VAE_DECODER[i], seq.VAE_DECODER[i + 1]
-        p["dkernel%d" % i] = (rng.standard_normal((1, 1, cin, cout * 16)) * np.sqrt(1.0 / (cin * 4))).astype(np.float32)
-        p["dbias%d" % i] = np.zeros((1, cin, 1, 1), np.float32)
-    return p
+def vae_parameters():
+    import vae
+    return vae.make_parameters()
 
 
 def test_config4_vae_against_oracle(gpu, oracle):
@@ -260,6 +242,29 @@ def test_config4_vae_against_oracle(gpu, oracle):
     # the encoder end to end on the device
     got = seq.vae_encoder_forward(gpu, params, x)
     assert rel_err(got["mu"], want["mu"]) <= 2e-3 and rel_err(got["logvar"], want["logvar"]) <= 2e-3
+
+
+def test_config4_device_resident_model(gpu, oracle):
+    """vae.Vae (every tensor on the device, fused entry points) at batch 4: latent statistics against the oracle's
+    encoder, the latent against the closed form on the device's own statistics, the decoder against the oracle's
+    decoder fed with the device's latent."""
+    import vae
+    params = vae.make_parameters()
+    x, eps = vae.make_batch(4)
+    net = vae.Vae(4, params)
+    net.set_batch(x, eps)
+    out = net.forward().numpy()
+    want = seq.vae_encoder_forward(oracle, params, x)
+    for i in range(4):   # four batch norms over four samples amplify rounding from layer to layer
+        assert rel_err(net.eh[i].numpy(), want["eh%d" % i]) <= 2e-3, "encoder stage %d" % i
+    mu, logvar = net.mu.numpy(), net.logvar.numpy()
+    assert rel_err(mu, want["mu"]) <= 2e-3 and rel_err(logvar, want["logvar"]) <= 2e-3
+    z, kl = oracle.vae_coder_output(mu, logvar, eps)
+    assert rel_err(net.z.numpy(), z) <= 1e-6 and abs(float(net.kl.numpy().ravel()[0]) - kl) <= 1e-5 * abs(kl)
+    dwant = seq.vae_decoder_forward(oracle, params, net.z.numpy())
+    for i in range(5):
+        assert rel_err(net.dh[i].numpy(), dwant["dh%d" % i]) <= REL, "decoder stage %d" % i
+    assert out.shape == (4, 3, 128, 128) and np.all((out > 0) & (out < 1))
 
 
 def test_config4_full_batch_properties(gpu, oracle):
