@@ -200,7 +200,7 @@ def secondary_forward(args):
     import mi355tensor as mt
     from mi355tensor import CTensor, CTensorConv, Fused
     mt.init(0)
-    rng = np.random.default_rng({"c1": 1, "c2": 2, "c4": 4}[args.workload])
+    rng = np.random.default_rng({"c1": 1, "c2": 2, "c4": 4, "gan": 6}[args.workload])
     if args.workload == "c1":
         batch, name = 16, "configs[0]: one convolution layer, batch 16: 3x64x64 -> 32 filters 5x5 stride 1 padding 2, leaky ReLU"
         image = CTensor.from_numpy(rng.uniform(-1, 1, (16, 3, 64, 64)).astype(np.float32))
@@ -220,6 +220,19 @@ def secondary_forward(args):
         def step():
             Fused.LinearForward(h, w1, x, b1, "relu")
             Fused.LinearForward(out, w2, h, b2)
+    elif args.workload == "gan":
+        import gan_generator as GG
+        batch, name = GG.BATCH, ("the reference's shipped GAN generator (cmodel_gan.cu.h), batch 32: Linear 1024 -> 3*4*512, six times (up-sampling x2, "
+                                 "conv 3x3, BN, leaky ReLU) 512 -> 512 -> 256 -> 128 -> 64 -> 32 -> 16, conv 3x3 -> 3, tanh: 192x256 images; "
+                                 + ("layer by layer" if args.literal else "up-sampling + convolution in one call"))
+        net = GG.GanGenerator(batch)
+        net.set_noise(GG.make_noise(batch))
+        layers = GG.conv_flops(batch)
+        # the one-call path multiplies 4 taps per output pixel where the layers multiply 9 (sums of coefficients)
+        executed = sum(layers) if args.literal else sum(layers[:6]) * 4.0 / 9.0 + layers[6]
+        flop = {"conv_executed": executed, "linear": 2.0 * batch * 1024 * 6144}
+        extra = {"conv_gflop_as_the_layers_count_it": sum(layers) / 1e9}
+        step = (lambda: net.forward(False)) if args.literal else (lambda: net.forward(True))
     else:
         import vae
         batch, name = 64, ("configs[3]: VAE forward, batch 64: conv 3x3 s2 p1 3->32->64->128->256 with BN + leaky ReLU, Linear 16384->128 x2, "
@@ -228,6 +241,8 @@ def secondary_forward(args):
         net.set_batch(*vae.make_batch(batch))
         flop = vae.flops(batch)
         step = net.forward
+    if args.workload != "gan":
+        extra = {}
     stream = mt.get_stream()
     create, record, elapsed_ms = hip_events()
     for _ in range(max(args.warmup, 1)):
@@ -260,7 +275,7 @@ def secondary_forward(args):
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic", "config": {"workload": name, "global_batch": batch, "path": "fused C-ABI entry points, step replayed as a HIP graph"},
         "gpu_ms_per_step_events": gpu_ms / args.steps, "host_ms_per_step_wall": wall_ms / args.steps, "kernel_ms_per_step_sum": kernel_ms,
-        "gflop_per_step": {k: v / 1e9 for k, v in flop.items()},
+        "gflop_per_step": dict({k: v / 1e9 for k, v in flop.items()}, **extra),
         "tflops_over_the_step": total / (ms_per_step * 1e-3) / 1e12,
         "frac_of_fp32_mfma_peak_over_the_step": total / (ms_per_step * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
         "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}}))
@@ -279,10 +294,12 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="time region 1 as replays of the step recorded once as a HIP graph (c5 does so by default: its step "
                          "is about a hundred short kernels and the Python host would be the bottleneck)")
-    ap.add_argument("--workload", choices=["c3", "c5", "ops", "c1", "c2", "c4"], default="c3",
+    ap.add_argument("--literal", action="store_true", help="workload gan: up-sampling and convolution as two layers")
+    ap.add_argument("--workload", choices=["c3", "c5", "ops", "c1", "c2", "c4", "gan"], default="c3",
                     help="c3 (default, the measured configuration): DCGAN-64 generator forward, batch 256; "
                          "c5 (secondary): DCGAN-64 discriminator training step, batch 128; "
                          "c1, c2, c4 (secondary): one convolution layer at batch 16, a two-layer MLP at batch 256, the VAE forward at batch 64; "
+                         "gan (secondary): the reference's shipped GAN generator at batch 32 (--literal: up-sampling and convolution as two layers); "
                          "ops (secondary): every HBM-bound tensor operation on a [256,64,32,32] activation, GB/s each")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -291,7 +308,7 @@ def main():
         return discriminator_step(args)
     if args.workload == "ops":
         return memory_bound_ops(args)
-    if args.workload in ("c1", "c2", "c4"):
+    if args.workload in ("c1", "c2", "c4", "gan"):
         return secondary_forward(args)
 
     import mi355tensor as mt

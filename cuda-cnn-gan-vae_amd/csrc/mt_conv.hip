@@ -1077,6 +1077,98 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
   return dbias_batch_sum(name, db->p, dbias_partial, delta->p, B, ka, DHW, chunks);
 }
 
+// ---- nearest-neighbour up-sampling x2 followed by a 3x3 convolution (stride 1, padding 1), without the up-sampled image --
+// Output row 2q reads up-sampled rows 2q-1, 2q, 2q+1 = input rows q-1, q, q; output row 2q+1 reads input rows q, q, q+1.
+// So each of the four output phases (row parity, column parity) is a 2x2 convolution of the input itself, with
+// coefficients that are sums of the 3x3 ones: 4 taps instead of 9, and the up-sampled image (four times the input)
+// is neither written nor read.  This is the phase structure of a transposed convolution 4x4 stride 2 padding 1, so the
+// same kernel runs it.  Rows outside the up-sampled image are rows outside the input: the zero padding carries over.
+// One thread per (co, ci): packed[phase][co][ci*4 + ty*2 + tx] = sum of w[co][ci][ky][kx] over ky in Y(phase_y, ty),
+// kx in X(phase_x, tx), with  (parity 0: tap 0 = {0}, tap 1 = {1, 2};  parity 1: tap 0 = {0, 1}, tap 1 = {2}).
+__global__ __launch_bounds__(256) void upconv_prepare_kernel(float *packed, const float *kernel, uint32_t ker_ld, uint32_t CO, uint32_t CI) {
+  const uint32_t ci = blockIdx.x * 256 + threadIdx.x, co = blockIdx.y;
+  if (ci >= CI) return;
+  float w[3][3];
+#pragma unroll
+  for (int i = 0; i < 9; i++) w[i / 3][i % 3] = kernel[(size_t)co * ker_ld + ci * 9 + i];
+  // rows summed per (parity, tap): r[parity][tap][kx]
+  float r[2][2][3];
+#pragma unroll
+  for (int x = 0; x < 3; x++) {
+    r[0][0][x] = w[0][x]; r[0][1][x] = w[1][x] + w[2][x];
+    r[1][0][x] = w[0][x] + w[1][x]; r[1][1][x] = w[2][x];
+  }
+  const uint32_t ld = CI * 4;
+#pragma unroll
+  for (int py = 0; py < 2; py++)
+#pragma unroll
+    for (int px = 0; px < 2; px++) {
+      float4 q;
+      const float(&a)[3] = r[py][0], (&b)[3] = r[py][1];
+      if (px == 0) q = make_float4(a[0], a[1] + a[2], b[0], b[1] + b[2]);
+      else q = make_float4(a[0] + a[1], a[2], b[0] + b[1], b[2]);
+      *reinterpret_cast<float4 *>(packed + ((size_t)(py * 2 + px) * CO + co) * ld + ci * 4) = q;
+    }
+}
+
+int upsampling_convolution(const char *name, const mt_tensor *out, const mt_tensor *image, uint32_t ux, uint32_t uy, const mt_tensor *kernel, int32_t kx,
+                           int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
+  if (mt::bad(out) || mt::bad(image) || mt::bad(kernel) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (ux == 0 || uy == 0) return mt::fail(MT_E_ARGUMENT, "%s: up-sampling factors must be positive", name);
+  if ((uint64_t)image->y * uy > 0x7fffffffu || (uint64_t)image->x * ux > 0x7fffffffu) return mt::fail(MT_E_ARGUMENT, "%s: image too large", name);
+  const mt_tensor up_shape{image->p, image->w, image->z, image->y * uy, image->x * ux};  // sizes only: the pointer is not used
+  int rc = check_forward(name, out, &up_shape, kernel, kx, ky, kz, ka, bias, sx, sy, px, py);
+  if (rc) return rc;
+  if (mt::count(out) == 0) return MT_OK;
+  if (image->w == 0 || bias->w == 0) return mt::fail(MT_E_ARGUMENT, "%s: empty operand", name);
+  const uint32_t K = (uint32_t)kz * kx * ky;
+  if ((rc = check_kernel_tensor(name, kernel, ka, K))) return rc;
+  const bool phases = ux == 2 && uy == 2 && kx == 3 && ky == 3 && sx == 1 && sy == 1 && px == 1 && py == 1 && kernel->w == 1 && bias->w == 1 &&
+                      image->w == out->w && g_conv_path != 1 && mt::fits_buffer(image) && kz <= 0x0fffffff / 16;
+  if (!phases) {
+    // any other geometry: the two layers one after the other, the up-sampled image in the workspace behind the
+    // region the convolution may use for re-ordered weights
+    const size_t head = ((size_t)ka * K + 63) & ~(size_t)63;
+    float *ws = nullptr;
+    if ((rc = workspace(head + mt::count(&up_shape), &ws))) return rc;
+    mt_tensor up = up_shape;
+    up.p = ws + head;
+    if ((rc = mt_upsampling(&up, image, ux, uy))) return rc;
+    return forward(name, out, &up, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);
+  }
+  const uint32_t ld = (uint32_t)kz * 4;
+  float *packed = nullptr;
+  if ((rc = workspace((size_t)4 * ka * ld, &packed))) return rc;
+  {
+    mt::ProfileScope prof("upconv_prepare");
+    upconv_prepare_kernel<<<dim3(cdiv((uint32_t)kz, 256), ka), 256, 0, mt::stream()>>>(packed, kernel->p, kernel->x, ka, (uint32_t)kz);
+    MT_LAUNCH_CHECK("upconv_prepare");
+  }
+  TconvArgs args{};
+  uint32_t max_n = 0;
+  for (int32_t phy = 0; phy < 2; phy++) {
+    const Phase1D Y = phase_1d(phy, 4, 2, 1, out->y);
+    for (int32_t phx = 0; phx < 2; phx++) {
+      const Phase1D X = phase_1d(phx, 4, 2, 1, out->x);
+      const uint32_t f = args.nphase++;
+      args.ph[f] = TconvPhase{packed + (size_t)(phy * 2 + phx) * ka * ld, ld, ld, (uint32_t)Y.q, (uint32_t)X.q, Y.taps, X.taps, Y.off, X.off, (uint32_t)phy, (uint32_t)phx};
+      const uint32_t n = out->w * Y.q * X.q;
+      if (n > max_n) max_n = n;
+    }
+  }
+  const uint32_t OHW = out->y * out->x;
+  args.M = ka; args.out_w = out->w;
+  args.delta = image->p; args.in_w = image->w; args.C = kz; args.H = image->y; args.W = image->x;
+  args.ep.C = out->p; args.ep.row_stride = OHW; args.ep.g_stride = (size_t)ka * OHW;
+  args.ep.sy = 2; args.ep.sx = 2; args.ep.OW = out->x;
+  args.ep.bias = bias->p; args.ep.bias_mode = 1; args.ep.bias_w = 1; args.ep.bias_stride = 0;
+  args.ep.IH = image->y; args.ep.IW = image->x;
+  const bool func_later = !mt::epilogue_func(func);
+  args.ep.func = func_later ? MT_F_NONE : func;
+  rc = launch_tconv(name, args, max_n);
+  return rc == MT_OK && func_later ? mt_apply_func(out, out, func) : rc;
+}
+
 }  // namespace
 
 namespace mt {
@@ -1114,6 +1206,12 @@ int mt_forward_convolution_func(const mt_tensor *out, const mt_tensor *image, co
                                 const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
   if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_forward_convolution_func: unknown function id %d", func);
   return forward("mt_forward_convolution_func", out, image, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);
+}
+
+int mt_upsampling_convolution_func(const mt_tensor *out, const mt_tensor *image, uint32_t ux, uint32_t uy, const mt_tensor *kernel, int32_t kx, int32_t ky,
+                                   int32_t kz, uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
+  if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_upsampling_convolution_func: unknown function id %d", func);
+  return upsampling_convolution("mt_upsampling_convolution_func", out, image, ux, uy, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);
 }
 
 int mt_backward_convolution(const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,

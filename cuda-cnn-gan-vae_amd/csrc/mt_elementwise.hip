@@ -999,7 +999,8 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
   bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(pm) && aligned16(pi) && (!xhat || aligned16(xhat->p));
   if (vec && mt::epilogue_func(func)) {
     // one pass: the widest column block that still gives every compute unit a few blocks, if the batch share fits
-    const int rb = S / 128 >= 512 ? 32 : S / 64 >= 512 ? 16 : 8;
+    // (a small batch on a large tensor: 64 column groups, so that a thread still has 8 to 16 loads in flight)
+    const int rb = S / 256 >= 512 && cdiv(W, 4) <= 16 ? 64 : S / 128 >= 512 ? 32 : S / 64 >= 512 ? 16 : 8;
     const uint32_t nw = cdiv(W, EW_THREADS / rb);
     if (nw <= 32) {
       mt::ProfileScope prof("bn_fused");
@@ -1008,7 +1009,8 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
   bn_fused_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func)
 #define MT_BN_FUSED_NW(RB) \
   do { if (nw <= 8) MT_BN_FUSED(RB, 8); else if (nw <= 16) MT_BN_FUSED(RB, 16); else MT_BN_FUSED(RB, 32); } while (0)
-      if (rb == 32) MT_BN_FUSED_NW(32); else if (rb == 16) MT_BN_FUSED_NW(16); else MT_BN_FUSED_NW(8);
+      if (rb == 64) { if (nw <= 8) MT_BN_FUSED(64, 8); else MT_BN_FUSED(64, 16); }
+      else if (rb == 32) MT_BN_FUSED_NW(32); else if (rb == 16) MT_BN_FUSED_NW(16); else MT_BN_FUSED_NW(8);
 #undef MT_BN_FUSED_NW
 #undef MT_BN_FUSED
       MT_LAUNCH_CHECK("bn_fused");

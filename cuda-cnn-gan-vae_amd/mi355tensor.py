@@ -396,6 +396,12 @@ class Fused:
             call("mt_batchnorm_backward_func", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), opt(beta), _d(xhat), _d(ivar), C.c_int(FUNC[func]))
 
     @staticmethod
+    def UpSamplingConvolution(out, image, upsampling_x, upsampling_y, kernel, kernel_x, kernel_y, kernel_z, kernel_amount, bias, stride_x, stride_y,
+                              padding_x, padding_y, func=None):
+        call("mt_upsampling_convolution_func", _d(out), _d(image), _u(upsampling_x), _u(upsampling_y), _d(kernel), _i(kernel_x), _i(kernel_y), _i(kernel_z),
+             _u(kernel_amount), _d(bias), _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y), C.c_int(FUNC[func]))
+
+    @staticmethod
     def FillMany(tensors, value):
         call("mt_fill_many", _u(len(tensors)), _list(tensors), _f(value))
 

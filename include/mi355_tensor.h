@@ -150,6 +150,15 @@ int mt_forward_convolution_func(const mt_tensor *output, const mt_tensor *image,
 int mt_backward_convolution_func(const mt_tensor *output, const mt_tensor *delta, const mt_tensor *kernel,
                                  int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
                                  const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y, int func);
+/* CNetLayerUpSampling::Forward (netlayer/cnetlayerupsampling.cu.h:233-252) + CNetLayerConvolution::Forward
+ * (netlayer/cnetlayerconvolution.cu.h:310-322) + CNetLayerFunction::Forward: output = func(conv(UpSampling(image))).
+ * `image` is the input of the up-sampling layer, [W,kernel_z,H,Wd]; output must be the convolution's output for the
+ * up-sampled image [W,kernel_z,H*upsampling_y,Wd*upsampling_x].  For x2 up-sampling and a 3x3 kernel with stride 1 and
+ * padding 1 (the reference's GAN generator) the up-sampled image is never formed: each output parity is a 2x2
+ * convolution of the input with sums of the 3x3 coefficients. */
+int mt_upsampling_convolution_func(const mt_tensor *output, const mt_tensor *image, uint32_t upsampling_x, uint32_t upsampling_y,
+                                   const mt_tensor *kernel, int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
+                                   const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y, int func);
 /* CNetLayerLinear::Forward + CNetLayerFunction::Forward (netlayer/cnetlayerlinear.cu.h:262-282): output[B,1,Out,1] =
  * func(weight[1,1,Out,In] * input[B,1,In,1] + bias[1,1,Out,1]); `input` may have any [B,Z,Y,X] with Z*Y*X == In. */
 int mt_linear_forward_func(const mt_tensor *output, const mt_tensor *weight, const mt_tensor *input, const mt_tensor *bias, int func);

@@ -11,6 +11,9 @@ def up(a):
     return CTensor.from_numpy(np.ascontiguousarray(a, dtype=np.float32))
 
 
+up_ = up   # for methods with a parameter called `up`
+
+
 class Gpu:
     def __init__(self):
         mt.init(0)
@@ -203,6 +206,13 @@ class Gpu:
         err, dg, db = CTensor(*delta.shape), up(dgamma0), up(dbeta0)
         Fused.BatchNormBackward(err, dg, db, up(delta), up(gamma), up(xhat), up(ivar), beta=up(beta) if beta is not None else None, func=func)
         return err.numpy(), dg.numpy(), db.numpy()
+
+    def upsampling_convolution(self, image, kernel, bias, k, kz, ka, up=2, s=1, p=1, func=None):
+        image = np.asarray(image, np.float32)
+        oy, ox = (image.shape[2] * up - k + 2 * p) // s + 1, (image.shape[3] * up - k + 2 * p) // s + 1
+        out = up_(np.full((image.shape[0], ka, oy, ox), 7.0, np.float32))
+        Fused.UpSamplingConvolution(out, up_(image), up, up, up_(kernel), k, k, kz, ka, up_(bias), s, s, p, p, func)
+        return out.numpy()
 
     def fill_many(self, arrays, value):
         ts = [up(a) for a in arrays]

@@ -178,20 +178,10 @@ def test_shipped_gan_generator_topology(gpu, oracle):
     """The generator of the reference's own GAN model (Linear, then up-sampling + conv 3x3 + BatchNorm + leaky ReLU six
     times, conv 3x3 + tanh; 3x4 -> 192x256), every layer output against the oracle, at a quarter of the shipped widths
     and batch 4 so that the CPU side finishes in seconds."""
+    import gan_generator as GG
     channels, noise_size, b = (128, 128, 64, 32, 16, 8, 4), 64, 4
-    rng = np.random.default_rng(6)
-    params = {"lin_w": (rng.standard_normal((1, 1, 12 * channels[0], noise_size)) * 0.1).astype(np.float32),
-              "lin_b": np.full((1, 1, 12 * channels[0], 1), 0.1, np.float32)}
-    size, widths = (3, 4), channels[1:] + (3,)
-    for i in range(7):
-        cin, cout = (channels[0] if i == 0 else widths[i - 1]), widths[i]
-        params["kernel%d" % i] = (rng.standard_normal((1, 1, cout, cin * 9)) * np.sqrt(2.0 / (cin * 9))).astype(np.float32)
-        params["bias%d" % i] = (rng.standard_normal((1, cout, 1, 1)) * 0.05).astype(np.float32)
-        if i < 6:
-            size = (size[0] * 2, size[1] * 2)
-            params["gamma%d" % i] = rng.uniform(0.5, 1.5, (1, cout) + size).astype(np.float32)
-            params["beta%d" % i] = rng.uniform(-0.2, 0.2, (1, cout) + size).astype(np.float32)
-    noise = rng.standard_normal((b, 1, noise_size, 1)).astype(np.float32)
+    params, noise = GG.make_parameters(channels, noise_size), GG.make_noise(b, noise_size)
+    widths = channels[1:] + (3,)
     want = seq.gan_generator_forward(oracle, params, noise, channels)
     # layer by layer on the oracle's own inputs: a batch norm over four samples divides by spreads that can be tiny, so
     # rounding differences of one layer would otherwise be amplified by the next ones
@@ -210,6 +200,16 @@ def test_shipped_gan_generator_topology(gpu, oracle):
     # end to end: the whole stack on the device, seven layers of accumulated rounding
     got = seq.gan_generator_forward(gpu, params, noise, channels)
     assert got["image"].shape == (b, 3, 192, 256) and rel_err(got["image"], want["image"]) <= 2e-3
+    # the same stack on device-resident tensors, layer by layer and with up-sampling + convolution as one call
+    net = GG.GanGenerator(b, params, channels, noise_size)
+    net.set_noise(noise)
+    for fused in (False, True):
+        image = net.forward(fused).numpy()
+        assert rel_err(net.c[0].numpy(), want["c0"]) <= REL        # same input as the oracle's first convolution
+        assert rel_err(image, want["image"]) <= 2e-3, "fused" if fused else "layer by layer"
+    for i in range(6):   # one call against two layers, each on the oracle's input
+        one = gpu.upsampling_convolution(want["h%d" % i], params["kernel%d" % i], params["bias%d" % i], 3, want["h%d" % i].shape[1], widths[i])
+        assert rel_err(one, want["c%d" % i]) <= REL, "up-sampling + conv %d" % i
 
 
 def vae_parameters():

@@ -263,6 +263,37 @@ def test_convolution_backward_weights_sum(gpu, oracle, path, case):
         close(got_b, want_b)
 
 
+@pytest.mark.parametrize("case", [
+    # B, C, H, W, KA
+    (2, 16, 6, 8, 32),      # channels tile the k step
+    (3, 5, 3, 4, 7),        # channel counts that do not
+    (1, 8, 1, 1, 4),        # one input pixel: every tap but one is padding
+    (2, 4, 5, 3, 70),       # odd input sizes, more filters than one tile
+    (2, 64, 12, 16, 32),    # a layer of the reference's GAN generator at a quarter of its width
+])
+def test_upsampling_convolution(gpu, oracle, path, case):
+    """Up-sampling x2 + convolution 3x3 stride 1 padding 1 (+ function) in one call, against the two layers on the
+    oracle (netlayer/cnetlayerupsampling.cu.h:233-252, netlayer/cnetlayerconvolution.cu.h:310-322): four 2x2
+    convolutions of the input with summed coefficients, so sums differ from the reference's by rounding only."""
+    B, C, H, Wd, KA = case
+    image, kernel, bias = U(1, B, C, H, Wd), Nrm(2, 1, 1, KA, C * 9, std=float(np.sqrt(2.0 / (C * 9)))), U(3, 1, KA, 1, 1) * 0.3
+    want = oracle.forward_convolution(oracle.upsampling(image, 2, 2), kernel, bias, 3, 3, C, KA, 1, 1, 1, 1)
+    close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA), want, 1e-5)
+    close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA, func="leaky_relu"), oracle.apply_func(want, "leaky_relu"), 1e-5)
+    close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA, func="tangence"), oracle.apply_func(want, "tangence"), 1e-5)
+
+
+def test_upsampling_convolution_other_geometries(gpu, oracle, path):
+    """Anything but (x2, 3x3, stride 1, padding 1) runs as the two layers one after the other inside the library."""
+    image = U(1, 2, 6, 5, 4)
+    for up, k, s, p in ((3, 3, 1, 1), (2, 5, 1, 2), (2, 3, 2, 1), (2, 3, 1, 0), (1, 3, 1, 1)):
+        kernel, bias = Nrm(2, 1, 1, 9, 6 * k * k, std=0.2), U(3, 1, 9, 1, 1)
+        want = oracle.forward_convolution(oracle.upsampling(image, up, up), kernel, bias, k, k, 6, 9, s, s, p, p)
+        close(gpu.upsampling_convolution(image, kernel, bias, k, 6, 9, up=up, s=s, p=p), want, 1e-5)
+    with pytest.raises(Exception):
+        gpu.upsampling_convolution(image, Nrm(2, 1, 1, 9, 54, std=0.2), U(3, 1, 8, 1, 1), 3, 6, 9)   # eight biases for nine filters
+
+
 def test_fused_conv_activation(gpu, oracle, path):
     image, kernel, bias = U(1, 3, 4, 10, 10), U(2, 1, 1, 6, 4 * 9), U(3, 1, 6, 1, 1)
     for func in ("leaky_relu", "relu", "tangence", "sigmoid"):
