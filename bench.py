@@ -80,14 +80,15 @@ def memory_bound_ops(args):
     import mi355tensor as mt
     from mi355tensor import CTensor, CTensorApplyFunc as F, CTensorMath as M, Fused
     mt.init(0)
-    shape, s1 = (256, 64, 32, 32), (1, 64, 32, 32)
-    n = 256 * 64 * 32 * 32
+    W = args.ops_batch   # 256: the activation of the measured configuration (67 MB, within the 256 MB Infinity Cache)
+    shape, s1 = (W, 64, 32, 32), (1, 64, 32, 32)
+    n = W * 64 * 32 * 32
     rng = np.random.default_rng(0)
     a, b, out = (CTensor.from_numpy(rng.standard_normal(shape).astype(np.float32)) for _ in range(3))
     g, be, m1, v1 = (CTensor.from_numpy(np.abs(rng.standard_normal(s1)).astype(np.float32) + 0.5) for _ in range(4))
-    xhat, sums, bias = CTensor(*shape), CTensor(256, 64, 1, 1), CTensor.from_numpy(np.ones((1, 64, 1, 1), np.float32))
-    half, pos, up = CTensor(256, 64, 16, 16), CTensor(256, 64, 16, 16, pos=True), CTensor(256, 64, 64, 64)
-    big = CTensor(256, 64, 64, 64)
+    xhat, sums, bias = CTensor(*shape), CTensor(W, 64, 1, 1), CTensor.from_numpy(np.ones((1, 64, 1, 1), np.float32))
+    half, pos, up = CTensor(W, 64, 16, 16), CTensor(W, 64, 16, 16, pos=True), CTensor(W, 64, 64, 64)
+    big = CTensor(W, 64, 64, 64)
     mom, vel = CTensor.from_numpy(np.zeros(shape, np.float32)), CTensor.from_numpy(np.zeros(shape, np.float32))
     B = 4.0 * n
     ops = [  # name, callable, algorithmic bytes
@@ -101,7 +102,7 @@ def memory_bound_ops(args):
         ("ApplyTangence", lambda: F.ApplyTangence(out, a), 2 * B),
         ("ApplyDifferentialLeakyReLU", lambda: F.ApplyDifferentialLeakyReLU(out, a), 2 * B),
         ("AddBias", lambda: M.AddBias(out, bias), 2 * B),
-        ("AddSumW (sum over the batch)", lambda: M.AddSumW(m1, m1, a, 1.0, 1.0 / 256), B),
+        ("AddSumW (sum over the batch)", lambda: M.AddSumW(m1, m1, a, 1.0, 1.0 / W), B),
         ("SummXY", lambda: M.SummXY(sums, a), B),
         ("batch norm forward, training mode, fused + ReLU", lambda: Fused.BatchNormForwardTrain(out, a, g, be, func="relu"), 2 * B),
         ("batch norm forward, training mode, keeping xhat", lambda: Fused.BatchNormForwardTrain(out, a, g, be, xhat, v1), 3 * B),
@@ -111,7 +112,7 @@ def memory_bound_ops(args):
         ("MaxPoolingBackward 2x2", lambda: M.MaxPoolingBackward(out, pos, half, 2, 2), B + 3 * B / 4),
         ("UpSampling x2", lambda: M.UpSampling(up, a, 2, 2), B + 4 * B),
         ("DownSampling x2", lambda: M.DownSampling(a, big, 2, 2), 4 * B + B),
-        ("Adam", lambda: M.Adam(out, a, mom, vel, 256, 2e-4, 0.5, 0.999, 1e-8, 1.0), 7 * B),
+        ("Adam", lambda: M.Adam(out, a, mom, vel, W, 2e-4, 0.5, 0.999, 1e-8, 1.0), 7 * B),
     ]
     stream = mt.get_stream()
     create, record, elapsed_ms = hip_events()
@@ -128,7 +129,7 @@ def memory_bound_ops(args):
         results[name] = {"us": us, "GB/s": nbytes / us / 1e3, "frac_of_hbm_peak": nbytes / us / 1e3 / 8000.0, "algorithmic_MB": nbytes / 1e6}
     rates = [r["GB/s"] for r in results.values()]
     print(json.dumps({
-        "metric": "GB/s of the HBM-bound tensor operations on a [256,64,32,32] fp32 activation (secondary workload)",
+        "metric": "GB/s of the HBM-bound tensor operations on a [%d,64,32,32] fp32 activation (secondary workload)" % W,
         "value": float(np.median(rates)), "unit": "GB/s (median over the operations)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": sum(r["us"] for r in results.values()) / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic", "config": {"workload": "every HBM-bound operation of the tensor-op layer, one launch each per step"},
@@ -294,6 +295,7 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="time region 1 as replays of the step recorded once as a HIP graph (c5 does so by default: its step "
                          "is about a hundred short kernels and the Python host would be the bottleneck)")
+    ap.add_argument("--ops-batch", type=int, default=256, help="workload ops: batch size of the [W,64,32,32] activation (1024: 268 MB per tensor)")
     ap.add_argument("--literal", action="store_true", help="workload gan: up-sampling and convolution as two layers")
     ap.add_argument("--workload", choices=["c3", "c5", "ops", "c1", "c2", "c4", "gan"], default="c3",
                     help="c3 (default, the measured configuration): DCGAN-64 generator forward, batch 256; "

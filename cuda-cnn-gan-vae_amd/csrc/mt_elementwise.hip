@@ -161,7 +161,16 @@ __global__ __launch_bounds__(EW_THREADS) void summ_xy_kernel(float *out, const f
   uint32_t w = row / Z, z = row % Z, lane = threadIdx.x % 64;
   const float *p = in + ((size_t)(w % Win) * Z + z) * YX;
   float s = 0.f;
-  for (uint32_t i = lane; i < YX; i += 64) s += p[i];
+  if (YX % 4 == 0 && ((uintptr_t)p & 15u) == 0) {  // 128-bit loads, four partial sums per lane
+    float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t i = lane; i < YX / 4; i += 64) {
+      const float4 v = reinterpret_cast<const float4 *>(p)[i];
+      q.x += v.x; q.y += v.y; q.z += v.z; q.w += v.w;
+    }
+    s = (q.x + q.y) + (q.z + q.w);
+  } else {
+    for (uint32_t i = lane; i < YX; i += 64) s += p[i];
+  }
   s = mt::wave_sum(s);
   if (lane == 0) out[row] = s;
 }
@@ -263,44 +272,81 @@ __global__ __launch_bounds__(EW_THREADS) void upsampling_kernel(float *out, cons
   }
 }
 
-// Four consecutive output columns per thread (one 128-bit store); ox is a multiple of 4.
+// Four consecutive output columns per thread (one 128-bit store); ox is a multiple of 4, the input is not empty.
+// Source indices are clamped into the input and the out-of-range columns zeroed afterwards, so the loads carry no
+// condition and four planes are in flight per thread.
 __global__ __launch_bounds__(EW_THREADS) void upsampling4_kernel(float *out, const float *in, Geo g, uint32_t ux, uint32_t uy, uint32_t planes) {
   const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ox4 = g.ox / 4, n4 = g.oy * ox4;
   if (i >= n4) return;
   const uint32_t y = i / ox4, x = (i % ox4) * 4, sy = y / uy;
+  const uint32_t syc = sy < g.iy ? sy : g.iy - 1;
   uint32_t sx[4];
+  bool ok[4];
 #pragma unroll
-  for (int k = 0; k < 4; k++) sx[k] = (x + k) / ux;
+  for (int k = 0; k < 4; k++) {
+    const uint32_t c = (x + k) / ux;
+    ok[k] = sy < g.iy && c < g.ix;
+    sx[k] = c < g.ix ? c : g.ix - 1;
+  }
+  const size_t plane_in = (size_t)g.iy * g.ix, plane_out = (size_t)g.oy * g.ox;
+  const bool same_w = g.Win * g.Z == planes;  // no broadcast over the batch: plane pl of the input
+#pragma unroll 4
   for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
-    const uint32_t w = pl / g.Z, z = pl % g.Z;
-    const float *src = in + (((size_t)(w % g.Win) * g.Z + z) * g.iy + sy) * g.ix;
+    const uint32_t ipl = same_w ? pl : (pl / g.Z % g.Win) * g.Z + pl % g.Z;
+    const float *src = in + (size_t)ipl * plane_in + (size_t)syc * g.ix;
     float v[4];
 #pragma unroll
-    for (int k = 0; k < 4; k++) v[k] = (sy < g.iy && sx[k] < g.ix) ? src[sx[k]] : 0.f;
-    reinterpret_cast<float4 *>(out + (size_t)pl * g.oy * g.ox)[i] = make_float4(v[0], v[1], v[2], v[3]);
+    for (int k = 0; k < 4; k++) v[k] = src[sx[k]];
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = ok[k] ? v[k] : 0.f;
+    reinterpret_cast<float4 *>(out + (size_t)pl * plane_out)[i] = make_float4(v[0], v[1], v[2], v[3]);
+  }
+}
+// x2 in both directions, output exactly twice the input, even input width: a thread reads two input pixels (64 bits)
+// and writes their 2x4 output pixels as two 128-bit stores; the same index map, without divisions.
+__global__ __launch_bounds__(EW_THREADS) void upsampling2x2_kernel(float *out, const float *in, Geo g, uint32_t planes) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ix2 = g.ix / 2, n2 = g.iy * ix2;
+  if (i >= n2) return;
+  const uint32_t y = i / ix2, x2 = i % ix2;
+  const size_t plane_in = (size_t)g.iy * g.ix, plane_out = (size_t)g.oy * g.ox;
+  const size_t o0 = (size_t)(2 * y) * g.ox + 4 * x2;
+  const bool same_w = g.Win * g.Z == planes;
+#pragma unroll 4
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const uint32_t ipl = same_w ? pl : (pl / g.Z % g.Win) * g.Z + pl % g.Z;
+    const float2 v = reinterpret_cast<const float2 *>(in + (size_t)ipl * plane_in)[i];
+    const float4 q = make_float4(v.x, v.x, v.y, v.y);
+    float *dst = out + (size_t)pl * plane_out + o0;
+    *reinterpret_cast<float4 *>(dst) = q;
+    *reinterpret_cast<float4 *>(dst + g.ox) = q;
   }
 }
 __global__ __launch_bounds__(EW_THREADS) void max_pooling_backward4_kernel(float *out, const mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t px_, uint32_t py_, uint32_t planes) {
   const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ox4 = g.ox / 4, n4 = g.oy * ox4;
   if (i >= n4) return;
   const uint32_t y = i / ox4, x = (i % ox4) * 4, sy = y / py_;
+  const uint32_t syc = sy < g.iy ? sy : g.iy - 1;
   uint32_t sx[4];
+  bool ok[4];
 #pragma unroll
-  for (int k = 0; k < 4; k++) sx[k] = (x + k) / px_;
+  for (int k = 0; k < 4; k++) {
+    const uint32_t c = (x + k) / px_;
+    ok[k] = sy < g.iy && c < g.ix;
+    sx[k] = c < g.ix ? c : g.ix - 1;
+  }
+  const size_t plane_in = (size_t)g.iy * g.ix, plane_out = (size_t)g.oy * g.ox;
+#pragma unroll 2
   for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
     const uint32_t w = pl / g.Z, z = pl % g.Z;
-    const mt_spos *prow = pos + (((size_t)(w % Wpos) * g.Z + z) * g.iy + sy) * g.ix;
-    const float *irow = in + ((size_t)pl * g.iy + sy) * g.ix;
+    const mt_spos *prow = pos + ((size_t)(w % Wpos) * g.Z + z) * plane_in + (size_t)syc * g.ix;
+    const float *irow = in + (size_t)pl * plane_in + (size_t)syc * g.ix;
+    mt_spos s[4];
     float v[4];
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-      v[k] = 0.f;
-      if (sy < g.iy && sx[k] < g.ix) {
-        const mt_spos s = prow[sx[k]];
-        if (s.X == x + k && s.Y == y) v[k] = irow[sx[k]];
-      }
-    }
-    reinterpret_cast<float4 *>(out + (size_t)pl * g.oy * g.ox)[i] = make_float4(v[0], v[1], v[2], v[3]);
+    for (int k = 0; k < 4; k++) { s[k] = prow[sx[k]]; v[k] = irow[sx[k]]; }
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = (ok[k] && s[k].X == x + k && s[k].Y == y) ? v[k] : 0.f;
+    reinterpret_cast<float4 *>(out + (size_t)pl * plane_out)[i] = make_float4(v[0], v[1], v[2], v[3]);
   }
 }
 __global__ __launch_bounds__(EW_THREADS) void downsampling_kernel(float *out, const float *in, Geo g, uint32_t dsx, uint32_t dsy, uint32_t planes) {
@@ -341,6 +387,55 @@ __global__ __launch_bounds__(EW_THREADS) void max_pooling_kernel(float *out, mt_
     out[(size_t)pl * n + i] = best;
     mt_spos s; s.X = bx; s.Y = by;
     pos[((size_t)(w % Wpos) * g.Z + z) * n + i] = s;
+  }
+}
+
+// 2x2 windows over an input of exactly twice the output and a width that is a multiple of four: a thread reads
+// 2x4 input pixels (two 128-bit loads) and produces two outputs; same arithmetic and scan order as the kernels above.
+__global__ __launch_bounds__(EW_THREADS) void downsampling2x2_kernel(float *out, const float *in, Geo g, uint32_t planes) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ox2 = g.ox / 2, n2 = g.oy * ox2;
+  if (i >= n2) return;
+  const uint32_t y = i / ox2, x2 = i % ox2;
+  const size_t plane_in = (size_t)g.iy * g.ix, plane_out = (size_t)g.oy * g.ox;
+  const size_t i0 = (size_t)(2 * y) * g.ix + 4 * x2;
+#pragma unroll 4
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const float *p = in + (size_t)pl * plane_in + i0;
+    const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + g.ix);
+    float2 r;
+    r.x = ((((0.f + a.x) + b.x) + a.y) + b.y) / 4.f;  // columns outer, rows inner
+    r.y = ((((0.f + a.z) + b.z) + a.w) + b.w) / 4.f;
+    reinterpret_cast<float2 *>(out + (size_t)pl * plane_out)[i] = r;
+  }
+}
+__global__ __launch_bounds__(EW_THREADS) void max_pooling2x2_kernel(float *out, mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t planes) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ox2 = g.ox / 2, n2 = g.oy * ox2;
+  if (i >= n2) return;
+  const uint32_t y = i / ox2, x2 = i % ox2, iy = 2 * y, ix = 4 * x2;
+  const size_t plane_in = (size_t)g.iy * g.ix, plane_out = (size_t)g.oy * g.ox;
+  const size_t i0 = (size_t)iy * g.ix + ix;
+  const bool same_w = Wpos * g.Z == planes;
+#pragma unroll 4
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const float *p = in + (size_t)pl * plane_in + i0;
+    const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + g.ix);
+    const float e[2][4] = {{a.x, a.y, b.x, b.y}, {a.z, a.w, b.z, b.w}};  // window scan order: rows, then columns
+    float best[2];
+    uint4 where;
+    uint32_t wh[4];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+      best[k] = e[k][0];
+      uint32_t bx = ix + 2 * k, by = iy;
+#pragma unroll
+      for (int t = 0; t < 4; t++)
+        if (e[k][t] > best[k]) { best[k] = e[k][t]; bx = ix + 2 * k + (t & 1); by = iy + (t >> 1); }  // first strict maximum
+      wh[2 * k] = bx; wh[2 * k + 1] = by;
+    }
+    where = make_uint4(wh[0], wh[1], wh[2], wh[3]);
+    reinterpret_cast<float2 *>(out + (size_t)pl * plane_out)[i] = make_float2(best[0], best[1]);
+    const uint32_t ppl = same_w ? pl : (pl / g.Z % Wpos) * g.Z + pl % g.Z;
+    reinterpret_cast<uint4 *>(pos + (size_t)ppl * plane_out)[i] = where;
   }
 }
 
@@ -850,7 +945,13 @@ int mt_upsampling(const mt_tensor *out, const mt_tensor *in, uint32_t ux, uint32
   if (planes == 0 || n == 0) return MT_OK;
   if (in->w == 0) return mt::fail(MT_E_ARGUMENT, "mt_upsampling: empty input");
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
-  if (out->x % 4 == 0 && aligned16(out->p)) {
+  if (ux == 2 && uy == 2 && out->x == 2 * in->x && out->y == 2 * in->y && in->x % 2 == 0 && in->x > 0 && aligned16(out->p) && ((uintptr_t)in->p & 7u) == 0) {
+    const unsigned bx = cdiv(n / 8, EW_THREADS);
+    upsampling2x2_kernel<<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, planes);
+    MT_LAUNCH_CHECK("mt_upsampling");
+    return MT_OK;
+  }
+  if (out->x % 4 == 0 && aligned16(out->p) && in->x > 0 && in->y > 0) {
     dim3 grid4(cdiv(n / 4, EW_THREADS), plane_blocks(cdiv(n / 4, EW_THREADS), planes));
     upsampling4_kernel<<<grid4, EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, ux, uy, planes);
     MT_LAUNCH_CHECK("mt_upsampling");
@@ -868,6 +969,12 @@ int mt_downsampling(const mt_tensor *out, const mt_tensor *in, uint32_t dx, uint
   uint32_t planes = out->w * out->z, n = out->y * out->x;
   if (planes == 0 || n == 0) return MT_OK;
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  if (dx == 2 && dy == 2 && in->x == 2 * out->x && in->y == 2 * out->y && out->x % 2 == 0 && aligned16(in->p) && ((uintptr_t)out->p & 7u) == 0) {
+    const unsigned bx = cdiv(n / 2, EW_THREADS);
+    downsampling2x2_kernel<<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, planes);
+    MT_LAUNCH_CHECK("mt_downsampling");
+    return MT_OK;
+  }
   dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
   downsampling_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, dx, dy, planes);
   MT_LAUNCH_CHECK("mt_downsampling");
@@ -882,6 +989,13 @@ int mt_max_pooling(const mt_tensor *out, const mt_pos_tensor *pos, const mt_tens
   if (pos->p == nullptr || pos->w == 0 || pos->z != out->z || pos->y != out->y || pos->x != out->x)
     return mt::fail(MT_E_ARGUMENT, "mt_max_pooling: position tensor must be [W',Z,Y,X] of the output");
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  if (px == 2 && py == 2 && in->x == 2 * out->x && in->y == 2 * out->y && out->x % 2 == 0 && aligned16(in->p) && ((uintptr_t)out->p & 7u) == 0 &&
+      aligned16(pos->p)) {
+    const unsigned bx = cdiv(n / 2, EW_THREADS);
+    max_pooling2x2_kernel<<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, planes);
+    MT_LAUNCH_CHECK("mt_max_pooling");
+    return MT_OK;
+  }
   dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
   max_pooling_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, px, py, planes);
   MT_LAUNCH_CHECK("mt_max_pooling");
@@ -896,7 +1010,7 @@ int mt_max_pooling_backward(const mt_tensor *out, const mt_pos_tensor *pos, cons
   if (pos->p == nullptr || pos->w == 0 || pos->z != in->z || pos->y != in->y || pos->x != in->x)
     return mt::fail(MT_E_ARGUMENT, "mt_max_pooling_backward: position tensor must be [W',Z,Y,X] of the input");
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
-  if (out->x % 4 == 0 && aligned16(out->p)) {
+  if (out->x % 4 == 0 && aligned16(out->p) && in->x > 0 && in->y > 0) {
     dim3 grid4(cdiv(n / 4, EW_THREADS), plane_blocks(cdiv(n / 4, EW_THREADS), planes));
     max_pooling_backward4_kernel<<<grid4, EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, px, py, planes);
     MT_LAUNCH_CHECK("mt_max_pooling_backward");

@@ -372,6 +372,20 @@ def test_resampling_and_pooling_bit_exact(gpu, oracle):
         assert np.array_equal(gpu.max_pooling_backward(d, o[1], dx, dy, a.shape), oracle.max_pooling_backward(d, o[1], dx, dy, a.shape))
 
 
+@pytest.mark.parametrize("shape", [(3, 2, 8, 16), (2, 5, 64, 64), (1, 1, 2, 4), (2, 3, 6, 12)])
+def test_resampling_and_pooling_2x2_bit_exact(gpu, oracle, shape):
+    """Widths that are multiples of four and 2x2 windows: the kernels with 128-bit accesses, ties and all."""
+    a = U(5, *shape)
+    ties = np.round(a * 2)
+    assert np.array_equal(gpu.upsampling(a, 2, 2), oracle.upsampling(a, 2, 2))
+    assert np.array_equal(gpu.downsampling(a, 2, 2), oracle.downsampling(a, 2, 2))
+    for t in (a, ties):
+        g, o = gpu.max_pooling(t, 2, 2), oracle.max_pooling(t, 2, 2)
+        assert np.array_equal(g[1], o[1]) and np.array_equal(g[0], o[0])
+        d = U(6, *o[0].shape)
+        assert np.array_equal(gpu.max_pooling_backward(d, o[1], 2, 2, a.shape), oracle.max_pooling_backward(d, o[1], 2, 2, a.shape))
+
+
 @pytest.mark.parametrize("name", sorted(oracle_api.FUNC))
 def test_activations(gpu, oracle, name):
     x = np.concatenate([U(1, 4000) * 12, U(2, 2000) * 40, np.array([0.0, -0.0, 30, -30, 30.000002, -30.000002], np.float32)]).reshape(1, 1, 1, -1)
