@@ -813,6 +813,73 @@ __global__ void vae_kl_kernel(float *kl, const float *partial, uint32_t blocks, 
   kl[0] = t / batch;
 }
 
+// ---- functions of the reference's GPU class that have no CPU counterpart (cuda/ctensormath.cu.h:473-598, 3029-3262) ----
+// ConcatecationZ / SplitZ: plane (w, z) of the wide tensor is plane (w % Wa, z) of A or (w % Wb, z - Za) of B.
+// TO_WIDE: the wide tensor is written (concatenation), else read (split; w then runs over the wide tensor's batch).
+template <bool TO_WIDE, class V>
+__global__ __launch_bounds__(EW_THREADS) void concat_split_z_kernel(V *wide, V *a, V *b, uint32_t Wwide, uint32_t Z, uint32_t Wa, uint32_t Za, uint32_t Wb,
+                                                                     uint32_t yx) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (i >= yx) return;
+  const uint32_t planes = Wwide * Z, Zb = Z - Za;
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const uint32_t w = pl / Z, z = pl % Z;
+    V *narrow = z < Za ? a + ((size_t)(w % Wa) * Za + z) * yx : b + ((size_t)(w % Wb) * Zb + (z - Za)) * yx;
+    if (TO_WIDE) wide[(size_t)pl * yx + i] = narrow[i];
+    else narrow[i] = wide[(size_t)pl * yx + i];
+  }
+}
+
+// SetTimeStep: out = in + (pos even ? sin : cos)(t[w] / 10000^(pos/size)), pos = element index within the sample
+__global__ __launch_bounds__(EW_THREADS) void set_time_step_kernel(float *out, const float *in, const uint32_t *time_step, uint32_t size, uint32_t W) {
+  const uint32_t pos = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (pos >= size) return;
+  const float scale = powf(10000.0f, (float)pos / (float)size);
+  for (uint32_t w = blockIdx.y; w < W; w += gridDim.y) {
+    const float angle = (float)time_step[w] / scale;
+    out[(size_t)w * size + pos] = in[(size_t)w * size + pos] + ((pos & 1u) == 0 ? sinf(angle) : cosf(angle));
+  }
+}
+
+// Philox4x32-10 (Salmon et al., SC'11): key = seed, counter = (element index, 0, 0); one block of four words per element.
+__device__ __forceinline__ void philox4x32_10(uint64_t seed, uint64_t index, uint32_t (&r)[4]) {
+  uint32_t c0 = (uint32_t)index, c1 = (uint32_t)(index >> 32), c2 = 0u, c3 = 0u, k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+#pragma unroll
+  for (int round = 0; round < 10; round++) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  r[0] = c0; r[1] = c1; r[2] = c2; r[3] = c3;
+}
+__device__ __forceinline__ float philox_uniform(const uint32_t (&r)[4]) { return (float)(r[0] >> 8) * (1.0f / 16777216.0f); }  // [0, 1)
+__device__ __forceinline__ float philox_normal(const uint32_t (&r)[4]) {  // Box-Muller: u1 in (0, 1], u2 in [0, 1)
+  const float u1 = (float)((r[0] >> 8) + 1u) * (1.0f / 16777216.0f), u2 = (float)(r[1] >> 8) * (1.0f / 16777216.0f);
+  return sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2);
+}
+__global__ __launch_bounds__(EW_THREADS) void drop_out_kernel(float *out, size_t n, float drop_out, float mult, uint64_t seed) {
+  for (size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += (size_t)gridDim.x * EW_THREADS) {
+    uint32_t r[4];
+    philox4x32_10(seed, i, r);
+    out[i] = philox_uniform(r) >= drop_out ? mult : 0.f;
+  }
+}
+// noise = N(0,1); with an image: noisy = sa[w] * image + sb[w] * noise
+__global__ __launch_bounds__(EW_THREADS) void normal_noise_kernel(float *noise, float *noisy, const float *image, const float *sa, uint32_t sa_stride,
+                                                                   const float *sb, uint32_t sb_stride, size_t per, size_t n, uint64_t seed) {
+  for (size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += (size_t)gridDim.x * EW_THREADS) {
+    uint32_t r[4];
+    philox4x32_10(seed, i, r);
+    const float e = philox_normal(r);
+    noise[i] = e;
+    if (noisy) {
+      const size_t w = i / per;
+      noisy[i] = (sa[w * sa_stride] * image[i]) + (sb[w * sb_stride] * e);
+    }
+  }
+}
+
 __global__ __launch_bounds__(EW_THREADS) void bn_ivar_kernel(float *ivar, const float *var, uint32_t S, float eps) {
   uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
   if (i < S) ivar[i] = (float)(1.0 / (double)sqrtf(var[i] + eps));
@@ -832,6 +899,34 @@ int bn_scratch(size_t floats, float **p) {
   }
   *p = g_bn_scratch;
   return MT_OK;
+}
+}  // namespace
+
+namespace {
+template <bool TO_WIDE>
+int concat_split(const char *name, const mt_tensor *wide, const mt_tensor *a, const mt_tensor *b) {
+  if (mt::bad(wide) || mt::bad(a) || mt::bad(b)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (wide->x != a->x || wide->x != b->x || wide->y != a->y || wide->y != b->y || wide->z != a->z + b->z)
+    return mt::fail(MT_E_SHAPE, "%s: sizes do not match", name);
+  const uint32_t yx = wide->y * wide->x, planes = wide->w * wide->z;
+  if (yx == 0 || planes == 0) return MT_OK;
+  if ((a->z && a->w == 0) || (b->z && b->w == 0)) return mt::fail(MT_E_ARGUMENT, "%s: empty operand", name);
+  const uint32_t wa = a->w ? a->w : 1, wb = b->w ? b->w : 1;
+  if (yx % 4 == 0 && aligned16(wide->p) && aligned16(a->p) && aligned16(b->p)) {
+    const unsigned bx = cdiv(yx / 4, EW_THREADS);
+    concat_split_z_kernel<TO_WIDE, float4><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(
+        (float4 *)wide->p, (float4 *)a->p, (float4 *)b->p, wide->w, wide->z, wa, a->z, wb, yx / 4);
+  } else {
+    const unsigned bx = cdiv(yx, EW_THREADS);
+    concat_split_z_kernel<TO_WIDE, float><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(wide->p, a->p, b->p, wide->w, wide->z, wa, a->z,
+                                                                                                               wb, yx);
+  }
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+unsigned stream_blocks(size_t n) {
+  const unsigned blocks = cdiv(n, EW_THREADS);
+  return blocks > 16384u ? 16384u : blocks;
 }
 }  // namespace
 
@@ -1019,6 +1114,60 @@ int mt_max_pooling_backward(const mt_tensor *out, const mt_pos_tensor *pos, cons
   dim3 grid(cdiv(n, EW_THREADS), planes < 65535u ? planes : 65535u);
   max_pooling_backward_kernel<<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, px, py, planes);
   MT_LAUNCH_CHECK("mt_max_pooling_backward");
+  return MT_OK;
+}
+
+int mt_concatecation_z(const mt_tensor *out, const mt_tensor *a, const mt_tensor *b) { return concat_split<true>("mt_concatecation_z", out, a, b); }
+int mt_split_z(const mt_tensor *out_a, const mt_tensor *out_b, const mt_tensor *in) { return concat_split<false>("mt_split_z", in, out_a, out_b); }
+
+int mt_set_time_step(const mt_tensor *out, const mt_tensor *in, const mt_u32_tensor *time_step) {
+  if (mt::bad(out) || mt::bad(in) || time_step == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_set_time_step: null tensor");
+  if (!mt::same_zyx(in, out) || in->w != out->w || time_step->w != in->w || time_step->z != 1 || time_step->y != 1 || time_step->x != 1)
+    return mt::fail(MT_E_SHAPE, "mt_set_time_step: sizes do not match");
+  const size_t size = (size_t)in->z * in->y * in->x;
+  if (size == 0 || in->w == 0) return MT_OK;
+  if (time_step->p == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_set_time_step: null tensor");
+  if (size > 0xffffffffu) return mt::fail(MT_E_ARGUMENT, "mt_set_time_step: sample too large");
+  const unsigned bx = cdiv(size, EW_THREADS);
+  set_time_step_kernel<<<dim3(bx, plane_blocks(bx, in->w)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, time_step->p, (uint32_t)size, in->w);
+  MT_LAUNCH_CHECK("mt_set_time_step");
+  return MT_OK;
+}
+
+int mt_create_drop_out_matrix(const mt_tensor *out, float drop_out, uint64_t seed) {
+  if (mt::bad(out)) return mt::fail(MT_E_ARGUMENT, "mt_create_drop_out_matrix: null tensor");
+  const size_t n = mt::count(out);
+  if (n == 0) return MT_OK;
+  drop_out_kernel<<<stream_blocks(n), EW_THREADS, 0, mt::stream()>>>(out->p, n, drop_out, (float)(1.0 / (1.0 - (double)drop_out)), seed);
+  MT_LAUNCH_CHECK("mt_create_drop_out_matrix");
+  return MT_OK;
+}
+
+int mt_set_normal_noise(const mt_tensor *out, uint64_t seed) {
+  if (mt::bad(out)) return mt::fail(MT_E_ARGUMENT, "mt_set_normal_noise: null tensor");
+  const size_t n = mt::count(out);
+  if (n == 0) return MT_OK;
+  normal_noise_kernel<<<stream_blocks(n), EW_THREADS, 0, mt::stream()>>>(out->p, nullptr, nullptr, nullptr, 0, nullptr, 0, 1, n, seed);
+  MT_LAUNCH_CHECK("mt_set_normal_noise");
+  return MT_OK;
+}
+
+int mt_get_noise_image_and_noise(const mt_tensor *noisy, const mt_tensor *noise, const mt_tensor *image, const mt_tensor *sqrt_alpha_bar,
+                                 const mt_tensor *sqrt_one_minus_alpha_bar, uint64_t seed) {
+  const mt_tensor *all[5] = {noisy, noise, image, sqrt_alpha_bar, sqrt_one_minus_alpha_bar};
+  for (auto t : all)
+    if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_get_noise_image_and_noise: null tensor");
+  if (!mt::same_zyx(noisy, noise) || noisy->w != noise->w) return mt::fail(MT_E_SHAPE, "mt_get_noise_image_and_noise: sizes of NoisyImage and Noise differ");
+  if (!mt::same_zyx(noisy, image) || noisy->w != image->w) return mt::fail(MT_E_SHAPE, "mt_get_noise_image_and_noise: sizes of NoisyImage and Image differ");
+  if (sqrt_alpha_bar->w != image->w || sqrt_one_minus_alpha_bar->w != image->w)
+    return mt::fail(MT_E_SHAPE, "mt_get_noise_image_and_noise: SqrtAlphaBar / SqrtOneMinusAlphaBar need one value per sample");
+  const size_t n = mt::count(image), per = (size_t)image->z * image->y * image->x;
+  if (n == 0) return MT_OK;
+  const size_t sa = (size_t)sqrt_alpha_bar->z * sqrt_alpha_bar->y * sqrt_alpha_bar->x, sb = (size_t)sqrt_one_minus_alpha_bar->z * sqrt_one_minus_alpha_bar->y * sqrt_one_minus_alpha_bar->x;
+  if (sa == 0 || sb == 0 || sa > 0xffffffffu || sb > 0xffffffffu) return mt::fail(MT_E_SHAPE, "mt_get_noise_image_and_noise: SqrtAlphaBar / SqrtOneMinusAlphaBar need one value per sample");
+  normal_noise_kernel<<<stream_blocks(n), EW_THREADS, 0, mt::stream()>>>(noise->p, noisy->p, image->p, sqrt_alpha_bar->p, (uint32_t)sa, sqrt_one_minus_alpha_bar->p,
+                                                                         (uint32_t)sb, per, n, seed);
+  MT_LAUNCH_CHECK("mt_get_noise_image_and_noise");
   return MT_OK;
 }
 

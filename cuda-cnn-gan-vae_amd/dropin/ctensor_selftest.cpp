@@ -2,6 +2,7 @@
 // (cuda/ctensortest.cu.h:725-928 and the five convolution tests at :77-652) written against the same public API,
 // plus the lazy host/device coherence and the error convention.  Every tensor op below runs on the GPU through
 // libmi355tensor.so.  Prints one line per check; exit code 0 when all pass.
+#include <math.h>
 #include <stdio.h>
 #include <string.h>
 #include <string>
@@ -199,6 +200,55 @@ static void CoherenceAndErrors(void)
  Report("MaxPooling positions and backward",ok);
 }
 
+// the functions that only the GPU class of the reference declares (cuda/ctensormath.cu.h:92-93, 128-134)
+static void GpuClassOnlyChecks(void)
+{
+ CTensor<type_t> a(2,2,2,2),b(2,1,2,2),cat(2,3,2,2),sa(2,2,2,2),sb(2,1,2,2);
+ for(uint32_t n=0;n<16;n++) a.SetElement(n/8,(n/4)%2,(n/2)%2,n%2,static_cast<type_t>(n));
+ for(uint32_t n=0;n<8;n++) b.SetElement(n/4,0,(n/2)%2,n%2,static_cast<type_t>(100+n));
+ CTensorMath<type_t>::ConcatecationZ(cat,a,b);
+ bool ok=cat.GetElement(1,1,1,0)==a.GetElement(1,1,1,0) && cat.GetElement(1,2,0,1)==b.GetElement(1,0,0,1);
+ CTensorMath<type_t>::SplitZ(sa,sb,cat);
+ ok=ok && sa.Compare(a,"",false) && sb.Compare(b,"",false);
+ Report("ConcatecationZ / SplitZ round trip",ok);
+
+ CTensor<uint32_t> step(2,1,1,1);
+ step.SetElement(0,0,0,0,0);
+ step.SetElement(1,0,0,0,3);
+ CTensor<type_t> x(2,1,2,2),y(2,1,2,2);
+ x.Fill(1);
+ CTensorMath<type_t>::SetTimeStep(y,x,step);
+ ok=y.GetElement(0,0,0,0)==1 && y.GetElement(0,0,0,1)==2;          // t=0: +sin 0 at even positions, +cos 0 at odd ones
+ ok=ok && fabs(y.GetElement(1,0,0,0)-(1+sin(3.0)))<1e-5;
+ Report("SetTimeStep",ok);
+
+ CTensor<type_t> mask(4,4,16,16),noise(4,4,16,16),noisy(4,4,16,16),image(4,4,16,16),alpha(4,1,1,1),beta(4,1,1,1);
+ CTensorMath<type_t>::CreateDropOutMatrix(mask,static_cast<type_t>(0.5));
+ uint32_t kept=0;
+ ok=true;
+ for(uint32_t n=0;n<4096;n++)
+ {
+  type_t v=mask.GetElement(n/1024,(n/256)%4,(n/16)%16,n%16);
+  if (v!=0) {kept++;ok=ok && v==2;}
+ }
+ Report("CreateDropOutMatrix keeps about half, scaled by 1/(1-p)",ok && kept>1850 && kept<2250);
+ image.Fill(2);alpha.Fill(static_cast<type_t>(0.5));beta.Fill(static_cast<type_t>(0.25));
+ CTensorMath<type_t>::GetNoiseImageAndNoise(noisy,noise,image,alpha,beta);
+ double sum=0,sum2=0;
+ ok=true;
+ for(uint32_t n=0;n<4096;n++)
+ {
+  type_t e=noise.GetElement(n/1024,(n/256)%4,(n/16)%16,n%16),v=noisy.GetElement(n/1024,(n/256)%4,(n/16)%16,n%16);
+  sum+=e;sum2+=e*e;
+  ok=ok && fabs(v-(1+0.25*e))<1e-6;
+ }
+ Report("GetNoiseImageAndNoise: standard normal noise, blended image",ok && fabs(sum/4096)<0.08 && fabs(sum2/4096-1)<0.12);
+ CTensorMath<type_t>::SetNormalNoise(noise);
+ sum=0;
+ for(uint32_t n=0;n<4096;n++) sum+=noise.GetElement(n/1024,(n/256)%4,(n/16)%16,n%16);
+ Report("SetNormalNoise",fabs(sum/4096)<0.08);
+}
+
 int main(void)
 {
  try
@@ -210,6 +260,7 @@ int main(void)
   BackwardConvolutionCheck();
   SummXYCheck();
   CoherenceAndErrors();
+  GpuClassOnlyChecks();
  }
  catch(const char *message)
  {

@@ -4,6 +4,7 @@
 #ifndef C_TENSOR_MATH_CU_H
 #define C_TENSOR_MATH_CU_H
 
+#include <stdlib.h>
 #include <type_traits>
 
 #include "ctensor.cu.h"
@@ -216,6 +217,56 @@ class CTensorMath
    mt_tensor o=cTensor.Device(true);
    mi355::Check(mt_signum(&o));
    cTensor.SetDeviceOnChange();
+  }
+  // the functions below exist in the GPU class only (cuda/ctensormath.cu.h:92-93, 128-134)
+  static void ConcatecationZ(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_InputA,const CTensor<type_t> &cTensor_InputB)
+  {
+   OnlyFloat();
+   mt_tensor a=cTensor_InputA.Device(true),b=cTensor_InputB.Device(true),o=cTensor_Output.Device(false);
+   mi355::Check(mt_concatecation_z(&o,&a,&b));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void SplitZ(CTensor<type_t> &cTensor_OutputA,CTensor<type_t> &cTensor_OutputB,const CTensor<type_t> &cTensor_Input)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),a=cTensor_OutputA.Device(false),b=cTensor_OutputB.Device(false);
+   mi355::Check(mt_split_z(&a,&b,&i));
+   cTensor_OutputA.SetDeviceOnChange();
+   cTensor_OutputB.SetDeviceOnChange();
+  }
+  static void SetTimeStep(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,const CTensor<uint32_t> &cTensor_TimeStep)
+  {
+   OnlyFloat();
+   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false),t=cTensor_TimeStep.Device(true);
+   mt_u32_tensor ts;
+   ts.p=reinterpret_cast<uint32_t*>(t.p);
+   ts.w=t.w;ts.z=t.z;ts.y=t.y;ts.x=t.x;
+   mi355::Check(mt_set_time_step(&o,&i,&ts));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  // the reference seeds its generator with rand() at each call (cuda/ctensormath.cu.h:3117, 3169, 3257); so does this
+  static void CreateDropOutMatrix(CTensor<type_t> &cTensor_Output,type_t drop_out)
+  {
+   OnlyFloat();
+   mt_tensor o=cTensor_Output.Device(false);
+   mi355::Check(mt_create_drop_out_matrix(&o,drop_out,static_cast<uint64_t>(rand())));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void SetNormalNoise(CTensor<type_t> &cTensor_Output)
+  {
+   OnlyFloat();
+   mt_tensor o=cTensor_Output.Device(false);
+   mi355::Check(mt_set_normal_noise(&o,static_cast<uint64_t>(rand())));
+   cTensor_Output.SetDeviceOnChange();
+  }
+  static void GetNoiseImageAndNoise(CTensor<type_t> &cTensor_NoisyImage,CTensor<type_t> &cTensor_Noise,const CTensor<type_t> &cTensor_Image,const CTensor<type_t> &cTensor_SqrtAlphaBar,const CTensor<type_t> &cTensor_SqrtOneMinusAlphaBar)
+  {
+   OnlyFloat();
+   mt_tensor im=cTensor_Image.Device(true),sa=cTensor_SqrtAlphaBar.Device(true),sb=cTensor_SqrtOneMinusAlphaBar.Device(true);
+   mt_tensor ni=cTensor_NoisyImage.Device(false),no=cTensor_Noise.Device(false);
+   mi355::Check(mt_get_noise_image_and_noise(&ni,&no,&im,&sa,&sb,static_cast<uint64_t>(rand())));
+   cTensor_Noise.SetDeviceOnChange();
+   cTensor_NoisyImage.SetDeviceOnChange();
   }
   static void Adam(CTensor<type_t> &cTensor_Weight,CTensor<type_t> &cTensor_dWeight,CTensor<type_t> &cTensor_M,CTensor<type_t> &cTensor_V,uint32_t batch_size,double speed,double beta1,double beta2,double epsilon,double iteration)
   {

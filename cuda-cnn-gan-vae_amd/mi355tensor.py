@@ -132,9 +132,9 @@ class Graph:
 class CTensor:
     """Device-resident [W,Z,Y,X] fp32 tensor (uint32 pairs for pooling positions when `pos` is set)."""
 
-    def __init__(self, size_w=1, size_z=1, size_y=1, size_x=1, pos=False):
+    def __init__(self, size_w=1, size_z=1, size_y=1, size_x=1, pos=False, u32=False):
         self.shape = (int(size_w), int(size_z), int(size_y), int(size_x))
-        self.pos = pos
+        self.pos, self.u32 = pos, u32     # u32: CTensor<uint32_t> (time steps)
         self.item = 8 if pos else 4
         self.ptr = C.c_void_p()
         self.owned = True
@@ -157,17 +157,17 @@ class CTensor:
     def wrap(cls, ptr, shape):
         """Borrow device memory owned by someone else (e.g. a torch tensor's data_ptr())."""
         t = cls.__new__(cls)
-        t.shape, t.pos, t.item, t.ptr, t.owned = tuple(int(s) for s in shape), False, 4, C.c_void_p(ptr), False
+        t.shape, t.pos, t.u32, t.item, t.ptr, t.owned = tuple(int(s) for s in shape), False, False, 4, C.c_void_p(ptr), False
         return t
 
     def upload(self, a):
-        a = np.ascontiguousarray(a, dtype=np.uint32 if self.pos else np.float32)
+        a = np.ascontiguousarray(a, dtype=np.uint32 if self.pos or self.u32 else np.float32)
         assert a.size == self.count * (2 if self.pos else 1)
         if a.size:
             call("mt_copy_h2d", self.ptr, C.c_void_p(a.ctypes.data), C.c_size_t(a.nbytes))
 
     def numpy(self):
-        out = np.empty(self.shape + ((2,) if self.pos else ()), np.uint32 if self.pos else np.float32)
+        out = np.empty(self.shape + ((2,) if self.pos else ()), np.uint32 if self.pos or self.u32 else np.float32)
         if out.size:
             call("mt_copy_d2h", C.c_void_p(out.ctypes.data), self.ptr, C.c_size_t(out.nbytes))
         else:
@@ -355,6 +355,32 @@ class CTensorMath:
     def Adam(weight, dweight, m, v, batch_size, speed, beta1, beta2, epsilon, iteration):
         call("mt_adam", _d(weight), _d(dweight), _d(m), _d(v), _u(batch_size), C.c_double(speed), C.c_double(beta1), C.c_double(beta2),
              C.c_double(epsilon), C.c_double(iteration))
+
+
+    # ---- functions of the reference's GPU class only (cuda/ctensormath.cu.h:92-93, 128-134); seeds are explicit here
+    @staticmethod
+    def ConcatecationZ(out, a, b):
+        call("mt_concatecation_z", _d(out), _d(a), _d(b))
+
+    @staticmethod
+    def SplitZ(out_a, out_b, inp):
+        call("mt_split_z", _d(out_a), _d(out_b), _d(inp))
+
+    @staticmethod
+    def SetTimeStep(out, inp, time_step):
+        call("mt_set_time_step", _d(out), _d(inp), _d(time_step))
+
+    @staticmethod
+    def CreateDropOutMatrix(out, drop_out, seed):
+        call("mt_create_drop_out_matrix", _d(out), _f(drop_out), C.c_uint64(seed))
+
+    @staticmethod
+    def SetNormalNoise(out, seed):
+        call("mt_set_normal_noise", _d(out), C.c_uint64(seed))
+
+    @staticmethod
+    def GetNoiseImageAndNoise(noisy_image, noise, image, sqrt_alpha_bar, sqrt_one_minus_alpha_bar, seed):
+        call("mt_get_noise_image_and_noise", _d(noisy_image), _d(noise), _d(image), _d(sqrt_alpha_bar), _d(sqrt_one_minus_alpha_bar), C.c_uint64(seed))
 
 
 class CTensorApplyFunc:

@@ -45,6 +45,12 @@ typedef struct {
   uint32_t w, z, y, x;
 } mt_pos_tensor;
 
+/* CTensor<uint32_t> (time steps of the diffusion model, cuda/ctensormath.cu.h:3064) */
+typedef struct {
+  uint32_t *p; /* device pointer */
+  uint32_t w, z, y, x;
+} mt_u32_tensor;
+
 enum {
   MT_OK = 0,
   MT_E_NO_KERNELS = 1,   /* kernel_amount == 0                                  (cpu/ctensorconv.h:88,199,321)  */
@@ -205,6 +211,24 @@ int mt_fill_many(uint32_t count, const mt_tensor *const *tensors, float value);
  * the other layers) as one launch: mt_adam on (weight[i], dweight[i], m[i], v[i]) for i < count, same arithmetic. */
 int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor *const *dweight, const mt_tensor *const *m,
                  const mt_tensor *const *v, uint32_t batch_size, double speed, double beta1, double beta2, double epsilon, double iteration);
+
+/* ---- functions that only the GPU class of the reference has (no CPU body) ----
+ * CTensorMath::ConcatecationZ, cuda/ctensormath.cu.h:473-533: output[w][z] = z < Za ? a[w % Wa][z] : b[w % Wb][z - Za]. */
+int mt_concatecation_z(const mt_tensor *output, const mt_tensor *input_a, const mt_tensor *input_b);
+/* CTensorMath::SplitZ, cuda/ctensormath.cu.h:538-598: the inverse; w runs over the input's W. */
+int mt_split_z(const mt_tensor *output_a, const mt_tensor *output_b, const mt_tensor *input);
+/* CTensorMath::SetTimeStep, cuda/ctensormath.cu.h:3029-3091: output = input + sin (even pos) or cos (odd pos) of
+ * time_step[w] / 10000^(pos/size), pos the element index within a sample; time_step is [W,1,1,1]. */
+int mt_set_time_step(const mt_tensor *output, const mt_tensor *input, const mt_u32_tensor *time_step);
+/* CTensorMath::CreateDropOutMatrix / SetNormalNoise / GetNoiseImageAndNoise, cuda/ctensormath.cu.h:3093-3262.  The
+ * reference seeds cuRAND with rand(); here the caller passes the seed and the generator is Philox4x32-10 with
+ * key = seed and counter = element index: element i of the output depends on (seed, i) only.
+ *   drop-out matrix: uniform[0,1) >= drop_out ? 1/(1-drop_out) : 0;   noise: standard normal (Box-Muller);
+ *   noisy_image = sqrt_alpha_bar[w] * image + sqrt_one_minus_alpha_bar[w] * noise. */
+int mt_create_drop_out_matrix(const mt_tensor *output, float drop_out, uint64_t seed);
+int mt_set_normal_noise(const mt_tensor *output, uint64_t seed);
+int mt_get_noise_image_and_noise(const mt_tensor *noisy_image, const mt_tensor *noise, const mt_tensor *image, const mt_tensor *sqrt_alpha_bar,
+                                 const mt_tensor *sqrt_one_minus_alpha_bar, uint64_t seed);
 
 /* ---- timing: replaces CCUDATimeSpent / CTimeStamp (cuda/ccudatimespent.cu:38-52, cuda/ctimestamp.cu:17-32) ----
  * While enabled, every kernel launch of the hot path is bracketed by two events on the work stream and its

@@ -249,6 +249,48 @@ class Oracle:
         self._call("vae_coder_output", self._p(out), C.byref(kl), self._p(mu), self._p(logvar), self._p(epsilon))
         return out, kl.value
 
+    # ---- functions of the reference's GPU class only ---------------------
+    def concatecation_z(self, a, b, out_w=None):
+        a, b = _f32(a), _f32(b)
+        out = np.zeros((out_w or max(a.shape[0], b.shape[0]), a.shape[1] + b.shape[1], a.shape[2], a.shape[3]), np.float32)
+        self._call("concatecation_z", self._p(out), self._p(a), self._p(b))
+        return out
+
+    def split_z(self, a, za, out_w=None):
+        a = _f32(a)
+        w = out_w or a.shape[0]
+        oa, ob = np.zeros((w, za) + a.shape[2:], np.float32), np.zeros((w, a.shape[1] - za) + a.shape[2:], np.float32)
+        self._call("split_z", self._p(oa), self._p(ob), self._p(a))
+        return oa, ob
+
+    def set_time_step(self, a, time_step):
+        a, t = _f32(a), np.ascontiguousarray(time_step, dtype=np.uint32).ravel()
+        out = np.zeros(a.shape, np.float32)
+        self._call("set_time_step", self._p(out), self._p(a), t.ctypes.data_as(C.POINTER(C.c_uint32)), C.c_uint32(t.size))
+        return out
+
+    def philox4x32_10(self, counter, key):
+        c, k, out = (C.c_uint32 * 4)(*counter), (C.c_uint32 * 2)(*key), (C.c_uint32 * 4)()
+        self.lib.oracle_philox4x32_10.restype = None
+        self.lib.oracle_philox4x32_10(c, k, out)
+        return tuple(out)
+
+    def create_drop_out_matrix(self, shape, drop_out, seed):
+        out = np.zeros(shape, np.float32)
+        self._call("create_drop_out_matrix", self._p(out), C.c_float(drop_out), C.c_uint64(seed))
+        return out
+
+    def set_normal_noise(self, shape, seed):
+        out = np.zeros(shape, np.float32)
+        self._call("set_normal_noise", self._p(out), C.c_uint64(seed))
+        return out
+
+    def get_noise_image_and_noise(self, image, sqrt_alpha_bar, sqrt_one_minus_alpha_bar, seed):
+        image, sa, sb = _f32(image), _f32(sqrt_alpha_bar), _f32(sqrt_one_minus_alpha_bar)
+        noisy, noise = np.zeros(image.shape, np.float32), np.zeros(image.shape, np.float32)
+        self._call("get_noise_image_and_noise", self._p(noisy), self._p(noise), self._p(image), self._p(sa), self._p(sb), C.c_uint64(seed))
+        return noisy, noise
+
     # ---- activations --------------------------------------------------
     def apply_func(self, a, func, differential=False):
         a = _f32(a)

@@ -529,6 +529,118 @@ int oracle_vae_coder_output(ot_tensor *out, float *kl, const ot_tensor *mu, cons
 }
 
 /* ------------------------------------------------------------------------ */
+/* Functions that exist only in the GPU class of the reference (no CPU body to follow): restated from the CUDA kernels. */
+
+/* cuda/ctensormath.cu.h:473-533: out[w][z] = z < Za ? a[w % Wa][z] : b[w % Wb][z - Za], w over the output's W */
+int oracle_concatecation_z(ot_tensor *out, const ot_tensor *a, const ot_tensor *b) {
+  if (out->x != a->x || out->x != b->x || out->y != a->y || out->y != b->y || out->z != a->z + b->z) return ORACLE_E_SHAPE;
+  size_t yx = (size_t)out->y * out->x;
+  for (uint32_t w = 0; w < out->w; w++)
+    for (uint32_t z = 0; z < out->z; z++) {
+      const float *src = z < a->z ? a->p + ((size_t)(w % a->w) * a->z + z) * yx : b->p + ((size_t)(w % b->w) * b->z + (z - a->z)) * yx;
+      memcpy(out->p + ((size_t)w * out->z + z) * yx, src, yx * sizeof(float));
+    }
+  return ORACLE_OK;
+}
+
+/* cuda/ctensormath.cu.h:538-598: the inverse; w runs over the input's W, outputs are indexed by w % their W */
+int oracle_split_z(ot_tensor *out_a, ot_tensor *out_b, const ot_tensor *in) {
+  if (out_a->x != in->x || out_b->x != in->x || out_a->y != in->y || out_b->y != in->y || out_a->z + out_b->z != in->z) return ORACLE_E_SHAPE;
+  size_t yx = (size_t)in->y * in->x;
+  for (uint32_t w = 0; w < in->w; w++)
+    for (uint32_t z = 0; z < in->z; z++) {
+      float *dst = z < out_a->z ? out_a->p + ((size_t)(w % out_a->w) * out_a->z + z) * yx
+                                : out_b->p + ((size_t)(w % out_b->w) * out_b->z + (z - out_a->z)) * yx;
+      memcpy(dst, in->p + ((size_t)w * in->z + z) * yx, yx * sizeof(float));
+    }
+  return ORACLE_OK;
+}
+
+/* cuda/ctensormath.cu.h:3029-3059, type_t = float: pos = x + X*y + X*Y*z, size = X*Y*Z,
+ * angle = t / powf(10000, (float)pos / (float)size); even pos adds sin(angle), odd pos adds cos(angle) */
+int oracle_set_time_step(ot_tensor *out, const ot_tensor *in, const uint32_t *time_step, uint32_t time_step_w) {
+  if (!same_zyx(in, out) || in->w != out->w || time_step_w != in->w) return ORACLE_E_SHAPE;
+  uint32_t size = in->x * in->y * in->z;
+  for (uint32_t w = 0; w < in->w; w++) {
+    float t = (float)time_step[w];
+    for (uint32_t pos = 0; pos < size; pos++) {
+      float angle = t / powf(10000.0f, (float)pos / (float)size);
+      float v = in->p[(size_t)w * size + pos];
+      v += (pos & 1u) == 0 ? sinf(angle) : cosf(angle);
+      out->p[(size_t)w * size + pos] = v;
+    }
+  }
+  return ORACLE_OK;
+}
+
+/* The reference draws with cuRAND seeded by rand() (cuda/ctensormath.cu.h:3117-3123, 3169-3174, 3218-3225): no
+ * sequence to reproduce.  The generator specified here instead is Philox4x32-10 (Salmon et al., SC'11) with
+ * key = (seed low, seed high) and counter = (element index low, element index high, 0, 0), one block per element. */
+void oracle_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c0 = counter[0], c1 = counter[1], c2 = counter[2], c3 = counter[3], k0 = key[0], k1 = key[1];
+  for (int r = 0; r < 10; r++) {
+    uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+static void element_random(uint64_t seed, uint64_t index, uint32_t r[4]) {
+  uint32_t counter[4] = {(uint32_t)index, (uint32_t)(index >> 32), 0u, 0u}, key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  oracle_philox4x32_10(counter, key, r);
+}
+/* uniform in [0, 1): the top 24 bits of word 0 */
+static float element_uniform(const uint32_t r[4]) { return (float)(r[0] >> 8) * (1.0f / 16777216.0f); }
+/* standard normal by Box-Muller from words 0 and 1: sqrt(-2 ln u1) cos(2 pi u2), u1 in (0, 1], u2 in [0, 1) */
+static float element_normal(const uint32_t r[4]) {
+  float u1 = (float)((r[0] >> 8) + 1u) * (1.0f / 16777216.0f), u2 = (float)(r[1] >> 8) * (1.0f / 16777216.0f);
+  return sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2);
+}
+
+/* cuda/ctensormath.cu.h:3093-3123: out = uniform >= drop_out ? (float)(1.0 / (1.0 - drop_out)) : 0 */
+int oracle_create_drop_out_matrix(ot_tensor *out, float drop_out, uint64_t seed) {
+  size_t n = count(out);
+  float mult = (float)(1.0 / (1.0 - drop_out));
+  for (size_t i = 0; i < n; i++) {
+    uint32_t r[4];
+    element_random(seed, i, r);
+    out->p[i] = element_uniform(r) >= drop_out ? mult : 0.0f;
+  }
+  return ORACLE_OK;
+}
+
+/* cuda/ctensormath.cu.h:3143-3174 */
+int oracle_set_normal_noise(ot_tensor *out, uint64_t seed) {
+  size_t n = count(out);
+  for (size_t i = 0; i < n; i++) {
+    uint32_t r[4];
+    element_random(seed, i, r);
+    out->p[i] = element_normal(r);
+  }
+  return ORACLE_OK;
+}
+
+/* cuda/ctensormath.cu.h:3179-3262: noise as above; noisy = sqrt_alpha_bar[w] * image + sqrt_one_minus_alpha_bar[w] * noise */
+int oracle_get_noise_image_and_noise(ot_tensor *noisy, ot_tensor *noise, const ot_tensor *image, const ot_tensor *sqrt_alpha_bar,
+                                     const ot_tensor *sqrt_one_minus_alpha_bar, uint64_t seed) {
+  if (!same_zyx(noisy, noise) || noisy->w != noise->w || !same_zyx(noisy, image) || noisy->w != image->w) return ORACLE_E_SHAPE;
+  if (sqrt_alpha_bar->w != image->w || sqrt_one_minus_alpha_bar->w != image->w) return ORACLE_E_SHAPE;
+  size_t per = (size_t)image->z * image->y * image->x;
+  size_t sa = (size_t)sqrt_alpha_bar->z * sqrt_alpha_bar->y * sqrt_alpha_bar->x;
+  size_t sb = (size_t)sqrt_one_minus_alpha_bar->z * sqrt_one_minus_alpha_bar->y * sqrt_one_minus_alpha_bar->x;
+  for (uint32_t w = 0; w < image->w; w++)
+    for (size_t i = 0; i < per; i++) {
+      uint32_t r[4];
+      element_random(seed, (size_t)w * per + i, r);
+      float e = element_normal(r);
+      noise->p[(size_t)w * per + i] = e;
+      noisy->p[(size_t)w * per + i] = sqrt_alpha_bar->p[w * sa] * image->p[(size_t)w * per + i] + sqrt_one_minus_alpha_bar->p[w * sb] * e;
+    }
+  return ORACLE_OK;
+}
+
+/* ------------------------------------------------------------------------ */
 /* cpu/ctensorapplyfunc.h:111-255.  The float/double mix follows the C++
  * overload resolution of the reference with type_t=float: math calls on a
  * float argument are the float versions, bare literals such as 1.0, 0.5, 0.1

@@ -111,6 +111,21 @@ int oracle_adam(ot_tensor *weight, const ot_tensor *dweight, ot_tensor *m, ot_te
  * special cases (tests/test_oracle_math.py); the layer itself draws from an unseedable generator. */
 int oracle_vae_coder_output(ot_tensor *out, float *kl, const ot_tensor *mu, const ot_tensor *logvar, const ot_tensor *epsilon);
 
+/* ---- functions of the GPU class only (cuda/ctensormath.cu.h:473-598, 3029-3262) -----------------------------------
+ * No CPU body exists in the reference: restated from the CUDA kernels.  Concatenation and split are data movement,
+ * pinned by numpy's concatenate / slicing; the time step by its float64 closed form.  The three random fills follow
+ * the reference's formulas, but the reference draws from cuRAND seeded with rand(), a sequence nobody can reproduce:
+ * the generator is specified here (Philox4x32-10, pinned by the published known-answer vectors of Random123) and
+ * the fills are checked for their distribution; their parity with the reference's own draws is unpinned by nature. */
+int oracle_concatecation_z(ot_tensor *out, const ot_tensor *a, const ot_tensor *b);
+int oracle_split_z(ot_tensor *out_a, ot_tensor *out_b, const ot_tensor *in);
+int oracle_set_time_step(ot_tensor *out, const ot_tensor *in, const uint32_t *time_step, uint32_t time_step_w);
+void oracle_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+int oracle_create_drop_out_matrix(ot_tensor *out, float drop_out, uint64_t seed);
+int oracle_set_normal_noise(ot_tensor *out, uint64_t seed);
+int oracle_get_noise_image_and_noise(ot_tensor *noisy, ot_tensor *noise, const ot_tensor *image, const ot_tensor *sqrt_alpha_bar,
+                                     const ot_tensor *sqrt_one_minus_alpha_bar, uint64_t seed);
+
 /* ---- activations (cpu/ctensorapplyfunc.h) -------------------------------
  * func ids: 0 sigmoid, 1 ReLU, 2 GeLU, 3 LeakyReLU(0.1), 4 linear, 5 tanh;
  * add 8 for the derivative of the same function. */

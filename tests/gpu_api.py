@@ -214,6 +214,44 @@ class Gpu:
         Fused.UpSamplingConvolution(out, up_(image), up, up, up_(kernel), k, k, kz, ka, up_(bias), s, s, p, p, func)
         return out.numpy()
 
+    # ---- functions of the reference's GPU class only ---------------------------
+    def concatecation_z(self, a, b, out_w=None):
+        a, b = np.asarray(a, np.float32), np.asarray(b, np.float32)
+        out = up(np.full((out_w or max(a.shape[0], b.shape[0]), a.shape[1] + b.shape[1], a.shape[2], a.shape[3]), 7.0, np.float32))
+        CTensorMath.ConcatecationZ(out, up(a), up(b))
+        return out.numpy()
+
+    def split_z(self, a, za, out_w=None):
+        a = np.asarray(a, np.float32)
+        w = out_w or a.shape[0]
+        oa, ob = up(np.full((w, za) + a.shape[2:], 7.0, np.float32)), up(np.full((w, a.shape[1] - za) + a.shape[2:], 7.0, np.float32))
+        CTensorMath.SplitZ(oa, ob, up(a))
+        return oa.numpy(), ob.numpy()
+
+    def set_time_step(self, a, time_step):
+        a = np.asarray(a, np.float32)
+        t = CTensor(a.shape[0], 1, 1, 1, u32=True)
+        t.upload(np.asarray(time_step, np.uint32))
+        out = CTensor(*a.shape)
+        CTensorMath.SetTimeStep(out, up(a), t)
+        return out.numpy()
+
+    def create_drop_out_matrix(self, shape, drop_out, seed):
+        out = CTensor(*shape)
+        CTensorMath.CreateDropOutMatrix(out, drop_out, seed)
+        return out.numpy()
+
+    def set_normal_noise(self, shape, seed):
+        out = CTensor(*shape)
+        CTensorMath.SetNormalNoise(out, seed)
+        return out.numpy()
+
+    def get_noise_image_and_noise(self, image, sqrt_alpha_bar, sqrt_one_minus_alpha_bar, seed):
+        image = np.asarray(image, np.float32)
+        noisy, noise = CTensor(*image.shape), CTensor(*image.shape)
+        CTensorMath.GetNoiseImageAndNoise(noisy, noise, up(image), up(sqrt_alpha_bar), up(sqrt_one_minus_alpha_bar), seed)
+        return noisy.numpy(), noise.numpy()
+
     def fill_many(self, arrays, value):
         ts = [up(a) for a in arrays]
         Fused.FillMany(ts, value)

@@ -386,6 +386,52 @@ def test_resampling_and_pooling_2x2_bit_exact(gpu, oracle, shape):
         assert np.array_equal(gpu.max_pooling_backward(d, o[1], 2, 2, a.shape), oracle.max_pooling_backward(d, o[1], 2, 2, a.shape))
 
 
+@pytest.mark.parametrize("shape", [(3, 2, 4, 8), (2, 5, 3, 7), (1, 1, 1, 1), (4, 16, 32, 32)])
+def test_concatenation_and_split_bit_exact(gpu, oracle, shape):
+    """ConcatecationZ / SplitZ (cuda/ctensormath.cu.h:473-598): data movement, with and without batch broadcast."""
+    w, z, y, x = shape
+    a, b = U(1, w, z, y, x), U(2, w, z + 1, y, x)
+    assert np.array_equal(gpu.concatecation_z(a, b), oracle.concatecation_z(a, b))
+    assert np.array_equal(gpu.concatecation_z(a, b[:1]), oracle.concatecation_z(a, b[:1]))
+    assert np.array_equal(gpu.concatecation_z(a[:1], b, out_w=w), oracle.concatecation_z(a[:1], b, out_w=w))
+    cat = oracle.concatecation_z(a, b)
+    for got, want in zip(gpu.split_z(cat, z), oracle.split_z(cat, z)):
+        assert np.array_equal(got, want)
+    import mi355tensor as mt
+    with pytest.raises(mt.TensorError) as e:
+        gpu.concatecation_z(a, U(3, w, z, y, x + 1))
+    assert e.value.code == 5
+
+
+def test_set_time_step(gpu, oracle):
+    """SetTimeStep (cuda/ctensormath.cu.h:3029-3091).  The angle t / 10000^(pos/size) reaches 1000 and carries the
+    rounding of powf (1e-7 relative, so 1e-4 absolute): that much of the sine is not determined in fp32."""
+    x = U(1, 5, 3, 8, 8)
+    steps = np.array([0, 1, 50, 500, 999], np.uint32)
+    got, want = gpu.set_time_step(x, steps), oracle.set_time_step(x, steps)
+    assert np.max(np.abs(got - want)) <= 4e-4
+    assert np.max(np.abs(got[:3] - want[:3])) <= 2e-5          # small angles: no such amplification
+    odd = U(2, 2, 1, 3, 5)                                      # a sample size that is no multiple of the block
+    assert np.max(np.abs(gpu.set_time_step(odd, [3, 4]) - oracle.set_time_step(odd, [3, 4]))) <= 2e-5
+
+
+def test_random_fills_follow_the_specified_generator(gpu, oracle):
+    """Drop-out matrix, normal noise and the noisy image of the diffusion model: element i is a function of (seed, i)
+    through Philox4x32-10, so the device and the oracle produce the same tensors (the mask bit for bit, the normal
+    draws up to the device's logf / cosf)."""
+    for shape in ((3, 4, 16, 16), (1, 1, 1, 5), (2, 3, 7, 9)):
+        for p in (0.0, 0.25, 0.5):
+            assert np.array_equal(gpu.create_drop_out_matrix(shape, p, 77), oracle.create_drop_out_matrix(shape, p, 77))
+        close(gpu.set_normal_noise(shape, 2 ** 40 + 3), oracle.set_normal_noise(shape, 2 ** 40 + 3), 2e-6)
+        image = U(3, *shape)
+        sa, sb = U(4, shape[0], 1, 1, 1) * 0.5 + 0.5, U(5, shape[0], 1, 1, 1) * 0.5 + 0.5
+        got, want = gpu.get_noise_image_and_noise(image, sa, sb, 9), oracle.get_noise_image_and_noise(image, sa, sb, 9)
+        close(got[0], want[0], 2e-6)
+        close(got[1], want[1], 2e-6)
+    big = gpu.set_normal_noise((8, 16, 64, 64), 1).astype(np.float64)      # 524288 draws on the device
+    assert abs(big.mean()) <= 4 / np.sqrt(big.size) and abs(big.var() - 1.0) <= 4 * np.sqrt(2.0 / big.size)
+
+
 @pytest.mark.parametrize("name", sorted(oracle_api.FUNC))
 def test_activations(gpu, oracle, name):
     x = np.concatenate([U(1, 4000) * 12, U(2, 2000) * 40, np.array([0.0, -0.0, 30, -30, 30.000002, -30.000002], np.float32)]).reshape(1, 1, 1, -1)

@@ -229,3 +229,61 @@ def test_vae_coder_output_closed_form(oracle):
     assert np.allclose(out, np.exp(5.0), rtol=1e-6)
     out, _ = oracle.vae_coder_output(zero, zero - 50, zero + 1)
     assert np.allclose(out, np.exp(-5.0), rtol=1e-6)
+
+
+# ---- functions that only the reference's GPU class has (cuda/ctensormath.cu.h:473-598, 3029-3262) ----------------
+
+def test_concatenation_and_split_are_numpy_slicing(oracle):
+    a, b = U(1, 3, 2, 4, 5), U(2, 3, 3, 4, 5)
+    cat = oracle.concatecation_z(a, b)
+    assert np.array_equal(cat, np.concatenate([a, b], axis=1))
+    # an operand with fewer samples repeats by w % W
+    one = oracle.concatecation_z(a, b[:1])
+    assert np.array_equal(one, np.concatenate([a, np.repeat(b[:1], 3, axis=0)], axis=1))
+    sa, sb = oracle.split_z(cat, 2)
+    assert np.array_equal(sa, a) and np.array_equal(sb, b)
+    with pytest.raises(Exception):
+        oracle.concatecation_z(a, U(3, 3, 3, 4, 6))
+
+
+def test_time_step_closed_form(oracle):
+    x = U(1, 3, 2, 4, 6)
+    steps = np.array([0, 7, 999], np.uint32)
+    got = oracle.set_time_step(x, steps)
+    size = 2 * 4 * 6
+    pos = np.arange(size, dtype=np.float64)
+    for w, t in enumerate(steps):
+        angle = float(t) / 10000.0 ** (pos / size)
+        want = x[w].ravel().astype(np.float64) + np.where(pos % 2 == 0, np.sin(angle), np.cos(angle))
+        # the angle is a float quotient of up to 1000: its rounding (6e-5) is the error of the sine
+        assert np.max(np.abs(got[w].ravel() - want)) <= 2e-4
+    assert np.array_equal(got[0].ravel()[0::2], x[0].ravel()[0::2])        # t = 0: sin 0 added to even positions
+    assert np.allclose(got[0].ravel()[1::2], x[0].ravel()[1::2] + 1.0)     # and cos 0 to odd ones
+
+
+def test_philox_known_answers(oracle):
+    """Philox4x32-10 against the known-answer vectors published with Random123 (kat_vectors)."""
+    assert oracle.philox4x32_10((0, 0, 0, 0), (0, 0)) == (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)
+    assert oracle.philox4x32_10((0xffffffff,) * 4, (0xffffffff,) * 2) == (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)
+    assert oracle.philox4x32_10((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0)) == (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)
+
+
+def test_random_fills_have_the_reference_distributions(oracle):
+    shape = (4, 8, 64, 64)   # 131072 draws
+    n = float(np.prod(shape))
+    for p in (0.0, 0.3, 0.5):
+        d = oracle.create_drop_out_matrix(shape, p, 11)
+        kept = d != 0
+        assert np.all(d[kept] == np.float32(1.0 / (1.0 - p)))
+        assert abs(kept.mean() - (1.0 - p)) <= 4 * np.sqrt(p * (1 - p) / n) + 1e-12          # four standard errors
+    assert not np.array_equal(oracle.create_drop_out_matrix(shape, 0.3, 11), oracle.create_drop_out_matrix(shape, 0.3, 12))
+    z = oracle.set_normal_noise(shape, 5).astype(np.float64)
+    assert abs(z.mean()) <= 4 / np.sqrt(n) and abs(z.var() - 1.0) <= 4 * np.sqrt(2.0 / n)
+    assert abs((z ** 3).mean()) <= 4 * np.sqrt(15.0 / n) and abs((z ** 4).mean() - 3.0) <= 4 * np.sqrt(96.0 / n)
+    assert abs((np.abs(z) < 1.0).mean() - 0.682689) <= 4 * np.sqrt(0.68 * 0.32 / n)
+    assert abs(np.corrcoef(z.ravel()[:-1], z.ravel()[1:])[0, 1]) <= 4 / np.sqrt(n)           # neighbours are independent
+    image = U(3, *shape)
+    sa, sb = U(4, 4, 1, 1, 1) * 0.5 + 0.5, U(5, 4, 1, 1, 1) * 0.5 + 0.5
+    noisy, noise = oracle.get_noise_image_and_noise(image, sa, sb, 5)
+    assert np.array_equal(noise, oracle.set_normal_noise(shape, 5))                          # the same draws per element
+    assert np.allclose(noisy, sa * image + sb * noise, rtol=0, atol=1e-6)
