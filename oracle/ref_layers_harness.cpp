@@ -13,6 +13,11 @@
 // Chain B: input [B,8,4,4]   -> BackConvolution 4x4 s2 p1 to 3 channels -> Tangence
 // Chain C: input [B,4,5,5]   -> BatchNormalization (training) -> ReLU            (layers_mi355 only: the reference's
 //          batch-norm layer does not compile on its own CPU classes, netlayer/cnetlayerbatchnormalization.cu.h:655)
+// Chain D: input [B,4,4,4]   -> UpSampling 2x2 -> AveragePooling 4x4, forward and backward
+// Chain E: inputs [B,2,4,4] and [B,3,4,4] -> Concatenator -> TimeEmbedding       (layers_mi355 only: ConcatecationZ and
+//          SetTimeStep exist in the reference's GPU tensor class only)
+// Chain F: input [B,4,8,8]   -> Linear function -> MaxPooling 2x2, forward and backward           (layers_mi355 only: the layer names the
+//          position type CTensorMath<type_t>::SPos, which the CPU class does not nest)
 // Each chain: TrainingStart, Forward, SetOutputError, TrainingBackward, TrainingUpdateWeight (gradient descent), Save.
 #include <math.h>
 #include <stdint.h>
@@ -36,8 +41,13 @@
 #include "netlayer/cnetlayerbackconvolution.cu.h"
 #include "netlayer/cnetlayerlinear.cu.h"
 #include "netlayer/cnetlayerfunction.cu.h"
+#include "netlayer/cnetlayerupsampling.cu.h"
+#include "netlayer/cnetlayeraveragepooling.cu.h"
 #ifndef USE_CPU
 #include "netlayer/cnetlayerbatchnormalization.cu.h"
+#include "netlayer/cnetlayerconcatenator.cu.h"
+#include "netlayer/cnetlayertimeembedding.cu.h"
+#include "netlayer/cnetlayermaxpooling.cu.h"
 #endif
 
 namespace SYSTEM
@@ -219,7 +229,75 @@ static void ChainB(void)
  DumpStream("B.tconv_updated",saved,8*sizeof(int32_t),2);
 }
 
+// Chain D: resampling layers, forward and backward (no weights)
+static void ChainD(void)
+{
+ CNetLayerConvolutionInput<type_t> input(4,4,4,BATCH);
+ CNetLayerUpSampling<type_t> up(2,2,&input,BATCH);
+ CNetLayerAveragePooling<type_t> avg(4,4,&up,BATCH);
+ CTensor<type_t> image(BATCH,4,4,4);
+ FillTensor(image,1.0);
+ input.SetOutput(image);
+ INetLayer<type_t> *layers[3]={&input,&up,&avg};
+ for(int n=0;n<3;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+ for(int n=0;n<3;n++) layers[n]->Forward();
+ Dump("D.input",image);
+ Dump("D.upsampling",up.GetOutputTensor());
+ Dump("D.average",avg.GetOutputTensor());
+ CTensor<type_t> error(BATCH,4,2,2);
+ FillTensor(error,0.5);
+ avg.SetOutputError(error);
+ for(int n=2;n>=1;n--) layers[n]->TrainingBackward(true);
+ Dump("D.delta_average",avg.GetDeltaTensor());
+ Dump("D.delta_upsampling",up.GetDeltaTensor());
+}
+
 #ifndef USE_CPU
+// Chain E: layers whose tensor functions exist in the GPU class only: two inputs -> Concatenator -> TimeEmbedding
+static void ChainE(void)
+{
+ CNetLayerConvolutionInput<type_t> input_a(2,4,4,BATCH),input_b(3,4,4,BATCH);
+ CNetLayerConcatenator<type_t> cat(&input_a,&input_b,BATCH);
+ CNetLayerTimeEmbedding<type_t> time(&cat,BATCH);
+ CTensor<type_t> a(BATCH,2,4,4),b(BATCH,3,4,4);
+ FillTensor(a,1.0);
+ FillTensor(b,1.0);
+ input_a.SetOutput(a);
+ input_b.SetOutput(b);
+ INetLayer<type_t> *layers[4]={&input_a,&input_b,&cat,&time};
+ for(int n=0;n<4;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+ CTensor<type_t> steps(BATCH,1,1,1);
+ for(uint32_t w=0;w<BATCH;w++) {time.SetTimeStep(w,w*7);steps.SetElement(w,0,0,0,static_cast<type_t>(w*7));}
+ for(int n=0;n<4;n++) layers[n]->Forward();
+ Dump("E.a",a);
+ Dump("E.b",b);
+ Dump("E.steps",steps);
+ Dump("E.concatenated",cat.GetOutputTensor());
+ Dump("E.time",time.GetOutputTensor());
+}
+
+// Chain F: the max-pooling layer keeps a CTensor<CTensorMath<type_t>::SPos>, a type only the GPU class nests
+static void ChainF(void)
+{
+ CNetLayerConvolutionInput<type_t> input(4,8,8,BATCH);
+ CNetLayerFunction<type_t> pass(NNeuron::NEURON_FUNCTION_LINEAR,&input,BATCH);   // keeps the error it is handed (derivative 1)
+ CNetLayerMaxPooling<type_t> pool(2,2,&pass,BATCH);
+ CTensor<type_t> image(BATCH,4,8,8);
+ FillTensor(image,1.0);
+ input.SetOutput(image);
+ INetLayer<type_t> *layers[3]={&input,&pass,&pool};
+ for(int n=0;n<3;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+ for(int n=0;n<3;n++) layers[n]->Forward();
+ Dump("F.input",image);
+ Dump("F.maxpool",pool.GetOutputTensor());
+ CTensor<type_t> error(BATCH,4,4,4);
+ FillTensor(error,0.5);
+ Dump("F.error",error);
+ pool.SetOutputError(error);
+ pool.TrainingBackward(true);
+ Dump("F.prev_error",pass.GetDeltaTensor());
+}
+
 static void ChainC(void)
 {
  CNetLayerConvolutionInput<type_t> input(4,5,5,BATCH);
@@ -265,8 +343,11 @@ int main(int argc,char **argv)
  {
   ChainA();
   ChainB();
+  ChainD();
 #ifndef USE_CPU
   ChainC();
+  ChainE();
+  ChainF();
 #endif
  }
  catch(const char *message)

@@ -77,3 +77,18 @@ def test_reference_batchnorm_layer_matches_the_oracle_sequence(dumps, oracle):
     assert rel_err(gpu["C.relu"], oracle.apply_func(want["out"], "relu")) <= 1e-4
     delta = oracle.tensor_item_production(err, oracle.apply_func(want["out"], "relu", differential=True))
     assert rel_err(gpu["C.delta_bn"], delta) <= 1e-4
+
+
+def test_reference_layers_of_the_gpu_class_only_match_the_oracle(dumps, oracle):
+    """Concatenator, time embedding and max pooling build on the reference's GPU tensor class only; their runs on the
+    drop-in classes are checked against the oracle (and the resampling chain D is among the shared keys above)."""
+    gpu, cpu = dumps
+    assert "D.average" in cpu and "D.delta_upsampling" in cpu
+    cat = oracle.concatecation_z(gpu["E.a"], gpu["E.b"])
+    assert np.array_equal(gpu["E.concatenated"], cat)
+    steps = gpu["E.steps"].ravel().astype(np.uint32)
+    assert steps.max() == 35
+    assert np.max(np.abs(gpu["E.time"] - oracle.set_time_step(cat, steps))) <= 2e-5
+    pooled, pos = oracle.max_pooling(gpu["F.input"], 2, 2)
+    assert np.array_equal(gpu["F.maxpool"], pooled)
+    assert np.array_equal(gpu["F.prev_error"], oracle.max_pooling_backward(gpu["F.error"], pos, 2, 2, gpu["F.input"].shape))
