@@ -48,6 +48,17 @@
 #include "netlayer/cnetlayerconcatenator.cu.h"
 #include "netlayer/cnetlayertimeembedding.cu.h"
 #include "netlayer/cnetlayermaxpooling.cu.h"
+// the remaining layers are only compiled: every member function of each is instantiated on the drop-in classes
+#include "netlayer/cnetlayermaxdepooling.cu.h"
+#include "netlayer/cnetlayerdropout.cu.h"
+#include "netlayer/cnetlayersplitter.cu.h"
+#include "netlayer/cnetlayervaecoderoutput.cu.h"
+#include "netlayer/cnetlayersoftmax.cu.h"
+template class CNetLayerMaxDePooling<float>;
+template class CNetLayerDropOut<float>;
+template class CNetLayerSplitter<float>;
+template class CNetLayerVAECoderOutput<float>;
+template class CNetLayerSoftMax<float>;
 #endif
 
 namespace SYSTEM
