@@ -948,6 +948,17 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   return rc == MT_OK ? mt_apply_func(out, out, func) : rc;
 }
 
+// Whether the weight gradient's image operand can use fixed per-thread offsets (SrcWgradImageFixed): the output
+// pixels must tile the k step for the number of pixels a thread loads in the block tile that will be chosen.
+bool wgrad_image_fixed(uint32_t M, uint32_t N, uint32_t batches, const mt_tensor *delta, const mt_tensor *image, int32_t kz, uint32_t per, int32_t px,
+                       int32_t py) {
+  if (px < 0 || py < 0) return false;
+  const Tile tile = pick_tile(M, N, batches);
+  const uint32_t pixels = (tile == T64x64 ? 64u : 128u) * BK / THREADS;
+  const size_t span = (size_t)per * kz * image->y * image->x + (size_t)py * image->x + px;
+  return SrcWgradImageFixed::fits(delta->y, delta->x, pixels) && mt::fits_buffer(span);
+}
+
 int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
           const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py, bool bias_too) {
   if (mt::bad(dk) || mt::bad(db) || mt::bad(image) || mt::bad(delta)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
@@ -977,7 +988,15 @@ int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t
     Epilogue ep{};
     ep.C = dk->p; ep.row_stride = dk->x; ep.inner = ncol; ep.g_stride = 0; ep.accumulate = true;
     ep.bt.wmod = dk->w; ep.bt.stride = (size_t)dk->z * dk->y * dk->x;
-    if ((rc = with_row_k(delta->p, DHW, ka, DHW, abt, [&](auto a) { return launch(name, a, b, ep, ka, ncol, DHW, dk->w); }))) return rc;
+    if (wgrad_image_fixed(ka, ncol, dk->w, delta, image, kz, 1, px, py)) {
+      SrcWgradImageFixed bf{};
+      bf.p = b.p; bf.C = b.C; bf.H = b.H; bf.W = b.W; bf.KY = b.KY; bf.KX = b.KX; bf.OW = b.OW; bf.OH = 0; bf.R = b.R; bf.K = b.K;
+      bf.sy = sy; bf.sx = sx; bf.py = py; bf.px = px; bf.bt = b.bt;
+      rc = with_row_k(delta->p, DHW, ka, DHW, abt, [&](auto a) { return launch(name, a, bf, ep, ka, ncol, DHW, dk->w); });
+    } else {
+      rc = with_row_k(delta->p, DHW, ka, DHW, abt, [&](auto a) { return launch(name, a, b, ep, ka, ncol, DHW, dk->w); });
+    }
+    if (rc) return rc;
   }
   if (!bias_too) return MT_OK;
   if (db->y != 1 || db->x != 1) return mt::fail(MT_E_ARGUMENT, "%s: bias gradient must be [W,Z,1,1]", name);
@@ -1063,7 +1082,14 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     ep.C = dk->p; ep.row_stride = dk->x; ep.accumulate = true;
   }
   if (DHW % 4 == 0 && ((uintptr_t)delta->p & 15u) == 0) {
-    rc = launch(name, a, b, ep, ka, ncol, per * DHW, groups);
+    if (wgrad_image_fixed(ka, ncol, groups, delta, image, kz, per, px, py)) {
+      SrcWgradImageFixed bf{};
+      bf.p = b.p; bf.C = b.C; bf.H = b.H; bf.W = b.W; bf.KY = b.KY; bf.KX = b.KX; bf.OW = b.OW; bf.OH = b.OH; bf.R = b.R; bf.K = b.K;
+      bf.sy = sy; bf.sx = sx; bf.py = py; bf.px = px; bf.bt = b.bt;
+      rc = launch(name, a, bf, ep, ka, ncol, per * DHW, groups);
+    } else {
+      rc = launch(name, a, b, ep, ka, ncol, per * DHW, groups);
+    }
   } else {
     SrcRowK<false> as{};
     as.p = a.p; as.ld = a.ld; as.R = a.R; as.K = a.K; as.seg = a.seg; as.seg_stride = a.seg_stride; as.bt = a.bt;

@@ -419,6 +419,73 @@ struct SrcWgradImage {
   }
 };
 
+// The same view when the 16 pixels of a k step are consecutive pixels of one output row (OW % 16 == 0) or a whole
+// number of output rows of one image (16 % OW == 0 and OH*OW % 16 == 0), and OW is a multiple of the E pixels a thread
+// loads: those pixels then keep their place inside the step's block of pixels, so their byte offsets relative to the
+// block's first pixel are computed once.  A step moves the block origin (scalar unit) and re-tests the image borders:
+// one test for the row, one per pixel for the column.  K is a multiple of 16 here, every step is complete.
+struct SrcWgradImageFixed {
+  static constexpr bool K_CONTIG = false;
+  const float *p;
+  uint32_t C, H, W, KY, KX, OW, R, K;
+  int32_t sy, sx, py, px;
+  Batch bt;
+  uint32_t OH = 0;  // > 0: k runs over the pixels of several images in turn
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff;       // byte offset of the thread's first pixel for the block origin (image 0, row 0, column 0), from p - bias
+  int32_t iyc, ixc;    // input row / column of that pixel for that origin
+  uint32_t oy, ox, woff, soff;
+  int32_t Y, X;        // input row / column displacement of the current origin
+  static __host__ __device__ bool fits(uint32_t OH_, uint32_t OW_, uint32_t e) {
+    return OW_ % e == 0 && (OW_ % BK == 0 || (BK % OW_ == 0 && (OH_ * OW_) % BK == 0));
+  }
+  __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
+  __device__ void bind(uint32_t row) {
+    // offsets are taken from (py rows + px pixels) in front of the image so that none is negative; elements that would
+    // lie in front of the image are masked before they are loaded
+    const uint32_t bias = (uint32_t)py * W + (uint32_t)px;
+    rsrc = make_rsrc(p - bias, ((OH ? K / (OH * OW) : 1u) * C * H * W + bias) * 4u);
+    const uint32_t r = row < R ? row : 0;
+    const uint32_t taps = KY * KX, c = r / taps, q = r % taps, i = q / KX, j = q % KX;
+    voff = (c * H * W + i * W + j) * 4u;
+    iyc = row < R ? (int32_t)i - py : 0x40000000;  // rows beyond R never pass the row test
+    ixc = (int32_t)j - px;
+  }
+  template <int E>
+  __device__ void seek(uint32_t k0) {
+    const uint32_t dy = k0 / OW, dx = k0 % OW;  // the thread's first pixel inside the block of 16
+    voff += (dy * (uint32_t)sy * W + dx * (uint32_t)sx) * 4u;
+    iyc += (int32_t)dy * sy;
+    ixc += (int32_t)dx * sx;
+    oy = 0; ox = 0; woff = 0; soff = 0; Y = 0; X = 0;
+  }
+  template <int E>
+  __device__ void next() {
+    if (OW > BK) {
+      ox += BK;
+      if (ox == OW) { ox = 0; oy++; }
+    } else {
+      oy += BK / OW;
+    }
+    if (OH && oy >= OH) { oy = 0; woff += C * H * W * 4u; }
+    Y = (int32_t)oy * sy;
+    X = (int32_t)ox * sx;
+    soff = woff + ((uint32_t)Y * W + (uint32_t)X) * 4u;
+  }
+  template <int E>
+  __device__ void fetch(float (&v)[E]) const {
+    const bool row_ok = (uint32_t)(iyc + Y) < H;
+    int32_t ix = ixc + X;
+    uint32_t off = voff;
+#pragma unroll
+    for (int i = 0; i < E; i++) {
+      v[i] = buf_load(rsrc, row_ok && (uint32_t)ix < W ? off : OOB, soff);
+      ix += sx;
+      off += (uint32_t)sx * 4u;
+    }
+  }
+};
+
 // Where C goes.  Column n decomposes as g = n / inner, r = n % inner; with qw > 0, r is a pixel (qy, qx) of a
 // stride phase and lands at ((qy*sy + py) * OW + qx*sx + px).  Element (m, n) is at col(n) + m*row_stride.
 // value = acc [+ old C] [+ bias (per row m, or per inner column r)] [+ tap_bias[g % bias_w] * taps(y, x)], then func.
