@@ -287,7 +287,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--cpu-sample-batch", type=int, default=4)
+    ap.add_argument("--cpu-sample-batch", type=int, default=40,
+                    help="images of the CPU baseline sample (about 0.3 s each on one core)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also launch one plain copy (mt_set) of this many MiB before the timed region: the known-size kernel "
