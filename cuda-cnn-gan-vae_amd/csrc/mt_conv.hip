@@ -942,9 +942,9 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     rc = launch_tconv_small(name, args, max_n);
     if (rc >= 0) return rc;
   }
-  if (mt::epilogue_func(func)) return launch_tconv(name, args, max_n);
+  if (mt::epilogue_func(func)) return launch_tconv(name, args, max_n, mt::count(out));
   args.ep.func = MT_F_NONE;
-  rc = launch_tconv(name, args, max_n);
+  rc = launch_tconv(name, args, max_n, mt::count(out));
   return rc == MT_OK ? mt_apply_func(out, out, func) : rc;
 }
 
@@ -1191,7 +1191,7 @@ int upsampling_convolution(const char *name, const mt_tensor *out, const mt_tens
   args.ep.IH = image->y; args.ep.IW = image->x;
   const bool func_later = !mt::epilogue_func(func);
   args.ep.func = func_later ? MT_F_NONE : func;
-  rc = launch_tconv(name, args, max_n);
+  rc = launch_tconv(name, args, max_n, mt::count(out));
   return rc == MT_OK && func_later ? mt_apply_func(out, out, func) : rc;
 }
 

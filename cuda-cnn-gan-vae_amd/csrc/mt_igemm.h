@@ -875,6 +875,8 @@ constexpr int MAX_PHASES = 16;
 struct TconvArgs {
   TconvPhase ph[MAX_PHASES];
   uint32_t nphase, tiles_m, M, out_w;
+  uint32_t nsplit = 1, ksplit = 0;  // split-K: slice s of nsplit covers k in [s*ksplit, (s+1)*ksplit) of every phase and
+  size_t split_stride = 0;          // writes its own copy of the output, split_stride floats after the previous one
   const float *delta;          // [in_w][C][H][W]
   uint32_t in_w, C, H, W;
   Epilogue ep;   // C, row_stride, g_stride, sy, sx, OW, tap_bias, bias_w, IH, IW, func filled in
@@ -886,11 +888,15 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN
   using TS = TileShape<TM, TN, WGM, WGN>;
   __shared__ float4 smem[TS::LDS_FLOATS / 4];
   uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
+  const uint32_t per_slice = gridDim.x / args.nsplit, slice = j / per_slice;
+  j %= per_slice;
   uint32_t group = args.tiles_m * args.nphase;
   uint32_t nt = j / group, rem = j % group, f = rem / args.tiles_m, mt = rem % args.tiles_m;
   const TconvPhase &ph = args.ph[f];
   const uint32_t qhw = ph.qh * ph.qw, N = args.out_w * qhw;
   if (nt * TS::BN >= N) return;  // phases of an odd-sized output differ in size
+  const uint32_t k_first = slice * args.ksplit;
+  if (k_first >= ph.kp && slice) return;  // a phase with fewer taps has fewer slices; its other copies stay zero
   SrcRowK<true> a{};
   a.p = ph.packed; a.ld = ph.ld; a.R = args.M; a.K = ph.ld;  // rows are zero-padded to ld (a multiple of 4)
   typename std::conditional<FIXED, SrcIm2colFixed, SrcIm2col>::type b{};
@@ -900,17 +906,54 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN
   Epilogue ep = args.ep;
   ep.inner = qhw; ep.qw = ph.qw; ep.py = ph.py; ep.px = ph.px;
   ep.ty_cnt = ph.taps_y; ep.tx_cnt = ph.taps_x; ep.offy = ph.offy; ep.offx = ph.offx;
-  igemm_body<TM, TN, WGM, WGN>(a, b, ep, args.M, N, ph.kp, mt * TS::BM, nt * TS::BN, reinterpret_cast<float *>(smem));
+  uint32_t klen = ph.kp;
+  if (args.nsplit > 1) {
+    a.ksplit = args.ksplit; a.batch(slice);   // A rows are zero-padded to ld: its K is ld, the slice may end inside the padding
+    b.ksplit = args.ksplit; b.batch(slice);
+    klen = ph.kp - k_first < args.ksplit ? ph.kp - k_first : args.ksplit;
+    ep.C += (size_t)slice * args.split_stride;
+    if (slice) { ep.bias = nullptr; ep.tap_bias = nullptr; }  // the biases enter once, through slice 0
+  }
+  igemm_body<TM, TN, WGM, WGN>(a, b, ep, args.M, N, klen, mt * TS::BM, nt * TS::BN, reinterpret_cast<float *>(smem));
 }
 
-inline int launch_tconv(const char *name, TconvArgs &args, uint32_t max_n) {
+// out_floats > 0: the whole output tensor (args.ep.C, out_floats values, every pixel written by exactly one phase) may be
+// produced as the sum of k ranges when the launch has few blocks and a long k axis (see launch_split): every range
+// writes its own copy of the output in the workspace, the copies are added in a fixed order, then the function.
+inline int launch_tconv(const char *name, TconvArgs &args, uint32_t max_n, size_t out_floats = 0) {
   if (args.M == 0 || max_n == 0 || args.nphase == 0) return MT_OK;
   hipStream_t s = stream();
   const Tile tile = pick_tile(args.M, max_n, args.nphase);
-  ProfileScope prof(profiling() ? shape_label(name, tile, args.M, max_n, args.ph[0].kp, args.nphase) : name);
   const uint32_t bm = tile == T128x128 ? 128 : tile == T32x128 ? 32 : 64, bn = tile == T64x64 ? 64 : 128;
   args.tiles_m = cdiv(args.M, bm);
-  const size_t total = (size_t)args.tiles_m * cdiv(max_n, bn) * args.nphase;
+  size_t total = (size_t)args.tiles_m * cdiv(max_n, bn) * args.nphase;
+  uint32_t kmax = 0, kmin = 0xffffffffu;
+  for (uint32_t f = 0; f < args.nphase; f++) {
+    kmax = args.ph[f].kp > kmax ? args.ph[f].kp : kmax;
+    kmin = args.ph[f].kp < kmin ? args.ph[f].kp : kmin;
+  }
+  float *out = args.ep.C;
+  const int func_in_kernel = args.ep.func;
+  args.nsplit = 1;
+  if (out_floats && out_floats <= (1u << 22) && total <= 512 && kmin >= 1024) {
+    const uint32_t want = (uint32_t)(1024 / total);
+    uint32_t kc = (cdiv(kmax, want) + BK - 1) / BK * BK;
+    if (kc < 32 * BK) kc = 32 * BK;
+    const uint32_t S = cdiv(kmax, kc);
+    if (S >= 2) {
+      float *partial = nullptr;
+      int rc = split_workspace((size_t)S * out_floats, &partial);
+      if (rc) return rc;
+      if (kmin != kmax) {  // phases with fewer taps leave some copies untouched: those must read as zero
+        const mt_tensor all{partial, 1, 1, S, (uint32_t)out_floats};
+        if ((rc = mt_fill(&all, 0.f))) return rc;
+      }
+      args.nsplit = S; args.ksplit = kc; args.split_stride = out_floats;
+      args.ep.C = partial; args.ep.func = MT_F_NONE;
+      total *= S;
+    }
+  }
+  ProfileScope prof(profiling() ? shape_label(name, tile, args.M, max_n, args.nsplit > 1 ? args.ksplit : args.ph[0].kp, args.nphase * args.nsplit) : name);
   if (total > 0x7fffffffu) return fail(MT_E_ARGUMENT, "%s: problem too large for one launch", name);
   bool fixed = true;
   for (uint32_t f = 0; f < args.nphase; f++) {
@@ -934,6 +977,12 @@ inline int launch_tconv(const char *name, TconvArgs &args, uint32_t max_n) {
     }
   }
   MT_LAUNCH_CHECK(name);
+  if (args.nsplit > 1) {
+    const float *partial = args.ep.C;
+    const uint32_t S = args.nsplit;
+    args.ep.C = out; args.ep.func = func_in_kernel; args.nsplit = 1;
+    return split_reduce(name, out, partial, S, out_floats, nullptr, 1, 1, func_in_kernel);
+  }
   return MT_OK;
 }
 

@@ -176,6 +176,8 @@ CONV_CASES = [
     (2, 48, 6, 6, 8, 3, 3, 1, 1, 1, 1, 1, 2),       # one bias set per sample: not split
     (3, 16, 20, 24, 3, 3, 3, 1, 1, 1, 1, 1, 1),     # 3x3 to three channels: LDS-tiled vector-ALU kernel
     (2, 8, 18, 36, 4, 3, 3, 1, 1, 1, 1, 1, 2),      # the same with partial tiles and one bias set per sample
+    (2, 8, 8, 8, 256, 4, 4, 2, 2, 1, 1, 1, 1),      # transposed conv with few blocks and k = 1024 per phase: split over k
+    (1, 8, 5, 5, 1024, 3, 3, 2, 2, 1, 1, 1, 1),     # the same with phases of 4, 2, 2 and 1 taps (k = 4096 ... 1024)
 ]
 
 
@@ -270,6 +272,7 @@ def test_convolution_backward_weights_sum(gpu, oracle, path, case):
     (1, 8, 1, 1, 4),        # one input pixel: every tap but one is padding
     (2, 4, 5, 3, 70),       # odd input sizes, more filters than one tile
     (2, 64, 12, 16, 32),    # a layer of the reference's GAN generator at a quarter of its width
+    (2, 512, 3, 4, 64),     # its first layer: few blocks, k = 2048 per phase, split over k
 ])
 def test_upsampling_convolution(gpu, oracle, path, case):
     """Up-sampling x2 + convolution 3x3 stride 1 padding 1 (+ function) in one call, against the two layers on the
