@@ -306,7 +306,7 @@ def main():
                          "ops (secondary): every HBM-bound tensor operation on a [256,64,32,32] activation, GB/s each")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the path shards along the batch axis, see DESIGN.md")
+        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the path would shard along the batch axis, one all-reduce of the batch-norm sums per layer")
     if args.workload == "c5":
         return discriminator_step(args)
     if args.workload == "ops":
