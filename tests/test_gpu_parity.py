@@ -223,6 +223,47 @@ def test_create_delta_weight_and_bias(gpu, oracle, path, case, back):
         assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
 
 
+def _random_conv_cases(n, seed):
+    """Seeded random geometries: every combination of ragged sizes, strides up to 3, paddings up to the kernel size,
+    channel counts around the tile and k-step sizes."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < n:
+        kx, ky = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        sx, sy = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        px, py = int(rng.integers(0, kx)), int(rng.integers(0, ky))
+        H, Wd = int(rng.integers(ky, ky + 12)), int(rng.integers(kx, kx + 12))
+        C = int(rng.choice([1, 2, 3, 4, 5, 8, 15, 16, 17, 32, 33]))
+        KA = int(rng.choice([1, 2, 3, 4, 5, 8, 16, 31, 32, 33, 64, 65, 130]))
+        W = int(rng.integers(1, 5))
+        if (H - ky + 2 * py) // sy + 1 < 1 or (Wd - kx + 2 * px) // sx + 1 < 1:
+            continue
+        cases.append((W, C, H, Wd, KA, kx, ky, sx, sy, px, py))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_conv_cases(40, 2024))
+def test_random_convolution_geometries(gpu, oracle, case):
+    """Forward, transposed and weight-gradient convolution on 40 seeded random geometries (per-shape kernel choice)."""
+    W, C, H, Wd, KA, kx, ky, sx, sy, px, py = case
+    oy, ox = (H - ky + 2 * py) // sy + 1, (Wd - kx + 2 * px) // sx + 1
+    image, kernel, bias = U(1, W, C, H, Wd), U(2, 1, 1, KA, C * kx * ky), U(3, 1, KA, 1, 1)
+    fwd = (image, kernel, bias, kx, ky, C, KA, sx, sy, px, py)
+    close(gpu.forward_convolution(*fwd), oracle.forward_convolution(*fwd))
+    delta = U(4, W, KA, oy, ox)
+    bwd = (delta, kernel, bias, kx, ky, C, KA, sx, sy, px, py, (W, C, H, Wd))
+    close(gpu.backward_convolution(*bwd), oracle.backward_convolution(*bwd))
+    dk0, db0 = U(5, W, 1, KA, C * kx * ky), U(6, W, KA, 1, 1)
+    wg = (dk0, db0, image, delta, kx, ky, C, KA, sx, sy, px, py)
+    got, want = gpu.create_delta_weight_and_bias(*wg), oracle.create_delta_weight_and_bias(*wg)
+    close(got[0], want[0])
+    close(got[1], want[1])
+    sk0, sb0 = U(7, 1, 1, KA, C * kx * ky), U(8, 1, KA, 1, 1)
+    want_k = oracle.add_sum_w(sk0, want[0] - dk0, out_init=sk0)
+    got_k, got_b = gpu.convolution_backward_weights_sum(sk0, sb0, image, delta, kx, ky, C, KA, sx, sy, px, py)
+    close(got_k, want_k, 2e-4)      # the per-sample gradients above went through fp32 subtraction
+
+
 def test_wgrad_w_broadcast(gpu, oracle, path):
     image, delta = U(1, 2, 2, 6, 6), U(2, 1, 3, 6, 6)
     args = (np.zeros((4, 1, 3, 18), np.float32), np.zeros((2, 3, 1, 1), np.float32), image, delta, 3, 3, 2, 3, 1, 1, 1, 1)
