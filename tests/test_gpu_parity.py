@@ -363,6 +363,26 @@ def test_products(gpu, oracle, m, k, n, wl, wr, z):
     assert np.array_equal(gpu.transponse(a), oracle.transponse(a))
 
 
+def _random_product_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        m, k, nn = (int(rng.choice([1, 2, 3, 15, 16, 17, 31, 33, 64, 65, 100, 129])) for _ in range(3))
+        if rng.random() < 0.3:
+            k = int(rng.choice([513, 640, 1024, 2050]))          # long k: split ranges
+        w = int(rng.integers(1, 6))
+        wl, wr = (w, w) if rng.random() < 0.4 else ((1, w) if rng.random() < 0.5 else (w, 1))
+        cases.append((m, k, nn, wl, wr, int(rng.integers(1, 3))))
+    return cases
+
+
+@pytest.mark.parametrize("m,k,n,wl,wr,z", _random_product_cases(30, 7))
+def test_random_products(gpu, oracle, m, k, n, wl, wr, z):
+    a, b, at = U(1, wl, z, m, k), U(2, wr, z, k, n), U(3, wl, z, k, m)
+    close(gpu.mul(a, b), oracle.mul(a, b), 1e-5)
+    close(gpu.transponse_mul(at, b), oracle.transponse_mul(at, b), 1e-5)
+
+
 def test_elementwise_bit_exact(gpu, oracle):
     l, r, one = U(1, 3, 2, 5, 7), U(2, 3, 2, 5, 7), U(3, 1, 2, 5, 7)
     l4, r4, one4 = U(4, 3, 2, 6, 8), U(5, 3, 2, 6, 8), U(6, 1, 2, 6, 8)   # element count a multiple of 4: vector path
