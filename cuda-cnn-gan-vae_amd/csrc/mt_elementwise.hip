@@ -611,30 +611,30 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
                                                               float *mean, float *var, float *ivar, float *new_mean, float *new_var, float mom_old,
                                                               float mom_new, const float *gamma, const float *beta, int func) {
   constexpr int WS = EW_THREADS / RB;
-  __shared__ float part[2][WS][RB * 4];
-  __shared__ float col_mean[RB * 4], col_ivar[RB * 4];
+  __shared__ __attribute__((aligned(16))) float part[2][WS][RB * 4];
+  __shared__ __attribute__((aligned(16))) float col_mean[RB * 4], col_ivar[RB * 4];
   const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
   const uint32_t r = (blockIdx.x * RB + rl) * 4;
   float4 q[NW];
-  float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f};
+  float4 s1 = make_float4(0.f, 0.f, 0.f, 0.f), s2 = s1;
   if (r < S) {
     const float4 sh = *reinterpret_cast<const float4 *>(x + r);
 #pragma unroll
     for (int i = 0; i < NW; i++) {
-      const uint32_t w = ws + i * WS;
-      q[i] = w < W ? *reinterpret_cast<const float4 *>(x + (size_t)w * S + r) : sh;
+      const uint32_t w = ws + i * WS;  // rows past the batch re-read its last row (a plain global load) and are not summed
+      q[i] = *reinterpret_cast<const float4 *>(x + (size_t)(w < W ? w : W - 1) * S + r);
     }
 #pragma unroll
     for (int i = 0; i < NW; i++) {
       if (ws + i * WS < W) {
         float d0 = q[i].x - sh.x, d1 = q[i].y - sh.y, d2 = q[i].z - sh.z, d3 = q[i].w - sh.w;
-        s1[0] += d0; s1[1] += d1; s1[2] += d2; s1[3] += d3;
-        s2[0] += d0 * d0; s2[1] += d1 * d1; s2[2] += d2 * d2; s2[3] += d3 * d3;
+        s1.x += d0; s1.y += d1; s1.z += d2; s1.w += d3;
+        s2.x += d0 * d0; s2.y += d1 * d1; s2.z += d2 * d2; s2.w += d3 * d3;
       }
     }
   }
-#pragma unroll
-  for (int v = 0; v < 4; v++) { part[0][ws][rl * 4 + v] = s1[v]; part[1][ws][rl * 4 + v] = s2[v]; }
+  *reinterpret_cast<float4 *>(&part[0][ws][rl * 4]) = s1;
+  *reinterpret_cast<float4 *>(&part[1][ws][rl * 4]) = s2;
   __syncthreads();
   const int c = threadIdx.x;
   const uint32_t rc = blockIdx.x * RB * 4 + c;
