@@ -597,13 +597,8 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
       float o[4];
 #pragma unroll
       for (int i = 0; i < 4; i++) o[i] = acc[i / 2][py][i % 2][co] + bsum * (float)(ny * nx[i]);
-      if (func == MT_F_TANGENCE) {  // the usual end of an image generator: inline, the other functions share one body
 #pragma unroll
-        for (int i = 0; i < 4; i++) o[i] = mt::f_tangence(o[i]);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; i++) o[i] = mt::apply_func_epilogue(func, o[i]);
-      }
+      for (int i = 0; i < 4; i++) o[i] = mt::apply_func_epilogue(func, o[i]);  // tanh / sigmoid: hardware exp and reciprocal
       float *dst = args.ep.C + ((size_t)g * M + co) * OHW + (size_t)(2 * qy + py) * OW + 2 * qx;
       *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
     }
