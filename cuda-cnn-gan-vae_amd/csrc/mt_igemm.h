@@ -935,7 +935,9 @@ inline int launch_tconv(const char *name, TconvArgs &args, uint32_t max_n, size_
   float *out = args.ep.C;
   const int func_in_kernel = args.ep.func;
   args.nsplit = 1;
-  if (out_floats && out_floats <= (1u << 22) && total <= 512 && kmin >= 1024) {
+  // (two blocks on every compute unit already keep the matrix pipes busy: splitting 512 blocks cost more in the extra
+  // pass over the output than it gained)
+  if (out_floats && out_floats <= (1u << 22) && total <= 384 && kmin >= 1024) {
     const uint32_t want = (uint32_t)(1024 / total);
     uint32_t kc = (cdiv(kmax, want) + BK - 1) / BK * BK;
     if (kc < 32 * BK) kc = 32 * BK;
