@@ -518,10 +518,12 @@ struct HaloTile {
 // instead of 9 global loads for 16*CO, which moves the kernel from the texture-address path to the vector ALUs.
 // Needs W % 4 == 0, C % CC == 0, 16-byte aligned rows, exactly CO output channels and the coefficients packed
 // as [ci][phase][co][taps].
-template <int CO>
+// PP = 2 as described; PP = 1: one input pixel per thread and tiles of 16 x 16, twice the wavefronts (and twice the LDS
+// reads per multiply-add) for inputs so small that the grid would otherwise not give every SIMD two wavefronts.
+template <int CO, int PP>
 __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
-  using Tile = HaloTile<32, 16, 8>;
-  constexpr int TW = 32, TH = 16, CC = 8, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
+  using Tile = HaloTile<16 * PP, 16, 8>;
+  constexpr int TW = 16 * PP, TH = 16, CC = 8, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
   __shared__ __attribute__((aligned(16))) float tile[2][CC][ROWS][PITCH];
   const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W, M = args.M;
   const uint32_t tiles_x = (W + TW - 1) / TW;
@@ -532,9 +534,9 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
   auto fetch = [&](uint32_t chunk) { stage.fetch(chunk); };
   auto put = [&](int buf) { stage.put(&tile[buf][0][0][0]); };
 
-  float acc[2][2][2][CO];  // [pixel][py][px][co]
+  float acc[PP][2][2][CO];  // [pixel][py][px][co]
 #pragma unroll
-  for (int i = 0; i < 8 * CO; i++) (&acc[0][0][0][0])[i] = 0.f;
+  for (int i = 0; i < PP * 4 * CO; i++) (&acc[0][0][0][0])[i] = 0.f;
   const uint32_t chunks = C / CC;
   const float *coeff = args.ph[0].packed;
   fetch(0);
@@ -546,12 +548,16 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
 #pragma unroll 2
     for (int c = 0; c < CC; c++) {
       const uint32_t ci = ch * CC + c;
-      float v[3][4];  // rows y-1..y+1, columns x-1..x+2 of the pixel pair (x, x+1)
+      float v[3][PP + 2];  // rows y-1..y+1, columns x-1..x+PP of the thread's pixels (x .. x+PP-1)
 #pragma unroll
       for (int dy = 0; dy < 3; dy++) {
-        const float *rowp = &tile[cur][c][ty + dy][2 * tx];
-        const float2 lo = *reinterpret_cast<const float2 *>(rowp), hi = *reinterpret_cast<const float2 *>(rowp + 2);
-        v[dy][0] = lo.x; v[dy][1] = lo.y; v[dy][2] = hi.x; v[dy][3] = hi.y;
+        const float *rowp = &tile[cur][c][ty + dy][PP * tx];
+        if constexpr (PP == 2) {
+          const float2 lo = *reinterpret_cast<const float2 *>(rowp), hi = *reinterpret_cast<const float2 *>(rowp + 2);
+          v[dy][0] = lo.x; v[dy][1] = lo.y; v[dy][2] = hi.x; v[dy][3] = hi.y;
+        } else {
+          v[dy][0] = rowp[0]; v[dy][1] = rowp[1]; v[dy][2] = rowp[2];
+        }
       }
       // all 16*CO coefficients of a channel are contiguous, [ci][phase][co][taps (ty,tx) = 00 01 10 11]: CO uniform
       // 64-byte loads through the scalar cache
@@ -567,7 +573,7 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
             const int f = ((py * 2 + px) * CO + co) * 4;
             const float4 w = make_float4(wv[f / 16][f % 16], wv[f / 16][f % 16 + 1], wv[f / 16][f % 16 + 2], wv[f / 16][f % 16 + 3]);
 #pragma unroll
-            for (int p = 0; p < 2; p++) {
+            for (int p = 0; p < PP; p++) {
               float a = acc[p][py][px][co];
               a = __builtin_fmaf(w.x, v[py][p + px], a);
               a = __builtin_fmaf(w.y, v[py][p + px + 1], a);
@@ -582,7 +588,7 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
     __syncthreads();
   }
 
-  const uint32_t qy = y0 + ty, qx = x0 + 2 * tx;
+  const uint32_t qy = y0 + ty, qx = x0 + PP * tx;
   if (qy >= H || qx >= W) return;  // W is even: a pair is inside or outside as a whole
   const uint32_t OW = 2 * W, OHW = 4 * HW;
   const float bsum = args.ep.tap_bias ? args.ep.tap_bias[g % args.ep.bias_w] : 0.f;
@@ -591,16 +597,21 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
   for (int py = 0; py < 2; py++) {
     // contributing taps of output row 2*qy+py are input rows qy+py-1 and qy+py; likewise along x
     const int ny = ((uint32_t)((int32_t)qy + py - 1) < H) + ((uint32_t)((int32_t)qy + py) < H);
-    const int nx[4] = {((uint32_t)((int32_t)qx - 1) < W) + 1, 2, 2, 1 + ((uint32_t)((int32_t)qx + 2) < W)};
+    int nx[2 * PP];  // output column 2*qx+i: two taps inside the row, one fewer at the image's left and right edge
+#pragma unroll
+    for (int i = 0; i < 2 * PP; i++) nx[i] = 2;
+    nx[0] = ((uint32_t)((int32_t)qx - 1) < W) + 1;
+    nx[2 * PP - 1] = 1 + ((uint32_t)((int32_t)qx + PP) < W);
 #pragma unroll
     for (int co = 0; co < CO; co++) {
-      float o[4];
+      float o[2 * PP];
 #pragma unroll
-      for (int i = 0; i < 4; i++) o[i] = acc[i / 2][py][i % 2][co] + bsum * (float)(ny * nx[i]);
+      for (int i = 0; i < 2 * PP; i++) o[i] = acc[i / 2][py][i % 2][co] + bsum * (float)(ny * nx[i]);
 #pragma unroll
-      for (int i = 0; i < 4; i++) o[i] = mt::apply_func_epilogue(func, o[i]);  // tanh / sigmoid: hardware exp and reciprocal
+      for (int i = 0; i < 2 * PP; i++) o[i] = mt::apply_func_epilogue(func, o[i]);  // tanh / sigmoid: hardware exp and reciprocal
       float *dst = args.ep.C + ((size_t)g * M + co) * OHW + (size_t)(2 * qy + py) * OW + 2 * qx;
-      *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+      if constexpr (PP == 2) *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+      else *reinterpret_cast<float2 *>(dst) = make_float2(o[0], o[1]);
     }
   }
 }
@@ -676,10 +687,16 @@ bool tile_kernel_fits(const mt_tensor *out, const mt_tensor *delta, int32_t kx, 
 int launch_tconv_tile(const char *name, TconvArgs &args) {
   mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "vector ALU, few output channels") : name);
   dim3 gt(cdiv(args.W, 32) * cdiv(args.H, 16), args.out_w);
-  if (args.M == 1) tconv_k4s2_tile_kernel<1><<<gt, 256, 0, mt::stream()>>>(args);
-  else if (args.M == 2) tconv_k4s2_tile_kernel<2><<<gt, 256, 0, mt::stream()>>>(args);
-  else if (args.M == 3) tconv_k4s2_tile_kernel<3><<<gt, 256, 0, mt::stream()>>>(args);
-  else tconv_k4s2_tile_kernel<4><<<gt, 256, 0, mt::stream()>>>(args);
+  if ((size_t)gt.x * gt.y < 512) {  // fewer than two blocks per compute unit: one pixel per thread, twice the blocks
+    dim3 g1(cdiv(args.W, 16) * cdiv(args.H, 16), args.out_w);
+    if (args.M == 1) tconv_k4s2_tile_kernel<1, 1><<<g1, 256, 0, mt::stream()>>>(args);
+    else if (args.M == 2) tconv_k4s2_tile_kernel<2, 1><<<g1, 256, 0, mt::stream()>>>(args);
+    else if (args.M == 3) tconv_k4s2_tile_kernel<3, 1><<<g1, 256, 0, mt::stream()>>>(args);
+    else tconv_k4s2_tile_kernel<4, 1><<<g1, 256, 0, mt::stream()>>>(args);
+  } else if (args.M == 1) tconv_k4s2_tile_kernel<1, 2><<<gt, 256, 0, mt::stream()>>>(args);
+  else if (args.M == 2) tconv_k4s2_tile_kernel<2, 2><<<gt, 256, 0, mt::stream()>>>(args);
+  else if (args.M == 3) tconv_k4s2_tile_kernel<3, 2><<<gt, 256, 0, mt::stream()>>>(args);
+  else tconv_k4s2_tile_kernel<4, 2><<<gt, 256, 0, mt::stream()>>>(args);
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }

@@ -338,6 +338,18 @@ def test_upsampling_convolution_other_geometries(gpu, oracle, path):
         gpu.upsampling_convolution(image, Nrm(2, 1, 1, 9, 54, std=0.2), U(3, 1, 8, 1, 1), 3, 6, 9)   # eight biases for nine filters
 
 
+def test_image_layer_kernels_both_tilings(gpu, oracle):
+    """Transposed convolution 4x4 stride 2 padding 1 to three channels: grids below two blocks per compute unit take
+    one input pixel per thread, larger ones two; both against the oracle, with tanh and a non-zero bias."""
+    kernel, bias = Nrm(2, 1, 1, 8, 3 * 16, std=0.2), U(3, 1, 8, 1, 1) * 0.1
+    for shape in ((2, 8, 16, 20), (32, 8, 128, 128)):          # 4 and 1024 blocks of 32 x 16 pixels
+        delta = U(1, *shape)
+        out_shape = (shape[0], 3, 2 * shape[2], 2 * shape[3])
+        want = oracle.apply_func(oracle.backward_convolution(delta, kernel, bias, 4, 4, 3, 8, 2, 2, 1, 1, out_shape), "tangence")
+        got = gpu.backward_convolution(delta, kernel, bias, 4, 4, 3, 8, 2, 2, 1, 1, out_shape, func="tangence")
+        close(got, want, 1e-5)
+
+
 def test_fused_conv_activation(gpu, oracle, path):
     image, kernel, bias = U(1, 3, 4, 10, 10), U(2, 1, 1, 6, 4 * 9), U(3, 1, 6, 1, 1)
     for func in ("leaky_relu", "relu", "tangence", "sigmoid"):
