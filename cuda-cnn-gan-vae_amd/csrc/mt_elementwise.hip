@@ -439,6 +439,35 @@ __global__ __launch_bounds__(EW_THREADS) void max_pooling2x2_kernel(float *out, 
   }
 }
 
+// MaxPoolingBackward for 2x2 windows and an output of exactly twice the input: a thread owns two neighbouring windows
+// (one 128-bit load of their positions, one 64-bit load of their deltas) and writes their 2 x 4 output pixels as two
+// 128-bit stores; same rule as the gather kernel below.
+__global__ __launch_bounds__(EW_THREADS) void max_pooling_backward2x2_kernel(float *out, const mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t planes) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ix2 = g.ix / 2, n2 = g.iy * ix2;
+  if (i >= n2) return;
+  const uint32_t y = i / ix2, x2 = i % ix2, oy = 2 * y, ox = 4 * x2;
+  const size_t plane_in = (size_t)g.iy * g.ix, plane_out = (size_t)g.oy * g.ox;
+  const size_t o0 = (size_t)oy * g.ox + ox;
+  const bool same_w = Wpos * g.Z == planes;
+#pragma unroll 4
+  for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
+    const uint32_t ppl = same_w ? pl : (pl / g.Z % Wpos) * g.Z + pl % g.Z;
+    const uint4 s = reinterpret_cast<const uint4 *>(pos + (size_t)ppl * plane_in)[i];  // {X0, Y0, X1, Y1}
+    const float2 d = reinterpret_cast<const float2 *>(in + (size_t)pl * plane_in)[i];
+    float4 r[2];
+#pragma unroll
+    for (uint32_t dy = 0; dy < 2; dy++) {
+      r[dy].x = (s.x == ox && s.y == oy + dy) ? d.x : 0.f;
+      r[dy].y = (s.x == ox + 1 && s.y == oy + dy) ? d.x : 0.f;
+      r[dy].z = (s.z == ox + 2 && s.w == oy + dy) ? d.y : 0.f;
+      r[dy].w = (s.z == ox + 3 && s.w == oy + dy) ? d.y : 0.f;
+    }
+    float *dst = out + (size_t)pl * plane_out + o0;
+    *reinterpret_cast<float4 *>(dst) = r[0];
+    *reinterpret_cast<float4 *>(dst + g.ox) = r[1];
+  }
+}
+
 // Gather form of the CPU path's scatter: output (y,x) takes the delta of its window when that window's stored
 // maximum is (x,y), else 0.  Equal to the scatter for positions that lie inside their own window, which is what
 // max_pooling writes.
@@ -732,7 +761,7 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
           add(qd[i], qx[i]);
         }
     } else {
-#pragma unroll 4
+#pragma unroll 8
       for (uint32_t w = ws; w < W; w += WS) {
         const float4 x = *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r);
         add(behind(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), x), x);
@@ -1105,6 +1134,13 @@ int mt_max_pooling_backward(const mt_tensor *out, const mt_pos_tensor *pos, cons
   if (pos->p == nullptr || pos->w == 0 || pos->z != in->z || pos->y != in->y || pos->x != in->x)
     return mt::fail(MT_E_ARGUMENT, "mt_max_pooling_backward: position tensor must be [W',Z,Y,X] of the input");
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
+  if (px == 2 && py == 2 && out->x == 2 * in->x && out->y == 2 * in->y && in->x % 2 == 0 && in->x > 0 && aligned16(out->p) && aligned16(pos->p) &&
+      ((uintptr_t)in->p & 7u) == 0) {
+    const unsigned bx = cdiv(n / 8, EW_THREADS);
+    max_pooling_backward2x2_kernel<<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, planes);
+    MT_LAUNCH_CHECK("mt_max_pooling_backward");
+    return MT_OK;
+  }
   if (out->x % 4 == 0 && aligned16(out->p) && in->x > 0 && in->y > 0) {
     dim3 grid4(cdiv(n / 4, EW_THREADS), plane_blocks(cdiv(n / 4, EW_THREADS), planes));
     max_pooling_backward4_kernel<<<grid4, EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, px, py, planes);
