@@ -105,6 +105,44 @@ int mt_set_option(const char *name, int value) {
   return mt::fail(MT_E_ARGUMENT, "mt_set_option: unknown option '%s'", name ? name : "(null)");
 }
 
+// ---- interval timer on the work stream: the two events of the reference's CCUDATimeSpent ----
+namespace {
+struct Timer {
+  hipEvent_t start, stop;
+};
+}  // namespace
+
+int mt_timer_create(void **timer) {
+  if (timer == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_timer_create: null pointer");
+  Timer *t = new Timer;
+  hipError_t e = hipEventCreate(&t->start);
+  if (e == hipSuccess && (e = hipEventCreate(&t->stop)) != hipSuccess) (void)hipEventDestroy(t->start);
+  if (e != hipSuccess) { delete t; return mt::hip_fail(e, "hipEventCreate"); }
+  *timer = t;
+  return MT_OK;
+}
+int mt_timer_start(void *timer) {
+  if (timer == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_timer_start: null timer");
+  MT_HIP(hipEventRecord(static_cast<Timer *>(timer)->start, mt::stream()));
+  return MT_OK;
+}
+int mt_timer_stop(void *timer, float *milliseconds) {
+  if (timer == nullptr || milliseconds == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_timer_stop: null argument");
+  Timer *t = static_cast<Timer *>(timer);
+  MT_HIP(hipEventRecord(t->stop, mt::stream()));
+  MT_HIP(hipEventSynchronize(t->stop));
+  MT_HIP(hipEventElapsedTime(milliseconds, t->start, t->stop));
+  return MT_OK;
+}
+int mt_timer_destroy(void *timer) {
+  if (timer == nullptr) return MT_OK;
+  Timer *t = static_cast<Timer *>(timer);
+  (void)hipEventDestroy(t->start);
+  (void)hipEventDestroy(t->stop);
+  delete t;
+  return MT_OK;
+}
+
 int mt_set_stream(void *hip_stream) {
   if (!g_ready) { int rc = mt_init(0); if (rc) return rc; }
   g_stream = hip_stream ? (hipStream_t)hip_stream : g_own_stream;

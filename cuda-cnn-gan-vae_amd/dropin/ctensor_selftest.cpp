@@ -8,6 +8,7 @@
 #include <string>
 
 #include "cuda/tensor.cu.h"
+#include "cuda/ctimestamp.cu.h"
 
 namespace SYSTEM
 {
@@ -249,6 +250,22 @@ static void GpuClassOnlyChecks(void)
  Report("SetNormalNoise",fabs(sum/4096)<0.08);
 }
 
+// the scope timer the reference's models wrap around their training phases (cuda/ctimestamp.cu.h)
+static void TimerCheck(void)
+{
+ CTensor<type_t> a(8,4,64,64),b(8,4,64,64),c(8,4,64,64);
+ a.Fill(1);b.Fill(2);
+ CCUDATimeSpent spent;
+ spent.Start();
+ for(int n=0;n<20;n++) CTensorMath<type_t>::Add(c,a,b);
+ float ms=spent.Stop();
+ {
+  CTimeStamp stamp("Add x20: ",true);   // prints through SYSTEM::PutMessageToConsole when it goes out of scope
+  for(int n=0;n<20;n++) CTensorMath<type_t>::Add(c,a,b);
+ }
+ Report("CCUDATimeSpent / CTimeStamp measure queued work",ms>0 && ms<1000 && c.GetElement(7,3,63,63)==3);
+}
+
 int main(void)
 {
  try
@@ -261,6 +278,7 @@ int main(void)
   SummXYCheck();
   CoherenceAndErrors();
   GpuClassOnlyChecks();
+  TimerCheck();
  }
  catch(const char *message)
  {

@@ -94,6 +94,30 @@ def set_stream(handle):
     call("mt_set_stream", C.c_void_p(handle))
 
 
+class Timer:
+    """Milliseconds of queued work between start() and stop() (two events on the work stream; the reference's
+    CCUDATimeSpent, cuda/ccudatimespent.cu:9-52)."""
+
+    def __init__(self):
+        self._t = C.c_void_p()
+        call("mt_timer_create", C.byref(self._t))
+
+    def start(self):
+        call("mt_timer_start", self._t)
+
+    def stop(self):
+        ms = C.c_float()
+        call("mt_timer_stop", self._t, C.byref(ms))
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self._t:
+                call("mt_timer_destroy", self._t)
+        except Exception:
+            pass
+
+
 class Graph:
     """A sequence of library calls recorded once as a HIP graph and replayed with one launch: for steps made of many
     short kernels, where the host would otherwise be the bottleneck.  Everything the calls allocate (workspaces) must

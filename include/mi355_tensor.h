@@ -81,6 +81,12 @@ int mt_copy_d2d(void *dst, const void *src, size_t bytes); /* operator= (device 
 int mt_synchronize(void);
 void *mt_get_stream(void);               /* the hipStream_t all work is queued on */
 int mt_set_stream(void *hip_stream);     /* queue on a caller-owned stream (NULL: back to the library's own) */
+/* CCUDATimeSpent (cuda/ccudatimespent.cu:9-52): two events on the work stream; stop waits for the second one and
+ * returns the milliseconds between them.  The timer must have been started before it is stopped. */
+int mt_timer_create(void **timer);
+int mt_timer_start(void *timer);
+int mt_timer_stop(void *timer, float *milliseconds);
+int mt_timer_destroy(void *timer);
 /* "conv_path": 0 choose per shape (default), 1 one-thread-per-output kernels in the CPU path's summation order,
  * 2 matrix-core kernels wherever they apply.  "igemm_tile": -1 choose per shape (default), 0..3 force the block
  * tile 128x128 / 64x128 / 32x128 / 64x64 of the matrix-core kernels.  "wgrad_groups": 0 choose per shape (default),

@@ -40,7 +40,7 @@ def test_cpp_selftest_on_the_dropin_classes():
     run = subprocess.run([SELFTEST], capture_output=True, text=True, timeout=120)
     print(run.stdout[-3000:], run.stderr[-2000:])
     assert run.returncode == 0 and "ALL PASS" in run.stdout and "FAIL" not in run.stdout
-    assert run.stdout.count("PASS") >= 23
+    assert run.stdout.count("PASS") >= 24
 
 
 @pytest.fixture(scope="module")
