@@ -26,6 +26,7 @@ int fail(int code, const char *fmt, ...) {
 }
 
 int hip_fail(hipError_t e, const char *what) {
+  (void)hipGetLastError();  // the runtime keeps the error until it is read: the next launch check must not see it again
   return fail(MT_E_HIP + (int)e, "%s: %s", what, hipGetErrorString(e));
 }
 

@@ -557,6 +557,18 @@ def test_precondition_codes_match_oracle(gpu, oracle):
     assert code(gpu, probes[0]) == 0 and code(gpu, probes[1]) == 1
 
 
+def test_failed_allocation_is_reported_and_forgotten(gpu):
+    """An allocation the device cannot serve returns 1000 + hipError_t (cuda/handle_error.cu.h exits there); the
+    library stays usable and the next launch is not blamed for it."""
+    import ctypes
+    import mi355tensor as mt
+    ptr = ctypes.c_void_p()
+    with pytest.raises(mt.TensorError) as e:
+        mt.call("mt_malloc", ctypes.byref(ptr), ctypes.c_size_t(1 << 46))
+    assert e.value.code >= 1000 and not ptr.value
+    assert np.array_equal(gpu.add(U(1, 2, 3, 4, 5), U(2, 2, 3, 4, 5)), (U(1, 2, 3, 4, 5) + U(2, 2, 3, 4, 5)).astype(np.float32))
+
+
 def test_empty_tensors(gpu):
     assert gpu.add(np.zeros((0, 2, 3, 4), np.float32), np.zeros((0, 2, 3, 4), np.float32)).shape == (0, 2, 3, 4)
     assert gpu.fill((2, 0, 3, 4), 1.0).size == 0
