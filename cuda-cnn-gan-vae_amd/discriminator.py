@@ -94,6 +94,47 @@ class Discriminator:
         self.x.upload(x)
         self.labels.upload(labels)
 
+    # ---- network file ----------------------------------------------------------------------------------------
+    LAYER_KINDS = ["input"] + ["convolution", "batchnorm", "function"] * 4 + ["linear", "function"]
+
+    def save_net(self, f):
+        """The parameters as the reference's SaveNetLayers would write this stack (cuda/netmodel/cmodelmain.cu.h:296-300):
+        a C++ network of the same layers on the drop-in classes loads the file.  This class keeps no running
+        statistics: mean 0 and variable 1 are written, the values a fresh layer holds (cnetlayerbatchnormalization.cu.h:239)."""
+        import wire_format
+        layers = [("input", {})]
+        for i in range(4):
+            host = {k: self.p["%s%d" % (k, i)].numpy() for k in ("kernel", "bias", "gamma", "beta")}
+            header = dict(kernel_amount=CHANNELS[i + 1], kernel_x=4, kernel_y=4, kernel_z=CHANNELS[i], stride_x=2, stride_y=2, padding_x=1, padding_y=1)
+            layers.append(("convolution", {"header": header, "kernel": host["kernel"], "bias": host["bias"]}))
+            layers.append(("batchnorm", {"beta": host["beta"], "gamma": host["gamma"], "mean": np.zeros_like(host["beta"]),
+                                         "variable": np.ones_like(host["beta"]), "momentum": MOMENTUM}))
+            layers.append(("function", {"name": "leaky_relu"}))
+        layers.append(("linear", {"weight": self.p["lin_w"].numpy(), "bias": self.p["lin_b"].numpy()}))
+        layers.append(("function", {"name": "sigmoid"}))
+        wire_format.write_net(f, layers)
+
+    def load_net(self, f):
+        """The inverse; sizes and layer settings in the file must be this stack's (the reference loads with check_size)."""
+        import wire_format
+        layers = wire_format.read_net(f, self.LAYER_KINDS)
+        for i in range(4):
+            conv, bn, func = (layers[1 + 3 * i + j][1] for j in range(3))
+            h = conv["header"]
+            want = (CHANNELS[i + 1], 4, 4, CHANNELS[i], 2, 2, 1, 1)
+            if tuple(h[k] for k in wire_format.CONV_HEADER) != want or func["name"] != "leaky_relu":
+                raise ValueError("layer %d of the file is not this network's: %r, %s" % (i, h, func["name"]))
+            for name, a in (("kernel", conv["kernel"]), ("bias", conv["bias"]), ("gamma", bn["gamma"]), ("beta", bn["beta"])):
+                t = self.p["%s%d" % (name, i)]
+                if a.shape != t.shape:
+                    raise ValueError("%s%d: the file holds %s, the network %s" % (name, i, a.shape, t.shape))
+                t.upload(a)
+        lin = layers[13][1]
+        if lin["weight"].shape != self.p["lin_w"].shape or lin["bias"].shape != self.p["lin_b"].shape or layers[14][1]["name"] != "sigmoid":
+            raise ValueError("the last layers of the file are not this network's")
+        self.p["lin_w"].upload(lin["weight"])
+        self.p["lin_b"].upload(lin["bias"])
+
     # ---- forward -------------------------------------------------------------------------------------------
     def forward(self, fused=False):
         h, p = self.x, self.p

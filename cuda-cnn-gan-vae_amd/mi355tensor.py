@@ -198,6 +198,28 @@ class CTensor:
             synchronize()
         return out
 
+    def Save(self, f):
+        """CTensor::Save (cuda/ctensor.cu.h:525-537): copy back from the device, four sizes, then the values as doubles."""
+        import wire_format
+        assert not (self.pos or self.u32), "only CTensor<type_t> tensors are part of a checkpoint"
+        wire_format.write_tensor(f, self.numpy())
+
+    def Load(self, f, check_size=True):
+        """CTensor::Load (cuda/ctensor.cu.h:541-571).  With `check_size` the sizes in the stream must be this tensor's own
+        (TensorError, as the reference throws); without it the tensor takes the stream's sizes and new device memory."""
+        import wire_format
+        a = wire_format.read_tensor(f)
+        if a.shape != self.shape:
+            if check_size:
+                axis = "WZYX"[[i for i in range(4) if a.shape[i] != self.shape[i]][0]]
+                raise TensorError("CTensor::Load", -1, "the stream holds %s, the tensor is %s: wrong size %s" % (a.shape, self.shape, axis))
+            assert self.owned, "a borrowed view cannot change its size"
+            self.free()
+            self.__dict__.pop("_ref", None)
+            self.shape = a.shape
+            call("mt_malloc", C.byref(self.ptr), C.c_size_t(self.count * self.item))
+        self.upload(a)
+
     def reinterpret(self, w, z, y, x):
         """ReinterpretSize: the same memory under other sizes (cuda/ctensor.cu.h:587-601)."""
         assert w * z * y * x == self.count, "the element count must not change"

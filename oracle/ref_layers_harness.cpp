@@ -83,6 +83,7 @@ class CMemoryStream:public IDataStream
  public:
   CMemoryStream(void):Pos(0) {}
   void Rewind(void) {Pos=0;}
+  const std::vector<uint8_t>& Bytes(void) const {return(Data);}
   int8_t LoadInt8(void) {return(Get<int8_t>());}
   int16_t LoadInt16(void) {return(Get<int16_t>());}
   int32_t LoadInt32(void) {return(Get<int32_t>());}
@@ -163,6 +164,19 @@ static void DumpStream(const char *name,CMemoryStream &stream,size_t skip_bytes,
  }
 }
 
+// the bytes of a stream as they would be in a checkpoint file, four per dump slot (the reader takes the bit patterns)
+static void DumpRaw(const char *name,CMemoryStream &stream)
+{
+ const std::vector<uint8_t> &bytes=stream.Bytes();
+ char label[32];
+ memset(label,0,sizeof(label));
+ strncpy(label,name,sizeof(label)-1);
+ uint32_t dims[4]={1,1,1,static_cast<uint32_t>(bytes.size()/4)};
+ fwrite(label,1,sizeof(label),out_file);
+ fwrite(dims,sizeof(uint32_t),4,out_file);
+ fwrite(&bytes[0],1,dims[3]*4,out_file);
+}
+
 static const uint32_t BATCH=6;
 
 static void ChainA(void)
@@ -207,6 +221,11 @@ static void ChainA(void)
  lin.Save(&lin_saved);
  DumpStream("A.conv_updated",conv_saved,8*sizeof(int32_t),2);
  DumpStream("A.linear_updated",lin_saved,0,2);
+ DumpRaw("A.conv_stream",conv_saved);
+ DumpRaw("A.linear_stream",lin_saved);
+ CMemoryStream net_saved;   // the whole chain, layer after layer, as CModelMain::SaveNetLayers writes a network
+ for(int n=0;n<5;n++) layers[n]->Save(&net_saved);
+ DumpRaw("A.net_stream",net_saved);
 }
 
 static void ChainB(void)
@@ -238,6 +257,7 @@ static void ChainB(void)
  CMemoryStream saved;
  tconv.Save(&saved);
  DumpStream("B.tconv_updated",saved,8*sizeof(int32_t),2);
+ DumpRaw("B.tconv_stream",saved);
 }
 
 // Chain D: resampling layers, forward and backward (no weights)
@@ -261,6 +281,9 @@ static void ChainD(void)
  for(int n=2;n>=1;n--) layers[n]->TrainingBackward(true);
  Dump("D.delta_average",avg.GetDeltaTensor());
  Dump("D.delta_upsampling",up.GetDeltaTensor());
+ CMemoryStream net_saved;
+ for(int n=0;n<3;n++) layers[n]->Save(&net_saved);
+ DumpRaw("D.net_stream",net_saved);
 }
 
 #ifndef USE_CPU
@@ -342,6 +365,9 @@ static void ChainC(void)
  for(int n=2;n>=1;n--) layers[n]->TrainingBackward(true);
  Dump("C.delta_bn",bn.GetDeltaTensor());
  Dump("C.prev_error",input.GetDeltaTensor());   // the input layer hands back its own tensor: unchanged input
+ CMemoryStream bn_saved;
+ bn.Save(&bn_saved);
+ DumpRaw("C.bn_stream",bn_saved);
 }
 #endif
 

@@ -130,6 +130,38 @@ def test_config5_training_step_against_oracle(gpu, oracle):
         assert rel_err(net.m[name].numpy(), m) <= 1e-6 and rel_err(net.v[name].numpy(), v) <= 1e-6, name
 
 
+def test_config5_network_file_round_trip(gpu):
+    """The discriminator's parameters after a training step, written in the reference's network-file layout, loaded
+    into a differently initialised copy: the copy computes the same outputs bit for bit; a file of another topology
+    is refused."""
+    import io
+    import discriminator as D
+    import wire_format as wf
+    x, labels = D.make_batch(4)
+    net = D.Discriminator(4)
+    net.set_batch(x, labels)
+    net.step(fused=True)
+    f = io.BytesIO()
+    net.save_net(f)
+    # size: 4 conv headers, 4 function ids + the last one, 4 momenta, 26 tensors
+    tensors = sum(int(np.prod(t.shape)) for t in net.p.values()) + 2 * sum(int(np.prod(net.p["beta%d" % i].shape)) for i in range(4))
+    assert len(f.getvalue()) == 4 * 32 + 5 * 4 + 4 * 8 + 26 * 16 + 8 * tensors
+    other = D.Discriminator(4, D.make_parameters(seed=77))
+    other.set_batch(x, labels)
+    f.seek(0)
+    other.load_net(f)
+    for name in net.p:
+        assert np.array_equal(net.p[name].numpy(), other.p[name].numpy()), name
+    assert np.array_equal(net.forward(True).numpy(), other.forward(True).numpy())
+    layers = wf.read_net(io.BytesIO(f.getvalue()), D.Discriminator.LAYER_KINDS)
+    layers[1][1]["header"]["stride_x"] = 1
+    g = io.BytesIO()
+    wf.write_net(g, layers)
+    g.seek(0)
+    with pytest.raises(ValueError):
+        other.load_net(g)
+
+
 def test_config5_full_batch_properties(gpu, oracle):
     """Batch 128: (1) the fused and the literal forward agree; (2) convolution, its input gradient and its per-sample
     weight gradient are independent per sample, so one sample of the big batch equals that sample alone through the

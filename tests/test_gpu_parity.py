@@ -754,3 +754,26 @@ def test_operands_beyond_two_gib(gpu, oracle):
     got = back.numpy()
     for w in (0, 31, 32, 35):
         close(got[w:w + 1], oracle.backward_convolution(host[w:w + 1], tk, zero, 3, 3, 1, C, 1, 1, 1, 1, (1, 1, H, H)))
+
+
+def test_tensor_save_and_load_in_the_wire_format(gpu):
+    """CTensor.Save / Load of the Python mirror: the bytes are the reference's layout (sizes, then doubles), a device
+    tensor survives the round trip bit for bit, a size mismatch is an error with check_size and a resize without it."""
+    import io
+    import struct
+    from mi355tensor import CTensor, TensorError
+    a = Nrm(60, 2, 3, 4, 5)
+    f = io.BytesIO()
+    CTensor.from_numpy(a).Save(f)
+    raw = f.getvalue()
+    assert struct.unpack_from("=4I", raw) == (2, 3, 4, 5)
+    assert np.array_equal(np.frombuffer(raw, np.float64, offset=16), a.reshape(-1).astype(np.float64))
+    t = CTensor(2, 3, 4, 5)
+    t.Load(io.BytesIO(raw))
+    assert np.array_equal(t.numpy(), a)
+    other = CTensor(2, 3, 5, 4)
+    with pytest.raises(TensorError, match="wrong size Y"):
+        other.Load(io.BytesIO(raw))
+    other.Load(io.BytesIO(raw), check_size=False)
+    assert other.shape == (2, 3, 4, 5) and np.array_equal(other.numpy(), a)
+    assert other.desc().w == 2 and other.desc().y == 4

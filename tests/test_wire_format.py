@@ -1,0 +1,150 @@
+"""The checkpoint wire format (wire_format.py): round trips, and the byte streams that the reference's OWN layer classes
+write with Save() -- `oracle/_ref/layers_cpu` is the reference's convolution and linear layers on its CPU tensor classes,
+compiled in the authoring container; it stores those streams byte for byte in its dump (entries `*_stream`)."""
+import io
+import os
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+
+import wire_format as wf
+from conftest import ROOT
+
+LAYERS_CPU = os.path.join(ROOT, "oracle", "_ref", "layers_cpu")
+
+
+def read_dump_bytes(path):
+    """name -> (dims, raw bytes of the float32 slots)"""
+    out, data, pos = {}, open(path, "rb").read(), 0
+    while pos < len(data):
+        name = data[pos:pos + 32].split(b"\0")[0].decode()
+        dims = struct.unpack_from("<4I", data, pos + 32)
+        n = int(np.prod(dims))
+        out[name] = (dims, data[pos + 48:pos + 48 + 4 * n])
+        pos += 48 + 4 * n
+    return out
+
+
+def as_array(entry):
+    return np.frombuffer(entry[1], np.float32).reshape(entry[0])
+
+
+def test_tensor_round_trip_is_exact():
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    a[0, 0, 0, :3] = (np.float32(1e-40), np.float32(3.4e38), np.float32(-0.0))       # denormal, near the maximum, signed zero
+    f = io.BytesIO()
+    wf.write_tensor(f, a)
+    assert len(f.getvalue()) == 16 + 8 * a.size
+    assert struct.unpack_from("=4I", f.getvalue()) == (2, 3, 4, 5)
+    f.seek(0)
+    b = wf.read_tensor(f)
+    assert b.dtype == np.float32 and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_empty_tensor_and_truncated_streams():
+    f = io.BytesIO()
+    wf.write_tensor(f, np.zeros((0, 1, 1, 1), np.float32))      # the reference writes the four sizes and no values
+    assert len(f.getvalue()) == 16
+    f.seek(0)
+    assert wf.read_tensor(f).shape == (0, 1, 1, 1)
+    with pytest.raises(EOFError):
+        wf.read_tensor(io.BytesIO(b"\x01\0\0\0"))
+    with pytest.raises(EOFError):
+        wf.read_tensor(io.BytesIO(struct.pack("=4I", 1, 1, 1, 2) + b"\0" * 8))
+
+
+def test_layer_round_trips():
+    rng = np.random.default_rng(2)
+    header = dict(kernel_amount=4, kernel_x=3, kernel_y=2, kernel_z=5, stride_x=2, stride_y=1, padding_x=1, padding_y=0)
+    kernel, bias = rng.standard_normal((1, 1, 4, 30)).astype(np.float32), rng.standard_normal((1, 4, 1, 1)).astype(np.float32)
+    f = io.BytesIO()
+    wf.write_convolution_layer(f, header, kernel, bias)
+    wf.write_linear_layer(f, kernel, bias.reshape(1, 1, 4, 1))
+    bn = [rng.standard_normal((1, 2, 3, 3)).astype(np.float32) for _ in range(4)]
+    wf.write_batchnorm_layer(f, *bn, momentum=0.9)
+    f.seek(0)
+    h, k, b = wf.read_convolution_layer(f)
+    assert h == header and np.array_equal(k, kernel) and np.array_equal(b, bias)
+    w, lb = wf.read_linear_layer(f)
+    assert np.array_equal(w, kernel) and lb.shape == (1, 1, 4, 1)
+    got = wf.read_batchnorm_layer(f)
+    assert all(np.array_equal(g, t) for g, t in zip(got[:4], bn)) and got[4] == 0.9
+    assert f.read() == b""
+
+
+@pytest.fixture(scope="module")
+def cpu_dump(tmp_path_factory):
+    if not os.path.exists(LAYERS_CPU):
+        pytest.skip("oracle/_ref/layers_cpu not built (it needs /root/reference)")
+    path = str(tmp_path_factory.mktemp("wire") / "cpu.bin")
+    run = subprocess.run([LAYERS_CPU, path], capture_output=True, text=True, timeout=180)
+    assert run.returncode == 0, run.stderr
+    return read_dump_bytes(path)
+
+
+def test_streams_written_by_the_reference_layers(cpu_dump):
+    """CNetLayerConvolution::Save and CNetLayerLinear::Save of the reference, parsed here; the tensors must equal the ones
+    the harness itself read back from the same streams with the reference's stream interface."""
+    header, kernel, bias = wf.read_convolution_layer(io.BytesIO(cpu_dump["A.conv_stream"][1]))
+    want_k, want_b = as_array(cpu_dump["A.conv_updated.0"]), as_array(cpu_dump["A.conv_updated.1"])
+    assert kernel.shape == want_k.shape and np.array_equal(kernel, want_k)
+    assert bias.shape == want_b.shape and np.array_equal(bias, want_b)
+    assert header["kernel_amount"] == kernel.shape[2]
+    assert header["kernel_x"] * header["kernel_y"] * header["kernel_z"] == kernel.shape[3]
+    assert header["stride_x"] >= 1 and header["stride_y"] >= 1 and header["padding_x"] >= 0 and header["padding_y"] >= 0
+
+    stream = io.BytesIO(cpu_dump["A.linear_stream"][1])
+    weight, lbias = wf.read_linear_layer(stream)
+    assert stream.read() == b""
+    assert np.array_equal(weight, as_array(cpu_dump["A.linear_updated.0"]))
+    assert np.array_equal(lbias, as_array(cpu_dump["A.linear_updated.1"]))
+
+    # written back, the bytes are the reference's own
+    f = io.BytesIO()
+    wf.write_convolution_layer(f, header, kernel, bias)
+    assert f.getvalue() == cpu_dump["A.conv_stream"][1]
+    f = io.BytesIO()
+    wf.write_linear_layer(f, weight, lbias)
+    assert f.getvalue() == cpu_dump["A.linear_stream"][1]
+
+
+def test_whole_networks_written_by_the_reference(cpu_dump):
+    """Every layer of a chain saved into one stream, the way CModelMain::SaveNetLayers writes a network file."""
+    raw = cpu_dump["A.net_stream"][1]
+    kinds = ["input", "convolution", "function", "linear", "function"]
+    net = wf.read_net(io.BytesIO(raw), kinds)
+    assert [k for k, _ in net] == kinds
+    assert net[2][1]["name"] == "leaky_relu" and net[4][1]["name"] == "sigmoid"
+    assert np.array_equal(net[1][1]["kernel"], as_array(cpu_dump["A.conv_updated.0"]))
+    assert np.array_equal(net[3][1]["bias"], as_array(cpu_dump["A.linear_updated.1"]))
+    f = io.BytesIO()
+    wf.write_net(f, net)
+    assert f.getvalue() == raw
+
+    raw = cpu_dump["D.net_stream"][1]
+    net = wf.read_net(io.BytesIO(raw), ["input", "upsampling", "averagepooling"])
+    assert net[1][1] == {"x": 2, "y": 2} and net[2][1] == {"x": 4, "y": 4}
+    f = io.BytesIO()
+    wf.write_net(f, net)
+    assert f.getvalue() == raw
+
+    header, kernel, _ = wf.read_convolution_layer(io.BytesIO(cpu_dump["B.tconv_stream"][1]))   # transposed convolution
+    assert np.array_equal(kernel, as_array(cpu_dump["B.tconv_updated.0"]))
+    assert (header["kernel_amount"], header["kernel_z"]) == (kernel.shape[2], kernel.shape[3] // 16)
+
+
+def test_net_round_trip_of_the_other_layer_kinds():
+    f = io.BytesIO()
+    layers = [("input", {}), ("dropout", {"rate": 0.25}), ("maxpooling", {"x": 2, "y": 3}), ("function", {"name": "gelu"}),
+              ("softmax", {}), ("splitter", {}), ("vae_coder_output", {}), ("concatenator", {}), ("time_embedding", {})]
+    wf.write_net(f, layers)
+    assert len(f.getvalue()) == 8 + 8 + 4
+    f.seek(0)
+    assert wf.read_net(f, [k for k, _ in layers]) == layers
+    with pytest.raises(ValueError):
+        wf.read_net(io.BytesIO(struct.pack("=I", 9)), ["function"])
+    with pytest.raises(EOFError):
+        wf.read_net(io.BytesIO(b""), ["upsampling"])
