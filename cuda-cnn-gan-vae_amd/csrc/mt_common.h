@@ -17,7 +17,8 @@ int hip_fail(hipError_t e, const char *what);
 int split_workspace(size_t floats, float **p);
 int split_reduce(const char *name, float *out, const float *partial, uint32_t S, size_t n, const float *bias, uint32_t bias_div, uint32_t bias_mod, int func);
 int set_conv_path(int v);  // 0 auto, 1 direct kernels, 2 matrix cores wherever they apply
-int set_igemm_tile(int v); // -1 auto, 0..3 force one block tile of the matrix-core kernels
+int set_igemm_tile(int v); // -1 auto, 0..4 force one block tile of the matrix-core kernels
+int set_patch_blocks(int v);  // persistent blocks of the input-patch transposed convolution (default 512)
 int set_wgrad_groups(int v);  // 0 auto, else batch groups of the batch-summed weight gradient
 
 // Brackets the launches made inside its lifetime with two events on the work stream when profiling is enabled

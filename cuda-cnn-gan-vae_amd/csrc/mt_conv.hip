@@ -966,7 +966,7 @@ bool wgrad_image_fixed(uint32_t M, uint32_t N, uint32_t batches, const mt_tensor
                        int32_t py) {
   if (px < 0 || py < 0) return false;
   const Tile tile = pick_tile(M, N, batches);
-  const uint32_t pixels = (tile == T64x64 ? 64u : 128u) * BK / THREADS;
+  const uint32_t pixels = tile_cols(tile) * BK / THREADS;
   const size_t span = (size_t)per * kz * image->y * image->x + (size_t)py * image->x + px;
   return SrcWgradImageFixed::fits(delta->y, delta->x, pixels) && mt::fits_buffer(span);
 }
@@ -1215,9 +1215,18 @@ int &tile_override() {
   static int v = -1;
   return v;
 }
+int &patch_blocks() {
+  static int v = 512;
+  return v;
+}
 }  // namespace igemm
+int set_patch_blocks(int v) {
+  if (v < 1 || v > 65536) return fail(MT_E_ARGUMENT, "patch_blocks must be 1..65536");
+  igemm::patch_blocks() = v;
+  return MT_OK;
+}
 int set_igemm_tile(int v) {
-  if (v < -1 || v > 3) return fail(MT_E_ARGUMENT, "igemm_tile must be -1 (auto) or 0..3");
+  if (v < -1 || v > 4) return fail(MT_E_ARGUMENT, "igemm_tile must be -1 (auto) or 0..4");
   igemm::tile_override() = v;
   return MT_OK;
 }

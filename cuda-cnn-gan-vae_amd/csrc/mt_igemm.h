@@ -1,7 +1,9 @@
 // Implicit-GEMM core for gfx950: C[M,N] (+)= A[M,K] * B[K,N] on the fp32 matrix cores.
 //
 //  * 256 threads = 4 wavefronts of 64 lanes; every wavefront owns a (TM*32) x (TN*32) block of C held in
-//    TM*TN accumulators of v_mfma_f32_32x32x2_f32 (16 VGPRs each).
+//    TM*TN accumulators of v_mfma_f32_32x32x2_f32 (16 VGPRs each).  Products of at most 16 rows use
+//    v_mfma_f32_16x16x4_f32 instead (R16: a 16 x 256 block, four 16 x 16 accumulators per wavefront), which
+//    runs at the same rate and leaves no half of the matrix unit multiplying padding.
 //  * A and B never exist as matrices in memory.  Each is an "operand source" that maps (row, k) to an
 //    address -- a row-major or column-major matrix, an im2col view of an NCHW image, one stride phase of a
 //    transposed convolution, the image view of a weight gradient -- and is staged through LDS as
@@ -24,6 +26,7 @@ constexpr int BK = 16;
 constexpr int THREADS = 256;
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4acc __attribute__((ext_vector_type(4)));
 
 // matrix index of batch entry bz = (w, z) for an operand with Wop layers of Z matrices each
 struct Batch {
@@ -240,7 +243,7 @@ struct SrcIm2colFixed {
   uint32_t imgoff;
   int32_t iy0, ix0;
   uint32_t ksplit = 0;  // > 0: batch entry bz covers k in [bz*ksplit, (bz+1)*ksplit), ksplit a multiple of BK (split-K)
-  uint32_t voff[8];
+  uint32_t voff[16];
   uint32_t soff, sstep, kpos, kend, kbase = 0;
   __device__ void batch(uint32_t bz) {
     if (ksplit) kbase = bz * ksplit;
@@ -260,7 +263,7 @@ struct SrcIm2colFixed {
   }
   template <int E>
   __device__ void seek(uint32_t k0) {  // k0 < BK
-    static_assert(E <= 8, "at most eight elements per thread");
+    static_assert(E <= 16, "at most sixteen elements per thread");
     const uint32_t taps = KY * KX;  // taps divides BK = 16, so taps and KX are powers of two
     const int lt = __builtin_ctz(taps), lx = __builtin_ctz(KX);
 #pragma unroll
@@ -298,7 +301,7 @@ struct SrcIm2colTap {
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t imgoff, kthread;
   int32_t iy0, ix0;
-  uint32_t voff[8];
+  uint32_t voff[16];
   uint32_t ky, kx, ctile, tiles_per_tap, kpos, kend, kbase = 0;
   __device__ void batch(uint32_t bz) {
     if (ksplit) kbase = bz * ksplit;
@@ -326,7 +329,7 @@ struct SrcIm2colTap {
   }
   template <int E>
   __device__ void seek(uint32_t k0) {  // k0 < BK: the thread's first channel within a tile
-    static_assert(E <= 8, "at most eight elements per thread");
+    static_assert(E <= 16, "at most sixteen elements per thread");
     kthread = k0;
     range();
     tiles_per_tap = C / BK;
@@ -567,6 +570,32 @@ struct Epilogue {
     MT_EACH_ROW(dst[(size_t)dm * row_stride] = v[r]);
 #undef MT_EACH_ROW
   }
+  // One accumulator of v_mfma_f32_16x16x4_f32 for column c: register r holds row m_base + r.  Same order of terms.
+  __device__ __forceinline__ void store_quad(const Col &c, uint32_t m_base, uint32_t M, floatx4acc &v) const {
+    if (m_base >= M) return;
+    float *dst = C + c.off + (size_t)m_base * row_stride;
+    const uint32_t rows = M - m_base < 4 ? M - m_base : 4;
+    if (accumulate) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) if ((uint32_t)r < rows) v[r] += dst[(size_t)r * row_stride];
+    }
+    if (bias && bias_mode == 1) {
+      const float *bp = bias + c.bias_row + m_base;
+#pragma unroll
+      for (int r = 0; r < 4; r++) if ((uint32_t)r < rows) v[r] += bp[r];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) v[r] += c.extra;
+    if (func == MT_F_RELU) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) v[r] = v[r] > 0.f ? v[r] : 0.f;
+    } else if (func == MT_F_LEAKY_RELU) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) v[r] = v[r] > 0.f ? v[r] : (float)(0.1 * (double)v[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) if ((uint32_t)r < rows) dst[(size_t)r * row_stride] = v[r];
+  }
   __device__ __forceinline__ void store_block(const Col &c, uint32_t m_base, uint32_t M, floatx16 &v) const {
     if (m_base >= M) return;
     if (m_base + 28 <= M) store_rows<true>(c, m_base, M, v);
@@ -610,9 +639,16 @@ __device__ __forceinline__ void lds_barrier() {
 // (lane % 32) of A and the column (lane % 32) of B.  Which k of the tile a step multiplies is free as long as A and
 // B agree, so lanes 0-31 take k = 0..3 and lanes 32-63 k = 4..7 from ONE 128-bit LDS read (steps 0-3), then
 // k = 8..11 / 12..15 from a second one (steps 4-7): two LDS reads per 32 rows and tile instead of eight.
-template <int TM, int TN, int WGM, int WGN, class SrcA, class SrcB>
+//
+// R16 (with TM = 1, WGM = 1): the block is 16 rows of C.  A is still staged 32 rows at a time (two k per thread,
+// rows beyond the sixteenth are never read back), and a wavefront's TN*32 columns are 2*TN accumulators of
+// v_mfma_f32_16x16x4_f32: lane l supplies row (or column) l % 16 at k slot l / 16, so ONE 128-bit LDS read at
+// k offset 4*(l/16) feeds four instructions that together cover the 16 k of a tile (instruction c multiplies
+// k = c, 4+c, 8+c, 12+c).  The two halves of a pipeline step are then the two halves of the wavefront's columns.
+template <int TM, int TN, int WGM, int WGN, bool R16, class SrcA, class SrcB>
 __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep, uint32_t M, uint32_t N, uint32_t K, uint32_t m0, uint32_t n0, float *smem) {
   static_assert(WGM * WGN == 4, "four wavefronts per block");
+  static_assert(!R16 || (TM == 1 && WGM == 1), "a 16-row block is one row of wavefronts");
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
   constexpr int EA = BM * BK / THREADS, EB = BN * BK / THREADS;
   static_assert(EA >= 2 && EB >= 2, "tile too small for the loader");
@@ -635,12 +671,17 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
 
   float ra[2][EA], rb[2][EB];  // two register sets: the global loads run two tiles ahead of the LDS writes
   floatx16 acc[TM][TN];
+  floatx4acc acc16[2 * TN];
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+#pragma unroll
+  for (int j = 0; j < 2 * TN; j++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc16[j][r] = 0.f;
 
   const uint32_t nk = (K + BK - 1) / BK;
   a.template seek<EA>(a_k);
@@ -667,18 +708,24 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
     lds_barrier();
   };
 
-  const int lrow = lane & 31, lk = lane >> 5;
+  const int lrow = R16 ? (lane & 15) : (lane & 31), lk = R16 ? (lane >> 4) : (lane >> 5);
   const float *a_get = As + (wm * TM * 32 + lrow) * LDK + lk * 4;
   const float *b_get = Bs + (wn * TN * 32 + lrow) * LDK + lk * 4;
-  // fragments of one half tile (8 k): one 128-bit LDS read per 32 rows
+  // fragments of one half: one 128-bit LDS read per 32 rows and 8 k, or (R16) per 16 rows and 16 k
   float4 fa[2][TM], fb[2][TN];
   auto read_half = [&](float4 (&av)[TM], float4 (&bv)[TN], int buf, int half) {
+    if constexpr (R16) {
+      av[0] = *reinterpret_cast<const float4 *>(a_get + buf * BM * LDK);
 #pragma unroll
-    for (int i = 0; i < TM; i++) av[i] = *reinterpret_cast<const float4 *>(a_get + buf * BM * LDK + i * 32 * LDK + half * 8);
+      for (int j = 0; j < TN; j++) bv[j] = *reinterpret_cast<const float4 *>(b_get + buf * BN * LDK + (half * TN + j) * 16 * LDK);
+    } else {
 #pragma unroll
-    for (int j = 0; j < TN; j++) bv[j] = *reinterpret_cast<const float4 *>(b_get + buf * BN * LDK + j * 32 * LDK + half * 8);
+      for (int i = 0; i < TM; i++) av[i] = *reinterpret_cast<const float4 *>(a_get + buf * BM * LDK + i * 32 * LDK + half * 8);
+#pragma unroll
+      for (int j = 0; j < TN; j++) bv[j] = *reinterpret_cast<const float4 *>(b_get + buf * BN * LDK + j * 32 * LDK + half * 8);
+    }
   };
-  auto multiply = [&](const float4 (&av)[TM], const float4 (&bv)[TN]) {
+  auto multiply = [&](auto half, const float4 (&av)[TM], const float4 (&bv)[TN]) {
 #pragma unroll
     for (int c = 0; c < 4; c++)  // consecutive matrix instructions go to different accumulators
 #pragma unroll
@@ -687,7 +734,12 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
         for (int j = 0; j < TN; j++) {
           float x = c == 0 ? av[i].x : c == 1 ? av[i].y : c == 2 ? av[i].z : av[i].w;
           float y = c == 0 ? bv[j].x : c == 1 ? bv[j].y : c == 2 ? bv[j].z : bv[j].w;
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[i][j], 0, 0, 0);
+          if constexpr (R16) {
+            constexpr int blk = decltype(half)::value * TN;
+            acc16[blk + j] = __builtin_amdgcn_mfma_f32_16x16x4f32(x, y, acc16[blk + j], 0, 0, 0);
+          } else {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[i][j], 0, 0, 0);
+          }
         }
   };
 
@@ -712,12 +764,12 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
     }
     if constexpr (decltype(load_ahead)::value) load_tile(nxt, true);
     __builtin_amdgcn_sched_barrier(0);  // memory instructions first, their latency hides behind the multiplies
-    multiply(fa[0], fb[0]);
+    multiply(std::integral_constant<int, 0>{}, fa[0], fb[0]);
     __builtin_amdgcn_sched_barrier(0);
     lds_barrier();
     if constexpr (decltype(write_next)::value) read_half(fa[0], fb[0], nxt, 0);
     __builtin_amdgcn_sched_barrier(0);
-    multiply(fa[1], fb[1]);
+    multiply(std::integral_constant<int, 1>{}, fa[1], fb[1]);
     __builtin_amdgcn_sched_barrier(0);
   };
   using Even = std::integral_constant<int, 0>;
@@ -753,6 +805,17 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
     step(Even{}, No{}, No{});
   }
 
+  if constexpr (R16) {
+    // accumulator layout of v_mfma_f32_16x16x4_f32: register r of lane l holds C[4*(l/16) + r][l%16]
+#pragma unroll
+    for (int j = 0; j < 2 * TN; j++) {
+      uint32_t n = n0 + wn * TN * 32 + j * 16 + lrow;
+      if (n >= N) continue;
+      Epilogue::Col col = ep.column(n);
+      ep.store_quad(col, m0 + 4 * lk, M, acc16[j]);
+    }
+    return;
+  }
   // accumulator layout of v_mfma_f32_32x32x2_f32: register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32]
 #pragma unroll
   for (int j = 0; j < TN; j++) {
@@ -775,7 +838,7 @@ __device__ __forceinline__ uint32_t xcd_swizzle(uint32_t L, uint32_t total) {
 
 // Generic launch: logical block index = (n tile, batch entry, m tile), n slowest, so concurrently running blocks
 // of one XCD share their B tile (the activations) and cycle through the A tiles (the weights).
-template <int TM, int TN, int WGM, int WGN, class SrcA, class SrcB>
+template <int TM, int TN, int WGM, int WGN, bool R16, class SrcA, class SrcB>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN == 1 ? 5 : TM * TN == 2 ? 3 : 2))) void igemm_kernel(SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, uint32_t tiles_m, uint32_t batches) {
   using TS = TileShape<TM, TN, WGM, WGN>;
   __shared__ float4 smem[TS::LDS_FLOATS / 4];
@@ -785,13 +848,16 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN
   a.batch(bz);
   b.batch(bz);
   ep.batch(bz);
-  igemm_body<TM, TN, WGM, WGN>(a, b, ep, M, N, K, mt * TS::BM, nt * TS::BN, reinterpret_cast<float *>(smem));
+  igemm_body<TM, TN, WGM, WGN, R16>(a, b, ep, M, N, K, mt * (R16 ? 16 : TS::BM), nt * TS::BN, reinterpret_cast<float *>(smem));
 }
 
-enum Tile { T128x128, T64x128, T32x128, T64x64 };
-static const char *const tile_names[] = {"128x128", "64x128", "32x128", "64x64"};
+enum Tile { T128x128, T64x128, T32x128, T64x64, T16x256 };
+static const char *const tile_names[] = {"128x128", "64x128", "32x128", "64x64", "16x256"};
+inline uint32_t tile_rows(Tile t) { return t == T128x128 ? 128 : t == T32x128 ? 32 : t == T16x256 ? 16 : 64; }
+inline uint32_t tile_cols(Tile t) { return t == T64x64 ? 64 : t == T16x256 ? 256 : 128; }
 
-int &tile_override();  // -1: choose per shape; 0..3: force a Tile (measurements only)
+int &tile_override();  // -1: choose per shape; 0..4: force a Tile (measurements only)
+int &patch_blocks();   // persistent blocks of tconv_patch16_kernel (measurements only); default two per compute unit
 
 inline const char *shape_label(const char *name, Tile tile, uint32_t M, uint32_t N, uint32_t K, uint32_t batches) {
   char buf[96];
@@ -801,6 +867,7 @@ inline const char *shape_label(const char *name, Tile tile, uint32_t M, uint32_t
 
 inline Tile pick_tile(uint32_t M, uint32_t N, uint32_t batches) {
   if (tile_override() >= 0) return (Tile)tile_override();
+  if (M <= 16) return T16x256;  // the 16x16x4 instruction: no half of the matrix unit multiplies padding
   if (M <= 32) return T32x128;
   if (M <= 64) return T64x64;
   // 64x64 blocks need only 20 KB of LDS and 60 registers, so eight of them share a compute unit and hide each
@@ -816,15 +883,16 @@ int launch(const char *name, SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N
   hipStream_t s = stream();
   const Tile tile = pick_tile(M, N, batches);
   ProfileScope prof(profiling() ? shape_label(name, tile, M, N, K, batches) : name);
-  const uint32_t bm = tile == T128x128 ? 128 : tile == T32x128 ? 32 : 64, bn = tile == T64x64 ? 64 : 128;
+  const uint32_t bm = tile_rows(tile), bn = tile_cols(tile);
   const uint32_t tm = cdiv(M, bm), tn = cdiv(N, bn);
   const size_t total = (size_t)tm * tn * batches;
   if (total > 0x7fffffffu) return fail(MT_E_ARGUMENT, "%s: problem too large for one launch", name);
   switch (tile) {
-    case T128x128: igemm_kernel<2, 2, 2, 2><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
-    case T64x128: igemm_kernel<2, 1, 1, 4><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
-    case T32x128: igemm_kernel<1, 1, 1, 4><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
-    case T64x64: igemm_kernel<1, 1, 2, 2><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+    case T128x128: igemm_kernel<2, 2, 2, 2, false><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+    case T64x128: igemm_kernel<2, 1, 1, 4, false><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+    case T32x128: igemm_kernel<1, 1, 1, 4, false><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+    case T64x64: igemm_kernel<1, 1, 2, 2, false><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
+    case T16x256: igemm_kernel<1, 2, 1, 4, true><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
   }
   MT_LAUNCH_CHECK(name);
   return MT_OK;
@@ -883,7 +951,7 @@ struct TconvArgs {
 };
 
 // FIXED: every phase has taps that tile the k step (see SrcIm2colFixed)
-template <int TM, int TN, int WGM, int WGN, bool FIXED>
+template <int TM, int TN, int WGM, int WGN, bool FIXED, bool R16>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN == 1 ? 5 : TM * TN == 2 ? 3 : 2))) void tconv_kernel(TconvArgs args) {
   using TS = TileShape<TM, TN, WGM, WGN>;
   __shared__ float4 smem[TS::LDS_FLOATS / 4];
@@ -914,7 +982,225 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN
     ep.C += (size_t)slice * args.split_stride;
     if (slice) { ep.bias = nullptr; ep.tap_bias = nullptr; }  // the biases enter once, through slice 0
   }
-  igemm_body<TM, TN, WGM, WGN>(a, b, ep, args.M, N, klen, mt * TS::BM, nt * TS::BN, reinterpret_cast<float *>(smem));
+  igemm_body<TM, TN, WGM, WGN, R16>(a, b, ep, args.M, N, klen, mt * (R16 ? 16 : TS::BM), nt * TS::BN, reinterpret_cast<float *>(smem));
+}
+
+
+// ---- stride-2 transposed convolution to at most 16 channels, operands taken from an input patch in LDS -----------
+// The four stride phases of a 4x4 stride-2 padding-1 transposed convolution (and of "up-sampling x2, then 3x3
+// convolution") are 2x2 convolutions of the SAME input pixels.  As implicit GEMMs every input value is gathered
+// 16 times (4 taps x 4 phases) through the texture path, which then limits a layer with few channels.  Here a block
+// loads the C x 10 x 34 input patch behind 8 x 32 input pixels once, and the matrix unit reads it in place:
+// v_mfma_f32_16x16x4_f32 takes k slot s from lanes 16s..16s+15; one instruction multiplies tap t of the four
+// channels 4i..4i+3, so lane l reads patch[4i + l/16][y + py + t/2][x + l%16 + px + t%2] -- a 32-bit LDS read whose
+// address differs between (i, t, phase, block of pixels) by constants -- and the four taps of channel 4i + l/16 of
+// its row l%16 as one 128-bit read of the packed sub-kernels (k order: channel, tap), which a block keeps in LDS too.
+// A wavefront owns 2 x 32 input pixels = four blocks of 16, for both px of one py at a time, and writes the two px
+// of an output pixel pair together: whole 128-byte lines.
+// Requires: 4 phases of 2x2 taps with offsets (py-1, px-1), phase size = input size, M <= 16, C = CH, bias per row
+// or per tap, output 8-byte aligned.
+//
+// Blocks are persistent (two per compute unit) and walk over the tiles: while the matrix unit works on a tile, the
+// next tile's patch is already on its way into registers (half of it requested before each of the two py passes,
+// so that never more loads are outstanding than the hardware counts), and the stores of a pass drain behind the
+// next pass.  Reads, matrix work and writes of the whole chip then overlap instead of coming in bursts.
+template <int CH>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void tconv_patch16_kernel(TconvArgs args, uint32_t tiles_x, uint32_t tiles_y, uint32_t tiles) {
+  constexpr int TY = 8, TX = 32, P = TX + 2, ROWS = TY + 2;
+  constexpr int PLANE = ROWS * P + 28;  // 368: planes of consecutive channels start 16 banks apart
+  static_assert(PLANE % 32 == 16 && CH % 4 == 0, "LDS layout");
+  constexpr int PAIRS = CH / 4 * ROWS;  // (channel, row) pairs per wavefront, requested in two halves
+  static_assert(CH % 8 == 0 && PAIRS / 2 <= 40, "two batches of loads, each within the outstanding-load counter");
+  constexpr int WROW = CH * 4 + 4;       // a row of coefficients plus 16 bytes: 128-bit reads of 8 rows hit 8 bank groups
+  __shared__ float patch[CH * PLANE];
+  __shared__ float coeff[4 * 16 * WROW];  // [phase][row][channel*4 + tap], rows beyond M zero
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int jj = lane & 15, slot = lane >> 4;
+  const uint32_t H = args.H, W = args.W, HW = H * W;
+
+  // the patch: every (channel, row) pair is one load instruction of 34 lanes; a wavefront takes a quarter of the
+  // channels.  The lane's column goes into the vector offset, channel and row into the scalar offset (additions
+  // only); either may be out of range.
+  float v[PAIRS];
+  auto request_patch = [&](uint32_t tile, auto half) {  // tile >= tiles: every load is out of range (no branch)
+    tile = __builtin_amdgcn_readfirstlane(tile);  // uniform by construction: keeps the offsets below on the scalar unit
+    const uint32_t none = tile < tiles ? 0u : OOB;
+    const uint32_t bx = tile % tiles_x, by = (tile / tiles_x) % tiles_y, w = tile / (tiles_x * tiles_y);
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta + (size_t)(w % args.in_w) * CH * HW, CH * HW * 4u);
+    const int32_t gx = (int32_t)(bx * TX) - 1 + lane;
+    const uint32_t voff = lane < P && (uint32_t)gx < W ? (uint32_t)gx * 4u : OOB;
+    constexpr int C0 = decltype(half)::value * (CH / 8);
+    // scalar offsets: one per row (exactly 2^31 for rows outside the image or a tile that does not exist: with the
+    // channel offset, below 2^31, the sum stays out of range) plus one per channel; a load costs one scalar addition
+    uint32_t row_off[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      const int32_t row = (int32_t)(by * TY) - 1 + r;
+      const uint32_t outside = (uint32_t)((row | ((int32_t)H - 1 - row)) >> 31) | (none ? ~0u : 0u);  // all ones for row < 0 or row >= H
+      row_off[r] = (((uint32_t)row * W * 4u) & ~outside) | (outside & OOB);
+    }
+    uint32_t s_chan = (uint32_t)(wave * (CH / 4) + C0) * HW * 4u;
+#pragma unroll
+    for (int cl = C0; cl < C0 + CH / 8; cl++) {
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) v[cl * ROWS + r] = buf_load(rsrc, voff, s_chan + row_off[r]);
+      s_chan += HW * 4u;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto store_patch = [&]() {
+    float *dst = patch + wave * (CH / 4) * PLANE + lane;
+#pragma unroll
+    for (int i = 0; i < PAIRS; i++)
+      if (lane < P) dst[(i / ROWS) * PLANE + (i % ROWS) * P] = v[i];
+  };
+  using First = std::integral_constant<int, 0>;
+  using Second = std::integral_constant<int, 1>;
+
+  uint32_t tile = __builtin_amdgcn_readfirstlane(blockIdx.x);
+  if (tile >= tiles) return;
+  request_patch(tile, First{});
+  request_patch(tile, Second{});
+  // the coefficients of all four phases, once per block (their loads travel with those of the first patch)
+  {
+    constexpr int VEC = 4 * 16 * CH;  // 128-bit pieces
+    static_assert(VEC % THREADS == 0, "whole rounds of loads");
+#pragma unroll
+    for (int i = 0; i < VEC / THREADS; i++) {
+      const int e = i * THREADS + tid, f = e / (16 * CH), row = (e / CH) % 16, piece = e % CH;
+      const TconvPhase &ph = args.ph[f];
+      const __amdgpu_buffer_rsrc_t rs = make_rsrc(ph.packed, args.M * ph.ld * 4u);
+      const floatx4 t = buf_load4(rs, (uint32_t)row < args.M ? ((uint32_t)row * ph.ld + (uint32_t)piece * 4u) * 4u : OOB, 0);
+      *reinterpret_cast<floatx4 *>(coeff + (f * 16 + row) * WROW + piece * 4) = t;
+    }
+  }
+  store_patch();
+  const float *b_lane = patch + slot * PLANE + wave * 2 * P + jj;
+  __syncthreads();
+
+#pragma unroll 1
+  for (; tile < tiles; tile = __builtin_amdgcn_readfirstlane(tile + gridDim.x)) {
+    const uint32_t bx = tile % tiles_x, by = (tile / tiles_x) % tiles_y, w = tile / (tiles_x * tiles_y);
+    const uint32_t y0 = by * TY, x0 = bx * TX;
+    const uint32_t next = tile + gridDim.x;
+    // bias of the lane's four rows (per row, and per sample where the caller has one set per sample)
+    float row_bias[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const uint32_t m = (uint32_t)(slot * 4 + r);
+      row_bias[r] = args.ep.bias && m < args.M ? args.ep.bias[(w % args.ep.bias_w) * args.ep.bias_stride + m] : 0.f;
+    }
+#pragma unroll
+    for (uint32_t py = 0; py < 2; py++) {
+      if (py == 0) request_patch(next, First{});
+      else request_patch(next, Second{});
+      floatx4acc acc[4][2];
+#pragma unroll
+      for (int b = 0; b < 4; b++)
+#pragma unroll
+        for (int px = 0; px < 2; px++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) acc[b][px][r] = 0.f;
+      // the patch values of step (i, t) + 1 are read while the eight matrix instructions of step (i, t) run; the
+      // two px of a block are neighbours in LDS
+      const float *b_py = b_lane + py * P;
+      float bv[2][4][2];
+      auto read_step = [&](int set, int step) {
+        const int i = step >> 2, t = step & 3;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+          const float *q = b_py + i * 4 * PLANE + ((b >> 1) + (t >> 1)) * P + (b & 1) * 16 + (t & 1);
+          bv[set][b][0] = q[0];
+          bv[set][b][1] = q[1];
+        }
+      };
+      // coefficients of the phases (py, 0) and (py, 1) for the lane's row and the channels 4i + slot: read one
+      // group of four steps ahead
+      const float *a_py = coeff + (py * 2 * 16 + jj) * WROW + slot * 4;
+      floatx4 av[2][2];
+      auto read_coefficients = [&](int set, int i) {
+#pragma unroll
+        for (int px = 0; px < 2; px++) av[set][px] = *reinterpret_cast<const floatx4 *>(a_py + px * 16 * WROW + i * 16);
+      };
+      read_coefficients(0, 0);
+      read_step(0, 0);
+#pragma unroll
+      for (int step = 0; step < CH; step++) {
+        if (step + 1 < CH) read_step((step + 1) & 1, step + 1);
+        if ((step & 3) == 0 && step + 4 < CH) read_coefficients(((step >> 2) + 1) & 1, (step >> 2) + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+          for (int px = 0; px < 2; px++)
+            acc[b][px] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[(step >> 2) & 1][px][step & 3], bv[step & 1][b][px], acc[b][px], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // accumulator layout: register r of lane l holds channel 4*(l/16) + r of pixel l%16.  value = acc + bias of
+      // the row + bias of every filter once per contributing tap (as the CPU path adds it), then the function: the
+      // order of the other kernels.  Output pixel (2*qy + py, 2*qx + px): the two px are written together.
+      float *image = args.ep.C + (size_t)w * args.ep.g_stride;
+      const float tap_bias = args.ep.tap_bias ? args.ep.tap_bias[w % args.ep.bias_w] : 0.f;
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        const uint32_t qy = y0 + wave * 2 + (b >> 1), qx = x0 + (b & 1) * 16 + jj;
+        const int ny = (int)((uint32_t)(qy + py - 1) < H) + (int)((uint32_t)(qy + py) < H);
+        const float extra0 = tap_bias * (float)(ny * ((int)((uint32_t)(qx - 1) < W) + 1));
+        const float extra1 = tap_bias * (float)(ny * (1 + (int)(qx + 1 < W)));
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          acc[b][0][r] = acc[b][0][r] + row_bias[r] + extra0;
+          acc[b][1][r] = acc[b][1][r] + row_bias[r] + extra1;
+        }
+      }
+      // the function is tested once for the 32 values (callers pass none, linear, ReLU or leaky ReLU)
+      if (args.ep.func == MT_F_RELU) {
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+          for (int px = 0; px < 2; px++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[b][px][r] = acc[b][px][r] > 0.f ? acc[b][px][r] : 0.f;
+      } else if (args.ep.func == MT_F_LEAKY_RELU) {
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+          for (int px = 0; px < 2; px++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[b][px][r] = acc[b][px][r] > 0.f ? acc[b][px][r] : (float)(0.1 * (double)acc[b][px][r]);
+      }
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        const uint32_t qy = y0 + wave * 2 + (b >> 1), qx = x0 + (b & 1) * 16 + jj;
+        const bool pixel = qy < H && qx < W;
+        const uint32_t off = (2 * qy + py) * args.ep.OW + 2 * qx;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const uint32_t m = (uint32_t)(slot * 4 + r);
+          if (pixel && m < args.M) *reinterpret_cast<float2 *>(image + (m * args.ep.row_stride + off)) = make_float2(acc[b][0][r], acc[b][1][r]);
+        }
+      }
+    }
+    if (next < tiles) {
+      __syncthreads();  // nobody reads the old patch any more
+      store_patch();
+      __syncthreads();
+    }
+  }
+}
+
+// whether the launch is the shape tconv_patch16_kernel covers; on success `order` maps (py, px) to the phase index
+inline bool tconv_patch16_fits(const TconvArgs &args) {
+  if (args.nphase != 4 || args.M > 16 || (args.C != 16 && args.C != 32) || args.ep.sy != 2 || args.ep.sx != 2 || args.ep.accumulate || !epilogue_func(args.ep.func)) return false;
+  if ((args.ep.bias && args.ep.bias_mode != 1) || ((uintptr_t)args.ep.C & 7u) || args.ep.row_stride % 2 || args.ep.g_stride % 2 || args.ep.OW != 2 * args.W) return false;
+  if ((uint64_t)args.M * args.ep.row_stride >= (1u << 30) || (args.ep.tap_bias && args.ep.IH != args.H) || (args.ep.tap_bias && args.ep.IW != args.W)) return false;
+  for (uint32_t f = 0; f < 4; f++) {
+    const TconvPhase &ph = args.ph[f];
+    if (ph.py != f / 2 || ph.px != f % 2 || ph.taps_y != 2 || ph.taps_x != 2 || ph.offy != (int32_t)ph.py - 1 || ph.offx != (int32_t)ph.px - 1 ||
+        ph.qh != args.H || ph.qw != args.W || ph.kp != args.C * 4)
+      return false;
+  }
+  return true;
 }
 
 // out_floats > 0: the whole output tensor (args.ep.C, out_floats values, every pixel written by exactly one phase) may be
@@ -923,8 +1209,22 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN
 inline int launch_tconv(const char *name, TconvArgs &args, uint32_t max_n, size_t out_floats = 0) {
   if (args.M == 0 || max_n == 0 || args.nphase == 0) return MT_OK;
   hipStream_t s = stream();
+  if (tile_override() < 0 && tconv_patch16_fits(args)) {
+    const uint32_t tiles_x = cdiv(args.W, 32), tiles_y = cdiv(args.H, 8);
+    const size_t tiles = (size_t)tiles_x * tiles_y * args.out_w;
+    if (tiles <= 0x7fffffffu) {
+      ProfileScope prof(profiling() ? shape_label(name, T16x256, args.M, max_n, args.C * 4, 4) : name);
+      args.nsplit = 1;
+      const uint32_t most = (uint32_t)patch_blocks();  // persistent blocks, two per compute unit
+      const uint32_t grid = tiles < most ? (uint32_t)tiles : most;
+      if (args.C == 16) tconv_patch16_kernel<16><<<grid, THREADS, 0, s>>>(args, tiles_x, tiles_y, (uint32_t)tiles);
+      else tconv_patch16_kernel<32><<<grid, THREADS, 0, s>>>(args, tiles_x, tiles_y, (uint32_t)tiles);
+      MT_LAUNCH_CHECK(name);
+      return MT_OK;
+    }
+  }
   const Tile tile = pick_tile(args.M, max_n, args.nphase);
-  const uint32_t bm = tile == T128x128 ? 128 : tile == T32x128 ? 32 : 64, bn = tile == T64x64 ? 64 : 128;
+  const uint32_t bm = tile_rows(tile), bn = tile_cols(tile);
   args.tiles_m = cdiv(args.M, bm);
   size_t total = (size_t)args.tiles_m * cdiv(max_n, bn) * args.nphase;
   uint32_t kmax = 0, kmin = 0xffffffffu;
@@ -965,17 +1265,19 @@ inline int launch_tconv(const char *name, TconvArgs &args, uint32_t max_n, size_
   const uint32_t grid = (uint32_t)total;
   if (fixed) {
     switch (tile) {
-      case T128x128: tconv_kernel<2, 2, 2, 2, true><<<grid, THREADS, 0, s>>>(args); break;
-      case T64x128: tconv_kernel<2, 1, 1, 4, true><<<grid, THREADS, 0, s>>>(args); break;
-      case T32x128: tconv_kernel<1, 1, 1, 4, true><<<grid, THREADS, 0, s>>>(args); break;
-      case T64x64: tconv_kernel<1, 1, 2, 2, true><<<grid, THREADS, 0, s>>>(args); break;
+      case T128x128: tconv_kernel<2, 2, 2, 2, true, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T64x128: tconv_kernel<2, 1, 1, 4, true, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T32x128: tconv_kernel<1, 1, 1, 4, true, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T64x64: tconv_kernel<1, 1, 2, 2, true, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T16x256: tconv_kernel<1, 2, 1, 4, true, true><<<grid, THREADS, 0, s>>>(args); break;
     }
   } else {
     switch (tile) {
-      case T128x128: tconv_kernel<2, 2, 2, 2, false><<<grid, THREADS, 0, s>>>(args); break;
-      case T64x128: tconv_kernel<2, 1, 1, 4, false><<<grid, THREADS, 0, s>>>(args); break;
-      case T32x128: tconv_kernel<1, 1, 1, 4, false><<<grid, THREADS, 0, s>>>(args); break;
-      case T64x64: tconv_kernel<1, 1, 2, 2, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T128x128: tconv_kernel<2, 2, 2, 2, false, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T64x128: tconv_kernel<2, 1, 1, 4, false, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T32x128: tconv_kernel<1, 1, 1, 4, false, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T64x64: tconv_kernel<1, 1, 2, 2, false, false><<<grid, THREADS, 0, s>>>(args); break;
+      case T16x256: tconv_kernel<1, 2, 1, 4, false, true><<<grid, THREADS, 0, s>>>(args); break;
     }
   }
   MT_LAUNCH_CHECK(name);

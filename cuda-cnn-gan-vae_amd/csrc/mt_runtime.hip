@@ -103,6 +103,7 @@ int mt_set_option(const char *name, int value) {
   if (name && strcmp(name, "conv_path") == 0) return mt::set_conv_path(value);
   if (name && strcmp(name, "igemm_tile") == 0) return mt::set_igemm_tile(value);
   if (name && strcmp(name, "wgrad_groups") == 0) return mt::set_wgrad_groups(value);
+  if (name && strcmp(name, "patch_blocks") == 0) return mt::set_patch_blocks(value);
   return mt::fail(MT_E_ARGUMENT, "mt_set_option: unknown option '%s'", name ? name : "(null)");
 }
 

@@ -23,7 +23,7 @@ def gpu():
     return Gpu()
 
 
-@pytest.fixture(params=[(2, -1), (2, 0), (2, 1), (2, 3), (1, -1)], ids=["auto", "mfma-128x128", "mfma-64x128", "mfma-64x64", "direct"])
+@pytest.fixture(params=[(2, -1), (2, 0), (2, 1), (2, 3), (2, 4), (1, -1)], ids=["auto", "mfma-128x128", "mfma-64x128", "mfma-64x64", "mfma-16x256", "direct"])
 def path(request, gpu):
     """Kernel family under test: per-shape choice (vector-ALU kernel for very few output channels, matrix cores
     otherwise), the matrix-core kernels with one forced block tile, or the one-thread-per-output kernels."""
@@ -314,6 +314,8 @@ def test_convolution_backward_weights_sum(gpu, oracle, path, case):
     (2, 4, 5, 3, 70),       # odd input sizes, more filters than one tile
     (2, 64, 12, 16, 32),    # a layer of the reference's GAN generator at a quarter of its width
     (2, 512, 3, 4, 64),     # its first layer: few blocks, k = 2048 per phase, split over k
+    (2, 32, 12, 16, 16),    # its last up-sampling layer at an eighth of the size: the input patch kernel
+    (3, 16, 9, 35, 7),      # the same kernel with sixteen channels, seven filters and partial tiles
 ])
 def test_upsampling_convolution(gpu, oracle, path, case):
     """Up-sampling x2 + convolution 3x3 stride 1 padding 1 (+ function) in one call, against the two layers on the
@@ -336,6 +338,66 @@ def test_upsampling_convolution_other_geometries(gpu, oracle, path):
         close(gpu.upsampling_convolution(image, kernel, bias, k, 6, 9, up=up, s=s, p=p), want, 1e-5)
     with pytest.raises(Exception):
         gpu.upsampling_convolution(image, Nrm(2, 1, 1, 9, 54, std=0.2), U(3, 1, 8, 1, 1), 3, 6, 9)   # eight biases for nine filters
+
+
+@pytest.mark.parametrize("case", [
+    # W, C (output channels of the transposed convolution), H, Wd, KA, k, s, p
+    (3, 16, 21, 19, 24, 4, 2, 1),     # sixteen rows exactly, 840 columns per phase: a partial last block of 256
+    (2, 13, 9, 40, 32, 4, 2, 1),      # thirteen rows: the last quad of accumulator rows holds one real row
+    (2, 9, 17, 15, 20, 3, 1, 1),      # taps that do not tile the k step
+    (1, 6, 30, 33, 7, 5, 3, 2),       # stride 3: nine phases of unequal size
+    (2, 16, 12, 12, 48, 2, 2, 0),     # 2x2 stride 2: one tap per phase
+])
+def test_transposed_convolution_sixteen_row_blocks(gpu, oracle, path, case):
+    """Transposed convolutions to 5..16 channels run on 16 x 256 blocks (the 16x16x4 matrix instruction): with and
+    without bias, with the functions the epilogue applies itself and one it does not."""
+    W, C, H, Wd, KA, k, s, p = case
+    oy, ox = (H - k + 2 * p) // s + 1, (Wd - k + 2 * p) // s + 1
+    delta, kernel = U(4, W, KA, oy, ox), Nrm(5, 1, 1, KA, C * k * k, std=0.2)
+    for bias, func in ((np.zeros((1, KA, 1, 1), np.float32), None), (U(6, 1, KA, 1, 1), "relu"), (U(6, 1, KA, 1, 1), "leaky_relu"), (U(6, 1, KA, 1, 1), "sigmoid")):
+        want = oracle.backward_convolution(delta, kernel, bias, k, k, C, KA, s, s, p, p, (W, C, H, Wd))
+        if func:
+            want = oracle.apply_func(want, func)
+        close(gpu.backward_convolution(delta, kernel, bias, k, k, C, KA, s, s, p, p, (W, C, H, Wd), func=func), want)
+
+
+@pytest.mark.parametrize("case", [
+    # W, out channels, delta H, delta W, in channels
+    (3, 13, 10, 9, 32),       # one partial tile of 8 x 32 input pixels
+    (2, 16, 13, 45, 16),      # partial tiles on both axes, sixteen channels
+    (1, 5, 24, 64, 32),       # whole tiles
+    (2, 16, 1, 1, 16),        # one input pixel: every tap but one is padding
+])
+def test_transposed_convolution_from_an_input_patch(gpu, oracle, path, case):
+    """4x4 stride 2 padding 1 to at most 16 channels from 16 or 32: the kernel that keeps the input patch in LDS and
+    computes all four stride phases from it.  Bias per contributing tap as on the CPU path, functions in the epilogue."""
+    W, C, H, Wd, KA = case
+    delta, kernel, bias = U(4, W, KA, H, Wd), Nrm(5, 1, 1, KA, C * 16, std=0.2), U(6, 1, KA, 1, 1) * 0.2
+    want = oracle.backward_convolution(delta, kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd))
+    close(gpu.backward_convolution(delta, kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd)), want)
+    close(gpu.backward_convolution(delta, kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd), func="tangence"), oracle.apply_func(want, "tangence"))
+    # delta broadcast over the batch of the output
+    want = oracle.backward_convolution(delta[:1], kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (2, C, 2 * H, 2 * Wd))
+    close(gpu.backward_convolution(delta[:1], kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (2, C, 2 * H, 2 * Wd)), want)
+
+
+def test_sixteen_row_blocks_forced_on_taller_products(gpu, oracle):
+    """The same block forced on 40 output channels: three row blocks, the last one half empty."""
+    import mi355tensor as mt
+    W, C, H, Wd, KA = 2, 40, 10, 14, 24
+    delta, kernel, bias = U(4, W, KA, 5, 7), Nrm(5, 1, 1, KA, C * 16, std=0.2), U(6, 1, KA, 1, 1)
+    want = oracle.backward_convolution(delta, kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (W, C, H, Wd))
+    mt.set_option("igemm_tile", 4)
+    try:
+        got = gpu.backward_convolution(delta, kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (W, C, H, Wd))
+        image, k3, b3 = U(1, 2, 8, 6, 10), Nrm(2, 1, 1, 40, 8 * 9, std=0.2), U(3, 1, 40, 1, 1)
+        got_up = gpu.upsampling_convolution(image, k3, b3, 3, 8, 40)
+        got_fwd = gpu.forward_convolution(image, k3, b3, 3, 3, 8, 40, 1, 1, 1, 1)
+    finally:
+        mt.set_option("igemm_tile", -1)
+    close(got, want)
+    close(got_up, oracle.forward_convolution(oracle.upsampling(image, 2, 2), k3, b3, 3, 3, 8, 40, 1, 1, 1, 1), 1e-5)
+    close(got_fwd, oracle.forward_convolution(image, k3, b3, 3, 3, 8, 40, 1, 1, 1, 1))
 
 
 def test_image_layer_kernels_both_tilings(gpu, oracle):
