@@ -88,8 +88,10 @@ int mt_timer_start(void *timer);
 int mt_timer_stop(void *timer, float *milliseconds);
 int mt_timer_destroy(void *timer);
 /* "conv_path": 0 choose per shape (default), 1 one-thread-per-output kernels in the CPU path's summation order,
- * 2 matrix-core kernels wherever they apply.  "igemm_tile": -1 choose per shape (default), 0..3 force the block
- * tile 128x128 / 64x128 / 32x128 / 64x64 of the matrix-core kernels.  "wgrad_groups": 0 choose per shape (default),
+ * 2 matrix-core kernels wherever they apply.  "igemm_tile": -1 choose per shape (default), 0..4 force the block
+ * tile 128x128 / 64x128 / 32x128 / 64x64 / 16x256 of the matrix-core kernels (a forced tile also switches off the
+ * kernels that are chosen by shape beside them).  "patch_blocks": persistent blocks of the input-patch transposed
+ * convolution (default 512, two per compute unit).  "wgrad_groups": 0 choose per shape (default),
  * n split the batch of mt_convolution_backward_weights_sum into n groups (when n divides the batch).  For tests and
  * measurements; results agree within fp32 rounding. */
 int mt_set_option(const char *name, int value);
