@@ -1140,18 +1140,28 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
       // the row + bias of every filter once per contributing tap (as the CPU path adds it), then the function: the
       // order of the other kernels.  Output pixel (2*qy + py, 2*qx + px): the two px are written together.
       float *image = args.ep.C + (size_t)w * args.ep.g_stride;
-      const float tap_bias = args.ep.tap_bias ? args.ep.tap_bias[w % args.ep.bias_w] : 0.f;
+      if (args.ep.tap_bias) {
+        const float tap_bias = args.ep.tap_bias[w % args.ep.bias_w];
 #pragma unroll
-      for (int b = 0; b < 4; b++) {
-        const uint32_t qy = y0 + wave * 2 + (b >> 1), qx = x0 + (b & 1) * 16 + jj;
-        const int ny = (int)((uint32_t)(qy + py - 1) < H) + (int)((uint32_t)(qy + py) < H);
-        const float extra0 = tap_bias * (float)(ny * ((int)((uint32_t)(qx - 1) < W) + 1));
-        const float extra1 = tap_bias * (float)(ny * (1 + (int)(qx + 1 < W)));
+        for (int b = 0; b < 4; b++) {
+          const uint32_t qy = y0 + wave * 2 + (b >> 1), qx = x0 + (b & 1) * 16 + jj;
+          const int ny = (int)((uint32_t)(qy + py - 1) < H) + (int)((uint32_t)(qy + py) < H);
+          const float extra0 = tap_bias * (float)(ny * ((int)((uint32_t)(qx - 1) < W) + 1));
+          const float extra1 = tap_bias * (float)(ny * (1 + (int)(qx + 1 < W)));
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          acc[b][0][r] = acc[b][0][r] + row_bias[r] + extra0;
-          acc[b][1][r] = acc[b][1][r] + row_bias[r] + extra1;
+          for (int r = 0; r < 4; r++) {
+            acc[b][0][r] = acc[b][0][r] + row_bias[r] + extra0;
+            acc[b][1][r] = acc[b][1][r] + row_bias[r] + extra1;
+          }
         }
+      } else {  // (vector instructions of one wavefront do not overlap with the matrix instructions of another: fewer is faster)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            acc[b][0][r] += row_bias[r];
+            acc[b][1][r] += row_bias[r];
+          }
       }
       // the function is tested once for the 32 values (callers pass none, linear, ReLU or leaky ReLU)
       if (args.ep.func == MT_F_RELU) {
@@ -1181,10 +1191,10 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
       }
     }
-    if (next < tiles) {
-      __syncthreads();  // nobody reads the old patch any more
+    if (next < tiles) {  // barriers that order LDS traffic only: the stores of this tile keep draining behind them
+      lds_barrier();     // nobody reads the old patch any more
       store_patch();
-      __syncthreads();
+      lds_barrier();
     }
   }
 }
