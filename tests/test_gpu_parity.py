@@ -379,6 +379,10 @@ def test_transposed_convolution_from_an_input_patch(gpu, oracle, path, case):
     # delta broadcast over the batch of the output
     want = oracle.backward_convolution(delta[:1], kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (2, C, 2 * H, 2 * Wd))
     close(gpu.backward_convolution(delta[:1], kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (2, C, 2 * H, 2 * Wd)), want)
+    # one set of biases per sample
+    biases = U(7, W, KA, 1, 1) * 0.2
+    want = oracle.backward_convolution(delta, kernel, biases, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd))
+    close(gpu.backward_convolution(delta, kernel, biases, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd), func="relu"), oracle.apply_func(want, "relu"))
 
 
 def test_sixteen_row_blocks_forced_on_taller_products(gpu, oracle):
