@@ -80,6 +80,50 @@ class GanGenerator:
     def set_noise(self, z):
         self.noise.upload(z)
 
+    # ---- network file ----------------------------------------------------------------------------------------
+    # cmodel_gan.cu.h:136-225: the input holder is a Linear layer without a predecessor, which saves two [1,1,1,1] tensors
+    # (netlayer/cnetlayerlinear.cu.h:175-178)
+    LAYER_KINDS = ["linear", "linear", "function"] + ["upsampling", "convolution", "batchnorm", "function"] * 6 + ["convolution", "function"]
+
+    def save_net(self, f):
+        """The parameters as SaveNetLayers writes the reference's generator (cuda/netmodel/cmodelmain.cu.h:296-300).  This
+        class keeps no running statistics: mean 0 and variable 1 are written, the values of a fresh layer."""
+        import wire_format
+        one = np.zeros((1, 1, 1, 1), np.float32)
+        layers = [("linear", {"weight": one, "bias": one}),
+                  ("linear", {"weight": self.p["lin_w"].numpy(), "bias": self.p["lin_b"].numpy()}), ("function", {"name": "leaky_relu"})]
+        widths = self.channels[1:] + (IMAGE_DEPTH,)
+        for i in range(7):
+            cin = self.channels[i]
+            header = dict(kernel_amount=widths[i], kernel_x=3, kernel_y=3, kernel_z=cin, stride_x=1, stride_y=1, padding_x=1, padding_y=1)
+            if i < 6:
+                layers.append(("upsampling", {"x": 2, "y": 2}))
+            layers.append(("convolution", {"header": header, "kernel": self.p["kernel%d" % i].numpy(), "bias": self.p["bias%d" % i].numpy()}))
+            if i < 6:
+                beta = self.p["beta%d" % i].numpy()
+                layers.append(("batchnorm", {"beta": beta, "gamma": self.p["gamma%d" % i].numpy(), "mean": np.zeros_like(beta),
+                                             "variable": np.ones_like(beta), "momentum": MOMENTUM}))
+                layers.append(("function", {"name": "leaky_relu"}))
+        layers.append(("function", {"name": "tangence"}))
+        wire_format.write_net(f, layers)
+
+    def load_net(self, f):
+        """The inverse; tensor sizes in the file must be this network's (the reference loads with check_size)."""
+        import wire_format
+        layers = wire_format.read_net(f, self.LAYER_KINDS)
+        found = {"lin_w": layers[1][1]["weight"], "lin_b": layers[1][1]["bias"]}
+        convs = [p for kind, p in layers if kind == "convolution"]
+        norms = [p for kind, p in layers if kind == "batchnorm"]
+        for i, c in enumerate(convs):
+            found["kernel%d" % i], found["bias%d" % i] = c["kernel"], c["bias"]
+        for i, n in enumerate(norms):
+            found["gamma%d" % i], found["beta%d" % i] = n["gamma"], n["beta"]
+        for name, a in found.items():
+            if a.shape != self.p[name].shape:
+                raise ValueError("%s: the file holds %s, the network %s" % (name, a.shape, self.p[name].shape))
+        for name, a in found.items():
+            self.p[name].upload(a)
+
     def forward(self, fused=True):
         p, ch = self.p, self.channels
         Fused.LinearForward(self.lin_out, p["lin_w"], self.noise, p["lin_b"], "leaky_relu")

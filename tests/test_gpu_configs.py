@@ -244,6 +244,31 @@ def test_shipped_gan_generator_topology(gpu, oracle):
         assert rel_err(one, want["c%d" % i]) <= REL, "up-sampling + conv %d" % i
 
 
+def test_gan_generator_network_file_round_trip(gpu):
+    """The generator's parameters in the layer order of the reference's GAN model (two Linear layers, the first one the
+    input holder with 1x1 tensors), loaded into a differently initialised copy: same image bit for bit."""
+    import io
+    import gan_generator as GG
+    import wire_format as wf
+    channels, noise_size, b = (64, 64, 32, 16, 16, 8, 4), 32, 2
+    net = GG.GanGenerator(b, GG.make_parameters(channels, noise_size), channels, noise_size)
+    other = GG.GanGenerator(b, GG.make_parameters(channels, noise_size, seed=99), channels, noise_size)
+    noise = GG.make_noise(b, noise_size)
+    net.set_noise(noise)
+    other.set_noise(noise)
+    f = io.BytesIO()
+    net.save_net(f)
+    raw = f.getvalue()
+    head = wf.read_net(io.BytesIO(raw), GG.GanGenerator.LAYER_KINDS[:5])
+    assert head[0][1]["weight"].shape == (1, 1, 1, 1) and head[2][1]["name"] == "leaky_relu" and head[3][1] == {"x": 2, "y": 2}
+    assert head[4][1]["header"]["kernel_amount"] == 64 and head[4][1]["kernel"].shape == (1, 1, 64, 64 * 9)
+    assert not np.array_equal(net.forward(True).numpy(), other.forward(True).numpy())
+    other.load_net(io.BytesIO(raw))
+    assert np.array_equal(net.forward(True).numpy(), other.forward(True).numpy())
+    with pytest.raises(ValueError):
+        GG.GanGenerator(b, None, (64, 64, 32, 16, 16, 8, 8), noise_size).load_net(io.BytesIO(raw))
+
+
 def vae_parameters():
     import vae
     return vae.make_parameters()
