@@ -84,6 +84,17 @@ class CMemoryStream:public IDataStream
   CMemoryStream(void):Pos(0) {}
   void Rewind(void) {Pos=0;}
   const std::vector<uint8_t>& Bytes(void) const {return(Data);}
+  bool ReadFile(const char *name)
+  {
+   FILE *file=fopen(name,"rb");
+   if (file==NULL) return(false);
+   uint8_t buffer[4096];
+   size_t n;
+   while((n=fread(buffer,1,sizeof(buffer),file))>0) Data.insert(Data.end(),buffer,buffer+n);
+   fclose(file);
+   Pos=0;
+   return(true);
+  }
   int8_t LoadInt8(void) {return(Get<int8_t>());}
   int16_t LoadInt16(void) {return(Get<int16_t>());}
   int32_t LoadInt32(void) {return(Get<int32_t>());}
@@ -371,13 +382,41 @@ static void ChainC(void)
 }
 #endif
 
+// Chain G: the layers of chain A loaded from a network file that somebody else wrote (every layer's Load() in order,
+// as CModelMain::LoadNetLayers does), forward only
+static void ChainG(const char *net_file)
+{
+ CNetLayerConvolutionInput<type_t> input(3,16,16,BATCH);
+ CNetLayerConvolution<type_t> conv(8,4,2,2,1,1,&input,BATCH);
+ CNetLayerFunction<type_t> f1(NNeuron::NEURON_FUNCTION_SIGMOID,&conv,BATCH);   // the file says leaky ReLU: Load() must take it from there
+ CNetLayerLinear<type_t> lin(24,&f1,BATCH);
+ CNetLayerFunction<type_t> f2(NNeuron::NEURON_FUNCTION_SIGMOID,&lin,BATCH);
+ CMemoryStream net;
+ if (net.ReadFile(net_file)==false) throw("network file not found");
+ INetLayer<type_t> *layers[5]={&input,&conv,&f1,&lin,&f2};
+ for(int n=0;n<5;n++) layers[n]->Load(&net,true);
+ CTensor<type_t> image(BATCH,3,16,16);
+ FillTensor(image,1.0);
+ input.SetOutput(image);
+ for(int n=0;n<5;n++) layers[n]->Forward();
+ Dump("G.input",image);
+ Dump("G.leaky",f1.GetOutputTensor());
+ Dump("G.sigmoid",f2.GetOutputTensor());
+}
+
 int main(int argc,char **argv)
 {
- if (argc<2) {fprintf(stderr,"usage: %s <output file>\n",argv[0]);return(2);}
+ if (argc<2) {fprintf(stderr,"usage: %s <output file> [network file for chain G]\n",argv[0]);return(2);}
  out_file=fopen(argv[1],"wb");
  if (out_file==NULL) return(2);
  try
  {
+  if (argc>2)   // only the chain that loads the given network file
+  {
+   ChainG(argv[2]);
+   fclose(out_file);
+   return(0);
+  }
   ChainA();
   ChainB();
   ChainD();

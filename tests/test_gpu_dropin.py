@@ -111,3 +111,16 @@ def test_reference_batchnorm_layer_saved_stream(dumps, oracle):
     # the conv and linear streams of the drop-in build carry the same layout as the reference's CPU build
     header, kernel, bias = wf.read_convolution_layer(io.BytesIO(gpu["A.conv_stream"].tobytes()))
     assert np.array_equal(kernel, gpu["A.conv_updated.0"]) and np.array_equal(bias, gpu["A.conv_updated.1"])
+
+
+def test_dropin_layers_load_a_network_written_from_python(oracle, tmp_path):
+    """A network file written by wire_format.py, loaded by the reference's layers on the drop-in classes: forward on the
+    GPU against the oracle on the same weights."""
+    if not os.path.exists(LAYERS_GPU):
+        pytest.skip("oracle/_ref/layers_mi355 not built (it needs /root/reference)")
+    from test_wire_format import chain_g_network, run_chain_g, expected_chain_g
+    layers = chain_g_network(seed=4)
+    got = run_chain_g(LAYERS_GPU, layers, tmp_path)
+    leaky, prob = expected_chain_g(oracle, layers, got["G.input"])
+    assert rel_err(got["G.leaky"], leaky) <= 1e-4
+    assert rel_err(got["G.sigmoid"], prob.reshape(got["G.sigmoid"].shape)) <= 1e-4

@@ -148,3 +148,46 @@ def test_net_round_trip_of_the_other_layer_kinds():
         wf.read_net(io.BytesIO(struct.pack("=I", 9)), ["function"])
     with pytest.raises(EOFError):
         wf.read_net(io.BytesIO(b""), ["upsampling"])
+
+
+def chain_g_network(seed=3):
+    """The layers of the harness's chain G with weights of our own."""
+    rng = np.random.default_rng(seed)
+    header = dict(kernel_amount=8, kernel_x=4, kernel_y=4, kernel_z=3, stride_x=2, stride_y=2, padding_x=1, padding_y=1)
+    return [("input", {}),
+            ("convolution", {"header": header, "kernel": (rng.standard_normal((1, 1, 8, 48)) * 0.2).astype(np.float32),
+                             "bias": (rng.standard_normal((1, 8, 1, 1)) * 0.1).astype(np.float32)}),
+            ("function", {"name": "leaky_relu"}),
+            ("linear", {"weight": (rng.standard_normal((1, 1, 24, 512)) * 0.08).astype(np.float32),
+                        "bias": (rng.standard_normal((1, 1, 24, 1)) * 0.1).astype(np.float32)}),
+            ("function", {"name": "sigmoid"})]
+
+
+def run_chain_g(exe, layers, tmp_path):
+    net, dump = str(tmp_path / "net.bin"), str(tmp_path / "g.bin")
+    with open(net, "wb") as f:
+        wf.write_net(f, layers)
+    run = subprocess.run([exe, dump, net], capture_output=True, text=True, timeout=180)
+    assert run.returncode == 0, run.stderr
+    return {k: as_array(v) for k, v in read_dump_bytes(dump).items()}
+
+
+def expected_chain_g(lib, layers, image):
+    import layer_sequences as seq
+    conv, lin = layers[1][1], layers[3][1]
+    a = lib.apply_func(seq.conv_forward(lib, image, conv["kernel"], conv["bias"], 4, 2, 1), "leaky_relu")
+    out = seq.linear_forward(lib, lin["weight"], a.reshape(a.shape[0], 1, -1, 1), lin["bias"])
+    return a, lib.apply_func(out, "sigmoid")
+
+
+def test_reference_layers_load_a_network_written_here(oracle, tmp_path):
+    """The other direction: a network file written by wire_format.py, loaded by the reference's own convolution, function
+    and linear layers (on the reference's CPU tensor classes) with Load(); their forward pass must be the oracle's on
+    the same weights.  The function layer is constructed as a sigmoid and becomes a leaky ReLU by loading."""
+    if not os.path.exists(LAYERS_CPU):
+        pytest.skip("oracle/_ref/layers_cpu not built (it needs /root/reference)")
+    layers = chain_g_network()
+    got = run_chain_g(LAYERS_CPU, layers, tmp_path)
+    leaky, prob = expected_chain_g(oracle, layers, got["G.input"])
+    assert np.array_equal(got["G.leaky"], leaky)
+    assert np.max(np.abs(got["G.sigmoid"] - prob.reshape(got["G.sigmoid"].shape))) <= 1e-6
