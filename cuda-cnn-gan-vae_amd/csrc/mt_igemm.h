@@ -867,7 +867,9 @@ inline const char *shape_label(const char *name, Tile tile, uint32_t M, uint32_t
 
 inline Tile pick_tile(uint32_t M, uint32_t N, uint32_t batches) {
   if (tile_override() >= 0) return (Tile)tile_override();
-  if (M <= 16) return T16x256;  // the 16x16x4 instruction: no half of the matrix unit multiplies padding
+  // the 16x16x4 instruction: no half of the matrix unit multiplies padding; with few columns the narrower block of the
+  // 32-row tile gives twice the blocks, which matters more
+  if (M <= 16 && (size_t)cdiv(N, 256) * batches >= 256) return T16x256;
   if (M <= 32) return T32x128;
   if (M <= 64) return T64x64;
   // 64x64 blocks need only 20 KB of LDS and 60 registers, so eight of them share a compute unit and hide each
