@@ -520,24 +520,30 @@ struct HaloTile {
 // as [ci][phase][co][taps].
 // PP = 2 as described; PP = 1: one input pixel per thread and tiles of 16 x 16, twice the wavefronts (and twice the LDS
 // reads per multiply-add) for inputs so small that the grid would otherwise not give every SIMD two wavefronts.
-template <int CO, int PP>
-__global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
-  using Tile = HaloTile<16 * PP, 16, 8>;
-  constexpr int TW = 16 * PP, TH = 16, CC = 8, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
-  __shared__ __attribute__((aligned(16))) float tile[2][CC][ROWS][PITCH];
+// SPLIT = 2: the block is two halves of 256 threads that take every other chunk of (then four) channels, each with its
+// own pair of LDS buffers, and add their sums at the end: twice the wavefronts per SIMD for a grid of two blocks per
+// compute unit, where the multiply-adds of one wavefront otherwise wait for its own LDS and scalar loads.
+template <int CO, int PP, int SPLIT>
+__global__ __launch_bounds__(256 * SPLIT) void tconv_k4s2_tile_kernel(TconvArgs args) {
+  constexpr int CC = SPLIT == 2 ? 4 : 8;
+  using Tile = HaloTile<16 * PP, 16, CC>;
+  constexpr int TW = 16 * PP, TH = 16, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
+  __shared__ __attribute__((aligned(16))) float tiles[SPLIT][2][CC][ROWS][PITCH];
+  static_assert(SPLIT == 1 || sizeof(tiles) >= sizeof(float) * 256 * PP * 4 * CO, "the sums of the second half fit into the tile memory");
   const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W, M = args.M;
   const uint32_t tiles_x = (W + TW - 1) / TW;
   const uint32_t x0 = (blockIdx.x % tiles_x) * TW, y0 = (blockIdx.x / tiles_x) * TH, g = blockIdx.y;
-  const uint32_t tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  const uint32_t half = SPLIT == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / 256) : 0u, tid = threadIdx.x % 256, tx = tid % 16, ty = tid / 16;
+  auto &tile = tiles[half];
   Tile stage;
   stage.setup(args.delta, args.in_w * C * HW * 4u, (g % args.in_w) * C * HW * 4u, H, W, x0, y0, tid);
-  auto fetch = [&](uint32_t chunk) { stage.fetch(chunk); };
+  auto fetch = [&](uint32_t step) { stage.fetch(step * SPLIT + half); };
   auto put = [&](int buf) { stage.put(&tile[buf][0][0][0]); };
 
   float acc[PP][2][2][CO];  // [pixel][py][px][co]
 #pragma unroll
   for (int i = 0; i < PP * 4 * CO; i++) (&acc[0][0][0][0])[i] = 0.f;
-  const uint32_t chunks = C / CC;
+  const uint32_t chunks = C / (CC * SPLIT);  // steps of a half
   const float *coeff = args.ph[0].packed;
   fetch(0);
   put(0);
@@ -547,7 +553,7 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
     if (ch + 1 < chunks) fetch(ch + 1);
 #pragma unroll 2
     for (int c = 0; c < CC; c++) {
-      const uint32_t ci = ch * CC + c;
+      const uint32_t ci = (ch * SPLIT + half) * CC + c;
       float v[3][PP + 2];  // rows y-1..y+1, columns x-1..x+PP of the thread's pixels (x .. x+PP-1)
 #pragma unroll
       for (int dy = 0; dy < 3; dy++) {
@@ -586,6 +592,17 @@ __global__ __launch_bounds__(256) void tconv_k4s2_tile_kernel(TconvArgs args) {
     }
     if (ch + 1 < chunks) put(cur ^ 1);
     __syncthreads();
+  }
+  if constexpr (SPLIT == 2) {  // the second half hands its sums over through the tile memory (nobody reads tiles any more)
+    float *sums = &tiles[0][0][0][0][0];
+    if (half == 1) {
+#pragma unroll
+      for (int i = 0; i < PP * 4 * CO; i++) sums[i * 256 + tid] = (&acc[0][0][0][0])[i];
+    }
+    __syncthreads();
+    if (half == 1) return;
+#pragma unroll
+    for (int i = 0; i < PP * 4 * CO; i++) (&acc[0][0][0][0])[i] += sums[i * 256 + tid];
   }
 
   const uint32_t qy = y0 + ty, qx = x0 + PP * tx;
@@ -689,14 +706,19 @@ int launch_tconv_tile(const char *name, TconvArgs &args) {
   dim3 gt(cdiv(args.W, 32) * cdiv(args.H, 16), args.out_w);
   if ((size_t)gt.x * gt.y < 512) {  // fewer than two blocks per compute unit: one pixel per thread, twice the blocks
     dim3 g1(cdiv(args.W, 16) * cdiv(args.H, 16), args.out_w);
-    if (args.M == 1) tconv_k4s2_tile_kernel<1, 1><<<g1, 256, 0, mt::stream()>>>(args);
-    else if (args.M == 2) tconv_k4s2_tile_kernel<2, 1><<<g1, 256, 0, mt::stream()>>>(args);
-    else if (args.M == 3) tconv_k4s2_tile_kernel<3, 1><<<g1, 256, 0, mt::stream()>>>(args);
-    else tconv_k4s2_tile_kernel<4, 1><<<g1, 256, 0, mt::stream()>>>(args);
-  } else if (args.M == 1) tconv_k4s2_tile_kernel<1, 2><<<gt, 256, 0, mt::stream()>>>(args);
-  else if (args.M == 2) tconv_k4s2_tile_kernel<2, 2><<<gt, 256, 0, mt::stream()>>>(args);
-  else if (args.M == 3) tconv_k4s2_tile_kernel<3, 2><<<gt, 256, 0, mt::stream()>>>(args);
-  else tconv_k4s2_tile_kernel<4, 2><<<gt, 256, 0, mt::stream()>>>(args);
+    if (args.M == 1) tconv_k4s2_tile_kernel<1, 1, 1><<<g1, 256, 0, mt::stream()>>>(args);
+    else if (args.M == 2) tconv_k4s2_tile_kernel<2, 1, 1><<<g1, 256, 0, mt::stream()>>>(args);
+    else if (args.M == 3) tconv_k4s2_tile_kernel<3, 1, 1><<<g1, 256, 0, mt::stream()>>>(args);
+    else tconv_k4s2_tile_kernel<4, 1, 1><<<g1, 256, 0, mt::stream()>>>(args);
+  } else if ((size_t)gt.x * gt.y < 1024 && args.C % 16 == 0) {  // two to four blocks per compute unit: the channels split over two halves of a block
+    if (args.M == 1) tconv_k4s2_tile_kernel<1, 2, 2><<<gt, 512, 0, mt::stream()>>>(args);
+    else if (args.M == 2) tconv_k4s2_tile_kernel<2, 2, 2><<<gt, 512, 0, mt::stream()>>>(args);
+    else if (args.M == 3) tconv_k4s2_tile_kernel<3, 2, 2><<<gt, 512, 0, mt::stream()>>>(args);
+    else tconv_k4s2_tile_kernel<4, 2, 2><<<gt, 512, 0, mt::stream()>>>(args);
+  } else if (args.M == 1) tconv_k4s2_tile_kernel<1, 2, 1><<<gt, 256, 0, mt::stream()>>>(args);
+  else if (args.M == 2) tconv_k4s2_tile_kernel<2, 2, 1><<<gt, 256, 0, mt::stream()>>>(args);
+  else if (args.M == 3) tconv_k4s2_tile_kernel<3, 2, 1><<<gt, 256, 0, mt::stream()>>>(args);
+  else tconv_k4s2_tile_kernel<4, 2, 1><<<gt, 256, 0, mt::stream()>>>(args);
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }

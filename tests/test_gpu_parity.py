@@ -414,6 +414,11 @@ def test_image_layer_kernels_both_tilings(gpu, oracle):
         want = oracle.apply_func(oracle.backward_convolution(delta, kernel, bias, 4, 4, 3, 8, 2, 2, 1, 1, out_shape), "tangence")
         got = gpu.backward_convolution(delta, kernel, bias, 4, 4, 3, 8, 2, 2, 1, 1, out_shape, func="tangence")
         close(got, want, 1e-5)
+    # 600 blocks and a multiple of 16 input channels: the halves of a block take every other chunk of channels
+    kernel, bias = Nrm(4, 1, 1, 32, 2 * 16, std=0.2), U(5, 1, 32, 1, 1) * 0.1
+    delta = U(6, 600, 32, 16, 32)
+    want = oracle.apply_func(oracle.backward_convolution(delta, kernel, bias, 4, 4, 2, 32, 2, 2, 1, 1, (600, 2, 32, 64)), "sigmoid")
+    close(gpu.backward_convolution(delta, kernel, bias, 4, 4, 2, 32, 2, 2, 1, 1, (600, 2, 32, 64), func="sigmoid"), want, 1e-5)
 
 
 def test_fused_conv_activation(gpu, oracle, path):
