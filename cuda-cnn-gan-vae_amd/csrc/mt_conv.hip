@@ -637,10 +637,12 @@ __global__ __launch_bounds__(256 * SPLIT) void tconv_k4s2_tile_kernel(TconvArgs 
 // vector ALUs, same staging: a thread computes two neighbouring output pixels for all KA channels, per input channel
 // 6 LDS reads and 18*KA multiply-adds; the 9 coefficients of (k, c) are contiguous in the kernel tensor and come
 // through the scalar cache.  Needs W % 4 == 0, C % 8 == 0, 16-byte aligned rows.
-template <int KA>
+// CC channels per chunk: 8, or 4 for images of few channels (more chunks to overlap loading with, and half the LDS,
+// so that more blocks share a compute unit).
+template <int KA, int CC>
 __global__ __launch_bounds__(256) void conv3x3_tile_kernel(float *out, const float *image, const float *kernel, const float *bias, ConvGeo g, int func) {
-  using Tile = HaloTile<32, 16, 8>;
-  constexpr int TW = 32, TH = 16, CC = 8, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
+  using Tile = HaloTile<32, 16, CC>;
+  constexpr int TW = 32, TH = 16, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
   __shared__ __attribute__((aligned(16))) float tile[2][CC][ROWS][PITCH];
   const uint32_t H = g.H, W = g.W, C = g.C, HW = H * W;
   const uint32_t tiles_x = (W + TW - 1) / TW;
@@ -826,10 +828,16 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
       image->x % 4 == 0 && kz % 8 == 0 && ((uintptr_t)image->p & 15u) == 0 && ((uintptr_t)out->p & 7u) == 0 && out->w <= 65535u) {
     mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "vector ALU, few output channels") : name);
     dim3 grid(cdiv(image->x, 32) * cdiv(image->y, 16), out->w);
-    if (ka == 1) conv3x3_tile_kernel<1><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);
-    else if (ka == 2) conv3x3_tile_kernel<2><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);
-    else if (ka == 3) conv3x3_tile_kernel<3><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);
-    else conv3x3_tile_kernel<4><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);
+#define MT_CONV3X3_TILE(KA)                                                                                                   \
+  do {                                                                                                                        \
+    if (kz <= 32) conv3x3_tile_kernel<KA, 4><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);  \
+    else conv3x3_tile_kernel<KA, 8><<<grid, 256, 0, mt::stream()>>>(out->p, image->p, kernel->p, bias->p, g, func);           \
+  } while (0)
+    if (ka == 1) MT_CONV3X3_TILE(1);
+    else if (ka == 2) MT_CONV3X3_TILE(2);
+    else if (ka == 3) MT_CONV3X3_TILE(3);
+    else MT_CONV3X3_TILE(4);
+#undef MT_CONV3X3_TILE
     MT_LAUNCH_CHECK(name);
     return MT_OK;
   }
