@@ -385,6 +385,28 @@ def test_transposed_convolution_from_an_input_patch(gpu, oracle, path, case):
     close(gpu.backward_convolution(delta, kernel, biases, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd), func="relu"), oracle.apply_func(want, "relu"))
 
 
+def _random_patch_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    return [(int(rng.integers(1, 4)), int(rng.integers(1, 17)), int(rng.integers(1, 40)), int(rng.integers(1, 75)), int(rng.choice([16, 32])),
+             [None, "relu", "leaky_relu"][int(rng.integers(0, 3))]) for _ in range(n)]
+
+
+@pytest.mark.parametrize("case", _random_patch_cases(16, 2025))
+def test_transposed_convolution_from_an_input_patch_random_sizes(gpu, oracle, case):
+    """Seeded random sizes in the domain of the input-patch kernel (and of the vector-ALU kernels for up to 4 channels):
+    ragged tiles in both directions, any number of output channels up to 16, both as a transposed convolution and as
+    up-sampling + 3x3 convolution."""
+    W, C, H, Wd, KA, func = case
+    delta, kernel, bias = U(4, W, KA, H, Wd), Nrm(5, 1, 1, KA, C * 16, std=0.2), U(6, 1, KA, 1, 1) * 0.2
+    want = oracle.backward_convolution(delta, kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd))
+    got = gpu.backward_convolution(delta, kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd), func=func)
+    close(got, oracle.apply_func(want, func) if func else want)
+    k3, b3 = Nrm(7, 1, 1, C, KA * 9, std=0.2), U(8, 1, C, 1, 1) * 0.2      # KA input channels, C filters
+    want = oracle.forward_convolution(oracle.upsampling(delta, 2, 2), k3, b3, 3, 3, KA, C, 1, 1, 1, 1)
+    got = gpu.upsampling_convolution(delta, k3, b3, 3, KA, C, func=func)
+    close(got, oracle.apply_func(want, func) if func else want, 1e-5)
+
+
 def test_sixteen_row_blocks_forced_on_taller_products(gpu, oracle):
     """The same block forced on 40 output channels: three row blocks, the last one half empty."""
     import mi355tensor as mt
