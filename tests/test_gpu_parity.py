@@ -407,6 +407,16 @@ def test_transposed_convolution_from_an_input_patch_random_sizes(gpu, oracle, ca
     close(got, oracle.apply_func(want, func) if func else want, 1e-5)
 
 
+def test_sixteen_row_blocks_chosen_for_wide_products(gpu, oracle):
+    """Sixteen filters over 98 304 output pixels: the shape for which the 16 x 256 block is chosen without being forced
+    (forward convolution, weight gradient with 16 filters, product of 16 rows)."""
+    image, kernel, bias = U(1, 2, 8, 192, 256), Nrm(2, 1, 1, 16, 8 * 9, std=0.2), U(3, 1, 16, 1, 1)
+    want = oracle.forward_convolution(image, kernel, bias, 3, 3, 8, 16, 1, 1, 1, 1)
+    close(gpu.forward_convolution(image, kernel, bias, 3, 3, 8, 16, 1, 1, 1, 1), want)
+    a, b = Nrm(4, 1, 1, 16, 40, std=0.3), Nrm(5, 1, 1, 40, 70000, std=0.3)
+    close(gpu.mul(a, b), oracle.mul(a, b), 1e-5)
+
+
 def test_sixteen_row_blocks_forced_on_taller_products(gpu, oracle):
     """The same block forced on 40 output channels: three row blocks, the last one half empty."""
     import mi355tensor as mt
