@@ -135,6 +135,35 @@ class Discriminator:
         self.p["lin_w"].upload(lin["weight"])
         self.p["lin_b"].upload(lin["bias"])
 
+    def save_training(self, f):
+        """Iteration and Adam moments in the layout of SaveNetLayersTrainingParam (cuda/netmodel/cmodelmain.cu.h:368-373):
+        per convolution, batch-norm and linear layer first and second moment of the weights, then of the biases (for a
+        batch norm: of gamma, then of beta)."""
+        import wire_format
+        pick = lambda w, b: {"m_weight": self.m[w].numpy(), "v_weight": self.v[w].numpy(), "m_bias": self.m[b].numpy(), "v_bias": self.v[b].numpy()}
+        layers = [("input", {})]
+        for i in range(4):
+            layers += [("convolution", pick("kernel%d" % i, "bias%d" % i)), ("batchnorm", pick("gamma%d" % i, "beta%d" % i)), ("function", {})]
+        layers += [("linear", pick("lin_w", "lin_b")), ("function", {})]
+        wire_format.write_training_params(f, self.iteration, layers)
+
+    def load_training(self, f):
+        import wire_format
+        iteration, layers = wire_format.read_training_params(f, self.LAYER_KINDS)
+        names = [None]
+        for i in range(4):
+            names += [("kernel%d" % i, "bias%d" % i), ("gamma%d" % i, "beta%d" % i), None]
+        names += [("lin_w", "lin_b"), None]
+        for (kind, p), pair in zip(layers, names):
+            if pair is None:
+                continue
+            for key, name in (("m_weight", pair[0]), ("v_weight", pair[0]), ("m_bias", pair[1]), ("v_bias", pair[1])):
+                target = (self.m if key[0] == "m" else self.v)[name]
+                if p[key].shape != target.shape:
+                    raise ValueError("%s of %s: the file holds %s, the network %s" % (key, name, p[key].shape, target.shape))
+                target.upload(p[key])
+        self.iteration = iteration
+
     # ---- forward -------------------------------------------------------------------------------------------
     def forward(self, fused=False):
         h, p = self.x, self.p

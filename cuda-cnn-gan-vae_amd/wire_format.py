@@ -150,3 +150,37 @@ def read_net(f, kinds):
             raise ValueError("unknown layer kind " + repr(kind))
         out.append((kind, p))
     return out
+
+
+# Training state.  CModelMain::SaveNetLayersTrainingParam (cuda/netmodel/cmodelmain.cu.h:368-373) writes the iteration
+# as one uint32, then SaveTrainingParam() of every layer in order: four tensors for the layers that Adam updates --
+# first moment and second moment of the weights, then of the biases (convolution / transposed convolution: MK, VK,
+# MB, VB, netlayer/cnetlayerconvolution.cu.h; linear: MW, VW, MB, VB; batch normalisation: MK, VK for gamma and MB, VB
+# for beta, netlayer/cnetlayerbatchnormalization.cu.h:639-640) -- and nothing for every other kind.
+_TRAINED = ("convolution", "backconvolution", "linear", "batchnorm")
+
+
+def write_training_params(f, iteration, layers):
+    """`layers`: a list of (kind, fields) in network order; for the kinds Adam updates the fields are "m_weight",
+    "v_weight", "m_bias", "v_bias" (for batch normalisation the weight is gamma, the bias beta)."""
+    f.write(struct.pack("=I", int(iteration)))
+    for kind, p in layers:
+        if kind in _TRAINED:
+            for name in ("m_weight", "v_weight", "m_bias", "v_bias"):
+                write_tensor(f, p[name])
+        elif kind not in _EMPTY and kind not in _PAIR and kind not in ("function", "dropout"):
+            raise ValueError("unknown layer kind " + repr(kind))
+
+
+def read_training_params(f, kinds):
+    """Returns (iteration, layers) as write_training_params takes them."""
+    iteration = _take(f, "=I", "the iteration")[0]
+    out = []
+    for kind in kinds:
+        if kind in _TRAINED:
+            out.append((kind, {name: read_tensor(f) for name in ("m_weight", "v_weight", "m_bias", "v_bias")}))
+        elif kind in _EMPTY or kind in _PAIR or kind in ("function", "dropout"):
+            out.append((kind, {}))
+        else:
+            raise ValueError("unknown layer kind " + repr(kind))
+    return iteration, out

@@ -237,6 +237,26 @@ static void ChainA(void)
  CMemoryStream net_saved;   // the whole chain, layer after layer, as CModelMain::SaveNetLayers writes a network
  for(int n=0;n<5;n++) layers[n]->Save(&net_saved);
  DumpRaw("A.net_stream",net_saved);
+ // known Adam moments into the convolution layer (this chain steps by plain gradient descent, its own moments are zero)
+ CMemoryStream moments;
+ const std::vector<double> mk=Values(8*48,0.3),vk=Values(8*48,0.2),mb=Values(8,0.3),vb=Values(8,0.2);
+ moments.PutTensor(1,1,8,3*16,mk);moments.PutTensor(1,1,8,3*16,vk);moments.PutTensor(1,8,1,1,mb);moments.PutTensor(1,8,1,1,vb);
+ conv.LoadTrainingParam(&moments);
+ {
+  CTensor<type_t> t(1,1,8,48),u(1,8,1,1);
+  for(uint32_t n=0;n<8*48;n++) t.SetElement(0,0,n/48,n%48,static_cast<type_t>(mk[n]));
+  Dump("A.mk",t);
+  for(uint32_t n=0;n<8*48;n++) t.SetElement(0,0,n/48,n%48,static_cast<type_t>(vk[n]));
+  Dump("A.vk",t);
+  for(uint32_t n=0;n<8;n++) u.SetElement(0,n,0,0,static_cast<type_t>(mb[n]));
+  Dump("A.mb",u);
+  for(uint32_t n=0;n<8;n++) u.SetElement(0,n,0,0,static_cast<type_t>(vb[n]));
+  Dump("A.vb",u);
+ }
+ CMemoryStream train_saved;   // the training state as CModelMain::SaveNetLayersTrainingParam writes it: iteration, then every layer
+ train_saved.SaveUInt32(7);
+ for(int n=0;n<5;n++) layers[n]->SaveTrainingParam(&train_saved);
+ DumpRaw("A.train_stream",train_saved);
 }
 
 static void ChainB(void)

@@ -153,6 +153,17 @@ def test_config5_network_file_round_trip(gpu):
     for name in net.p:
         assert np.array_equal(net.p[name].numpy(), other.p[name].numpy()), name
     assert np.array_equal(net.forward(True).numpy(), other.forward(True).numpy())
+    # the training state (iteration, Adam moments) travels the same way: after loading both, the next step is the same
+    g = io.BytesIO()
+    net.save_training(g)
+    g.seek(0)
+    other.load_training(g)
+    assert other.iteration == net.iteration == 1
+    net.step(fused=True)
+    other.step(fused=True)
+    for name in net.p:
+        assert np.array_equal(net.p[name].numpy(), other.p[name].numpy()), name
+        assert np.array_equal(net.m[name].numpy(), other.m[name].numpy()), name
     layers = wf.read_net(io.BytesIO(f.getvalue()), D.Discriminator.LAYER_KINDS)
     layers[1][1]["header"]["stride_x"] = 1
     g = io.BytesIO()

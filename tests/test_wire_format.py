@@ -191,3 +191,23 @@ def test_reference_layers_load_a_network_written_here(oracle, tmp_path):
     leaky, prob = expected_chain_g(oracle, layers, got["G.input"])
     assert np.array_equal(got["G.leaky"], leaky)
     assert np.max(np.abs(got["G.sigmoid"] - prob.reshape(got["G.sigmoid"].shape))) <= 1e-6
+
+
+def test_training_state_written_by_the_reference(cpu_dump):
+    """Iteration and Adam moments of chain A as SaveNetLayersTrainingParam writes them: the moments have the shapes of
+    the parameters, the convolution's come back in the order they were loaded in, and the bytes survive a round trip."""
+    raw = cpu_dump["A.train_stream"][1]
+    kinds = ["input", "convolution", "function", "linear", "function"]
+    iteration, layers = wf.read_training_params(io.BytesIO(raw), kinds)
+    assert iteration == 7
+    conv, lin = layers[1][1], layers[3][1]
+    assert conv["m_weight"].shape == conv["v_weight"].shape == as_array(cpu_dump["A.conv_updated.0"]).shape
+    assert conv["m_bias"].shape == as_array(cpu_dump["A.conv_updated.1"]).shape
+    assert lin["m_weight"].shape == as_array(cpu_dump["A.linear_updated.0"]).shape and lin["v_bias"].shape == as_array(cpu_dump["A.linear_updated.1"]).shape
+    # the convolution layer was given known moments through its LoadTrainingParam: their order in the stream
+    for name, key in (("m_weight", "A.mk"), ("v_weight", "A.vk"), ("m_bias", "A.mb"), ("v_bias", "A.vb")):
+        assert np.array_equal(conv[name], as_array(cpu_dump[key])) and np.abs(conv[name]).max() > 0, name
+    assert not np.array_equal(conv["m_weight"], conv["v_weight"])
+    f = io.BytesIO()
+    wf.write_training_params(f, iteration, layers)
+    assert f.getvalue() == raw
