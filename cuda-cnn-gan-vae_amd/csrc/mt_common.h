@@ -21,6 +21,24 @@ int set_igemm_tile(int v); // -1 auto, 0..4 force one block tile of the matrix-c
 int set_patch_blocks(int v);  // persistent blocks of the input-patch transposed convolution (default 512)
 int set_wgrad_groups(int v);  // 0 auto, else batch groups of the batch-summed weight gradient
 
+// A library-owned device buffer that grows on demand.  Recorded HIP graphs keep the pointers of the recording:
+// a request that does not fit while the stream is being captured is an error (run the sequence once eagerly
+// first), and a block that a capture may have seen is kept alive when a later request outgrows it.
+struct Workspace {
+  float *p = nullptr;
+  size_t floats = 0;
+  bool captured = false;  // handed out while the work stream was being captured
+};
+int workspace_get(Workspace &ws, const char *what, size_t floats, float **p);
+size_t retired_workspaces();
+void count_driver_allocation();  // every hipMalloc of the library is counted (mt_get_info "driver_allocations")
+// Re-ordered copies of weights are kept between calls, keyed by the weights' address and shape.  Every library call
+// that writes device memory reports the range here (so does mt_invalidate for writers outside the library); copies
+// made from an overlapping range are then made again on their next use.
+void note_write(const void *p, size_t bytes);
+int set_pack_cache(int on);
+bool pack_cache_info(const char *name, int64_t *value);
+
 // Brackets the launches made inside its lifetime with two events on the work stream when profiling is enabled
 // (mt_profile_enable); `label` must be a string literal.
 struct ProfileScope {
@@ -46,6 +64,7 @@ const char *intern_label(const char *name, const char *suffix);  // "name[suffix
 
 inline bool same_zyx(const mt_tensor *a, const mt_tensor *b) { return a->x == b->x && a->y == b->y && a->z == b->z; }
 inline size_t count(const mt_tensor *t) { return (size_t)t->w * t->z * t->y * t->x; }
+inline void note_write(const mt_tensor *t) { if (t && t->p) note_write(t->p, count(t) * sizeof(float)); }
 inline bool bad(const mt_tensor *t) { return t == nullptr || (t->p == nullptr && count(t) != 0); }
 inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 // The matrix-core kernels address an operand through a 32-bit buffer descriptor, with 0x80000000 as "outside".

@@ -10,6 +10,11 @@
 // Slow path ("direct"): one thread per output element, same loop and summation order as the CPU path, used
 // for shapes the fast path does not cover (kernels that differ per sample, strides above 4) and as a
 // bit-for-bit cross-check of the fast path in the tests.
+#include <string.h>
+
+#include <initializer_list>
+#include <vector>
+
 #include "mt_igemm.h"
 
 namespace {
@@ -35,18 +40,105 @@ int with_row_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, Batch bt, F 
   return f(s);
 }
 
-// ---- library-owned workspace: packed phase kernels and bias sums of the transposed convolution ----------------
-float *g_ws = nullptr;
-size_t g_ws_floats = 0;
-int workspace(size_t floats, float **p) {
-  if (floats > g_ws_floats) {
-    if (g_ws) { MT_HIP(hipStreamSynchronize(mt::stream())); MT_HIP(hipFree(g_ws)); g_ws = nullptr; g_ws_floats = 0; }
-    size_t want = floats + floats / 4 + 1024;
-    MT_HIP(hipMalloc((void **)&g_ws, want * sizeof(float)));
-    g_ws_floats = want;
+// ---- library-owned workspace: the partial sums of the batch-summed gradients, up-sampled images, and re-ordered
+// weights while they cannot be kept (see below)
+mt::Workspace g_ws;
+int workspace(size_t floats, float **p) { return mt::workspace_get(g_ws, "convolution workspace", floats, p); }
+
+// ---- re-ordered weights, kept between calls ---------------------------------------------------------------------
+// A layer passes the same kernel tensor on every forward call (netlayer/cnetlayerbackconvolution.cu.h:303-315); it
+// changes only when the optimiser steps.  The per-phase sub-kernels and bias sums of a transposed convolution, the
+// tap-major order of a 3x3 / 5x5 forward kernel and the coefficient sums of "up-sampling, then 3x3" are therefore
+// made once per (kernel address and sizes, bias address and sizes, geometry, layout) and made again only after a write
+// to the kernel's or the bias' memory: every library call that writes device memory reports its output range
+// (mt::note_write), and writers outside the library call mt_invalidate.  Every entry owns its buffer, so the order of
+// uses on the stream keeps readers of the old contents ahead of the kernel that re-makes them.  While the stream is
+// being captured nothing is kept or looked up (the recorded graph must re-order the weights it will meet at every
+// replay): the re-ordered weights then live in the workspace, as they do with the cache switched off.
+struct PackKey {
+  int kind;  // 0 transposed convolution, 1 tap-major forward kernel, 2 up-sampling + 3x3 coefficient sums
+  const float *kernel, *bias;
+  uint32_t kernel_dims[4], bias_dims[4];
+  int32_t geo[12];
+  bool operator==(const PackKey &o) const {
+    if (kind != o.kind || kernel != o.kernel || bias != o.bias) return false;
+    for (int i = 0; i < 4; i++)
+      if (kernel_dims[i] != o.kernel_dims[i] || bias_dims[i] != o.bias_dims[i]) return false;
+    for (int i = 0; i < 12; i++)
+      if (geo[i] != o.geo[i]) return false;
+    return true;
   }
-  *p = g_ws;
+};
+struct PackEntry {
+  PackKey key;
+  float *buf = nullptr;
+  size_t floats = 0;
+  bool valid = false;
+  uint64_t used = 0;
+};
+constexpr size_t PACK_MAX_ENTRIES = 64, PACK_MAX_BYTES = (size_t)512 << 20;
+std::vector<PackEntry> g_packs;
+bool g_pack_cache = true;
+uint64_t g_pack_clock = 0, g_pack_hits = 0, g_pack_made = 0;
+
+PackKey pack_key(int kind, const mt_tensor *kernel, const mt_tensor *bias, std::initializer_list<int32_t> geo) {
+  PackKey k{};
+  k.kind = kind;
+  k.kernel = kernel->p;
+  k.kernel_dims[0] = kernel->w; k.kernel_dims[1] = kernel->z; k.kernel_dims[2] = kernel->y; k.kernel_dims[3] = kernel->x;
+  if (bias) { k.bias = bias->p; k.bias_dims[0] = bias->w; k.bias_dims[1] = bias->z; k.bias_dims[2] = bias->y; k.bias_dims[3] = bias->x; }
+  int i = 0;
+  for (int32_t g : geo) k.geo[i++] = g;
+  return k;
+}
+
+bool capturing() {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (mt::stream() != nullptr) (void)hipStreamIsCapturing(mt::stream(), &st);
+  return st != hipStreamCaptureStatusNone;
+}
+
+// Where the re-ordered weights of `key` live: *fresh tells the caller to make them (again).
+int pack_buffer(const PackKey &key, size_t floats, float **buf, bool *fresh) {
+  if (!g_pack_cache || floats * sizeof(float) > PACK_MAX_BYTES / 4 || capturing()) {
+    *fresh = true;
+    return workspace(floats, buf);
+  }
+  g_pack_clock++;
+  for (PackEntry &e : g_packs)
+    if (e.key == key && e.floats == floats) {
+      e.used = g_pack_clock;
+      *buf = e.buf;
+      *fresh = !e.valid;
+      e.valid = true;
+      if (*fresh) g_pack_made++; else g_pack_hits++;
+      return MT_OK;
+    }
+  size_t bytes = floats * sizeof(float);
+  for (const PackEntry &e : g_packs) bytes += e.floats * sizeof(float);
+  while (!g_packs.empty() && (g_packs.size() >= PACK_MAX_ENTRIES || bytes > PACK_MAX_BYTES)) {  // least recently used goes
+    size_t lru = 0;
+    for (size_t i = 1; i < g_packs.size(); i++)
+      if (g_packs[i].used < g_packs[lru].used) lru = i;
+    MT_HIP(hipStreamSynchronize(mt::stream()));
+    MT_HIP(hipFree(g_packs[lru].buf));
+    bytes -= g_packs[lru].floats * sizeof(float);
+    g_packs.erase(g_packs.begin() + lru);
+  }
+  PackEntry e;
+  e.key = key; e.floats = floats; e.valid = true; e.used = g_pack_clock;
+  MT_HIP(hipMalloc((void **)&e.buf, floats * sizeof(float)));
+  mt::count_driver_allocation();
+  g_packs.push_back(e);
+  g_pack_made++;
+  *buf = e.buf;
+  *fresh = true;
   return MT_OK;
+}
+
+inline bool overlaps(const float *p, size_t floats, uintptr_t lo, uintptr_t hi) {
+  const uintptr_t a = (uintptr_t)p, b = a + floats * sizeof(float);
+  return p != nullptr && a < hi && lo < b;
 }
 
 struct ConvGeo {
@@ -774,6 +866,7 @@ __global__ __launch_bounds__(256) void conv_pack_tap_major_kernel(float *packed,
 int check_forward(const char *name, const mt_tensor *out, const mt_tensor *image, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz,
                   uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py) {
   if (mt::bad(out) || mt::bad(image) || mt::bad(kernel) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  mt::note_write(out);
   if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel is required", name);
   if (ka != bias->z) return mt::fail(MT_E_BIAS_COUNT, "%s: kernel_amount %u but %u biases", name, ka, bias->z);
   if (kx <= 0 || ky <= 0 || sx <= 0 || sy <= 0 || px < 0 || py < 0) return mt::fail(MT_E_ARGUMENT, "%s: kernel and stride must be positive, padding non-negative", name);
@@ -867,8 +960,9 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
     } else if ((uint32_t)kz % BK == 0 && ka >= 16) {
       // k ordered tap-major, 16 channels of one tap per k step; the weights are re-ordered to match (one small launch)
       float *packed = nullptr;
-      if ((rc = workspace((size_t)ka * K, &packed))) return rc;
-      {
+      bool fresh = true;
+      if ((rc = pack_buffer(pack_key(1, kernel, nullptr, {kx, ky, kz, (int32_t)ka}), (size_t)ka * K, &packed, &fresh))) return rc;
+      if (fresh) {
         mt::ProfileScope prof("conv_pack_tap_major");
         unsigned gx = cdiv((size_t)ka * K, 256 * 4);
         conv_pack_tap_major_kernel<<<gx > 2048 ? 2048 : gx, 256, 0, mt::stream()>>>(packed, kernel->p, kernel->x, ka, (uint32_t)kz, taps);
@@ -895,6 +989,7 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
 int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
              const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
   if (mt::bad(out) || mt::bad(delta) || mt::bad(kernel) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  mt::note_write(out);
   if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel is required", name);
   if (ka != bias->z) return mt::fail(MT_E_BIAS_COUNT, "%s: kernel_amount %u but %u biases", name, ka, bias->z);
   if (kx <= 0 || ky <= 0 || kz <= 0 || sx <= 0 || sy <= 0) return mt::fail(MT_E_ARGUMENT, "%s: kernel and stride must be positive", name);
@@ -932,7 +1027,12 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   // workspace: [bias sums (bias_w, padded to 64)] [packed sub-kernels of all phases: kz*ka*ky*kx floats + alignment]
   size_t sums = (bias->w + 63u) & ~(size_t)63u;
   float *ws = nullptr;
-  if ((rc = workspace(sums + (size_t)kz * ka * ky * kx + (size_t)4 * kz * sy * sx + 64, &ws))) return rc;
+  bool fresh = true;
+  const bool tile = mt::igemm::tile_override() < 0 && tile_kernel_fits(out, delta, kx, ky, kz, ka, sx, sy, px, py);
+  // the phases depend on the output size as well (an odd output has phases of different sizes and may lack one)
+  if ((rc = pack_buffer(pack_key(0, kernel, bias, {kx, ky, kz, (int32_t)ka, sx, sy, px, py, (int32_t)out->x, (int32_t)out->y, tile ? 1 : 0}),
+                        sums + (size_t)kz * ka * ky * kx + (size_t)4 * kz * sy * sx + 64, &ws, &fresh)))
+    return rc;
   float *packed = ws + sums;
 
   TconvArgs args{};
@@ -940,7 +1040,6 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   pa.ker_ld = kernel->x; pa.bias_w = bias->w; pa.CO = kz; pa.CI = ka; pa.KY = ky; pa.KX = kx; pa.SY = sy; pa.SX = sx;
   uint32_t max_n = 0, max_pack = 0, begin = 0;
   const uint32_t OHW = out->y * out->x;
-  const bool tile = mt::igemm::tile_override() < 0 && tile_kernel_fits(out, delta, kx, ky, kz, ka, sx, sy, px, py);
   for (int32_t phy = 0; phy < sy; phy++) {
     Phase1D Y = phase_1d(phy, ky, sy, py, out->y);
     if (Y.q == 0) continue;
@@ -960,7 +1059,7 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     }
   }
   pa.nphase = args.nphase;
-  {
+  if (fresh) {
     mt::ProfileScope prof("tconv_prepare");
     bool k4s2 = kx == 4 && ky == 4 && sx == 2 && sy == 2 && args.nphase == 4 && kernel->x % 4 == 0 && ((uintptr_t)kernel->p & 15u) == 0 && kz <= 65534;
     for (uint32_t f = 0; k4s2 && f < 4; f++) k4s2 = pa.ph[f].ty == 2 && pa.ph[f].tx == 2 && pa.ph[f].ci_stride % 4 == 0 && pa.ph[f].co_stride % 4 == 0;
@@ -1004,6 +1103,8 @@ bool wgrad_image_fixed(uint32_t M, uint32_t N, uint32_t batches, const mt_tensor
 int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
           const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py, bool bias_too) {
   if (mt::bad(dk) || mt::bad(db) || mt::bad(image) || mt::bad(delta)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  mt::note_write(dk);
+  mt::note_write(db);
   if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel gradient is required", name);
   if (db->z != ka) return mt::fail(MT_E_BIAS_COUNT, "%s: kernel_amount %u but %u bias gradients", name, ka, db->z);
   if (kx <= 0 || ky <= 0 || kz <= 0 || sx <= 0 || sy <= 0) return mt::fail(MT_E_ARGUMENT, "%s: kernel and stride must be positive", name);
@@ -1060,6 +1161,8 @@ int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t
 int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,
                     const mt_tensor *delta, int32_t sx, int32_t sy, int32_t px, int32_t py) {
   if (mt::bad(dk) || mt::bad(db) || mt::bad(image) || mt::bad(delta)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  mt::note_write(dk);
+  mt::note_write(db);
   if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel gradient is required", name);
   if (db->z != ka) return mt::fail(MT_E_BIAS_COUNT, "%s: kernel_amount %u but %u bias gradients", name, ka, db->z);
   if (kx <= 0 || ky <= 0 || kz <= 0 || sx <= 0 || sy <= 0) return mt::fail(MT_E_ARGUMENT, "%s: kernel and stride must be positive", name);
@@ -1182,6 +1285,7 @@ __global__ __launch_bounds__(256) void upconv_prepare_kernel(float *packed, cons
 int upsampling_convolution(const char *name, const mt_tensor *out, const mt_tensor *image, uint32_t ux, uint32_t uy, const mt_tensor *kernel, int32_t kx,
                            int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
   if (mt::bad(out) || mt::bad(image) || mt::bad(kernel) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  mt::note_write(out);
   if (ux == 0 || uy == 0) return mt::fail(MT_E_ARGUMENT, "%s: up-sampling factors must be positive", name);
   if ((uint64_t)image->y * uy > 0x7fffffffu || (uint64_t)image->x * ux > 0x7fffffffu) return mt::fail(MT_E_ARGUMENT, "%s: image too large", name);
   const mt_tensor up_shape{image->p, image->w, image->z, image->y * uy, image->x * ux};  // sizes only: the pointer is not used
@@ -1206,8 +1310,9 @@ int upsampling_convolution(const char *name, const mt_tensor *out, const mt_tens
   }
   const uint32_t ld = (uint32_t)kz * 4;
   float *packed = nullptr;
-  if ((rc = workspace((size_t)4 * ka * ld, &packed))) return rc;
-  {
+  bool fresh = true;
+  if ((rc = pack_buffer(pack_key(2, kernel, nullptr, {kz, (int32_t)ka}), (size_t)4 * ka * ld, &packed, &fresh))) return rc;
+  if (fresh) {
     mt::ProfileScope prof("upconv_prepare");
     upconv_prepare_kernel<<<dim3(cdiv((uint32_t)kz, 256), ka), 256, 0, mt::stream()>>>(packed, kernel->p, kernel->x, ka, (uint32_t)kz);
     MT_LAUNCH_CHECK("upconv_prepare");
@@ -1250,6 +1355,34 @@ int &patch_blocks() {
   return v;
 }
 }  // namespace igemm
+void note_write(const void *p, size_t bytes) {
+  if (g_packs.empty() || p == nullptr || bytes == 0) return;
+  const uintptr_t lo = (uintptr_t)p, hi = lo + bytes < lo ? ~(uintptr_t)0 : lo + bytes;
+  for (PackEntry &e : g_packs) {
+    if (!e.valid) continue;
+    const size_t kernel_floats = (size_t)e.key.kernel_dims[0] * e.key.kernel_dims[1] * e.key.kernel_dims[2] * e.key.kernel_dims[3];
+    const size_t bias_floats = (size_t)e.key.bias_dims[0] * e.key.bias_dims[1] * e.key.bias_dims[2] * e.key.bias_dims[3];
+    if (overlaps(e.key.kernel, kernel_floats, lo, hi) || overlaps(e.key.bias, bias_floats, lo, hi)) e.valid = false;
+  }
+}
+int set_pack_cache(int on) {
+  if (on != 0 && on != 1) return fail(MT_E_ARGUMENT, "pack_cache must be 0 (re-order the weights on every call) or 1 (keep them between calls)");
+  g_pack_cache = on != 0;
+  if (!g_pack_cache && !g_packs.empty()) {
+    MT_HIP(hipStreamSynchronize(stream()));
+    for (PackEntry &e : g_packs) MT_HIP(hipFree(e.buf));
+    g_packs.clear();
+  }
+  return MT_OK;
+}
+bool pack_cache_info(const char *name, int64_t *value) {
+  if (strcmp(name, "pack_cache_entries") == 0) { *value = (int64_t)g_packs.size(); return true; }
+  if (strcmp(name, "pack_cache_valid") == 0) { int64_t n = 0; for (const PackEntry &e : g_packs) n += e.valid; *value = n; return true; }
+  if (strcmp(name, "pack_cache_hits") == 0) { *value = (int64_t)g_pack_hits; return true; }
+  if (strcmp(name, "pack_cache_made") == 0) { *value = (int64_t)g_pack_made; return true; }
+  if (strcmp(name, "pack_cache_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_packs) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
+  return false;
+}
 int set_patch_blocks(int v) {
   if (v < 1 || v > 65536) return fail(MT_E_ARGUMENT, "patch_blocks must be 1..65536");
   igemm::patch_blocks() = v;

@@ -71,6 +71,7 @@ inline unsigned plane_blocks(unsigned blocks_x, uint32_t planes) {
 template <class F>
 int launch1(const char *name, const mt_tensor *out, const mt_tensor *in, F f) {
   if (mt::bad(out) || mt::bad(in)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  mt::note_write(out);
   if (!mt::same_zyx(in, out)) return mt::fail(MT_E_SHAPE, "%s: Z/Y/X of input and output differ", name);
   size_t S = (size_t)out->z * out->y * out->x;
   if (S == 0 || out->w == 0) return MT_OK;
@@ -86,6 +87,7 @@ int launch1(const char *name, const mt_tensor *out, const mt_tensor *in, F f) {
 template <class F>
 int launch2(const char *name, const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, F f) {
   if (mt::bad(out) || mt::bad(l) || mt::bad(r)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  mt::note_write(out);
   if (!mt::same_zyx(l, r) || !mt::same_zyx(out, r)) return mt::fail(MT_E_SHAPE, "%s: Z/Y/X of the operands differ", name);
   size_t S = (size_t)out->z * out->y * out->x;
   if (S == 0 || out->w == 0) return MT_OK;
@@ -918,23 +920,16 @@ __global__ __launch_bounds__(EW_THREADS) void bn_ivar_kernel(float *ivar, const 
 
 // a small pool of scratch statistics for the fused batch-norm entry points when the caller passes NULL
 namespace {
-float *g_bn_scratch = nullptr;
-size_t g_bn_scratch_floats = 0;
-int bn_scratch(size_t floats, float **p) {
-  if (floats > g_bn_scratch_floats) {
-    if (g_bn_scratch) { MT_HIP(hipStreamSynchronize(mt::stream())); MT_HIP(hipFree(g_bn_scratch)); g_bn_scratch = nullptr; g_bn_scratch_floats = 0; }
-    MT_HIP(hipMalloc((void **)&g_bn_scratch, floats * sizeof(float)));
-    g_bn_scratch_floats = floats;
-  }
-  *p = g_bn_scratch;
-  return MT_OK;
-}
+mt::Workspace g_bn_ws;
+int bn_scratch(size_t floats, float **p) { return mt::workspace_get(g_bn_ws, "batch-norm scratch", floats, p); }
+
 }  // namespace
 
 namespace {
 template <bool TO_WIDE>
 int concat_split(const char *name, const mt_tensor *wide, const mt_tensor *a, const mt_tensor *b) {
   if (mt::bad(wide) || mt::bad(a) || mt::bad(b)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (TO_WIDE) mt::note_write(wide); else { mt::note_write(a); mt::note_write(b); }
   if (wide->x != a->x || wide->x != b->x || wide->y != a->y || wide->y != b->y || wide->z != a->z + b->z)
     return mt::fail(MT_E_SHAPE, "%s: sizes do not match", name);
   const uint32_t yx = wide->y * wide->x, planes = wide->w * wide->z;
@@ -963,6 +958,7 @@ extern "C" {
 
 int mt_fill(const mt_tensor *out, float value) {
   if (mt::bad(out)) return mt::fail(MT_E_ARGUMENT, "mt_fill: null tensor");
+  mt::note_write(out);
   size_t n = mt::count(out);
   if (n == 0) return MT_OK;
   if (n % 4 == 0 && aligned16(out->p)) {
@@ -1003,6 +999,7 @@ int mt_apply_func(const mt_tensor *out, const mt_tensor *in, int func) {
 
 int mt_add_sum_w(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, float ls, float rs) {
   if (mt::bad(out) || mt::bad(l) || mt::bad(r)) return mt::fail(MT_E_ARGUMENT, "mt_add_sum_w: null tensor");
+  mt::note_write(out);
   if (!mt::same_zyx(l, r) || !mt::same_zyx(out, r)) return mt::fail(MT_E_SHAPE, "mt_add_sum_w: Z/Y/X of the operands differ");
   size_t S = (size_t)out->z * out->y * out->x;
   if (S == 0 || out->w == 0) return MT_OK;
@@ -1020,6 +1017,7 @@ int mt_add_sum_w(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, f
 
 int mt_summ_xy(const mt_tensor *out, const mt_tensor *in) {
   if (mt::bad(out) || mt::bad(in)) return mt::fail(MT_E_ARGUMENT, "mt_summ_xy: null tensor");
+  mt::note_write(out);
   if (in->z != out->z) return mt::fail(MT_E_SHAPE, "mt_summ_xy: depth of input and output differ");
   uint32_t rows = out->w * out->z;
   if (rows == 0) return MT_OK;
@@ -1034,6 +1032,7 @@ int mt_summ_xy(const mt_tensor *out, const mt_tensor *in) {
 
 int mt_add_bias(const mt_tensor *t, const mt_tensor *bias) {
   if (mt::bad(t) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "mt_add_bias: null tensor");
+  mt::note_write(t);
   if (t->z != bias->z) return mt::fail(MT_E_SHAPE, "mt_add_bias: depth of tensor and bias differ");
   uint32_t rows = t->w * t->z, YX = t->y * t->x;
   if (rows == 0 || YX == 0) return MT_OK;
@@ -1052,6 +1051,7 @@ int mt_add_bias(const mt_tensor *t, const mt_tensor *bias) {
 
 int mt_transponse(const mt_tensor *out, const mt_tensor *in) {
   if (mt::bad(out) || mt::bad(in)) return mt::fail(MT_E_ARGUMENT, "mt_transponse: null tensor");
+  mt::note_write(out);
   if (out->y != in->x || out->x != in->y || out->z != in->z || out->w != in->w) return mt::fail(MT_E_SHAPE, "mt_transponse: sizes do not match");
   if (mt::count(in) == 0) return MT_OK;
   uint32_t planes = in->w * in->z;
@@ -1064,6 +1064,7 @@ int mt_transponse(const mt_tensor *out, const mt_tensor *in) {
 
 int mt_upsampling(const mt_tensor *out, const mt_tensor *in, uint32_t ux, uint32_t uy) {
   if (mt::bad(out) || mt::bad(in) || ux == 0 || uy == 0) return mt::fail(MT_E_ARGUMENT, "mt_upsampling: bad argument");
+  mt::note_write(out);
   if (in->x != out->x / ux || in->y != out->y / uy || in->z != out->z) return mt::fail(MT_E_SHAPE, "mt_upsampling: sizes do not match");
   uint32_t planes = out->w * out->z, n = out->y * out->x;
   if (planes == 0 || n == 0) return MT_OK;
@@ -1089,6 +1090,7 @@ int mt_upsampling(const mt_tensor *out, const mt_tensor *in, uint32_t ux, uint32
 
 int mt_downsampling(const mt_tensor *out, const mt_tensor *in, uint32_t dx, uint32_t dy) {
   if (mt::bad(out) || mt::bad(in) || dx == 0 || dy == 0) return mt::fail(MT_E_ARGUMENT, "mt_downsampling: bad argument");
+  mt::note_write(out);
   if (in->x / dx != out->x || in->y / dy != out->y || in->z != out->z || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_downsampling: sizes do not match");
   uint32_t planes = out->w * out->z, n = out->y * out->x;
   if (planes == 0 || n == 0) return MT_OK;
@@ -1107,6 +1109,8 @@ int mt_downsampling(const mt_tensor *out, const mt_tensor *in, uint32_t dx, uint
 
 int mt_max_pooling(const mt_tensor *out, const mt_pos_tensor *pos, const mt_tensor *in, uint32_t px, uint32_t py) {
   if (mt::bad(out) || mt::bad(in) || pos == nullptr || px == 0 || py == 0) return mt::fail(MT_E_ARGUMENT, "mt_max_pooling: bad argument");
+  mt::note_write(out);
+  mt::note_write(pos->p, (size_t)pos->w * pos->z * pos->y * pos->x * sizeof(mt_spos));
   if (in->x / px != out->x || in->y / py != out->y || in->z != out->z || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_max_pooling: sizes do not match");
   uint32_t planes = out->w * out->z, n = out->y * out->x;
   if (planes == 0 || n == 0) return MT_OK;
@@ -1128,6 +1132,7 @@ int mt_max_pooling(const mt_tensor *out, const mt_pos_tensor *pos, const mt_tens
 
 int mt_max_pooling_backward(const mt_tensor *out, const mt_pos_tensor *pos, const mt_tensor *in, uint32_t px, uint32_t py) {
   if (mt::bad(out) || mt::bad(in) || pos == nullptr || px == 0 || py == 0) return mt::fail(MT_E_ARGUMENT, "mt_max_pooling_backward: bad argument");
+  mt::note_write(out);
   if (in->x != out->x / px || in->y != out->y / py || in->z != out->z || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_max_pooling_backward: sizes do not match");
   uint32_t planes = out->w * out->z, n = out->y * out->x;
   if (planes == 0 || n == 0) return MT_OK;
@@ -1158,6 +1163,7 @@ int mt_split_z(const mt_tensor *out_a, const mt_tensor *out_b, const mt_tensor *
 
 int mt_set_time_step(const mt_tensor *out, const mt_tensor *in, const mt_u32_tensor *time_step) {
   if (mt::bad(out) || mt::bad(in) || time_step == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_set_time_step: null tensor");
+  mt::note_write(out);
   if (!mt::same_zyx(in, out) || in->w != out->w || time_step->w != in->w || time_step->z != 1 || time_step->y != 1 || time_step->x != 1)
     return mt::fail(MT_E_SHAPE, "mt_set_time_step: sizes do not match");
   const size_t size = (size_t)in->z * in->y * in->x;
@@ -1172,6 +1178,7 @@ int mt_set_time_step(const mt_tensor *out, const mt_tensor *in, const mt_u32_ten
 
 int mt_create_drop_out_matrix(const mt_tensor *out, float drop_out, uint64_t seed) {
   if (mt::bad(out)) return mt::fail(MT_E_ARGUMENT, "mt_create_drop_out_matrix: null tensor");
+  mt::note_write(out);
   const size_t n = mt::count(out);
   if (n == 0) return MT_OK;
   drop_out_kernel<<<stream_blocks(n), EW_THREADS, 0, mt::stream()>>>(out->p, n, drop_out, (float)(1.0 / (1.0 - (double)drop_out)), seed);
@@ -1181,6 +1188,7 @@ int mt_create_drop_out_matrix(const mt_tensor *out, float drop_out, uint64_t see
 
 int mt_set_normal_noise(const mt_tensor *out, uint64_t seed) {
   if (mt::bad(out)) return mt::fail(MT_E_ARGUMENT, "mt_set_normal_noise: null tensor");
+  mt::note_write(out);
   const size_t n = mt::count(out);
   if (n == 0) return MT_OK;
   normal_noise_kernel<<<stream_blocks(n), EW_THREADS, 0, mt::stream()>>>(out->p, nullptr, nullptr, nullptr, 0, nullptr, 0, 1, n, seed);
@@ -1193,6 +1201,8 @@ int mt_get_noise_image_and_noise(const mt_tensor *noisy, const mt_tensor *noise,
   const mt_tensor *all[5] = {noisy, noise, image, sqrt_alpha_bar, sqrt_one_minus_alpha_bar};
   for (auto t : all)
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_get_noise_image_and_noise: null tensor");
+  mt::note_write(noisy);
+  mt::note_write(noise);
   if (!mt::same_zyx(noisy, noise) || noisy->w != noise->w) return mt::fail(MT_E_SHAPE, "mt_get_noise_image_and_noise: sizes of NoisyImage and Noise differ");
   if (!mt::same_zyx(noisy, image) || noisy->w != image->w) return mt::fail(MT_E_SHAPE, "mt_get_noise_image_and_noise: sizes of NoisyImage and Image differ");
   if (sqrt_alpha_bar->w != image->w || sqrt_one_minus_alpha_bar->w != image->w)
@@ -1210,6 +1220,9 @@ int mt_get_noise_image_and_noise(const mt_tensor *noisy, const mt_tensor *noise,
 int mt_adam(const mt_tensor *weight, const mt_tensor *dweight, const mt_tensor *m, const mt_tensor *v, uint32_t batch_size, double speed,
             double beta1, double beta2, double epsilon, double iteration) {
   if (mt::bad(weight) || mt::bad(dweight) || mt::bad(m) || mt::bad(v)) return mt::fail(MT_E_ARGUMENT, "mt_adam: null tensor");
+  mt::note_write(weight);
+  mt::note_write(m);
+  mt::note_write(v);
   const mt_tensor *o[3] = {dweight, m, v};
   for (auto t : o)
     if (!mt::same_zyx(weight, t) || weight->w != t->w) return mt::fail(MT_E_SHAPE, "mt_adam: sizes do not match");
@@ -1225,6 +1238,7 @@ int mt_fill_many(uint32_t count, const mt_tensor *const *tensors, float value) {
   if (count && tensors == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_fill_many: null list");
   for (uint32_t i = 0; i < count; i++)
     if (mt::bad(tensors[i])) return mt::fail(MT_E_ARGUMENT, "mt_fill_many: null tensor (entry %u)", i);
+  for (uint32_t i = 0; i < count; i++) mt::note_write(tensors[i]);
   for (uint32_t first = 0; first < count;) {
     ManyFill a{};
     uint32_t used = 0;
@@ -1249,6 +1263,9 @@ int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor
   if (count && (weight == nullptr || dweight == nullptr || m == nullptr || v == nullptr)) return mt::fail(MT_E_ARGUMENT, "mt_adam_many: null list");
   for (uint32_t i = 0; i < count; i++) {
     if (mt::bad(weight[i]) || mt::bad(dweight[i]) || mt::bad(m[i]) || mt::bad(v[i])) return mt::fail(MT_E_ARGUMENT, "mt_adam_many: null tensor (entry %u)", i);
+    mt::note_write(weight[i]);
+    mt::note_write(m[i]);
+    mt::note_write(v[i]);
     const mt_tensor *o[3] = {dweight[i], m[i], v[i]};
     for (auto t : o)
       if (!mt::same_zyx(weight[i], t) || weight[i]->w != t->w) return mt::fail(MT_E_SHAPE, "mt_adam_many: sizes do not match (entry %u)", i);
@@ -1274,11 +1291,12 @@ int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor
   return MT_OK;
 }
 
-int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
-                                    const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
-                                    const mt_tensor *new_variable, float momentum, float epsilon, int func) {
+static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
+                            const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
+                            const mt_tensor *new_variable, float momentum, float epsilon, int func) {
   if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: unknown function id %d", func);
   if (mt::bad(out) || mt::bad(in) || mt::bad(gamma) || mt::bad(beta)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: null tensor");
+  for (auto t : {out, xhat, ivar, batch_mean, batch_var, new_mean, new_variable}) mt::note_write(t);
   if (!mt::same_zyx(in, out) || in->w != out->w || !mt::same_zyx(gamma, in) || !mt::same_zyx(beta, in) || gamma->w == 0 || beta->w == 0)
     return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_func: sizes do not match");
   const mt_tensor *stats[5] = {ivar, batch_mean, batch_var, new_mean, new_variable};
@@ -1288,10 +1306,10 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
   size_t S = (size_t)in->z * in->y * in->x;
   uint32_t W = in->w;
   if (S == 0 || W == 0) return MT_OK;
-  float *scratch = nullptr;
-  int rc = bn_scratch(3 * S, &scratch);
+  float *spare = nullptr;
+  int rc = bn_scratch(3 * S, &spare);
   if (rc) return rc;
-  float *pm = batch_mean ? batch_mean->p : scratch, *pv = batch_var ? batch_var->p : scratch + S, *pi = ivar ? ivar->p : scratch + 2 * S;
+  float *pm = batch_mean ? batch_mean->p : spare, *pv = batch_var ? batch_var->p : spare + S, *pi = ivar ? ivar->p : spare + 2 * S;
   float inv_n = (float)(1.0 / (double)(float)W);  // the layer passes 1.0/N with N a float
   float mom_new = (float)(1.0 - (double)momentum);  // and 1.0-Momentum, rounded once
   float *nm = new_mean ? new_mean->p : nullptr, *nv = new_variable ? new_variable->p : nullptr;
@@ -1332,12 +1350,19 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
   return MT_OK;
 }
 
+int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
+                                    const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
+                                    const mt_tensor *new_variable, float momentum, float epsilon, int func) {
+  return bn_forward_train(out, in, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func);
+}
+
 int mt_batchnorm_forward_infer_func(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *mean,
                                     const mt_tensor *variable, float epsilon, int func) {
   if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_infer_func: unknown function id %d", func);
   const mt_tensor *all[6] = {out, in, gamma, beta, mean, variable};
   for (auto t : all)
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_infer_func: null tensor");
+  mt::note_write(out);
   if (!mt::same_zyx(in, out) || in->w != out->w) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_infer_func: sizes do not match");
   for (int i = 2; i < 6; i++)
     if (!mt::same_zyx(all[i], in) || all[i]->w == 0) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_infer_func: parameters must be [1,Z,Y,X]");
@@ -1369,6 +1394,7 @@ int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, 
   const mt_tensor *need[5] = {error, delta, gamma, xhat, ivar};
   for (auto t : need)
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: null tensor");
+  for (auto t : {error, dgamma, dbeta}) mt::note_write(t);
   if (func != MT_F_NONE && (mt::bad(beta) || !mt::same_zyx(beta, delta) || beta->w == 0))
     return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: beta must be [1,Z,Y,X] when a function is given");
   if (!mt::same_zyx(error, delta) || error->w != delta->w || !mt::same_zyx(xhat, delta) || xhat->w != delta->w || !mt::same_zyx(gamma, delta) ||
@@ -1428,6 +1454,8 @@ int mt_vae_coder_output(const mt_tensor *out, const mt_tensor *kl_loss, const mt
   const mt_tensor *need[4] = {out, mu, logvar, epsilon};
   for (auto t : need)
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_vae_coder_output: null tensor");
+  mt::note_write(out);
+  mt::note_write(kl_loss);
   for (auto t : {mu, logvar, epsilon})
     if (!mt::same_zyx(t, out) || t->w != out->w) return mt::fail(MT_E_SHAPE, "mt_vae_coder_output: sizes do not match");
   if (kl_loss && (mt::bad(kl_loss) || mt::count(kl_loss) < 1)) return mt::fail(MT_E_ARGUMENT, "mt_vae_coder_output: kl_loss must hold one value");

@@ -35,8 +35,7 @@ SrcColK col_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, uint32_t inne
 }
 
 // ---- split-K support (see launch_split in mt_igemm.h): workspace for the partial results and the kernel that adds them
-float *g_split_ws = nullptr;
-size_t g_split_floats = 0;
+mt::Workspace g_split_ws;
 
 // out[i] = func(sum_s partial[s][i] + bias[(i / bias_div) % bias_mod])
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *out, const float *partial, uint32_t S, size_t n, const float *bias, uint32_t bias_div,
@@ -78,6 +77,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_small_kernel(float *out, co
 // bias (optional) holds one value per output row m; func is applied last.
 int product(const char *name, const mt_tensor *out, const mt_tensor *left, const mt_tensor *right, bool ta, const float *bias, int func) {
   if (mt::bad(out) || mt::bad(left) || mt::bad(right)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  mt::note_write(out);
   const uint32_t M = ta ? left->x : left->y, K = ta ? left->y : left->x, N = right->x, Z = left->z;
   if (K != right->y || left->z != right->z || out->y != M || out->x != N || out->z != right->z)
     return mt::fail(MT_E_SHAPE, "%s: sizes do not match", name);
@@ -140,15 +140,7 @@ int product(const char *name, const mt_tensor *out, const mt_tensor *left, const
 }  // namespace
 
 namespace mt {
-int split_workspace(size_t floats, float **p) {
-  if (floats > g_split_floats) {
-    if (g_split_ws) { MT_HIP(hipStreamSynchronize(stream())); MT_HIP(hipFree(g_split_ws)); g_split_ws = nullptr; g_split_floats = 0; }
-    MT_HIP(hipMalloc((void **)&g_split_ws, (floats + floats / 4 + 1024) * sizeof(float)));
-    g_split_floats = floats + floats / 4 + 1024;
-  }
-  *p = g_split_ws;
-  return MT_OK;
-}
+int split_workspace(size_t floats, float **p) { return workspace_get(g_split_ws, "split-K workspace", floats, p); }
 int split_reduce(const char *name, float *out, const float *partial, uint32_t S, size_t n, const float *bias, uint32_t bias_div, uint32_t bias_mod, int func) {
   if (n <= 16384 && S >= 32)
     splitk_reduce_small_kernel<<<cdiv(n, 16), 256, 0, stream()>>>(out, partial, S, (uint32_t)n, bias, bias_div, bias_mod, func);

@@ -20,6 +20,7 @@ struct Total {
 };
 
 bool g_on = false;
+int g_open = 0;    // ProfileScope objects alive that hold a slot of g_pending
 std::vector<Pending> g_pending;
 std::vector<hipEvent_t> g_free_events;
 std::vector<Total> g_totals;
@@ -63,6 +64,7 @@ namespace mt {
 
 bool profiling() { return g_on; }
 
+
 const char *intern_label(const char *name, const char *suffix) {
   static std::map<std::string, std::string> labels;
   std::string key = std::string(name) + "[" + suffix + "]";
@@ -71,16 +73,27 @@ const char *intern_label(const char *name, const char *suffix) {
 
 ProfileScope::ProfileScope(const char *label) : slot(-1) {
   if (!g_on) return;
-  if (g_pending.size() >= 16384 && flush() != MT_OK) return;
-  Pending p{label, take_event(), take_event()};
-  if (!p.start || !p.stop) return;
-  if (hipEventRecord(p.start, stream()) != hipSuccess) return;
+  if (g_pending.size() >= 16384) {
+    // the pending list is emptied only while no scope holds a slot of it; otherwise this sample is dropped
+    if (g_open > 0 || flush() != MT_OK) return;
+  }
+  Pending p{label, take_event(), nullptr};
+  if (!p.start) return;
+  p.stop = take_event();
+  if (!p.stop || hipEventRecord(p.start, stream()) != hipSuccess) {
+    g_free_events.push_back(p.start);
+    if (p.stop) g_free_events.push_back(p.stop);
+    return;
+  }
   slot = (int)g_pending.size();
   g_pending.push_back(p);
+  g_open++;
 }
 
 ProfileScope::~ProfileScope() {
-  if (slot >= 0) (void)hipEventRecord(g_pending[slot].stop, stream());
+  if (slot < 0) return;
+  g_open--;
+  (void)hipEventRecord(g_pending[slot].stop, stream());
 }
 
 }  // namespace mt

@@ -4,6 +4,10 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <map>
+#include <unordered_map>
+#include <vector>
+
 #include "mt_common.h"
 
 namespace {
@@ -11,6 +15,9 @@ char g_error[512] = "";
 hipStream_t g_own_stream = nullptr;
 hipStream_t g_stream = nullptr;
 bool g_ready = false;
+int g_device = -1;
+uint64_t g_driver_allocs = 0;
+std::vector<float *> g_retired;  // outgrown workspace blocks that a recorded graph may still use
 }  // namespace
 
 namespace mt {
@@ -30,6 +37,37 @@ int hip_fail(hipError_t e, const char *what) {
   return fail(MT_E_HIP + (int)e, "%s: %s", what, hipGetErrorString(e));
 }
 
+int workspace_get(Workspace &ws, const char *what, size_t floats, float **p) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (g_stream != nullptr) (void)hipStreamIsCapturing(g_stream, &capture);
+  const bool capturing = capture != hipStreamCaptureStatusNone;
+  if (floats > ws.floats) {
+    if (capturing)
+      return fail(MT_E_ARGUMENT, "%s: %zu bytes are needed but %zu exist, and the stream is being captured: run the sequence once before recording it",
+                  what, floats * sizeof(float), ws.floats * sizeof(float));
+    const size_t want = floats + floats / 4 + 1024;
+    float *fresh = nullptr;
+    MT_HIP(hipMalloc((void **)&fresh, want * sizeof(float)));
+    g_driver_allocs++;
+    if (ws.p != nullptr) {
+      if (ws.captured) {
+        g_retired.push_back(ws.p);  // a recorded graph may still name it: kept until the process ends
+      } else {
+        hipError_t e = hipStreamSynchronize(g_stream);  // queued kernels may still use the old block
+        if (e == hipSuccess) e = hipFree(ws.p);
+        if (e != hipSuccess) { (void)hipFree(fresh); return hip_fail(e, "workspace growth"); }
+      }
+    }
+    ws.p = fresh; ws.floats = want; ws.captured = false;
+  }
+  if (capturing) ws.captured = true;
+  *p = ws.p;
+  return MT_OK;
+}
+
+size_t retired_workspaces() { return g_retired.size(); }
+void count_driver_allocation() { g_driver_allocs++; }
+
 }  // namespace mt
 
 extern "C" {
@@ -41,29 +79,93 @@ int mt_init(int device) {
   hipError_t e = hipGetDeviceCount(&n);
   if (e != hipSuccess || n <= 0) return mt::fail(MT_E_UNAVAILABLE, "mt_init: no HIP device (%s)", hipGetErrorString(e));
   if (device < 0 || device >= n) return mt::fail(MT_E_ARGUMENT, "mt_init: device %d out of range (0..%d)", device, n - 1);
+  if (g_ready && device != g_device)
+    return mt::fail(MT_E_ARGUMENT, "mt_init: the library already runs on device %d (its stream, workspaces and memory pool live there)", g_device);
   hipDeviceProp_t prop;
   MT_HIP(hipGetDeviceProperties(&prop, device));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return mt::fail(MT_E_UNAVAILABLE, "mt_init: device %d is %s, this library holds gfx950 code only", device, prop.gcnArchName);
   MT_HIP(hipSetDevice(device));
   if (g_own_stream == nullptr) MT_HIP(hipStreamCreateWithFlags(&g_own_stream, hipStreamNonBlocking));
-  g_stream = g_own_stream;
+  if (!g_ready) g_stream = g_own_stream;
+  g_device = device;
   g_ready = true;
   return MT_OK;
 }
+
+// ---- device memory: a stream-ordered pool ---------------------------------------------------------------------------
+// All work of the library runs on one stream.  A block that the caller frees may still be read by kernels that are
+// queued, but whatever the next owner of the block does is queued behind them on the same stream: the block can be
+// handed out again at once, without waiting.  Freed blocks are kept per size; memory goes back to the driver only when
+// the pool holds more than its limit or an allocation fails (then the stream is drained first).  The unchanged layers
+// of the reference create temporaries on every call (netlayer/cnetlayerconvolution.cu.h:494), which this makes cheap.
+namespace {
+constexpr size_t POOL_GRANULE = 512;                  // block sizes are multiples of this
+constexpr size_t POOL_LARGEST = (size_t)1 << 30;      // larger blocks are not kept
+size_t g_pool_limit = (size_t)4 << 30;                // bytes the pool may hold in free blocks
+size_t g_pool_bytes = 0;
+bool g_pool_on = true;
+uint64_t g_pool_reused = 0;
+std::unordered_map<void *, size_t> g_block_size;      // every live or pooled block of mt_malloc
+std::map<size_t, std::vector<void *>> g_pool;         // free blocks by size
+
+int pool_release_all() {
+  if (g_pool_bytes == 0) return MT_OK;
+  MT_HIP(hipStreamSynchronize(g_stream));
+  for (auto &kv : g_pool)
+    for (void *p : kv.second) {
+      g_block_size.erase(p);
+      MT_HIP(hipFree(p));
+    }
+  g_pool.clear();
+  g_pool_bytes = 0;
+  return MT_OK;
+}
+}  // namespace
 
 int mt_malloc(void **ptr, size_t bytes) {
   if (ptr == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_malloc: null result pointer");
   if (!g_ready) { int rc = mt_init(0); if (rc) return rc; }
   *ptr = nullptr;
   if (bytes == 0) return MT_OK;
-  MT_HIP(hipMalloc(ptr, bytes));
+  const size_t size = (bytes + POOL_GRANULE - 1) / POOL_GRANULE * POOL_GRANULE;
+  auto it = g_pool.find(size);
+  if (it != g_pool.end() && !it->second.empty()) {
+    *ptr = it->second.back();
+    it->second.pop_back();
+    g_pool_bytes -= size;
+    g_pool_reused++;
+    return MT_OK;
+  }
+  hipError_t e = hipMalloc(ptr, size);
+  if (e == hipErrorOutOfMemory && g_pool_bytes) {
+    (void)hipGetLastError();
+    int rc = pool_release_all();
+    if (rc) return rc;
+    e = hipMalloc(ptr, size);
+  }
+  if (e != hipSuccess) { *ptr = nullptr; return mt::hip_fail(e, "hipMalloc"); }
+  g_driver_allocs++;
+  g_block_size[*ptr] = size;
   return MT_OK;
 }
 
 int mt_free(void *ptr) {
   if (ptr == nullptr) return MT_OK;
-  MT_HIP(hipStreamSynchronize(g_stream));  // queued kernels may still use it
+  auto it = g_block_size.find(ptr);
+  const size_t size = it == g_block_size.end() ? 0 : it->second;
+  // whatever was derived from the block's contents (re-ordered weights) must not outlive it: the address may come back
+  mt::note_write(ptr, size ? size : ~(size_t)0 - (size_t)(uintptr_t)ptr);
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (g_stream != nullptr) (void)hipStreamIsCapturing(g_stream, &capture);
+  if (g_pool_on && size && size <= POOL_LARGEST) {
+    if (g_pool_bytes + size > g_pool_limit && capture == hipStreamCaptureStatusNone) { int rc = pool_release_all(); if (rc) return rc; }
+    g_pool[size].push_back(ptr);
+    g_pool_bytes += size;
+    return MT_OK;
+  }
+  if (it != g_block_size.end()) g_block_size.erase(it);
+  if (capture == hipStreamCaptureStatusNone) MT_HIP(hipStreamSynchronize(g_stream));  // queued kernels may still use it
   MT_HIP(hipFree(ptr));
   return MT_OK;
 }
@@ -71,6 +173,7 @@ int mt_free(void *ptr) {
 int mt_copy_h2d(void *dst, const void *src, size_t bytes) {
   if (bytes == 0) return MT_OK;
   if (dst == nullptr || src == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_copy_h2d: null pointer");
+  mt::note_write(dst, bytes);
   MT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
   MT_HIP(hipStreamSynchronize(g_stream));  // the host buffer may be reused on return
   return MT_OK;
@@ -87,7 +190,14 @@ int mt_copy_d2h(void *dst, const void *src, size_t bytes) {
 int mt_copy_d2d(void *dst, const void *src, size_t bytes) {
   if (bytes == 0) return MT_OK;
   if (dst == nullptr || src == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_copy_d2d: null pointer");
+  mt::note_write(dst, bytes);
   MT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
+  return MT_OK;
+}
+
+int mt_invalidate(const void *ptr, size_t bytes) {
+  if (ptr == nullptr || bytes == 0) return MT_OK;
+  mt::note_write(ptr, bytes);
   return MT_OK;
 }
 
@@ -104,6 +214,17 @@ int mt_set_option(const char *name, int value) {
   if (name && strcmp(name, "igemm_tile") == 0) return mt::set_igemm_tile(value);
   if (name && strcmp(name, "wgrad_groups") == 0) return mt::set_wgrad_groups(value);
   if (name && strcmp(name, "patch_blocks") == 0) return mt::set_patch_blocks(value);
+  if (name && strcmp(name, "pack_cache") == 0) return mt::set_pack_cache(value);
+  if (name && strcmp(name, "pool") == 0) {
+    if (value != 0 && value != 1) return mt::fail(MT_E_ARGUMENT, "pool must be 0 (every mt_free goes to the driver) or 1");
+    g_pool_on = value != 0;
+    return g_pool_on ? MT_OK : pool_release_all();
+  }
+  if (name && strcmp(name, "pool_limit_mib") == 0) {
+    if (value < 0) return mt::fail(MT_E_ARGUMENT, "pool_limit_mib must not be negative");
+    g_pool_limit = (size_t)value << 20;
+    return g_pool_bytes > g_pool_limit ? pool_release_all() : MT_OK;
+  }
   return mt::fail(MT_E_ARGUMENT, "mt_set_option: unknown option '%s'", name ? name : "(null)");
 }
 
@@ -147,8 +268,23 @@ int mt_timer_destroy(void *timer) {
 
 int mt_set_stream(void *hip_stream) {
   if (!g_ready) { int rc = mt_init(0); if (rc) return rc; }
-  g_stream = hip_stream ? (hipStream_t)hip_stream : g_own_stream;
+  hipStream_t next = hip_stream ? (hipStream_t)hip_stream : g_own_stream;
+  if (next == g_stream) return MT_OK;
+  // pooled blocks, workspaces and re-ordered weights are reused in the order of ONE stream: the old stream's work
+  // must be complete before anything is queued on the new one
+  MT_HIP(hipStreamSynchronize(g_stream));
+  g_stream = next;
   return MT_OK;
+}
+
+int mt_get_info(const char *name, int64_t *value) {
+  if (name == nullptr || value == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_get_info: null argument");
+  if (strcmp(name, "pool_bytes") == 0) { *value = (int64_t)g_pool_bytes; return MT_OK; }
+  if (strcmp(name, "pool_reused") == 0) { *value = (int64_t)g_pool_reused; return MT_OK; }
+  if (strcmp(name, "driver_allocations") == 0) { *value = (int64_t)g_driver_allocs; return MT_OK; }
+  if (strcmp(name, "retired_workspaces") == 0) { *value = (int64_t)mt::retired_workspaces(); return MT_OK; }
+  if (mt::pack_cache_info(name, value)) return MT_OK;
+  return mt::fail(MT_E_ARGUMENT, "mt_get_info: unknown name '%s'", name);
 }
 
 }  // extern "C"

@@ -48,6 +48,8 @@ def lib():
             getattr(_lib, f).argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         _lib.mt_set_stream.argtypes = [C.c_void_p]
         _lib.mt_set_option.argtypes = [C.c_char_p, C.c_int]
+        _lib.mt_get_info.argtypes = [C.c_char_p, C.POINTER(C.c_int64)]
+        _lib.mt_invalidate.argtypes = [C.c_void_p, C.c_size_t]
     return _lib
 
 
@@ -67,6 +69,18 @@ def synchronize():
 
 def set_option(name, value):
     call("mt_set_option", name.encode(), C.c_int(value))
+
+
+def get_info(name):
+    """A counter of the runtime (memory pool, kept re-ordered weights, retired workspaces); see mt_get_info."""
+    v = C.c_int64()
+    call("mt_get_info", name.encode(), C.byref(v))
+    return v.value
+
+
+def invalidate(ptr, nbytes):
+    """Announce a write to device memory that did not go through this library (see mt_invalidate)."""
+    call("mt_invalidate", C.c_void_p(ptr), C.c_size_t(nbytes))
 
 
 def profile_enable(on=True):
@@ -223,7 +237,9 @@ class CTensor:
     def reinterpret(self, w, z, y, x):
         """ReinterpretSize: the same memory under other sizes (cuda/ctensor.cu.h:587-601)."""
         assert w * z * y * x == self.count, "the element count must not change"
-        return CTensor.wrap(self.ptr.value, (w, z, y, x))
+        t = CTensor.wrap(self.ptr.value, (w, z, y, x))
+        t._base = self   # the view must not outlive the memory it looks at
+        return t
 
     def desc(self):
         return MtTensor(self.ptr.value, *self.shape)
@@ -232,6 +248,8 @@ class CTensor:
         """Pointer to this tensor's descriptor for a C-ABI call (built once: pointer and sizes never change)."""
         r = self.__dict__.get("_ref")
         if r is None:
+            if not self.ptr and self.count:
+                raise RuntimeError("the tensor's device memory has been freed")
             self._desc = self.desc()
             r = self._ref = C.byref(self._desc)
         return r
@@ -240,6 +258,8 @@ class CTensor:
         if self.owned and self.ptr:
             call("mt_free", self.ptr)
             self.ptr = C.c_void_p()
+            self.__dict__.pop("_ref", None)
+            self.__dict__.pop("_desc", None)
 
     def __del__(self):
         try:

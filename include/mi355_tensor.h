@@ -78,6 +78,12 @@ int mt_free(void *ptr);                  /* ccudadevicevector.cu.h clear    */
 int mt_copy_h2d(void *dst, const void *src, size_t bytes); /* copy_host_to_device */
 int mt_copy_d2h(void *dst, const void *src, size_t bytes); /* copy_device_to_host; waits for queued work */
 int mt_copy_d2d(void *dst, const void *src, size_t bytes); /* operator= (device copy, :159-170) */
+/* Tells the library that someone else (another library's kernel, a hipMemcpy of the caller's) wrote [ptr, ptr+bytes).
+ * The library keeps re-ordered copies of convolution weights between calls (the layers pass the same kernel tensor on
+ * every forward call, netlayer/cnetlayerbackconvolution.cu.h:303-315) and makes them again after any write to the
+ * weights that goes through this ABI -- mt_copy_h2d, mt_copy_d2d, mt_free, every function with an output tensor --
+ * or is announced here.  No counterpart in the reference: its CTensor writes device memory through its own calls only. */
+int mt_invalidate(const void *ptr, size_t bytes);
 int mt_synchronize(void);
 void *mt_get_stream(void);               /* the hipStream_t all work is queued on */
 int mt_set_stream(void *hip_stream);     /* queue on a caller-owned stream (NULL: back to the library's own) */
@@ -95,6 +101,13 @@ int mt_timer_destroy(void *timer);
  * n split the batch of mt_convolution_backward_weights_sum into n groups (when n divides the batch).  For tests and
  * measurements; results agree within fp32 rounding. */
 int mt_set_option(const char *name, int value);
+/* More options: "pack_cache" 1 (default) keep re-ordered weights between calls / 0 re-order on every call;
+ * "pool" 1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no wait) /
+ * 0 every mt_free waits for the stream and returns the block to the driver; "pool_limit_mib" bytes the pool may hold.
+ * mt_get_info reads counters of the runtime, for tests and measurements (no counterpart in the reference):
+ * "pool_bytes", "pool_reused", "driver_allocations", "retired_workspaces", "pack_cache_entries", "pack_cache_valid",
+ * "pack_cache_hits", "pack_cache_made", "pack_cache_bytes". */
+int mt_get_info(const char *name, int64_t *value);
 
 /* ---- convolutions: CTensorConv<T> (cuda/ctensorconv.cu.h:63-66) ---- */
 /* ForwardConvolution, cuda/ctensorconv.cu.h:276-315 (+ the AddBias launch it ends with); CPU: cpu/ctensorconv.h:84-148 */
