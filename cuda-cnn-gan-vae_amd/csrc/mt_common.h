@@ -38,6 +38,7 @@ void count_driver_allocation();  // every hipMalloc of the library is counted (m
 void note_write(const void *p, size_t bytes);
 int set_pack_cache(int on);
 bool pack_cache_info(const char *name, int64_t *value);
+int static_scratch_setup();  // looks up the device address of the fixed scratch array for the current device
 
 // Brackets the launches made inside its lifetime with two events on the work stream when profiling is enabled
 // (mt_profile_enable); `label` must be a string literal.
@@ -47,6 +48,11 @@ struct ProfileScope {
   int slot;
 };
 bool profiling();
+struct ProfileMute {  // while alive (and `on`): scopes record nothing, so no event is created
+  explicit ProfileMute(bool on);
+  ~ProfileMute();
+  bool on;
+};
 const char *intern_label(const char *name, const char *suffix);  // "name[suffix]" with process lifetime
 
 #define MT_HIP(call)                                         \

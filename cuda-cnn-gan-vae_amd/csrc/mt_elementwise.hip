@@ -923,7 +923,34 @@ namespace {
 mt::Workspace g_bn_ws;
 int bn_scratch(size_t floats, float **p) { return mt::workspace_get(g_bn_ws, "batch-norm scratch", floats, p); }
 
+// The same scratch for callers that cannot allocate: a fixed array in the code object's own device memory, one copy
+// per device that loads the library, held until the process ends.  Host code never uses the array's name as an
+// address: the device address is looked up once per device (with that device current) and kept.
+constexpr size_t STATIC_SCRATCH_FLOATS = 3u * 262144u;  // mean, variance, 1/sqrt(variance + eps) of up to 262144 elements: 3 MiB
+constexpr int MAX_DEVICES = 64;
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+float *g_static_scratch[MAX_DEVICES] = {};
+int static_scratch(float **p) {
+  int dev = -1;
+  MT_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= MAX_DEVICES) return mt::fail(MT_E_UNAVAILABLE, "static scratch: device %d is beyond the %d devices the library keeps an address for", dev, MAX_DEVICES);
+  if (g_static_scratch[dev] == nullptr) {
+    void *q = nullptr;
+    MT_HIP(hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)));
+    if (q == nullptr) return mt::fail(MT_E_UNAVAILABLE, "static scratch: no device address for the array on device %d", dev);
+    g_static_scratch[dev] = static_cast<float *>(q);
+  }
+  *p = g_static_scratch[dev];
+  return MT_OK;
+}
 }  // namespace
+
+namespace mt {
+int static_scratch_setup() {
+  float *p = nullptr;
+  return static_scratch(&p);
+}
+}  // namespace mt
 
 namespace {
 template <bool TO_WIDE>
@@ -1291,9 +1318,11 @@ int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor
   return MT_OK;
 }
 
+// fixed_scratch: the entry point that allocates nothing -- statistics the caller does not ask for go to the library's
+// fixed array (at most STATIC_SCRATCH_FLOATS / 3 elements per sample) and no launch is bracketed by profiling events.
 static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
                             const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
-                            const mt_tensor *new_variable, float momentum, float epsilon, int func) {
+                            const mt_tensor *new_variable, float momentum, float epsilon, int func, bool fixed_scratch) {
   if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: unknown function id %d", func);
   if (mt::bad(out) || mt::bad(in) || mt::bad(gamma) || mt::bad(beta)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: null tensor");
   for (auto t : {out, xhat, ivar, batch_mean, batch_var, new_mean, new_variable}) mt::note_write(t);
@@ -1307,8 +1336,17 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
   uint32_t W = in->w;
   if (S == 0 || W == 0) return MT_OK;
   float *spare = nullptr;
-  int rc = bn_scratch(3 * S, &spare);
+  int rc = MT_OK;
+  if (fixed_scratch) {
+    if (3 * S > STATIC_SCRATCH_FLOATS)
+      return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func_noalloc: %zu elements per sample, the fixed scratch array holds statistics for at most %zu",
+                      S, STATIC_SCRATCH_FLOATS / 3);
+    rc = static_scratch(&spare);
+  } else {
+    rc = bn_scratch(3 * S, &spare);
+  }
   if (rc) return rc;
+  mt::ProfileMute mute(fixed_scratch);
   float *pm = batch_mean ? batch_mean->p : spare, *pv = batch_var ? batch_var->p : spare + S, *pi = ivar ? ivar->p : spare + 2 * S;
   float inv_n = (float)(1.0 / (double)(float)W);  // the layer passes 1.0/N with N a float
   float mom_new = (float)(1.0 - (double)momentum);  // and 1.0-Momentum, rounded once
@@ -1353,7 +1391,13 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
 int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
                                     const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
                                     const mt_tensor *new_variable, float momentum, float epsilon, int func) {
-  return bn_forward_train(out, in, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func);
+  return bn_forward_train(out, in, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func, false);
+}
+
+int mt_batchnorm_forward_train_func_noalloc(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
+                                            const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
+                                            const mt_tensor *new_variable, float momentum, float epsilon, int func) {
+  return bn_forward_train(out, in, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func, true);
 }
 
 int mt_batchnorm_forward_infer_func(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *mean,

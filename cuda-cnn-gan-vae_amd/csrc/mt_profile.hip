@@ -20,6 +20,7 @@ struct Total {
 };
 
 bool g_on = false;
+int g_muted = 0;   // ProfileMute objects alive
 int g_open = 0;    // ProfileScope objects alive that hold a slot of g_pending
 std::vector<Pending> g_pending;
 std::vector<hipEvent_t> g_free_events;
@@ -62,8 +63,10 @@ int flush() {
 
 namespace mt {
 
-bool profiling() { return g_on; }
+bool profiling() { return g_on && g_muted == 0; }
 
+ProfileMute::ProfileMute(bool on_) : on(on_) { if (on) g_muted++; }
+ProfileMute::~ProfileMute() { if (on) g_muted--; }
 
 const char *intern_label(const char *name, const char *suffix) {
   static std::map<std::string, std::string> labels;
@@ -72,7 +75,7 @@ const char *intern_label(const char *name, const char *suffix) {
 }
 
 ProfileScope::ProfileScope(const char *label) : slot(-1) {
-  if (!g_on) return;
+  if (!g_on || g_muted) return;
   if (g_pending.size() >= 16384) {
     // the pending list is emptied only while no scope holds a slot of it; otherwise this sample is dropped
     if (g_open > 0 || flush() != MT_OK) return;

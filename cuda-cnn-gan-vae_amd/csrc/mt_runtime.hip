@@ -88,6 +88,8 @@ int mt_init(int device) {
   MT_HIP(hipSetDevice(device));
   if (g_own_stream == nullptr) MT_HIP(hipStreamCreateWithFlags(&g_own_stream, hipStreamNonBlocking));
   if (!g_ready) g_stream = g_own_stream;
+  int rc = mt::static_scratch_setup();  // the entry point that allocates nothing finds its array's address here
+  if (rc) return rc;
   g_device = device;
   g_ready = true;
   return MT_OK;

@@ -475,6 +475,14 @@ class Fused:
              opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
 
     @staticmethod
+    def BatchNormForwardTrainNoAlloc(out, inp, gamma, beta, xhat=None, ivar=None, batch_mean=None, batch_var=None, new_mean=None, new_variable=None,
+                                     momentum=0.9, epsilon=1e-6, func=None):
+        """The same call through the entry point that allocates nothing (statistics in the library's fixed array)."""
+        opt = lambda t: _d(t) if t is not None else None
+        call("mt_batchnorm_forward_train_func_noalloc", _d(out), _d(inp), _d(gamma), _d(beta), opt(xhat), opt(ivar), opt(batch_mean), opt(batch_var),
+             opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
+
+    @staticmethod
     def VaeCoderOutput(out, kl_loss, mu, logvar, epsilon):
         call("mt_vae_coder_output", _d(out), _d(kl_loss) if kl_loss is not None else None, _d(mu), _d(logvar), _d(epsilon))
 

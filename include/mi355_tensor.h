@@ -196,6 +196,15 @@ int mt_linear_forward_func(const mt_tensor *output, const mt_tensor *weight, con
 int mt_batchnorm_forward_train_func(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
                                     const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var,
                                     const mt_tensor *new_mean, const mt_tensor *new_variable, float momentum, float epsilon, int func);
+/* The same call for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Statistics the caller does not ask for go to a
+ * fixed array inside the library's code object (3 MiB per GPU, held until the process ends) instead of a workspace
+ * that grows: Z*Y*X of the input must not exceed 262144 (MT_E_ARGUMENT otherwise); nothing is allocated or freed, no
+ * profiling event is created.  Same kernels and results as mt_batchnorm_forward_train_func.  All calls on one GPU
+ * share the array: calls that overlap in time on one GPU (two streams, two threads) race. */
+int mt_batchnorm_forward_train_func_noalloc(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
+                                            const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var,
+                                            const mt_tensor *new_mean, const mt_tensor *new_variable, float momentum, float epsilon, int func);
 /* The same layer in inference mode (lines 326-371): stored mean / variable instead of batch statistics. */
 int mt_batchnorm_forward_infer_func(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
                                     const mt_tensor *mean, const mt_tensor *variable, float epsilon, int func);
