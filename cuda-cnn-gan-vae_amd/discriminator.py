@@ -39,6 +39,55 @@ def make_parameters(seed=5, std=0.02):
     return p
 
 
+def make_statistics():
+    """Running mean and variable of the four batch-norm layers as a fresh layer holds them
+    (Reset, netlayer/cnetlayerbatchnormalization.cu.h:239-240): 0 and 1."""
+    s, size = {}, IMAGE
+    for i in range(4):
+        size //= 2
+        s["mean%d" % i] = np.zeros((1, CHANNELS[i + 1], size, size), np.float32)
+        s["variable%d" % i] = np.ones((1, CHANNELS[i + 1], size, size), np.float32)
+    return s
+
+
+LAYER_KINDS = ["input"] + ["convolution", "batchnorm", "function"] * 4 + ["linear", "function"]
+
+
+def net_layers(host):
+    """Parameters and running statistics (numpy, keys of make_parameters + make_statistics) as the layer list that
+    wire_format.write_net takes, in the order SaveNetLayers writes this stack (cuda/netmodel/cmodelmain.cu.h:296-300)."""
+    layers = [("input", {})]
+    for i in range(4):
+        header = dict(kernel_amount=CHANNELS[i + 1], kernel_x=4, kernel_y=4, kernel_z=CHANNELS[i], stride_x=2, stride_y=2, padding_x=1, padding_y=1)
+        layers.append(("convolution", {"header": header, "kernel": host["kernel%d" % i], "bias": host["bias%d" % i]}))
+        layers.append(("batchnorm", {"beta": host["beta%d" % i], "gamma": host["gamma%d" % i], "mean": host["mean%d" % i],
+                                     "variable": host["variable%d" % i], "momentum": MOMENTUM}))
+        layers.append(("function", {"name": "leaky_relu"}))
+    layers.append(("linear", {"weight": host["lin_w"], "bias": host["lin_b"]}))
+    layers.append(("function", {"name": "sigmoid"}))
+    return layers
+
+
+def host_from_layers(layers):
+    """The inverse, for a list read with wire_format.read_net(f, LAYER_KINDS); layer settings in the file must be this
+    stack's (the reference loads with check_size)."""
+    import wire_format
+    host = {}
+    for i in range(4):
+        conv, bn, func = (layers[1 + 3 * i + j][1] for j in range(3))
+        h = conv["header"]
+        want = (CHANNELS[i + 1], 4, 4, CHANNELS[i], 2, 2, 1, 1)
+        if tuple(h[k] for k in wire_format.CONV_HEADER) != want or func["name"] != "leaky_relu":
+            raise ValueError("layer %d of the file is not this network's: %r, %s" % (i, h, func["name"]))
+        for name, a in (("kernel", conv["kernel"]), ("bias", conv["bias"]), ("gamma", bn["gamma"]), ("beta", bn["beta"]), ("mean", bn["mean"]),
+                        ("variable", bn["variable"])):
+            host["%s%d" % (name, i)] = a
+    if layers[14][1]["name"] != "sigmoid":
+        raise ValueError("the last layers of the file are not this network's")
+    host["lin_w"], host["lin_b"] = layers[13][1]["weight"], layers[13][1]["bias"]
+    return host
+
+
 def make_batch(batch, seed=5):
     rng = np.random.default_rng(seed + 1000)
     x = rng.uniform(-1, 1, size=(batch, 3, IMAGE, IMAGE)).astype(np.float32)
@@ -61,7 +110,12 @@ class Discriminator:
         mt.init(0)
         self.batch = b = batch
         host = params or make_parameters()
-        self.p = {k: CTensor.from_numpy(v) for k, v in host.items()}
+        self.p = {k: CTensor.from_numpy(v) for k, v in host.items() if not k.startswith(("mean", "variable"))}
+        # Running statistics of the batch-norm layers.  The layer keeps Mean / Variable (saved, used in inference mode)
+        # and NewMean / NewVariable (blended by every training-mode forward pass), and copies one pair to the other at
+        # both ends of a training step (netlayer/cnetlayerbatchnormalization.cu.h:620-621, 650-651).  Here one tensor
+        # serves as both: the training-mode forward pass blends into it, the two copies are no-ops.
+        self.stats = {k: CTensor.from_numpy(host[k] if k in host else v) for k, v in make_statistics().items()}
         self.x, self.labels = CTensor(b, 3, IMAGE, IMAGE), CTensor(b, 1, 1, 1)
         self.c, self.bn, self.a, self.xhat, self.ivar = [], [], [], [], []
         self.d_a, self.d_bn, self.d_c = [], [], []
@@ -86,8 +140,8 @@ class Discriminator:
         self.tmp_dw = CTensor(b, 1, 1, CHANNELS[4] * 16)
         self.g["lin_w"], self.g["lin_b"] = CTensor(1, 1, 1, CHANNELS[4] * 16), CTensor(1, 1, 1, 1)
         self.zero_bias = [CTensor.from_numpy(np.zeros((1, CHANNELS[i + 1], 1, 1), np.float32)) for i in range(4)]
-        self.m = {k: CTensor.from_numpy(np.zeros(v.shape, np.float32)) for k, v in host.items()}
-        self.v = {k: CTensor.from_numpy(np.zeros(v.shape, np.float32)) for k, v in host.items()}
+        self.m = {k: CTensor.from_numpy(np.zeros(t.shape, np.float32)) for k, t in self.p.items()}
+        self.v = {k: CTensor.from_numpy(np.zeros(t.shape, np.float32)) for k, t in self.p.items()}
         self.iteration = 0
 
     def set_batch(self, x, labels):
@@ -95,45 +149,32 @@ class Discriminator:
         self.labels.upload(labels)
 
     # ---- network file ----------------------------------------------------------------------------------------
-    LAYER_KINDS = ["input"] + ["convolution", "batchnorm", "function"] * 4 + ["linear", "function"]
+    LAYER_KINDS = LAYER_KINDS
+
+    def host_state(self):
+        """Parameters and running statistics as numpy arrays."""
+        host = {k: t.numpy() for k, t in self.p.items()}
+        host.update({k: t.numpy() for k, t in self.stats.items()})
+        return host
 
     def save_net(self, f):
-        """The parameters as the reference's SaveNetLayers would write this stack (cuda/netmodel/cmodelmain.cu.h:296-300):
-        a C++ network of the same layers on the drop-in classes loads the file.  This class keeps no running
-        statistics: mean 0 and variable 1 are written, the values a fresh layer holds (cnetlayerbatchnormalization.cu.h:239)."""
+        """The parameters and the running statistics as the reference's SaveNetLayers would write this stack
+        (cuda/netmodel/cmodelmain.cu.h:296-300; batch norm: beta, gamma, mean, variable, momentum,
+        netlayer/cnetlayerbatchnormalization.cu.h:409-417): a C++ network of the same layers on the drop-in classes
+        loads the file and runs inference with the statistics trained here."""
         import wire_format
-        layers = [("input", {})]
-        for i in range(4):
-            host = {k: self.p["%s%d" % (k, i)].numpy() for k in ("kernel", "bias", "gamma", "beta")}
-            header = dict(kernel_amount=CHANNELS[i + 1], kernel_x=4, kernel_y=4, kernel_z=CHANNELS[i], stride_x=2, stride_y=2, padding_x=1, padding_y=1)
-            layers.append(("convolution", {"header": header, "kernel": host["kernel"], "bias": host["bias"]}))
-            layers.append(("batchnorm", {"beta": host["beta"], "gamma": host["gamma"], "mean": np.zeros_like(host["beta"]),
-                                         "variable": np.ones_like(host["beta"]), "momentum": MOMENTUM}))
-            layers.append(("function", {"name": "leaky_relu"}))
-        layers.append(("linear", {"weight": self.p["lin_w"].numpy(), "bias": self.p["lin_b"].numpy()}))
-        layers.append(("function", {"name": "sigmoid"}))
-        wire_format.write_net(f, layers)
+        wire_format.write_net(f, net_layers(self.host_state()))
 
     def load_net(self, f):
         """The inverse; sizes and layer settings in the file must be this stack's (the reference loads with check_size)."""
         import wire_format
-        layers = wire_format.read_net(f, self.LAYER_KINDS)
-        for i in range(4):
-            conv, bn, func = (layers[1 + 3 * i + j][1] for j in range(3))
-            h = conv["header"]
-            want = (CHANNELS[i + 1], 4, 4, CHANNELS[i], 2, 2, 1, 1)
-            if tuple(h[k] for k in wire_format.CONV_HEADER) != want or func["name"] != "leaky_relu":
-                raise ValueError("layer %d of the file is not this network's: %r, %s" % (i, h, func["name"]))
-            for name, a in (("kernel", conv["kernel"]), ("bias", conv["bias"]), ("gamma", bn["gamma"]), ("beta", bn["beta"])):
-                t = self.p["%s%d" % (name, i)]
-                if a.shape != t.shape:
-                    raise ValueError("%s%d: the file holds %s, the network %s" % (name, i, a.shape, t.shape))
-                t.upload(a)
-        lin = layers[13][1]
-        if lin["weight"].shape != self.p["lin_w"].shape or lin["bias"].shape != self.p["lin_b"].shape or layers[14][1]["name"] != "sigmoid":
-            raise ValueError("the last layers of the file are not this network's")
-        self.p["lin_w"].upload(lin["weight"])
-        self.p["lin_b"].upload(lin["bias"])
+        host = host_from_layers(wire_format.read_net(f, self.LAYER_KINDS))
+        for name, a in host.items():
+            t = self.stats[name] if name in self.stats else self.p[name]
+            if a.shape != t.shape:
+                raise ValueError("%s: the file holds %s, the network %s" % (name, a.shape, t.shape))
+        for name, a in host.items():
+            (self.stats[name] if name in self.stats else self.p[name]).upload(a)
 
     def save_training(self, f):
         """Iteration and Adam moments in the layout of SaveNetLayersTrainingParam (cuda/netmodel/cmodelmain.cu.h:368-373):
@@ -172,6 +213,7 @@ class Discriminator:
             CTensorConv.ForwardConvolution(self.c[i], h, p["kernel%d" % i], 4, 4, cin, cout, p["bias%d" % i], 2, 2, 1, 1)
             if fused:  # batch norm and the function layer behind it in one pass
                 Fused.BatchNormForwardTrain(self.a[i], self.c[i], p["gamma%d" % i], p["beta%d" % i], self.xhat[i], self.ivar[i],
+                                            new_mean=self.stats["mean%d" % i], new_variable=self.stats["variable%d" % i],
                                             momentum=MOMENTUM, epsilon=BN_EPSILON, func="leaky_relu")
             else:
                 self._batchnorm_literal(i)
@@ -193,11 +235,14 @@ class Discriminator:
         inv_n = float(np.float32(1.0 / np.float64(np.float32(self.batch))))
         CTensorMath.Fill(mean, 0.0)
         CTensorMath.AddSumW(mean, mean, x, 1.0, inv_n)
+        keep = float(np.float32(1.0 - np.float64(np.float32(MOMENTUM))))      # the layer passes 1.0-Momentum, rounded to float
+        CTensorMath.Add(self.stats["mean%d" % i], self.stats["mean%d" % i], mean, MOMENTUM, keep)
         xmu = self.tmp[i]
         CTensorMath.Sub(xmu, x, mean, 1.0, 1.0)
         CTensorMath.Pow2(self.xhat[i], xmu, 1.0)
         CTensorMath.Fill(var, 0.0)
         CTensorMath.AddSumW(var, var, self.xhat[i], 1.0, inv_n)
+        CTensorMath.Add(self.stats["variable%d" % i], self.stats["variable%d" % i], var, MOMENTUM, keep)
         CTensorMath.SQRT(sq, var, 1.0, BN_EPSILON)
         CTensorMath.Inv(self.ivar[i], sq)
         CTensorMath.TensorItemProduction(self.xhat[i], xmu, self.ivar[i])

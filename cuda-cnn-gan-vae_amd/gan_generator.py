@@ -42,6 +42,53 @@ def make_parameters(channels=CHANNELS, noise=NOISE, seed=6):
     return p
 
 
+def make_statistics(channels=CHANNELS):
+    """Running mean and variable of the six batch-norm layers as a fresh layer holds them
+    (Reset, netlayer/cnetlayerbatchnormalization.cu.h:239-240): 0 and 1."""
+    s, size = {}, (3, 4)
+    for i in range(6):
+        size = (size[0] * 2, size[1] * 2)
+        s["mean%d" % i] = np.zeros((1, channels[i + 1]) + size, np.float32)
+        s["variable%d" % i] = np.ones((1, channels[i + 1]) + size, np.float32)
+    return s
+
+
+# cmodel_gan.cu.h:136-225: the input holder is a Linear layer without a predecessor, which saves two [1,1,1,1] tensors
+# (netlayer/cnetlayerlinear.cu.h:175-178)
+LAYER_KINDS = ["linear", "linear", "function"] + ["upsampling", "convolution", "batchnorm", "function"] * 6 + ["convolution", "function"]
+
+
+def net_layers(host, channels=CHANNELS):
+    """Parameters and running statistics (numpy, keys of make_parameters + make_statistics) as the layer list that
+    wire_format.write_net takes, in the order SaveNetLayers writes the reference's generator
+    (cuda/netmodel/cmodelmain.cu.h:296-300)."""
+    one = np.zeros((1, 1, 1, 1), np.float32)
+    layers = [("linear", {"weight": one, "bias": one}), ("linear", {"weight": host["lin_w"], "bias": host["lin_b"]}), ("function", {"name": "leaky_relu"})]
+    widths = tuple(channels[1:]) + (IMAGE_DEPTH,)
+    for i in range(7):
+        header = dict(kernel_amount=widths[i], kernel_x=3, kernel_y=3, kernel_z=channels[i], stride_x=1, stride_y=1, padding_x=1, padding_y=1)
+        if i < 6:
+            layers.append(("upsampling", {"x": 2, "y": 2}))
+        layers.append(("convolution", {"header": header, "kernel": host["kernel%d" % i], "bias": host["bias%d" % i]}))
+        if i < 6:
+            layers.append(("batchnorm", {"beta": host["beta%d" % i], "gamma": host["gamma%d" % i], "mean": host["mean%d" % i],
+                                         "variable": host["variable%d" % i], "momentum": MOMENTUM}))
+            layers.append(("function", {"name": "leaky_relu"}))
+    layers.append(("function", {"name": "tangence"}))
+    return layers
+
+
+def host_from_layers(layers):
+    """The inverse, for a list read with wire_format.read_net(f, LAYER_KINDS)."""
+    host = {"lin_w": layers[1][1]["weight"], "lin_b": layers[1][1]["bias"]}
+    for i, c in enumerate(p for kind, p in layers if kind == "convolution"):
+        host["kernel%d" % i], host["bias%d" % i] = c["kernel"], c["bias"]
+    for i, n in enumerate(p for kind, p in layers if kind == "batchnorm"):
+        for name in ("gamma", "beta", "mean", "variable"):
+            host["%s%d" % (name, i)] = n[name]
+    return host
+
+
 def make_noise(batch, noise=NOISE, seed=6):
     return np.random.default_rng(seed + 1000).standard_normal((batch, 1, noise, 1)).astype(np.float32)
 
@@ -63,7 +110,11 @@ class GanGenerator:
         mt.init(0)
         self.batch, self.channels = batch, tuple(channels)
         host = params or make_parameters(channels, noise)
-        self.p = {k: CTensor.from_numpy(v) for k, v in host.items()}
+        self.p = {k: CTensor.from_numpy(v) for k, v in host.items() if not k.startswith(("mean", "variable"))}
+        # running statistics: one tensor serves as the layer's Mean / Variable and as its NewMean / NewVariable, which the
+        # layer copies into each other at both ends of a training step (netlayer/cnetlayerbatchnormalization.cu.h:620-621,
+        # 650-651); the training-mode forward pass blends into it
+        self.stats = {k: CTensor.from_numpy(host[k] if k in host else v) for k, v in make_statistics(self.channels).items()}
         b = batch
         self.noise = CTensor(b, 1, noise, 1)
         self.h = [CTensor(b, channels[0], 3, 4)]          # layer outputs after the function
@@ -81,48 +132,29 @@ class GanGenerator:
         self.noise.upload(z)
 
     # ---- network file ----------------------------------------------------------------------------------------
-    # cmodel_gan.cu.h:136-225: the input holder is a Linear layer without a predecessor, which saves two [1,1,1,1] tensors
-    # (netlayer/cnetlayerlinear.cu.h:175-178)
-    LAYER_KINDS = ["linear", "linear", "function"] + ["upsampling", "convolution", "batchnorm", "function"] * 6 + ["convolution", "function"]
+    LAYER_KINDS = LAYER_KINDS
+
+    def host_state(self):
+        host = {k: t.numpy() for k, t in self.p.items()}
+        host.update({k: t.numpy() for k, t in self.stats.items()})
+        return host
 
     def save_net(self, f):
-        """The parameters as SaveNetLayers writes the reference's generator (cuda/netmodel/cmodelmain.cu.h:296-300).  This
-        class keeps no running statistics: mean 0 and variable 1 are written, the values of a fresh layer."""
+        """Parameters and running statistics as SaveNetLayers writes the reference's generator
+        (cuda/netmodel/cmodelmain.cu.h:296-300)."""
         import wire_format
-        one = np.zeros((1, 1, 1, 1), np.float32)
-        layers = [("linear", {"weight": one, "bias": one}),
-                  ("linear", {"weight": self.p["lin_w"].numpy(), "bias": self.p["lin_b"].numpy()}), ("function", {"name": "leaky_relu"})]
-        widths = self.channels[1:] + (IMAGE_DEPTH,)
-        for i in range(7):
-            cin = self.channels[i]
-            header = dict(kernel_amount=widths[i], kernel_x=3, kernel_y=3, kernel_z=cin, stride_x=1, stride_y=1, padding_x=1, padding_y=1)
-            if i < 6:
-                layers.append(("upsampling", {"x": 2, "y": 2}))
-            layers.append(("convolution", {"header": header, "kernel": self.p["kernel%d" % i].numpy(), "bias": self.p["bias%d" % i].numpy()}))
-            if i < 6:
-                beta = self.p["beta%d" % i].numpy()
-                layers.append(("batchnorm", {"beta": beta, "gamma": self.p["gamma%d" % i].numpy(), "mean": np.zeros_like(beta),
-                                             "variable": np.ones_like(beta), "momentum": MOMENTUM}))
-                layers.append(("function", {"name": "leaky_relu"}))
-        layers.append(("function", {"name": "tangence"}))
-        wire_format.write_net(f, layers)
+        wire_format.write_net(f, net_layers(self.host_state(), self.channels))
 
     def load_net(self, f):
         """The inverse; tensor sizes in the file must be this network's (the reference loads with check_size)."""
         import wire_format
-        layers = wire_format.read_net(f, self.LAYER_KINDS)
-        found = {"lin_w": layers[1][1]["weight"], "lin_b": layers[1][1]["bias"]}
-        convs = [p for kind, p in layers if kind == "convolution"]
-        norms = [p for kind, p in layers if kind == "batchnorm"]
-        for i, c in enumerate(convs):
-            found["kernel%d" % i], found["bias%d" % i] = c["kernel"], c["bias"]
-        for i, n in enumerate(norms):
-            found["gamma%d" % i], found["beta%d" % i] = n["gamma"], n["beta"]
+        found = host_from_layers(wire_format.read_net(f, self.LAYER_KINDS))
         for name, a in found.items():
-            if a.shape != self.p[name].shape:
-                raise ValueError("%s: the file holds %s, the network %s" % (name, a.shape, self.p[name].shape))
+            t = self.stats[name] if name in self.stats else self.p[name]
+            if a.shape != t.shape:
+                raise ValueError("%s: the file holds %s, the network %s" % (name, a.shape, t.shape))
         for name, a in found.items():
-            self.p[name].upload(a)
+            (self.stats[name] if name in self.stats else self.p[name]).upload(a)
 
     def forward(self, fused=True):
         p, ch = self.p, self.channels
@@ -137,6 +169,7 @@ class GanGenerator:
                     self.up[i] = CTensor(s[0], s[1], s[2] * 2, s[3] * 2)
                 CTensorMath.UpSampling(self.up[i], self.h[i], 2, 2)
                 CTensorConv.ForwardConvolution(self.c[i], self.up[i], p["kernel%d" % i], 3, 3, cin, cout, p["bias%d" % i], 1, 1, 1, 1)
-            Fused.BatchNormForwardTrain(self.h[i + 1], self.c[i], p["gamma%d" % i], p["beta%d" % i], momentum=MOMENTUM, epsilon=BN_EPSILON, func="leaky_relu")
+            Fused.BatchNormForwardTrain(self.h[i + 1], self.c[i], p["gamma%d" % i], p["beta%d" % i], new_mean=self.stats["mean%d" % i],
+                                        new_variable=self.stats["variable%d" % i], momentum=MOMENTUM, epsilon=BN_EPSILON, func="leaky_relu")
         CTensorConv.ForwardConvolution(self.image, self.h[6], p["kernel6"], 3, 3, ch[6], IMAGE_DEPTH, p["bias6"], 1, 1, 1, 1, func="tangence")
         return self.image

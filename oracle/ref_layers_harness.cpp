@@ -399,6 +399,25 @@ static void ChainC(void)
  CMemoryStream bn_saved;
  bn.Save(&bn_saved);
  DumpRaw("C.bn_stream",bn_saved);
+ // the end of a training step: Mean and Variable take the statistics blended by the forward pass, then a second step
+ for(int n=1;n<3;n++) layers[n]->TrainingUpdateWeight(0.05,1);
+ CMemoryStream bn_trained;
+ bn.Save(&bn_trained);
+ DumpRaw("C.bn_trained_stream",bn_trained);
+ CTensor<type_t> x2(BATCH,4,5,5);
+ FillTensor(x2,1.5);
+ input.SetOutput(x2);
+ Dump("C.input2",x2);
+ for(int n=0;n<3;n++) layers[n]->TrainingResetDeltaWeight();
+ for(int n=0;n<3;n++) layers[n]->Forward();
+ for(int n=1;n<3;n++) layers[n]->TrainingUpdateWeight(0.0,2);
+ CMemoryStream bn_trained2;
+ bn.Save(&bn_trained2);
+ DumpRaw("C.bn_trained2_stream",bn_trained2);
+ // inference mode with the trained statistics
+ for(int n=0;n<3;n++) layers[n]->TrainingStop();
+ for(int n=0;n<3;n++) layers[n]->Forward();
+ Dump("C.bn_inference",bn.GetOutputTensor());
 }
 #endif
 

@@ -144,7 +144,7 @@ def test_config5_network_file_round_trip(gpu):
     f = io.BytesIO()
     net.save_net(f)
     # size: 4 conv headers, 4 function ids + the last one, 4 momenta, 26 tensors
-    tensors = sum(int(np.prod(t.shape)) for t in net.p.values()) + 2 * sum(int(np.prod(net.p["beta%d" % i].shape)) for i in range(4))
+    tensors = sum(int(np.prod(t.shape)) for t in net.p.values()) + sum(int(np.prod(t.shape)) for t in net.stats.values())
     assert len(f.getvalue()) == 4 * 32 + 5 * 4 + 4 * 8 + 26 * 16 + 8 * tensors
     other = D.Discriminator(4, D.make_parameters(seed=77))
     other.set_batch(x, labels)
@@ -152,6 +152,11 @@ def test_config5_network_file_round_trip(gpu):
     other.load_net(f)
     for name in net.p:
         assert np.array_equal(net.p[name].numpy(), other.p[name].numpy()), name
+    for name in net.stats:      # the running statistics travel too, and saving what was loaded gives the same bytes
+        assert np.array_equal(net.stats[name].numpy(), other.stats[name].numpy()), name
+    again = io.BytesIO()
+    other.save_net(again)
+    assert again.getvalue() == f.getvalue()
     assert np.array_equal(net.forward(True).numpy(), other.forward(True).numpy())
     # the training state (iteration, Adam moments) travels the same way: after loading both, the next step is the same
     g = io.BytesIO()
@@ -171,6 +176,29 @@ def test_config5_network_file_round_trip(gpu):
     g.seek(0)
     with pytest.raises(ValueError):
         other.load_net(g)
+
+
+def test_config5_running_statistics(gpu, oracle):
+    """The running mean and variable of the batch-norm layers after two training steps, fused and literal: the
+    oracle's blend Add(momentum, 1-momentum) of the batch statistics of the layer's input
+    (netlayer/cnetlayerbatchnormalization.cu.h:311, 324), starting from 0 and 1."""
+    import discriminator as D
+    for fused in (True, False):
+        net = D.Discriminator(6)
+        want = D.make_statistics()
+        for seed in (70, 71):
+            net.set_batch(*D.make_batch(6, seed=seed))
+            net.forward(fused)
+            for i in range(4):
+                zero = np.zeros_like(want["mean%d" % i])
+                r = seq.batchnorm_forward_train(oracle, net.c[i].numpy(), zero + 1, zero, new_mean=want["mean%d" % i], new_var=want["variable%d" % i],
+                                                momentum=D.MOMENTUM)
+                want["mean%d" % i], want["variable%d" % i] = r["new_mean"], r["new_var"]
+            net.backward(fused)
+            net.update(fused=fused)
+        for name in want:
+            assert rel_err(net.stats[name].numpy(), want[name]) <= 1e-5, (fused, name)
+            assert np.abs(want[name] - D.make_statistics()[name]).max() > 1e-3, name
 
 
 def test_config5_full_batch_properties(gpu, oracle):

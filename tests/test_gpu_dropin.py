@@ -113,6 +113,28 @@ def test_reference_batchnorm_layer_saved_stream(dumps, oracle):
     assert np.array_equal(kernel, gpu["A.conv_updated.0"]) and np.array_equal(bias, gpu["A.conv_updated.1"])
 
 
+def test_reference_batchnorm_layer_trained_statistics(dumps, oracle):
+    """The running statistics the reference's batch-norm layer saves after one and two training steps on the drop-in
+    classes are the oracle's blends Add(momentum, 1-momentum) of the batch statistics (cnetlayerbatchnormalization.cu.h:311,
+    324, 650-651), and its inference-mode forward pass uses them."""
+    import io
+    import wire_format as wf
+    gpu, _ = dumps
+    beta, gamma = gpu["C.beta"], gpu["C.gamma"]
+    zero, one = np.zeros_like(beta), np.ones_like(beta)
+    first = seq.batchnorm_forward_train(oracle, gpu["C.input"], gamma, beta, new_mean=zero, new_var=one, momentum=0.9)
+    _, _, mean1, var1, momentum = wf.read_batchnorm_layer(io.BytesIO(gpu["C.bn_trained_stream"].tobytes()))
+    assert momentum == float(np.float32(0.9))
+    assert rel_err(mean1, first["new_mean"]) <= 1e-6 and rel_err(var1, first["new_var"]) <= 1e-6
+    assert np.abs(mean1).max() > 0.01 and np.abs(var1 - 1.0).max() > 0.01        # non-trivial
+    # the second step runs with gamma and beta after one gradient step; the statistics do not depend on them
+    second = seq.batchnorm_forward_train(oracle, gpu["C.input2"], gamma, beta, new_mean=first["new_mean"], new_var=first["new_var"], momentum=0.9)
+    beta2, gamma2, mean2, var2, _ = wf.read_batchnorm_layer(io.BytesIO(gpu["C.bn_trained2_stream"].tobytes()))
+    assert rel_err(mean2, second["new_mean"]) <= 1e-6 and rel_err(var2, second["new_var"]) <= 1e-6
+    want = seq.batchnorm_forward_infer(oracle, gpu["C.input2"], gamma2, beta2, mean2, var2)
+    assert rel_err(gpu["C.bn_inference"], want) <= 1e-4
+
+
 def test_dropin_layers_load_a_network_written_from_python(oracle, tmp_path):
     """A network file written by wire_format.py, loaded by the reference's layers on the drop-in classes: forward on the
     GPU against the oracle on the same weights."""

@@ -211,3 +211,37 @@ def test_training_state_written_by_the_reference(cpu_dump):
     f = io.BytesIO()
     wf.write_training_params(f, iteration, layers)
     assert f.getvalue() == raw
+
+
+@pytest.mark.parametrize("model", ["discriminator", "gan_generator"])
+def test_model_files_keep_the_running_statistics(model):
+    """What the Python models write for a network and read back (host side, no device): a stream whose batch-norm layers
+    carry trained running statistics, read into the model's parameter dictionary and written again, is the same bytes,
+    so loading a trained network and saving it loses nothing."""
+    import importlib
+    mod = importlib.import_module(model)
+    rng = np.random.default_rng(7)
+    if model == "discriminator":
+        host = dict(mod.make_parameters(), **mod.make_statistics())
+        layers_of, kinds = mod.net_layers, mod.LAYER_KINDS
+    else:
+        channels = (8, 8, 4, 4, 2, 2, 2)
+        host = dict(mod.make_parameters(channels, 16), **mod.make_statistics(channels))
+        layers_of, kinds = (lambda h: mod.net_layers(h, channels)), mod.LAYER_KINDS
+    for name in host:
+        if name.startswith("mean"):
+            host[name] = rng.standard_normal(host[name].shape).astype(np.float32)
+        if name.startswith("variable"):
+            host[name] = rng.uniform(0.2, 3.0, host[name].shape).astype(np.float32)
+    first = io.BytesIO()
+    wf.write_net(first, layers_of(host))
+    back = mod.host_from_layers(wf.read_net(io.BytesIO(first.getvalue()), kinds))
+    assert sorted(back) == sorted(host)
+    for name in host:
+        assert np.array_equal(back[name], host[name]), name
+    second = io.BytesIO()
+    wf.write_net(second, layers_of(back))
+    assert second.getvalue() == first.getvalue()
+    # the statistics sit where the reference's layer reads them: third and fourth tensor of a batch-norm layer
+    norm = [p for kind, p in wf.read_net(io.BytesIO(first.getvalue()), kinds) if kind == "batchnorm"][0]
+    assert np.array_equal(norm["mean"], host["mean0"]) and np.array_equal(norm["variable"], host["variable0"])
