@@ -298,6 +298,10 @@ def main():
                          "is about a hundred short kernels and the Python host would be the bottleneck)")
     ap.add_argument("--ops-batch", type=int, default=256, help="workload ops: batch size of the [W,64,32,32] activation (1024: 268 MB per tensor)")
     ap.add_argument("--literal", action="store_true", help="workload gan: up-sampling and convolution as two layers")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="mt_set_option before the run (measurements: tconv_walk=0, pack_cache=0, igemm_tile=3 ...); may be repeated")
+    ap.add_argument("--fold", default=None, metavar="LAYERS",
+                    help="workload c3: batch norms folded into the convolutions around them, e.g. 3 or 1,2,3 or none (default: the generator's own choice)")
     ap.add_argument("--workload", choices=["c3", "c5", "ops", "c1", "c2", "c4", "gan"], default="c3",
                     help="c3 (default, the measured configuration): DCGAN-64 generator forward, batch 256; "
                          "c5 (secondary): DCGAN-64 discriminator training step, batch 128; "
@@ -307,6 +311,12 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the path would shard along the batch axis, one all-reduce of the batch-norm sums per layer")
+    if args.option:
+        import mi355tensor as mt_
+        mt_.init(0)
+        for item in args.option:
+            name, value = item.split("=")
+            mt_.set_option(name, int(value))
     if args.workload == "c5":
         return discriminator_step(args)
     if args.workload == "ops":
@@ -318,6 +328,8 @@ def main():
     import generator as G
 
     net = G.DcganGenerator(BATCH)
+    if args.fold is not None:
+        net.fold = () if args.fold == "none" else tuple(int(v) for v in args.fold.split(","))
     net.set_latent(G.make_latent(BATCH))
     stream = mt.get_stream()
     create, record, elapsed_ms = hip_events()

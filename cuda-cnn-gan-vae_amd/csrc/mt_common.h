@@ -18,7 +18,17 @@ int split_workspace(size_t floats, float **p);
 int split_reduce(const char *name, float *out, const float *partial, uint32_t S, size_t n, const float *bias, uint32_t bias_div, uint32_t bias_mod, int func);
 int set_conv_path(int v);  // 0 auto, 1 direct kernels, 2 matrix cores wherever they apply
 int set_igemm_tile(int v); // -1 auto, 0..4 force one block tile of the matrix-core kernels
-int set_patch_blocks(int v);  // persistent blocks of the input-patch transposed convolution (default 512)
+int set_patch_blocks(int v);
+int set_walk_blocks(int v);
+int set_walk_waves(int v);
+int set_walk_tm(int v);
+int set_tconv_walk(int v);    // blocks of a transposed convolution that walk over the batch: 0 never for plain calls, 1 wherever the shape allows
+// out = func(scale * in + shift) with the pairs (scale, shift) per element [Z][Y][X] of one sample (func: a cheap one)
+int norm_apply(const mt_tensor *out, const mt_tensor *in, const float *scale_shift, int func);
+// statistics of x over the batch as a separate pass: (scale, shift) pairs of the batch normalisation that follows, and
+// the optional outputs of mt_batchnorm_forward_train_func
+int bn_statistics(const mt_tensor *x, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *scale_shift, const mt_tensor *ivar,
+                  const mt_tensor *mean, const mt_tensor *var, const mt_tensor *new_mean, const mt_tensor *new_var, float momentum, float epsilon);  // persistent blocks of the input-patch transposed convolution (default 512)
 int set_wgrad_groups(int v);  // 0 auto, else batch groups of the batch-summed weight gradient
 
 // A library-owned device buffer that grows on demand.  Recorded HIP graphs keep the pointers of the recording:

@@ -13,9 +13,11 @@
 #include <string.h>
 
 #include <initializer_list>
+#include <utility>
 #include <vector>
 
 #include "mt_igemm.h"
+#include "mt_walk.h"
 
 namespace {
 
@@ -42,7 +44,7 @@ int with_row_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, Batch bt, F 
 
 // ---- library-owned workspace: the partial sums of the batch-summed gradients, up-sampled images, and re-ordered
 // weights while they cannot be kept (see below)
-mt::Workspace g_ws;
+mt::Workspace g_ws, g_stats_ws, g_norm_ws;
 int workspace(size_t floats, float **p) { return mt::workspace_get(g_ws, "convolution workspace", floats, p); }
 
 // ---- re-ordered weights, kept between calls ---------------------------------------------------------------------
@@ -74,12 +76,18 @@ struct PackEntry {
   float *buf = nullptr;
   size_t floats = 0;
   bool valid = false;
+  bool pinned = false;  // a recorded graph writes and reads the buffer: it is never freed
   uint64_t used = 0;
 };
 constexpr size_t PACK_MAX_ENTRIES = 64, PACK_MAX_BYTES = (size_t)512 << 20;
 std::vector<PackEntry> g_packs;
 bool g_pack_cache = true;
 uint64_t g_pack_clock = 0, g_pack_hits = 0, g_pack_made = 0;
+// Memory that calls recorded into a graph write.  A replay changes it without the library seeing a call, so copies made
+// from such memory are never trusted: they are made again on every use (training weights that a recorded step updates).
+std::vector<std::pair<uintptr_t, uintptr_t>> g_graph_written;
+bool g_graph_writes_anything = false;  // the list overflowed: nothing is trusted any more
+constexpr size_t GRAPH_WRITTEN_MAX = 4096;
 
 PackKey pack_key(int kind, const mt_tensor *kernel, const mt_tensor *bias, std::initializer_list<int32_t> geo) {
   PackKey k{};
@@ -98,22 +106,43 @@ bool capturing() {
   return st != hipStreamCaptureStatusNone;
 }
 
+inline bool overlaps(const float *p, size_t floats, uintptr_t lo, uintptr_t hi) {
+  const uintptr_t a = (uintptr_t)p, b = a + floats * sizeof(float);
+  return p != nullptr && a < hi && lo < b;
+}
+inline size_t key_floats(const uint32_t (&d)[4]) { return (size_t)d[0] * d[1] * d[2] * d[3]; }
+
+bool written_by_a_graph(const PackKey &k) {
+  if (g_graph_writes_anything) return true;
+  for (const auto &r : g_graph_written)
+    if (overlaps(k.kernel, key_floats(k.kernel_dims), r.first, r.second) || overlaps(k.bias, key_floats(k.bias_dims), r.first, r.second)) return true;
+  return false;
+}
+
+void drop_entry(size_t i) {  // the stream is idle
+  if (!g_packs[i].pinned) (void)hipFree(g_packs[i].buf);   // a pinned buffer stays allocated: a graph may still name it
+  g_packs.erase(g_packs.begin() + i);
+}
+
 // Where the re-ordered weights of `key` live: *fresh tells the caller to make them (again).
+// While the stream is captured the recording makes them itself at every replay -- into the entry's own buffer when
+// the weights have been used before (the buffer is then never freed), else into the workspace.
 int pack_buffer(const PackKey &key, size_t floats, float **buf, bool *fresh) {
-  if (!g_pack_cache || floats * sizeof(float) > PACK_MAX_BYTES / 4 || capturing()) {
-    *fresh = true;
-    return workspace(floats, buf);
-  }
+  *fresh = true;
+  if (!g_pack_cache || floats * sizeof(float) > PACK_MAX_BYTES / 4) return workspace(floats, buf);
+  const bool recording = capturing();
   g_pack_clock++;
   for (PackEntry &e : g_packs)
     if (e.key == key && e.floats == floats) {
       e.used = g_pack_clock;
       *buf = e.buf;
-      *fresh = !e.valid;
+      if (recording) { e.pinned = true; return MT_OK; }
+      *fresh = !e.valid || written_by_a_graph(key);
       e.valid = true;
       if (*fresh) g_pack_made++; else g_pack_hits++;
       return MT_OK;
     }
+  if (recording) return workspace(floats, buf);
   size_t bytes = floats * sizeof(float);
   for (const PackEntry &e : g_packs) bytes += e.floats * sizeof(float);
   while (!g_packs.empty() && (g_packs.size() >= PACK_MAX_ENTRIES || bytes > PACK_MAX_BYTES)) {  // least recently used goes
@@ -121,9 +150,8 @@ int pack_buffer(const PackKey &key, size_t floats, float **buf, bool *fresh) {
     for (size_t i = 1; i < g_packs.size(); i++)
       if (g_packs[i].used < g_packs[lru].used) lru = i;
     MT_HIP(hipStreamSynchronize(mt::stream()));
-    MT_HIP(hipFree(g_packs[lru].buf));
     bytes -= g_packs[lru].floats * sizeof(float);
-    g_packs.erase(g_packs.begin() + lru);
+    drop_entry(lru);
   }
   PackEntry e;
   e.key = key; e.floats = floats; e.valid = true; e.used = g_pack_clock;
@@ -132,13 +160,7 @@ int pack_buffer(const PackKey &key, size_t floats, float **buf, bool *fresh) {
   g_packs.push_back(e);
   g_pack_made++;
   *buf = e.buf;
-  *fresh = true;
   return MT_OK;
-}
-
-inline bool overlaps(const float *p, size_t floats, uintptr_t lo, uintptr_t hi) {
-  const uintptr_t a = (uintptr_t)p, b = a + floats * sizeof(float);
-  return p != nullptr && a < hi && lo < b;
 }
 
 struct ConvGeo {
@@ -551,17 +573,28 @@ __global__ __launch_bounds__(256) void tconv_k4s2_small_kernel(TconvArgs args) {
 // channels per chunk.  The tile columns are fetched with 128-bit buffer loads, the two halo columns with 32-bit ones;
 // everything outside the image comes back as zero through the range check.  The byte offsets of a thread's pieces are
 // computed once; the chunk advances through the scalar offset.  Needs W % 4 == 0 and 16-byte aligned rows.
-template <int TW, int TH, int CC>
+// NORM: the input still owes func(scale * x + shift) with one (scale, shift) pair per element [C][H][W]; the pairs of a
+// piece are fetched beside it (two 128-bit loads for the four pairs of a 128-bit piece) and applied on the way to LDS.
+// Pieces outside the image load their pairs out of range as well: func(0 * 0 + 0) = 0 keeps the padding zero.
+template <int TW, int TH, int CC, bool NORM = false>
 struct HaloTile {
   static constexpr int PITCH = TW + 4, ROWS = TH + 2, FLOATS = CC * ROWS * PITCH;
   static constexpr int VEC = CC * ROWS * (TW / 4), NVEC = (VEC + 255) / 256;
   static constexpr int EDGE = CC * ROWS * 2, NEDGE = (EDGE + 255) / 256;
-  __amdgpu_buffer_rsrc_t rsrc;
-  uint32_t voff[NVEC], eoff[NEDGE], vdst[NVEC], edst[NEDGE], chunk_bytes;
+  __amdgpu_buffer_rsrc_t rsrc, prsrc;
+  uint32_t voff[NVEC], eoff[NEDGE], vdst[NVEC], edst[NEDGE], chunk_bytes, image_bytes;
+  int in_func;
   floatx4 rv[NVEC];
   float re[NEDGE];
-  __device__ void setup(const float *p, uint32_t bytes, uint32_t imgoff, uint32_t H, uint32_t W, uint32_t x0, uint32_t y0, uint32_t tid) {
+  floatx4 pv[NORM ? NVEC : 1][2];
+  floatx2 pe[NORM ? NEDGE : 1];
+  __device__ void setup(const float *p, uint32_t bytes, uint32_t imgoff, uint32_t H, uint32_t W, uint32_t x0, uint32_t y0, uint32_t tid,
+                        const float *pairs = nullptr, uint32_t channels = 0, int func = MT_F_NONE) {
     rsrc = make_rsrc(p, bytes);
+    prsrc = rsrc;
+    if (NORM) prsrc = make_rsrc(pairs, channels * H * W * 8u);
+    in_func = func;
+    image_bytes = imgoff;
     chunk_bytes = CC * H * W * 4u;
 #pragma unroll
     for (int i = 0; i < NVEC; i++) {
@@ -587,18 +620,39 @@ struct HaloTile {
     for (int i = 0; i < NVEC; i++) rv[i] = buf_load4(rsrc, voff[i], soff);
 #pragma unroll
     for (int i = 0; i < NEDGE; i++) re[i] = buf_load(rsrc, eoff[i], soff);
+    if constexpr (NORM) {  // the pairs of an element sit at twice its byte offset inside the sample
+#pragma unroll
+      for (int i = 0; i < NVEC; i++) {
+        const uint32_t po = voff[i] == OOB ? OOB : (voff[i] - image_bytes) * 2u;
+        pv[i][0] = buf_load4(prsrc, po, 2u * soff);
+        pv[i][1] = buf_load4(prsrc, po == OOB ? OOB : po + 16u, 2u * soff);
+      }
+#pragma unroll
+      for (int i = 0; i < NEDGE; i++) pe[i] = buf_load2(prsrc, eoff[i] == OOB ? OOB : (eoff[i] - image_bytes) * 2u, 2u * soff);
+    }
   }
   __device__ void put(float *t) const {
 #pragma unroll
     for (int i = 0; i < NVEC; i++)
       if (vdst[i] != 0xffffffffu) {  // the tile starts at an odd column: 4 + 8 + 4 bytes
-        t[vdst[i]] = rv[i].x;
-        *reinterpret_cast<float2 *>(t + vdst[i] + 1) = make_float2(rv[i].y, rv[i].z);
-        t[vdst[i] + 3] = rv[i].w;
+        floatx4 v = rv[i];
+        if constexpr (NORM) {
+          v.x = mt::apply_func_cheap(in_func, pv[i][0].x * v.x + pv[i][0].y);
+          v.y = mt::apply_func_cheap(in_func, pv[i][0].z * v.y + pv[i][0].w);
+          v.z = mt::apply_func_cheap(in_func, pv[i][1].x * v.z + pv[i][1].y);
+          v.w = mt::apply_func_cheap(in_func, pv[i][1].z * v.w + pv[i][1].w);
+        }
+        t[vdst[i]] = v.x;
+        *reinterpret_cast<float2 *>(t + vdst[i] + 1) = make_float2(v.y, v.z);
+        t[vdst[i] + 3] = v.w;
       }
 #pragma unroll
     for (int i = 0; i < NEDGE; i++)
-      if (edst[i] != 0xffffffffu) t[edst[i]] = re[i];
+      if (edst[i] != 0xffffffffu) {
+        float v = re[i];
+        if constexpr (NORM) v = mt::apply_func_cheap(in_func, pe[i].x * v + pe[i].y);
+        t[edst[i]] = v;
+      }
   }
 };
 
@@ -615,10 +669,10 @@ struct HaloTile {
 // SPLIT = 2: the block is two halves of 256 threads that take every other chunk of (then four) channels, each with its
 // own pair of LDS buffers, and add their sums at the end: twice the wavefronts per SIMD for a grid of two blocks per
 // compute unit, where the multiply-adds of one wavefront otherwise wait for its own LDS and scalar loads.
-template <int CO, int PP, int SPLIT>
+template <int CO, int PP, int SPLIT, bool NORM>
 __global__ __launch_bounds__(256 * SPLIT) void tconv_k4s2_tile_kernel(TconvArgs args) {
   constexpr int CC = SPLIT == 2 ? 4 : 8;
-  using Tile = HaloTile<16 * PP, 16, CC>;
+  using Tile = HaloTile<16 * PP, 16, CC, NORM>;
   constexpr int TW = 16 * PP, TH = 16, PITCH = Tile::PITCH, ROWS = Tile::ROWS;
   __shared__ __attribute__((aligned(16))) float tiles[SPLIT][2][CC][ROWS][PITCH];
   static_assert(SPLIT == 1 || sizeof(tiles) >= sizeof(float) * 256 * PP * 4 * CO, "the sums of the second half fit into the tile memory");
@@ -628,7 +682,7 @@ __global__ __launch_bounds__(256 * SPLIT) void tconv_k4s2_tile_kernel(TconvArgs 
   const uint32_t half = SPLIT == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / 256) : 0u, tid = threadIdx.x % 256, tx = tid % 16, ty = tid / 16;
   auto &tile = tiles[half];
   Tile stage;
-  stage.setup(args.delta, args.in_w * C * HW * 4u, (g % args.in_w) * C * HW * 4u, H, W, x0, y0, tid);
+  stage.setup(args.delta, args.in_w * C * HW * 4u, (g % args.in_w) * C * HW * 4u, H, W, x0, y0, tid, args.in_scale_shift, C, args.in_func);
   auto fetch = [&](uint32_t step) { stage.fetch(step * SPLIT + half); };
   auto put = [&](int buf) { stage.put(&tile[buf][0][0][0]); };
 
@@ -795,26 +849,30 @@ bool tile_kernel_fits(const mt_tensor *out, const mt_tensor *delta, int32_t kx, 
   return kz <= 4 && kx == 4 && ky == 4 && sx == 2 && sy == 2 && px == 1 && py == 1 && out->y == 2 * delta->y && out->x == 2 * delta->x &&
          delta->x % 4 == 0 && ka % 8 == 0 && ka >= 16 && ((uintptr_t)out->p & 15u) == 0 && ((uintptr_t)delta->p & 15u) == 0 && out->w <= 65535u;
 }
-int launch_tconv_tile(const char *name, TconvArgs &args) {
+template <bool NORM>
+int launch_tconv_tile_norm(const char *name, TconvArgs &args) {
   mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "vector ALU, few output channels") : name);
   dim3 gt(cdiv(args.W, 32) * cdiv(args.H, 16), args.out_w);
   if ((size_t)gt.x * gt.y < 512) {  // fewer than two blocks per compute unit: one pixel per thread, twice the blocks
     dim3 g1(cdiv(args.W, 16) * cdiv(args.H, 16), args.out_w);
-    if (args.M == 1) tconv_k4s2_tile_kernel<1, 1, 1><<<g1, 256, 0, mt::stream()>>>(args);
-    else if (args.M == 2) tconv_k4s2_tile_kernel<2, 1, 1><<<g1, 256, 0, mt::stream()>>>(args);
-    else if (args.M == 3) tconv_k4s2_tile_kernel<3, 1, 1><<<g1, 256, 0, mt::stream()>>>(args);
-    else tconv_k4s2_tile_kernel<4, 1, 1><<<g1, 256, 0, mt::stream()>>>(args);
+    if (args.M == 1) tconv_k4s2_tile_kernel<1, 1, 1, NORM><<<g1, 256, 0, mt::stream()>>>(args);
+    else if (args.M == 2) tconv_k4s2_tile_kernel<2, 1, 1, NORM><<<g1, 256, 0, mt::stream()>>>(args);
+    else if (args.M == 3) tconv_k4s2_tile_kernel<3, 1, 1, NORM><<<g1, 256, 0, mt::stream()>>>(args);
+    else tconv_k4s2_tile_kernel<4, 1, 1, NORM><<<g1, 256, 0, mt::stream()>>>(args);
   } else if ((size_t)gt.x * gt.y < 1024 && args.C % 16 == 0) {  // two to four blocks per compute unit: the channels split over two halves of a block
-    if (args.M == 1) tconv_k4s2_tile_kernel<1, 2, 2><<<gt, 512, 0, mt::stream()>>>(args);
-    else if (args.M == 2) tconv_k4s2_tile_kernel<2, 2, 2><<<gt, 512, 0, mt::stream()>>>(args);
-    else if (args.M == 3) tconv_k4s2_tile_kernel<3, 2, 2><<<gt, 512, 0, mt::stream()>>>(args);
-    else tconv_k4s2_tile_kernel<4, 2, 2><<<gt, 512, 0, mt::stream()>>>(args);
-  } else if (args.M == 1) tconv_k4s2_tile_kernel<1, 2, 1><<<gt, 256, 0, mt::stream()>>>(args);
-  else if (args.M == 2) tconv_k4s2_tile_kernel<2, 2, 1><<<gt, 256, 0, mt::stream()>>>(args);
-  else if (args.M == 3) tconv_k4s2_tile_kernel<3, 2, 1><<<gt, 256, 0, mt::stream()>>>(args);
-  else tconv_k4s2_tile_kernel<4, 2, 1><<<gt, 256, 0, mt::stream()>>>(args);
+    if (args.M == 1) tconv_k4s2_tile_kernel<1, 2, 2, NORM><<<gt, 512, 0, mt::stream()>>>(args);
+    else if (args.M == 2) tconv_k4s2_tile_kernel<2, 2, 2, NORM><<<gt, 512, 0, mt::stream()>>>(args);
+    else if (args.M == 3) tconv_k4s2_tile_kernel<3, 2, 2, NORM><<<gt, 512, 0, mt::stream()>>>(args);
+    else tconv_k4s2_tile_kernel<4, 2, 2, NORM><<<gt, 512, 0, mt::stream()>>>(args);
+  } else if (args.M == 1) tconv_k4s2_tile_kernel<1, 2, 1, NORM><<<gt, 256, 0, mt::stream()>>>(args);
+  else if (args.M == 2) tconv_k4s2_tile_kernel<2, 2, 1, NORM><<<gt, 256, 0, mt::stream()>>>(args);
+  else if (args.M == 3) tconv_k4s2_tile_kernel<3, 2, 1, NORM><<<gt, 256, 0, mt::stream()>>>(args);
+  else tconv_k4s2_tile_kernel<4, 2, 1, NORM><<<gt, 256, 0, mt::stream()>>>(args);
   MT_LAUNCH_CHECK(name);
   return MT_OK;
+}
+int launch_tconv_tile(const char *name, TconvArgs &args) {
+  return args.in_scale_shift ? launch_tconv_tile_norm<true>(name, args) : launch_tconv_tile_norm<false>(name, args);
 }
 
 int launch_tconv_small(const char *name, TconvArgs &args, uint32_t max_n) {
@@ -986,8 +1044,24 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
   return rc == MT_OK && func_later ? mt_apply_func(out, out, func) : rc;
 }
 
+// What a transposed convolution can take over from the batch-norm layers around it (see mt_walk.h).
+struct NormIn {   // the input tensor stands for func(scale * x + shift), the pairs (scale, shift) per element [C][H][W]
+  const float *scale_shift;
+  int func;
+};
+struct BnOut {    // statistics of the output over the batch, turned into (scale, shift) for the consumer of the output
+  const mt_tensor *gamma, *beta, *scale_shift, *ivar, *mean, *var, *new_mean, *new_var;
+  float momentum, epsilon;
+};
+int g_tconv_walk = 1;  // plain calls (no batch norm folded in): 0 never walk, 1 walk wherever the shape allows
+
+// norm / bn: only the kernel that walks over the batch implements them.  `handled` (required with either) tells the
+// caller whether it ran; if not, nothing was launched and the caller composes the result from separate passes.
 int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
-             const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
+             const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func, const NormIn *norm = nullptr, const BnOut *bn = nullptr,
+             bool *handled = nullptr) {
+  const bool fused = norm != nullptr || bn != nullptr;
+  if (handled) *handled = false;
   if (mt::bad(out) || mt::bad(delta) || mt::bad(kernel) || mt::bad(bias)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
   mt::note_write(out);
   if (ka == 0) return mt::fail(MT_E_NO_KERNELS, "%s: at least one kernel is required", name);
@@ -1002,6 +1076,7 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   ConvGeo g{out->w, delta->w, kernel->w, bias->w, (int32_t)ka, (int32_t)delta->y, (int32_t)delta->x, (int32_t)ka, ky, kx, sy, sx, py, px,
             (int32_t)out->y, (int32_t)out->x, kz, kernel->x, kernel->z * kernel->y};
   bool direct = g_conv_path == 1 || kernel->w != 1 || sx > 4 || sy > 4 || delta->y == 0 || delta->x == 0;
+  if (!direct && fused && !mt::fits_buffer(delta)) return MT_OK;
   if (!direct && !mt::fits_buffer(delta)) {
     // the batch is addressed through one 32-bit descriptor: run it in parts of less than 2 GiB of input
     const size_t delta_sample = (size_t)ka * delta->y * delta->x, out_sample = (size_t)kz * out->y * out->x;
@@ -1016,6 +1091,7 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     }
     direct = true;
   }
+  if (direct && fused) return MT_OK;
   if (direct) {
     size_t total = mt::count(out);
     mt::ProfileScope prof("tconv_direct");
@@ -1029,6 +1105,8 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   float *ws = nullptr;
   bool fresh = true;
   const bool tile = mt::igemm::tile_override() < 0 && tile_kernel_fits(out, delta, kx, ky, kz, ka, sx, sy, px, py);
+  const bool tile_norm = tile && norm && !bn;   // the image layer's kernel normalises its input on the way to LDS
+  if (fused && !tile_norm && (tile || kz <= 4 || mt::igemm::tile_override() >= 0)) return MT_OK;
   // the phases depend on the output size as well (an odd output has phases of different sizes and may lack one)
   if ((rc = pack_buffer(pack_key(0, kernel, bias, {kx, ky, kz, (int32_t)ka, sx, sy, px, py, (int32_t)out->x, (int32_t)out->y, tile ? 1 : 0}),
                         sums + (size_t)kz * ka * ky * kx + (size_t)4 * kz * sy * sx + 64, &ws, &fresh)))
@@ -1059,6 +1137,24 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     }
   }
   pa.nphase = args.nphase;
+  // blocks that walk over the batch: the statistics of the output, the normalisation of the input, and for plain calls
+  // the saving of a cold start per tile
+  WalkArgs walk{};
+  bool walks = false;
+  uint32_t walk_tm = 1;
+  if (!tile && kz > 4 && mt::igemm::tile_override() < 0 && (fused || g_tconv_walk) && bias->w == 1 && delta->w == out->w && (int32_t)args.nphase == sy * sx &&
+      mt::fits_buffer((size_t)ka * delta->y * delta->x * 2)) {
+    for (uint32_t f = 0; f < args.nphase; f++) walk.ph[f] = args.ph[f];
+    walk.nphase = args.nphase; walk.M = (uint32_t)kz; walk.batch = out->w;
+    walk.delta = delta->p; walk.C = ka; walk.H = delta->y; walk.W = delta->x;
+    walk.out = out->p; walk.OW = out->x; walk.OHW = OHW; walk.sy = (uint32_t)sy; walk.sx = (uint32_t)sx;
+    walk.func = bn || !mt::epilogue_func(func) ? MT_F_NONE : func;   // any other function runs as a pass of its own afterwards
+    if (norm) { walk.scale_shift = norm->scale_shift; walk.in_func = norm->func; }
+    size_t covered = 0;
+    for (uint32_t f = 0; f < args.nphase; f++) covered += (size_t)args.ph[f].qh * args.ph[f].qw;
+    walk_tm = mt::igemm::walk_tm() == 2 && kz % 128 == 0 ? 2u : 1u;
+    walks = covered == OHW && tconv_walk_plan(walk, (uint32_t)mt::igemm::walk_blocks(), walk_tm);
+  }
   if (fresh) {
     mt::ProfileScope prof("tconv_prepare");
     bool k4s2 = kx == 4 && ky == 4 && sx == 2 && sy == 2 && args.nphase == 4 && kernel->x % 4 == 0 && ((uintptr_t)kernel->p & 15u) == 0 && kz <= 65534;
@@ -1078,6 +1174,36 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   args.ep.sy = sy; args.ep.sx = sx; args.ep.OW = out->x;
   args.ep.tap_bias = ws; args.ep.bias_w = bias->w; args.ep.IH = delta->y; args.ep.IW = delta->x;
   args.ep.func = func;
+  if (fused && !walks && !tile_norm) return MT_OK;
+  if (walks) {
+    const size_t S = (size_t)kz * OHW;
+    if (bn) {
+      float *part = nullptr;
+      if ((rc = mt::workspace_get(g_stats_ws, "batch-norm partial statistics", 2 * (size_t)walk.groups * S, &part))) return rc;
+      walk.part_mean = part; walk.part_m2 = part + (size_t)walk.groups * S;
+    }
+    walk.tap_bias = ws;
+    {
+      mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, walk.M, out->w * args.ph[0].qh * args.ph[0].qw, args.ph[0].kp, args.nphase) : name);
+      if ((rc = launch_tconv_walk(name, walk, norm != nullptr, bn != nullptr, walk_tm))) return rc;
+    }
+    if (bn) {
+      mt::ProfileScope prof("bn_finish");
+      const float mom_new = (float)(1.0 - (double)bn->momentum);
+      bn_finish_kernel<<<cdiv(S, 64), 256, 0, mt::stream()>>>(bn->scale_shift->p, bn->mean ? bn->mean->p : nullptr, bn->var ? bn->var->p : nullptr,
+                                                              bn->ivar ? bn->ivar->p : nullptr, bn->new_mean ? bn->new_mean->p : nullptr,
+                                                              bn->new_var ? bn->new_var->p : nullptr, walk.part_mean, walk.part_m2, walk.groups,
+                                                              (float)(walk.per * (64u >> walk.px_log)), (uint32_t)S, bn->gamma->p, bn->beta->p, bn->epsilon,
+                                                              bn->momentum, mom_new);
+      MT_LAUNCH_CHECK("bn_finish");
+    }
+    if (handled) *handled = true;
+    return !bn && !mt::epilogue_func(func) ? mt_apply_func(out, out, func) : MT_OK;
+  }
+  if (tile_norm) {
+    args.in_scale_shift = norm->scale_shift; args.in_func = norm->func;
+    if (handled) *handled = true;
+  }
   if (tile) return launch_tconv_tile(name, args);
   if (kz <= 4 && mt::igemm::tile_override() < 0) {
     rc = launch_tconv_small(name, args, max_n);
@@ -1087,6 +1213,46 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
   args.ep.func = MT_F_NONE;
   rc = launch_tconv(name, args, max_n, mt::count(out));
   return rc == MT_OK ? mt_apply_func(out, out, func) : rc;
+}
+
+// A transposed convolution between two batch-norm layers: the input may still owe its normalisation and activation
+// (scale_shift [1,C,H,2*W], delta_func), and the statistics of the output may be wanted as the (scale, shift) pairs of
+// the NEXT batch normalisation.  One kernel when the blocks can walk over the batch; otherwise the same result from
+// separate passes: normalise into the workspace, convolve, statistics over the output.
+int backward_between_norms(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *scale_shift, int delta_func, const mt_tensor *kernel,
+                           int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func,
+                           const BnOut *bn) {
+  if (mt::bad(out) || mt::bad(delta)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  if (scale_shift) {
+    if (mt::bad(scale_shift) || scale_shift->w == 0 || scale_shift->z != delta->z || scale_shift->y != delta->y || scale_shift->x != 2 * delta->x)
+      return mt::fail(MT_E_SHAPE, "%s: the (scale, shift) pairs of the input must be [1,%u,%u,%u]", name, delta->z, delta->y, 2 * delta->x);
+    if (!mt::epilogue_func(delta_func)) return mt::fail(MT_E_ARGUMENT, "%s: the input's function must be none, linear, ReLU or leaky ReLU", name);
+  }
+  if (bn) {
+    const mt_tensor *same[7] = {bn->gamma, bn->beta, bn->ivar, bn->mean, bn->var, bn->new_mean, bn->new_var};
+    for (int i = 0; i < 7; i++) {
+      if (i < 2 && mt::bad(same[i])) return mt::fail(MT_E_ARGUMENT, "%s: gamma and beta are required", name);
+      if (same[i] && (mt::bad(same[i]) || !mt::same_zyx(same[i], out) || same[i]->w == 0)) return mt::fail(MT_E_SHAPE, "%s: statistics and parameters must be [1,Z,Y,X] of the output", name);
+    }
+    if (mt::bad(bn->scale_shift) || bn->scale_shift->w == 0 || bn->scale_shift->z != out->z || bn->scale_shift->y != out->y || bn->scale_shift->x != 2 * out->x)
+      return mt::fail(MT_E_SHAPE, "%s: the (scale, shift) pairs of the output must be [1,%u,%u,%u]", name, out->z, out->y, 2 * out->x);
+    for (auto t : {bn->scale_shift, bn->ivar, bn->mean, bn->var, bn->new_mean, bn->new_var}) mt::note_write(t);
+  }
+  NormIn norm{scale_shift ? scale_shift->p : nullptr, delta_func};
+  bool handled = false;
+  int rc = backward(name, out, delta, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func, scale_shift ? &norm : nullptr, bn, &handled);
+  if (rc || handled) return rc;
+  if (!scale_shift && !bn) return backward(name, out, delta, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);
+  mt_tensor in = *delta;
+  if (scale_shift && mt::count(delta)) {
+    float *tmp = nullptr;
+    if ((rc = mt::workspace_get(g_norm_ws, "normalised input", mt::count(delta), &tmp))) return rc;
+    in.p = tmp;
+    if ((rc = mt::norm_apply(&in, delta, scale_shift->p, delta_func))) return rc;
+  }
+  if ((rc = backward(name, out, &in, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, bn ? MT_F_NONE : func))) return rc;
+  if (!bn) return MT_OK;
+  return mt::bn_statistics(out, bn->gamma, bn->beta, bn->scale_shift, bn->ivar, bn->mean, bn->var, bn->new_mean, bn->new_var, bn->momentum, bn->epsilon);
 }
 
 // Whether the weight gradient's image operand can use fixed per-thread offsets (SrcWgradImageFixed): the output
@@ -1354,15 +1520,33 @@ int &patch_blocks() {
   static int v = 512;
   return v;
 }
+int &walk_blocks() {
+  static int v = 1024;
+  return v;
+}
+int &walk_waves() {
+  static int v = 4;
+  return v;
+}
+int &walk_tm() {
+  static int v = 1;
+  return v;
+}
 }  // namespace igemm
 void note_write(const void *p, size_t bytes) {
-  if (g_packs.empty() || p == nullptr || bytes == 0) return;
+  if (p == nullptr || bytes == 0) return;
   const uintptr_t lo = (uintptr_t)p, hi = lo + bytes < lo ? ~(uintptr_t)0 : lo + bytes;
+  if (g_pack_cache && !g_graph_writes_anything && capturing()) {  // a replay will write this range unseen
+    bool known = false;
+    for (const auto &r : g_graph_written) known = known || (r.first <= lo && hi <= r.second);
+    if (!known) {
+      if (g_graph_written.size() >= GRAPH_WRITTEN_MAX) g_graph_writes_anything = true;
+      else g_graph_written.emplace_back(lo, hi);
+    }
+  }
   for (PackEntry &e : g_packs) {
     if (!e.valid) continue;
-    const size_t kernel_floats = (size_t)e.key.kernel_dims[0] * e.key.kernel_dims[1] * e.key.kernel_dims[2] * e.key.kernel_dims[3];
-    const size_t bias_floats = (size_t)e.key.bias_dims[0] * e.key.bias_dims[1] * e.key.bias_dims[2] * e.key.bias_dims[3];
-    if (overlaps(e.key.kernel, kernel_floats, lo, hi) || overlaps(e.key.bias, bias_floats, lo, hi)) e.valid = false;
+    if (overlaps(e.key.kernel, key_floats(e.key.kernel_dims), lo, hi) || overlaps(e.key.bias, key_floats(e.key.bias_dims), lo, hi)) e.valid = false;
   }
 }
 int set_pack_cache(int on) {
@@ -1370,8 +1554,7 @@ int set_pack_cache(int on) {
   g_pack_cache = on != 0;
   if (!g_pack_cache && !g_packs.empty()) {
     MT_HIP(hipStreamSynchronize(stream()));
-    for (PackEntry &e : g_packs) MT_HIP(hipFree(e.buf));
-    g_packs.clear();
+    while (!g_packs.empty()) drop_entry(g_packs.size() - 1);
   }
   return MT_OK;
 }
@@ -1382,6 +1565,26 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "pack_cache_made") == 0) { *value = (int64_t)g_pack_made; return true; }
   if (strcmp(name, "pack_cache_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_packs) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
   return false;
+}
+int set_tconv_walk(int v) {
+  if (v < 0 || v > 1) return fail(MT_E_ARGUMENT, "tconv_walk must be 0 (never for plain calls) or 1 (wherever the shape allows)");
+  g_tconv_walk = v;
+  return MT_OK;
+}
+int set_walk_blocks(int v) {
+  if (v < 1 || v > 65536) return fail(MT_E_ARGUMENT, "walk_blocks must be 1..65536");
+  igemm::walk_blocks() = v;
+  return MT_OK;
+}
+int set_walk_tm(int v) {
+  if (v != 1 && v != 2) return fail(MT_E_ARGUMENT, "walk_tm must be 1 or 2");
+  igemm::walk_tm() = v;
+  return MT_OK;
+}
+int set_walk_waves(int v) {
+  if (v != 4 && v != 5) return fail(MT_E_ARGUMENT, "walk_waves must be 4 or 5");
+  igemm::walk_waves() = v;
+  return MT_OK;
 }
 int set_patch_blocks(int v) {
   if (v < 1 || v > 65536) return fail(MT_E_ARGUMENT, "patch_blocks must be 1..65536");
@@ -1433,6 +1636,23 @@ int mt_backward_convolution_func(const mt_tensor *out, const mt_tensor *delta, c
                                  const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
   if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_backward_convolution_func: unknown function id %d", func);
   return backward("mt_backward_convolution_func", out, delta, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);
+}
+
+int mt_backward_convolution_norm_func(const mt_tensor *out, const mt_tensor *delta, const mt_tensor *delta_scale_shift, int delta_func, const mt_tensor *kernel,
+                                      int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func) {
+  if (!mt::valid_func(func, true) || !mt::valid_func(delta_func, true)) return mt::fail(MT_E_ARGUMENT, "mt_backward_convolution_norm_func: unknown function id");
+  return backward_between_norms("mt_backward_convolution_norm_func", out, delta, delta_scale_shift, delta_func, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func, nullptr);
+}
+
+int mt_backward_convolution_norm_stats(const mt_tensor *out, const mt_tensor *delta, const mt_tensor *delta_scale_shift, int delta_func, const mt_tensor *kernel,
+                                       int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py,
+                                       const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *scale_shift, const mt_tensor *ivar,
+                                       const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean, const mt_tensor *new_variable,
+                                       float momentum, float epsilon) {
+  if (!mt::valid_func(delta_func, true)) return mt::fail(MT_E_ARGUMENT, "mt_backward_convolution_norm_stats: unknown function id %d", delta_func);
+  const BnOut bn{gamma, beta, scale_shift, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon};
+  return backward_between_norms("mt_backward_convolution_norm_stats", out, delta, delta_scale_shift, delta_func, kernel, kx, ky, kz, ka, bias, sx, sy, px, py,
+                                MT_F_NONE, &bn);
 }
 
 int mt_create_delta_weight_and_bias(const mt_tensor *dk, int32_t kx, int32_t ky, int32_t kz, uint32_t ka, const mt_tensor *db, const mt_tensor *image,

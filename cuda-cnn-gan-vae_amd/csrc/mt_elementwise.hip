@@ -945,7 +945,56 @@ int static_scratch(float **p) {
 }
 }  // namespace
 
+namespace {
+__global__ __launch_bounds__(EW_THREADS) void norm_apply_kernel(float *out, const float *in, const float2 *ss, uint32_t S, uint32_t W, int func) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (i >= S) return;
+  const float2 p = ss[i];
+  for (uint32_t w = blockIdx.y; w < W; w += gridDim.y) out[(size_t)w * S + i] = mt::apply_func_cheap(func, p.x * in[(size_t)w * S + i] + p.y);
+}
+__global__ __launch_bounds__(EW_THREADS) void bn_scale_shift_kernel(float2 *ss, const float *mean, const float *ivar, const float *gamma, const float *beta, uint32_t S) {
+  const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (i >= S) return;
+  const float scale = gamma[i] * ivar[i];
+  ss[i] = make_float2(scale, beta[i] - mean[i] * scale);
+}
+}  // namespace
+
 namespace mt {
+int norm_apply(const mt_tensor *out, const mt_tensor *in, const float *scale_shift, int func) {
+  const size_t S = (size_t)in->z * in->y * in->x;
+  if (S == 0 || in->w == 0) return MT_OK;
+  mt::ProfileScope prof("norm_apply");
+  norm_apply_kernel<<<dim3(cdiv(S, EW_THREADS), in->w < 16 ? in->w : 16), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, reinterpret_cast<const float2 *>(scale_shift),
+                                                                                                         (uint32_t)S, in->w, func);
+  MT_LAUNCH_CHECK("norm_apply");
+  return MT_OK;
+}
+
+int bn_statistics(const mt_tensor *x, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *scale_shift, const mt_tensor *ivar,
+                  const mt_tensor *mean, const mt_tensor *var, const mt_tensor *new_mean, const mt_tensor *new_var, float momentum, float epsilon) {
+  const size_t S = (size_t)x->z * x->y * x->x;
+  const uint32_t W = x->w;
+  if (S == 0 || W == 0) return MT_OK;
+  float *spare = nullptr;
+  int rc = bn_scratch(3 * S, &spare);
+  if (rc) return rc;
+  float *pm = mean ? mean->p : spare, *pv = var ? var->p : spare + S, *pi = ivar ? ivar->p : spare + 2 * S;
+  const float inv_n = (float)(1.0 / (double)(float)W), mom_new = (float)(1.0 - (double)momentum);
+  float *nm = new_mean ? new_mean->p : nullptr, *nv = new_var ? new_var->p : nullptr;
+  {
+    mt::ProfileScope prof("bn_stats");
+    if (S % 4 == 0 && aligned16(x->p))
+      bn_stats_kernel<4><<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(x->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new);
+    else
+      bn_stats_kernel<1><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(x->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new);
+    MT_LAUNCH_CHECK("bn_stats");
+  }
+  bn_scale_shift_kernel<<<cdiv(S, EW_THREADS), EW_THREADS, 0, mt::stream()>>>(reinterpret_cast<float2 *>(scale_shift->p), pm, pi, gamma->p, beta->p, (uint32_t)S);
+  MT_LAUNCH_CHECK("bn_scale_shift");
+  return MT_OK;
+}
+
 int static_scratch_setup() {
   float *p = nullptr;
   return static_scratch(&p);

@@ -15,6 +15,7 @@
 //    rows of one k (coalesced NCHW rows); for k-contiguous sources each thread reads a 16/32-byte vector.
 #pragma once
 
+#include <initializer_list>
 #include <type_traits>
 
 #include "mt_common.h"
@@ -949,6 +950,8 @@ struct TconvArgs {
   size_t split_stride = 0;          // writes its own copy of the output, split_stride floats after the previous one
   const float *delta;          // [in_w][C][H][W]
   uint32_t in_w, C, H, W;
+  const float *in_scale_shift = nullptr;  // kernels that normalise their input: (scale, shift) pairs [C][H][W][2], and the
+  int in_func = MT_F_NONE;                // function applied to scale * x + shift
   Epilogue ep;   // C, row_stride, g_stride, sy, sx, OW, tap_bias, bias_w, IH, IW, func filled in
 };
 

@@ -217,6 +217,10 @@ int mt_set_option(const char *name, int value) {
   if (name && strcmp(name, "wgrad_groups") == 0) return mt::set_wgrad_groups(value);
   if (name && strcmp(name, "patch_blocks") == 0) return mt::set_patch_blocks(value);
   if (name && strcmp(name, "pack_cache") == 0) return mt::set_pack_cache(value);
+  if (name && strcmp(name, "tconv_walk") == 0) return mt::set_tconv_walk(value);
+  if (name && strcmp(name, "walk_blocks") == 0) return mt::set_walk_blocks(value);
+  if (name && strcmp(name, "walk_waves") == 0) return mt::set_walk_waves(value);
+  if (name && strcmp(name, "walk_tm") == 0) return mt::set_walk_tm(value);
   if (name && strcmp(name, "pool") == 0) {
     if (value != 0 && value != 1) return mt::fail(MT_E_ARGUMENT, "pool must be 0 (every mt_free goes to the driver) or 1");
     g_pool_on = value != 0;

@@ -1,0 +1,419 @@
+// Transposed convolution on the fp32 matrix cores whose blocks walk over the batch, with the two halves of a batch
+// normalisation folded into it: the statistics of the layer's own output (epilogue) and the normalisation + activation
+// that its input still owes (loader).
+//
+// A block owns one stride phase, 64 output channels and one tile of PX pixels x SP samples (PX * SP = 64 columns), and
+// walks from one group of SP samples to the next, `per` groups in all.  Going to the next group changes nothing but a
+// scalar byte offset of the operand loads, so the walk is ONE long k loop: the loads of the next group's first tiles
+// are in flight while the last tiles of the current one are multiplied, and the only pause of the matrix pipe is the
+// epilogue itself (the stores of a group drain behind the multiplications of the next).  The one-tile blocks of
+// tconv_kernel pay a cold start and a drain per tile.
+//
+// STATS.  Walking the batch is what makes the statistics cheap: a block sees per * SP samples of every output element
+// it owns.  Each lane keeps a running mean and sum of squared deviations (Welford) of its sixteen elements over the
+// groups it walks, merges the SP samples of a tile at the end (lane shuffles for samples that sit in one wavefront's
+// columns, LDS between the two wavefronts along the columns) and writes ONE (mean, M2) pair per element and block.
+// The pairs of the blocks are combined in a fixed order by a small kernel afterwards: no pass over the activation, and
+// a result that does not depend on timing.
+//
+// NORM.  The input is the raw output of a layer whose batch normalisation and activation are still owed: every value
+// becomes func(scale * x + shift) on its way from the load to LDS, with (scale, shift) per element (c, y, x) fetched as
+// one 64-bit value beside it.  Elements outside the image stay exactly zero: their pair is loaded out of range as well,
+// and func(0 * 0 + 0) = 0 for the functions allowed here.
+#pragma once
+
+#include "mt_igemm.h"
+
+namespace mt {
+namespace igemm {
+
+struct WalkArgs {
+  TconvPhase ph[MAX_PHASES];
+  uint32_t nphase, tiles_m, M, batch;
+  uint32_t px_log, qtiles, groups, per;  // PX = 1 << px_log pixels per tile; pixel tiles per phase; batch groups; steps per block
+  uint32_t nk;                           // k steps of one tile (the same for every phase)
+  const float *delta;                    // [batch][C][H][W]
+  const float *scale_shift;              // NORM: [C][H][W][2]
+  int in_func;                           // NORM: none, linear, ReLU or leaky ReLU
+  uint32_t C, H, W;
+  float *out;                            // [batch][M][OH][OW]
+  uint32_t OW, OHW, sy, sx;
+  const float *tap_bias;                 // sum of the filters' biases, added once per contributing tap (may be null)
+  int func;                              // applied to the output (cheap functions only); with STATS: none
+  float *part_mean, *part_m2;            // STATS: [groups][M * OHW] each
+};
+
+// Merges two sets of n samples each, given as (mean, sum of squared deviations): Chan's update for equal counts.
+__device__ __forceinline__ void welford_merge_equal(float &mean, float &m2, float other_mean, float other_m2, float half_n) {
+  const float d = other_mean - mean;
+  mean = mean + 0.5f * d;
+  m2 = (m2 + other_m2) + (d * d) * half_n;
+}
+
+// TM: 32-row accumulators per wavefront (the block is 64*TM rows x 64 columns, 2 x 2 wavefronts)
+template <bool NORM, bool STATS, int WAVES, int TM>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void tconv_walk_kernel(WalkArgs a) {
+  constexpr int BM = 64 * TM, BN = 64, E = 4;  // four elements per thread, operand and 64 rows
+  __shared__ float4 smem4[2 * (BM + BN) * LDK / 4];
+  float *smem = reinterpret_cast<float *>(smem4);
+  float *As = smem, *Bs = smem + 2 * BM * LDK;
+
+  uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
+  const uint32_t mt = j % a.tiles_m; j /= a.tiles_m;
+  const uint32_t f = j % a.nphase; j /= a.nphase;
+  const uint32_t qt = j % a.qtiles, g = j / a.qtiles;
+  const TconvPhase &ph = a.ph[f];
+  const uint32_t m0 = mt * BM, HW = a.H * a.W, sp = (uint32_t)BN >> a.px_log, px_mask = (1u << a.px_log) - 1u;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // ---- operand A: packed sub-kernel of the phase, [M][ld], one 128-bit load per thread and step
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ph.packed, a.M * ph.ld * 4u);
+  const uint32_t a_row = (uint32_t)tid / 4u, a_k = ((uint32_t)tid % 4u) * E;
+  const uint32_t a_voff = ((m0 + a_row) * ph.ld + a_k) * 4u;  // M is a multiple of the block's rows; the next 64 rows are 64*ld further
+  // ---- operand B: the thread's column (pixel p of sample s of the group) and its E consecutive k (channel, tap)
+  const uint32_t b_col = (uint32_t)tid % BN, b_k = (uint32_t)__builtin_amdgcn_readfirstlane((tid / BN) * E);
+  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(a.delta, a.batch * a.C * HW * 4u);
+  __amdgpu_buffer_rsrc_t s_rsrc = b_rsrc;
+  if (NORM) s_rsrc = make_rsrc(a.scale_shift, a.C * HW * 8u);
+  uint32_t b_voff[E], sample_bytes;  // (the offsets of the pairs follow from b_voff: twice the offset inside the sample)
+  uint32_t sstep;
+  {
+    const uint32_t q = qt * (px_mask + 1u) + (b_col & px_mask), s = b_col >> a.px_log;
+    const uint32_t qy = q / ph.qw, qx = q % ph.qw;
+    const uint32_t sample = g * a.per * sp + s;
+    const uint32_t tx_cnt = (uint32_t)ph.taps_x, taps = (uint32_t)(ph.taps_y * ph.taps_x);  // taps divides BK: powers of two
+    const int lt = __builtin_ctz(taps), lx = __builtin_ctz(tx_cnt);
+    const bool col_ok = q < ph.qh * ph.qw && sample < a.batch;
+#pragma unroll
+    for (int i = 0; i < E; i++) {
+      const uint32_t kk = b_k + i, cc = kk >> lt, t = kk & (taps - 1u), ty = t >> lx, tx = t & (tx_cnt - 1u);
+      const int32_t iy = (int32_t)qy + ph.offy + (int32_t)ty, ix = (int32_t)qx + ph.offx + (int32_t)tx;
+      const bool ok = col_ok && (uint32_t)iy < a.H && (uint32_t)ix < a.W;
+      const uint32_t pixel = (cc * a.H + (uint32_t)iy) * a.W + (uint32_t)ix;
+      b_voff[i] = ok ? (sample * a.C * HW + pixel) * 4u : OOB;
+    }
+    sample_bytes = sample * a.C * HW * 4u;
+    sstep = (BK / taps) * HW * 4u;
+  }
+  const uint32_t group_step = sp * a.C * HW * 4u, nk = a.nk;
+  uint32_t a_soff = 0, b_soff = 0, ctile = 0;
+  auto advance = [&]() {  // scalar unit only
+    ctile++;
+    a_soff += BK * 4u; b_soff += sstep;
+    if (ctile == nk) { ctile = 0; a_soff = 0; b_soff += group_step - nk * sstep; }
+  };
+
+  // Register sets: A and B are loaded two steps before they are written to LDS (two sets, tile t+3 requested while
+  // tile t is multiplied).  The (scale, shift) pairs come from the L2 cache and are requested one step ahead into a
+  // single set -- in front of the A and B loads of the same step, so that waiting for them leaves those in flight.
+  float ra[2][TM][E], rb[2][E];
+  floatx2 rs[NORM ? E : 1];
+  uint32_t s_next = 0;  // scalar offset of the pairs of the tile that is written to LDS next
+  auto load_pairs = [&]() {
+    if constexpr (NORM) {
+#pragma unroll
+      for (int i = 0; i < E; i++) rs[i] = buf_load2(s_rsrc, b_voff[i] == OOB ? OOB : (b_voff[i] - sample_bytes) * 2u, s_next);
+      s_next += 2u * sstep;
+      if (s_next == 2u * sstep * nk) s_next = 0;
+    }
+  };
+  auto load_tile = [&](int set, bool adv) {
+    if (adv) advance();
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const floatx4 t = buf_load4(a_rsrc, a_voff + (uint32_t)i * 64u * ph.ld * 4u, a_soff);
+      ra[set][i][0] = t.x; ra[set][i][1] = t.y; ra[set][i][2] = t.z; ra[set][i][3] = t.w;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < E; i++) rb[set][i] = buf_load(b_rsrc, b_voff[i], b_soff);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  float *a_put = As + a_row * LDK + a_k, *b_put = Bs + b_col * LDK + b_k;
+  const int in_func = a.in_func;
+  auto put_tile = [&](int set, int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) lds_put<E>(a_put + buf * BM * LDK + i * 64 * LDK, ra[set][i]);
+    if constexpr (NORM) {
+      float v[E];
+#pragma unroll
+      for (int i = 0; i < E; i++) v[i] = apply_func_cheap(in_func, rs[i].x * rb[set][i] + rs[i].y);
+      lds_put<E>(b_put + buf * BN * LDK, v);
+    } else {
+      lds_put<E>(b_put + buf * BN * LDK, rb[set]);
+    }
+  };
+
+  const int lrow = lane & 31, lk = lane >> 5;
+  const float *a_get = As + (wm * TM * 32 + lrow) * LDK + lk * 4;
+  const float *b_get = Bs + (wn * 32 + lrow) * LDK + lk * 4;
+  floatx16 acc[TM];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+  float4 fa[2][TM], fb[2];
+  auto read_half = [&](float4 (&av)[TM], float4 &bv, int buf, int half) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) av[i] = *reinterpret_cast<const float4 *>(a_get + buf * BM * LDK + i * 32 * LDK + half * 8);
+    bv = *reinterpret_cast<const float4 *>(b_get + buf * BN * LDK + half * 8);
+  };
+  auto multiply = [&](const float4 (&av)[TM], const float4 &bv) {
+#pragma unroll
+    for (int c = 0; c < 4; c++)  // consecutive matrix instructions go to different accumulators
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        const float x = c == 0 ? av[i].x : c == 1 ? av[i].y : c == 2 ? av[i].z : av[i].w;
+        const float y = c == 0 ? bv.x : c == 1 ? bv.y : c == 2 ? bv.z : bv.w;
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, acc[i], 0, 0, 0);
+      }
+  };
+  auto step = [&](auto parity, auto write_next, auto load_ahead, auto pairs_ahead) {
+    constexpr int cur = decltype(parity)::value, nxt = cur ^ 1;
+    read_half(fa[1], fb[1], cur, 1);
+    if constexpr (decltype(write_next)::value) {
+      put_tile(nxt, nxt);
+      if constexpr (decltype(pairs_ahead)::value) load_pairs();  // the pairs of tile t+2, wanted by the next step
+    }
+    if constexpr (decltype(load_ahead)::value) load_tile(nxt, true);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(fa[0], fb[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    lds_barrier();
+    if constexpr (decltype(write_next)::value) read_half(fa[0], fb[0], nxt, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(fa[1], fb[1]);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- the lane's column of C: pixel and sample of the first group; register r is row m_lane + 8*(r/4) + r%4
+  const uint32_t c_col = (uint32_t)(wn * 32 + lrow);
+  const uint32_t c_q = qt * (px_mask + 1u) + (c_col & px_mask), c_s = c_col >> a.px_log;
+  const uint32_t c_qy = c_q / ph.qw, c_qx = c_q % ph.qw;
+  const uint32_t pix = (c_qy * a.sy + ph.py) * a.OW + c_qx * a.sx + ph.px;
+  const uint32_t m_lane = m0 + (uint32_t)(wm * TM * 32 + 4 * lk);  // whole blocks of rows and whole pixel tiles: no row or column tests
+  float extra = 0.f;
+  if (a.tap_bias) {  // the CPU path adds the bias of every filter once per contributing tap
+    int ny = 0, nx = 0;
+    for (int t = 0; t < ph.taps_y; t++) ny += (uint32_t)((int32_t)c_qy + ph.offy + t) < a.H;
+    for (int t = 0; t < ph.taps_x; t++) nx += (uint32_t)((int32_t)c_qx + ph.offx + t) < a.W;
+    extra = a.tap_bias[0] * (float)(ny * nx);
+  }
+  // element offsets fit 32 bits (the output is addressed like the input: less than 2 GiB)
+  uint32_t dst = ((g * a.per * sp + c_s) * a.M + m_lane) * a.OHW + pix;
+  const uint32_t dst_step = sp * a.M * a.OHW;
+  const int func = a.func;
+  constexpr int NS = STATS ? 16 * TM : 1;
+  float w_mean[NS], w_m2[NS];
+  if constexpr (STATS) {
+#pragma unroll
+    for (int r = 0; r < NS; r++) { w_mean[r] = 0.f; w_m2[r] = 0.f; }
+  }
+  uint32_t seen = 0;  // groups finished
+  auto flush = [&]() {
+    seen++;
+    const float inv_seen = 1.0f / (float)seen;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const uint32_t dm = 32u * i + 8u * (r / 4) + (r & 3);
+        float v = acc[i][r] + extra;
+        if constexpr (STATS) {
+          const float d = v - w_mean[16 * i + r];
+          w_mean[16 * i + r] = w_mean[16 * i + r] + d * inv_seen;
+          w_m2[16 * i + r] = w_m2[16 * i + r] + d * (v - w_mean[16 * i + r]);
+        } else {
+          v = apply_func_cheap(func, v);
+        }
+        a.out[dst + dm * a.OHW] = v;
+        acc[i][r] = 0.f;
+      }
+    dst += dst_step;
+  };
+
+  // ---- the walk: per * nk steps as one software pipeline (see igemm_body for the pipeline itself)
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
+  using Yes = std::true_type;
+  using No = std::false_type;
+  load_pairs();              // pairs of tile 0
+  load_tile(0, false);
+  put_tile(0, 0);
+  load_pairs();              // pairs of tile 1
+  load_tile(1, true);
+  load_tile(0, true);
+  lds_barrier();
+  read_half(fa[0], fb[0], 0, 0);
+  uint32_t left = a.per * nk, kleft = nk;  // nk is even and at least 4, so the last four steps belong to the last group
+  for (; left > 4; left -= 2) {
+    step(Even{}, Yes{}, Yes{}, Yes{});
+    step(Odd{}, Yes{}, Yes{}, Yes{});
+    kleft -= 2;
+    if (kleft == 0) { flush(); kleft = nk; }
+  }
+  step(Even{}, Yes{}, Yes{}, Yes{});   // writes tile left-3, requests the pairs of tile left-2
+  step(Odd{}, Yes{}, No{}, Yes{});     // writes tile left-2, requests the pairs of the last tile
+  step(Even{}, Yes{}, No{}, No{});     // writes the last tile
+  step(Odd{}, No{}, No{}, No{});
+  flush();
+
+  if constexpr (STATS) {
+    // samples of the tile that sit in one wavefront's 32 columns: lanes that differ in the bits at and above px_log
+    float half_n = 0.5f * (float)a.per;  // half of the samples each side of a merge holds
+    for (uint32_t bit = px_mask + 1u; bit < 32u; bit <<= 1) {
+#pragma unroll
+      for (int r = 0; r < NS; r++) {
+        const float om = __shfl_xor(w_mean[r], (int)bit, 64), o2 = __shfl_xor(w_m2[r], (int)bit, 64);
+        welford_merge_equal(w_mean[r], w_m2[r], om, o2, half_n);
+      }
+      half_n *= 2.f;
+    }
+    const bool across = a.px_log <= 5;  // both wavefronts along the columns hold the same pixels (other samples)
+    if (across) {
+      // no wavefront reads operand tiles any more: every LDS read of the last step came before its barrier
+      float *xch = smem + (wm * 64 + lane) * (NS + 1);  // 2 x 64 x (NS + 1) floats, used twice: within the tiles' memory
+      static_assert(2 * 64 * (NS + 1) <= 2 * (BM + BN) * LDK, "the exchange fits into the tiles' memory");
+      float other_mean[NS];
+      if (wn == 1) {
+#pragma unroll
+        for (int r = 0; r < NS; r++) xch[r] = w_mean[r];
+      }
+      __syncthreads();
+      if (wn == 0) {
+#pragma unroll
+        for (int r = 0; r < NS; r++) other_mean[r] = xch[r];
+      }
+      __syncthreads();
+      if (wn == 1) {
+#pragma unroll
+        for (int r = 0; r < NS; r++) xch[r] = w_m2[r];
+      }
+      __syncthreads();
+      if (wn == 0) {
+#pragma unroll
+        for (int r = 0; r < NS; r++) welford_merge_equal(w_mean[r], w_m2[r], other_mean[r], xch[r], half_n);
+      }
+    }
+    const uint32_t keep = px_mask + 1u < 32u ? px_mask + 1u : 32u;  // lanes that hold distinct pixels
+    if ((!across || wn == 0) && (uint32_t)lrow < keep) {
+      const size_t S = (size_t)a.M * a.OHW;
+      float *pm = a.part_mean + (size_t)g * S + (size_t)m_lane * a.OHW + pix, *p2 = a.part_m2 + (size_t)g * S + (size_t)m_lane * a.OHW + pix;
+#pragma unroll
+      for (int r = 0; r < NS; r++) {
+        const uint32_t dm = 32u * (r / 16) + 8u * ((r % 16) / 4) + (r & 3);
+        pm[(size_t)dm * a.OHW] = w_mean[r];
+        p2[(size_t)dm * a.OHW] = w_m2[r];
+      }
+    }
+  }
+}
+
+// Chan's update: (n, mean, m2) takes in another set of samples given the same way
+__device__ __forceinline__ void welford_merge(float &n, float &mean, float &m2, float on, float om, float o2) {
+  if (on == 0.f) return;
+  if (n == 0.f) { n = on; mean = om; m2 = o2; return; }
+  const float total = n + on, d = om - mean, w = __frcp_rn(total);
+  mean = mean + d * (on * w);
+  m2 = (m2 + o2) + (d * d) * (n * on * w);
+  n = total;
+}
+
+// Combines the per-block (mean, M2) pairs of one element in a fixed order (every block holds n_block samples) and turns
+// them into what the consumer of the normalised tensor needs:
+//   mean, biased variance, ivar = 1/sqrt(var + eps);  scale = gamma * ivar,  shift = beta - mean * scale
+// scale_shift is [S][2]; the other outputs are optional.  A block finishes 64 elements: thread (element, quarter) merges
+// the blocks quarter, quarter + 4, ... with eight loads in flight, then the four quarters are merged in order.
+__global__ __launch_bounds__(256) void bn_finish_kernel(float *scale_shift, float *mean_out, float *var_out, float *ivar_out, float *new_mean, float *new_var,
+                                                        const float *part_mean, const float *part_m2, uint32_t blocks, float n_block, uint32_t S,
+                                                        const float *gamma, const float *beta, float eps, float mom_old, float mom_new) {
+  __shared__ float xn[3][64], xm[3][64], x2[3][64];
+  const uint32_t el = threadIdx.x % 64, quarter = threadIdx.x / 64, e = blockIdx.x * 64 + el;
+  float n = 0.f, mean = 0.f, m2 = 0.f;
+  if (e < S) {
+    uint32_t b = quarter;
+    for (; b + 12 < blocks; b += 16) {
+      float om[4], o2[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) { om[i] = part_mean[(size_t)(b + 4 * i) * S + e]; o2[i] = part_m2[(size_t)(b + 4 * i) * S + e]; }
+#pragma unroll
+      for (int i = 0; i < 4; i++) welford_merge(n, mean, m2, n_block, om[i], o2[i]);
+    }
+    for (; b < blocks; b += 4) welford_merge(n, mean, m2, n_block, part_mean[(size_t)b * S + e], part_m2[(size_t)b * S + e]);
+  }
+  if (quarter) { xn[quarter - 1][el] = n; xm[quarter - 1][el] = mean; x2[quarter - 1][el] = m2; }
+  __syncthreads();
+  if (quarter || e >= S) return;
+#pragma unroll
+  for (int q = 0; q < 3; q++) welford_merge(n, mean, m2, xn[q][el], xm[q][el], x2[q][el]);
+  float var = m2 / n;
+  if (var < 0.f) var = 0.f;
+  const float ivar = (float)(1.0 / (double)sqrtf(var + eps));
+  const float scale = gamma[e] * ivar;
+  reinterpret_cast<float2 *>(scale_shift)[e] = make_float2(scale, beta[e] - mean * scale);
+  if (mean_out) mean_out[e] = mean;
+  if (var_out) var_out[e] = var;
+  if (ivar_out) ivar_out[e] = ivar;
+  if (new_mean) new_mean[e] = (mom_old * new_mean[e]) + (mom_new * mean);
+  if (new_var) new_var[e] = (mom_old * new_var[e]) + (mom_new * var);
+}
+
+// Whether (and how) a transposed convolution can walk: fills px_log, qtiles, groups, per, nk.
+inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
+  if (a.nphase == 0 || a.M == 0 || a.batch == 0) return false;
+  const TconvPhase &p0 = a.ph[0];
+  const uint32_t qhw = p0.qh * p0.qw;
+  for (uint32_t f = 0; f < a.nphase; f++) {
+    const TconvPhase &ph = a.ph[f];
+    const uint32_t taps = (uint32_t)(ph.taps_y * ph.taps_x);
+    if (ph.qh * ph.qw != qhw || ph.kp != p0.kp || taps == 0 || BK % taps != 0 || (taps & (taps - 1)) != 0 || (ph.taps_x & (ph.taps_x - 1)) != 0) return false;
+    if (a.C % (BK / taps) != 0 || ph.ld != ph.kp) return false;
+  }
+  if (p0.kp % (2 * BK) != 0 || p0.kp < 4 * BK || a.M % (64 * tm) != 0) return false;
+  if ((uint64_t)a.batch * a.M * a.OHW * 4u >= 0x80000000ull) return false;
+  a.nk = p0.kp / BK;
+  // pixels per tile: 16 (four samples per tile: two per wavefront, merged by a lane shuffle), else 32 or 64
+  uint32_t px_log = 0;
+  for (uint32_t cand : {4u, 5u, 6u})
+    if (qhw % (1u << cand) == 0 && a.batch % (64u >> cand) == 0) { px_log = cand; break; }
+  if (px_log == 0) return false;
+  a.px_log = px_log;
+  a.qtiles = qhw >> px_log;
+  const uint32_t sp = 64u >> px_log, sample_groups = a.batch / sp;
+  a.tiles_m = a.M / (64 * tm);
+  const uint32_t base = a.nphase * a.tiles_m * a.qtiles;
+  // batch groups: as many as give about want_blocks blocks, a divisor of the number of sample groups
+  uint32_t groups = base >= want_blocks ? 1u : want_blocks / base;
+  if (groups > sample_groups) groups = sample_groups;
+  while (groups > 1 && sample_groups % groups) groups--;
+  a.groups = groups;
+  a.per = sample_groups / groups;
+  return (uint64_t)base * groups <= 0x7fffffffu;
+}
+
+int &walk_blocks();   // blocks wanted per launch (measurements only); default 1024, or 1280 for the plain variant
+int &walk_waves();
+int &walk_tm();       // 1 or 2 accumulators per wavefront (2 where the output channels allow; measurements only)    // 4 or 5 wavefronts per SIMD for the plain variant (measurements only)
+
+inline int launch_tconv_walk(const char *name, const WalkArgs &a, bool norm, bool stats, uint32_t tm) {
+  const uint32_t grid = a.nphase * a.tiles_m * a.qtiles * a.groups;
+  hipStream_t s = stream();
+  if (tm == 2) {
+    if (norm && stats) tconv_walk_kernel<true, true, 2, 2><<<grid, THREADS, 0, s>>>(a);
+    else if (norm) tconv_walk_kernel<true, false, 3, 2><<<grid, THREADS, 0, s>>>(a);
+    else if (stats) tconv_walk_kernel<false, true, 3, 2><<<grid, THREADS, 0, s>>>(a);
+    else tconv_walk_kernel<false, false, 4, 2><<<grid, THREADS, 0, s>>>(a);
+  } else if (norm && stats) tconv_walk_kernel<true, true, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  else if (norm) tconv_walk_kernel<true, false, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  else if (stats) tconv_walk_kernel<false, true, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  else if (walk_waves() == 5) tconv_walk_kernel<false, false, 5, 1><<<grid, THREADS, 0, s>>>(a);
+  else tconv_walk_kernel<false, false, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
+}  // namespace igemm
+}  // namespace mt

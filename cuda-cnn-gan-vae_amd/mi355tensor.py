@@ -502,6 +502,22 @@ class Fused:
              _u(kernel_amount), _d(bias), _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y), C.c_int(FUNC[func]))
 
     @staticmethod
+    def BackwardConvolutionNorm(out, delta, delta_scale_shift, delta_func, kernel, kernel_x, kernel_y, kernel_z, kernel_amount, bias, stride_x, stride_y,
+                                padding_x, padding_y, func=None, bn=None):
+        """A transposed convolution whose input still owes func(scale*x+shift) (delta_scale_shift may be None).  With
+        `bn` (a dict: gamma, beta, scale_shift and optionally ivar, batch_mean, batch_var, new_mean, new_variable, momentum,
+        epsilon) the statistics of the output for the batch normalisation that follows are produced as well."""
+        opt = lambda t: _d(t) if t is not None else None
+        head = (_d(out), _d(delta), opt(delta_scale_shift), C.c_int(FUNC[delta_func]), _d(kernel), _i(kernel_x), _i(kernel_y), _i(kernel_z), _u(kernel_amount),
+                _d(bias), _i(stride_x), _i(stride_y), _i(padding_x), _i(padding_y))
+        if bn is None:
+            call("mt_backward_convolution_norm_func", *head, C.c_int(FUNC[func]))
+        else:
+            g = bn.get
+            call("mt_backward_convolution_norm_stats", *head, _d(bn["gamma"]), _d(bn["beta"]), _d(bn["scale_shift"]), opt(g("ivar")), opt(g("batch_mean")),
+                 opt(g("batch_var")), opt(g("new_mean")), opt(g("new_variable")), _f(g("momentum", 0.9)), _f(g("epsilon", 1e-6)))
+
+    @staticmethod
     def FillMany(tensors, value):
         call("mt_fill_many", _u(len(tensors)), _list(tensors), _f(value))
 

@@ -102,7 +102,9 @@ int mt_timer_destroy(void *timer);
  * measurements; results agree within fp32 rounding. */
 int mt_set_option(const char *name, int value);
 /* More options: "pack_cache" 1 (default) keep re-ordered weights between calls / 0 re-order on every call;
- * "pool" 1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no wait) /
+ * "tconv_walk" 1 (default) plain transposed convolutions use the kernel whose blocks walk over the batch wherever the
+ * shape allows / 0 never; "walk_blocks", "walk_waves", "walk_tm": grid size, wavefronts per SIMD and accumulators per
+ * wavefront of that kernel (measurements); "pool" 1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no wait) /
  * 0 every mt_free waits for the stream and returns the block to the driver; "pool_limit_mib" bytes the pool may hold.
  * mt_get_info reads counters of the runtime, for tests and measurements (no counterpart in the reference):
  * "pool_bytes", "pool_reused", "driver_allocations", "retired_workspaces", "pack_cache_entries", "pack_cache_valid",
@@ -186,6 +188,35 @@ int mt_backward_convolution_func(const mt_tensor *output, const mt_tensor *delta
 int mt_upsampling_convolution_func(const mt_tensor *output, const mt_tensor *image, uint32_t upsampling_x, uint32_t upsampling_y,
                                    const mt_tensor *kernel, int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
                                    const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y, int func);
+/* A transposed-convolution layer between two batch-norm layers, with the batch normalisations folded into it
+ * (CNetLayerBatchNormalization::Forward in training mode + CNetLayerFunction::Forward,
+ * netlayer/cnetlayerbatchnormalization.cu.h:301-371, around CNetLayerBackConvolution::Forward,
+ * netlayer/cnetlayerbackconvolution.cu.h:303-315).  A batch normalisation is split at its statistics: the layer in
+ * front of it produces, beside its raw output x, the pair (scale, shift) = (gamma*ivar, beta - mean*gamma*ivar) per
+ * element, and the layer behind it applies func(scale*x + shift) as it loads x.  The normalised tensor is never
+ * written or read.  A tensor of pairs is [1,Z,Y,2*X]: element (z,y,x) holds its scale at 2*x and its shift at 2*x+1.
+ *
+ * mt_backward_convolution_norm_func:  output = func(BackwardConvolution(delta_func(scale*delta + shift), kernel, bias)).
+ *   delta_scale_shift [1,kernel_amount,H,2*W] may be NULL (delta is used as it is); delta_func is none, linear, ReLU or
+ *   leaky ReLU.
+ * mt_backward_convolution_norm_stats: the same with func none, plus the statistics of `output` over the batch for the batch
+ *   normalisation (gamma, beta [1,Z,Y,X] of the output) that follows: scale_shift [1,Z,Y,2*X] of the output, and
+ *   optionally ivar, batch mean, batch variance and the blended running statistics exactly as
+ *   mt_batchnorm_forward_train_func gives them.  xhat of that layer is (output - batch_mean) * ivar.
+ * Where the shape allows (one kernel set and one bias set for the batch, equal batch sizes, output channels a
+ * multiple of 64, phase images of a multiple of 16 pixels, batch a multiple of 4) this is one matrix-core kernel whose
+ * blocks walk over the batch and a small kernel that combines per-block statistics in a fixed order; otherwise the
+ * same results come from separate passes.  Results equal the layer-by-layer path within fp32 rounding
+ * (scale*x + shift against gamma*((x - mean)*ivar) + beta: a few units in the last place of |mean*scale| + |x*scale|). */
+int mt_backward_convolution_norm_func(const mt_tensor *output, const mt_tensor *delta, const mt_tensor *delta_scale_shift, int delta_func,
+                                      const mt_tensor *kernel, int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
+                                      const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y, int func);
+int mt_backward_convolution_norm_stats(const mt_tensor *output, const mt_tensor *delta, const mt_tensor *delta_scale_shift, int delta_func,
+                                       const mt_tensor *kernel, int32_t kernel_x, int32_t kernel_y, int32_t kernel_z, uint32_t kernel_amount,
+                                       const mt_tensor *bias, int32_t stride_x, int32_t stride_y, int32_t padding_x, int32_t padding_y,
+                                       const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *scale_shift, const mt_tensor *ivar,
+                                       const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean, const mt_tensor *new_variable,
+                                       float momentum, float epsilon);
 /* CNetLayerLinear::Forward + CNetLayerFunction::Forward (netlayer/cnetlayerlinear.cu.h:262-282): output[B,1,Out,1] =
  * func(weight[1,1,Out,In] * input[B,1,In,1] + bias[1,1,Out,1]); `input` may have any [B,Z,Y,X] with Z*Y*X == In. */
 int mt_linear_forward_func(const mt_tensor *output, const mt_tensor *weight, const mt_tensor *input, const mt_tensor *bias, int func);

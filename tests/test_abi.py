@@ -32,7 +32,7 @@ def test_header_cites_the_reference_for_every_op():
         if decl in ("mt_init", "mt_malloc", "mt_free", "mt_copy_h2d", "mt_copy_d2h", "mt_copy_d2d", "mt_synchronize", "mt_set_stream", "mt_set_option", "mt_get_info"):
             continue
         pos = header.index("int " + decl + "(")
-        context = header[max(0, pos - 900):pos + 400]
+        context = header[max(0, pos - 3000):pos + 400]
         # a citation of the function it replaces, or the statement that the reference has no such function
         assert re.search(r"(cuda|cpu|netlayer)/[a-z_.]+:\d+|:\d{3,4}|[Nn]o counterpart in the reference", context), decl
 

@@ -46,48 +46,60 @@ def test_config2_linear_stack(gpu, oracle):
 
 
 def test_config3_generator_against_oracle(gpu, oracle):
-    """DCGAN-64 generator forward, every layer output, batch 8 (the oracle needs ~0.2 GFLOP per image)."""
+    """DCGAN-64 generator forward, every layer output, batch 8 (the oracle needs ~0.2 GFLOP per image): the literal op
+    sequence, and the fused path with no, one and all batch norms folded into the convolutions around them."""
     import generator as G
     params, z = G.make_parameters(), G.make_latent(8)
     want = seq.dcgan_generator_forward(oracle, params, z)
     net = G.DcganGenerator(8, params)
     net.set_latent(z)
-    for forward in (net.forward_fused, net.forward_literal):
+    for forward, fold in ((net.forward_fused, ()), (net.forward_fused, (3,)), (net.forward_fused, (1, 2, 3)), (net.forward_literal, ())):
+        net.fold = fold
+        for t in net.h + net.a:
+            mt_fill(t, 7.0)
         forward()
         assert rel_err(net.h[0].numpy(), want["h0"]) <= REL
         for i in range(4):
-            assert rel_err(net.a[i].numpy(), want["a%d" % i]) <= REL, "a%d" % i
+            assert rel_err(net.activation(i), want["a%d" % i]) <= REL, ("a%d" % i, fold)
             if i < 3:
-                assert rel_err(net.h[i + 1].numpy(), want["h%d" % (i + 1)]) <= REL, "h%d" % (i + 1)
+                assert rel_err(net.h[i + 1].numpy(), want["h%d" % (i + 1)]) <= REL, ("h%d" % (i + 1), fold)
         image = net.output.numpy()
-        assert image.shape == (8, 3, 64, 64) and rel_err(image, want["image"]) <= REL
+        assert image.shape == (8, 3, 64, 64) and rel_err(image, want["image"]) <= REL, fold
+
+
+def mt_fill(t, value):
+    import mi355tensor as mt
+    mt.CTensorMath.Fill(t, value)
 
 
 def test_config3_full_batch_properties(gpu, oracle):
-    """Batch 256: (1) the fused and the literal op sequences agree; (2) the transposed convolutions are linear and
-    per-sample independent, so any sample of the big batch equals the same sample run alone through the oracle."""
+    """Batch 256: (1) the fused path (with the batch norms folded that the benchmark folds, and with all of them) and the
+    literal op sequences agree; (2) the transposed convolutions are linear and per-sample independent, so any sample of
+    the big batch equals the same sample run alone through the oracle."""
     import generator as G
     params, z = G.make_parameters(), G.make_latent(256)
     net = G.DcganGenerator(256, params)
     net.set_latent(z)
-    fused = net.forward_fused().numpy()
-    a = [t.numpy() for t in net.a]
-    h = [t.numpy() for t in net.h[:4]]
     literal = net.forward_literal().numpy()
-    assert fused.shape == (256, 3, 64, 64) and np.all(np.isfinite(fused)) and np.all(np.abs(fused) <= 1)
-    assert rel_err(fused, literal) <= REL
-    for i in range(4):
-        # batch-norm output before ReLU has zero mean and unit variance over the batch, per element
-        x = h[i].astype(np.float64)
-        xhat = (x - x.mean(0)) / np.sqrt(x.var(0) + G.BN_EPSILON)
-        assert rel_err(a[i], np.maximum(xhat, 0)) <= REL
-    for i, sample in ((0, 255), (1, 17), (2, 100), (3, 3)):
-        cin, cout = G.CHANNELS[i], G.CHANNELS[i + 1]
-        want = seq.backconv_forward(oracle, a[i][sample:sample + 1], params["kernel%d" % i], params["bias%d" % i], 4, 2, 1, cout)
-        got = h[i + 1][sample:sample + 1] if i < 3 else None
-        if i == 3:
-            want, got = oracle.apply_func(want, "tangence"), fused[sample:sample + 1]
-        assert rel_err(got, want) <= REL, "layer %d" % i
+    for fold in ((), G.FOLD, (1, 2, 3)):
+        net.fold = fold
+        fused = net.forward_fused().numpy()
+        a = [net.activation(i) for i in range(4)]
+        h = [t.numpy() for t in net.h[:4]]
+        assert fused.shape == (256, 3, 64, 64) and np.all(np.isfinite(fused)) and np.all(np.abs(fused) <= 1)
+        assert rel_err(fused, literal) <= REL, fold
+        for i in range(4):
+            # batch-norm output before ReLU has zero mean and unit variance over the batch, per element
+            x = h[i].astype(np.float64)
+            xhat = (x - x.mean(0)) / np.sqrt(x.var(0) + G.BN_EPSILON)
+            assert rel_err(a[i], np.maximum(xhat, 0)) <= REL, (i, fold)
+        for i, sample in ((0, 255), (1, 17), (2, 100), (3, 3)):
+            cin, cout = G.CHANNELS[i], G.CHANNELS[i + 1]
+            want = seq.backconv_forward(oracle, a[i][sample:sample + 1], params["kernel%d" % i], params["bias%d" % i], 4, 2, 1, cout)
+            got = h[i + 1][sample:sample + 1] if i < 3 else None
+            if i == 3:
+                want, got = oracle.apply_func(want, "tangence"), fused[sample:sample + 1]
+            assert rel_err(got, want) <= REL, ("layer %d" % i, fold)
 
 
 def test_config5_training_step_against_oracle(gpu, oracle):

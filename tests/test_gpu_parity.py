@@ -880,3 +880,91 @@ def test_tensor_save_and_load_in_the_wire_format(gpu):
     other.Load(io.BytesIO(raw), check_size=False)
     assert other.shape == (2, 3, 4, 5) and np.array_equal(other.numpy(), a)
     assert other.desc().w == 2 and other.desc().y == 4
+
+
+# ---- transposed convolution between two batch-norm layers ---------------------------------------------------------
+
+def _norm_case(oracle, B, cin, cout, H, W, seed, bias_std=0.0, func="relu"):
+    """Raw input x with batch-norm parameters, its pairs (scale, shift) from float64 statistics, and the oracle's layer
+    by layer result: batch norm (training mode) -> function -> transposed convolution 4x4 stride 2 padding 1."""
+    x = Nrm(seed, B, cin, H, W) * 2.0 + 0.6
+    gin, bin_ = U(seed + 1, 1, cin, H, W, lo=0.5, hi=1.5), U(seed + 2, 1, cin, H, W, lo=-0.3, hi=0.3)
+    kernel, bias = Nrm(seed + 3, 1, 1, cin, cout * 16, std=0.05), Nrm(seed + 4, 1, cin, 1, 1, std=bias_std) if bias_std else np.zeros((1, cin, 1, 1), np.float32)
+    a = oracle.apply_func(seq.batchnorm_forward_train(oracle, x, gin, bin_)["out"], func) if func else seq.batchnorm_forward_train(oracle, x, gin, bin_)["out"]
+    y = oracle.backward_convolution(a, kernel, bias, 4, 4, cout, cin, 2, 2, 1, 1, (B, cout, 2 * H, 2 * W))
+    x64 = x.astype(np.float64)
+    scale = gin / np.sqrt(x64.var(0, keepdims=True) + seq.BN_EPSILON)
+    pairs = np.stack([scale, bin_ - x64.mean(0, keepdims=True) * scale], -1).reshape(1, cin, H, 2 * W).astype(np.float32)
+    return x, pairs, kernel, bias, y
+
+
+@pytest.mark.parametrize("shape", [(8, 16, 64, 4, 4), (16, 32, 128, 8, 8), (12, 8, 64, 16, 16), (4, 8, 192, 4, 8),      # blocks that walk over the batch
+                                   (6, 16, 64, 4, 4), (8, 16, 48, 4, 4), (8, 12, 64, 5, 3), (3, 16, 3, 8, 8), (5, 10, 2, 6, 4)],  # separate passes
+                         ids=lambda s: "x".join(str(v) for v in s))
+@pytest.mark.parametrize("bias_std", [0.0, 0.05], ids=["no-bias", "bias"])
+def test_transposed_convolution_between_batch_norms(gpu, oracle, shape, bias_std):
+    """mt_backward_convolution_norm_func / _norm_stats against the layers one after the other on the oracle: the input
+    is normalised as it is loaded, the raw output comes with the statistics of the batch norm that follows."""
+    from mi355tensor import CTensor, Fused
+    B, cin, cout, H, W = shape
+    x, pairs, kernel, bias, y = _norm_case(oracle, B, cin, cout, H, W, seed=sum(shape), bias_std=bias_std)
+    tx, tp, tk, tb = (CTensor.from_numpy(v) for v in (x, pairs, kernel, bias))
+    out = CTensor(B, cout, 2 * H, 2 * W)
+    for func in ("tangence", None, "leaky_relu"):
+        Fused.BackwardConvolutionNorm(out, tx, tp, "relu", tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func=func)
+        close(out.numpy(), oracle.apply_func(y, func) if func else y)
+    gout, bout = U(7, 1, cout, 2 * H, 2 * W, lo=0.5, hi=1.5), U(8, 1, cout, 2 * H, 2 * W, lo=-0.3, hi=0.3)
+    nm0, nv0 = U(9, 1, cout, 2 * H, 2 * W), U(10, 1, cout, 2 * H, 2 * W, lo=0.5, hi=2.0)
+    want = seq.batchnorm_forward_train(oracle, y, gout, bout, new_mean=nm0, new_var=nv0, momentum=0.9)
+    one = (1, cout, 2 * H, 2 * W)
+    t = dict(gamma=CTensor.from_numpy(gout), beta=CTensor.from_numpy(bout), scale_shift=CTensor(1, cout, 2 * H, 4 * W), ivar=CTensor(*one), batch_mean=CTensor(*one),
+             batch_var=CTensor(*one), new_mean=CTensor.from_numpy(nm0), new_variable=CTensor.from_numpy(nv0), momentum=0.9, epsilon=seq.BN_EPSILON)
+    Fused.BackwardConvolutionNorm(out, tx, tp, "relu", tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, bn=t)
+    close(out.numpy(), y)
+    close(t["batch_mean"].numpy(), want["mean"], 1e-5)
+    close(t["batch_var"].numpy(), want["var"], 1e-5)
+    close(t["ivar"].numpy(), want["ivar"], 1e-5)
+    close(t["new_mean"].numpy(), want["new_mean"], 1e-5)
+    close(t["new_variable"].numpy(), want["new_var"], 1e-5)
+    # the pairs turn the raw output into the next layer's output: func(scale*y + shift) == func(batch norm(y))
+    ss = t["scale_shift"].numpy().reshape(1, cout, 2 * H, 2 * W, 2)
+    close(ss[..., 0] * y + ss[..., 1], want["out"])
+    # without pairs for the input the entry points are the plain layer (+ statistics)
+    a = np.maximum(pairs.reshape(1, cin, H, W, 2)[..., 0] * x + pairs.reshape(1, cin, H, W, 2)[..., 1], 0).astype(np.float32)
+    Fused.BackwardConvolutionNorm(out, CTensor.from_numpy(a), None, None, tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func="relu")
+    close(out.numpy(), oracle.apply_func(y, "relu"))
+
+
+def test_statistics_in_the_epilogue_survive_a_large_mean(gpu, oracle):
+    """Running mean and squared deviations (not sums of squares): an output whose mean is a hundred times its spread."""
+    from mi355tensor import CTensor, Fused
+    B, cin, cout, H = 32, 16, 64, 4
+    x = np.abs(Nrm(70, B, cin, H, H)) + 1.0
+    kernel = np.abs(Nrm(71, 1, 1, cin, cout * 16, std=0.05)) + 0.5      # positive weights, positive input: every output is large
+    bias = np.zeros((1, cin, 1, 1), np.float32)
+    y = oracle.backward_convolution(x, kernel, bias, 4, 4, cout, cin, 2, 2, 1, 1, (B, cout, 8, 8))
+    y64 = y.astype(np.float64)
+    assert np.median(np.abs(y64.mean(0)) / y64.std(0)) > 5
+    one = (1, cout, 8, 8)
+    ones, zeros = np.ones(one, np.float32), np.zeros(one, np.float32)
+    t = dict(gamma=CTensor.from_numpy(ones), beta=CTensor.from_numpy(zeros), scale_shift=CTensor(1, cout, 8, 16), batch_mean=CTensor(*one), batch_var=CTensor(*one))
+    out = CTensor(B, cout, 8, 8)
+    Fused.BackwardConvolutionNorm(out, CTensor.from_numpy(x), None, None, CTensor.from_numpy(kernel), 4, 4, cout, cin, CTensor.from_numpy(bias), 2, 2, 1, 1, bn=t)
+    close(t["batch_mean"].numpy(), y64.mean(0, keepdims=True), 1e-6)
+    close(t["batch_var"].numpy(), y64.var(0, keepdims=True), 1e-4)
+
+
+def test_transposed_convolution_between_batch_norms_argument_checks(gpu):
+    import mi355tensor as mt
+    from mi355tensor import CTensor, Fused
+    x, k, b, out = CTensor(4, 8, 4, 4), CTensor(1, 1, 8, 64 * 16), CTensor(1, 8, 1, 1), CTensor(4, 64, 8, 8)
+    with pytest.raises(mt.TensorError) as e:
+        Fused.BackwardConvolutionNorm(out, x, CTensor(1, 8, 4, 4), "relu", k, 4, 4, 64, 8, b, 2, 2, 1, 1)      # pairs must be [1,C,H,2W]
+    assert e.value.code == 5
+    with pytest.raises(mt.TensorError) as e:
+        Fused.BackwardConvolutionNorm(out, x, CTensor(1, 8, 4, 8), "tangence", k, 4, 4, 64, 8, b, 2, 2, 1, 1)  # only the cheap functions
+    assert e.value.code == 6
+    with pytest.raises(mt.TensorError) as e:
+        Fused.BackwardConvolutionNorm(out, x, None, None, k, 4, 4, 64, 8, b, 2, 2, 1, 1,
+                                      bn=dict(gamma=CTensor(1, 64, 8, 8), beta=CTensor(1, 64, 8, 8), scale_shift=CTensor(1, 64, 8, 8)))
+    assert e.value.code == 5

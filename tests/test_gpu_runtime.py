@@ -121,6 +121,37 @@ def test_recording_never_uses_kept_weights(mt):
         assert np.array_equal(out.numpy(), eager)
 
 
+def test_weights_that_a_recording_updates_are_never_trusted(mt):
+    """A recorded step that changes the weights (an optimiser step inside the graph): replays write the weights without
+    the library seeing a call, so an eager call after a replay must re-order them again although no eager write happened;
+    and a recording made after eager use of the weights needs no workspace of its own."""
+    from mi355tensor import CTensor, CTensorMath as M
+    cin, cout = 32, 64
+    x, out = CTensor.from_numpy(Nrm(60, 4, cin, 4, 4)), CTensor(4, cout, 8, 8)
+    kernel, bias = CTensor.from_numpy(Nrm(61, 1, 1, cin, cout * 16, std=0.05)), CTensor.from_numpy(np.zeros((1, cin, 1, 1), np.float32))
+    other = CTensor.from_numpy(Nrm(62, 1, 1, cin, cout * 16, std=0.05))
+    conv = lambda: mt.CTensorConv.BackwardConvolution(out, x, kernel, 4, 4, cout, cin, bias, 2, 2, 1, 1)
+
+    def step():
+        M.Add(kernel, kernel, other, 1.0, 0.5)
+        conv()
+    conv()                      # the kept copy exists and is valid
+    mt.synchronize()
+    graph = mt.Graph(step)      # records into the kept copy's own buffer
+    for _ in range(3):
+        graph.launch()
+        replayed = out.numpy()
+        hits = mt.get_info("pack_cache_hits")
+        conv()                  # eager, after an unseen write
+        assert mt.get_info("pack_cache_hits") == hits, "the copy of weights that a graph writes was trusted"
+        eager = out.numpy()
+        mt.set_option("pack_cache", 0)
+        conv()
+        mt.set_option("pack_cache", 1)
+        assert np.array_equal(eager, out.numpy()) and np.array_equal(replayed, eager)
+        conv()
+
+
 def test_pool_reuses_blocks_in_stream_order(mt):
     """A temporary that is freed while the kernel that reads it is still queued (the reference's layers do this on
     every backward call, netlayer/cnetlayerconvolution.cu.h:494) and whose block is handed out again at once."""
