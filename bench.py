@@ -4,7 +4,10 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
 A step is one forward pass of the generator over one batch of synthetic latents that are already resident in HBM
-(the fused C-ABI path: Linear, 4 x (BatchNorm + ReLU, transposed conv 4x4 s2 p1), tanh).  Prints ONE JSON line:
+(the fused C-ABI path: Linear, 4 x (BatchNorm + ReLU, transposed conv 4x4 s2 p1), tanh).  Order of the run: W warm-up +
+K timed steps from a cold start (reported), a sustained stretch of load (reported; the clocks settle), then the W
+warm-up + K timed steps that `value` comes from, the same steps with the latents uploaded from the host, and the K
+steps with per-kernel events.  Prints ONE JSON line:
 value = images/s of the whole step; conv_gflops / conv_frac_of_fp32_mfma_peak = algorithmic FLOPs (2*MAC, non-zero
 taps only) of the four transposed convolutions over the time of their kernels; roofline = the dominant kernel
 (the matrix-core implicit GEMM of the three large transposed convolutions) measured with HIP events on the
@@ -334,9 +337,43 @@ def main():
     stream = mt.get_stream()
     create, record, elapsed_ms = hip_events()
 
-    for _ in range(args.warmup):
-        net.forward_fused()
-    mt.synchronize()
+    step = net.forward_fused
+    if args.graph:
+        step()                       # workspaces and kept weights exist before the recording
+        mt.synchronize()
+        graph = mt.Graph(net.forward_fused)
+        step = graph.launch
+
+    def timed_region(steps):
+        """W untimed warm-up steps, then `steps` steps with one event per step boundary on the work stream and the host
+        wall clock beside them.  Returns (milliseconds between first and last event, wall milliseconds, per-step list)."""
+        for _ in range(args.warmup):
+            step()
+        marks = [create() for _ in range(steps + 1)]
+        mt.synchronize()
+        t0 = time.perf_counter()
+        record(marks[0], stream)
+        for i in range(steps):
+            step()
+            record(marks[i + 1], stream)
+        mt.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3
+        per_step = [elapsed_ms(marks[i], marks[i + 1]) for i in range(steps)]
+        return elapsed_ms(marks[0], marks[steps]), wall, per_step
+
+    # Region 0 (reported, not `value`): the first K steps of the process after W warm-up steps.  The GPU raises its
+    # clocks over the first tens of milliseconds of load, so these steps run slower than the same steps of a job that
+    # has been running for a moment.
+    cold_gpu_ms, cold_wall_ms, _ = timed_region(args.steps)
+    # Sustained load: long enough (about 0.3 s) for the clocks to settle, and for a GPU-busy sample from outside to
+    # see the GPU working; its average is reported as ms_per_step_sustained.
+    sustained_steps = max(500, 4 * args.steps)
+    s0, s1 = create(), create()
+    record(s0, stream)
+    for _ in range(sustained_steps):
+        step()
+    record(s1, stream)
+    sustained_ms = elapsed_ms(s0, s1) / sustained_steps
     if args.copy_mib:
         n = args.copy_mib * 1024 * 1024 // 4
         src, dst = mt.CTensor(1, 1, n // 1024, 1024), mt.CTensor(1, 1, n // 1024, 1024)
@@ -344,23 +381,21 @@ def main():
         mt.CTensorMath.Set(dst, src, 1.0, 0.0)   # reads and writes copy_mib MiB each
         mt.synchronize()
 
-    # Timed region 1 (-> value): K steps between two events on the work stream, host wall clock beside it.
-    step = net.forward_fused
-    if args.graph:
-        graph = mt.Graph(net.forward_fused)
-        step = graph.launch
-        for _ in range(3):
-            step()
-    e0, e1 = create(), create()
+    # Timed region 1 (-> value): W warm-up steps, then exactly K steps between events on the work stream, host wall clock
+    # beside it; the larger of the two counts.  The median of the per-step times is reported beside the mean.
+    gpu_ms, wall_ms, per_step_ms = timed_region(args.steps)
+    median_ms = sorted(per_step_ms)[len(per_step_ms) // 2]
+
+    # The same K steps with the latents coming from the host: one 100 KB upload (mt_copy_h2d, which waits for the copy)
+    # in front of every step, wall clock around the K steps.
+    latent_host = G.make_latent(BATCH)
     mt.synchronize()
     t0 = time.perf_counter()
-    record(e0, stream)
     for _ in range(args.steps):
+        net.set_latent(latent_host)
         step()
-    record(e1, stream)
     mt.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    gpu_ms = elapsed_ms(e0, e1)
+    h2d_ms = (time.perf_counter() - t0) * 1e3
 
     # Timed region 2 (-> roofline, per-kernel times): the same K steps with every kernel launch bracketed by two HIP
     # events on the work stream.  The ~40 extra event records per step cost about 0.1 ms of stream time between the
@@ -417,9 +452,14 @@ def main():
         "conv_frac_of_fp32_mfma_peak": conv_tflops / FP32_MFMA_PEAK_TFLOPS,
         "gpu_ms_per_step_events": gpu_ms / args.steps,
         "host_ms_per_step_wall": wall_ms / args.steps,
+        "ms_per_step_median": median_ms,
+        "ms_per_step_with_h2d": h2d_ms / args.steps,
+        "ms_per_step_first_steps_of_the_process": max(cold_gpu_ms, cold_wall_ms) / args.steps,
+        "ms_per_step_sustained": sustained_ms, "sustained_steps": sustained_steps,
         "ms_per_step_with_per_kernel_events": profiled_wall_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": measured_traffic(), "traffic_unit": "bytes per launch",
+                     "traffic_source": "profiles/dcgan64_b256_forward_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, not measured in this run)",
                      "kernel": dom_label,
                      "launches_per_step": dom_launches / args.steps, "avg_launch_ms": dom_ms / dom_launches if dom_launches else None,
                      "flop_per_launch": flop_per_launch,
