@@ -660,9 +660,13 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
   const int wm = wave / WGN, wn = wave % WGN;
 
   int a_row, a_k, b_row, b_k;
-  if (SrcA::K_CONTIG) { constexpr int TPR = BK / EA; a_row = tid / TPR; a_k = (tid % TPR) * EA; }
+  // k-contiguous sources: TPR threads share a row.  With four threads per row (128 bits each) the LDS takes two rows
+  // per cycle, and rows of 80 bytes fill the 32 banks exactly when they are r and r+4 (r and r+1 would share four
+  // banks): eight consecutive threads take rows r, r+4.
+  auto row_of = [](int t, int tpr) { return tpr == 4 ? ((t / 8) / 4) * 8 + ((t / 8) % 4) + 4 * ((t % 8) / 4) : t / tpr; };
+  if (SrcA::K_CONTIG) { constexpr int TPR = BK / EA; a_row = row_of(tid, TPR); a_k = (tid % TPR) * EA; }
   else { a_row = tid % BM; a_k = (tid / BM) * EA; }
-  if (SrcB::K_CONTIG) { constexpr int TPR = BK / EB; b_row = tid / TPR; b_k = (tid % TPR) * EB; }
+  if (SrcB::K_CONTIG) { constexpr int TPR = BK / EB; b_row = row_of(tid, TPR); b_k = (tid % TPR) * EB; }
   else { b_row = tid % BN; b_k = (tid / BN) * EB; }
   // with 64 or more rows per tile a wavefront shares one k range: keep its decomposition on the scalar unit
   if (!SrcA::K_CONTIG && BM >= 64) a_k = __builtin_amdgcn_readfirstlane(a_k);

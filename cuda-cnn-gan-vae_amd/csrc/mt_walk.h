@@ -70,7 +70,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
 
   // ---- operand A: packed sub-kernel of the phase, [M][ld], one 128-bit load per thread and step
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ph.packed, a.M * ph.ld * 4u);
-  const uint32_t a_row = (uint32_t)tid / 4u, a_k = ((uint32_t)tid % 4u) * E;
+  // Four threads write one 64-byte piece of a row to LDS (128-bit each); the LDS takes eight lanes per cycle, i.e. two
+  // rows, and rows of 80 bytes that are r and r+4 apart fill the 32 banks exactly (r and r+1 would share four banks).
+  const uint32_t a_oct = (uint32_t)tid / 8u, a_row = (a_oct / 4u) * 8u + (a_oct % 4u) + 4u * (((uint32_t)tid % 8u) / 4u), a_k = ((uint32_t)tid % 4u) * E;
   const uint32_t a_voff = ((m0 + a_row) * ph.ld + a_k) * 4u;  // M is a multiple of the block's rows; the next 64 rows are 64*ld further
   // ---- operand B: the thread's column (pixel p of sample s of the group) and its E consecutive k (channel, tap)
   const uint32_t b_col = (uint32_t)tid % BN, b_k = (uint32_t)__builtin_amdgcn_readfirstlane((tid / BN) * E);
