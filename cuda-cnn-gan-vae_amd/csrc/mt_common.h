@@ -19,6 +19,7 @@ int split_reduce(const char *name, float *out, const float *partial, uint32_t S,
 int set_conv_path(int v);  // 0 auto, 1 direct kernels, 2 matrix cores wherever they apply
 int set_igemm_tile(int v); // -1 auto, 0..4 force one block tile of the matrix-core kernels
 int set_patch_blocks(int v);
+int set_image_mfma(int v);
 int set_walk_blocks(int v);
 int set_walk_waves(int v);
 int set_walk_tm(int v);

@@ -779,6 +779,149 @@ __global__ __launch_bounds__(256 * SPLIT) void tconv_k4s2_tile_kernel(TconvArgs 
   }
 }
 
+template <int... I, class F>
+__device__ __forceinline__ void static_for(std::integer_sequence<int, I...>, F &&f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+
+// The same layer on the matrix cores.  v_mfma_f32_4x4x1_16B_f32 multiplies sixteen independent 4x1 by 1x4 blocks: with
+// the four rows as output channels (at most 4: the image layer has 3) and the 64 lanes as 64 input pixels, one
+// instruction adds one (channel, tap) term to 4 output channels of 64 pixels -- the same rate as the large matrix
+// instructions, 3/4 of it useful.  Lane l supplies the input value of ITS pixel (operand B); operand A, the coefficients,
+// uses the instruction's block broadcast: a register holds in lanes 4b..4b+3 the coefficients of the four output
+// channels for input channel b of a chunk of 16, and the instruction with broadcast block b takes just those -- one
+// register per (phase, tap) carries 16 channels, so the 16 (phase, tap) combinations of a chunk are 16 registers read
+// from LDS once per chunk.
+//
+// A block (4 wavefronts) owns 8 rows x 32 columns of input pixels of one image; a wavefront two rows.  The input patch
+// behind the tile (10 x 34 pixels) is staged per chunk of 16 channels in LDS as [pixel][channel], 80 bytes per pixel:
+// a lane's 3x3 neighbours are 128-bit reads of four channels each, free of bank conflicts like the operand tiles of
+// the large kernels.  Global loads walk the image rows (lanes along x, four channels per thread gathered into one
+// 128-bit LDS write); the next chunk's values travel while the current chunk is multiplied (two LDS buffers).  NORM:
+// func(scale * x + shift) on the way to LDS, see HaloTile.  The four phases of an output row pair are stored as 8-byte
+// pairs (px = 0, 1), whole lines per wavefront.
+// Needs W % 32 == 0, C % 16 == 0, at most 4 output channels, coefficients packed [ci][phase][co][taps].
+template <bool NORM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void tconv_k4s2_mfma_kernel(TconvArgs args, uint32_t tiles_x, uint32_t tiles_y) {
+  constexpr int TR = 8, TC = 32, PR = TR + 2, PC = TC + 2, PS = 20, CH = 16;
+  constexpr int PIX = PR * PC, ITEMS = PIX * (CH / 4), NIT = (ITEMS + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float patch[2][PIX * PS];
+  __shared__ __attribute__((aligned(16))) float coeff[2][64 * 16];  // [lane][phase * 4 + tap]
+  const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W, M = args.M;
+  const uint32_t tile = blockIdx.x % (tiles_x * tiles_y), g = blockIdx.x / (tiles_x * tiles_y);
+  const uint32_t x0 = (tile % tiles_x) * TC, y0 = (tile / tiles_x) * TR;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta, args.in_w * C * HW * 4u);
+  __amdgpu_buffer_rsrc_t prsrc = rsrc;
+  if (NORM) prsrc = make_rsrc(args.in_scale_shift, C * HW * 8u);
+  const uint32_t image_bytes = (g % args.in_w) * C * HW * 4u;
+
+  // staging items: (pixel of the patch, quad of channels); byte offset of channel 4*quad at that pixel, or out of range
+  uint32_t it_off[NIT], it_dst[NIT];
+#pragma unroll
+  for (int i = 0; i < NIT; i++) {
+    const uint32_t id = (uint32_t)tid + i * 256u, quad = id / PIX, pix = id % PIX, yy = pix / PC, xx = pix % PC;
+    const int32_t y = (int32_t)(y0 + yy) - 1, x = (int32_t)(x0 + xx) - 1;
+    const bool ok = id < ITEMS && (uint32_t)y < H && (uint32_t)x < W;
+    it_off[i] = ok ? ((quad * 4u * H + (uint32_t)y) * W + (uint32_t)x) * 4u : OOB;
+    it_dst[i] = id < ITEMS ? pix * PS + quad * 4u : 0xffffffffu;
+  }
+  floatx4 sv[NIT];
+  floatx2 sp[NORM ? NIT : 1][4];
+  float cw[4];
+  const int in_func = args.in_func;
+  const float *packed = args.ph[0].packed;
+  auto fetch = [&](uint32_t chunk) {
+    const uint32_t soff = image_bytes + chunk * CH * HW * 4u;
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) sv[i][j] = buf_load(rsrc, it_off[i] == OOB ? OOB : it_off[i] + (uint32_t)j * HW * 4u, soff);
+      if constexpr (NORM) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) sp[i][j] = buf_load2(prsrc, it_off[i] == OOB ? OOB : (it_off[i] + (uint32_t)j * HW * 4u) * 2u, 2u * chunk * CH * HW * 4u);
+      }
+    }
+    // coefficients of the chunk: thread (lane l = 4b + i, four of the 16 combinations) reads packed[ci = chunk*16 + b][phase][co = i][tap]
+    const uint32_t l = (uint32_t)tid & 63u, b = l >> 2, co = l & 3u, f = (uint32_t)tid >> 6;
+    const float *src = packed + ((size_t)(chunk * CH + b) * 4u + f) * (4u * M) + co * 4u;
+#pragma unroll
+    for (int t = 0; t < 4; t++) cw[t] = co < M ? src[t] : 0.f;
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NIT; i++)
+      if (it_dst[i] != 0xffffffffu) {
+        floatx4 v = sv[i];
+        if constexpr (NORM) {
+#pragma unroll
+          for (int j = 0; j < 4; j++) v[j] = mt::apply_func_cheap(in_func, sp[i][j].x * v[j] + sp[i][j].y);
+        }
+        *reinterpret_cast<floatx4 *>(&patch[buf][it_dst[i]]) = v;
+      }
+    *reinterpret_cast<floatx4 *>(&coeff[buf][((uint32_t)tid & 63u) * 16u + ((uint32_t)tid >> 6) * 4u]) = floatx4{cw[0], cw[1], cw[2], cw[3]};
+  };
+
+  floatx4acc acc[4];
+#pragma unroll
+  for (int f = 0; f < 4; f++) acc[f] = floatx4acc{0.f, 0.f, 0.f, 0.f};
+  const uint32_t rr = (uint32_t)lane >> 5, lx = (uint32_t)lane & 31u;
+  const float *centre = &patch[0][((wave * 2 + rr + 1) * PC + lx + 1) * PS];  // the lane's pixel in the patch (buffer 0)
+  const uint32_t chunks = C / CH;
+  fetch(0);
+  put(0);
+  __syncthreads();
+  for (uint32_t ch = 0; ch < chunks; ch++) {
+    const int cur = ch & 1;
+    if (ch + 1 < chunks) fetch(ch + 1);
+    floatx4 av[4];  // av[f][t]: coefficients of phase f, tap t for the 16 channels of the chunk (this lane's slot)
+#pragma unroll
+    for (int f = 0; f < 4; f++) av[f] = *reinterpret_cast<const floatx4 *>(&coeff[cur][lane * 16 + f * 4]);
+    const float *pc = centre + cur * PIX * PS;
+    static_for(std::make_integer_sequence<int, CH / 4>{}, [&](auto qc) {
+      constexpr int q = decltype(qc)::value;
+      floatx4 xv[3][3];  // four channels of the nine neighbours
+#pragma unroll
+      for (int dy = 0; dy < 3; dy++)
+#pragma unroll
+        for (int dx = 0; dx < 3; dx++) xv[dy][dx] = *reinterpret_cast<const floatx4 *>(pc + ((dy - 1) * PC + (dx - 1)) * PS + q * 4);
+      static_for(std::make_integer_sequence<int, 4>{}, [&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        // channel 4q+j of the chunk (broadcast block 4q+j): tap (ty, tx) of phase (py, px) reads neighbour
+        // (py + ty - 1, px + tx - 1); consecutive instructions go to different accumulators
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+          for (int f = 0; f < 4; f++) {
+            const int py = f >> 1, px = f & 1, ty = t >> 1, tx = t & 1;
+            acc[f] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[f][t], xv[py + ty][px + tx][j], acc[f], 4, q * 4 + j, 0);
+          }
+      });
+    });
+    if (ch + 1 < chunks) put(cur ^ 1);
+    __syncthreads();
+  }
+
+  const uint32_t qy = y0 + wave * 2 + rr, qx = x0 + lx;
+  if (qy >= H) return;
+  const uint32_t OW = 2 * W, OHW = 4 * HW;
+  const float bsum = args.ep.tap_bias ? args.ep.tap_bias[g % args.ep.bias_w] : 0.f;
+  const int func = args.ep.func;
+#pragma unroll
+  for (int py = 0; py < 2; py++) {
+    const int ny = ((uint32_t)((int32_t)qy + py - 1) < H) + ((uint32_t)((int32_t)qy + py) < H);
+    const int nx0 = ((uint32_t)((int32_t)qx - 1) < W) + 1, nx1 = 1 + ((uint32_t)((int32_t)qx + 1) < W);
+#pragma unroll
+    for (int co = 0; co < 4; co++) {
+      if ((uint32_t)co >= M) break;
+      float2 o;
+      o.x = mt::apply_func_epilogue(func, acc[py * 2][co] + bsum * (float)(ny * nx0));
+      o.y = mt::apply_func_epilogue(func, acc[py * 2 + 1][co] + bsum * (float)(ny * nx1));
+      *reinterpret_cast<float2 *>(args.ep.C + ((size_t)g * M + co) * OHW + (size_t)(2 * qy + py) * OW + 2 * qx) = o;
+    }
+  }
+}
+
 // Forward convolution 3x3, stride 1, padding 1 with at most 4 output channels (an image-producing last layer) on the
 // vector ALUs, same staging: a thread computes two neighbouring output pixels for all KA channels, per input channel
 // 6 LDS reads and 18*KA multiply-adds; the 9 coefficients of (k, c) are contiguous in the kernel tensor and come
@@ -871,7 +1014,22 @@ int launch_tconv_tile_norm(const char *name, TconvArgs &args) {
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }
+// 0 (default): the image layer runs on the vector ALUs; 1: on the matrix cores where the shape allows.  Measured on an
+// MI355X for [256,64,32,32] -> [256,3,64,64]: 35.0 us against 35.3 us (with the normalising loader 47.8 against
+// 40.3 us), so the vector-ALU kernel stays the default; the matrix-core kernel is kept selectable and tested.
+int g_image_mfma = 0;
 int launch_tconv_tile(const char *name, TconvArgs &args) {
+  if (g_image_mfma && args.W % 32 == 0 && args.C % 16 == 0 && args.M <= 4) {
+    mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "4x4x1 matrix instructions, few output channels") : name);
+    const uint32_t tiles_x = args.W / 32, tiles_y = cdiv(args.H, 8);
+    const size_t blocks = (size_t)tiles_x * tiles_y * args.out_w;
+    if (blocks <= 0x7fffffffu) {
+      if (args.in_scale_shift) tconv_k4s2_mfma_kernel<true><<<(uint32_t)blocks, 256, 0, mt::stream()>>>(args, tiles_x, tiles_y);
+      else tconv_k4s2_mfma_kernel<false><<<(uint32_t)blocks, 256, 0, mt::stream()>>>(args, tiles_x, tiles_y);
+      MT_LAUNCH_CHECK(name);
+      return MT_OK;
+    }
+  }
   return args.in_scale_shift ? launch_tconv_tile_norm<true>(name, args) : launch_tconv_tile_norm<false>(name, args);
 }
 
@@ -1565,6 +1723,11 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "pack_cache_made") == 0) { *value = (int64_t)g_pack_made; return true; }
   if (strcmp(name, "pack_cache_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_packs) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
   return false;
+}
+int set_image_mfma(int v) {
+  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "image_mfma must be 0 or 1");
+  g_image_mfma = v;
+  return MT_OK;
 }
 int set_tconv_walk(int v) {
   if (v < 0 || v > 1) return fail(MT_E_ARGUMENT, "tconv_walk must be 0 (never for plain calls) or 1 (wherever the shape allows)");

@@ -968,3 +968,31 @@ def test_transposed_convolution_between_batch_norms_argument_checks(gpu):
         Fused.BackwardConvolutionNorm(out, x, None, None, k, 4, 4, 64, 8, b, 2, 2, 1, 1,
                                       bn=dict(gamma=CTensor(1, 64, 8, 8), beta=CTensor(1, 64, 8, 8), scale_shift=CTensor(1, 64, 8, 8)))
     assert e.value.code == 5
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 3, 8, 32), (3, 32, 3, 5, 32), (2, 64, 2, 16, 64), (1, 16, 4, 9, 32), (2, 48, 1, 8, 32)], ids=lambda s: "x".join(str(v) for v in s))
+def test_image_layer_on_the_4x4x1_matrix_instructions(gpu, oracle, shape):
+    """The selectable matrix-core kernel of the image layer (16 blocks of 4 output channels x 4 pixels per instruction,
+    coefficients broadcast from one block) against the oracle, plain and with the normalising loader, beside the
+    vector-ALU kernel that is the default."""
+    import mi355tensor as mt
+    from mi355tensor import CTensor, CTensorConv, Fused
+    B, cin, cout, H, W = shape
+    x, kernel, bias = Nrm(sum(shape), B, cin, H, W), Nrm(sum(shape) + 1, 1, 1, cin, cout * 16, std=0.1), Nrm(sum(shape) + 2, 1, cin, 1, 1, std=0.05)
+    out_shape = (B, cout, 2 * H, 2 * W)
+    want = oracle.apply_func(oracle.backward_convolution(x, kernel, bias, 4, 4, cout, cin, 2, 2, 1, 1, out_shape), "tangence")
+    pairs = np.stack([U(5, 1, cin, H, W, lo=0.5, hi=1.5), U(6, 1, cin, H, W, lo=-0.5, hi=0.5)], -1)
+    a = np.maximum(pairs[..., 0] * x + pairs[..., 1], 0).astype(np.float32)
+    want_norm = oracle.apply_func(oracle.backward_convolution(a, kernel, bias, 4, 4, cout, cin, 2, 2, 1, 1, out_shape), "tangence")
+    tx, tk, tb, tp, out = CTensor.from_numpy(x), CTensor.from_numpy(kernel), CTensor.from_numpy(bias), CTensor.from_numpy(pairs.reshape(1, cin, H, 2 * W)), CTensor(*out_shape)
+    try:
+        for matrix in (1, 0):
+            mt.set_option("image_mfma", matrix)
+            mt.CTensorMath.Fill(out, 9.0)
+            CTensorConv.BackwardConvolution(out, tx, tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func="tangence")
+            close(out.numpy(), want, 1e-5)
+            mt.CTensorMath.Fill(out, 9.0)
+            Fused.BackwardConvolutionNorm(out, tx, tp, "relu", tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func="tangence")
+            close(out.numpy(), want_norm, 1e-5)
+    finally:
+        mt.set_option("image_mfma", 0)
