@@ -250,6 +250,102 @@ static void GpuClassOnlyChecks(void)
  Report("SetNormalNoise",fabs(sum/4096)<0.08);
 }
 
+// The weight-gradient sequence of the reference's convolution layer (netlayer/cnetlayerconvolution.cu.h:501-508) at a
+// size where the drop-in classes defer the per-sample gradients (mi355::CDeferredGradient), against the same calls
+// with the deferral switched off.
+static type_t Pattern(uint32_t n,type_t scale) {return(static_cast<type_t>(static_cast<int>((n*2654435761u)>>20)%2001-1000)*scale/1000);}
+static void FillPattern(CTensor<type_t> &t,uint32_t seed,type_t scale)
+{
+ uint32_t n=seed;
+ for(uint32_t w=0;w<t.GetSizeW();w++)
+  for(uint32_t z=0;z<t.GetSizeZ();z++)
+   for(uint32_t y=0;y<t.GetSizeY();y++)
+    for(uint32_t x=0;x<t.GetSizeX();x++,n++) t.SetElement(w,z,y,x,Pattern(n,scale));
+}
+static double MaxDifference(const CTensor<type_t> &a,const CTensor<type_t> &b,double &largest)
+{
+ double diff=0;
+ largest=0;
+ for(uint32_t w=0;w<a.GetSizeW();w++)
+  for(uint32_t z=0;z<a.GetSizeZ();z++)
+   for(uint32_t y=0;y<a.GetSizeY();y++)
+    for(uint32_t x=0;x<a.GetSizeX();x++)
+    {
+     double va=a.GetElement(w,z,y,x),vb=b.GetElement(w,z,y,x);
+     if (fabs(va-vb)>diff) diff=fabs(va-vb);
+     if (fabs(vb)>largest) largest=fabs(vb);
+    }
+ return(diff);
+}
+static void DeferredGradientChecks(void)
+{
+ const uint32_t batch=8,amount=128,depth=64,size=4;
+ CTensor<type_t> image(batch,depth,8,8),delta(batch,amount,4,4);
+ FillPattern(image,1,1.0f);
+ FillPattern(delta,77,0.5f);
+ // [0]: every call runs when it is made; [1]: deferred
+ CTensor<type_t> dkernel[2],dbias[2],dkernel_batch[2],dbias_batch[2];
+ for(int n=0;n<2;n++)
+ {
+  mi355::DeferGradients()=(n==1);
+  dkernel[n]=CTensor<type_t>(1,1,amount,depth*size*size);
+  dbias[n]=CTensor<type_t>(1,amount,1,1);
+  dkernel_batch[n]=CTensor<type_t>(batch,1,amount,depth*size*size);
+  dbias_batch[n]=CTensor<type_t>(batch,amount,1,1);
+  FillPattern(dkernel[n],5,0.25f);   // the sums accumulate onto what the layer holds
+  FillPattern(dbias[n],9,0.25f);
+  CTensorMath<type_t>::Fill(dkernel_batch[n],0);
+  CTensorMath<type_t>::Fill(dbias_batch[n],0);
+  CTensorConv<type_t>::CreateDeltaWeightAndBias(dkernel_batch[n],size,size,depth,amount,dbias_batch[n],image,delta,2,2,1,1);
+  CTensorMath<type_t>::AddSumW(dkernel[n],dkernel[n],dkernel_batch[n]);
+  CTensorMath<type_t>::AddSumW(dbias[n],dbias[n],dbias_batch[n],0.5f,2.0f);
+ }
+ double largest=0;
+ double diff=MaxDifference(dkernel[1],dkernel[0],largest);
+ bool ok=diff<=2e-5*largest && largest>1;
+ diff=MaxDifference(dbias[1],dbias[0],largest);
+ ok=ok && diff<=2e-5*largest && largest>1;
+ Report("deferred per-sample gradients: the sums over the batch",ok);
+ // the operands change (the next step's forward pass), then somebody reads the per-sample gradients after all
+ CTensorMath<type_t>::Fill(image,3);
+ CTensorMath<type_t>::Fill(delta,-2);
+ CTensor<type_t> copy=dkernel_batch[1];   // a copy is a reader
+ diff=MaxDifference(copy,dkernel_batch[0],largest);
+ ok=diff<=2e-5*largest && largest>0.1;
+ diff=MaxDifference(dkernel_batch[1],dkernel_batch[0],largest);
+ ok=ok && diff<=2e-5*largest;
+ diff=MaxDifference(dbias_batch[1],dbias_batch[0],largest);
+ ok=ok && diff<=2e-5*largest && largest>0.1;
+ Report("deferred per-sample gradients: read later, operands changed",ok);
+ // a zeroed tensor that nothing was added to is zeros; zeroed and then written by the host, it is what was written
+ CTensor<type_t> zero(batch,2,3,3),other(batch,2,3,3);
+ FillPattern(zero,3,1.0f);
+ CTensorMath<type_t>::Fill(zero,0);
+ ok=(zero.GetElement(batch-1,1,2,2)==0 && zero.GetElement(0,0,0,0)==0);
+ CTensorMath<type_t>::Fill(zero,0);
+ zero.SetElement(1,1,1,1,7);
+ ok=ok && zero.GetElement(1,1,1,1)==7 && zero.GetElement(1,1,1,0)==0;
+ FillPattern(other,4,1.0f);
+ CTensorMath<type_t>::Fill(zero,0);
+ CTensorMath<type_t>::Add(zero,zero,other);
+ diff=MaxDifference(zero,other,largest);
+ ok=ok && diff==0;
+ // gradients added onto a tensor that is not zero take the plain path
+ FillPattern(dkernel_batch[1],11,0.5f);
+ dkernel_batch[0]=dkernel_batch[1];
+ CTensorMath<type_t>::Fill(dbias_batch[0],0);
+ CTensorMath<type_t>::Fill(dbias_batch[1],0);
+ FillPattern(image,1,1.0f);
+ FillPattern(delta,77,0.5f);
+ mi355::DeferGradients()=false;
+ CTensorConv<type_t>::CreateDeltaWeightAndBias(dkernel_batch[0],size,size,depth,amount,dbias_batch[0],image,delta,2,2,1,1);
+ mi355::DeferGradients()=true;
+ CTensorConv<type_t>::CreateDeltaWeightAndBias(dkernel_batch[1],size,size,depth,amount,dbias_batch[1],image,delta,2,2,1,1);
+ diff=MaxDifference(dkernel_batch[1],dkernel_batch[0],largest);
+ ok=ok && diff==0 && largest>0.5;
+ Report("deferred zero fill: reads, host writes, accumulation onto data",ok);
+}
+
 // the scope timer the reference's models wrap around their training phases (cuda/ctimestamp.cu.h)
 static void TimerCheck(void)
 {
@@ -275,6 +371,7 @@ int main(void)
   ForwardConvolutionCheck();
   DeltaWeightChecks();
   BackwardConvolutionCheck();
+  DeferredGradientChecks();
   SummXYCheck();
   CoherenceAndErrors();
   GpuClassOnlyChecks();

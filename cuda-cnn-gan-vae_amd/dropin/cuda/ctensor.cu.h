@@ -9,6 +9,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
+#include <memory>
 #include <string>
 #include <utility>
 #include <vector>
@@ -53,10 +54,43 @@ namespace mi355
     if (bytes!=0) Check(mt_malloc(&Ptr,bytes));
     Bytes=bytes;
    }
+   void assign(const void *device_source,size_t bytes)
+   {
+    resize(bytes);
+    if (Bytes!=0) Check(mt_copy_d2d(Ptr,device_source,Bytes));
+   }
    void swap(CDeviceBuffer &other) {std::swap(Ptr,other.Ptr);std::swap(Bytes,other.Bytes);}
    void* get(void) const {return(Ptr);}
    size_t size(void) const {return(Bytes);}
  };
+
+ // Per-sample weight gradients of a convolution layer that were asked for and not computed.  The reference's layer
+ // (netlayer/cnetlayerconvolution.cu.h:501-508) fills a [B,1,Kamt,C*Ky*Kx] tensor with zeros, has
+ // CreateDeltaWeightAndBias add every sample's gradient into its slice and then sums the slices with AddSumW: at
+ // 512 kernels of 256x4x4 and a batch of 128 that tensor is 1 GiB, written twice and read twice per step, to obtain
+ // 8 MiB.  The drop-in classes defer the three steps: Fill(0) of a batch tensor only marks it, CreateDeltaWeightAndBias
+ // on two marked tensors computes the sums over the batch directly (mt_convolution_backward_weights_sum) and keeps
+ // copies of its two operands, AddSumW of such a tensor adds the sum.  Whoever reads the per-sample gradients in any
+ // other way gets them: they are then computed from the kept operands (CTensor::Materialise).
+ struct CDeferredGradient
+ {
+  CDeviceBuffer Image;///<the operands as they were when the gradients were asked for
+  CDeviceBuffer Delta;
+  mt_tensor ImageTensor;
+  mt_tensor DeltaTensor;
+  int32_t Kernel_X,Kernel_Y,Kernel_Z,Stride_X,Stride_Y,Padding_X,Padding_Y;
+  uint32_t Kernel_Amount;
+  uint32_t KernelSize[4];///<sizes of the two per-sample tensors when the gradients were asked for
+  uint32_t BiasSize[4];
+  CDeviceBuffer KernelSum;///<[1,Z,Y,X] of the kernel tensor: the sum over the batch
+  CDeviceBuffer BiasSum;
+ };
+ // switch for the deferral (on by default): with `false` every call runs when it is made
+ inline bool& DeferGradients(void)
+ {
+  static bool on=true;
+  return(on);
+ }
 }
 
 template<class type_t> class CTensorMath;
@@ -90,9 +124,15 @@ class CTensor
   mutable mi355::CDeviceBuffer DeviceItem;
   mutable bool HostOnChange;
   mutable bool DeviceOnChange;
+  // What the device copy holds when it was not written yet (mi355::CDeferredGradient): while Lazy is not LAZY_NONE the
+  // device copy is the current one (DeviceOnChange) and every access goes through Materialise() first.
+  enum {LAZY_NONE=0,LAZY_ZERO,LAZY_GRADIENT_KERNEL,LAZY_GRADIENT_BIAS};
+  mutable uint8_t Lazy;
+  mutable std::shared_ptr<mi355::CDeferredGradient> Deferred;
  public:
   CTensor(uint32_t size_w=1,uint32_t size_z=1,uint32_t size_y=1,uint32_t size_x=1)
   {
+   Lazy=LAZY_NONE;
    Size_X=size_x;Size_Y=size_y;Size_Z=size_z;Size_W=size_w;
    BasedSize_X=Size_X;BasedSize_Y=Size_Y;BasedSize_Z=Size_Z;BasedSize_W=Size_W;
    Item.resize(Count());
@@ -102,12 +142,10 @@ class CTensor
   }
   CTensor(const CTensor<type_t> &cTensor)
   {
-   Item=cTensor.Item;
-   DeviceItem=cTensor.DeviceItem;
+   Lazy=LAZY_NONE;
+   CopyValues(cTensor);
    Size_X=cTensor.Size_X;Size_Y=cTensor.Size_Y;Size_Z=cTensor.Size_Z;Size_W=cTensor.Size_W;
    BasedSize_X=Size_X;BasedSize_Y=Size_Y;BasedSize_Z=Size_Z;BasedSize_W=Size_W;
-   HostOnChange=cTensor.HostOnChange;
-   DeviceOnChange=cTensor.DeviceOnChange;
   }
   ~CTensor() {}
  public:
@@ -160,6 +198,8 @@ class CTensor
   void Move(CTensor<type_t> &cTensor)
   {
    if (this==&cTensor) return;
+   cTensor.Materialise();
+   DropLazy();
    Item=std::move(cTensor.Item);
    DeviceItem.swap(cTensor.DeviceItem);
    Size_X=cTensor.Size_X;Size_Y=cTensor.Size_Y;Size_Z=cTensor.Size_Z;Size_W=cTensor.Size_W;
@@ -189,6 +229,7 @@ class CTensor
   void CopyItemToDevice(type_t *item_array,uint32_t size)
   {
    if (Item.size()<size) throw("CTensor::CopyItemToDevice: array larger than the tensor");
+   Materialise();
    CopyToDevice();
    mi355::Check(mt_copy_h2d(DeviceItem.get(),item_array,size*sizeof(type_t)));
    SetDeviceOnChange();
@@ -205,6 +246,7 @@ class CTensor
   {
    size_t offset=static_cast<size_t>(w)*Size_X*Size_Y*Size_Z;
    if (Item.size()<size+offset) throw("CTensor::CopyItemLayerWToDevice: array larger than the tensor");
+   Materialise();
    CopyToDevice();
    mi355::Check(mt_copy_h2d(static_cast<type_t*>(DeviceItem.get())+offset,item_array,size*sizeof(type_t)));
    SetDeviceOnChange();
@@ -213,12 +255,9 @@ class CTensor
   {
    if (this!=&cTensor)
    {
-    Item=cTensor.Item;
-    DeviceItem=cTensor.DeviceItem;
+    CopyValues(cTensor);
     Size_X=cTensor.Size_X;Size_Y=cTensor.Size_Y;Size_Z=cTensor.Size_Z;Size_W=cTensor.Size_W;
     BasedSize_X=cTensor.BasedSize_X;BasedSize_Y=cTensor.BasedSize_Y;BasedSize_Z=cTensor.BasedSize_Z;BasedSize_W=cTensor.BasedSize_W;
-    HostOnChange=cTensor.HostOnChange;
-    DeviceOnChange=cTensor.DeviceOnChange;
    }
    return(*this);
   }
@@ -256,6 +295,7 @@ class CTensor
     Size_Y=iDataStream_Ptr->LoadUInt32();
     Size_X=iDataStream_Ptr->LoadUInt32();
    }
+   DropLazy();
    Item.assign(Count(),type_t());
    DeviceItem.resize(Item.size()*sizeof(type_t));
    for(size_t n=0;n<Count();n++) Item[n]=static_cast<type_t>(iDataStream_Ptr->LoadDouble());
@@ -306,19 +346,56 @@ class CTensor
   void CopyToDevice(bool force=false) const
   {
    if (HostOnChange==false && force==false) return;
+   DropLazy();
    if (!Item.empty()) mi355::Check(mt_copy_h2d(DeviceItem.get(),&Item[0],Item.size()*sizeof(type_t)));
    HostOnChange=false;
    DeviceOnChange=false;
   }
   void CopyFromDevice(bool force=false) const
   {
+   Materialise();
    if (DeviceOnChange==false && force==false) return;
    if (!Item.empty()) mi355::Check(mt_copy_d2h(&Item[0],DeviceItem.get(),Item.size()*sizeof(type_t)));
    HostOnChange=false;
    DeviceOnChange=false;
   }
   void SetDeviceOnChange(void) const {DeviceOnChange=true;HostOnChange=false;}
-  void SetHostOnChange(void) const {DeviceOnChange=false;HostOnChange=true;}
+  void SetHostOnChange(void) const {DropLazy();DeviceOnChange=false;HostOnChange=true;}
+  // Writes what the device copy was only said to hold: zeros, or the per-sample gradients computed from the operands
+  // that were kept (CreateDeltaWeightAndBias of the reference adds into the zeroed tensor, netlayer/
+  // cnetlayerconvolution.cu.h:503-506; a sample's bias gradient is the sum of its delta over the pixels).
+  void Materialise(void) const
+  {
+   if (Lazy==LAZY_NONE) return;
+   const uint8_t kind=Lazy;
+   std::shared_ptr<mi355::CDeferredGradient> record;
+   record.swap(Deferred);
+   Lazy=LAZY_NONE;
+   mt_tensor own;
+   own.p=static_cast<float*>(DeviceItem.get());
+   own.w=Size_W;own.z=Size_Z;own.y=Size_Y;own.x=Size_X;
+   if (kind==LAZY_ZERO)
+   {
+    mi355::Check(mt_fill(&own,0));
+    return;
+   }
+   const uint32_t *size=(kind==LAZY_GRADIENT_KERNEL)?record->KernelSize:record->BiasSize;
+   own.w=size[0];own.z=size[1];own.y=size[2];own.x=size[3];
+   if (kind==LAZY_GRADIENT_BIAS)
+   {
+    mi355::Check(mt_summ_xy(&own,&record->DeltaTensor));
+    return;
+   }
+   mi355::CDeviceBuffer bias;
+   bias.resize(static_cast<size_t>(record->BiasSize[0])*record->BiasSize[1]*sizeof(float));
+   mt_tensor db;
+   db.p=static_cast<float*>(bias.get());
+   db.w=record->BiasSize[0];db.z=record->BiasSize[1];db.y=1;db.x=1;
+   mi355::Check(mt_fill(&own,0));
+   mi355::Check(mt_fill(&db,0));
+   mi355::Check(mt_create_delta_weight_and_bias(&own,record->Kernel_X,record->Kernel_Y,record->Kernel_Z,record->Kernel_Amount,&db,&record->ImageTensor,&record->DeltaTensor,
+                                                record->Stride_X,record->Stride_Y,record->Padding_X,record->Padding_Y));
+  }
 
   void Print(const std::string &name,bool print_value=true) const
   {
@@ -379,11 +456,40 @@ class CTensor
    return(ret);
   }
  private:
+  // Values and coherence state of another tensor.  Only the side that is current is copied: the layers hand their
+  // errors on with operator= on every step (netlayer/cnetlayerconvolution.cu.h:571), and a host copy that the device
+  // copy has overtaken would cost a memcpy of the whole activation for values nobody may read.
+  void CopyValues(const CTensor<type_t> &cTensor)
+  {
+   cTensor.Materialise();
+   DropLazy();
+   if (cTensor.DeviceOnChange==true)
+   {
+    Item.resize(cTensor.Item.size());
+    DeviceItem=cTensor.DeviceItem;
+   }
+   else if (cTensor.HostOnChange==true)
+   {
+    Item=cTensor.Item;
+    DeviceItem.resize(cTensor.DeviceItem.size());
+   }
+   else
+   {
+    Item=cTensor.Item;
+    DeviceItem=cTensor.DeviceItem;
+   }
+   HostOnChange=cTensor.HostOnChange;
+   DeviceOnChange=cTensor.DeviceOnChange;
+  }
+  void DropLazy(void) const {Lazy=LAZY_NONE;Deferred.reset();}
+  // the device copy is said to hold zeros; nothing is launched (CTensorMath::Fill)
+  void SetLazyZero(void) const {DropLazy();Lazy=LAZY_ZERO;DeviceOnChange=true;HostOnChange=false;}
   size_t Count(void) const {return(static_cast<size_t>(Size_X)*Size_Y*Size_Z*Size_W);}
   size_t Index(uint32_t w,uint32_t z,uint32_t y,uint32_t x) const {return(x+static_cast<size_t>(Size_X)*(y+static_cast<size_t>(Size_Y)*(z+static_cast<size_t>(Size_Z)*w)));}
   // descriptor of the device copy for the C ABI; `upload` first brings the device copy up to date
   mt_tensor Device(bool upload) const
   {
+   Materialise();
    if (upload==true) CopyToDevice();
    mt_tensor t;
    t.p=static_cast<float*>(DeviceItem.get());

@@ -11,6 +11,19 @@ class CTensorConv
 {
  private:
   static void OnlyFloat(void) {static_assert(std::is_same<type_t,float>::value,"the MI355X tensor path computes in fp32 only");}
+  // Whether CreateDeltaWeightAndBias may keep the per-sample gradients uncomputed (mi355::CDeferredGradient): both
+  // tensors were zeroed and not touched since, one slice per sample of the batch, the bias gradient [B,Kamt,1,1], and
+  // the gradients are at least four times the operands (keeping copies of those must be the cheaper side).
+  static bool Deferrable(const CTensor<type_t> &dkernel,const CTensor<type_t> &dbias,const CTensor<type_t> &image,const CTensor<type_t> &delta)
+  {
+   if (mi355::DeferGradients()==false) return(false);
+   if (dkernel.Lazy!=CTensor<type_t>::LAZY_ZERO || dbias.Lazy!=CTensor<type_t>::LAZY_ZERO || &dkernel==&dbias) return(false);
+   const uint32_t batch=dkernel.GetSizeW();
+   if (batch<2 || dbias.GetSizeW()!=batch || image.GetSizeW()!=batch || delta.GetSizeW()!=batch) return(false);
+   if (dbias.GetSizeY()!=1 || dbias.GetSizeX()!=1) return(false);
+   const size_t gradients=dkernel.Count(),operands=image.Count()+delta.Count();
+   return(gradients>=(static_cast<size_t>(1)<<20) && gradients>=4*operands);
+  }
  public:
   static void ForwardConvolution(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Image,const CTensor<type_t> &cTensor_Kernel,int32_t kernel_x,int32_t kernel_y,int32_t kernel_z,uint32_t kernel_amount,const CTensor<type_t> &cTensor_Bias,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)
   {
@@ -29,6 +42,37 @@ class CTensorConv
   static void CreateDeltaWeightAndBias(CTensor<type_t> &cTensor_dKernel,int32_t dkernel_x,int32_t dkernel_y,int32_t dkernel_z,uint32_t dkernel_amount,CTensor<type_t> &cTensor_dBias,const CTensor<type_t> &cTensor_Image,CTensor<type_t> &cTensor_Delta,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)
   {
    OnlyFloat();
+   if (Deferrable(cTensor_dKernel,cTensor_dBias,cTensor_Image,cTensor_Delta)==true)
+   {
+    // Two zeroed per-sample tensors: the sums over the batch now, from the operands as they are; copies of the operands
+    // for whoever reads a sample's gradient later (mi355::CDeferredGradient).
+    std::shared_ptr<mi355::CDeferredGradient> record(new mi355::CDeferredGradient);
+    mt_tensor i=cTensor_Image.Device(true),d=cTensor_Delta.Device(true);
+    record->Kernel_X=dkernel_x;record->Kernel_Y=dkernel_y;record->Kernel_Z=dkernel_z;record->Kernel_Amount=dkernel_amount;
+    record->Stride_X=stride_x;record->Stride_Y=stride_y;record->Padding_X=padding_x;record->Padding_Y=padding_y;
+    const CTensor<type_t> *batch[2]={&cTensor_dKernel,&cTensor_dBias};
+    uint32_t *size[2]={record->KernelSize,record->BiasSize};
+    mi355::CDeviceBuffer *sum[2]={&record->KernelSum,&record->BiasSum};
+    mt_tensor total[2];
+    for(int n=0;n<2;n++)
+    {
+     size[n][0]=batch[n]->GetSizeW();size[n][1]=batch[n]->GetSizeZ();size[n][2]=batch[n]->GetSizeY();size[n][3]=batch[n]->GetSizeX();
+     sum[n]->resize(static_cast<size_t>(size[n][1])*size[n][2]*size[n][3]*sizeof(float));
+     total[n].p=static_cast<float*>(sum[n]->get());
+     total[n].w=1;total[n].z=size[n][1];total[n].y=size[n][2];total[n].x=size[n][3];
+     mi355::Check(mt_fill(&total[n],0));
+    }
+    // the summed kernel gradient is addressed as [1,1,Kamt,C*Ky*Kx] whatever Z x Y split the layer gave its tensor
+    total[0].y*=total[0].z;total[0].z=1;
+    mi355::Check(mt_convolution_backward_weights_sum(&total[0],dkernel_x,dkernel_y,dkernel_z,dkernel_amount,&total[1],&i,&d,stride_x,stride_y,padding_x,padding_y));
+    record->Image.assign(i.p,static_cast<size_t>(i.w)*i.z*i.y*i.x*sizeof(float));
+    record->Delta.assign(d.p,static_cast<size_t>(d.w)*d.z*d.y*d.x*sizeof(float));
+    record->ImageTensor=i;record->ImageTensor.p=static_cast<float*>(record->Image.get());
+    record->DeltaTensor=d;record->DeltaTensor.p=static_cast<float*>(record->Delta.get());
+    cTensor_dKernel.Lazy=CTensor<type_t>::LAZY_GRADIENT_KERNEL;cTensor_dKernel.Deferred=record;
+    cTensor_dBias.Lazy=CTensor<type_t>::LAZY_GRADIENT_BIAS;cTensor_dBias.Deferred=record;
+    return;
+   }
    // both gradients accumulate: bring their device copies up to date first
    mt_tensor dk=cTensor_dKernel.Device(true),db=cTensor_dBias.Device(true),i=cTensor_Image.Device(true),d=cTensor_Delta.Device(true);
    mi355::Check(mt_create_delta_weight_and_bias(&dk,dkernel_x,dkernel_y,dkernel_z,dkernel_amount,&db,&i,&d,stride_x,stride_y,padding_x,padding_y));

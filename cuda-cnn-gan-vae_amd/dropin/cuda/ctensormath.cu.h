@@ -32,6 +32,13 @@ class CTensorMath
   static void Fill(CTensor<type_t> &cTensor_Output,type_t value=0)
   {
    OnlyFloat();
+   cTensor_Output.DropLazy();   // whatever the tensor was said to hold is overwritten
+   if (value==0 && cTensor_Output.GetSizeW()>1 && mi355::DeferGradients()==true)
+   {
+    // zeros for a tensor with a batch axis: written when somebody asks for them (mi355::CDeferredGradient)
+    cTensor_Output.SetLazyZero();
+    return;
+   }
    mt_tensor o=cTensor_Output.Device(false);
    mi355::Check(mt_fill(&o,value));
    cTensor_Output.SetDeviceOnChange();
@@ -66,6 +73,20 @@ class CTensorMath
   static void AddSumW(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
   {
    OnlyFloat();
+   if (&cTensor_Right!=&cTensor_Output && &cTensor_Right!=&cTensor_Left &&
+       (cTensor_Right.Lazy==CTensor<type_t>::LAZY_GRADIENT_KERNEL || cTensor_Right.Lazy==CTensor<type_t>::LAZY_GRADIENT_BIAS))
+   {
+    // per-sample gradients that were not computed: their sum over the batch was, and is a one-sample tensor
+    const std::shared_ptr<mi355::CDeferredGradient> record=cTensor_Right.Deferred;
+    const bool kernel=(cTensor_Right.Lazy==CTensor<type_t>::LAZY_GRADIENT_KERNEL);
+    mt_tensor r;
+    r.p=static_cast<float*>(kernel?record->KernelSum.get():record->BiasSum.get());
+    r.w=1;r.z=cTensor_Right.GetSizeZ();r.y=cTensor_Right.GetSizeY();r.x=cTensor_Right.GetSizeX();
+    mt_tensor l=cTensor_Left.Device(true),o=cTensor_Output.Device(false);
+    mi355::Check(mt_add_sum_w(&o,&l,&r,left_scale,right_scale));
+    cTensor_Output.SetDeviceOnChange();
+    return;
+   }
    mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
    mi355::Check(mt_add_sum_w(&o,&l,&r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();

@@ -82,13 +82,13 @@ def write_batchnorm_layer(f, beta, gamma, mean, variable, momentum):
 # Whole networks.  CModelMain::SaveNetLayers (cuda/netmodel/cmodelmain.cu.h:296-300) calls Save() of every layer in
 # order, with nothing between them; what the other layer kinds write:
 #     function                 uint32 id of netlayer/neuron.cu.h:21-26 (not the id of the tensor-level function)
-#     up-sampling, max pooling, average pooling      2 x uint32 (x, y)
+#     up-sampling, max pooling, max de-pooling, average pooling      2 x uint32 (x, y)
 #     drop-out                 one double
 #     input, time embedding, concatenator, splitter, VAE coder output, soft-max      nothing
 NEURON_FUNCTION = {"sigmoid": 0, "relu": 1, "leaky_relu": 2, "linear": 3, "tangence": 4, "gelu": 5}
 _NEURON_NAME = {v: k for k, v in NEURON_FUNCTION.items()}
 _EMPTY = ("input", "time_embedding", "concatenator", "splitter", "vae_coder_output", "softmax")
-_PAIR = ("upsampling", "maxpooling", "averagepooling")
+_PAIR = ("upsampling", "maxpooling", "maxdepooling", "averagepooling")
 
 
 def _take(f, fmt, what):
@@ -184,3 +184,38 @@ def read_training_params(f, kinds):
         else:
             raise ValueError("unknown layer kind " + repr(kind))
     return iteration, out
+
+
+# Averaged weights.  CModelMain::SaveNetLayersEMAWeight (cuda/netmodel/cmodelmain.cu.h:332-336) calls SaveEMAWeight() of
+# every layer in order (backwards through the vector when asked to), and every layer writes the record of its Save()
+# with the averaged tensors in place of the trained ones: convolution / transposed convolution the eight header values,
+# Kernel_EMA, Bias_EMA (netlayer/cnetlayerconvolution.cu.h:679-692); linear W_EMA, B_EMA (cnetlayerlinear.cu.h:590-595);
+# batch normalisation Beta_EMA, Gamma_EMA, Mean_EMA, Variable_EMA and the momentum (cnetlayerbatchnormalization.cu.h:
+# 770-778); the other kinds what their Save() writes.  A layer whose averaging was never enabled holds [1,1,1,1] tensors
+# there (EnableEMA(false), the constructors' state) and writes those.  TrainingUpdateWeight blends
+# ema = EMA_K * ema + (1 - EMA_K) * weight with EMA_K = 0.999 (netlayer/inetlayer.cu.h:67) after every step.
+EMA_K = 0.999
+
+
+def write_ema(f, layers, backward=False):
+    """`layers` as write_net takes them, the tensor fields holding the averaged weights."""
+    write_net(f, list(reversed(layers)) if backward else layers)
+
+
+def read_ema(f, kinds, backward=False):
+    """Returns the layers in network order, whichever way the stream was written."""
+    if not backward:
+        return read_net(f, kinds)
+    return list(reversed(read_net(f, list(reversed(kinds)))))
+
+
+def ema_disabled(kind):
+    """The fields a layer of this kind writes when its averaging was never enabled (for write_ema)."""
+    one = np.zeros((1, 1, 1, 1), np.float32)
+    if kind in ("convolution", "backconvolution"):
+        return {"kernel": one, "bias": one}
+    if kind == "linear":
+        return {"weight": one, "bias": one}
+    if kind == "batchnorm":
+        return {"beta": one, "gamma": one, "mean": one, "variable": one}
+    return {}

@@ -18,10 +18,17 @@
 //          SetTimeStep exist in the reference's GPU tensor class only)
 // Chain F: input [B,4,8,8]   -> Linear function -> MaxPooling 2x2, forward and backward           (layers_mi355 only: the layer names the
 //          position type CTensorMath<type_t>::SPos, which the CPU class does not nest)
+// Chain H: the layers that work element by element on the host through GetElement/SetElement: SoftMax; Splitter with two
+//          consumers; DropOut and VAECoderOutput (both draw from std::random_device: the test recovers mask and noise
+//          from the outputs and checks the rest against them); MaxDePooling
+// "time" as the second argument (layers_mi355 only): the DCGAN-64 generator's forward pass at batch 256 and the
+//          discriminator's training step at batch 128 on the reference's layer classes, timed with the drop-in CTimeStamp
 // Each chain: TrainingStart, Forward, SetOutputError, TrainingBackward, TrainingUpdateWeight (gradient descent), Save.
+// SYSTEM::PutMessage* come from the reference's own system/system.cpp, compiled beside this file.
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 #include <algorithm>
 #include <memory>
@@ -34,6 +41,7 @@
 #include "cuda/tensor.cu.h"   // with USE_CPU this is the reference's cpu/tensor.h
 #else
 #include "cuda/tensor.cu.h"   // the drop-in, found first on the include path
+#include "cuda/ctimestamp.cu.h"
 #endif
 
 #include "netlayer/cnetlayerconvolutioninput.cu.h"
@@ -48,24 +56,19 @@
 #include "netlayer/cnetlayerconcatenator.cu.h"
 #include "netlayer/cnetlayertimeembedding.cu.h"
 #include "netlayer/cnetlayermaxpooling.cu.h"
-// the remaining layers are only compiled: every member function of each is instantiated on the drop-in classes
+#endif
 #include "netlayer/cnetlayermaxdepooling.cu.h"
 #include "netlayer/cnetlayerdropout.cu.h"
 #include "netlayer/cnetlayersplitter.cu.h"
 #include "netlayer/cnetlayervaecoderoutput.cu.h"
 #include "netlayer/cnetlayersoftmax.cu.h"
+// every member function of each, also those no chain calls
 template class CNetLayerMaxDePooling<float>;
 template class CNetLayerDropOut<float>;
 template class CNetLayerSplitter<float>;
 template class CNetLayerVAECoderOutput<float>;
 template class CNetLayerSoftMax<float>;
-#endif
 
-namespace SYSTEM
-{
- void PutMessage(const std::string &) {}
- void PutMessageToConsole(const std::string &) {}
-}
 // the reference's IDataStream declares a file factory that nothing here calls
 #ifdef USE_CPU
 IDataStream* IDataStream::CreateNewDataStreamFile(std::string,bool) {return(NULL);}
@@ -212,6 +215,12 @@ static void ChainA(void)
  FillTensor(image,1.0);
  input.SetOutput(image);
  INetLayer<type_t> *layers[5]={&input,&conv,&f1,&lin,&f2};
+ DumpStream("A.conv_loaded",conv_w,8*sizeof(int32_t),2);
+ DumpStream("A.linear_loaded",lin_w,0,2);
+ CMemoryStream ema_off;   // averaged weights of a network that never enabled them
+ for(int n=0;n<5;n++) layers[n]->SaveEMAWeight(&ema_off);
+ DumpRaw("A.ema_off_stream",ema_off);
+ for(int n=0;n<5;n++) layers[n]->EnableEMA(true);   // the averages start as copies of the loaded weights
  for(int n=0;n<5;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
  for(int n=0;n<5;n++) layers[n]->Forward();
  Dump("A.conv",conv.GetOutputTensor());
@@ -237,6 +246,21 @@ static void ChainA(void)
  CMemoryStream net_saved;   // the whole chain, layer after layer, as CModelMain::SaveNetLayers writes a network
  for(int n=0;n<5;n++) layers[n]->Save(&net_saved);
  DumpRaw("A.net_stream",net_saved);
+ CMemoryStream ema_saved;   // the averaged weights after one update, layer after layer, as CModelMain::SaveNetLayersEMAWeight writes them
+ for(int n=0;n<5;n++) layers[n]->SaveEMAWeight(&ema_saved);
+ DumpRaw("A.ema_stream",ema_saved);
+ {
+  CMemoryStream conv_ema,lin_ema;
+  conv.SaveEMAWeight(&conv_ema);
+  lin.SaveEMAWeight(&lin_ema);
+  DumpStream("A.conv_ema",conv_ema,8*sizeof(int32_t),2);
+  DumpStream("A.linear_ema",lin_ema,0,2);
+ }
+ // forward with the averaged weights
+ for(int n=0;n<5;n++) layers[n]->SetUseEMA(true);
+ for(int n=0;n<5;n++) layers[n]->Forward();
+ Dump("A.sigmoid_ema",f2.GetOutputTensor());
+ for(int n=0;n<5;n++) layers[n]->SetUseEMA(false);
  // known Adam moments into the convolution layer (this chain steps by plain gradient descent, its own moments are zero)
  CMemoryStream moments;
  const std::vector<double> mk=Values(8*48,0.3),vk=Values(8*48,0.2),mb=Values(8,0.3),vb=Values(8,0.2);
@@ -317,6 +341,137 @@ static void ChainD(void)
  DumpRaw("D.net_stream",net_saved);
 }
 
+
+// Chain H: layers that work on the host, element by element
+static void ChainH(void)
+{
+ // soft-max over all elements of a sample, forward and the full Jacobian backward
+ {
+  CNetLayerConvolutionInput<type_t> input(2,3,4,BATCH);
+  CNetLayerFunction<type_t> pass(NNeuron::NEURON_FUNCTION_LINEAR,&input,BATCH);
+  CNetLayerSoftMax<type_t> soft(&pass,BATCH);
+  CTensor<type_t> x(BATCH,2,3,4);
+  FillTensor(x,2.0);
+  input.SetOutput(x);
+  INetLayer<type_t> *layers[3]={&input,&pass,&soft};
+  for(int n=0;n<3;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+  for(int n=0;n<3;n++) layers[n]->Forward();
+  Dump("H.soft_input",x);
+  Dump("H.softmax",soft.GetOutputTensor());
+  CTensor<type_t> error(BATCH,2,3,4);
+  FillTensor(error,0.5);
+  Dump("H.soft_error",error);
+  soft.SetOutputError(error);
+  soft.TrainingBackward(true);
+  Dump("H.soft_delta",pass.GetDeltaTensor());
+ }
+ // splitter with two consumers: the output is the input, the errors of both consumers add up
+ {
+  CNetLayerConvolutionInput<type_t> input(3,4,4,BATCH);
+  CNetLayerFunction<type_t> pass(NNeuron::NEURON_FUNCTION_LINEAR,&input,BATCH);
+  CNetLayerSplitter<type_t> split(2,&pass,BATCH);
+  CNetLayerFunction<type_t> branch_a(NNeuron::NEURON_FUNCTION_LINEAR,&split,BATCH),branch_b(NNeuron::NEURON_FUNCTION_TANGENCE,&split,BATCH);
+  CTensor<type_t> x(BATCH,3,4,4);
+  FillTensor(x,1.0);
+  input.SetOutput(x);
+  INetLayer<type_t> *layers[5]={&input,&pass,&split,&branch_a,&branch_b};
+  for(int n=0;n<5;n++) layers[n]->Forward();   // the splitter's training tensors are copies of its output
+  for(int n=0;n<5;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+  for(int n=0;n<5;n++) layers[n]->Forward();
+  Dump("H.split_input",x);
+  Dump("H.split_output",split.GetOutputTensor());
+  Dump("H.split_tanh",branch_b.GetOutputTensor());
+  CTensor<type_t> error_a(BATCH,3,4,4),error_b(BATCH,3,4,4);
+  FillTensor(error_a,0.5);
+  FillTensor(error_b,0.5);
+  Dump("H.split_error_a",error_a);
+  Dump("H.split_error_b",error_b);
+  branch_a.SetOutputError(error_a);
+  branch_b.SetOutputError(error_b);
+  branch_a.TrainingBackward(true);
+  branch_b.TrainingBackward(true);
+  Dump("H.split_delta",split.GetDeltaTensor());
+  split.TrainingBackward(true);
+  Dump("H.split_prev_delta",pass.GetDeltaTensor());
+ }
+ // drop-out: the mask comes from std::random_device
+ {
+  CNetLayerConvolutionInput<type_t> input(4,8,8,BATCH);
+  CNetLayerFunction<type_t> pass(NNeuron::NEURON_FUNCTION_LINEAR,&input,BATCH);
+  CNetLayerDropOut<type_t> drop(0.25,&pass,BATCH);
+  CTensor<type_t> x(BATCH,4,8,8);
+  FillTensor(x,1.0);
+  input.SetOutput(x);
+  INetLayer<type_t> *layers[3]={&input,&pass,&drop};
+  for(int n=0;n<3;n++) layers[n]->Forward();
+  Dump("H.drop_inference",drop.GetOutputTensor());   // not training: the layer hands its input through
+  for(int n=0;n<3;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+  for(int n=0;n<3;n++) layers[n]->Forward();
+  Dump("H.drop_input",x);
+  Dump("H.drop_output",drop.GetOutputTensor());
+  CTensor<type_t> error(BATCH,4,8,8);
+  FillTensor(error,0.5);
+  Dump("H.drop_error",error);
+  drop.SetOutputError(error);
+  drop.TrainingBackward(true);
+  Dump("H.drop_prev_delta",pass.GetDeltaTensor());
+  CMemoryStream saved;
+  drop.Save(&saved);
+  DumpRaw("H.drop_stream",saved);
+ }
+ // output of a VAE coder: mu + exp(logvar/2)*noise, the noise from std::random_device; Kullback-Leibler terms in the error
+ {
+  CNetLayerConvolutionInput<type_t> input_mu(1,16,1,BATCH),input_logvar(1,16,1,BATCH);
+  CNetLayerFunction<type_t> mu(NNeuron::NEURON_FUNCTION_LINEAR,&input_mu,BATCH),logvar(NNeuron::NEURON_FUNCTION_LINEAR,&input_logvar,BATCH);
+  CNetLayerVAECoderOutput<type_t> coder(0.125f,&mu,&logvar,BATCH);
+  CTensor<type_t> m(BATCH,1,16,1),l(BATCH,1,16,1);
+  FillTensor(m,1.0);
+  FillTensor(l,12.0);   // beyond the clamp at +-10 in places
+  input_mu.SetOutput(m);
+  input_logvar.SetOutput(l);
+  INetLayer<type_t> *layers[5]={&input_mu,&input_logvar,&mu,&logvar,&coder};
+  for(int n=0;n<5;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+  for(int n=0;n<5;n++) layers[n]->Forward();
+  Dump("H.vae_mu",m);
+  Dump("H.vae_logvar",l);
+  Dump("H.vae_output",coder.GetOutputTensor());
+  CTensor<type_t> error(BATCH,1,16,1);
+  FillTensor(error,0.5);
+  Dump("H.vae_error",error);
+  coder.SetOutputError(error);   // the Kullback-Leibler weight is 0 until iteration 6
+  Dump("H.vae_delta_mu0",mu.GetDeltaTensor());
+  Dump("H.vae_delta_logvar0",logvar.GetDeltaTensor());
+  coder.TrainingUpdateWeight(0.05,6);
+  coder.SetOutputError(error);
+  Dump("H.vae_delta_mu",mu.GetDeltaTensor());
+  Dump("H.vae_delta_logvar",logvar.GetDeltaTensor());
+ }
+ // max de-pooling: every input element fills its block; backward through the layer
+ {
+  CNetLayerConvolutionInput<type_t> input(3,4,4,BATCH);
+  CNetLayerFunction<type_t> pass(NNeuron::NEURON_FUNCTION_LINEAR,&input,BATCH);
+  CNetLayerMaxDePooling<type_t> depool(2,3,&pass,BATCH);
+  CTensor<type_t> x(BATCH,3,4,4);
+  FillTensor(x,1.0);
+  input.SetOutput(x);
+  INetLayer<type_t> *layers[3]={&input,&pass,&depool};
+  for(int n=0;n<3;n++) layers[n]->Forward();
+  for(int n=0;n<3;n++) {layers[n]->TrainingStart();layers[n]->TrainingResetDeltaWeight();}
+  for(int n=0;n<3;n++) layers[n]->Forward();
+  Dump("H.depool_input",x);
+  Dump("H.depool_output",depool.GetOutputTensor());
+  CTensor<type_t> error(BATCH,3,8,12);
+  FillTensor(error,0.5);
+  Dump("H.depool_error",error);
+  depool.SetOutputError(error);
+  depool.TrainingBackward(true);
+  Dump("H.depool_prev_delta",pass.GetDeltaTensor());
+  CMemoryStream saved;
+  depool.Save(&saved);
+  DumpRaw("H.depool_stream",saved);
+ }
+}
+
 #ifndef USE_CPU
 // Chain E: layers whose tensor functions exist in the GPU class only: two inputs -> Concatenator -> TimeEmbedding
 static void ChainE(void)
@@ -363,6 +518,120 @@ static void ChainF(void)
  Dump("F.prev_error",pass.GetDeltaTensor());
 }
 
+
+// Timing of the unchanged layer classes on the drop-in tensors at the sizes of the two networks the library is tuned
+// for; CTimeStamp (the reference's own scope timer, here the drop-in's) prints each figure through SYSTEM::PutMessageToConsole
+// and CCUDATimeSpent returns it.  One JSON line per chain on stdout.
+static void LoadConvolutionWeights(INetLayer<type_t> &layer,uint32_t rows,uint32_t amount_field,int32_t size,int32_t depth_field,uint32_t columns,uint32_t biases,double scale)
+{
+ CMemoryStream w;
+ w.SaveUInt32(amount_field);w.SaveInt32(size);w.SaveInt32(size);w.SaveInt32(depth_field);w.SaveInt32(2);w.SaveInt32(2);w.SaveInt32(1);w.SaveInt32(1);
+ w.PutTensor(1,1,rows,columns,Values(static_cast<size_t>(rows)*columns,scale));
+ w.PutTensor(1,biases,1,1,std::vector<double>(biases,0.0));
+ layer.Load(&w);
+}
+
+static double TimeSteps(const char *name,std::vector<INetLayer<type_t>*> &net,CTensor<type_t> *error,uint32_t warmup,uint32_t steps)
+{
+ double ms=0;
+ for(uint32_t pass=0;pass<2;pass++)
+ {
+  const uint32_t count=(pass==0)?warmup:steps;
+  CCUDATimeSpent timer;
+  timer.Start();
+  {
+   CTimeStamp stamp(std::string(name)+(pass==0?" (warm-up): ":": "),true);
+   for(uint32_t step=0;step<count;step++)
+   {
+    for(size_t n=0;n<net.size();n++) net[n]->Forward();
+    if (error==NULL) continue;
+    for(size_t n=0;n<net.size();n++) net[n]->TrainingResetDeltaWeight();
+    net[net.size()-1]->SetOutputError(*error);
+    for(size_t n=net.size()-1;n>=1;n--) net[n]->TrainingBackward(true);
+    for(size_t n=1;n<net.size();n++) net[n]->TrainingUpdateWeight(0.0002,step+1);
+   }
+  }
+  ms=timer.Stop();
+ }
+ return(ms/steps);
+}
+
+// DCGAN-64 generator, forward pass in training mode (batch statistics), batch 256
+static void TimeGenerator(uint32_t batch,uint32_t warmup,uint32_t steps)
+{
+ static const uint32_t channels[5]={512,256,128,64,3};
+ std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
+ std::vector<INetLayer<type_t>*> net;
+#define PUSH(LAYER) {owner.push_back(std::shared_ptr<INetLayer<type_t> >(LAYER));net.push_back(owner.back().get());}
+ PUSH(new CNetLayerLinear<type_t>(100,NULL,batch));
+ PUSH(new CNetLayerLinear<type_t>(channels[0]*16,net.back(),batch));
+ {
+  CMemoryStream w;
+  w.PutTensor(1,1,channels[0]*16,100,Values(channels[0]*16*100,0.02));
+  w.PutTensor(1,1,channels[0]*16,1,std::vector<double>(channels[0]*16,0.0));
+  net.back()->Load(&w);
+ }
+ for(uint32_t i=0;i<4;i++)
+ {
+  PUSH(new CNetLayerBatchNormalization<type_t>(0.9f,net.back(),batch));
+  net.back()->Reset();
+  PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_RELU,net.back(),batch));
+  // the first transposed convolution takes the vector as [512,4,4]: it remembers the shape it was constructed on and
+  // reinterprets its input to it in every Forward (netlayer/cnetlayerbackconvolution.cu.h:305-315)
+  if (i==0) net.back()->GetOutputTensor().ReinterpretSize(batch,channels[0],4,4);
+  INetLayer<type_t> *function=net.back();
+  PUSH(new CNetLayerBackConvolution<type_t>(4,channels[i+1],2,2,1,1,net.back(),batch));
+  if (i==0) function->GetOutputTensor().ReinterpretSize(batch,1,channels[0]*16,1);
+  LoadConvolutionWeights(*net.back(),channels[i],channels[i],4,channels[i+1],channels[i+1]*16,channels[i],0.02);
+ }
+ PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_TANGENCE,net.back(),batch));
+ CTensor<type_t> latent(batch,1,100,1);
+ FillTensor(latent,1.0);
+ net[0]->SetOutput(latent);
+ for(size_t n=0;n<net.size();n++) net[n]->TrainingStart();
+ double ms=TimeSteps("generator forward",net,NULL,warmup,steps);
+ CTensor<type_t> &image=net.back()->GetOutputTensor();
+ double sum=0;
+ for(uint32_t x=0;x<64;x++) sum+=fabs(image.GetElement(batch-1,2,63,x));
+ printf("{\"chain\": \"dcgan64_generator_forward\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"last_row_abs_sum\": %.6f}\n",
+        batch,steps,ms,image.GetSizeW(),image.GetSizeZ(),image.GetSizeY(),image.GetSizeX(),sum);
+}
+
+// DCGAN-64 discriminator, whole training step (forward, backward with weight gradients, Adam), batch 128
+static void TimeDiscriminator(uint32_t batch,uint32_t warmup,uint32_t steps)
+{
+ static const uint32_t channels[5]={3,64,128,256,512};
+ std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
+ std::vector<INetLayer<type_t>*> net;
+ PUSH(new CNetLayerConvolutionInput<type_t>(3,64,64,batch));
+ for(uint32_t i=0;i<4;i++)
+ {
+  PUSH(new CNetLayerConvolution<type_t>(channels[i+1],4,2,2,1,1,net.back(),batch));
+  LoadConvolutionWeights(*net.back(),channels[i+1],channels[i+1],4,channels[i],channels[i]*16,channels[i+1],0.02);
+  PUSH(new CNetLayerBatchNormalization<type_t>(0.9f,net.back(),batch));
+  net.back()->Reset();
+  PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_LEAKY_RELU,net.back(),batch));
+ }
+ PUSH(new CNetLayerLinear<type_t>(1,net.back(),batch));
+ {
+  CMemoryStream w;
+  w.PutTensor(1,1,1,512*16,Values(512*16,0.02));
+  w.PutTensor(1,1,1,1,std::vector<double>(1,0.0));
+  net.back()->Load(&w);
+ }
+ PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_SIGMOID,net.back(),batch));
+#undef PUSH
+ CTensor<type_t> image(batch,3,64,64),error(batch,1,1,1);
+ FillTensor(image,1.0);
+ FillTensor(error,0.5);
+ net[0]->SetOutput(image);
+ for(size_t n=0;n<net.size();n++) {net[n]->TrainingModeAdam();net[n]->TrainingStart();}
+ double ms=TimeSteps("discriminator step",net,&error,warmup,steps);
+ CTensor<type_t> &out=net.back()->GetOutputTensor();
+ printf("{\"chain\": \"dcgan64_discriminator_step\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"first\": %.6f}\n",
+        batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),out.GetElement(0,0,0,0));
+}
+
 static void ChainC(void)
 {
  CNetLayerConvolutionInput<type_t> input(4,5,5,BATCH);
@@ -376,6 +645,7 @@ static void ChainC(void)
  w.PutTensor(1,4,5,5,std::vector<double>(100,1.0));
  w.SaveDouble(0.9);
  bn.Load(&w);
+ bn.EnableEMA(true);
  CTensor<type_t> x(BATCH,4,5,5);
  FillTensor(x,2.0);
  input.SetOutput(x);
@@ -404,6 +674,9 @@ static void ChainC(void)
  CMemoryStream bn_trained;
  bn.Save(&bn_trained);
  DumpRaw("C.bn_trained_stream",bn_trained);
+ CMemoryStream bn_ema;
+ bn.SaveEMAWeight(&bn_ema);
+ DumpRaw("C.bn_ema_stream",bn_ema);
  CTensor<type_t> x2(BATCH,4,5,5);
  FillTensor(x2,1.5);
  input.SetOutput(x2);
@@ -450,6 +723,16 @@ int main(int argc,char **argv)
  if (out_file==NULL) return(2);
  try
  {
+#ifndef USE_CPU
+  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up]]
+  {
+   const uint32_t steps=(argc>3)?static_cast<uint32_t>(atoi(argv[3])):50,warmup=(argc>4)?static_cast<uint32_t>(atoi(argv[4])):20;
+   TimeGenerator(256,warmup,steps);
+   TimeDiscriminator(128,warmup,steps);
+   fclose(out_file);
+   return(0);
+  }
+#endif
   if (argc>2)   // only the chain that loads the given network file
   {
    ChainG(argv[2]);
@@ -459,6 +742,7 @@ int main(int argc,char **argv)
   ChainA();
   ChainB();
   ChainD();
+  ChainH();
 #ifndef USE_CPU
   ChainC();
   ChainE();

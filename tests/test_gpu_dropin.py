@@ -24,6 +24,9 @@ LAYERS_GPU = os.path.join(ROOT, "oracle", "_ref", "layers_mi355")
 LAYERS_CPU = os.path.join(ROOT, "oracle", "_ref", "layers_cpu")
 
 
+RANDOM = ("H.drop_output", "H.drop_prev_delta", "H.vae_output", "H.vae_delta_logvar0", "H.vae_delta_logvar")
+
+
 def read_dump(path):
     out, data, pos = {}, open(path, "rb").read(), 0
     while pos < len(data):
@@ -40,7 +43,7 @@ def test_cpp_selftest_on_the_dropin_classes():
     run = subprocess.run([SELFTEST], capture_output=True, text=True, timeout=120)
     print(run.stdout[-3000:], run.stderr[-2000:])
     assert run.returncode == 0 and "ALL PASS" in run.stdout and "FAIL" not in run.stdout
-    assert run.stdout.count("PASS") >= 24
+    assert run.stdout.count("PASS") >= 27
 
 
 @pytest.fixture(scope="module")
@@ -58,7 +61,9 @@ def dumps(tmp_path_factory):
 
 def test_reference_layers_agree_on_both_tensor_paths(dumps):
     gpu, cpu = dumps
-    shared = [k for k in cpu if k in gpu and not k.endswith("_stream")]   # streams are bytes, compared by a test of their own
+    # streams are bytes, compared by tests of their own; drop-out and the VAE coder output draw from std::random_device
+    shared = [k for k in cpu if k in gpu and not k.endswith("_stream") and k not in RANDOM]
+    assert "A.sigmoid_ema" in shared and "H.soft_delta" in shared and "H.split_delta" in shared and "H.depool_prev_delta" in shared
     assert len(shared) >= 16 and any(k.startswith("B.") for k in shared)
     for key in shared:
         assert gpu[key].shape == cpu[key].shape, key
@@ -146,3 +151,35 @@ def test_dropin_layers_load_a_network_written_from_python(oracle, tmp_path):
     leaky, prob = expected_chain_g(oracle, layers, got["G.input"])
     assert rel_err(got["G.leaky"], leaky) <= 1e-4
     assert rel_err(got["G.sigmoid"], prob.reshape(got["G.sigmoid"].shape)) <= 1e-4
+
+
+def test_reference_host_side_layers_on_the_dropin_classes(dumps):
+    """Soft-max, splitter, drop-out, VAE coder output and max de-pooling read and write their tensors element by element
+    (GetElement / SetElement on device-resident drop-in tensors) and mix that with tensor-library calls; the same checks
+    that pin the numpy restatements on the reference's CPU build."""
+    import host_layers
+    gpu, _ = dumps
+    host_layers.check_chain_h({k: v for k, v in gpu.items() if k.startswith("H.")}, tol=1e-5)
+
+
+def test_reference_layers_averaged_weights_on_the_dropin_classes(dumps):
+    """SaveEMAWeight on the drop-in classes: the convolution and linear streams against the CPU build's (same layout, values
+    within rounding), the batch-norm layer's (GPU class only) against EMA_K * loaded + (1 - EMA_K) * trained."""
+    import io
+    import wire_format as wf
+    gpu, cpu = dumps
+    kinds = ["input", "convolution", "function", "linear", "function"]
+    mine, theirs = (wf.read_ema(io.BytesIO(d["A.ema_stream"].tobytes()), kinds) for d in (gpu, cpu))
+    assert mine[1][1]["header"] == theirs[1][1]["header"] and mine[2][1] == theirs[2][1]
+    for i, field in ((1, "kernel"), (1, "bias"), (3, "weight"), (3, "bias")):
+        assert rel_err(mine[i][1][field], theirs[i][1][field]) <= 1e-5, field
+    off = wf.read_ema(io.BytesIO(gpu["A.ema_off_stream"].tobytes()), kinds)
+    assert off[1][1]["kernel"].shape == off[3][1]["weight"].shape == (1, 1, 1, 1)
+    beta, gamma, mean, variable, momentum = wf.read_batchnorm_layer(io.BytesIO(gpu["C.bn_ema_stream"].tobytes()))
+    trained = wf.read_batchnorm_layer(io.BytesIO(gpu["C.bn_trained_stream"].tobytes()))
+    loaded = (gpu["C.beta"], gpu["C.gamma"], np.zeros_like(beta), np.ones_like(beta))
+    assert momentum == trained[4]
+    k = np.float32(wf.EMA_K)
+    for got, w0, w1 in zip((beta, gamma, mean, variable), loaded, trained[:4]):
+        assert np.abs(w1 - w0).max() > 1e-3
+        assert rel_err(got, k * w0 + (np.float32(1) - k) * w1) <= 1e-6

@@ -245,3 +245,55 @@ def test_model_files_keep_the_running_statistics(model):
     # the statistics sit where the reference's layer reads them: third and fourth tensor of a batch-norm layer
     norm = [p for kind, p in wf.read_net(io.BytesIO(first.getvalue()), kinds) if kind == "batchnorm"][0]
     assert np.array_equal(norm["mean"], host["mean0"]) and np.array_equal(norm["variable"], host["variable0"])
+
+
+def test_averaged_weights_written_by_the_reference(cpu_dump):
+    """SaveEMAWeight of every layer of chain A after one update step with averaging enabled: the stream has the layout of
+    the network stream, its tensors are EMA_K * loaded + (1 - EMA_K) * updated (netlayer/cnetlayerconvolution.cu.h:547-551,
+    cnetlayerlinear.cu.h:478-482), and writing them back gives the reference's bytes."""
+    kinds = ["input", "convolution", "function", "linear", "function"]
+    raw = cpu_dump["A.ema_stream"][1]
+    net = wf.read_ema(io.BytesIO(raw), kinds)
+    conv, lin = net[1][1], net[3][1]
+    assert np.array_equal(conv["kernel"], as_array(cpu_dump["A.conv_ema.0"])) and np.array_equal(conv["bias"], as_array(cpu_dump["A.conv_ema.1"]))
+    assert np.array_equal(lin["weight"], as_array(cpu_dump["A.linear_ema.0"])) and np.array_equal(lin["bias"], as_array(cpu_dump["A.linear_ema.1"]))
+    assert net[2][1]["name"] == "leaky_relu" and conv["header"]["kernel_amount"] == 8
+    k, rest = np.float32(wf.EMA_K), np.float32(1.0 - wf.EMA_K)
+    for got, loaded, updated in ((conv["kernel"], "A.conv_loaded.0", "A.conv_updated.0"), (conv["bias"], "A.conv_loaded.1", "A.conv_updated.1"),
+                                 (lin["weight"], "A.linear_loaded.0", "A.linear_updated.0"), (lin["bias"], "A.linear_loaded.1", "A.linear_updated.1")):
+        w0, w1 = as_array(cpu_dump[loaded]), as_array(cpu_dump[updated])
+        assert np.abs(w1 - w0).max() > 1e-4                               # the step moved the weights
+        assert np.array_equal(got, k * w0 + rest * w1), loaded            # rounded product by product, like CTensorMath::Add
+        assert not np.array_equal(got, w0) and not np.array_equal(got, w1)
+    f = io.BytesIO()
+    wf.write_ema(f, net)
+    assert f.getvalue() == raw
+    # written from the last layer to the first (SaveNetLayersEMAWeight with backward = true) and read back in network order
+    f = io.BytesIO()
+    wf.write_ema(f, net, backward=True)
+    assert f.getvalue() != raw and len(f.getvalue()) == len(raw)
+    back = wf.read_ema(io.BytesIO(f.getvalue()), kinds, backward=True)
+    assert [k for k, _ in back] == kinds and np.array_equal(back[3][1]["weight"], lin["weight"])
+
+
+def test_averaged_weights_of_a_network_that_never_enabled_them(cpu_dump):
+    """Before EnableEMA(true) the layers hold [1,1,1,1] tensors in place of the averages and write those."""
+    kinds = ["input", "convolution", "function", "linear", "function"]
+    raw = cpu_dump["A.ema_off_stream"][1]
+    net = wf.read_ema(io.BytesIO(raw), kinds)
+    assert net[1][1]["kernel"].shape == net[1][1]["bias"].shape == net[3][1]["weight"].shape == (1, 1, 1, 1)
+    header = net[1][1]["header"]
+    mine = [("input", {}), ("convolution", dict(wf.ema_disabled("convolution"), header=header)), ("function", {"name": "leaky_relu"}),
+            ("linear", wf.ema_disabled("linear")), ("function", {"name": "sigmoid"})]
+    f = io.BytesIO()
+    wf.write_ema(f, mine)
+    assert f.getvalue() == raw
+
+
+def test_host_side_layers_of_the_reference(cpu_dump):
+    """Soft-max, splitter, drop-out, VAE coder output and max de-pooling of the reference on its CPU tensor classes against
+    the numpy restatements in host_layers.py (which the GPU tests then use on the drop-in build of the same classes)."""
+    import host_layers
+    host_layers.check_chain_h({k: as_array(v) for k, v in cpu_dump.items() if k.startswith("H.")})
+    layers = wf.read_net(io.BytesIO(cpu_dump["H.drop_stream"][1] + cpu_dump["H.depool_stream"][1]), ["dropout", "maxdepooling"])
+    assert layers == [("dropout", {"rate": 0.25}), ("maxdepooling", {"x": 3, "y": 2})]
