@@ -104,7 +104,8 @@ int mt_set_option(const char *name, int value);
 /* More options: "pack_cache" 1 (default) keep re-ordered weights between calls / 0 re-order on every call;
  * "tconv_walk" 1 (default) plain transposed convolutions use the kernel whose blocks walk over the batch wherever the
  * shape allows / 0 never; "walk_blocks", "walk_waves", "walk_tm": grid size, wavefronts per SIMD and accumulators per
- * wavefront of that kernel (measurements); "pool" 1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no wait) /
+ * wavefront of that kernel (measurements); "image_mfma" 0 (default) / 1 the image layer of a generator (at most 4 output
+ * channels) on the 4x4x1 matrix instruction instead of the vector ALU; "pool" 1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no wait) /
  * 0 every mt_free waits for the stream and returns the block to the driver; "pool_limit_mib" bytes the pool may hold.
  * mt_get_info reads counters of the runtime, for tests and measurements (no counterpart in the reference):
  * "pool_bytes", "pool_reused", "driver_allocations", "retired_workspaces", "pack_cache_entries", "pack_cache_valid",
@@ -168,7 +169,12 @@ int mt_apply_func(const mt_tensor *output, const mt_tensor *input, int func);
 
 /* ---- fused entry points -----------------------------------------------------------------------
  * Each one is the exact op sequence of one reference layer's Forward(), lowered to fewer launches.
- * They have no single counterpart function in the reference; the sequence each replaces is cited. */
+ * They have no single counterpart function in the reference; the sequence each replaces is cited.
+ * Numerics of `func`: ReLU, leaky ReLU, linear and GeLU are the arithmetic of mt_apply_func.  Sigmoid and tangence,
+ * where they run at the end of a convolution or transposed-convolution kernel (the image layer of a generator and the
+ * small-channel-count kernels), use the hardware's exponential and reciprocal (v_exp_f32, v_rcp_f32) with the same
+ * clamp at +-30 instead of the library exp and the division of mt_apply_func, and differ from mt_apply_func on the
+ * same input by at most 3e-7 absolute (outputs lie in [-1, 1]). */
 
 /* CNetLayerConvolution::Forward + CNetLayerFunction::Forward (netlayer/cnetlayerconvolution.cu.h:310-322,
  * netlayer/cnetlayerfunction.cu.h:203-213): convolution, bias and activation `func` in one kernel. */
