@@ -1690,6 +1690,10 @@ int &walk_tm() {
   static int v = 1;
   return v;
 }
+int &walk_order() {
+  static int v = -1;
+  return v;
+}
 }  // namespace igemm
 void note_write(const void *p, size_t bytes) {
   if (p == nullptr || bytes == 0) return;
@@ -1737,6 +1741,11 @@ int set_tconv_walk(int v) {
 int set_walk_blocks(int v) {
   if (v < 1 || v > 65536) return fail(MT_E_ARGUMENT, "walk_blocks must be 1..65536");
   igemm::walk_blocks() = v;
+  return MT_OK;
+}
+int set_walk_order(int v) {
+  if (v < -1 || v > 1) return fail(MT_E_ARGUMENT, "walk_order must be -1 (per layer), 0 (batch groups first) or 1 (row tiles first)");
+  igemm::walk_order() = v;
   return MT_OK;
 }
 int set_walk_tm(int v) {

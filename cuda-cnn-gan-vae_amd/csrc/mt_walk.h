@@ -32,6 +32,7 @@ struct WalkArgs {
   uint32_t nphase, tiles_m, M, batch;
   uint32_t px_log, qtiles, groups, per;  // PX = 1 << px_log pixels per tile; pixel tiles per phase; batch groups; steps per block
   uint32_t nk;                           // k steps of one tile (the same for every phase)
+  uint32_t weights_major;                // block order, see tconv_walk_kernel
   const float *delta;                    // [batch][C][H][W]
   const float *scale_shift;              // NORM: [C][H][W][2]
   int in_func;                           // NORM: none, linear, ReLU or leaky ReLU
@@ -58,10 +59,21 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   float *smem = reinterpret_cast<float *>(smem4);
   float *As = smem, *Bs = smem + 2 * BM * LDK;
 
-  uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
-  const uint32_t mt = j % a.tiles_m; j /= a.tiles_m;
-  const uint32_t f = j % a.nphase; j /= a.nphase;
-  const uint32_t qt = j % a.qtiles, g = j / a.qtiles;
+  // An XCD runs a contiguous range of logical blocks.  Ordered by batch group first, the blocks of an XCD share the
+  // samples of a few groups in its L2 and between them read every packed weight.  When the weights of the layer do not
+  // fit an L2 beside the rest (weights_major), the order is by row tile first: an XCD then reads one row tile's weights
+  // (all phases) again and again from its own L2 and streams its share of the input through once; the phases of a
+  // tile stay neighbours, so their stores, which interleave pixel by pixel, still meet in one L2.
+  uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x), mt, f, qt, g;
+  if (a.weights_major) {
+    f = j % a.nphase; j /= a.nphase;
+    qt = j % a.qtiles; j /= a.qtiles;
+    g = j % a.groups; mt = j / a.groups;
+  } else {
+    mt = j % a.tiles_m; j /= a.tiles_m;
+    f = j % a.nphase; j /= a.nphase;
+    qt = j % a.qtiles; g = j / a.qtiles;
+  }
   const TconvPhase &ph = a.ph[f];
   const uint32_t m0 = mt * BM, HW = a.H * a.W, sp = (uint32_t)BN >> a.px_log, px_mask = (1u << a.px_log) - 1u;
 
@@ -364,6 +376,7 @@ __global__ __launch_bounds__(256) void bn_finish_kernel(float *scale_shift, floa
 }
 
 // Whether (and how) a transposed convolution can walk: fills px_log, qtiles, groups, per, nk.
+int &walk_order();    // -1 choose per layer (default), 0 batch groups first, 1 row tiles first (measurements only)
 inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
   if (a.nphase == 0 || a.M == 0 || a.batch == 0) return false;
   const TconvPhase &p0 = a.ph[0];
@@ -393,6 +406,8 @@ inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
   while (groups > 1 && sample_groups % groups) groups--;
   a.groups = groups;
   a.per = sample_groups / groups;
+  // more packed weights than an XCD's L2 holds (4 MiB), and several row tiles to deal out
+  a.weights_major = walk_order() >= 0 ? (uint32_t)walk_order() : ((uint64_t)a.nphase * a.M * p0.kp * 4u > (4u << 20) && a.tiles_m > 1 ? 1u : 0u);
   return (uint64_t)base * groups <= 0x7fffffffu;
 }
 

@@ -902,11 +902,18 @@ def _norm_case(oracle, B, cin, cout, H, W, seed, bias_std=0.0, func="relu"):
                                    (6, 16, 64, 4, 4), (8, 16, 48, 4, 4), (8, 12, 64, 5, 3), (3, 16, 3, 8, 8), (5, 10, 2, 6, 4)],  # separate passes
                          ids=lambda s: "x".join(str(v) for v in s))
 @pytest.mark.parametrize("bias_std", [0.0, 0.05], ids=["no-bias", "bias"])
-def test_transposed_convolution_between_batch_norms(gpu, oracle, shape, bias_std):
+@pytest.mark.parametrize("order", [0, 1], ids=["groups-first", "row-tiles-first"])
+def test_transposed_convolution_between_batch_norms(gpu, oracle, shape, bias_std, order, request):
     """mt_backward_convolution_norm_func / _norm_stats against the layers one after the other on the oracle: the input
-    is normalised as it is loaded, the raw output comes with the statistics of the batch norm that follows."""
+    is normalised as it is loaded, the raw output comes with the statistics of the batch norm that follows.  Both block
+    orders of the kernel that walks over the batch (the library picks by the size of the weights)."""
+    import mi355tensor as mt
     from mi355tensor import CTensor, Fused
     B, cin, cout, H, W = shape
+    if order == 1 and cout % 64 != 0:
+        pytest.skip("shapes that do not walk have no block order")
+    mt.set_option("walk_order", order)
+    request.addfinalizer(lambda: mt.set_option("walk_order", -1))
     x, pairs, kernel, bias, y = _norm_case(oracle, B, cin, cout, H, W, seed=sum(shape), bias_std=bias_std)
     tx, tp, tk, tb = (CTensor.from_numpy(v) for v in (x, pairs, kernel, bias))
     out = CTensor(B, cout, 2 * H, 2 * W)
