@@ -531,12 +531,15 @@ static void LoadConvolutionWeights(INetLayer<type_t> &layer,uint32_t rows,uint32
  layer.Load(&w);
 }
 
+static long long driver_allocations_in_the_timed_steps=0;   // blocks asked of the driver during the last TimeSteps' timed pass
 static double TimeSteps(const char *name,std::vector<INetLayer<type_t>*> &net,CTensor<type_t> *error,uint32_t warmup,uint32_t steps)
 {
  double ms=0;
+ int64_t before=0,after=0;
  for(uint32_t pass=0;pass<2;pass++)
  {
   const uint32_t count=(pass==0)?warmup:steps;
+  mt_get_info("driver_allocations",&before);
   CCUDATimeSpent timer;
   timer.Start();
   {
@@ -552,7 +555,9 @@ static double TimeSteps(const char *name,std::vector<INetLayer<type_t>*> &net,CT
    }
   }
   ms=timer.Stop();
+  mt_get_info("driver_allocations",&after);
  }
+ driver_allocations_in_the_timed_steps=after-before;
  return(ms/steps);
 }
 
@@ -593,8 +598,8 @@ static void TimeGenerator(uint32_t batch,uint32_t warmup,uint32_t steps)
  CTensor<type_t> &image=net.back()->GetOutputTensor();
  double sum=0;
  for(uint32_t x=0;x<64;x++) sum+=fabs(image.GetElement(batch-1,2,63,x));
- printf("{\"chain\": \"dcgan64_generator_forward\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"last_row_abs_sum\": %.6f}\n",
-        batch,steps,ms,image.GetSizeW(),image.GetSizeZ(),image.GetSizeY(),image.GetSizeX(),sum);
+ printf("{\"chain\": \"dcgan64_generator_forward\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"last_row_abs_sum\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
+        batch,steps,ms,image.GetSizeW(),image.GetSizeZ(),image.GetSizeY(),image.GetSizeX(),sum,driver_allocations_in_the_timed_steps);
 }
 
 // DCGAN-64 discriminator, whole training step (forward, backward with weight gradients, Adam), batch 128
@@ -628,8 +633,8 @@ static void TimeDiscriminator(uint32_t batch,uint32_t warmup,uint32_t steps)
  for(size_t n=0;n<net.size();n++) {net[n]->TrainingModeAdam();net[n]->TrainingStart();}
  double ms=TimeSteps("discriminator step",net,&error,warmup,steps);
  CTensor<type_t> &out=net.back()->GetOutputTensor();
- printf("{\"chain\": \"dcgan64_discriminator_step\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"first\": %.6f}\n",
-        batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),out.GetElement(0,0,0,0));
+ printf("{\"chain\": \"dcgan64_discriminator_step\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"first\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
+        batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),out.GetElement(0,0,0,0),driver_allocations_in_the_timed_steps);
 }
 
 static void ChainC(void)
