@@ -365,9 +365,9 @@ def main():
     # clocks over the first tens of milliseconds of load, so these steps run slower than the same steps of a job that
     # has been running for a moment.
     cold_gpu_ms, cold_wall_ms, _ = timed_region(args.steps)
-    # Sustained load: long enough (about 0.3 s) for the clocks to settle, and for a GPU-busy sample from outside to
+    # Sustained load: long enough (about 1 s) for the clocks to settle, and for a GPU-busy sample from outside to
     # see the GPU working; its average is reported as ms_per_step_sustained.
-    sustained_steps = max(500, 4 * args.steps)
+    sustained_steps = max(2000, 4 * args.steps)
     s0, s1 = create(), create()
     record(s0, stream)
     for _ in range(sustained_steps):

@@ -21,6 +21,8 @@
 // Chain H: the layers that work element by element on the host through GetElement/SetElement: SoftMax; Splitter with two
 //          consumers; DropOut and VAECoderOutput (both draw from std::random_device: the test recovers mask and noise
 //          from the outputs and checks the rest against them); MaxDePooling
+// "deferred" as the second argument (layers_mi355 only): chain K, two training steps of the DCGAN-64 discriminator at batch
+//          16 with and without the drop-in classes' deferral of the per-sample weight gradients
 // "time" as the second argument (layers_mi355 only): the DCGAN-64 generator's forward pass at batch 256 and the
 //          discriminator's training step at batch 128 on the reference's layer classes, timed with the drop-in CTimeStamp
 // Each chain: TrainingStart, Forward, SetOutputError, TrainingBackward, TrainingUpdateWeight (gradient descent), Save.
@@ -603,11 +605,10 @@ static void TimeGenerator(uint32_t batch,uint32_t warmup,uint32_t steps)
 }
 
 // DCGAN-64 discriminator, whole training step (forward, backward with weight gradients, Adam), batch 128
-static void TimeDiscriminator(uint32_t batch,uint32_t warmup,uint32_t steps)
+// the discriminator's layers with seeded weights, in training mode (Adam or plain gradient descent)
+static void BuildDiscriminator(uint32_t batch,std::vector<std::shared_ptr<INetLayer<type_t> > > &owner,std::vector<INetLayer<type_t>*> &net,bool adam=true)
 {
  static const uint32_t channels[5]={3,64,128,256,512};
- std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
- std::vector<INetLayer<type_t>*> net;
  PUSH(new CNetLayerConvolutionInput<type_t>(3,64,64,batch));
  for(uint32_t i=0;i<4;i++)
  {
@@ -626,15 +627,66 @@ static void TimeDiscriminator(uint32_t batch,uint32_t warmup,uint32_t steps)
  }
  PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_SIGMOID,net.back(),batch));
 #undef PUSH
+ for(size_t n=0;n<net.size();n++)
+ {
+  if (adam==true) net[n]->TrainingModeAdam();
+  net[n]->TrainingStart();
+ }
+}
+
+static void TimeDiscriminator(uint32_t batch,uint32_t warmup,uint32_t steps)
+{
+ std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
+ std::vector<INetLayer<type_t>*> net;
+ BuildDiscriminator(batch,owner,net);
  CTensor<type_t> image(batch,3,64,64),error(batch,1,1,1);
  FillTensor(image,1.0);
  FillTensor(error,0.5);
  net[0]->SetOutput(image);
- for(size_t n=0;n<net.size();n++) {net[n]->TrainingModeAdam();net[n]->TrainingStart();}
  double ms=TimeSteps("discriminator step",net,&error,warmup,steps);
  CTensor<type_t> &out=net.back()->GetOutputTensor();
  printf("{\"chain\": \"dcgan64_discriminator_step\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"first\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
         batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),out.GetElement(0,0,0,0),driver_allocations_in_the_timed_steps);
+}
+
+// Chain K: two training steps (gradient descent) of the discriminator at batch 16, once with the per-sample weight gradients deferred by the
+// drop-in classes (mi355::CDeferredGradient; the last two convolution layers qualify) and once with every call run when
+// it is made: same seeds, the updated convolution weights of both runs go to the dump
+static void ChainK(void)
+{
+ const uint32_t batch=16;
+ for(int deferred=1;deferred>=0;deferred--)
+ {
+  mi355::DeferGradients()=(deferred==1);
+  rng_state=0x0123456789ABCDEFull;
+  std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
+  std::vector<INetLayer<type_t>*> net;
+  // gradient descent: Adam would turn the rounding noise of gradients that are zero by construction (the biases in
+  // front of a batch normalisation) into steps of the full learning rate
+  BuildDiscriminator(batch,owner,net,false);
+  CTensor<type_t> image(batch,3,64,64),error(batch,1,1,1);
+  FillTensor(image,1.0);
+  FillTensor(error,0.5);
+  net[0]->SetOutput(image);
+  for(uint32_t step=0;step<2;step++)
+  {
+   for(size_t n=0;n<net.size();n++) net[n]->Forward();
+   for(size_t n=0;n<net.size();n++) net[n]->TrainingResetDeltaWeight();
+   net[net.size()-1]->SetOutputError(error);
+   for(size_t n=net.size()-1;n>=1;n--) net[n]->TrainingBackward(true);
+   for(size_t n=1;n<net.size();n++) net[n]->TrainingUpdateWeight(0.05,step+1);
+  }
+  for(int layer=0;layer<4;layer++)
+  {
+   CMemoryStream saved;
+   net[1+3*layer]->Save(&saved);
+   char label[32];
+   snprintf(label,sizeof(label),"K.%s.conv%d",deferred==1?"deferred":"eager",layer+1);
+   DumpStream(label,saved,8*sizeof(int32_t),2);
+  }
+  Dump(deferred==1?"K.deferred.out":"K.eager.out",net.back()->GetOutputTensor());
+ }
+ mi355::DeferGradients()=true;
 }
 
 static void ChainC(void)
@@ -729,6 +781,12 @@ int main(int argc,char **argv)
  try
  {
 #ifndef USE_CPU
+  if (argc>2 && strcmp(argv[2],"deferred")==0)   // only the chain that compares deferred and eager weight gradients
+  {
+   ChainK();
+   fclose(out_file);
+   return(0);
+  }
   if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up]]
   {
    const uint32_t steps=(argc>3)?static_cast<uint32_t>(atoi(argv[3])):50,warmup=(argc>4)?static_cast<uint32_t>(atoi(argv[4])):20;

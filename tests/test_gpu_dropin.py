@@ -183,3 +183,24 @@ def test_reference_layers_averaged_weights_on_the_dropin_classes(dumps):
     for got, w0, w1 in zip((beta, gamma, mean, variable), loaded, trained[:4]):
         assert np.abs(w1 - w0).max() > 1e-3
         assert rel_err(got, k * w0 + (np.float32(1) - k) * w1) <= 1e-6
+
+
+def test_deferred_weight_gradients_in_the_reference_layers(tmp_path):
+    """Two training steps (forward, backward, gradient descent) of the DCGAN-64 discriminator at batch 16 on the reference's own layer
+    classes: the drop-in classes defer the per-sample weight gradients of the last two convolution layers (their sums
+    over the batch are computed directly); the updated weights must be those of the run with every call made at once."""
+    if not os.path.exists(LAYERS_GPU):
+        pytest.skip("oracle/_ref/layers_mi355 not built (it needs /root/reference)")
+    path = str(tmp_path / "k.bin")
+    run = subprocess.run([LAYERS_GPU, path, "deferred"], capture_output=True, text=True, timeout=180)
+    assert run.returncode == 0, run.stderr + run.stdout[-2000:]
+    d = read_dump(path)
+    for layer in (1, 2, 3, 4):
+        for part in (0, 1):
+            a, b = d["K.deferred.conv%d.%d" % (layer, part)], d["K.eager.conv%d.%d" % (layer, part)]
+            assert a.shape == b.shape
+            # (the biases sit in front of a batch normalisation: their gradients are rounding noise around zero)
+            assert np.abs(a - b).max() <= 1e-6 + 1e-4 * np.abs(b).max(), (layer, part, np.abs(a - b).max(), np.abs(b).max())
+    assert rel_err(d["K.deferred.out"], d["K.eager.out"]) <= 1e-4
+    kernel = d["K.eager.conv4.0"]
+    assert kernel.shape == (1, 1, 512, 4096) and kernel.std() > 0.005
