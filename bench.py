@@ -296,6 +296,9 @@ def main():
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also launch one plain copy (mt_set) of this many MiB before the timed region: the known-size kernel "
                          "that calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--sustained-steps", type=int, default=0,
+                    help="steps of the sustained region (default: at least 2000, about a second of GPU work; counter runs of "
+                         "rocprofv3 --pmc, which intercept every dispatch, use a few hundred)")
     ap.add_argument("--graph", action="store_true",
                     help="time region 1 as replays of the step recorded once as a HIP graph (c5 does so by default: its step "
                          "is about a hundred short kernels and the Python host would be the bottleneck)")
@@ -367,7 +370,7 @@ def main():
     cold_gpu_ms, cold_wall_ms, _ = timed_region(args.steps)
     # Sustained load: long enough (about 1 s) for the clocks to settle, and for a GPU-busy sample from outside to
     # see the GPU working; its average is reported as ms_per_step_sustained.
-    sustained_steps = max(2000, 4 * args.steps)
+    sustained_steps = args.sustained_steps if args.sustained_steps > 0 else max(2000, 4 * args.steps)
     s0, s1 = create(), create()
     record(s0, stream)
     for _ in range(sustained_steps):
