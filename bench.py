@@ -329,6 +329,8 @@ def main():
     ap.add_argument("--literal", action="store_true", help="workload gan: up-sampling and convolution as two layers")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="mt_set_option before the run (measurements: tconv_walk=0, pack_cache=0, igemm_tile=3 ...); may be repeated")
+    ap.add_argument("--linear-bn", type=int, default=None, metavar="0|1",
+                    help="workload c3: Linear layer and its batch norm as one launch (1) or two (0); default: the generator's own choice")
     ap.add_argument("--fold", default=None, metavar="LAYERS",
                     help="workload c3: batch norms folded into the convolutions around them, e.g. 3 or 1,2,3 or none (default: the generator's own choice)")
     ap.add_argument("--workload", choices=["c3", "c5", "ops", "c1", "c2", "c4", "gan"], default="c3",
@@ -359,6 +361,8 @@ def main():
     net = G.DcganGenerator(BATCH)
     if args.fold is not None:
         net.fold = () if args.fold == "none" else tuple(int(v) for v in args.fold.split(","))
+    if args.linear_bn is not None:
+        net.fuse_linear_bn = bool(args.linear_bn)
     net.set_latent(G.make_latent(BATCH))
     stream = mt.get_stream()
     create, record, elapsed_ms = hip_events()

@@ -174,4 +174,67 @@ int mt_linear_forward_func(const mt_tensor *out, const mt_tensor *weight, const 
   return rc == MT_OK ? mt_apply_func(out, out, func) : rc;
 }
 
+// CNetLayerLinear::Forward, CNetLayerBatchNormalization::Forward in training mode and CNetLayerFunction::Forward as one
+// launch: features are the rows of the product, the batch its columns, and a 16 x 256 block holds the whole batch of its
+// 16 features, so the statistics over the batch are sums inside the block (lane shuffles, then the four wavefronts
+// through LDS).  Batches above 256 take the two calls.
+int mt_linear_batchnorm_forward_func(const mt_tensor *out, const mt_tensor *weight, const mt_tensor *input, const mt_tensor *bias, const mt_tensor *gamma,
+                                     const mt_tensor *beta, const mt_tensor *linear_output, const mt_tensor *xhat, const mt_tensor *ivar,
+                                     const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean, const mt_tensor *new_variable,
+                                     float momentum, float epsilon, int func) {
+  const char *name = "mt_linear_batchnorm_forward_func";
+  if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "%s: unknown function id %d", name, func);
+  if (mt::bad(out) || mt::bad(weight) || mt::bad(input) || mt::bad(bias) || mt::bad(gamma) || mt::bad(beta)) return mt::fail(MT_E_ARGUMENT, "%s: null tensor", name);
+  for (auto t : {out, linear_output, xhat, ivar, batch_mean, batch_var, new_mean, new_variable}) mt::note_write(t);
+  const uint32_t B = input->w, In = input->z * input->y * input->x, Out = weight->y;
+  if (weight->w != 1 || weight->z != 1 || weight->x != In || bias->w != 1 || bias->z != 1 || bias->x != 1 || bias->y != Out)
+    return mt::fail(MT_E_SHAPE, "%s: weight must be [1,1,Out,In], bias [1,1,Out,1]", name);
+  const size_t S = Out;
+  if (out->w != B || (size_t)out->z * out->y * out->x != S) return mt::fail(MT_E_SHAPE, "%s: output must hold [B,Out] values", name);
+  for (auto t : {gamma, beta, ivar, batch_mean, batch_var, new_mean, new_variable})
+    if (t && (t->p == nullptr || t->w == 0 || (size_t)t->z * t->y * t->x != S)) return mt::fail(MT_E_SHAPE, "%s: parameters and statistics are [1,...] tensors of Out values", name);
+  for (auto t : {linear_output, xhat})
+    if (t && (t->p == nullptr || t->w != B || (size_t)t->z * t->y * t->x != S)) return mt::fail(MT_E_SHAPE, "%s: linear_output and xhat hold [B,Out] values", name);
+  if (B == 0 || Out == 0) return MT_OK;
+  const bool fast = B <= 256 && In > 0 && mt::fits_buffer((size_t)Out * In) && mt::fits_buffer((size_t)B * In) && aligned16(out->p) && (!xhat || aligned16(xhat->p)) &&
+                    Out <= 0x7fffffffu / 16u;
+  if (!fast) {
+    // the layers one after the other; the Linear output goes to its own tensor if there is one, else through `out`
+    mt_tensor lin = linear_output ? *linear_output : *out;
+    lin.z = 1; lin.y = Out; lin.x = 1;
+    int rc = mt_linear_forward_func(&lin, weight, input, bias, MT_F_NONE);
+    if (rc) return rc;
+    mt_tensor x = *out;   // the same values seen with the output's sizes
+    x.p = lin.p;
+    return mt_batchnorm_forward_train_func(out, &x, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func);
+  }
+  Epilogue ep{};
+  ep.C = out->p; ep.row_stride = 1; ep.inner = 1; ep.g_stride = Out;
+  ep.bias = bias->p; ep.bias_mode = 1; ep.func = func;
+  ep.bn.gamma = gamma->p; ep.bn.beta = beta->p;
+  ep.bn.raw = linear_output ? linear_output->p : nullptr;
+  ep.bn.xhat = xhat ? xhat->p : nullptr;
+  ep.bn.ivar = ivar ? ivar->p : nullptr;
+  ep.bn.mean = batch_mean ? batch_mean->p : nullptr;
+  ep.bn.var = batch_var ? batch_var->p : nullptr;
+  ep.bn.new_mean = new_mean ? new_mean->p : nullptr;
+  ep.bn.new_var = new_variable ? new_variable->p : nullptr;
+  ep.bn.inv_n = (float)(1.0 / (double)(float)B);
+  ep.bn.eps = epsilon;
+  ep.bn.mom_old = momentum;
+  ep.bn.mom_new = (float)(1.0 - (double)momentum);
+  const uint32_t tiles = cdiv(Out, 16);
+  mt::ProfileScope prof(mt::profiling() ? shape_label(name, T16x256, Out, B, In, 1) : name);
+  const Batch none{};
+  int rc = with_row_k(weight->p, In, Out, In, none, [&](auto a) {
+    return with_row_k(input->p, In, B, In, none, [&](auto b) {
+      igemm_kernel<1, 2, 1, 4, true, true><<<tiles, THREADS, 0, mt::stream()>>>(a, b, ep, Out, B, In, tiles, 1);
+      return MT_OK;
+    });
+  });
+  if (rc) return rc;
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
 }  // extern "C"

@@ -509,6 +509,13 @@ struct Epilogue {
   bool accumulate = false;
   Batch bt;
   uint32_t g0 = 0;  // batched launches: the batch entry's w, so that per-sample biases still index by w
+  // Batch normalisation over the columns of a block that holds all of them (BN_TAIL kernels only): row m is a feature,
+  // the N columns are the batch.  gamma, beta and the statistics are indexed by m.
+  struct BnTail {
+    const float *gamma = nullptr, *beta = nullptr;
+    float *raw = nullptr, *xhat = nullptr, *ivar = nullptr, *mean = nullptr, *var = nullptr, *new_mean = nullptr, *new_var = nullptr;
+    float inv_n = 0.f, eps = 0.f, mom_old = 0.f, mom_new = 0.f;
+  } bn;
 
   struct Col {
     size_t off;
@@ -646,10 +653,11 @@ __device__ __forceinline__ void lds_barrier() {
 // v_mfma_f32_16x16x4_f32: lane l supplies row (or column) l % 16 at k slot l / 16, so ONE 128-bit LDS read at
 // k offset 4*(l/16) feeds four instructions that together cover the 16 k of a tile (instruction c multiplies
 // k = c, 4+c, 8+c, 12+c).  The two halves of a pipeline step are then the two halves of the wavefront's columns.
-template <int TM, int TN, int WGM, int WGN, bool R16, class SrcA, class SrcB>
+template <int TM, int TN, int WGM, int WGN, bool R16, bool BN_TAIL = false, class SrcA, class SrcB>
 __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep, uint32_t M, uint32_t N, uint32_t K, uint32_t m0, uint32_t n0, float *smem) {
   static_assert(WGM * WGN == 4, "four wavefronts per block");
   static_assert(!R16 || (TM == 1 && WGM == 1), "a 16-row block is one row of wavefronts");
+  static_assert(!BN_TAIL || R16, "the batch-norm tail belongs to the 16-row block, whose 256 columns hold a whole batch");
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
   constexpr int EA = BM * BK / THREADS, EB = BN * BK / THREADS;
   static_assert(EA >= 2 && EB >= 2, "tile too small for the loader");
@@ -810,6 +818,102 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
     step(Even{}, No{}, No{});
   }
 
+  if constexpr (BN_TAIL) {
+    // The block's columns are the whole batch (n0 == 0, N <= BN): Linear bias, then the batch normalisation of the
+    // layer behind it (netlayer/cnetlayerbatchnormalization.cu.h:301-371) on the accumulators, then the function.
+    // Register r of accumulator j of lane l holds C[4*(l/16) + r][wn*TN*32 + 16*j + l%16]: a row's values sit in the 16
+    // lanes that share l/16 (lane shuffles), in the 2*TN accumulators of a lane and in the four wavefronts (LDS).
+    __syncthreads();                           // every wavefront has read its last operand fragments: the tiles' memory is free
+    float *red = smem;                         // [4 wavefronts][16 rows]
+    const uint32_t m4 = m0 + 4 * lk;
+    const Epilogue::BnTail &bn = ep.bn;
+    float v[2 * TN][4];
+    bool ok[2 * TN];
+    float bias_r[4], gamma_r[4], beta_r[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const bool row = m4 + r < M;
+      bias_r[r] = ep.bias && row ? ep.bias[m4 + r] : 0.f;
+      gamma_r[r] = row ? bn.gamma[m4 + r] : 0.f;
+      beta_r[r] = row ? bn.beta[m4 + r] : 0.f;
+    }
+    auto row_sums = [&](float (&s)[4]) {       // over the batch: lanes, then wavefronts; every lane gets the totals of its rows
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1)
+#pragma unroll
+        for (int r = 0; r < 4; r++) s[r] += __shfl_xor(s[r], off, 64);
+      if (lrow == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[wave * 16 + 4 * lk + r] = s[r];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < 4; r++) s[r] = ((red[4 * lk + r] + red[16 + 4 * lk + r]) + red[32 + 4 * lk + r]) + red[48 + 4 * lk + r];
+      __syncthreads();
+    };
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 2 * TN; j++) {
+      ok[j] = n0 + wn * TN * 32 + j * 16 + lrow < N;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        v[j][r] = acc16[j][r] + bias_r[r];
+        s[r] += ok[j] ? v[j][r] : 0.f;
+      }
+    }
+    row_sums(s);
+    float mean[4], q[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 4; r++) mean[r] = s[r] * bn.inv_n;
+#pragma unroll
+    for (int j = 0; j < 2 * TN; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const float raw = v[j][r];
+        if (bn.raw && ok[j] && m4 + r < M) bn.raw[(size_t)(n0 + wn * TN * 32 + j * 16 + lrow) * M + m4 + r] = raw;
+        v[j][r] = raw - mean[r];
+        q[r] += ok[j] ? v[j][r] * v[j][r] : 0.f;
+      }
+    row_sums(q);
+    float iv[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float vr = q[r] * bn.inv_n;
+      iv[r] = (float)(1.0 / (double)sqrtf(vr + bn.eps));
+      if (wave == 0 && lrow == 0 && m4 + r < M) {
+        const uint32_t m = m4 + r;
+        if (bn.mean) bn.mean[m] = mean[r];
+        if (bn.var) bn.var[m] = vr;
+        if (bn.ivar) bn.ivar[m] = iv[r];
+        if (bn.new_mean) bn.new_mean[m] = (bn.mom_old * bn.new_mean[m]) + (bn.mom_new * mean[r]);
+        if (bn.new_var) bn.new_var[m] = (bn.mom_old * bn.new_var[m]) + (bn.mom_new * vr);
+      }
+    }
+    const bool whole = m4 + 4 <= M && M % 4 == 0;   // the lane's four rows are one aligned 16-byte piece of a sample
+#pragma unroll
+    for (int j = 0; j < 2 * TN; j++) {
+      if (!ok[j]) continue;
+      const size_t at = (size_t)(n0 + wn * TN * 32 + j * 16 + lrow) * M + m4;   // output [batch][features]
+      float xh[4], o[4];
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        xh[r] = v[j][r] * iv[r];
+        o[r] = apply_func_epilogue(ep.func, gamma_r[r] * xh[r] + beta_r[r]);
+      }
+      if (whole) {
+        *reinterpret_cast<float4 *>(ep.C + at) = make_float4(o[0], o[1], o[2], o[3]);
+        if (bn.xhat) *reinterpret_cast<float4 *>(bn.xhat + at) = make_float4(xh[0], xh[1], xh[2], xh[3]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          if (m4 + r < M) {
+            ep.C[at + r] = o[r];
+            if (bn.xhat) bn.xhat[at + r] = xh[r];
+          }
+      }
+    }
+    return;
+  }
   if constexpr (R16) {
     // accumulator layout of v_mfma_f32_16x16x4_f32: register r of lane l holds C[4*(l/16) + r][l%16]
 #pragma unroll
@@ -843,7 +947,7 @@ __device__ __forceinline__ uint32_t xcd_swizzle(uint32_t L, uint32_t total) {
 
 // Generic launch: logical block index = (n tile, batch entry, m tile), n slowest, so concurrently running blocks
 // of one XCD share their B tile (the activations) and cycle through the A tiles (the weights).
-template <int TM, int TN, int WGM, int WGN, bool R16, class SrcA, class SrcB>
+template <int TM, int TN, int WGM, int WGN, bool R16, bool BN_TAIL = false, class SrcA, class SrcB>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN == 1 ? 5 : TM * TN == 2 ? 3 : 2))) void igemm_kernel(SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N, uint32_t K, uint32_t tiles_m, uint32_t batches) {
   using TS = TileShape<TM, TN, WGM, WGN>;
   __shared__ float4 smem[TS::LDS_FLOATS / 4];
@@ -853,7 +957,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN
   a.batch(bz);
   b.batch(bz);
   ep.batch(bz);
-  igemm_body<TM, TN, WGM, WGN, R16>(a, b, ep, M, N, K, mt * (R16 ? 16 : TS::BM), nt * TS::BN, reinterpret_cast<float *>(smem));
+  igemm_body<TM, TN, WGM, WGN, R16, BN_TAIL>(a, b, ep, M, N, K, mt * (R16 ? 16 : TS::BM), nt * TS::BN, reinterpret_cast<float *>(smem));
 }
 
 enum Tile { T128x128, T64x128, T32x128, T64x64, T16x256 };

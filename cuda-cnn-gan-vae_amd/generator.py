@@ -22,6 +22,7 @@ CHANNELS = (512, 256, 128, 64, 3)
 BN_EPSILON = 1e-6
 MOMENTUM = 0.9
 FOLD = (3,)
+FUSE_LINEAR_BN = False
 
 
 def make_parameters(seed=3, std=0.02):
@@ -77,6 +78,10 @@ class DcganGenerator:
         # the transposed convolution in front of it and its normalisation + ReLU happen in the loader of the one behind
         # it.  Measured per layer on an MI355X at batch 256; the others keep the one-pass batch-norm kernel.
         self.fold = FOLD
+        # forward_fused can run the Linear layer and its batch norm as one launch (the Linear layer's own output h[0] is
+        # then written only when somebody wants to look at it) or as two
+        self.fuse_linear_bn = FUSE_LINEAR_BN
+        self.keep_linear_output = False
 
     def set_latent(self, z):
         self.latent.upload(z)
@@ -94,14 +99,20 @@ class DcganGenerator:
         return self.a[i].numpy()
 
     def forward_fused(self):
-        """One or two launches per layer.  Batch norm 0 (behind the Linear layer) is always the one-pass kernel; a batch
-        norm i in self.fold never writes its output: the convolution in front of it leaves the raw activation h[i] and the
-        pairs (scale, shift), the convolution behind it normalises as it loads."""
+        """One or two launches per layer.  Batch norm 0 sits in the epilogue of the Linear layer's product (a block holds
+        the whole batch of its features); a batch norm i in self.fold never writes its output: the convolution in front of
+        it leaves the raw activation h[i] and the pairs (scale, shift), the convolution behind it normalises as it loads."""
         p = self.p
-        Fused.LinearForward(self.lin_out, p["lin_w"], self.latent, p["lin_b"], None)
+        if self.fuse_linear_bn:
+            Fused.LinearBatchNormForwardTrain(self.a[0], p["lin_w"], self.latent, p["lin_b"], p["gamma0"], p["beta0"],
+                                              linear_output=self.lin_out if self.keep_linear_output else None,
+                                              momentum=MOMENTUM, epsilon=BN_EPSILON, func="relu")
+        else:
+            Fused.LinearForward(self.lin_out, p["lin_w"], self.latent, p["lin_b"], None)
+            Fused.BatchNormForwardTrain(self.a[0], self.h[0], p["gamma0"], p["beta0"], momentum=MOMENTUM, epsilon=BN_EPSILON, func="relu")
         for i in range(4):
             folded, next_folded = i in self.fold and i > 0, (i + 1) in self.fold and i < 3
-            if not folded:
+            if not folded and i > 0:
                 Fused.BatchNormForwardTrain(self.a[i], self.h[i], p["gamma%d" % i], p["beta%d" % i], momentum=MOMENTUM, epsilon=BN_EPSILON, func="relu")
             if not folded and not next_folded:
                 CTensorConv.BackwardConvolution(self.h[i + 1], self.a[i], p["kernel%d" % i], 4, 4, CHANNELS[i + 1], CHANNELS[i], p["bias%d" % i], 2, 2, 1, 1,

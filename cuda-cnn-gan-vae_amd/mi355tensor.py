@@ -468,6 +468,15 @@ class Fused:
         call("mt_linear_forward_func", _d(out), _d(weight), _d(inp), _d(bias), C.c_int(FUNC[func]))
 
     @staticmethod
+    def LinearBatchNormForwardTrain(out, weight, inp, bias, gamma, beta, linear_output=None, xhat=None, ivar=None, batch_mean=None, batch_var=None,
+                                    new_mean=None, new_variable=None, momentum=0.9, epsilon=1e-6, func=None):
+        """Linear layer, batch normalisation in training mode and function layer in one launch (batches of at most 256;
+        larger ones run as the two calls inside the library)."""
+        opt = lambda t: _d(t) if t is not None else None
+        call("mt_linear_batchnorm_forward_func", _d(out), _d(weight), _d(inp), _d(bias), _d(gamma), _d(beta), opt(linear_output), opt(xhat), opt(ivar),
+             opt(batch_mean), opt(batch_var), opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
+
+    @staticmethod
     def BatchNormForwardTrain(out, inp, gamma, beta, xhat=None, ivar=None, batch_mean=None, batch_var=None, new_mean=None, new_variable=None,
                               momentum=0.9, epsilon=1e-6, func=None):
         opt = lambda t: _d(t) if t is not None else None

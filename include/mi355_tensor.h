@@ -226,6 +226,17 @@ int mt_backward_convolution_norm_stats(const mt_tensor *output, const mt_tensor 
 /* CNetLayerLinear::Forward + CNetLayerFunction::Forward (netlayer/cnetlayerlinear.cu.h:262-282): output[B,1,Out,1] =
  * func(weight[1,1,Out,In] * input[B,1,In,1] + bias[1,1,Out,1]); `input` may have any [B,Z,Y,X] with Z*Y*X == In. */
 int mt_linear_forward_func(const mt_tensor *output, const mt_tensor *weight, const mt_tensor *input, const mt_tensor *bias, int func);
+/* CNetLayerLinear::Forward (netlayer/cnetlayerlinear.cu.h:262-282), CNetLayerBatchNormalization::Forward in training mode
+ * (netlayer/cnetlayerbatchnormalization.cu.h:301-371) and CNetLayerFunction::Forward as one launch for batches of at most
+ * 256: output [B,...] = func(gamma * xhat + beta) with xhat = (weight * input + bias - mean) * ivar, mean and variance per
+ * output feature over the batch, computed on the product's accumulators (a block holds the whole batch of its 16
+ * features).  weight, input, bias as for mt_linear_forward_func; gamma, beta and the optional statistics hold Out values
+ * ([1,Z,Y,X] with Z*Y*X == Out, like the output's sample); optional linear_output (the Linear layer's own output) and
+ * xhat hold [B,Out] values; NULL skips an optional tensor.  Larger batches run as the two calls. */
+int mt_linear_batchnorm_forward_func(const mt_tensor *output, const mt_tensor *weight, const mt_tensor *input, const mt_tensor *bias,
+                                     const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *linear_output, const mt_tensor *xhat,
+                                     const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
+                                     const mt_tensor *new_variable, float momentum, float epsilon, int func);
 /* CNetLayerBatchNormalization::Forward in training mode followed by CNetLayerFunction::Forward
  * (netlayer/cnetlayerbatchnormalization.cu.h:301-371): statistics per element (z,y,x) over the batch axis W.
  * Writes output = func(gamma*xhat+beta); optionally xhat [B,Z,Y,X], ivar / batch mean / batch variance [1,Z,Y,X]

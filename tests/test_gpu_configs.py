@@ -52,9 +52,12 @@ def test_config3_generator_against_oracle(gpu, oracle):
     params, z = G.make_parameters(), G.make_latent(8)
     want = seq.dcgan_generator_forward(oracle, params, z)
     net = G.DcganGenerator(8, params)
+    net.keep_linear_output = True
     net.set_latent(z)
-    for forward, fold in ((net.forward_fused, ()), (net.forward_fused, (3,)), (net.forward_fused, (1, 2, 3)), (net.forward_literal, ())):
+    for forward, fold, one_launch in ((net.forward_fused, (), False), (net.forward_fused, (3,), True), (net.forward_fused, (3,), False),
+                                      (net.forward_fused, (1, 2, 3), False), (net.forward_literal, (), False)):
         net.fold = fold
+        net.fuse_linear_bn = one_launch   # the Linear layer and its batch norm as one launch or two
         for t in net.h + net.a:
             mt_fill(t, 7.0)
         forward()
@@ -79,10 +82,12 @@ def test_config3_full_batch_properties(gpu, oracle):
     import generator as G
     params, z = G.make_parameters(), G.make_latent(256)
     net = G.DcganGenerator(256, params)
+    net.keep_linear_output = True
     net.set_latent(z)
     literal = net.forward_literal().numpy()
-    for fold in ((), G.FOLD, (1, 2, 3)):
+    for fold, one_launch in (((), False), (G.FOLD, False), (G.FOLD, True), ((1, 2, 3), False)):
         net.fold = fold
+        net.fuse_linear_bn = one_launch
         fused = net.forward_fused().numpy()
         a = [net.activation(i) for i in range(4)]
         h = [t.numpy() for t in net.h[:4]]

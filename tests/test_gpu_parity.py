@@ -1003,3 +1003,41 @@ def test_image_layer_on_the_4x4x1_matrix_instructions(gpu, oracle, shape):
             close(out.numpy(), want_norm, 1e-5)
     finally:
         mt.set_option("image_mfma", 0)
+
+
+@pytest.mark.parametrize("shape", [(256, 100, 8192, "relu"), (6, 37, 50, "leaky_relu"), (64, 128, 96, None), (255, 20, 18, "tangence"),
+                                   (300, 24, 64, "relu")],   # the last one: more than 256 samples, the two calls inside the library
+                         ids=lambda s: "x".join(str(v) for v in s))
+def test_linear_layer_with_the_batch_norm_in_its_epilogue(gpu, oracle, shape):
+    """mt_linear_batchnorm_forward_func against the layers one after the other on the oracle (Linear, batch normalisation
+    in training mode, function): output, every statistic it can leave, the blended running statistics and the Linear
+    layer's own output."""
+    from mi355tensor import CTensor, Fused
+    B, n_in, n_out, func = shape
+    seed = sum(v for v in shape[:3])
+    x, w, b = Nrm(seed, B, 1, n_in, 1), Nrm(seed + 1, 1, 1, n_out, n_in, std=0.3), U(seed + 2, 1, 1, n_out, 1)
+    gamma, beta = U(seed + 3, 1, 1, n_out, 1, lo=0.5, hi=1.5), U(seed + 4, 1, 1, n_out, 1, lo=-0.3, hi=0.3)
+    nm0, nv0 = U(seed + 5, 1, 1, n_out, 1), U(seed + 6, 1, 1, n_out, 1, lo=0.5, hi=2.0)
+    lin = seq.linear_forward(oracle, w, x, b)
+    want = seq.batchnorm_forward_train(oracle, lin, gamma, beta, new_mean=nm0, new_var=nv0, momentum=0.9)
+    y = oracle.apply_func(want["out"], func) if func else want["out"]
+    one, full = (1, 1, n_out, 1), (B, 1, n_out, 1)
+    t = dict(linear_output=CTensor(*full), xhat=CTensor(*full), ivar=CTensor(*one), batch_mean=CTensor(*one), batch_var=CTensor(*one),
+             new_mean=CTensor.from_numpy(nm0), new_variable=CTensor.from_numpy(nv0))
+    out = CTensor(*full)
+    tx, tw, tb, tg, tbe = (CTensor.from_numpy(v) for v in (x, w, b, gamma, beta))
+    Fused.LinearBatchNormForwardTrain(out, tw, tx, tb, tg, tbe, momentum=0.9, epsilon=seq.BN_EPSILON, func=func, **t)
+    close(t["linear_output"].numpy(), lin)
+    close(t["batch_mean"].numpy(), want["mean"], 1e-5)
+    close(t["batch_var"].numpy(), want["var"], 1e-5)
+    close(t["ivar"].numpy(), want["ivar"], 1e-5)
+    close(t["new_mean"].numpy(), want["new_mean"], 1e-5)
+    close(t["new_variable"].numpy(), want["new_var"], 1e-5)
+    close(t["xhat"].numpy(), want["xhat"])
+    close(out.numpy(), y)
+    # nothing optional asked for, and the output shaped as the [512,4,4]-like tensor a convolution will read
+    if n_out % 16 == 0:
+        shaped = CTensor(B, n_out // 16, 4, 4)
+        g4, b4 = (CTensor.from_numpy(v.reshape(1, n_out // 16, 4, 4)) for v in (gamma, beta))
+        Fused.LinearBatchNormForwardTrain(shaped, tw, tx, tb, g4, b4, epsilon=seq.BN_EPSILON, func=func)
+        close(shaped.numpy().reshape(y.shape), y)
