@@ -174,6 +174,24 @@ __device__ __forceinline__ float apply_func_epilogue(int func, float v) {
   if (func == MT_F_SIGMOID) return f_sigmoid_fast(v);
   return apply_func_outlined(func, v);
 }
+// The same for N values at once: one look at the (uniform) function, then straight-line code.
+template <int N>
+__device__ __forceinline__ void apply_func_epilogue_many(int func, float *v) {
+  if (func == MT_F_NONE || func == MT_F_LINEAR) return;
+  if (func == MT_F_TANGENCE) {
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = f_tangence_fast(v[i]);
+  } else if (func == MT_F_SIGMOID) {
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = f_sigmoid_fast(v[i]);
+  } else if (func == MT_F_RELU) {
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = v[i] > 0.f ? v[i] : 0.f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = apply_func_epilogue(func, v[i]);
+  }
+}
 
 inline bool valid_func(int func, bool allow_none) {
   if (func == MT_F_NONE) return allow_none;

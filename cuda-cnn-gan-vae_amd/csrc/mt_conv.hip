@@ -922,6 +922,152 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
 }
 
+// The same layer as a product WITHOUT neighbourhoods, then a cheap combination.  A stride-2 transposed convolution
+// scatters: input pixel (y, x) adds kernel tap (phase, tap) times its value to one output pixel near (2y, 2x).  So
+//   P[(tap of 16, co)][pixel] = sum over ci of coefficient[(tap, co)][ci] * in[ci][pixel]
+// is an ordinary product with 16*CO rows, K = C and the raw input pixels as columns -- no patch, no halo, no padding
+// rows: with CO = 3 the 48 rows are exactly three 16-row tiles of v_mfma_f32_16x16x4_f32.  Every output pixel is then
+// the sum of four P values of neighbouring input pixels.
+//
+// A block owns one image (W = 32, H <= 32 rows, one wavefront per two rows).  Lane (n, g) of a wavefront supplies, per
+// k step of four channels, channel 4s + g of pixels x = 2n, 2n+1 in both rows: two 64-bit loads straight from global
+// memory into the matrix operand (the input is read exactly once, in whole lines; no LDS for it), DEPTH k steps ahead
+// in a register ring.  The coefficients are re-ordered once per block into LDS as [k step][tile][lane], one 32-bit read
+// per tile and k step, from the [ci][phase][co][taps] order of the tile kernel.  NORM: func(scale * x + shift) on the
+// operand registers, the pairs fetched beside the values.
+//
+// Rows of a tile are (a, b) = ((py, ty), (px, tx)): the product of category a lands in output row 2y + {2, 0, 1, -1}[a],
+// of category b in output column 2x + {2, 0, 1, -1}[b].  The accumulator layout puts a into the lane group g and b into
+// the register index, so the combination along x is four additions per output row piece, two of them with the
+// neighbouring lane's value (a DPP shift inside the 16 lanes that hold one image row: what it shifts in at either end is
+// the zero beyond the image), and the combination along y goes once through LDS ([row][a][co][64 columns]), from where
+// every lane takes the two pieces of its output row, adds the bias term, applies the function and stores 16 bytes of a
+// whole output line.
+// Needs W == 32, H even and at most 32, C a multiple of 4 * DEPTH, exactly CO output channels, 8-byte aligned input.
+template <int CO, int NORM, int DEPTH>   // NORM: 0 plain input, 1 ReLU(scale * x + shift), 2 any of the cheap functions
+__global__ __launch_bounds__(1024) void tconv_k4s2_products_kernel(TconvArgs args) {
+  extern __shared__ __attribute__((aligned(16))) float pieces[];  // [H][4][CO][64], then the coefficients [C/4][CO][64]
+  const uint32_t H = args.H, C = args.C, HW = H * 32u;
+  const uint32_t img = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t n = (uint32_t)lane & 15u, g = (uint32_t)lane >> 4;
+  const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta, args.in_w * C * HW * 4u);
+  __amdgpu_buffer_rsrc_t prsrc = rsrc;
+  if (NORM) prsrc = make_rsrc(args.in_scale_shift, C * HW * 8u);
+  // value offsets: channel g of the k step, row 2*wave (the next row is 128 bytes on), pixels 2n, 2n+1
+  const uint32_t in_sample = ((g * H + 2u * (uint32_t)wave) * 32u + 2u * n) * 4u;
+  const uint32_t b_voff = (img % args.in_w) * C * HW * 4u + in_sample, b_step = 4u * HW * 4u;
+  const uint32_t steps = C / 4u;
+  const int in_func = args.in_func;
+  float *coeff = pieces + H * 4u * CO * 64u;
+
+  floatx2 rb[DEPTH][2];
+  floatx4 rp[NORM ? DEPTH : 1][2];
+  float rc[2][CO];
+  auto fetch = [&](int slot, uint32_t s) {
+    const bool live = s < steps;   // uniform; loads beyond the last step are dropped by the range check
+    const uint32_t bo = live ? b_voff : OOB;
+#pragma unroll
+    for (int yy = 0; yy < 2; yy++) rb[slot][yy] = buf_load2(rsrc, bo == OOB ? OOB : bo + (uint32_t)yy * 128u, s * b_step);
+    if constexpr (NORM != 0) {
+      const uint32_t po = live ? in_sample * 2u : OOB;
+#pragma unroll
+      for (int yy = 0; yy < 2; yy++) rp[slot][yy] = buf_load4(prsrc, po == OOB ? OOB : po + (uint32_t)yy * 256u, s * b_step * 2u);
+    }
+  };
+
+  floatx4acc acc[CO][4];   // [tile = co][pixel group (yy, xx)]
+#pragma unroll
+  for (int co = 0; co < CO; co++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[co][j] = floatx4acc{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int d = 0; d < DEPTH; d++) fetch(d, (uint32_t)d);
+  // The coefficients in the order the matrix instruction takes them.  Row i = lane % 16 of a tile is
+  // (a, b) = (i / 4, i % 4) = ((py, ty), (px, tx)); lane / 16 is the channel within the k step.
+  for (uint32_t idx = (uint32_t)tid; idx < steps * CO * 64u; idx += blockDim.x) {
+    const uint32_t l = idx & 63u, co = (idx >> 6) % CO, s = idx / (64u * CO), i = l & 15u;
+    const uint32_t f = ((i >> 2) >> 1) * 2u + ((i & 3u) >> 1), t = ((i >> 2) & 1u) * 2u + (i & 1u);
+    coeff[idx] = args.ph[0].packed[((4u * s + (l >> 4)) * 16u + f * 4u) * CO + co * 4u + t];
+  }
+  __syncthreads();
+  const float *cget = coeff + lane;
+#pragma unroll
+  for (int co = 0; co < CO; co++) rc[0][co] = cget[co * 64];
+  for (uint32_t s0 = 0; s0 < steps; s0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+      {
+        const uint32_t sn = s0 + (uint32_t)d + 1u < steps ? s0 + (uint32_t)d + 1u : 0u;   // (the last step reads something it does not use)
+#pragma unroll
+        for (int co = 0; co < CO; co++) rc[(d + 1) & 1][co] = cget[(sn * CO + co) * 64u];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      float v[4] = {rb[d][0].x, rb[d][0].y, rb[d][1].x, rb[d][1].y};   // (yy, xx) = 00 01 10 11
+      if constexpr (NORM != 0) {
+        const float sc[4] = {rp[d][0].x, rp[d][0].z, rp[d][1].x, rp[d][1].z}, sh[4] = {rp[d][0].y, rp[d][0].w, rp[d][1].y, rp[d][1].w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const float u = sc[j] * v[j] + sh[j];
+          v[j] = NORM == 1 ? (u > 0.f ? u : 0.f) : mt::apply_func_cheap(in_func, u);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int co = 0; co < CO; co++) acc[co][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(rc[d & 1][co], v[j], acc[co][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(d, s0 + (uint32_t)d + DEPTH);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // ---- along x: output columns 4n .. 4n+3 of row category a = g, for both input rows and every channel
+  auto from_left = [](float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x111, 0xf, 0xf, true)); };   // row_shr:1
+  auto from_right = [](float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x101, 0xf, 0xf, true)); };  // row_shl:1
+#pragma unroll
+  for (int yy = 0; yy < 2; yy++)
+#pragma unroll
+    for (int co = 0; co < CO; co++) {
+      const floatx4acc &e = acc[co][yy * 2], &o = acc[co][yy * 2 + 1];   // pixels x = 2n and 2n + 1; register = category b
+      floatx4 r;
+      r.x = e[1] + from_left(o[0]);    // column 4n:     x = 2n as 2x, x = 2n - 1 as 2x + 2
+      r.y = e[2] + o[3];               // column 4n + 1: x = 2n as 2x + 1, x = 2n + 1 as 2x - 1
+      r.z = o[1] + e[0];               // column 4n + 2: x = 2n + 1 as 2x, x = 2n as 2x + 2
+      r.w = o[2] + from_right(e[3]);   // column 4n + 3: x = 2n + 1 as 2x + 1, x = 2n + 2 as 2x - 1
+      *reinterpret_cast<floatx4 *>(&pieces[((((uint32_t)(2 * wave + yy)) * 4u + g) * CO + co) * 64u + 4u * n]) = r;
+    }
+
+  __syncthreads();
+
+  // ---- along y: output row 2m is input row m in category 1 plus row m - 1 in category 0; output row 2m + 1 is row m in
+  // category 2 plus row m + 1 in category 3.  The lane takes row 4*wave + g, columns 4n .. 4n+3, every channel.
+  const uint32_t oy = 4u * (uint32_t)wave + g, m = oy >> 1, odd = oy & 1u;
+  const uint32_t a_own = odd ? 2u : 1u, a_other = odd ? 3u : 0u;
+  const int32_t y_other = odd ? (int32_t)m + 1 : (int32_t)m - 1;
+  const bool other = (uint32_t)y_other < H;
+  const uint32_t OHW = 4u * HW;
+  const float bsum = args.ep.tap_bias ? args.ep.tap_bias[img % args.ep.bias_w] : 0.f;
+  const float ny = other ? 2.f : 1.f;
+  // contributing input columns of an output column: two, one at the image's left and right edge
+  const float nx[4] = {n == 0 ? 1.f : 2.f, 2.f, 2.f, n == 15 ? 1.f : 2.f};
+  float o[CO][4];
+#pragma unroll
+  for (int co = 0; co < CO; co++) {
+    floatx4 r = *reinterpret_cast<const floatx4 *>(&pieces[((m * 4u + a_own) * CO + co) * 64u + 4u * n]);
+    if (other) {
+      const floatx4 q = *reinterpret_cast<const floatx4 *>(&pieces[(((uint32_t)y_other * 4u + a_other) * CO + co) * 64u + 4u * n]);
+      r.x = r.x + q.x; r.y = r.y + q.y; r.z = r.z + q.z; r.w = r.w + q.w;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[co][i] = r[i] + bsum * (ny * nx[i]);
+  }
+  mt::apply_func_epilogue_many<4 * CO>(args.ep.func, &o[0][0]);
+#pragma unroll
+  for (int co = 0; co < CO; co++)
+    *reinterpret_cast<float4 *>(args.ep.C + ((size_t)img * CO + co) * OHW + (size_t)oy * 64u + 4u * n) = make_float4(o[co][0], o[co][1], o[co][2], o[co][3]);
+}
+
 // Forward convolution 3x3, stride 1, padding 1 with at most 4 output channels (an image-producing last layer) on the
 // vector ALUs, same staging: a thread computes two neighbouring output pixels for all KA channels, per input channel
 // 6 LDS reads and 18*KA multiply-adds; the 9 coefficients of (k, c) are contiguous in the kernel tensor and come
@@ -1014,12 +1160,46 @@ int launch_tconv_tile_norm(const char *name, TconvArgs &args) {
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }
-// 0 (default): the image layer runs on the vector ALUs; 1: on the matrix cores where the shape allows.  Measured on an
-// MI355X for [256,64,32,32] -> [256,3,64,64]: 35.0 us against 35.3 us (with the normalising loader 47.8 against
-// 40.3 us), so the vector-ALU kernel stays the default; the matrix-core kernel is kept selectable and tested.
-int g_image_mfma = 0;
+// Which kernel runs the image layer: 0 the vector ALUs; 1 the 4x4x1 matrix instruction where the shape allows (measured
+// on an MI355X for [256,64,32,32] -> [256,3,64,64]: 35.0 us against 35.3 us, with the normalising loader 47.8 against
+// 40.3 us: kept selectable and tested); 2 (default) products per input pixel on the 16x16x4 matrix instruction where the
+// shape allows (22.7 us, 25.1 us with the normalising loader), the vector ALUs elsewhere.
+int g_image_mfma = 2;
+template <int CO, int NORM>
+int launch_tconv_products(const char *name, const TconvArgs &args) {
+  constexpr int DEPTH = NORM == 2 || (CO == 4 && NORM != 0) ? 2 : 4;   // k steps in flight: what 128 registers hold beside the accumulators
+  static bool prepared = false;
+  const size_t lds = ((size_t)args.H * 4u * CO * 64u + (size_t)args.C / 4u * CO * 64u) * sizeof(float);   // the pieces, then the coefficients
+  if (!prepared) {
+    MT_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&tconv_k4s2_products_kernel<CO, NORM, DEPTH>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               160 * 1024));
+    prepared = true;
+  }
+  tconv_k4s2_products_kernel<CO, NORM, DEPTH><<<args.out_w, args.H * 32u, lds, mt::stream()>>>(args);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+template <int CO>
+int launch_tconv_products_norm(const char *name, const TconvArgs &args) {
+  if (!args.in_scale_shift) return launch_tconv_products<CO, 0>(name, args);
+  return args.in_func == MT_F_RELU ? launch_tconv_products<CO, 1>(name, args) : launch_tconv_products<CO, 2>(name, args);
+}
+bool products_kernel_fits(const TconvArgs &args) {
+  // (the pieces of the output rows and the coefficients share the 160 KB of LDS)
+  return args.W == 32 && args.H % 2 == 0 && args.H >= 2 && args.H <= 32 && args.C % 16 == 0 && args.M >= 1 && args.M <= 4 && args.out_w <= 0x7fffffffu &&
+         ((size_t)args.H * 4u + args.C / 4u) * args.M * 64u * sizeof(float) <= 160u * 1024u;
+}
 int launch_tconv_tile(const char *name, TconvArgs &args) {
-  if (g_image_mfma && args.W % 32 == 0 && args.C % 16 == 0 && args.M <= 4) {
+  if (g_image_mfma == 2 && products_kernel_fits(args)) {
+    mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "products per input pixel on 16x16x4, few output channels") : name);
+    switch (args.M) {
+      case 1: return launch_tconv_products_norm<1>(name, args);
+      case 2: return launch_tconv_products_norm<2>(name, args);
+      case 3: return launch_tconv_products_norm<3>(name, args);
+      default: return launch_tconv_products_norm<4>(name, args);
+    }
+  }
+  if (g_image_mfma == 1 && args.W % 32 == 0 && args.C % 16 == 0 && args.M <= 4) {
     mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, "4x4x1 matrix instructions, few output channels") : name);
     const uint32_t tiles_x = args.W / 32, tiles_y = cdiv(args.H, 8);
     const size_t blocks = (size_t)tiles_x * tiles_y * args.out_w;
@@ -1729,7 +1909,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   return false;
 }
 int set_image_mfma(int v) {
-  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "image_mfma must be 0 or 1");
+  if (v < 0 || v > 2) return fail(MT_E_ARGUMENT, "image_mfma must be 0, 1 or 2");
   g_image_mfma = v;
   return MT_OK;
 }

@@ -437,20 +437,26 @@ def test_sixteen_row_blocks_forced_on_taller_products(gpu, oracle):
 
 
 def test_image_layer_kernels_both_tilings(gpu, oracle):
-    """Transposed convolution 4x4 stride 2 padding 1 to three channels: grids below two blocks per compute unit take
-    one input pixel per thread, larger ones two; both against the oracle, with tanh and a non-zero bias."""
-    kernel, bias = Nrm(2, 1, 1, 8, 3 * 16, std=0.2), U(3, 1, 8, 1, 1) * 0.1
-    for shape in ((2, 8, 16, 20), (32, 8, 128, 128)):          # 4 and 1024 blocks of 32 x 16 pixels
-        delta = U(1, *shape)
-        out_shape = (shape[0], 3, 2 * shape[2], 2 * shape[3])
-        want = oracle.apply_func(oracle.backward_convolution(delta, kernel, bias, 4, 4, 3, 8, 2, 2, 1, 1, out_shape), "tangence")
-        got = gpu.backward_convolution(delta, kernel, bias, 4, 4, 3, 8, 2, 2, 1, 1, out_shape, func="tangence")
-        close(got, want, 1e-5)
-    # 600 blocks and a multiple of 16 input channels: the halves of a block take every other chunk of channels
-    kernel, bias = Nrm(4, 1, 1, 32, 2 * 16, std=0.2), U(5, 1, 32, 1, 1) * 0.1
-    delta = U(6, 600, 32, 16, 32)
-    want = oracle.apply_func(oracle.backward_convolution(delta, kernel, bias, 4, 4, 2, 32, 2, 2, 1, 1, (600, 2, 32, 64)), "sigmoid")
-    close(gpu.backward_convolution(delta, kernel, bias, 4, 4, 2, 32, 2, 2, 1, 1, (600, 2, 32, 64), func="sigmoid"), want, 1e-5)
+    """Transposed convolution 4x4 stride 2 padding 1 to three channels on the vector ALUs (the kernel for the shapes that
+    the matrix-core kernels leave, selected here for all of them): grids below two blocks per compute unit take one input
+    pixel per thread, larger ones two; both against the oracle, with tanh and a non-zero bias."""
+    import mi355tensor as mt
+    mt.set_option("image_mfma", 0)
+    try:
+        kernel, bias = Nrm(2, 1, 1, 8, 3 * 16, std=0.2), U(3, 1, 8, 1, 1) * 0.1
+        for shape in ((2, 8, 16, 20), (32, 8, 128, 128)):          # 4 and 1024 blocks of 32 x 16 pixels
+            delta = U(1, *shape)
+            out_shape = (shape[0], 3, 2 * shape[2], 2 * shape[3])
+            want = oracle.apply_func(oracle.backward_convolution(delta, kernel, bias, 4, 4, 3, 8, 2, 2, 1, 1, out_shape), "tangence")
+            got = gpu.backward_convolution(delta, kernel, bias, 4, 4, 3, 8, 2, 2, 1, 1, out_shape, func="tangence")
+            close(got, want, 1e-5)
+        # 600 blocks and a multiple of 16 input channels: the halves of a block take every other chunk of channels
+        kernel, bias = Nrm(4, 1, 1, 32, 2 * 16, std=0.2), U(5, 1, 32, 1, 1) * 0.1
+        delta = U(6, 600, 32, 16, 32)
+        want = oracle.apply_func(oracle.backward_convolution(delta, kernel, bias, 4, 4, 2, 32, 2, 2, 1, 1, (600, 2, 32, 64)), "sigmoid")
+        close(gpu.backward_convolution(delta, kernel, bias, 4, 4, 2, 32, 2, 2, 1, 1, (600, 2, 32, 64), func="sigmoid"), want, 1e-5)
+    finally:
+        mt.set_option("image_mfma", 2)
 
 
 def test_fused_conv_activation(gpu, oracle, path):
@@ -1002,7 +1008,42 @@ def test_image_layer_on_the_4x4x1_matrix_instructions(gpu, oracle, shape):
             Fused.BackwardConvolutionNorm(out, tx, tp, "relu", tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func="tangence")
             close(out.numpy(), want_norm, 1e-5)
     finally:
-        mt.set_option("image_mfma", 0)
+        mt.set_option("image_mfma", 2)
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 3, 8, 32), (3, 32, 3, 32, 32), (2, 64, 2, 16, 32), (1, 16, 4, 2, 32), (2, 48, 1, 6, 32), (5, 64, 3, 32, 32),
+                                   (2, 32, 4, 30, 32), (2, 16, 3, 7, 32), (2, 24, 3, 8, 32)],   # the last two: shapes it leaves to the vector-ALU kernel
+                         ids=lambda s: "x".join(str(v) for v in s))
+def test_image_layer_as_products_per_input_pixel(gpu, oracle, shape):
+    """The image layer as a product of the coefficients with the raw input pixels on the 16x16x4 matrix instruction,
+    combined along x by lane shifts and along y through LDS: against the oracle, plain and with the normalising loader
+    (ReLU and leaky ReLU), with a bias (the CPU path adds it once per contributing tap, fewer at the borders), and with
+    one input sample shared by the whole batch."""
+    import mi355tensor as mt
+    from mi355tensor import CTensor, CTensorConv, Fused
+    B, cin, cout, H, W = shape
+    x, kernel, bias = Nrm(sum(shape), B, cin, H, W), Nrm(sum(shape) + 1, 1, 1, cin, cout * 16, std=0.1), Nrm(sum(shape) + 2, 1, cin, 1, 1, std=0.05)
+    out_shape = (B, cout, 2 * H, 2 * W)
+    want = oracle.apply_func(oracle.backward_convolution(x, kernel, bias, 4, 4, cout, cin, 2, 2, 1, 1, out_shape), "tangence")
+    want_shared = oracle.backward_convolution(x[:1], kernel, bias, 4, 4, cout, cin, 2, 2, 1, 1, out_shape)
+    pairs = np.stack([U(5, 1, cin, H, W, lo=0.5, hi=1.5), U(6, 1, cin, H, W, lo=-0.5, hi=0.5)], -1)
+    u = pairs[..., 0] * x + pairs[..., 1]
+    tx, tk, tb, tp, out = CTensor.from_numpy(x), CTensor.from_numpy(kernel), CTensor.from_numpy(bias), CTensor.from_numpy(pairs.reshape(1, cin, H, 2 * W)), CTensor(*out_shape)
+    try:
+        mt.set_option("image_mfma", 2)
+        mt.CTensorMath.Fill(out, 9.0)
+        CTensorConv.BackwardConvolution(out, tx, tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func="tangence")
+        close(out.numpy(), want, 1e-5)
+        mt.CTensorMath.Fill(out, 9.0)
+        CTensorConv.BackwardConvolution(out, CTensor.from_numpy(x[:1]), tk, 4, 4, cout, cin, tb, 2, 2, 1, 1)
+        close(out.numpy(), want_shared, 1e-5)
+        for func, a in (("relu", np.maximum(u, 0)), ("leaky_relu", np.where(u > 0, u, 0.1 * u))):
+            want_norm = oracle.apply_func(oracle.backward_convolution(a.astype(np.float32), kernel, bias, 4, 4, cout, cin, 2, 2, 1, 1, out_shape), "sigmoid")
+            mt.CTensorMath.Fill(out, 9.0)
+            Fused.BackwardConvolutionNorm(out, tx, tp, func, tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func="sigmoid")
+            close(out.numpy(), want_norm, 1e-5)
+    finally:
+        mt.set_option("image_mfma", 2)
 
 
 @pytest.mark.parametrize("shape", [(256, 100, 8192, "relu"), (6, 37, 50, "leaky_relu"), (64, 128, 96, None), (255, 20, 18, "tangence"),
