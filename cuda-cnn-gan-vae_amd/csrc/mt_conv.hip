@@ -1874,6 +1874,10 @@ int &walk_order() {
   static int v = -1;
   return v;
 }
+int &walk_fair() {
+  static int v = 0x842;
+  return v;
+}
 }  // namespace igemm
 void note_write(const void *p, size_t bytes) {
   if (p == nullptr || bytes == 0) return;
@@ -1926,6 +1930,11 @@ int set_walk_blocks(int v) {
 int set_walk_order(int v) {
   if (v < -1 || v > 1) return fail(MT_E_ARGUMENT, "walk_order must be -1 (per layer), 0 (batch groups first) or 1 (row tiles first)");
   igemm::walk_order() = v;
+  return MT_OK;
+}
+int set_walk_fair(int v) {
+  if (v < 0 || v > 0xfff) return fail(MT_E_ARGUMENT, "walk_fair must be 0 or three hexadecimal digits (sixteenths of a block's steps)");
+  igemm::walk_fair() = v;
   return MT_OK;
 }
 int set_walk_tm(int v) {

@@ -33,6 +33,7 @@ struct WalkArgs {
   uint32_t px_log, qtiles, groups, per;  // PX = 1 << px_log pixels per tile; pixel tiles per phase; batch groups; steps per block
   uint32_t nk;                           // k steps of one tile (the same for every phase)
   uint32_t weights_major;                // block order, see tconv_walk_kernel
+  uint32_t fair;                         // 0, or three hexadecimal digits: sixteenths of the steps left at which a wavefront's priority drops to 2, 1, 0
   const float *delta;                    // [batch][C][H][W]
   const float *scale_shift;              // NORM: [C][H][W][2]
   int in_func;                           // NORM: none, linear, ReLU or leaky ReLU
@@ -263,7 +264,21 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   lds_barrier();
   read_half(fa[0], fb[0], 0, 0);
   uint32_t left = a.per * nk, kleft = nk;  // nk is even and at least 4, so the last four steps belong to the last group
+  // The blocks that share a compute unit (one wavefront each per SIMD) do the same work, but a SIMD serves the oldest
+  // ready wavefront first: left alone, one block runs ahead and finishes early (the first after less than half of the
+  // kernel's time), and the last ones multiply with ever fewer neighbours to cover their waits.  A wavefront therefore
+  // lowers its own priority as its work shrinks -- four levels, at 1/2, 1/4 and 1/8 of its steps left -- so whoever is
+  // behind is served first and the blocks of a compute unit stay together to the end (they also ask for the same
+  // weights at the same time).
+  uint32_t lower2 = 0, lower1 = 0, lower0 = 0;   // steps left at which the priority drops to 2, 1, 0 (even numbers)
+  if (a.fair) { lower2 = (left * ((a.fair >> 8) & 15u) / 16u) & ~1u; lower1 = (left * ((a.fair >> 4) & 15u) / 16u) & ~1u; lower0 = (left * (a.fair & 15u) / 16u) & ~1u; }
+  if (a.fair) __builtin_amdgcn_s_setprio(3);
   for (; left > 4; left -= 2) {
+    if (a.fair) {
+      if (left == lower2) __builtin_amdgcn_s_setprio(2);
+      else if (left == lower1) __builtin_amdgcn_s_setprio(1);
+      else if (left == lower0) __builtin_amdgcn_s_setprio(0);
+    }
     step(Even{}, Yes{}, Yes{}, Yes{});
     step(Odd{}, Yes{}, Yes{}, Yes{});
     kleft -= 2;
@@ -377,6 +392,7 @@ __global__ __launch_bounds__(256) void bn_finish_kernel(float *scale_shift, floa
 
 // Whether (and how) a transposed convolution can walk: fills px_log, qtiles, groups, per, nk.
 int &walk_order();    // -1 choose per layer (default), 0 batch groups first, 1 row tiles first (measurements only)
+int &walk_fair();     // 0x842 (default): wavefronts lower their priority at 8/16, 4/16, 2/16 of their steps left; 0: no priorities (measurements only)
 inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
   if (a.nphase == 0 || a.M == 0 || a.batch == 0) return false;
   const TconvPhase &p0 = a.ph[0];
@@ -407,6 +423,7 @@ inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
   a.groups = groups;
   a.per = sample_groups / groups;
   // more packed weights than an XCD's L2 holds (4 MiB), and several row tiles to deal out
+  a.fair = (uint32_t)walk_fair();
   a.weights_major = walk_order() >= 0 ? (uint32_t)walk_order() : ((uint64_t)a.nphase * a.M * p0.kp * 4u > (4u << 20) && a.tiles_m > 1 ? 1u : 0u);
   return (uint64_t)base * groups <= 0x7fffffffu;
 }
