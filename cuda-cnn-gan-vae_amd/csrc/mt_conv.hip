@@ -1874,6 +1874,10 @@ int &walk_order() {
   static int v = -1;
   return v;
 }
+int &igemm_fair() {
+  static int v = -1;
+  return v;
+}
 int &walk_fair() {
   static int v = 0x842;
   return v;
@@ -1935,6 +1939,11 @@ int set_walk_order(int v) {
 int set_walk_fair(int v) {
   if (v < 0 || v > 0xfff) return fail(MT_E_ARGUMENT, "walk_fair must be 0 or three hexadecimal digits (sixteenths of a block's steps)");
   igemm::walk_fair() = v;
+  return MT_OK;
+}
+int set_igemm_fair(int v) {
+  if (v < -1 || v > 0xfff) return fail(MT_E_ARGUMENT, "igemm_fair must be -1 (per launch), 0 or three hexadecimal digits (sixteenths of a block's steps)");
+  igemm::igemm_fair() = v;
   return MT_OK;
 }
 int set_walk_tm(int v) {

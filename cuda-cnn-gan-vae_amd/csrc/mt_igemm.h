@@ -505,6 +505,7 @@ struct Epilogue {
   const float *tap_bias = nullptr;
   int32_t ty_cnt = 0, tx_cnt = 0, offy = 0, offx = 0;
   uint32_t IH = 0, IW = 0;
+  uint32_t fair = 0;    // wavefront priorities by remaining k steps (three hexadecimal digits, sixteenths), 0: none
   int func = MT_F_NONE;
   bool accumulate = false;
   Batch bt;
@@ -793,7 +794,17 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
     prologue(std::integral_constant<int, 3>{});
     read_half(fa[0], fb[0], 0, 0);
     uint32_t left = nk;
+    uint32_t lower2 = 0, lower1 = 0, lower0 = 0;   // see tconv_walk_kernel
+    if (ep.fair) {
+      lower2 = (left * ((ep.fair >> 8) & 15u) / 16u) & ~1u; lower1 = (left * ((ep.fair >> 4) & 15u) / 16u) & ~1u; lower0 = (left * (ep.fair & 15u) / 16u) & ~1u;
+      __builtin_amdgcn_s_setprio(3);
+    }
     for (; left > 4; left -= 2) {
+      if (ep.fair) {
+        if (left == lower2) __builtin_amdgcn_s_setprio(2);
+        else if (left == lower1) __builtin_amdgcn_s_setprio(1);
+        else if (left == lower0) __builtin_amdgcn_s_setprio(0);
+      }
       step(Even{}, Yes{}, Yes{});
       step(Odd{}, Yes{}, Yes{});
     }
@@ -974,6 +985,14 @@ inline const char *shape_label(const char *name, Tile tile, uint32_t M, uint32_t
   return intern_label(name, buf);
 }
 
+int &igemm_fair();   // wavefront priorities of the one-tile kernels: -1 choose per launch (default), 0 none, else Epilogue::fair as given (measurements only)
+// A grid that the chip holds all at once (at least two blocks per compute unit) with long k loops behaves like the kernel
+// whose blocks walk over the batch: its blocks start together, and should finish together (see tconv_walk_kernel).
+inline uint32_t fair_for(Tile tile, size_t blocks, uint32_t k) {
+  if (igemm_fair() >= 0) return (uint32_t)igemm_fair();
+  const size_t per_cu = tile == T128x128 ? 2 : tile == T64x128 ? 3 : 5;
+  return blocks >= 512 && blocks <= 256 * per_cu && k >= 16 * BK ? 0x842u : 0u;
+}
 inline Tile pick_tile(uint32_t M, uint32_t N, uint32_t batches) {
   if (tile_override() >= 0) return (Tile)tile_override();
   // the 16x16x4 instruction: no half of the matrix unit multiplies padding; with few columns the narrower block of the
@@ -998,6 +1017,7 @@ int launch(const char *name, SrcA a, SrcB b, Epilogue ep, uint32_t M, uint32_t N
   const uint32_t tm = cdiv(M, bm), tn = cdiv(N, bn);
   const size_t total = (size_t)tm * tn * batches;
   if (total > 0x7fffffffu) return fail(MT_E_ARGUMENT, "%s: problem too large for one launch", name);
+  ep.fair = fair_for(tile, total, K);
   switch (tile) {
     case T128x128: igemm_kernel<2, 2, 2, 2, false><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
     case T64x128: igemm_kernel<2, 1, 1, 4, false><<<(uint32_t)total, THREADS, 0, s>>>(a, b, ep, M, N, K, tm, batches); break;
@@ -1386,6 +1406,7 @@ inline int launch_tconv(const char *name, TconvArgs &args, uint32_t max_n, size_
     fixed = fixed && taps != 0 && BK % taps == 0 && args.C % (BK / taps) == 0;
   }
   const uint32_t grid = (uint32_t)total;
+  args.ep.fair = fair_for(tile, total, args.nsplit > 1 ? args.ksplit : args.ph[0].kp);
   if (fixed) {
     switch (tile) {
       case T128x128: tconv_kernel<2, 2, 2, 2, true, false><<<grid, THREADS, 0, s>>>(args); break;

@@ -224,6 +224,7 @@ int mt_set_option(const char *name, int value) {
   if (name && strcmp(name, "walk_tm") == 0) return mt::set_walk_tm(value);
   if (name && strcmp(name, "walk_order") == 0) return mt::set_walk_order(value);
   if (name && strcmp(name, "walk_fair") == 0) return mt::set_walk_fair(value);
+  if (name && strcmp(name, "igemm_fair") == 0) return mt::set_igemm_fair(value);
   if (name && strcmp(name, "pool") == 0) {
     if (value != 0 && value != 1) return mt::fail(MT_E_ARGUMENT, "pool must be 0 (every mt_free goes to the driver) or 1");
     g_pool_on = value != 0;

@@ -105,7 +105,8 @@ int mt_set_option(const char *name, int value);
  * "tconv_walk" 1 (default) plain transposed convolutions use the kernel whose blocks walk over the batch wherever the
  * shape allows / 0 never; "walk_blocks", "walk_waves", "walk_tm", "walk_order", "walk_fair": grid size, wavefronts per SIMD, accumulators
  * per wavefront, block order (-1 per layer, 0 batch groups first, 1 row tiles first) and wavefront priorities (0 none, default 0x842: a wavefront's priority drops
- * at 8/16, 4/16 and 2/16 of its steps left) of that kernel (measurements); "image_mfma": which kernel runs the image layer of a generator
+ * at 8/16, 4/16 and 2/16 of its steps left) of that kernel (measurements); "igemm_fair" the same priorities in the one-tile matrix kernels (-1, default: where the
+ * chip holds the whole grid at once, 0 never, else as given); "image_mfma": which kernel runs the image layer of a generator
  * (transposed convolution 4x4, stride 2 to at most 4 output channels): 2 (default) products per input pixel on the 16x16x4 matrix instruction where the shape
  * allows, 1 the 4x4x1 matrix instruction where the shape allows, 0 the vector ALUs; "pool" 1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no wait) /
  * 0 every mt_free waits for the stream and returns the block to the driver; "pool_limit_mib" bytes the pool may hold.
