@@ -948,6 +948,39 @@ def test_transposed_convolution_between_batch_norms(gpu, oracle, shape, bias_std
     close(out.numpy(), oracle.apply_func(y, "relu"))
 
 
+def test_wavefront_priorities_change_no_result(gpu):
+    """The priorities that keep the blocks of a compute unit together only change which wavefront is served first: the
+    walking transposed convolution (plain and with statistics) and a one-tile product give bit-identical results with
+    them, without them and with other thresholds."""
+    import mi355tensor as mt
+    from mi355tensor import CTensor, CTensorConv, CTensorMath, Fused
+    B, cin, cout, H = 64, 128, 64, 16
+    x, kernel, bias = Nrm(1, B, cin, H, H), Nrm(2, 1, 1, cin, cout * 16, std=0.05), Nrm(3, 1, cin, 1, 1, std=0.01)
+    tx, tk, tb, out = CTensor.from_numpy(x), CTensor.from_numpy(kernel), CTensor.from_numpy(bias), CTensor(B, cout, 2 * H, 2 * H)
+    one = (1, cout, 2 * H, 2 * H)
+    left, right, prod = CTensor.from_numpy(Nrm(4, 1, 1, 1024, 2048)), CTensor.from_numpy(Nrm(5, 1, 1, 2048, 768)), CTensor(1, 1, 1024, 768)
+    results = []
+    try:
+        for walk, tile in ((0x842, -1), (0, 0), (0xc84, 0x842), (0x421, 0xfff)):
+            mt.set_option("walk_fair", walk)
+            mt.set_option("igemm_fair", tile)
+            CTensorConv.BackwardConvolution(out, tx, tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func="relu")
+            plain = out.numpy().copy()
+            t = dict(gamma=CTensor.from_numpy(U(7, *one, lo=0.5, hi=1.5)), beta=CTensor.from_numpy(U(8, *one)), scale_shift=CTensor(1, cout, 2 * H, 4 * H),
+                     batch_mean=CTensor(*one), batch_var=CTensor(*one), momentum=0.9, epsilon=seq.BN_EPSILON)
+            Fused.BackwardConvolutionNorm(out, tx, None, None, tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, bn=t)
+            CTensorMath.Mul(prod, left, right)
+            results.append((plain, out.numpy().copy(), t["scale_shift"].numpy().copy(), t["batch_var"].numpy().copy(), prod.numpy().copy()))
+    finally:
+        mt.set_option("walk_fair", 0x842)
+        mt.set_option("igemm_fair", -1)
+    for other in results[1:]:
+        for a, b in zip(results[0], other):
+            assert np.array_equal(a, b)
+    with pytest.raises(mt.TensorError):
+        mt.set_option("walk_fair", 0x1000)
+
+
 def test_statistics_in_the_epilogue_survive_a_large_mean(gpu, oracle):
     """Running mean and squared deviations (not sums of squares): an output whose mean is a hundred times its spread."""
     from mi355tensor import CTensor, Fused
