@@ -150,6 +150,18 @@ __device__ __forceinline__ float apply_func_cheap(int func, float v) {  // func 
   return v;
 }
 
+// The same for N values at once: one look at the (uniform) function, then straight-line code.
+template <int N>
+__device__ __forceinline__ void apply_func_cheap_many(int func, float *v) {
+  if (func == MT_F_RELU) {
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = v[i] > 0.f ? v[i] : 0.f;
+  } else if (func == MT_F_LEAKY_RELU) {
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = v[i] > 0.f ? v[i] : (float)(0.1 * (double)v[i]);
+  }
+}
+
 // tanh and sigmoid for the end of a compute-bound kernel (the image layer of a generator applies one of them to 24
 // values per thread; with the library routines that was a third of the kernel's vector-ALU time).  Hardware exp and
 // reciprocal: absolute error below 3e-7 against the functions above, the same results beyond their clamps.

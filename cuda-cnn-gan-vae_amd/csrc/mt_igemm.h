@@ -62,6 +62,9 @@ __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t vof
 __device__ __forceinline__ floatx2 buf_load2(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
   return __builtin_bit_cast(floatx2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0));
 }
+__device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, float v, uint32_t voff, uint32_t soff) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v), r, (int)voff, (int)soff, 0);
+}
 __device__ __forceinline__ floatx4 buf_load4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
   return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
 }

@@ -53,7 +53,9 @@ __device__ __forceinline__ void welford_merge_equal(float &mean, float &m2, floa
 }
 
 // TM: 32-row accumulators per wavefront (the block is 64*TM rows x 64 columns, 2 x 2 wavefronts)
-template <bool NORM, bool STATS, int WAVES, int TM>
+// NORM: 0 the input is used as it is, 1 ReLU(scale * x + shift), 2 any of the cheap functions of it (chosen at run time: a
+// branch per element in the loader, which the one case that generators use should not pay)
+template <int NORM, bool STATS, int WAVES, int TM>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void tconv_walk_kernel(WalkArgs a) {
   constexpr int BM = 64 * TM, BN = 64, E = 4;  // four elements per thread, operand and 64 rows
   __shared__ float4 smem4[2 * (BM + BN) * LDK / 4];
@@ -155,7 +157,10 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
     if constexpr (NORM) {
       float v[E];
 #pragma unroll
-      for (int i = 0; i < E; i++) v[i] = apply_func_cheap(in_func, rs[i].x * rb[set][i] + rs[i].y);
+      for (int i = 0; i < E; i++) {
+        const float u = rs[i].x * rb[set][i] + rs[i].y;
+        v[i] = NORM == 1 ? (u > 0.f ? u : 0.f) : apply_func_cheap(in_func, u);
+      }
       lds_put<E>(b_put + buf * BN * LDK, v);
     } else {
       lds_put<E>(b_put + buf * BN * LDK, rb[set]);
@@ -228,23 +233,35 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
     for (int r = 0; r < NS; r++) { w_mean[r] = 0.f; w_m2[r] = 0.f; }
   }
   uint32_t seen = 0;  // groups finished
+  // The output is addressed like the input, through a buffer descriptor (less than 2 GiB): the lane's first element as
+  // a 32-bit byte offset, the row of register r as a scalar offset -- no 64-bit address arithmetic per store, and one
+  // look at the output function for all sixteen values instead of a chain of branches per value.
+  const __amdgpu_buffer_rsrc_t o_rsrc = make_rsrc(a.out, a.batch * a.M * a.OHW * 4u);
+  const uint32_t row_bytes = a.OHW * 4u;
   auto flush = [&]() {
     seen++;
     const float inv_seen = 1.0f / (float)seen;
+    float v[16 * TM];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) v[16 * i + r] = acc[i][r] + extra;
+    if constexpr (STATS) {
+#pragma unroll
+      for (int e = 0; e < 16 * TM; e++) {
+        const float d = v[e] - w_mean[e];
+        w_mean[e] = w_mean[e] + d * inv_seen;
+        w_m2[e] = w_m2[e] + d * (v[e] - w_mean[e]);
+      }
+    } else {
+      apply_func_cheap_many<16 * TM>(func, v);
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const uint32_t dm = 32u * i + 8u * (r / 4) + (r & 3);
-        float v = acc[i][r] + extra;
-        if constexpr (STATS) {
-          const float d = v - w_mean[16 * i + r];
-          w_mean[16 * i + r] = w_mean[16 * i + r] + d * inv_seen;
-          w_m2[16 * i + r] = w_m2[16 * i + r] + d * (v - w_mean[16 * i + r]);
-        } else {
-          v = apply_func_cheap(func, v);
-        }
-        a.out[dst + dm * a.OHW] = v;
+        buf_store(o_rsrc, v[16 * i + r], dst * 4u, dm * row_bytes);
         acc[i][r] = 0.f;
       }
     dst += dst_step;
@@ -435,16 +452,21 @@ int &walk_tm();       // 1 or 2 accumulators per wavefront (2 where the output c
 inline int launch_tconv_walk(const char *name, const WalkArgs &a, bool norm, bool stats, uint32_t tm) {
   const uint32_t grid = a.nphase * a.tiles_m * a.qtiles * a.groups;
   hipStream_t s = stream();
+  const int n = !norm ? 0 : a.in_func == MT_F_RELU ? 1 : 2;
   if (tm == 2) {
-    if (norm && stats) tconv_walk_kernel<true, true, 2, 2><<<grid, THREADS, 0, s>>>(a);
-    else if (norm) tconv_walk_kernel<true, false, 3, 2><<<grid, THREADS, 0, s>>>(a);
-    else if (stats) tconv_walk_kernel<false, true, 3, 2><<<grid, THREADS, 0, s>>>(a);
-    else tconv_walk_kernel<false, false, 4, 2><<<grid, THREADS, 0, s>>>(a);
-  } else if (norm && stats) tconv_walk_kernel<true, true, 4, 1><<<grid, THREADS, 0, s>>>(a);
-  else if (norm) tconv_walk_kernel<true, false, 4, 1><<<grid, THREADS, 0, s>>>(a);
-  else if (stats) tconv_walk_kernel<false, true, 4, 1><<<grid, THREADS, 0, s>>>(a);
-  else if (walk_waves() == 5) tconv_walk_kernel<false, false, 5, 1><<<grid, THREADS, 0, s>>>(a);
-  else tconv_walk_kernel<false, false, 4, 1><<<grid, THREADS, 0, s>>>(a);
+    if (n == 1 && stats) tconv_walk_kernel<1, true, 2, 2><<<grid, THREADS, 0, s>>>(a);
+    else if (n == 2 && stats) tconv_walk_kernel<2, true, 2, 2><<<grid, THREADS, 0, s>>>(a);
+    else if (n == 1) tconv_walk_kernel<1, false, 3, 2><<<grid, THREADS, 0, s>>>(a);
+    else if (n == 2) tconv_walk_kernel<2, false, 3, 2><<<grid, THREADS, 0, s>>>(a);
+    else if (stats) tconv_walk_kernel<0, true, 3, 2><<<grid, THREADS, 0, s>>>(a);
+    else tconv_walk_kernel<0, false, 4, 2><<<grid, THREADS, 0, s>>>(a);
+  } else if (n == 1 && stats) tconv_walk_kernel<1, true, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  else if (n == 2 && stats) tconv_walk_kernel<2, true, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  else if (n == 1) tconv_walk_kernel<1, false, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  else if (n == 2) tconv_walk_kernel<2, false, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  else if (stats) tconv_walk_kernel<0, true, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  else if (walk_waves() == 5) tconv_walk_kernel<0, false, 5, 1><<<grid, THREADS, 0, s>>>(a);
+  else tconv_walk_kernel<0, false, 4, 1><<<grid, THREADS, 0, s>>>(a);
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }
