@@ -5,6 +5,7 @@
 // blockIdx.y is the output layer w, so a broadcast operand (w % W_operand) costs no per-element
 // division, and threads along blockIdx.x/threadIdx.x touch consecutive addresses (coalesced,
 // 16-byte vectors when S and the pointers allow it).
+#include <type_traits>
 #include "mt_common.h"
 
 namespace {
@@ -691,17 +692,25 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
   if (r >= S) return;
   const float4 mu = *reinterpret_cast<const float4 *>(col_mean + rl * 4), iv = *reinterpret_cast<const float4 *>(col_ivar + rl * 4);
   const float4 g = *reinterpret_cast<const float4 *>(gamma + r), b = *reinterpret_cast<const float4 *>(beta + r);
+  // one look at the function and at the optional output for the whole loop, not one per value
+  auto emit = [&](auto f, auto keep) {
 #pragma unroll
-  for (int i = 0; i < NW; i++) {
-    const uint32_t w = ws + i * WS;
-    if (w >= W) break;
-    float4 h, o;
-    h.x = (q[i].x - mu.x) * iv.x; h.y = (q[i].y - mu.y) * iv.y; h.z = (q[i].z - mu.z) * iv.z; h.w = (q[i].w - mu.w) * iv.w;
-    o.x = mt::apply_func_cheap(func, (g.x * h.x) + b.x); o.y = mt::apply_func_cheap(func, (g.y * h.y) + b.y);
-    o.z = mt::apply_func_cheap(func, (g.z * h.z) + b.z); o.w = mt::apply_func_cheap(func, (g.w * h.w) + b.w);
-    if (xhat) *reinterpret_cast<float4 *>(xhat + (size_t)w * S + r) = h;
-    *reinterpret_cast<float4 *>(out + (size_t)w * S + r) = o;
-  }
+    for (int i = 0; i < NW; i++) {
+      const uint32_t w = ws + i * WS;
+      if (w >= W) break;
+      float4 h, o;
+      h.x = (q[i].x - mu.x) * iv.x; h.y = (q[i].y - mu.y) * iv.y; h.z = (q[i].z - mu.z) * iv.z; h.w = (q[i].w - mu.w) * iv.w;
+      o.x = f((g.x * h.x) + b.x); o.y = f((g.y * h.y) + b.y); o.z = f((g.z * h.z) + b.z); o.w = f((g.w * h.w) + b.w);
+      if constexpr (decltype(keep)::value) *reinterpret_cast<float4 *>(xhat + (size_t)w * S + r) = h;
+      *reinterpret_cast<float4 *>(out + (size_t)w * S + r) = o;
+    }
+  };
+  auto with_func = [&](auto keep) {
+    if (func == MT_F_RELU) emit([](float v) { return v > 0.f ? v : 0.f; }, keep);
+    else if (func == MT_F_LEAKY_RELU) emit([](float v) { return v > 0.f ? v : (float)(0.1 * (double)v); }, keep);
+    else emit([](float v) { return v; }, keep);
+  };
+  if (xhat) with_func(std::true_type{}); else with_func(std::false_type{});
 }
 
 // Backward pass of the same layer in one kernel (netlayer/cnetlayerbatchnormalization.cu.h:578-604):
