@@ -904,25 +904,29 @@ __device__ __forceinline__ void igemm_body(SrcA &a, SrcB &b, const Epilogue &ep,
       }
     }
     const bool whole = m4 + 4 <= M && M % 4 == 0;   // the lane's four rows are one aligned 16-byte piece of a sample
+    // xhat in place of the centred values, then the outputs: one look at the function for all of them
+    float o[2 * TN][4];
+#pragma unroll
+    for (int j = 0; j < 2 * TN; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        v[j][r] = v[j][r] * iv[r];
+        o[j][r] = gamma_r[r] * v[j][r] + beta_r[r];
+      }
+    apply_func_epilogue_many<8 * TN>(ep.func, &o[0][0]);
 #pragma unroll
     for (int j = 0; j < 2 * TN; j++) {
       if (!ok[j]) continue;
       const size_t at = (size_t)(n0 + wn * TN * 32 + j * 16 + lrow) * M + m4;   // output [batch][features]
-      float xh[4], o[4];
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        xh[r] = v[j][r] * iv[r];
-        o[r] = apply_func_epilogue(ep.func, gamma_r[r] * xh[r] + beta_r[r]);
-      }
       if (whole) {
-        *reinterpret_cast<float4 *>(ep.C + at) = make_float4(o[0], o[1], o[2], o[3]);
-        if (bn.xhat) *reinterpret_cast<float4 *>(bn.xhat + at) = make_float4(xh[0], xh[1], xh[2], xh[3]);
+        *reinterpret_cast<float4 *>(ep.C + at) = make_float4(o[j][0], o[j][1], o[j][2], o[j][3]);
+        if (bn.xhat) *reinterpret_cast<float4 *>(bn.xhat + at) = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
       } else {
 #pragma unroll
         for (int r = 0; r < 4; r++)
           if (m4 + r < M) {
-            ep.C[at + r] = o[r];
-            if (bn.xhat) bn.xhat[at + r] = xh[r];
+            ep.C[at + r] = o[j][r];
+            if (bn.xhat) bn.xhat[at + r] = v[j][r];
           }
       }
     }
