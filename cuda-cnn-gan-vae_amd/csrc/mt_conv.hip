@@ -119,8 +119,17 @@ bool written_by_a_graph(const PackKey &k) {
   return false;
 }
 
+// Buffers of evicted entries that a recorded graph may still name: they stay allocated, are counted
+// ("pack_cache_spare_bytes") and serve the same key again when it comes back.
+std::vector<PackEntry> g_pack_spare;
+
 void drop_entry(size_t i) {  // the stream is idle
-  if (!g_packs[i].pinned) (void)hipFree(g_packs[i].buf);   // a pinned buffer stays allocated: a graph may still name it
+  if (g_packs[i].pinned) {
+    g_packs[i].valid = false;
+    g_pack_spare.push_back(g_packs[i]);
+  } else {
+    (void)hipFree(g_packs[i].buf);
+  }
   g_packs.erase(g_packs.begin() + i);
 }
 
@@ -155,8 +164,17 @@ int pack_buffer(const PackKey &key, size_t floats, float **buf, bool *fresh) {
   }
   PackEntry e;
   e.key = key; e.floats = floats; e.valid = true; e.used = g_pack_clock;
-  MT_HIP(hipMalloc((void **)&e.buf, floats * sizeof(float)));
-  mt::count_driver_allocation();
+  for (size_t i = 0; i < g_pack_spare.size(); i++)
+    if (g_pack_spare[i].key == key && g_pack_spare[i].floats == floats) {  // the buffer a graph still names: the same weights again
+      e.buf = g_pack_spare[i].buf;
+      e.pinned = true;
+      g_pack_spare.erase(g_pack_spare.begin() + i);
+      break;
+    }
+  if (e.buf == nullptr) {
+    MT_HIP(hipMalloc((void **)&e.buf, floats * sizeof(float)));
+    mt::count_driver_allocation();
+  }
   g_packs.push_back(e);
   g_pack_made++;
   *buf = e.buf;
@@ -1576,11 +1594,11 @@ int backward_between_norms(const char *name, const mt_tensor *out, const mt_tens
       return mt::fail(MT_E_SHAPE, "%s: the (scale, shift) pairs of the output must be [1,%u,%u,%u]", name, out->z, out->y, 2 * out->x);
     for (auto t : {bn->scale_shift, bn->ivar, bn->mean, bn->var, bn->new_mean, bn->new_var}) mt::note_write(t);
   }
+  if (!scale_shift && !bn) return backward(name, out, delta, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);  // nothing folded in: the plain call, once
   NormIn norm{scale_shift ? scale_shift->p : nullptr, delta_func};
   bool handled = false;
   int rc = backward(name, out, delta, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func, scale_shift ? &norm : nullptr, bn, &handled);
   if (rc || handled) return rc;
-  if (!scale_shift && !bn) return backward(name, out, delta, kernel, kx, ky, kz, ka, bias, sx, sy, px, py, func);
   mt_tensor in = *delta;
   if (scale_shift && mt::count(delta)) {
     float *tmp = nullptr;
@@ -1914,6 +1932,9 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "pack_cache_hits") == 0) { *value = (int64_t)g_pack_hits; return true; }
   if (strcmp(name, "pack_cache_made") == 0) { *value = (int64_t)g_pack_made; return true; }
   if (strcmp(name, "pack_cache_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_packs) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
+  if (strcmp(name, "pack_cache_spare_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_pack_spare) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
+  if (strcmp(name, "graph_written_ranges") == 0) { *value = (int64_t)g_graph_written.size(); return true; }
+  if (strcmp(name, "graph_writes_anything") == 0) { *value = g_graph_writes_anything ? 1 : 0; return true; }
   return false;
 }
 int set_image_mfma(int v) {

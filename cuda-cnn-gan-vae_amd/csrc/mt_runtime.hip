@@ -108,20 +108,40 @@ size_t g_pool_limit = (size_t)4 << 30;                // bytes the pool may hold
 size_t g_pool_bytes = 0;
 bool g_pool_on = true;
 uint64_t g_pool_reused = 0;
-std::unordered_map<void *, size_t> g_block_size;      // every live or pooled block of mt_malloc
+// A block is LIVE (the caller holds it), POOLED (free, waiting for the next mt_malloc of its size) or RETIRED: freed
+// while the stream was being captured, or handed out during a capture.  A recorded graph names such a block's address
+// in its kernels, and every replay writes there again; handing the block to another tensor would let replays scribble
+// over it.  A retired block stays allocated and is never handed out again (the cost of recording a sequence that creates
+// temporaries: its temporaries, once per recording).
+enum BlockState : uint8_t { LIVE, POOLED, RETIRED };
+struct Block {
+  size_t size;
+  BlockState state;
+  bool in_capture;  // handed out while the stream was being captured
+};
+std::unordered_map<void *, Block> g_blocks;           // every block mt_malloc ever got from the driver and still holds
 std::map<size_t, std::vector<void *>> g_pool;         // free blocks by size
+size_t g_retired_blocks = 0, g_retired_bytes = 0;
 
+bool capturing_now() {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (g_stream != nullptr) (void)hipStreamIsCapturing(g_stream, &capture);
+  return capture != hipStreamCaptureStatusNone;
+}
+
+// gives every pooled block back to the driver; the bookkeeping is complete before a failure is reported
 int pool_release_all() {
   if (g_pool_bytes == 0) return MT_OK;
-  MT_HIP(hipStreamSynchronize(g_stream));
+  hipError_t first = hipStreamSynchronize(g_stream);
   for (auto &kv : g_pool)
     for (void *p : kv.second) {
-      g_block_size.erase(p);
-      MT_HIP(hipFree(p));
+      g_blocks.erase(p);
+      const hipError_t e = hipFree(p);
+      if (first == hipSuccess) first = e;
     }
   g_pool.clear();
   g_pool_bytes = 0;
-  return MT_OK;
+  return first == hipSuccess ? MT_OK : mt::hip_fail(first, "returning pooled blocks to the driver");
 }
 }  // namespace
 
@@ -131,16 +151,20 @@ int mt_malloc(void **ptr, size_t bytes) {
   *ptr = nullptr;
   if (bytes == 0) return MT_OK;
   const size_t size = (bytes + POOL_GRANULE - 1) / POOL_GRANULE * POOL_GRANULE;
+  const bool capturing = capturing_now();
   auto it = g_pool.find(size);
   if (it != g_pool.end() && !it->second.empty()) {
     *ptr = it->second.back();
     it->second.pop_back();
     g_pool_bytes -= size;
     g_pool_reused++;
+    Block &b = g_blocks[*ptr];
+    b.state = LIVE;
+    b.in_capture = capturing;
     return MT_OK;
   }
   hipError_t e = hipMalloc(ptr, size);
-  if (e == hipErrorOutOfMemory && g_pool_bytes) {
+  if (e == hipErrorOutOfMemory && g_pool_bytes && !capturing) {
     (void)hipGetLastError();
     int rc = pool_release_all();
     if (rc) return rc;
@@ -148,26 +172,34 @@ int mt_malloc(void **ptr, size_t bytes) {
   }
   if (e != hipSuccess) { *ptr = nullptr; return mt::hip_fail(e, "hipMalloc"); }
   g_driver_allocs++;
-  g_block_size[*ptr] = size;
+  g_blocks[*ptr] = Block{size, LIVE, capturing};
   return MT_OK;
 }
 
 int mt_free(void *ptr) {
   if (ptr == nullptr) return MT_OK;
-  auto it = g_block_size.find(ptr);
-  const size_t size = it == g_block_size.end() ? 0 : it->second;
+  auto it = g_blocks.find(ptr);
+  if (it != g_blocks.end() && it->second.state != LIVE)
+    return mt::fail(MT_E_ARGUMENT, "mt_free: block %p was freed already (%s)", ptr, it->second.state == POOLED ? "it waits in the pool" : "a recorded graph holds it");
+  const size_t size = it == g_blocks.end() ? 0 : it->second.size;
   // whatever was derived from the block's contents (re-ordered weights) must not outlive it: the address may come back
   mt::note_write(ptr, size ? size : ~(size_t)0 - (size_t)(uintptr_t)ptr);
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  if (g_stream != nullptr) (void)hipStreamIsCapturing(g_stream, &capture);
+  const bool capturing = capturing_now();
+  if (it != g_blocks.end() && (capturing || it->second.in_capture)) {
+    it->second.state = RETIRED;  // a recorded graph may write here on every replay
+    g_retired_blocks++;
+    g_retired_bytes += size;
+    return MT_OK;
+  }
   if (g_pool_on && size && size <= POOL_LARGEST) {
-    if (g_pool_bytes + size > g_pool_limit && capture == hipStreamCaptureStatusNone) { int rc = pool_release_all(); if (rc) return rc; }
+    if (g_pool_bytes + size > g_pool_limit) { int rc = pool_release_all(); if (rc) return rc; }
+    it->second.state = POOLED;
     g_pool[size].push_back(ptr);
     g_pool_bytes += size;
     return MT_OK;
   }
-  if (it != g_block_size.end()) g_block_size.erase(it);
-  if (capture == hipStreamCaptureStatusNone) MT_HIP(hipStreamSynchronize(g_stream));  // queued kernels may still use it
+  if (it != g_blocks.end()) g_blocks.erase(it);
+  if (!capturing) MT_HIP(hipStreamSynchronize(g_stream));  // queued kernels may still use it
   MT_HIP(hipFree(ptr));
   return MT_OK;
 }
@@ -293,6 +325,8 @@ int mt_get_info(const char *name, int64_t *value) {
   if (strcmp(name, "pool_reused") == 0) { *value = (int64_t)g_pool_reused; return MT_OK; }
   if (strcmp(name, "driver_allocations") == 0) { *value = (int64_t)g_driver_allocs; return MT_OK; }
   if (strcmp(name, "retired_workspaces") == 0) { *value = (int64_t)mt::retired_workspaces(); return MT_OK; }
+  if (strcmp(name, "retired_blocks") == 0) { *value = (int64_t)g_retired_blocks; return MT_OK; }
+  if (strcmp(name, "retired_bytes") == 0) { *value = (int64_t)g_retired_bytes; return MT_OK; }
   if (mt::pack_cache_info(name, value)) return MT_OK;
   return mt::fail(MT_E_ARGUMENT, "mt_get_info: unknown name '%s'", name);
 }

@@ -93,26 +93,47 @@ int mt_timer_create(void **timer);
 int mt_timer_start(void *timer);
 int mt_timer_stop(void *timer, float *milliseconds);
 int mt_timer_destroy(void *timer);
-/* "conv_path": 0 choose per shape (default), 1 one-thread-per-output kernels in the CPU path's summation order,
- * 2 matrix-core kernels wherever they apply.  "igemm_tile": -1 choose per shape (default), 0..4 force the block
- * tile 128x128 / 64x128 / 32x128 / 64x64 / 16x256 of the matrix-core kernels (a forced tile also switches off the
- * kernels that are chosen by shape beside them).  "patch_blocks": persistent blocks of the input-patch transposed
- * convolution (default 512, two per compute unit).  "wgrad_groups": 0 choose per shape (default),
- * n split the batch of mt_convolution_backward_weights_sum into n groups (when n divides the batch).  For tests and
- * measurements; results agree within fp32 rounding. */
+/* Options, for tests and measurements (results agree within fp32 rounding whatever is chosen).  No counterpart in the
+ * reference.  One line per option: name, values, meaning.
+ *   "conv_path"      0 (default) choose per shape / 1 one-thread-per-output kernels in the CPU path's summation order /
+ *                    2 matrix-core kernels wherever they apply
+ *   "igemm_tile"     -1 (default) choose per shape / 0..4 force the block tile 128x128, 64x128, 32x128, 64x64, 16x256 of the
+ *                    matrix-core kernels (a forced tile also switches off the kernels chosen by shape beside them)
+ *   "igemm_fair"     -1 (default) falling wavefront priorities where the chip holds the whole grid at once / 0 never /
+ *                    three hexadecimal digits: sixteenths of a block's k steps left at which the priority drops to 2, 1, 0
+ *   "split_reduce"   1 (default) the block that finishes last adds the partial results of a product split over k (or over
+ *                    batch groups) in a fixed order / 0 a separate launch adds them
+ *   "patch_blocks"   persistent blocks of the input-patch transposed convolution (default 512, two per compute unit)
+ *   "wgrad_groups"   0 (default) choose per shape / n split the batch of mt_convolution_backward_weights_sum into n groups
+ *                    (when n divides the batch)
+ *   "pack_cache"     1 (default) keep re-ordered weights between calls / 0 re-order on every call
+ *   "tconv_walk"     1 (default) plain transposed convolutions use the kernel whose blocks walk over the batch wherever
+ *                    the shape allows / 0 never
+ *   "conv_walk"      1 (default) forward convolutions whose taps tile the k step use the same walking kernel wherever the
+ *                    shape allows / 0 never
+ *   "walk_blocks"    blocks wanted per launch of the walking kernel (default 1024)
+ *   "walk_waves"     4 (default) or 5 wavefronts per SIMD for its plain variant
+ *   "walk_tm"        1 (default) or 2 accumulators per wavefront
+ *   "walk_order"     -1 (default) per layer / 0 batch groups first / 1 row tiles first
+ *   "walk_fair"      0x842 (default): a wavefront's priority drops at 8/16, 4/16 and 2/16 of its steps left / 0 none
+ *   "image_mfma"     kernel of a generator's image layer (transposed convolution 4x4, stride 2, to at most 4 channels):
+ *                    2 (default) products per input pixel on the 16x16x4 matrix instruction where the shape allows /
+ *                    1 the 4x4x1 matrix instruction where the shape allows / 0 the vector ALUs
+ *   "pool"           1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no
+ *                    wait) / 0 every mt_free waits for the stream and returns the block to the driver
+ *   "pool_limit_mib" MiB the pool may hold in free blocks (default 4096) */
 int mt_set_option(const char *name, int value);
-/* More options: "pack_cache" 1 (default) keep re-ordered weights between calls / 0 re-order on every call;
- * "tconv_walk" 1 (default) plain transposed convolutions use the kernel whose blocks walk over the batch wherever the
- * shape allows / 0 never; "walk_blocks", "walk_waves", "walk_tm", "walk_order", "walk_fair": grid size, wavefronts per SIMD, accumulators
- * per wavefront, block order (-1 per layer, 0 batch groups first, 1 row tiles first) and wavefront priorities (0 none, default 0x842: a wavefront's priority drops
- * at 8/16, 4/16 and 2/16 of its steps left) of that kernel (measurements); "igemm_fair" the same priorities in the one-tile matrix kernels (-1, default: where the
- * chip holds the whole grid at once, 0 never, else as given); "image_mfma": which kernel runs the image layer of a generator
- * (transposed convolution 4x4, stride 2 to at most 4 output channels): 2 (default) products per input pixel on the 16x16x4 matrix instruction where the shape
- * allows, 1 the 4x4x1 matrix instruction where the shape allows, 0 the vector ALUs; "pool" 1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no wait) /
- * 0 every mt_free waits for the stream and returns the block to the driver; "pool_limit_mib" bytes the pool may hold.
- * mt_get_info reads counters of the runtime, for tests and measurements (no counterpart in the reference):
- * "pool_bytes", "pool_reused", "driver_allocations", "retired_workspaces", "pack_cache_entries", "pack_cache_valid",
- * "pack_cache_hits", "pack_cache_made", "pack_cache_bytes". */
+/* Counters of the runtime, for tests and measurements (no counterpart in the reference):
+ *   "pool_bytes", "pool_reused", "driver_allocations"      the memory pool behind mt_malloc / mt_free
+ *   "retired_blocks", "retired_bytes"                      blocks freed (or handed out) while the stream was being captured:
+ *                                                          a recorded graph names them, so they are never handed out again
+ *   "retired_workspaces"                                   outgrown workspaces that a recorded graph may still use
+ *   "pack_cache_entries", "pack_cache_valid", "pack_cache_hits", "pack_cache_made", "pack_cache_bytes"
+ *                                                          the re-ordered weights kept between calls
+ *   "pack_cache_spare_bytes"                               buffers of evicted entries that a recorded graph still names
+ *   "graph_written_ranges", "graph_writes_anything"        memory written by recorded calls: weights inside such a range
+ *                                                          are re-ordered on every use; after 4096 ranges everything is
+ *                                                          (graph_writes_anything = 1, for the rest of the process) */
 int mt_get_info(const char *name, int64_t *value);
 
 /* ---- convolutions: CTensorConv<T> (cuda/ctensorconv.cu.h:63-66) ---- */
@@ -256,7 +277,8 @@ int mt_batchnorm_forward_train_func(const mt_tensor *output, const mt_tensor *in
 int mt_batchnorm_forward_train_func_noalloc(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
                                             const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var,
                                             const mt_tensor *new_mean, const mt_tensor *new_variable, float momentum, float epsilon, int func);
-/* The same layer in inference mode (lines 326-371): stored mean / variable instead of batch statistics. */
+/* The same layer in inference mode (netlayer/cnetlayerbatchnormalization.cu.h:326-371): stored mean / variable instead of
+ * batch statistics. */
 int mt_batchnorm_forward_infer_func(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
                                     const mt_tensor *mean, const mt_tensor *variable, float epsilon, int func);
 

@@ -182,6 +182,62 @@ def test_pool_reuses_blocks_in_stream_order(mt):
     mt.set_option("pool", 1)
 
 
+def test_temporaries_of_a_recording_are_never_handed_out_again(mt):
+    """A recorded sequence that creates and frees a temporary, as the reference's layers do on every backward call
+    (netlayer/cnetlayerconvolution.cu.h:494): the graph's kernels name the temporary's address, so its block must not
+    serve another tensor afterwards -- replays would write over that tensor.  A block freed twice is refused."""
+    from mi355tensor import CTensor, CTensorMath as M, Graph
+    shape = (1, 1, 1 << 10, 1 << 10)
+    a = CTensor.from_numpy(np.arange(1 << 20, dtype=np.float32).reshape(shape) % 977.0)
+    out = CTensor(*shape)
+    seen = {}
+
+    def step():
+        tmp = CTensor(*shape)
+        seen["ptr"] = tmp.ptr.value
+        M.Set(tmp, a, 2.0, 1.0)
+        M.Add(out, tmp, a, 1.0, 1.0)
+        tmp.free()
+
+    step()                                       # eager first: the temporary's block now waits in the pool
+    want = out.numpy()
+    retired = mt.get_info("retired_blocks")
+    graph = Graph(step)
+    assert mt.get_info("retired_blocks") == retired + 1
+    later = [CTensor(*shape) for _ in range(3)]  # same size as the temporary
+    assert all(t.ptr.value != seen["ptr"] for t in later)
+    for t in later:
+        M.Fill(t, 7.0)
+    for _ in range(3):
+        M.Fill(out, 0.0)
+        graph.launch()
+        assert np.array_equal(out.numpy(), want)
+        for t in later:
+            assert np.array_equal(t.numpy(), np.full(shape, 7.0, np.float32))
+    # a block handed out during a recording is retired when it is freed later, too
+    held = {}
+
+    def allocate_only():
+        held["t"] = CTensor(*shape)
+        M.Set(held["t"], a, 1.0, 0.0)
+
+    graph2 = Graph(allocate_only)
+    ptr = held["t"].ptr.value
+    retired = mt.get_info("retired_blocks")
+    held["t"].free()
+    assert mt.get_info("retired_blocks") == retired + 1
+    again = CTensor(*shape)
+    assert again.ptr.value != ptr
+    del graph2
+    # double free: the second call names a block that waits in the pool
+    t = CTensor(1, 1, 8, 8)
+    raw = C.c_void_p(t.ptr.value)
+    t.free()
+    with pytest.raises(mt.TensorError) as e:
+        mt.call("mt_free", raw)
+    assert "freed already" in str(e.value)
+
+
 def test_workspace_growth_around_a_recording(mt):
     """A request that outgrows a workspace while the stream is captured is refused with a message; a workspace that a
     recording has seen is kept alive when a later call outgrows it."""
