@@ -142,7 +142,7 @@ def memory_bound_ops(args):
 
 def discriminator_step(args):
     """Secondary workload (configs[4]): forward, backward and Adam update of the DCGAN-64 discriminator at batch 128
-    through the fused entry points.  Same two timed regions as the main workload; one JSON line."""
+    through the fused entry points.  Same two timed regions as the main workload; returns the JSON object."""
     import mi355tensor as mt
     import discriminator as D
     batch = 128
@@ -183,7 +183,7 @@ def discriminator_step(args):
     conv = {k: v for k, v in prof.items() if k.startswith(("mt_forward_convolution", "mt_backward_convolution", "mt_convolution_backward_weights_sum"))}
     conv_ms = sum(v[1] for v in conv.values()) / args.steps
     flop = 3.0 * sum(D.conv_flops(batch))   # forward, input gradient, weight gradient
-    print(json.dumps({
+    return ({
         "metric": "images/sec, DCGAN-64 discriminator training step fp32 b=128 (secondary workload)",
         "value": batch / (ms_per_step * 1e-3), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
@@ -197,13 +197,16 @@ def discriminator_step(args):
         "kernel_ms_per_step_sum": sum(v[1] for v in prof.values()) / args.steps,
         "conv_gflops": flop / (conv_ms * 1e-3) / 1e9, "conv_ms_per_step": conv_ms,
         "conv_frac_of_fp32_mfma_peak": flop / (conv_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
-        "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}}))
+        "gflop_per_step": {"conv": flop / 1e9},
+        "tflops_over_the_step": flop / (ms_per_step * 1e-3) / 1e12,
+        "frac_of_fp32_mfma_peak_over_the_step": flop / (ms_per_step * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+        "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}})
 
 
 def secondary_forward(args):
     """Secondary workloads configs[0], configs[1], configs[3]: one forward pass per step, timed twice -- recorded once as a
     HIP graph and replayed, and issued call by call from Python -- the faster of the two is the step; then the steps with
-    per-kernel events."""
+    per-kernel events.  Returns the JSON object."""
     import numpy as np
     import mi355tensor as mt
     from mi355tensor import CTensor, CTensorConv, Fused
@@ -295,7 +298,7 @@ def secondary_forward(args):
         gpu_ms, wall_ms = eager_gpu_ms, eager_wall_ms
     kernel_ms = sum(v[1] for v in prof.values()) / args.steps
     total = sum(flop.values())
-    print(json.dumps({
+    return ({
         "metric": "images/sec, forward fp32 (secondary workload)" if args.workload != "c2" else "samples/sec, forward fp32 (secondary workload)",
         "value": batch / (ms_per_step * 1e-3), "unit": "images/s" if args.workload != "c2" else "samples/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
@@ -305,7 +308,27 @@ def secondary_forward(args):
         "gflop_per_step": dict({k: v / 1e9 for k, v in flop.items()}, **extra),
         "tflops_over_the_step": total / (ms_per_step * 1e-3) / 1e12,
         "frac_of_fp32_mfma_peak_over_the_step": total / (ms_per_step * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
-        "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}}))
+        "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])}})
+
+
+def secondary_workloads(steps, warmup):
+    """The other configurations and the shipped GAN generator, a few hundred steps each, in this process after the
+    measured workload: {name: {ms_per_step, tflops, frac_of_fp32_mfma_peak, ...}} for the `secondary` object of the
+    default run's JSON line.  Algorithmic FLOP over the whole step, convolution kernels beside it where they dominate."""
+    out = {}
+    for wl in ("c1", "c2", "c4", "c5", "gan"):
+        a = argparse.Namespace(workload=wl, steps=steps, warmup=warmup, literal=False)
+        full = discriminator_step(a) if wl == "c5" else secondary_forward(a)
+        brief = {"workload": full["config"]["workload"], "steps": steps, "warmup": warmup, "ms_per_step": full["ms_per_step"],
+                 "value": full["value"], "unit": full["unit"], "gflop_per_step": sum(v for k, v in full["gflop_per_step"].items() if not k.startswith("conv_gflop_as")),
+                 "tflops": full["tflops_over_the_step"], "frac_of_fp32_mfma_peak": full["frac_of_fp32_mfma_peak_over_the_step"],
+                 "path": full["config"]["path"]}
+        if "conv_frac_of_fp32_mfma_peak" in full:
+            brief["conv_kernels_frac_of_fp32_mfma_peak"] = full["conv_frac_of_fp32_mfma_peak"]
+        top = sorted(full["kernels_ms_per_step"].items(), key=lambda kv: -kv[1])[:4]
+        brief["largest_kernels_ms_per_step"] = {k: round(v, 5) for k, v in top}
+        out[wl] = brief
+    return out
 
 
 def main():
@@ -316,6 +339,8 @@ def main():
     ap.add_argument("--cpu-sample-batch", type=int, default=40,
                     help="images of the CPU baseline sample (about 0.3 s each on one core)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true", help="workload c3: leave out the `secondary` object (the other configurations, about 3 s)")
+    ap.add_argument("--secondary-steps", type=int, default=200, help="steps per secondary workload inside the default run")
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also launch one plain copy (mt_set) of this many MiB before the timed region: the known-size kernel "
                          "that calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -349,11 +374,15 @@ def main():
             name, value = item.split("=")
             mt_.set_option(name, int(value))
     if args.workload == "c5":
-        return discriminator_step(args)
+        return print(json.dumps(discriminator_step(args)))
     if args.workload == "ops":
         return memory_bound_ops(args)
     if args.workload in ("c1", "c2", "c4", "gan"):
-        return secondary_forward(args)
+        return print(json.dumps(secondary_forward(args)))
+
+    # The CPU baseline runs first (about 12 s of host work), so that everything that follows is GPU work back to back:
+    # a coarse GPU-busy sample taken from outside during the second half of the run sees the GPU at work.
+    baseline = None if args.no_cpu_baseline else cpu_baseline(args.cpu_sample_batch)
 
     import mi355tensor as mt
     import generator as G
@@ -496,8 +525,12 @@ def main():
                      "per_layer": {b[0]: {"avg_launch_ms": b[2] / b[1], "tflops": b[3] / (b[2] / b[1] * 1e-3) / 1e12} for b in big}},
         "kernels_ms_per_step": {k: v[1] / args.steps for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])},
     }
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch)
+    if baseline is not None:
+        result["cpu_baseline"] = baseline
+    if not args.no_secondary:
+        # the other configurations, measured by the same process right after the measured workload (python bench.py --workload
+        # c1|c2|c4|c5|gan prints each one's full line)
+        result["secondary"] = secondary_workloads(args.secondary_steps, 20)
     print(json.dumps(result))
 
 

@@ -25,6 +25,7 @@ using namespace mt::igemm;
 using mt::cdiv;
 
 int g_conv_path = 0;  // 0 auto, 1 direct, 2 implicit GEMM wherever it applies
+int g_conv_walk = 1;   // forward convolutions whose taps tile the k step: 0 never on the kernel whose blocks walk over the batch, 1 wherever the shape allows and gives 512 blocks, 2 wherever the shape allows
 int g_wgrad_groups = 0;  // 0 auto, else the number of batch groups of the batch-summed weight gradient (if it divides the batch)
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
@@ -1349,6 +1350,28 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
     return MT_OK;
   }
   uint32_t OHW = out->y * out->x;
+  // Taps that tile the k step (4x4, 2x2, 1x1 kernels), one kernel and bias set, whole 64-channel row tiles: the kernel whose
+  // blocks walk over the batch runs it (see mt_walk.h) when that gives at least two blocks per compute unit; products
+  // with fewer tiles and a long k axis are better cut over k (launch_split below).
+  if (g_conv_walk && kernel->w == 1 && bias->w == 1 && image->w == out->w && mt::igemm::tile_override() < 0 && BK % ((uint32_t)ky * kx) == 0 &&
+      ((uintptr_t)kernel->p & 15u) == 0 && mt::fits_buffer(out)) {
+    WalkArgs walk{};
+    walk.nphase = 1;
+    walk.ph[0] = TconvPhase{kernel->p, K, kernel->x, out->y, out->x, ky, kx, -py, -px, 0u, 0u};
+    walk.M = ka; walk.batch = out->w;
+    walk.delta = image->p; walk.C = (uint32_t)kz; walk.H = image->y; walk.W = image->x;
+    walk.in_sy = (uint32_t)sy; walk.in_sx = (uint32_t)sx;
+    walk.out = out->p; walk.OW = out->x; walk.OHW = OHW; walk.sy = 1; walk.sx = 1;
+    walk.row_bias = bias->p; walk.tap_bias = nullptr;
+    walk.func = mt::epilogue_func(func) ? func : MT_F_NONE;
+    if (tconv_walk_plan(walk, (uint32_t)mt::igemm::walk_blocks(), 1) && ((size_t)walk.tiles_m * walk.qtiles * walk.groups >= 512 || g_conv_walk == 2)) {
+      {
+        mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, out->w * OHW, K, 1) : name);
+        if ((rc = launch_tconv_walk(name, walk, false, false, 1))) return rc;
+      }
+      return mt::epilogue_func(func) ? MT_OK : mt_apply_func(out, out, func);
+    }
+  }
   SrcIm2col b{};
   b.p = image->p; b.in_w = image->w; b.C = kz; b.H = image->y; b.W = image->x; b.KY = ky; b.KX = kx; b.OHW = OHW; b.OW = out->x; b.K = K;
   b.sy = sy; b.sx = sx; b.py = py; b.px = px;
@@ -1945,6 +1968,11 @@ int set_image_mfma(int v) {
 int set_tconv_walk(int v) {
   if (v < 0 || v > 1) return fail(MT_E_ARGUMENT, "tconv_walk must be 0 (never for plain calls) or 1 (wherever the shape allows)");
   g_tconv_walk = v;
+  return MT_OK;
+}
+int set_conv_walk(int v) {
+  if (v < 0 || v > 2) return fail(MT_E_ARGUMENT, "conv_walk must be 0 (never), 1 (wherever the shape allows and the grid fills the chip) or 2 (wherever the shape allows)");
+  g_conv_walk = v;
   return MT_OK;
 }
 int set_walk_blocks(int v) {

@@ -1,6 +1,8 @@
 // Transposed convolution on the fp32 matrix cores whose blocks walk over the batch, with the two halves of a batch
 // normalisation folded into it: the statistics of the layer's own output (epilogue) and the normalisation + activation
-// that its input still owes (loader).
+// that its input still owes (loader).  A forward convolution whose taps tile the k step (4x4, 2x2, 1x1 kernels) is the
+// same kernel with one "phase": the operand is gathered with the convolution's stride (in_sy, in_sx), the weights are
+// the layer's kernel tensor as it is, and every output channel has its bias (ROWBIAS).
 //
 // A block owns one stride phase, 64 output channels and one tile of PX pixels x SP samples (PX * SP = 64 columns), and
 // walks from one group of SP samples to the next, `per` groups in all.  Going to the next group changes nothing but a
@@ -40,6 +42,8 @@ struct WalkArgs {
   uint32_t C, H, W;
   float *out;                            // [batch][M][OH][OW]
   uint32_t OW, OHW, sy, sx;
+  uint32_t in_sy = 1, in_sx = 1;         // stride of the gather: input pixel = output pixel * stride + offset + tap (1 for a transposed convolution)
+  const float *row_bias = nullptr;       // ROWBIAS: one value per output channel, [M]
   const float *tap_bias;                 // sum of the filters' biases, added once per contributing tap (may be null)
   int func;                              // applied to the output (cheap functions only); with STATS: none
   float *part_mean, *part_m2;            // STATS: [groups][M * OHW] each
@@ -55,7 +59,7 @@ __device__ __forceinline__ void welford_merge_equal(float &mean, float &m2, floa
 // TM: 32-row accumulators per wavefront (the block is 64*TM rows x 64 columns, 2 x 2 wavefronts)
 // NORM: 0 the input is used as it is, 1 ReLU(scale * x + shift), 2 any of the cheap functions of it (chosen at run time: a
 // branch per element in the loader, which the one case that generators use should not pay)
-template <int NORM, bool STATS, int WAVES, int TM>
+template <int NORM, bool STATS, int WAVES, int TM, bool ROWBIAS = false>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void tconv_walk_kernel(WalkArgs a) {
   constexpr int BM = 64 * TM, BN = 64, E = 4;  // four elements per thread, operand and 64 rows
   __shared__ float4 smem4[2 * (BM + BN) * LDK / 4];
@@ -106,7 +110,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
 #pragma unroll
     for (int i = 0; i < E; i++) {
       const uint32_t kk = b_k + i, cc = kk >> lt, t = kk & (taps - 1u), ty = t >> lx, tx = t & (tx_cnt - 1u);
-      const int32_t iy = (int32_t)qy + ph.offy + (int32_t)ty, ix = (int32_t)qx + ph.offx + (int32_t)tx;
+      const int32_t iy = (int32_t)(qy * a.in_sy) + ph.offy + (int32_t)ty, ix = (int32_t)(qx * a.in_sx) + ph.offx + (int32_t)tx;
       const bool ok = col_ok && (uint32_t)iy < a.H && (uint32_t)ix < a.W;
       const uint32_t pixel = (cc * a.H + (uint32_t)iy) * a.W + (uint32_t)ix;
       b_voff[i] = ok ? (sample * a.C * HW + pixel) * 4u : OOB;
@@ -215,6 +219,11 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   const uint32_t c_qy = c_q / ph.qw, c_qx = c_q % ph.qw;
   const uint32_t pix = (c_qy * a.sy + ph.py) * a.OW + c_qx * a.sx + ph.px;
   const uint32_t m_lane = m0 + (uint32_t)(wm * TM * 32 + 4 * lk);  // whole blocks of rows and whole pixel tiles: no row or column tests
+  float rbias[ROWBIAS ? 16 * TM : 1];
+  if constexpr (ROWBIAS) {
+#pragma unroll
+    for (int r = 0; r < 16 * TM; r++) rbias[r] = a.row_bias[m_lane + 32u * (r / 16) + 8u * ((r % 16) / 4) + (r & 3)];
+  }
   float extra = 0.f;
   if (a.tap_bias) {  // the CPU path adds the bias of every filter once per contributing tap
     int ny = 0, nx = 0;
@@ -245,7 +254,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) v[16 * i + r] = acc[i][r] + extra;
+      for (int r = 0; r < 16; r++) v[16 * i + r] = ROWBIAS ? acc[i][r] + rbias[16 * i + r] : acc[i][r] + extra;
     if constexpr (STATS) {
 #pragma unroll
       for (int e = 0; e < 16 * TM; e++) {
@@ -418,7 +427,7 @@ inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
     const TconvPhase &ph = a.ph[f];
     const uint32_t taps = (uint32_t)(ph.taps_y * ph.taps_x);
     if (ph.qh * ph.qw != qhw || ph.kp != p0.kp || taps == 0 || BK % taps != 0 || (taps & (taps - 1)) != 0 || (ph.taps_x & (ph.taps_x - 1)) != 0) return false;
-    if (a.C % (BK / taps) != 0 || ph.ld != ph.kp) return false;
+    if (a.C % (BK / taps) != 0 || ph.ld < ph.kp || ph.ld % 4 != 0) return false;
   }
   if (p0.kp % (2 * BK) != 0 || p0.kp < 4 * BK || a.M % (64 * tm) != 0) return false;
   if ((uint64_t)a.batch * a.M * a.OHW * 4u >= 0x80000000ull) return false;
@@ -453,6 +462,12 @@ inline int launch_tconv_walk(const char *name, const WalkArgs &a, bool norm, boo
   const uint32_t grid = a.nphase * a.tiles_m * a.qtiles * a.groups;
   hipStream_t s = stream();
   const int n = !norm ? 0 : a.in_func == MT_F_RELU ? 1 : 2;
+  if (a.row_bias) {  // forward convolution: plain variant only
+    if (norm || stats || tm != 1) return fail(MT_E_ARGUMENT, "%s: a forward convolution walks without batch-norm folding", name);
+    tconv_walk_kernel<0, false, 4, 1, true><<<grid, THREADS, 0, s>>>(a);
+    MT_LAUNCH_CHECK(name);
+    return MT_OK;
+  }
   if (tm == 2) {
     if (n == 1 && stats) tconv_walk_kernel<1, true, 2, 2><<<grid, THREADS, 0, s>>>(a);
     else if (n == 2 && stats) tconv_walk_kernel<2, true, 2, 2><<<grid, THREADS, 0, s>>>(a);

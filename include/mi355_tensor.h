@@ -101,16 +101,14 @@ int mt_timer_destroy(void *timer);
  *                    matrix-core kernels (a forced tile also switches off the kernels chosen by shape beside them)
  *   "igemm_fair"     -1 (default) falling wavefront priorities where the chip holds the whole grid at once / 0 never /
  *                    three hexadecimal digits: sixteenths of a block's k steps left at which the priority drops to 2, 1, 0
- *   "split_reduce"   1 (default) the block that finishes last adds the partial results of a product split over k (or over
- *                    batch groups) in a fixed order / 0 a separate launch adds them
  *   "patch_blocks"   persistent blocks of the input-patch transposed convolution (default 512, two per compute unit)
  *   "wgrad_groups"   0 (default) choose per shape / n split the batch of mt_convolution_backward_weights_sum into n groups
  *                    (when n divides the batch)
  *   "pack_cache"     1 (default) keep re-ordered weights between calls / 0 re-order on every call
  *   "tconv_walk"     1 (default) plain transposed convolutions use the kernel whose blocks walk over the batch wherever
  *                    the shape allows / 0 never
- *   "conv_walk"      1 (default) forward convolutions whose taps tile the k step use the same walking kernel wherever the
- *                    shape allows / 0 never
+ *   "conv_walk"      1 (default) forward convolutions whose taps tile the k step (4x4, 2x2, 1x1) use the same walking kernel
+ *                    wherever the shape allows and gives at least 512 blocks / 2 wherever the shape allows / 0 never
  *   "walk_blocks"    blocks wanted per launch of the walking kernel (default 1024)
  *   "walk_waves"     4 (default) or 5 wavefronts per SIMD for its plain variant
  *   "walk_tm"        1 (default) or 2 accumulators per wavefront

@@ -193,6 +193,38 @@ def test_forward_convolution(gpu, oracle, path, case):
     close(gpu.forward_convolution(*args, out_w=W + 2), oracle.forward_convolution(*args, out_w=W + 2))  # image broadcast
 
 
+@pytest.mark.parametrize("case", [
+    # W, C, H, Wd, KA, k, s, p
+    (8, 8, 16, 16, 64, 4, 2, 1),      # the discriminator's geometry: 64 output pixels, four samples... one tile of 64 pixels
+    (4, 16, 8, 8, 128, 2, 2, 0),      # 2x2 taps, four channels per k step, 16 output pixels: four samples per tile
+    (4, 64, 4, 4, 64, 1, 1, 0),       # 1x1 kernel: sixteen channels per k step
+    (12, 6, 10, 18, 192, 4, 2, 1),    # 5 x 9 = 45 output pixels: not a multiple of 16, stays on the one-tile kernel
+    (6, 12, 12, 20, 64, 4, 1, 2),     # stride 1 with padding 2: 13 x 21 pixels, no walk; and
+    (2, 4, 34, 34, 64, 4, 2, 1),      # 17 x 17 pixels, no walk
+    (16, 4, 32, 32, 64, 4, 2, 1),     # 256 output pixels, 16 samples: several groups per block
+])
+@pytest.mark.parametrize("func", [None, "leaky_relu", "tangence"])
+def test_forward_convolution_whose_blocks_walk_over_the_batch(gpu, oracle, case, func):
+    """Forward convolutions whose taps tile the k step on the kernel of the transposed convolutions (gather with the
+    layer's stride, the kernel tensor as it is, bias per output channel), against the oracle and the one-tile kernel."""
+    import mi355tensor as mt
+    W, C, H, Wd, KA, k, s, p = case
+    image, kernel, bias = U(1, W, C, H, Wd), U(2, 1, 1, KA, C * k * k) * 0.2, U(3, 1, KA, 1, 1)
+    args = (image, kernel, bias, k, k, C, KA, s, s, p, p)
+    want = oracle.forward_convolution(*args)
+    if func:
+        want = oracle.apply_func(want, func)
+    got = {}
+    try:
+        for mode in (2, 0):
+            mt.set_option("conv_walk", mode)
+            got[mode] = gpu.forward_convolution(*args, func=func)
+    finally:
+        mt.set_option("conv_walk", 1)
+    close(got[2], want, 1e-5 if func != "tangence" else 1e-4)
+    close(got[2], got[0], 2e-6)
+
+
 @pytest.mark.parametrize("case", CONV_CASES)
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_backward_convolution(gpu, oracle, path, case, with_bias):
