@@ -723,7 +723,7 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
 template <int RB, int NW>
 __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, float *dgamma, float *dbeta, const float *delta, const float *gamma,
                                                                  const float *beta, const float *xhat, const float *ivar, uint32_t W, uint32_t S, float n,
-                                                                 float inv_n, int func) {
+                                                                 float inv_n, int func, float *keep_dxhat, float *keep_s1, float *keep_s2) {
   constexpr int WS = EW_THREADS / RB, HOLD = NW > 0 ? NW : 1;
   __shared__ float part[4][WS][RB * 4];
   __shared__ float col_s1[RB * 4], col_s2[RB * 4];
@@ -794,6 +794,8 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
       for (int q = 0; q < 4; q++) t[q] += part[q][i][c];
     col_s1[c] = t[0];
     col_s2[c] = t[1];
+    if (keep_s1) keep_s1[rc] = t[0];
+    if (keep_s2) keep_s2[rc] = t[1];
     if (dgamma) dgamma[rc] = dgamma[rc] + t[2];
     if (dbeta) dbeta[rc] = dbeta[rc] + t[3];
   }
@@ -809,7 +811,16 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
     e.w = (((n * (d.w * g.w)) - (x.w * s2.w)) - s1.w) * iv.w * inv_n;
     return e;
   };
+  auto times_gamma = [&](const float4 &d) { return make_float4(d.x * g.x, d.y * g.y, d.z * g.z, d.w * g.w); };
   if constexpr (NW > 0) {
+    if (keep_dxhat) {  // (one look at the optional output for the whole loop)
+#pragma unroll
+      for (int i = 0; i < NW; i++) {
+        const uint32_t w = ws + i * WS;
+        if (w >= W) break;
+        *reinterpret_cast<float4 *>(keep_dxhat + (size_t)w * S + r) = times_gamma(qd[i]);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NW; i++) {
       const uint32_t w = ws + i * WS;
@@ -819,7 +830,9 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
   } else {
     for (uint32_t w = ws; w < W; w += WS) {
       const float4 x = *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r);
-      *reinterpret_cast<float4 *>(err + (size_t)w * S + r) = error(behind(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), x), x);
+      const float4 d = behind(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), x);
+      if (keep_dxhat) *reinterpret_cast<float4 *>(keep_dxhat + (size_t)w * S + r) = times_gamma(d);
+      *reinterpret_cast<float4 *>(err + (size_t)w * S + r) = error(d, x);
     }
   }
 }
@@ -1038,6 +1051,10 @@ unsigned stream_blocks(size_t n) {
   return blocks > 16384u ? 16384u : blocks;
 }
 }  // namespace
+
+static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
+                           const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func, const mt_tensor *keep_dxhat, const mt_tensor *keep_s1,
+                           const mt_tensor *keep_s2);
 
 extern "C" {
 
@@ -1491,12 +1508,29 @@ int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const
 
 int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
                                const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func) {
+  return bn_backward_any(error, dgamma, dbeta, delta, gamma, beta, xhat, ivar, func, nullptr, nullptr, nullptr);
+}
+
+int mt_batchnorm_backward_keep(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
+                               const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *dxhat, const mt_tensor *sum_dxhat, const mt_tensor *sum_dxhat_xhat) {
+  return bn_backward_any(error, dgamma, dbeta, delta, gamma, nullptr, xhat, ivar, MT_F_NONE, dxhat, sum_dxhat, sum_dxhat_xhat);
+}
+
+}  // extern "C"
+
+static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
+                           const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func, const mt_tensor *keep_dxhat, const mt_tensor *keep_s1,
+                           const mt_tensor *keep_s2) {
   if (!mt::valid_func(func, true) || (func != MT_F_NONE && (func & MT_F_DIFFERENTIAL))) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: unknown function id %d", func);
   if (func == MT_F_LINEAR) func = MT_F_NONE;  // derivative 1
   const mt_tensor *need[5] = {error, delta, gamma, xhat, ivar};
   for (auto t : need)
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: null tensor");
-  for (auto t : {error, dgamma, dbeta}) mt::note_write(t);
+  for (auto t : {error, dgamma, dbeta, keep_dxhat, keep_s1, keep_s2}) mt::note_write(t);
+  if (keep_dxhat && (mt::bad(keep_dxhat) || !mt::same_zyx(keep_dxhat, delta) || keep_dxhat->w != delta->w || keep_dxhat->p == delta->p || keep_dxhat->p == error->p))
+    return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward_keep: dxhat must be a tensor of its own with the sizes of delta");
+  for (auto t : {keep_s1, keep_s2})
+    if (t && (mt::bad(t) || !mt::same_zyx(t, delta) || t->w == 0)) return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward_keep: the sums must be [1,Z,Y,X]");
   if (func != MT_F_NONE && (mt::bad(beta) || !mt::same_zyx(beta, delta) || beta->w == 0))
     return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward: beta must be [1,Z,Y,X] when a function is given");
   if (!mt::same_zyx(error, delta) || error->w != delta->w || !mt::same_zyx(xhat, delta) || xhat->w != delta->w || !mt::same_zyx(gamma, delta) ||
@@ -1511,14 +1545,14 @@ int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, 
   float *pg = dgamma ? dgamma->p : nullptr, *pb = dbeta ? dbeta->p : nullptr;
   const bool cheap = func == MT_F_NONE || func == MT_F_RELU || func == MT_F_LEAKY_RELU;
   const bool vec = cheap && S % 4 == 0 && aligned16(error->p) && aligned16(delta->p) && aligned16(gamma->p) && aligned16(xhat->p) && aligned16(ivar->p) &&
-                   (func == MT_F_NONE || aligned16(beta->p));
+                   (func == MT_F_NONE || aligned16(beta->p)) && (!keep_dxhat || aligned16(keep_dxhat->p));
   if (!vec) {
     // any layout, any function: the layers' own sequences of tensor operations, on workspace tensors
     float *ws = nullptr;
     int rc = bn_scratch(2 * S + 3 * (size_t)W * S, &ws);
     if (rc) return rc;
-    mt_tensor s1{ws, 1, delta->z, delta->y, delta->x}, s2{ws + S, 1, delta->z, delta->y, delta->x};
-    mt_tensor dx{ws + 2 * S, W, delta->z, delta->y, delta->x}, t{ws + 2 * S + (size_t)W * S, W, delta->z, delta->y, delta->x};
+    mt_tensor s1{keep_s1 ? keep_s1->p : ws, 1, delta->z, delta->y, delta->x}, s2{keep_s2 ? keep_s2->p : ws + S, 1, delta->z, delta->y, delta->x};
+    mt_tensor dx{keep_dxhat ? keep_dxhat->p : ws + 2 * S, W, delta->z, delta->y, delta->x}, t{ws + 2 * S + (size_t)W * S, W, delta->z, delta->y, delta->x};
     mt_tensor front{ws + 2 * S + 2 * (size_t)W * S, W, delta->z, delta->y, delta->x};
     if (func != MT_F_NONE) {  // the function layer: delta * f'(gamma*xhat + beta)
       if ((rc = mt_tensor_item_production(&t, gamma, xhat)) || (rc = mt_add(&t, &t, beta, 1.f, 1.f))) return rc;
@@ -1542,7 +1576,8 @@ int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, 
   const unsigned grid = cdiv(S, (size_t)rb * 4);
 #define MT_BN_BWD(RB, NW) \
   bn_backward_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(error->p, pg, pb, delta->p, gamma->p, beta ? beta->p : nullptr, xhat->p, ivar->p, W, \
-                                                                    (uint32_t)S, n, inv_n, func)
+                                                                    (uint32_t)S, n, inv_n, func, keep_dxhat ? keep_dxhat->p : nullptr, keep_s1 ? keep_s1->p : nullptr, \
+                                                                    keep_s2 ? keep_s2->p : nullptr)
 #define MT_BN_BWD_NW(RB) \
   do { if (nw <= 4) MT_BN_BWD(RB, 4); else if (nw <= 8) MT_BN_BWD(RB, 8); else if (nw <= 16) MT_BN_BWD(RB, 16); else MT_BN_BWD(RB, 0); } while (0)
   if (rb == 32) MT_BN_BWD_NW(32); else if (rb == 16) MT_BN_BWD_NW(16); else MT_BN_BWD_NW(8);
@@ -1551,6 +1586,8 @@ int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, 
   MT_LAUNCH_CHECK("mt_batchnorm_backward");
   return MT_OK;
 }
+
+extern "C" {
 
 int mt_vae_coder_output(const mt_tensor *out, const mt_tensor *kl_loss, const mt_tensor *mu, const mt_tensor *logvar, const mt_tensor *epsilon) {
   const mt_tensor *need[4] = {out, mu, logvar, epsilon};

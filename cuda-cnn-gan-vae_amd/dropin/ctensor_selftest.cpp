@@ -346,6 +346,185 @@ static void DeferredGradientChecks(void)
  Report("deferred zero fill: reads, host writes, accumulation onto data",ok);
 }
 
+// The call sequences of the reference's batch-norm layer (netlayer/cnetlayerbatchnormalization.cu.h:301-371 forward in
+// training and in inference mode, :578-604 backward) and the per-layer Fill / Adam loops, written out as the layer
+// writes them, with the deferral of mi355::COpQueue on and off: every tensor a reader could look at afterwards --
+// outputs, statistics and the scratch tensors -- must hold the same values, and the counters must show that the
+// sequences ran as one kernel each.
+struct SBatchNormTensors
+{
+ CTensor<type_t> X,H,XHat,TmpAH,TmpA,TmpB,TmpC,IVar,Gamma,Beta,Mean,Variable,NewMean,NewVariable,Delta,DXHat,Prev,DGamma,DBeta;
+ SBatchNormTensors(uint32_t w,uint32_t z,uint32_t y,uint32_t x)
+  :X(w,z,y,x),H(w,z,y,x),XHat(w,z,y,x),TmpAH(w,z,y,x),TmpA(1,z,y,x),TmpB(1,z,y,x),TmpC(1,z,y,x),IVar(1,z,y,x),Gamma(1,z,y,x),Beta(1,z,y,x),Mean(1,z,y,x),
+   Variable(1,z,y,x),NewMean(1,z,y,x),NewVariable(1,z,y,x),Delta(w,z,y,x),DXHat(w,z,y,x),Prev(w,z,y,x),DGamma(1,z,y,x),DBeta(1,z,y,x)
+ {
+  FillPattern(X,1,2.0f);FillPattern(Gamma,2,0.5f);FillPattern(Beta,3,0.5f);FillPattern(NewMean,4,0.3f);FillPattern(NewVariable,5,0.3f);
+  FillPattern(Delta,6,1.0f);FillPattern(DGamma,7,0.2f);FillPattern(DBeta,8,0.2f);FillPattern(Mean,9,0.3f);FillPattern(Variable,10,0.3f);
+  for(uint32_t n=0;n<z*y*x;n++) Gamma.SetElement(0,n/(y*x),(n/x)%y,n%x,Gamma.GetElement(0,n/(y*x),(n/x)%y,n%x)+1.5f);
+  for(uint32_t n=0;n<z*y*x;n++) Variable.SetElement(0,n/(y*x),(n/x)%y,n%x,static_cast<type_t>(fabs(Variable.GetElement(0,n/(y*x),(n/x)%y,n%x))+0.2));
+ }
+ void ForwardTraining(int read_at=-1)///<read_at >= 0: somebody reads a tensor after that many calls
+ {
+  const type_t N=static_cast<type_t>(X.GetSizeW()),Momentum=0.9f,EPSILON=0.000001f;
+  CTensor<type_t> &VAR=TmpB;
+  int call=0;
+  #define STEP(code) {code;if (call++==read_at) XHat.GetElement(0,0,0,0);}
+  STEP(CTensorMath<type_t>::Fill(TmpA,0))
+  STEP(CTensorMath<type_t>::AddSumW(TmpA,TmpA,X,1,1.0/N))
+  STEP(CTensorMath<type_t>::Add(NewMean,NewMean,TmpA,Momentum,1.0-Momentum))
+  STEP(CTensorMath<type_t>::Sub(XHat,X,TmpA,1.0,1.0))
+  STEP(CTensorMath<type_t>::Fill(VAR,0))
+  STEP(CTensorMath<type_t>::Pow2(TmpAH,XHat,1))
+  STEP(CTensorMath<type_t>::AddSumW(VAR,VAR,TmpAH,1,1.0/N))
+  STEP(CTensorMath<type_t>::Add(NewVariable,NewVariable,VAR,Momentum,1.0-Momentum))
+  STEP(CTensorMath<type_t>::SQRT(TmpC,VAR,1,EPSILON))
+  STEP(CTensorMath<type_t>::Inv(IVar,TmpC))
+  STEP(CTensorMath<type_t>::TensorItemProduction(XHat,XHat,IVar))
+  STEP(CTensorMath<type_t>::TensorItemProduction(TmpAH,Gamma,XHat))
+  STEP(CTensorMath<type_t>::Add(H,TmpAH,Beta))
+ }
+ void ForwardInference(void)
+ {
+  const type_t EPSILON=0.000001f;
+  CTensor<type_t> &VAR=TmpB;
+  VAR=Variable;
+  CTensorMath<type_t>::Sub(XHat,X,Mean,1.0,1.0);
+  CTensorMath<type_t>::SQRT(TmpC,VAR,1,EPSILON);
+  CTensorMath<type_t>::Inv(IVar,TmpC);
+  CTensorMath<type_t>::TensorItemProduction(XHat,XHat,IVar);
+  CTensorMath<type_t>::TensorItemProduction(TmpAH,Gamma,XHat);
+  CTensorMath<type_t>::Add(H,TmpAH,Beta);
+ }
+ void Backward(bool create_delta_weight,int read_at=-1)
+ {
+  const type_t N=static_cast<type_t>(X.GetSizeW());
+  int call=0;
+  STEP(CTensorMath<type_t>::Fill(TmpB,0))
+  STEP(CTensorMath<type_t>::Fill(TmpC,0))
+  STEP(CTensorMath<type_t>::TensorItemProduction(DXHat,Delta,Gamma))
+  STEP(CTensorMath<type_t>::AddSumW(TmpB,TmpB,DXHat))
+  STEP(CTensorMath<type_t>::TensorItemProduction(TmpAH,DXHat,XHat))
+  STEP(CTensorMath<type_t>::AddSumW(TmpC,TmpC,TmpAH))
+  if (create_delta_weight==true)
+  {
+   STEP(CTensorMath<type_t>::TensorItemProduction(TmpAH,Delta,XHat))
+   STEP(CTensorMath<type_t>::AddSumW(DGamma,DGamma,TmpAH))
+   STEP(CTensorMath<type_t>::AddSumW(DBeta,DBeta,Delta))
+  }
+  STEP(CTensorMath<type_t>::Mul(Prev,DXHat,N))
+  STEP(CTensorMath<type_t>::TensorItemProduction(TmpAH,XHat,TmpC))
+  STEP(CTensorMath<type_t>::Sub(Prev,Prev,TmpAH))
+  STEP(CTensorMath<type_t>::Sub(Prev,Prev,TmpB))
+  STEP(CTensorMath<type_t>::TensorItemProduction(Prev,Prev,IVar))
+  STEP(CTensorMath<type_t>::Mul(Prev,Prev,static_cast<type_t>(1.0/N)))
+  #undef STEP
+ }
+ // every tensor against the same tensor of a run without deferral; differences are measured against the largest value
+ bool Agrees(const SBatchNormTensors &eager,double tolerance) const
+ {
+  const CTensor<type_t> *mine[16]={&H,&XHat,&TmpAH,&TmpA,&TmpB,&TmpC,&IVar,&NewMean,&NewVariable,&DXHat,&Prev,&DGamma,&DBeta,&Gamma,&Beta,&X};
+  const CTensor<type_t> *theirs[16]={&eager.H,&eager.XHat,&eager.TmpAH,&eager.TmpA,&eager.TmpB,&eager.TmpC,&eager.IVar,&eager.NewMean,&eager.NewVariable,
+                                     &eager.DXHat,&eager.Prev,&eager.DGamma,&eager.DBeta,&eager.Gamma,&eager.Beta,&eager.X};
+  bool ok=true;
+  for(int n=0;n<16;n++)
+  {
+   double largest=0;
+   const double diff=MaxDifference(*mine[n],*theirs[n],largest);
+   if (diff>tolerance*(largest>1e-3?largest:1e-3))
+   {
+    printf("  tensor %d differs by %g (largest value %g)\n",n,diff,largest);
+    ok=false;
+   }
+  }
+  return(ok);
+ }
+};
+
+static void FusedSequenceChecks(void)
+{
+ mi355::COpQueue &queue=mi355::Queue();
+ const uint32_t shapes[3][4]={{16,3,6,8},{5,2,3,3},{64,8,16,16}};
+ for(int s=0;s<3;s++)
+ {
+  const uint32_t *d=shapes[s];
+  char name[128];
+  // training: forward, backward with and without the parameter gradients, a second forward (the layer's next step)
+  mi355::FuseSequences()=false;
+  SBatchNormTensors eager(d[0],d[1],d[2],d[3]);
+  eager.ForwardTraining();eager.Backward(true);eager.Backward(false);eager.ForwardTraining();eager.Backward(true);
+  mi355::FuseSequences()=true;
+  SBatchNormTensors fused(d[0],d[1],d[2],d[3]);
+  const size_t forward=queue.ForwardFused,backward=queue.BackwardFused,literal=queue.LiteralCalls;
+  fused.ForwardTraining();fused.Backward(true);fused.Backward(false);fused.ForwardTraining();fused.Backward(true);
+  bool ok=queue.ForwardFused==forward+2 && queue.BackwardFused==backward+3 && queue.LiteralCalls==literal;
+  ok=fused.Agrees(eager,2e-5) && ok;   // (the statistics of the one-pass kernel against sums over the batch: fp32 rounding)
+  snprintf(name,sizeof(name),"batch-norm sequences as one kernel each, batch %u x %ux%ux%u",d[0],d[1],d[2],d[3]);
+  Report(name,ok);
+  // a reader in the middle of a sequence gets what the calls so far have left; the rest then runs as written
+  bool all=true;
+  for(int read_at=0;read_at<13;read_at+=3)
+  {
+   mi355::FuseSequences()=false;
+   SBatchNormTensors a(d[0],d[1],d[2],d[3]);
+   a.ForwardTraining(read_at);a.Backward(true,read_at);
+   mi355::FuseSequences()=true;
+   SBatchNormTensors b(d[0],d[1],d[2],d[3]);
+   b.ForwardTraining(read_at);b.Backward(true,read_at);
+   all=b.Agrees(a,2e-5) && all;
+  }
+  snprintf(name,sizeof(name),"a sequence interrupted by a reader, batch %u",d[0]);
+  Report(name,all);
+  // inference mode, twice (the scratch tensors of the first pass are overwritten unread by the second)
+  mi355::FuseSequences()=false;
+  SBatchNormTensors ei(d[0],d[1],d[2],d[3]);
+  ei.ForwardInference();ei.ForwardInference();
+  mi355::FuseSequences()=true;
+  SBatchNormTensors fi(d[0],d[1],d[2],d[3]);
+  const size_t inference=queue.InferenceFused,dropped=queue.PendingDropped;
+  fi.ForwardInference();fi.ForwardInference();
+  ok=queue.InferenceFused==inference+2 && queue.PendingDropped>dropped;
+  ok=fi.Agrees(ei,2e-5) && ok;
+  snprintf(name,sizeof(name),"batch-norm inference sequence as one kernel, batch %u",d[0]);
+  Report(name,ok);
+ }
+ // the per-layer loops: gradients cleared and Adam run tensor by tensor collect into one launch each, whatever the
+ // layers do to other tensors in between; a reader of one of the tensors gets the call-by-call result
+ const int count=6;
+ CTensor<type_t> w[2][count],dw[2][count],m[2][count],v[2][count],unrelated(4,4,4,4),copy(4,4,4,4);
+ FillPattern(unrelated,1,1.0f);
+ size_t runs[2]={0,0};
+ for(int mode=0;mode<2;mode++)
+ {
+  mi355::FuseSequences()=(mode==1);
+  for(int n=0;n<count;n++)
+  {
+   w[mode][n]=CTensor<type_t>(1,1,8+n,16);dw[mode][n]=w[mode][n];m[mode][n]=w[mode][n];v[mode][n]=w[mode][n];
+   FillPattern(w[mode][n],10+n,1.0f);FillPattern(dw[mode][n],20+n,1.0f);
+  }
+  const size_t fill_runs=queue.FillRuns,adam_runs=queue.AdamRuns;
+  for(int n=0;n<count;n++)
+  {
+   CTensorMath<type_t>::Fill(m[mode][n],0);
+   CTensorMath<type_t>::Fill(v[mode][n],0);
+   copy=unrelated;   // what a layer does between its calls (the batch-norm layer copies its running statistics)
+  }
+  for(int step=1;step<=2;step++)
+   for(int n=0;n<count;n++)
+   {
+    CTensorMath<type_t>::Adam(w[mode][n],dw[mode][n],m[mode][n],v[mode][n],8,0.01,0.9,0.999,1e-8,step);
+    copy=unrelated;
+   }
+  queue.Flush();
+  runs[mode]=(queue.FillRuns-fill_runs)+(queue.AdamRuns-adam_runs);
+ }
+ bool ok=(runs[0]==0);
+ double largest=0;
+ for(int n=0;n<count;n++) ok=ok && MaxDifference(w[1][n],w[0][n],largest)==0 && MaxDifference(m[1][n],m[0][n],largest)==0 && MaxDifference(v[1][n],v[0][n],largest)==0;
+ ok=ok && runs[1]==3 && copy.GetElement(3,3,3,3)==unrelated.GetElement(3,3,3,3);   // one Fill launch, one Adam launch per step
+ Report("Fill and Adam loops over the layers' tensors as one launch each",ok);
+ mi355::FuseSequences()=true;
+}
+
 // the scope timer the reference's models wrap around their training phases (cuda/ctimestamp.cu.h)
 static void TimerCheck(void)
 {
@@ -372,6 +551,7 @@ int main(void)
   DeltaWeightChecks();
   BackwardConvolutionCheck();
   DeferredGradientChecks();
+  FusedSequenceChecks();
   SummXYCheck();
   CoherenceAndErrors();
   GpuClassOnlyChecks();

@@ -6,6 +6,7 @@
 // the queued work took in between.  Header-only: there is no ccudatimespent.cu to compile.
 
 #include "mi355_tensor.h"
+#include "copqueue.cu.h"
 
 class CCUDATimeSpent
 {
@@ -16,10 +17,12 @@ class CCUDATimeSpent
  public:
   CCUDATimeSpent(void):Timer(0) {mt_timer_create(&Timer);}
   ~CCUDATimeSpent() {mt_timer_destroy(Timer);}
-  void Start(void) {if (Timer!=0) mt_timer_start(Timer);}
+  // calls that the tensor classes have deferred belong to the side of the mark on which they were made
+  void Start(void) {mi355::Queue().Flush();if (Timer!=0) mt_timer_start(Timer);}
   float Stop(void)
   {
    float gpu_time=0;
+   mi355::Queue().Flush();
    if (Timer!=0) mt_timer_stop(Timer,&gpu_time);
    return(gpu_time);
   }

@@ -1,0 +1,540 @@
+// Deferred tensor operations of the drop-in classes.  No counterpart in the reference, whose CTensorMath runs every call
+// when it is made.
+//
+// The reference's layers are written as long sequences of small tensor operations: the batch-norm layer's forward pass
+// in training mode is 13 calls (netlayer/cnetlayerbatchnormalization.cu.h:301-371), its backward pass 12 or 15
+// (:578-604), and every layer clears its gradients and runs Adam tensor by tensor
+// (netlayer/cnetlayerconvolution.cu.h:522-539).  The library has one kernel for each of these sequences
+// (mt_batchnorm_forward_train_func, mt_batchnorm_forward_infer_func, mt_batchnorm_backward_keep, mt_fill_many,
+// mt_adam_many).  So the elementwise calls of CTensorMath are not run at once: they are appended to a queue, and
+//   * while the queue is the beginning of one of the known sequences (same operations, same tensors in the same roles,
+//     same scalars), it waits;
+//   * when it is a whole sequence, the sequence's one kernel runs instead;
+//   * consecutive Fill calls (one value) and consecutive Adam calls (one set of hyper-parameters) collect, across
+//     layers, into one launch each;
+//   * anything else -- an operation that fits no sequence, any other call of the tensor classes that touches a tensor of
+//     the queue, any host access to one -- runs the queue call by call, exactly as written, first (calls and accesses
+//     that touch none of the queue's tensors pass it: neither side depends on the other).
+// A sequence's kernel does not write the sequence's scratch tensors that nobody can have read yet (sqrt(var + eps) and
+// gamma * xhat of the forward pass; xhat * sum of the backward pass).  Their defining calls stay "pending": they run the
+// moment somebody reads such a tensor or is about to change one of their inputs, and are forgotten when the tensor is
+// overwritten without having been read (which is what the layer does on its next pass).  Every tensor therefore holds,
+// whenever it is looked at, what the call-by-call path would have left in it, within fp32 rounding of the fused kernels.
+// mi355::FuseSequences() = false switches all of this off.
+#ifndef C_OP_QUEUE_CU_H
+#define C_OP_QUEUE_CU_H
+
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <vector>
+
+#include "mi355_tensor.h"
+
+namespace mi355
+{
+ inline void Check(int rc)
+ {
+  if (rc!=MT_OK) throw static_cast<const char*>(mt_last_error());
+ }
+ // switch for the deferral of elementwise sequences (on by default)
+ inline bool& FuseSequences(void)
+ {
+  static bool on=true;
+  return(on);
+ }
+
+ enum {OP_FILL=0,OP_ADD_SUM_W,OP_ADD,OP_SUB,OP_POW2,OP_SQRT,OP_INV,OP_ITEM_PRODUCTION,OP_MUL_VALUE,OP_ADAM};
+
+ // one call of CTensorMath as it was made: T[0] is the output (Adam: the weights), the inputs follow
+ struct SOp
+ {
+  int Kind;
+  mt_tensor T[4];
+  uint8_t Count;///<tensors in use
+  uint8_t Reads;///<bit i: T[i] is read
+  uint8_t Writes;///<bit i: all of T[i] is written
+  float A;
+  float B;
+  uint32_t BatchSize;
+  double Speed,Beta1,Beta2,Epsilon,Iteration;
+ };
+
+ inline SOp MakeOp(int kind,uint8_t count,uint8_t reads,uint8_t writes,float a=0,float b=0)
+ {
+  SOp op;
+  op.Kind=kind;op.Count=count;op.Reads=reads;op.Writes=writes;op.A=a;op.B=b;
+  op.BatchSize=0;op.Speed=0;op.Beta1=0;op.Beta2=0;op.Epsilon=0;op.Iteration=0;
+  for(int n=0;n<4;n++) {op.T[n].p=NULL;op.T[n].w=0;op.T[n].z=0;op.T[n].y=0;op.T[n].x=0;}
+  return(op);
+ }
+ inline SOp MakeFill(const mt_tensor &o,float value)
+ {
+  SOp op=MakeOp(OP_FILL,1,0,1,value);
+  op.T[0]=o;
+  return(op);
+ }
+ inline SOp MakeUnary(int kind,const mt_tensor &o,const mt_tensor &i,float a=0,float b=0)
+ {
+  SOp op=MakeOp(kind,2,2,1,a,b);
+  op.T[0]=o;op.T[1]=i;
+  return(op);
+ }
+ inline SOp MakeBinary(int kind,const mt_tensor &o,const mt_tensor &l,const mt_tensor &r,float a=0,float b=0)
+ {
+  SOp op=MakeOp(kind,3,6,1,a,b);
+  op.T[0]=o;op.T[1]=l;op.T[2]=r;
+  return(op);
+ }
+ inline SOp MakeAdam(const mt_tensor &w,const mt_tensor &dw,const mt_tensor &m,const mt_tensor &v,uint32_t batch_size,double speed,double beta1,double beta2,double epsilon,double iteration)
+ {
+  SOp op=MakeOp(OP_ADAM,4,15,13);
+  op.T[0]=w;op.T[1]=dw;op.T[2]=m;op.T[3]=v;
+  op.BatchSize=batch_size;op.Speed=speed;op.Beta1=beta1;op.Beta2=beta2;op.Epsilon=epsilon;op.Iteration=iteration;
+  return(op);
+ }
+
+ inline size_t Bytes(const mt_tensor &t) {return(static_cast<size_t>(t.w)*t.z*t.y*t.x*sizeof(float));}
+ inline bool Same(const mt_tensor &a,const mt_tensor &b) {return(a.p==b.p && a.w==b.w && a.z==b.z && a.y==b.y && a.x==b.x);}
+ inline bool SameSample(const mt_tensor &a,const mt_tensor &b) {return(a.z==b.z && a.y==b.y && a.x==b.x);}
+ inline bool Overlap(const void *p,size_t bytes,const mt_tensor &t)
+ {
+  const char *a=static_cast<const char*>(p);
+  const char *b=reinterpret_cast<const char*>(t.p);
+  return(bytes!=0 && Bytes(t)!=0 && a<b+Bytes(t) && b<a+bytes);
+ }
+ inline bool Overlap(const mt_tensor &a,const mt_tensor &b) {return(Overlap(a.p,Bytes(a),b));}
+ inline bool Covers(const void *p,size_t bytes,const mt_tensor &t)///<[p,p+bytes) holds all of t
+ {
+  const char *a=static_cast<const char*>(p);
+  const char *b=reinterpret_cast<const char*>(t.p);
+  return(a<=b && b+Bytes(t)<=a+bytes);
+ }
+ inline bool Near(float a,double b) {return(fabs(static_cast<double>(a)-b)<=1e-6*(fabs(b)>1?fabs(b):1));}
+
+ // the call as the reference's layer wrote it
+ inline void RunLiteral(const SOp &op)
+ {
+  switch(op.Kind)
+  {
+   case OP_FILL:Check(mt_fill(&op.T[0],op.A));break;
+   case OP_ADD_SUM_W:Check(mt_add_sum_w(&op.T[0],&op.T[1],&op.T[2],op.A,op.B));break;
+   case OP_ADD:Check(mt_add(&op.T[0],&op.T[1],&op.T[2],op.A,op.B));break;
+   case OP_SUB:Check(mt_sub(&op.T[0],&op.T[1],&op.T[2],op.A,op.B));break;
+   case OP_POW2:Check(mt_pow2(&op.T[0],&op.T[1],op.A));break;
+   case OP_SQRT:Check(mt_sqrt(&op.T[0],&op.T[1],op.A,op.B));break;
+   case OP_INV:Check(mt_inv(&op.T[0],&op.T[1]));break;
+   case OP_ITEM_PRODUCTION:Check(mt_tensor_item_production(&op.T[0],&op.T[1],&op.T[2]));break;
+   case OP_MUL_VALUE:Check(mt_mul_value(&op.T[0],&op.T[1],op.A));break;
+   case OP_ADAM:Check(mt_adam(&op.T[0],&op.T[1],&op.T[2],&op.T[3],op.BatchSize,op.Speed,op.Beta1,op.Beta2,op.Epsilon,op.Iteration));break;
+   default:throw("mi355::RunLiteral: unknown operation");
+  }
+ }
+
+ // ---- the known sequences ---------------------------------------------------------------------------------------------
+ // A matcher walks the queue from `first` and returns 0 (not this sequence), 1 (its beginning) or 2 (all of it).
+ struct SBatchNormForward///<netlayer/cnetlayerbatchnormalization.cu.h:301-371, training mode
+ {
+  mt_tensor Mean,X,NewMean,XHat,Var,Scratch,NewVar,SqrtVar,IVar,Gamma,Beta,H;
+  float Momentum,Epsilon;
+  enum {LENGTH=13};
+ };
+ struct SBatchNormInference///<the same lines in inference mode (:326-371)
+ {
+  mt_tensor X,Mean,XHat,Var,SqrtVar,IVar,Scratch,Gamma,Beta,H;
+  float Epsilon;
+  enum {LENGTH=6};
+ };
+ struct SBatchNormBackward///<:578-604
+ {
+  mt_tensor SumA,SumB,DXHat,Delta,Gamma,Scratch,XHat,DGamma,DBeta,Prev,IVar;
+  bool Gradients;
+  size_t Length;
+ };
+ inline bool Distinct(const mt_tensor *const *list,size_t count)
+ {
+  for(size_t a=0;a<count;a++)
+   for(size_t b=a+1;b<count;b++)
+    if (Overlap(*list[a],*list[b])==true) return(false);
+  return(true);
+ }
+ inline bool OneSampleOf(const mt_tensor &t,const mt_tensor &batch) {return(t.w==1 && SameSample(t,batch)==true);}
+
+ inline int MatchBatchNormForward(const std::vector<SOp> &q,size_t first,SBatchNormForward &m)
+ {
+  const size_t n=q.size()-first;
+  if (n>SBatchNormForward::LENGTH) return(0);
+  for(size_t i=0;i<n;i++)
+  {
+   const SOp &o=q[first+i];
+   switch(i)
+   {
+    case 0:if (o.Kind!=OP_FILL || o.A!=0 || o.T[0].w!=1) return(0);
+           m.Mean=o.T[0];break;
+    case 1:if (o.Kind!=OP_ADD_SUM_W || !Same(o.T[0],m.Mean) || !Same(o.T[1],m.Mean) || o.A!=1 || o.T[2].w==0 || !Near(o.B,1.0/o.T[2].w) || !SameSample(o.T[2],m.Mean)) return(0);
+           m.X=o.T[2];break;
+    case 2:if (o.Kind!=OP_ADD || !Same(o.T[0],o.T[1]) || !Same(o.T[2],m.Mean) || !OneSampleOf(o.T[0],m.X) || !Near(o.B,1.0-static_cast<double>(o.A))) return(0);
+           m.NewMean=o.T[0];m.Momentum=o.A;break;
+    case 3:if (o.Kind!=OP_SUB || !Same(o.T[1],m.X) || !Same(o.T[2],m.Mean) || o.A!=1 || o.B!=1 || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
+           m.XHat=o.T[0];break;
+    case 4:if (o.Kind!=OP_FILL || o.A!=0 || !OneSampleOf(o.T[0],m.X)) return(0);
+           m.Var=o.T[0];break;
+    case 5:if (o.Kind!=OP_POW2 || !Same(o.T[1],m.XHat) || o.A!=1 || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
+           m.Scratch=o.T[0];break;
+    case 6:if (o.Kind!=OP_ADD_SUM_W || !Same(o.T[0],m.Var) || !Same(o.T[1],m.Var) || !Same(o.T[2],m.Scratch) || o.A!=1 || !Near(o.B,1.0/m.X.w)) return(0);
+           break;
+    case 7:if (o.Kind!=OP_ADD || !Same(o.T[0],o.T[1]) || !Same(o.T[2],m.Var) || !OneSampleOf(o.T[0],m.X) || o.A!=m.Momentum || !Near(o.B,1.0-static_cast<double>(o.A))) return(0);
+           m.NewVar=o.T[0];break;
+    case 8:if (o.Kind!=OP_SQRT || !Same(o.T[1],m.Var) || o.A!=1 || !OneSampleOf(o.T[0],m.X)) return(0);
+           m.SqrtVar=o.T[0];m.Epsilon=o.B;break;
+    case 9:if (o.Kind!=OP_INV || !Same(o.T[1],m.SqrtVar) || !OneSampleOf(o.T[0],m.X)) return(0);
+           m.IVar=o.T[0];break;
+    case 10:if (o.Kind!=OP_ITEM_PRODUCTION || !Same(o.T[0],m.XHat) || !Same(o.T[1],m.XHat) || !Same(o.T[2],m.IVar)) return(0);
+            break;
+    case 11:if (o.Kind!=OP_ITEM_PRODUCTION || !Same(o.T[0],m.Scratch) || !Same(o.T[2],m.XHat) || !OneSampleOf(o.T[1],m.X)) return(0);
+            m.Gamma=o.T[1];break;
+    case 12:if (o.Kind!=OP_ADD || !Same(o.T[1],m.Scratch) || !OneSampleOf(o.T[2],m.X) || o.A!=1 || o.B!=1 || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
+            m.Beta=o.T[2];m.H=o.T[0];break;
+   }
+  }
+  if (n<SBatchNormForward::LENGTH) return(1);
+  const mt_tensor *all[12]={&m.Mean,&m.X,&m.NewMean,&m.XHat,&m.Var,&m.Scratch,&m.NewVar,&m.SqrtVar,&m.IVar,&m.Gamma,&m.Beta,&m.H};
+  return(Distinct(all,12)==true?2:0);
+ }
+
+ inline int MatchBatchNormInference(const std::vector<SOp> &q,size_t first,SBatchNormInference &m)
+ {
+  const size_t n=q.size()-first;
+  if (n>SBatchNormInference::LENGTH) return(0);
+  for(size_t i=0;i<n;i++)
+  {
+   const SOp &o=q[first+i];
+   switch(i)
+   {
+    case 0:if (o.Kind!=OP_SUB || o.A!=1 || o.B!=1 || o.T[1].w==0 || o.T[0].w!=o.T[1].w || !SameSample(o.T[0],o.T[1]) || !OneSampleOf(o.T[2],o.T[1])) return(0);
+           m.XHat=o.T[0];m.X=o.T[1];m.Mean=o.T[2];break;
+    case 1:if (o.Kind!=OP_SQRT || o.A!=1 || !OneSampleOf(o.T[0],m.X) || !OneSampleOf(o.T[1],m.X)) return(0);
+           m.SqrtVar=o.T[0];m.Var=o.T[1];m.Epsilon=o.B;break;
+    case 2:if (o.Kind!=OP_INV || !Same(o.T[1],m.SqrtVar) || !OneSampleOf(o.T[0],m.X)) return(0);
+           m.IVar=o.T[0];break;
+    case 3:if (o.Kind!=OP_ITEM_PRODUCTION || !Same(o.T[0],m.XHat) || !Same(o.T[1],m.XHat) || !Same(o.T[2],m.IVar)) return(0);
+           break;
+    case 4:if (o.Kind!=OP_ITEM_PRODUCTION || !Same(o.T[2],m.XHat) || !OneSampleOf(o.T[1],m.X) || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
+           m.Scratch=o.T[0];m.Gamma=o.T[1];break;
+    case 5:if (o.Kind!=OP_ADD || !Same(o.T[1],m.Scratch) || !OneSampleOf(o.T[2],m.X) || o.A!=1 || o.B!=1 || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
+           m.Beta=o.T[2];m.H=o.T[0];break;
+   }
+  }
+  if (n<SBatchNormInference::LENGTH) return(1);
+  const mt_tensor *all[10]={&m.X,&m.Mean,&m.XHat,&m.Var,&m.SqrtVar,&m.IVar,&m.Scratch,&m.Gamma,&m.Beta,&m.H};
+  return(Distinct(all,10)==true?2:0);
+ }
+
+ inline int MatchBatchNormBackward(const std::vector<SOp> &q,size_t first,SBatchNormBackward &m)
+ {
+  const size_t n=q.size()-first;
+  if (n>15) return(0);
+  m.Gradients=false;
+  m.Length=12;
+  for(size_t i=0;i<n;i++)
+  {
+   const SOp &o=q[first+i];
+   size_t step=i;
+   if (i>=6)
+   {
+    // with create_delta_weight three more calls follow the two sums (:586-592); the seventh call tells which form this is
+    if (i==6) m.Gradients=(o.Kind==OP_ITEM_PRODUCTION);
+    if (m.Gradients==true) m.Length=15;
+    else step=i+3;
+   }
+   switch(step)
+   {
+    case 0:if (o.Kind!=OP_FILL || o.A!=0 || o.T[0].w!=1) return(0);
+           m.SumA=o.T[0];break;
+    case 1:if (o.Kind!=OP_FILL || o.A!=0 || o.T[0].w!=1 || !SameSample(o.T[0],m.SumA)) return(0);
+           m.SumB=o.T[0];break;
+    case 2:if (o.Kind!=OP_ITEM_PRODUCTION || o.T[1].w==0 || o.T[0].w!=o.T[1].w || !SameSample(o.T[0],o.T[1]) || !SameSample(o.T[1],m.SumA) || !OneSampleOf(o.T[2],o.T[1])) return(0);
+           m.DXHat=o.T[0];m.Delta=o.T[1];m.Gamma=o.T[2];break;
+    case 3:if (o.Kind!=OP_ADD_SUM_W || !Same(o.T[0],m.SumA) || !Same(o.T[1],m.SumA) || !Same(o.T[2],m.DXHat) || o.A!=1 || o.B!=1) return(0);
+           break;
+    case 4:if (o.Kind!=OP_ITEM_PRODUCTION || !Same(o.T[1],m.DXHat) || o.T[0].w!=m.Delta.w || !SameSample(o.T[0],m.Delta) || o.T[2].w!=m.Delta.w || !SameSample(o.T[2],m.Delta)) return(0);
+           m.Scratch=o.T[0];m.XHat=o.T[2];break;
+    case 5:if (o.Kind!=OP_ADD_SUM_W || !Same(o.T[0],m.SumB) || !Same(o.T[1],m.SumB) || !Same(o.T[2],m.Scratch) || o.A!=1 || o.B!=1) return(0);
+           break;
+    case 6:if (o.Kind!=OP_ITEM_PRODUCTION || !Same(o.T[0],m.Scratch) || !Same(o.T[1],m.Delta) || !Same(o.T[2],m.XHat)) return(0);
+           break;
+    case 7:if (o.Kind!=OP_ADD_SUM_W || !Same(o.T[0],o.T[1]) || !Same(o.T[2],m.Scratch) || !OneSampleOf(o.T[0],m.Delta) || o.A!=1 || o.B!=1) return(0);
+           m.DGamma=o.T[0];break;
+    case 8:if (o.Kind!=OP_ADD_SUM_W || !Same(o.T[0],o.T[1]) || !Same(o.T[2],m.Delta) || !OneSampleOf(o.T[0],m.Delta) || o.A!=1 || o.B!=1) return(0);
+           m.DBeta=o.T[0];break;
+    case 9:if (o.Kind!=OP_MUL_VALUE || !Same(o.T[1],m.DXHat) || o.A!=static_cast<float>(m.Delta.w) || o.T[0].w!=m.Delta.w || !SameSample(o.T[0],m.Delta)) return(0);
+           m.Prev=o.T[0];break;
+    case 10:if (o.Kind!=OP_ITEM_PRODUCTION || !Same(o.T[0],m.Scratch) || !Same(o.T[1],m.XHat) || !Same(o.T[2],m.SumB)) return(0);
+            break;
+    case 11:if (o.Kind!=OP_SUB || !Same(o.T[0],m.Prev) || !Same(o.T[1],m.Prev) || !Same(o.T[2],m.Scratch) || o.A!=1 || o.B!=1) return(0);
+            break;
+    case 12:if (o.Kind!=OP_SUB || !Same(o.T[0],m.Prev) || !Same(o.T[1],m.Prev) || !Same(o.T[2],m.SumA) || o.A!=1 || o.B!=1) return(0);
+            break;
+    case 13:if (o.Kind!=OP_ITEM_PRODUCTION || !Same(o.T[0],m.Prev) || !Same(o.T[1],m.Prev) || !OneSampleOf(o.T[2],m.Delta)) return(0);
+            m.IVar=o.T[2];break;
+    case 14:if (o.Kind!=OP_MUL_VALUE || !Same(o.T[0],m.Prev) || !Same(o.T[1],m.Prev) || !Near(o.A,1.0/m.Delta.w)) return(0);
+            break;
+   }
+  }
+  if (n>m.Length) return(0);
+  if (n<=6 || n<m.Length) return(1);
+  const mt_tensor *all[11]={&m.SumA,&m.SumB,&m.DXHat,&m.Delta,&m.Gamma,&m.Scratch,&m.XHat,&m.Prev,&m.IVar,&m.DGamma,&m.DBeta};
+  return(Distinct(all,m.Gradients==true?11:9)==true?2:0);
+ }
+
+ // consecutive Fill calls with one value, or consecutive Adam calls with one set of hyper-parameters
+ inline bool IsRun(const std::vector<SOp> &q,size_t count)
+ {
+  if (count==0) return(true);
+  const SOp &h=q[0];
+  if (h.Kind!=OP_FILL && h.Kind!=OP_ADAM) return(false);
+  for(size_t i=1;i<count;i++)
+  {
+   const SOp &o=q[i];
+   if (o.Kind!=h.Kind) return(false);
+   if (h.Kind==OP_FILL && o.A!=h.A) return(false);
+   if (h.Kind==OP_ADAM && (o.BatchSize!=h.BatchSize || o.Speed!=h.Speed || o.Beta1!=h.Beta1 || o.Beta2!=h.Beta2 || o.Epsilon!=h.Epsilon || o.Iteration!=h.Iteration)) return(false);
+  }
+  return(true);
+ }
+
+ class COpQueue
+ {
+  private:
+   std::vector<SOp> Queue;///<calls made and not yet run, in order
+   std::vector<SOp> Pending;///<defining calls of scratch tensors that a sequence's kernel did not write, in order
+  public:
+   // counters, for tests and measurements
+   size_t ForwardFused,InferenceFused,BackwardFused,FillRuns,AdamRuns,RunCalls,LiteralCalls,PendingRun,PendingDropped;
+   COpQueue(void):ForwardFused(0),InferenceFused(0),BackwardFused(0),FillRuns(0),AdamRuns(0),RunCalls(0),LiteralCalls(0),PendingRun(0),PendingDropped(0) {}
+
+   // a call of CTensorMath; operands are up to date on the device, the output is marked device-side by the caller
+   void Submit(const SOp &op)
+   {
+    if (FuseSequences()==false)
+    {
+     Flush();
+     Settle(&op,1);
+     RunLiteral(op);
+     return;
+    }
+    Queue.push_back(op);
+    for(;;)
+    {
+     // the queue may begin with a run that is still collecting; a known sequence may start anywhere behind it
+     for(size_t first=0;first<Queue.size();first++)
+     {
+      if (IsRun(Queue,first)==false) break;
+      SBatchNormForward f;
+      SBatchNormInference i;
+      SBatchNormBackward b;
+      const int mf=MatchBatchNormForward(Queue,first,f),mi=MatchBatchNormInference(Queue,first,i),mb=MatchBatchNormBackward(Queue,first,b);
+      if (mf==2 || mi==2 || mb==2)
+      {
+       std::vector<SOp> sequence(Queue.begin()+first,Queue.end());
+       Queue.resize(first);
+       RunQueue();
+       if (mf==2) RunForward(sequence,f);
+       else if (mi==2) RunInference(sequence,i);
+       else RunBackward(sequence,b);
+       return;
+      }
+      if (mf==1 || mi==1 || mb==1) return;
+     }
+     if (IsRun(Queue,Queue.size())==true) return;
+     if (Queue.size()==1) {RunQueue();return;}
+     // the last call fits nothing the queue was waiting for: the calls before it run as written, it starts anew
+     const SOp last=Queue.back();
+     Queue.pop_back();
+     RunQueue();
+     Queue.push_back(last);
+    }
+   }
+   // everything queued runs now, call by call (a collected run as its one launch)
+   void Flush(void)
+   {
+    if (Queue.empty()==false) RunQueue();
+   }
+   // Somebody outside the queue is about to read and/or write device memory [p,p+bytes): a call of the tensor classes
+   // that is not deferred, a copy to or from the host, a buffer that is freed.  `write` means all of it is overwritten
+   // (or goes away); with `read` as well the old contents are used first.
+   void Access(const void *p,size_t bytes,bool read,bool write)
+   {
+    if (p==NULL || bytes==0) return;
+    if (Queue.empty()==false)
+    {
+     bool touches=false;///<calls on other tensors pass: they depend on nothing the queue holds, and nothing in it on them
+     for(size_t i=0;i<Queue.size() && touches==false;i++)
+      for(uint8_t t=0;t<Queue[i].Count;t++)
+       if (Overlap(p,bytes,Queue[i].T[t])==true) touches=true;
+     if (touches==true) RunQueue();
+    }
+    if (Pending.empty()==false) SettleRange(p,bytes,read,write);
+   }
+   bool Idle(void) const {return(Queue.empty() && Pending.empty());}
+   size_t QueuedCalls(void) const {return(Queue.size());}
+   size_t PendingCalls(void) const {return(Pending.size());}
+  private:
+   void RunQueue(void)
+   {
+    std::vector<SOp> q;
+    q.swap(Queue);
+    if (q.size()>=2 && IsRun(q,q.size())==true)
+    {
+     Settle(&q[0],q.size());
+     RunCalls+=q.size();
+     std::vector<const mt_tensor*> a(q.size()),b(q.size()),c(q.size()),d(q.size());
+     for(size_t i=0;i<q.size();i++) {a[i]=&q[i].T[0];b[i]=&q[i].T[1];c[i]=&q[i].T[2];d[i]=&q[i].T[3];}
+     if (q[0].Kind==OP_FILL)
+     {
+      FillRuns++;
+      Check(mt_fill_many(static_cast<uint32_t>(q.size()),&a[0],q[0].A));
+     }
+     else
+     {
+      AdamRuns++;
+      Check(mt_adam_many(static_cast<uint32_t>(q.size()),&a[0],&b[0],&c[0],&d[0],q[0].BatchSize,q[0].Speed,q[0].Beta1,q[0].Beta2,q[0].Epsilon,q[0].Iteration));
+     }
+     return;
+    }
+    for(size_t i=0;i<q.size();i++)
+    {
+     Settle(&q[i],1);
+     LiteralCalls++;
+     RunLiteral(q[i]);
+    }
+   }
+   void RunForward(const std::vector<SOp> &sequence,const SBatchNormForward &m)
+   {
+    Settle(&sequence[0],sequence.size());
+    ForwardFused++;
+    Check(mt_batchnorm_forward_train_func(&m.H,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,m.Momentum,m.Epsilon,MT_F_NONE));
+    Pending.push_back(sequence[8]);///<SqrtVar = sqrt(Var + epsilon)
+    Pending.push_back(sequence[11]);///<Scratch = Gamma * XHat
+   }
+   void RunInference(const std::vector<SOp> &sequence,const SBatchNormInference &m)
+   {
+    Settle(&sequence[0],sequence.size());
+    InferenceFused++;
+    Check(mt_batchnorm_forward_infer_func(&m.H,&m.X,&m.Gamma,&m.Beta,&m.Mean,&m.Var,m.Epsilon,MT_F_NONE));
+    for(size_t i=0;i<5;i++) Pending.push_back(sequence[i]);///<everything but the output itself
+   }
+   void RunBackward(const std::vector<SOp> &sequence,const SBatchNormBackward &m)
+   {
+    Settle(&sequence[0],sequence.size());
+    BackwardFused++;
+    Check(mt_batchnorm_backward_keep(&m.Prev,m.Gradients==true?&m.DGamma:NULL,m.Gradients==true?&m.DBeta:NULL,&m.Delta,&m.Gamma,&m.XHat,&m.IVar,&m.DXHat,&m.SumA,&m.SumB));
+    Pending.push_back(sequence[m.Gradients==true?10:7]);///<Scratch = XHat * SumB
+   }
+
+   // ---- pending calls ------------------------------------------------------------------------------------------------
+   // Runs pending call `j` after every earlier pending call that shares a tensor with it (program order among related calls).
+   void RunPending(size_t j,std::vector<uint8_t> &state)///<state: 0 waiting, 1 done or dropped
+   {
+    if (state[j]!=0) return;
+    for(size_t i=0;i<j;i++)
+    {
+     if (state[i]!=0) continue;
+     bool related=false;
+     for(uint8_t a=0;a<Pending[i].Count && related==false;a++)
+      for(uint8_t b=0;b<Pending[j].Count;b++)
+       if (Overlap(Pending[i].T[a],Pending[j].T[b])==true) {related=true;break;}
+     if (related==true) RunPending(i,state);
+    }
+    state[j]=1;
+    PendingRun++;
+    RunLiteral(Pending[j]);
+   }
+   // Before `count` calls run as one unit (a sequence's kernel, a run, one literal call): pending calls whose output the
+   // unit overwrites without anybody having read it are forgotten; those whose output the unit reads, or whose inputs
+   // it changes, run first.
+   void Settle(const SOp *unit,size_t count)
+   {
+    if (Pending.empty()==true) return;
+    // what the unit reads from outside itself, and what it overwrites
+    std::vector<mt_tensor> reads,writes;
+    for(size_t i=0;i<count;i++)
+    {
+     const SOp &o=unit[i];
+     for(uint8_t t=0;t<o.Count;t++)
+     {
+      if ((o.Reads&(1u<<t))==0) continue;
+      bool inside=false;
+      for(size_t w=0;w<writes.size();w++)
+       if (Covers(writes[w].p,Bytes(writes[w]),o.T[t])==true) inside=true;
+      if (inside==false) reads.push_back(o.T[t]);
+     }
+     for(uint8_t t=0;t<o.Count;t++)
+      if ((o.Writes&(1u<<t))!=0) writes.push_back(o.T[t]);
+    }
+    SettleSets(reads,writes);
+   }
+   void SettleRange(const void *p,size_t bytes,bool read,bool write)
+   {
+    mt_tensor range;
+    range.p=static_cast<float*>(const_cast<void*>(p));
+    range.w=1;range.z=1;range.y=1;range.x=static_cast<uint32_t>(bytes/sizeof(float));
+    if (static_cast<size_t>(range.x)*sizeof(float)!=bytes) {range.y=static_cast<uint32_t>((bytes/sizeof(float)+0xffffu)>>16);range.x=1u<<16;}///<(a buffer of 16 GiB or more, or one that is no whole number of floats: a range that covers it)
+    std::vector<mt_tensor> reads,writes;
+    if (read==true) reads.push_back(range);
+    if (write==true) writes.push_back(range);
+    SettleSets(reads,writes);
+   }
+   void SettleSets(const std::vector<mt_tensor> &reads,const std::vector<mt_tensor> &writes)
+   {
+    const size_t n=Pending.size();
+    std::vector<uint8_t> state(n,0);
+    std::vector<uint8_t> dead(n,0);
+    // from the last pending call to the first: forgotten when its output is overwritten whole, read by nobody outside
+    // and by no later pending call that stays
+    for(size_t k=n;k>0;k--)
+    {
+     const size_t j=k-1;
+     const mt_tensor &out=Pending[j].T[0];
+     bool overwritten=false,wanted=false;
+     for(size_t w=0;w<writes.size();w++)
+      if (Covers(writes[w].p,Bytes(writes[w]),out)==true) overwritten=true;
+     for(size_t r=0;r<reads.size();r++)
+      if (Overlap(reads[r],out)==true) wanted=true;
+     for(size_t l=j+1;l<n && wanted==false;l++)
+     {
+      if (dead[l]!=0) continue;
+      for(uint8_t t=0;t<Pending[l].Count;t++)
+       if ((Pending[l].Reads&(1u<<t))!=0 && Overlap(Pending[l].T[t],out)==true) wanted=true;
+     }
+     if (overwritten==true && wanted==false) dead[j]=1;
+    }
+    for(size_t j=0;j<n;j++)
+     if (dead[j]!=0) {state[j]=1;PendingDropped++;}
+    // the others run when the unit reads their output, or writes into their output or one of their inputs
+    for(size_t j=0;j<n;j++)
+    {
+     if (state[j]!=0) continue;
+     bool now=false;
+     for(size_t r=0;r<reads.size() && now==false;r++)
+      if (Overlap(reads[r],Pending[j].T[0])==true) now=true;
+     for(size_t w=0;w<writes.size() && now==false;w++)
+      for(uint8_t t=0;t<Pending[j].Count;t++)
+       if (Overlap(writes[w],Pending[j].T[t])==true) {now=true;break;}
+     if (now==true) RunPending(j,state);
+    }
+    std::vector<SOp> left;
+    for(size_t j=0;j<n;j++)
+     if (state[j]==0) left.push_back(Pending[j]);
+    Pending.swap(left);
+   }
+ };
+
+ inline COpQueue& Queue(void)
+ {
+  static COpQueue *queue=new COpQueue;///<never destroyed: tensors with static lifetime may outlive any static object
+  return(*queue);
+ }
+}
+
+#endif

@@ -17,14 +17,10 @@
 #include "../common/idatastream.h"
 #include "../system/system.h"
 #include "mi355_tensor.h"
+#include "copqueue.cu.h"
 
 namespace mi355
 {
- inline void Check(int rc)
- {
-  if (rc!=MT_OK) throw static_cast<const char*>(mt_last_error());
- }
-
  // owning device buffer with value semantics (copying copies the device data, :159-170 of the reference vector)
  class CDeviceBuffer
  {
@@ -38,12 +34,21 @@ namespace mi355
    {
     if (this==&other) return(*this);
     resize(other.Bytes);
-    if (Bytes!=0) Check(mt_copy_d2d(Ptr,other.Ptr,Bytes));
+    if (Bytes!=0)
+    {
+     Queue().Access(other.Ptr,other.Bytes,true,false);
+     Queue().Access(Ptr,Bytes,false,true);
+     Check(mt_copy_d2d(Ptr,other.Ptr,Bytes));
+    }
     return(*this);
    }
    void clear(void)
    {
-    if (Ptr!=NULL) mt_free(Ptr);
+    if (Ptr!=NULL)
+    {
+     Queue().Access(Ptr,Bytes,false,true);///<deferred calls that name the block run (or are forgotten) before it goes
+     mt_free(Ptr);
+    }
     Ptr=NULL;
     Bytes=0;
    }
@@ -57,7 +62,12 @@ namespace mi355
    void assign(const void *device_source,size_t bytes)
    {
     resize(bytes);
-    if (Bytes!=0) Check(mt_copy_d2d(Ptr,device_source,Bytes));
+    if (Bytes!=0)
+    {
+     Queue().Access(device_source,bytes,true,false);
+     Queue().Access(Ptr,Bytes,false,true);
+     Check(mt_copy_d2d(Ptr,device_source,Bytes));
+    }
    }
    void swap(CDeviceBuffer &other) {std::swap(Ptr,other.Ptr);std::swap(Bytes,other.Bytes);}
    void* get(void) const {return(Ptr);}
@@ -231,6 +241,7 @@ class CTensor
    if (Item.size()<size) throw("CTensor::CopyItemToDevice: array larger than the tensor");
    Materialise();
    CopyToDevice();
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),true,true);
    mi355::Check(mt_copy_h2d(DeviceItem.get(),item_array,size*sizeof(type_t)));
    SetDeviceOnChange();
   }
@@ -248,6 +259,7 @@ class CTensor
    if (Item.size()<size+offset) throw("CTensor::CopyItemLayerWToDevice: array larger than the tensor");
    Materialise();
    CopyToDevice();
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),true,true);
    mi355::Check(mt_copy_h2d(static_cast<type_t*>(DeviceItem.get())+offset,item_array,size*sizeof(type_t)));
    SetDeviceOnChange();
   }
@@ -347,6 +359,7 @@ class CTensor
   {
    if (HostOnChange==false && force==false) return;
    DropLazy();
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),false,true);
    if (!Item.empty()) mi355::Check(mt_copy_h2d(DeviceItem.get(),&Item[0],Item.size()*sizeof(type_t)));
    HostOnChange=false;
    DeviceOnChange=false;
@@ -355,6 +368,7 @@ class CTensor
   {
    Materialise();
    if (DeviceOnChange==false && force==false) return;
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),true,false);
    if (!Item.empty()) mi355::Check(mt_copy_d2h(&Item[0],DeviceItem.get(),Item.size()*sizeof(type_t)));
    HostOnChange=false;
    DeviceOnChange=false;
@@ -367,6 +381,7 @@ class CTensor
   void Materialise(void) const
   {
    if (Lazy==LAZY_NONE) return;
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),false,true);
    const uint8_t kind=Lazy;
    std::shared_ptr<mi355::CDeferredGradient> record;
    record.swap(Deferred);
@@ -483,14 +498,34 @@ class CTensor
   }
   void DropLazy(void) const {Lazy=LAZY_NONE;Deferred.reset();}
   // the device copy is said to hold zeros; nothing is launched (CTensorMath::Fill)
-  void SetLazyZero(void) const {DropLazy();Lazy=LAZY_ZERO;DeviceOnChange=true;HostOnChange=false;}
+  void SetLazyZero(void) const
+  {
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),false,true);///<as far as deferred calls are concerned the tensor is overwritten now
+   DropLazy();
+   Lazy=LAZY_ZERO;
+   DeviceOnChange=true;
+   HostOnChange=false;
+  }
   size_t Count(void) const {return(static_cast<size_t>(Size_X)*Size_Y*Size_Z*Size_W);}
   size_t Index(uint32_t w,uint32_t z,uint32_t y,uint32_t x) const {return(x+static_cast<size_t>(Size_X)*(y+static_cast<size_t>(Size_Y)*(z+static_cast<size_t>(Size_Z)*w)));}
-  // descriptor of the device copy for the C ABI; `upload` first brings the device copy up to date
+  // descriptor of the device copy for a call that is deferred (mi355::COpQueue): the queue itself keeps the order
+  mt_tensor DeviceQueued(bool upload) const
+  {
+   Materialise();
+   if (upload==true) CopyToDevice();
+   mt_tensor t;
+   t.p=static_cast<float*>(DeviceItem.get());
+   t.w=Size_W;t.z=Size_Z;t.y=Size_Y;t.x=Size_X;
+   return(t);
+  }
+  // descriptor of the device copy for the C ABI; `upload` first brings the device copy up to date (the tensor is read,
+  // and may be written as well); without it the call overwrites the whole tensor.  Deferred calls that involve the
+  // tensor run first.
   mt_tensor Device(bool upload) const
   {
    Materialise();
    if (upload==true) CopyToDevice();
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),upload,true);
    mt_tensor t;
    t.p=static_cast<float*>(DeviceItem.get());
    t.w=Size_W;t.z=Size_Z;t.y=Size_Y;t.x=Size_X;

@@ -1,6 +1,8 @@
 // Drop-in for the reference's cuda/ctensormath.cu.h (class at :52-138): every static function keeps the reference's
 // name, argument order and defaults and forwards to one C-ABI call.  Inputs are brought up to date on the device
-// first and the output is marked device-side, as the reference does (:845-870).
+// first and the output is marked device-side, as the reference does (:845-870).  The elementwise calls that the layers
+// string into long sequences (Fill, Add, Sub, AddSumW, Pow2, SQRT, Inv, TensorItemProduction, Mul by a value, Adam) go
+// through mi355::COpQueue, which runs a whole known sequence as its one kernel and everything else as written.
 #ifndef C_TENSOR_MATH_CU_H
 #define C_TENSOR_MATH_CU_H
 
@@ -39,15 +41,14 @@ class CTensorMath
     cTensor_Output.SetLazyZero();
     return;
    }
-   mt_tensor o=cTensor_Output.Device(false);
-   mi355::Check(mt_fill(&o,value));
+   mi355::Queue().Submit(mi355::MakeFill(cTensor_Output.DeviceQueued(false),value));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Inv(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
-   mi355::Check(mt_inv(&o,&i));
+   mt_tensor i=cTensor_Input.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mi355::Queue().Submit(mi355::MakeUnary(mi355::OP_INV,o,i));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Div(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
@@ -60,8 +61,8 @@ class CTensorMath
   static void Add(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
-   mi355::Check(mt_add(&o,&l,&r,left_scale,right_scale));
+   mt_tensor l=cTensor_Left.DeviceQueued(true),r=cTensor_Right.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_ADD,o,l,r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();
   }
   // The batch-norm layer of the reference calls Add(out,left,right,EMA_K,1,0-EMA_K) (netlayer/cnetlayerbatchnormalization.cu.h:655-658,
@@ -87,8 +88,8 @@ class CTensorMath
     cTensor_Output.SetDeviceOnChange();
     return;
    }
-   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
-   mi355::Check(mt_add_sum_w(&o,&l,&r,left_scale,right_scale));
+   mt_tensor l=cTensor_Left.DeviceQueued(true),r=cTensor_Right.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_ADD_SUM_W,o,l,r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();
   }
   static void AddValue(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t tensor_scale,type_t value)
@@ -101,8 +102,8 @@ class CTensorMath
   static void Sub(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
-   mi355::Check(mt_sub(&o,&l,&r,left_scale,right_scale));
+   mt_tensor l=cTensor_Left.DeviceQueued(true),r=cTensor_Right.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_SUB,o,l,r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();
   }
   static void SubValue(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t tensor_scale,type_t value)
@@ -122,15 +123,15 @@ class CTensorMath
   static void Pow2(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t scale=1)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
-   mi355::Check(mt_pow2(&o,&i,scale));
+   mt_tensor i=cTensor_Input.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mi355::Queue().Submit(mi355::MakeUnary(mi355::OP_POW2,o,i,scale));
    cTensor_Output.SetDeviceOnChange();
   }
   static void SQRT(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t scale,type_t add_sqrt_value)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
-   mi355::Check(mt_sqrt(&o,&i,scale,add_sqrt_value));
+   mt_tensor i=cTensor_Input.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mi355::Queue().Submit(mi355::MakeUnary(mi355::OP_SQRT,o,i,scale,add_sqrt_value));
    cTensor_Output.SetDeviceOnChange();
   }
   static void AddBias(CTensor<type_t> &cTensor_Working,const CTensor<type_t> &cTensor_Bias)
@@ -166,8 +167,8 @@ class CTensorMath
   static void Mul(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const type_t &value_right)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.Device(true),o=cTensor_Output.Device(false);
-   mi355::Check(mt_mul_value(&o,&l,value_right));
+   mt_tensor l=cTensor_Left.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mi355::Queue().Submit(mi355::MakeUnary(mi355::OP_MUL_VALUE,o,l,value_right));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Mul(CTensor<type_t> &cTensor_Output,const type_t &value_left,const CTensor<type_t> &cTensor_Right)
@@ -184,8 +185,8 @@ class CTensorMath
   static void TensorItemProduction(CTensor<type_t> &cTensor_Output,CTensor<type_t> &cTensor_Left,CTensor<type_t> &cTensor_Right)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
-   mi355::Check(mt_tensor_item_production(&o,&l,&r));
+   mt_tensor l=cTensor_Left.DeviceQueued(true),r=cTensor_Right.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_ITEM_PRODUCTION,o,l,r));
    cTensor_Output.SetDeviceOnChange();
   }
   static CTensor<type_t> Transpose(const CTensor<type_t> &cTensor_Input)
@@ -292,8 +293,8 @@ class CTensorMath
   static void Adam(CTensor<type_t> &cTensor_Weight,CTensor<type_t> &cTensor_dWeight,CTensor<type_t> &cTensor_M,CTensor<type_t> &cTensor_V,uint32_t batch_size,double speed,double beta1,double beta2,double epsilon,double iteration)
   {
    OnlyFloat();
-   mt_tensor w=cTensor_Weight.Device(true),dw=cTensor_dWeight.Device(true),m=cTensor_M.Device(true),v=cTensor_V.Device(true);
-   mi355::Check(mt_adam(&w,&dw,&m,&v,batch_size,speed,beta1,beta2,epsilon,iteration));
+   mt_tensor w=cTensor_Weight.DeviceQueued(true),dw=cTensor_dWeight.DeviceQueued(true),m=cTensor_M.DeviceQueued(true),v=cTensor_V.DeviceQueued(true);
+   mi355::Queue().Submit(mi355::MakeAdam(w,dw,m,v,batch_size,speed,beta1,beta2,epsilon,iteration));
    cTensor_Weight.SetDeviceOnChange();
    cTensor_M.SetDeviceOnChange();
    cTensor_V.SetDeviceOnChange();

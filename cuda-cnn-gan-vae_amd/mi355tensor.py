@@ -505,6 +505,12 @@ class Fused:
             call("mt_batchnorm_backward_func", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), opt(beta), _d(xhat), _d(ivar), C.c_int(FUNC[func]))
 
     @staticmethod
+    def BatchNormBackwardKeep(error, dgamma, dbeta, delta, gamma, xhat, ivar, dxhat=None, sum_dxhat=None, sum_dxhat_xhat=None):
+        """The backward pass that also leaves the intermediate tensors of the layer's own sequence."""
+        opt = lambda t: _d(t) if t is not None else None
+        call("mt_batchnorm_backward_keep", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), _d(xhat), _d(ivar), opt(dxhat), opt(sum_dxhat), opt(sum_dxhat_xhat))
+
+    @staticmethod
     def UpSamplingConvolution(out, image, upsampling_x, upsampling_y, kernel, kernel_x, kernel_y, kernel_z, kernel_amount, bias, stride_x, stride_y,
                               padding_x, padding_y, func=None):
         call("mt_upsampling_convolution_func", _d(out), _d(image), _u(upsampling_x), _u(upsampling_y), _d(kernel), _i(kernel_x), _i(kernel_y), _i(kernel_z),

@@ -298,6 +298,13 @@ int mt_batchnorm_backward(const mt_tensor *error, const mt_tensor *dgamma, const
  * multiplied by f'(gamma*xhat+beta) on the way in.  `beta` [1,Z,Y,X] is needed unless func is MT_F_NONE / MT_F_LINEAR. */
 int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta,
                                const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func);
+/* CNetLayerBatchNormalization::TrainingBackward (netlayer/cnetlayerbatchnormalization.cu.h:578-604) as one kernel that also
+ * leaves the tensors the literal sequence leaves behind, for callers that replace the sequence behind an unchanged layer:
+ * dxhat [B,Z,Y,X] = delta*gamma (line 581), sum_dxhat [1,Z,Y,X] = sum_w dxhat (line 582), sum_dxhat_xhat = sum_w dxhat*xhat
+ * (line 585); NULL skips any of them.  dxhat must not be the error or the delta tensor. */
+int mt_batchnorm_backward_keep(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta,
+                               const mt_tensor *gamma, const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *dxhat,
+                               const mt_tensor *sum_dxhat, const mt_tensor *sum_dxhat_xhat);
 /* CNetLayerConvolution::TrainingBackward, netlayer/cnetlayerconvolution.cu.h:501-508, without the per-sample round trip:
  * dkernel [1,1,Kamt,C*Ky*Kx] += sum over the batch of the per-sample weight gradients (CreateDeltaWeightAndBias into a
  * zeroed batch tensor, then AddSumW), dbias [1,Kamt,1,1] += sum over the batch and the pixels of delta. */

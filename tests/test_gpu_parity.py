@@ -804,6 +804,18 @@ def test_batchnorm_backward_fused(gpu, oracle, shape):
     assert np.max(np.abs(err - want_err)) <= 1e-5 * max(scale, np.abs(want_err).max())
     close(dg - dg0, want_dg, 1e-5)
     close(db - db0, want_db, 1e-5)
+    # the variant that leaves the sequence's intermediate tensors: same results, and dxhat and the two sums beside them
+    from mi355tensor import CTensor, Fused
+    from gpu_api import up
+    one = (1,) + tuple(shape[1:])
+    t_err, t_dg, t_db, t_dx, t_s1, t_s2 = CTensor(*shape), up(dg0), up(db0), CTensor(*shape), CTensor(*one), CTensor(*one)
+    Fused.BatchNormBackwardKeep(t_err, t_dg, t_db, up(delta), up(gamma), up(fwd["xhat"]), up(fwd["ivar"]), t_dx, t_s1, t_s2)
+    assert np.array_equal(t_err.numpy(), err) and np.array_equal(t_dg.numpy(), dg) and np.array_equal(t_db.numpy(), db)
+    dxhat = oracle.tensor_item_production(delta, gamma)
+    zero = np.zeros(one, np.float32)
+    assert np.array_equal(t_dx.numpy(), dxhat)
+    close(t_s1.numpy(), oracle.add_sum_w(zero, dxhat, out_init=zero), 1e-5)
+    close(t_s2.numpy(), oracle.add_sum_w(zero, oracle.tensor_item_production(dxhat, fwd["xhat"]), out_init=zero), 1e-5)
 
 
 @pytest.mark.parametrize("shape", [(16, 3, 6, 6), (5, 2, 3, 3), (130, 4, 8, 8), (300, 1, 4, 8)])
