@@ -525,6 +525,53 @@ static void FusedSequenceChecks(void)
  mi355::FuseSequences()=true;
 }
 
+// Copies share their device block until one side is written (mi355::CDeviceBuffer): every way of writing one side must
+// leave the other as it was.
+static void SharedBlockChecks(void)
+{
+ CTensor<type_t> a(4,2,8,8),b(4,2,8,8),ones(4,2,8,8),bias(1,2,1,1);
+ FillPattern(a,1,1.0f);
+ CTensorMath<type_t>::Fill(ones,1);
+ bias.SetElement(0,0,0,0,10);bias.SetElement(0,1,0,0,20);
+ CTensorMath<type_t>::Add(a,a,ones,1,0);        // a lives on the device now
+ CTensor<type_t> original=a;
+ original.GetElement(0,0,0,0);                   // ... and `original` on the host as well: a reference that no later write can reach
+ double largest=0;
+ bool ok=true;
+ // overwritten as a whole
+ b=a;
+ CTensorMath<type_t>::Fill(a,5);
+ ok=ok && MaxDifference(b,original,largest)==0 && a.GetElement(3,1,7,7)==5;
+ // written in place by a deferred call, and by a call that is not deferred
+ a=b;
+ CTensorMath<type_t>::Add(a,a,ones,1,1);
+ ok=ok && MaxDifference(b,original,largest)==0 && a.GetElement(0,0,0,1)==original.GetElement(0,0,0,1)+1;
+ a=b;
+ CTensorMath<type_t>::AddBias(a,bias);
+ ok=ok && MaxDifference(b,original,largest)==0 && a.GetElement(2,1,3,3)==original.GetElement(2,1,3,3)+20;
+ // the copy is written, the source stays
+ a=b;
+ CTensorMath<type_t>::Mul(b,b,static_cast<type_t>(2));
+ ok=ok && MaxDifference(a,original,largest)==0 && b.GetElement(1,0,2,2)==2*original.GetElement(1,0,2,2);
+ // written from the host, partly and as a whole
+ b=a;
+ type_t row[8]={9,9,9,9,9,9,9,9};
+ b.CopyItemToDevice(row,8);
+ ok=ok && MaxDifference(a,original,largest)==0 && b.GetElement(0,0,0,7)==9 && b.GetElement(0,0,1,0)==original.GetElement(0,0,1,0);
+ b=a;
+ b.SetElement(0,0,0,0,-3);
+ CTensorMath<type_t>::Add(b,b,ones,1,0);
+ ok=ok && MaxDifference(a,original,largest)==0 && b.GetElement(0,0,0,0)==-3 && b.GetElement(3,1,7,7)==original.GetElement(3,1,7,7);
+ // a chain of copies, the middle one updated by Adam (reads and writes weights and both moments)
+ CTensor<type_t> w1=original,w2,w3,m(4,2,8,8),v(4,2,8,8);
+ w2=w1;w3=w2;
+ CTensor<type_t> m_copy=m;
+ CTensorMath<type_t>::Fill(m,0);CTensorMath<type_t>::Fill(v,0);
+ CTensorMath<type_t>::Adam(w2,ones,m,v,4,0.01,0.9,0.999,1e-8,1);
+ ok=ok && MaxDifference(w1,original,largest)==0 && MaxDifference(w3,original,largest)==0 && MaxDifference(w2,original,largest)>0;
+ Report("copies share a device block until one side is written",ok);
+}
+
 // the scope timer the reference's models wrap around their training phases (cuda/ctimestamp.cu.h)
 static void TimerCheck(void)
 {
@@ -552,6 +599,7 @@ int main(void)
   BackwardConvolutionCheck();
   DeferredGradientChecks();
   FusedSequenceChecks();
+  SharedBlockChecks();
   SummXYCheck();
   CoherenceAndErrors();
   GpuClassOnlyChecks();

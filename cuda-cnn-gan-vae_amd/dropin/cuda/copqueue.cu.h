@@ -136,6 +136,7 @@ namespace mi355
  struct SBatchNormForward///<netlayer/cnetlayerbatchnormalization.cu.h:301-371, training mode
  {
   mt_tensor Mean,X,NewMean,XHat,Var,Scratch,NewVar,SqrtVar,IVar,Gamma,Beta,H;
+  mt_tensor OldMean,OldVar;///<what the running statistics are blended from: the same tensors, unless they shared their block with a copy
   float Momentum,Epsilon;
   enum {LENGTH=13};
  };
@@ -173,8 +174,8 @@ namespace mi355
            m.Mean=o.T[0];break;
     case 1:if (o.Kind!=OP_ADD_SUM_W || !Same(o.T[0],m.Mean) || !Same(o.T[1],m.Mean) || o.A!=1 || o.T[2].w==0 || !Near(o.B,1.0/o.T[2].w) || !SameSample(o.T[2],m.Mean)) return(0);
            m.X=o.T[2];break;
-    case 2:if (o.Kind!=OP_ADD || !Same(o.T[0],o.T[1]) || !Same(o.T[2],m.Mean) || !OneSampleOf(o.T[0],m.X) || !Near(o.B,1.0-static_cast<double>(o.A))) return(0);
-           m.NewMean=o.T[0];m.Momentum=o.A;break;
+    case 2:if (o.Kind!=OP_ADD || !OneSampleOf(o.T[1],m.X) || !Same(o.T[2],m.Mean) || !OneSampleOf(o.T[0],m.X) || !Near(o.B,1.0-static_cast<double>(o.A))) return(0);
+           m.NewMean=o.T[0];m.OldMean=o.T[1];m.Momentum=o.A;break;
     case 3:if (o.Kind!=OP_SUB || !Same(o.T[1],m.X) || !Same(o.T[2],m.Mean) || o.A!=1 || o.B!=1 || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
            m.XHat=o.T[0];break;
     case 4:if (o.Kind!=OP_FILL || o.A!=0 || !OneSampleOf(o.T[0],m.X)) return(0);
@@ -183,8 +184,8 @@ namespace mi355
            m.Scratch=o.T[0];break;
     case 6:if (o.Kind!=OP_ADD_SUM_W || !Same(o.T[0],m.Var) || !Same(o.T[1],m.Var) || !Same(o.T[2],m.Scratch) || o.A!=1 || !Near(o.B,1.0/m.X.w)) return(0);
            break;
-    case 7:if (o.Kind!=OP_ADD || !Same(o.T[0],o.T[1]) || !Same(o.T[2],m.Var) || !OneSampleOf(o.T[0],m.X) || o.A!=m.Momentum || !Near(o.B,1.0-static_cast<double>(o.A))) return(0);
-           m.NewVar=o.T[0];break;
+    case 7:if (o.Kind!=OP_ADD || !OneSampleOf(o.T[1],m.X) || !Same(o.T[2],m.Var) || !OneSampleOf(o.T[0],m.X) || o.A!=m.Momentum || !Near(o.B,1.0-static_cast<double>(o.A))) return(0);
+           m.NewVar=o.T[0];m.OldVar=o.T[1];break;
     case 8:if (o.Kind!=OP_SQRT || !Same(o.T[1],m.Var) || o.A!=1 || !OneSampleOf(o.T[0],m.X)) return(0);
            m.SqrtVar=o.T[0];m.Epsilon=o.B;break;
     case 9:if (o.Kind!=OP_INV || !Same(o.T[1],m.SqrtVar) || !OneSampleOf(o.T[0],m.X)) return(0);
@@ -199,7 +200,15 @@ namespace mi355
   }
   if (n<SBatchNormForward::LENGTH) return(1);
   const mt_tensor *all[12]={&m.Mean,&m.X,&m.NewMean,&m.XHat,&m.Var,&m.Scratch,&m.NewVar,&m.SqrtVar,&m.IVar,&m.Gamma,&m.Beta,&m.H};
-  return(Distinct(all,12)==true?2:0);
+  if (Distinct(all,12)==false) return(0);
+  // a running statistic blended from another block (its tensor shared the old one with a copy) must not be one of the outputs
+  for(int n=0;n<12;n++)
+  {
+   if (Same(m.OldMean,m.NewMean)==false && Overlap(m.OldMean,*all[n])==true && all[n]!=&m.NewMean) return(0);
+   if (Same(m.OldVar,m.NewVar)==false && Overlap(m.OldVar,*all[n])==true && all[n]!=&m.NewVar) return(0);
+  }
+  if ((Same(m.OldMean,m.NewMean)==false && Overlap(m.OldMean,m.NewMean)==true) || (Same(m.OldVar,m.NewVar)==false && Overlap(m.OldVar,m.NewVar)==true)) return(0);
+  return(2);
  }
 
  inline int MatchBatchNormInference(const std::vector<SOp> &q,size_t first,SBatchNormInference &m)
@@ -413,7 +422,12 @@ namespace mi355
    {
     Settle(&sequence[0],sequence.size());
     ForwardFused++;
-    Check(mt_batchnorm_forward_train_func(&m.H,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,m.Momentum,m.Epsilon,MT_F_NONE));
+    // the kernel blends a running statistic in place; one that comes from another block is blended by its own call
+    const bool mean_in_place=Same(m.OldMean,m.NewMean),var_in_place=Same(m.OldVar,m.NewVar);
+    Check(mt_batchnorm_forward_train_func(&m.H,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,mean_in_place==true?&m.NewMean:NULL,var_in_place==true?&m.NewVar:NULL,
+                                          m.Momentum,m.Epsilon,MT_F_NONE));
+    if (mean_in_place==false) RunLiteral(sequence[2]);
+    if (var_in_place==false) RunLiteral(sequence[7]);
     Pending.push_back(sequence[8]);///<SqrtVar = sqrt(Var + epsilon)
     Pending.push_back(sequence[11]);///<Scratch = Gamma * XHat
    }

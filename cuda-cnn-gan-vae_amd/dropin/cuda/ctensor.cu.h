@@ -21,57 +21,70 @@
 
 namespace mi355
 {
- // owning device buffer with value semantics (copying copies the device data, :159-170 of the reference vector)
+ // Device buffer with value semantics (copying a CCUDADeviceVector copies the device data, cuda/ccudadevicevector.cu.h:159-170)
+ // whose copies share one block until one of them is written: the layers hand whole activations on with operator= on
+ // every step (cTensor_Delta=error in every SetOutputError, netlayer/cnetlayerconvolution.cu.h:571; the batch-norm layer's
+ // running statistics, netlayer/cnetlayerbatchnormalization.cu.h:617-618), and the copy is almost always replaced as a whole
+ // before anybody changes one side.  Whoever is about to write calls Own() first: a block of its own, with the present
+ // contents only if the write keeps part of them.  The block goes back to the library when its last owner lets go.
  class CDeviceBuffer
  {
-   void *Ptr;
-   size_t Bytes;
-  public:
-   CDeviceBuffer(void):Ptr(NULL),Bytes(0) {}
-   CDeviceBuffer(const CDeviceBuffer &other):Ptr(NULL),Bytes(0) {*this=other;}
-   ~CDeviceBuffer() {clear();}
-   CDeviceBuffer& operator=(const CDeviceBuffer &other)
+   struct SBlock
    {
-    if (this==&other) return(*this);
-    resize(other.Bytes);
-    if (Bytes!=0)
+    void *Ptr;
+    size_t Bytes;
+    SBlock(void):Ptr(NULL),Bytes(0) {}
+    ~SBlock()
     {
-     Queue().Access(other.Ptr,other.Bytes,true,false);
-     Queue().Access(Ptr,Bytes,false,true);
-     Check(mt_copy_d2d(Ptr,other.Ptr,Bytes));
-    }
-    return(*this);
-   }
-   void clear(void)
-   {
-    if (Ptr!=NULL)
-    {
-     Queue().Access(Ptr,Bytes,false,true);///<deferred calls that name the block run (or are forgotten) before it goes
+     if (Ptr==NULL) return;
+     try {Queue().Access(Ptr,Bytes,false,true);} catch(const char*) {}///<deferred calls that name the block run (or are forgotten) before it goes
      mt_free(Ptr);
     }
-    Ptr=NULL;
-    Bytes=0;
+   };
+   std::shared_ptr<SBlock> Block;
+   static std::shared_ptr<SBlock> Make(size_t bytes)
+   {
+    std::shared_ptr<SBlock> block(new SBlock);
+    Check(mt_malloc(&block->Ptr,bytes));
+    block->Bytes=bytes;
+    return(block);
    }
+  public:
+   CDeviceBuffer(void) {}
+   CDeviceBuffer(const CDeviceBuffer &other):Block(other.Block) {}
+   CDeviceBuffer& operator=(const CDeviceBuffer &other) {Block=other.Block;return(*this);}
+   void clear(void) {Block.reset();}
+   // a block of `bytes` bytes that nobody else holds; the contents are undefined
    void resize(size_t bytes)
    {
-    if (bytes==Bytes) return;
-    clear();
-    if (bytes!=0) Check(mt_malloc(&Ptr,bytes));
-    Bytes=bytes;
+    if (bytes==size() && (bytes==0 || Block.use_count()==1)) return;
+    Block.reset();
+    if (bytes!=0) Block=Make(bytes);
    }
    void assign(const void *device_source,size_t bytes)
    {
     resize(bytes);
-    if (Bytes!=0)
-    {
-     Queue().Access(device_source,bytes,true,false);
-     Queue().Access(Ptr,Bytes,false,true);
-     Check(mt_copy_d2d(Ptr,device_source,Bytes));
-    }
+    if (bytes==0) return;
+    Queue().Access(device_source,bytes,true,false);
+    Queue().Access(Block->Ptr,bytes,false,true);
+    Check(mt_copy_d2d(Block->Ptr,device_source,bytes));
    }
-   void swap(CDeviceBuffer &other) {std::swap(Ptr,other.Ptr);std::swap(Bytes,other.Bytes);}
-   void* get(void) const {return(Ptr);}
-   size_t size(void) const {return(Bytes);}
+   // before a write: the block becomes this object's alone; `keep` carries the present contents over
+   void Own(bool keep)
+   {
+    if (!Block || Block.use_count()==1) return;
+    std::shared_ptr<SBlock> mine=Make(Block->Bytes);
+    if (keep==true)
+    {
+     Queue().Access(Block->Ptr,Block->Bytes,true,false);
+     Check(mt_copy_d2d(mine->Ptr,Block->Ptr,Block->Bytes));
+    }
+    Block.swap(mine);
+   }
+   bool Shared(void) const {return(Block && Block.use_count()>1);}
+   void swap(CDeviceBuffer &other) {Block.swap(other.Block);}
+   void* get(void) const {return(Block?Block->Ptr:NULL);}
+   size_t size(void) const {return(Block?Block->Bytes:0);}
  };
 
  // Per-sample weight gradients of a convolution layer that were asked for and not computed.  The reference's layer
@@ -241,6 +254,7 @@ class CTensor
    if (Item.size()<size) throw("CTensor::CopyItemToDevice: array larger than the tensor");
    Materialise();
    CopyToDevice();
+   DeviceItem.Own(true);
    mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),true,true);
    mi355::Check(mt_copy_h2d(DeviceItem.get(),item_array,size*sizeof(type_t)));
    SetDeviceOnChange();
@@ -259,6 +273,7 @@ class CTensor
    if (Item.size()<size+offset) throw("CTensor::CopyItemLayerWToDevice: array larger than the tensor");
    Materialise();
    CopyToDevice();
+   DeviceItem.Own(true);
    mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),true,true);
    mi355::Check(mt_copy_h2d(static_cast<type_t*>(DeviceItem.get())+offset,item_array,size*sizeof(type_t)));
    SetDeviceOnChange();
@@ -359,6 +374,7 @@ class CTensor
   {
    if (HostOnChange==false && force==false) return;
    DropLazy();
+   DeviceItem.Own(false);
    mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),false,true);
    if (!Item.empty()) mi355::Check(mt_copy_h2d(DeviceItem.get(),&Item[0],Item.size()*sizeof(type_t)));
    HostOnChange=false;
@@ -381,6 +397,7 @@ class CTensor
   void Materialise(void) const
   {
    if (Lazy==LAZY_NONE) return;
+   DeviceItem.Own(false);
    mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),false,true);
    const uint8_t kind=Lazy;
    std::shared_ptr<mi355::CDeferredGradient> record;
@@ -500,6 +517,7 @@ class CTensor
   // the device copy is said to hold zeros; nothing is launched (CTensorMath::Fill)
   void SetLazyZero(void) const
   {
+   DeviceItem.Own(false);
    mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),false,true);///<as far as deferred calls are concerned the tensor is overwritten now
    DropLazy();
    Lazy=LAZY_ZERO;
@@ -508,28 +526,45 @@ class CTensor
   }
   size_t Count(void) const {return(static_cast<size_t>(Size_X)*Size_Y*Size_Z*Size_W);}
   size_t Index(uint32_t w,uint32_t z,uint32_t y,uint32_t x) const {return(x+static_cast<size_t>(Size_X)*(y+static_cast<size_t>(Size_Y)*(z+static_cast<size_t>(Size_Z)*w)));}
-  // descriptor of the device copy for a call that is deferred (mi355::COpQueue): the queue itself keeps the order
-  mt_tensor DeviceQueued(bool upload) const
+  // Descriptors of the device copy for the C ABI.  Read: the tensor is an input (brought up to date first).  Device(true):
+  // the call reads and writes it (an accumulator, an in-place operation); Device(false): the call overwrites all of it.
+  // A tensor that is about to be written stops sharing its block with its copies (CDeviceBuffer::Own).  Deferred calls
+  // (mi355::COpQueue) that involve the tensor run first; the *Queued forms are for calls that are deferred themselves,
+  // whose order the queue keeps.
+  mt_tensor Descriptor(void) const
   {
-   Materialise();
-   if (upload==true) CopyToDevice();
    mt_tensor t;
    t.p=static_cast<float*>(DeviceItem.get());
    t.w=Size_W;t.z=Size_Z;t.y=Size_Y;t.x=Size_X;
    return(t);
   }
-  // descriptor of the device copy for the C ABI; `upload` first brings the device copy up to date (the tensor is read,
-  // and may be written as well); without it the call overwrites the whole tensor.  Deferred calls that involve the
-  // tensor run first.
+  mt_tensor DeviceQueuedRead(void) const
+  {
+   Materialise();
+   CopyToDevice();
+   return(Descriptor());
+  }
+  mt_tensor DeviceQueued(bool upload) const
+  {
+   Materialise();
+   if (upload==true) CopyToDevice();
+   DeviceItem.Own(upload);
+   return(Descriptor());
+  }
+  mt_tensor DeviceRead(void) const
+  {
+   Materialise();
+   CopyToDevice();
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),true,false);
+   return(Descriptor());
+  }
   mt_tensor Device(bool upload) const
   {
    Materialise();
    if (upload==true) CopyToDevice();
+   DeviceItem.Own(upload);
    mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),upload,true);
-   mt_tensor t;
-   t.p=static_cast<float*>(DeviceItem.get());
-   t.w=Size_W;t.z=Size_Z;t.y=Size_Y;t.x=Size_X;
-   return(t);
+   return(Descriptor());
   }
 };
 

@@ -15,7 +15,7 @@ class CTensorApplyFunc
   static void Apply(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,int func)
   {
    static_assert(std::is_same<type_t,float>::value,"the MI355X tensor path computes in fp32 only");
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_apply_func(&o,&i,func));
    cTensor_Output.SetDeviceOnChange();
   }

@@ -28,14 +28,14 @@ class CTensorConv
   static void ForwardConvolution(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Image,const CTensor<type_t> &cTensor_Kernel,int32_t kernel_x,int32_t kernel_y,int32_t kernel_z,uint32_t kernel_amount,const CTensor<type_t> &cTensor_Bias,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Image.Device(true),k=cTensor_Kernel.Device(true),b=cTensor_Bias.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Image.DeviceRead(),k=cTensor_Kernel.DeviceRead(),b=cTensor_Bias.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_forward_convolution(&o,&i,&k,kernel_x,kernel_y,kernel_z,kernel_amount,&b,stride_x,stride_y,padding_x,padding_y));
    cTensor_Output.SetDeviceOnChange();
   }
   static void BackwardConvolution(CTensor<type_t> &cTensor_OutputDelta,const CTensor<type_t> &cTensor_Delta,const CTensor<type_t> &cTensor_Kernel,int32_t kernel_x,int32_t kernel_y,int32_t kernel_z,uint32_t kernel_amount,const CTensor<type_t> &cTensor_Bias,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)
   {
    OnlyFloat();
-   mt_tensor d=cTensor_Delta.Device(true),k=cTensor_Kernel.Device(true),b=cTensor_Bias.Device(true),o=cTensor_OutputDelta.Device(false);
+   mt_tensor d=cTensor_Delta.DeviceRead(),k=cTensor_Kernel.DeviceRead(),b=cTensor_Bias.DeviceRead(),o=cTensor_OutputDelta.Device(false);
    mi355::Check(mt_backward_convolution(&o,&d,&k,kernel_x,kernel_y,kernel_z,kernel_amount,&b,stride_x,stride_y,padding_x,padding_y));
    cTensor_OutputDelta.SetDeviceOnChange();
   }
@@ -47,7 +47,7 @@ class CTensorConv
     // Two zeroed per-sample tensors: the sums over the batch now, from the operands as they are; copies of the operands
     // for whoever reads a sample's gradient later (mi355::CDeferredGradient).
     std::shared_ptr<mi355::CDeferredGradient> record(new mi355::CDeferredGradient);
-    mt_tensor i=cTensor_Image.Device(true),d=cTensor_Delta.Device(true);
+    mt_tensor i=cTensor_Image.DeviceRead(),d=cTensor_Delta.DeviceRead();
     record->Kernel_X=dkernel_x;record->Kernel_Y=dkernel_y;record->Kernel_Z=dkernel_z;record->Kernel_Amount=dkernel_amount;
     record->Stride_X=stride_x;record->Stride_Y=stride_y;record->Padding_X=padding_x;record->Padding_Y=padding_y;
     const CTensor<type_t> *batch[2]={&cTensor_dKernel,&cTensor_dBias};
@@ -65,16 +65,17 @@ class CTensorConv
     // the summed kernel gradient is addressed as [1,1,Kamt,C*Ky*Kx] whatever Z x Y split the layer gave its tensor
     total[0].y*=total[0].z;total[0].z=1;
     mi355::Check(mt_convolution_backward_weights_sum(&total[0],dkernel_x,dkernel_y,dkernel_z,dkernel_amount,&total[1],&i,&d,stride_x,stride_y,padding_x,padding_y));
-    record->Image.assign(i.p,static_cast<size_t>(i.w)*i.z*i.y*i.x*sizeof(float));
-    record->Delta.assign(d.p,static_cast<size_t>(d.w)*d.z*d.y*d.x*sizeof(float));
-    record->ImageTensor=i;record->ImageTensor.p=static_cast<float*>(record->Image.get());
-    record->DeltaTensor=d;record->DeltaTensor.p=static_cast<float*>(record->Delta.get());
+    // the operands as they are now: the record shares their blocks, and a tensor that is written later takes a new one
+    record->Image=cTensor_Image.DeviceItem;
+    record->Delta=cTensor_Delta.DeviceItem;
+    record->ImageTensor=i;
+    record->DeltaTensor=d;
     cTensor_dKernel.Lazy=CTensor<type_t>::LAZY_GRADIENT_KERNEL;cTensor_dKernel.Deferred=record;
     cTensor_dBias.Lazy=CTensor<type_t>::LAZY_GRADIENT_BIAS;cTensor_dBias.Deferred=record;
     return;
    }
    // both gradients accumulate: bring their device copies up to date first
-   mt_tensor dk=cTensor_dKernel.Device(true),db=cTensor_dBias.Device(true),i=cTensor_Image.Device(true),d=cTensor_Delta.Device(true);
+   mt_tensor dk=cTensor_dKernel.Device(true),db=cTensor_dBias.Device(true),i=cTensor_Image.DeviceRead(),d=cTensor_Delta.DeviceRead();
    mi355::Check(mt_create_delta_weight_and_bias(&dk,dkernel_x,dkernel_y,dkernel_z,dkernel_amount,&db,&i,&d,stride_x,stride_y,padding_x,padding_y));
    cTensor_dKernel.SetDeviceOnChange();
    cTensor_dBias.SetDeviceOnChange();
@@ -82,7 +83,7 @@ class CTensorConv
   static void CreateBackDeltaWeightAndBias(CTensor<type_t> &cTensor_dKernel,int32_t dkernel_x,int32_t dkernel_y,int32_t dkernel_z,uint32_t dkernel_amount,CTensor<type_t> &cTensor_dBias,CTensor<type_t> &cTensor_Image,const CTensor<type_t> &cTensor_Delta,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)
   {
    OnlyFloat();
-   mt_tensor dk=cTensor_dKernel.Device(true),db=cTensor_dBias.Device(true),i=cTensor_Image.Device(true),d=cTensor_Delta.Device(true);
+   mt_tensor dk=cTensor_dKernel.Device(true),db=cTensor_dBias.Device(true),i=cTensor_Image.DeviceRead(),d=cTensor_Delta.DeviceRead();
    mi355::Check(mt_create_back_delta_weight_and_bias(&dk,dkernel_x,dkernel_y,dkernel_z,dkernel_amount,&db,&i,&d,stride_x,stride_y,padding_x,padding_y));
    cTensor_dKernel.SetDeviceOnChange();
    cTensor_dBias.SetDeviceOnChange();

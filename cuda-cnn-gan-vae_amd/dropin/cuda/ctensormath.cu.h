@@ -24,7 +24,7 @@ class CTensorMath
   static void OnlyFloat(void) {static_assert(std::is_same<type_t,float>::value,"the MI355X tensor path computes in fp32 only");}
   static mt_pos_tensor Position(const CTensor<SPos> &cTensor,bool upload)
   {
-   mt_tensor t=cTensor.Device(upload);
+   mt_tensor t=(upload==true)?cTensor.DeviceRead():cTensor.Device(false);
    mt_pos_tensor p;
    p.p=reinterpret_cast<mt_spos*>(t.p);
    p.w=t.w;p.z=t.z;p.y=t.y;p.x=t.x;
@@ -47,21 +47,21 @@ class CTensorMath
   static void Inv(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mt_tensor i=cTensor_Input.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeUnary(mi355::OP_INV,o,i));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Div(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor l=cTensor_Left.DeviceRead(),r=cTensor_Right.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_div(&o,&l,&r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Add(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.DeviceQueued(true),r=cTensor_Right.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mt_tensor l=cTensor_Left.DeviceQueuedRead(),r=cTensor_Right.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_ADD,o,l,r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();
   }
@@ -83,68 +83,68 @@ class CTensorMath
     mt_tensor r;
     r.p=static_cast<float*>(kernel?record->KernelSum.get():record->BiasSum.get());
     r.w=1;r.z=cTensor_Right.GetSizeZ();r.y=cTensor_Right.GetSizeY();r.x=cTensor_Right.GetSizeX();
-    mt_tensor l=cTensor_Left.Device(true),o=cTensor_Output.Device(false);
+    mt_tensor l=cTensor_Left.DeviceRead(),o=cTensor_Output.Device(false);
     mi355::Check(mt_add_sum_w(&o,&l,&r,left_scale,right_scale));
     cTensor_Output.SetDeviceOnChange();
     return;
    }
-   mt_tensor l=cTensor_Left.DeviceQueued(true),r=cTensor_Right.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mt_tensor l=cTensor_Left.DeviceQueuedRead(),r=cTensor_Right.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_ADD_SUM_W,o,l,r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();
   }
   static void AddValue(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t tensor_scale,type_t value)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_add_value(&o,&i,tensor_scale,value));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Sub(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const CTensor<type_t> &cTensor_Right,type_t left_scale=1,type_t right_scale=1)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.DeviceQueued(true),r=cTensor_Right.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mt_tensor l=cTensor_Left.DeviceQueuedRead(),r=cTensor_Right.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_SUB,o,l,r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();
   }
   static void SubValue(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t tensor_scale,type_t value)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_sub_value(&o,&i,tensor_scale,value));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Set(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t scale=1,type_t add_value=0)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_set(&o,&i,scale,add_value));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Pow2(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t scale=1)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mt_tensor i=cTensor_Input.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeUnary(mi355::OP_POW2,o,i,scale));
    cTensor_Output.SetDeviceOnChange();
   }
   static void SQRT(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,type_t scale,type_t add_sqrt_value)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mt_tensor i=cTensor_Input.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeUnary(mi355::OP_SQRT,o,i,scale,add_sqrt_value));
    cTensor_Output.SetDeviceOnChange();
   }
   static void AddBias(CTensor<type_t> &cTensor_Working,const CTensor<type_t> &cTensor_Bias)
   {
    OnlyFloat();
-   mt_tensor b=cTensor_Bias.Device(true),o=cTensor_Working.Device(true);
+   mt_tensor b=cTensor_Bias.DeviceRead(),o=cTensor_Working.Device(true);
    mi355::Check(mt_add_bias(&o,&b));
    cTensor_Working.SetDeviceOnChange();
   }
   static void SummXY(CTensor<type_t> &cTensor_Output,CTensor<type_t> &cTensor_Input)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(true);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(true);
    mi355::Check(mt_summ_xy(&o,&i));
    cTensor_Output.SetDeviceOnChange();
   }
@@ -152,7 +152,7 @@ class CTensorMath
   {
    OnlyFloat();
    (void)tensor_core;  // the reference's fp16 tensor-core switch; this path is always fp32 on the matrix cores
-   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor l=cTensor_Left.DeviceRead(),r=cTensor_Right.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_mul(&o,&l,&r));
    cTensor_Output.SetDeviceOnChange();
   }
@@ -160,14 +160,14 @@ class CTensorMath
   {
    OnlyFloat();
    (void)tensor_core;
-   mt_tensor l=cTensor_Left.Device(true),r=cTensor_Right.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor l=cTensor_Left.DeviceRead(),r=cTensor_Right.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_transponse_mul(&o,&l,&r));
    cTensor_Output.SetDeviceOnChange();
   }
   static void Mul(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Left,const type_t &value_right)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mt_tensor l=cTensor_Left.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeUnary(mi355::OP_MUL_VALUE,o,l,value_right));
    cTensor_Output.SetDeviceOnChange();
   }
@@ -178,14 +178,14 @@ class CTensorMath
   static void Transponse(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_transponse(&o,&i));
    cTensor_Output.SetDeviceOnChange();
   }
   static void TensorItemProduction(CTensor<type_t> &cTensor_Output,CTensor<type_t> &cTensor_Left,CTensor<type_t> &cTensor_Right)
   {
    OnlyFloat();
-   mt_tensor l=cTensor_Left.DeviceQueued(true),r=cTensor_Right.DeviceQueued(true),o=cTensor_Output.DeviceQueued(false);
+   mt_tensor l=cTensor_Left.DeviceQueuedRead(),r=cTensor_Right.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_ITEM_PRODUCTION,o,l,r));
    cTensor_Output.SetDeviceOnChange();
   }
@@ -198,21 +198,21 @@ class CTensorMath
   static void UpSampling(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,uint32_t upsampling_x,uint32_t upsampling_y)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_upsampling(&o,&i,upsampling_x,upsampling_y));
    cTensor_Output.SetDeviceOnChange();
   }
   static void DownSampling(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,uint32_t downsampling_x,uint32_t downsampling_y)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_downsampling(&o,&i,downsampling_x,downsampling_y));
    cTensor_Output.SetDeviceOnChange();
   }
   static void MaxPooling(CTensor<type_t> &cTensor_Output,const CTensor<SPos> &cTensor_Position,const CTensor<type_t> &cTensor_Input,uint32_t pooling_x,uint32_t pooling_y)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mt_pos_tensor p=Position(cTensor_Position,false);
    mi355::Check(mt_max_pooling(&o,&p,&i,pooling_x,pooling_y));
    cTensor_Output.SetDeviceOnChange();
@@ -221,7 +221,7 @@ class CTensorMath
   static void MaxPoolingBackward(CTensor<type_t> &cTensor_Output,const CTensor<SPos> &cTensor_Position,const CTensor<type_t> &cTensor_Input,uint32_t pooling_x,uint32_t pooling_y)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mt_pos_tensor p=Position(cTensor_Position,true);
    mi355::Check(mt_max_pooling_backward(&o,&p,&i,pooling_x,pooling_y));
    cTensor_Output.SetDeviceOnChange();
@@ -244,14 +244,14 @@ class CTensorMath
   static void ConcatecationZ(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_InputA,const CTensor<type_t> &cTensor_InputB)
   {
    OnlyFloat();
-   mt_tensor a=cTensor_InputA.Device(true),b=cTensor_InputB.Device(true),o=cTensor_Output.Device(false);
+   mt_tensor a=cTensor_InputA.DeviceRead(),b=cTensor_InputB.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_concatecation_z(&o,&a,&b));
    cTensor_Output.SetDeviceOnChange();
   }
   static void SplitZ(CTensor<type_t> &cTensor_OutputA,CTensor<type_t> &cTensor_OutputB,const CTensor<type_t> &cTensor_Input)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),a=cTensor_OutputA.Device(false),b=cTensor_OutputB.Device(false);
+   mt_tensor i=cTensor_Input.DeviceRead(),a=cTensor_OutputA.Device(false),b=cTensor_OutputB.Device(false);
    mi355::Check(mt_split_z(&a,&b,&i));
    cTensor_OutputA.SetDeviceOnChange();
    cTensor_OutputB.SetDeviceOnChange();
@@ -259,7 +259,7 @@ class CTensorMath
   static void SetTimeStep(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,const CTensor<uint32_t> &cTensor_TimeStep)
   {
    OnlyFloat();
-   mt_tensor i=cTensor_Input.Device(true),o=cTensor_Output.Device(false),t=cTensor_TimeStep.Device(true);
+   mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false),t=cTensor_TimeStep.DeviceRead();
    mt_u32_tensor ts;
    ts.p=reinterpret_cast<uint32_t*>(t.p);
    ts.w=t.w;ts.z=t.z;ts.y=t.y;ts.x=t.x;
@@ -284,7 +284,7 @@ class CTensorMath
   static void GetNoiseImageAndNoise(CTensor<type_t> &cTensor_NoisyImage,CTensor<type_t> &cTensor_Noise,const CTensor<type_t> &cTensor_Image,const CTensor<type_t> &cTensor_SqrtAlphaBar,const CTensor<type_t> &cTensor_SqrtOneMinusAlphaBar)
   {
    OnlyFloat();
-   mt_tensor im=cTensor_Image.Device(true),sa=cTensor_SqrtAlphaBar.Device(true),sb=cTensor_SqrtOneMinusAlphaBar.Device(true);
+   mt_tensor im=cTensor_Image.DeviceRead(),sa=cTensor_SqrtAlphaBar.DeviceRead(),sb=cTensor_SqrtOneMinusAlphaBar.DeviceRead();
    mt_tensor ni=cTensor_NoisyImage.Device(false),no=cTensor_Noise.Device(false);
    mi355::Check(mt_get_noise_image_and_noise(&ni,&no,&im,&sa,&sb,static_cast<uint64_t>(rand())));
    cTensor_Noise.SetDeviceOnChange();
@@ -293,7 +293,7 @@ class CTensorMath
   static void Adam(CTensor<type_t> &cTensor_Weight,CTensor<type_t> &cTensor_dWeight,CTensor<type_t> &cTensor_M,CTensor<type_t> &cTensor_V,uint32_t batch_size,double speed,double beta1,double beta2,double epsilon,double iteration)
   {
    OnlyFloat();
-   mt_tensor w=cTensor_Weight.DeviceQueued(true),dw=cTensor_dWeight.DeviceQueued(true),m=cTensor_M.DeviceQueued(true),v=cTensor_V.DeviceQueued(true);
+   mt_tensor w=cTensor_Weight.DeviceQueued(true),dw=cTensor_dWeight.DeviceQueuedRead(),m=cTensor_M.DeviceQueued(true),v=cTensor_V.DeviceQueued(true);
    mi355::Queue().Submit(mi355::MakeAdam(w,dw,m,v,batch_size,speed,beta1,beta2,epsilon,iteration));
    cTensor_Weight.SetDeviceOnChange();
    cTensor_M.SetDeviceOnChange();
