@@ -554,7 +554,8 @@ __global__ __launch_bounds__(EW_THREADS) void adam_many_kernel(ManyAdam a, uint3
 // Produces mean, biased variance and 1/sqrt(var+eps), and blends the running statistics.
 template <int V>
 __global__ __launch_bounds__(EW_THREADS) void bn_stats_kernel(const float *x, uint32_t W, uint32_t S, float inv_n, float eps, float *mean,
-                                                              float *var, float *ivar, float *new_mean, float *new_var, float mom_old, float mom_new) {
+                                                              float *var, float *ivar, float *new_mean, float *new_var, float mom_old, float mom_new,
+                                                              const float *old_mean, const float *old_var) {
   constexpr int RB = 32, WS = EW_THREADS / RB;
   __shared__ float part[2][WS][RB * V];
   const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
@@ -603,8 +604,8 @@ __global__ __launch_bounds__(EW_THREADS) void bn_stats_kernel(const float *x, ui
   mean[rc] = mu;
   var[rc] = vr;
   ivar[rc] = iv;
-  if (new_mean) new_mean[rc] = (mom_old * new_mean[rc]) + (mom_new * mu);
-  if (new_var) new_var[rc] = (mom_old * new_var[rc]) + (mom_new * vr);
+  if (new_mean) new_mean[rc] = (mom_old * old_mean[rc]) + (mom_new * mu);   // (old_*: the same tensors unless the caller blends from others)
+  if (new_var) new_var[rc] = (mom_old * old_var[rc]) + (mom_new * vr);
 }
 
 // Pass 2: out = func(gamma * ((x - mean) * ivar) + beta), optionally storing xhat.
@@ -641,7 +642,8 @@ __global__ __launch_bounds__(EW_THREADS) void bn_apply_kernel(float *out, float 
 template <int RB, int NW>
 __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float *xhat, const float *x, uint32_t W, uint32_t S, float inv_n, float eps,
                                                               float *mean, float *var, float *ivar, float *new_mean, float *new_var, float mom_old,
-                                                              float mom_new, const float *gamma, const float *beta, int func) {
+                                                              float mom_new, const float *gamma, const float *beta, int func, const float *old_mean,
+                                                              const float *old_var) {
   constexpr int WS = EW_THREADS / RB;
   __shared__ __attribute__((aligned(16))) float part[2][WS][RB * 4];
   __shared__ __attribute__((aligned(16))) float col_mean[RB * 4], col_ivar[RB * 4];
@@ -683,8 +685,8 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
     mean[rc] = mu;
     var[rc] = vr;
     ivar[rc] = iv;
-    if (new_mean) new_mean[rc] = (mom_old * new_mean[rc]) + (mom_new * mu);
-    if (new_var) new_var[rc] = (mom_old * new_var[rc]) + (mom_new * vr);
+    if (new_mean) new_mean[rc] = (mom_old * old_mean[rc]) + (mom_new * mu);
+    if (new_var) new_var[rc] = (mom_old * old_var[rc]) + (mom_new * vr);
     col_mean[c] = mu;
     col_ivar[c] = iv;
   }
@@ -1007,9 +1009,9 @@ int bn_statistics(const mt_tensor *x, const mt_tensor *gamma, const mt_tensor *b
   {
     mt::ProfileScope prof("bn_stats");
     if (S % 4 == 0 && aligned16(x->p))
-      bn_stats_kernel<4><<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(x->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new);
+      bn_stats_kernel<4><<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(x->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, nm, nv);
     else
-      bn_stats_kernel<1><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(x->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new);
+      bn_stats_kernel<1><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(x->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, nm, nv);
     MT_LAUNCH_CHECK("bn_stats");
   }
   bn_scale_shift_kernel<<<cdiv(S, EW_THREADS), EW_THREADS, 0, mt::stream()>>>(reinterpret_cast<float2 *>(scale_shift->p), pm, pi, gamma->p, beta->p, (uint32_t)S);
@@ -1397,8 +1399,12 @@ int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor
 // fixed array (at most STATIC_SCRATCH_FLOATS / 3 elements per sample) and no launch is bracketed by profiling events.
 static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
                             const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
-                            const mt_tensor *new_variable, float momentum, float epsilon, int func, bool fixed_scratch) {
+                            const mt_tensor *new_variable, float momentum, float epsilon, int func, bool fixed_scratch,
+                            const mt_tensor *old_mean = nullptr, const mt_tensor *old_variable = nullptr) {
   if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: unknown function id %d", func);
+  if ((old_mean && !new_mean) || (old_variable && !new_variable)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_from: a statistic to blend from needs one to blend into");
+  for (auto t : {old_mean, old_variable})
+    if (t && (mt::bad(t) || !mt::same_zyx(t, in) || t->w == 0)) return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_from: statistics must be [1,Z,Y,X]");
   if (mt::bad(out) || mt::bad(in) || mt::bad(gamma) || mt::bad(beta)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: null tensor");
   for (auto t : {out, xhat, ivar, batch_mean, batch_var, new_mean, new_variable}) mt::note_write(t);
   if (!mt::same_zyx(in, out) || in->w != out->w || !mt::same_zyx(gamma, in) || !mt::same_zyx(beta, in) || gamma->w == 0 || beta->w == 0)
@@ -1426,6 +1432,7 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
   float inv_n = (float)(1.0 / (double)(float)W);  // the layer passes 1.0/N with N a float
   float mom_new = (float)(1.0 - (double)momentum);  // and 1.0-Momentum, rounded once
   float *nm = new_mean ? new_mean->p : nullptr, *nv = new_variable ? new_variable->p : nullptr;
+  const float *om = old_mean ? old_mean->p : nm, *ov = old_variable ? old_variable->p : nv;
   bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(pm) && aligned16(pi) && (!xhat || aligned16(xhat->p));
   if (vec && mt::epilogue_func(func)) {
     // one pass: the widest column block that still gives every compute unit a few blocks, if the batch share fits
@@ -1436,7 +1443,7 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
       mt::ProfileScope prof("bn_fused");
       const unsigned grid = cdiv(S, (size_t)rb * 4);
 #define MT_BN_FUSED(RB, NW) \
-  bn_fused_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func)
+  bn_fused_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func, om, ov)
 #define MT_BN_FUSED_NW(RB) \
   do { if (nw <= 8) MT_BN_FUSED(RB, 8); else if (nw <= 16) MT_BN_FUSED(RB, 16); else MT_BN_FUSED(RB, 32); } while (0)
       if (rb == 64) { if (nw <= 8) MT_BN_FUSED(64, 8); else MT_BN_FUSED(64, 16); }
@@ -1450,9 +1457,9 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
   {
   mt::ProfileScope prof("bn_stats");
   if (S % 4 == 0 && aligned16(in->p))
-    bn_stats_kernel<4><<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new);
+    bn_stats_kernel<4><<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, om, ov);
   else
-    bn_stats_kernel<1><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new);
+    bn_stats_kernel<1><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, om, ov);
   }
   MT_LAUNCH_CHECK("bn_stats");
   unsigned gx = cdiv(vec ? S / 4 : S, EW_THREADS);
@@ -1467,6 +1474,13 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
                                     const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
                                     const mt_tensor *new_variable, float momentum, float epsilon, int func) {
   return bn_forward_train(out, in, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func, false);
+}
+
+int mt_batchnorm_forward_train_from(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
+                                    const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
+                                    const mt_tensor *new_variable, const mt_tensor *old_mean, const mt_tensor *old_variable, float momentum, float epsilon,
+                                    int func) {
+  return bn_forward_train(out, in, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func, false, old_mean, old_variable);
 }
 
 int mt_batchnorm_forward_train_func_noalloc(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,

@@ -5,7 +5,7 @@
 // in training mode is 13 calls (netlayer/cnetlayerbatchnormalization.cu.h:301-371), its backward pass 12 or 15
 // (:578-604), and every layer clears its gradients and runs Adam tensor by tensor
 // (netlayer/cnetlayerconvolution.cu.h:522-539).  The library has one kernel for each of these sequences
-// (mt_batchnorm_forward_train_func, mt_batchnorm_forward_infer_func, mt_batchnorm_backward_keep, mt_fill_many,
+// (mt_batchnorm_forward_train_from, mt_batchnorm_forward_infer_func, mt_batchnorm_backward_keep, mt_fill_many,
 // mt_adam_many).  So the elementwise calls of CTensorMath are not run at once: they are appended to a queue, and
 //   * while the queue is the beginning of one of the known sequences (same operations, same tensors in the same roles,
 //     same scalars), it waits;
@@ -422,12 +422,7 @@ namespace mi355
    {
     Settle(&sequence[0],sequence.size());
     ForwardFused++;
-    // the kernel blends a running statistic in place; one that comes from another block is blended by its own call
-    const bool mean_in_place=Same(m.OldMean,m.NewMean),var_in_place=Same(m.OldVar,m.NewVar);
-    Check(mt_batchnorm_forward_train_func(&m.H,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,mean_in_place==true?&m.NewMean:NULL,var_in_place==true?&m.NewVar:NULL,
-                                          m.Momentum,m.Epsilon,MT_F_NONE));
-    if (mean_in_place==false) RunLiteral(sequence[2]);
-    if (var_in_place==false) RunLiteral(sequence[7]);
+    Check(mt_batchnorm_forward_train_from(&m.H,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,&m.OldMean,&m.OldVar,m.Momentum,m.Epsilon,MT_F_NONE));
     Pending.push_back(sequence[8]);///<SqrtVar = sqrt(Var + epsilon)
     Pending.push_back(sequence[11]);///<Scratch = Gamma * XHat
    }

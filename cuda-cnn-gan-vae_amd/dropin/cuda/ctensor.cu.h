@@ -97,7 +97,7 @@ namespace mi355
  // other way gets them: they are then computed from the kept operands (CTensor::Materialise).
  struct CDeferredGradient
  {
-  CDeviceBuffer Image;///<the operands as they were when the gradients were asked for
+  CDeviceBuffer Image;///<the operands as they were when the gradients were asked for (their blocks, shared)
   CDeviceBuffer Delta;
   mt_tensor ImageTensor;
   mt_tensor DeltaTensor;
@@ -105,8 +105,40 @@ namespace mi355
   uint32_t Kernel_Amount;
   uint32_t KernelSize[4];///<sizes of the two per-sample tensors when the gradients were asked for
   uint32_t BiasSize[4];
-  CDeviceBuffer KernelSum;///<[1,Z,Y,X] of the kernel tensor: the sum over the batch
+  CDeviceBuffer KernelSum;///<[1,Z,Y,X] of the kernel tensor: the sum over the batch, once somebody needs it on its own
   CDeviceBuffer BiasSum;
+  bool KernelReady;
+  bool BiasReady;
+  CDeferredGradient(void):KernelReady(false),BiasReady(false) {}
+  mt_tensor Sum(bool kernel)
+  {
+   const uint32_t *size=kernel?KernelSize:BiasSize;
+   CDeviceBuffer &buffer=kernel?KernelSum:BiasSum;
+   buffer.resize(static_cast<size_t>(size[1])*size[2]*size[3]*sizeof(float));
+   mt_tensor t;
+   t.p=static_cast<float*>(buffer.get());
+   t.w=1;t.z=size[1];t.y=size[2];t.x=size[3];
+   return(t);
+  }
+  // The sums over the batch from the kept operands.  `onto`: the kernel gradients are added straight onto this tensor
+  // (the layer's AddSumW(dKernel,dKernel,per-sample tensor)); without it they go to KernelSum.  The bias sums always go
+  // to BiasSum (a few hundred values).
+  void Compute(const mt_tensor *onto)
+  {
+   mt_tensor bias=Sum(false),kernel;
+   Check(mt_fill(&bias,0));
+   if (onto!=NULL) kernel=*onto;
+   else
+   {
+    kernel=Sum(true);
+    Check(mt_fill(&kernel,0));
+   }
+   // the summed kernel gradient is addressed as [1,1,Kamt,C*Ky*Kx] whatever Z x Y split the layer gave its tensor
+   kernel.y*=kernel.z;kernel.z=1;
+   Check(mt_convolution_backward_weights_sum(&kernel,Kernel_X,Kernel_Y,Kernel_Z,Kernel_Amount,&bias,&ImageTensor,&DeltaTensor,Stride_X,Stride_Y,Padding_X,Padding_Y));
+   BiasReady=true;
+   if (onto==NULL) KernelReady=true;
+  }
  };
  // switch for the deferral (on by default): with `false` every call runs when it is made
  inline bool& DeferGradients(void)

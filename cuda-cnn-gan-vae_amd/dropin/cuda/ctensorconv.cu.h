@@ -44,28 +44,19 @@ class CTensorConv
    OnlyFloat();
    if (Deferrable(cTensor_dKernel,cTensor_dBias,cTensor_Image,cTensor_Delta)==true)
    {
-    // Two zeroed per-sample tensors: the sums over the batch now, from the operands as they are; copies of the operands
-    // for whoever reads a sample's gradient later (mi355::CDeferredGradient).
+    // Two zeroed per-sample tensors: nothing is computed yet.  The record keeps the operands as they are (it shares their
+    // blocks; a tensor that is written later takes a new one); AddSumW of the per-sample tensors computes their sums over
+    // the batch, anybody else who reads them gets them computed then (mi355::CDeferredGradient).
     std::shared_ptr<mi355::CDeferredGradient> record(new mi355::CDeferredGradient);
     mt_tensor i=cTensor_Image.DeviceRead(),d=cTensor_Delta.DeviceRead();
     record->Kernel_X=dkernel_x;record->Kernel_Y=dkernel_y;record->Kernel_Z=dkernel_z;record->Kernel_Amount=dkernel_amount;
     record->Stride_X=stride_x;record->Stride_Y=stride_y;record->Padding_X=padding_x;record->Padding_Y=padding_y;
     const CTensor<type_t> *batch[2]={&cTensor_dKernel,&cTensor_dBias};
     uint32_t *size[2]={record->KernelSize,record->BiasSize};
-    mi355::CDeviceBuffer *sum[2]={&record->KernelSum,&record->BiasSum};
-    mt_tensor total[2];
     for(int n=0;n<2;n++)
     {
      size[n][0]=batch[n]->GetSizeW();size[n][1]=batch[n]->GetSizeZ();size[n][2]=batch[n]->GetSizeY();size[n][3]=batch[n]->GetSizeX();
-     sum[n]->resize(static_cast<size_t>(size[n][1])*size[n][2]*size[n][3]*sizeof(float));
-     total[n].p=static_cast<float*>(sum[n]->get());
-     total[n].w=1;total[n].z=size[n][1];total[n].y=size[n][2];total[n].x=size[n][3];
-     mi355::Check(mt_fill(&total[n],0));
     }
-    // the summed kernel gradient is addressed as [1,1,Kamt,C*Ky*Kx] whatever Z x Y split the layer gave its tensor
-    total[0].y*=total[0].z;total[0].z=1;
-    mi355::Check(mt_convolution_backward_weights_sum(&total[0],dkernel_x,dkernel_y,dkernel_z,dkernel_amount,&total[1],&i,&d,stride_x,stride_y,padding_x,padding_y));
-    // the operands as they are now: the record shares their blocks, and a tensor that is written later takes a new one
     record->Image=cTensor_Image.DeviceItem;
     record->Delta=cTensor_Delta.DeviceItem;
     record->ImageTensor=i;

@@ -77,12 +77,20 @@ class CTensorMath
    if (&cTensor_Right!=&cTensor_Output && &cTensor_Right!=&cTensor_Left &&
        (cTensor_Right.Lazy==CTensor<type_t>::LAZY_GRADIENT_KERNEL || cTensor_Right.Lazy==CTensor<type_t>::LAZY_GRADIENT_BIAS))
    {
-    // per-sample gradients that were not computed: their sum over the batch was, and is a one-sample tensor
+    // per-sample gradients that were not computed: their sum over the batch is, from the operands the record keeps
     const std::shared_ptr<mi355::CDeferredGradient> record=cTensor_Right.Deferred;
     const bool kernel=(cTensor_Right.Lazy==CTensor<type_t>::LAZY_GRADIENT_KERNEL);
-    mt_tensor r;
-    r.p=static_cast<float*>(kernel?record->KernelSum.get():record->BiasSum.get());
-    r.w=1;r.z=cTensor_Right.GetSizeZ();r.y=cTensor_Right.GetSizeY();r.x=cTensor_Right.GetSizeX();
+    if (kernel==true && record->KernelReady==false && &cTensor_Left==&cTensor_Output && left_scale==1 && right_scale==1 && cTensor_Output.GetSizeW()==1 &&
+        cTensor_Output.GetSizeZ()==cTensor_Right.GetSizeZ() && cTensor_Output.GetSizeY()==cTensor_Right.GetSizeY() && cTensor_Output.GetSizeX()==cTensor_Right.GetSizeX())
+    {
+     // the layer's own call, AddSumW(dKernel,dKernel,per-sample tensor): the sums are added straight onto dKernel
+     mt_tensor o=cTensor_Output.Device(true);
+     record->Compute(&o);
+     cTensor_Output.SetDeviceOnChange();
+     return;
+    }
+    if ((kernel==true && record->KernelReady==false) || (kernel==false && record->BiasReady==false)) record->Compute(NULL);
+    mt_tensor r=record->Sum(kernel);
     mt_tensor l=cTensor_Left.DeviceRead(),o=cTensor_Output.Device(false);
     mi355::Check(mt_add_sum_w(&o,&l,&r,left_scale,right_scale));
     cTensor_Output.SetDeviceOnChange();

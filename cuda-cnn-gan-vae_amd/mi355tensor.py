@@ -478,8 +478,12 @@ class Fused:
 
     @staticmethod
     def BatchNormForwardTrain(out, inp, gamma, beta, xhat=None, ivar=None, batch_mean=None, batch_var=None, new_mean=None, new_variable=None,
-                              momentum=0.9, epsilon=1e-6, func=None):
+                              momentum=0.9, epsilon=1e-6, func=None, old_mean=None, old_variable=None):
+        """old_mean / old_variable: the running statistics are blended from these tensors into new_mean / new_variable."""
         opt = lambda t: _d(t) if t is not None else None
+        if old_mean is not None or old_variable is not None:
+            return call("mt_batchnorm_forward_train_from", _d(out), _d(inp), _d(gamma), _d(beta), opt(xhat), opt(ivar), opt(batch_mean), opt(batch_var),
+                        opt(new_mean), opt(new_variable), opt(old_mean), opt(old_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
         call("mt_batchnorm_forward_train_func", _d(out), _d(inp), _d(gamma), _d(beta), opt(xhat), opt(ivar), opt(batch_mean), opt(batch_var),
              opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
 

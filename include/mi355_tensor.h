@@ -266,6 +266,14 @@ int mt_linear_batchnorm_forward_func(const mt_tensor *output, const mt_tensor *w
 int mt_batchnorm_forward_train_func(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
                                     const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var,
                                     const mt_tensor *new_mean, const mt_tensor *new_variable, float momentum, float epsilon, int func);
+/* The same call with the running statistics blended FROM other tensors: new_mean = momentum * old_mean + (1 - momentum) * batch
+ * mean, likewise the variance (lines 311 and 324 with cTensor_NewMean sharing its memory with cTensor_Mean, as it does after
+ * TrainingResetDeltaWeight, netlayer/cnetlayerbatchnormalization.cu.h:617-618, in a container whose copies share storage);
+ * old_mean / old_variable NULL: blended in place. */
+int mt_batchnorm_forward_train_from(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
+                                    const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var,
+                                    const mt_tensor *new_mean, const mt_tensor *new_variable, const mt_tensor *old_mean,
+                                    const mt_tensor *old_variable, float momentum, float epsilon, int func);
 /* The same call for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Statistics the caller does not ask for go to a
  * fixed array inside the library's code object (3 MiB per GPU, held until the process ends) instead of a workspace

@@ -789,6 +789,23 @@ def test_batchnorm_layer(gpu, oracle):
         close(got, exp, 1e-5)
 
 
+@pytest.mark.parametrize("shape", [(16, 3, 6, 6), (5, 2, 3, 3), (300, 1, 4, 8), (7, 64, 32, 32)])
+def test_batchnorm_running_statistics_blended_from_other_tensors(gpu, shape):
+    """new_mean = momentum * old_mean + (1 - momentum) * batch mean with old and new in different tensors: bit for bit what
+    the in-place call leaves in a copy of the old ones, and the old ones untouched."""
+    from mi355tensor import CTensor, Fused
+    from gpu_api import up
+    one = (1,) + tuple(shape[1:])
+    x, gamma, beta, om, ov = Nrm(1, *shape) + 0.3, U(2, *one) + 1.5, U(3, *one), U(4, *one), np.abs(U(5, *one))
+    tx, tg, tb = up(x), up(gamma), up(beta)
+    want_m, want_v, out_a = up(om), up(ov), CTensor(*shape)
+    Fused.BatchNormForwardTrain(out_a, tx, tg, tb, new_mean=want_m, new_variable=want_v, momentum=0.8)
+    old_m, old_v, new_m, new_v, out_b = up(om), up(ov), CTensor(*one), CTensor(*one), CTensor(*shape)
+    Fused.BatchNormForwardTrain(out_b, tx, tg, tb, new_mean=new_m, new_variable=new_v, momentum=0.8, old_mean=old_m, old_variable=old_v)
+    assert np.array_equal(new_m.numpy(), want_m.numpy()) and np.array_equal(new_v.numpy(), want_v.numpy())
+    assert np.array_equal(old_m.numpy(), om) and np.array_equal(old_v.numpy(), ov) and np.array_equal(out_a.numpy(), out_b.numpy())
+
+
 @pytest.mark.parametrize("shape", [(16, 3, 6, 6), (5, 2, 3, 3), (40, 8, 16, 16), (130, 4, 8, 8), (300, 1, 4, 8), (7, 64, 32, 32)])
 def test_batchnorm_backward_fused(gpu, oracle, shape):
     """The one-kernel backward pass against the layer's sequence of tensor operations, gradients accumulating into
