@@ -18,6 +18,7 @@
 
 #include "mt_igemm.h"
 #include "mt_walk.h"
+#include "mt_firstlayer.h"
 
 namespace {
 
@@ -25,6 +26,7 @@ using namespace mt::igemm;
 using mt::cdiv;
 
 int g_conv_path = 0;  // 0 auto, 1 direct, 2 implicit GEMM wherever it applies
+int g_first_layer = 1; // forward convolutions of 3-channel images: 0 never on the kernel that keeps the input patch in LDS and the weights in registers, 1 wherever the shape allows
 int g_conv_walk = 1;   // forward convolutions whose taps tile the k step: 0 never on the kernel whose blocks walk over the batch, 1 wherever the shape allows and gives 512 blocks, 2 wherever the shape allows
 int g_wgrad_groups = 0;  // 0 auto, else the number of batch groups of the batch-summed weight gradient (if it divides the batch)
 
@@ -1350,6 +1352,20 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
     return MT_OK;
   }
   uint32_t OHW = out->y * out->x;
+  // an image of three channels (a first layer): input patch in LDS, weights in registers, 128-bit stores (mt_firstlayer.h)
+  if (g_first_layer && kz == 3 && kernel->w == 1 && bias->w == 1 && image->w == out->w && mt::igemm::tile_override() < 0 && sx == sy && px >= 0 && py >= 0 &&
+      mt::fits_buffer(image)) {
+    FirstLayerArgs fl{};
+    fl.image = image->p; fl.kernel = kernel->p; fl.bias = bias->p; fl.out = out->p;
+    fl.ld = kernel->x; fl.KA = ka; fl.H = image->y; fl.W = image->x; fl.OH = out->y; fl.OW = out->x; fl.batch = out->w;
+    fl.pad_y = py; fl.pad_x = px;
+    fl.func = mt::epilogue_func(func) ? func : MT_F_NONE;
+    mt::ProfileScope prof(mt::profiling() ? shape_label(name, T32x128, ka, out->w * OHW, K, 1) : name);
+    if (first_layer_launch(name, fl, kz, ky, kx, sx, &rc)) {
+      if (rc) return rc;
+      return mt::epilogue_func(func) ? MT_OK : mt_apply_func(out, out, func);
+    }
+  }
   // Taps that tile the k step (4x4, 2x2, 1x1 kernels), one kernel and bias set, whole 64-channel row tiles: the kernel whose
   // blocks walk over the batch runs it (see mt_walk.h) when that gives at least two blocks per compute unit; products
   // with fewer tiles and a long k axis are better cut over k (launch_split below).
@@ -1968,6 +1984,11 @@ int set_image_mfma(int v) {
 int set_tconv_walk(int v) {
   if (v < 0 || v > 1) return fail(MT_E_ARGUMENT, "tconv_walk must be 0 (never for plain calls) or 1 (wherever the shape allows)");
   g_tconv_walk = v;
+  return MT_OK;
+}
+int set_first_layer(int v) {
+  if (v < 0 || v > 1) return fail(MT_E_ARGUMENT, "first_layer must be 0 (never) or 1 (wherever the shape allows)");
+  g_first_layer = v;
   return MT_OK;
 }
 int set_conv_walk(int v) {

@@ -109,6 +109,8 @@ int mt_timer_destroy(void *timer);
  *                    the shape allows / 0 never
  *   "conv_walk"      1 (default) forward convolutions whose taps tile the k step (4x4, 2x2, 1x1) use the same walking kernel
  *                    wherever the shape allows and gives at least 512 blocks / 2 wherever the shape allows / 0 never
+ *   "first_layer"    1 (default) forward convolutions of 3-channel images (3x3, 4x4, 5x5 kernels to 32 or 64 filters) keep the
+ *                    input patch in LDS and the weights in registers wherever the shape allows / 0 never
  *   "walk_blocks"    blocks wanted per launch of the walking kernel (default 1024)
  *   "walk_waves"     4 (default) or 5 wavefronts per SIMD for its plain variant
  *   "walk_tm"        1 (default) or 2 accumulators per wavefront

@@ -225,6 +225,39 @@ def test_forward_convolution_whose_blocks_walk_over_the_batch(gpu, oracle, case,
     close(got[2], got[0], 2e-6)
 
 
+@pytest.mark.parametrize("case", [
+    # W, H, Wd, KA, k, s, p
+    (3, 64, 64, 32, 5, 1, 2),      # configs[0]: 5x5, odd kernel: pairs along a row, the last column row by row, one tap alone
+    (2, 128, 128, 32, 3, 2, 1),    # the VAE encoder's first layer: 3x3 stride 2
+    (3, 64, 64, 64, 4, 2, 1),      # the discriminator's first layer: 4x4 stride 2 to 64 filters (two filter blocks)
+    (2, 64, 64, 32, 4, 2, 1),      # the same to 32 filters
+    (1, 30, 64, 32, 3, 1, 1),      # 3x3 stride 1, 30 rows: the last tile has two rows beyond the image
+    (5, 18, 128, 32, 3, 2, 1),     # 9 output rows with tiles of four; more tiles than one pass of some blocks... and
+    (40, 16, 64, 64, 4, 2, 1),     # 40 x 2 tiles of 4 x 32 pixels: blocks walk over the samples
+    (2, 64, 60, 32, 5, 1, 2),      # 60 output columns: not this kernel (the general one runs)
+])
+@pytest.mark.parametrize("func", [None, "leaky_relu"])
+def test_first_layer_from_an_input_patch(gpu, oracle, case, func):
+    """Forward convolution of a 3-channel image on the kernel that keeps the input patch in LDS and the weights in registers,
+    against the oracle and against the general kernel."""
+    import mi355tensor as mt
+    W, H, Wd, KA, k, s, p = case
+    image, kernel, bias = U(1, W, 3, H, Wd), U(2, 1, 1, KA, 3 * k * k) * 0.3, U(3, 1, KA, 1, 1)
+    args = (image, kernel, bias, k, k, 3, KA, s, s, p, p)
+    want = oracle.forward_convolution(*args)
+    if func:
+        want = oracle.apply_func(want, func)
+    got = {}
+    try:
+        for mode in (1, 0):
+            mt.set_option("first_layer", mode)
+            got[mode] = gpu.forward_convolution(*args, func=func)
+    finally:
+        mt.set_option("first_layer", 1)
+    close(got[1], want, 1e-5)
+    close(got[1], got[0], 2e-6)
+
+
 @pytest.mark.parametrize("case", CONV_CASES)
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_backward_convolution(gpu, oracle, path, case, with_bias):
