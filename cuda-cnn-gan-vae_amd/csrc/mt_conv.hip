@@ -28,6 +28,8 @@ using mt::cdiv;
 int g_conv_path = 0;  // 0 auto, 1 direct, 2 implicit GEMM wherever it applies
 int g_first_layer = 1; // forward convolutions of 3-channel images: 0 never on the kernel that keeps the input patch in LDS and the weights in registers, 1 wherever the shape allows
 int g_conv_walk = 1;   // forward convolutions whose taps tile the k step: 0 never on the kernel whose blocks walk over the batch, 1 wherever the shape allows and gives 512 blocks, 2 wherever the shape allows
+uint64_t g_wgrad_walk_launches = 0;
+int g_wgrad_walk = 1;    // 1: the batch-summed weight gradient runs as one k loop per block where its shape allows (wgrad_walk_kernel), 0: never
 int g_wgrad_groups = 0;  // 0 auto, else the number of batch groups of the batch-summed weight gradient (if it divides the batch)
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
@@ -1764,14 +1766,35 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     groups = g;
   }
   const uint32_t per = B / groups;
+  // rows of delta against a gather from the image with fixed offsets, one k loop per block (wgrad_walk_kernel), where the
+  // shape allows; it may cut the samples themselves into groups when the batch alone gives few blocks
+  mt::igemm::WgradWalkArgs wa{};
+  bool walks = false;
+  if (g_wgrad_walk && dk->x == ncol && dk->z * dk->y == ka) {
+    wa.delta = delta->p; wa.image = image->p;
+    wa.M = ka; wa.N = ncol; wa.C = (uint32_t)kz; wa.H = image->y; wa.W = image->x; wa.OH = delta->y; wa.OW = delta->x; wa.KY = (uint32_t)ky; wa.KX = (uint32_t)kx;
+    wa.sy = sy; wa.sx = sx; wa.py = py; wa.px = px; wa.groups = groups;
+    walks = mt::igemm::wgrad_walk_plan(wa, B, g_wgrad_groups == 0);
+  }
   float *partial = nullptr, *dbias_partial = nullptr;
   const uint32_t chunks = dbias_chunks(B, ka, DHW);
-  const size_t wgrad_floats = groups > 1 ? (size_t)groups * ka * ncol : 0;
+  const size_t wgrad_floats = walks ? (size_t)wa.groups * ka * ncol : groups > 1 ? (size_t)groups * ka * ncol : 0;
   if (groups > 1 && (dk->x != ncol || dk->z * dk->y != ka))
     return mt::fail(MT_E_ARGUMENT, "%s: the summed kernel gradient must be exactly [1,1,%u,%u]", name, ka, ncol);
   if (wgrad_floats + (chunks > 1 ? (size_t)ka * chunks : 0) > 0) {
     if ((rc = workspace(wgrad_floats + (size_t)ka * chunks, &partial))) return rc;
     dbias_partial = partial + wgrad_floats;
+  }
+  if (walks) {
+    wa.partial = partial;
+    {
+      mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, ncol, wa.steps * BK, wa.groups) : name);
+      if ((rc = mt::igemm::launch_wgrad_walk(name, wa))) return rc;
+    }
+    g_wgrad_walk_launches++;
+    mt_tensor pt{partial, wa.groups, 1, ka, ncol}, flat{dk->p, 1, 1, ka, ncol};
+    if ((rc = mt_add_sum_w(&flat, &flat, &pt, 1.f, 1.f))) return rc;
+    return dbias_batch_sum(name, db->p, dbias_partial, delta->p, B, ka, DHW, chunks);
   }
   SrcRowK<true> a{};
   a.p = delta->p; a.ld = DHW; a.R = ka; a.K = per * DHW; a.seg = DHW; a.seg_stride = (uint32_t)sample_delta;
@@ -1974,6 +1997,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "pack_cache_spare_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_pack_spare) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
   if (strcmp(name, "graph_written_ranges") == 0) { *value = (int64_t)g_graph_written.size(); return true; }
   if (strcmp(name, "graph_writes_anything") == 0) { *value = g_graph_writes_anything ? 1 : 0; return true; }
+  if (strcmp(name, "wgrad_walk_launches") == 0) { *value = (int64_t)g_wgrad_walk_launches; return true; }
   return false;
 }
 int set_image_mfma(int v) {
@@ -2036,6 +2060,12 @@ int set_igemm_tile(int v) {
   igemm::tile_override() = v;
   return MT_OK;
 }
+int set_wgrad_walk(int v) {
+  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "wgrad_walk must be 0 or 1");
+  g_wgrad_walk = v;
+  return MT_OK;
+}
+
 int set_wgrad_groups(int v) {
   if (v < 0) return fail(MT_E_ARGUMENT, "wgrad_groups must be 0 (auto) or a positive divisor of the batch");
   g_wgrad_groups = v;

@@ -179,12 +179,17 @@ __global__ __launch_bounds__(EW_THREADS) void summ_xy_kernel(float *out, const f
 }
 
 // ---- AddBias: working[w][z][.] += bias[w%Wb][z] ------------------------------------------------------------------
-// The same with 128-bit accesses: a block owns 32 groups of four columns and splits the batch over 8 slices that are
-// combined in LDS; the slice loop is unrolled so that several loads per thread are in flight.
+// The same with 128-bit accesses: a block owns RB groups of four columns and splits the batch over WS = 256 / RB slices;
+// the slice loops are unrolled so that several loads per thread are in flight.  Slices are combined inside a wavefront by
+// lane exchanges (the lanes that differ above the column bits), the four wavefronts in LDS.  RB = 256 is one thread per
+// group of columns, no exchange at all: tensors with few samples and many columns (two or eight partial weight gradients);
+// RB = 4 gives 64 slices: few columns and many samples (hundreds of partial gradients of a first layer).
+template <int RB>
 __global__ __launch_bounds__(EW_THREADS) void add_sum_w_vec_kernel(float *out, uint32_t Wout, const float *L, uint32_t Wl, const float *R, uint32_t Wr,
                                                                    uint32_t S, float ls, float rs) {
-  constexpr int RB = 32, WS = EW_THREADS / RB;
-  __shared__ float4 part[2][WS][RB];
+  constexpr int WS = EW_THREADS / RB, WAVES = EW_THREADS / 64;
+  constexpr int IN_WAVE = RB >= 64 ? 1 : 64 / RB;   // slices inside one wavefront
+  __shared__ float4 part[2][WS > 1 ? WAVES : 1][RB < 64 ? RB : 64];
   const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
   const uint32_t r = (blockIdx.x * RB + rl) * 4;
   float4 sl = make_float4(0.f, 0.f, 0.f, 0.f), sr = sl;
@@ -194,24 +199,36 @@ __global__ __launch_bounds__(EW_THREADS) void add_sum_w_vec_kernel(float *out, u
       const float4 q = *reinterpret_cast<const float4 *>(L + (size_t)w * S + r);
       sl.x += q.x; sl.y += q.y; sl.z += q.z; sl.w += q.w;
     }
-#pragma unroll 4
+#pragma unroll 8
     for (uint32_t w = ws; w < Wr; w += WS) {
       const float4 q = *reinterpret_cast<const float4 *>(R + (size_t)w * S + r);
       sr.x += q.x; sr.y += q.y; sr.z += q.z; sr.w += q.w;
     }
   }
-  part[0][ws][rl] = sl;
-  part[1][ws][rl] = sr;
-  __syncthreads();
-  if (r >= S) return;
-  if (ws == 0) {
-    sl = make_float4(0.f, 0.f, 0.f, 0.f); sr = sl;
+  if constexpr (WS > 1) {
 #pragma unroll
-    for (int i = 0; i < WS; i++) {
-      const float4 a = part[0][i][rl], b = part[1][i][rl];
-      sl.x += a.x; sl.y += a.y; sl.z += a.z; sl.w += a.w;
-      sr.x += b.x; sr.y += b.y; sr.z += b.z; sr.w += b.w;
+    for (int d = RB; d < RB * IN_WAVE; d <<= 1) {
+      sl.x += __shfl_xor(sl.x, d, 64); sl.y += __shfl_xor(sl.y, d, 64); sl.z += __shfl_xor(sl.z, d, 64); sl.w += __shfl_xor(sl.w, d, 64);
+      sr.x += __shfl_xor(sr.x, d, 64); sr.y += __shfl_xor(sr.y, d, 64); sr.z += __shfl_xor(sr.z, d, 64); sr.w += __shfl_xor(sr.w, d, 64);
     }
+    static_assert(RB <= 64, "several slices: a wavefront holds whole slices");
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    if (lane < RB) { part[0][wave][lane] = sl; part[1][wave][lane] = sr; }
+    __syncthreads();
+    if (r >= S) return;
+    if (ws == 0) {
+      sl = make_float4(0.f, 0.f, 0.f, 0.f); sr = sl;
+#pragma unroll
+      for (int i = 0; i < WAVES; i++) {
+        const float4 a = part[0][i][rl], b = part[1][i][rl];
+        sl.x += a.x; sl.y += a.y; sl.z += a.z; sl.w += a.w;
+        sr.x += b.x; sr.y += b.y; sr.z += b.z; sr.w += b.w;
+      }
+    }
+  } else {
+    if (r >= S) return;
+  }
+  if (ws == 0) {
     float4 o;
     o.x = sl.x * ls + sr.x * rs; o.y = sl.y * ls + sr.y * rs; o.z = sl.z * ls + sr.z * rs; o.w = sl.w * ls + sr.w * rs;
     *reinterpret_cast<float4 *>(out + r) = o;
@@ -1107,11 +1124,25 @@ int mt_add_sum_w(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, f
   if (!mt::same_zyx(l, r) || !mt::same_zyx(out, r)) return mt::fail(MT_E_SHAPE, "mt_add_sum_w: Z/Y/X of the operands differ");
   size_t S = (size_t)out->z * out->y * out->x;
   if (S == 0 || out->w == 0) return MT_OK;
-  mt::ProfileScope prof("mt_add_sum_w");
+  char shape[64];
+  if (mt::profiling()) snprintf(shape, sizeof shape, "S %zu W %u + %u", S, l->w, r->w);
+  mt::ProfileScope prof(mt::profiling() ? mt::intern_label("mt_add_sum_w", shape) : "mt_add_sum_w");
   // the output may alias an operand (dW = dW + sum_w TmpdW): every column is read completely before it is written
-  if (S % 4 == 0 && S >= 4096 && aligned16(out->p) && aligned16(l->p) && aligned16(r->p))
-    add_sum_w_vec_kernel<<<cdiv(S, 128), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
-  else if (S >= 65536)
+  if (S % 4 == 0 && S >= 1024 && aligned16(out->p) && aligned16(l->p) && aligned16(r->p)) {
+    // groups of four columns per block: as many as still give about a thousand blocks, but no more slices than samples
+    const size_t cols = S / 4;
+    const uint32_t W = l->w > r->w ? l->w : r->w;
+    int rb = cols / 256 >= 1024 ? 256 : cols / 32 >= 1024 ? 32 : cols / 8 >= 256 ? 8 : 4;
+    if (rb == 4 && W < 64) rb = 8;
+    if (rb == 8 && W < 32) rb = 32;
+    if (rb == 32 && W < 8 && cols / 256 >= 64) rb = 256;
+    hipStream_t st = mt::stream();
+    const uint32_t n = (uint32_t)S;
+    if (rb == 256) add_sum_w_vec_kernel<256><<<cdiv(cols, 256), EW_THREADS, 0, st>>>(out->p, out->w, l->p, l->w, r->p, r->w, n, ls, rs);
+    else if (rb == 32) add_sum_w_vec_kernel<32><<<cdiv(cols, 32), EW_THREADS, 0, st>>>(out->p, out->w, l->p, l->w, r->p, r->w, n, ls, rs);
+    else if (rb == 8) add_sum_w_vec_kernel<8><<<cdiv(cols, 8), EW_THREADS, 0, st>>>(out->p, out->w, l->p, l->w, r->p, r->w, n, ls, rs);
+    else add_sum_w_vec_kernel<4><<<cdiv(cols, 4), EW_THREADS, 0, st>>>(out->p, out->w, l->p, l->w, r->p, r->w, n, ls, rs);
+  } else if (S >= 65536)
     add_sum_w_kernel<256><<<cdiv(S, 256), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
   else
     add_sum_w_kernel<32><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);

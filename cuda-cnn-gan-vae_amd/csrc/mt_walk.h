@@ -367,6 +367,186 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   }
 }
 
+// ---- batch-summed weight gradient on the same pipeline ----------------------------------------------------------------
+//   dK[f][(c,i,j)] = sum over (w, oy, ox) of delta[w][f][oy][ox] * image[w][c][oy*sy + i - py][ox*sx + j - px]
+// as one product per group of k steps: rows = filters (operand A: rows of delta, 16 consecutive pixels per k step, one
+// 128-bit load per thread), columns = kernel coefficients (c, i, j) (operand B: a gather from the image whose per-thread
+// byte offsets never change: a k step is a block of 16 output pixels -- whole output rows, 16 / OW of them, or a 16-pixel
+// piece of one row -- so the pixels keep their place inside the block and a step moves a scalar offset), k = (sample,
+// output pixel).  A block owns one 64 x 64 tile of dK for its group -- whole samples, or an equal share of one sample's
+// steps -- and runs it as ONE k loop; the groups' tiles are added afterwards in group order.
+// Image borders: rows can only fall outside the image in the first row block of a sample (above it) and in the last one
+// (below it), so a thread keeps one mask for each and a step ORs in the one that applies -- two vector instructions per
+// step and one per load, against a bounds test per element in the general kernel.  Columns outside the image are out of
+// range for good when a step covers whole rows (folded into the offsets); when a row takes several steps (WIDE) they can
+// only occur in its first and last step, with a mask per element for each.
+struct WgradWalkArgs {
+  const float *delta;   // [B][M][OH][OW]
+  const float *image;   // [B][C][H][W]
+  float *partial;       // [groups][M][N]
+  uint32_t M, N, C, H, W, OH, OW, KY, KX;
+  int32_t sy, sx, py, px;
+  uint32_t steps, groups, tiles_m, tiles_n, fair;   // steps: k steps of a group (of B * OH * OW / 16 in all)
+};
+
+template <bool WIDE, int WAVES>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void wgrad_walk_kernel(WgradWalkArgs a) {
+  constexpr int BM = 64, BN = 64, E = 4;
+  __shared__ float4 smem4[2 * (BM + BN) * LDK / 4];
+  float *smem = reinterpret_cast<float *>(smem4);
+  float *As = smem, *Bs = smem + 2 * BM * LDK;
+
+  // an XCD runs a contiguous range of logical blocks: a few groups (their slices of delta and of the image) per range
+  uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
+  const uint32_t mt = j % a.tiles_m; j /= a.tiles_m;
+  const uint32_t nt = j % a.tiles_n, g = j / a.tiles_n;
+  const uint32_t m0 = mt * BM, n0 = nt * BN, DHW = a.OH * a.OW, HW = a.H * a.W;
+  // a sample is yblocks row blocks of xsteps k steps each
+  const uint32_t rows_per_step = WIDE ? 1u : BK / a.OW, xsteps = WIDE ? a.OW / BK : 1u, yblocks = a.OH / rows_per_step, nb = yblocks * xsteps;
+  const uint32_t first = g * a.steps, sample0 = first / nb, rem = first % nb;   // the group's first step: sample and step inside it
+  const uint32_t samples = (rem + a.steps + nb - 1) / nb;                        // samples the group touches (1 when it is a share of one)
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // ---- operand A: delta[w][m0 + row][16 pixels of the step], four pixels per thread
+  const uint32_t a_oct = (uint32_t)tid / 8u, a_row = (a_oct / 4u) * 8u + (a_oct % 4u) + 4u * (((uint32_t)tid % 8u) / 4u), a_k = ((uint32_t)tid % 4u) * E;
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.delta + (size_t)sample0 * a.M * DHW, samples * a.M * DHW * 4u);
+  const uint32_t a_voff = ((m0 + a_row) * DHW + a_k) * 4u;
+  // ---- operand B: column n = (c, i, j), pixels b_k .. b_k + 3 of the step's block
+  const uint32_t b_col = (uint32_t)tid % BN, b_k = (uint32_t)__builtin_amdgcn_readfirstlane((tid / BN) * E);
+  const uint32_t front = (uint32_t)a.py * a.W + (uint32_t)a.px;   // offsets are taken from (py rows + px pixels) in front of the image: none is negative
+  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(a.image + (size_t)sample0 * a.C * HW - front, (samples * a.C * HW + front) * 4u);
+  uint32_t b_voff[E], m_top, m_bottom, m_left[WIDE ? E : 1], m_right[WIDE ? E : 1];
+  {
+    const uint32_t n = n0 + b_col, taps = a.KY * a.KX, c = n / taps, t = n % taps, ki = t / a.KX, kj = t % a.KX;
+    const uint32_t dy = WIDE ? 0u : b_k / a.OW, dx0 = WIDE ? b_k : b_k % a.OW;   // the four pixels are neighbours in one output row (OW is a multiple of 4)
+    const int32_t iy_first = (int32_t)(dy * a.sy + ki) - a.py;                                  // input row in the first row block of a sample
+    const int32_t iy_last = (int32_t)((a.OH - rows_per_step + dy) * a.sy + ki) - a.py;          // ... and in the last one
+    m_top = iy_first < 0 ? OOB : 0u;
+    m_bottom = iy_last >= (int32_t)a.H ? OOB : 0u;
+#pragma unroll
+    for (int e = 0; e < E; e++) {
+      const int32_t ix = (int32_t)((dx0 + e) * a.sx + kj) - a.px;   // input column in the first step of a row
+      bool ok = n < a.N;
+      if constexpr (WIDE) {
+        m_left[e] = ix < 0 ? OOB : 0u;
+        m_right[e] = ix + (int32_t)((a.OW - BK) * a.sx) >= (int32_t)a.W ? OOB : 0u;
+      } else {
+        ok = ok && (uint32_t)ix < a.W;
+      }
+      b_voff[e] = ok ? ((c * a.H + dy * a.sy + ki) * a.W + (dx0 + e) * a.sx + kj) * 4u : OOB;
+    }
+  }
+  const uint32_t a_sample = (a.M * DHW - DHW) * 4u;
+  const uint32_t x_bytes = WIDE ? BK * (uint32_t)a.sx * 4u : 0u;                                  // a step along a row
+  const uint32_t y_bytes = rows_per_step * (uint32_t)a.sy * a.W * 4u, y_jump = y_bytes - xsteps * x_bytes;   // to the next row block
+  const uint32_t b_sample = (a.C * HW) * 4u - yblocks * y_bytes;
+  uint32_t yb = rem / xsteps, xb = rem % xsteps;   // the step's row block inside its sample, its place in the row
+  uint32_t a_soff = rem * BK * 4u, b_soff = yb * y_bytes + xb * x_bytes;
+  auto edges = [&]() { return (yb == 0 ? 1u : 0u) | (yb == yblocks - 1 ? 2u : 0u) | (xb == 0 ? 4u : 0u) | (xb == xsteps - 1 ? 8u : 0u); };
+  uint32_t edge = edges();
+  auto advance = [&]() {  // scalar unit only
+    a_soff += BK * 4u;
+    if constexpr (WIDE) { b_soff += x_bytes; xb++; }
+    if (!WIDE || xb == xsteps) {
+      xb = 0; yb++; b_soff += y_jump;
+      if (yb == yblocks) { yb = 0; a_soff += a_sample; b_soff += b_sample; }
+    }
+    edge = edges();
+  };
+  float ra[2][E], rb[2][E];
+  auto load_tile = [&](int set, bool adv) {
+    if (adv) advance();
+    const uint32_t top = edge & 1u ? ~0u : 0u, bottom = edge & 2u ? ~0u : 0u;   // (scalar selects)
+    const uint32_t mask = (m_top & top) | (m_bottom & bottom);
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      const floatx4 t = buf_load4(a_rsrc, a_voff, a_soff);
+      ra[set][0] = t.x; ra[set][1] = t.y; ra[set][2] = t.z; ra[set][3] = t.w;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (WIDE) {
+      const uint32_t left = edge & 4u ? ~0u : 0u, right = edge & 8u ? ~0u : 0u;
+#pragma unroll
+      for (int i = 0; i < E; i++) rb[set][i] = buf_load(b_rsrc, b_voff[i] | mask | (m_left[i] & left) | (m_right[i] & right), b_soff);
+    } else {
+#pragma unroll
+      for (int i = 0; i < E; i++) rb[set][i] = buf_load(b_rsrc, b_voff[i] | mask, b_soff);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  float *a_put = As + a_row * LDK + a_k, *b_put = Bs + b_col * LDK + b_k;
+  auto put_tile = [&](int set, int buf) {
+    lds_put<E>(a_put + buf * BM * LDK, ra[set]);
+    lds_put<E>(b_put + buf * BN * LDK, rb[set]);
+  };
+  const int lrow = lane & 31, lk = lane >> 5;
+  const float *a_get = As + (wm * 32 + lrow) * LDK + lk * 4;
+  const float *b_get = Bs + (wn * 32 + lrow) * LDK + lk * 4;
+  floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  float4 fa[2], fb[2];
+  auto read_half = [&](float4 &av, float4 &bv, int buf, int half) {
+    av = *reinterpret_cast<const float4 *>(a_get + buf * BM * LDK + half * 8);
+    bv = *reinterpret_cast<const float4 *>(b_get + buf * BN * LDK + half * 8);
+  };
+  auto multiply = [&](const float4 &av, const float4 &bv) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, acc, 0, 0, 0);
+  };
+  auto step = [&](auto parity, auto write_next, auto load_ahead) {   // (the pipeline of igemm_body)
+    constexpr int cur = decltype(parity)::value, nxt = cur ^ 1;
+    read_half(fa[1], fb[1], cur, 1);
+    if constexpr (decltype(write_next)::value) put_tile(nxt, nxt);
+    if constexpr (decltype(load_ahead)::value) load_tile(nxt, true);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(fa[0], fb[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    lds_barrier();
+    if constexpr (decltype(write_next)::value) read_half(fa[0], fb[0], nxt, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(fa[1], fb[1]);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
+  using Yes = std::true_type;
+  using No = std::false_type;
+  load_tile(0, false);
+  put_tile(0, 0);
+  load_tile(1, true);
+  load_tile(0, true);
+  lds_barrier();
+  read_half(fa[0], fb[0], 0, 0);
+  uint32_t left = a.steps;   // even and at least 4 (checked on the host)
+  uint32_t lower2 = 0, lower1 = 0, lower0 = 0;   // wavefront priorities that fall with the work left (see tconv_walk_kernel)
+  if (a.fair) { lower2 = (left * ((a.fair >> 8) & 15u) / 16u) & ~1u; lower1 = (left * ((a.fair >> 4) & 15u) / 16u) & ~1u; lower0 = (left * (a.fair & 15u) / 16u) & ~1u; }
+  if (a.fair) __builtin_amdgcn_s_setprio(3);
+  for (; left > 4; left -= 2) {
+    if (a.fair) {
+      if (left == lower2) __builtin_amdgcn_s_setprio(2);
+      else if (left == lower1) __builtin_amdgcn_s_setprio(1);
+      else if (left == lower0) __builtin_amdgcn_s_setprio(0);
+    }
+    step(Even{}, Yes{}, Yes{});
+    step(Odd{}, Yes{}, Yes{});
+  }
+  step(Even{}, Yes{}, Yes{});
+  step(Odd{}, Yes{}, No{});
+  step(Even{}, Yes{}, No{});
+  step(Odd{}, No{}, No{});
+  // the group's tile: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the wavefront's 32 x 32 quarter
+  const uint32_t n = n0 + (uint32_t)(wn * 32 + lrow), m_lane = m0 + (uint32_t)(wm * 32 + 4 * lk);
+  const __amdgpu_buffer_rsrc_t o_rsrc = make_rsrc(a.partial, a.groups * a.M * a.N * 4u);
+  const uint32_t dst = n < a.N ? ((g * a.M + m_lane) * a.N + n) * 4u : OOB, row_bytes = a.N * 4u;
+#pragma unroll
+  for (int r = 0; r < 16; r++) buf_store(o_rsrc, acc[r], dst, (8u * (r / 4) + (r & 3)) * row_bytes);
+}
+
 // Chan's update: (n, mean, m2) takes in another set of samples given the same way
 __device__ __forceinline__ void welford_merge(float &n, float &mean, float &m2, float on, float om, float o2) {
   if (on == 0.f) return;
@@ -482,6 +662,55 @@ inline int launch_tconv_walk(const char *name, const WalkArgs &a, bool norm, boo
   else if (stats) tconv_walk_kernel<0, true, 4, 1><<<grid, THREADS, 0, s>>>(a);
   else if (walk_waves() == 5) tconv_walk_kernel<0, false, 5, 1><<<grid, THREADS, 0, s>>>(a);
   else tconv_walk_kernel<0, false, 4, 1><<<grid, THREADS, 0, s>>>(a);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
+
+// Whether the batch-summed weight gradient can run as wgrad_walk_kernel, and with how many groups: `groups` comes in as
+// the caller's choice (a divisor of the batch) and may go up to an equal share of one sample's steps per group when the
+// batch alone gives too few blocks.  Fills steps, groups, tiles_m, tiles_n.
+inline bool wgrad_walk_plan(WgradWalkArgs &a, uint32_t batch, bool may_split_samples) {
+  if (a.groups == 0 || batch % a.groups != 0 || a.M % 64 != 0 || a.py < 0 || a.px < 0) return false;
+  const bool wide = a.OW > (uint32_t)BK;
+  if (wide ? a.OW % BK != 0 : (a.OW < 4 || BK % a.OW != 0 || a.OH % (BK / a.OW) != 0)) return false;   // a k step is whole output rows or a piece of one
+  const uint32_t rows = wide ? 1u : BK / a.OW, yblocks = a.OH / rows, xsteps = wide ? a.OW / BK : 1u, nb = yblocks * xsteps;
+  // rows above the image only in the first row block of a sample, rows below it only in the last one; columns left and
+  // right of it only in the first and last step of a row
+  for (uint32_t yb = 0; yb < yblocks; yb++)
+    for (uint32_t dy = 0; dy < rows; dy++)
+      for (uint32_t ki = 0; ki < a.KY; ki++) {
+        const int64_t iy = (int64_t)(yb * rows + dy) * a.sy + ki - a.py;
+        if (iy < 0 && yb != 0) return false;
+        if (iy >= (int64_t)a.H && yb != yblocks - 1) return false;
+      }
+  if (wide)
+    for (uint32_t xb = 0; xb < xsteps; xb++)
+      for (uint32_t dx = 0; dx < (uint32_t)BK; dx++)
+        for (uint32_t kj = 0; kj < a.KX; kj++) {
+          const int64_t ix = (int64_t)(xb * BK + dx) * a.sx + kj - a.px;
+          if (ix < 0 && xb != 0) return false;
+          if (ix >= (int64_t)a.W && xb != xsteps - 1) return false;
+        }
+  a.tiles_m = a.M / 64;
+  a.tiles_n = (a.N + 63) / 64;
+  uint32_t steps = batch / a.groups * nb;
+  if (may_split_samples && a.groups == batch)   // one sample per group and still few blocks: equal shares of a sample's steps
+    while (steps % 2 == 0 && steps / 2 >= 16 && (uint64_t)a.tiles_m * a.tiles_n * a.groups < 512) { steps /= 2; a.groups *= 2; }
+  if (a.groups < 2 || steps < 4 || steps % 2 != 0) return false;
+  a.steps = steps;
+  const uint64_t samples = (steps + nb - 1) / nb, front = (uint64_t)a.py * a.W + a.px;
+  if (samples * a.M * a.OH * a.OW * 4u >= 0x80000000ull || (samples * a.C * a.H * a.W + front + (uint64_t)a.KY * a.W) * 4u >= 0x80000000ull ||
+      (uint64_t)a.groups * a.M * a.N * 4u >= 0x80000000ull)
+    return false;
+  if (((uintptr_t)a.delta & 15u) != 0) return false;
+  a.fair = (uint32_t)walk_fair();
+  return (uint64_t)a.tiles_m * a.tiles_n * a.groups <= 0x7fffffffu;
+}
+
+inline int launch_wgrad_walk(const char *name, const WgradWalkArgs &a) {
+  const uint32_t grid = a.tiles_m * a.tiles_n * a.groups;
+  if (a.OW > (uint32_t)BK) wgrad_walk_kernel<true, 4><<<grid, THREADS, 0, stream()>>>(a);
+  else wgrad_walk_kernel<false, 4><<<grid, THREADS, 0, stream()>>>(a);
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }

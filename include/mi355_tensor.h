@@ -109,6 +109,9 @@ int mt_timer_destroy(void *timer);
  *                    the shape allows / 0 never
  *   "conv_walk"      1 (default) forward convolutions whose taps tile the k step (4x4, 2x2, 1x1) use the same walking kernel
  *                    wherever the shape allows and gives at least 512 blocks / 2 wherever the shape allows / 0 never
+ *   "wgrad_walk"     1 (default) mt_convolution_backward_weights_sum runs each group of samples as one k loop per block, with
+ *                    fixed gather offsets, where the shape allows (output rows of 4, 8 or 16 pixels, filters a multiple of 64) /
+ *                    0 never
  *   "first_layer"    1 (default) forward convolutions of 3-channel images (3x3, 4x4, 5x5 kernels to 32 or 64 filters) keep the
  *                    input patch in LDS and the weights in registers wherever the shape allows / 0 never
  *   "walk_blocks"    blocks wanted per launch of the walking kernel (default 1024)
@@ -133,7 +136,9 @@ int mt_set_option(const char *name, int value);
  *   "pack_cache_spare_bytes"                               buffers of evicted entries that a recorded graph still names
  *   "graph_written_ranges", "graph_writes_anything"        memory written by recorded calls: weights inside such a range
  *                                                          are re-ordered on every use; after 4096 ranges everything is
- *                                                          (graph_writes_anything = 1, for the rest of the process) */
+ *                                                          (graph_writes_anything = 1, for the rest of the process)
+ *   "wgrad_walk_launches"                                  calls of mt_convolution_backward_weights_sum that ran as one k loop
+ *                                                          per block (option "wgrad_walk") */
 int mt_get_info(const char *name, int64_t *value);
 
 /* ---- convolutions: CTensorConv<T> (cuda/ctensorconv.cu.h:63-66) ---- */

@@ -372,6 +372,49 @@ def test_convolution_backward_weights_sum(gpu, oracle, path, case):
 
 
 @pytest.mark.parametrize("case", [
+    # B, C, H, W, KA, k, s, p, groups
+    (16, 64, 32, 32, 128, 4, 2, 1, 0),   # output rows of 16 pixels: a k step is one row
+    (16, 32, 16, 16, 64, 4, 2, 1, 0),    # rows of 8 pixels: two rows per k step, four steps per sample
+    (32, 16, 8, 8, 64, 4, 2, 1, 4),      # 4 x 4 output pixels: a sample is one k step, both borders in every step
+    (8, 64, 16, 16, 64, 3, 1, 1, 0),     # 3 x 3, stride 1: 576 columns
+    (8, 7, 16, 16, 64, 3, 1, 1, 0),      # 63 columns: a partial column tile
+    (6, 8, 8, 16, 128, 4, 2, 1, 3),      # 4 x 8 output pixels, two samples per group
+    (4, 3, 64, 64, 64, 4, 2, 1, 0),      # rows of 32 pixels: two k steps per row, left and right border in different steps; a
+                                         # sample's steps are shared out over four groups
+    (2, 5, 32, 64, 64, 3, 1, 1, 0),      # rows of 64 pixels, 3 x 3, stride 1
+    (2, 8, 64, 32, 64, 4, 2, 1, 0),      # rows of 16 pixels, half a sample per group
+    (2, 3, 64, 64, 64, 5, 1, 2, 0),      # 5 x 5, padding 2: rows outside the image beyond the first k step -- the general kernel
+])
+def test_weights_sum_as_one_k_loop_per_block(gpu, oracle, case):
+    """The batch-summed weight gradient on the kernel whose blocks run a group of samples as one k loop with fixed gather
+    offsets (border rows masked per step), against the layer's own sequence on the oracle
+    (netlayer/cnetlayerconvolution.cu.h:501-508) and against the general kernel."""
+    B, C, H, Wd, KA, k, s, p, groups = case
+    oy, ox = (H - k + 2 * p) // s + 1, (Wd - k + 2 * p) // s + 1
+    image, delta = U(21, B, C, H, Wd), U(22, B, KA, oy, ox)
+    dk0, db0 = U(23, 1, 1, KA, C * k * k), U(24, 1, KA, 1, 1)
+    dkb, dbb = oracle.create_delta_weight_and_bias(np.zeros((B, 1, KA, C * k * k), np.float32), np.zeros((B, KA, 1, 1), np.float32),
+                                                   image, delta, k, k, C, KA, s, s, p, p)
+    want_k, want_b = oracle.add_sum_w(dk0, dkb, out_init=dk0), oracle.add_sum_w(db0, dbb, out_init=db0)
+    import mi355tensor as mt
+    got = {}
+    mt.set_option("wgrad_groups", groups)
+    try:
+        for walk in (1, 0):
+            mt.set_option("wgrad_walk", walk)
+            before = mt.get_info("wgrad_walk_launches")
+            got[walk] = gpu.convolution_backward_weights_sum(dk0, db0, image, delta, k, k, C, KA, s, s, p, p)
+            assert mt.get_info("wgrad_walk_launches") - before == (walk if p < 2 else 0)
+    finally:
+        mt.set_option("wgrad_groups", 0)
+        mt.set_option("wgrad_walk", 1)
+    for walk in (1, 0):
+        close(got[walk][0], want_k)
+        close(got[walk][1], want_b)
+    close(got[1][0], got[0][0], 2e-6)
+
+
+@pytest.mark.parametrize("case", [
     # B, C, H, W, KA
     (2, 16, 6, 8, 32),      # channels tile the k step
     (3, 5, 3, 4, 7),        # channel counts that do not
