@@ -333,6 +333,15 @@ __global__ __launch_bounds__(256) void dbias_finish_kernel(float *dbias, const f
   for (uint32_t c = 0; c < chunks; c++) s += partial[f * chunks + c];
   dbias[f] += s;
 }
+// The same with one wavefront per filter: many partial sums per filter (the groups of the walking weight-gradient kernel).
+__global__ __launch_bounds__(256) void dbias_finish_wave_kernel(float *dbias, const float *partial, uint32_t KA, uint32_t chunks) {
+  const uint32_t f = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x % 64;
+  if (f >= KA) return;
+  float s = 0.f;
+  for (uint32_t c = lane; c < chunks; c += 64) s += partial[f * chunks + c];
+  s = mt::wave_sum(s);
+  if (lane == 0) dbias[f] += s;
+}
 // chunks of the batch per filter: enough blocks to fill the device, each with at least a few thousand values
 uint32_t dbias_chunks(uint32_t B, uint32_t KA, uint32_t DHW) {
   uint32_t chunks = 1;
@@ -1781,12 +1790,14 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
   const size_t wgrad_floats = walks ? (size_t)wa.groups * ka * ncol : groups > 1 ? (size_t)groups * ka * ncol : 0;
   if (groups > 1 && (dk->x != ncol || dk->z * dk->y != ka))
     return mt::fail(MT_E_ARGUMENT, "%s: the summed kernel gradient must be exactly [1,1,%u,%u]", name, ka, ncol);
-  if (wgrad_floats + (chunks > 1 ? (size_t)ka * chunks : 0) > 0) {
-    if ((rc = workspace(wgrad_floats + (size_t)ka * chunks, &partial))) return rc;
+  const size_t dbias_floats = walks ? (size_t)ka * wa.groups : chunks > 1 ? (size_t)ka * chunks : 0;   // (the walking kernel sums delta as it passes)
+  if (wgrad_floats + dbias_floats > 0) {
+    if ((rc = workspace(wgrad_floats + dbias_floats, &partial))) return rc;
     dbias_partial = partial + wgrad_floats;
   }
   if (walks) {
     wa.partial = partial;
+    wa.bias_partial = dbias_partial;
     {
       mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, ncol, wa.steps * BK, wa.groups) : name);
       if ((rc = mt::igemm::launch_wgrad_walk(name, wa))) return rc;
@@ -1794,7 +1805,9 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     g_wgrad_walk_launches++;
     mt_tensor pt{partial, wa.groups, 1, ka, ncol}, flat{dk->p, 1, 1, ka, ncol};
     if ((rc = mt_add_sum_w(&flat, &flat, &pt, 1.f, 1.f))) return rc;
-    return dbias_batch_sum(name, db->p, dbias_partial, delta->p, B, ka, DHW, chunks);
+    dbias_finish_wave_kernel<<<cdiv(ka, 4), 256, 0, mt::stream()>>>(db->p, dbias_partial, ka, wa.groups);
+    MT_LAUNCH_CHECK(name);
+    return MT_OK;
   }
   SrcRowK<true> a{};
   a.p = delta->p; a.ld = DHW; a.R = ka; a.K = per * DHW; a.seg = DHW; a.seg_stride = (uint32_t)sample_delta;

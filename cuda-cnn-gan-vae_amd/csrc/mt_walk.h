@@ -384,6 +384,7 @@ struct WgradWalkArgs {
   const float *delta;   // [B][M][OH][OW]
   const float *image;   // [B][C][H][W]
   float *partial;       // [groups][M][N]
+  float *bias_partial;  // [M][groups]: the groups' sums of delta per filter (the bias gradient), or null
   uint32_t M, N, C, H, W, OH, OW, KY, KX;
   int32_t sy, sx, py, px;
   uint32_t steps, groups, tiles_m, tiles_n, fair;   // steps: k steps of a group (of B * OH * OW / 16 in all)
@@ -477,9 +478,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
     __builtin_amdgcn_sched_barrier(0);
   };
   float *a_put = As + a_row * LDK + a_k, *b_put = Bs + b_col * LDK + b_k;
+  // the bias gradient is the sum of delta over samples and pixels: the row sums of operand A, which the blocks of the
+  // first column tile add up as the tiles pass through their registers
+  const bool row_sums = a.bias_partial != nullptr && nt == 0;
+  float row_sum = 0.f;
   auto put_tile = [&](int set, int buf) {
     lds_put<E>(a_put + buf * BM * LDK, ra[set]);
     lds_put<E>(b_put + buf * BN * LDK, rb[set]);
+    if (row_sums) row_sum += (ra[set][0] + ra[set][1]) + (ra[set][2] + ra[set][3]);
   };
   const int lrow = lane & 31, lk = lane >> 5;
   const float *a_get = As + (wm * 32 + lrow) * LDK + lk * 4;
@@ -545,6 +551,11 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   const uint32_t dst = n < a.N ? ((g * a.M + m_lane) * a.N + n) * 4u : OOB, row_bytes = a.N * 4u;
 #pragma unroll
   for (int r = 0; r < 16; r++) buf_store(o_rsrc, acc[r], dst, (8u * (r / 4) + (r & 3)) * row_bytes);
+  if (row_sums) {  // four neighbouring lanes hold the four quarters of a row's k steps
+    row_sum += __shfl_xor(row_sum, 1, 64);
+    row_sum += __shfl_xor(row_sum, 2, 64);
+    if ((tid & 3) == 0) a.bias_partial[(size_t)(m0 + a_row) * a.groups + g] = row_sum;
+  }
 }
 
 // Chan's update: (n, mean, m2) takes in another set of samples given the same way
