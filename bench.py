@@ -4,10 +4,12 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
 A step is one forward pass of the generator over one batch of synthetic latents that are already resident in HBM
-(the fused C-ABI path: Linear, 4 x (BatchNorm + ReLU, transposed conv 4x4 s2 p1), tanh).  Order of the run: W warm-up +
-K timed steps from a cold start (reported), a sustained stretch of load (reported; the clocks settle), then the W
-warm-up + K timed steps that `value` comes from, the same steps with the latents uploaded from the host, and the K
-steps with per-kernel events.  Prints ONE JSON line:
+(the fused C-ABI path: Linear, 4 x (BatchNorm + ReLU, transposed conv 4x4 s2 p1), tanh).  Order of the run: the CPU
+baseline (before anything touches the GPU), W warm-up + K timed steps from a cold start (reported), a sustained
+stretch of load (reported; the clocks settle; at most 300 steps under a counter run of rocprofv3), then the W warm-up +
+K timed steps that `value` comes from, the same steps with the latents uploaded from the host, the K steps with
+per-kernel events, and the other configurations (c1, c2, c4, c5, gan: `secondary`, --no-secondary skips them).
+Prints ONE JSON line:
 value = images/s of the whole step; conv_gflops / conv_frac_of_fp32_mfma_peak = algorithmic FLOPs (2*MAC, non-zero
 taps only) of the four transposed convolutions over the time of their kernels; roofline = the dominant kernel
 (the matrix-core implicit GEMM of the three large transposed convolutions) measured with HIP events on the
@@ -427,6 +429,12 @@ def main():
     # Sustained load: long enough (about 1 s) for the clocks to settle, and for a GPU-busy sample from outside to
     # see the GPU working; its average is reported as ms_per_step_sustained.
     sustained_steps = args.sustained_steps if args.sustained_steps > 0 else max(2000, 4 * args.steps)
+    # A counter run of rocprofv3 (--pmc sets ROCPROF_COUNTER_COLLECTION for the program it starts) serialises and
+    # intercepts every dispatch; with tens of thousands of them its own tool library has ended in a segmentation fault.
+    # The counters of a kernel do not depend on the number of steps: a few hundred are enough there.
+    counters_on = os.environ.get("ROCPROF_COUNTER_COLLECTION", "").lower() not in ("", "0", "false")
+    if counters_on and sustained_steps > 300:
+        sustained_steps = 300
     s0, s1 = create(), create()
     record(s0, stream)
     for _ in range(sustained_steps):
