@@ -710,7 +710,10 @@ __global__ __launch_bounds__(256 * SPLIT) void tconv_k4s2_tile_kernel(TconvArgs 
   static_assert(SPLIT == 1 || sizeof(tiles) >= sizeof(float) * 256 * PP * 4 * CO, "the sums of the second half fit into the tile memory");
   const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W, M = args.M;
   const uint32_t tiles_x = (W + TW - 1) / TW;
-  const uint32_t x0 = (blockIdx.x % tiles_x) * TW, y0 = (blockIdx.x / tiles_x) * TH, g = blockIdx.y;
+  // (an XCD takes a contiguous range of (image, tile): neighbouring tiles read each other's edge lines from one L2)
+  const uint32_t logical = xcd_swizzle(blockIdx.y * gridDim.x + blockIdx.x, gridDim.x * gridDim.y);
+  const uint32_t tile_id = logical % gridDim.x, g = logical / gridDim.x;
+  const uint32_t x0 = (tile_id % tiles_x) * TW, y0 = (tile_id / tiles_x) * TH;
   const uint32_t half = SPLIT == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / 256) : 0u, tid = threadIdx.x % 256, tx = tid % 16, ty = tid / 16;
   auto &tile = tiles[half];
   Tile stage;
@@ -976,28 +979,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // every lane takes the two pieces of its output row, adds the bias term, applies the function and stores 16 bytes of a
 // whole output line.
 // Needs W == 32, H even and at most 32, C a multiple of 4 * DEPTH, exactly CO output channels, 8-byte aligned input.
-template <int CO, int NORM, int DEPTH>   // NORM: 0 plain input, 1 ReLU(scale * x + shift), 2 any of the cheap functions
+//
+// STRIP: images of W == 64.  A block owns a strip of R input rows of one image and has R + 2 wavefronts, one per input
+// row from the row above the strip to the row below it (the neighbours' pieces are computed again rather than fetched
+// from another block; rows outside the image load zeros and contribute zeros).  A wavefront's four pixel groups are the
+// two halves of its row (the second half is 128 bytes on, exactly where the next row is for W == 32, so the loads and
+// the products are the same instructions); along x the two halves exchange their edge pixels through a DPP rotation of
+// the 16 lanes; the first R wavefronts then finish two output rows each, 32 lanes per row.
+template <int CO, int NORM, int DEPTH, bool STRIP = false>   // NORM: 0 plain input, 1 ReLU(scale * x + shift), 2 any of the cheap functions
 __global__ __launch_bounds__(1024) void tconv_k4s2_products_kernel(TconvArgs args) {
-  extern __shared__ __attribute__((aligned(16))) float pieces[];  // [H][4][CO][64], then the coefficients [C/4][CO][64]
-  const uint32_t H = args.H, C = args.C, HW = H * 32u;
-  const uint32_t img = blockIdx.x;
+  extern __shared__ __attribute__((aligned(16))) float pieces[];  // [rows][4][CO][2 W], then the coefficients [C/4][CO][64]
+  constexpr uint32_t W = STRIP ? 64u : 32u, OW = 2u * W;
+  const uint32_t H = args.H, C = args.C, HW = H * W;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t R = STRIP ? blockDim.x / 64u - 2u : H;            // input rows whose output rows the block writes
+  const uint32_t strips = STRIP ? H / R : 1u;
+  const uint32_t block = STRIP ? xcd_swizzle(blockIdx.x, gridDim.x) : blockIdx.x;   // neighbouring strips share two input rows: one L2 for both
+  const uint32_t img = block / strips, y0 = (block % strips) * R;
   const uint32_t n = (uint32_t)lane & 15u, g = (uint32_t)lane >> 4;
   const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta, args.in_w * C * HW * 4u);
   __amdgpu_buffer_rsrc_t prsrc = rsrc;
   if (NORM) prsrc = make_rsrc(args.in_scale_shift, C * HW * 8u);
-  // value offsets: channel g of the k step, row 2*wave (the next row is 128 bytes on), pixels 2n, 2n+1
-  const uint32_t in_sample = ((g * H + 2u * (uint32_t)wave) * 32u + 2u * n) * 4u;
-  const uint32_t b_voff = (img % args.in_w) * C * HW * 4u + in_sample, b_step = 4u * HW * 4u;
+  // value offsets: channel g of the k step, the wavefront's (first) row, pixels 2n, 2n+1; the second pair is 128 bytes on
+  const int32_t row = STRIP ? (int32_t)y0 - 1 + wave : 2 * wave;
+  const bool row_in = !STRIP || (uint32_t)row < H;
+  const uint32_t in_sample = row_in ? ((g * H + (uint32_t)row) * W + 2u * n) * 4u : 0u;
+  const uint32_t b_voff = row_in ? (img % args.in_w) * C * HW * 4u + in_sample : OOB, b_step = 4u * HW * 4u;
   const uint32_t steps = C / 4u;
   const int in_func = args.in_func;
-  float *coeff = pieces + H * 4u * CO * 64u;
+  float *coeff = pieces + (STRIP ? R + 2u : H) * 4u * CO * OW;
 
   floatx2 rb[DEPTH][2];
   floatx4 rp[NORM ? DEPTH : 1][2];
   float rc[2][CO];
   auto fetch = [&](int slot, uint32_t s) {
-    const bool live = s < steps;   // uniform; loads beyond the last step are dropped by the range check
+    const bool live = s < steps && row_in;   // uniform; loads beyond the last step are dropped by the range check
     const uint32_t bo = live ? b_voff : OOB;
 #pragma unroll
     for (int yy = 0; yy < 2; yy++) rb[slot][yy] = buf_load2(rsrc, bo == OOB ? OOB : bo + (uint32_t)yy * 128u, s * b_step);
@@ -1067,10 +1083,47 @@ __global__ __launch_bounds__(1024) void tconv_k4s2_products_kernel(TconvArgs arg
       r.y = e[2] + o[3];               // column 4n + 1: x = 2n as 2x + 1, x = 2n + 1 as 2x - 1
       r.z = o[1] + e[0];               // column 4n + 2: x = 2n + 1 as 2x, x = 2n as 2x + 2
       r.w = o[2] + from_right(e[3]);   // column 4n + 3: x = 2n + 1 as 2x + 1, x = 2n + 2 as 2x - 1
-      *reinterpret_cast<floatx4 *>(&pieces[((((uint32_t)(2 * wave + yy)) * 4u + g) * CO + co) * 64u + 4u * n]) = r;
+      if constexpr (STRIP) {
+        // yy is the half of the row: pixel 31's neighbour to the right is pixel 32, lane 0 of the other half, and the other
+        // way round (a rotation of the 16 lanes; lanes without a source in the shift keep that value)
+        if (yy == 0) {
+          const float edge = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc[co][2][3]), 0x12f, 0xf, 0xf, false));   // row_ror:15: lane 15 <- lane 0
+          r.w = o[2] + __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(edge), __float_as_int(e[3]), 0x101, 0xf, 0xf, false));
+        } else {
+          const float edge = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc[co][1][0]), 0x121, 0xf, 0xf, false));   // row_ror:1: lane 0 <- lane 15
+          r.x = e[1] + __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(edge), __float_as_int(o[0]), 0x111, 0xf, 0xf, false));
+        }
+        *reinterpret_cast<floatx4 *>(&pieces[((((uint32_t)wave) * 4u + g) * CO + co) * OW + 64u * (uint32_t)yy + 4u * n]) = r;
+      } else {
+        *reinterpret_cast<floatx4 *>(&pieces[((((uint32_t)(2 * wave + yy)) * 4u + g) * CO + co) * 64u + 4u * n]) = r;
+      }
     }
 
   __syncthreads();
+  if constexpr (STRIP) {
+    // ---- along y: wavefront w finishes output rows 2m and 2m + 1 of input row m = y0 + w (local row w + 1), 32 lanes each
+    if ((uint32_t)wave >= R) return;
+    const uint32_t odd = (uint32_t)lane >> 5, q = (uint32_t)lane & 31u, m = y0 + (uint32_t)wave, local = (uint32_t)wave + 1u;
+    const uint32_t a_own = odd ? 2u : 1u, a_other = odd ? 3u : 0u, local_other = odd ? local + 1u : local - 1u;
+    const bool other = (uint32_t)((int32_t)m + (odd ? 1 : -1)) < H;   // (a row outside the image holds zeros: only the bias count differs)
+    const uint32_t OHW = 4u * HW, oy = 2u * m + odd;
+    const float bsum = args.ep.tap_bias ? args.ep.tap_bias[img % args.ep.bias_w] : 0.f;
+    const float ny = other ? 2.f : 1.f;
+    const float nx[4] = {q == 0 ? 1.f : 2.f, 2.f, 2.f, q == 31 ? 1.f : 2.f};
+    float o[CO][4];
+#pragma unroll
+    for (int co = 0; co < CO; co++) {
+      floatx4 r = *reinterpret_cast<const floatx4 *>(&pieces[((local * 4u + a_own) * CO + co) * OW + 4u * q]);
+      const floatx4 t = *reinterpret_cast<const floatx4 *>(&pieces[((local_other * 4u + a_other) * CO + co) * OW + 4u * q]);
+#pragma unroll
+      for (int i = 0; i < 4; i++) o[co][i] = (r[i] + t[i]) + bsum * (ny * nx[i]);
+    }
+    mt::apply_func_epilogue_many<4 * CO>(args.ep.func, &o[0][0]);
+#pragma unroll
+    for (int co = 0; co < CO; co++)
+      *reinterpret_cast<float4 *>(args.ep.C + ((size_t)img * CO + co) * OHW + (size_t)oy * OW + 4u * q) = make_float4(o[co][0], o[co][1], o[co][2], o[co][3]);
+    return;
+  }
 
   // ---- along y: output row 2m is input row m in category 1 plus row m - 1 in category 0; output row 2m + 1 is row m in
   // category 2 plus row m + 1 in category 3.  The lane takes row 4*wave + g, columns 4n .. 4n+3, every channel.
@@ -1113,7 +1166,12 @@ __global__ __launch_bounds__(256) void conv3x3_tile_kernel(float *out, const flo
   __shared__ __attribute__((aligned(16))) float tile[2][CC][ROWS][PITCH];
   const uint32_t H = g.H, W = g.W, C = g.C, HW = H * W;
   const uint32_t tiles_x = (W + TW - 1) / TW;
-  const uint32_t x0 = (blockIdx.x % tiles_x) * TW, y0 = (blockIdx.x / tiles_x) * TH, w = blockIdx.y;
+  // Neighbouring tiles read each other's edge columns and rows: an XCD (its own L2) takes a contiguous range of
+  // (image, tile) instead of every eighth block, so that those lines are fetched once (2.8 times the input was read
+  // from the fabric before, 5.9 TB/s of it: the kernel was bound by its own re-reads).
+  const uint32_t logical = mt::igemm::xcd_swizzle(blockIdx.y * gridDim.x + blockIdx.x, gridDim.x * gridDim.y);
+  const uint32_t tile_id = logical % gridDim.x, w = logical / gridDim.x;
+  const uint32_t x0 = (tile_id % tiles_x) * TW, y0 = (tile_id / tiles_x) * TH;
   const uint32_t tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
   Tile stage;
   stage.setup(image, g.in_w * C * HW * 4u, (w % g.in_w) * C * HW * 4u, H, W, x0, y0, tid);
@@ -1211,14 +1269,45 @@ int launch_tconv_products(const char *name, const TconvArgs &args) {
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }
+// Rows per strip of the same kernel for images of 64 columns: 8 (two blocks of ten wavefronts per compute unit), else 4
+int g_image_strip = 0;   // 0: choose; else rows per strip (measurements only; must divide the image height)
+uint32_t products_strip_rows(const TconvArgs &args) {
+  if (g_image_strip > 0 && args.H % (uint32_t)g_image_strip == 0) return (uint32_t)g_image_strip;
+  return args.H % 8 == 0 ? 8u : 4u;
+}
+template <int CO, int NORM>
+int launch_tconv_products_strip(const char *name, const TconvArgs &args) {
+  constexpr int DEPTH = NORM == 2 || (CO == 4 && NORM != 0) ? 2 : 4;
+  static bool prepared = false;
+  const uint32_t rows = products_strip_rows(args);
+  const size_t lds = ((size_t)(rows + 2u) * 4u * CO * 128u + (size_t)args.C / 4u * CO * 64u) * sizeof(float);
+  if (!prepared) {
+    MT_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&tconv_k4s2_products_kernel<CO, NORM, DEPTH, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               160 * 1024));
+    prepared = true;
+  }
+  tconv_k4s2_products_kernel<CO, NORM, DEPTH, true><<<args.out_w * (args.H / rows), (rows + 2u) * 64u, lds, mt::stream()>>>(args);
+  MT_LAUNCH_CHECK(name);
+  return MT_OK;
+}
 template <int CO>
 int launch_tconv_products_norm(const char *name, const TconvArgs &args) {
+  if (args.W == 64) {
+    if (!args.in_scale_shift) return launch_tconv_products_strip<CO, 0>(name, args);
+    return args.in_func == MT_F_RELU ? launch_tconv_products_strip<CO, 1>(name, args) : launch_tconv_products_strip<CO, 2>(name, args);
+  }
   if (!args.in_scale_shift) return launch_tconv_products<CO, 0>(name, args);
   return args.in_func == MT_F_RELU ? launch_tconv_products<CO, 1>(name, args) : launch_tconv_products<CO, 2>(name, args);
 }
 bool products_kernel_fits(const TconvArgs &args) {
+  if (args.C % 16 != 0 || args.M < 1 || args.M > 4) return false;
+  if (args.W == 64) {  // strips of rows, one wavefront per input row
+    const uint32_t rows = products_strip_rows(args);
+    return args.H % 4 == 0 && args.H >= 4 && (uint64_t)args.out_w * (args.H / rows) <= 0x7fffffffu &&
+           ((size_t)(rows + 2u) * 4u * 128u + args.C / 4u * 64u) * args.M * sizeof(float) <= 160u * 1024u;
+  }
   // (the pieces of the output rows and the coefficients share the 160 KB of LDS)
-  return args.W == 32 && args.H % 2 == 0 && args.H >= 2 && args.H <= 32 && args.C % 16 == 0 && args.M >= 1 && args.M <= 4 && args.out_w <= 0x7fffffffu &&
+  return args.W == 32 && args.H % 2 == 0 && args.H >= 2 && args.H <= 32 && args.out_w <= 0x7fffffffu &&
          ((size_t)args.H * 4u + args.C / 4u) * args.M * 64u * sizeof(float) <= 160u * 1024u;
 }
 int launch_tconv_tile(const char *name, TconvArgs &args) {
@@ -2012,6 +2101,11 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "graph_writes_anything") == 0) { *value = g_graph_writes_anything ? 1 : 0; return true; }
   if (strcmp(name, "wgrad_walk_launches") == 0) { *value = (int64_t)g_wgrad_walk_launches; return true; }
   return false;
+}
+int set_image_strip(int v) {
+  if (v < 0 || v > 14) return fail(MT_E_ARGUMENT, "image_strip must be 0 (choose) or 1..14 rows");
+  g_image_strip = v;
+  return MT_OK;
 }
 int set_image_mfma(int v) {
   if (v < 0 || v > 2) return fail(MT_E_ARGUMENT, "image_mfma must be 0, 1 or 2");

@@ -121,7 +121,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 4)))
   using Slot0 = std::integral_constant<int, 0>;
   using Slot1 = std::integral_constant<int, 1>;
 
-  uint32_t tile = __builtin_amdgcn_readfirstlane(blockIdx.x);
+  // neighbouring tiles share patch rows and columns: the blocks of an XCD (one L2) take neighbouring tiles of every round
+  uint32_t tile = __builtin_amdgcn_readfirstlane(xcd_swizzle(blockIdx.x, gridDim.x));
   if (tile >= a.tiles) return;
   request(tile, Slot0{});
   request(tile + gridDim.x, Slot1{});

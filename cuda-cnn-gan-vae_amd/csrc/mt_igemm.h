@@ -1197,7 +1197,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   using First = std::integral_constant<int, 0>;
   using Second = std::integral_constant<int, 1>;
 
-  uint32_t tile = __builtin_amdgcn_readfirstlane(blockIdx.x);
+  // neighbouring tiles share patch rows and columns: the blocks of an XCD (one L2) take neighbouring tiles of every round
+  uint32_t tile = __builtin_amdgcn_readfirstlane(xcd_swizzle(blockIdx.x, gridDim.x));
   if (tile >= tiles) return;
   request_patch(tile, First{});
   request_patch(tile, Second{});

@@ -1182,7 +1182,9 @@ def test_image_layer_on_the_4x4x1_matrix_instructions(gpu, oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(2, 16, 3, 8, 32), (3, 32, 3, 32, 32), (2, 64, 2, 16, 32), (1, 16, 4, 2, 32), (2, 48, 1, 6, 32), (5, 64, 3, 32, 32),
-                                   (2, 32, 4, 30, 32), (2, 16, 3, 7, 32), (2, 24, 3, 8, 32)],   # the last two: shapes it leaves to the vector-ALU kernel
+                                   (2, 32, 4, 30, 32), (2, 16, 3, 7, 32), (2, 24, 3, 8, 32),   # the last two: shapes it leaves to the vector-ALU kernel
+                                   # images of 64 columns: strips of 8 or 4 rows, one wavefront per input row, the halves of a row exchange edge pixels
+                                   (2, 32, 3, 64, 64), (2, 16, 3, 8, 64), (1, 16, 4, 12, 64), (3, 16, 1, 4, 64), (2, 48, 2, 16, 64), (2, 16, 3, 6, 64)],
                          ids=lambda s: "x".join(str(v) for v in s))
 def test_image_layer_as_products_per_input_pixel(gpu, oracle, shape):
     """The image layer as a product of the coefficients with the raw input pixels on the 16x16x4 matrix instruction,
@@ -1199,10 +1201,15 @@ def test_image_layer_as_products_per_input_pixel(gpu, oracle, shape):
     pairs = np.stack([U(5, 1, cin, H, W, lo=0.5, hi=1.5), U(6, 1, cin, H, W, lo=-0.5, hi=0.5)], -1)
     u = pairs[..., 0] * x + pairs[..., 1]
     tx, tk, tb, tp, out = CTensor.from_numpy(x), CTensor.from_numpy(kernel), CTensor.from_numpy(bias), CTensor.from_numpy(pairs.reshape(1, cin, H, 2 * W)), CTensor(*out_shape)
+    fits = cin % 16 == 0 and ((W == 32 and H % 2 == 0 and H <= 32) or (W == 64 and H % 4 == 0))
     try:
         mt.set_option("image_mfma", 2)
         mt.CTensorMath.Fill(out, 9.0)
+        mt.profile_enable(True)
         CTensorConv.BackwardConvolution(out, tx, tk, 4, 4, cout, cin, tb, 2, 2, 1, 1, func="tangence")
+        labels = list(mt.profile_report())
+        mt.profile_enable(False)
+        assert any("products per input pixel" in label for label in labels) == fits, labels
         close(out.numpy(), want, 1e-5)
         mt.CTensorMath.Fill(out, 9.0)
         CTensorConv.BackwardConvolution(out, CTensor.from_numpy(x[:1]), tk, 4, 4, cout, cin, tb, 2, 2, 1, 1)
