@@ -27,6 +27,7 @@ int set_walk_order(int v);
 int set_walk_fair(int v);
 int set_igemm_fair(int v);
 int set_first_layer(int v);   // forward convolutions of 3-channel images on the input-patch kernel: 0 never, 1 wherever the shape allows
+int set_nontemporal(int v);   // streaming kernels read and write past the caches: 0 never, 1 always, 2 tensors of 128 MiB and more
 int set_image_strip(int v);   // rows per strip of the image layer's product kernel on 64-column images (0: choose)
 int set_wgrad_walk(int v);    // batch-summed weight gradients as one k loop per block: 0 never, 1 wherever the shape allows
 int set_conv_walk(int v);     // forward convolutions on the kernel whose blocks walk over the batch: 0 never, 1 wherever the shape allows

@@ -13,6 +13,16 @@ namespace {
 using mt::cdiv;
 
 constexpr int EW_THREADS = 256;
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// Tensors that are streamed once and exceed what the caches hold (4 MiB of L2 per XCD, 256 MiB of Infinity Cache) are
+// read and written with non-temporal accesses: measured on 268 MB and 1 GB tensors, 2x2 up-sampling goes from 4.9 to
+// 6.7 TB/s, max pooling backward from 5.1 to 6.7, max pooling from 5.2 to 6.2, down-sampling from 4.9 to 5.7.  Tensors that
+// fit are left to the caches: the next kernel finds them there (max pooling of a 67 MB input: 6.6 TB/s, 5.6 when
+// it is read past the caches).  The plain elementwise kernels (one contiguous store per thread) measured no difference
+// and keep ordinary accesses.
+int g_nontemporal = 2;   // 0 never, 1 always, 2 by size (default)
+inline bool streamed(size_t bytes) { return g_nontemporal == 1 || (g_nontemporal == 2 && bytes >= ((size_t)128 << 20)); }
 
 struct Operand {
   const float *p;
@@ -324,6 +334,7 @@ __global__ __launch_bounds__(EW_THREADS) void upsampling4_kernel(float *out, con
 }
 // x2 in both directions, output exactly twice the input, even input width: a thread reads two input pixels (64 bits)
 // and writes their 2x4 output pixels as two 128-bit stores; the same index map, without divisions.
+template <bool NT>
 __global__ __launch_bounds__(EW_THREADS) void upsampling2x2_kernel(float *out, const float *in, Geo g, uint32_t planes) {
   const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ix2 = g.ix / 2, n2 = g.iy * ix2;
   if (i >= n2) return;
@@ -335,10 +346,15 @@ __global__ __launch_bounds__(EW_THREADS) void upsampling2x2_kernel(float *out, c
   for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
     const uint32_t ipl = same_w ? pl : (pl / g.Z % g.Win) * g.Z + pl % g.Z;
     const float2 v = reinterpret_cast<const float2 *>(in + (size_t)ipl * plane_in)[i];
-    const float4 q = make_float4(v.x, v.x, v.y, v.y);
+    const floatx4 q = {v.x, v.x, v.y, v.y};
     float *dst = out + (size_t)pl * plane_out + o0;
-    *reinterpret_cast<float4 *>(dst) = q;
-    *reinterpret_cast<float4 *>(dst + g.ox) = q;
+    if constexpr (NT) {  // an output beyond what the caches hold: written once, not kept
+      __builtin_nontemporal_store(q, reinterpret_cast<floatx4 *>(dst));
+      __builtin_nontemporal_store(q, reinterpret_cast<floatx4 *>(dst + g.ox));
+    } else {
+      *reinterpret_cast<floatx4 *>(dst) = q;
+      *reinterpret_cast<floatx4 *>(dst + g.ox) = q;
+    }
   }
 }
 __global__ __launch_bounds__(EW_THREADS) void max_pooling_backward4_kernel(float *out, const mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t px_, uint32_t py_, uint32_t planes) {
@@ -412,6 +428,7 @@ __global__ __launch_bounds__(EW_THREADS) void max_pooling_kernel(float *out, mt_
 
 // 2x2 windows over an input of exactly twice the output and a width that is a multiple of four: a thread reads
 // 2x4 input pixels (two 128-bit loads) and produces two outputs; same arithmetic and scan order as the kernels above.
+template <bool NT>
 __global__ __launch_bounds__(EW_THREADS) void downsampling2x2_kernel(float *out, const float *in, Geo g, uint32_t planes) {
   const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ox2 = g.ox / 2, n2 = g.oy * ox2;
   if (i >= n2) return;
@@ -421,13 +438,21 @@ __global__ __launch_bounds__(EW_THREADS) void downsampling2x2_kernel(float *out,
 #pragma unroll 4
   for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
     const float *p = in + (size_t)pl * plane_in + i0;
-    const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + g.ix);
+    floatx4 a, b;
+    if constexpr (NT) {  // an input beyond what the caches hold: read once, not kept
+      a = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(p));
+      b = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(p + g.ix));
+    } else {
+      a = *reinterpret_cast<const floatx4 *>(p);
+      b = *reinterpret_cast<const floatx4 *>(p + g.ix);
+    }
     float2 r;
     r.x = ((((0.f + a.x) + b.x) + a.y) + b.y) / 4.f;  // columns outer, rows inner
     r.y = ((((0.f + a.z) + b.z) + a.w) + b.w) / 4.f;
     reinterpret_cast<float2 *>(out + (size_t)pl * plane_out)[i] = r;
   }
 }
+template <bool NT>
 __global__ __launch_bounds__(EW_THREADS) void max_pooling2x2_kernel(float *out, mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t planes) {
   const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ox2 = g.ox / 2, n2 = g.oy * ox2;
   if (i >= n2) return;
@@ -438,7 +463,14 @@ __global__ __launch_bounds__(EW_THREADS) void max_pooling2x2_kernel(float *out, 
 #pragma unroll 4
   for (uint32_t pl = blockIdx.y; pl < planes; pl += gridDim.y) {
     const float *p = in + (size_t)pl * plane_in + i0;
-    const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + g.ix);
+    floatx4 a, b;
+    if constexpr (NT) {
+      a = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(p));
+      b = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(p + g.ix));
+    } else {
+      a = *reinterpret_cast<const floatx4 *>(p);
+      b = *reinterpret_cast<const floatx4 *>(p + g.ix);
+    }
     const float e[2][4] = {{a.x, a.y, b.x, b.y}, {a.z, a.w, b.z, b.w}};  // window scan order: rows, then columns
     float best[2];
     uint4 where;
@@ -462,6 +494,7 @@ __global__ __launch_bounds__(EW_THREADS) void max_pooling2x2_kernel(float *out, 
 // MaxPoolingBackward for 2x2 windows and an output of exactly twice the input: a thread owns two neighbouring windows
 // (one 128-bit load of their positions, one 64-bit load of their deltas) and writes their 2 x 4 output pixels as two
 // 128-bit stores; same rule as the gather kernel below.
+template <bool NT>
 __global__ __launch_bounds__(EW_THREADS) void max_pooling_backward2x2_kernel(float *out, const mt_spos *pos, uint32_t Wpos, const float *in, Geo g, uint32_t planes) {
   const uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x, ix2 = g.ix / 2, n2 = g.iy * ix2;
   if (i >= n2) return;
@@ -474,7 +507,7 @@ __global__ __launch_bounds__(EW_THREADS) void max_pooling_backward2x2_kernel(flo
     const uint32_t ppl = same_w ? pl : (pl / g.Z % Wpos) * g.Z + pl % g.Z;
     const uint4 s = reinterpret_cast<const uint4 *>(pos + (size_t)ppl * plane_in)[i];  // {X0, Y0, X1, Y1}
     const float2 d = reinterpret_cast<const float2 *>(in + (size_t)pl * plane_in)[i];
-    float4 r[2];
+    floatx4 r[2];
 #pragma unroll
     for (uint32_t dy = 0; dy < 2; dy++) {
       r[dy].x = (s.x == ox && s.y == oy + dy) ? d.x : 0.f;
@@ -483,8 +516,13 @@ __global__ __launch_bounds__(EW_THREADS) void max_pooling_backward2x2_kernel(flo
       r[dy].w = (s.z == ox + 3 && s.w == oy + dy) ? d.y : 0.f;
     }
     float *dst = out + (size_t)pl * plane_out + o0;
-    *reinterpret_cast<float4 *>(dst) = r[0];
-    *reinterpret_cast<float4 *>(dst + g.ox) = r[1];
+    if constexpr (NT) {
+      __builtin_nontemporal_store(r[0], reinterpret_cast<floatx4 *>(dst));
+      __builtin_nontemporal_store(r[1], reinterpret_cast<floatx4 *>(dst + g.ox));
+    } else {
+      *reinterpret_cast<floatx4 *>(dst) = r[0];
+      *reinterpret_cast<floatx4 *>(dst + g.ox) = r[1];
+    }
   }
 }
 
@@ -656,13 +694,15 @@ __global__ __launch_bounds__(EW_THREADS) void bn_apply_kernel(float *out, float 
 // columns and splits the batch over 256/RB slices; a thread keeps its NW rows (128-bit each) in registers between
 // the statistics and the normalisation, so the input is read once.  Same sums, in the same order per thread, as
 // bn_stats_kernel<4>; only the cheap functions are applied here (see mt::epilogue_func).
-template <int RB, int NW>
-__global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float *xhat, const float *x, uint32_t W, uint32_t S, float inv_n, float eps,
-                                                              float *mean, float *var, float *ivar, float *new_mean, float *new_var, float mom_old,
-                                                              float mom_new, const float *gamma, const float *beta, int func, const float *old_mean,
-                                                              const float *old_var) {
-  constexpr int WS = EW_THREADS / RB;
-  __shared__ __attribute__((aligned(16))) float part[2][WS][RB * 4];
+// T = 1024 threads for batches of more than 512: 64 or 128 slices, so that a thread's share is still 16 rows at most; the
+// slices that sit in one wavefront are added by lane exchanges first, one partial per wavefront goes through LDS.
+template <int RB, int NW, int T = EW_THREADS, bool NT = false>
+__global__ __launch_bounds__(T) void bn_fused_kernel(float *out, float *xhat, const float *x, uint32_t W, uint32_t S, float inv_n, float eps,
+                                                     float *mean, float *var, float *ivar, float *new_mean, float *new_var, float mom_old,
+                                                     float mom_new, const float *gamma, const float *beta, int func, const float *old_mean,
+                                                     const float *old_var) {
+  constexpr int WS = T / RB, PARTS = T > EW_THREADS ? T / 64 : WS;
+  __shared__ __attribute__((aligned(16))) float part[2][PARTS][RB * 4];
   __shared__ __attribute__((aligned(16))) float col_mean[RB * 4], col_ivar[RB * 4];
   const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
   const uint32_t r = (blockIdx.x * RB + rl) * 4;
@@ -673,7 +713,12 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
 #pragma unroll
     for (int i = 0; i < NW; i++) {
       const uint32_t w = ws + i * WS;  // rows past the batch re-read its last row (a plain global load) and are not summed
-      q[i] = *reinterpret_cast<const float4 *>(x + (size_t)(w < W ? w : W - 1) * S + r);
+      if constexpr (NT) {
+        const floatx4 t = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(x + (size_t)(w < W ? w : W - 1) * S + r));
+        q[i] = make_float4(t.x, t.y, t.z, t.w);
+      } else {
+        q[i] = *reinterpret_cast<const float4 *>(x + (size_t)(w < W ? w : W - 1) * S + r);
+      }
     }
 #pragma unroll
     for (int i = 0; i < NW; i++) {
@@ -684,15 +729,28 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
       }
     }
   }
-  *reinterpret_cast<float4 *>(&part[0][ws][rl * 4]) = s1;
-  *reinterpret_cast<float4 *>(&part[1][ws][rl * 4]) = s2;
+  if constexpr (T > EW_THREADS) {
+    static_assert(RB < 64, "several slices per wavefront");
+#pragma unroll
+    for (int d = RB; d < 64; d <<= 1) {
+      s1.x += __shfl_xor(s1.x, d, 64); s1.y += __shfl_xor(s1.y, d, 64); s1.z += __shfl_xor(s1.z, d, 64); s1.w += __shfl_xor(s1.w, d, 64);
+      s2.x += __shfl_xor(s2.x, d, 64); s2.y += __shfl_xor(s2.y, d, 64); s2.z += __shfl_xor(s2.z, d, 64); s2.w += __shfl_xor(s2.w, d, 64);
+    }
+    if ((threadIdx.x & 63) < RB) {
+      *reinterpret_cast<float4 *>(&part[0][threadIdx.x / 64][rl * 4]) = s1;
+      *reinterpret_cast<float4 *>(&part[1][threadIdx.x / 64][rl * 4]) = s2;
+    }
+  } else {
+    *reinterpret_cast<float4 *>(&part[0][ws][rl * 4]) = s1;
+    *reinterpret_cast<float4 *>(&part[1][ws][rl * 4]) = s2;
+  }
   __syncthreads();
   const int c = threadIdx.x;
   const uint32_t rc = blockIdx.x * RB * 4 + c;
   if (c < RB * 4 && rc < S) {  // the first RB*4 threads finish one column each
     float a1 = 0.f, a2 = 0.f;
 #pragma unroll
-    for (int i = 0; i < WS; i++) { a1 += part[0][i][c]; a2 += part[1][i][c]; }
+    for (int i = 0; i < PARTS; i++) { a1 += part[0][i][c]; a2 += part[1][i][c]; }
     const float sh = x[rc];
     float md = a1 * inv_n;
     float mu = sh + md;
@@ -720,8 +778,13 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
       float4 h, o;
       h.x = (q[i].x - mu.x) * iv.x; h.y = (q[i].y - mu.y) * iv.y; h.z = (q[i].z - mu.z) * iv.z; h.w = (q[i].w - mu.w) * iv.w;
       o.x = f((g.x * h.x) + b.x); o.y = f((g.y * h.y) + b.y); o.z = f((g.z * h.z) + b.z); o.w = f((g.w * h.w) + b.w);
-      if constexpr (decltype(keep)::value) *reinterpret_cast<float4 *>(xhat + (size_t)w * S + r) = h;
-      *reinterpret_cast<float4 *>(out + (size_t)w * S + r) = o;
+      if constexpr (NT) {
+        if constexpr (decltype(keep)::value) __builtin_nontemporal_store(floatx4{h.x, h.y, h.z, h.w}, reinterpret_cast<floatx4 *>(xhat + (size_t)w * S + r));
+        __builtin_nontemporal_store(floatx4{o.x, o.y, o.z, o.w}, reinterpret_cast<floatx4 *>(out + (size_t)w * S + r));
+      } else {
+        if constexpr (decltype(keep)::value) *reinterpret_cast<float4 *>(xhat + (size_t)w * S + r) = h;
+        *reinterpret_cast<float4 *>(out + (size_t)w * S + r) = o;
+      }
     }
   };
   auto with_func = [&](auto keep) {
@@ -739,12 +802,12 @@ __global__ __launch_bounds__(EW_THREADS) void bn_fused_kernel(float *out, float 
 // sums and the error; NW == 0: any batch size, the rows are read a second time.
 // func (ReLU or leaky ReLU, else MT_F_NONE): the layer's output went through that function and `delta` is the
 // gradient behind it; the function layer's step delta * f'(gamma*xhat + beta) happens as delta is loaded.
-template <int RB, int NW>
-__global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, float *dgamma, float *dbeta, const float *delta, const float *gamma,
-                                                                 const float *beta, const float *xhat, const float *ivar, uint32_t W, uint32_t S, float n,
-                                                                 float inv_n, int func, float *keep_dxhat, float *keep_s1, float *keep_s2) {
-  constexpr int WS = EW_THREADS / RB, HOLD = NW > 0 ? NW : 1;
-  __shared__ float part[4][WS][RB * 4];
+template <int RB, int NW, int T = EW_THREADS>   // T = 1024: see bn_fused_kernel
+__global__ __launch_bounds__(T) void bn_backward_kernel(float *err, float *dgamma, float *dbeta, const float *delta, const float *gamma,
+                                                        const float *beta, const float *xhat, const float *ivar, uint32_t W, uint32_t S, float n,
+                                                        float inv_n, int func, float *keep_dxhat, float *keep_s1, float *keep_s2) {
+  constexpr int WS = T / RB, HOLD = NW > 0 ? NW : 1, PARTS = T > EW_THREADS ? T / 64 : WS;
+  __shared__ float part[4][PARTS][RB * 4];
   __shared__ float col_s1[RB * 4], col_s2[RB * 4];
   const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
   const uint32_t r = (blockIdx.x * RB + rl) * 4;
@@ -798,17 +861,33 @@ __global__ __launch_bounds__(EW_THREADS) void bn_backward_kernel(float *err, flo
       }
     }
   }
+  if constexpr (T > EW_THREADS) {
+    static_assert(RB < 64, "several slices per wavefront");
 #pragma unroll
-  for (int q = 0; q < 4; q++)
+    for (int d = RB; d < 64; d <<= 1)
 #pragma unroll
-    for (int v = 0; v < 4; v++) part[q][ws][rl * 4 + v] = acc[q][v];
+      for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[q][v] += __shfl_xor(acc[q][v], d, 64);
+    if ((threadIdx.x & 63) < RB) {
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) part[q][threadIdx.x / 64][rl * 4 + v] = acc[q][v];
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) part[q][ws][rl * 4 + v] = acc[q][v];
+  }
   __syncthreads();
   const int c = threadIdx.x;
   const uint32_t rc = blockIdx.x * RB * 4 + c;
   if (c < RB * 4 && rc < S) {  // the first RB*4 threads finish one column each
     float t[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < WS; i++)
+    for (int i = 0; i < PARTS; i++)
 #pragma unroll
       for (int q = 0; q < 4; q++) t[q] += part[q][i][c];
     col_s1[c] = t[0];
@@ -1002,6 +1081,11 @@ __global__ __launch_bounds__(EW_THREADS) void bn_scale_shift_kernel(float2 *ss, 
 }  // namespace
 
 namespace mt {
+int set_nontemporal(int v) {
+  if (v < 0 || v > 2) return fail(MT_E_ARGUMENT, "nontemporal must be 0 (never), 1 (always) or 2 (tensors of 128 MiB and more)");
+  g_nontemporal = v;
+  return MT_OK;
+}
 int norm_apply(const mt_tensor *out, const mt_tensor *in, const float *scale_shift, int func) {
   const size_t S = (size_t)in->z * in->y * in->x;
   if (S == 0 || in->w == 0) return MT_OK;
@@ -1132,7 +1216,7 @@ int mt_add_sum_w(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, f
     // groups of four columns per block: as many as still give about a thousand blocks, but no more slices than samples
     const size_t cols = S / 4;
     const uint32_t W = l->w > r->w ? l->w : r->w;
-    int rb = cols / 256 >= 1024 ? 256 : cols / 32 >= 1024 ? 32 : cols / 8 >= 256 ? 8 : 4;
+    int rb = cols / 256 >= 1024 && W <= 4 ? 256 : cols / 32 >= 256 ? 32 : cols / 8 >= 256 ? 8 : 4;
     if (rb == 4 && W < 64) rb = 8;
     if (rb == 8 && W < 32) rb = 32;
     if (rb == 32 && W < 8 && cols / 256 >= 64) rb = 256;
@@ -1207,7 +1291,8 @@ int mt_upsampling(const mt_tensor *out, const mt_tensor *in, uint32_t ux, uint32
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
   if (ux == 2 && uy == 2 && out->x == 2 * in->x && out->y == 2 * in->y && in->x % 2 == 0 && in->x > 0 && aligned16(out->p) && ((uintptr_t)in->p & 7u) == 0) {
     const unsigned bx = cdiv(n / 8, EW_THREADS);
-    upsampling2x2_kernel<<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, planes);
+    if (streamed(mt::count(out) * sizeof(float))) upsampling2x2_kernel<true><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, planes);
+    else upsampling2x2_kernel<false><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, planes);
     MT_LAUNCH_CHECK("mt_upsampling");
     return MT_OK;
   }
@@ -1232,7 +1317,8 @@ int mt_downsampling(const mt_tensor *out, const mt_tensor *in, uint32_t dx, uint
   Geo g{in->w, in->z, in->y, in->x, out->y, out->x};
   if (dx == 2 && dy == 2 && in->x == 2 * out->x && in->y == 2 * out->y && out->x % 2 == 0 && aligned16(in->p) && ((uintptr_t)out->p & 7u) == 0) {
     const unsigned bx = cdiv(n / 2, EW_THREADS);
-    downsampling2x2_kernel<<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, planes);
+    if (streamed(mt::count(in) * sizeof(float))) downsampling2x2_kernel<true><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, planes);
+    else downsampling2x2_kernel<false><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, in->p, g, planes);
     MT_LAUNCH_CHECK("mt_downsampling");
     return MT_OK;
   }
@@ -1255,7 +1341,8 @@ int mt_max_pooling(const mt_tensor *out, const mt_pos_tensor *pos, const mt_tens
   if (px == 2 && py == 2 && in->x == 2 * out->x && in->y == 2 * out->y && out->x % 2 == 0 && aligned16(in->p) && ((uintptr_t)out->p & 7u) == 0 &&
       aligned16(pos->p)) {
     const unsigned bx = cdiv(n / 2, EW_THREADS);
-    max_pooling2x2_kernel<<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, planes);
+    if (streamed(mt::count(in) * sizeof(float))) max_pooling2x2_kernel<true><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, planes);
+    else max_pooling2x2_kernel<false><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, planes);
     MT_LAUNCH_CHECK("mt_max_pooling");
     return MT_OK;
   }
@@ -1277,7 +1364,8 @@ int mt_max_pooling_backward(const mt_tensor *out, const mt_pos_tensor *pos, cons
   if (px == 2 && py == 2 && out->x == 2 * in->x && out->y == 2 * in->y && in->x % 2 == 0 && in->x > 0 && aligned16(out->p) && aligned16(pos->p) &&
       ((uintptr_t)in->p & 7u) == 0) {
     const unsigned bx = cdiv(n / 8, EW_THREADS);
-    max_pooling_backward2x2_kernel<<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, planes);
+    if (streamed(mt::count(out) * sizeof(float))) max_pooling_backward2x2_kernel<true><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, planes);
+    else max_pooling_backward2x2_kernel<false><<<dim3(bx, plane_blocks(bx, planes)), EW_THREADS, 0, mt::stream()>>>(out->p, pos->p, pos->w, in->p, g, planes);
     MT_LAUNCH_CHECK("mt_max_pooling_backward");
     return MT_OK;
   }
@@ -1468,7 +1556,21 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
   if (vec && mt::epilogue_func(func)) {
     // one pass: the widest column block that still gives every compute unit a few blocks, if the batch share fits
     // (a small batch on a large tensor: 64 column groups, so that a thread still has 8 to 16 loads in flight)
-    const int rb = S / 256 >= 512 && cdiv(W, 4) <= 16 ? 64 : S / 128 >= 512 ? 32 : S / 64 >= 512 ? 16 : 8;
+    int rb = S / 256 >= 512 && cdiv(W, 4) <= 16 ? 64 : S / 128 >= 512 ? 32 : S / 64 >= 512 ? 16 : 8;
+    if (W > 512 && W <= 2048) {
+      // a large batch: blocks of 1024 threads, 64 slices of 16 column groups (128 of 8 beyond a batch of 1024)
+      mt::ProfileScope prof("bn_fused");
+      const int big_rb = W <= 1024 ? 16 : 8;
+      const unsigned grid = cdiv(S, (size_t)big_rb * 4);
+#define MT_BN_FUSED_BIG(RB, NT) \
+  bn_fused_kernel<RB, 16, 1024, NT><<<grid, 1024, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func, om, ov)
+      const bool past_caches = streamed(S * W * sizeof(float));   // (116 against 125 us for a 268 MB tensor)
+      if (big_rb == 16 && past_caches) MT_BN_FUSED_BIG(16, true); else if (big_rb == 16) MT_BN_FUSED_BIG(16, false);
+      else if (past_caches) MT_BN_FUSED_BIG(8, true); else MT_BN_FUSED_BIG(8, false);
+#undef MT_BN_FUSED_BIG
+      MT_LAUNCH_CHECK("bn_fused");
+      return MT_OK;
+    }
     const uint32_t nw = cdiv(W, EW_THREADS / rb);
     if (nw <= 32) {
       mt::ProfileScope prof("bn_fused");
@@ -1615,6 +1717,13 @@ static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, cons
     return mt_mul_value(error, error, inv_n);
   }
   mt::ProfileScope prof("bn_backward");
+  if (W > 512 && W <= 1024) {  // a large batch: 1024 threads, 128 slices of 8 column groups, 8 rows of both tensors per thread
+    bn_backward_kernel<8, 8, 1024><<<cdiv(S, (size_t)32), 1024, 0, mt::stream()>>>(error->p, pg, pb, delta->p, gamma->p, beta ? beta->p : nullptr, xhat->p, ivar->p, W,
+                                                                               (uint32_t)S, n, inv_n, func, keep_dxhat ? keep_dxhat->p : nullptr,
+                                                                               keep_s1 ? keep_s1->p : nullptr, keep_s2 ? keep_s2->p : nullptr);
+    MT_LAUNCH_CHECK("mt_batchnorm_backward");
+    return MT_OK;
+  }
   int rb = S / 128 >= 512 ? 32 : S / 64 >= 512 ? 16 : 8;
   while (rb > 8 && cdiv(W, EW_THREADS / rb) > 16) rb /= 2;
   const uint32_t nw = cdiv(W, EW_THREADS / rb);

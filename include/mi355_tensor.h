@@ -122,6 +122,9 @@ int mt_timer_destroy(void *timer);
  *   "image_mfma"     kernel of a generator's image layer (transposed convolution 4x4, stride 2, to at most 4 channels):
  *                    2 (default) products per input pixel on the 16x16x4 matrix instruction where the shape allows /
  *                    1 the 4x4x1 matrix instruction where the shape allows / 0 the vector ALUs
+ *   "image_strip"    rows per strip of the image layer's product kernel on images of 64 columns (0, default: 8 or 4)
+ *   "nontemporal"    2 (default) the re-sampling, pooling and large-batch batch-norm kernels read and write tensors of 128 MiB
+ *                    and more past the caches (each element is touched once) / 1 always / 0 never
  *   "pool"           1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no
  *                    wait) / 0 every mt_free waits for the stream and returns the block to the driver
  *   "pool_limit_mib" MiB the pool may hold in free blocks (default 4096) */

@@ -666,17 +666,24 @@ def test_resampling_and_pooling_bit_exact(gpu, oracle):
 
 
 @pytest.mark.parametrize("shape", [(3, 2, 8, 16), (2, 5, 64, 64), (1, 1, 2, 4), (2, 3, 6, 12)])
-def test_resampling_and_pooling_2x2_bit_exact(gpu, oracle, shape):
-    """Widths that are multiples of four and 2x2 windows: the kernels with 128-bit accesses, ties and all."""
+@pytest.mark.parametrize("past_caches", [0, 1])
+def test_resampling_and_pooling_2x2_bit_exact(gpu, oracle, shape, past_caches):
+    """Widths that are multiples of four and 2x2 windows: the kernels with 128-bit accesses, ties and all; with ordinary
+    accesses and with the non-temporal ones that tensors of 128 MiB and more get."""
+    import mi355tensor as mt
     a = U(5, *shape)
     ties = np.round(a * 2)
-    assert np.array_equal(gpu.upsampling(a, 2, 2), oracle.upsampling(a, 2, 2))
-    assert np.array_equal(gpu.downsampling(a, 2, 2), oracle.downsampling(a, 2, 2))
-    for t in (a, ties):
-        g, o = gpu.max_pooling(t, 2, 2), oracle.max_pooling(t, 2, 2)
-        assert np.array_equal(g[1], o[1]) and np.array_equal(g[0], o[0])
-        d = U(6, *o[0].shape)
-        assert np.array_equal(gpu.max_pooling_backward(d, o[1], 2, 2, a.shape), oracle.max_pooling_backward(d, o[1], 2, 2, a.shape))
+    mt.set_option("nontemporal", past_caches)
+    try:
+        assert np.array_equal(gpu.upsampling(a, 2, 2), oracle.upsampling(a, 2, 2))
+        assert np.array_equal(gpu.downsampling(a, 2, 2), oracle.downsampling(a, 2, 2))
+        for t in (a, ties):
+            g, o = gpu.max_pooling(t, 2, 2), oracle.max_pooling(t, 2, 2)
+            assert np.array_equal(g[1], o[1]) and np.array_equal(g[0], o[0])
+            d = U(6, *o[0].shape)
+            assert np.array_equal(gpu.max_pooling_backward(d, o[1], 2, 2, a.shape), oracle.max_pooling_backward(d, o[1], 2, 2, a.shape))
+    finally:
+        mt.set_option("nontemporal", 2)
 
 
 @pytest.mark.parametrize("shape", [(3, 2, 4, 8), (2, 5, 3, 7), (1, 1, 1, 1), (4, 16, 32, 32)])
@@ -882,7 +889,28 @@ def test_batchnorm_running_statistics_blended_from_other_tensors(gpu, shape):
     assert np.array_equal(old_m.numpy(), om) and np.array_equal(old_v.numpy(), ov) and np.array_equal(out_a.numpy(), out_b.numpy())
 
 
-@pytest.mark.parametrize("shape", [(16, 3, 6, 6), (5, 2, 3, 3), (40, 8, 16, 16), (130, 4, 8, 8), (300, 1, 4, 8), (7, 64, 32, 32)])
+@pytest.mark.parametrize("shape", [(600, 2, 4, 8), (1024, 1, 8, 8), (1500, 1, 4, 8), (2100, 1, 4, 4), (700, 1, 3, 3)])
+def test_batchnorm_forward_of_large_batches(gpu, oracle, shape):
+    """Batches of more than 512: blocks of 1024 threads keep a thread's share of the batch in registers up to 2048 samples
+    (64 or 128 slices, added by lane exchanges and through LDS); beyond that, and for layouts without 128-bit rows, the
+    two-pass kernels.  Every output of the layer against the oracle's op sequence."""
+    import mi355tensor as mt
+    one = (1,) + tuple(shape[1:])
+    x, gamma, beta, nm, nv = Nrm(1, *shape) * 1.5 + 0.3, U(2, *one) + 1.5, U(3, *one), U(4, *one), np.abs(U(5, *one))
+    want = seq.batchnorm_forward_train(oracle, x, gamma, beta, nm, nv, 0.9)
+    try:
+        for past_caches in (2, 1):   # by size (ordinary accesses here); non-temporal ones, as for tensors of 128 MiB and more
+            mt.set_option("nontemporal", past_caches)
+            fused = gpu.batchnorm_train(x, gamma, beta, 0.9, seq.BN_EPSILON, None, nm, nv)
+            for key in ("out", "xhat", "ivar", "mean", "var", "new_mean", "new_var"):
+                close(fused[key], want[key], 1e-5)
+            close(gpu.batchnorm_train(x, gamma, beta, func="leaky_relu")["out"], oracle.apply_func(want["out"], "leaky_relu"), 1e-5)
+    finally:
+        mt.set_option("nontemporal", 2)
+
+
+@pytest.mark.parametrize("shape", [(16, 3, 6, 6), (5, 2, 3, 3), (40, 8, 16, 16), (130, 4, 8, 8), (300, 1, 4, 8), (7, 64, 32, 32),
+                                   (600, 2, 4, 8), (1024, 1, 8, 8), (1100, 1, 4, 8)])   # the last three: 1024 threads per block; rows read twice
 def test_batchnorm_backward_fused(gpu, oracle, shape):
     """The one-kernel backward pass against the layer's sequence of tensor operations, gradients accumulating into
     non-zero tensors; shapes cover register-resident and re-read batches, vector and scalar layouts."""
