@@ -663,9 +663,10 @@ __global__ __launch_bounds__(EW_THREADS) void bn_stats_kernel(const float *x, ui
   if (new_var) new_var[rc] = (mom_old * old_var[rc]) + (mom_new * vr);
 }
 
-// Pass 2: out = func(gamma * ((x - mean) * ivar) + beta), optionally storing xhat.
+// Pass 2: out = func(gamma * ((x - mean) * ivar) + beta), optionally storing xhat and the value in front of the function.
 __global__ __launch_bounds__(EW_THREADS) void bn_apply_kernel(float *out, float *xhat, const float *x, const float *mean, const float *ivar,
-                                                              const float *gamma, const float *beta, uint32_t S, uint32_t W, bool vec, int func) {
+                                                              const float *gamma, const float *beta, uint32_t S, uint32_t W, bool vec, int func,
+                                                              float *pre = nullptr) {
   uint32_t i = blockIdx.x * EW_THREADS + threadIdx.x;
   if (vec) {
     if (i * 4 >= S) return;
@@ -674,9 +675,11 @@ __global__ __launch_bounds__(EW_THREADS) void bn_apply_kernel(float *out, float 
     for (uint32_t w = blockIdx.y; w < W; w += gridDim.y) {
       float4 v = reinterpret_cast<const float4 *>(x + (size_t)w * S)[i], h, o;
       h.x = (v.x - mu.x) * iv.x; h.y = (v.y - mu.y) * iv.y; h.z = (v.z - mu.z) * iv.z; h.w = (v.w - mu.w) * iv.w;
-      o.x = mt::apply_func(func, (g.x * h.x) + b.x); o.y = mt::apply_func(func, (g.y * h.y) + b.y);
-      o.z = mt::apply_func(func, (g.z * h.z) + b.z); o.w = mt::apply_func(func, (g.w * h.w) + b.w);
+      const float4 z = make_float4((g.x * h.x) + b.x, (g.y * h.y) + b.y, (g.z * h.z) + b.z, (g.w * h.w) + b.w);
+      o.x = mt::apply_func(func, z.x); o.y = mt::apply_func(func, z.y);
+      o.z = mt::apply_func(func, z.z); o.w = mt::apply_func(func, z.w);
       if (xhat) reinterpret_cast<float4 *>(xhat + (size_t)w * S)[i] = h;
+      if (pre) reinterpret_cast<float4 *>(pre + (size_t)w * S)[i] = z;
       reinterpret_cast<float4 *>(out + (size_t)w * S)[i] = o;
     }
   } else {
@@ -685,6 +688,7 @@ __global__ __launch_bounds__(EW_THREADS) void bn_apply_kernel(float *out, float 
     for (uint32_t w = blockIdx.y; w < W; w += gridDim.y) {
       float h = (x[(size_t)w * S + i] - mu) * iv;
       if (xhat) xhat[(size_t)w * S + i] = h;
+      if (pre) pre[(size_t)w * S + i] = (g * h) + b;
       out[(size_t)w * S + i] = mt::apply_func(func, (g * h) + b);
     }
   }
@@ -700,7 +704,7 @@ template <int RB, int NW, int T = EW_THREADS, bool NT = false>
 __global__ __launch_bounds__(T) void bn_fused_kernel(float *out, float *xhat, const float *x, uint32_t W, uint32_t S, float inv_n, float eps,
                                                      float *mean, float *var, float *ivar, float *new_mean, float *new_var, float mom_old,
                                                      float mom_new, const float *gamma, const float *beta, int func, const float *old_mean,
-                                                     const float *old_var) {
+                                                     const float *old_var, float *pre) {
   constexpr int WS = T / RB, PARTS = T > EW_THREADS ? T / 64 : WS;
   __shared__ __attribute__((aligned(16))) float part[2][PARTS][RB * 4];
   __shared__ __attribute__((aligned(16))) float col_mean[RB * 4], col_ivar[RB * 4];
@@ -777,7 +781,9 @@ __global__ __launch_bounds__(T) void bn_fused_kernel(float *out, float *xhat, co
       if (w >= W) break;
       float4 h, o;
       h.x = (q[i].x - mu.x) * iv.x; h.y = (q[i].y - mu.y) * iv.y; h.z = (q[i].z - mu.z) * iv.z; h.w = (q[i].w - mu.w) * iv.w;
-      o.x = f((g.x * h.x) + b.x); o.y = f((g.y * h.y) + b.y); o.z = f((g.z * h.z) + b.z); o.w = f((g.w * h.w) + b.w);
+      const float4 z = make_float4((g.x * h.x) + b.x, (g.y * h.y) + b.y, (g.z * h.z) + b.z, (g.w * h.w) + b.w);
+      o.x = f(z.x); o.y = f(z.y); o.z = f(z.z); o.w = f(z.w);
+      if (pre) *reinterpret_cast<float4 *>(pre + (size_t)w * S + r) = z;   // (the value in front of the function, for callers that keep both)
       if constexpr (NT) {
         if constexpr (decltype(keep)::value) __builtin_nontemporal_store(floatx4{h.x, h.y, h.z, h.w}, reinterpret_cast<floatx4 *>(xhat + (size_t)w * S + r));
         __builtin_nontemporal_store(floatx4{o.x, o.y, o.z, o.w}, reinterpret_cast<floatx4 *>(out + (size_t)w * S + r));
@@ -801,11 +807,12 @@ __global__ __launch_bounds__(T) void bn_fused_kernel(float *out, float *xhat, co
 // Block layout as bn_fused_kernel.  NW > 0: a thread keeps its NW rows of delta and xhat in registers between the
 // sums and the error; NW == 0: any batch size, the rows are read a second time.
 // func (ReLU or leaky ReLU, else MT_F_NONE): the layer's output went through that function and `delta` is the
-// gradient behind it; the function layer's step delta * f'(gamma*xhat + beta) happens as delta is loaded.
+// gradient behind it; the function layer's step delta * f'(gamma*xhat + beta) happens as delta is loaded (keep_front:
+// that product is stored too, where the function layer itself leaves it).
 template <int RB, int NW, int T = EW_THREADS>   // T = 1024: see bn_fused_kernel
 __global__ __launch_bounds__(T) void bn_backward_kernel(float *err, float *dgamma, float *dbeta, const float *delta, const float *gamma,
                                                         const float *beta, const float *xhat, const float *ivar, uint32_t W, uint32_t S, float n,
-                                                        float inv_n, int func, float *keep_dxhat, float *keep_s1, float *keep_s2) {
+                                                        float inv_n, int func, float *keep_dxhat, float *keep_s1, float *keep_s2, float *keep_front) {
   constexpr int WS = T / RB, HOLD = NW > 0 ? NW : 1, PARTS = T > EW_THREADS ? T / 64 : WS;
   __shared__ float part[4][PARTS][RB * 4];
   __shared__ float col_s1[RB * 4], col_s2[RB * 4];
@@ -919,6 +926,14 @@ __global__ __launch_bounds__(T) void bn_backward_kernel(float *err, float *dgamm
         *reinterpret_cast<float4 *>(keep_dxhat + (size_t)w * S + r) = times_gamma(qd[i]);
       }
     }
+    if (keep_front) {
+#pragma unroll
+      for (int i = 0; i < NW; i++) {
+        const uint32_t w = ws + i * WS;
+        if (w >= W) break;
+        *reinterpret_cast<float4 *>(keep_front + (size_t)w * S + r) = qd[i];
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NW; i++) {
       const uint32_t w = ws + i * WS;
@@ -930,6 +945,7 @@ __global__ __launch_bounds__(T) void bn_backward_kernel(float *err, float *dgamm
       const float4 x = *reinterpret_cast<const float4 *>(xhat + (size_t)w * S + r);
       const float4 d = behind(*reinterpret_cast<const float4 *>(delta + (size_t)w * S + r), x);
       if (keep_dxhat) *reinterpret_cast<float4 *>(keep_dxhat + (size_t)w * S + r) = times_gamma(d);
+      if (keep_front) *reinterpret_cast<float4 *>(keep_front + (size_t)w * S + r) = d;
       *reinterpret_cast<float4 *>(err + (size_t)w * S + r) = error(d, x);
     }
   }
@@ -1157,7 +1173,7 @@ unsigned stream_blocks(size_t n) {
 
 static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
                            const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func, const mt_tensor *keep_dxhat, const mt_tensor *keep_s1,
-                           const mt_tensor *keep_s2);
+                           const mt_tensor *keep_s2, const mt_tensor *keep_front = nullptr);
 
 extern "C" {
 
@@ -1519,7 +1535,10 @@ int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor
 static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
                             const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
                             const mt_tensor *new_variable, float momentum, float epsilon, int func, bool fixed_scratch,
-                            const mt_tensor *old_mean = nullptr, const mt_tensor *old_variable = nullptr) {
+                            const mt_tensor *old_mean = nullptr, const mt_tensor *old_variable = nullptr, const mt_tensor *pre = nullptr) {
+  if (pre && (mt::bad(pre) || !mt::same_zyx(pre, in) || pre->w != in->w || pre->p == out->p || (xhat && pre->p == xhat->p) || pre->p == in->p))
+    return mt::fail(MT_E_SHAPE, "mt_batchnorm_forward_train_from: the tensor for gamma*xhat+beta must have the input's sizes and be a tensor of its own");
+  mt::note_write(pre);
   if (!mt::valid_func(func, true)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_func: unknown function id %d", func);
   if ((old_mean && !new_mean) || (old_variable && !new_variable)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_forward_train_from: a statistic to blend from needs one to blend into");
   for (auto t : {old_mean, old_variable})
@@ -1552,7 +1571,9 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
   float mom_new = (float)(1.0 - (double)momentum);  // and 1.0-Momentum, rounded once
   float *nm = new_mean ? new_mean->p : nullptr, *nv = new_variable ? new_variable->p : nullptr;
   const float *om = old_mean ? old_mean->p : nm, *ov = old_variable ? old_variable->p : nv;
-  bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(pm) && aligned16(pi) && (!xhat || aligned16(xhat->p));
+  float *pp = pre ? pre->p : nullptr;
+  bool vec = (S % 4 == 0) && aligned16(out->p) && aligned16(in->p) && aligned16(gamma->p) && aligned16(beta->p) && aligned16(pm) && aligned16(pi) && (!xhat || aligned16(xhat->p)) &&
+             (!pp || aligned16(pp));
   if (vec && mt::epilogue_func(func)) {
     // one pass: the widest column block that still gives every compute unit a few blocks, if the batch share fits
     // (a small batch on a large tensor: 64 column groups, so that a thread still has 8 to 16 loads in flight)
@@ -1563,7 +1584,7 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
       const int big_rb = W <= 1024 ? 16 : 8;
       const unsigned grid = cdiv(S, (size_t)big_rb * 4);
 #define MT_BN_FUSED_BIG(RB, NT) \
-  bn_fused_kernel<RB, 16, 1024, NT><<<grid, 1024, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func, om, ov)
+  bn_fused_kernel<RB, 16, 1024, NT><<<grid, 1024, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func, om, ov, pp)
       const bool past_caches = streamed(S * W * sizeof(float));   // (116 against 125 us for a 268 MB tensor)
       if (big_rb == 16 && past_caches) MT_BN_FUSED_BIG(16, true); else if (big_rb == 16) MT_BN_FUSED_BIG(16, false);
       else if (past_caches) MT_BN_FUSED_BIG(8, true); else MT_BN_FUSED_BIG(8, false);
@@ -1576,7 +1597,7 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
       mt::ProfileScope prof("bn_fused");
       const unsigned grid = cdiv(S, (size_t)rb * 4);
 #define MT_BN_FUSED(RB, NW) \
-  bn_fused_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func, om, ov)
+  bn_fused_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func, om, ov, pp)
 #define MT_BN_FUSED_NW(RB) \
   do { if (nw <= 8) MT_BN_FUSED(RB, 8); else if (nw <= 16) MT_BN_FUSED(RB, 16); else MT_BN_FUSED(RB, 32); } while (0)
       if (rb == 64) { if (nw <= 8) MT_BN_FUSED(64, 8); else MT_BN_FUSED(64, 16); }
@@ -1598,7 +1619,7 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
   unsigned gx = cdiv(vec ? S / 4 : S, EW_THREADS);
   unsigned gy = W < 16 ? W : 16;  // a few batch slices per column block keeps the per-column loads in registers
   mt::ProfileScope prof("bn_apply");
-  bn_apply_kernel<<<dim3(gx, gy), EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, pm, pi, gamma->p, beta->p, (uint32_t)S, W, vec, func);
+  bn_apply_kernel<<<dim3(gx, gy), EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, pm, pi, gamma->p, beta->p, (uint32_t)S, W, vec, func, pp);
   MT_LAUNCH_CHECK("bn_apply");
   return MT_OK;
 }
@@ -1612,8 +1633,9 @@ int mt_batchnorm_forward_train_func(const mt_tensor *out, const mt_tensor *in, c
 int mt_batchnorm_forward_train_from(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
                                     const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var, const mt_tensor *new_mean,
                                     const mt_tensor *new_variable, const mt_tensor *old_mean, const mt_tensor *old_variable, float momentum, float epsilon,
-                                    int func) {
-  return bn_forward_train(out, in, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func, false, old_mean, old_variable);
+                                    int func, const mt_tensor *pre_function) {
+  return bn_forward_train(out, in, gamma, beta, xhat, ivar, batch_mean, batch_var, new_mean, new_variable, momentum, epsilon, func, false, old_mean, old_variable,
+                          pre_function);
 }
 
 int mt_batchnorm_forward_train_func_noalloc(const mt_tensor *out, const mt_tensor *in, const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat,
@@ -1663,17 +1685,26 @@ int mt_batchnorm_backward_keep(const mt_tensor *error, const mt_tensor *dgamma, 
   return bn_backward_any(error, dgamma, dbeta, delta, gamma, nullptr, xhat, ivar, MT_F_NONE, dxhat, sum_dxhat, sum_dxhat_xhat);
 }
 
+int mt_batchnorm_backward_func_keep(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
+                                    const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func, const mt_tensor *dxhat,
+                                    const mt_tensor *sum_dxhat, const mt_tensor *sum_dxhat_xhat, const mt_tensor *delta_front) {
+  return bn_backward_any(error, dgamma, dbeta, delta, gamma, beta, xhat, ivar, func, dxhat, sum_dxhat, sum_dxhat_xhat, delta_front);
+}
+
 }  // extern "C"
 
 static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta, const mt_tensor *gamma,
                            const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func, const mt_tensor *keep_dxhat, const mt_tensor *keep_s1,
-                           const mt_tensor *keep_s2) {
+                           const mt_tensor *keep_s2, const mt_tensor *keep_front) {
   if (!mt::valid_func(func, true) || (func != MT_F_NONE && (func & MT_F_DIFFERENTIAL))) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: unknown function id %d", func);
   if (func == MT_F_LINEAR) func = MT_F_NONE;  // derivative 1
   const mt_tensor *need[5] = {error, delta, gamma, xhat, ivar};
   for (auto t : need)
     if (mt::bad(t)) return mt::fail(MT_E_ARGUMENT, "mt_batchnorm_backward: null tensor");
-  for (auto t : {error, dgamma, dbeta, keep_dxhat, keep_s1, keep_s2}) mt::note_write(t);
+  for (auto t : {error, dgamma, dbeta, keep_dxhat, keep_s1, keep_s2, keep_front}) mt::note_write(t);
+  if (keep_front && (mt::bad(keep_front) || !mt::same_zyx(keep_front, delta) || keep_front->w != delta->w || keep_front->p == error->p ||
+                     (keep_dxhat && keep_front->p == keep_dxhat->p)))
+    return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward_func_keep: delta_front must have the sizes of delta and be neither the error nor dxhat");
   if (keep_dxhat && (mt::bad(keep_dxhat) || !mt::same_zyx(keep_dxhat, delta) || keep_dxhat->w != delta->w || keep_dxhat->p == delta->p || keep_dxhat->p == error->p))
     return mt::fail(MT_E_SHAPE, "mt_batchnorm_backward_keep: dxhat must be a tensor of its own with the sizes of delta");
   for (auto t : {keep_s1, keep_s2})
@@ -1692,7 +1723,7 @@ static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, cons
   float *pg = dgamma ? dgamma->p : nullptr, *pb = dbeta ? dbeta->p : nullptr;
   const bool cheap = func == MT_F_NONE || func == MT_F_RELU || func == MT_F_LEAKY_RELU;
   const bool vec = cheap && S % 4 == 0 && aligned16(error->p) && aligned16(delta->p) && aligned16(gamma->p) && aligned16(xhat->p) && aligned16(ivar->p) &&
-                   (func == MT_F_NONE || aligned16(beta->p)) && (!keep_dxhat || aligned16(keep_dxhat->p));
+                   (func == MT_F_NONE || aligned16(beta->p)) && (!keep_dxhat || aligned16(keep_dxhat->p)) && (!keep_front || aligned16(keep_front->p));
   if (!vec) {
     // any layout, any function: the layers' own sequences of tensor operations, on workspace tensors
     float *ws = nullptr;
@@ -1700,11 +1731,13 @@ static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, cons
     if (rc) return rc;
     mt_tensor s1{keep_s1 ? keep_s1->p : ws, 1, delta->z, delta->y, delta->x}, s2{keep_s2 ? keep_s2->p : ws + S, 1, delta->z, delta->y, delta->x};
     mt_tensor dx{keep_dxhat ? keep_dxhat->p : ws + 2 * S, W, delta->z, delta->y, delta->x}, t{ws + 2 * S + (size_t)W * S, W, delta->z, delta->y, delta->x};
-    mt_tensor front{ws + 2 * S + 2 * (size_t)W * S, W, delta->z, delta->y, delta->x};
+    mt_tensor front{keep_front ? keep_front->p : ws + 2 * S + 2 * (size_t)W * S, W, delta->z, delta->y, delta->x};
     if (func != MT_F_NONE) {  // the function layer: delta * f'(gamma*xhat + beta)
       if ((rc = mt_tensor_item_production(&t, gamma, xhat)) || (rc = mt_add(&t, &t, beta, 1.f, 1.f))) return rc;
       if ((rc = mt_apply_func(&t, &t, MT_F_DIFFERENTIAL + func)) || (rc = mt_tensor_item_production(&front, delta, &t))) return rc;
       delta = &front;
+    } else if (keep_front && keep_front->p != delta->p) {
+      if ((rc = mt_set(&front, delta, 1.f, 0.f))) return rc;
     }
     if ((rc = mt_fill(&s1, 0.f)) || (rc = mt_fill(&s2, 0.f))) return rc;
     if ((rc = mt_tensor_item_production(&dx, delta, gamma)) || (rc = mt_add_sum_w(&s1, &s1, &dx, 1.f, 1.f))) return rc;
@@ -1720,7 +1753,8 @@ static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, cons
   if (W > 512 && W <= 1024) {  // a large batch: 1024 threads, 128 slices of 8 column groups, 8 rows of both tensors per thread
     bn_backward_kernel<8, 8, 1024><<<cdiv(S, (size_t)32), 1024, 0, mt::stream()>>>(error->p, pg, pb, delta->p, gamma->p, beta ? beta->p : nullptr, xhat->p, ivar->p, W,
                                                                                (uint32_t)S, n, inv_n, func, keep_dxhat ? keep_dxhat->p : nullptr,
-                                                                               keep_s1 ? keep_s1->p : nullptr, keep_s2 ? keep_s2->p : nullptr);
+                                                                               keep_s1 ? keep_s1->p : nullptr, keep_s2 ? keep_s2->p : nullptr,
+                                                                               keep_front ? keep_front->p : nullptr);
     MT_LAUNCH_CHECK("mt_batchnorm_backward");
     return MT_OK;
   }
@@ -1731,7 +1765,7 @@ static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, cons
 #define MT_BN_BWD(RB, NW) \
   bn_backward_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(error->p, pg, pb, delta->p, gamma->p, beta ? beta->p : nullptr, xhat->p, ivar->p, W, \
                                                                     (uint32_t)S, n, inv_n, func, keep_dxhat ? keep_dxhat->p : nullptr, keep_s1 ? keep_s1->p : nullptr, \
-                                                                    keep_s2 ? keep_s2->p : nullptr)
+                                                                    keep_s2 ? keep_s2->p : nullptr, keep_front ? keep_front->p : nullptr)
 #define MT_BN_BWD_NW(RB) \
   do { if (nw <= 4) MT_BN_BWD(RB, 4); else if (nw <= 8) MT_BN_BWD(RB, 8); else if (nw <= 16) MT_BN_BWD(RB, 16); else MT_BN_BWD(RB, 0); } while (0)
   if (rb == 32) MT_BN_BWD_NW(32); else if (rb == 16) MT_BN_BWD_NW(16); else MT_BN_BWD_NW(8);

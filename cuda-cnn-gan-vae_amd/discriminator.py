@@ -114,7 +114,11 @@ class Discriminator:
         # Running statistics of the batch-norm layers.  The layer keeps Mean / Variable (saved, used in inference mode)
         # and NewMean / NewVariable (blended by every training-mode forward pass), and copies one pair to the other at
         # both ends of a training step (netlayer/cnetlayerbatchnormalization.cu.h:620-621, 650-651).  Here one tensor
-        # serves as both: the training-mode forward pass blends into it, the two copies are no-ops.
+        # serves as both: the training-mode forward pass blends into it, the two copies are no-ops.  Inside a complete
+        # step (reset, forward, backward, update) the two are the same.  They differ for a training-mode forward pass that
+        # is NOT followed by the update: the layer throws its blend away at the next reset (NewMean = Mean), this class
+        # keeps it.  step() always runs the whole sequence; a caller that only wants outputs in training mode and the
+        # reference's statistics afterwards saves self.stats before and restores them after.
         self.stats = {k: CTensor.from_numpy(host[k] if k in host else v) for k, v in make_statistics().items()}
         self.x, self.labels = CTensor(b, 3, IMAGE, IMAGE), CTensor(b, 1, 1, 1)
         self.c, self.bn, self.a, self.xhat, self.ivar = [], [], [], [], []

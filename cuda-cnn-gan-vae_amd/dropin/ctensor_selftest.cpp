@@ -354,11 +354,13 @@ static void DeferredGradientChecks(void)
 struct SBatchNormTensors
 {
  CTensor<type_t> X,H,XHat,TmpAH,TmpA,TmpB,TmpC,IVar,Gamma,Beta,Mean,Variable,NewMean,NewVariable,Delta,DXHat,Prev,DGamma,DBeta;
+ CTensor<type_t> Error,FunctionDelta,F;///<what a function layer behind the batch norm is handed, its own delta tensor, its output
  SBatchNormTensors(uint32_t w,uint32_t z,uint32_t y,uint32_t x)
   :X(w,z,y,x),H(w,z,y,x),XHat(w,z,y,x),TmpAH(w,z,y,x),TmpA(1,z,y,x),TmpB(1,z,y,x),TmpC(1,z,y,x),IVar(1,z,y,x),Gamma(1,z,y,x),Beta(1,z,y,x),Mean(1,z,y,x),
-   Variable(1,z,y,x),NewMean(1,z,y,x),NewVariable(1,z,y,x),Delta(w,z,y,x),DXHat(w,z,y,x),Prev(w,z,y,x),DGamma(1,z,y,x),DBeta(1,z,y,x)
+   Variable(1,z,y,x),NewMean(1,z,y,x),NewVariable(1,z,y,x),Delta(w,z,y,x),DXHat(w,z,y,x),Prev(w,z,y,x),DGamma(1,z,y,x),DBeta(1,z,y,x),Error(w,z,y,x),FunctionDelta(w,z,y,x),F(w,z,y,x)
  {
   FillPattern(X,1,2.0f);FillPattern(Gamma,2,0.5f);FillPattern(Beta,3,0.5f);FillPattern(NewMean,4,0.3f);FillPattern(NewVariable,5,0.3f);
+  FillPattern(Error,11,1.0f);
   FillPattern(Delta,6,1.0f);FillPattern(DGamma,7,0.2f);FillPattern(DBeta,8,0.2f);FillPattern(Mean,9,0.3f);FillPattern(Variable,10,0.3f);
   for(uint32_t n=0;n<z*y*x;n++) Gamma.SetElement(0,n/(y*x),(n/x)%y,n%x,Gamma.GetElement(0,n/(y*x),(n/x)%y,n%x)+1.5f);
   for(uint32_t n=0;n<z*y*x;n++) Variable.SetElement(0,n/(y*x),(n/x)%y,n%x,static_cast<type_t>(fabs(Variable.GetElement(0,n/(y*x),(n/x)%y,n%x))+0.2));
@@ -395,6 +397,24 @@ struct SBatchNormTensors
   CTensorMath<type_t>::TensorItemProduction(TmpAH,Gamma,XHat);
   CTensorMath<type_t>::Add(H,TmpAH,Beta);
  }
+ // a function layer behind the batch norm: its Forward (netlayer/cnetlayerfunction.cu.h:202-212)
+ void Function(bool leaky)
+ {
+  if (leaky==true) CTensorApplyFunc<type_t>::ApplyLeakyReLU(F,H);
+              else CTensorApplyFunc<type_t>::ApplyReLU(F,H);
+ }
+ // a function layer behind the batch norm: its SetOutputError (netlayer/cnetlayerfunction.cu.h:347-358), the batch-norm
+ // layer's (a copy of the tensor, :677-680), then the backward pass
+ void FunctionBackward(bool leaky,bool create_delta_weight,int read_at=-1)
+ {
+  if (leaky==true) CTensorApplyFunc<type_t>::ApplyDifferentialLeakyReLU(FunctionDelta,H);
+              else CTensorApplyFunc<type_t>::ApplyDifferentialReLU(FunctionDelta,H);
+  if (read_at==100) H.GetElement(0,0,0,0);
+  CTensorMath<type_t>::TensorItemProduction(FunctionDelta,Error,FunctionDelta);
+  if (read_at==101) FunctionDelta.GetElement(0,0,0,0);
+  Delta=FunctionDelta;
+  Backward(create_delta_weight,read_at);
+ }
  void Backward(bool create_delta_weight,int read_at=-1)
  {
   const type_t N=static_cast<type_t>(X.GetSizeW());
@@ -422,11 +442,11 @@ struct SBatchNormTensors
  // every tensor against the same tensor of a run without deferral; differences are measured against the largest value
  bool Agrees(const SBatchNormTensors &eager,double tolerance) const
  {
-  const CTensor<type_t> *mine[16]={&H,&XHat,&TmpAH,&TmpA,&TmpB,&TmpC,&IVar,&NewMean,&NewVariable,&DXHat,&Prev,&DGamma,&DBeta,&Gamma,&Beta,&X};
-  const CTensor<type_t> *theirs[16]={&eager.H,&eager.XHat,&eager.TmpAH,&eager.TmpA,&eager.TmpB,&eager.TmpC,&eager.IVar,&eager.NewMean,&eager.NewVariable,
-                                     &eager.DXHat,&eager.Prev,&eager.DGamma,&eager.DBeta,&eager.Gamma,&eager.Beta,&eager.X};
+  const CTensor<type_t> *mine[20]={&H,&XHat,&TmpAH,&TmpA,&TmpB,&TmpC,&IVar,&NewMean,&NewVariable,&DXHat,&Prev,&DGamma,&DBeta,&Gamma,&Beta,&X,&Error,&FunctionDelta,&Delta,&F};
+  const CTensor<type_t> *theirs[20]={&eager.H,&eager.XHat,&eager.TmpAH,&eager.TmpA,&eager.TmpB,&eager.TmpC,&eager.IVar,&eager.NewMean,&eager.NewVariable,
+                                     &eager.DXHat,&eager.Prev,&eager.DGamma,&eager.DBeta,&eager.Gamma,&eager.Beta,&eager.X,&eager.Error,&eager.FunctionDelta,&eager.Delta,&eager.F};
   bool ok=true;
-  for(int n=0;n<16;n++)
+  for(int n=0;n<20;n++)
   {
    double largest=0;
    const double diff=MaxDifference(*mine[n],*theirs[n],largest);
@@ -474,6 +494,70 @@ static void FusedSequenceChecks(void)
   }
   snprintf(name,sizeof(name),"a sequence interrupted by a reader, batch %u",d[0]);
   Report(name,all);
+  // a function layer behind the batch norm: its two calls and the backward pass as one kernel while the forward pass is
+  // on record; as two calls and one kernel after somebody has written gamma; as written when a reader comes between
+  mi355::FuseSequences()=false;
+  SBatchNormTensors ef(d[0],d[1],d[2],d[3]);
+  ef.ForwardTraining();ef.FunctionBackward(true,true);ef.ForwardTraining();ef.FunctionBackward(false,false);
+  mi355::FuseSequences()=true;
+  SBatchNormTensors ff(d[0],d[1],d[2],d[3]);
+  const size_t function=queue.FunctionBackwardFused,plain=queue.BackwardFused,calls=queue.LiteralCalls;
+  ff.ForwardTraining();ff.FunctionBackward(true,true);ff.ForwardTraining();ff.FunctionBackward(false,false);
+  ok=queue.FunctionBackwardFused==function+2 && queue.BackwardFused==plain && queue.LiteralCalls==calls;
+  ok=ff.Agrees(ef,2e-5) && ok;
+  mi355::FuseSequences()=false;
+  SBatchNormTensors eg(d[0],d[1],d[2],d[3]);
+  eg.ForwardTraining();CTensorMath<type_t>::Mul(eg.Gamma,eg.Gamma,static_cast<type_t>(1));eg.FunctionBackward(true,true);
+  mi355::FuseSequences()=true;
+  SBatchNormTensors fg(d[0],d[1],d[2],d[3]);
+  const size_t function2=queue.FunctionBackwardFused,plain2=queue.BackwardFused;
+  fg.ForwardTraining();CTensorMath<type_t>::Mul(fg.Gamma,fg.Gamma,static_cast<type_t>(1));fg.FunctionBackward(true,true);
+  ok=queue.FunctionBackwardFused==function2 && queue.BackwardFused==plain2+1 && ok;
+  ok=fg.Agrees(eg,2e-5) && ok;
+  for(int read_at=100;read_at<=101;read_at++)
+  {
+   mi355::FuseSequences()=false;
+   SBatchNormTensors a(d[0],d[1],d[2],d[3]);
+   a.ForwardTraining();a.FunctionBackward(true,true,read_at);
+   mi355::FuseSequences()=true;
+   SBatchNormTensors b(d[0],d[1],d[2],d[3]);
+   b.ForwardTraining();b.FunctionBackward(true,true,read_at);
+   ok=b.Agrees(a,2e-5) && ok;
+  }
+  for(int read_at=1;read_at<15;read_at+=4)
+  {
+   mi355::FuseSequences()=false;
+   SBatchNormTensors a(d[0],d[1],d[2],d[3]);
+   a.ForwardTraining();a.FunctionBackward(false,true,read_at);
+   mi355::FuseSequences()=true;
+   SBatchNormTensors b(d[0],d[1],d[2],d[3]);
+   b.ForwardTraining();b.FunctionBackward(false,true,read_at);
+   ok=b.Agrees(a,2e-5) && ok;
+  }
+  snprintf(name,sizeof(name),"function layer and batch-norm layer backward as one kernel, batch %u",d[0]);
+  Report(name,ok);
+  // the function layer's Forward behind the batch-norm layer's: one kernel leaves both outputs (training mode), or the
+  // function layer's with the batch-norm layer's own pending (inference mode); a whole training step through both layers
+  mi355::FuseSequences()=false;
+  SBatchNormTensors eh(d[0],d[1],d[2],d[3]);
+  eh.ForwardTraining();eh.Function(true);eh.FunctionBackward(true,true);eh.ForwardInference();eh.Function(false);eh.ForwardInference();eh.Function(false);
+  mi355::FuseSequences()=true;
+  SBatchNormTensors fh(d[0],d[1],d[2],d[3]);
+  const size_t forward2=queue.ForwardFused,inference2=queue.InferenceFused,function3=queue.FunctionBackwardFused,calls2=queue.LiteralCalls;
+  fh.ForwardTraining();fh.Function(true);fh.FunctionBackward(true,true);fh.ForwardInference();fh.Function(false);fh.ForwardInference();fh.Function(false);
+  queue.Flush();
+  ok=queue.ForwardFused==forward2+1 && queue.InferenceFused==inference2+2 && queue.FunctionBackwardFused==function3+1 && queue.LiteralCalls==calls2;
+  ok=fh.Agrees(eh,2e-5) && ok;
+  // ... and when a reader looks at the batch-norm layer's output between the two layers
+  mi355::FuseSequences()=false;
+  SBatchNormTensors ej(d[0],d[1],d[2],d[3]);
+  ej.ForwardTraining();ej.H.GetElement(0,0,0,0);ej.Function(false);ej.ForwardInference();ej.H.GetElement(0,0,0,0);ej.Function(true);
+  mi355::FuseSequences()=true;
+  SBatchNormTensors fj(d[0],d[1],d[2],d[3]);
+  fj.ForwardTraining();fj.H.GetElement(0,0,0,0);fj.Function(false);fj.ForwardInference();fj.H.GetElement(0,0,0,0);fj.Function(true);
+  ok=fj.Agrees(ej,2e-5) && ok;
+  snprintf(name,sizeof(name),"function layer forward behind the batch-norm layer's as one kernel, batch %u",d[0]);
+  Report(name,ok);
   // inference mode, twice (the scratch tensors of the first pass are overwritten unread by the second)
   mi355::FuseSequences()=false;
   SBatchNormTensors ei(d[0],d[1],d[2],d[3]);
@@ -482,6 +566,7 @@ static void FusedSequenceChecks(void)
   SBatchNormTensors fi(d[0],d[1],d[2],d[3]);
   const size_t inference=queue.InferenceFused,dropped=queue.PendingDropped;
   fi.ForwardInference();fi.ForwardInference();
+  queue.Flush();   // (a whole forward sequence waits for the function layer's call that may follow)
   ok=queue.InferenceFused==inference+2 && queue.PendingDropped>dropped;
   ok=fi.Agrees(ei,2e-5) && ok;
   snprintf(name,sizeof(name),"batch-norm inference sequence as one kernel, batch %u",d[0]);

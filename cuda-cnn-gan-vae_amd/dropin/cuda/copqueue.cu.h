@@ -3,10 +3,11 @@
 //
 // The reference's layers are written as long sequences of small tensor operations: the batch-norm layer's forward pass
 // in training mode is 13 calls (netlayer/cnetlayerbatchnormalization.cu.h:301-371), its backward pass 12 or 15
-// (:578-604), and every layer clears its gradients and runs Adam tensor by tensor
+// (:578-604), with the two calls of a function layer's SetOutputError in front of it when one follows the batch norm
+// (netlayer/cnetlayerfunction.cu.h:347-358), and every layer clears its gradients and runs Adam tensor by tensor
 // (netlayer/cnetlayerconvolution.cu.h:522-539).  The library has one kernel for each of these sequences
-// (mt_batchnorm_forward_train_from, mt_batchnorm_forward_infer_func, mt_batchnorm_backward_keep, mt_fill_many,
-// mt_adam_many).  So the elementwise calls of CTensorMath are not run at once: they are appended to a queue, and
+// (mt_batchnorm_forward_train_from, mt_batchnorm_forward_infer_func, mt_batchnorm_backward_keep,
+// mt_batchnorm_backward_func_keep, mt_fill_many, mt_adam_many).  So the elementwise calls of CTensorMath are not run at once: they are appended to a queue, and
 //   * while the queue is the beginning of one of the known sequences (same operations, same tensors in the same roles,
 //     same scalars), it waits;
 //   * when it is a whole sequence, the sequence's one kernel runs instead;
@@ -44,7 +45,7 @@ namespace mi355
   return(on);
  }
 
- enum {OP_FILL=0,OP_ADD_SUM_W,OP_ADD,OP_SUB,OP_POW2,OP_SQRT,OP_INV,OP_ITEM_PRODUCTION,OP_MUL_VALUE,OP_ADAM};
+ enum {OP_FILL=0,OP_ADD_SUM_W,OP_ADD,OP_SUB,OP_POW2,OP_SQRT,OP_INV,OP_ITEM_PRODUCTION,OP_MUL_VALUE,OP_ADAM,OP_DIFFERENTIAL,OP_FUNCTION};
 
  // one call of CTensorMath as it was made: T[0] is the output (Adam: the weights), the inputs follow
  struct SOp
@@ -56,6 +57,7 @@ namespace mi355
   uint8_t Writes;///<bit i: all of T[i] is written
   float A;
   float B;
+  int Func;///<OP_FUNCTION: the function applied; OP_DIFFERENTIAL: the function whose derivative is applied (MT_F_*)
   uint32_t BatchSize;
   double Speed,Beta1,Beta2,Epsilon,Iteration;
  };
@@ -63,7 +65,7 @@ namespace mi355
  inline SOp MakeOp(int kind,uint8_t count,uint8_t reads,uint8_t writes,float a=0,float b=0)
  {
   SOp op;
-  op.Kind=kind;op.Count=count;op.Reads=reads;op.Writes=writes;op.A=a;op.B=b;
+  op.Kind=kind;op.Count=count;op.Reads=reads;op.Writes=writes;op.A=a;op.B=b;op.Func=MT_F_NONE;
   op.BatchSize=0;op.Speed=0;op.Beta1=0;op.Beta2=0;op.Epsilon=0;op.Iteration=0;
   for(int n=0;n<4;n++) {op.T[n].p=NULL;op.T[n].w=0;op.T[n].z=0;op.T[n].y=0;op.T[n].x=0;}
   return(op);
@@ -78,6 +80,18 @@ namespace mi355
  {
   SOp op=MakeOp(kind,2,2,1,a,b);
   op.T[0]=o;op.T[1]=i;
+  return(op);
+ }
+ inline SOp MakeDifferential(const mt_tensor &o,const mt_tensor &i,int func)///<o = f'(i), CTensorApplyFunc::ApplyDifferential...
+ {
+  SOp op=MakeOp(OP_DIFFERENTIAL,2,2,1);
+  op.T[0]=o;op.T[1]=i;op.Func=func;
+  return(op);
+ }
+ inline SOp MakeFunction(const mt_tensor &o,const mt_tensor &i,int func)///<o = f(i), CTensorApplyFunc::Apply...
+ {
+  SOp op=MakeOp(OP_FUNCTION,2,2,1);
+  op.T[0]=o;op.T[1]=i;op.Func=func;
   return(op);
  }
  inline SOp MakeBinary(int kind,const mt_tensor &o,const mt_tensor &l,const mt_tensor &r,float a=0,float b=0)
@@ -110,6 +124,8 @@ namespace mi355
   const char *b=reinterpret_cast<const char*>(t.p);
   return(a<=b && b+Bytes(t)<=a+bytes);
  }
+ // the functions (and derivatives) that the batch-norm kernels apply themselves
+ inline bool FusedFunction(int func) {return(func==MT_F_RELU || func==MT_F_LEAKY_RELU || func==MT_F_LINEAR);}
  inline bool Near(float a,double b) {return(fabs(static_cast<double>(a)-b)<=1e-6*(fabs(b)>1?fabs(b):1));}
 
  // the call as the reference's layer wrote it
@@ -126,24 +142,34 @@ namespace mi355
    case OP_INV:Check(mt_inv(&op.T[0],&op.T[1]));break;
    case OP_ITEM_PRODUCTION:Check(mt_tensor_item_production(&op.T[0],&op.T[1],&op.T[2]));break;
    case OP_MUL_VALUE:Check(mt_mul_value(&op.T[0],&op.T[1],op.A));break;
+   case OP_FUNCTION:Check(mt_apply_func(&op.T[0],&op.T[1],op.Func));break;
+   case OP_DIFFERENTIAL:Check(mt_apply_func(&op.T[0],&op.T[1],MT_F_DIFFERENTIAL+op.Func));break;
    case OP_ADAM:Check(mt_adam(&op.T[0],&op.T[1],&op.T[2],&op.T[3],op.BatchSize,op.Speed,op.Beta1,op.Beta2,op.Epsilon,op.Iteration));break;
    default:throw("mi355::RunLiteral: unknown operation");
   }
  }
 
  // ---- the known sequences ---------------------------------------------------------------------------------------------
- // A matcher walks the queue from `first` and returns 0 (not this sequence), 1 (its beginning) or 2 (all of it).
+ // A matcher walks the queue from `first` and returns 0 (not this sequence), 1 (its beginning), 2 (all of it) or 3 (all
+ // of it, and the next call may still belong to it: the function layer's Forward behind a batch-norm layer's,
+ // netlayer/cnetlayerfunction.cu.h:202-212).
  struct SBatchNormForward///<netlayer/cnetlayerbatchnormalization.cu.h:301-371, training mode
  {
   mt_tensor Mean,X,NewMean,XHat,Var,Scratch,NewVar,SqrtVar,IVar,Gamma,Beta,H;
   mt_tensor OldMean,OldVar;///<what the running statistics are blended from: the same tensors, unless they shared their block with a copy
   float Momentum,Epsilon;
+  bool HasFunction;
+  int Func;
+  mt_tensor F;///<the function layer's output, when its call follows
   enum {LENGTH=13};
  };
  struct SBatchNormInference///<the same lines in inference mode (:326-371)
  {
   mt_tensor X,Mean,XHat,Var,SqrtVar,IVar,Scratch,Gamma,Beta,H;
   float Epsilon;
+  bool HasFunction;
+  int Func;
+  mt_tensor F;
   enum {LENGTH=6};
  };
  struct SBatchNormBackward///<:578-604
@@ -164,7 +190,8 @@ namespace mi355
  inline int MatchBatchNormForward(const std::vector<SOp> &q,size_t first,SBatchNormForward &m)
  {
   const size_t n=q.size()-first;
-  if (n>SBatchNormForward::LENGTH) return(0);
+  if (n>SBatchNormForward::LENGTH+1) return(0);
+  m.HasFunction=false;m.Func=MT_F_NONE;
   for(size_t i=0;i<n;i++)
   {
    const SOp &o=q[first+i];
@@ -196,11 +223,14 @@ namespace mi355
             m.Gamma=o.T[1];break;
     case 12:if (o.Kind!=OP_ADD || !Same(o.T[1],m.Scratch) || !OneSampleOf(o.T[2],m.X) || o.A!=1 || o.B!=1 || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
             m.Beta=o.T[2];m.H=o.T[0];break;
+    case 13:if (o.Kind!=OP_FUNCTION || FusedFunction(o.Func)==false || !Same(o.T[1],m.H) || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
+            m.F=o.T[0];m.Func=o.Func;m.HasFunction=true;break;
    }
   }
   if (n<SBatchNormForward::LENGTH) return(1);
-  const mt_tensor *all[12]={&m.Mean,&m.X,&m.NewMean,&m.XHat,&m.Var,&m.Scratch,&m.NewVar,&m.SqrtVar,&m.IVar,&m.Gamma,&m.Beta,&m.H};
-  if (Distinct(all,12)==false) return(0);
+  const mt_tensor *all[13]={&m.Mean,&m.X,&m.NewMean,&m.XHat,&m.Var,&m.Scratch,&m.NewVar,&m.SqrtVar,&m.IVar,&m.Gamma,&m.Beta,&m.H,&m.F};
+  if (Distinct(all,m.HasFunction==true?13:12)==false) return(0);
+  if (m.HasFunction==true && (Overlap(m.F,m.OldMean)==true || Overlap(m.F,m.OldVar)==true)) return(0);
   // a running statistic blended from another block (its tensor shared the old one with a copy) must not be one of the outputs
   for(int n=0;n<12;n++)
   {
@@ -208,13 +238,14 @@ namespace mi355
    if (Same(m.OldVar,m.NewVar)==false && Overlap(m.OldVar,*all[n])==true && all[n]!=&m.NewVar) return(0);
   }
   if ((Same(m.OldMean,m.NewMean)==false && Overlap(m.OldMean,m.NewMean)==true) || (Same(m.OldVar,m.NewVar)==false && Overlap(m.OldVar,m.NewVar)==true)) return(0);
-  return(2);
+  return(m.HasFunction==true?2:3);
  }
 
  inline int MatchBatchNormInference(const std::vector<SOp> &q,size_t first,SBatchNormInference &m)
  {
   const size_t n=q.size()-first;
-  if (n>SBatchNormInference::LENGTH) return(0);
+  if (n>SBatchNormInference::LENGTH+1) return(0);
+  m.HasFunction=false;m.Func=MT_F_NONE;
   for(size_t i=0;i<n;i++)
   {
    const SOp &o=q[first+i];
@@ -232,11 +263,14 @@ namespace mi355
            m.Scratch=o.T[0];m.Gamma=o.T[1];break;
     case 5:if (o.Kind!=OP_ADD || !Same(o.T[1],m.Scratch) || !OneSampleOf(o.T[2],m.X) || o.A!=1 || o.B!=1 || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
            m.Beta=o.T[2];m.H=o.T[0];break;
+    case 6:if (o.Kind!=OP_FUNCTION || FusedFunction(o.Func)==false || !Same(o.T[1],m.H) || o.T[0].w!=m.X.w || !SameSample(o.T[0],m.X)) return(0);
+           m.F=o.T[0];m.Func=o.Func;m.HasFunction=true;break;
    }
   }
   if (n<SBatchNormInference::LENGTH) return(1);
-  const mt_tensor *all[10]={&m.X,&m.Mean,&m.XHat,&m.Var,&m.SqrtVar,&m.IVar,&m.Scratch,&m.Gamma,&m.Beta,&m.H};
-  return(Distinct(all,10)==true?2:0);
+  const mt_tensor *all[11]={&m.X,&m.Mean,&m.XHat,&m.Var,&m.SqrtVar,&m.IVar,&m.Scratch,&m.Gamma,&m.Beta,&m.H,&m.F};
+  if (Distinct(all,m.HasFunction==true?11:10)==false) return(0);
+  return(m.HasFunction==true?2:3);
  }
 
  inline int MatchBatchNormBackward(const std::vector<SOp> &q,size_t first,SBatchNormBackward &m)
@@ -296,6 +330,39 @@ namespace mi355
   return(Distinct(all,m.Gradients==true?11:9)==true?2:0);
  }
 
+ // The two calls of CNetLayerFunction::SetOutputError (netlayer/cnetlayerfunction.cu.h:347-358) followed by the batch-norm
+ // layer's backward pass on the tensor they produce:  Front = f'(Output of the batch norm);  Front = Error * Front;  then
+ // the sequence above with Delta = Front (the batch-norm layer's copy of it shares its block).
+ struct SFunctionBackward
+ {
+  mt_tensor Front,Output,Error;
+  int Func;
+  SBatchNormBackward Norm;
+ };
+ inline int MatchFunctionBackward(const std::vector<SOp> &q,size_t first,SFunctionBackward &m)
+ {
+  const size_t n=q.size()-first;
+  if (n>17) return(0);
+  const SOp &d=q[first];
+  if (d.Kind!=OP_DIFFERENTIAL || FusedFunction(d.Func)==false || d.T[0].w==0 || d.T[0].w!=d.T[1].w || !SameSample(d.T[0],d.T[1]) || Overlap(d.T[0],d.T[1])) return(0);
+  m.Front=d.T[0];m.Output=d.T[1];m.Func=d.Func;
+  if (n==1) return(1);
+  const SOp &p=q[first+1];
+  if (p.Kind!=OP_ITEM_PRODUCTION || !Same(p.T[0],m.Front) || !Same(p.T[2],m.Front) || p.T[1].w!=m.Front.w || !SameSample(p.T[1],m.Front) || Overlap(p.T[1],m.Front) || Overlap(p.T[1],m.Output)) return(0);
+  m.Error=p.T[1];
+  if (n==2) return(1);
+  const int inner=MatchBatchNormBackward(q,first+2,m.Norm);
+  if (inner==0) return(0);
+  if (n>=5 && Same(m.Norm.Delta,m.Front)==false) return(0);///<(the third call of the inner sequence names its Delta)
+  if (inner==1) return(1);
+  const mt_tensor *mine[2]={&m.Error,&m.Output};
+  const mt_tensor *theirs[10]={&m.Norm.SumA,&m.Norm.SumB,&m.Norm.DXHat,&m.Norm.Gamma,&m.Norm.Scratch,&m.Norm.XHat,&m.Norm.Prev,&m.Norm.IVar,&m.Norm.DGamma,&m.Norm.DBeta};
+  for(int a=0;a<2;a++)
+   for(int b=0;b<(m.Norm.Gradients==true?10:8);b++)
+    if (Overlap(*mine[a],*theirs[b])==true) return(0);
+  return(2);
+ }
+
  // consecutive Fill calls with one value, or consecutive Adam calls with one set of hyper-parameters
  inline bool IsRun(const std::vector<SOp> &q,size_t count)
  {
@@ -317,10 +384,15 @@ namespace mi355
   private:
    std::vector<SOp> Queue;///<calls made and not yet run, in order
    std::vector<SOp> Pending;///<defining calls of scratch tensors that a sequence's kernel did not write, in order
+   // What a forward pass in training mode established: Output = Gamma * XHat + Beta, element by element, for as long as
+   // none of the four tensors is written.  The backward pass behind a function layer needs Beta, which its own calls
+   // never name, to take the function's derivative at Gamma * XHat + Beta instead of reading Output.
+   struct SNormFact {mt_tensor Output,Gamma,Beta,XHat;};
+   std::vector<SNormFact> Facts;
   public:
    // counters, for tests and measurements
-   size_t ForwardFused,InferenceFused,BackwardFused,FillRuns,AdamRuns,RunCalls,LiteralCalls,PendingRun,PendingDropped;
-   COpQueue(void):ForwardFused(0),InferenceFused(0),BackwardFused(0),FillRuns(0),AdamRuns(0),RunCalls(0),LiteralCalls(0),PendingRun(0),PendingDropped(0) {}
+   size_t ForwardFused,InferenceFused,BackwardFused,FunctionBackwardFused,FillRuns,AdamRuns,RunCalls,LiteralCalls,PendingRun,PendingDropped;
+   COpQueue(void):ForwardFused(0),InferenceFused(0),BackwardFused(0),FunctionBackwardFused(0),FillRuns(0),AdamRuns(0),RunCalls(0),LiteralCalls(0),PendingRun(0),PendingDropped(0) {}
 
    // a call of CTensorMath; operands are up to date on the device, the output is marked device-side by the caller
    void Submit(const SOp &op)
@@ -335,29 +407,11 @@ namespace mi355
     Queue.push_back(op);
     for(;;)
     {
-     // the queue may begin with a run that is still collecting; a known sequence may start anywhere behind it
-     for(size_t first=0;first<Queue.size();first++)
-     {
-      if (IsRun(Queue,first)==false) break;
-      SBatchNormForward f;
-      SBatchNormInference i;
-      SBatchNormBackward b;
-      const int mf=MatchBatchNormForward(Queue,first,f),mi=MatchBatchNormInference(Queue,first,i),mb=MatchBatchNormBackward(Queue,first,b);
-      if (mf==2 || mi==2 || mb==2)
-      {
-       std::vector<SOp> sequence(Queue.begin()+first,Queue.end());
-       Queue.resize(first);
-       RunQueue();
-       if (mf==2) RunForward(sequence,f);
-       else if (mi==2) RunInference(sequence,i);
-       else RunBackward(sequence,b);
-       return;
-      }
-      if (mf==1 || mi==1 || mb==1) return;
-     }
+     if (Scan(false)!=0) return;
      if (IsRun(Queue,Queue.size())==true) return;
      if (Queue.size()==1) {RunQueue();return;}
-     // the last call fits nothing the queue was waiting for: the calls before it run as written, it starts anew
+     // the last call fits nothing the queue was waiting for: the calls before it run (as the sequence they are, if they
+     // are a whole one; else as written), it starts anew
      const SOp last=Queue.back();
      Queue.pop_back();
      RunQueue();
@@ -384,13 +438,51 @@ namespace mi355
      if (touches==true) RunQueue();
     }
     if (Pending.empty()==false) SettleRange(p,bytes,read,write);
+    if (write==true && Facts.empty()==false)
+    {
+     mt_tensor range=Range(p,bytes);
+     Forget(&range,1);
+    }
    }
    bool Idle(void) const {return(Queue.empty() && Pending.empty());}
+   size_t ForwardPassesOnRecord(void) const {return(Facts.size());}
    size_t QueuedCalls(void) const {return(Queue.size());}
    size_t PendingCalls(void) const {return(Pending.size());}
   private:
+   // Looks for a known sequence in the queue, which may begin with a run that is still collecting.  Returns 2 when a
+   // whole sequence was found and has run (with everything in front of it), 1 when the queue is the beginning of one (or a
+   // whole one that the next call may extend) and waits, 0 when it is neither.  `final`: nothing more will be added --
+   // beginnings do not count, a whole sequence that could have been extended runs as it is.
+   int Scan(bool final)
+   {
+    for(size_t first=0;first<Queue.size();first++)
+    {
+     if (IsRun(Queue,first)==false) break;
+     SBatchNormForward f;
+     SBatchNormInference i;
+     SBatchNormBackward b;
+     SFunctionBackward fb;
+     const int mf=MatchBatchNormForward(Queue,first,f),mi=MatchBatchNormInference(Queue,first,i),mb=MatchBatchNormBackward(Queue,first,b);
+     const int mfb=MatchFunctionBackward(Queue,first,fb);
+     const bool forward=(mf==2 || (final==true && mf==3)),inference=(mi==2 || (final==true && mi==3));
+     if (forward==true || inference==true || mb==2 || mfb==2)
+     {
+      std::vector<SOp> sequence(Queue.begin()+first,Queue.end());
+      Queue.resize(first);
+      if (Queue.empty()==false) RunQueue();
+      if (forward==true) RunForward(sequence,f);
+      else if (inference==true) RunInference(sequence,i);
+      else if (mb==2) RunBackward(sequence,b);
+      else RunFunctionBackward(sequence,fb);
+      return(2);
+     }
+     if (final==false && (mf==1 || mi==1 || mb==1 || mfb==1 || mf==3 || mi==3)) return(1);
+    }
+    return(0);
+   }
    void RunQueue(void)
    {
+    if (Scan(true)==2) return;
     std::vector<SOp> q;
     q.swap(Queue);
     if (q.size()>=2 && IsRun(q,q.size())==true)
@@ -422,14 +514,26 @@ namespace mi355
    {
     Settle(&sequence[0],sequence.size());
     ForwardFused++;
-    Check(mt_batchnorm_forward_train_from(&m.H,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,&m.OldMean,&m.OldVar,m.Momentum,m.Epsilon,MT_F_NONE));
+    // with the function layer's call behind it: both layers' outputs from the one kernel
+    if (m.HasFunction==true) Check(mt_batchnorm_forward_train_from(&m.F,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,&m.OldMean,&m.OldVar,m.Momentum,m.Epsilon,m.Func,&m.H));
+    else Check(mt_batchnorm_forward_train_from(&m.H,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,&m.OldMean,&m.OldVar,m.Momentum,m.Epsilon,MT_F_NONE,NULL));
     Pending.push_back(sequence[8]);///<SqrtVar = sqrt(Var + epsilon)
     Pending.push_back(sequence[11]);///<Scratch = Gamma * XHat
+    SNormFact fact;
+    fact.Output=m.H;fact.Gamma=m.Gamma;fact.Beta=m.Beta;fact.XHat=m.XHat;
+    Facts.push_back(fact);
    }
    void RunInference(const std::vector<SOp> &sequence,const SBatchNormInference &m)
    {
     Settle(&sequence[0],sequence.size());
     InferenceFused++;
+    if (m.HasFunction==true)
+    {
+     // the function layer's output from the kernel; the batch-norm layer's own output stays pending with the scratch tensors
+     Check(mt_batchnorm_forward_infer_func(&m.F,&m.X,&m.Gamma,&m.Beta,&m.Mean,&m.Var,m.Epsilon,m.Func));
+     for(size_t i=0;i<6;i++) Pending.push_back(sequence[i]);
+     return;
+    }
     Check(mt_batchnorm_forward_infer_func(&m.H,&m.X,&m.Gamma,&m.Beta,&m.Mean,&m.Var,m.Epsilon,MT_F_NONE));
     for(size_t i=0;i<5;i++) Pending.push_back(sequence[i]);///<everything but the output itself
    }
@@ -439,6 +543,34 @@ namespace mi355
     BackwardFused++;
     Check(mt_batchnorm_backward_keep(&m.Prev,m.Gradients==true?&m.DGamma:NULL,m.Gradients==true?&m.DBeta:NULL,&m.Delta,&m.Gamma,&m.XHat,&m.IVar,&m.DXHat,&m.SumA,&m.SumB));
     Pending.push_back(sequence[m.Gradients==true?10:7]);///<Scratch = XHat * SumB
+   }
+
+   // The function layer's two calls and the batch-norm layer's backward pass as one kernel, when the forward pass that
+   // produced the function layer's input is on record (Beta); else the two calls as written and the backward pass as its
+   // own kernel.
+   void RunFunctionBackward(const std::vector<SOp> &sequence,const SFunctionBackward &m)
+   {
+    const SNormFact *fact=NULL;
+    for(size_t i=0;i<Facts.size();i++)
+     if (Same(Facts[i].Output,m.Output)==true && Same(Facts[i].Gamma,m.Norm.Gamma)==true && Same(Facts[i].XHat,m.Norm.XHat)==true) fact=&Facts[i];
+    if (fact==NULL)
+    {
+     for(size_t i=0;i<2;i++)
+     {
+      Settle(&sequence[i],1);
+      LiteralCalls++;
+      RunLiteral(sequence[i]);
+     }
+     const std::vector<SOp> rest(sequence.begin()+2,sequence.end());
+     RunBackward(rest,m.Norm);
+     return;
+    }
+    const mt_tensor beta=fact->Beta;///<(Settle below may drop the record)
+    Settle(&sequence[0],sequence.size());
+    FunctionBackwardFused++;
+    const SBatchNormBackward &b=m.Norm;
+    Check(mt_batchnorm_backward_func_keep(&b.Prev,b.Gradients==true?&b.DGamma:NULL,b.Gradients==true?&b.DBeta:NULL,&m.Error,&b.Gamma,&beta,&b.XHat,&b.IVar,m.Func,&b.DXHat,&b.SumA,&b.SumB,&m.Front));
+    Pending.push_back(sequence[2+(b.Gradients==true?10:7)]);///<Scratch = XHat * SumB
    }
 
    // ---- pending calls ------------------------------------------------------------------------------------------------
@@ -464,6 +596,14 @@ namespace mi355
    // it changes, run first.
    void Settle(const SOp *unit,size_t count)
    {
+    if (Facts.empty()==false)
+    {
+     std::vector<mt_tensor> written;
+     for(size_t i=0;i<count;i++)
+      for(uint8_t t=0;t<unit[i].Count;t++)
+       if ((unit[i].Writes&(1u<<t))!=0) written.push_back(unit[i].T[t]);
+     if (written.empty()==false) Forget(&written[0],written.size());
+    }
     if (Pending.empty()==true) return;
     // what the unit reads from outside itself, and what it overwrites
     std::vector<mt_tensor> reads,writes;
@@ -483,12 +623,30 @@ namespace mi355
     }
     SettleSets(reads,writes);
    }
-   void SettleRange(const void *p,size_t bytes,bool read,bool write)
+   // a forward pass on record is forgotten when any of its four tensors is written
+   void Forget(const mt_tensor *written,size_t count)
+   {
+    std::vector<SNormFact> left;
+    for(size_t f=0;f<Facts.size();f++)
+    {
+     bool touched=false;
+     for(size_t w=0;w<count && touched==false;w++)
+      touched=Overlap(written[w],Facts[f].Output) || Overlap(written[w],Facts[f].Gamma) || Overlap(written[w],Facts[f].Beta) || Overlap(written[w],Facts[f].XHat);
+     if (touched==false) left.push_back(Facts[f]);
+    }
+    Facts.swap(left);
+   }
+   static mt_tensor Range(const void *p,size_t bytes)
    {
     mt_tensor range;
     range.p=static_cast<float*>(const_cast<void*>(p));
     range.w=1;range.z=1;range.y=1;range.x=static_cast<uint32_t>(bytes/sizeof(float));
     if (static_cast<size_t>(range.x)*sizeof(float)!=bytes) {range.y=static_cast<uint32_t>((bytes/sizeof(float)+0xffffu)>>16);range.x=1u<<16;}///<(a buffer of 16 GiB or more, or one that is no whole number of floats: a range that covers it)
+    return(range);
+   }
+   void SettleRange(const void *p,size_t bytes,bool read,bool write)
+   {
+    const mt_tensor range=Range(p,bytes);
     std::vector<mt_tensor> reads,writes;
     if (read==true) reads.push_back(range);
     if (write==true) writes.push_back(range);

@@ -15,6 +15,16 @@ class CTensorApplyFunc
   static void Apply(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,int func)
   {
    static_assert(std::is_same<type_t,float>::value,"the MI355X tensor path computes in fp32 only");
+   if (&cTensor_Output!=&cTensor_Input && mi355::FusedFunction(func>=MT_F_DIFFERENTIAL?func-MT_F_DIFFERENTIAL:func)==true)
+   {
+    // A function layer's Forward, or the first call of its SetOutputError: deferred, since it may be the end of a
+    // batch-norm layer's forward sequence or the beginning of its backward sequence (mi355::COpQueue).
+    mt_tensor i=cTensor_Input.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
+    if (func>=MT_F_DIFFERENTIAL) mi355::Queue().Submit(mi355::MakeDifferential(o,i,func-MT_F_DIFFERENTIAL));
+                            else mi355::Queue().Submit(mi355::MakeFunction(o,i,func));
+    cTensor_Output.SetDeviceOnChange();
+    return;
+   }
    mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_apply_func(&o,&i,func));
    cTensor_Output.SetDeviceOnChange();

@@ -13,7 +13,8 @@ class CTensorConv
   static void OnlyFloat(void) {static_assert(std::is_same<type_t,float>::value,"the MI355X tensor path computes in fp32 only");}
   // Whether CreateDeltaWeightAndBias may keep the per-sample gradients uncomputed (mi355::CDeferredGradient): both
   // tensors were zeroed and not touched since, one slice per sample of the batch, the bias gradient [B,Kamt,1,1], and
-  // the gradients are at least four times the operands (keeping copies of those must be the cheaper side).
+  // enough gradients for the bookkeeping to matter (the record shares the operands' device blocks: holding them costs
+  // nothing unless somebody overwrites an operand before the sums are taken, and then only a new block).
   static bool Deferrable(const CTensor<type_t> &dkernel,const CTensor<type_t> &dbias,const CTensor<type_t> &image,const CTensor<type_t> &delta)
   {
    if (mi355::DeferGradients()==false) return(false);
@@ -21,8 +22,7 @@ class CTensorConv
    const uint32_t batch=dkernel.GetSizeW();
    if (batch<2 || dbias.GetSizeW()!=batch || image.GetSizeW()!=batch || delta.GetSizeW()!=batch) return(false);
    if (dbias.GetSizeY()!=1 || dbias.GetSizeX()!=1) return(false);
-   const size_t gradients=dkernel.Count(),operands=image.Count()+delta.Count();
-   return(gradients>=(static_cast<size_t>(1)<<20) && gradients>=4*operands);
+   return(dkernel.Count()>=(static_cast<size_t>(1)<<16));
   }
  public:
   static void ForwardConvolution(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Image,const CTensor<type_t> &cTensor_Kernel,int32_t kernel_x,int32_t kernel_y,int32_t kernel_z,uint32_t kernel_amount,const CTensor<type_t> &cTensor_Bias,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)

@@ -113,7 +113,9 @@ class GanGenerator:
         self.p = {k: CTensor.from_numpy(v) for k, v in host.items() if not k.startswith(("mean", "variable"))}
         # running statistics: one tensor serves as the layer's Mean / Variable and as its NewMean / NewVariable, which the
         # layer copies into each other at both ends of a training step (netlayer/cnetlayerbatchnormalization.cu.h:620-621,
-        # 650-651); the training-mode forward pass blends into it
+        # 650-651); the training-mode forward pass blends into it.  The layer itself discards the blend of a forward pass
+        # that no weight update follows (NewMean = Mean at the next reset); this class keeps it: forward passes here are
+        # meant as the forward half of training steps
         self.stats = {k: CTensor.from_numpy(host[k] if k in host else v) for k, v in make_statistics(self.channels).items()}
         b = batch
         self.noise = CTensor(b, 1, noise, 1)

@@ -101,7 +101,10 @@ class DcganGenerator:
     def forward_fused(self):
         """One or two launches per layer.  Batch norm 0 sits in the epilogue of the Linear layer's product (a block holds
         the whole batch of its features); a batch norm i in self.fold never writes its output: the convolution in front of
-        it leaves the raw activation h[i] and the pairs (scale, shift), the convolution behind it normalises as it loads."""
+        it leaves the raw activation h[i] and the pairs (scale, shift), the convolution behind it normalises as it loads.
+        Running statistics: this class measures the forward pass in training mode and keeps none (no new_mean /
+        new_variable is passed; the reference's layer would blend its NewMean / NewVariable here and, without a weight update
+        behind the pass, discard the blend at its next reset, netlayer/cnetlayerbatchnormalization.cu.h:620-621)."""
         p = self.p
         if self.fuse_linear_bn:
             Fused.LinearBatchNormForwardTrain(self.a[0], p["lin_w"], self.latent, p["lin_b"], p["gamma0"], p["beta0"],

@@ -478,12 +478,13 @@ class Fused:
 
     @staticmethod
     def BatchNormForwardTrain(out, inp, gamma, beta, xhat=None, ivar=None, batch_mean=None, batch_var=None, new_mean=None, new_variable=None,
-                              momentum=0.9, epsilon=1e-6, func=None, old_mean=None, old_variable=None):
-        """old_mean / old_variable: the running statistics are blended from these tensors into new_mean / new_variable."""
+                              momentum=0.9, epsilon=1e-6, func=None, old_mean=None, old_variable=None, pre_function=None):
+        """old_mean / old_variable: the running statistics are blended from these tensors into new_mean / new_variable;
+        pre_function: gamma*xhat+beta is written there beside func of it."""
         opt = lambda t: _d(t) if t is not None else None
-        if old_mean is not None or old_variable is not None:
+        if old_mean is not None or old_variable is not None or pre_function is not None:
             return call("mt_batchnorm_forward_train_from", _d(out), _d(inp), _d(gamma), _d(beta), opt(xhat), opt(ivar), opt(batch_mean), opt(batch_var),
-                        opt(new_mean), opt(new_variable), opt(old_mean), opt(old_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
+                        opt(new_mean), opt(new_variable), opt(old_mean), opt(old_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]), opt(pre_function))
         call("mt_batchnorm_forward_train_func", _d(out), _d(inp), _d(gamma), _d(beta), opt(xhat), opt(ivar), opt(batch_mean), opt(batch_var),
              opt(new_mean), opt(new_variable), _f(momentum), _f(epsilon), C.c_int(FUNC[func]))
 
@@ -513,6 +514,13 @@ class Fused:
         """The backward pass that also leaves the intermediate tensors of the layer's own sequence."""
         opt = lambda t: _d(t) if t is not None else None
         call("mt_batchnorm_backward_keep", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), _d(xhat), _d(ivar), opt(dxhat), opt(sum_dxhat), opt(sum_dxhat_xhat))
+
+    @staticmethod
+    def BatchNormBackwardFuncKeep(error, dgamma, dbeta, delta, gamma, beta, xhat, ivar, func, dxhat=None, sum_dxhat=None, sum_dxhat_xhat=None, delta_front=None):
+        """The function layer's backward step and the batch-norm layer's backward pass in one kernel, leaving what both sequences leave."""
+        opt = lambda t: _d(t) if t is not None else None
+        call("mt_batchnorm_backward_func_keep", _d(error), opt(dgamma), opt(dbeta), _d(delta), _d(gamma), opt(beta), _d(xhat), _d(ivar), C.c_int(FUNC[func]),
+             opt(dxhat), opt(sum_dxhat), opt(sum_dxhat_xhat), opt(delta_front))
 
     @staticmethod
     def UpSamplingConvolution(out, image, upsampling_x, upsampling_y, kernel, kernel_x, kernel_y, kernel_z, kernel_amount, bias, stride_x, stride_y,

@@ -101,6 +101,9 @@ class Vae:
         return self.dh[4]
 
     def forward(self):
+        # batch norm in training mode (batch statistics); running statistics are not kept here: a forward pass without a
+        # weight update leaves the reference's Mean / Variable unchanged too (its NewMean is reset from Mean,
+        # netlayer/cnetlayerbatchnormalization.cu.h:620-621)
         p, h = self.p, self.x
         for i in range(4):
             CTensorConv.ForwardConvolution(self.ec[i], h, p["ekernel%d" % i], 3, 3, ENCODER[i], ENCODER[i + 1], p["ebias%d" % i], 2, 2, 1, 1)

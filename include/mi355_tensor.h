@@ -279,11 +279,13 @@ int mt_batchnorm_forward_train_func(const mt_tensor *output, const mt_tensor *in
 /* The same call with the running statistics blended FROM other tensors: new_mean = momentum * old_mean + (1 - momentum) * batch
  * mean, likewise the variance (lines 311 and 324 with cTensor_NewMean sharing its memory with cTensor_Mean, as it does after
  * TrainingResetDeltaWeight, netlayer/cnetlayerbatchnormalization.cu.h:617-618, in a container whose copies share storage);
- * old_mean / old_variable NULL: blended in place. */
+ * old_mean / old_variable NULL: blended in place.  pre_function [B,Z,Y,X] (NULL to skip): gamma*xhat+beta, the batch-norm
+ * layer's own output tensor when `output` is the function layer's (netlayer/cnetlayerfunction.cu.h:202-212); a tensor of
+ * its own. */
 int mt_batchnorm_forward_train_from(const mt_tensor *output, const mt_tensor *input, const mt_tensor *gamma, const mt_tensor *beta,
                                     const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *batch_mean, const mt_tensor *batch_var,
                                     const mt_tensor *new_mean, const mt_tensor *new_variable, const mt_tensor *old_mean,
-                                    const mt_tensor *old_variable, float momentum, float epsilon, int func);
+                                    const mt_tensor *old_variable, float momentum, float epsilon, int func, const mt_tensor *pre_function);
 /* The same call for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Statistics the caller does not ask for go to a
  * fixed array inside the library's code object (3 MiB per GPU, held until the process ends) instead of a workspace
@@ -323,6 +325,14 @@ int mt_batchnorm_backward_func(const mt_tensor *error, const mt_tensor *dgamma, 
 int mt_batchnorm_backward_keep(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta,
                                const mt_tensor *gamma, const mt_tensor *xhat, const mt_tensor *ivar, const mt_tensor *dxhat,
                                const mt_tensor *sum_dxhat, const mt_tensor *sum_dxhat_xhat);
+/* Both of the above: CNetLayerFunction::SetOutputError (netlayer/cnetlayerfunction.cu.h:347-358) and the batch-norm layer's
+ * TrainingBackward (netlayer/cnetlayerbatchnormalization.cu.h:578-604) as one kernel that leaves what the two literal sequences
+ * leave: delta_front [B,Z,Y,X] = delta * f'(gamma*xhat+beta) (the function layer's own delta tensor; may be the same tensor
+ * as delta, not the error or dxhat), dxhat = delta_front*gamma, the two sums; NULL skips any of them. */
+int mt_batchnorm_backward_func_keep(const mt_tensor *error, const mt_tensor *dgamma, const mt_tensor *dbeta, const mt_tensor *delta,
+                                    const mt_tensor *gamma, const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func,
+                                    const mt_tensor *dxhat, const mt_tensor *sum_dxhat, const mt_tensor *sum_dxhat_xhat,
+                                    const mt_tensor *delta_front);
 /* CNetLayerConvolution::TrainingBackward, netlayer/cnetlayerconvolution.cu.h:501-508, without the per-sample round trip:
  * dkernel [1,1,Kamt,C*Ky*Kx] += sum over the batch of the per-sample weight gradients (CreateDeltaWeightAndBias into a
  * zeroed batch tensor, then AddSumW), dbias [1,Kamt,1,1] += sum over the batch and the pixels of delta. */

@@ -887,6 +887,17 @@ def test_batchnorm_running_statistics_blended_from_other_tensors(gpu, shape):
     Fused.BatchNormForwardTrain(out_b, tx, tg, tb, new_mean=new_m, new_variable=new_v, momentum=0.8, old_mean=old_m, old_variable=old_v)
     assert np.array_equal(new_m.numpy(), want_m.numpy()) and np.array_equal(new_v.numpy(), want_v.numpy())
     assert np.array_equal(old_m.numpy(), om) and np.array_equal(old_v.numpy(), ov) and np.array_equal(out_a.numpy(), out_b.numpy())
+    # the value in front of the function beside the function's: the batch-norm layer's output and the function layer's in one call
+    for func in ("leaky_relu", "tangence"):   # inside the one-pass kernel; through the two-pass kernels
+        out_f, pre = CTensor(*shape), CTensor(*shape)
+        Fused.BatchNormForwardTrain(out_f, tx, tg, tb, func=func, pre_function=pre)
+        if func == "leaky_relu":
+            assert np.array_equal(pre.numpy(), out_a.numpy())
+        else:   # (the two-pass kernels add the batch up in another order than the one-pass kernel)
+            close(pre.numpy(), out_a.numpy(), 1e-6)
+        plain = CTensor(*shape)
+        Fused.BatchNormForwardTrain(plain, tx, tg, tb, func=func)
+        assert np.array_equal(out_f.numpy(), plain.numpy())
 
 
 @pytest.mark.parametrize("shape", [(600, 2, 4, 8), (1024, 1, 8, 8), (1500, 1, 4, 8), (2100, 1, 4, 4), (700, 1, 3, 3)])
@@ -956,6 +967,19 @@ def test_batchnorm_backward_behind_a_function(gpu, oracle, shape, func):
     assert np.max(np.abs(err - want_err)) <= 1e-5 * max(scale, np.abs(want_err).max())
     close(dg, want_dg, 1e-5)
     close(db, want_db, 1e-5)
+    # the variant that also leaves what the two layers' sequences leave: the function layer's delta (in place of the error
+    # it was given), dxhat and the two sums
+    from mi355tensor import CTensor, Fused
+    from gpu_api import up
+    one = (1,) + tuple(shape[1:])
+    t_err, t_dg, t_db, t_dx, t_s1, t_s2, t_delta = CTensor(*shape), up(zero), up(zero), CTensor(*shape), CTensor(*one), CTensor(*one), up(error)
+    Fused.BatchNormBackwardFuncKeep(t_err, t_dg, t_db, t_delta, up(gamma), up(beta), up(fwd["xhat"]), up(fwd["ivar"]), func, t_dx, t_s1, t_s2, t_delta)
+    assert np.array_equal(t_err.numpy(), err) and np.array_equal(t_dg.numpy(), dg) and np.array_equal(t_db.numpy(), db)
+    close(t_delta.numpy(), delta, 1e-6)
+    dxhat = oracle.tensor_item_production(delta, gamma)
+    close(t_dx.numpy(), dxhat, 1e-6)
+    close(t_s1.numpy(), oracle.add_sum_w(zero, dxhat, out_init=zero), 1e-5)
+    close(t_s2.numpy(), oracle.add_sum_w(zero, oracle.tensor_item_production(dxhat, fwd["xhat"]), out_init=zero), 1e-5)
 
 
 def test_fill_and_adam_over_many_tensors(gpu, oracle):
