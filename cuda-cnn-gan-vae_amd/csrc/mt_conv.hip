@@ -1460,7 +1460,9 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
     fl.ld = kernel->x; fl.KA = ka; fl.H = image->y; fl.W = image->x; fl.OH = out->y; fl.OW = out->x; fl.batch = out->w;
     fl.pad_y = py; fl.pad_x = px;
     fl.func = mt::epilogue_func(func) ? func : MT_F_NONE;
-    mt::ProfileScope prof(mt::profiling() ? shape_label(name, T32x128, ka, out->w * OHW, K, 1) : name);
+    char tag[96];
+    snprintf(tag, sizeof tag, "input patch M%u N%u K%u x1", ka, out->w * OHW, K);
+    mt::ProfileScope prof(mt::profiling() ? mt::intern_label(name, tag) : name);
     if (first_layer_launch(name, fl, kz, ky, kx, sx, &rc)) {
       if (rc) return rc;
       return mt::epilogue_func(func) ? MT_OK : mt_apply_func(out, out, func);
