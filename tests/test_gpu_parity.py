@@ -414,6 +414,40 @@ def test_weights_sum_as_one_k_loop_per_block(gpu, oracle, case):
     close(got[1][0], got[0][0], 2e-6)
 
 
+def _random_walk_wgrad_cases(n, seed):
+    """Seeded random geometries the walking weight-gradient kernel takes: 64 or 128 filters, output rows of 4 to 64 pixels
+    that tile (or are tiled by) the k step, kernels 3x3 stride 1 and 4x4 stride 2 (padding 1), ragged channel counts."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < n:
+        k, s = ((3, 1), (4, 2))[int(rng.integers(0, 2))]
+        ow = int(rng.choice([4, 8, 16, 32, 64]))
+        rows_per_step = max(1, 16 // ow)
+        oh = rows_per_step * int(rng.integers(1, 5)) * (2 if ow >= 16 else 1)
+        C, KA, B = int(rng.integers(1, 24)), int(rng.choice([64, 128])), int(rng.integers(2, 9))
+        H, Wd = (oh - 1) * s + k - 2, (ow - 1) * s + k - 2
+        if s == 2:
+            H, Wd = H + int(rng.integers(0, 2)), Wd + int(rng.integers(0, 2))   # the last input row / column may go unused
+        if H < 1 or Wd < 1 or (H - k + 2) // s + 1 != oh or (Wd - k + 2) // s + 1 != ow:
+            continue
+        cases.append((B, C, H, Wd, KA, k, s))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_walk_wgrad_cases(14, 77))
+def test_weights_sum_walk_random_geometries(gpu, oracle, case):
+    B, C, H, Wd, KA, k, s = case
+    oy, ox = (H - k + 2) // s + 1, (Wd - k + 2) // s + 1
+    image, delta = U(31, B, C, H, Wd), U(32, B, KA, oy, ox)
+    dk0, db0 = U(33, 1, 1, KA, C * k * k), U(34, 1, KA, 1, 1)
+    dkb, dbb = oracle.create_delta_weight_and_bias(np.zeros((B, 1, KA, C * k * k), np.float32), np.zeros((B, KA, 1, 1), np.float32),
+                                                   image, delta, k, k, C, KA, s, s, 1, 1)
+    want_k, want_b = oracle.add_sum_w(dk0, dkb, out_init=dk0), oracle.add_sum_w(db0, dbb, out_init=db0)
+    got_k, got_b = gpu.convolution_backward_weights_sum(dk0, db0, image, delta, k, k, C, KA, s, s, 1, 1)
+    close(got_k, want_k)
+    close(got_b, want_b)
+
+
 @pytest.mark.parametrize("case", [
     # B, C, H, W, KA
     (2, 16, 6, 8, 32),      # channels tile the k step
