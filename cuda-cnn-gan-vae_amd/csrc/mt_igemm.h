@@ -963,6 +963,8 @@ __device__ __forceinline__ uint32_t xcd_swizzle(uint32_t L, uint32_t total) {
   return (L % 8) * per + L / 8;
 }
 
+__device__ __forceinline__ constexpr uint32_t igemm_group_n() { return 8; }
+
 // Generic launch: logical block index = (n tile, batch entry, m tile), n slowest, so concurrently running blocks
 // of one XCD share their B tile (the activations) and cycle through the A tiles (the weights).
 template <int TM, int TN, int WGM, int WGN, bool R16, bool BN_TAIL = false, class SrcA, class SrcB>
@@ -972,6 +974,15 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(TM * TN
   uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x);
   uint32_t group = tiles_m * batches;
   uint32_t nt = j / group, rem = j % group, bz = rem / tiles_m, mt = rem % tiles_m;
+  if (batches == 1 && tiles_m >= 16) {
+    // One large product: with m fastest, the blocks that run together (some 160 per XCD) would cover all row tiles of two or
+    // three column tiles and stream the whole of A through the L2 once per column tile.  Groups of eight column tiles, column
+    // fastest inside a group: the same blocks cover a patch of about 20 x 8 tiles and fetch 28 operand panels instead of 66.
+    const uint32_t tiles_n = gridDim.x / tiles_m, per_group = igemm_group_n() * tiles_m, g = j / per_group, idx = j % per_group;
+    const uint32_t first = g * igemm_group_n(), gn = tiles_n - first < igemm_group_n() ? tiles_n - first : igemm_group_n();
+    mt = idx / gn;
+    nt = first + idx % gn;
+  }
   a.batch(bz);
   b.batch(bz);
   ep.batch(bz);
@@ -1010,7 +1021,10 @@ inline Tile pick_tile(uint32_t M, uint32_t N, uint32_t batches) {
   // 64x64 blocks need only 20 KB of LDS and 60 registers, so eight of them share a compute unit and hide each
   // other's barriers and load latency; larger blocks only pay off when the grid is huge anyway
   size_t big = (size_t)cdiv(M, 128) * cdiv(N, 128) * batches;
-  if (big >= 8192) return T128x128;
+  // (two 128x128 blocks share a compute unit: a grid that is a whole number of rounds of 512, or many rounds.  Measured after
+  // a warm-up: 4096^3 1040 us against 1135 us with 64x64 blocks, 4096 x 4096 x 2048 522 against 586; but 3072^3, 576 blocks,
+  // 639 against 506, and 2048^3 174 against 172)
+  if (big >= 512 && (big % 512 == 0 || big >= 2048)) return T128x128;
   return T64x64;
 }
 
