@@ -112,6 +112,8 @@ int mt_timer_destroy(void *timer);
  *   "wgrad_walk"     1 (default) mt_convolution_backward_weights_sum runs each group of samples as one k loop per block, with
  *                    fixed gather offsets, where the shape allows (output rows of 4, 8 or 16 pixels, filters a multiple of 64) /
  *                    0 never
+ *   "upconv_walk"    512 (default) mt_upsampling_convolution_func (x2, 3x3) uses the walking kernel when that gives at least this
+ *                    many blocks / 1 wherever the shape allows / 0 never
  *   "first_layer"    1 (default) forward convolutions of 3-channel images (3x3, 4x4, 5x5 kernels to 32 or 64 filters) keep the
  *                    input patch in LDS and the weights in registers wherever the shape allows / 0 never
  *   "walk_blocks"    blocks wanted per launch of the walking kernel (default 1024)

@@ -455,6 +455,8 @@ def test_weights_sum_walk_random_geometries(gpu, oracle, case):
     (1, 8, 1, 1, 4),        # one input pixel: every tap but one is padding
     (2, 4, 5, 3, 70),       # odd input sizes, more filters than one tile
     (2, 64, 12, 16, 32),    # a layer of the reference's GAN generator at a quarter of its width
+    (4, 32, 8, 16, 64),     # 64 filters, 128 pixels per sample: whole tiles for the walking kernel
+    (8, 16, 4, 4, 128),     # 16 pixels per sample: four samples share a tile of the walking kernel
     (2, 512, 3, 4, 64),     # its first layer: few blocks, k = 2048 per phase, split over k
     (2, 32, 12, 16, 16),    # its last up-sampling layer at an eighth of the size: the input patch kernel
     (3, 16, 9, 35, 7),      # the same kernel with sixteen channels, seven filters and partial tiles
@@ -463,12 +465,18 @@ def test_upsampling_convolution(gpu, oracle, path, case):
     """Up-sampling x2 + convolution 3x3 stride 1 padding 1 (+ function) in one call, against the two layers on the
     oracle (netlayer/cnetlayerupsampling.cu.h:233-252, netlayer/cnetlayerconvolution.cu.h:310-322): four 2x2
     convolutions of the input with summed coefficients, so sums differ from the reference's by rounding only."""
+    import mi355tensor as mt
     B, C, H, Wd, KA = case
     image, kernel, bias = U(1, B, C, H, Wd), Nrm(2, 1, 1, KA, C * 9, std=float(np.sqrt(2.0 / (C * 9)))), U(3, 1, KA, 1, 1) * 0.3
     want = oracle.forward_convolution(oracle.upsampling(image, 2, 2), kernel, bias, 3, 3, C, KA, 1, 1, 1, 1)
-    close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA), want, 1e-5)
-    close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA, func="leaky_relu"), oracle.apply_func(want, "leaky_relu"), 1e-5)
-    close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA, func="tangence"), oracle.apply_func(want, "tangence"), 1e-5)
+    try:
+        for walk in (512, 1):   # the library's choice; the kernel whose blocks walk over the batch wherever the shape allows
+            mt.set_option("upconv_walk", walk)
+            close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA), want, 1e-5)
+            close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA, func="leaky_relu"), oracle.apply_func(want, "leaky_relu"), 1e-5)
+            close(gpu.upsampling_convolution(image, kernel, bias, 3, C, KA, func="tangence"), oracle.apply_func(want, "tangence"), 1e-5)
+    finally:
+        mt.set_option("upconv_walk", 512)
 
 
 def test_upsampling_convolution_other_geometries(gpu, oracle, path):
