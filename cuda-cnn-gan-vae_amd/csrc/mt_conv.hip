@@ -28,6 +28,7 @@ using mt::cdiv;
 int g_conv_path = 0;  // 0 auto, 1 direct, 2 implicit GEMM wherever it applies
 int g_first_layer = 1; // forward convolutions of 3-channel images: 0 never on the kernel that keeps the input patch in LDS and the weights in registers, 1 wherever the shape allows
 int g_conv_walk = 1;   // forward convolutions whose taps tile the k step: 0 never on the kernel whose blocks walk over the batch, 1 wherever the shape allows and gives 512 blocks, 2 wherever the shape allows
+int g_upconv_split = 1;    // 1: up-sampling convolutions with fewer than 512 walking blocks share a tile's k steps between blocks
 int g_upconv_walk = 512;   // blocks from which the up-sampling convolution takes the walking kernel (0: never; measured on the
                            // shipped GAN generator at batch 32: 768 blocks 67.7 -> 54.6 and 58.6 -> 54.0 us, 384 blocks 65.1 -> 69 us)
 uint64_t g_wgrad_walk_launches = 0;
@@ -2036,13 +2037,29 @@ int upsampling_convolution(const char *name, const mt_tensor *out, const mt_tens
     walk.M = ka; walk.batch = out->w; walk.delta = image->p; walk.C = (uint32_t)kz; walk.H = image->y; walk.W = image->x;
     walk.out = out->p; walk.OW = out->x; walk.OHW = OHW; walk.sy = 2; walk.sx = 2;
     walk.row_bias = bias->p; walk.tap_bias = nullptr; walk.func = args.ep.func;
-    if (mt::igemm::tconv_walk_plan(walk, (uint32_t)mt::igemm::walk_blocks(), 1) &&
-        (size_t)walk.nphase * walk.tiles_m * walk.qtiles * walk.groups >= (size_t)g_upconv_walk) {
-      {
-        mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, out->w * args.ph[0].qh * args.ph[0].qw, args.ph[0].kp, args.nphase) : name);
+    if (mt::igemm::tconv_walk_plan(walk, (uint32_t)mt::igemm::walk_blocks(), 1) || mt::igemm::tconv_walk_plan_flat(walk)) {
+      // too few tiles for the chip (small images, many channels): two or four blocks share a tile's k steps, their sums
+      // are added afterwards together with the bias and the function
+      const size_t blocks = (size_t)walk.nphase * walk.tiles_m * walk.qtiles * walk.groups;
+      uint32_t share = 1;
+      if (g_upconv_split && walk.per == 1 && blocks < 512 && mt::count(out) <= (1u << 22))
+        while (share < 4 && blocks * share < 512 && walk.nk % (4 * share) == 0 && walk.nk / (2 * share) >= 8) share *= 2;
+      if (share > 1) {
+        float *partial = nullptr;
+        if ((rc = mt::split_workspace((size_t)share * mt::count(out), &partial))) return rc;
+        walk.ksplit = share; walk.nk /= share; walk.split_stride = mt::count(out);
+        walk.out = partial; walk.row_bias = nullptr; walk.func = MT_F_NONE;
+        mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, out->w * args.ph[0].qh * args.ph[0].qw, walk.nk * mt::igemm::BK, args.nphase * share) : name);
         if ((rc = mt::igemm::launch_tconv_walk(name, walk, false, false, 1))) return rc;
+        return mt::split_reduce(name, out->p, partial, share, mt::count(out), bias->p, OHW, ka, func);
       }
-      return func_later ? mt_apply_func(out, out, func) : MT_OK;
+      if (blocks >= (size_t)g_upconv_walk) {
+        {
+          mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, out->w * args.ph[0].qh * args.ph[0].qw, args.ph[0].kp, args.nphase) : name);
+          if ((rc = mt::igemm::launch_tconv_walk(name, walk, false, false, 1))) return rc;
+        }
+        return func_later ? mt_apply_func(out, out, func) : MT_OK;
+      }
     }
   }
   rc = launch_tconv(name, args, max_n, mt::count(out));
@@ -2186,6 +2203,11 @@ int set_patch_blocks(int v) {
 int set_igemm_tile(int v) {
   if (v < -1 || v > 4) return fail(MT_E_ARGUMENT, "igemm_tile must be -1 (auto) or 0..4");
   igemm::tile_override() = v;
+  return MT_OK;
+}
+int set_upconv_split(int v) {
+  if (v < 0 || v > 1) return fail(MT_E_ARGUMENT, "upconv_split must be 0 (never) or 1 (where too few tiles would fill the chip)");
+  g_upconv_split = v;
   return MT_OK;
 }
 int set_upconv_walk(int v) {

@@ -33,7 +33,11 @@ struct WalkArgs {
   TconvPhase ph[MAX_PHASES];
   uint32_t nphase, tiles_m, M, batch;
   uint32_t px_log, qtiles, groups, per;  // PX = 1 << px_log pixels per tile; pixel tiles per phase; batch groups; steps per block
-  uint32_t nk;                           // k steps of one tile (the same for every phase)
+  uint32_t nk;                           // k steps of one block's tile (the same for every phase): all of them, or one of ksplit equal shares
+  uint32_t ksplit = 1;                   // blocks that share a tile's k steps; block ks writes its sums to out + ks * split_stride (per = 1 then)
+  size_t split_stride = 0;               // floats
+  uint32_t flat = 0;                     // 1: the columns are (sample, pixel) pairs counted through the whole batch, 64 to a tile (qtiles of
+                                         // them, the last one may be ragged), for pixel counts that no tile of 16, 32 or 64 divides; no walk
   uint32_t weights_major;                // block order, see tconv_walk_kernel
   uint32_t fair;                         // 0, or three hexadecimal digits: sixteenths of the steps left at which a wavefront's priority drops to 2, 1, 0
   const float *delta;                    // [batch][C][H][W]
@@ -71,7 +75,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   // fit an L2 beside the rest (weights_major), the order is by row tile first: an XCD then reads one row tile's weights
   // (all phases) again and again from its own L2 and streams its share of the input through once; the phases of a
   // tile stay neighbours, so their stores, which interleave pixel by pixel, still meet in one L2.
-  uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x), mt, f, qt, g;
+  uint32_t j = xcd_swizzle(blockIdx.x, gridDim.x), mt, f, qt, g, ks = 0;
+  if (a.ksplit > 1) { ks = j % a.ksplit; j /= a.ksplit; }
   if (a.weights_major) {
     f = j % a.nphase; j /= a.nphase;
     qt = j % a.qtiles; j /= a.qtiles;
@@ -101,9 +106,10 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   uint32_t b_voff[E], sample_bytes;  // (the offsets of the pairs follow from b_voff: twice the offset inside the sample)
   uint32_t sstep;
   {
-    const uint32_t q = qt * (px_mask + 1u) + (b_col & px_mask), s = b_col >> a.px_log;
+    const uint32_t qhw = ph.qh * ph.qw, n = qt * BN + b_col;
+    const uint32_t q = a.flat ? n % qhw : qt * (px_mask + 1u) + (b_col & px_mask);
     const uint32_t qy = q / ph.qw, qx = q % ph.qw;
-    const uint32_t sample = g * a.per * sp + s;
+    const uint32_t sample = a.flat ? n / qhw : g * a.per * sp + (b_col >> a.px_log);
     const uint32_t tx_cnt = (uint32_t)ph.taps_x, taps = (uint32_t)(ph.taps_y * ph.taps_x);  // taps divides BK: powers of two
     const int lt = __builtin_ctz(taps), lx = __builtin_ctz(tx_cnt);
     const bool col_ok = q < ph.qh * ph.qw && sample < a.batch;
@@ -119,11 +125,12 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
     sstep = (BK / taps) * HW * 4u;
   }
   const uint32_t group_step = sp * a.C * HW * 4u, nk = a.nk;
-  uint32_t a_soff = 0, b_soff = 0, ctile = 0;
+  const uint32_t a_first = ks * nk * BK * 4u;  // the block's share of the k steps starts here
+  uint32_t a_soff = a_first, b_soff = ks * nk * sstep, ctile = 0;
   auto advance = [&]() {  // scalar unit only
     ctile++;
     a_soff += BK * 4u; b_soff += sstep;
-    if (ctile == nk) { ctile = 0; a_soff = 0; b_soff += group_step - nk * sstep; }
+    if (ctile == nk) { ctile = 0; a_soff = a_first; b_soff += group_step - nk * sstep; }
   };
 
   // Register sets: A and B are loaded two steps before they are written to LDS (two sets, tile t+3 requested while
@@ -131,13 +138,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   // single set -- in front of the A and B loads of the same step, so that waiting for them leaves those in flight.
   float ra[2][TM][E], rb[2][E];
   floatx2 rs[NORM ? E : 1];
-  uint32_t s_next = 0;  // scalar offset of the pairs of the tile that is written to LDS next
+  const uint32_t s_first = 2u * ks * nk * sstep;
+  uint32_t s_next = s_first;  // scalar offset of the pairs of the tile that is written to LDS next
   auto load_pairs = [&]() {
     if constexpr (NORM) {
 #pragma unroll
       for (int i = 0; i < E; i++) rs[i] = buf_load2(s_rsrc, b_voff[i] == OOB ? OOB : (b_voff[i] - sample_bytes) * 2u, s_next);
       s_next += 2u * sstep;
-      if (s_next == 2u * sstep * nk) s_next = 0;
+      if (s_next == s_first + 2u * sstep * nk) s_next = s_first;
     }
   };
   auto load_tile = [&](int set, bool adv) {
@@ -215,7 +223,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
 
   // ---- the lane's column of C: pixel and sample of the first group; register r is row m_lane + 8*(r/4) + r%4
   const uint32_t c_col = (uint32_t)(wn * 32 + lrow);
-  const uint32_t c_q = qt * (px_mask + 1u) + (c_col & px_mask), c_s = c_col >> a.px_log;
+  const uint32_t c_n = qt * BN + c_col, c_qhw = ph.qh * ph.qw;
+  const uint32_t c_q = a.flat ? c_n % c_qhw : qt * (px_mask + 1u) + (c_col & px_mask);
+  const uint32_t c_sample = a.flat ? c_n / c_qhw : g * a.per * sp + (c_col >> a.px_log);
   const uint32_t c_qy = c_q / ph.qw, c_qx = c_q % ph.qw;
   const uint32_t pix = (c_qy * a.sy + ph.py) * a.OW + c_qx * a.sx + ph.px;
   const uint32_t m_lane = m0 + (uint32_t)(wm * TM * 32 + 4 * lk);  // whole blocks of rows and whole pixel tiles: no row or column tests
@@ -232,7 +242,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
     extra = a.tap_bias[0] * (float)(ny * nx);
   }
   // element offsets fit 32 bits (the output is addressed like the input: less than 2 GiB)
-  uint32_t dst = ((g * a.per * sp + c_s) * a.M + m_lane) * a.OHW + pix;
+  uint32_t dst = c_sample < a.batch ? (c_sample * a.M + m_lane) * a.OHW + pix : OOB / 4u;  // (columns past the batch: only in a ragged flat tile)
   const uint32_t dst_step = sp * a.M * a.OHW;
   const int func = a.func;
   constexpr int NS = STATS ? 16 * TM : 1;
@@ -245,7 +255,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   // The output is addressed like the input, through a buffer descriptor (less than 2 GiB): the lane's first element as
   // a 32-bit byte offset, the row of register r as a scalar offset -- no 64-bit address arithmetic per store, and one
   // look at the output function for all sixteen values instead of a chain of branches per value.
-  const __amdgpu_buffer_rsrc_t o_rsrc = make_rsrc(a.out, a.batch * a.M * a.OHW * 4u);
+  const __amdgpu_buffer_rsrc_t o_rsrc = make_rsrc(a.out + (size_t)ks * a.split_stride, a.batch * a.M * a.OHW * 4u);
   const uint32_t row_bytes = a.OHW * 4u;
   auto flush = [&]() {
     seen++;
@@ -607,10 +617,10 @@ __global__ __launch_bounds__(256) void bn_finish_kernel(float *scale_shift, floa
   if (new_var) new_var[e] = (mom_old * new_var[e]) + (mom_new * var);
 }
 
-// Whether (and how) a transposed convolution can walk: fills px_log, qtiles, groups, per, nk.
 int &walk_order();    // -1 choose per layer (default), 0 batch groups first, 1 row tiles first (measurements only)
 int &walk_fair();     // 0x842 (default): wavefronts lower their priority at 8/16, 4/16, 2/16 of their steps left; 0: no priorities (measurements only)
-inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
+// What every use of tconv_walk_kernel needs of the phases and the sizes.
+inline bool tconv_walk_fits(const WalkArgs &a, uint32_t tm) {
   if (a.nphase == 0 || a.M == 0 || a.batch == 0) return false;
   const TconvPhase &p0 = a.ph[0];
   const uint32_t qhw = p0.qh * p0.qw;
@@ -621,7 +631,14 @@ inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
     if (a.C % (BK / taps) != 0 || ph.ld < ph.kp || ph.ld % 4 != 0) return false;
   }
   if (p0.kp % (2 * BK) != 0 || p0.kp < 4 * BK || a.M % (64 * tm) != 0) return false;
-  if ((uint64_t)a.batch * a.M * a.OHW * 4u >= 0x80000000ull) return false;
+  return (uint64_t)a.batch * a.M * a.OHW * 4u < 0x80000000ull && (uint64_t)a.batch * a.C * a.H * a.W * 4u < 0x80000000ull;
+}
+// Whether (and how) a transposed convolution can walk: fills px_log, qtiles, groups, per, nk.
+inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
+  if (!tconv_walk_fits(a, tm)) return false;
+  const TconvPhase &p0 = a.ph[0];
+  const uint32_t qhw = p0.qh * p0.qw;
+  a.flat = 0;
   a.nk = p0.kp / BK;
   // pixels per tile: 16 (four samples per tile: two per wavefront, merged by a lane shuffle), else 32 or 64
   uint32_t px_log = 0;
@@ -641,8 +658,25 @@ inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
   a.per = sample_groups / groups;
   // more packed weights than an XCD's L2 holds (4 MiB), and several row tiles to deal out
   a.fair = (uint32_t)walk_fair();
+  a.ksplit = 1; a.split_stride = 0;
   a.weights_major = walk_order() >= 0 ? (uint32_t)walk_order() : ((uint64_t)a.nphase * a.M * p0.kp * 4u > (4u << 20) && a.tiles_m > 1 ? 1u : 0u);
   return (uint64_t)base * groups <= 0x7fffffffu;
+}
+
+// The same kernel without a walk, for any number of pixels per sample: tiles of 64 (sample, pixel) columns through the
+// whole batch, every block one tile over all k steps (64-row blocks only, no statistics).
+inline bool tconv_walk_plan_flat(WalkArgs &a) {
+  if (!tconv_walk_fits(a, 1)) return false;
+  const TconvPhase &p0 = a.ph[0];
+  const uint64_t n = (uint64_t)a.batch * p0.qh * p0.qw;
+  a.flat = 1;
+  a.nk = p0.kp / BK;
+  a.px_log = 6; a.qtiles = (uint32_t)((n + 63) / 64); a.groups = 1; a.per = 1;
+  a.tiles_m = a.M / 64;
+  a.fair = (uint32_t)walk_fair();
+  a.ksplit = 1; a.split_stride = 0;
+  a.weights_major = walk_order() >= 0 ? (uint32_t)walk_order() : ((uint64_t)a.nphase * a.M * p0.kp * 4u > (4u << 20) && a.tiles_m > 1 ? 1u : 0u);
+  return (uint64_t)a.nphase * a.tiles_m * a.qtiles <= 0x7fffffu;
 }
 
 int &walk_blocks();   // blocks wanted per launch (measurements only); default 1024, or 1280 for the plain variant
@@ -650,9 +684,12 @@ int &walk_waves();
 int &walk_tm();       // 1 or 2 accumulators per wavefront (2 where the output channels allow; measurements only)    // 4 or 5 wavefronts per SIMD for the plain variant (measurements only)
 
 inline int launch_tconv_walk(const char *name, const WalkArgs &a, bool norm, bool stats, uint32_t tm) {
-  const uint32_t grid = a.nphase * a.tiles_m * a.qtiles * a.groups;
+  const uint32_t grid = a.nphase * a.tiles_m * a.qtiles * a.groups * a.ksplit;
   hipStream_t s = stream();
   const int n = !norm ? 0 : a.in_func == MT_F_RELU ? 1 : 2;
+  if (a.flat && (stats || tm != 1 || a.per != 1 || a.groups != 1)) return fail(MT_E_ARGUMENT, "%s: flat column tiles do not walk and keep no statistics", name);
+  if (a.ksplit > 1 && (stats || a.per != 1 || a.nk < 4 || a.nk % 2 != 0 || a.row_bias || a.tap_bias || a.func != MT_F_NONE))
+    return fail(MT_E_ARGUMENT, "%s: blocks that share a tile's k steps write plain sums of one batch group", name);
   if (a.row_bias) {  // forward convolution: plain variant only
     if (norm || stats || tm != 1) return fail(MT_E_ARGUMENT, "%s: a forward convolution walks without batch-norm folding", name);
     tconv_walk_kernel<0, false, 4, 1, true><<<grid, THREADS, 0, s>>>(a);

@@ -114,6 +114,9 @@ int mt_timer_destroy(void *timer);
  *                    0 never
  *   "upconv_walk"    512 (default) mt_upsampling_convolution_func (x2, 3x3) uses the walking kernel when that gives at least this
  *                    many blocks / 1 wherever the shape allows / 0 never
+ *   "upconv_split"   1 (default) where that kernel would get fewer than 512 blocks (small images, many channels), two or four
+ *                    blocks share a tile's sum over (channel, tap) and a second kernel adds their parts, the bias and the function /
+ *                    0 never
  *   "first_layer"    1 (default) forward convolutions of 3-channel images (3x3, 4x4, 5x5 kernels to 32 or 64 filters) keep the
  *                    input patch in LDS and the weights in registers wherever the shape allows / 0 never
  *   "walk_blocks"    blocks wanted per launch of the walking kernel (default 1024)

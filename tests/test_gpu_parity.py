@@ -457,6 +457,11 @@ def test_weights_sum_walk_random_geometries(gpu, oracle, case):
     (2, 64, 12, 16, 32),    # a layer of the reference's GAN generator at a quarter of its width
     (4, 32, 8, 16, 64),     # 64 filters, 128 pixels per sample: whole tiles for the walking kernel
     (8, 16, 4, 4, 128),     # 16 pixels per sample: four samples share a tile of the walking kernel
+    (4, 64, 4, 4, 64),      # few tiles, 16 k steps: two blocks share a tile's k steps
+    (8, 128, 4, 8, 64),     # few tiles, 32 k steps: four blocks share them
+    (4, 64, 3, 4, 64),      # 12 pixels per sample: one ragged tile of (sample, pixel) columns, two blocks share its k steps
+    (6, 32, 3, 5, 64),      # 15 pixels per sample: two such tiles, the second ragged
+    (32, 128, 3, 4, 128),   # the shape of the shipped GAN generator's first layer at a quarter of its channels
     (2, 512, 3, 4, 64),     # its first layer: few blocks, k = 2048 per phase, split over k
     (2, 32, 12, 16, 16),    # its last up-sampling layer at an eighth of the size: the input patch kernel
     (3, 16, 9, 35, 7),      # the same kernel with sixteen channels, seven filters and partial tiles
