@@ -484,6 +484,31 @@ def test_upsampling_convolution(gpu, oracle, path, case):
         mt.set_option("upconv_walk", 512)
 
 
+def test_upsampling_convolution_walk_random_geometries(gpu, oracle, path):
+    """The walking routes of the fused call (whole tiles of 16, 32 or 64 pixels, flat (sample, pixel) tiles, blocks that
+    share a tile's k steps) on sixteen seeded random shapes whose filters fill 64-row blocks, against the two layers on
+    the oracle; the second pass forbids sharing, so the same shapes also run as one block per tile."""
+    import mi355tensor as mt
+    rng = np.random.default_rng(77)
+    try:
+        mt.set_option("upconv_walk", 1)
+        for n in range(16):
+            KA = 64 * int(rng.integers(1, 3))
+            C = 16 * int(rng.integers(1, 9))
+            H, Wd = int(rng.integers(1, 10)), int(rng.integers(1, 10))
+            B = int(rng.integers(1, 9))
+            image = U(100 + n, B, C, H, Wd)
+            kernel, bias = Nrm(200 + n, 1, 1, KA, C * 9, std=float(np.sqrt(2.0 / (C * 9)))), U(300 + n, 1, KA, 1, 1) * 0.3
+            want = oracle.apply_func(oracle.forward_convolution(oracle.upsampling(image, 2, 2), kernel, bias, 3, 3, C, KA, 1, 1, 1, 1), "leaky_relu")
+            for share in (1, 0):
+                mt.set_option("upconv_split", share)
+                got = gpu.upsampling_convolution(image, kernel, bias, 3, C, KA, func="leaky_relu")
+                assert np.allclose(got, want, rtol=1e-5, atol=1e-5), (n, B, C, H, Wd, KA, share, float(np.abs(got - want).max()))
+    finally:
+        mt.set_option("upconv_walk", 512)
+        mt.set_option("upconv_split", 1)
+
+
 def test_upsampling_convolution_other_geometries(gpu, oracle, path):
     """Anything but (x2, 3x3, stride 1, padding 1) runs as the two layers one after the other inside the library."""
     image = U(1, 2, 6, 5, 4)
