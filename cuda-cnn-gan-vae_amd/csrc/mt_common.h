@@ -57,7 +57,18 @@ void count_driver_allocation();  // every hipMalloc of the library is counted (m
 // that writes device memory reports the range here (so does mt_invalidate for writers outside the library); copies
 // made from an overlapping range are then made again on their next use.
 void note_write(const void *p, size_t bytes);
+int add_sum_w_pair(float *out1, const float *r1, size_t S1, float *out2, const float *r2, size_t S2, uint32_t W);  // two batch sums, one launch
 int set_pack_cache(int on);
+int set_adam_vec(int v);      // mt_adam_many updates four elements per thread: 1 (default) in the tiles that also write a re-ordered copy, 2 wherever the tensors allow, 0 never (measurements only)
+int set_pack_refresh(int v);  // 1 (default): mt_adam_many keeps the re-ordered copies of 4x4 stride-2 transposed-convolution weights current; 0: never
+struct PackRefresh {          // where mt_adam_many writes such a copy: tap t of (channel co, filter ci) in phase f at packed[begin[f] + co*co_stride + ci*ci_stride + t]
+  float *packed;
+  uint32_t ker_ld, co_stride, ci_stride, begin[4];
+  uint8_t phase_of[4];
+  size_t entry;
+};
+bool pack_refresh_find(const float *kernel, size_t floats, PackRefresh *r);
+void pack_refresh_commit(const PackRefresh &r, const mt_tensor *const *weight, const mt_tensor *const *m, const mt_tensor *const *v, uint32_t count);
 bool pack_cache_info(const char *name, int64_t *value);
 int static_scratch_setup();  // looks up the device address of the fixed scratch array for the current device
 

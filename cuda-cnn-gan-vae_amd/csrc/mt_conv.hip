@@ -79,8 +79,17 @@ struct PackKey {
     return true;
   }
 };
+// What an optimiser step needs to write the re-ordered copy of a 4x4 stride-2 transposed convolution itself (see
+// mt::pack_refresh_find): where the sub-kernel of each phase starts behind the bias sums, and which phase owns which
+// parity of a flipped coefficient.
+struct PackK4S2 {
+  bool on = false;
+  uint32_t sums = 0, CO = 0, CI = 0, co_stride = 0, ci_stride = 0, begin[4] = {0, 0, 0, 0};  // coefficient (co, ci, tap) of phase f: begin[f] + co*co_stride + ci*ci_stride + tap
+  uint8_t phase_of[4] = {0, 0, 0, 0};  // [(3 - ky) % 2 * 2 + (3 - kx) % 2]
+};
 struct PackEntry {
   PackKey key;
+  PackK4S2 k4s2;
   float *buf = nullptr;
   size_t floats = 0;
   bool valid = false;
@@ -90,7 +99,8 @@ struct PackEntry {
 constexpr size_t PACK_MAX_ENTRIES = 64, PACK_MAX_BYTES = (size_t)512 << 20;
 std::vector<PackEntry> g_packs;
 bool g_pack_cache = true;
-uint64_t g_pack_clock = 0, g_pack_hits = 0, g_pack_made = 0;
+uint64_t g_pack_clock = 0, g_pack_hits = 0, g_pack_made = 0, g_pack_refreshed = 0;
+int g_pack_refresh = 1;  // 1: mt_adam_many writes the re-ordered copies of the weights it updates (4x4 stride-2 transposed convolutions), 0: never
 // Memory that calls recorded into a graph write.  A replay changes it without the library seeing a call, so copies made
 // from such memory are never trusted: they are made again on every use (training weights that a recorded step updates).
 std::vector<std::pair<uintptr_t, uintptr_t>> g_graph_written;
@@ -335,15 +345,6 @@ __global__ __launch_bounds__(256) void dbias_finish_kernel(float *dbias, const f
   float s = 0.f;
   for (uint32_t c = 0; c < chunks; c++) s += partial[f * chunks + c];
   dbias[f] += s;
-}
-// The same with one wavefront per filter: many partial sums per filter (the groups of the walking weight-gradient kernel).
-__global__ __launch_bounds__(256) void dbias_finish_wave_kernel(float *dbias, const float *partial, uint32_t KA, uint32_t chunks) {
-  const uint32_t f = blockIdx.x * 4 + threadIdx.x / 64, lane = threadIdx.x % 64;
-  if (f >= KA) return;
-  float s = 0.f;
-  for (uint32_t c = lane; c < chunks; c += 64) s += partial[f * chunks + c];
-  s = mt::wave_sum(s);
-  if (lane == 0) dbias[f] += s;
 }
 // chunks of the batch per filter: enough blocks to fill the device, each with at least a few thousand values
 uint32_t dbias_chunks(uint32_t B, uint32_t KA, uint32_t DHW) {
@@ -1655,10 +1656,24 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     walk_tm = mt::igemm::walk_tm() == 2 && kz % 128 == 0 ? 2u : 1u;
     walks = covered == OHW && tconv_walk_plan(walk, (uint32_t)mt::igemm::walk_blocks(), walk_tm);
   }
+  bool k4s2 = kx == 4 && ky == 4 && sx == 2 && sy == 2 && args.nphase == 4 && kernel->x % 4 == 0 && ((uintptr_t)kernel->p & 15u) == 0 && kz <= 65534;
+  for (uint32_t f = 0; k4s2 && f < 4; f++) k4s2 = pa.ph[f].ty == 2 && pa.ph[f].tx == 2 && pa.ph[f].ci_stride % 4 == 0 && pa.ph[f].co_stride % 4 == 0;
+  if (k4s2 && kernel->x == (uint32_t)kz * 16u) {
+    // an optimiser step may keep this copy current: tell the cache entry (if the copy lives in one) how it is laid out
+    PackK4S2 info;
+    info.on = true; info.sums = (uint32_t)sums; info.CO = (uint32_t)kz; info.CI = ka; info.co_stride = pa.ph[0].co_stride; info.ci_stride = pa.ph[0].ci_stride;
+    uint32_t seen = 0;
+    for (uint32_t f = 0; f < 4; f++) {
+      info.begin[f] = pa.ph[f].begin;
+      info.on = info.on && (uint32_t)pa.ph[f].ky0 < 2u && (uint32_t)pa.ph[f].kx0 < 2u && pa.ph[f].co_stride == info.co_stride && pa.ph[f].ci_stride == info.ci_stride;
+      if (info.on) { info.phase_of[pa.ph[f].ky0 * 2 + pa.ph[f].kx0] = (uint8_t)f; seen |= 1u << (pa.ph[f].ky0 * 2 + pa.ph[f].kx0); }
+    }
+    if (info.on && seen == 15u)
+      for (PackEntry &e : g_packs)
+        if (e.buf == ws) e.k4s2 = info;
+  }
   if (fresh) {
     mt::ProfileScope prof("tconv_prepare");
-    bool k4s2 = kx == 4 && ky == 4 && sx == 2 && sy == 2 && args.nphase == 4 && kernel->x % 4 == 0 && ((uintptr_t)kernel->p & 15u) == 0 && kz <= 65534;
-    for (uint32_t f = 0; k4s2 && f < 4; f++) k4s2 = pa.ph[f].ty == 2 && pa.ph[f].tx == 2 && pa.ph[f].ci_stride % 4 == 0 && pa.ph[f].co_stride % 4 == 0;
     if (k4s2) {
       tconv_prepare_k4s2_kernel<<<dim3(cdiv(ka, 256), kz + 1), 256, 0, mt::stream()>>>(packed, ws, kernel->p, bias->p, pa);
     } else {
@@ -1897,11 +1912,7 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
       if ((rc = mt::igemm::launch_wgrad_walk(name, wa))) return rc;
     }
     g_wgrad_walk_launches++;
-    mt_tensor pt{partial, wa.groups, 1, ka, ncol}, flat{dk->p, 1, 1, ka, ncol};
-    if ((rc = mt_add_sum_w(&flat, &flat, &pt, 1.f, 1.f))) return rc;
-    dbias_finish_wave_kernel<<<cdiv(ka, 4), 256, 0, mt::stream()>>>(db->p, dbias_partial, ka, wa.groups);
-    MT_LAUNCH_CHECK(name);
-    return MT_OK;
+    return mt::add_sum_w_pair(dk->p, partial, (size_t)ka * ncol, db->p, dbias_partial, ka, wa.groups);  // the groups in order, one launch for both
   }
   SrcRowK<true> a{};
   a.p = delta->p; a.ld = DHW; a.R = ka; a.K = per * DHW; a.seg = DHW; a.seg_stride = (uint32_t)sample_delta;
@@ -2119,6 +2130,40 @@ void note_write(const void *p, size_t bytes) {
     if (overlaps(e.key.kernel, key_floats(e.key.kernel_dims), lo, hi) || overlaps(e.key.bias, key_floats(e.key.bias_dims), lo, hi)) e.valid = false;
   }
 }
+// The kept re-ordered copy of the weights at `kernel` that mt_adam_many can write while it updates them, if there is one:
+// a 4x4 stride-2 transposed convolution's, not while a graph is recorded (a replay would write a copy that the cache
+// cannot vouch for) and not for weights that a recorded graph writes.
+bool pack_refresh_find(const float *kernel, size_t floats, PackRefresh *r) {
+  if (!g_pack_cache || !g_pack_refresh || capturing()) return false;
+  for (size_t i = 0; i < g_packs.size(); i++) {
+    const PackEntry &e = g_packs[i];
+    if (e.key.kind != 0 || !e.valid || !e.k4s2.on || e.key.kernel != kernel || key_floats(e.key.kernel_dims) != floats || floats != (size_t)e.k4s2.CI * e.k4s2.CO * 16u) continue;
+    if (written_by_a_graph(e.key)) continue;
+    r->packed = e.buf + e.k4s2.sums; r->ker_ld = e.k4s2.CO * 16u; r->co_stride = e.k4s2.co_stride; r->ci_stride = e.k4s2.ci_stride; r->entry = i;
+    for (int f = 0; f < 4; f++) { r->begin[f] = e.k4s2.begin[f]; r->phase_of[f] = e.k4s2.phase_of[f]; }
+    return true;
+  }
+  return false;
+}
+// After the launch that wrote the copy (and after the write to the weights was reported, which marked the entry stale):
+// the copy is current again unless the same step also wrote the bias whose sums the entry holds.
+void pack_refresh_commit(const PackRefresh &r, const mt_tensor *const *weight, const mt_tensor *const *m, const mt_tensor *const *v, uint32_t count) {
+  if (r.entry >= g_packs.size()) return;
+  PackEntry &e = g_packs[r.entry];
+  for (const mt_tensor *const *written : {weight, m, v})
+    for (uint32_t i = 0; i < count; i++) {
+      const uintptr_t lo = (uintptr_t)written[i]->p, hi = lo + mt::count(written[i]) * sizeof(float);
+      if (overlaps(e.key.bias, key_floats(e.key.bias_dims), lo, hi)) return;
+      if (written != weight && overlaps(e.key.kernel, key_floats(e.key.kernel_dims), lo, hi)) return;  // (moments that alias the weights: nothing to vouch for)
+    }
+  e.valid = true;
+  g_pack_refreshed++;
+}
+int set_pack_refresh(int v) {
+  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "pack_refresh must be 0 or 1");
+  g_pack_refresh = v;
+  return MT_OK;
+}
 int set_pack_cache(int on) {
   if (on != 0 && on != 1) return fail(MT_E_ARGUMENT, "pack_cache must be 0 (re-order the weights on every call) or 1 (keep them between calls)");
   g_pack_cache = on != 0;
@@ -2133,6 +2178,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "pack_cache_valid") == 0) { int64_t n = 0; for (const PackEntry &e : g_packs) n += e.valid; *value = n; return true; }
   if (strcmp(name, "pack_cache_hits") == 0) { *value = (int64_t)g_pack_hits; return true; }
   if (strcmp(name, "pack_cache_made") == 0) { *value = (int64_t)g_pack_made; return true; }
+  if (strcmp(name, "pack_cache_refreshed") == 0) { *value = (int64_t)g_pack_refreshed; return true; }
   if (strcmp(name, "pack_cache_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_packs) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
   if (strcmp(name, "pack_cache_spare_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_pack_spare) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
   if (strcmp(name, "graph_written_ranges") == 0) { *value = (int64_t)g_graph_written.size(); return true; }

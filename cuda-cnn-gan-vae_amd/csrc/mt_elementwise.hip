@@ -195,13 +195,13 @@ __global__ __launch_bounds__(EW_THREADS) void summ_xy_kernel(float *out, const f
 // group of columns, no exchange at all: tensors with few samples and many columns (two or eight partial weight gradients);
 // RB = 4 gives 64 slices: few columns and many samples (hundreds of partial gradients of a first layer).
 template <int RB>
-__global__ __launch_bounds__(EW_THREADS) void add_sum_w_vec_kernel(float *out, uint32_t Wout, const float *L, uint32_t Wl, const float *R, uint32_t Wr,
-                                                                   uint32_t S, float ls, float rs) {
+__device__ __forceinline__ void add_sum_w_vec_body(uint32_t block, float *out, uint32_t Wout, const float *L, uint32_t Wl, const float *R, uint32_t Wr,
+                                                   uint32_t S, float ls, float rs) {
   constexpr int WS = EW_THREADS / RB, WAVES = EW_THREADS / 64;
   constexpr int IN_WAVE = RB >= 64 ? 1 : 64 / RB;   // slices inside one wavefront
   __shared__ float4 part[2][WS > 1 ? WAVES : 1][RB < 64 ? RB : 64];
   const int rl = threadIdx.x % RB, ws = threadIdx.x / RB;
-  const uint32_t r = (blockIdx.x * RB + rl) * 4;
+  const uint32_t r = (block * RB + rl) * 4;
   float4 sl = make_float4(0.f, 0.f, 0.f, 0.f), sr = sl;
   if (r < S) {
 #pragma unroll 4
@@ -244,6 +244,25 @@ __global__ __launch_bounds__(EW_THREADS) void add_sum_w_vec_kernel(float *out, u
     *reinterpret_cast<float4 *>(out + r) = o;
   }
   for (uint32_t w = 1 + ws; w < Wout; w += WS) *reinterpret_cast<float4 *>(out + (size_t)w * S + r) = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+template <int RB>
+__global__ __launch_bounds__(EW_THREADS) void add_sum_w_vec_kernel(float *out, uint32_t Wout, const float *L, uint32_t Wl, const float *R, uint32_t Wr,
+                                                                   uint32_t S, float ls, float rs) {
+  add_sum_w_vec_body<RB>(blockIdx.x, out, Wout, L, Wl, R, Wr, S, ls, rs);
+}
+// Two sums in one launch, out[i] += sum over w of R[w][i] for each: the first `blocks` blocks own the first one.  (The
+// partial weight gradients of a layer and the partial sums of its bias gradient: the second is too small for a launch of
+// its own to be worth its start.)
+struct SumJob {
+  float *out;
+  const float *R;
+  uint32_t S, blocks;
+};
+template <int RB>
+__global__ __launch_bounds__(EW_THREADS) void add_sum_w_pair_kernel(SumJob a, SumJob b, uint32_t W) {
+  const bool first = blockIdx.x < a.blocks;  // (uniform over the block: the barrier inside the body is reached by all of its threads)
+  const SumJob &j = first ? a : b;
+  add_sum_w_vec_body<RB>(first ? blockIdx.x : blockIdx.x - a.blocks, j.out, 1, j.out, 1, j.R, W, j.S, 1.f, 1.f);
 }
 
 __global__ __launch_bounds__(EW_THREADS) void add_bias4_kernel(float *t, const float *bias, uint32_t Wb, uint32_t Z, uint32_t YX4, uint32_t rows) {
@@ -550,18 +569,37 @@ struct AdamStep {
   float batch;
   double speed, beta1, beta2, epsilon, c1, c2;
 };
-__device__ __forceinline__ void adam_update(float *weight, const float *dweight, float *m, float *v, size_t i, const AdamStep &a) {
-  const float batch = a.batch;
+// one element: the new weight; mi and vi are updated in place
+__device__ __forceinline__ float adam_element(float w, float dw, float &mi, float &vi, const AdamStep &a) {
   const double speed = a.speed, beta1 = a.beta1, beta2 = a.beta2, epsilon = a.epsilon, c1 = a.c1, c2 = a.c2;
-  float dw = dweight[i] / batch, mi = m[i], vi = v[i];
+  dw = dw / a.batch;
   mi = (float)(beta1 * (double)mi + (1.0 - beta1) * (double)dw);
   vi = (float)(beta2 * (double)vi + (1.0 - beta2) * (double)dw * (double)dw);
   float mc = (float)((double)mi / c1);  // c1 = 1 - beta1^iteration
   float vc = (float)((double)vi / c2);
   dw = (float)(speed * (double)mc / ((double)sqrtf(vc) + epsilon));
+  return w - dw;
+}
+__device__ __forceinline__ float adam_update(float *weight, const float *dweight, float *m, float *v, size_t i, const AdamStep &a) {
+  float mi = m[i], vi = v[i];
+  const float w = adam_element(weight[i], dweight[i], mi, vi, a);
   m[i] = mi;
   v[i] = vi;
-  weight[i] = weight[i] - dw;
+  weight[i] = w;
+  return w;
+}
+// four consecutive elements (16-byte aligned tensors), the same arithmetic per element
+__device__ __forceinline__ float4 adam_update4(float *weight, const float *dweight, float *m, float *v, size_t i4, const AdamStep &a) {
+  float4 w = reinterpret_cast<const float4 *>(weight)[i4], mi = reinterpret_cast<const float4 *>(m)[i4], vi = reinterpret_cast<const float4 *>(v)[i4];
+  const float4 dw = reinterpret_cast<const float4 *>(dweight)[i4];
+  w.x = adam_element(w.x, dw.x, mi.x, vi.x, a);
+  w.y = adam_element(w.y, dw.y, mi.y, vi.y, a);
+  w.z = adam_element(w.z, dw.z, mi.z, vi.z, a);
+  w.w = adam_element(w.w, dw.w, mi.w, vi.w, a);
+  reinterpret_cast<float4 *>(m)[i4] = mi;
+  reinterpret_cast<float4 *>(v)[i4] = vi;
+  reinterpret_cast<float4 *>(weight)[i4] = w;
+  return w;
 }
 __global__ __launch_bounds__(EW_THREADS) void adam_kernel(float *weight, const float *dweight, float *m, float *v, size_t n, AdamStep a) {
   size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
@@ -582,6 +620,7 @@ struct ManyAdam {
   float *m[MANY], *v[MANY];
   size_t n[MANY];
   uint32_t first_block[MANY + 1];
+  uint32_t vec;  // bit t: tensor t is updated four elements at a time (a multiple of four elements, 16-byte aligned)
 };
 template <class T>
 __device__ __forceinline__ uint32_t many_owner(const T &a, uint32_t count) {
@@ -595,11 +634,89 @@ __global__ __launch_bounds__(EW_THREADS) void fill_many_kernel(ManyFill a, uint3
   float *p = a.p[t];
   for (size_t i = (size_t)(blockIdx.x - a.first_block[t]) * EW_THREADS + threadIdx.x; i < a.n[t]; i += stride) p[i] = value;
 }
-__global__ __launch_bounds__(EW_THREADS) void adam_many_kernel(ManyAdam a, uint32_t count, AdamStep step) {
-  const uint32_t t = many_owner(a, count);
+// Weights whose re-ordered copy for the transposed convolution 4x4 stride 2 (the input gradient of a 4x4 stride-2
+// convolution layer) is kept between calls: the step writes the new value to its place in the copy as well, so the next
+// backward pass finds it current.  Coefficient (ky, kx) of filter ci, channel co is tap ((3-ky)/2, (3-kx)/2) of the phase
+// that owns the parities of (3-ky, 3-kx); a phase's sub-kernel is [co][ci*4 + tap].
+constexpr int MANY_PACKS = 8;
+int g_adam_vec = 1;  // 1: mt_adam_many updates four elements per thread in the tiles that also write a re-ordered copy; 2: wherever the tensors allow; 0: never (measurements only)
+struct AdamPack {
+  float *packed;
+  uint32_t ker_ld, co_stride, ci_stride, begin[4];
+  uint8_t phase_of[4];
+  uint32_t tiles_co;  // 0: element by element; else tiles of 16 filters x 16 channels, this many along the channels
+};
+struct ManyAdamPacks {
+  int8_t slot[MANY];  // -1: no copy to keep
+  AdamPack pack[MANY_PACKS];
+};
+__device__ __forceinline__ void adam_many_plain(const ManyAdam &a, uint32_t t, const AdamStep &step) {
   const size_t stride = (size_t)(a.first_block[t + 1] - a.first_block[t]) * EW_THREADS;
-  for (size_t i = (size_t)(blockIdx.x - a.first_block[t]) * EW_THREADS + threadIdx.x; i < a.n[t]; i += stride)
-    adam_update(a.weight[t], a.dweight[t], a.m[t], a.v[t], i, step);
+  const size_t first = (size_t)(blockIdx.x - a.first_block[t]) * EW_THREADS + threadIdx.x;
+  if (a.vec >> t & 1u) {
+    for (size_t i = first; i < a.n[t] / 4; i += stride) adam_update4(a.weight[t], a.dweight[t], a.m[t], a.v[t], i, step);
+  } else {
+    for (size_t i = first; i < a.n[t]; i += stride) adam_update(a.weight[t], a.dweight[t], a.m[t], a.v[t], i, step);
+  }
+}
+__global__ __launch_bounds__(EW_THREADS) void adam_many_kernel(ManyAdam a, uint32_t count, AdamStep step) {
+  adam_many_plain(a, many_owner(a, count), step);
+}
+__global__ __launch_bounds__(EW_THREADS) void adam_many_packs_kernel(ManyAdam a, ManyAdamPacks packs, uint32_t count, AdamStep step) {
+  const uint32_t t = many_owner(a, count);
+  const int slot = packs.slot[t];
+  if (slot < 0) {
+    adam_many_plain(a, t, step);
+    return;
+  }
+  const AdamPack &p = packs.pack[slot];
+  const uint32_t begin[4] = {p.begin[0], p.begin[1], p.begin[2], p.begin[3]};
+  const uint32_t phase_of = (uint32_t)p.phase_of[0] | (uint32_t)p.phase_of[1] << 8 | (uint32_t)p.phase_of[2] << 16 | (uint32_t)p.phase_of[3] << 24;
+  if (p.tiles_co) {
+    // Tiles of 16 filters x 16 channels (16 rows of 256 consecutive weights): updated with 128-bit accesses along the
+    // rows, the new values staged in LDS, then written to the copy as the 256 contiguous bytes that sixteen filters fill
+    // of a (phase, channel) row -- whole lines instead of 16-byte pieces from blocks that run at different times.
+    constexpr int ROW = 256 + 1;
+    __shared__ float tile[16 * ROW];
+    const uint32_t tiles = (uint32_t)(a.n[t] / 4096), blocks = a.first_block[t + 1] - a.first_block[t];
+    const uint32_t tid = threadIdx.x, r4 = tid / 64, c4 = tid % 64;   // row within a pass of four rows, float4 within the row
+    for (uint32_t tl = blockIdx.x - a.first_block[t]; tl < tiles; tl += blocks) {
+      const uint32_t ci0 = (tl / p.tiles_co) * 16u, co0 = (tl % p.tiles_co) * 16u;
+#pragma unroll
+      for (int pass = 0; pass < 4; pass++) {
+        const uint32_t r = pass * 4 + r4;
+        const size_t i4 = ((size_t)(ci0 + r) * p.ker_ld + co0 * 16u) / 4 + c4;
+        const float4 w = adam_update4(a.weight[t], a.dweight[t], a.m[t], a.v[t], i4, step);
+        float *d = tile + r * ROW + c4 * 4;
+        d[0] = w.x; d[1] = w.y; d[2] = w.z; d[3] = w.w;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < 4; j++) {   // j = parities of the flipped coefficient: (ky' % 2, kx' % 2)
+        const uint32_t ci = tid % 16, co = tid / 16, f = (phase_of >> (8u * j)) & 255u;
+        const uint32_t b = f == 0 ? begin[0] : f == 1 ? begin[1] : f == 2 ? begin[2] : begin[3];
+        const float *src = tile + ci * ROW + co * 16;
+        float4 q;   // taps (ty, tx): coefficient (3 - (ky0 + 2 ty), 3 - (kx0 + 2 tx)) with ky0 = j / 2, kx0 = j % 2
+        const uint32_t ky0 = (uint32_t)j >> 1, kx0 = (uint32_t)j & 1u;
+        q.x = src[(3 - ky0) * 4 + (3 - kx0)];
+        q.y = src[(3 - ky0) * 4 + (1 - kx0)];
+        q.z = src[(1 - ky0) * 4 + (3 - kx0)];
+        q.w = src[(1 - ky0) * 4 + (1 - kx0)];
+        *reinterpret_cast<float4 *>(p.packed + (size_t)b + (size_t)(co0 + co) * p.co_stride + (ci0 + ci) * 4u) = q;
+      }
+      __syncthreads();
+    }
+    return;
+  }
+  const size_t stride = (size_t)(a.first_block[t + 1] - a.first_block[t]) * EW_THREADS;
+  for (size_t i = (size_t)(blockIdx.x - a.first_block[t]) * EW_THREADS + threadIdx.x; i < a.n[t]; i += stride) {
+    const float w = adam_update(a.weight[t], a.dweight[t], a.m[t], a.v[t], i, step);
+    const uint32_t e = (uint32_t)i, ci = e / p.ker_ld, col = e - ci * p.ker_ld, co = col >> 4, tap = col & 15u;
+    const uint32_t ky = 3u - (tap >> 2), kx = 3u - (tap & 3u);
+    const uint32_t f = (phase_of >> (8u * ((ky & 1u) * 2u + (kx & 1u)))) & 255u;
+    const uint32_t b = f == 0 ? begin[0] : f == 1 ? begin[1] : f == 2 ? begin[2] : begin[3];
+    p.packed[(size_t)b + (size_t)co * p.co_stride + (size_t)ci * p.ci_stride + (ky >> 1) * 2u + (kx >> 1)] = w;
+  }
 }
 
 // ---- batch normalisation over the batch axis, statistics per element (z,y,x) --------------------------------------
@@ -1175,6 +1292,45 @@ static int bn_backward_any(const mt_tensor *error, const mt_tensor *dgamma, cons
                            const mt_tensor *beta, const mt_tensor *xhat, const mt_tensor *ivar, int func, const mt_tensor *keep_dxhat, const mt_tensor *keep_s1,
                            const mt_tensor *keep_s2, const mt_tensor *keep_front = nullptr);
 
+namespace mt {
+int set_adam_vec(int v) {
+  if (v < 0 || v > 2) return fail(MT_E_ARGUMENT, "adam_vec must be 0, 1 or 2");
+  g_adam_vec = v;
+  return MT_OK;
+}
+// out1[i] += sum over w of r1[w][i] and out2[i] += sum over w of r2[w][i], both over the same W: one launch where the
+// 128-bit kernel takes both (sizes that are multiples of four, aligned), else two calls of mt_add_sum_w.
+int add_sum_w_pair(float *out1, const float *r1, size_t S1, float *out2, const float *r2, size_t S2, uint32_t W) {
+  if (S1 == 0 || S2 == 0 || W == 0) return fail(MT_E_ARGUMENT, "add_sum_w_pair: empty operand");
+  if (S1 % 4 || S2 % 4 || S1 < 1024 || S1 > 0xffffffffu || S2 > 0xffffffffu || !aligned16(out1) || !aligned16(r1) || !aligned16(out2) || !aligned16(r2)) {
+    const mt_tensor o1{out1, 1, 1, 1, (uint32_t)S1}, p1{const_cast<float *>(r1), W, 1, 1, (uint32_t)S1};
+    const mt_tensor o2{out2, 1, 1, 1, (uint32_t)S2}, p2{const_cast<float *>(r2), W, 1, 1, (uint32_t)S2};
+    if (S1 > 0xffffffffu || S2 > 0xffffffffu) return fail(MT_E_ARGUMENT, "add_sum_w_pair: more than 2^32 elements");
+    const int rc = mt_add_sum_w(&o1, &o1, &p1, 1.f, 1.f);
+    return rc ? rc : mt_add_sum_w(&o2, &o2, &p2, 1.f, 1.f);
+  }
+  note_write(out1, S1 * sizeof(float));
+  note_write(out2, S2 * sizeof(float));
+  char shape[64];
+  if (profiling()) snprintf(shape, sizeof shape, "S %zu and %zu W 1 + %u", S1, S2, W);
+  ProfileScope prof(profiling() ? intern_label("mt_add_sum_w", shape) : "mt_add_sum_w");
+  const size_t cols = S1 / 4;
+  int rb = cols / 256 >= 1024 && W <= 4 ? 256 : cols / 32 >= 256 ? 32 : cols / 8 >= 256 ? 8 : 4;   // as in mt_add_sum_w, chosen for the first sum
+  if (rb == 4 && W < 64) rb = 8;
+  if (rb == 8 && W < 32) rb = 32;
+  if (rb == 32 && W < 8 && cols / 256 >= 64) rb = 256;
+  SumJob a{out1, r1, (uint32_t)S1, cdiv(cols, (size_t)rb)}, b{out2, r2, (uint32_t)S2, cdiv(S2 / 4, (size_t)rb)};
+  const uint32_t grid = a.blocks + b.blocks;
+  hipStream_t st = stream();
+  if (rb == 256) add_sum_w_pair_kernel<256><<<grid, EW_THREADS, 0, st>>>(a, b, W);
+  else if (rb == 32) add_sum_w_pair_kernel<32><<<grid, EW_THREADS, 0, st>>>(a, b, W);
+  else if (rb == 8) add_sum_w_pair_kernel<8><<<grid, EW_THREADS, 0, st>>>(a, b, W);
+  else add_sum_w_pair_kernel<4><<<grid, EW_THREADS, 0, st>>>(a, b, W);
+  MT_LAUNCH_CHECK("mt_add_sum_w");
+  return MT_OK;
+}
+}  // namespace mt
+
 extern "C" {
 
 int mt_fill(const mt_tensor *out, float value) {
@@ -1500,8 +1656,12 @@ int mt_fill_many(uint32_t count, const mt_tensor *const *tensors, float value) {
 int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor *const *dweight, const mt_tensor *const *m, const mt_tensor *const *v,
                  uint32_t batch_size, double speed, double beta1, double beta2, double epsilon, double iteration) {
   if (count && (weight == nullptr || dweight == nullptr || m == nullptr || v == nullptr)) return mt::fail(MT_E_ARGUMENT, "mt_adam_many: null list");
+  mt::PackRefresh found[MANY_PACKS];
+  uint32_t found_for[MANY_PACKS], nfound = 0;
   for (uint32_t i = 0; i < count; i++) {
     if (mt::bad(weight[i]) || mt::bad(dweight[i]) || mt::bad(m[i]) || mt::bad(v[i])) return mt::fail(MT_E_ARGUMENT, "mt_adam_many: null tensor (entry %u)", i);
+    // (looked up before the write is reported: only a copy that is current now can be kept current by this step)
+    if (nfound < (uint32_t)MANY_PACKS && mt::count(weight[i]) <= 0xffffffffu && mt::pack_refresh_find(weight[i]->p, mt::count(weight[i]), &found[nfound])) found_for[nfound++] = i;
     mt::note_write(weight[i]);
     mt::note_write(m[i]);
     mt::note_write(v[i]);
@@ -1512,20 +1672,44 @@ int mt_adam_many(uint32_t count, const mt_tensor *const *weight, const mt_tensor
   const AdamStep step{(float)batch_size, speed, beta1, beta2, epsilon, 1.0 - pow(beta1, iteration), 1.0 - pow(beta2, iteration)};
   for (uint32_t first = 0; first < count;) {
     ManyAdam a{};
-    uint32_t used = 0;
+    ManyAdamPacks packs{};
+    uint32_t refresh[MANY_PACKS];
+    uint32_t used = 0, kept = 0;
     for (; first < count && used < (uint32_t)MANY; first++) {
       const size_t n = mt::count(weight[first]);
       if (n == 0) continue;
-      unsigned blocks = cdiv(n, EW_THREADS);
-      if (blocks > 4096u) blocks = 4096u;
+      const bool vec = g_adam_vec && n % 4 == 0 && aligned16(weight[first]->p) && aligned16(dweight[first]->p) && aligned16(m[first]->p) && aligned16(v[first]->p);
+      unsigned blocks = cdiv(vec ? n / 4 : n, EW_THREADS);
       a.weight[used] = weight[first]->p; a.dweight[used] = dweight[first]->p; a.m[used] = m[first]->p; a.v[used] = v[first]->p;
-      a.n[used] = n; a.first_block[used + 1] = a.first_block[used] + blocks;
+      a.n[used] = n;
+      if (vec) a.vec |= 1u << used;
+      packs.slot[used] = -1;
+      uint32_t k = 0;
+      while (k < nfound && found_for[k] != first) k++;
+      if (k < nfound) {
+        const mt::PackRefresh &r = found[k];
+        refresh[kept] = k;
+        AdamPack &p = packs.pack[kept];
+        p.packed = r.packed; p.ker_ld = r.ker_ld; p.co_stride = r.co_stride; p.ci_stride = r.ci_stride;
+        for (int f = 0; f < 4; f++) { p.begin[f] = r.begin[f]; p.phase_of[f] = r.phase_of[f]; }
+        const uint32_t CO = r.ker_ld / 16u, CI = (uint32_t)(n / r.ker_ld);
+        p.tiles_co = vec && CO % 16 == 0 && CI % 16 == 0 && r.ci_stride == 4 && r.co_stride % 4 == 0 && aligned16(r.packed) ? CO / 16u : 0u;
+        if (p.tiles_co) blocks = (unsigned)(n / 4096);
+        else { blocks = cdiv(n, EW_THREADS); a.vec &= ~(1u << used); }
+        packs.slot[used] = (int8_t)kept++;
+      } else if (vec && g_adam_vec == 1) {
+        blocks = cdiv(n, EW_THREADS); a.vec &= ~(1u << used);
+      }
+      if (blocks > 4096u) blocks = 4096u;
+      a.first_block[used + 1] = a.first_block[used] + blocks;
       used++;
     }
     if (used == 0) continue;
     mt::ProfileScope prof("mt_adam_many");
-    adam_many_kernel<<<a.first_block[used], EW_THREADS, 0, mt::stream()>>>(a, used, step);
+    if (kept) adam_many_packs_kernel<<<a.first_block[used], EW_THREADS, 0, mt::stream()>>>(a, packs, used, step);
+    else adam_many_kernel<<<a.first_block[used], EW_THREADS, 0, mt::stream()>>>(a, used, step);
     MT_LAUNCH_CHECK("mt_adam_many");
+    for (uint32_t k = 0; k < kept; k++) mt::pack_refresh_commit(found[refresh[k]], weight, m, v, count);
   }
   return MT_OK;
 }

@@ -254,6 +254,8 @@ int mt_set_option(const char *name, int value) {
   if (name && strcmp(name, "wgrad_walk") == 0) return mt::set_wgrad_walk(value);
   if (name && strcmp(name, "upconv_walk") == 0) return mt::set_upconv_walk(value);
   if (name && strcmp(name, "upconv_split") == 0) return mt::set_upconv_split(value);
+  if (name && strcmp(name, "pack_refresh") == 0) return mt::set_pack_refresh(value);
+  if (name && strcmp(name, "adam_vec") == 0) return mt::set_adam_vec(value);
   if (name && strcmp(name, "nontemporal") == 0) return mt::set_nontemporal(value);
   if (name && strcmp(name, "image_strip") == 0) return mt::set_image_strip(value);
   if (name && strcmp(name, "first_layer") == 0) return mt::set_first_layer(value);

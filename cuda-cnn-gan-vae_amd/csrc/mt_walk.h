@@ -394,7 +394,7 @@ struct WgradWalkArgs {
   const float *delta;   // [B][M][OH][OW]
   const float *image;   // [B][C][H][W]
   float *partial;       // [groups][M][N]
-  float *bias_partial;  // [M][groups]: the groups' sums of delta per filter (the bias gradient), or null
+  float *bias_partial;  // [groups][M]: the groups' sums of delta per filter (the bias gradient), or null
   uint32_t M, N, C, H, W, OH, OW, KY, KX;
   int32_t sy, sx, py, px;
   uint32_t steps, groups, tiles_m, tiles_n, fair;   // steps: k steps of a group (of B * OH * OW / 16 in all)
@@ -564,7 +564,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   if (row_sums) {  // four neighbouring lanes hold the four quarters of a row's k steps
     row_sum += __shfl_xor(row_sum, 1, 64);
     row_sum += __shfl_xor(row_sum, 2, 64);
-    if ((tid & 3) == 0) a.bias_partial[(size_t)(m0 + a_row) * a.groups + g] = row_sum;
+    if ((tid & 3) == 0) a.bias_partial[(size_t)g * a.M + (m0 + a_row)] = row_sum;
   }
 }
 

@@ -117,6 +117,9 @@ int mt_timer_destroy(void *timer);
  *   "upconv_split"   1 (default) where that kernel would get fewer than 512 blocks (small images, many channels), two or four
  *                    blocks share a tile's sum over (channel, tap) and a second kernel adds their parts, the bias and the function /
  *                    0 never
+ *   "pack_refresh"   1 (default) mt_adam_many writes each new weight also into the kept re-ordered copy that the 4x4 stride-2
+ *                    transposed convolution (the input gradient of a 4x4 stride-2 convolution layer) made of those weights, so a
+ *                    training loop re-orders nothing per step; not while a graph is recorded / 0 the step only reports its write
  *   "first_layer"    1 (default) forward convolutions of 3-channel images (3x3, 4x4, 5x5 kernels to 32 or 64 filters) keep the
  *                    input patch in LDS and the weights in registers wherever the shape allows / 0 never
  *   "walk_blocks"    blocks wanted per launch of the walking kernel (default 1024)
@@ -141,6 +144,7 @@ int mt_set_option(const char *name, int value);
  *   "retired_workspaces"                                   outgrown workspaces that a recorded graph may still use
  *   "pack_cache_entries", "pack_cache_valid", "pack_cache_hits", "pack_cache_made", "pack_cache_bytes"
  *                                                          the re-ordered weights kept between calls
+ *   "pack_cache_refreshed"                                 copies that an mt_adam_many call wrote itself (option "pack_refresh")
  *   "pack_cache_spare_bytes"                               buffers of evicted entries that a recorded graph still names
  *   "graph_written_ranges", "graph_writes_anything"        memory written by recorded calls: weights inside such a range
  *                                                          are re-ordered on every use; after 4096 ranges everything is

@@ -42,7 +42,8 @@ def test_kept_weights_follow_every_write_path(mt):
         ("mt_copy_d2d", lambda: mt.call("mt_copy_d2d", kernel.ptr, other.ptr, C.c_size_t(kernel.count * 4)), True),
         ("mt_fill", lambda: M.Fill(kernel, 0.01), True),
         ("mt_adam", lambda: M.Adam(kernel, other, mom, vel, 4, 1e-2, 0.9, 0.999, 1e-8, 1.0), True),
-        ("mt_adam_many", lambda: Fused.AdamMany([kernel], [other], [mom], [vel], 4, 1e-2, 0.9, 0.999, 1e-8, 2.0), True),
+        # (the step over several tensors writes the re-ordered copy itself: nothing is made again, the result is the same)
+        ("mt_adam_many", lambda: Fused.AdamMany([kernel], [other], [mom], [vel], 4, 1e-2, 0.9, 0.999, 1e-8, 2.0), False),
         ("mt_fill_many", lambda: Fused.FillMany([kernel, mom], 0.02), True),
         ("mt_add into the weights", lambda: M.Add(kernel, kernel, other, 1.0, 0.5), True),
         ("mt_mul_value on a view of the weights", lambda: M.Mul(part, part, 1.5), True),
@@ -66,6 +67,67 @@ def test_kept_weights_follow_every_write_path(mt):
     hits = mt.get_info("pack_cache_hits")
     tconv(mt, out, x, kernel, bias, cout, cin)
     assert mt.get_info("pack_cache_hits") == hits + 1
+
+
+def test_optimiser_step_keeps_the_reordered_copy_current(mt):
+    """mt_adam_many writes every new weight into the kept copy for the 4x4 stride-2 transposed convolution as well: the
+    next input gradient re-orders nothing and is bit for bit what a fresh re-ordering gives, over several steps and four
+    layers in one call.  A step that also changes the bias whose sums the copy holds, a copy that was stale before the
+    step, and the option switched off all fall back to re-ordering."""
+    from mi355tensor import CTensor, CTensorMath as M, Fused
+    layers = []
+    # (the third: no tiles of 16 x 16, element by element; the last: an image layer, whose kernel has a layout of its own)
+    for n, (cin, cout, hw) in enumerate([(64, 32, 8), (128, 64, 4), (24, 20, 4), (64, 3, 16)]):
+        kernel, grad = CTensor.from_numpy(Nrm(160 + n, 1, 1, cin, cout * 16, std=0.05)), CTensor.from_numpy(Nrm(62 + n, 1, 1, cin, cout * 16, std=0.05))
+        mom, vel = CTensor(1, 1, cin, cout * 16), CTensor(1, 1, cin, cout * 16)
+        M.Fill(mom, 0.0)
+        M.Fill(vel, 0.0)
+        layers.append(dict(cin=cin, cout=cout, x=CTensor.from_numpy(Nrm(64 + n, 4, cin, hw, hw)), out=CTensor(4, cout, 2 * hw, 2 * hw), kernel=kernel, grad=grad,
+                           mom=mom, vel=vel, bias=CTensor.from_numpy(Nrm(66 + n, 1, cin, 1, 1, std=0.1))))
+    run = lambda l: tconv(mt, l["out"], l["x"], l["kernel"], l["bias"], l["cout"], l["cin"])
+    fresh = lambda l: (mt.set_option("pack_cache", 0), run(l), mt.set_option("pack_cache", 1))[1]
+    lists = lambda key: [l[key] for l in layers]
+    for l in layers:
+        run(l)
+    for step in range(1, 4):
+        refreshed, made = mt.get_info("pack_cache_refreshed"), mt.get_info("pack_cache_made")
+        Fused.AdamMany(lists("kernel"), lists("grad"), lists("mom"), lists("vel"), 4, 1e-2, 0.9, 0.999, 1e-8, float(step))
+        assert mt.get_info("pack_cache_refreshed") == refreshed + 4
+        got = [run(l) for l in layers]
+        assert mt.get_info("pack_cache_made") == made, "the copies were re-ordered again"
+        for l, g in zip(layers, got):
+            assert np.array_equal(g, fresh(l)), step
+        for l in layers:
+            run(l)  # (switching the cache off dropped every entry: they exist again for the next step)
+    # the bias in the same step: its sums in the entry are stale, so the copy is made again
+    l = layers[0]
+    bias_grad, bias_mom, bias_vel = CTensor.from_numpy(Nrm(70, 1, l["cin"], 1, 1)), CTensor(1, l["cin"], 1, 1), CTensor(1, l["cin"], 1, 1)
+    M.Fill(bias_mom, 0.0)
+    M.Fill(bias_vel, 0.0)
+    made = mt.get_info("pack_cache_made")
+    Fused.AdamMany([l["kernel"], l["bias"]], [l["grad"], bias_grad], [l["mom"], bias_mom], [l["vel"], bias_vel], 4, 1e-2, 0.9, 0.999, 1e-8, 4.0)
+    got = run(l)
+    assert mt.get_info("pack_cache_made") == made + 1
+    assert np.array_equal(got, fresh(l))
+    run(l)
+    # a copy that is stale before the step (the bias was written on its own) is not vouched for by the step
+    M.Fill(l["bias"], 0.125)
+    made = mt.get_info("pack_cache_made")
+    Fused.AdamMany([l["kernel"]], [l["grad"]], [l["mom"]], [l["vel"]], 4, 1e-2, 0.9, 0.999, 1e-8, 5.0)
+    got = run(l)
+    assert mt.get_info("pack_cache_made") == made + 1
+    assert np.array_equal(got, fresh(l))
+    run(l)
+    # switched off: the step only reports its write
+    mt.set_option("pack_refresh", 0)
+    try:
+        made, refreshed = mt.get_info("pack_cache_made"), mt.get_info("pack_cache_refreshed")
+        Fused.AdamMany([l["kernel"]], [l["grad"]], [l["mom"]], [l["vel"]], 4, 1e-2, 0.9, 0.999, 1e-8, 6.0)
+        got = run(l)
+        assert mt.get_info("pack_cache_made") == made + 1 and mt.get_info("pack_cache_refreshed") == refreshed
+        assert np.array_equal(got, fresh(l))
+    finally:
+        mt.set_option("pack_refresh", 1)
 
 
 def test_kept_weights_of_the_other_layouts(mt):
