@@ -120,6 +120,8 @@ int mt_timer_destroy(void *timer);
  *   "pack_refresh"   1 (default) mt_adam_many writes each new weight also into the kept re-ordered copy that the 4x4 stride-2
  *                    transposed convolution (the input gradient of a 4x4 stride-2 convolution layer) made of those weights, so a
  *                    training loop re-orders nothing per step; not while a graph is recorded / 0 the step only reports its write
+ *   "adam_vec"       1 (default) mt_adam_many updates four elements per thread in the tiles that also write a re-ordered copy /
+ *                    2 wherever the tensors allow / 0 never (measurements only; the results are the same bit for bit)
  *   "first_layer"    1 (default) forward convolutions of 3-channel images (3x3, 4x4, 5x5 kernels to 32 or 64 filters) keep the
  *                    input patch in LDS and the weights in registers wherever the shape allows / 0 never
  *   "walk_blocks"    blocks wanted per launch of the walking kernel (default 1024)
