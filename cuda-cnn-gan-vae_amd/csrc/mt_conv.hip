@@ -28,6 +28,7 @@ using mt::cdiv;
 int g_conv_path = 0;  // 0 auto, 1 direct, 2 implicit GEMM wherever it applies
 int g_first_layer = 1; // forward convolutions of 3-channel images: 0 never on the kernel that keeps the input patch in LDS and the weights in registers, 1 wherever the shape allows
 int g_conv_walk = 1;   // forward convolutions whose taps tile the k step: 0 never on the kernel whose blocks walk over the batch, 1 wherever the shape allows and gives 512 blocks, 2 wherever the shape allows
+int g_walk_wide = 1;       // 1: layers whose output channels are a multiple of 32 but not of 64 walk in blocks of 32 rows x 128 columns, 0: never
 int g_upconv_split = 1;    // 1: up-sampling convolutions with fewer than 512 walking blocks share a tile's k steps between blocks
 int g_upconv_walk = 512;   // blocks from which the up-sampling convolution takes the walking kernel (0: never; measured on the
                            // shipped GAN generator at batch 32: 768 blocks 67.7 -> 54.6 and 58.6 -> 54.0 us, 384 blocks 65.1 -> 69 us)
@@ -1654,6 +1655,8 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     size_t covered = 0;
     for (uint32_t f = 0; f < args.nphase; f++) covered += (size_t)args.ph[f].qh * args.ph[f].qw;
     walk_tm = mt::igemm::walk_tm() == 2 && kz % 128 == 0 ? 2u : 1u;
+    walk.wide = g_walk_wide && !norm && !bn && kz % 64 != 0 && kz % 32 == 0 ? 1u : 0u;
+    if (walk.wide) walk_tm = 1;
     walks = covered == OHW && tconv_walk_plan(walk, (uint32_t)mt::igemm::walk_blocks(), walk_tm);
   }
   bool k4s2 = kx == 4 && ky == 4 && sx == 2 && sy == 2 && args.nphase == 4 && kernel->x % 4 == 0 && ((uintptr_t)kernel->p & 15u) == 0 && kz <= 65534;
@@ -1699,7 +1702,7 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     }
     walk.tap_bias = ws;
     {
-      mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, walk.M, out->w * args.ph[0].qh * args.ph[0].qw, args.ph[0].kp, args.nphase) : name);
+      mt::ProfileScope prof(mt::profiling() ? shape_label(name, walk.wide ? T32x128 : T64x64, walk.M, out->w * args.ph[0].qh * args.ph[0].qw, args.ph[0].kp, args.nphase) : name);
       if ((rc = launch_tconv_walk(name, walk, norm != nullptr, bn != nullptr, walk_tm))) return rc;
     }
     if (bn) {
@@ -2048,6 +2051,7 @@ int upsampling_convolution(const char *name, const mt_tensor *out, const mt_tens
     walk.M = ka; walk.batch = out->w; walk.delta = image->p; walk.C = (uint32_t)kz; walk.H = image->y; walk.W = image->x;
     walk.out = out->p; walk.OW = out->x; walk.OHW = OHW; walk.sy = 2; walk.sx = 2;
     walk.row_bias = bias->p; walk.tap_bias = nullptr; walk.func = args.ep.func;
+    walk.wide = g_walk_wide && ka % 64 != 0 && ka % 32 == 0 ? 1u : 0u;   // 32 filters (or 96, ...): blocks of 32 rows x 128 columns
     if (mt::igemm::tconv_walk_plan(walk, (uint32_t)mt::igemm::walk_blocks(), 1) || mt::igemm::tconv_walk_plan_flat(walk)) {
       // too few tiles for the chip (small images, many channels): two or four blocks share a tile's k steps, their sums
       // are added afterwards together with the bias and the function
@@ -2060,13 +2064,13 @@ int upsampling_convolution(const char *name, const mt_tensor *out, const mt_tens
         if ((rc = mt::split_workspace((size_t)share * mt::count(out), &partial))) return rc;
         walk.ksplit = share; walk.nk /= share; walk.split_stride = mt::count(out);
         walk.out = partial; walk.row_bias = nullptr; walk.func = MT_F_NONE;
-        mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, out->w * args.ph[0].qh * args.ph[0].qw, walk.nk * mt::igemm::BK, args.nphase * share) : name);
+        mt::ProfileScope prof(mt::profiling() ? shape_label(name, walk.wide ? T32x128 : T64x64, ka, out->w * args.ph[0].qh * args.ph[0].qw, walk.nk * mt::igemm::BK, args.nphase * share) : name);
         if ((rc = mt::igemm::launch_tconv_walk(name, walk, false, false, 1))) return rc;
         return mt::split_reduce(name, out->p, partial, share, mt::count(out), bias->p, OHW, ka, func);
       }
       if (blocks >= (size_t)g_upconv_walk) {
         {
-          mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, out->w * args.ph[0].qh * args.ph[0].qw, args.ph[0].kp, args.nphase) : name);
+          mt::ProfileScope prof(mt::profiling() ? shape_label(name, walk.wide ? T32x128 : T64x64, ka, out->w * args.ph[0].qh * args.ph[0].qw, args.ph[0].kp, args.nphase) : name);
           if ((rc = mt::igemm::launch_tconv_walk(name, walk, false, false, 1))) return rc;
         }
         return func_later ? mt_apply_func(out, out, func) : MT_OK;
@@ -2249,6 +2253,11 @@ int set_patch_blocks(int v) {
 int set_igemm_tile(int v) {
   if (v < -1 || v > 4) return fail(MT_E_ARGUMENT, "igemm_tile must be -1 (auto) or 0..4");
   igemm::tile_override() = v;
+  return MT_OK;
+}
+int set_walk_wide(int v) {
+  if (v < 0 || v > 1) return fail(MT_E_ARGUMENT, "walk_wide must be 0 or 1");
+  g_walk_wide = v;
   return MT_OK;
 }
 int set_upconv_split(int v) {

@@ -36,6 +36,7 @@ struct WalkArgs {
   uint32_t nk;                           // k steps of one block's tile (the same for every phase): all of them, or one of ksplit equal shares
   uint32_t ksplit = 1;                   // blocks that share a tile's k steps; block ks writes its sums to out + ks * split_stride (per = 1 then)
   size_t split_stride = 0;               // floats
+  uint32_t wide = 0;                     // 1: blocks of 32 rows x 128 columns (set by the caller before planning; plain variant only)
   uint32_t flat = 0;                     // 1: the columns are (sample, pixel) pairs counted through the whole batch, 64 to a tile (qtiles of
                                          // them, the last one may be ragged), for pixel counts that no tile of 16, 32 or 64 divides; no walk
   uint32_t weights_major;                // block order, see tconv_walk_kernel
@@ -63,9 +64,13 @@ __device__ __forceinline__ void welford_merge_equal(float &mean, float &m2, floa
 // TM: 32-row accumulators per wavefront (the block is 64*TM rows x 64 columns, 2 x 2 wavefronts)
 // NORM: 0 the input is used as it is, 1 ReLU(scale * x + shift), 2 any of the cheap functions of it (chosen at run time: a
 // branch per element in the loader, which the one case that generators use should not pay)
-template <int NORM, bool STATS, int WAVES, int TM, bool ROWBIAS = false>
+// WIDE: the block is 32 rows x 128 columns, four wavefronts side by side (layers with 32 output channels; plain variant
+// only: no statistics, no normalisation of the input, one accumulator per wavefront)
+template <int NORM, bool STATS, int WAVES, int TM, bool ROWBIAS = false, bool WIDE = false>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void tconv_walk_kernel(WalkArgs a) {
-  constexpr int BM = 64 * TM, BN = 64, E = 4;  // four elements per thread, operand and 64 rows
+  static_assert(!WIDE || (NORM == 0 && !STATS && TM == 1), "the 32 x 128 block exists as the plain variant only");
+  constexpr int BM = WIDE ? 32 : 64 * TM, BN = WIDE ? 128 : 64, E = 4;  // four elements per thread, operand and 64 rows
+  constexpr int NB = BN / 64;   // sets of four k per thread and step in operand B (a step is 16 k of BN columns)
   __shared__ float4 smem4[2 * (BM + BN) * LDK / 4];
   float *smem = reinterpret_cast<float *>(smem4);
   float *As = smem, *Bs = smem + 2 * BM * LDK;
@@ -90,7 +95,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   const uint32_t m0 = mt * BM, HW = a.H * a.W, sp = (uint32_t)BN >> a.px_log, px_mask = (1u << a.px_log) - 1u;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = WIDE ? 0 : wave >> 1, wn = WIDE ? wave : wave & 1;
+  const bool a_loader = !WIDE || wave < 2;   // 32 rows of A are one 128-bit load for 128 threads
 
   // ---- operand A: packed sub-kernel of the phase, [M][ld], one 128-bit load per thread and step
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ph.packed, a.M * ph.ld * 4u);
@@ -99,11 +105,13 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   const uint32_t a_oct = (uint32_t)tid / 8u, a_row = (a_oct / 4u) * 8u + (a_oct % 4u) + 4u * (((uint32_t)tid % 8u) / 4u), a_k = ((uint32_t)tid % 4u) * E;
   const uint32_t a_voff = ((m0 + a_row) * ph.ld + a_k) * 4u;  // M is a multiple of the block's rows; the next 64 rows are 64*ld further
   // ---- operand B: the thread's column (pixel p of sample s of the group) and its E consecutive k (channel, tap)
+  // (with 128 columns a thread's two sets are k = b_k .. b_k+3 and b_k+8 .. b_k+11)
   const uint32_t b_col = (uint32_t)tid % BN, b_k = (uint32_t)__builtin_amdgcn_readfirstlane((tid / BN) * E);
+  constexpr uint32_t B_SET = (THREADS / BN) * E;
   const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(a.delta, a.batch * a.C * HW * 4u);
   __amdgpu_buffer_rsrc_t s_rsrc = b_rsrc;
   if (NORM) s_rsrc = make_rsrc(a.scale_shift, a.C * HW * 8u);
-  uint32_t b_voff[E], sample_bytes;  // (the offsets of the pairs follow from b_voff: twice the offset inside the sample)
+  uint32_t b_voff[NB][E], sample_bytes;  // (the offsets of the pairs follow from b_voff: twice the offset inside the sample)
   uint32_t sstep;
   {
     const uint32_t qhw = ph.qh * ph.qw, n = qt * BN + b_col;
@@ -114,13 +122,15 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
     const int lt = __builtin_ctz(taps), lx = __builtin_ctz(tx_cnt);
     const bool col_ok = q < ph.qh * ph.qw && sample < a.batch;
 #pragma unroll
-    for (int i = 0; i < E; i++) {
-      const uint32_t kk = b_k + i, cc = kk >> lt, t = kk & (taps - 1u), ty = t >> lx, tx = t & (tx_cnt - 1u);
-      const int32_t iy = (int32_t)(qy * a.in_sy) + ph.offy + (int32_t)ty, ix = (int32_t)(qx * a.in_sx) + ph.offx + (int32_t)tx;
-      const bool ok = col_ok && (uint32_t)iy < a.H && (uint32_t)ix < a.W;
-      const uint32_t pixel = (cc * a.H + (uint32_t)iy) * a.W + (uint32_t)ix;
-      b_voff[i] = ok ? (sample * a.C * HW + pixel) * 4u : OOB;
-    }
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+      for (int i = 0; i < E; i++) {
+        const uint32_t kk = b_k + (uint32_t)j * B_SET + i, cc = kk >> lt, t = kk & (taps - 1u), ty = t >> lx, tx = t & (tx_cnt - 1u);
+        const int32_t iy = (int32_t)(qy * a.in_sy) + ph.offy + (int32_t)ty, ix = (int32_t)(qx * a.in_sx) + ph.offx + (int32_t)tx;
+        const bool ok = col_ok && (uint32_t)iy < a.H && (uint32_t)ix < a.W;
+        const uint32_t pixel = (cc * a.H + (uint32_t)iy) * a.W + (uint32_t)ix;
+        b_voff[j][i] = ok ? (sample * a.C * HW + pixel) * 4u : OOB;
+      }
     sample_bytes = sample * a.C * HW * 4u;
     sstep = (BK / taps) * HW * 4u;
   }
@@ -136,14 +146,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   // Register sets: A and B are loaded two steps before they are written to LDS (two sets, tile t+3 requested while
   // tile t is multiplied).  The (scale, shift) pairs come from the L2 cache and are requested one step ahead into a
   // single set -- in front of the A and B loads of the same step, so that waiting for them leaves those in flight.
-  float ra[2][TM][E], rb[2][E];
+  float ra[2][TM][E], rb[2][NB][E];
   floatx2 rs[NORM ? E : 1];
   const uint32_t s_first = 2u * ks * nk * sstep;
   uint32_t s_next = s_first;  // scalar offset of the pairs of the tile that is written to LDS next
   auto load_pairs = [&]() {
     if constexpr (NORM) {
 #pragma unroll
-      for (int i = 0; i < E; i++) rs[i] = buf_load2(s_rsrc, b_voff[i] == OOB ? OOB : (b_voff[i] - sample_bytes) * 2u, s_next);
+      for (int i = 0; i < E; i++) rs[i] = buf_load2(s_rsrc, b_voff[0][i] == OOB ? OOB : (b_voff[0][i] - sample_bytes) * 2u, s_next);
       s_next += 2u * sstep;
       if (s_next == s_first + 2u * sstep * nk) s_next = s_first;
     }
@@ -151,31 +161,38 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, 
   auto load_tile = [&](int set, bool adv) {
     if (adv) advance();
     __builtin_amdgcn_sched_barrier(0);
+    if (a_loader) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-      const floatx4 t = buf_load4(a_rsrc, a_voff + (uint32_t)i * 64u * ph.ld * 4u, a_soff);
-      ra[set][i][0] = t.x; ra[set][i][1] = t.y; ra[set][i][2] = t.z; ra[set][i][3] = t.w;
+      for (int i = 0; i < TM; i++) {
+        const floatx4 t = buf_load4(a_rsrc, a_voff + (uint32_t)i * 64u * ph.ld * 4u, a_soff);
+        ra[set][i][0] = t.x; ra[set][i][1] = t.y; ra[set][i][2] = t.z; ra[set][i][3] = t.w;
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < E; i++) rb[set][i] = buf_load(b_rsrc, b_voff[i], b_soff);
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+      for (int i = 0; i < E; i++) rb[set][j][i] = buf_load(b_rsrc, b_voff[j][i], b_soff);
     __builtin_amdgcn_sched_barrier(0);
   };
   float *a_put = As + a_row * LDK + a_k, *b_put = Bs + b_col * LDK + b_k;
   const int in_func = a.in_func;
   auto put_tile = [&](int set, int buf) {
+    if (a_loader) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) lds_put<E>(a_put + buf * BM * LDK + i * 64 * LDK, ra[set][i]);
+      for (int i = 0; i < TM; i++) lds_put<E>(a_put + buf * BM * LDK + i * 64 * LDK, ra[set][i]);
+    }
     if constexpr (NORM) {
       float v[E];
 #pragma unroll
       for (int i = 0; i < E; i++) {
-        const float u = rs[i].x * rb[set][i] + rs[i].y;
+        const float u = rs[i].x * rb[set][0][i] + rs[i].y;
         v[i] = NORM == 1 ? (u > 0.f ? u : 0.f) : apply_func_cheap(in_func, u);
       }
       lds_put<E>(b_put + buf * BN * LDK, v);
     } else {
-      lds_put<E>(b_put + buf * BN * LDK, rb[set]);
+#pragma unroll
+      for (int j = 0; j < NB; j++) lds_put<E>(b_put + buf * BN * LDK + j * (int)B_SET, rb[set][j]);
     }
   };
 
@@ -630,7 +647,7 @@ inline bool tconv_walk_fits(const WalkArgs &a, uint32_t tm) {
     if (ph.qh * ph.qw != qhw || ph.kp != p0.kp || taps == 0 || BK % taps != 0 || (taps & (taps - 1)) != 0 || (ph.taps_x & (ph.taps_x - 1)) != 0) return false;
     if (a.C % (BK / taps) != 0 || ph.ld < ph.kp || ph.ld % 4 != 0) return false;
   }
-  if (p0.kp % (2 * BK) != 0 || p0.kp < 4 * BK || a.M % (64 * tm) != 0) return false;
+  if (p0.kp % (2 * BK) != 0 || p0.kp < 4 * BK || a.M % (a.wide ? 32 : 64 * tm) != 0 || (a.wide && tm != 1)) return false;
   return (uint64_t)a.batch * a.M * a.OHW * 4u < 0x80000000ull && (uint64_t)a.batch * a.C * a.H * a.W * 4u < 0x80000000ull;
 }
 // Whether (and how) a transposed convolution can walk: fills px_log, qtiles, groups, per, nk.
@@ -640,15 +657,17 @@ inline bool tconv_walk_plan(WalkArgs &a, uint32_t want_blocks, uint32_t tm) {
   const uint32_t qhw = p0.qh * p0.qw;
   a.flat = 0;
   a.nk = p0.kp / BK;
-  // pixels per tile: 16 (four samples per tile: two per wavefront, merged by a lane shuffle), else 32 or 64
+  // pixels per tile: 16 (four samples per tile: two per wavefront, merged by a lane shuffle), else 32 or 64; twice
+  // that for the blocks of 128 columns
+  const uint32_t cols = a.wide ? 128u : 64u, lo = a.wide ? 5u : 4u;
   uint32_t px_log = 0;
-  for (uint32_t cand : {4u, 5u, 6u})
-    if (qhw % (1u << cand) == 0 && a.batch % (64u >> cand) == 0) { px_log = cand; break; }
+  for (uint32_t cand = lo; cand < lo + 3u; cand++)
+    if (qhw % (1u << cand) == 0 && a.batch % (cols >> cand) == 0) { px_log = cand; break; }
   if (px_log == 0) return false;
   a.px_log = px_log;
   a.qtiles = qhw >> px_log;
-  const uint32_t sp = 64u >> px_log, sample_groups = a.batch / sp;
-  a.tiles_m = a.M / (64 * tm);
+  const uint32_t sp = cols >> px_log, sample_groups = a.batch / sp;
+  a.tiles_m = a.M / (a.wide ? 32 : 64 * tm);
   const uint32_t base = a.nphase * a.tiles_m * a.qtiles;
   // batch groups: as many as give about want_blocks blocks, a divisor of the number of sample groups
   uint32_t groups = base >= want_blocks ? 1u : want_blocks / base;
@@ -671,8 +690,9 @@ inline bool tconv_walk_plan_flat(WalkArgs &a) {
   const uint64_t n = (uint64_t)a.batch * p0.qh * p0.qw;
   a.flat = 1;
   a.nk = p0.kp / BK;
-  a.px_log = 6; a.qtiles = (uint32_t)((n + 63) / 64); a.groups = 1; a.per = 1;
-  a.tiles_m = a.M / 64;
+  const uint32_t cols = a.wide ? 128u : 64u;
+  a.px_log = a.wide ? 7 : 6; a.qtiles = (uint32_t)((n + cols - 1) / cols); a.groups = 1; a.per = 1;
+  a.tiles_m = a.M / (a.wide ? 32 : 64);
   a.fair = (uint32_t)walk_fair();
   a.ksplit = 1; a.split_stride = 0;
   a.weights_major = walk_order() >= 0 ? (uint32_t)walk_order() : ((uint64_t)a.nphase * a.M * p0.kp * 4u > (4u << 20) && a.tiles_m > 1 ? 1u : 0u);
@@ -690,6 +710,13 @@ inline int launch_tconv_walk(const char *name, const WalkArgs &a, bool norm, boo
   if (a.flat && (stats || tm != 1 || a.per != 1 || a.groups != 1)) return fail(MT_E_ARGUMENT, "%s: flat column tiles do not walk and keep no statistics", name);
   if (a.ksplit > 1 && (stats || a.per != 1 || a.nk < 4 || a.nk % 2 != 0 || a.row_bias || a.tap_bias || a.func != MT_F_NONE))
     return fail(MT_E_ARGUMENT, "%s: blocks that share a tile's k steps write plain sums of one batch group", name);
+  if (a.wide) {
+    if (norm || stats || tm != 1) return fail(MT_E_ARGUMENT, "%s: blocks of 32 rows walk without batch-norm folding", name);
+    if (a.row_bias) tconv_walk_kernel<0, false, 4, 1, true, true><<<grid, THREADS, 0, s>>>(a);
+    else tconv_walk_kernel<0, false, 4, 1, false, true><<<grid, THREADS, 0, s>>>(a);
+    MT_LAUNCH_CHECK(name);
+    return MT_OK;
+  }
   if (a.row_bias) {  // forward convolution: plain variant only
     if (norm || stats || tm != 1) return fail(MT_E_ARGUMENT, "%s: a forward convolution walks without batch-norm folding", name);
     tconv_walk_kernel<0, false, 4, 1, true><<<grid, THREADS, 0, s>>>(a);

@@ -114,6 +114,8 @@ int mt_timer_destroy(void *timer);
  *                    0 never
  *   "upconv_walk"    512 (default) mt_upsampling_convolution_func (x2, 3x3) uses the walking kernel when that gives at least this
  *                    many blocks / 1 wherever the shape allows / 0 never
+ *   "walk_wide"      1 (default) transposed and up-sampling convolutions whose output channels are a multiple of 32 but not of 64
+ *                    walk in blocks of 32 rows x 128 columns / 0 they run on the one-tile kernels
  *   "upconv_split"   1 (default) where that kernel would get fewer than 512 blocks (small images, many channels), two or four
  *                    blocks share a tile's sum over (channel, tap) and a second kernel adds their parts, the bias and the function /
  *                    0 never

@@ -486,14 +486,14 @@ def test_upsampling_convolution(gpu, oracle, path, case):
 
 def test_upsampling_convolution_walk_random_geometries(gpu, oracle, path):
     """The walking routes of the fused call (whole tiles of 16, 32 or 64 pixels, flat (sample, pixel) tiles, blocks that
-    share a tile's k steps) on sixteen seeded random shapes whose filters fill 64-row blocks, against the two layers on
+    share a tile's k steps) on sixteen seeded random shapes whose filters fill 32- or 64-row blocks, against the two layers on
     the oracle; the second pass forbids sharing, so the same shapes also run as one block per tile."""
     import mi355tensor as mt
     rng = np.random.default_rng(77)
     try:
         mt.set_option("upconv_walk", 1)
         for n in range(16):
-            KA = 64 * int(rng.integers(1, 3))
+            KA = 32 * int(rng.integers(1, 5))   # (32 and 96: blocks of 32 rows x 128 columns)
             C = 16 * int(rng.integers(1, 9))
             H, Wd = int(rng.integers(1, 10)), int(rng.integers(1, 10))
             B = int(rng.integers(1, 9))
