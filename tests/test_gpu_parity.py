@@ -273,6 +273,36 @@ def test_backward_convolution(gpu, oracle, path, case, with_bias):
             assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("case", [
+    # W, C (channels of the result), H, Wd (input size), KA (input channels)
+    (4, 32, 8, 16, 64),      # 128 pixels per sample and phase: one sample per tile
+    (8, 32, 4, 8, 32),       # 32 pixels: four samples share a tile
+    (6, 96, 8, 8, 16),       # 96 channels: three row tiles; 64 pixels, two samples per tile, three groups to walk
+    (3, 32, 5, 6, 48),       # 30 pixels per sample: no tile divides them, the one-tile kernel runs either way
+    (16, 32, 16, 16, 64),    # the VAE decoder's 64 -> 32 layer at a quarter of its batch and size
+])
+@pytest.mark.parametrize("func", [None, "leaky_relu", "sigmoid"])
+def test_transposed_convolution_walking_in_32_row_blocks(gpu, oracle, path, case, func):
+    """Transposed convolution 4x4 stride 2 padding 1 to 32 (or 96) channels: the kernel whose blocks walk over the batch in
+    blocks of 32 rows x 128 columns, against the oracle and against the one-tile kernels (option walk_wide)."""
+    import mi355tensor as mt
+    W, C, H, Wd, KA = case
+    delta, kernel, bias = U(4, W, KA, H, Wd), U(5, 1, 1, KA, C * 16) * 0.2, U(6, 1, KA, 1, 1)
+    args = (delta, kernel, bias, 4, 4, C, KA, 2, 2, 1, 1, (W, C, 2 * H, 2 * Wd))
+    want = oracle.backward_convolution(*args)
+    if func:
+        want = oracle.apply_func(want, func)
+    got = {}
+    try:
+        for mode in (1, 0):
+            mt.set_option("walk_wide", mode)
+            got[mode] = gpu.backward_convolution(*args, func=func)
+    finally:
+        mt.set_option("walk_wide", 1)
+    close(got[1], want, 1e-5)
+    close(got[0], want, 1e-5)
+
+
 @pytest.mark.parametrize("case", CONV_CASES)
 @pytest.mark.parametrize("back", [False, True])
 def test_create_delta_weight_and_bias(gpu, oracle, path, case, back):
