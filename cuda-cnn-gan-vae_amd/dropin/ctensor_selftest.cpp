@@ -146,6 +146,49 @@ static void BackwardConvolutionCheck(void)
  Report("BackwardConvolution 5x5, stride 2, padding 2",out.Compare(control,"",false));
 }
 
+// A bias that is known to hold zeros reaches the library as one shared block of zeros (mi355::ZeroBlock) and is not read:
+// the result is that of a tensor whose zeros were written element by element, and every later write to the tensor ends it.
+static void ZeroBiasCheck(void)
+{
+ type_t delta[16];
+ for(int n=0;n<16;n++) delta[n]=n+1;
+ CTensor<type_t> kernel(1,1,2,3*16),trained(1,2,1,1),dl(BATCH,2,4,4),out(BATCH,3,8,8),control(BATCH,3,8,8);
+ for(uint32_t f=0;f<2;f++)
+  for(uint32_t n=0;n<48;n++) kernel.SetElement(0,0,f,n,static_cast<type_t>((n*7+f*5)%11)-5);
+ trained.SetElement(0,0,0,0,0.5f);trained.SetElement(0,1,0,0,-0.25f);
+ for(uint32_t w=0;w<BATCH;w++)
+  for(uint32_t f=0;f<2;f++)
+   for(uint32_t n=0;n<16;n++) dl.SetElement(w,f,n/4,n%4,delta[n]*(f+1)+w);
+ CTensor<type_t> written(1,2,1,1);
+ written.SetElement(0,0,0,0,0);written.SetElement(0,1,0,0,0);   // zeros that the class does not know to be zeros
+ CTensorConv<type_t>::BackwardConvolution(control,dl,kernel,4,4,3,2,written,2,2,1,1);
+ CTensor<type_t> zeroed=trained;                                   // the layer's own sequence: a copy of the bias, filled with 0
+ CTensorMath<type_t>::Fill(zeroed,0);
+ CTensorConv<type_t>::BackwardConvolution(out,dl,kernel,4,4,3,2,zeroed,2,2,1,1);
+ bool ok=out.Compare(control,"",false) && zeroed.GetElement(0,1,0,0)==0 && trained.GetElement(0,1,0,0)==-0.25f;
+ Report("BackwardConvolution with a bias filled with zeros",ok);
+ // writes end it: an element set on the host, a device operation into the tensor, a copy of other values
+ zeroed.SetElement(0,0,0,0,0.5f);zeroed.SetElement(0,1,0,0,-0.25f);
+ CTensorConv<type_t>::BackwardConvolution(out,dl,kernel,4,4,3,2,zeroed,2,2,1,1);
+ CTensorConv<type_t>::BackwardConvolution(control,dl,kernel,4,4,3,2,trained,2,2,1,1);
+ ok=out.Compare(control,"",false) && out.GetElement(0,0,3,3)!=0;
+ CTensorMath<type_t>::Fill(zeroed,0);
+ CTensorMath<type_t>::Add(zeroed,zeroed,trained);
+ CTensorConv<type_t>::BackwardConvolution(out,dl,kernel,4,4,3,2,zeroed,2,2,1,1);
+ ok=ok && out.Compare(control,"",false);
+ CTensorMath<type_t>::Fill(zeroed,0);
+ zeroed=trained;
+ CTensorConv<type_t>::BackwardConvolution(out,dl,kernel,4,4,3,2,zeroed,2,2,1,1);
+ ok=ok && out.Compare(control,"",false);
+ CTensor<type_t> copy_of_zeros;
+ CTensorMath<type_t>::Fill(zeroed,0);
+ copy_of_zeros=zeroed;                                               // a copy of zeros holds zeros
+ CTensorConv<type_t>::BackwardConvolution(out,dl,kernel,4,4,3,2,copy_of_zeros,2,2,1,1);
+ CTensorConv<type_t>::BackwardConvolution(control,dl,kernel,4,4,3,2,written,2,2,1,1);
+ ok=ok && out.Compare(control,"",false);
+ Report("a write to the bias ends it",ok);
+}
+
 static void SummXYCheck(void)
 {
  bool ok=true;
@@ -682,6 +725,7 @@ int main(void)
   ForwardConvolutionCheck();
   DeltaWeightChecks();
   BackwardConvolutionCheck();
+  ZeroBiasCheck();
   DeferredGradientChecks();
   FusedSequenceChecks();
   SharedBlockChecks();

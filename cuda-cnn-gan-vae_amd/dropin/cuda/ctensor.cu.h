@@ -9,6 +9,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
+#include <map>
 #include <memory>
 #include <string>
 #include <utility>
@@ -21,6 +22,26 @@
 
 namespace mi355
 {
+ // `floats` zeros on the device, made once per size and kept until the process ends.  CTensorConv::BackwardConvolution
+ // hands them to the library in place of a bias tensor that is known to hold zeros: the convolution layer zeroes a fresh
+ // copy of its bias on every backward pass (netlayer/cnetlayerconvolution.cu.h:494-497), and the library keeps its
+ // re-ordered weights per (kernel, bias) pair -- with one address for all those zeros the pair stays the same from step
+ // to step, with a new temporary per step it never does.
+ inline float* ZeroBlock(size_t floats)
+ {
+  static std::map<size_t,float*> blocks;
+  std::map<size_t,float*>::iterator found=blocks.find(floats);
+  if (found!=blocks.end()) return(found->second);
+  void *ptr=NULL;
+  Check(mt_malloc(&ptr,floats*sizeof(float)));
+  mt_tensor t;
+  t.p=static_cast<float*>(ptr);
+  t.w=1;t.z=1;t.y=1;t.x=static_cast<uint32_t>(floats);
+  Check(mt_fill(&t,0));
+  blocks[floats]=t.p;
+  return(t.p);
+ }
+
  // Device buffer with value semantics (copying a CCUDADeviceVector copies the device data, cuda/ccudadevicevector.cu.h:159-170)
  // whose copies share one block until one of them is written: the layers hand whole activations on with operator= on
  // every step (cTensor_Delta=error in every SetOutputError, netlayer/cnetlayerconvolution.cu.h:571; the batch-norm layer's
@@ -184,10 +205,14 @@ class CTensor
   enum {LAZY_NONE=0,LAZY_ZERO,LAZY_GRADIENT_KERNEL,LAZY_GRADIENT_BIAS};
   mutable uint8_t Lazy;
   mutable std::shared_ptr<mi355::CDeferredGradient> Deferred;
+  // The last write was a fill with zeros (set by the fills, cleared by everything that hands out the tensor for writing
+  // and by every change of either copy): see mi355::ZeroBlock.
+  mutable bool KnownZero;
  public:
   CTensor(uint32_t size_w=1,uint32_t size_z=1,uint32_t size_y=1,uint32_t size_x=1)
   {
    Lazy=LAZY_NONE;
+   KnownZero=false;
    Size_X=size_x;Size_Y=size_y;Size_Z=size_z;Size_W=size_w;
    BasedSize_X=Size_X;BasedSize_Y=Size_Y;BasedSize_Z=Size_Z;BasedSize_W=Size_W;
    Item.resize(Count());
@@ -198,6 +223,7 @@ class CTensor
   CTensor(const CTensor<type_t> &cTensor)
   {
    Lazy=LAZY_NONE;
+   KnownZero=false;
    CopyValues(cTensor);
    Size_X=cTensor.Size_X;Size_Y=cTensor.Size_Y;Size_Z=cTensor.Size_Z;Size_W=cTensor.Size_W;
    BasedSize_X=Size_X;BasedSize_Y=Size_Y;BasedSize_Z=Size_Z;BasedSize_W=Size_W;
@@ -249,6 +275,7 @@ class CTensor
   {
    for(size_t n=0;n<Item.size();n++) Item[n]=value;
    SetHostOnChange();
+   KnownZero=(value==0);
   }
   void Move(CTensor<type_t> &cTensor)
   {
@@ -261,6 +288,7 @@ class CTensor
    BasedSize_X=cTensor.BasedSize_X;BasedSize_Y=cTensor.BasedSize_Y;BasedSize_Z=cTensor.BasedSize_Z;BasedSize_W=cTensor.BasedSize_W;
    HostOnChange=cTensor.HostOnChange;
    DeviceOnChange=cTensor.DeviceOnChange;
+   KnownZero=cTensor.KnownZero;
    cTensor.Size_X=0;cTensor.Size_Y=0;cTensor.Size_Z=0;cTensor.Size_W=0;
    cTensor.BasedSize_X=0;cTensor.BasedSize_Y=0;cTensor.BasedSize_Z=0;cTensor.BasedSize_W=0;
    cTensor.Item.clear();
@@ -421,8 +449,10 @@ class CTensor
    HostOnChange=false;
    DeviceOnChange=false;
   }
-  void SetDeviceOnChange(void) const {DeviceOnChange=true;HostOnChange=false;}
-  void SetHostOnChange(void) const {DropLazy();DeviceOnChange=false;HostOnChange=true;}
+  void SetDeviceOnChange(void) const {DeviceOnChange=true;HostOnChange=false;KnownZero=false;}
+  void SetHostOnChange(void) const {DropLazy();DeviceOnChange=false;HostOnChange=true;KnownZero=false;}
+  void SetKnownZero(void) const {KnownZero=true;}///<CTensorMath::Fill, after its write was noted
+  bool HoldsZeros(void) const {return(Lazy==LAZY_ZERO || (Lazy==LAZY_NONE && KnownZero==true));}
   // Writes what the device copy was only said to hold: zeros, or the per-sample gradients computed from the operands
   // that were kept (CreateDeltaWeightAndBias of the reference adds into the zeroed tensor, netlayer/
   // cnetlayerconvolution.cu.h:503-506; a sample's bias gradient is the sum of its delta over the pixels).
@@ -435,6 +465,7 @@ class CTensor
    std::shared_ptr<mi355::CDeferredGradient> record;
    record.swap(Deferred);
    Lazy=LAZY_NONE;
+   KnownZero=(kind==LAZY_ZERO);
    mt_tensor own;
    own.p=static_cast<float*>(DeviceItem.get());
    own.w=Size_W;own.z=Size_Z;own.y=Size_Y;own.x=Size_X;
@@ -544,6 +575,7 @@ class CTensor
    }
    HostOnChange=cTensor.HostOnChange;
    DeviceOnChange=cTensor.DeviceOnChange;
+   KnownZero=cTensor.KnownZero;
   }
   void DropLazy(void) const {Lazy=LAZY_NONE;Deferred.reset();}
   // the device copy is said to hold zeros; nothing is launched (CTensorMath::Fill)
@@ -581,6 +613,7 @@ class CTensor
    Materialise();
    if (upload==true) CopyToDevice();
    DeviceItem.Own(upload);
+   KnownZero=false;
    return(Descriptor());
   }
   mt_tensor DeviceRead(void) const
@@ -596,6 +629,7 @@ class CTensor
    if (upload==true) CopyToDevice();
    DeviceItem.Own(upload);
    mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),upload,true);
+   KnownZero=false;
    return(Descriptor());
   }
 };

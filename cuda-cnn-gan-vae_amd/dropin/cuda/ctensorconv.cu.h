@@ -35,7 +35,14 @@ class CTensorConv
   static void BackwardConvolution(CTensor<type_t> &cTensor_OutputDelta,const CTensor<type_t> &cTensor_Delta,const CTensor<type_t> &cTensor_Kernel,int32_t kernel_x,int32_t kernel_y,int32_t kernel_z,uint32_t kernel_amount,const CTensor<type_t> &cTensor_Bias,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)
   {
    OnlyFloat();
-   mt_tensor d=cTensor_Delta.DeviceRead(),k=cTensor_Kernel.DeviceRead(),b=cTensor_Bias.DeviceRead(),o=cTensor_OutputDelta.Device(false);
+   const bool zeros=cTensor_Bias.HoldsZeros(),unwritten=(cTensor_Bias.Lazy==CTensor<type_t>::LAZY_ZERO);
+   mt_tensor d=cTensor_Delta.DeviceRead(),k=cTensor_Kernel.DeviceRead(),b,o=cTensor_OutputDelta.Device(false);
+   // Zeros come from one address for every call (mi355::ZeroBlock).  A tensor whose zeros were never written stays
+   // unwritten; one that was filled is still brought up to date like any operand, so that the calls that wait in the
+   // queue keep their order.
+   if (unwritten==true) b=cTensor_Bias.Descriptor();
+   else b=cTensor_Bias.DeviceRead();
+   if (zeros==true) b.p=mi355::ZeroBlock(static_cast<size_t>(b.w)*b.z*b.y*b.x);
    mi355::Check(mt_backward_convolution(&o,&d,&k,kernel_x,kernel_y,kernel_z,kernel_amount,&b,stride_x,stride_y,padding_x,padding_y));
    cTensor_OutputDelta.SetDeviceOnChange();
   }

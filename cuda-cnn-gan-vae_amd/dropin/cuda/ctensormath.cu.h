@@ -43,6 +43,7 @@ class CTensorMath
    }
    mi355::Queue().Submit(mi355::MakeFill(cTensor_Output.DeviceQueued(false),value));
    cTensor_Output.SetDeviceOnChange();
+   if (value==0) cTensor_Output.SetKnownZero();
   }
   static void Inv(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input)
   {
