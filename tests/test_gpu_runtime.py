@@ -89,12 +89,16 @@ def test_optimiser_step_keeps_the_reordered_copy_current(mt):
     lists = lambda key: [l[key] for l in layers]
     for l in layers:
         run(l)
+    # (weights at an address that a graph recorded by an earlier test wrote are never vouched for: the pool may hand such a
+    # block to this test, and that layer is then re-ordered on every use, as it must be)
+    trusted = mt.get_info("graph_written_ranges") == 0 and mt.get_info("graph_writes_anything") == 0
     for step in range(1, 4):
         refreshed, made = mt.get_info("pack_cache_refreshed"), mt.get_info("pack_cache_made")
         Fused.AdamMany(lists("kernel"), lists("grad"), lists("mom"), lists("vel"), 4, 1e-2, 0.9, 0.999, 1e-8, float(step))
-        assert mt.get_info("pack_cache_refreshed") == refreshed + 4
+        kept = mt.get_info("pack_cache_refreshed") - refreshed
+        assert kept == 4 if trusted else 0 <= kept <= 4
         got = [run(l) for l in layers]
-        assert mt.get_info("pack_cache_made") == made, "the copies were re-ordered again"
+        assert mt.get_info("pack_cache_made") - made == 4 - kept, "a copy was neither kept current nor made again"
         for l, g in zip(layers, got):
             assert np.array_equal(g, fresh(l)), step
         for l in layers:
@@ -113,9 +117,10 @@ def test_optimiser_step_keeps_the_reordered_copy_current(mt):
     # a copy that is stale before the step (the bias was written on its own) is not vouched for by the step
     M.Fill(l["bias"], 0.125)
     made = mt.get_info("pack_cache_made")
+    refreshed = mt.get_info("pack_cache_refreshed")
     Fused.AdamMany([l["kernel"]], [l["grad"]], [l["mom"]], [l["vel"]], 4, 1e-2, 0.9, 0.999, 1e-8, 5.0)
     got = run(l)
-    assert mt.get_info("pack_cache_made") == made + 1
+    assert mt.get_info("pack_cache_made") == made + 1 and mt.get_info("pack_cache_refreshed") == refreshed
     assert np.array_equal(got, fresh(l))
     run(l)
     # switched off: the step only reports its write
@@ -237,7 +242,7 @@ def test_pool_reuses_blocks_in_stream_order(mt):
         assert np.array_equal(out1.numpy(), 3.0 * want + 1.0)
         assert np.array_equal(out2.numpy(), want - 5.0)
         again.free()
-    assert mt.get_info("driver_allocations") == allocs + 1
+    assert mt.get_info("driver_allocations") <= allocs + 1   # (one block for all three rounds; none when an earlier test left one of this size in the pool)
     assert mt.get_info("pool_reused") >= 5
     mt.set_option("pool", 0)
     assert mt.get_info("pool_bytes") == 0
