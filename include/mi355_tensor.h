@@ -114,11 +114,11 @@ int mt_timer_destroy(void *timer);
  *                    0 never
  *   "upconv_walk"    512 (default) mt_upsampling_convolution_func (x2, 3x3) uses the walking kernel when that gives at least this
  *                    many blocks / 1 wherever the shape allows / 0 never
- *   "walk_wide"      1 (default) transposed and up-sampling convolutions whose output channels are a multiple of 32 but not of 64
- *                    walk in blocks of 32 rows x 128 columns / 0 they run on the one-tile kernels
  *   "upconv_split"   1 (default) where that kernel would get fewer than 512 blocks (small images, many channels), two or four
  *                    blocks share a tile's sum over (channel, tap) and a second kernel adds their parts, the bias and the function /
  *                    0 never
+ *   "walk_wide"      1 (default) transposed and up-sampling convolutions whose output channels are a multiple of 32 but not of 64
+ *                    walk in blocks of 32 rows x 128 columns / 0 they run on the one-tile kernels
  *   "pack_refresh"   1 (default) mt_adam_many writes each new weight also into the kept re-ordered copy that the 4x4 stride-2
  *                    transposed convolution (the input gradient of a 4x4 stride-2 convolution layer) made of those weights, so a
  *                    training loop re-orders nothing per step; not while a graph is recorded / 0 the step only reports its write
