@@ -503,6 +503,51 @@ struct SBatchNormTensors
  }
 };
 
+// UpSampling by 2 x 2 writes nothing; a 3x3 convolution (stride 1, padding 1) of the tensor is computed from the source,
+// every other reader gets the up-sampled values, and the source may change in between.
+static void DeferredUpSamplingChecks(void)
+{
+ CTensor<type_t> source(BATCH,16,5,6),kernel(1,1,8,16*9),bias(1,8,1,1),wide(1,1,8,16*25);
+ CTensor<type_t> up(BATCH,16,10,12),up_now(BATCH,16,10,12),out(BATCH,8,10,12),control(BATCH,8,10,12),out5(BATCH,8,10,12),control5(BATCH,8,10,12);
+ FillPattern(source,3,1.0f);FillPattern(kernel,5,0.1f);FillPattern(bias,7,0.5f);FillPattern(wide,9,0.05f);
+ mi355::DeferGradients()=false;   // the two calls one after the other
+ CTensorMath<type_t>::UpSampling(up_now,source,2,2);
+ CTensorConv<type_t>::ForwardConvolution(control,up_now,kernel,3,3,16,8,bias,1,1,1,1);
+ CTensorConv<type_t>::ForwardConvolution(control5,up_now,wide,5,5,16,8,bias,1,1,2,2);
+ mi355::DeferGradients()=true;
+ CTensorMath<type_t>::UpSampling(up,source,2,2);
+ CTensor<type_t> kept=source;
+ CTensorMath<type_t>::Fill(source,7);   // the source changes after the call: the tensor stands for the values it had
+ CTensorConv<type_t>::ForwardConvolution(out,up,kernel,3,3,16,8,bias,1,1,1,1);
+ double largest=0;
+ bool ok=MaxDifference(out,control,largest)<=2e-5*largest && largest>0.1;
+ // (coefficient sums: not the same roundings as the two calls, so not the same bits either -- the fused call ran)
+ bool fused=false;
+ for(uint32_t x=0;x<12 && fused==false;x++) fused=(out.GetElement(1,3,4,x)!=control.GetElement(1,3,4,x));
+ Report("3x3 convolution of an up-sampled tensor that was never written",ok && fused);
+ // a reader of the tensor itself: the up-sampled values of the source as it was
+ ok=up.GetElement(1,3,7,9)==kept.GetElement(1,3,3,4) && up.GetElement(0,15,9,11)==kept.GetElement(0,15,4,5) && up.GetElement(1,0,0,1)==kept.GetElement(1,0,0,0);
+ CTensorConv<type_t>::ForwardConvolution(out,up,kernel,3,3,16,8,bias,1,1,1,1);   // written now: the convolution as it always was
+ ok=ok && MaxDifference(out,control,largest)==0;
+ Report("a reader of the up-sampled tensor gets it written",ok);
+ // another geometry writes the tensor first
+ CTensorMath<type_t>::UpSampling(up,kept,2,2);
+ CTensorConv<type_t>::ForwardConvolution(out5,up,wide,5,5,16,8,bias,1,1,2,2);
+ ok=MaxDifference(out5,control5,largest)==0;
+ // a copy and a later write to the tensor end the deferral
+ CTensorMath<type_t>::UpSampling(up,kept,2,2);
+ CTensor<type_t> copy=up;
+ ok=ok && MaxDifference(copy,up_now,largest)==0;
+ CTensorMath<type_t>::UpSampling(up,kept,2,2);
+ CTensorMath<type_t>::Add(up,up_now,up_now,1.0f,1.0f);
+ ok=ok && up.GetElement(1,3,7,9)==2*kept.GetElement(1,3,3,4);
+ // other factors are written at once
+ CTensor<type_t> up3(BATCH,16,15,18);
+ CTensorMath<type_t>::UpSampling(up3,kept,3,3);
+ ok=ok && up3.GetElement(1,3,11,13)==kept.GetElement(1,3,3,4);
+ Report("other kernels, copies, writes and factors",ok);
+}
+
 static void FusedSequenceChecks(void)
 {
  mi355::COpQueue &queue=mi355::Queue();
@@ -727,6 +772,7 @@ int main(void)
   BackwardConvolutionCheck();
   ZeroBiasCheck();
   DeferredGradientChecks();
+  DeferredUpSamplingChecks();
   FusedSequenceChecks();
   SharedBlockChecks();
   SummXYCheck();

@@ -161,6 +161,19 @@ namespace mi355
    if (onto==NULL) KernelReady=true;
   }
  };
+ // An up-sampled tensor that was not written yet (CTensorMath::UpSampling by 2 x 2): the source as it was (its block,
+ // shared) and the factors.  The generator of the reference's GAN model follows every up-sampling layer by a 3x3
+ // convolution (cuda/netmodel/cmodel_gan.cu.h:153-170); CTensorConv::ForwardConvolution on such a tensor computes the
+ // convolution of the up-sampled image from the source itself (mt_upsampling_convolution_func: four 2x2 convolutions,
+ // 4/9 of the multiplications, the image of four times the size neither written nor read).  Whoever reads the tensor
+ // in any other way gets it written first (CTensor::Materialise), e.g. the layer's weight gradient in training.
+ struct CDeferredUpSampling
+ {
+  CDeviceBuffer Source;
+  mt_tensor SourceTensor;
+  uint32_t Factor_X;
+  uint32_t Factor_Y;
+ };
  // switch for the deferral (on by default): with `false` every call runs when it is made
  inline bool& DeferGradients(void)
  {
@@ -202,9 +215,10 @@ class CTensor
   mutable bool DeviceOnChange;
   // What the device copy holds when it was not written yet (mi355::CDeferredGradient): while Lazy is not LAZY_NONE the
   // device copy is the current one (DeviceOnChange) and every access goes through Materialise() first.
-  enum {LAZY_NONE=0,LAZY_ZERO,LAZY_GRADIENT_KERNEL,LAZY_GRADIENT_BIAS};
+  enum {LAZY_NONE=0,LAZY_ZERO,LAZY_GRADIENT_KERNEL,LAZY_GRADIENT_BIAS,LAZY_UPSAMPLING};
   mutable uint8_t Lazy;
   mutable std::shared_ptr<mi355::CDeferredGradient> Deferred;
+  mutable std::shared_ptr<mi355::CDeferredUpSampling> DeferredUpSampling;
   // The last write was a fill with zeros (set by the fills, cleared by everything that hands out the tensor for writing
   // and by every change of either copy): see mi355::ZeroBlock.
   mutable bool KnownZero;
@@ -464,11 +478,20 @@ class CTensor
    const uint8_t kind=Lazy;
    std::shared_ptr<mi355::CDeferredGradient> record;
    record.swap(Deferred);
+   std::shared_ptr<mi355::CDeferredUpSampling> up;
+   up.swap(DeferredUpSampling);
    Lazy=LAZY_NONE;
    KnownZero=(kind==LAZY_ZERO);
    mt_tensor own;
    own.p=static_cast<float*>(DeviceItem.get());
    own.w=Size_W;own.z=Size_Z;own.y=Size_Y;own.x=Size_X;
+   if (kind==LAZY_UPSAMPLING)
+   {
+    // (the sizes of the source as it was: the tensor may have been reinterpreted since)
+    own.w=up->SourceTensor.w;own.z=up->SourceTensor.z;own.y=up->SourceTensor.y*up->Factor_Y;own.x=up->SourceTensor.x*up->Factor_X;
+    mi355::Check(mt_upsampling(&own,&up->SourceTensor,up->Factor_X,up->Factor_Y));
+    return;
+   }
    if (kind==LAZY_ZERO)
    {
     mi355::Check(mt_fill(&own,0));
@@ -577,7 +600,23 @@ class CTensor
    DeviceOnChange=cTensor.DeviceOnChange;
    KnownZero=cTensor.KnownZero;
   }
-  void DropLazy(void) const {Lazy=LAZY_NONE;Deferred.reset();}
+  void DropLazy(void) const {Lazy=LAZY_NONE;Deferred.reset();DeferredUpSampling.reset();}
+  // the device copy is said to hold `source` up-sampled by the factors; nothing is launched (CTensorMath::UpSampling)
+  void SetLazyUpSampling(const mi355::CDeviceBuffer &source,const mt_tensor &source_tensor,uint32_t factor_x,uint32_t factor_y) const
+  {
+   DeviceItem.Own(false);
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),false,true);
+   DropLazy();
+   std::shared_ptr<mi355::CDeferredUpSampling> record(new mi355::CDeferredUpSampling);
+   record->Source=source;
+   record->SourceTensor=source_tensor;
+   record->Factor_X=factor_x;record->Factor_Y=factor_y;
+   DeferredUpSampling=record;
+   Lazy=LAZY_UPSAMPLING;
+   DeviceOnChange=true;
+   HostOnChange=false;
+   KnownZero=false;
+  }
   // the device copy is said to hold zeros; nothing is launched (CTensorMath::Fill)
   void SetLazyZero(void) const
   {

@@ -28,6 +28,20 @@ class CTensorConv
   static void ForwardConvolution(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Image,const CTensor<type_t> &cTensor_Kernel,int32_t kernel_x,int32_t kernel_y,int32_t kernel_z,uint32_t kernel_amount,const CTensor<type_t> &cTensor_Bias,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)
   {
    OnlyFloat();
+   if (cTensor_Image.Lazy==CTensor<type_t>::LAZY_UPSAMPLING && &cTensor_Output!=&cTensor_Image && kernel_x==3 && kernel_y==3 && stride_x==1 && stride_y==1 && padding_x==1 && padding_y==1)
+   {
+    // the image was never written: the convolution of the up-sampled image from its source (mi355::CDeferredUpSampling)
+    const std::shared_ptr<mi355::CDeferredUpSampling> up=cTensor_Image.DeferredUpSampling;///<(kept alive over the call)
+    const mt_tensor &source=up->SourceTensor;
+    if (up->Factor_X==2 && up->Factor_Y==2 && cTensor_Image.GetSizeW()==source.w && cTensor_Image.GetSizeZ()==source.z &&
+        cTensor_Image.GetSizeY()==2*source.y && cTensor_Image.GetSizeX()==2*source.x && source.z==static_cast<uint32_t>(kernel_z))
+    {
+     mt_tensor k=cTensor_Kernel.DeviceRead(),b=cTensor_Bias.DeviceRead(),o=cTensor_Output.Device(false);
+     mi355::Check(mt_upsampling_convolution_func(&o,&source,2,2,&k,kernel_x,kernel_y,kernel_z,kernel_amount,&b,stride_x,stride_y,padding_x,padding_y,MT_F_NONE));
+     cTensor_Output.SetDeviceOnChange();
+     return;
+    }
+   }
    mt_tensor i=cTensor_Image.DeviceRead(),k=cTensor_Kernel.DeviceRead(),b=cTensor_Bias.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_forward_convolution(&o,&i,&k,kernel_x,kernel_y,kernel_z,kernel_amount,&b,stride_x,stride_y,padding_x,padding_y));
    cTensor_Output.SetDeviceOnChange();

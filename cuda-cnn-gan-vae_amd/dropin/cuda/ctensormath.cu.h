@@ -207,6 +207,15 @@ class CTensorMath
   static void UpSampling(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Input,uint32_t upsampling_x,uint32_t upsampling_y)
   {
    OnlyFloat();
+   if (mi355::DeferGradients()==true && upsampling_x==2 && upsampling_y==2 && &cTensor_Output!=&cTensor_Input &&
+       cTensor_Output.GetSizeW()==cTensor_Input.GetSizeW() && cTensor_Output.GetSizeZ()==cTensor_Input.GetSizeZ() &&
+       cTensor_Output.GetSizeY()==2*cTensor_Input.GetSizeY() && cTensor_Output.GetSizeX()==2*cTensor_Input.GetSizeX())
+   {
+    // written when somebody asks for it; a 3x3 convolution that follows never does (mi355::CDeferredUpSampling)
+    mt_tensor source=cTensor_Input.DeviceRead();
+    cTensor_Output.SetLazyUpSampling(cTensor_Input.DeviceItem,source,upsampling_x,upsampling_y);
+    return;
+   }
    mt_tensor i=cTensor_Input.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_upsampling(&o,&i,upsampling_x,upsampling_y));
    cTensor_Output.SetDeviceOnChange();

@@ -14,6 +14,9 @@
 // Chain C: input [B,4,5,5]   -> BatchNormalization (training) -> ReLU            (layers_mi355 only: the reference's
 //          batch-norm layer does not compile on its own CPU classes, netlayer/cnetlayerbatchnormalization.cu.h:655)
 // Chain D: input [B,4,4,4]   -> UpSampling 2x2 -> AveragePooling 4x4, forward and backward
+// Chain U: input [B,16,6,8]  -> UpSampling 2x2 -> Convolution 8 x 3x3 s1 p1 -> LeakyReLU, two training steps (a layer pair of the
+//          reference's GAN generator, cuda/netmodel/cmodel_gan.cu.h:153-170: the drop-in classes compute the convolution from
+//          the input of the up-sampling layer and write the up-sampled image only for the weight gradient)
 // Chain E: inputs [B,2,4,4] and [B,3,4,4] -> Concatenator -> TimeEmbedding       (layers_mi355 only: ConcatecationZ and
 //          SetTimeStep exist in the reference's GPU tensor class only)
 // Chain F: input [B,4,8,8]   -> Linear function -> MaxPooling 2x2, forward and backward           (layers_mi355 only: the layer names the
@@ -23,8 +26,9 @@
 //          from the outputs and checks the rest against them); MaxDePooling
 // "deferred" as the second argument (layers_mi355 only): chain K, two training steps of the DCGAN-64 discriminator at batch
 //          16 with and without the drop-in classes' deferral of the per-sample weight gradients
-// "time" as the second argument (layers_mi355 only): the DCGAN-64 generator's forward pass at batch 256 and the
-//          discriminator's training step at batch 128 on the reference's layer classes, timed with the drop-in CTimeStamp
+// "time" as the second argument (layers_mi355 only): the DCGAN-64 generator's forward pass at batch 256, the
+//          discriminator's training step at batch 128 and the forward pass of the reference's own GAN generator (192x256
+//          images, batch 32) on the reference's layer classes, timed with the drop-in CTimeStamp
 // Each chain: TrainingStart, Forward, SetOutputError, TrainingBackward, TrainingUpdateWeight (gradient descent), Save.
 // SYSTEM::PutMessage* come from the reference's own system/system.cpp, compiled beside this file.
 #include <math.h>
@@ -343,6 +347,42 @@ static void ChainD(void)
  DumpRaw("D.net_stream",net_saved);
 }
 
+static void ChainU(void)
+{
+ CNetLayerConvolutionInput<type_t> input(16,6,8,BATCH);
+ CNetLayerUpSampling<type_t> up(2,2,&input,BATCH);
+ CNetLayerConvolution<type_t> conv(8,3,1,1,1,1,&up,BATCH);
+ CNetLayerFunction<type_t> f(NNeuron::NEURON_FUNCTION_LEAKY_RELU,&conv,BATCH);
+ CMemoryStream conv_w;
+ conv_w.SaveUInt32(8);conv_w.SaveInt32(3);conv_w.SaveInt32(3);conv_w.SaveInt32(16);conv_w.SaveInt32(1);conv_w.SaveInt32(1);conv_w.SaveInt32(1);conv_w.SaveInt32(1);
+ conv_w.PutTensor(1,1,8,16*9,Values(8*144,0.15));
+ conv_w.PutTensor(1,8,1,1,Values(8,0.1));
+ conv.Load(&conv_w);
+ CTensor<type_t> image(BATCH,16,6,8),error(BATCH,8,12,16);
+ INetLayer<type_t> *layers[4]={&input,&up,&conv,&f};
+ for(int n=0;n<4;n++) layers[n]->TrainingStart();
+ for(int step=0;step<2;step++)
+ {
+  FillTensor(image,1.0+step);
+  input.SetOutput(image);
+  for(int n=0;n<4;n++) layers[n]->TrainingResetDeltaWeight();
+  for(int n=0;n<4;n++) layers[n]->Forward();
+  const std::string tag=std::string("U.")+(step==0?"first.":"second.");
+  Dump((tag+"conv").c_str(),conv.GetOutputTensor());
+  Dump((tag+"leaky").c_str(),f.GetOutputTensor());
+  FillTensor(error,0.5);
+  f.SetOutputError(error);
+  for(int n=3;n>=1;n--) layers[n]->TrainingBackward(true);
+  Dump((tag+"delta_conv").c_str(),conv.GetDeltaTensor());
+  Dump((tag+"delta_upsampling").c_str(),up.GetDeltaTensor());
+  for(int n=1;n<4;n++) layers[n]->TrainingUpdateWeight(0.05,step+1);
+  CMemoryStream saved;
+  conv.Save(&saved);
+  DumpStream((tag+"conv_updated").c_str(),saved,8*sizeof(int32_t),2);
+ }
+ Dump("U.upsampling",up.GetOutputTensor());   // read at last: whoever asks for the up-sampled image gets it
+}
+
 
 // Chain H: layers that work on the host, element by element
 static void ChainH(void)
@@ -604,6 +644,61 @@ static void TimeGenerator(uint32_t batch,uint32_t warmup,uint32_t steps)
         batch,steps,ms,image.GetSizeW(),image.GetSizeZ(),image.GetSizeY(),image.GetSizeX(),sum,driver_allocations_in_the_timed_steps);
 }
 
+// The generator of the reference's GAN model (cuda/netmodel/cmodel_gan.cu.h:136-225), forward pass in training mode, batch 32:
+// Linear 1024 -> 512x3x4, leaky ReLU, six times (UpSampling 2x2, Convolution 3x3, BatchNormalization, leaky ReLU) through
+// 512, 256, 128, 64, 32, 16 channels, Convolution 3x3 to 3 channels, Tangence: 192x256 images
+static void TimeGanGenerator(uint32_t batch,uint32_t warmup,uint32_t steps)
+{
+ static const uint32_t channels[8]={512,512,256,128,64,32,16,3};
+ rng_state=0x243F6A8885A308D3ull;   // the same weights and latent vectors on every call (the chain may run twice)
+ std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
+ std::vector<INetLayer<type_t>*> net;
+ PUSH(new CNetLayerLinear<type_t>(1024,NULL,batch));
+ PUSH(new CNetLayerLinear<type_t>(channels[0]*12,net.back(),batch));
+ {
+  CMemoryStream w;
+  w.PutTensor(1,1,channels[0]*12,1024,Values(static_cast<size_t>(channels[0])*12*1024,0.025));
+  w.PutTensor(1,1,channels[0]*12,1,std::vector<double>(channels[0]*12,0.1));
+  net.back()->Load(&w);
+ }
+ PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_LEAKY_RELU,net.back(),batch));
+ // the first up-sampling layer takes the vector as [512,3,4]: it remembers the shape it was constructed on and reinterprets
+ // its input to it in every Forward (netlayer/cnetlayerupsampling.cu.h:243-252)
+ INetLayer<type_t> *function=net.back();
+ function->GetOutputTensor().ReinterpretSize(batch,channels[0],3,4);
+ for(uint32_t i=0;i<7;i++)
+ {
+  if (i<6) PUSH(new CNetLayerUpSampling<type_t>(2,2,net.back(),batch));
+  if (i==0) function->GetOutputTensor().ReinterpretSize(batch,1,channels[0]*12,1);
+  PUSH(new CNetLayerConvolution<type_t>(channels[i+1],3,1,1,1,1,net.back(),batch));
+  {
+   const uint32_t columns=channels[i]*9;
+   CMemoryStream w;
+   w.SaveUInt32(channels[i+1]);w.SaveInt32(3);w.SaveInt32(3);w.SaveInt32(channels[i]);w.SaveInt32(1);w.SaveInt32(1);w.SaveInt32(1);w.SaveInt32(1);
+   w.PutTensor(1,1,channels[i+1],columns,Values(static_cast<size_t>(channels[i+1])*columns,sqrt(6.0/columns)));
+   w.PutTensor(1,channels[i+1],1,1,Values(channels[i+1],0.05));
+   net.back()->Load(&w);
+  }
+  if (i<6)
+  {
+   PUSH(new CNetLayerBatchNormalization<type_t>(0.9f,net.back(),batch));
+   net.back()->Reset();
+   PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_LEAKY_RELU,net.back(),batch));
+  }
+ }
+ PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_TANGENCE,net.back(),batch));
+ CTensor<type_t> latent(batch,1,1024,1);
+ FillTensor(latent,1.0);
+ net[0]->SetOutput(latent);
+ for(size_t n=0;n<net.size();n++) net[n]->TrainingStart();
+ double ms=TimeSteps("GAN generator forward",net,NULL,warmup,steps);
+ CTensor<type_t> &image=net.back()->GetOutputTensor();
+ double sum=0;
+ for(uint32_t x=0;x<256;x++) sum+=fabs(image.GetElement(batch-1,2,191,x));
+ printf("{\"chain\": \"gan_generator_forward\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"last_row_abs_sum\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
+        batch,steps,ms,image.GetSizeW(),image.GetSizeZ(),image.GetSizeY(),image.GetSizeX(),sum,driver_allocations_in_the_timed_steps);
+}
+
 // DCGAN-64 discriminator, whole training step (forward, backward with weight gradients, Adam), batch 128
 // the discriminator's layers with seeded weights, in training mode (Adam or plain gradient descent)
 static void BuildDiscriminator(uint32_t batch,std::vector<std::shared_ptr<INetLayer<type_t> > > &owner,std::vector<INetLayer<type_t>*> &net,bool adam=true)
@@ -787,11 +882,18 @@ int main(int argc,char **argv)
    fclose(out_file);
    return(0);
   }
-  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up]]
+  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up [literal]]]
   {
    const uint32_t steps=(argc>3)?static_cast<uint32_t>(atoi(argv[3])):50,warmup=(argc>4)?static_cast<uint32_t>(atoi(argv[4])):20;
    TimeGenerator(256,warmup,steps);
    TimeDiscriminator(128,warmup,steps);
+   TimeGanGenerator(32,warmup,steps);
+   if (argc>5 && strcmp(argv[5],"literal")==0)   // and the last chain once more with every call run when it is made
+   {
+    mi355::DeferGradients()=false;
+    TimeGanGenerator(32,warmup,steps);
+    mi355::DeferGradients()=true;
+   }
    fclose(out_file);
    return(0);
   }
@@ -805,6 +907,7 @@ int main(int argc,char **argv)
   ChainA();
   ChainB();
   ChainD();
+  ChainU();
   ChainH();
 #ifndef USE_CPU
   ChainC();

@@ -43,7 +43,7 @@ def test_cpp_selftest_on_the_dropin_classes():
     run = subprocess.run([SELFTEST], capture_output=True, text=True, timeout=120)
     print(run.stdout[-3000:], run.stderr[-2000:])
     assert run.returncode == 0 and "ALL PASS" in run.stdout and "FAIL" not in run.stdout
-    assert run.stdout.count("PASS") >= 27
+    assert run.stdout.count("PASS") >= 32
 
 
 @pytest.fixture(scope="module")
@@ -183,6 +183,22 @@ def test_reference_layers_averaged_weights_on_the_dropin_classes(dumps):
     for got, w0, w1 in zip((beta, gamma, mean, variable), loaded, trained[:4]):
         assert np.abs(w1 - w0).max() > 1e-3
         assert rel_err(got, k * w0 + (np.float32(1) - k) * w1) <= 1e-6
+
+
+def test_reference_gan_generator_with_deferred_upsampling(tmp_path):
+    """The generator of the reference's GAN model on its own layer classes (six times UpSampling 2x2 + Convolution 3x3):
+    the drop-in classes compute each convolution from the up-sampling layer's input; the images are those of the run
+    with every call made at once (same weights: a row of the last image summed, 256 values after seven layers)."""
+    import json
+    if not os.path.exists(LAYERS_GPU):
+        pytest.skip("oracle/_ref/layers_mi355 not built (it needs /root/reference)")
+    run = subprocess.run([LAYERS_GPU, str(tmp_path / "t.bin"), "time", "2", "1", "literal"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr + run.stdout[-2000:]
+    lines = [json.loads(l) for l in run.stdout.splitlines() if l.startswith("{")]
+    gan = [l for l in lines if l["chain"] == "gan_generator_forward"]
+    assert len(gan) == 2 and gan[0]["output"] == [32, 3, 192, 256]
+    deferred, literal = gan[0]["last_row_abs_sum"], gan[1]["last_row_abs_sum"]
+    assert literal > 1.0 and abs(deferred - literal) <= 1e-5 * literal
 
 
 def test_deferred_weight_gradients_in_the_reference_layers(tmp_path):
