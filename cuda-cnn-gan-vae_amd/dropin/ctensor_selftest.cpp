@@ -646,6 +646,34 @@ static void FusedSequenceChecks(void)
   ok=fj.Agrees(ej,2e-5) && ok;
   snprintf(name,sizeof(name),"function layer forward behind the batch-norm layer's as one kernel, batch %u",d[0]);
   Report(name,ok);
+  // Forward passes on their own: the batch-norm layer's own output is not written (pending, then dropped by the next
+  // pass); a reader gets it from its two calls, and from then on the kernel writes it.
+  {
+   mi355::FuseSequences()=false;
+   SBatchNormTensors ek(d[0],d[1],d[2],d[3]);
+   ek.ForwardTraining();ek.Function(true);
+   mi355::FuseSequences()=true;
+   SBatchNormTensors fk(d[0],d[1],d[2],d[3]);
+   const size_t kept=queue.OwnOutputsPending,ran=queue.PendingRun;
+   for(int pass=0;pass<3;pass++) {fk.ForwardTraining();fk.Function(true);}
+   queue.Flush();
+   ok=queue.OwnOutputsPending==kept+3 && queue.PendingRun==ran;
+   double largest=0;
+   ok=ok && MaxDifference(fk.F,ek.F,largest)<=2e-5*largest;
+   ok=ok && MaxDifference(fk.H,ek.H,largest)<=2e-5*largest && queue.PendingRun>ran;   // the reader: the two calls run now
+   const size_t kept2=queue.OwnOutputsPending;
+   fk.ForwardTraining();fk.Function(true);
+   queue.Flush();
+   ok=ok && queue.OwnOutputsPending==kept2 && MaxDifference(fk.H,ek.H,largest)<=2e-5*largest && MaxDifference(fk.F,ek.F,largest)<=2e-5*largest;
+   // the optimiser's write to Gamma reaches a pending output before the new values do
+   SBatchNormTensors fl(d[0],d[1],d[2],d[3]);
+   fl.ForwardTraining();fl.Function(true);
+   queue.Flush();
+   CTensorMath<type_t>::Mul(fl.Gamma,fl.Gamma,static_cast<type_t>(3));
+   ok=ok && MaxDifference(fl.H,ek.H,largest)<=2e-5*largest;
+   snprintf(name,sizeof(name),"the batch-norm layer's own output behind a fused forward pass, batch %u",d[0]);
+   Report(name,ok);
+  }
   // inference mode, twice (the scratch tensors of the first pass are overwritten unread by the second)
   mi355::FuseSequences()=false;
   SBatchNormTensors ei(d[0],d[1],d[2],d[3]);

@@ -60,13 +60,14 @@ namespace mi355
   int Func;///<OP_FUNCTION: the function applied; OP_DIFFERENTIAL: the function whose derivative is applied (MT_F_*)
   uint32_t BatchSize;
   double Speed,Beta1,Beta2,Epsilon,Iteration;
+  uint8_t Own;///<1: writes a batch-norm layer's own output that a fused forward pass left pending (COpQueue::RunForward)
  };
 
  inline SOp MakeOp(int kind,uint8_t count,uint8_t reads,uint8_t writes,float a=0,float b=0)
  {
   SOp op;
   op.Kind=kind;op.Count=count;op.Reads=reads;op.Writes=writes;op.A=a;op.B=b;op.Func=MT_F_NONE;
-  op.BatchSize=0;op.Speed=0;op.Beta1=0;op.Beta2=0;op.Epsilon=0;op.Iteration=0;
+  op.BatchSize=0;op.Speed=0;op.Beta1=0;op.Beta2=0;op.Epsilon=0;op.Iteration=0;op.Own=0;
   for(int n=0;n<4;n++) {op.T[n].p=NULL;op.T[n].w=0;op.T[n].z=0;op.T[n].y=0;op.T[n].x=0;}
   return(op);
  }
@@ -389,10 +390,11 @@ namespace mi355
    // never name, to take the function's derivative at Gamma * XHat + Beta instead of reading Output.
    struct SNormFact {mt_tensor Output,Gamma,Beta,XHat;};
    std::vector<SNormFact> Facts;
+   std::vector<const void*> OwnOutputsRead;///<batch-norm outputs that were left pending once and had to be written after all
   public:
    // counters, for tests and measurements
-   size_t ForwardFused,InferenceFused,BackwardFused,FunctionBackwardFused,FillRuns,AdamRuns,RunCalls,LiteralCalls,PendingRun,PendingDropped;
-   COpQueue(void):ForwardFused(0),InferenceFused(0),BackwardFused(0),FunctionBackwardFused(0),FillRuns(0),AdamRuns(0),RunCalls(0),LiteralCalls(0),PendingRun(0),PendingDropped(0) {}
+   size_t ForwardFused,InferenceFused,BackwardFused,FunctionBackwardFused,FillRuns,AdamRuns,RunCalls,LiteralCalls,PendingRun,PendingDropped,OwnOutputsPending;
+   COpQueue(void):ForwardFused(0),InferenceFused(0),BackwardFused(0),FunctionBackwardFused(0),FillRuns(0),AdamRuns(0),RunCalls(0),LiteralCalls(0),PendingRun(0),PendingDropped(0),OwnOutputsPending(0) {}
 
    // a call of CTensorMath; operands are up to date on the device, the output is marked device-side by the caller
    void Submit(const SOp &op)
@@ -514,11 +516,26 @@ namespace mi355
    {
     Settle(&sequence[0],sequence.size());
     ForwardFused++;
-    // with the function layer's call behind it: both layers' outputs from the one kernel
-    if (m.HasFunction==true) Check(mt_batchnorm_forward_train_from(&m.F,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,&m.OldMean,&m.OldVar,m.Momentum,m.Epsilon,m.Func,&m.H));
+    // With the function layer's call behind it the kernel writes that layer's output.  The batch-norm layer's own output
+    // is one more store of the whole activation that a forward pass on its own never reads (the next layer takes the
+    // function's output, the next pass overwrites it): it stays pending as H = Gamma * XHat, H = H + Beta -- the layer's
+    // own two calls with H in place of the scratch tensor, which the backward pass reuses.  In a training loop the
+    // optimiser changes Gamma and Beta, and the pending calls have to run first: two launches instead of one store.  So
+    // an output whose pending calls ever ran is written by the kernel from then on (OwnOutputsRead).
+    const bool written=(m.HasFunction==false || WasRead(m.H.p)==true);
+    if (m.HasFunction==true) Check(mt_batchnorm_forward_train_from(&m.F,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,&m.OldMean,&m.OldVar,m.Momentum,m.Epsilon,m.Func,written==true?&m.H:NULL));
     else Check(mt_batchnorm_forward_train_from(&m.H,&m.X,&m.Gamma,&m.Beta,&m.XHat,&m.IVar,&m.Mean,&m.Var,&m.NewMean,&m.NewVar,&m.OldMean,&m.OldVar,m.Momentum,m.Epsilon,MT_F_NONE,NULL));
     Pending.push_back(sequence[8]);///<SqrtVar = sqrt(Var + epsilon)
     Pending.push_back(sequence[11]);///<Scratch = Gamma * XHat
+    if (written==false)
+    {
+     SOp product=sequence[11],sum=sequence[12];
+     product.T[0]=m.H;product.Own=1;
+     sum.T[1]=m.H;sum.Own=1;
+     Pending.push_back(product);
+     Pending.push_back(sum);
+     OwnOutputsPending++;
+    }
     SNormFact fact;
     fact.Output=m.H;fact.Gamma=m.Gamma;fact.Beta=m.Beta;fact.XHat=m.XHat;
     Facts.push_back(fact);
@@ -566,7 +583,7 @@ namespace mi355
      return;
     }
     const mt_tensor beta=fact->Beta;///<(Settle below may drop the record)
-    Settle(&sequence[0],sequence.size());
+    Settle(&sequence[0],sequence.size(),&m.Output);///<(the kernel does not read the function's input: it has Gamma, XHat and Beta)
     FunctionBackwardFused++;
     const SBatchNormBackward &b=m.Norm;
     Check(mt_batchnorm_backward_func_keep(&b.Prev,b.Gradients==true?&b.DGamma:NULL,b.Gradients==true?&b.DBeta:NULL,&m.Error,&b.Gamma,&beta,&b.XHat,&b.IVar,m.Func,&b.DXHat,&b.SumA,&b.SumB,&m.Front));
@@ -589,12 +606,20 @@ namespace mi355
     }
     state[j]=1;
     PendingRun++;
+    if (Pending[j].Own!=0 && WasRead(Pending[j].T[0].p)==false && OwnOutputsRead.size()<1024) OwnOutputsRead.push_back(Pending[j].T[0].p);
     RunLiteral(Pending[j]);
+   }
+   bool WasRead(const void *p) const
+   {
+    for(size_t i=0;i<OwnOutputsRead.size();i++)
+     if (OwnOutputsRead[i]==p) return(true);
+    return(false);
    }
    // Before `count` calls run as one unit (a sequence's kernel, a run, one literal call): pending calls whose output the
    // unit overwrites without anybody having read it are forgotten; those whose output the unit reads, or whose inputs
    // it changes, run first.
-   void Settle(const SOp *unit,size_t count)
+   // `unread`: a tensor that the unit's calls name as an input but the kernel that stands for them does not touch.
+   void Settle(const SOp *unit,size_t count,const mt_tensor *unread=NULL)
    {
     if (Facts.empty()==false)
     {
@@ -613,6 +638,7 @@ namespace mi355
      for(uint8_t t=0;t<o.Count;t++)
      {
       if ((o.Reads&(1u<<t))==0) continue;
+      if (unread!=NULL && Same(o.T[t],*unread)==true) continue;
       bool inside=false;
       for(size_t w=0;w<writes.size();w++)
        if (Covers(writes[w].p,Bytes(writes[w]),o.T[t])==true) inside=true;
