@@ -58,6 +58,7 @@ void count_driver_allocation();  // every hipMalloc of the library is counted (m
 // that writes device memory reports the range here (so does mt_invalidate for writers outside the library); copies
 // made from an overlapping range are then made again on their next use.
 void note_write(const void *p, size_t bytes);
+void forget_graph_writes(const void *p, size_t bytes);  // the block at p is released: recorded writes into it no longer count
 int add_sum_w_pair(float *out1, const float *r1, size_t S1, float *out2, const float *r2, size_t S2, uint32_t W);  // two batch sums, one launch
 int set_pack_cache(int on);
 int set_adam_vec(int v);      // mt_adam_many updates four elements per thread: 1 (default) in the tiles that also write a re-ordered copy, 2 wherever the tensors allow, 0 never (measurements only)

@@ -2163,6 +2163,18 @@ void pack_refresh_commit(const PackRefresh &r, const mt_tensor *const *weight, c
   e.valid = true;
   g_pack_refreshed++;
 }
+// A block goes back to the pool or the driver (not under capture): what recorded graphs write into it no longer matters
+// to the cache.  Replaying such a graph now would write into whoever owns the block next -- the caller's error, as
+// with any use of freed memory -- so nothing recorded can change what the next owner keeps there, and copies made of the
+// next owner's weights can be trusted again.
+void forget_graph_writes(const void *p, size_t bytes) {
+  if (p == nullptr || bytes == 0 || g_graph_written.empty()) return;
+  const uintptr_t lo = (uintptr_t)p, hi = lo + bytes < lo ? ~(uintptr_t)0 : lo + bytes;
+  size_t kept = 0;
+  for (size_t i = 0; i < g_graph_written.size(); i++)
+    if (!(lo <= g_graph_written[i].first && g_graph_written[i].second <= hi)) g_graph_written[kept++] = g_graph_written[i];
+  g_graph_written.resize(kept);
+}
 int set_pack_refresh(int v) {
   if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "pack_refresh must be 0 or 1");
   g_pack_refresh = v;

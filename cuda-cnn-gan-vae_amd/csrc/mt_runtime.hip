@@ -191,6 +191,7 @@ int mt_free(void *ptr) {
     g_retired_bytes += size;
     return MT_OK;
   }
+  mt::forget_graph_writes(ptr, size);
   if (g_pool_on && size && size <= POOL_LARGEST) {
     if (g_pool_bytes + size > g_pool_limit) { int rc = pool_release_all(); if (rc) return rc; }
     it->second.state = POOLED;

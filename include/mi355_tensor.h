@@ -151,7 +151,8 @@ int mt_set_option(const char *name, int value);
  *   "pack_cache_refreshed"                                 copies that an mt_adam_many call wrote itself (option "pack_refresh")
  *   "pack_cache_spare_bytes"                               buffers of evicted entries that a recorded graph still names
  *   "graph_written_ranges", "graph_writes_anything"        memory written by recorded calls: weights inside such a range
- *                                                          are re-ordered on every use; after 4096 ranges everything is
+ *                                                          are re-ordered on every use, until the block that holds the
+ *                                                          range is freed; after 4096 ranges everything is
  *                                                          (graph_writes_anything = 1, for the rest of the process)
  *   "wgrad_walk_launches"                                  calls of mt_convolution_backward_weights_sum that ran as one k loop
  *                                                          per block (option "wgrad_walk") */

@@ -217,6 +217,17 @@ def test_weights_that_a_recording_updates_are_never_trusted(mt):
         mt.set_option("pack_cache", 1)
         assert np.array_equal(eager, out.numpy()) and np.array_equal(replayed, eager)
         conv()
+    # Once the weights' block is given back, what the recording writes there no longer counts (replaying it now would be a
+    # use of freed memory): the next tensor at that address is trusted like any other.
+    ranges, address = mt.get_info("graph_written_ranges"), kernel.ptr.value
+    kernel.free()
+    assert mt.get_info("graph_written_ranges") < ranges
+    kernel = CTensor.from_numpy(Nrm(63, 1, 1, cin, cout * 16, std=0.05))
+    assert kernel.ptr.value == address, "the pool hands the freed block to the next tensor of the same size"
+    conv()
+    hits = mt.get_info("pack_cache_hits")
+    conv()
+    assert mt.get_info("pack_cache_hits") == hits + 1
 
 
 def test_pool_reuses_blocks_in_stream_order(mt):
