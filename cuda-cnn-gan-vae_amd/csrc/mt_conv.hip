@@ -33,6 +33,7 @@ int g_upconv_split = 1;    // 1: up-sampling convolutions with fewer than 512 wa
 int g_upconv_walk = 512;   // blocks from which the up-sampling convolution takes the walking kernel (0: never; measured on the
                            // shipped GAN generator at batch 32: 768 blocks 67.7 -> 54.6 and 58.6 -> 54.0 us, 384 blocks 65.1 -> 69 us)
 uint64_t g_wgrad_walk_launches = 0;
+int g_wgrad_parts = 1;   // 1: the general batch-summed weight gradient cuts samples into bands of output rows when samples x tiles are too few blocks, 0: never, n > 1: n bands
 int g_wgrad_walk = 1;    // 1: the batch-summed weight gradient runs as one k loop per block where its shape allows (wgrad_walk_kernel), 0: never
 int g_wgrad_groups = 0;  // 0 auto, else the number of batch groups of the batch-summed weight gradient (if it divides the batch)
 
@@ -1917,6 +1918,38 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     g_wgrad_walk_launches++;
     return mt::add_sum_w_pair(dk->p, partial, (size_t)ka * ncol, db->p, dbias_partial, ka, wa.groups);  // the groups in order, one launch for both
   }
+  // Few filters on large images (the last layers of a generator: 16 filters at 192 x 256) leave fewer tiles x samples than
+  // the chip has compute units even with one group per sample: the groups then become equal bands of output rows of one
+  // sample each (`parts` per sample), for the source that gathers with fixed offsets
+  uint32_t parts = 1;
+  if (g_wgrad_parts && groups == B && DHW % 4 == 0 && ((uintptr_t)delta->p & 15u) == 0 && dk->x == ncol && dk->z * dk->y == ka) {
+    const uint32_t OH = delta->y, OW = delta->x;
+    auto fits = [&](uint32_t n) {
+      return OH % n == 0 && ((OH / n) * OW) % BK == 0 && (OH / n) * OW >= 32u * BK && (size_t)B * n * ka * ncol <= ((size_t)1 << 26) &&
+             wgrad_image_fixed(ka, ncol, B * n, delta, image, kz, 1, px, py);
+    };
+    while ((size_t)tiles * B * parts < 1024 && parts < 256 && fits(parts * 2)) parts *= 2;
+    if (g_wgrad_parts > 1 && fits((uint32_t)g_wgrad_parts)) parts = (uint32_t)g_wgrad_parts;
+  }
+  if (parts > 1) {
+    const uint32_t total = B * parts, rows = delta->y / parts, chunk = rows * delta->x;
+    float *band_sums = nullptr;
+    if ((rc = workspace((size_t)total * ka * ncol + (chunks > 1 ? (size_t)ka * chunks : 0), &band_sums))) return rc;
+    SrcRowK<true> a{};
+    a.p = delta->p; a.ld = DHW; a.R = ka; a.K = chunk;
+    a.bt.wmod = B; a.bt.zcount = parts; a.bt.wstride = sample_delta; a.bt.stride = chunk;
+    SrcWgradImageFixed bf{};
+    bf.p = image->p; bf.C = kz; bf.H = image->y; bf.W = image->x; bf.KY = ky; bf.KX = kx; bf.OW = delta->x; bf.OH = 0; bf.R = ncol; bf.K = chunk;
+    bf.sy = sy; bf.sx = sx; bf.py = py; bf.px = px; bf.part_rows = rows;
+    bf.bt.wmod = B; bf.bt.zcount = parts; bf.bt.wstride = sample_image; bf.bt.stride = 0;
+    Epilogue ep{};
+    ep.inner = ncol; ep.g_stride = 0;
+    ep.C = band_sums; ep.row_stride = ncol; ep.bt.wmod = total; ep.bt.stride = (size_t)ka * ncol;
+    if ((rc = launch(name, a, bf, ep, ka, ncol, chunk, total))) return rc;
+    mt_tensor pt{band_sums, total, 1, ka, ncol}, flat{dk->p, 1, 1, ka, ncol};
+    if ((rc = mt_add_sum_w(&flat, &flat, &pt, 1.f, 1.f))) return rc;
+    return dbias_batch_sum(name, db->p, band_sums + (size_t)total * ka * ncol, delta->p, B, ka, DHW, chunks);
+  }
   SrcRowK<true> a{};
   a.p = delta->p; a.ld = DHW; a.R = ka; a.K = per * DHW; a.seg = DHW; a.seg_stride = (uint32_t)sample_delta;
   a.bt.wmod = groups; a.bt.stride = (size_t)per * sample_delta;
@@ -2280,6 +2313,11 @@ int set_upconv_split(int v) {
 int set_upconv_walk(int v) {
   if (v < 0) return fail(MT_E_ARGUMENT, "upconv_walk must be 0 (never) or the number of blocks from which the walking kernel is taken");
   g_upconv_walk = v;
+  return MT_OK;
+}
+int set_wgrad_parts(int v) {
+  if (v < 0 || v > 256) return fail(MT_E_ARGUMENT, "wgrad_parts must be 0 (never), 1 (choose) or the number of bands per sample (2..256)");
+  g_wgrad_parts = v;
   return MT_OK;
 }
 int set_wgrad_walk(int v) {

@@ -33,8 +33,10 @@ typedef float floatx4acc __attribute__((ext_vector_type(4)));
 struct Batch {
   uint32_t wmod = 1, zcount = 1;
   size_t stride = 0;
+  size_t wstride = 0;  // > 0: entry (w, z) lies at (w % wmod) * wstride + z * stride (parts of a sample that are not the whole sample)
   __device__ size_t offset(uint32_t bz) const {
     uint32_t w = bz / zcount, z = bz % zcount;
+    if (wstride) return (size_t)(w % wmod) * wstride + (size_t)z * stride;
     return (size_t)((w % wmod) * zcount + z) * stride;
   }
 };
@@ -438,15 +440,19 @@ struct SrcWgradImageFixed {
   int32_t sy, sx, py, px;
   Batch bt;
   uint32_t OH = 0;  // > 0: k runs over the pixels of several images in turn
+  uint32_t part_rows = 0;  // > 0: batch entry (w, z) covers the output rows z * part_rows .. of image w only (OH = 0 then)
   __amdgpu_buffer_rsrc_t rsrc;
   uint32_t voff;       // byte offset of the thread's first pixel for the block origin (image 0, row 0, column 0), from p - bias
   int32_t iyc, ixc;    // input row / column of that pixel for that origin
-  uint32_t oy, ox, woff, soff;
+  uint32_t oy, ox, woff, soff, oy0 = 0;
   int32_t Y, X;        // input row / column displacement of the current origin
   static __host__ __device__ bool fits(uint32_t OH_, uint32_t OW_, uint32_t e) {
     return OW_ % e == 0 && (OW_ % BK == 0 || (BK % OW_ == 0 && (OH_ * OW_) % BK == 0));
   }
-  __device__ void batch(uint32_t bz) { p += bt.offset(bz); }
+  __device__ void batch(uint32_t bz) {
+    p += bt.offset(bz);
+    if (part_rows) oy0 = (bz % bt.zcount) * part_rows;
+  }
   __device__ void bind(uint32_t row) {
     // offsets are taken from (py rows + px pixels) in front of the image so that none is negative; elements that would
     // lie in front of the image are masked before they are loaded
@@ -464,7 +470,9 @@ struct SrcWgradImageFixed {
     voff += (dy * (uint32_t)sy * W + dx * (uint32_t)sx) * 4u;
     iyc += (int32_t)dy * sy;
     ixc += (int32_t)dx * sx;
-    oy = 0; ox = 0; woff = 0; soff = 0; Y = 0; X = 0;
+    oy = oy0; ox = 0; woff = 0; X = 0;
+    Y = (int32_t)oy * sy;
+    soff = (uint32_t)Y * W * 4u;
   }
   template <int E>
   __device__ void next() {

@@ -22,7 +22,9 @@ class CTensorConv
    const uint32_t batch=dkernel.GetSizeW();
    if (batch<2 || dbias.GetSizeW()!=batch || image.GetSizeW()!=batch || delta.GetSizeW()!=batch) return(false);
    if (dbias.GetSizeY()!=1 || dbias.GetSizeX()!=1) return(false);
-   return(dkernel.Count()>=(static_cast<size_t>(1)<<16));
+   // (... or enough pixels: a layer with few filters on large images, whose per-sample gradients are small but each of
+   // them is a sum over a whole image -- summed over the batch directly, that work spreads over the chip)
+   return(dkernel.Count()>=(static_cast<size_t>(1)<<16) || delta.Count()>=(static_cast<size_t>(1)<<20));
   }
  public:
   static void ForwardConvolution(CTensor<type_t> &cTensor_Output,const CTensor<type_t> &cTensor_Image,const CTensor<type_t> &cTensor_Kernel,int32_t kernel_x,int32_t kernel_y,int32_t kernel_z,uint32_t kernel_amount,const CTensor<type_t> &cTensor_Bias,int32_t stride_x,int32_t stride_y,int32_t padding_x,int32_t padding_y)

@@ -104,6 +104,9 @@ int mt_timer_destroy(void *timer);
  *   "patch_blocks"   persistent blocks of the input-patch transposed convolution (default 512, two per compute unit)
  *   "wgrad_groups"   0 (default) choose per shape / n split the batch of mt_convolution_backward_weights_sum into n groups
  *                    (when n divides the batch)
+ *   "wgrad_parts"    1 (default) the general kernel of mt_convolution_backward_weights_sum cuts every sample into equal bands of
+ *                    output rows (one partial sum per band) when samples x tiles are fewer blocks than the chip needs: layers
+ *                    with few filters on large images / 0 never / n bands per sample (2..256, where the rows divide)
  *   "pack_cache"     1 (default) keep re-ordered weights between calls / 0 re-order on every call
  *   "tconv_walk"     1 (default) plain transposed convolutions use the kernel whose blocks walk over the batch wherever
  *                    the shape allows / 0 never

@@ -28,7 +28,8 @@
 //          16 with and without the drop-in classes' deferral of the per-sample weight gradients
 // "time" as the second argument (layers_mi355 only): the DCGAN-64 generator's forward pass at batch 256, the
 //          discriminator's training step at batch 128 and the forward pass of the reference's own GAN generator (192x256
-//          images, batch 32) on the reference's layer classes, timed with the drop-in CTimeStamp
+//          images, batch 32) on the reference's layer classes, timed with the drop-in CTimeStamp; a fifth argument "literal"
+//          repeats the last chain with every call run when it is made, "train" adds that generator's whole training step
 // Each chain: TrainingStart, Forward, SetOutputError, TrainingBackward, TrainingUpdateWeight (gradient descent), Save.
 // SYSTEM::PutMessage* come from the reference's own system/system.cpp, compiled beside this file.
 #include <math.h>
@@ -647,7 +648,7 @@ static void TimeGenerator(uint32_t batch,uint32_t warmup,uint32_t steps)
 // The generator of the reference's GAN model (cuda/netmodel/cmodel_gan.cu.h:136-225), forward pass in training mode, batch 32:
 // Linear 1024 -> 512x3x4, leaky ReLU, six times (UpSampling 2x2, Convolution 3x3, BatchNormalization, leaky ReLU) through
 // 512, 256, 128, 64, 32, 16 channels, Convolution 3x3 to 3 channels, Tangence: 192x256 images
-static void TimeGanGenerator(uint32_t batch,uint32_t warmup,uint32_t steps)
+static void TimeGanGenerator(uint32_t batch,uint32_t warmup,uint32_t steps,bool train=false)
 {
  static const uint32_t channels[8]={512,512,256,128,64,32,16,3};
  rng_state=0x243F6A8885A308D3ull;   // the same weights and latent vectors on every call (the chain may run twice)
@@ -691,10 +692,18 @@ static void TimeGanGenerator(uint32_t batch,uint32_t warmup,uint32_t steps)
  FillTensor(latent,1.0);
  net[0]->SetOutput(latent);
  for(size_t n=0;n<net.size();n++) net[n]->TrainingStart();
- double ms=TimeSteps("GAN generator forward",net,NULL,warmup,steps);
+ CTensor<type_t> error(batch,3,192,256);
+ if (train==true) FillTensor(error,0.01);
+ double ms=TimeSteps(train==true?"GAN generator step":"GAN generator forward",net,train==true?&error:NULL,warmup,steps);
  CTensor<type_t> &image=net.back()->GetOutputTensor();
  double sum=0;
  for(uint32_t x=0;x<256;x++) sum+=fabs(image.GetElement(batch-1,2,191,x));
+ if (train==true)
+ {
+  printf("{\"chain\": \"gan_generator_step\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"last_row_abs_sum\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
+         batch,steps,ms,image.GetSizeW(),image.GetSizeZ(),image.GetSizeY(),image.GetSizeX(),sum,driver_allocations_in_the_timed_steps);
+  return;
+ }
  printf("{\"chain\": \"gan_generator_forward\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"last_row_abs_sum\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
         batch,steps,ms,image.GetSizeW(),image.GetSizeZ(),image.GetSizeY(),image.GetSizeX(),sum,driver_allocations_in_the_timed_steps);
 }
@@ -882,12 +891,13 @@ int main(int argc,char **argv)
    fclose(out_file);
    return(0);
   }
-  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up [literal]]]
+  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up [literal | train]]]
   {
    const uint32_t steps=(argc>3)?static_cast<uint32_t>(atoi(argv[3])):50,warmup=(argc>4)?static_cast<uint32_t>(atoi(argv[4])):20;
    TimeGenerator(256,warmup,steps);
    TimeDiscriminator(128,warmup,steps);
    TimeGanGenerator(32,warmup,steps);
+   if (argc>5 && strcmp(argv[5],"train")==0) TimeGanGenerator(32,warmup,steps,true);   // and its whole training step (forward, backward, Adam)
    if (argc>5 && strcmp(argv[5],"literal")==0)   // and the last chain once more with every call run when it is made
    {
     mi355::DeferGradients()=false;

@@ -402,6 +402,36 @@ def test_convolution_backward_weights_sum(gpu, oracle, path, case):
 
 
 @pytest.mark.parametrize("case", [
+    # B, C, H, W, KA, k, s, p, bands
+    (2, 8, 64, 64, 16, 3, 1, 1, 1),      # 16 filters at 64 x 64: the library's choice (8 bands of 8 rows)
+    (2, 8, 64, 64, 16, 3, 1, 1, 4),      # four bands of 16 rows
+    (3, 16, 32, 64, 32, 3, 1, 1, 2),     # 32 filters, rows of 64 pixels, two bands
+    (2, 4, 64, 32, 3, 3, 1, 1, 4),       # 3 filters (an image layer), rows of 32 pixels
+    (4, 16, 64, 64, 16, 5, 2, 2, 2),     # 5 x 5 stride 2 padding 2: 32 x 32 output pixels
+    (2, 8, 48, 16, 24, 4, 2, 1, 3),      # 24 rows of 8 output pixels in three bands
+    (5, 8, 32, 32, 16, 3, 1, 1, 0),      # bands switched off: one group per sample
+])
+def test_weights_sum_in_bands_of_rows(gpu, oracle, case):
+    """The batch-summed weight gradient of layers with few filters on large images: the general kernel with every sample cut
+    into bands of output rows (one partial sum per band), against the layer's own sequence on the oracle."""
+    import mi355tensor as mt
+    B, C, H, Wd, KA, k, s, p, bands = case
+    oy, ox = (H - k + 2 * p) // s + 1, (Wd - k + 2 * p) // s + 1
+    image, delta = U(41, B, C, H, Wd), U(42, B, KA, oy, ox)
+    dk0, db0 = U(43, 1, 1, KA, C * k * k), U(44, 1, KA, 1, 1)
+    dkb, dbb = oracle.create_delta_weight_and_bias(np.zeros((B, 1, KA, C * k * k), np.float32), np.zeros((B, KA, 1, 1), np.float32),
+                                                   image, delta, k, k, C, KA, s, s, p, p)
+    want_k, want_b = oracle.add_sum_w(dk0, dkb, out_init=dk0), oracle.add_sum_w(db0, dbb, out_init=db0)
+    mt.set_option("wgrad_parts", bands)
+    try:
+        got_k, got_b = gpu.convolution_backward_weights_sum(dk0, db0, image, delta, k, k, C, KA, s, s, p, p)
+    finally:
+        mt.set_option("wgrad_parts", 1)
+    close(got_k, want_k)
+    close(got_b, want_b)
+
+
+@pytest.mark.parametrize("case", [
     # B, C, H, W, KA, k, s, p, groups
     (16, 64, 32, 32, 128, 4, 2, 1, 0),   # output rows of 16 pixels: a k step is one row
     (16, 32, 16, 16, 64, 4, 2, 1, 0),    # rows of 8 pixels: two rows per k step, four steps per sample
