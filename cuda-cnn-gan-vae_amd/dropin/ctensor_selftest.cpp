@@ -548,6 +548,46 @@ static void DeferredUpSamplingChecks(void)
  Report("other kernels, copies, writes and factors",ok);
 }
 
+// The linear layer's weight gradient: per-sample outer products, then their sum over the batch (netlayer/cnetlayerlinear.cu.h:
+// 436-444).  The products are not computed; their sum is one product over the batch.
+static void DeferredProductChecks(void)
+{
+ const uint32_t batch=8,m=64,n=160;
+ CTensor<type_t> delta(batch,1,m,1),input(batch,1,1,n),products(batch,1,m,n),control_products(batch,1,m,n),dw(1,1,m,n),control_dw(1,1,m,n);
+ FillPattern(delta,31,1.0f);FillPattern(input,37,1.0f);FillPattern(dw,41,0.5f);
+ control_dw=dw;
+ mi355::DeferGradients()=false;   // every call when it is made
+ CTensorMath<type_t>::Mul(control_products,delta,input);
+ CTensorMath<type_t>::AddSumW(control_dw,control_dw,control_products);
+ mi355::DeferGradients()=true;
+ CTensorMath<type_t>::Mul(products,delta,input);
+ CTensor<type_t> kept=delta;
+ CTensorMath<type_t>::Fill(delta,3);   // an operand changes after the call: the products are those of the values it had
+ CTensorMath<type_t>::AddSumW(dw,dw,products);
+ double largest=0;
+ bool ok=MaxDifference(dw,control_dw,largest)<=1e-5*largest && largest>1;
+ Report("sum over the batch of per-sample outer products that were never computed",ok);
+ ok=MaxDifference(products,control_products,largest)==0;   // a reader: the products themselves, bit for bit
+ // other shapes and small products run at once; a scaled sum takes the products
+ CTensor<type_t> small(batch,1,4,8),column(batch,1,4,1),row(batch,1,1,8),sum(1,1,4,8),control_sum(1,1,4,8);
+ FillPattern(column,43,1.0f);FillPattern(row,47,1.0f);
+ CTensorMath<type_t>::Mul(small,column,row);
+ CTensorMath<type_t>::Fill(sum,0);
+ CTensorMath<type_t>::AddSumW(sum,sum,small);
+ for(uint32_t y=0;y<4;y++)
+  for(uint32_t x=0;x<8;x++)
+  {
+   double expected=0;
+   for(uint32_t w=0;w<batch;w++) expected+=static_cast<double>(column.GetElement(w,0,y,0))*row.GetElement(w,0,0,x);
+   ok=ok && fabs(sum.GetElement(0,0,y,x)-expected)<=1e-5*(1+fabs(expected));
+  }
+ CTensorMath<type_t>::Mul(products,kept,input);
+ CTensorMath<type_t>::AddSumW(dw,control_dw,products,0.5f,2.0f);   // not the layer's call: out = 0.5 control_dw + 2 sum
+ CTensorMath<type_t>::AddSumW(control_dw,control_dw,control_products,0.5f,2.0f);
+ ok=ok && MaxDifference(dw,control_dw,largest)<=1e-5*largest;
+ Report("readers of the products, small products, scaled sums",ok);
+}
+
 static void FusedSequenceChecks(void)
 {
  mi355::COpQueue &queue=mi355::Queue();
@@ -801,6 +841,7 @@ int main(void)
   ZeroBiasCheck();
   DeferredGradientChecks();
   DeferredUpSamplingChecks();
+  DeferredProductChecks();
   FusedSequenceChecks();
   SharedBlockChecks();
   SummXYCheck();

@@ -174,6 +174,17 @@ namespace mi355
   uint32_t Factor_X;
   uint32_t Factor_Y;
  };
+ // Per-sample outer products that were not computed (CTensorMath::Mul of a column [B,1,M,1] by a row [B,1,1,N]): the
+ // linear layer forms its weight gradient that way and sums it over the batch at once (netlayer/cnetlayerlinear.cu.h:
+ // 436-444), B x M x N values written and read back for an M x N result.  AddSumW of such a tensor onto the layer's
+ // gradient is one product over the batch instead, columns^T x rows; any other reader gets the products computed.
+ struct CDeferredProduct
+ {
+  CDeviceBuffer Left;
+  CDeviceBuffer Right;
+  mt_tensor LeftTensor;
+  mt_tensor RightTensor;
+ };
  // switch for the deferral (on by default): with `false` every call runs when it is made
  inline bool& DeferGradients(void)
  {
@@ -215,10 +226,11 @@ class CTensor
   mutable bool DeviceOnChange;
   // What the device copy holds when it was not written yet (mi355::CDeferredGradient): while Lazy is not LAZY_NONE the
   // device copy is the current one (DeviceOnChange) and every access goes through Materialise() first.
-  enum {LAZY_NONE=0,LAZY_ZERO,LAZY_GRADIENT_KERNEL,LAZY_GRADIENT_BIAS,LAZY_UPSAMPLING};
+  enum {LAZY_NONE=0,LAZY_ZERO,LAZY_GRADIENT_KERNEL,LAZY_GRADIENT_BIAS,LAZY_UPSAMPLING,LAZY_PRODUCT};
   mutable uint8_t Lazy;
   mutable std::shared_ptr<mi355::CDeferredGradient> Deferred;
   mutable std::shared_ptr<mi355::CDeferredUpSampling> DeferredUpSampling;
+  mutable std::shared_ptr<mi355::CDeferredProduct> DeferredProduct;
   // The last write was a fill with zeros (set by the fills, cleared by everything that hands out the tensor for writing
   // and by every change of either copy): see mi355::ZeroBlock.
   mutable bool KnownZero;
@@ -480,11 +492,19 @@ class CTensor
    record.swap(Deferred);
    std::shared_ptr<mi355::CDeferredUpSampling> up;
    up.swap(DeferredUpSampling);
+   std::shared_ptr<mi355::CDeferredProduct> product;
+   product.swap(DeferredProduct);
    Lazy=LAZY_NONE;
    KnownZero=(kind==LAZY_ZERO);
    mt_tensor own;
    own.p=static_cast<float*>(DeviceItem.get());
    own.w=Size_W;own.z=Size_Z;own.y=Size_Y;own.x=Size_X;
+   if (kind==LAZY_PRODUCT)
+   {
+    own.w=product->LeftTensor.w;own.z=product->LeftTensor.z;own.y=product->LeftTensor.y;own.x=product->RightTensor.x;
+    mi355::Check(mt_mul(&own,&product->LeftTensor,&product->RightTensor));
+    return;
+   }
    if (kind==LAZY_UPSAMPLING)
    {
     // (the sizes of the source as it was: the tensor may have been reinterpreted since)
@@ -600,7 +620,22 @@ class CTensor
    DeviceOnChange=cTensor.DeviceOnChange;
    KnownZero=cTensor.KnownZero;
   }
-  void DropLazy(void) const {Lazy=LAZY_NONE;Deferred.reset();DeferredUpSampling.reset();}
+  void DropLazy(void) const {Lazy=LAZY_NONE;Deferred.reset();DeferredUpSampling.reset();DeferredProduct.reset();}
+  // the device copy is said to hold the per-sample products left x right; nothing is launched (CTensorMath::Mul)
+  void SetLazyProduct(const mi355::CDeviceBuffer &left,const mt_tensor &left_tensor,const mi355::CDeviceBuffer &right,const mt_tensor &right_tensor) const
+  {
+   DeviceItem.Own(false);
+   mi355::Queue().Access(DeviceItem.get(),DeviceItem.size(),false,true);
+   DropLazy();
+   std::shared_ptr<mi355::CDeferredProduct> record(new mi355::CDeferredProduct);
+   record->Left=left;record->LeftTensor=left_tensor;
+   record->Right=right;record->RightTensor=right_tensor;
+   DeferredProduct=record;
+   Lazy=LAZY_PRODUCT;
+   DeviceOnChange=true;
+   HostOnChange=false;
+   KnownZero=false;
+  }
   // the device copy is said to hold `source` up-sampled by the factors; nothing is launched (CTensorMath::UpSampling)
   void SetLazyUpSampling(const mi355::CDeviceBuffer &source,const mt_tensor &source_tensor,uint32_t factor_x,uint32_t factor_y) const
   {

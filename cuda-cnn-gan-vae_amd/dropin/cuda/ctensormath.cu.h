@@ -97,6 +97,29 @@ class CTensorMath
     cTensor_Output.SetDeviceOnChange();
     return;
    }
+   if (&cTensor_Right!=&cTensor_Output && cTensor_Right.Lazy==CTensor<type_t>::LAZY_PRODUCT && &cTensor_Left==&cTensor_Output && left_scale==1 && right_scale==1 &&
+       cTensor_Output.GetSizeW()==1 && cTensor_Output.GetSizeZ()==1)
+   {
+    // the linear layer's own call, AddSumW(dW,dW,per-sample products): dW += columns^T x rows, one product over the batch
+    const std::shared_ptr<mi355::CDeferredProduct> record=cTensor_Right.DeferredProduct;
+    mt_tensor columns=record->LeftTensor,rows=record->RightTensor;
+    const uint32_t batch=columns.w,m=columns.y,n=rows.x;
+    if (cTensor_Output.GetSizeY()==m && cTensor_Output.GetSizeX()==n)
+    {
+     columns.w=1;columns.y=batch;columns.x=m;   // [B,1,M,1] read as the matrix [B][M]
+     rows.w=1;rows.y=batch;rows.x=n;            // [B,1,1,N] read as the matrix [B][N]
+     mi355::CDeviceBuffer sum;
+     sum.resize(static_cast<size_t>(m)*n*sizeof(float));
+     mt_tensor s;
+     s.p=static_cast<float*>(sum.get());
+     s.w=1;s.z=1;s.y=m;s.x=n;
+     mi355::Check(mt_transponse_mul(&s,&columns,&rows));
+     mt_tensor o=cTensor_Output.Device(true);
+     mi355::Check(mt_add(&o,&o,&s,1,1));
+     cTensor_Output.SetDeviceOnChange();
+     return;
+    }
+   }
    mt_tensor l=cTensor_Left.DeviceQueuedRead(),r=cTensor_Right.DeviceQueuedRead(),o=cTensor_Output.DeviceQueued(false);
    mi355::Queue().Submit(mi355::MakeBinary(mi355::OP_ADD_SUM_W,o,l,r,left_scale,right_scale));
    cTensor_Output.SetDeviceOnChange();
@@ -161,6 +184,16 @@ class CTensorMath
   {
    OnlyFloat();
    (void)tensor_core;  // the reference's fp16 tensor-core switch; this path is always fp32 on the matrix cores
+   if (mi355::DeferGradients()==true && &cTensor_Output!=&cTensor_Left && &cTensor_Output!=&cTensor_Right && cTensor_Left.GetSizeX()==1 && cTensor_Right.GetSizeY()==1 &&
+       cTensor_Left.GetSizeW()>=2 && cTensor_Right.GetSizeW()==cTensor_Left.GetSizeW() && cTensor_Output.GetSizeW()==cTensor_Left.GetSizeW() &&
+       cTensor_Left.GetSizeZ()==1 && cTensor_Right.GetSizeZ()==1 && cTensor_Output.GetSizeZ()==1 &&
+       cTensor_Output.GetSizeY()==cTensor_Left.GetSizeY() && cTensor_Output.GetSizeX()==cTensor_Right.GetSizeX() && cTensor_Output.Count()>=(static_cast<size_t>(1)<<16))
+   {
+    // per-sample outer products: computed when somebody reads them; their sum over the batch never needs them (mi355::CDeferredProduct)
+    mt_tensor l=cTensor_Left.DeviceRead(),r=cTensor_Right.DeviceRead();
+    cTensor_Output.SetLazyProduct(cTensor_Left.DeviceItem,l,cTensor_Right.DeviceItem,r);
+    return;
+   }
    mt_tensor l=cTensor_Left.DeviceRead(),r=cTensor_Right.DeviceRead(),o=cTensor_Output.Device(false);
    mi355::Check(mt_mul(&o,&l,&r));
    cTensor_Output.SetDeviceOnChange();
