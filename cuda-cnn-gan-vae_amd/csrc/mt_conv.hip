@@ -1928,7 +1928,11 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
       return OH % n == 0 && ((OH / n) * OW) % BK == 0 && (OH / n) * OW >= 32u * BK && (size_t)B * n * ka * ncol <= ((size_t)1 << 26) &&
              wgrad_image_fixed(ka, ncol, B * n, delta, image, kz, 1, px, py);
     };
-    while ((size_t)tiles * B * parts < 1024 && parts < 256 && fits(parts * 2)) parts *= 2;
+    auto blocks = [&](uint32_t n) {   // with the tile that the product of B * n groups will get
+      const Tile tile = pick_tile(ka, ncol, B * n);
+      return (size_t)cdiv(ka, tile_rows(tile)) * cdiv(ncol, tile_cols(tile)) * B * n;
+    };
+    while (blocks(parts) < 1024 && parts < 256 && fits(parts * 2)) parts *= 2;
     if (g_wgrad_parts > 1 && fits((uint32_t)g_wgrad_parts)) parts = (uint32_t)g_wgrad_parts;
   }
   if (parts > 1) {
