@@ -19,6 +19,7 @@
 #include "mt_igemm.h"
 #include "mt_walk.h"
 #include "mt_firstlayer.h"
+#include "mt_wgradpatch.h"
 
 namespace {
 
@@ -32,7 +33,8 @@ int g_walk_wide = 1;       // 1: layers whose output channels are a multiple of 
 int g_upconv_split = 1;    // 1: up-sampling convolutions with fewer than 512 walking blocks share a tile's k steps between blocks
 int g_upconv_walk = 512;   // blocks from which the up-sampling convolution takes the walking kernel (0: never; measured on the
                            // shipped GAN generator at batch 32: 768 blocks 67.7 -> 54.6 and 58.6 -> 54.0 us, 384 blocks 65.1 -> 69 us)
-uint64_t g_wgrad_walk_launches = 0;
+uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0;
+int g_wgrad_patch = 1;   // 1: the batch-summed weight gradient of a 3x3 stride-1 layer with at most 32 filters on large images multiplies patches held in LDS (wgrad_patch3x3_kernel), 0: never
 int g_wgrad_parts = 1;   // 1: the general batch-summed weight gradient cuts samples into bands of output rows when samples x tiles are too few blocks, 0: never, n > 1: n bands
 int g_wgrad_walk = 1;    // 1: the batch-summed weight gradient runs as one k loop per block where its shape allows (wgrad_walk_kernel), 0: never
 int g_wgrad_groups = 0;  // 0 auto, else the number of batch groups of the batch-summed weight gradient (if it divides the batch)
@@ -1873,6 +1875,26 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     if ((rc = mt_add_sum_w(dst, dst, &dkb, 1.f, 1.f))) return rc;
     return mt_add_sum_w(db, db, &dbb, 1.f, 1.f);
   }
+  // few filters of 3 x 3, stride 1, padding 1 on large images: the nine taps share one patch in LDS
+  if (g_wgrad_patch && kx == 3 && ky == 3 && sx == 1 && sy == 1 && px == 1 && py == 1 && image->y == delta->y && image->x == delta->x &&
+      dk->x == ncol && dk->z * dk->y == ka) {
+    mt::igemm::WgradPatchArgs pa{};
+    pa.delta = delta->p; pa.image = image->p; pa.B = B; pa.KA = ka; pa.C = (uint32_t)kz; pa.H = delta->y; pa.W = delta->x;
+    if (mt::igemm::wgrad_patch_plan(pa)) {
+      const uint32_t sums = 2 * pa.groups, chunks = dbias_chunks(B, ka, DHW);
+      float *ws = nullptr;
+      if ((rc = workspace((size_t)sums * ka * ncol + (chunks > 1 ? (size_t)ka * chunks : 0), &ws))) return rc;
+      pa.partial = ws;
+      {
+        mt::ProfileScope prof(mt::profiling() ? shape_label(name, T64x64, ka, ncol, B * DHW, pa.groups * pa.slabs) : name);
+        if ((rc = mt::igemm::launch_wgrad_patch(name, pa))) return rc;
+      }
+      g_wgrad_patch_launches++;
+      mt_tensor pt{ws, sums, 1, ka, ncol}, flat{dk->p, 1, 1, ka, ncol};
+      if ((rc = mt_add_sum_w(&flat, &flat, &pt, 1.f, 1.f))) return rc;
+      return dbias_batch_sum(name, db->p, ws + (size_t)sums * ka * ncol, delta->p, B, ka, DHW, chunks);
+    }
+  }
   // groups: enough blocks for every compute unit, and a divisor of the batch so that all groups have the same K
   const uint32_t tiles = cdiv(ka, 64) * cdiv(ncol, 64);
   uint32_t groups = 1;
@@ -2237,6 +2259,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "graph_written_ranges") == 0) { *value = (int64_t)g_graph_written.size(); return true; }
   if (strcmp(name, "graph_writes_anything") == 0) { *value = g_graph_writes_anything ? 1 : 0; return true; }
   if (strcmp(name, "wgrad_walk_launches") == 0) { *value = (int64_t)g_wgrad_walk_launches; return true; }
+  if (strcmp(name, "wgrad_patch_launches") == 0) { *value = (int64_t)g_wgrad_patch_launches; return true; }
   return false;
 }
 int set_image_strip(int v) {
@@ -2317,6 +2340,11 @@ int set_upconv_split(int v) {
 int set_upconv_walk(int v) {
   if (v < 0) return fail(MT_E_ARGUMENT, "upconv_walk must be 0 (never) or the number of blocks from which the walking kernel is taken");
   g_upconv_walk = v;
+  return MT_OK;
+}
+int set_wgrad_patch(int v) {
+  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "wgrad_patch must be 0 or 1");
+  g_wgrad_patch = v;
   return MT_OK;
 }
 int set_wgrad_parts(int v) {

@@ -432,6 +432,43 @@ def test_weights_sum_in_bands_of_rows(gpu, oracle, case):
 
 
 @pytest.mark.parametrize("case", [
+    # B, C, H, W, KA, taken
+    (4, 32, 64, 512, 16, 1),     # 16 filters over 32 channels: one slab, one block of filters
+    (8, 16, 32, 512, 3, 1),      # an image layer: 3 filters over 16 channels (half a slab)
+    (4, 64, 128, 256, 32, 1),    # 32 filters over 64 channels: two slabs, two blocks of filters
+    (16, 48, 16, 512, 17, 1),    # ragged: 17 filters, a slab and a half
+    (2, 5, 64, 1024, 9, 1),      # 5 channels, rows of 16 segments
+    (1, 20, 256, 512, 4, 1),     # one sample
+    (4, 40, 64, 512, 8, 0),      # a second slab of 8 channels: mostly padding, the general kernel
+    (4, 8, 62, 512, 8, 0),       # rows of 512 pixels but too few tiles: the general kernel
+])
+def test_weights_sum_from_patches_in_lds(gpu, oracle, case):
+    """The batch-summed weight gradient of 3 x 3 stride-1 layers with few filters on large images on the kernel that holds
+    delta's tile and the image patch behind it in LDS (nine taps per patch), against the layer's own sequence on the oracle
+    (netlayer/cnetlayerconvolution.cu.h:501-508) and against the general kernel."""
+    import mi355tensor as mt
+    B, C, H, Wd, KA, taken = case
+    image, delta = U(51, B, C, H, Wd), U(52, B, KA, H, Wd)
+    dk0, db0 = U(53, 1, 1, KA, C * 9), U(54, 1, KA, 1, 1)
+    dkb, dbb = oracle.create_delta_weight_and_bias(np.zeros((B, 1, KA, C * 9), np.float32), np.zeros((B, KA, 1, 1), np.float32),
+                                                   image, delta, 3, 3, C, KA, 1, 1, 1, 1)
+    want_k, want_b = oracle.add_sum_w(dk0, dkb, out_init=dk0), oracle.add_sum_w(db0, dbb, out_init=db0)
+    got = {}
+    try:
+        for on in (1, 0):
+            mt.set_option("wgrad_patch", on)
+            before = mt.get_info("wgrad_patch_launches")
+            got[on] = gpu.convolution_backward_weights_sum(dk0, db0, image, delta, 3, 3, C, KA, 1, 1, 1, 1)
+            assert mt.get_info("wgrad_patch_launches") - before == (taken if on else 0)
+    finally:
+        mt.set_option("wgrad_patch", 1)
+    for on in (1, 0):
+        close(got[on][0], want_k)
+        close(got[on][1], want_b)
+    close(got[1][0], got[0][0], 2e-6)
+
+
+@pytest.mark.parametrize("case", [
     # B, C, H, W, KA, k, s, p, groups
     (16, 64, 32, 32, 128, 4, 2, 1, 0),   # output rows of 16 pixels: a k step is one row
     (16, 32, 16, 16, 64, 4, 2, 1, 0),    # rows of 8 pixels: two rows per k step, four steps per sample
