@@ -1400,6 +1400,8 @@ int mt_add_sum_w(const mt_tensor *out, const mt_tensor *l, const mt_tensor *r, f
     else add_sum_w_vec_kernel<4><<<cdiv(cols, 4), EW_THREADS, 0, st>>>(out->p, out->w, l->p, l->w, r->p, r->w, n, ls, rs);
   } else if (S >= 65536)
     add_sum_w_kernel<256><<<cdiv(S, 256), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
+  else if ((l->w >= 512 || r->w >= 512) && S <= 4096)   // many short slices (partial sums of a small gradient): 64 threads share a column
+    add_sum_w_kernel<4><<<cdiv(S, 4), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
   else
     add_sum_w_kernel<32><<<cdiv(S, 32), EW_THREADS, 0, mt::stream()>>>(out->p, out->w, l->p, l->w, r->p, r->w, (uint32_t)S, ls, rs);
   MT_LAUNCH_CHECK("mt_add_sum_w");

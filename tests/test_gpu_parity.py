@@ -817,6 +817,11 @@ def test_reductions(gpu, oracle):
     assert np.all(out[1] == 0)
     wide = U(6, 32, 4, 128, 160)  # 81920 columns: the one-slice variant
     close(gpu.add_sum_w(wide[:1], wide, 1.0, 1.0 / 32), oracle.add_sum_w(wide[:1], wide, 1.0, 1.0 / 32), 1e-6)
+    many = U(7, 1536, 1, 3, 145)  # 1536 short slices of 435 columns: 64 threads share a column
+    close(gpu.add_sum_w(many[:1], many, 1.0, 1.0), oracle.add_sum_w(many[:1], many, 1.0, 1.0), 2e-6)
+    out = gpu.add_sum_w(many[:1], many, 1.0, 0.5, out_w=2)
+    close(out, oracle.add_sum_w(many[:1], many, 1.0, 0.5, out_w=2), 2e-6)
+    assert np.all(out[1] == 0)
 
 
 def test_resampling_and_pooling_bit_exact(gpu, oracle):
