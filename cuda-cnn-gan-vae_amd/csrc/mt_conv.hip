@@ -20,6 +20,7 @@
 #include "mt_walk.h"
 #include "mt_firstlayer.h"
 #include "mt_wgradpatch.h"
+#include "mt_convpatch.h"
 
 namespace {
 
@@ -33,7 +34,8 @@ int g_walk_wide = 1;       // 1: layers whose output channels are a multiple of 
 int g_upconv_split = 1;    // 1: up-sampling convolutions with fewer than 512 walking blocks share a tile's k steps between blocks
 int g_upconv_walk = 512;   // blocks from which the up-sampling convolution takes the walking kernel (0: never; measured on the
                            // shipped GAN generator at batch 32: 768 blocks 67.7 -> 54.6 and 58.6 -> 54.0 us, 384 blocks 65.1 -> 69 us)
-uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0;
+uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0, g_tconv_patch_launches = 0;
+int g_tconv_patch = 1;   // 1: a 3x3 stride-1 transposed convolution from at most 32 filters to at most 64 channels on large images multiplies patches held in LDS (tconv3x3_patch_kernel), 0: never
 int g_wgrad_patch = 1;   // 1: the batch-summed weight gradient of a 3x3 stride-1 layer with at most 32 filters on large images multiplies patches held in LDS (wgrad_patch3x3_kernel), 0: never
 int g_wgrad_parts = 1;   // 1: the general batch-summed weight gradient cuts samples into bands of output rows when samples x tiles are too few blocks, 0: never, n > 1: n bands
 int g_wgrad_walk = 1;    // 1: the batch-summed weight gradient runs as one k loop per block where its shape allows (wgrad_walk_kernel), 0: never
@@ -1605,6 +1607,22 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     return MT_OK;
   }
 
+  // few filters of 3 x 3, stride 1, padding 1 on large images: the nine taps share one patch of delta in LDS, the weights are
+  // read as they lie
+  if (g_tconv_patch && !fused && mt::igemm::tile_override() < 0 && kx == 3 && ky == 3 && sx == 1 && sy == 1 && px == 1 && py == 1 && bias->w == 1 &&
+      delta->w == out->w && delta->y == out->y && delta->x == out->x) {
+    mt::igemm::TconvPatchArgs tp{};
+    tp.delta = delta->p; tp.kernel = kernel->p; tp.bias = bias->p; tp.out = out->p;
+    tp.B = out->w; tp.F = ka; tp.C = (uint32_t)kz; tp.H = out->y; tp.W = out->x; tp.ld = kernel->x;
+    if (mt::igemm::tconv_patch_plan(tp)) {
+      {
+        mt::ProfileScope prof(mt::profiling() ? shape_label(name, T16x256, (uint32_t)kz, out->w * out->y * out->x, ka * 9, 1) : name);
+        if ((rc = mt::igemm::launch_tconv_patch(name, tp))) return rc;
+      }
+      g_tconv_patch_launches++;
+      return func == MT_F_NONE ? MT_OK : mt_apply_func(out, out, func);
+    }
+  }
   // workspace: [bias sums (bias_w, padded to 64)] [packed sub-kernels of all phases: kz*ka*ky*kx floats + alignment]
   size_t sums = (bias->w + 63u) & ~(size_t)63u;
   float *ws = nullptr;
@@ -2260,6 +2278,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "graph_writes_anything") == 0) { *value = g_graph_writes_anything ? 1 : 0; return true; }
   if (strcmp(name, "wgrad_walk_launches") == 0) { *value = (int64_t)g_wgrad_walk_launches; return true; }
   if (strcmp(name, "wgrad_patch_launches") == 0) { *value = (int64_t)g_wgrad_patch_launches; return true; }
+  if (strcmp(name, "tconv_patch_launches") == 0) { *value = (int64_t)g_tconv_patch_launches; return true; }
   return false;
 }
 int set_image_strip(int v) {
@@ -2340,6 +2359,11 @@ int set_upconv_split(int v) {
 int set_upconv_walk(int v) {
   if (v < 0) return fail(MT_E_ARGUMENT, "upconv_walk must be 0 (never) or the number of blocks from which the walking kernel is taken");
   g_upconv_walk = v;
+  return MT_OK;
+}
+int set_tconv_patch(int v) {
+  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "tconv_patch must be 0 or 1");
+  g_tconv_patch = v;
   return MT_OK;
 }
 int set_wgrad_patch(int v) {

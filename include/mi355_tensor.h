@@ -107,6 +107,9 @@ int mt_timer_destroy(void *timer);
  *   "wgrad_parts"    1 (default) the general kernel of mt_convolution_backward_weights_sum cuts every sample into equal bands of
  *                    output rows (one partial sum per band) when samples x tiles are fewer blocks than the chip needs: layers
  *                    with few filters on large images / 0 never / n bands per sample (2..256, where the rows divide)
+ *   "tconv_patch"    1 (default) mt_backward_convolution of a 3x3 layer with stride 1, padding 1, at most 32 filters and at most 64
+ *                    channels on large images (rows a multiple of 64 pixels, an even number of rows, at least 1024 tiles of
+ *                    2 x 64 pixels in the batch) multiplies patches of delta held in LDS, nine taps per patch / 0 never
  *   "wgrad_patch"    1 (default) mt_convolution_backward_weights_sum of a 3x3 layer with stride 1, padding 1 and at most 32
  *                    filters on large images (rows a multiple of 64 pixels, an even number of rows, at least 1024 tiles of
  *                    2 x 64 pixels in the batch) multiplies image patches held in LDS, nine taps per patch / 0 never
@@ -162,7 +165,8 @@ int mt_set_option(const char *name, int value);
  *                                                          (graph_writes_anything = 1, for the rest of the process)
  *   "wgrad_walk_launches"                                  calls of mt_convolution_backward_weights_sum that ran as one k loop
  *                                                          per block (option "wgrad_walk")
- *   "wgrad_patch_launches"                                 calls of it that multiplied patches held in LDS (option "wgrad_patch") */
+ *   "wgrad_patch_launches"                                 calls of it that multiplied patches held in LDS (option "wgrad_patch")
+ *   "tconv_patch_launches"                                 calls of mt_backward_convolution that did (option "tconv_patch") */
 int mt_get_info(const char *name, int64_t *value);
 
 /* ---- convolutions: CTensorConv<T> (cuda/ctensorconv.cu.h:63-66) ---- */

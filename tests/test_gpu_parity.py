@@ -432,6 +432,44 @@ def test_weights_sum_in_bands_of_rows(gpu, oracle, case):
 
 
 @pytest.mark.parametrize("case", [
+    # B, C, H, W, KA, func, taken
+    (4, 32, 64, 512, 16, None, 1),        # 16 filters to 32 channels: a wave per (16 channels, row of the tile)
+    (8, 16, 32, 512, 3, None, 1),         # an image layer's backward pass: 3 filters to 16 channels
+    (4, 64, 128, 256, 32, None, 1),       # 32 filters to 64 channels: a wave per 16 channels
+    (16, 40, 16, 512, 17, "leaky_relu", 1),   # ragged: 17 filters, 40 channels, a function afterwards
+    (2, 5, 64, 1024, 9, None, 1),         # 5 channels, rows of 16 segments
+    (1, 20, 256, 512, 6, "tangence", 1),  # one sample
+    (4, 80, 64, 512, 8, None, 0),         # more than 64 channels: the general kernel
+    (4, 8, 62, 512, 8, None, 0),          # too few tiles: the general kernel
+])
+def test_transposed_convolution_from_patches_in_lds(gpu, oracle, case):
+    """The backward pass of 3 x 3 stride-1 layers with few filters on large images on the kernel that holds the patch of
+    delta in LDS and the weights in registers, with a non-zero bias (added once per tap inside the image,
+    cpu/ctensorconv.h:204-268), against the oracle and against the general kernel."""
+    import mi355tensor as mt
+    B, C, H, Wd, KA, func, taken = case
+    delta = U(61, B, KA, H, Wd)
+    kernel = U(62, 1, 1, KA, C * 9) * np.float32(0.2)
+    bias = U(63, 1, KA, 1, 1) * np.float32(0.1)
+    args = (delta, kernel, bias, 3, 3, C, KA, 1, 1, 1, 1, (B, C, H, Wd))
+    want = oracle.backward_convolution(*args)
+    if func:
+        want = oracle.apply_func(want, func)
+    got = {}
+    try:
+        for on in (1, 0):
+            mt.set_option("tconv_patch", on)
+            before = mt.get_info("tconv_patch_launches")
+            got[on] = gpu.backward_convolution(*args, func=func)
+            assert mt.get_info("tconv_patch_launches") - before == (taken if on else 0)
+    finally:
+        mt.set_option("tconv_patch", 1)
+    close(got[1], want)
+    close(got[0], want)
+    close(got[1], got[0], 2e-6)
+
+
+@pytest.mark.parametrize("case", [
     # B, C, H, W, KA, taken
     (4, 32, 64, 512, 16, 1),     # 16 filters over 32 channels: one slab, one block of filters
     (8, 16, 32, 512, 3, 1),      # an image layer: 3 filters over 16 channels (half a slab)
