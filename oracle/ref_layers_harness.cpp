@@ -691,7 +691,11 @@ static void TimeGanGenerator(uint32_t batch,uint32_t warmup,uint32_t steps,bool 
  CTensor<type_t> latent(batch,1,1024,1);
  FillTensor(latent,1.0);
  net[0]->SetOutput(latent);
- for(size_t n=0;n<net.size();n++) net[n]->TrainingStart();
+ for(size_t n=0;n<net.size();n++)
+ {
+  if (train==true) net[n]->TrainingModeAdam(0.5,0.9);   // as the model trains it (cuda/netmodel/cmodel_basicgan.cu.h:852)
+  net[n]->TrainingStart();
+ }
  CTensor<type_t> error(batch,3,192,256);
  if (train==true) FillTensor(error,0.01);
  double ms=TimeSteps(train==true?"GAN generator step":"GAN generator forward",net,train==true?&error:NULL,warmup,steps);
