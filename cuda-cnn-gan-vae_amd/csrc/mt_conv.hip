@@ -2276,6 +2276,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "pack_cache_spare_bytes") == 0) { int64_t n = 0; for (const PackEntry &e : g_pack_spare) n += (int64_t)(e.floats * sizeof(float)); *value = n; return true; }
   if (strcmp(name, "graph_written_ranges") == 0) { *value = (int64_t)g_graph_written.size(); return true; }
   if (strcmp(name, "graph_writes_anything") == 0) { *value = g_graph_writes_anything ? 1 : 0; return true; }
+  if (strcmp(name, "convolution_workspace_bytes") == 0) { *value = (int64_t)(g_ws.floats * sizeof(float)); return true; }
   if (strcmp(name, "wgrad_walk_launches") == 0) { *value = (int64_t)g_wgrad_walk_launches; return true; }
   if (strcmp(name, "wgrad_patch_launches") == 0) { *value = (int64_t)g_wgrad_patch_launches; return true; }
   if (strcmp(name, "tconv_patch_launches") == 0) { *value = (int64_t)g_tconv_patch_launches; return true; }

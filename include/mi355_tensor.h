@@ -155,6 +155,7 @@ int mt_set_option(const char *name, int value);
  *   "retired_blocks", "retired_bytes"                      blocks freed (or handed out) while the stream was being captured:
  *                                                          a recorded graph names them, so they are never handed out again
  *   "retired_workspaces"                                   outgrown workspaces that a recorded graph may still use
+ *   "convolution_workspace_bytes"                          size of the convolutions' workspace (it only grows)
  *   "pack_cache_entries", "pack_cache_valid", "pack_cache_hits", "pack_cache_made", "pack_cache_bytes"
  *                                                          the re-ordered weights kept between calls
  *   "pack_cache_refreshed"                                 copies that an mt_adam_many call wrote itself (option "pack_refresh")

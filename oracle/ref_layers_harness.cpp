@@ -565,10 +565,10 @@ static void ChainF(void)
 // Timing of the unchanged layer classes on the drop-in tensors at the sizes of the two networks the library is tuned
 // for; CTimeStamp (the reference's own scope timer, here the drop-in's) prints each figure through SYSTEM::PutMessageToConsole
 // and CCUDATimeSpent returns it.  One JSON line per chain on stdout.
-static void LoadConvolutionWeights(INetLayer<type_t> &layer,uint32_t rows,uint32_t amount_field,int32_t size,int32_t depth_field,uint32_t columns,uint32_t biases,double scale)
+static void LoadConvolutionWeights(INetLayer<type_t> &layer,uint32_t rows,uint32_t amount_field,int32_t size,int32_t depth_field,uint32_t columns,uint32_t biases,double scale,int32_t padding=1)
 {
  CMemoryStream w;
- w.SaveUInt32(amount_field);w.SaveInt32(size);w.SaveInt32(size);w.SaveInt32(depth_field);w.SaveInt32(2);w.SaveInt32(2);w.SaveInt32(1);w.SaveInt32(1);
+ w.SaveUInt32(amount_field);w.SaveInt32(size);w.SaveInt32(size);w.SaveInt32(depth_field);w.SaveInt32(2);w.SaveInt32(2);w.SaveInt32(padding);w.SaveInt32(padding);
  w.PutTensor(1,1,rows,columns,Values(static_cast<size_t>(rows)*columns,scale));
  w.PutTensor(1,biases,1,1,std::vector<double>(biases,0.0));
  layer.Load(&w);
@@ -757,6 +757,51 @@ static void TimeDiscriminator(uint32_t batch,uint32_t warmup,uint32_t steps)
         batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),out.GetElement(0,0,0,0),driver_allocations_in_the_timed_steps);
 }
 
+// The discriminator of the reference's GAN model (cuda/netmodel/cmodel_gan.cu.h:236-287), whole training step in Adam mode, batch 32:
+// Convolution 5x5 stride 2 padding 2 to 16 filters, leaky ReLU, five times (Convolution 5x5 stride 2 padding 2, BatchNormalization,
+// leaky ReLU) through 32, 64, 128, 256, 512 filters, Linear to one output; 192x256 images
+static void TimeGanDiscriminator(uint32_t batch,uint32_t warmup,uint32_t steps)
+{
+ static const uint32_t channels[7]={3,16,32,64,128,256,512};
+ rng_state=0x13198A2E03707344ull;
+ std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
+ std::vector<INetLayer<type_t>*> net;
+#define PUSH(LAYER) {owner.push_back(std::shared_ptr<INetLayer<type_t> >(LAYER));net.push_back(owner.back().get());}
+ PUSH(new CNetLayerConvolutionInput<type_t>(3,192,256,batch));
+ for(uint32_t i=0;i<6;i++)
+ {
+  PUSH(new CNetLayerConvolution<type_t>(channels[i+1],5,2,2,2,2,net.back(),batch));
+  LoadConvolutionWeights(*net.back(),channels[i+1],channels[i+1],5,channels[i],channels[i]*25,channels[i+1],sqrt(2.0/(channels[i]*25)),2);
+  if (i>0)
+  {
+   PUSH(new CNetLayerBatchNormalization<type_t>(0.9f,net.back(),batch));
+   net.back()->Reset();
+  }
+  PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_LEAKY_RELU,net.back(),batch));
+ }
+ PUSH(new CNetLayerLinear<type_t>(1,net.back(),batch));
+ {
+  CMemoryStream w;
+  w.PutTensor(1,1,1,512*12,Values(512*12,0.02));
+  w.PutTensor(1,1,1,1,std::vector<double>(1,0.0));
+  net.back()->Load(&w);
+ }
+#undef PUSH
+ for(size_t n=0;n<net.size();n++)
+ {
+  net[n]->TrainingModeAdam(0.5,0.9);
+  net[n]->TrainingStart();
+ }
+ CTensor<type_t> image(batch,3,192,256),error(batch,1,1,1);
+ FillTensor(image,1.0);
+ FillTensor(error,0.5);
+ net[0]->SetOutput(image);
+ double ms=TimeSteps("GAN discriminator step",net,&error,warmup,steps);
+ CTensor<type_t> &out=net.back()->GetOutputTensor();
+ printf("{\"chain\": \"gan_discriminator_step\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"first\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
+        batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),out.GetElement(0,0,0,0),driver_allocations_in_the_timed_steps);
+}
+
 // Chain K: two training steps (gradient descent) of the discriminator at batch 16, once with the per-sample weight gradients deferred by the
 // drop-in classes (mi355::CDeferredGradient; the last two convolution layers qualify) and once with every call run when
 // it is made: same seeds, the updated convolution weights of both runs go to the dump
@@ -901,7 +946,11 @@ int main(int argc,char **argv)
    TimeGenerator(256,warmup,steps);
    TimeDiscriminator(128,warmup,steps);
    TimeGanGenerator(32,warmup,steps);
-   if (argc>5 && strcmp(argv[5],"train")==0) TimeGanGenerator(32,warmup,steps,true);   // and its whole training step (forward, backward, Adam)
+   if (argc>5 && strcmp(argv[5],"train")==0)   // and the whole training steps (forward, backward, Adam) of the reference's GAN generator and discriminator
+   {
+    TimeGanGenerator(32,warmup,steps,true);
+    TimeGanDiscriminator(32,warmup,steps);
+   }
    if (argc>5 && strcmp(argv[5],"literal")==0)   // and the last chain once more with every call run when it is made
    {
     mi355::DeferGradients()=false;

@@ -333,7 +333,8 @@ def test_workspace_growth_around_a_recording(mt):
         hip = C.CDLL("libamdhip64.so")
         stream, graph = C.c_void_p(mt.get_stream()), C.c_void_p()
         # larger than anything the process has run so far, so the workspace must grow
-        huge, _ = layer(1024, 1024 + 16 * retired, 2)
+        exists = mt.get_info("convolution_workspace_bytes") // 4
+        huge, _ = layer(1024, max(1024, 16 * (exists // (1024 * 16 * 16) + 2)) + 16 * retired, 2)
         assert hip.hipStreamBeginCapture(stream, C.c_int(2)) == 0
         try:
             small()
