@@ -364,19 +364,23 @@ namespace mi355
   return(2);
  }
 
- // consecutive Fill calls with one value, or consecutive Adam calls with one set of hyper-parameters
+ // Fill calls with one value, or Adam calls with one set of hyper-parameters: neighbours in the queue run as one launch
+ inline bool SameRun(const SOp &h,const SOp &o)
+ {
+  if (h.Kind!=OP_FILL && h.Kind!=OP_ADAM) return(false);
+  if (o.Kind!=h.Kind) return(false);
+  if (h.Kind==OP_FILL && o.A!=h.A) return(false);
+  if (h.Kind==OP_ADAM && (o.BatchSize!=h.BatchSize || o.Speed!=h.Speed || o.Beta1!=h.Beta1 || o.Beta2!=h.Beta2 || o.Epsilon!=h.Epsilon || o.Iteration!=h.Iteration)) return(false);
+  return(true);
+ }
+
+ // whether the first `count` calls of the queue are one such run
  inline bool IsRun(const std::vector<SOp> &q,size_t count)
  {
   if (count==0) return(true);
-  const SOp &h=q[0];
-  if (h.Kind!=OP_FILL && h.Kind!=OP_ADAM) return(false);
+  if (q[0].Kind!=OP_FILL && q[0].Kind!=OP_ADAM) return(false);
   for(size_t i=1;i<count;i++)
-  {
-   const SOp &o=q[i];
-   if (o.Kind!=h.Kind) return(false);
-   if (h.Kind==OP_FILL && o.A!=h.A) return(false);
-   if (h.Kind==OP_ADAM && (o.BatchSize!=h.BatchSize || o.Speed!=h.Speed || o.Beta1!=h.Beta1 || o.Beta2!=h.Beta2 || o.Epsilon!=h.Epsilon || o.Iteration!=h.Iteration)) return(false);
-  }
+   if (SameRun(q[0],q[i])==false) return(false);
   return(true);
  }
 
@@ -487,29 +491,36 @@ namespace mi355
     if (Scan(true)==2) return;
     std::vector<SOp> q;
     q.swap(Queue);
-    if (q.size()>=2 && IsRun(q,q.size())==true)
+    size_t first=0;
+    while(first<q.size())
     {
-     Settle(&q[0],q.size());
-     RunCalls+=q.size();
-     std::vector<const mt_tensor*> a(q.size()),b(q.size()),c(q.size()),d(q.size());
-     for(size_t i=0;i<q.size();i++) {a[i]=&q[i].T[0];b[i]=&q[i].T[1];c[i]=&q[i].T[2];d[i]=&q[i].T[3];}
-     if (q[0].Kind==OP_FILL)
+     size_t end=first+1;
+     while(end<q.size() && SameRun(q[first],q[end])==true) end++;
+     const size_t count=end-first;
+     if (count>=2)   // a run of fills or of Adam updates (other calls may stand in front of it and behind it)
      {
-      FillRuns++;
-      Check(mt_fill_many(static_cast<uint32_t>(q.size()),&a[0],q[0].A));
+      Settle(&q[first],count);
+      RunCalls+=count;
+      std::vector<const mt_tensor*> a(count),b(count),c(count),d(count);
+      for(size_t i=0;i<count;i++) {a[i]=&q[first+i].T[0];b[i]=&q[first+i].T[1];c[i]=&q[first+i].T[2];d[i]=&q[first+i].T[3];}
+      if (q[first].Kind==OP_FILL)
+      {
+       FillRuns++;
+       Check(mt_fill_many(static_cast<uint32_t>(count),&a[0],q[first].A));
+      }
+      else
+      {
+       AdamRuns++;
+       Check(mt_adam_many(static_cast<uint32_t>(count),&a[0],&b[0],&c[0],&d[0],q[first].BatchSize,q[first].Speed,q[first].Beta1,q[first].Beta2,q[first].Epsilon,q[first].Iteration));
+      }
      }
      else
      {
-      AdamRuns++;
-      Check(mt_adam_many(static_cast<uint32_t>(q.size()),&a[0],&b[0],&c[0],&d[0],q[0].BatchSize,q[0].Speed,q[0].Beta1,q[0].Beta2,q[0].Epsilon,q[0].Iteration));
+      Settle(&q[first],1);
+      LiteralCalls++;
+      RunLiteral(q[first]);
      }
-     return;
-    }
-    for(size_t i=0;i<q.size();i++)
-    {
-     Settle(&q[i],1);
-     LiteralCalls++;
-     RunLiteral(q[i]);
+     first=end;
     }
    }
    void RunForward(const std::vector<SOp> &sequence,const SBatchNormForward &m)
