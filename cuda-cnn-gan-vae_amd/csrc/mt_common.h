@@ -31,6 +31,7 @@ int set_nontemporal(int v);   // streaming kernels read and write past the cache
 int set_image_strip(int v);   // rows per strip of the image layer's product kernel on 64-column images (0: choose)
 int set_tconv_patch(int v);  // 3x3 stride-1 transposed convolutions from at most 32 filters on large images from patches in LDS: 1 (default) / 0 never
 int set_wgrad_patch(int v);  // the batch-summed weight gradient of 3x3 stride-1 layers with at most 32 filters on large images from patches in LDS: 1 (default) / 0 never
+int set_wgrad_pad(int v);    // the batch-summed weight gradient on delta padded with rows of zeros where its images do not fill whole k steps: 1 (default) / 0 never
 int set_wgrad_parts(int v);  // the general batch-summed weight gradient in bands of output rows per sample: 1 (default) where samples x tiles are few, 0 never, n bands
 int set_walk_wide(int v);    // 1 (default): the walking kernel in blocks of 32 rows x 128 columns for 32 (96, ...) output channels; 0: never
 int set_upconv_split(int v); // 1 (default): up-sampling convolutions with too few tiles share a tile's k steps between blocks; 0: never

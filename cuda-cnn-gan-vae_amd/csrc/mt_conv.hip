@@ -37,6 +37,7 @@ int g_upconv_walk = 512;   // blocks from which the up-sampling convolution take
 uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0, g_tconv_patch_launches = 0;
 int g_tconv_patch = 1;   // 1: a 3x3 stride-1 transposed convolution from at most 32 filters to at most 64 channels on large images multiplies patches held in LDS (tconv3x3_patch_kernel), 0: never
 int g_wgrad_patch = 1;   // 1: the batch-summed weight gradient of a 3x3 stride-1 layer with at most 32 filters on large images multiplies patches held in LDS (wgrad_patch3x3_kernel), 0: never
+int g_wgrad_pad = 1;     // 1: the batch-summed weight gradient pads delta's images with rows of zeros when their pixels do not fill whole k steps, 0: per-sample gradients then
 int g_wgrad_parts = 1;   // 1: the general batch-summed weight gradient cuts samples into bands of output rows when samples x tiles are too few blocks, 0: never, n > 1: n bands
 int g_wgrad_walk = 1;    // 1: the batch-summed weight gradient runs as one k loop per block where its shape allows (wgrad_walk_kernel), 0: never
 int g_wgrad_groups = 0;  // 0 auto, else the number of batch groups of the batch-summed weight gradient (if it divides the batch)
@@ -1859,6 +1860,15 @@ int wgrad(const char *name, const mt_tensor *dk, int32_t kx, int32_t ky, int32_t
   return MT_OK;
 }
 
+// delta with rows of zeros appended to every image: [rows][hw] -> [rows][hw2]
+__global__ __launch_bounds__(256) void pad_rows_kernel(float *out, const float *in, uint32_t hw, uint32_t hw2, size_t total) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const size_t row = i / hw2;
+  const uint32_t k = (uint32_t)(i - row * hw2);
+  out[i] = k < hw ? in[row * hw + k] : 0.f;
+}
+
 // Weight and bias gradient of a convolution layer summed over the batch in one product: K runs over (sample, output
 // pixel), so dK[f][(c,i,j)] += sum_w sum_(oy,ox) delta[w][f][oy][ox] * image[w][c][oy*s-p+i][ox*s-p+j] without the
 // per-sample gradients ever being written.  When the product has few output tiles the batch is split into groups
@@ -1880,6 +1890,25 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
   if (rc) return rc;
   if (B == 0 || DHW == 0) return MT_OK;
   const size_t sample_image = (size_t)kz * image->y * image->x, sample_delta = (size_t)ka * DHW;
+  if (g_conv_path != 1 && DHW % BK != 0 && g_wgrad_pad && sample_image * 4 < 0x80000000ull) {
+    // Output images whose pixels do not fill whole k steps (3 x 4 at the end of a discriminator): the same sums with rows of
+    // zeros appended to every image of delta -- the image rows those would meet are inside the tensor or masked like any
+    // row below the image, and a zero times either adds nothing
+    uint32_t oh2 = delta->y;
+    while ((oh2 * delta->x) % BK != 0 && oh2 <= 2 * delta->y) oh2++;
+    const size_t padded_floats = (size_t)B * ka * oh2 * delta->x;
+    if ((oh2 * delta->x) % BK == 0 && oh2 <= 2 * delta->y && padded_floats * 4 < 0x80000000ull) {
+      float *buf = nullptr;
+      if ((rc = mt::workspace_get(g_norm_ws, "padded delta", padded_floats, &buf))) return rc;
+      {
+        mt::ProfileScope prof("pad_rows");
+        pad_rows_kernel<<<cdiv(padded_floats, 256), 256, 0, mt::stream()>>>(buf, delta->p, DHW, oh2 * delta->x, padded_floats);
+        MT_LAUNCH_CHECK(name);
+      }
+      mt_tensor padded{buf, B, ka, oh2, delta->x};
+      return wgrad_batch_sum(name, dk, kx, ky, kz, ka, db, image, &padded, sx, sy, px, py);
+    }
+  }
   if (g_conv_path == 1 || DHW % BK != 0 || sample_image * 4 >= 0x80000000ull || sample_delta * 4 >= 0x80000000ull) {
     // per-sample gradients into the workspace, then their sum: the op sequence of the layer itself
     float *ws = nullptr;
@@ -2370,6 +2399,11 @@ int set_tconv_patch(int v) {
 int set_wgrad_patch(int v) {
   if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "wgrad_patch must be 0 or 1");
   g_wgrad_patch = v;
+  return MT_OK;
+}
+int set_wgrad_pad(int v) {
+  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "wgrad_pad must be 0 or 1");
+  g_wgrad_pad = v;
   return MT_OK;
 }
 int set_wgrad_parts(int v) {

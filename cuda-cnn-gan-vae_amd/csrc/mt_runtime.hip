@@ -257,6 +257,7 @@ int mt_set_option(const char *name, int value) {
   if (name && strcmp(name, "upconv_split") == 0) return mt::set_upconv_split(value);
   if (name && strcmp(name, "walk_wide") == 0) return mt::set_walk_wide(value);
   if (name && strcmp(name, "wgrad_parts") == 0) return mt::set_wgrad_parts(value);
+  if (name && strcmp(name, "wgrad_pad") == 0) return mt::set_wgrad_pad(value);
   if (name && strcmp(name, "wgrad_patch") == 0) return mt::set_wgrad_patch(value);
   if (name && strcmp(name, "tconv_patch") == 0) return mt::set_tconv_patch(value);
   if (name && strcmp(name, "pack_refresh") == 0) return mt::set_pack_refresh(value);

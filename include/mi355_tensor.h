@@ -107,6 +107,9 @@ int mt_timer_destroy(void *timer);
  *   "wgrad_parts"    1 (default) the general kernel of mt_convolution_backward_weights_sum cuts every sample into equal bands of
  *                    output rows (one partial sum per band) when samples x tiles are fewer blocks than the chip needs: layers
  *                    with few filters on large images / 0 never / n bands per sample (2..256, where the rows divide)
+ *   "wgrad_pad"      1 (default) mt_convolution_backward_weights_sum appends rows of zeros to delta's images when their pixels
+ *                    are not a multiple of 16 (3 x 4 at the end of a discriminator), so that the sum over the batch stays
+ *                    one product / 0 per-sample gradients and their sum then
  *   "tconv_patch"    1 (default) mt_backward_convolution of a 3x3 layer with stride 1, padding 1, at most 32 filters and at most 64
  *                    channels on large images (rows a multiple of 64 pixels, an even number of rows, at least 1024 tiles of
  *                    2 x 64 pixels in the batch) multiplies patches of delta held in LDS, nine taps per patch / 0 never

@@ -377,6 +377,9 @@ def test_wgrad_w_broadcast(gpu, oracle, path):
     (7, 1, 4, 4, 1, 1, 1, 0),        # 1x1 kernel, one channel, odd batch
     (16, 2, 64, 64, 3, 4, 2, 1),     # 1024 output pixels, 16 samples: the bias sum runs over the batch in four chunks
     (8, 1, 35, 35, 2, 3, 1, 0),      # 33x33 output pixels: rows that are no multiple of four floats, two chunks
+    (32, 16, 6, 8, 64, 5, 2, 2),     # 3x4 output pixels (the end of a discriminator): a row of zeros appended, one k loop per block
+    (8, 8, 6, 8, 24, 5, 2, 2),       # the same with 24 filters: the general kernel
+    (4, 3, 14, 14, 6, 3, 2, 1),      # 7x7 output pixels: no acceptable padding, per-sample path
 ])
 def test_convolution_backward_weights_sum(gpu, oracle, path, case):
     """The batch-summed weight gradient against the layer's own sequence: per-sample gradients into zeroed batch
