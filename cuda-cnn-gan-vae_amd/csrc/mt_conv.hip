@@ -611,6 +611,96 @@ __global__ __launch_bounds__(256) void tconv_k4s2_small_kernel(TconvArgs args) {
   }
 }
 
+// The same for kernel 5x5, stride 2, padding 2 (output exactly twice the input: the first layer of a discriminator on
+// images, backwards): output pixel (2*qy + py, 2*qx + px) reads input rows qy + py - 1 .. qy + 1 and columns
+// qx + px - 1 .. qx + 1, so the four phases -- 3x3, 3x2, 2x3 and 2x2 taps -- again share the 3x3 neighbourhood of the input
+// pixel: per input channel a thread issues 9 loads for 25*CO multiply-adds.  Phase (py, px) has 3-py by 3-px taps with
+// offsets (py-1, px-1); tap (ty, tx) multiplies neighbour (py + ty, px + tx).
+template <int CO>
+__global__ __launch_bounds__(256) void tconv_k5s2_small_kernel(TconvArgs args) {
+  constexpr int SLICES = 4, PIX = 64;
+  __shared__ float part[SLICES - 1][4 * CO][PIX];
+  const uint32_t H = args.H, W = args.W, C = args.C, HW = H * W;
+  const uint32_t pix = threadIdx.x % PIX, slice = threadIdx.x / PIX;   // the slice is uniform over a wavefront
+  const uint32_t n = blockIdx.x * PIX + pix;
+  const bool live = n < args.out_w * HW;
+  const uint32_t g = (live ? n : 0) / HW, r = (live ? n : 0) % HW, qy = r / W, qx = r % W;
+  __amdgpu_buffer_rsrc_t rsrc = make_rsrc(args.delta, args.in_w * C * HW * 4u);
+  const uint32_t imgoff = (g % args.in_w) * C * HW * 4u;
+  uint32_t voff[3][3];
+#pragma unroll
+  for (int dy = 0; dy < 3; dy++)
+#pragma unroll
+    for (int dx = 0; dx < 3; dx++) {
+      int32_t iy = (int32_t)qy + dy - 1, ix = (int32_t)qx + dx - 1;
+      bool ok = live && (uint32_t)iy < H && (uint32_t)ix < W;
+      voff[dy][dx] = ok ? imgoff + ((uint32_t)iy * W + (uint32_t)ix) * 4u : OOB;
+    }
+  float acc[2][2][CO];
+#pragma unroll
+  for (int i = 0; i < 4 * CO; i++) (&acc[0][0][0])[i] = 0.f;
+  const uint32_t M = args.M;
+  const uint32_t per = (C + SLICES - 1) / SLICES;
+  const uint32_t c_begin = __builtin_amdgcn_readfirstlane(slice * per);
+  const uint32_t c_end = c_begin + per < C ? c_begin + per : C;
+#pragma unroll 2
+  for (uint32_t ci = c_begin; ci < c_end; ci++) {
+    const uint32_t soff = ci * HW * 4u;
+    float v[3][3];
+#pragma unroll
+    for (int dy = 0; dy < 3; dy++)
+#pragma unroll
+      for (int dx = 0; dx < 3; dx++) v[dy][dx] = buf_load(rsrc, voff[dy][dx], soff);
+#pragma unroll
+    for (int py = 0; py < 2; py++)
+#pragma unroll
+      for (int px = 0; px < 2; px++) {
+        const TconvPhase &ph = args.ph[py * 2 + px];
+        const int ty_cnt = 3 - py, tx_cnt = 3 - px;
+#pragma unroll
+        for (int co = 0; co < CO; co++) {
+          if (co >= (int)M) continue;
+          const float *w = ph.packed + (size_t)co * ph.ld + ci * (uint32_t)(ty_cnt * tx_cnt);   // uniform: through the scalar cache
+          float a = acc[py][px][co];
+#pragma unroll
+          for (int ty = 0; ty < ty_cnt; ty++)
+#pragma unroll
+            for (int tx = 0; tx < tx_cnt; tx++) a = __builtin_fmaf(w[ty * tx_cnt + tx], v[py + ty][px + tx], a);
+          acc[py][px][co] = a;
+        }
+      }
+  }
+  if (slice > 0) {
+#pragma unroll
+    for (int i = 0; i < 4 * CO; i++) part[slice - 1][i][pix] = (&acc[0][0][0])[i];
+  }
+  __syncthreads();
+  if (slice > 0 || !live) return;
+#pragma unroll
+  for (int i = 0; i < 4 * CO; i++)
+#pragma unroll
+    for (int sl = 0; sl < SLICES - 1; sl++) (&acc[0][0][0])[i] += part[sl][i][pix];
+  const uint32_t OW = 2 * W, OHW = 4 * HW;
+  const float bsum = args.ep.tap_bias ? args.ep.tap_bias[g % args.ep.bias_w] : 0.f;
+  const int up = (uint32_t)((int32_t)qy - 1) < H, down = (uint32_t)((int32_t)qy + 1) < H;
+  const int left = (uint32_t)((int32_t)qx - 1) < W, right = (uint32_t)((int32_t)qx + 1) < W;
+#pragma unroll
+  for (int py = 0; py < 2; py++) {
+    // contributing input rows of output row 2*qy+py: qy-1 (py = 0 only), qy, qy+1; columns alike
+    const int ny = (py == 0 ? up : 0) + 1 + down;
+    const int nx0 = left + 1 + right, nx1 = 1 + right;
+#pragma unroll
+    for (int co = 0; co < CO; co++) {
+      if (co >= (int)M) continue;
+      float2 o;
+      o.x = mt::apply_func_epilogue(args.ep.func, acc[py][0][co] + bsum * (float)(ny * nx0));
+      o.y = mt::apply_func_epilogue(args.ep.func, acc[py][1][co] + bsum * (float)(ny * nx1));
+      float *dst = args.ep.C + ((size_t)g * M + co) * OHW + (size_t)(2 * qy + py) * OW + 2 * qx;
+      *reinterpret_cast<float2 *>(dst) = o;
+    }
+  }
+}
+
 // Staging of an input tile with a one-pixel halo through registers into LDS, shared by the vector-ALU kernels below:
 // per channel (TH+2) rows of [x0-1 | x0 .. x0+TW-1 | x0+TW] (PITCH floats, the tile itself starts at column 1), CC
 // channels per chunk.  The tile columns are fetched with 128-bit buffer loads, the two halo columns with 32-bit ones;
@@ -1366,6 +1456,21 @@ int launch_tconv_small(const char *name, TconvArgs &args, uint32_t max_n) {
     else if (args.M <= 2) tconv_k4s2_small_kernel<2><<<g4, 256, 0, mt::stream()>>>(args);
     else if (args.M == 3) tconv_k4s2_small_kernel<3><<<g4, 256, 0, mt::stream()>>>(args);
     else tconv_k4s2_small_kernel<4><<<g4, 256, 0, mt::stream()>>>(args);
+    MT_LAUNCH_CHECK(name);
+    return MT_OK;
+  }
+  // kernel 5x5, stride 2, padding 2 with the natural output size: phases of 3-py by 3-px taps with offsets py-1, px-1
+  bool k5s2 = args.nphase == 4 && args.ep.sy == 2 && args.ep.sx == 2 && args.ep.OW == 2 * args.W && args.ep.row_stride == 4 * args.H * args.W &&
+              ((uintptr_t)args.ep.C & 7u) == 0 && mt::fits_buffer((size_t)args.in_w * args.C * args.H * args.W);
+  for (uint32_t f = 0; k5s2 && f < 4; f++)
+    k5s2 = args.ph[f].py == f / 2 && args.ph[f].px == f % 2 && args.ph[f].offy == (int32_t)(f / 2) - 1 && args.ph[f].offx == (int32_t)(f % 2) - 1 &&
+           args.ph[f].taps_y == 3 - (int32_t)(f / 2) && args.ph[f].taps_x == 3 - (int32_t)(f % 2) && args.ph[f].qh == args.H && args.ph[f].qw == args.W;
+  if (k5s2) {
+    dim3 g5(cdiv((size_t)args.out_w * args.H * args.W, 64));
+    if (args.M <= 1) tconv_k5s2_small_kernel<1><<<g5, 256, 0, mt::stream()>>>(args);
+    else if (args.M <= 2) tconv_k5s2_small_kernel<2><<<g5, 256, 0, mt::stream()>>>(args);
+    else if (args.M == 3) tconv_k5s2_small_kernel<3><<<g5, 256, 0, mt::stream()>>>(args);
+    else tconv_k5s2_small_kernel<4><<<g5, 256, 0, mt::stream()>>>(args);
     MT_LAUNCH_CHECK(name);
     return MT_OK;
   }
