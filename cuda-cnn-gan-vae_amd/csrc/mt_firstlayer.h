@@ -217,7 +217,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 4)))
 // the shapes the kernel is built for; returns false when the layer is not one of them
 inline bool first_layer_launch(const char *name, FirstLayerArgs &a, int C, int KY, int KX, int S, int *rc) {
   *rc = MT_OK;
-  if (a.OW % 32 != 0 || a.OW % 4 != 0 || ((uintptr_t)a.out & 15u) || a.KA % 32 != 0 || a.KA > 64 || !epilogue_func(a.func)) return false;
+  if (a.OW % 32 != 0 || a.OW % 4 != 0 || ((uintptr_t)a.out & 15u) || a.KA < 8 || a.KA > 64 || !epilogue_func(a.func)) return false;   // (filters beyond KA in the last block of 32: zero weights, stores out of range)
   if (!fits_buffer((size_t)a.batch * a.KA * a.OH * a.OW)) return false;
   hipStream_t s = stream();
   auto go = [&](auto kernel, int th, int gx) {
@@ -232,8 +232,9 @@ inline bool first_layer_launch(const char *name, FirstLayerArgs &a, int C, int K
     if (e != hipSuccess) *rc = hip_fail(e, name);
     return true;
   };
-  const int nf = (int)a.KA / 32;
+  const int nf = ((int)a.KA + 31) / 32;
   if (C == 3 && KY == 5 && KX == 5 && S == 1 && nf == 1 && a.OW % 64 == 0) return go(first_layer_kernel<3, 5, 5, 1, 1, 2, 2>, 2, 2);
+  if (C == 3 && KY == 5 && KX == 5 && S == 2 && nf == 1) return go(first_layer_kernel<3, 5, 5, 2, 1, 4, 1>, 4, 1);
   if (C == 3 && KY == 3 && KX == 3 && S == 2 && nf == 1 && a.OW % 64 == 0) return go(first_layer_kernel<3, 3, 3, 2, 1, 4, 2>, 4, 2);
   if (C == 3 && KY == 3 && KX == 3 && S == 1 && nf == 1 && a.OW % 64 == 0) return go(first_layer_kernel<3, 3, 3, 1, 1, 4, 2>, 4, 2);
   if (C == 3 && KY == 4 && KX == 4 && S == 2 && nf == 2) return go(first_layer_kernel<3, 4, 4, 2, 2, 4, 1>, 4, 1);

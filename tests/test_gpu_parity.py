@@ -239,6 +239,9 @@ def test_forward_convolution_whose_blocks_walk_over_the_batch(gpu, oracle, case,
     (5, 18, 128, 32, 3, 2, 1),     # 9 output rows with tiles of four; more tiles than one pass of some blocks... and
     (40, 16, 64, 64, 4, 2, 1),     # 40 x 2 tiles of 4 x 32 pixels: blocks walk over the samples
     (2, 64, 60, 32, 5, 1, 2),      # 60 output columns: not this kernel (the general one runs)
+    (2, 48, 64, 16, 5, 2, 2),      # 5x5 stride 2 to 16 filters (the first layer of the reference's GAN discriminator): half a filter block
+    (3, 32, 64, 48, 4, 2, 1),      # 48 filters: a block and a half
+    (2, 16, 128, 12, 3, 1, 1),     # 12 filters
 ])
 @pytest.mark.parametrize("func", [None, "leaky_relu"])
 def test_first_layer_from_an_input_patch(gpu, oracle, case, func):
