@@ -34,7 +34,8 @@ int g_walk_wide = 1;       // 1: layers whose output channels are a multiple of 
 int g_upconv_split = 1;    // 1: up-sampling convolutions with fewer than 512 walking blocks share a tile's k steps between blocks
 int g_upconv_walk = 512;   // blocks from which the up-sampling convolution takes the walking kernel (0: never; measured on the
                            // shipped GAN generator at batch 32: 768 blocks 67.7 -> 54.6 and 58.6 -> 54.0 us, 384 blocks 65.1 -> 69 us)
-uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0, g_tconv_patch_launches = 0;
+uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0, g_tconv_patch_launches = 0, g_tconv_merge_launches = 0;
+int g_tconv_merge = 1;   // 1: a 5x5 stride-2 padding-2 transposed convolution to 5..16 channels runs as one 3x3 convolution to (channel, phase) rows, 0: never
 int g_tconv_patch = 1;   // 1: a 3x3 stride-1 transposed convolution from at most 32 filters to at most 64 channels on large images multiplies patches held in LDS (tconv3x3_patch_kernel), 0: never
 int g_wgrad_patch = 1;   // 1: the batch-summed weight gradient of a 3x3 stride-1 layer with at most 32 filters on large images multiplies patches held in LDS (wgrad_patch3x3_kernel), 0: never
 int g_wgrad_pad = 1;     // 1: the batch-summed weight gradient pads delta's images with rows of zeros when their pixels do not fill whole k steps, 0: per-sample gradients then
@@ -1670,6 +1671,47 @@ int g_tconv_walk = 1;  // plain calls (no batch norm folded in): 0 never walk, 1
 
 // norm / bn: only the kernel that walks over the batch implements them.  `handled` (required with either) tells the
 // caller whether it ran; if not, nothing was launched and the caller composes the result from separate passes.
+// ---- transposed convolution 5x5, stride 2, padding 2 to few channels as ONE 3x3 convolution ------------------------
+// Output pixel (2*qy + py, 2*qx + px) reads input rows qy + py - 1 .. qy + 1 and columns qx + px - 1 .. qx + 1: the four
+// stride phases are 3x3 stride-1 convolutions of the same input with (3 - py) x (3 - px) of the nine taps set, so all of
+// them are one convolution to 4 x CO "channels" (c, phase) -- 64 rows instead of four products of 16 -- whose result is
+// spread over the output afterwards.  36/25 of the multiplications, but one gather of the input instead of four, and
+// tiles of the size the matrix-core kernels are built for.
+// merged[(c*4 + py*2 + px)][f*9 + a*3 + b] = kernel[f][c*25 + (4 - (py + 2*(a - py)))*5 + (4 - (px + 2*(b - px)))] for
+// a >= py, b >= px (tap (a - py, b - px) of the phase, whose first coefficient is py, px), else 0; `zeros`: 4*CO zeros
+// behind it (the convolution's bias).
+__global__ __launch_bounds__(256) void tconv_k5s2_merge_kernel(float *merged, const float *kernel, uint32_t ker_ld, uint32_t CO, uint32_t F) {
+  const uint32_t cols = F * 9, total = 4 * CO * cols;
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= total + 4 * CO) return;
+  if (i >= total) { merged[i] = 0.f; return; }
+  const uint32_t r = i / cols, k = i % cols, c = r / 4, py = (r / 2) % 2, px = r % 2, f = k / 9, a = (k % 9) / 3, b = k % 3;
+  float v = 0.f;
+  if (a >= py && b >= px) v = kernel[(size_t)f * ker_ld + c * 25 + (4 - (py + 2 * (a - py))) * 5 + (4 - (px + 2 * (b - px)))];
+  merged[i] = v;
+}
+// out[w][c][2y + py][2x + px] = func(planes[w][c*4 + py*2 + px][y][x] + bias_sum * taps inside the image)
+__global__ __launch_bounds__(256) void tconv_k5s2_spread_kernel(float *out, const float *planes, const float *bias, uint32_t F, uint32_t rows, uint32_t H, uint32_t W, int func) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;   // (w, c, y, x)
+  if (i >= (size_t)rows * H * W) return;
+  const uint32_t x = (uint32_t)(i % W), y = (uint32_t)((i / W) % H);
+  const size_t row = i / ((size_t)W * H);   // w * CO + c
+  float bias_sum = 0.f;
+  for (uint32_t f = 0; f < F; f++) bias_sum += bias[f];
+  const size_t HW = (size_t)H * W;
+  const float *p = planes + row * 4 * HW + (size_t)y * W + x;
+  const float up = y > 0 ? 1.f : 0.f, down = y + 1 < H ? 1.f : 0.f, left = x > 0 ? 1.f : 0.f, right = x + 1 < W ? 1.f : 0.f;
+  const float ny0 = up + 1.f + down, ny1 = 1.f + down, nx0 = left + 1.f + right, nx1 = 1.f + right;
+  float2 top, bottom;
+  top.x = mt::apply_func_epilogue(func, p[0] + bias_sum * (ny0 * nx0));
+  top.y = mt::apply_func_epilogue(func, p[HW] + bias_sum * (ny0 * nx1));
+  bottom.x = mt::apply_func_epilogue(func, p[2 * HW] + bias_sum * (ny1 * nx0));
+  bottom.y = mt::apply_func_epilogue(func, p[3 * HW] + bias_sum * (ny1 * nx1));
+  float *dst = out + row * 4 * HW + (size_t)(2 * y) * (2 * W) + 2 * x;
+  *reinterpret_cast<float2 *>(dst) = top;
+  *reinterpret_cast<float2 *>(dst + 2 * W) = bottom;
+}
+
 int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
              const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func, const NormIn *norm = nullptr, const BnOut *bn = nullptr,
              bool *handled = nullptr) {
@@ -1713,6 +1755,32 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     return MT_OK;
   }
 
+  // 5 x 5, stride 2, padding 2 to 5..16 channels at twice the input size: the four phases as one 3 x 3 convolution to
+  // (channel, phase) rows, spread over the output afterwards
+  if (g_tconv_merge && !fused && mt::igemm::tile_override() < 0 && kx == 5 && ky == 5 && sx == 2 && sy == 2 && px == 2 && py == 2 && bias->w == 1 &&
+      delta->w == out->w && out->y == 2 * delta->y && out->x == 2 * delta->x && kz > 4 && kz <= 16 && ka >= 16 && mt::epilogue_func(func) &&
+      ((uintptr_t)out->p & 7u) == 0 && mt::fits_buffer(mt::count(out)) && (size_t)out->w * delta->y * delta->x >= 16384) {
+    const uint32_t rows4 = 4u * (uint32_t)kz, cols = ka * 9u;
+    const size_t merged_floats = ((size_t)rows4 * cols + rows4 + 3) & ~(size_t)3, plane_floats = mt::count(out);
+    float *buf = nullptr;
+    if ((rc = mt::workspace_get(g_norm_ws, "merged phases", merged_floats + plane_floats, &buf))) return rc;
+    float *planes = buf + merged_floats;
+    {
+      mt::ProfileScope prof("tconv_prepare");
+      tconv_k5s2_merge_kernel<<<cdiv((size_t)rows4 * cols + rows4, 256), 256, 0, mt::stream()>>>(buf, kernel->p, kernel->x, (uint32_t)kz, ka);
+      MT_LAUNCH_CHECK(name);
+    }
+    mt::note_write(buf, (merged_floats + plane_floats) * sizeof(float));   // (a copy of these weights that the forward pass kept is stale)
+    mt_tensor merged{buf, 1, 1, rows4, cols}, zeros{buf + (size_t)rows4 * cols, 1, rows4, 1, 1}, wide{planes, out->w, rows4, delta->y, delta->x};
+    if ((rc = forward(name, &wide, delta, &merged, 3, 3, (int32_t)ka, rows4, &zeros, 1, 1, 1, 1, MT_F_NONE))) return rc;
+    {
+      mt::ProfileScope prof("tconv_spread");
+      tconv_k5s2_spread_kernel<<<cdiv(plane_floats / 4, 256), 256, 0, mt::stream()>>>(out->p, planes, bias->p, ka, out->w * (uint32_t)kz, delta->y, delta->x, func);
+      MT_LAUNCH_CHECK(name);
+    }
+    g_tconv_merge_launches++;
+    return MT_OK;
+  }
   // few filters of 3 x 3, stride 1, padding 1 on large images: the nine taps share one patch of delta in LDS, the weights are
   // read as they lie
   if (g_tconv_patch && !fused && mt::igemm::tile_override() < 0 && kx == 3 && ky == 3 && sx == 1 && sy == 1 && px == 1 && py == 1 && bias->w == 1 &&
@@ -2413,6 +2481,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "convolution_workspace_bytes") == 0) { *value = (int64_t)(g_ws.floats * sizeof(float)); return true; }
   if (strcmp(name, "wgrad_walk_launches") == 0) { *value = (int64_t)g_wgrad_walk_launches; return true; }
   if (strcmp(name, "wgrad_patch_launches") == 0) { *value = (int64_t)g_wgrad_patch_launches; return true; }
+  if (strcmp(name, "tconv_merge_launches") == 0) { *value = (int64_t)g_tconv_merge_launches; return true; }
   if (strcmp(name, "tconv_patch_launches") == 0) { *value = (int64_t)g_tconv_patch_launches; return true; }
   return false;
 }
@@ -2494,6 +2563,11 @@ int set_upconv_split(int v) {
 int set_upconv_walk(int v) {
   if (v < 0) return fail(MT_E_ARGUMENT, "upconv_walk must be 0 (never) or the number of blocks from which the walking kernel is taken");
   g_upconv_walk = v;
+  return MT_OK;
+}
+int set_tconv_merge(int v) {
+  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "tconv_merge must be 0 or 1");
+  g_tconv_merge = v;
   return MT_OK;
 }
 int set_tconv_patch(int v) {

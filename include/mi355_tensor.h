@@ -110,6 +110,8 @@ int mt_timer_destroy(void *timer);
  *   "wgrad_pad"      1 (default) mt_convolution_backward_weights_sum appends rows of zeros to delta's images when their pixels
  *                    are not a multiple of 16 (3 x 4 at the end of a discriminator), so that the sum over the batch stays
  *                    one product / 0 per-sample gradients and their sum then
+ *   "tconv_merge"    1 (default) mt_backward_convolution 5x5 stride 2 padding 2 to 5..16 channels at twice the input size runs its
+ *                    four stride phases as one 3x3 convolution to (channel, phase) rows and spreads them over the output / 0 never
  *   "tconv_patch"    1 (default) mt_backward_convolution of a 3x3 layer with stride 1, padding 1, at most 32 filters and at most 64
  *                    channels on large images (rows a multiple of 64 pixels, an even number of rows, at least 1024 tiles of
  *                    2 x 64 pixels in the batch) multiplies patches of delta held in LDS, nine taps per patch / 0 never
@@ -170,6 +172,7 @@ int mt_set_option(const char *name, int value);
  *   "wgrad_walk_launches"                                  calls of mt_convolution_backward_weights_sum that ran as one k loop
  *                                                          per block (option "wgrad_walk")
  *   "wgrad_patch_launches"                                 calls of it that multiplied patches held in LDS (option "wgrad_patch")
+ *   "tconv_merge_launches"                                 calls of mt_backward_convolution that ran as one merged convolution (option "tconv_merge")
  *   "tconv_patch_launches"                                 calls of mt_backward_convolution that did (option "tconv_patch") */
 int mt_get_info(const char *name, int64_t *value);
 

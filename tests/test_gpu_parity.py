@@ -442,6 +442,42 @@ def test_weights_sum_in_bands_of_rows(gpu, oracle, case):
 
 
 @pytest.mark.parametrize("case", [
+    # B, C (output channels), H, W (of delta), KA (filters), func, taken
+    (4, 16, 64, 64, 32, None, 1),          # the second layer of a discriminator on images, backwards: 32 filters to 16 channels
+    (5, 8, 48, 80, 16, "leaky_relu", 1),   # 16 filters to 8 channels, a function in the same pass
+    (16, 13, 32, 32, 20, None, 1),         # ragged counts
+    (4, 16, 64, 64, 8, None, 0),           # 8 filters: too short a k axis, the phases one by one
+    (4, 20, 64, 64, 32, None, 0),          # 20 channels: the phases one by one
+    (2, 16, 32, 32, 32, None, 0),          # too few pixels
+])
+def test_transposed_convolution_5x5_stride_2_as_one_3x3_convolution(gpu, oracle, case):
+    """The backward pass of a 5 x 5 stride-2 padding-2 layer to few channels as one 3 x 3 convolution to (channel, phase)
+    rows that is spread over the output afterwards, with a non-zero bias (added once per tap inside the image,
+    cpu/ctensorconv.h:204-268), against the oracle and against the phases run one by one."""
+    import mi355tensor as mt
+    B, C, H, Wd, KA, func, taken = case
+    delta = U(71, B, KA, H, Wd)
+    kernel = U(72, 1, 1, KA, C * 25) * np.float32(0.2)
+    bias = U(73, 1, KA, 1, 1) * np.float32(0.1)
+    args = (delta, kernel, bias, 5, 5, C, KA, 2, 2, 2, 2, (B, C, 2 * H, 2 * Wd))
+    want = oracle.backward_convolution(*args)
+    if func:
+        want = oracle.apply_func(want, func)
+    got = {}
+    try:
+        for on in (1, 0):
+            mt.set_option("tconv_merge", on)
+            before = mt.get_info("tconv_merge_launches")
+            got[on] = gpu.backward_convolution(*args, func=func)
+            assert mt.get_info("tconv_merge_launches") - before == (taken if on else 0)
+    finally:
+        mt.set_option("tconv_merge", 1)
+    close(got[1], want)
+    close(got[0], want)
+    close(got[1], got[0], 2e-6)
+
+
+@pytest.mark.parametrize("case", [
     # B, C, H, W, KA, func, taken
     (4, 32, 64, 512, 16, None, 1),        # 16 filters to 32 channels: a wave per (16 channels, row of the tile)
     (8, 16, 32, 512, 3, None, 1),         # an image layer's backward pass: 3 filters to 16 channels
