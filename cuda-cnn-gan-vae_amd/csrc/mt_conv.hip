@@ -60,7 +60,7 @@ int with_row_k(const float *p, uint32_t ld, uint32_t R, uint32_t K, Batch bt, F 
 
 // ---- library-owned workspace: the partial sums of the batch-summed gradients, up-sampled images, and re-ordered
 // weights while they cannot be kept (see below)
-mt::Workspace g_ws, g_stats_ws, g_norm_ws;
+mt::Workspace g_ws, g_stats_ws, g_norm_ws, g_pad_ws, g_merge_ws;   // (one per use: a call that takes its input from one of them may need another)
 int workspace(size_t floats, float **p) { return mt::workspace_get(g_ws, "convolution workspace", floats, p); }
 
 // ---- re-ordered weights, kept between calls ---------------------------------------------------------------------
@@ -1763,7 +1763,7 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     const uint32_t rows4 = 4u * (uint32_t)kz, cols = ka * 9u;
     const size_t merged_floats = ((size_t)rows4 * cols + rows4 + 3) & ~(size_t)3, plane_floats = mt::count(out);
     float *buf = nullptr;
-    if ((rc = mt::workspace_get(g_norm_ws, "merged phases", merged_floats + plane_floats, &buf))) return rc;
+    if ((rc = mt::workspace_get(g_merge_ws, "merged phases", merged_floats + plane_floats, &buf))) return rc;
     float *planes = buf + merged_floats;
     {
       mt::ProfileScope prof("tconv_prepare");
@@ -2072,7 +2072,7 @@ int wgrad_batch_sum(const char *name, const mt_tensor *dk, int32_t kx, int32_t k
     const size_t padded_floats = (size_t)B * ka * oh2 * delta->x;
     if ((oh2 * delta->x) % BK == 0 && oh2 <= 2 * delta->y && padded_floats * 4 < 0x80000000ull) {
       float *buf = nullptr;
-      if ((rc = mt::workspace_get(g_norm_ws, "padded delta", padded_floats, &buf))) return rc;
+      if ((rc = mt::workspace_get(g_pad_ws, "padded delta", padded_floats, &buf))) return rc;
       {
         mt::ProfileScope prof("pad_rows");
         pad_rows_kernel<<<cdiv(padded_floats, 256), 256, 0, mt::stream()>>>(buf, delta->p, DHW, oh2 * delta->x, padded_floats);

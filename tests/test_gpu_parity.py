@@ -1395,6 +1395,26 @@ def test_transposed_convolution_between_batch_norms(gpu, oracle, shape, bias_std
     close(out.numpy(), oracle.apply_func(y, "relu"))
 
 
+def test_normalised_input_in_front_of_the_merged_5x5_route(gpu, oracle):
+    """mt_backward_convolution_norm_func on a shape that does not walk normalises its input into a workspace and runs the plain
+    layer on it; a 5 x 5 stride-2 layer to 16 channels then takes the route that needs a workspace of its own (the phases as
+    one 3 x 3 convolution): the two must not share one."""
+    import mi355tensor as mt
+    from mi355tensor import CTensor, Fused
+    B, cin, cout, H, W = 4, 32, 16, 64, 64
+    x = Nrm(81, B, cin, H, W)
+    pairs = np.stack([U(82, 1, cin, H, W, lo=0.5, hi=1.5), U(83, 1, cin, H, W, lo=-0.3, hi=0.3)], -1).reshape(1, cin, H, 2 * W).astype(np.float32)
+    kernel, bias = Nrm(84, 1, 1, cin, cout * 25, std=0.05), Nrm(85, 1, cin, 1, 1, std=0.02)
+    a = np.maximum(pairs.reshape(1, cin, H, W, 2)[..., 0] * x + pairs.reshape(1, cin, H, W, 2)[..., 1], 0).astype(np.float32)
+    want = oracle.backward_convolution(a, kernel, bias, 5, 5, cout, cin, 2, 2, 2, 2, (B, cout, 2 * H, 2 * W))
+    out = CTensor(B, cout, 2 * H, 2 * W)
+    before = mt.get_info("tconv_merge_launches")
+    Fused.BackwardConvolutionNorm(out, CTensor.from_numpy(x), CTensor.from_numpy(pairs), "relu", CTensor.from_numpy(kernel), 5, 5, cout, cin,
+                                  CTensor.from_numpy(bias), 2, 2, 2, 2)
+    assert mt.get_info("tconv_merge_launches") == before + 1
+    close(out.numpy(), want)
+
+
 def test_wavefront_priorities_change_no_result(gpu):
     """The priorities that keep the blocks of a compute unit together only change which wavefront is served first: the
     walking transposed convolution (plain and with statistics) and a one-tile product give bit-identical results with
