@@ -1669,8 +1669,6 @@ struct BnOut {    // statistics of the output over the batch, turned into (scale
 };
 int g_tconv_walk = 1;  // plain calls (no batch norm folded in): 0 never walk, 1 walk wherever the shape allows
 
-// norm / bn: only the kernel that walks over the batch implements them.  `handled` (required with either) tells the
-// caller whether it ran; if not, nothing was launched and the caller composes the result from separate passes.
 // ---- transposed convolution 5x5, stride 2, padding 2 to few channels as ONE 3x3 convolution ------------------------
 // Output pixel (2*qy + py, 2*qx + px) reads input rows qy + py - 1 .. qy + 1 and columns qx + px - 1 .. qx + 1: the four
 // stride phases are 3x3 stride-1 convolutions of the same input with (3 - py) x (3 - px) of the nine taps set, so all of
@@ -1712,6 +1710,8 @@ __global__ __launch_bounds__(256) void tconv_k5s2_spread_kernel(float *out, cons
   *reinterpret_cast<float2 *>(dst + 2 * W) = bottom;
 }
 
+// norm / bn: only the kernel that walks over the batch implements them.  `handled` (required with either) tells the
+// caller whether it ran; if not, nothing was launched and the caller composes the result from separate passes.
 int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
              const mt_tensor *bias, int32_t sx, int32_t sy, int32_t px, int32_t py, int func, const NormIn *norm = nullptr, const BnOut *bn = nullptr,
              bool *handled = nullptr) {
