@@ -1918,7 +1918,10 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
     if (handled) *handled = true;
   }
   if (tile) return launch_tconv_tile(name, args);
-  if (kz <= 4 && mt::igemm::tile_override() < 0) {
+  // (a small output behind a long k axis -- 128 filters to one channel at 16 x 16 -- has too few pixels for one thread each:
+  // the matrix-core path cuts its k axis over blocks)
+  const bool few_pixels = (size_t)max_n * args.nphase < 32768 && (size_t)ka * ky * kx >= 512;
+  if (kz <= 4 && mt::igemm::tile_override() < 0 && !few_pixels) {
     rc = launch_tconv_small(name, args, max_n);
     if (rc >= 0) return rc;
   }

@@ -802,6 +802,78 @@ static void TimeGanDiscriminator(uint32_t batch,uint32_t warmup,uint32_t steps)
         batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),out.GetElement(0,0,0,0),driver_allocations_in_the_timed_steps);
 }
 
+// a convolution layer's weights as the layer saves them: uniform in +-scale (scale 0: sqrt(6 / columns)), small biases
+static void LoadConvolution(INetLayer<type_t> &layer,uint32_t amount,int32_t size,uint32_t depth,int32_t stride,int32_t padding,double scale=0)
+{
+ const uint32_t columns=depth*size*size;
+ CMemoryStream w;
+ w.SaveUInt32(amount);w.SaveInt32(size);w.SaveInt32(size);w.SaveInt32(depth);w.SaveInt32(stride);w.SaveInt32(stride);w.SaveInt32(padding);w.SaveInt32(padding);
+ w.PutTensor(1,1,amount,columns,Values(static_cast<size_t>(amount)*columns,scale>0?scale:sqrt(6.0/columns)));
+ w.PutTensor(1,amount,1,1,Values(amount,0.05));
+ layer.Load(&w);
+}
+
+// The reference's VAE model (cuda/netmodel/cmodel_vae.cu.h:130-230), whole training step in Adam mode, batch 32, 256x256 images.
+// Coder: three times (Convolution 5x5 stride 2 padding 2, BatchNormalization, leaky ReLU) to 32, 64, 128 filters, Splitter, two
+// Convolutions 5x5 stride 2 to one filter (mu, log variance: 16x16), VAECoderOutput.  Decoder: seven Convolutions 3x3 (128, 128, 128,
+// 64, 64, 32 filters with BatchNormalization and leaky ReLU, UpSampling 2x2 in front of the third to the sixth; then 3 filters and
+// leaky ReLU): 256x256 images.
+static void TimeVae(uint32_t batch,uint32_t warmup,uint32_t steps)
+{
+ rng_state=0xA4093822299F31D0ull;
+ std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
+ std::vector<INetLayer<type_t>*> net;
+#define PUSH(LAYER) {owner.push_back(std::shared_ptr<INetLayer<type_t> >(LAYER));net.push_back(owner.back().get());}
+ PUSH(new CNetLayerConvolutionInput<type_t>(3,256,256,batch));
+ static const uint32_t coder[4]={3,32,64,128};
+ for(uint32_t i=0;i<3;i++)
+ {
+  PUSH(new CNetLayerConvolution<type_t>(coder[i+1],5,2,2,2,2,net.back(),batch));
+  LoadConvolution(*net.back(),coder[i+1],5,coder[i],2,2);
+  PUSH(new CNetLayerBatchNormalization<type_t>(0.9f,net.back(),batch));
+  net.back()->Reset();
+  PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_LEAKY_RELU,net.back(),batch));
+ }
+ PUSH(new CNetLayerSplitter<type_t>(2,net.back(),batch));
+ INetLayer<type_t> *splitter=net.back();
+ PUSH(new CNetLayerConvolution<type_t>(1,5,2,2,2,2,splitter,batch));
+ LoadConvolution(*net.back(),1,5,128,2,2);
+ INetLayer<type_t> *mu=net.back();
+ PUSH(new CNetLayerConvolution<type_t>(1,5,2,2,2,2,splitter,batch));
+ LoadConvolution(*net.back(),1,5,128,2,2,0.01);
+ INetLayer<type_t> *logvar=net.back();
+ PUSH(new CNetLayerVAECoderOutput<type_t>(0.001f,mu,logvar,batch));
+ static const uint32_t decoder[8]={1,128,128,128,64,64,32,3};
+ for(uint32_t i=0;i<7;i++)
+ {
+  if (i>=2 && i<=5) PUSH(new CNetLayerUpSampling<type_t>(2,2,net.back(),batch));
+  PUSH(new CNetLayerConvolution<type_t>(decoder[i+1],3,1,1,1,1,net.back(),batch));
+  LoadConvolution(*net.back(),decoder[i+1],3,decoder[i],1,1);
+  if (i<6)
+  {
+   PUSH(new CNetLayerBatchNormalization<type_t>(0.9f,net.back(),batch));
+   net.back()->Reset();
+  }
+  PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_LEAKY_RELU,net.back(),batch));
+ }
+#undef PUSH
+ for(size_t n=0;n<net.size();n++)
+ {
+  net[n]->TrainingModeAdam(0.9,0.999);   // as the model trains it (cuda/netmodel/cmodel_basicvae.cu.h:487-492)
+  net[n]->TrainingStart();
+ }
+ CTensor<type_t> image(batch,3,256,256),error(batch,3,256,256);
+ FillTensor(image,1.0);
+ FillTensor(error,0.01);
+ net[0]->SetOutput(image);
+ double ms=TimeSteps("VAE step",net,&error,warmup,steps);
+ CTensor<type_t> &out=net.back()->GetOutputTensor();
+ double sum=0;
+ for(uint32_t x=0;x<256;x++) sum+=fabs(out.GetElement(batch-1,2,255,x));
+ printf("{\"chain\": \"vae_step\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"last_row_abs_sum\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
+        batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),sum,driver_allocations_in_the_timed_steps);
+}
+
 // Chain K: two training steps (gradient descent) of the discriminator at batch 16, once with the per-sample weight gradients deferred by the
 // drop-in classes (mi355::CDeferredGradient; the last two convolution layers qualify) and once with every call run when
 // it is made: same seeds, the updated convolution weights of both runs go to the dump
@@ -940,7 +1012,7 @@ int main(int argc,char **argv)
    fclose(out_file);
    return(0);
   }
-  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up [literal | train]]]
+  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up [literal | train | vae]]]
   {
    const uint32_t steps=(argc>3)?static_cast<uint32_t>(atoi(argv[3])):50,warmup=(argc>4)?static_cast<uint32_t>(atoi(argv[4])):20;
    TimeGenerator(256,warmup,steps);
@@ -951,6 +1023,7 @@ int main(int argc,char **argv)
     TimeGanGenerator(32,warmup,steps,true);
     TimeGanDiscriminator(32,warmup,steps);
    }
+   if (argc>5 && strcmp(argv[5],"vae")==0) TimeVae(32,warmup,steps);   // or the whole training step of the reference's VAE model
    if (argc>5 && strcmp(argv[5],"literal")==0)   // and the last chain once more with every call run when it is made
    {
     mi355::DeferGradients()=false;

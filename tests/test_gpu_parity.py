@@ -178,6 +178,7 @@ CONV_CASES = [
     (2, 8, 18, 36, 4, 3, 3, 1, 1, 1, 1, 1, 2),      # the same with partial tiles and one bias set per sample
     (2, 8, 8, 8, 256, 4, 4, 2, 2, 1, 1, 1, 1),      # transposed conv with few blocks and k = 1024 per phase: split over k
     (1, 8, 5, 5, 1024, 3, 3, 2, 2, 1, 1, 1, 1),     # the same with phases of 4, 2, 2 and 1 taps (k = 4096 ... 1024)
+    (8, 1, 16, 16, 128, 3, 3, 1, 1, 1, 1, 1, 1),    # 128 filters to one channel at 16 x 16: few pixels behind a long k axis, split over k
     (3, 3, 24, 32, 16, 5, 5, 2, 2, 2, 2, 1, 1),     # 5x5 stride 2 padding 2 to three channels (a discriminator's first layer, backwards):
                                                     # the four phases from the 3x3 neighbourhood of an input pixel
     (2, 1, 10, 12, 5, 5, 5, 2, 2, 2, 2, 1, 2),      # the same to one channel, one bias set per sample
