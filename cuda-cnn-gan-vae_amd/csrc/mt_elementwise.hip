@@ -1786,7 +1786,13 @@ static int bn_forward_train(const mt_tensor *out, const mt_tensor *in, const mt_
   bn_fused_kernel<RB, NW><<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func, om, ov, pp)
 #define MT_BN_FUSED_NW(RB) \
   do { if (nw <= 8) MT_BN_FUSED(RB, 8); else if (nw <= 16) MT_BN_FUSED(RB, 16); else MT_BN_FUSED(RB, 32); } while (0)
-      if (rb == 64) { if (nw <= 8) MT_BN_FUSED(64, 8); else MT_BN_FUSED(64, 16); }
+      if (rb == 64 && streamed(S * W * sizeof(float))) {   // a large tensor, every element touched once: past the caches
+#define MT_BN_FUSED_NT(NW) \
+  bn_fused_kernel<64, NW, EW_THREADS, true><<<grid, EW_THREADS, 0, mt::stream()>>>(out->p, xhat ? xhat->p : nullptr, in->p, W, (uint32_t)S, inv_n, epsilon, pm, pv, pi, nm, nv, momentum, mom_new, gamma->p, beta->p, func, om, ov, pp)
+        if (nw <= 8) MT_BN_FUSED_NT(8); else MT_BN_FUSED_NT(16);
+#undef MT_BN_FUSED_NT
+      }
+      else if (rb == 64) { if (nw <= 8) MT_BN_FUSED(64, 8); else MT_BN_FUSED(64, 16); }
       else if (rb == 32) MT_BN_FUSED_NW(32); else if (rb == 16) MT_BN_FUSED_NW(16); else MT_BN_FUSED_NW(8);
 #undef MT_BN_FUSED_NW
 #undef MT_BN_FUSED

@@ -1179,6 +1179,28 @@ def test_batchnorm_forward_of_large_batches(gpu, oracle, shape):
         mt.set_option("nontemporal", 2)
 
 
+@pytest.mark.parametrize("shape", [(8, 8, 128, 128), (40, 2, 256, 256)])
+def test_batchnorm_forward_of_small_batches_on_large_tensors(gpu, oracle, shape):
+    """A small batch on a large tensor: blocks of 64 column groups, 8 or 16 rows per thread; with ordinary accesses and with the
+    non-temporal ones that tensors of 128 MiB and more get.  Every output of the layer against the oracle's op sequence."""
+    import mi355tensor as mt
+    one = (1,) + tuple(shape[1:])
+    x, gamma, beta, nm, nv = Nrm(1, *shape) * 1.5 + 0.3, U(2, *one) + 1.5, U(3, *one), U(4, *one), np.abs(U(5, *one))
+    want = seq.batchnorm_forward_train(oracle, x, gamma, beta, nm, nv, 0.9)
+    got = {}
+    try:
+        for past_caches in (2, 1):
+            mt.set_option("nontemporal", past_caches)
+            got[past_caches] = gpu.batchnorm_train(x, gamma, beta, 0.9, seq.BN_EPSILON, None, nm, nv)
+            for key in ("out", "xhat", "ivar", "mean", "var", "new_mean", "new_var"):
+                close(got[past_caches][key], want[key], 1e-5)
+            close(gpu.batchnorm_train(x, gamma, beta, func="leaky_relu")["out"], oracle.apply_func(want["out"], "leaky_relu"), 1e-5)
+    finally:
+        mt.set_option("nontemporal", 2)
+    for key in ("out", "xhat"):
+        assert np.array_equal(got[1][key], got[2][key])
+
+
 @pytest.mark.parametrize("shape", [(16, 3, 6, 6), (5, 2, 3, 3), (40, 8, 16, 16), (130, 4, 8, 8), (300, 1, 4, 8), (7, 64, 32, 32),
                                    (600, 2, 4, 8), (1024, 1, 8, 8), (1100, 1, 4, 8)])   # the last three: 1024 threads per block; rows read twice
 def test_batchnorm_backward_fused(gpu, oracle, shape):
