@@ -771,6 +771,22 @@ inline bool wgrad_walk_plan(WgradWalkArgs &a, uint32_t batch, bool may_split_sam
   uint32_t steps = batch / a.groups * nb;
   if (may_split_samples && a.groups == batch)   // one sample per group and still few blocks: equal shares of a sample's steps
     while (steps % 2 == 0 && steps / 2 >= 16 && (uint64_t)a.tiles_m * a.tiles_n * a.groups < 512) { steps /= 2; a.groups *= 2; }
+  if (may_split_samples && steps >= 48) {
+    // The blocks come in rounds of one per compute unit: 576 blocks are three rounds, the last an eighth full.  More groups of
+    // fewer steps each can fill the rounds (a group need not end with a sample); a group's first loads and its tile's way
+    // out cost about eight steps' time.
+    const uint64_t tiles = (uint64_t)a.tiles_m * a.tiles_n;
+    auto cost = [&](uint64_t groups, uint32_t st) { return (double)((tiles * groups + 255) / 256) / (double)groups * (1.0 + 8.0 / (double)st); };
+    double best = cost(a.groups, steps);
+    uint32_t pick = 1;
+    for (uint32_t m : {2u, 3u, 4u, 6u, 8u, 12u, 16u}) {
+      if (steps % m != 0 || (steps / m) % 2 != 0 || steps / m < 24) continue;
+      if ((uint64_t)a.groups * m * a.M * a.N > ((uint64_t)1 << 26)) continue;   // (the groups' tiles: at most 256 MB)
+      const double c = cost((uint64_t)a.groups * m, steps / m);
+      if (c < 0.97 * best) { best = c; pick = m; }
+    }
+    steps /= pick; a.groups *= pick;
+  }
   if (a.groups < 2 || steps < 4 || steps % 2 != 0) return false;
   a.steps = steps;
   const uint64_t samples = (steps + nb - 1) / nb, front = (uint64_t)a.py * a.W + a.px;
