@@ -34,7 +34,8 @@ int g_walk_wide = 1;       // 1: layers whose output channels are a multiple of 
 int g_upconv_split = 1;    // 1: up-sampling convolutions with fewer than 512 walking blocks share a tile's k steps between blocks
 int g_upconv_walk = 512;   // blocks from which the up-sampling convolution takes the walking kernel (0: never; measured on the
                            // shipped GAN generator at batch 32: 768 blocks 67.7 -> 54.6 and 58.6 -> 54.0 us, 384 blocks 65.1 -> 69 us)
-uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0, g_tconv_patch_launches = 0, g_tconv_merge_launches = 0;
+uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0, g_tconv_patch_launches = 0, g_tconv_merge_launches = 0, g_tconv_as_conv_launches = 0;
+int g_tconv_as_conv = 1;   // 1: a stride-1 transposed convolution whose taps do not tile the k step (3x3) runs as the forward convolution with flipped kernels, 0: never
 int g_tconv_merge = 1;   // 1: a 5x5 stride-2 padding-2 transposed convolution to 5..16 channels runs as one 3x3 convolution to (channel, phase) rows, 0: never
 int g_tconv_patch = 1;   // 1: a 3x3 stride-1 transposed convolution from at most 32 filters to at most 64 channels on large images multiplies patches held in LDS (tconv3x3_patch_kernel), 0: never
 int g_wgrad_patch = 1;   // 1: the batch-summed weight gradient of a 3x3 stride-1 layer with at most 32 filters on large images multiplies patches held in LDS (wgrad_patch3x3_kernel), 0: never
@@ -1710,6 +1711,42 @@ __global__ __launch_bounds__(256) void tconv_k5s2_spread_kernel(float *out, cons
   *reinterpret_cast<float2 *>(dst + 2 * W) = bottom;
 }
 
+// ---- stride-1 transposed convolution as the forward convolution it is ---------------------------------------------------
+// out[c][y][x] = sum over (f, a, b) of kernel[f][c*taps + a*KX + b] * delta[f][y - a + py][x - b + px] is the forward
+// convolution of delta with the kernels flipped and transposed, padding K - 1 - p: flipped[c][f*taps + t] =
+// kernel[f][c*taps + taps - 1 - t].  The forward path orders k tap-major (16 channels of one tap per k step: one input
+// offset per step), which a kernel whose taps do not tile the k step (3 x 3) cannot have in the phase formulation above.
+// Behind the flipped weights: CO zeros (the convolution's bias) and the sum of the filters' biases, which the reference
+// adds once per tap inside the image (cpu/ctensorconv.h:204-268).
+__global__ __launch_bounds__(256) void tconv_s1_flip_kernel(float *flipped, const float *kernel, const float *bias, uint32_t ker_ld, uint32_t CO, uint32_t F, uint32_t taps) {
+  const uint32_t cols = F * taps, total = CO * cols;
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i < total) {
+    const uint32_t c = i / cols, k = i % cols, f = k / taps, t = k % taps;
+    flipped[i] = kernel[(size_t)f * ker_ld + c * taps + (taps - 1 - t)];
+  } else if (i < total + CO) {
+    flipped[i] = 0.f;
+  } else if (i == total + CO) {
+    float sum = 0.f;
+    for (uint32_t f = 0; f < F; f++) sum += bias[f];
+    flipped[i] = sum;
+  }
+}
+// out[row][y][x] += bias_sum * (taps of (y, x) inside the input image); nothing to do when the sum is zero (a layer's
+// backward pass hands over zeroed biases)
+__global__ __launch_bounds__(256) void tconv_s1_bias_kernel(float *out, const float *bias_sum, size_t total, uint32_t OH, uint32_t OW, uint32_t IH, uint32_t IW,
+                                                            int32_t KY, int32_t KX, int32_t pad_y, int32_t pad_x) {
+  const float sum = *bias_sum;
+  if (sum == 0.f) return;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    const uint32_t x = (uint32_t)(i % OW), y = (uint32_t)((i / OW) % OH);
+    int ny = 0, nx = 0;
+    for (int32_t t = 0; t < KY; t++) ny += (uint32_t)((int32_t)y + t - pad_y) < IH;
+    for (int32_t t = 0; t < KX; t++) nx += (uint32_t)((int32_t)x + t - pad_x) < IW;
+    out[i] += sum * (float)(ny * nx);
+  }
+}
+
 // norm / bn: only the kernel that walks over the batch implements them.  `handled` (required with either) tells the
 // caller whether it ran; if not, nothing was launched and the caller composes the result from separate passes.
 int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, const mt_tensor *kernel, int32_t kx, int32_t ky, int32_t kz, uint32_t ka,
@@ -1796,6 +1833,32 @@ int backward(const char *name, const mt_tensor *out, const mt_tensor *delta, con
       g_tconv_patch_launches++;
       return func == MT_F_NONE ? MT_OK : mt_apply_func(out, out, func);
     }
+  }
+  // stride 1, taps that do not tile the k step (3 x 3, 5 x 5): the forward convolution with flipped, transposed kernels
+  if (g_tconv_as_conv && !fused && mt::igemm::tile_override() < 0 && sx == 1 && sy == 1 && BK % (uint32_t)(kx * ky) != 0 && ka % BK == 0 && kz >= 16 &&
+      bias->w == 1 && delta->w == out->w && px <= kx - 1 && py <= ky - 1 && out->y == delta->y + (uint32_t)(ky - 1 - 2 * py) &&
+      out->x == delta->x + (uint32_t)(kx - 1 - 2 * px) && func == MT_F_NONE && kernel->x == (uint32_t)(kz * kx * ky) &&
+      (size_t)ka * kx * ky >= 256 && mt::fits_buffer(out) && mt::fits_buffer(delta)) {
+    const uint32_t taps = (uint32_t)(kx * ky), cols = ka * taps;
+    const size_t flip_floats = ((size_t)kz * cols + (size_t)kz + 1 + 3) & ~(size_t)3;
+    float *buf = nullptr;
+    if ((rc = mt::workspace_get(g_merge_ws, "flipped kernels", flip_floats, &buf))) return rc;
+    {
+      mt::ProfileScope prof("tconv_prepare");
+      tconv_s1_flip_kernel<<<cdiv((size_t)kz * cols + kz + 1, 256), 256, 0, mt::stream()>>>(buf, kernel->p, bias->p, kernel->x, (uint32_t)kz, ka, taps);
+      MT_LAUNCH_CHECK(name);
+    }
+    mt::note_write(buf, flip_floats * sizeof(float));   // (a re-ordered copy of these weights that the forward path kept is stale)
+    mt_tensor flipped{buf, 1, 1, (uint32_t)kz, cols}, zeros{buf + (size_t)kz * cols, 1, (uint32_t)kz, 1, 1};
+    if ((rc = forward(name, out, delta, &flipped, kx, ky, (int32_t)ka, (uint32_t)kz, &zeros, 1, 1, kx - 1 - px, ky - 1 - py, MT_F_NONE))) return rc;
+    {
+      mt::ProfileScope prof("tconv_tap_bias");
+      tconv_s1_bias_kernel<<<1024, 256, 0, mt::stream()>>>(out->p, buf + (size_t)kz * cols + kz, mt::count(out), out->y, out->x, delta->y, delta->x, ky, kx,
+                                                           ky - 1 - py, kx - 1 - px);
+      MT_LAUNCH_CHECK(name);
+    }
+    g_tconv_as_conv_launches++;
+    return MT_OK;
   }
   // workspace: [bias sums (bias_w, padded to 64)] [packed sub-kernels of all phases: kz*ka*ky*kx floats + alignment]
   size_t sums = (bias->w + 63u) & ~(size_t)63u;
@@ -2484,6 +2547,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "convolution_workspace_bytes") == 0) { *value = (int64_t)(g_ws.floats * sizeof(float)); return true; }
   if (strcmp(name, "wgrad_walk_launches") == 0) { *value = (int64_t)g_wgrad_walk_launches; return true; }
   if (strcmp(name, "wgrad_patch_launches") == 0) { *value = (int64_t)g_wgrad_patch_launches; return true; }
+  if (strcmp(name, "tconv_as_conv_launches") == 0) { *value = (int64_t)g_tconv_as_conv_launches; return true; }
   if (strcmp(name, "tconv_merge_launches") == 0) { *value = (int64_t)g_tconv_merge_launches; return true; }
   if (strcmp(name, "tconv_patch_launches") == 0) { *value = (int64_t)g_tconv_patch_launches; return true; }
   return false;
@@ -2566,6 +2630,11 @@ int set_upconv_split(int v) {
 int set_upconv_walk(int v) {
   if (v < 0) return fail(MT_E_ARGUMENT, "upconv_walk must be 0 (never) or the number of blocks from which the walking kernel is taken");
   g_upconv_walk = v;
+  return MT_OK;
+}
+int set_tconv_as_conv(int v) {
+  if (v != 0 && v != 1) return fail(MT_E_ARGUMENT, "tconv_as_conv must be 0 or 1");
+  g_tconv_as_conv = v;
   return MT_OK;
 }
 int set_tconv_merge(int v) {

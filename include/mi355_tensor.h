@@ -110,6 +110,9 @@ int mt_timer_destroy(void *timer);
  *   "wgrad_pad"      1 (default) mt_convolution_backward_weights_sum appends rows of zeros to delta's images when their pixels
  *                    are not a multiple of 16 (3 x 4 at the end of a discriminator), so that the sum over the batch stays
  *                    one product / 0 per-sample gradients and their sum then
+ *   "tconv_as_conv"  1 (default) mt_backward_convolution with stride 1 and a kernel whose taps do not tile a k step of 16 (3x3, 5x5),
+ *                    a multiple of 16 filters and at least 16 channels runs as the forward convolution with flipped, transposed
+ *                    kernels (k ordered tap-major) / 0 as a transposed convolution
  *   "tconv_merge"    1 (default) mt_backward_convolution 5x5 stride 2 padding 2 to 5..16 channels at twice the input size runs its
  *                    four stride phases as one 3x3 convolution to (channel, phase) rows and spreads them over the output / 0 never
  *   "tconv_patch"    1 (default) mt_backward_convolution of a 3x3 layer with stride 1, padding 1, at most 32 filters and at most 64
@@ -172,6 +175,7 @@ int mt_set_option(const char *name, int value);
  *   "wgrad_walk_launches"                                  calls of mt_convolution_backward_weights_sum that ran as one k loop
  *                                                          per block (option "wgrad_walk")
  *   "wgrad_patch_launches"                                 calls of it that multiplied patches held in LDS (option "wgrad_patch")
+ *   "tconv_as_conv_launches"                               calls of mt_backward_convolution that ran as a forward convolution (option "tconv_as_conv")
  *   "tconv_merge_launches"                                 calls of mt_backward_convolution that ran as one merged convolution (option "tconv_merge")
  *   "tconv_patch_launches"                                 calls of mt_backward_convolution that did (option "tconv_patch") */
 int mt_get_info(const char *name, int64_t *value);

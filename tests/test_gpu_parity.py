@@ -178,6 +178,10 @@ CONV_CASES = [
     (2, 8, 18, 36, 4, 3, 3, 1, 1, 1, 1, 1, 2),      # the same with partial tiles and one bias set per sample
     (2, 8, 8, 8, 256, 4, 4, 2, 2, 1, 1, 1, 1),      # transposed conv with few blocks and k = 1024 per phase: split over k
     (1, 8, 5, 5, 1024, 3, 3, 2, 2, 1, 1, 1, 1),     # the same with phases of 4, 2, 2 and 1 taps (k = 4096 ... 1024)
+    (2, 32, 12, 16, 32, 3, 3, 1, 1, 1, 1, 1, 1),    # 3x3 stride 1, 32 filters to 32 channels: backwards it is the forward convolution with flipped kernels
+    (3, 48, 9, 10, 64, 3, 3, 1, 1, 1, 1, 1, 1),     # the same with 64 filters to 48 channels, ragged image
+    (2, 16, 8, 8, 16, 5, 5, 1, 1, 2, 2, 1, 1),      # 5x5 stride 1 padding 2
+    (2, 16, 6, 6, 32, 3, 3, 1, 1, 0, 0, 1, 1),      # no padding: backwards the output is larger than the input
     (8, 1, 16, 16, 128, 3, 3, 1, 1, 1, 1, 1, 1),    # 128 filters to one channel at 16 x 16: few pixels behind a long k axis, split over k
     (3, 3, 24, 32, 16, 5, 5, 2, 2, 2, 2, 1, 1),     # 5x5 stride 2 padding 2 to three channels (a discriminator's first layer, backwards):
                                                     # the four phases from the 3x3 neighbourhood of an input pixel
@@ -440,6 +444,41 @@ def test_weights_sum_in_bands_of_rows(gpu, oracle, case):
         mt.set_option("wgrad_parts", 1)
     close(got_k, want_k)
     close(got_b, want_b)
+
+
+@pytest.mark.parametrize("case", [
+    # B, C (output channels), H, W (of delta), KA (filters), k, p, taken
+    (4, 128, 24, 32, 64, 3, 1, 1),     # a generator's middle layer backwards: 64 filters to 128 channels
+    (2, 512, 6, 8, 512, 3, 1, 1),      # few pixels behind a long k axis: the forward path splits it over k
+    (3, 40, 10, 12, 32, 5, 2, 1),      # 5x5, 40 channels
+    (3, 40, 10, 12, 32, 3, 0, 1),      # no padding: the output is two pixels larger each way
+    (3, 40, 10, 12, 24, 3, 1, 0),      # 24 filters: not a multiple of a k step, the transposed convolution's own kernels
+    (3, 8, 10, 12, 32, 3, 1, 0),       # 8 channels: too few rows
+])
+def test_stride_1_transposed_convolution_as_forward_convolution(gpu, oracle, case):
+    """The backward pass of a stride-1 layer whose taps do not tile a k step as the forward convolution with flipped,
+    transposed kernels, with a non-zero bias (added once per tap inside the image, cpu/ctensorconv.h:204-268) and with a
+    zero one, against the oracle and against the transposed convolution's own kernels."""
+    import mi355tensor as mt
+    B, C, H, Wd, KA, k, p, taken = case
+    oh, ow = H + k - 1 - 2 * p, Wd + k - 1 - 2 * p
+    delta = U(91, B, KA, H, Wd)
+    kernel = U(92, 1, 1, KA, C * k * k) * np.float32(0.2)
+    for bias in (U(93, 1, KA, 1, 1) * np.float32(0.1), np.zeros((1, KA, 1, 1), np.float32)):
+        args = (delta, kernel, bias, k, k, C, KA, 1, 1, p, p, (B, C, oh, ow))
+        want = oracle.backward_convolution(*args)
+        got = {}
+        try:
+            for on in (1, 0):
+                mt.set_option("tconv_as_conv", on)
+                before = mt.get_info("tconv_as_conv_launches")
+                got[on] = gpu.backward_convolution(*args)
+                assert mt.get_info("tconv_as_conv_launches") - before == (taken if on else 0)
+        finally:
+            mt.set_option("tconv_as_conv", 1)
+        close(got[1], want)
+        close(got[0], want)
+        close(got[1], got[0], 2e-6)
 
 
 @pytest.mark.parametrize("case", [
