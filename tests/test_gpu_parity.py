@@ -543,6 +543,7 @@ def test_transposed_convolution_from_patches_in_lds(gpu, oracle, case):
         want = oracle.apply_func(want, func)
     got = {}
     try:
+        mt.set_option("tconv_as_conv", 0)   # (which takes a multiple of 16 filters from 32 on)
         for on in (1, 0):
             mt.set_option("tconv_patch", on)
             before = mt.get_info("tconv_patch_launches")
@@ -550,9 +551,14 @@ def test_transposed_convolution_from_patches_in_lds(gpu, oracle, case):
             assert mt.get_info("tconv_patch_launches") - before == (taken if on else 0)
     finally:
         mt.set_option("tconv_patch", 1)
+        mt.set_option("tconv_as_conv", 1)
     close(got[1], want)
     close(got[0], want)
     close(got[1], got[0], 2e-6)
+    if KA == 32 and taken and func is None:   # both routes on: 32 filters go to the forward convolution, 16 stay here
+        before = mt.get_info("tconv_as_conv_launches")
+        close(gpu.backward_convolution(*args), want)
+        assert mt.get_info("tconv_as_conv_launches") == before + 1
 
 
 @pytest.mark.parametrize("case", [
