@@ -205,10 +205,43 @@ int mt_free(void *ptr) {
   return MT_OK;
 }
 
+// Small uploads (a layer's time steps, a batch of noise, a label) go through pinned staging slots: the caller's buffer is
+// copied at once and may be reused on return, the copy to the device is queued like a kernel -- waiting for it here would
+// wait for everything queued in front of it, and a layer that uploads 128 bytes per forward pass would drain the queue
+// every time.  A slot is taken again when its own copy is over (an event per slot).
+namespace {
+constexpr size_t STAGE_SLOT_BYTES = (size_t)64 << 10;
+constexpr int STAGE_SLOTS = 64;
+char *g_stage = nullptr;
+hipEvent_t g_stage_done[STAGE_SLOTS];
+bool g_stage_used[STAGE_SLOTS];
+int g_stage_next = 0, g_staged_uploads = 1;
+uint64_t g_staged_count = 0;
+}  // namespace
+
 int mt_copy_h2d(void *dst, const void *src, size_t bytes) {
   if (bytes == 0) return MT_OK;
   if (dst == nullptr || src == nullptr) return mt::fail(MT_E_ARGUMENT, "mt_copy_h2d: null pointer");
   mt::note_write(dst, bytes);
+  if (g_staged_uploads && bytes <= STAGE_SLOT_BYTES && !capturing_now()) {
+    if (g_stage == nullptr) {
+      MT_HIP(hipHostMalloc((void **)&g_stage, STAGE_SLOT_BYTES * STAGE_SLOTS, hipHostMallocPortable));
+      for (int i = 0; i < STAGE_SLOTS; i++) {
+        MT_HIP(hipEventCreateWithFlags(&g_stage_done[i], hipEventDisableTiming));
+        g_stage_used[i] = false;
+      }
+    }
+    const int slot = g_stage_next;
+    g_stage_next = (slot + 1) % STAGE_SLOTS;
+    if (g_stage_used[slot]) MT_HIP(hipEventSynchronize(g_stage_done[slot]));
+    char *staged = g_stage + (size_t)slot * STAGE_SLOT_BYTES;
+    memcpy(staged, src, bytes);
+    MT_HIP(hipMemcpyAsync(dst, staged, bytes, hipMemcpyHostToDevice, g_stream));
+    MT_HIP(hipEventRecord(g_stage_done[slot], g_stream));
+    g_stage_used[slot] = true;
+    g_staged_count++;
+    return MT_OK;
+  }
   MT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
   MT_HIP(hipStreamSynchronize(g_stream));  // the host buffer may be reused on return
   return MT_OK;
@@ -274,6 +307,11 @@ int mt_set_option(const char *name, int value) {
   if (name && strcmp(name, "walk_order") == 0) return mt::set_walk_order(value);
   if (name && strcmp(name, "walk_fair") == 0) return mt::set_walk_fair(value);
   if (name && strcmp(name, "igemm_fair") == 0) return mt::set_igemm_fair(value);
+  if (name && strcmp(name, "staged_uploads") == 0) {
+    if (value != 0 && value != 1) return mt::fail(MT_E_ARGUMENT, "staged_uploads must be 0 or 1");
+    g_staged_uploads = value;
+    return MT_OK;
+  }
   if (name && strcmp(name, "pool") == 0) {
     if (value != 0 && value != 1) return mt::fail(MT_E_ARGUMENT, "pool must be 0 (every mt_free goes to the driver) or 1");
     g_pool_on = value != 0;
@@ -341,6 +379,7 @@ int mt_get_info(const char *name, int64_t *value) {
   if (strcmp(name, "pool_bytes") == 0) { *value = (int64_t)g_pool_bytes; return MT_OK; }
   if (strcmp(name, "pool_reused") == 0) { *value = (int64_t)g_pool_reused; return MT_OK; }
   if (strcmp(name, "driver_allocations") == 0) { *value = (int64_t)g_driver_allocs; return MT_OK; }
+  if (strcmp(name, "staged_uploads") == 0) { *value = (int64_t)g_staged_count; return MT_OK; }
   if (strcmp(name, "retired_workspaces") == 0) { *value = (int64_t)mt::retired_workspaces(); return MT_OK; }
   if (strcmp(name, "retired_blocks") == 0) { *value = (int64_t)g_retired_blocks; return MT_OK; }
   if (strcmp(name, "retired_bytes") == 0) { *value = (int64_t)g_retired_bytes; return MT_OK; }

@@ -154,6 +154,8 @@ int mt_timer_destroy(void *timer);
  *   "image_strip"    rows per strip of the image layer's product kernel on images of 64 columns (0, default: 8 or 4)
  *   "nontemporal"    2 (default) the re-sampling, pooling and large-batch batch-norm kernels read and write tensors of 128 MiB
  *                    and more past the caches (each element is touched once) / 1 always / 0 never
+ *   "staged_uploads" 1 (default) mt_copy_h2d of at most 64 KiB copies the caller's buffer into a pinned slot at once and queues
+ *                    the copy to the device behind the work already queued, without waiting for it / 0 every upload waits
  *   "pool"           1 (default) mt_free keeps blocks for the next mt_malloc of the same size (stream-ordered reuse, no
  *                    wait) / 0 every mt_free waits for the stream and returns the block to the driver
  *   "pool_limit_mib" MiB the pool may hold in free blocks (default 4096) */
@@ -162,6 +164,7 @@ int mt_set_option(const char *name, int value);
  *   "pool_bytes", "pool_reused", "driver_allocations"      the memory pool behind mt_malloc / mt_free
  *   "retired_blocks", "retired_bytes"                      blocks freed (or handed out) while the stream was being captured:
  *                                                          a recorded graph names them, so they are never handed out again
+ *   "staged_uploads"                                       uploads that went through a pinned slot (option "staged_uploads")
  *   "retired_workspaces"                                   outgrown workspaces that a recorded graph may still use
  *   "convolution_workspace_bytes"                          size of the convolutions' workspace (it only grows)
  *   "pack_cache_entries", "pack_cache_valid", "pack_cache_hits", "pack_cache_made", "pack_cache_bytes"

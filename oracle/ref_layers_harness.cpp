@@ -874,6 +874,87 @@ static void TimeVae(uint32_t batch,uint32_t warmup,uint32_t steps)
         batch,steps,ms,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),sum,driver_allocations_in_the_timed_steps);
 }
 
+// The reference's diffusion model (cuda/netmodel/cmodel_diffusion.cu.h:106-230), whole training step in Adam mode, batch 32, 192x256 images:
+// a U-net.  Down: five blocks (Convolution 3x3, TimeEmbedding, leaky ReLU, Splitter, Convolution 3x3 stride 2) with 16, 32, 64, 128, 256
+// filters; bottom: three times (Convolution 3x3 to 512 filters, TimeEmbedding, leaky ReLU) at 6x8; up: five blocks (UpSampling 2x2,
+// Concatenator with the splitter of the same size, Convolution 3x3, TimeEmbedding, leaky ReLU) with 256, 128, 64, 32, 16 filters; then
+// Convolution 3x3 to 16 filters, leaky ReLU, Convolution 3x3 to the image.  The time steps are set before every step, sample by sample
+// and layer by layer, as the model does (cuda/netmodel/cmodel_basicdiffusion.cu.h:303).
+static void TimeDiffusion(uint32_t batch,uint32_t warmup,uint32_t steps)
+{
+ rng_state=0x082EFA98EC4E6C89ull;
+ std::vector<std::shared_ptr<INetLayer<type_t> > > owner;
+ std::vector<INetLayer<type_t>*> net;
+#define PUSH(LAYER) {owner.push_back(std::shared_ptr<INetLayer<type_t> >(LAYER));net.push_back(owner.back().get());}
+#define BLOCK(FILTERS,DEPTH) {PUSH(new CNetLayerConvolution<type_t>(FILTERS,3,1,1,1,1,net.back(),batch));LoadConvolution(*net.back(),FILTERS,3,DEPTH,1,1);\
+                              PUSH(new CNetLayerTimeEmbedding<type_t>(net.back(),batch));\
+                              PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_LEAKY_RELU,net.back(),batch));}
+ PUSH(new CNetLayerConvolutionInput<type_t>(3,192,256,batch));
+ static const uint32_t down[6]={3,16,32,64,128,256};
+ INetLayer<type_t> *split[5];
+ for(uint32_t i=0;i<5;i++)
+ {
+  BLOCK(down[i+1],down[i]);
+  PUSH(new CNetLayerSplitter<type_t>(2,net.back(),batch));
+  split[i]=net.back();
+  PUSH(new CNetLayerConvolution<type_t>(down[i+1],3,2,2,1,1,net.back(),batch));
+  LoadConvolution(*net.back(),down[i+1],3,down[i+1],2,1);
+ }
+ BLOCK(512,256);
+ BLOCK(512,512);
+ BLOCK(512,512);
+ uint32_t depth=512;
+ for(int i=4;i>=0;i--)
+ {
+  PUSH(new CNetLayerUpSampling<type_t>(2,2,net.back(),batch));
+  PUSH(new CNetLayerConcatenator<type_t>(net.back(),split[i],batch));
+  BLOCK(down[i+1],depth+down[i+1]);
+  depth=down[i+1];
+ }
+ PUSH(new CNetLayerConvolution<type_t>(16,3,1,1,1,1,net.back(),batch));
+ LoadConvolution(*net.back(),16,3,16,1,1);
+ PUSH(new CNetLayerFunction<type_t>(NNeuron::NEURON_FUNCTION_LEAKY_RELU,net.back(),batch));
+ PUSH(new CNetLayerConvolution<type_t>(3,3,1,1,1,1,net.back(),batch));
+ LoadConvolution(*net.back(),3,3,16,1,1);
+#undef BLOCK
+#undef PUSH
+ for(size_t n=0;n<net.size();n++)
+ {
+  net[n]->TrainingModeAdam(0.9,0.999);   // as the model trains it (cuda/netmodel/cmodel_basicdiffusion.cu.h:598)
+  net[n]->TrainingStart();
+ }
+ CTensor<type_t> image(batch,3,192,256),error(batch,3,192,256);
+ FillTensor(image,1.0);
+ FillTensor(error,0.01);
+ net[0]->SetOutput(image);
+ double ms=0;
+ int64_t before=0,after=0;
+ for(uint32_t pass=0;pass<2;pass++)
+ {
+  const uint32_t count=(pass==0)?warmup:steps;
+  mt_get_info("driver_allocations",&before);
+  CCUDATimeSpent timer;
+  timer.Start();
+  for(uint32_t step=0;step<count;step++)
+  {
+   for(uint32_t b=0;b<batch;b++)
+    for(size_t n=0;n<net.size();n++) net[n]->SetTimeStep(b,(b*37+step*11)%1000);
+   for(size_t n=0;n<net.size();n++) net[n]->Forward();
+   for(size_t n=0;n<net.size();n++) net[n]->TrainingResetDeltaWeight();
+   net[net.size()-1]->SetOutputError(error);
+   for(size_t n=net.size()-1;n>=1;n--) net[n]->TrainingBackward(true);
+   for(size_t n=1;n<net.size();n++) net[n]->TrainingUpdateWeight(0.0002,step+1);
+  }
+  ms=timer.Stop();
+  mt_get_info("driver_allocations",&after);
+ }
+ CTensor<type_t> &out=net.back()->GetOutputTensor();
+ double sum=0;
+ for(uint32_t x=0;x<256;x++) sum+=fabs(out.GetElement(batch-1,2,191,x));
+ printf("{\"chain\": \"diffusion_step\", \"batch\": %u, \"steps\": %u, \"ms_per_step\": %.4f, \"output\": [%u,%u,%u,%u], \"last_row_abs_sum\": %.6f, \"driver_allocations_in_the_timed_steps\": %lld}\n",
+        batch,steps,ms/steps,out.GetSizeW(),out.GetSizeZ(),out.GetSizeY(),out.GetSizeX(),sum,static_cast<long long>(after-before));
+}
+
 // Chain K: two training steps (gradient descent) of the discriminator at batch 16, once with the per-sample weight gradients deferred by the
 // drop-in classes (mi355::CDeferredGradient; the last two convolution layers qualify) and once with every call run when
 // it is made: same seeds, the updated convolution weights of both runs go to the dump
@@ -1012,7 +1093,7 @@ int main(int argc,char **argv)
    fclose(out_file);
    return(0);
   }
-  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up [literal | train | vae]]]
+  if (argc>2 && strcmp(argv[2],"time")==0)   // only the timed chains: time [steps [warm-up [literal | train | vae | diffusion]]]
   {
    const uint32_t steps=(argc>3)?static_cast<uint32_t>(atoi(argv[3])):50,warmup=(argc>4)?static_cast<uint32_t>(atoi(argv[4])):20;
    TimeGenerator(256,warmup,steps);
@@ -1024,6 +1105,7 @@ int main(int argc,char **argv)
     TimeGanDiscriminator(32,warmup,steps);
    }
    if (argc>5 && strcmp(argv[5],"vae")==0) TimeVae(32,warmup,steps);   // or the whole training step of the reference's VAE model
+   if (argc>5 && strcmp(argv[5],"diffusion")==0) TimeDiffusion(32,warmup,steps);   // or that of its diffusion model
    if (argc>5 && strcmp(argv[5],"literal")==0)   // and the last chain once more with every call run when it is made
    {
     mi355::DeferGradients()=false;

@@ -351,3 +351,35 @@ def test_workspace_growth_around_a_recording(mt):
         assert np.array_equal(small_out.numpy(), eager)
     finally:
         mt.set_option("pack_cache", 1)
+
+
+def test_small_uploads_go_through_pinned_slots(mt):
+    """Uploads of at most 64 KiB are queued behind the work already queued instead of waiting for it: the caller's buffer is
+    copied at once (it is overwritten right after the call here), the slots are taken again after 64 uploads, and the
+    order with the kernels around them is kept.  Larger uploads and the option's other value wait as before."""
+    from mi355tensor import CTensor, CTensorMath as M
+    big = CTensor.from_numpy(Nrm(60, 8, 16, 64, 64))         # some queued work in front of every upload
+    acc = CTensor.from_numpy(np.zeros((1, 1, 8, 16), np.float32))
+    want = np.zeros((1, 1, 8, 16), np.float32)
+    try:
+        for staged in (1, 0):
+            mt.set_option("staged_uploads", staged)
+            before = mt.get_info("staged_uploads")
+            buf = np.zeros((1, 1, 8, 16), np.float32)
+            t = CTensor(1, 1, 8, 16)
+            for i in range(150):                              # more uploads than there are slots
+                buf[...] = float(i + 1)
+                t.upload(buf)
+                buf[...] = -1.0                               # the caller's buffer is free again
+                M.Add(big, big, big, 0.5, 0.5)                # queued work between the uploads
+                M.Add(acc, acc, t, 1.0, 1.0)
+                want += float(i + 1)
+            assert mt.get_info("staged_uploads") - before == (150 if staged else 0)
+            assert np.array_equal(acc.numpy(), want)
+        mt.set_option("staged_uploads", 1)
+        before = mt.get_info("staged_uploads")
+        large = Nrm(61, 1, 1, 256, 128)                       # 128 KiB: waits, as before
+        assert np.array_equal(CTensor.from_numpy(large).numpy(), large)
+        assert mt.get_info("staged_uploads") == before
+    finally:
+        mt.set_option("staged_uploads", 1)
