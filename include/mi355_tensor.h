@@ -75,7 +75,8 @@ int mt_init(int device);                 /* cuda/cuda.cu:81 (cudaSetDevice); che
 const char *mt_last_error(void);
 int mt_malloc(void **ptr, size_t bytes); /* ccudadevicevector.cu.h resize   */
 int mt_free(void *ptr);                  /* ccudadevicevector.cu.h clear    */
-int mt_copy_h2d(void *dst, const void *src, size_t bytes); /* copy_host_to_device */
+int mt_copy_h2d(void *dst, const void *src, size_t bytes); /* copy_host_to_device; src may be reused on return; the copy is in
+                                                             stream order (at most 64 KiB: queued, not waited for) */
 int mt_copy_d2h(void *dst, const void *src, size_t bytes); /* copy_device_to_host; waits for queued work */
 int mt_copy_d2d(void *dst, const void *src, size_t bytes); /* operator= (device copy, :159-170) */
 /* Tells the library that someone else (another library's kernel, a hipMemcpy of the caller's) wrote [ptr, ptr+bytes).
