@@ -29,6 +29,7 @@ int set_igemm_fair(int v);
 int set_first_layer(int v);   // forward convolutions of 3-channel images on the input-patch kernel: 0 never, 1 wherever the shape allows
 int set_nontemporal(int v);   // streaming kernels read and write past the caches: 0 never, 1 always, 2 tensors of 128 MiB and more
 int set_image_strip(int v);   // rows per strip of the image layer's product kernel on 64-column images (0: choose)
+int set_conv_patch(int v);     // 3x3 stride-1 forward convolutions from at most 32 channels on large images from patches in LDS: 1 (default) / 0 never / n: from n filters on
 int set_tconv_as_conv(int v);  // stride-1 transposed convolutions with 3x3 (5x5 ...) taps as forward convolutions with flipped kernels: 1 (default) / 0 never
 int set_tconv_merge(int v);  // 5x5 stride-2 padding-2 transposed convolutions to 5..16 channels as one 3x3 convolution to (channel, phase) rows: 1 (default) / 0 never
 int set_tconv_patch(int v);  // 3x3 stride-1 transposed convolutions from at most 32 filters on large images from patches in LDS: 1 (default) / 0 never

@@ -34,7 +34,9 @@ int g_walk_wide = 1;       // 1: layers whose output channels are a multiple of 
 int g_upconv_split = 1;    // 1: up-sampling convolutions with fewer than 512 walking blocks share a tile's k steps between blocks
 int g_upconv_walk = 512;   // blocks from which the up-sampling convolution takes the walking kernel (0: never; measured on the
                            // shipped GAN generator at batch 32: 768 blocks 67.7 -> 54.6 and 58.6 -> 54.0 us, 384 blocks 65.1 -> 69 us)
-uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0, g_tconv_patch_launches = 0, g_tconv_merge_launches = 0, g_tconv_as_conv_launches = 0;
+uint64_t g_wgrad_walk_launches = 0, g_wgrad_patch_launches = 0, g_tconv_patch_launches = 0, g_tconv_merge_launches = 0, g_tconv_as_conv_launches = 0, g_conv_patch_launches = 0;
+int g_conv_patch = 1;     // 1: a 3x3 stride-1 forward convolution from at most 32 channels to g_conv_patch_min..64 filters on large images multiplies patches held in LDS, 0: never
+int g_conv_patch_min = 5;
 int g_tconv_as_conv = 1;   // 1: a stride-1 transposed convolution whose taps do not tile the k step (3x3) runs as the forward convolution with flipped kernels, 0: never
 int g_tconv_merge = 1;   // 1: a 5x5 stride-2 padding-2 transposed convolution to 5..16 channels runs as one 3x3 convolution to (channel, phase) rows, 0: never
 int g_tconv_patch = 1;   // 1: a 3x3 stride-1 transposed convolution from at most 32 filters to at most 64 channels on large images multiplies patches held in LDS (tconv3x3_patch_kernel), 0: never
@@ -1586,6 +1588,24 @@ int forward(const char *name, const mt_tensor *out, const mt_tensor *image, cons
       return mt::epilogue_func(func) ? MT_OK : mt_apply_func(out, out, func);
     }
   }
+  // 3 x 3, stride 1, padding 1 from at most 32 channels on large images: the nine taps share one patch of the image in LDS,
+  // the weights live in registers (mt_convpatch.h)
+  if (g_conv_patch && kx == 3 && ky == 3 && sx == 1 && sy == 1 && px == 1 && py == 1 && kernel->w == 1 && bias->w == 1 && image->w == out->w &&
+      mt::igemm::tile_override() < 0 && kz <= 32 && ka >= (uint32_t)g_conv_patch_min && ka <= 64 && (kz <= 16 || ka <= 16) && image->y == out->y &&
+      image->x == out->x) {   // (32 channels to 32 or 64 filters: the general kernel is as fast or faster, 322 against 364 us at 192 x 256, batch 32)
+    mt::igemm::TconvPatchArgs cp{};
+    cp.delta = image->p; cp.kernel = kernel->p; cp.bias = bias->p; cp.out = out->p;
+    cp.B = out->w; cp.F = (uint32_t)kz; cp.C = ka; cp.H = out->y; cp.W = out->x; cp.ld = kernel->x;
+    cp.func = mt::epilogue_func(func) ? func : MT_F_NONE;
+    if (mt::igemm::tconv_patch_plan(cp)) {
+      {
+        mt::ProfileScope prof(mt::profiling() ? shape_label(name, T16x256, ka, out->w * OHW, K, 1) : name);
+        if ((rc = mt::igemm::launch_conv_patch(name, cp))) return rc;
+      }
+      g_conv_patch_launches++;
+      return mt::epilogue_func(func) ? MT_OK : mt_apply_func(out, out, func);
+    }
+  }
   // Taps that tile the k step (4x4, 2x2, 1x1 kernels), one kernel and bias set, whole 64-channel row tiles: the kernel whose
   // blocks walk over the batch runs it (see mt_walk.h) when that gives at least two blocks per compute unit; products
   // with fewer tiles and a long k axis are better cut over k (launch_split below).
@@ -2550,6 +2570,7 @@ bool pack_cache_info(const char *name, int64_t *value) {
   if (strcmp(name, "convolution_workspace_bytes") == 0) { *value = (int64_t)(g_ws.floats * sizeof(float)); return true; }
   if (strcmp(name, "wgrad_walk_launches") == 0) { *value = (int64_t)g_wgrad_walk_launches; return true; }
   if (strcmp(name, "wgrad_patch_launches") == 0) { *value = (int64_t)g_wgrad_patch_launches; return true; }
+  if (strcmp(name, "conv_patch_launches") == 0) { *value = (int64_t)g_conv_patch_launches; return true; }
   if (strcmp(name, "tconv_as_conv_launches") == 0) { *value = (int64_t)g_tconv_as_conv_launches; return true; }
   if (strcmp(name, "tconv_merge_launches") == 0) { *value = (int64_t)g_tconv_merge_launches; return true; }
   if (strcmp(name, "tconv_patch_launches") == 0) { *value = (int64_t)g_tconv_patch_launches; return true; }
@@ -2633,6 +2654,12 @@ int set_upconv_split(int v) {
 int set_upconv_walk(int v) {
   if (v < 0) return fail(MT_E_ARGUMENT, "upconv_walk must be 0 (never) or the number of blocks from which the walking kernel is taken");
   g_upconv_walk = v;
+  return MT_OK;
+}
+int set_conv_patch(int v) {
+  if (v < 0 || v > 64) return fail(MT_E_ARGUMENT, "conv_patch must be 0 (never), 1 (from 5 filters on) or the smallest number of filters (2..64)");
+  g_conv_patch = v != 0;
+  g_conv_patch_min = v <= 1 ? 5 : v;
   return MT_OK;
 }
 int set_tconv_as_conv(int v) {

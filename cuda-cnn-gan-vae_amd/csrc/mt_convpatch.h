@@ -30,6 +30,7 @@ struct TconvPatchArgs {
   float *out;            // [B][C][H][W]
   uint32_t B, F, C, H, W, ld;
   uint32_t groups;       // persistent blocks
+  int func;              // forward convolution only: the function behind it (none, linear, ReLU, leaky ReLU)
 };
 
 namespace tpatch {
@@ -38,8 +39,11 @@ constexpr int P_ROW = PX + 8;                       // the 64 pixels at 4 .. 67 
 constexpr int P_PLANE = (ROWS + 2) * P_ROW + 16;    // = 16 mod 32 banks: the four filters of an instruction read disjoint banks
 }  // namespace tpatch
 
-// FQ: filters / 4, rounded up to 1, 2, 4 or 8; NC: output channels / 16, rounded up (1, 2 or 4)
-template <int FQ, int NC>
+// FQ: filters / 4, rounded up to 1, 2, 4 or 8; NC: output channels / 16, rounded up (1, 2 or 4).
+// FWD: the forward convolution of such a layer on the same machine -- `delta` is the image (F channels), `kernel` is
+// [C][ld] with column f*9 + a*3 + b, tap (a, b) reads image[f][y + a - 1][x + b - 1], `bias` holds one value per output
+// channel and `func` follows:  out[c][y][x] = func(bias[c] + sum kernel[c][f*9 + a*3 + b] * image[f][y + a - 1][x + b - 1]).
+template <int FQ, int NC, bool FWD = false>
 __global__ __launch_bounds__(THREADS) void tconv3x3_patch_kernel(TconvPatchArgs a) {
   using namespace tpatch;
   constexpr int NP = FQ * 4;             // planes of the patch
@@ -57,10 +61,15 @@ __global__ __launch_bounds__(THREADS) void tconv3x3_patch_kernel(TconvPatchArgs 
   for (int q = 0; q < FQ; q++) {
     const uint32_t f = 4 * q + (lane >> 4);
 #pragma unroll
-    for (int t = 0; t < 9; t++) wreg[t][q] = f < a.F && c < a.C ? a.kernel[(size_t)f * a.ld + c * 9 + t] : 0.f;
+    for (int t = 0; t < 9; t++)
+      wreg[t][q] = f < a.F && c < a.C ? (FWD ? a.kernel[(size_t)c * a.ld + f * 9 + t] : a.kernel[(size_t)f * a.ld + c * 9 + t]) : 0.f;
   }
-  float bias_sum = 0.f;
-  for (uint32_t f = 0; f < a.F; f++) bias_sum += a.bias[f];
+  float bias_sum = 0.f;   // backward: the sum of the filters' biases; forward: the output channel's own
+  if constexpr (FWD) {
+    bias_sum = c < a.C ? a.bias[c] : 0.f;
+  } else {
+    for (uint32_t f = 0; f < a.F; f++) bias_sum += a.bias[f];
+  }
   // loader: 16 neighbouring threads load one row of 64 pixels; a thread keeps its patch row and quad and steps over the
   // filters.  The halo: thread -> (filter, patch row, side).
   const uint32_t p_q = tid & 15u, p_rr = (tid >> 4) & 3u;
@@ -101,18 +110,20 @@ __global__ __launch_bounds__(THREADS) void tconv3x3_patch_kernel(TconvPatchArgs 
 #pragma unroll
     for (int i = 0; i < NPB; i++) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
     // lane l reads pixel l % 16 of filter 4q + l / 16; output row r needs patch rows r + 2 - a, column x + 5 - b
-    const float *pa = patch + (lane >> 4) * P_PLANE + (lane & 15u) + 5;
+    // (forward: rows r + a, column x + 3 + b)
+    const float *pa = patch + (lane >> 4) * P_PLANE + (lane & 15u) + (FWD ? 3 : 5);
 #pragma unroll
     for (int i = 0; i < NPB; i++) {
       const uint32_t pb = pb0 + i, r = pb >> 2, xb = pb & 3u;
-      const float *pr = pa + (r + 2) * P_ROW + xb * 16;
+      const float *pr = pa + (r + (FWD ? 0 : 2)) * P_ROW + xb * 16;
 #pragma unroll
       for (int ta = 0; ta < 3; ta++)
 #pragma unroll
         for (int tb = 0; tb < 3; tb++)
 #pragma unroll
           for (int q = 0; q < FQ; q++)
-            acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[4 * q * P_PLANE - ta * P_ROW - tb], wreg[ta * 3 + tb][q], acc[i], 0, 0, 0);
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(FWD ? pr[4 * q * P_PLANE + ta * P_ROW + tb] : pr[4 * q * P_PLANE - ta * P_ROW - tb], wreg[ta * 3 + tb][q],
+                                                          acc[i], 0, 0, 0);
     }
     // register v of lane l holds (pixel 4 * (l / 16) + v, channel l % 16) of its block of 16 pixels
     if (c < a.C) {
@@ -120,13 +131,20 @@ __global__ __launch_bounds__(THREADS) void tconv3x3_patch_kernel(TconvPatchArgs 
       for (int i = 0; i < NPB; i++) {
         const uint32_t pb = pb0 + i, r = pb >> 2, xb = pb & 3u;
         const uint32_t y = y0 + r, x = x0 + xb * 16 + 4 * (lane >> 4);
-        const float ny = 3.f - (y == 0 ? 1.f : 0.f) - (y + 1 == a.H ? 1.f : 0.f);
         floatx4 v = acc[i];
-        const float inner = bias_sum * (ny * 3.f);
-        v.x += x == 0 ? bias_sum * (ny * 2.f) : inner;
-        v.y += inner;
-        v.z += inner;
-        v.w += x + 4 == a.W ? bias_sum * (ny * 2.f) : inner;
+        if constexpr (FWD) {
+          v.x = apply_func_epilogue(a.func, v.x + bias_sum);
+          v.y = apply_func_epilogue(a.func, v.y + bias_sum);
+          v.z = apply_func_epilogue(a.func, v.z + bias_sum);
+          v.w = apply_func_epilogue(a.func, v.w + bias_sum);
+        } else {
+          const float ny = 3.f - (y == 0 ? 1.f : 0.f) - (y + 1 == a.H ? 1.f : 0.f);
+          const float inner = bias_sum * (ny * 3.f);
+          v.x += x == 0 ? bias_sum * (ny * 2.f) : inner;
+          v.y += inner;
+          v.z += inner;
+          v.w += x + 4 == a.W ? bias_sum * (ny * 2.f) : inner;
+        }
         *(floatx4 *)(a.out + ((size_t)w * a.C + c) * plane + (size_t)y * a.W + x) = v;
       }
     }
@@ -144,22 +162,25 @@ inline bool tconv_patch_plan(TconvPatchArgs &a) {
   return true;
 }
 
-template <int FQ>
+template <int FQ, bool FWD>
 inline void launch_tconv_patch_nc(const TconvPatchArgs &a) {
   const uint32_t nc = (a.C + 15) / 16;
-  if (nc == 1) tconv3x3_patch_kernel<FQ, 1><<<a.groups, THREADS, 0, stream()>>>(a);
-  else if (nc == 2) tconv3x3_patch_kernel<FQ, 2><<<a.groups, THREADS, 0, stream()>>>(a);
-  else tconv3x3_patch_kernel<FQ, 4><<<a.groups, THREADS, 0, stream()>>>(a);
+  if (nc == 1) tconv3x3_patch_kernel<FQ, 1, FWD><<<a.groups, THREADS, 0, stream()>>>(a);
+  else if (nc == 2) tconv3x3_patch_kernel<FQ, 2, FWD><<<a.groups, THREADS, 0, stream()>>>(a);
+  else tconv3x3_patch_kernel<FQ, 4, FWD><<<a.groups, THREADS, 0, stream()>>>(a);
 }
 
-inline int launch_tconv_patch(const char *name, const TconvPatchArgs &a) {
-  if (a.F <= 4) launch_tconv_patch_nc<1>(a);
-  else if (a.F <= 8) launch_tconv_patch_nc<2>(a);
-  else if (a.F <= 16) launch_tconv_patch_nc<4>(a);
-  else launch_tconv_patch_nc<8>(a);
+template <bool FWD>
+inline int launch_patch(const char *name, const TconvPatchArgs &a) {
+  if (a.F <= 4) launch_tconv_patch_nc<1, FWD>(a);
+  else if (a.F <= 8) launch_tconv_patch_nc<2, FWD>(a);
+  else if (a.F <= 16) launch_tconv_patch_nc<4, FWD>(a);
+  else launch_tconv_patch_nc<8, FWD>(a);
   MT_LAUNCH_CHECK(name);
   return MT_OK;
 }
+inline int launch_tconv_patch(const char *name, const TconvPatchArgs &a) { return launch_patch<false>(name, a); }
+inline int launch_conv_patch(const char *name, const TconvPatchArgs &a) { return launch_patch<true>(name, a); }
 
 }  // namespace igemm
 }  // namespace mt

@@ -295,6 +295,7 @@ int mt_set_option(const char *name, int value) {
   if (name && strcmp(name, "tconv_patch") == 0) return mt::set_tconv_patch(value);
   if (name && strcmp(name, "tconv_merge") == 0) return mt::set_tconv_merge(value);
   if (name && strcmp(name, "tconv_as_conv") == 0) return mt::set_tconv_as_conv(value);
+  if (name && strcmp(name, "conv_patch") == 0) return mt::set_conv_patch(value);
   if (name && strcmp(name, "pack_refresh") == 0) return mt::set_pack_refresh(value);
   if (name && strcmp(name, "adam_vec") == 0) return mt::set_adam_vec(value);
   if (name && strcmp(name, "nontemporal") == 0) return mt::set_nontemporal(value);

@@ -111,6 +111,9 @@ int mt_timer_destroy(void *timer);
  *   "wgrad_pad"      1 (default) mt_convolution_backward_weights_sum appends rows of zeros to delta's images when their pixels
  *                    are not a multiple of 16 (3 x 4 at the end of a discriminator), so that the sum over the batch stays
  *                    one product / 0 per-sample gradients and their sum then
+ *   "conv_patch"     1 (default) mt_forward_convolution 3x3, stride 1, padding 1 from at most 32 channels to 5..64 filters on large
+ *                    images (rows a multiple of 64 pixels, an even number of rows, at least 1024 tiles of 2 x 64 pixels in the
+ *                    batch) multiplies image patches held in LDS, nine taps per patch / 0 never / n (2..64) from n filters on
  *   "tconv_as_conv"  1 (default) mt_backward_convolution with stride 1 and a kernel whose taps do not tile a k step of 16 (3x3, 5x5),
  *                    a multiple of 16 filters and at least 16 channels runs as the forward convolution with flipped, transposed
  *                    kernels (k ordered tap-major) / 0 as a transposed convolution
@@ -179,6 +182,7 @@ int mt_set_option(const char *name, int value);
  *   "wgrad_walk_launches"                                  calls of mt_convolution_backward_weights_sum that ran as one k loop
  *                                                          per block (option "wgrad_walk")
  *   "wgrad_patch_launches"                                 calls of it that multiplied patches held in LDS (option "wgrad_patch")
+ *   "conv_patch_launches"                                  calls of mt_forward_convolution that multiplied patches held in LDS (option "conv_patch")
  *   "tconv_as_conv_launches"                               calls of mt_backward_convolution that ran as a forward convolution (option "tconv_as_conv")
  *   "tconv_merge_launches"                                 calls of mt_backward_convolution that ran as one merged convolution (option "tconv_merge")
  *   "tconv_patch_launches"                                 calls of mt_backward_convolution that did (option "tconv_patch") */

@@ -447,6 +447,43 @@ def test_weights_sum_in_bands_of_rows(gpu, oracle, case):
 
 
 @pytest.mark.parametrize("case", [
+    # B, C (channels), H, W, KA (filters), func, taken
+    (4, 16, 64, 512, 16, None, 1),           # 16 channels to 16 filters: a wave per pair of 16-pixel blocks
+    (8, 8, 32, 512, 16, "leaky_relu", 1),    # 8 channels, the function in the same pass
+    (4, 16, 128, 256, 64, "relu", 1),        # 16 channels to 64 filters: a wave per 16 filters
+    (16, 31, 16, 512, 13, "tangence", 1),    # ragged: 31 channels, 13 filters, a function afterwards
+    (2, 5, 64, 1024, 9, None, 1),            # 5 channels
+    (1, 20, 256, 512, 6, "linear", 1),       # one sample
+    (4, 32, 64, 512, 32, None, 0),           # 32 channels to 32 filters: the general kernel
+    (4, 8, 62, 512, 8, None, 0),             # too few tiles: the general kernel
+])
+def test_forward_convolution_from_patches_in_lds(gpu, oracle, case):
+    """The forward pass of 3 x 3 stride-1 layers with few channels on large images on the kernel that holds the image patch in
+    LDS and the weights in registers, with bias and function, against the oracle and against the general kernel."""
+    import mi355tensor as mt
+    B, C, H, Wd, KA, func, taken = case
+    image = U(101, B, C, H, Wd)
+    kernel = U(102, 1, 1, KA, C * 9) * np.float32(0.2)
+    bias = U(103, 1, KA, 1, 1)
+    args = (image, kernel, bias, 3, 3, C, KA, 1, 1, 1, 1)
+    want = oracle.forward_convolution(*args)
+    if func:
+        want = oracle.apply_func(want, func)
+    got = {}
+    try:
+        for on in (1, 0):
+            mt.set_option("conv_patch", on)
+            before = mt.get_info("conv_patch_launches")
+            got[on] = gpu.forward_convolution(*args, func=func)
+            assert mt.get_info("conv_patch_launches") - before == (taken if on else 0)
+    finally:
+        mt.set_option("conv_patch", 1)
+    close(got[1], want)
+    close(got[0], want)
+    close(got[1], got[0], 5e-6)   # (two orders of summation)
+
+
+@pytest.mark.parametrize("case", [
     # B, C (output channels), H, W (of delta), KA (filters), k, p, taken
     (4, 128, 24, 32, 64, 3, 1, 1),     # a generator's middle layer backwards: 64 filters to 128 channels
     (2, 512, 6, 8, 512, 3, 1, 1),      # few pixels behind a long k axis: the forward path splits it over k
